@@ -1,0 +1,319 @@
+"""ctypes bindings of the CPU oracle (liboracle.so) and, when it has been built, of the reference's own
+ggml shared object (oracle/_ref/libggml_ref.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by bench.py's cpu_baseline leg,
+as the checker.  The product package never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(HERE, "liboracle.so")
+REF_SO = os.path.join(HERE, "_ref", "libggml_ref.so")
+
+# lm_ggml_type values (reference ggml.h:351-391)
+F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
+TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K"}
+BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256}
+BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292}
+VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K)
+
+
+def row_size(t, k):
+    return (k // BLOCK_ELEMS[t]) * BLOCK_BYTES[t]
+
+
+def build(force=False):
+    """Compile liboracle.so (and oracle/_ref when the reference tree is mounted)."""
+    if force or not os.path.exists(ORACLE_SO):
+        subprocess.check_call(["make", "-C", HERE, "oracle"] + (["-B"] if force else []))
+    if os.path.isdir("/root/reference/cactus") and (force or not os.path.exists(REF_SO)):
+        subprocess.check_call(["make", "-C", HERE, "-j8", "ref"])
+
+
+_vp, _i64, _i32, _f32p = C.c_void_p, C.c_int64, C.c_int, C.POINTER(C.c_float)
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a
+
+
+class Oracle:
+    """The restatement.  Arrays in, arrays out; all quantized data travel as uint8 arrays."""
+
+    def __init__(self, path=ORACLE_SO):
+        if not os.path.exists(path):
+            build()
+        self.lib = L = C.CDLL(path)
+        L.orc_fp16_to_fp32.restype = C.c_float
+        L.orc_fp16_to_fp32.argtypes = [C.c_uint16]
+        L.orc_fp32_to_fp16.restype = C.c_uint16
+        L.orc_fp32_to_fp16.argtypes = [C.c_float]
+        for n in ("q8_0", "q8_K", "q4_0_ref", "q8_0_ref", "q4_K_ref", "q6_K_ref"):
+            f = getattr(L, "orc_quantize_row_" + n)
+            f.restype = None
+            f.argtypes = [_vp, _vp, _i64]
+        L.orc_quantize_rows.restype = C.c_size_t
+        L.orc_quantize_rows.argtypes = [_i32, _vp, _vp, _i64, _i64]
+        L.orc_dequantize_row.restype = None
+        L.orc_dequantize_row.argtypes = [_i32, _vp, _vp, _i64]
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K"):
+            f = getattr(L, "orc_vec_dot_" + n)
+            f.restype = C.c_float
+            f.argtypes = [_i64, _vp, _vp, _vp]
+        L.orc_vec_dot_q4_K_q8_K.restype = C.c_float
+        L.orc_vec_dot_q4_K_q8_K.argtypes = [_i64, _vp, _vp, _vp, _vp]
+        L.orc_vec_dot_exact.restype = C.c_double
+        L.orc_vec_dot_exact.argtypes = [_i32, _i64, _vp, _vp, _vp]
+        L.orc_mul_mat.restype = None
+        L.orc_mul_mat.argtypes = [_i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i32]
+
+    # -- scalars
+    def h2f(self, h):
+        return self.lib.orc_fp16_to_fp32(int(h))
+
+    def f2h(self, f):
+        return self.lib.orc_fp32_to_fp16(float(np.float32(f)))
+
+    # -- quantizers
+    def quantize_activation(self, act_type, x):
+        """x [..., K] fp32 -> uint8 [..., row_size]; act_type is Q8_0 (AVX2 semantics) or Q8_K."""
+        x = _f32(x)
+        k = x.shape[-1]
+        rows = x.reshape(-1, k)
+        out = np.zeros((rows.shape[0], row_size(act_type, k)), np.uint8)
+        fn = {Q8_0: self.lib.orc_quantize_row_q8_0, Q8_K: self.lib.orc_quantize_row_q8_K}[act_type]
+        for r in range(rows.shape[0]):
+            fn(_ptr(rows[r]), _ptr(out[r]), k)
+        return out.reshape(x.shape[:-1] + (out.shape[1],))
+
+    def quantize_q8_0_ref(self, x):
+        x = _f32(x)
+        out = np.zeros(row_size(Q8_0, x.size), np.uint8)
+        self.lib.orc_quantize_row_q8_0_ref(_ptr(x), _ptr(out), x.size)
+        return out
+
+    def quantize_weights(self, wtype, w):
+        """w [N, K] fp32 -> uint8 [N, row_size] with the reference's *_ref weight quantizer."""
+        w = _f32(w)
+        n, k = w.shape
+        out = np.zeros((n, row_size(wtype, k)), np.uint8)
+        got = self.lib.orc_quantize_rows(wtype, _ptr(w), _ptr(out), n, k)
+        assert got == out.size
+        return out
+
+    def dequantize(self, t, q, k):
+        q = np.ascontiguousarray(q, np.uint8)
+        rows = q.reshape(-1, row_size(t, k))
+        out = np.zeros((rows.shape[0], k), np.float32)
+        for r in range(rows.shape[0]):
+            self.lib.orc_dequantize_row(t, _ptr(rows[r]), _ptr(out[r]), k)
+        return out.reshape(q.shape[:-1] + (k,))
+
+    # -- dots
+    def vec_dot(self, wtype, k, wrow, arow, want_sums=False):
+        wrow = np.ascontiguousarray(wrow, np.uint8)
+        arow = np.ascontiguousarray(arow, np.uint8)
+        nb = k // BLOCK_ELEMS[wtype]
+        isum = np.zeros(nb, np.int32)
+        imin = np.zeros(nb, np.int32)
+        if wtype == Q4_0:
+            v = self.lib.orc_vec_dot_q4_0_q8_0(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == Q8_0:
+            v = self.lib.orc_vec_dot_q8_0_q8_0(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == Q4_K:
+            v = self.lib.orc_vec_dot_q4_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
+        elif wtype == Q6_K:
+            v = self.lib.orc_vec_dot_q6_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        else:
+            raise ValueError(wtype)
+        v = np.float32(v)
+        return (v, isum, imin) if want_sums else v
+
+    def vec_dot_exact(self, wtype, k, wrow, arow):
+        wrow = np.ascontiguousarray(wrow, np.uint8)
+        arow = np.ascontiguousarray(arow, np.uint8)
+        sa = C.c_double(0)
+        v = self.lib.orc_vec_dot_exact(wtype, k, _ptr(wrow), _ptr(arow), C.byref(sa))
+        return v, sa.value
+
+    def mul_mat(self, wtype, W, x, nthreads=1, want=()):
+        """W uint8 [N, row_size(wtype,K)], x fp32 [n, K] -> y fp32 [n, N].
+        want may name 'wdata' (quantized activations) and/or 'sum_abs' (tolerance yardstick)."""
+        W = np.ascontiguousarray(W, np.uint8)
+        x = _f32(x)
+        n, k = x.shape
+        N = W.shape[0]
+        assert W.shape[1] == row_size(wtype, k)
+        y = np.zeros((n, N), np.float32)
+        wd = np.zeros((n, row_size(VEC_DOT_TYPE[wtype], k)), np.uint8) if "wdata" in want else None
+        sa = np.zeros((n, N), np.float64) if "sum_abs" in want else None
+        self.lib.orc_mul_mat(wtype, k, N, n, _ptr(W), _ptr(x), _ptr(y), _ptr(wd), _ptr(sa), nthreads)
+        out = {"y": y}
+        if wd is not None:
+            out["wdata"] = wd
+        if sa is not None:
+            out["sum_abs"] = sa
+        return out
+
+
+class _InitParams(C.Structure):
+    _fields_ = [("mem_size", C.c_size_t), ("mem_buffer", C.c_void_p), ("no_alloc", C.c_bool)]
+
+
+class Reference:
+    """The reference's own compiled code (oracle/_ref/libggml_ref.so), when present.
+
+    Exposes the hot-path functions directly and the CPU backend's LM_GGML_OP_MUL_MAT through a one-node graph
+    with a persistent threadpool (reference ggml-cpu/ggml-cpu.c:3079, ggml-cpu/ggml-cpu.cpp:238-248)."""
+
+    @staticmethod
+    def available():
+        return os.path.exists(REF_SO)
+
+    def __init__(self, path=REF_SO, mode=C.RTLD_GLOBAL):
+        self.lib = L = C.CDLL(path, mode=mode)
+        L.lm_ggml_cpu_init.restype = None
+        L.lm_ggml_cpu_init()
+        # fp16 table is filled by the first lm_ggml_init (reference ggml.c:1418-1431)
+        L.lm_ggml_init.restype = _vp
+        L.lm_ggml_init.argtypes = [_InitParams]
+        L.lm_ggml_free.argtypes = [_vp]
+        ctx = L.lm_ggml_init(_InitParams(1 << 20, None, False))
+        L.lm_ggml_free(ctx)
+        for n in ("quantize_row_q8_0", "quantize_row_q8_K", "quantize_row_q4_0_ref", "quantize_row_q8_0_ref",
+                  "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref"):
+            f = getattr(L, n)
+            f.restype = None
+            f.argtypes = [_vp, _vp, _i64]
+        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K"):
+            f = getattr(L, "dequantize_row_" + n)
+            f.restype = None
+            f.argtypes = [_vp, _vp, _i64]
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K"):
+            f = getattr(L, "lm_ggml_vec_dot_" + n)
+            f.restype = None
+            f.argtypes = [C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, _vp, C.c_size_t, C.c_int]
+        L.lm_ggml_quantize_chunk.restype = C.c_size_t
+        L.lm_ggml_quantize_chunk.argtypes = [_i32, _vp, _vp, _i64, _i64, _i64, _vp]
+        # graph / backend API (opaque pointers)
+        L.lm_ggml_new_tensor_2d.restype = _vp
+        L.lm_ggml_new_tensor_2d.argtypes = [_vp, _i32, _i64, _i64]
+        L.lm_ggml_mul_mat.restype = _vp
+        L.lm_ggml_mul_mat.argtypes = [_vp, _vp, _vp]
+        L.lm_ggml_new_graph.restype = _vp
+        L.lm_ggml_new_graph.argtypes = [_vp]
+        L.lm_ggml_build_forward_expand.restype = None
+        L.lm_ggml_build_forward_expand.argtypes = [_vp, _vp]
+        L.lm_ggml_backend_cpu_init.restype = _vp
+        L.lm_ggml_backend_cpu_set_n_threads.argtypes = [_vp, _i32]
+        L.lm_ggml_backend_cpu_set_threadpool.argtypes = [_vp, _vp]
+        L.lm_ggml_backend_alloc_ctx_tensors.restype = _vp
+        L.lm_ggml_backend_alloc_ctx_tensors.argtypes = [_vp, _vp]
+        L.lm_ggml_backend_tensor_set.argtypes = [_vp, _vp, C.c_size_t, C.c_size_t]
+        L.lm_ggml_backend_tensor_get.argtypes = [_vp, _vp, C.c_size_t, C.c_size_t]
+        L.lm_ggml_backend_graph_compute.restype = _i32
+        L.lm_ggml_backend_graph_compute.argtypes = [_vp, _vp]
+        L.lm_ggml_backend_buffer_free.argtypes = [_vp]
+        L.lm_ggml_backend_free.argtypes = [_vp]
+        L.lm_ggml_tensor_overhead.restype = C.c_size_t
+        L.lm_ggml_graph_overhead.restype = C.c_size_t
+        L.lm_ggml_threadpool_new.restype = _vp
+        L.lm_ggml_threadpool_new.argtypes = [_vp]
+        L.lm_ggml_threadpool_free.argtypes = [_vp]
+        L.lm_ggml_threadpool_params_init.argtypes = [_vp, _i32]
+
+    _ACT = {Q8_0: "quantize_row_q8_0", Q8_K: "quantize_row_q8_K"}
+    _WQ = {Q4_0: "quantize_row_q4_0_ref", Q8_0: "quantize_row_q8_0_ref",
+           Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref"}
+    _DOT = {Q4_0: "lm_ggml_vec_dot_q4_0_q8_0", Q8_0: "lm_ggml_vec_dot_q8_0_q8_0",
+            Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K"}
+
+    def quantize_activation(self, act_type, x):
+        x = _f32(x)
+        k = x.shape[-1]
+        rows = x.reshape(-1, k)
+        # bsums of an all-zero Q8_K block are left unwritten by the reference: start from zeros
+        out = np.zeros((rows.shape[0], row_size(act_type, k)), np.uint8)
+        fn = getattr(self.lib, self._ACT[act_type])
+        for r in range(rows.shape[0]):
+            fn(_ptr(rows[r]), _ptr(out[r]), k)
+        return out.reshape(x.shape[:-1] + (out.shape[1],))
+
+    def quantize_q8_0_ref(self, x):
+        x = _f32(x)
+        out = np.zeros(row_size(Q8_0, x.size), np.uint8)
+        self.lib.quantize_row_q8_0_ref(_ptr(x), _ptr(out), x.size)
+        return out
+
+    def quantize_weights(self, wtype, w):
+        w = _f32(w)
+        n, k = w.shape
+        out = np.zeros((n, row_size(wtype, k)), np.uint8)
+        fn = getattr(self.lib, self._WQ[wtype])
+        for r in range(n):
+            fn(_ptr(w[r]), _ptr(out[r]), k)
+        return out
+
+    def dequantize(self, t, q, k):
+        q = np.ascontiguousarray(q, np.uint8)
+        rows = q.reshape(-1, row_size(t, k))
+        out = np.zeros((rows.shape[0], k), np.float32)
+        fn = getattr(self.lib, "dequantize_row_" + TYPE_NAMES[t])
+        for r in range(rows.shape[0]):
+            fn(_ptr(rows[r]), _ptr(out[r]), k)
+        return out.reshape(q.shape[:-1] + (k,))
+
+    def vec_dot(self, wtype, k, wrow, arow):
+        wrow = np.ascontiguousarray(wrow, np.uint8)
+        arow = np.ascontiguousarray(arow, np.uint8)
+        s = C.c_float(0)
+        getattr(self.lib, self._DOT[wtype])(k, C.byref(s), 0, _ptr(wrow), 0, _ptr(arow), 0, 1)
+        return np.float32(s.value)
+
+    def mul_mat_graph(self, wtype, W, x, nthreads=1, repeat=1):
+        """LM_GGML_OP_MUL_MAT on the reference CPU backend.  Returns (y [n,N], seconds per compute: list)."""
+        import time
+        L = self.lib
+        W = np.ascontiguousarray(W, np.uint8)
+        x = _f32(x)
+        n, k = x.shape
+        N = W.shape[0]
+        ctx = L.lm_ggml_init(_InitParams(L.lm_ggml_tensor_overhead() * 8 + L.lm_ggml_graph_overhead() + 4096,
+                                         None, True))
+        a = L.lm_ggml_new_tensor_2d(ctx, wtype, k, N)
+        b = L.lm_ggml_new_tensor_2d(ctx, F32, k, n)
+        c = L.lm_ggml_mul_mat(ctx, a, b)
+        g = L.lm_ggml_new_graph(ctx)
+        L.lm_ggml_build_forward_expand(g, c)
+        be = L.lm_ggml_backend_cpu_init()
+        L.lm_ggml_backend_cpu_set_n_threads(be, nthreads)
+        tpp = (C.c_char * 1024)()          # struct lm_ggml_threadpool_params (opaque, generously sized)
+        L.lm_ggml_threadpool_params_init(C.byref(tpp), nthreads)
+        tp = L.lm_ggml_threadpool_new(C.byref(tpp))
+        L.lm_ggml_backend_cpu_set_threadpool(be, tp)
+        buf = L.lm_ggml_backend_alloc_ctx_tensors(ctx, be)
+        L.lm_ggml_backend_tensor_set(a, _ptr(W), 0, W.size)
+        L.lm_ggml_backend_tensor_set(b, _ptr(x), 0, x.size * 4)
+        times = []
+        for _ in range(repeat):
+            t0 = time.perf_counter()
+            st = L.lm_ggml_backend_graph_compute(be, g)
+            times.append(time.perf_counter() - t0)
+            assert st == 0
+        y = np.zeros((n, N), np.float32)
+        L.lm_ggml_backend_tensor_get(c, _ptr(y), 0, y.size * 4)
+        L.lm_ggml_backend_buffer_free(buf)
+        L.lm_ggml_backend_free(be)
+        L.lm_ggml_threadpool_free(tp)
+        L.lm_ggml_free(ctx)
+        return y, times

@@ -1,0 +1,715 @@
+/*
+ * oracle.c -- CPU restatement of the reference's quantized MUL_MAT path (see oracle.h for scope and pinning).
+ * TEST INFRASTRUCTURE ONLY: never linked into, loaded by, or used as a fallback for the product library.
+ *
+ * Reference paths are relative to the reference's cactus/ directory.  Build with -ffp-contract=off: the only
+ * fused multiply-adds are the explicit fmaf() calls that mirror the reference's _mm256_fmadd_ps/_mm_fmadd_ps.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---------------------------------------------------------------- block layouts (ggml-common.h:167-172,
+ * 209-214, 285-296, 320-326, 329-334).  On-disk == in-memory; all little endian. */
+#pragma pack(push, 1)
+typedef struct { uint16_t d; uint8_t qs[16]; } blk_q4_0;
+typedef struct { uint16_t d; int8_t qs[32]; } blk_q8_0;
+typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[128]; } blk_q4_K;
+typedef struct { uint8_t ql[128]; uint8_t qh[64]; int8_t scales[16]; uint16_t d; } blk_q6_K;
+typedef struct { float d; int8_t qs[256]; int16_t bsums[16]; } blk_q8_K;
+#pragma pack(pop)
+
+_Static_assert(sizeof(blk_q4_0) == 18, "q4_0");
+_Static_assert(sizeof(blk_q8_0) == 34, "q8_0");
+_Static_assert(sizeof(blk_q4_K) == 144, "q4_K");
+_Static_assert(sizeof(blk_q6_K) == 210, "q6_K");
+_Static_assert(sizeof(blk_q8_K) == 292, "q8_K");
+
+int orc_block_elems(int type) {
+    switch (type) {
+        case ORC_TYPE_F32: return 1;
+        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: return 32;
+        case ORC_TYPE_Q4_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
+        default: return 0;
+    }
+}
+size_t orc_block_bytes(int type) {
+    switch (type) {
+        case ORC_TYPE_F32: return 4;
+        case ORC_TYPE_Q4_0: return 18;
+        case ORC_TYPE_Q8_0: return 34;
+        case ORC_TYPE_Q4_K: return 144;
+        case ORC_TYPE_Q6_K: return 210;
+        case ORC_TYPE_Q8_K: return 292;
+        default: return 0;
+    }
+}
+size_t orc_row_size(int type, int64_t k) {
+    int be = orc_block_elems(type);
+    return be ? (size_t)(k / be) * orc_block_bytes(type) : 0;
+}
+int orc_vec_dot_type(int type) {
+    switch (type) { /* ggml-cpu/ggml-cpu.c:213,245,272,284 */
+        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: return ORC_TYPE_Q8_0;
+        case ORC_TYPE_Q4_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
+        default: return -1;
+    }
+}
+
+/* ---------------------------------------------------------------- fp16 <-> fp32, IEEE round-to-nearest-even.
+ * The x86 reference uses the F16C instructions (ggml-impl.h:346-353) and a 65536-entry table filled with
+ * them (ggml.c:1418-1431); both are plain IEEE conversions, restated here in integer arithmetic. */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+float orc_fp16_to_fp32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp  = (h >> 10) & 0x1f;
+    uint32_t man  = h & 0x3ffu;
+    if (exp == 0) {
+        if (man == 0) return u2f(sign);
+        /* subnormal half: value = man * 2^-24, exact in fp32 */
+        float v = (float)man * 0x1.0p-24f;
+        return u2f(f2u(v) | sign);
+    }
+    if (exp == 31) return u2f(sign | 0x7f800000u | (man << 13));
+    return u2f(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+uint16_t orc_fp32_to_fp16(float f) {
+    uint32_t u = f2u(f);
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x3ffu)); /* NaN (quieted) */
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);   /* >= 65520 rounds to inf */
+    if (a < 0x33000001u) return sign;                            /* <= 2^-25 rounds to zero (tie -> even 0) */
+    int32_t e = (int32_t)(a >> 23) - 127;
+    uint32_t m = (a & 0x7fffffu) | 0x800000u;                    /* 24-bit significand */
+    int shift;                                                   /* bits dropped from m */
+    uint32_t base;
+    if (e >= -14) { shift = 13; base = (uint32_t)(e + 15) << 10; m &= 0x7fffffu; }
+    else          { shift = 13 + (-14 - e); base = 0; }
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | (base + q));                        /* carry out of q bumps the exponent */
+}
+
+#define H2F(h) orc_fp16_to_fp32(h)
+#define F2H(f) orc_fp32_to_fp16(f)
+
+/* ggml-quants.c:366-371: round to nearest (ties to even) through the 1.5*2^23 magic constant. */
+static inline int nearest_i(float v) {
+    float t = v + 12582912.f;
+    return (int)(f2u(t) & 0x007fffffu) - 0x00400000;
+}
+static inline int imin_(int a, int b) { return a < b ? a : b; }
+static inline int imax_(int a, int b) { return a > b ? a : b; }
+
+/* ---------------------------------------------------------------- activation quantizers */
+
+/* ggml-cpu/ggml-cpu-quants.c:802-885 (AVX2 branch of quantize_row_q8_0):
+ *   d = amax/127 ; id = amax != 0 ? 127/amax : 0 ; q = round_half_even(x*id).
+ * This differs from the scalar _ref (id = 1/d, roundf) in the last ulp of id and on exact .5 ties. */
+void orc_quantize_row_q8_0(const float *x, void *vy, int64_t k) {
+    blk_q8_0 *y = (blk_q8_0 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) { float a = fabsf(x[j]); if (a > amax) amax = a; }
+        const float d = amax / 127.f;
+        const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+        y[b].d = F2H(d);
+        for (int j = 0; j < 32; j++) {
+            const float r = nearbyintf(x[j] * id);    /* default rounding mode: to nearest even */
+            /* cvtps_epi32 turns NaN and anything outside int32 into 0x80000000 ("integer indefinite"),
+             * which the two saturating packs carry down to -128; reachable when 127/amax overflows. */
+            const int q = fabsf(r) < 2147483648.f ? (int)r : INT32_MIN;
+            y[b].qs[j] = (int8_t)imax_(-128, imin_(127, q));
+        }
+    }
+}
+
+/* ggml-quants.c:188-211 (scalar reference, used for Q8_0 *weights*). */
+void orc_quantize_row_q8_0_ref(const float *x, void *vy, int64_t k) {
+    blk_q8_0 *y = (blk_q8_0 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) { float a = fabsf(x[j]); if (a > amax) amax = a; }
+        const float d = amax / 127;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = F2H(d);
+        for (int j = 0; j < 32; j++) y[b].qs[j] = (int8_t)roundf(x[j] * id);
+    }
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:1740,1819-1821 -> ggml-quants.c:2473-2510.  An all-zero block leaves bsums
+ * unwritten in the reference (they are multiplied by d == 0 downstream); here they are set to 0. */
+void orc_quantize_row_q8_K(const float *x, void *vy, int64_t k) {
+    blk_q8_K *y = (blk_q8_K *)vy;
+    for (int64_t b = 0; b < k / 256; b++, x += 256) {
+        float amax = 0.0f, mx = 0.0f;
+        for (int j = 0; j < 256; j++) {
+            float a = fabsf(x[j]);
+            if (a > amax) { amax = a; mx = x[j]; }    /* strict >: the first largest wins, sign kept */
+        }
+        if (amax == 0.0f) { memset(&y[b], 0, sizeof(blk_q8_K)); continue; }
+        const float iscale = -127.f / mx;
+        for (int j = 0; j < 256; j++) y[b].qs[j] = (int8_t)imin_(127, nearest_i(iscale * x[j]));
+        for (int g = 0; g < 16; g++) {
+            int s = 0;
+            for (int j = 0; j < 16; j++) s += y[b].qs[16 * g + j];
+            y[b].bsums[g] = (int16_t)s;
+        }
+        y[b].d = 1 / iscale;
+    }
+}
+
+/* ---------------------------------------------------------------- weight quantizers */
+
+/* ggml-quants.c:25-60. */
+void orc_quantize_row_q4_0_ref(const float *x, void *vy, int64_t k) {
+    blk_q4_0 *y = (blk_q4_0 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float amax = 0.0f, mx = 0.0f;
+        for (int j = 0; j < 32; j++) {
+            if (amax < fabsf(x[j])) { amax = fabsf(x[j]); mx = x[j]; }
+        }
+        const float d = mx / -8;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = F2H(d);
+        for (int j = 0; j < 16; j++) {
+            const float lo = x[j] * id, hi = x[j + 16] * id;
+            const uint8_t qlo = (uint8_t)imin_(15, (int8_t)(lo + 8.5f));
+            const uint8_t qhi = (uint8_t)imin_(15, (int8_t)(hi + 8.5f));
+            y[b].qs[j] = (uint8_t)(qlo | (qhi << 4));
+        }
+    }
+}
+
+/* ggml-quants.c:544-623 with the arguments quantize_row_q4_K_ref passes (n=32, nmax=15, rmin=-1,
+ * rdelta=0.1, nstep=20, use_mad=false).  Returns the scale, writes -min to *neg_min. */
+static float fit_scale_min_32(const float *x, const float *w, uint8_t *L, float *neg_min, uint8_t *Laux) {
+    const int n = 32, nmax = 15, nstep = 20;
+    const float rmin = -1.f, rdelta = 0.1f;
+    float lo = x[0], hi = x[0];
+    float sum_w = w[0];
+    float sum_x = sum_w * x[0];
+    for (int i = 1; i < n; i++) {
+        if (x[i] < lo) lo = x[i];
+        if (x[i] > hi) hi = x[i];
+        sum_w += w[i];
+        sum_x += w[i] * x[i];
+    }
+    if (lo > 0) lo = 0;
+    if (hi == lo) {
+        for (int i = 0; i < n; i++) L[i] = 0;
+        *neg_min = -lo;
+        return 0.f;
+    }
+    float iscale = nmax / (hi - lo);
+    float scale = 1 / iscale;
+    float best = 0;
+    for (int i = 0; i < n; i++) {
+        int l = nearest_i(iscale * (x[i] - lo));
+        L[i] = (uint8_t)imax_(0, imin_(nmax, l));
+        float diff = scale * L[i] + lo - x[i];
+        diff = diff * diff;
+        best += w[i] * diff;
+    }
+    for (int is = 0; is <= nstep; is++) {
+        iscale = (rmin + rdelta * is + nmax) / (hi - lo);
+        float sum_l = 0, sum_l2 = 0, sum_xl = 0;
+        for (int i = 0; i < n; i++) {
+            int l = nearest_i(iscale * (x[i] - lo));
+            l = imax_(0, imin_(nmax, l));
+            Laux[i] = (uint8_t)l;
+            sum_l  += w[i] * l;
+            sum_l2 += w[i] * l * l;
+            sum_xl += w[i] * l * x[i];
+        }
+        float D = sum_w * sum_l2 - sum_l * sum_l;
+        if (D > 0) {
+            float s = (sum_w * sum_xl - sum_x * sum_l) / D;
+            float m = (sum_l2 * sum_x - sum_l * sum_xl) / D;
+            if (m > 0) { m = 0; s = sum_xl / sum_l2; }
+            float mad = 0;
+            for (int i = 0; i < n; i++) {
+                float diff = s * Laux[i] + m - x[i];
+                diff = diff * diff;
+                mad += w[i] * diff;
+            }
+            if (mad < best) {
+                for (int i = 0; i < n; i++) L[i] = Laux[i];
+                best = mad; scale = s; lo = m;
+            }
+        }
+    }
+    *neg_min = -lo;
+    return scale;
+}
+
+/* ggml-quants.c:625-632: 6-bit scale and min of sub-block j from the 12 packed bytes. */
+static inline void unpack_sc_m(int j, const uint8_t *q, uint8_t *sc, uint8_t *m) {
+    if (j < 4) { *sc = q[j] & 63; *m = q[j + 4] & 63; }
+    else {
+        *sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m  = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* ggml-quants.c:1202-1272. */
+void orc_quantize_row_q4_K_ref(const float *x, void *vy, int64_t k) {
+    blk_q4_K *y = (blk_q4_K *)vy;
+    uint8_t L[256], Laux[32];
+    float w[32], mins[8], scales[8];
+    for (int64_t b = 0; b < k / 256; b++, x += 256) {
+        float max_scale = 0, max_min = 0;
+        for (int j = 0; j < 8; j++) {
+            const float *xs = x + 32 * j;
+            float sum_x2 = 0;
+            for (int l = 0; l < 32; l++) sum_x2 += xs[l] * xs[l];
+            float av = sqrtf(sum_x2 / 32);
+            for (int l = 0; l < 32; l++) w[l] = av + fabsf(xs[l]);
+            scales[j] = fit_scale_min_32(xs, w, L + 32 * j, &mins[j], Laux);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+        const float inv_min   = max_min   > 0 ? 63.f / max_min   : 0.f;
+        for (int j = 0; j < 8; j++) {
+            uint8_t ls = (uint8_t)nearest_i(inv_scale * scales[j]);
+            uint8_t lm = (uint8_t)nearest_i(inv_min * mins[j]);
+            if (ls > 63) ls = 63;
+            if (lm > 63) lm = 63;
+            if (j < 4) { y[b].scales[j] = ls; y[b].scales[j + 4] = lm; }
+            else {
+                y[b].scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                y[b].scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                y[b].scales[j]     |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        y[b].d    = F2H(max_scale / 63.f);
+        y[b].dmin = F2H(max_min / 63.f);
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            unpack_sc_m(j, y[b].scales, &sc, &m);
+            const float d = H2F(y[b].d) * sc;
+            if (!d) continue;
+            const float dm = H2F(y[b].dmin) * m;
+            for (int i = 0; i < 32; i++) {
+                int l = nearest_i((x[32 * j + i] + dm) / d);
+                L[32 * j + i] = (uint8_t)imax_(0, imin_(15, l));
+            }
+        }
+        uint8_t *q = y[b].qs;
+        for (int j = 0; j < 256; j += 64, q += 32)
+            for (int l = 0; l < 32; l++) q[l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
+    }
+}
+
+/* ggml-quants.c:373-440 with the arguments quantize_row_q6_K_ref passes (n=16, nmax=32, rmse_type=1,
+ * no external weights: w_i = x_i^2). */
+static float fit_scale_16(const float *x, int8_t *L) {
+    const int n = 16, nmax = 32;
+    float mx = 0, amax = 0;
+    for (int i = 0; i < n; i++) {
+        float a = fabsf(x[i]);
+        if (a > amax) { amax = a; mx = x[i]; }
+    }
+    if (amax < 1e-15f) {
+        for (int i = 0; i < n; i++) L[i] = 0;
+        return 0.f;
+    }
+    float iscale = -nmax / mx;
+    float sumlx = 0, suml2 = 0;
+    for (int i = 0; i < n; i++) {
+        int l = nearest_i(iscale * x[i]);
+        l = imax_(-nmax, imin_(nmax - 1, l));
+        L[i] = (int8_t)(l + nmax);
+        float w = x[i] * x[i];
+        sumlx += w * x[i] * l;
+        suml2 += w * l * l;
+    }
+    float scale = suml2 ? sumlx / suml2 : 0.0f;
+    float best = scale * sumlx;
+    for (int is = -9; is <= 9; is++) {
+        if (is == 0) continue;
+        iscale = -(nmax + 0.1f * is) / mx;
+        sumlx = suml2 = 0;
+        for (int i = 0; i < n; i++) {
+            int l = nearest_i(iscale * x[i]);
+            l = imax_(-nmax, imin_(nmax - 1, l));
+            float w = x[i] * x[i];
+            sumlx += w * x[i] * l;
+            suml2 += w * l * l;
+        }
+        if (suml2 > 0 && sumlx * sumlx > best * suml2) {
+            for (int i = 0; i < n; i++) {
+                int l = nearest_i(iscale * x[i]);
+                L[i] = (int8_t)(nmax + imax_(-nmax, imin_(nmax - 1, l)));
+            }
+            scale = sumlx / suml2;
+            best = scale * sumlx;
+        }
+    }
+    return scale;
+}
+
+/* ggml-quants.c:1614-1682. */
+void orc_quantize_row_q6_K_ref(const float *x, void *vy, int64_t k) {
+    blk_q6_K *y = (blk_q6_K *)vy;
+    int8_t L[256];
+    float scales[16];
+    for (int64_t b = 0; b < k / 256; b++, x += 256) {
+        float max_scale = 0, max_abs = 0;
+        for (int g = 0; g < 16; g++) {
+            const float s = fit_scale_16(x + 16 * g, L + 16 * g);
+            scales[g] = s;
+            const float a = fabsf(s);
+            if (a > max_abs) { max_abs = a; max_scale = s; }
+        }
+        if (max_abs < 1e-15f) { memset(&y[b], 0, sizeof(blk_q6_K)); continue; }
+        const float iscale = -128.f / max_scale;
+        y[b].d = F2H(1 / iscale);
+        for (int g = 0; g < 16; g++) y[b].scales[g] = (int8_t)imin_(127, nearest_i(iscale * scales[g]));
+        for (int g = 0; g < 16; g++) {
+            const float d = H2F(y[b].d) * y[b].scales[g];
+            if (!d) continue;
+            for (int i = 0; i < 16; i++) {
+                int l = nearest_i(x[16 * g + i] / d);
+                L[16 * g + i] = (int8_t)(imax_(-32, imin_(31, l)) + 32);
+            }
+        }
+        uint8_t *ql = y[b].ql, *qh = y[b].qh;
+        for (int j = 0; j < 256; j += 128, ql += 64, qh += 32) {
+            for (int l = 0; l < 32; l++) {
+                const uint8_t a = (uint8_t)L[j + l], c = (uint8_t)L[j + l + 32];
+                const uint8_t e = (uint8_t)L[j + l + 64], g = (uint8_t)L[j + l + 96];
+                ql[l]      = (uint8_t)((a & 0xF) | ((e & 0xF) << 4));
+                ql[l + 32] = (uint8_t)((c & 0xF) | ((g & 0xF) << 4));
+                qh[l] = (uint8_t)((a >> 4) | ((c >> 4) << 2) | ((e >> 4) << 4) | ((g >> 4) << 6));
+            }
+        }
+    }
+}
+
+size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64_t k) {
+    const size_t rs = orc_row_size(type, k);
+    for (int64_t r = 0; r < nrows; r++) {
+        void *dst = (char *)y + r * rs;
+        const float *src = x + r * k;
+        switch (type) {
+            case ORC_TYPE_Q4_0: orc_quantize_row_q4_0_ref(src, dst, k); break;
+            case ORC_TYPE_Q8_0: orc_quantize_row_q8_0_ref(src, dst, k); break;
+            case ORC_TYPE_Q4_K: orc_quantize_row_q4_K_ref(src, dst, k); break;
+            case ORC_TYPE_Q6_K: orc_quantize_row_q6_K_ref(src, dst, k); break;
+            default: return 0;
+        }
+    }
+    return rs * (size_t)nrows;
+}
+
+/* ---------------------------------------------------------------- dequantizers (closed forms)
+ * q4_0 ggml-quants.c:249-267 ; q8_0 :343-357 ; q4_K :1274-1296 ; q6_K :1684-1713 ; q8_K :2512-2521 */
+void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
+    if (type == ORC_TYPE_Q4_0) {
+        const blk_q4_0 *x = (const blk_q4_0 *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d);
+            for (int j = 0; j < 16; j++) {
+                y[j]      = ((x[b].qs[j] & 0xF) - 8) * d;
+                y[j + 16] = ((x[b].qs[j] >> 4) - 8) * d;
+            }
+        }
+    } else if (type == ORC_TYPE_Q8_0) {
+        const blk_q8_0 *x = (const blk_q8_0 *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d);
+            for (int j = 0; j < 32; j++) y[j] = x[b].qs[j] * d;
+        }
+    } else if (type == ORC_TYPE_Q4_K) {
+        const blk_q4_K *x = (const blk_q4_K *)vx;
+        for (int64_t b = 0; b < k / 256; b++) {
+            const float d = H2F(x[b].d), mn = H2F(x[b].dmin);
+            const uint8_t *q = x[b].qs;
+            for (int j = 0; j < 4; j++, q += 32) {
+                uint8_t sc, m;
+                unpack_sc_m(2 * j, x[b].scales, &sc, &m);
+                const float d1 = d * sc, m1 = mn * m;
+                unpack_sc_m(2 * j + 1, x[b].scales, &sc, &m);
+                const float d2 = d * sc, m2 = mn * m;
+                for (int l = 0; l < 32; l++) *y++ = d1 * (q[l] & 0xF) - m1;
+                for (int l = 0; l < 32; l++) *y++ = d2 * (q[l] >> 4) - m2;
+            }
+        }
+    } else if (type == ORC_TYPE_Q6_K) {
+        const blk_q6_K *x = (const blk_q6_K *)vx;
+        for (int64_t b = 0; b < k / 256; b++) {
+            const float d = H2F(x[b].d);
+            const uint8_t *ql = x[b].ql, *qh = x[b].qh;
+            const int8_t *sc = x[b].scales;
+            for (int h = 0; h < 2; h++, y += 128, ql += 64, qh += 32, sc += 8) {
+                for (int l = 0; l < 32; l++) {
+                    const int is = l / 16;
+                    const int8_t q1 = (int8_t)((ql[l]      & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                    const int8_t q2 = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                    const int8_t q3 = (int8_t)((ql[l]      >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                    const int8_t q4 = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                    y[l]      = d * sc[is + 0] * q1;
+                    y[l + 32] = d * sc[is + 2] * q2;
+                    y[l + 64] = d * sc[is + 4] * q3;
+                    y[l + 96] = d * sc[is + 6] * q4;
+                }
+            }
+        }
+    } else if (type == ORC_TYPE_Q8_K) {
+        const blk_q8_K *x = (const blk_q8_K *)vx;
+        for (int64_t b = 0; b < k / 256; b++)
+            for (int j = 0; j < 256; j++) *y++ = x[b].d * x[b].qs[j];
+    }
+}
+
+/* ---------------------------------------------------------------- dot products (AVX2 lane structure) */
+
+/* ggml-cpu/ggml-cpu-quants.c:43-49: horizontal sum of 8 lanes, in the order the shuffles impose. */
+static inline float hsum8(const float a[8]) {
+    const float r0 = a[4] + a[0], r1 = a[5] + a[1], r2 = a[6] + a[2], r3 = a[7] + a[3];
+    const float s0 = r0 + r2, s1 = r1 + r3;
+    return s0 + s1;
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:2267-2290.  Lane j of the 8-wide accumulator takes the four products of bytes
+ * 4j..4j+3 of the 32-byte vectors (low nibbles are bytes 0..15, high nibbles 16..31; :79-85,116-128). */
+float orc_vec_dot_q4_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q4_0 *x = (const blk_q4_0 *)vx;
+    const blk_q8_0 *y = (const blk_q8_0 *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 32; b++) {
+        const float d = H2F(x[b].d) * H2F(y[b].d);
+        int8_t w[32];
+        for (int j = 0; j < 16; j++) {
+            w[j]      = (int8_t)((x[b].qs[j] & 0xF) - 8);
+            w[j + 16] = (int8_t)((x[b].qs[j] >> 4) - 8);
+        }
+        int32_t tot = 0;
+        for (int j = 0; j < 8; j++) {
+            int32_t p = 0;
+            for (int t = 0; t < 4; t++) p += (int32_t)w[4 * j + t] * y[b].qs[4 * j + t];
+            tot += p;
+            acc[j] = fmaf(d, (float)p, acc[j]);
+        }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc);
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:3863-3880. */
+float orc_vec_dot_q8_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q8_0 *x = (const blk_q8_0 *)vx;
+    const blk_q8_0 *y = (const blk_q8_0 *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 32; b++) {
+        const float d = H2F(x[b].d) * H2F(y[b].d);
+        int32_t tot = 0;
+        for (int j = 0; j < 8; j++) {
+            int32_t p = 0;
+            for (int t = 0; t < 4; t++) p += (int32_t)x[b].qs[4 * j + t] * y[b].qs[4 * j + t];
+            tot += p;
+            acc[j] = fmaf(d, (float)p, acc[j]);
+        }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc);
+}
+
+/* The shuffle the SIMD paths use to unpack the 12 scale bytes (ggml-cpu/ggml-cpu-quants.c:7048-7053):
+ * out[0..7] = 6-bit scales, out[8..15] = 6-bit mins.  Equivalent to unpack_sc_m for j = 0..7. */
+static void unpack_scales_kmask(const uint8_t *s12, uint8_t out[16]) {
+    uint32_t u[4];
+    memcpy(u, s12, 12);
+    u[3] = ((u[2] >> 4) & 0x0f0f0f0fu) | (((u[1] >> 6) & 0x03030303u) << 4);
+    const uint32_t t = u[1] & 0x3f3f3f3fu;
+    u[1] = (u[2] & 0x0f0f0f0fu) | (((u[0] >> 6) & 0x03030303u) << 4);
+    u[2] = t;
+    u[0] &= 0x3f3f3f3fu;
+    memcpy(out, u, 16);
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:7036-7099. */
+float orc_vec_dot_q4_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin) {
+    const blk_q4_K *x = (const blk_q4_K *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    float acc[8] = {0};
+    float accm[4] = {0};
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float d = y[b].d * H2F(x[b].d);
+        const float dmin = -y[b].d * H2F(x[b].dmin);
+        uint8_t sm[16];
+        unpack_scales_kmask(x[b].scales, sm);
+        const uint8_t *sc = sm, *mn = sm + 8;
+
+        /* mins: pairwise bsums as int16 (hadd), then madd by pairs of mins -> 4 int32 lanes */
+        int32_t mtot = 0;
+        for (int i = 0; i < 4; i++) {
+            const int16_t s0 = (int16_t)(y[b].bsums[4 * i + 0] + y[b].bsums[4 * i + 1]);
+            const int16_t s1 = (int16_t)(y[b].bsums[4 * i + 2] + y[b].bsums[4 * i + 3]);
+            const int32_t p = (int32_t)mn[2 * i] * s0 + (int32_t)mn[2 * i + 1] * s1;
+            mtot += p;
+            accm[i] = fmaf(dmin, (float)p, accm[i]);
+        }
+
+        int32_t lane[8] = {0};
+        const uint8_t *q4 = x[b].qs;
+        const int8_t *q8 = y[b].qs;
+        for (int j = 0; j < 4; j++, q4 += 32, q8 += 64) {
+            for (int m = 0; m < 8; m++) {
+                int32_t pl = 0, ph = 0;
+                for (int t = 0; t < 4; t++) {
+                    pl += (int32_t)(q4[4 * m + t] & 0xF) * q8[4 * m + t];
+                    ph += (int32_t)(q4[4 * m + t] >> 4) * q8[32 + 4 * m + t];
+                }
+                lane[m] += (int32_t)sc[2 * j] * pl + (int32_t)sc[2 * j + 1] * ph;
+            }
+        }
+        int32_t tot = 0;
+        for (int m = 0; m < 8; m++) { tot += lane[m]; acc[m] = fmaf(d, (float)lane[m], acc[m]); }
+        if (isum) isum[b] = tot;
+        if (imin) imin[b] = mtot;
+    }
+    const float m0 = accm[0] + accm[2], m1 = accm[1] + accm[3];
+    return hsum8(acc) + (m0 + m1);
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:8972-9049. */
+float orc_vec_dot_q6_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q6_K *x = (const blk_q6_K *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float d = y[b].d * H2F(x[b].d);
+        int32_t lane[8] = {0};
+        const uint8_t *ql = x[b].ql, *qh = x[b].qh;
+        const int8_t *q8 = y[b].qs, *sc = x[b].scales;
+        for (int h = 0; h < 2; h++, ql += 64, qh += 32, q8 += 128, sc += 8) {
+            for (int v = 0; v < 4; v++) {                 /* the four 32-value vectors of this half */
+                for (int m = 0; m < 8; m++) {
+                    int32_t p = 0;
+                    for (int t = 0; t < 4; t++) {
+                        const int i = 4 * m + t;
+                        int q;
+                        switch (v) {
+                            case 0:  q = (ql[i]      & 0xF) | (((qh[i] >> 0) & 3) << 4); break;
+                            case 1:  q = (ql[i + 32] & 0xF) | (((qh[i] >> 2) & 3) << 4); break;
+                            case 2:  q = (ql[i]      >> 4) | (((qh[i] >> 4) & 3) << 4); break;
+                            default: q = (ql[i + 32] >> 4) | (((qh[i] >> 6) & 3) << 4); break;
+                        }
+                        p += (q - 32) * (int32_t)q8[32 * v + i];
+                    }
+                    lane[m] += (int32_t)sc[2 * v + (m >= 4)] * p;
+                }
+            }
+        }
+        int32_t tot = 0;
+        for (int m = 0; m < 8; m++) { tot += lane[m]; acc[m] = fmaf(d, (float)lane[m], acc[m]); }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc);
+}
+
+float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
+    switch (type) {
+        case ORC_TYPE_Q4_0: return orc_vec_dot_q4_0_q8_0(k, vx, vy, NULL);
+        case ORC_TYPE_Q8_0: return orc_vec_dot_q8_0_q8_0(k, vx, vy, NULL);
+        case ORC_TYPE_Q4_K: return orc_vec_dot_q4_K_q8_K(k, vx, vy, NULL, NULL);
+        case ORC_TYPE_Q6_K: return orc_vec_dot_q6_K_q8_K(k, vx, vy, NULL);
+        default: return NAN;
+    }
+}
+
+double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, double *sum_abs) {
+    double s = 0, sa = 0;
+    const int be = orc_block_elems(type);
+    if (!be) return NAN;
+    const int64_t nb = k / be;
+    int32_t *is = (int32_t *)malloc(sizeof(int32_t) * (size_t)(nb > 0 ? nb : 1) * 2);
+    int32_t *im = is + (nb > 0 ? nb : 1);
+    if (type == ORC_TYPE_Q4_0 || type == ORC_TYPE_Q8_0) {
+        if (type == ORC_TYPE_Q4_0) orc_vec_dot_q4_0_q8_0(k, vx, vy, is);
+        else                       orc_vec_dot_q8_0_q8_0(k, vx, vy, is);
+        const blk_q8_0 *y = (const blk_q8_0 *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const uint16_t hx = type == ORC_TYPE_Q4_0 ? ((const blk_q4_0 *)vx)[b].d : ((const blk_q8_0 *)vx)[b].d;
+            const double t = (double)H2F(hx) * (double)H2F(y[b].d) * (double)is[b];
+            s += t; sa += fabs(t);
+        }
+    } else if (type == ORC_TYPE_Q4_K) {
+        orc_vec_dot_q4_K_q8_K(k, vx, vy, is, im);
+        const blk_q4_K *x = (const blk_q4_K *)vx;
+        const blk_q8_K *y = (const blk_q8_K *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const double t1 = (double)y[b].d * (double)H2F(x[b].d) * (double)is[b];
+            const double t2 = (double)y[b].d * (double)H2F(x[b].dmin) * (double)im[b];
+            s += t1 - t2; sa += fabs(t1) + fabs(t2);
+        }
+    } else if (type == ORC_TYPE_Q6_K) {
+        orc_vec_dot_q6_K_q8_K(k, vx, vy, is);
+        const blk_q6_K *x = (const blk_q6_K *)vx;
+        const blk_q8_K *y = (const blk_q8_K *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const double t = (double)y[b].d * (double)H2F(x[b].d) * (double)is[b];
+            s += t; sa += fabs(t);
+        }
+    } else { s = NAN; }
+    free(is);
+    if (sum_abs) *sum_abs = sa;
+    return s;
+}
+
+/* ---------------------------------------------------------------- MUL_MAT (ggml-cpu/ggml-cpu.c:1257-1449) */
+typedef struct {
+    int type; int64_t K, N, n; const char *W; const char *wd; float *y; double *sa;
+    int64_t r0, r1;
+} mm_job;
+
+static void *mm_worker(void *p) {
+    mm_job *j = (mm_job *)p;
+    const size_t wrs = orc_row_size(j->type, j->K);
+    const size_t ars = orc_row_size(orc_vec_dot_type(j->type), j->K);
+    for (int64_t t = 0; t < j->n; t++) {
+        for (int64_t r = j->r0; r < j->r1; r++) {
+            const void *wr = j->W + (size_t)r * wrs;
+            const void *ar = j->wd + (size_t)t * ars;
+            j->y[t * j->N + r] = orc_vec_dot(j->type, j->K, wr, ar);
+            if (j->sa) orc_vec_dot_exact(j->type, j->K, wr, ar, &j->sa[t * j->N + r]);
+        }
+    }
+    return NULL;
+}
+
+void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const float *x, float *y,
+                 void *wdata, double *sum_abs, int nthreads) {
+    const int vdt = orc_vec_dot_type(type);
+    if (vdt < 0) return;
+    const size_t ars = orc_row_size(vdt, K);
+    char *wd = wdata ? (char *)wdata : (char *)malloc(ars * (size_t)(n > 0 ? n : 1));
+    for (int64_t t = 0; t < n; t++) {
+        if (vdt == ORC_TYPE_Q8_0) orc_quantize_row_q8_0(x + t * K, wd + (size_t)t * ars, K);
+        else                      orc_quantize_row_q8_K(x + t * K, wd + (size_t)t * ars, K);
+    }
+    if (nthreads < 1) nthreads = 1;
+    if (nthreads > 256) nthreads = 256;
+    if ((int64_t)nthreads > N) nthreads = (int)(N > 0 ? N : 1);
+    pthread_t th[256];
+    mm_job jobs[256];
+    for (int i = 0; i < nthreads; i++) {
+        jobs[i] = (mm_job){type, K, N, n, (const char *)W, wd, y, sum_abs, N * i / nthreads, N * (i + 1) / nthreads};
+        if (i > 0) pthread_create(&th[i], NULL, mm_worker, &jobs[i]);
+    }
+    mm_worker(&jobs[0]);
+    for (int i = 1; i < nthreads; i++) pthread_join(th[i], NULL);
+    if (!wdata) free(wd);
+}

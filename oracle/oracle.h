@@ -1,0 +1,106 @@
+/*
+ * oracle.h -- CPU restatement of the reference's quantized MUL_MAT path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load
+ * this library, and there only as the checker.  The product (libcactus_hip.so, libggml-hip.so) never links,
+ * loads or falls back to anything in this directory.
+ *
+ * Every function restates, in plain scalar C, what the reference computes on an x86-64 AVX2 build, citing the
+ * reference file:line it follows (paths relative to the reference's cactus/ directory).  Pinning status:
+ *
+ *   function                         pinned by
+ *   -------------------------------  -------------------------------------------------------------------------
+ *   orc_fp16_to_fp32/fp32_to_fp16    exhaustive over all 65536 halves / edge+random floats vs numpy (IEEE RNE)
+ *   orc_quantize_row_q8_0            bit-exact vs oracle/_ref on seeded data + committed golden vectors;
+ *                                    invariants (max element -> +-127, zero block, ties-to-even cases)
+ *   orc_quantize_row_q8_0_ref        bit-exact vs oracle/_ref + golden; half-away-from-zero tie cases
+ *   orc_quantize_row_q8_K            bit-exact vs oracle/_ref + golden; bsums == sum of 16, first-max sign rule
+ *   orc_quantize_row_q4_0_ref        bit-exact vs oracle/_ref + golden; dequant closed form d*(nib-8)
+ *   orc_quantize_row_q4_K_ref        bit-exact vs oracle/_ref + golden (iterative search: only the oracle run
+ *   orc_quantize_row_q6_K_ref          pins the bytes); reconstruction-error bound as a sanity invariant
+ *   orc_dequantize_row_*             closed forms; vs oracle/_ref + golden
+ *   orc_vec_dot_*                    integer sums: brute force from dequantised integers; float result: bit-exact
+ *                                    vs oracle/_ref (the AVX2 lane structure is restated) + golden; fp64 identity
+ *                                    sum(dequant(x)*dequant(y))
+ *   orc_mul_mat                      == n*N independent vec_dots; vs oracle/_ref's LM_GGML_OP_MUL_MAT graph
+ *
+ * No function here is "parity unpinned".
+ */
+#ifndef CACTUS_ORACLE_H
+#define CACTUS_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* type ids are the reference's lm_ggml_type values (ggml.h:351-391) */
+enum orc_type {
+    ORC_TYPE_F32  = 0,
+    ORC_TYPE_Q4_0 = 2,
+    ORC_TYPE_Q8_0 = 8,
+    ORC_TYPE_Q4_K = 12,
+    ORC_TYPE_Q6_K = 14,
+    ORC_TYPE_Q8_K = 15,
+};
+
+/* elements per block / bytes per block / bytes per row of k elements; 0 for an unknown type */
+int    orc_block_elems(int type);
+size_t orc_block_bytes(int type);
+size_t orc_row_size(int type, int64_t k);
+/* activation type a weight type is dotted with (type_traits_cpu[].vec_dot_type, ggml-cpu/ggml-cpu.c:198-367) */
+int    orc_vec_dot_type(int type);
+
+float    orc_fp16_to_fp32(uint16_t h);
+uint16_t orc_fp32_to_fp16(float f);
+
+/* activation quantizers (the two the MUL_MAT op calls on the fly) */
+void orc_quantize_row_q8_0(const float *x, void *y, int64_t k);      /* AVX2 semantics */
+void orc_quantize_row_q8_K(const float *x, void *y, int64_t k);
+
+/* weight quantizers (offline; their output bytes are the op's input) */
+void orc_quantize_row_q4_0_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q8_0_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q4_K_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q6_K_ref(const float *x, void *y, int64_t k);
+/* dispatch on weight type, nrows rows of k elements, rows packed back to back; returns bytes written */
+size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64_t k);
+
+void orc_dequantize_row(int type, const void *x, float *y, int64_t k);
+
+/*
+ * Dot products.  Each returns the fp32 value the reference's AVX2 branch produces (same lane structure, same
+ * fused multiply-adds, same horizontal-sum order) and optionally the exact integer sums:
+ *   q4_0/q8_0 : isum[k/32]   = sum over the block of wq*aq                (wq already offset by -8 for q4_0)
+ *   q4_K      : isum[k/256]  = sum_j sc_j * sum_{i<32} q4*q8 ; imin[k/256] = sum_j m_j*(bsums[2j]+bsums[2j+1])
+ *   q6_K      : isum[k/256]  = sum_j sc_j * sum_{i<16} (q6-32)*q8
+ * Pass NULL to skip an output.
+ */
+float orc_vec_dot_q4_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot_q8_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot_q4_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin);
+float orc_vec_dot_q6_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
+
+/* fp64 evaluation of sum_b scale_b*isum_b (returned) and of sum_b |scale_b*isum_b| (*sum_abs; for Q4_K the
+ * |dmin term| is included): the tolerance yardstick 1e-5 * sum_abs and an order-free reference value. */
+double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, double *sum_abs);
+
+/*
+ * MUL_MAT as the CPU backend computes it (ggml-cpu/ggml-cpu.c:1257-1449): quantize each of the n activation
+ * rows x[t][0..K) to the weight type's vec_dot_type, then y[t][r] = vec_dot(W row r, quantized row t).
+ *   W     : N rows of orc_row_size(type, K) bytes, packed
+ *   x     : n rows of K floats;   y : n rows of N floats
+ *   wdata : optional out, n rows of orc_row_size(vec_dot_type, K) bytes (the quantized activations)
+ *   sum_abs : optional out, n*N doubles (tolerance yardstick per output)
+ *   nthreads: rows are split over this many pthreads (>=1)
+ */
+void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const float *x, float *y,
+                 void *wdata, double *sum_abs, int nthreads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

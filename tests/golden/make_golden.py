@@ -1,0 +1,50 @@
+"""Writes tests/golden/*.npz from the reference's own compiled code (oracle/_ref/libggml_ref.so).
+
+Run in the build container, where the reference tree is mounted:  python tests/golden/make_golden.py
+The fixtures hold data only: seeded inputs and the bytes / floats the reference produced for them.
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+sys.path.insert(0, os.path.dirname(HERE))
+
+import oracle as O            # noqa: E402
+import common                 # noqa: E402
+
+
+def main():
+    O.build()
+    r = O.Reference()
+    K, N, n = 512, 3, 2
+    for wt in O.WEIGHT_TYPES:
+        name = O.TYPE_NAMES[wt]
+        w = common.weights_f32(100 + wt, N, K, outliers=(wt in (O.Q4_K, O.Q6_K)))
+        x = common.activations_f32(100 + wt, n, K)
+        wq = r.quantize_weights(wt, w)
+        at = O.VEC_DOT_TYPE[wt]
+        xq = r.quantize_activation(at, x)
+        y_dot = np.zeros((n, N), np.float32)
+        for t in range(n):
+            for i in range(N):
+                y_dot[t, i] = r.vec_dot(wt, K, wq[i], xq[t])
+        y_graph, _ = r.mul_mat_graph(wt, wq, x, nthreads=2)
+        np.savez_compressed(os.path.join(HERE, "mul_mat_%s.npz" % name),
+                            wtype=np.int32(wt), K=np.int32(K), w=w, x=x, wq=wq, xq=xq,
+                            w_deq=r.dequantize(wt, wq, K), y_dot=y_dot, y_graph=y_graph)
+    e0 = common.q8_0_edge_rows()
+    with np.errstate(all="ignore"):
+        np.savez_compressed(os.path.join(HERE, "quantize_q8_0_edges.npz"), x=e0,
+                            q_avx2=r.quantize_activation(O.Q8_0, e0),
+                            q_ref=np.stack([r.quantize_q8_0_ref(row) for row in e0]))
+        ek = common.q8_K_edge_rows()
+        np.savez_compressed(os.path.join(HERE, "quantize_q8_K_edges.npz"), x=ek,
+                            q=r.quantize_activation(O.Q8_K, ek))
+    print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
+
+
+if __name__ == "__main__":
+    main()
