@@ -1,0 +1,207 @@
+"""cactus_amd -- MI355X (gfx950) backend for Cactus's quantized MUL_MAT path.
+
+The product is two shared libraries built from cactus_amd/csrc:
+
+  lib/libcactus_hip.so   hand-written HIP kernels behind the C-ABI of include/cactus_hip.h
+  lib/libggml-hip.so     the ggml backend (reg / device / buffer type / graph_compute) on top of it
+
+This Python package is a thin ctypes binding of the C-ABI for tests and benchmarks.  There is no CPU or
+PyTorch fallback: if the library is missing or no gfx950 device is present, loading raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(HERE, "lib")
+KERNEL_LIB = os.path.join(LIB_DIR, "libcactus_hip.so")
+BACKEND_LIB = os.path.join(LIB_DIR, "libggml-hip.so")
+
+F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
+TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K"}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K)
+
+# every symbol include/cactus_hip.h declares
+EXPORTS = (
+    "chip_init", "chip_device_count", "chip_get_device_info", "chip_error_string", "chip_malloc", "chip_free",
+    "chip_memcpy_h2d", "chip_memcpy_d2h", "chip_memcpy_d2d", "chip_memset", "chip_stream_create",
+    "chip_stream_destroy", "chip_stream_synchronize", "chip_block_elems", "chip_block_bytes", "chip_row_size",
+    "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
+    "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_block_isums",
+    "chip_workspace_to_blocks",
+)
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("device", C.c_int), ("compute_units", C.c_int), ("wavefront_size", C.c_int),
+                ("max_lds_per_block", C.c_int), ("clock_khz", C.c_int), ("xcd_count", C.c_int),
+                ("hbm_total", C.c_size_t), ("hbm_free", C.c_size_t), ("name", C.c_char * 128), ("arch", C.c_char * 64)]
+
+
+class ChipError(RuntimeError):
+    pass
+
+
+def build():
+    """Compile the libraries in-tree with hipcc for gfx950 (cross-compiles without a GPU)."""
+    import subprocess
+    subprocess.check_call(["make", "-C", os.path.join(HERE, "csrc"), "-j8", "all"])
+
+
+def load_library(path=KERNEL_LIB):
+    """dlopen libcactus_hip.so and declare the prototypes.  Raises if the library has not been built."""
+    if not os.path.exists(path):
+        raise ChipError("%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                        "(there is no fallback implementation)" % path)
+    L = C.CDLL(path)
+    vp, i64, sz, i32 = C.c_void_p, C.c_int64, C.c_size_t, C.c_int
+    L.chip_init.argtypes = [i32]
+    L.chip_get_device_info.argtypes = [C.POINTER(DeviceInfo)]
+    L.chip_error_string.restype = C.c_char_p
+    L.chip_error_string.argtypes = [i32]
+    L.chip_malloc.argtypes = [C.POINTER(vp), sz]
+    L.chip_free.argtypes = [vp]
+    for n in ("chip_memcpy_h2d", "chip_memcpy_d2h", "chip_memcpy_d2d"):
+        getattr(L, n).argtypes = [vp, vp, sz, vp]
+    L.chip_memset.argtypes = [vp, i32, sz, vp]
+    L.chip_stream_create.argtypes = [C.POINTER(vp)]
+    L.chip_stream_destroy.argtypes = [vp]
+    L.chip_stream_synchronize.argtypes = [vp]
+    L.chip_block_elems.argtypes = [i32]
+    L.chip_block_bytes.restype = sz
+    L.chip_block_bytes.argtypes = [i32]
+    L.chip_row_size.restype = sz
+    L.chip_row_size.argtypes = [i32, i64]
+    L.chip_vec_dot_type.argtypes = [i32]
+    L.chip_mul_mat_supported.argtypes = [i32, i64]
+    L.chip_quantize_q8_0.argtypes = [vp, i64, i64, i64, vp, vp]
+    L.chip_quantize_q8_K.argtypes = [vp, i64, i64, i64, vp, vp]
+    L.chip_mul_mat_workspace_size.restype = sz
+    L.chip_mul_mat_workspace_size.argtypes = [i32, i64, i64]
+    L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
+    L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
+    L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
+    L.chip_block_isums.argtypes = [i32, vp, sz, i64, i64, vp, i64, vp, vp, vp]
+    L.chip_workspace_to_blocks.argtypes = [i32, i64, i64, vp, vp, vp]
+    return L
+
+
+class DeviceBuffer:
+    """A hipMalloc'd region owned through the C-ABI."""
+
+    def __init__(self, dev, nbytes):
+        self.dev, self.nbytes = dev, int(nbytes)
+        p = C.c_void_p()
+        dev.check(dev.lib.chip_malloc(C.byref(p), max(self.nbytes, 16)))
+        self.ptr = p.value
+
+    def upload(self, arr, offset=0):
+        arr = np.ascontiguousarray(arr)
+        assert offset + arr.nbytes <= max(self.nbytes, 16)
+        self.dev.check(self.dev.lib.chip_memcpy_h2d(self.ptr + offset, arr.ctypes.data, arr.nbytes, None))
+        return self
+
+    def download(self, dtype, count, offset=0):
+        out = np.empty(count, dtype)
+        assert offset + out.nbytes <= max(self.nbytes, 16)
+        self.dev.check(self.dev.lib.chip_memcpy_d2h(out.ctypes.data, self.ptr + offset, out.nbytes, None))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.dev.lib.chip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Device:
+    """One gfx950 GPU seen through the C-ABI; numpy in, numpy out (host<->device copies are synchronous)."""
+
+    def __init__(self, ordinal=0):
+        self.lib = load_library()
+        rc = self.lib.chip_init(ordinal)
+        if rc != 0:
+            raise ChipError("chip_init(%d) failed: %s" % (ordinal, self.error_string(rc)))
+        self.info = DeviceInfo()
+        self.check(self.lib.chip_get_device_info(C.byref(self.info)))
+
+    def error_string(self, rc):
+        return self.lib.chip_error_string(rc).decode()
+
+    def check(self, rc):
+        if rc != 0:
+            raise ChipError("libcactus_hip: %s (code %d)" % (self.error_string(rc), rc))
+
+    def alloc(self, nbytes):
+        return DeviceBuffer(self, nbytes)
+
+    def to_device(self, arr):
+        arr = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, arr.nbytes).upload(arr)
+
+    def sync(self, stream=None):
+        self.check(self.lib.chip_stream_synchronize(stream))
+
+    def row_size(self, t, k):
+        return self.lib.chip_row_size(t, k)
+
+    # -- the hot path -------------------------------------------------------------------------------------
+    def quantize(self, act_type, x):
+        """x fp32 [n, K] -> uint8 [n, row_size] in the reference block layout."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, k = x.shape
+        dx = self.to_device(x)
+        rs = self.row_size(act_type, k)
+        dy = self.alloc(n * rs)
+        fn = {Q8_0: self.lib.chip_quantize_q8_0, Q8_K: self.lib.chip_quantize_q8_K}[act_type]
+        self.check(fn(dx.ptr, k, n, k, dy.ptr, None))
+        self.sync()
+        return dy.download(np.uint8, n * rs).reshape(n, rs)
+
+    def mul_mat(self, wtype, W, x, dW=None, want_workspace_blocks=False):
+        """LM_GGML_OP_MUL_MAT: W uint8 [N, row_size(wtype, K)] (or a DeviceBuffer via dW), x fp32 [n, K] -> y [n, N]."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, k = x.shape
+        if dW is None:
+            W = np.ascontiguousarray(W, np.uint8)
+            N = W.shape[0]
+            dW = self.to_device(W)
+        else:
+            N = dW.nbytes // self.row_size(wtype, k)
+        nb01 = self.row_size(wtype, k)
+        dx = self.to_device(x)
+        dy = self.alloc(n * N * 4)
+        wsz = self.lib.chip_mul_mat_workspace_size(wtype, k, n)
+        ws = self.alloc(wsz)
+        self.check(self.lib.chip_mul_mat(wtype, dW.ptr, nb01, k, N, dx.ptr, k, n, dy.ptr, N, ws.ptr, wsz, None))
+        self.sync()
+        y = dy.download(np.float32, n * N).reshape(n, N)
+        if want_workspace_blocks:
+            at = self.lib.chip_vec_dot_type(wtype)
+            rs = self.row_size(at, k)
+            db = self.alloc(n * rs)
+            self.check(self.lib.chip_workspace_to_blocks(wtype, k, n, ws.ptr, db.ptr, None))
+            self.sync()
+            return y, db.download(np.uint8, n * rs).reshape(n, rs)
+        return y
+
+    def block_isums(self, wtype, W, aq, k):
+        """Per-block integer sums [n, N, K/block] (and imin for Q4_K) from reference-layout activation blocks."""
+        W = np.ascontiguousarray(W, np.uint8)
+        aq = np.ascontiguousarray(aq, np.uint8)
+        N, n = W.shape[0], aq.shape[0]
+        nblk = k // self.lib.chip_block_elems(wtype)
+        dW, da = self.to_device(W), self.to_device(aq)
+        di = self.alloc(n * N * nblk * 4)
+        dm = self.alloc(n * N * nblk * 4)
+        self.check(self.lib.chip_block_isums(wtype, dW.ptr, W.shape[1], k, N, da.ptr, n, di.ptr, dm.ptr, None))
+        self.sync()
+        isum = di.download(np.int32, n * N * nblk).reshape(n, N, nblk)
+        imin = dm.download(np.int32, n * N * nblk).reshape(n, N, nblk) if wtype == Q4_K else None
+        return isum, imin

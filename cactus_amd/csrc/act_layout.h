@@ -1,0 +1,35 @@
+// Kernel-private layout of quantized activations in the MUL_MAT workspace ("split" layout).
+//
+// The reference keeps quantized activations as arrays of block_q8_0 / block_q8_K (34 / 292-byte records that
+// interleave scale and quants).  On the GPU the same numbers are kept per token as three aligned planes so
+// that every consumer reads 16-byte aligned vectors:
+//
+//   Q8_0 activations (for Q4_0 and Q8_0 weights), token stride = q8_0_stride(K):
+//       qs  int8  [K]        at +0                 quants, block b at 32*b
+//       d   float [K/32]     at +K                 the block scale after rounding to fp16 (exactly as stored
+//                                                  in block_q8_0.d), widened back to fp32
+//       sum int32 [K/32]     at +K + 4*(K/32)      sum of the 32 quants of the block (Q4_0's -8 offset)
+//
+//   Q8_K activations (for Q4_K and Q6_K weights), token stride = q8_K_stride(K):
+//       qs    int8  [K]      at +0
+//       d     float [K/256]  at +K
+//       bsums int16 [K/16]   at +K + 4*(K/256)     block_q8_K.bsums
+//
+// K is a multiple of 256, so every plane starts 16-byte aligned.
+#pragma once
+#include <stdint.h>
+#include <stddef.h>
+
+namespace chip {
+
+__host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
+
+__host__ __device__ constexpr size_t q8_0_off_d(int64_t K)   { return (size_t)K; }
+__host__ __device__ constexpr size_t q8_0_off_sum(int64_t K) { return (size_t)K + 4 * (size_t)(K / 32); }
+__host__ __device__ constexpr size_t q8_0_stride(int64_t K)  { return align16((size_t)K + 8 * (size_t)(K / 32)); }
+
+__host__ __device__ constexpr size_t q8_K_off_d(int64_t K)     { return (size_t)K; }
+__host__ __device__ constexpr size_t q8_K_off_bsums(int64_t K) { return (size_t)K + 4 * (size_t)(K / 256); }
+__host__ __device__ constexpr size_t q8_K_stride(int64_t K)    { return align16((size_t)K + 4 * (size_t)(K / 256) + 2 * (size_t)(K / 16)); }
+
+}  // namespace chip

@@ -1,0 +1,289 @@
+// C-ABI of libcactus_hip.so (declared in include/cactus_hip.h): argument checking, device plumbing and the
+// dispatch from LM_GGML_OP_MUL_MAT shapes to the gfx950 kernels.  No CPU fallback exists anywhere in this
+// library: an unsupported request returns an error code, it is never computed on the host.
+#include "../../include/cactus_hip.h"
+#include "act_layout.h"
+#include "dev_common.h"
+#include "kernels.h"
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+using namespace chip;
+
+namespace {
+
+std::mutex g_mu;
+bool g_limits_ready[64] = {};
+DeviceLimits g_limits[64];
+
+int hip_rc(hipError_t e) { return e == hipSuccess ? CHIP_OK : (int)e; }
+
+// Limits of the current device, read once per device.
+int current_limits(DeviceLimits &out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return CHIP_EINVAL;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_limits_ready[dev]) {
+        hipDeviceProp_t p;
+        e = hipGetDeviceProperties(&p, dev);
+        if (e != hipSuccess) return (int)e;
+        int optin = 0;
+        if (hipDeviceGetAttribute(&optin, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) optin = 0;
+        size_t lds = p.sharedMemPerBlock;
+        if ((size_t)optin > lds) lds = (size_t)optin;
+        if (p.maxSharedMemoryPerMultiProcessor > lds) lds = p.maxSharedMemoryPerMultiProcessor;
+        if (lds > 160 * 1024) lds = 160 * 1024;
+        g_limits[dev].compute_units = p.multiProcessorCount;
+        g_limits[dev].max_lds_per_block = (int)lds;
+        g_limits_ready[dev] = true;
+    }
+    out = g_limits[dev];
+    return CHIP_OK;
+}
+
+bool is_weight_type(int t) { return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K; }
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// Q4_0 / Q8_0 / Q4_K rows of K % 256 == 0 elements are multiples of 16 bytes and the kernels load them with
+// 4- and 16-byte aligned vectors.  Q6_K rows are multiples of 210 bytes: only 2-byte alignment can be asked for,
+// and that kernel loads with 2-byte aligned vectors throughout.
+bool weights_aligned(int type, const void *W, size_t nb01) {
+    const size_t a = (type == T_Q6_K) ? 2 : 16;
+    return ((uintptr_t)W % a) == 0 && (nb01 % a) == 0;
+}
+
+size_t act_stride(int act_type, int64_t K) { return act_type == T_Q8_0 ? q8_0_stride(K) : q8_K_stride(K); }
+
+}  // namespace
+
+extern "C" {
+
+int chip_device_count(void) {
+    int n = 0;
+    return hipGetDeviceCount(&n) == hipSuccess ? n : 0;
+}
+
+int chip_init(int device) {
+    int n = chip_device_count();
+    if (n <= 0) return CHIP_ENODEVICE;
+    if (device < 0 || device >= n) return CHIP_EINVAL;
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t p;
+    e = hipGetDeviceProperties(&p, device);
+    if (e != hipSuccess) return (int)e;
+    if (std::strncmp(p.gcnArchName, "gfx950", 6) != 0) return CHIP_ENODEVICE;   // the kernels are built for gfx950 only
+    DeviceLimits lim;
+    return current_limits(lim);
+}
+
+int chip_get_device_info(chip_device_info *out) {
+    if (!out) return CHIP_EINVAL;
+    std::memset(out, 0, sizeof(*out));
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t p;
+    e = hipGetDeviceProperties(&p, dev);
+    if (e != hipSuccess) return (int)e;
+    DeviceLimits lim;
+    int rc = current_limits(lim);
+    if (rc) return rc;
+    out->device = dev;
+    out->compute_units = p.multiProcessorCount;
+    out->wavefront_size = p.warpSize;
+    out->max_lds_per_block = lim.max_lds_per_block;
+    out->clock_khz = p.clockRate;
+    out->xcd_count = 0;
+    size_t fr = 0, tot = 0;
+    if (hipMemGetInfo(&fr, &tot) == hipSuccess) { out->hbm_free = fr; out->hbm_total = tot; }
+    std::snprintf(out->name, sizeof(out->name), "%s", p.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+    return CHIP_OK;
+}
+
+const char *chip_error_string(int code) {
+    switch (code) {
+        case CHIP_OK: return "ok";
+        case CHIP_EINVAL: return "invalid argument (null, negative, or misaligned)";
+        case CHIP_EUNSUPPORTED: return "unsupported type or shape";
+        case CHIP_ENOMEM: return "workspace too small";
+        case CHIP_ENODEVICE: return "no gfx950 device";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}
+
+int chip_malloc(void **dptr, size_t bytes) {
+    if (!dptr) return CHIP_EINVAL;
+    *dptr = nullptr;
+    if (bytes == 0) return CHIP_OK;
+    return hip_rc(hipMalloc(dptr, bytes));
+}
+int chip_free(void *dptr) { return dptr ? hip_rc(hipFree(dptr)) : CHIP_OK; }
+
+int chip_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return CHIP_OK;
+    if (!dst || !src) return CHIP_EINVAL;
+    if (!stream) return hip_rc(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return hip_rc(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+}
+int chip_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return CHIP_OK;
+    if (!dst || !src) return CHIP_EINVAL;
+    if (!stream) return hip_rc(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return hip_rc(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+}
+int chip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return CHIP_OK;
+    if (!dst || !src) return CHIP_EINVAL;
+    return hip_rc(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+}
+int chip_memset(void *dst, int value, size_t bytes, void *stream) {
+    if (bytes == 0) return CHIP_OK;
+    if (!dst) return CHIP_EINVAL;
+    return hip_rc(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream));
+}
+int chip_stream_create(void **stream) {
+    if (!stream) return CHIP_EINVAL;
+    hipStream_t s = nullptr;
+    hipError_t e = hipStreamCreate(&s);                                  // default priority
+    *stream = (void *)s;
+    return hip_rc(e);
+}
+int chip_stream_destroy(void *stream) { return stream ? hip_rc(hipStreamDestroy((hipStream_t)stream)) : CHIP_OK; }
+int chip_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((hipStream_t)stream)); }
+
+int chip_block_elems(int type) {
+    switch (type) {
+        case T_F32: return 1;
+        case T_Q4_0: case T_Q8_0: return 32;
+        case T_Q4_K: case T_Q6_K: case T_Q8_K: return 256;
+        default: return 0;
+    }
+}
+size_t chip_block_bytes(int type) {
+    switch (type) {
+        case T_F32: return 4;
+        case T_Q4_0: return BYTES_Q4_0;
+        case T_Q8_0: return BYTES_Q8_0;
+        case T_Q4_K: return BYTES_Q4_K;
+        case T_Q6_K: return BYTES_Q6_K;
+        case T_Q8_K: return BYTES_Q8_K;
+        default: return 0;
+    }
+}
+size_t chip_row_size(int type, int64_t k) {
+    const int be = chip_block_elems(type);
+    return (be && k > 0) ? (size_t)(k / be) * chip_block_bytes(type) : 0;
+}
+int chip_vec_dot_type(int type) {
+    switch (type) {
+        case T_Q4_0: case T_Q8_0: return T_Q8_0;
+        case T_Q4_K: case T_Q6_K: return T_Q8_K;
+        default: return -1;
+    }
+}
+int chip_mul_mat_supported(int type, int64_t K) { return is_weight_type(type) && K > 0 && K % 256 == 0 && K <= (1 << 20); }
+
+static int quantize_public(int act_type, const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
+    if (n < 0 || k < 0) return CHIP_EINVAL;
+    if (n == 0 || k == 0) return CHIP_OK;
+    if (!x || !y || ldx < k) return CHIP_EINVAL;
+    if (k % chip_block_elems(act_type) != 0) return CHIP_EUNSUPPORTED;
+    if (!aligned16(x) || (ldx % 4) != 0) return CHIP_EINVAL;             // float4 loads
+    if (((uintptr_t)y & 3) != 0) return CHIP_EINVAL;
+    if (n > 65535) return CHIP_EUNSUPPORTED;
+    return hip_rc(launch_quantize(act_type, false, x, ldx, n, k, y, chip_row_size(act_type, k), (hipStream_t)stream));
+}
+int chip_quantize_q8_0(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
+    return quantize_public(T_Q8_0, x, ldx, n, k, y, stream);
+}
+int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
+    return quantize_public(T_Q8_K, x, ldx, n, k, y, stream);
+}
+
+size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n) {
+    if (!chip_mul_mat_supported(type, K) || n <= 0) return 0;
+    return act_stride(chip_vec_dot_type(type), K) * (size_t)n;
+}
+
+int chip_mul_mat_prepare(int type, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    if (n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (n == 0) return CHIP_OK;
+    if (!x || !workspace || ldx < K) return CHIP_EINVAL;
+    if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace)) return CHIP_EINVAL;
+    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+    const int at = chip_vec_dot_type(type);
+    const size_t stride = act_stride(at, K);
+    // grid.y carries the token index: split very long prompts
+    for (int64_t t0 = 0; t0 < n; t0 += 32768) {
+        const int64_t nt = (n - t0 < 32768) ? n - t0 : 32768;
+        hipError_t e = launch_quantize(at, true, x + t0 * ldx, ldx, nt, K, (uint8_t *)workspace + t0 * stride, stride,
+                                       (hipStream_t)stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    return CHIP_OK;
+}
+
+int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
+                     float *y, int64_t ldy, void *stream) {
+    if (N < 0 || n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n == 0) return CHIP_OK;
+    if (!W || !workspace || !y || ldy < N) return CHIP_EINVAL;
+    if (!weights_aligned(type, W, nb01) || nb01 < chip_row_size(type, K) || !aligned16(workspace)) return CHIP_EINVAL;
+    if (((uintptr_t)y & 3) != 0) return CHIP_EINVAL;
+    DeviceLimits lim;
+    int rc = current_limits(lim);
+    if (rc) return rc;
+    const size_t stride = act_stride(chip_vec_dot_type(type), K);
+    hipStream_t st = (hipStream_t)stream;
+
+    if (type == T_Q4_0 && n >= 16 && gemm_q4_0_supported(K, N, n))
+        return hip_rc(launch_gemm_q4_0(W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
+
+    const int group = gemv_max_tokens(type, K, lim);
+    if (group < 1) return CHIP_EUNSUPPORTED;
+    for (int64_t t0 = 0; t0 < n; t0 += group) {
+        const int nt = (int)((n - t0 < group) ? n - t0 : group);
+        hipError_t e = launch_gemv(type, W, nb01, K, N, (const uint8_t *)workspace + t0 * stride, stride, nt, y + t0 * ldy,
+                                   ldy, lim, st);
+        if (e != hipSuccess) return (int)e;
+    }
+    return CHIP_OK;
+}
+
+int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
+                 float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = chip_mul_mat_prepare(type, K, x, ldx, n, workspace, workspace_bytes, stream);
+    if (rc) return rc;
+    return chip_mul_mat_run(type, W, nb01, K, N, n, workspace, y, ldy, stream);
+}
+
+int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
+                     int32_t *isum, int32_t *imin, void *stream) {
+    if (N < 0 || n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n == 0) return CHIP_OK;
+    if (!W || !aq || !isum) return CHIP_EINVAL;
+    if (!weights_aligned(type, W, nb01) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;
+    return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, type == T_Q4_K ? imin : nullptr, (hipStream_t)stream));
+}
+
+int chip_workspace_to_blocks(int type, int64_t K, int64_t n, const void *workspace, void *y, void *stream) {
+    if (n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (n == 0) return CHIP_OK;
+    if (!workspace || !y || n > 65535) return CHIP_EINVAL;
+    const int at = chip_vec_dot_type(type);
+    return hip_rc(launch_split_to_blocks(at, workspace, act_stride(at, K), n, K, y, chip_row_size(at, K), (hipStream_t)stream));
+}
+
+}  // extern "C"

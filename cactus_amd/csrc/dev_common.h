@@ -1,0 +1,70 @@
+// Device-side helpers shared by the gfx950 kernels: block layout constants, exact fp16 conversion,
+// 4-way int8 dot, funnel shift, and a wave64 butterfly sum built from DPP moves (no LDS traffic).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+namespace chip {
+
+// GGUF block sizes in bytes (reference ggml-common.h:172,214,296,326,334).
+constexpr int QK_SMALL = 32;     // elements per Q4_0 / Q8_0 block
+constexpr int QK_K     = 256;    // elements per K-quant super-block
+constexpr int BYTES_Q4_0 = 18, BYTES_Q8_0 = 34, BYTES_Q4_K = 144, BYTES_Q6_K = 210, BYTES_Q8_K = 292;
+
+enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15 };
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+// Same vectors with relaxed alignment: gfx950 global loads need no more than the element alignment given
+// here, and GGUF blocks (18/34/210 bytes) are only 2-byte aligned inside a 16-byte aligned row.
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ float h2f(uint32_t h16) {
+    return __half2float(__ushort_as_half((unsigned short)(h16 & 0xffffu)));     // exact
+}
+__device__ __forceinline__ unsigned short f2h_rne(float f) {
+    return __half_as_ushort(__float2half_rn(f));                               // IEEE round-to-nearest-even
+}
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);                    // v_dot4_i32_i8, signed x signed
+}
+// low 32 bits of ((hi:lo) >> 16): re-slices a byte stream that starts 2 bytes into a dword
+__device__ __forceinline__ uint32_t shr16(uint32_t hi, uint32_t lo) {
+    return __builtin_amdgcn_alignbit(hi, lo, 16);
+}
+
+template <int CTRL, int ROW_MASK = 0xf, bool BOUND = true>
+__device__ __forceinline__ float dpp_get(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, BOUND));
+}
+// Sum over the 64 lanes of a wave in a fixed butterfly order; the total ends up in lane 63.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+    v += dpp_get<0xB1>(v);               // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E>(v);               // quad_perm [2,3,0,1]
+    v += dpp_get<0x141>(v);              // row_half_mirror
+    v += dpp_get<0x140>(v);              // row_mirror: every lane of a 16-lane row holds the row sum
+    v += dpp_get<0x142, 0xa, false>(v);  // row_bcast15 into rows 1 and 3
+    v += dpp_get<0x143, 0xc, false>(v);  // row_bcast31 into rows 2 and 3
+    return v;
+}
+__device__ __forceinline__ float wave_max_all(float v) {
+    v = fmaxf(v, dpp_get<0xB1>(v));
+    v = fmaxf(v, dpp_get<0x4E>(v));
+    v = fmaxf(v, dpp_get<0x141>(v));
+    v = fmaxf(v, dpp_get<0x140>(v));
+    // rows hold their own maxima; finish through the scalar unit (values are >= 0 here, so 0 is neutral)
+    float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+__host__ __device__ constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace chip

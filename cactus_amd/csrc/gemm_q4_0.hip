@@ -1,0 +1,291 @@
+// Prefill GEMM for gfx950: Y[t][r] = sum_b dw[r][b] * dx[t][b] * isum[t][r][b] over Q4_0 weights and Q8_0
+// activations, the batched form of lm_ggml_vec_dot_q4_0_q8_0 (reference ggml-cpu/ggml-cpu-quants.c:1906-2602)
+// as driven by lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449).
+//
+// Structure
+//   * One v_mfma_i32_32x32x32_i8 multiplies a 32-row x 32-k weight tile by a 32-k x 32-token activation tile:
+//     its K extent is exactly one 32-value quantization block, so each of the 1024 int32 results is one
+//     per-block integer sum isum[t][r][b], bit-exact.
+//   * Weight tiles are staged through LDS once per workgroup and k-stage: the Q4_0 nibbles are split into the
+//     low-nibble half (elements 0..15) and the high-nibble half (16..31) and turned into signed int8 (nib - 8);
+//     activations arrive as int8 from the split workspace layout.  Both sit in LDS as [k-block][half][row]
+//     16-byte cells, which is exactly what one lane feeds the MFMA (row = lane % 32, half = lane / 32).
+//   * Per-block scales are applied in fp32 after the integer accumulate.  The MFMA's C input is a register
+//     vector holding the bit pattern of 12582912.0f (1.5 * 2^23): adding |isum| < 2^22 to those bits gives the
+//     bits of the float 12582912 + isum, so the accumulator can be used as a float with no conversion.  Then
+//         t   = fma(acc_as_float, dx, -12582912 * dx)      exactly round(isum * dx): 12582912*dx is exact
+//                                                           because dx comes from fp16 (11-bit significand)
+//         out = fma(t, dw, out)                            dw read as fp16 by the mixed-precision fma
+//     i.e. two VALU operations per integer sum, 32 per MFMA.  That VALU work, not the matrix pipe, bounds this
+//     kernel: an MFMA occupies the matrix unit for 32 cycles, 32 wave-wide fp32 operations occupy the vector
+//     unit for 128.
+//   * A workgroup is WR x WC waves, each wave owns TM x TN MFMA tiles (32*TM rows x 32*TN tokens); LDS is
+//     double buffered over stages of KB = 4 blocks with one barrier per stage and the next stage's global
+//     loads in flight during the current stage's arithmetic.
+#include "dev_common.h"
+#include "act_layout.h"
+#include "kernels.h"
+
+namespace chip {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int GEMM_KB = 4;                    // 32-value blocks per LDS stage
+constexpr float MAGIC_F = 12582912.f;         // 1.5 * 2^23
+constexpr int MAGIC_I = 0x4B400000;
+
+// nibbles 0..15 in the four bytes of x  ->  signed bytes (nibble - 8)
+__device__ __forceinline__ uint32_t nib_to_i8(uint32_t x) {
+    return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+}
+
+template <int TM, int TN, int WR, int WC>
+struct GemmCfg {
+    static constexpr int NW = WR * WC, NT = NW * 64;
+    static constexpr int BM = 32 * TM * WR;                        // weight rows per workgroup
+    static constexpr int BN = 32 * TN * WC;                        // tokens per workgroup
+    static constexpr int A_CELLS = GEMM_KB * 2 * BM;               // 16-byte cells
+    static constexpr int B_CELLS = GEMM_KB * 2 * BN;
+    static constexpr size_t OFF_A = 0;
+    static constexpr size_t OFF_B = OFF_A + (size_t)A_CELLS * 16;
+    static constexpr size_t OFF_SW = OFF_B + (size_t)B_CELLS * 16;                 // fp16 [KB][BM], permuted per 32 rows
+    static constexpr size_t OFF_SX = OFF_SW + (size_t)GEMM_KB * BM * 2;            // fp32 [KB][BN]
+    static constexpr size_t STAGE = OFF_SX + (size_t)GEMM_KB * BN * 4;
+    static constexpr int W_ITEMS = BM * GEMM_KB;                   // (row, block) pairs per stage
+    static constexpr int W_PER_T = (W_ITEMS + NT - 1) / NT;
+    static constexpr int X_ITEMS = BN * GEMM_KB * 2;               // 16-byte activation cells per stage
+    static constexpr int X_PER_T = (X_ITEMS + NT - 1) / NT;
+    static constexpr int S_ITEMS = BN * GEMM_KB;                   // activation scales per stage
+    static constexpr int S_PER_T = (S_ITEMS + NT - 1) / NT;
+};
+
+template <int TM, int TN, int WR, int WC>
+__global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
+                                                                int64_t N, const uint8_t *__restrict__ ws,
+                                                                size_t ws_stride, int64_t M, float *__restrict__ y,
+                                                                int64_t ldy) {
+    using C = GemmCfg<TM, TN, WR, WC>;
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wr = wave / WC, wc = wave % WC;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t row_base = (int64_t)blockIdx.x * C::BM;
+    const int64_t tok_base = (int64_t)blockIdx.y * C::BN;
+    const int nstages = (int)(K / (32 * GEMM_KB));
+    const size_t off_d = q8_0_off_d(K);
+
+    // ---- per-thread prefetch registers for one stage ----
+    u32x4 wq[C::W_PER_T];
+    uint32_t wd[C::W_PER_T];
+    u32x4 xq[C::X_PER_T];
+    float xs[C::S_PER_T];
+
+    auto fetch = [&](int stage) {
+        const int64_t kb0 = (int64_t)stage * GEMM_KB;
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
+                const int r = item / GEMM_KB, b = item % GEMM_KB;
+                const int64_t row = min(row_base + r, N - 1);
+                const uint8_t *p = W + (size_t)row * nb01 + (size_t)(kb0 + b) * BYTES_Q4_0;
+                wd[i] = *reinterpret_cast<const unsigned short *>(p);
+                wq[i] = *reinterpret_cast<const u32x4_a2 *>(p + 2);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
+                const int c = item % (GEMM_KB * 2), n = item / (GEMM_KB * 2);       // c = 2*b + half
+                const int64_t tok = min(tok_base + n, M - 1);
+                xq[i] = *reinterpret_cast<const u32x4 *>(ws + (size_t)tok * ws_stride + (size_t)kb0 * 32 + 16 * c);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::S_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
+                const int b = item % GEMM_KB, n = item / GEMM_KB;
+                const int64_t tok = min(tok_base + n, M - 1);
+                xs[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_d)[kb0 + b];
+            }
+        }
+    };
+
+    auto commit = [&](int buf) {
+        uint8_t *base = lds + (size_t)buf * C::STAGE;
+        u32x4 *A = reinterpret_cast<u32x4 *>(base + C::OFF_A);
+        u32x4 *B = reinterpret_cast<u32x4 *>(base + C::OFF_B);
+        unsigned short *SW = reinterpret_cast<unsigned short *>(base + C::OFF_SW);
+        float *SX = reinterpret_cast<float *>(base + C::OFF_SX);
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
+                const int r = item / GEMM_KB, b = item % GEMM_KB;
+                u32x4 lo, hi;
+                lo.x = nib_to_i8(wq[i].x & 0x0f0f0f0fu); hi.x = nib_to_i8((wq[i].x >> 4) & 0x0f0f0f0fu);
+                lo.y = nib_to_i8(wq[i].y & 0x0f0f0f0fu); hi.y = nib_to_i8((wq[i].y >> 4) & 0x0f0f0f0fu);
+                lo.z = nib_to_i8(wq[i].z & 0x0f0f0f0fu); hi.z = nib_to_i8((wq[i].z >> 4) & 0x0f0f0f0fu);
+                lo.w = nib_to_i8(wq[i].w & 0x0f0f0f0fu); hi.w = nib_to_i8((wq[i].w >> 4) & 0x0f0f0f0fu);
+                A[(b * 2 + 0) * C::BM + r] = lo;
+                A[(b * 2 + 1) * C::BM + r] = hi;
+                // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4;
+                // store the scale of row i at half*16 + (i/8)*4 + i%4 so each lane reads its 16 scales contiguously
+                const int i32 = r & 31;
+                const int pos = ((i32 >> 2) & 1) * 16 + (i32 >> 3) * 4 + (i32 & 3);
+                SW[b * C::BM + (r & ~31) + pos] = (unsigned short)wd[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
+                const int c = item % (GEMM_KB * 2), n = item / (GEMM_KB * 2);
+                B[c * C::BN + n] = xq[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::S_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
+                const int b = item % GEMM_KB, n = item / GEMM_KB;
+                SX[b * C::BN + n] = xs[i];
+            }
+        }
+    };
+
+    float acc[TM][TN][16];
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+
+    // The magic constant lives in 16 registers for the whole kernel; the empty asm keeps the compiler from
+    // re-materialising it with 16 moves in front of every MFMA.
+    i32x16 magic;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        int m = MAGIC_I;
+        asm volatile("" : "+v"(m));
+        magic[v] = m;
+    }
+
+    fetch(0);
+    commit(0);
+    __syncthreads();
+
+    for (int s = 0; s < nstages; s++) {
+        const int buf = s & 1;
+        if (s + 1 < nstages) fetch(s + 1);
+
+        const uint8_t *base = lds + (size_t)buf * C::STAGE;
+        const u32x4 *A = reinterpret_cast<const u32x4 *>(base + C::OFF_A);
+        const u32x4 *B = reinterpret_cast<const u32x4 *>(base + C::OFF_B);
+        const u32x4 *SW = reinterpret_cast<const u32x4 *>(base + C::OFF_SW);
+        const float *SX = reinterpret_cast<const float *>(base + C::OFF_SX);
+
+#pragma unroll 1
+        for (int b = 0; b < GEMM_KB; b++) {
+            i32x4 af[TM], bf[TN];
+            u32x4 sw[TM][2];
+            float dx[TN], ndx[TN];
+#pragma unroll
+            for (int a = 0; a < TM; a++) {
+                const int r0 = (wr * TM + a) * 32;
+                const u32x4 t = A[(b * 2 + half) * C::BM + r0 + l32];
+                af[a] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
+                const u32x4 *sp = SW + ((size_t)b * C::BM + r0 + half * 16) / 8;    // 8 halves per 16-byte cell
+                sw[a][0] = sp[0];
+                sw[a][1] = sp[1];
+            }
+#pragma unroll
+            for (int c = 0; c < TN; c++) {
+                const int n0 = (wc * TN + c) * 32;
+                const u32x4 t = B[(b * 2 + half) * C::BN + n0 + l32];
+                bf[c] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
+                dx[c] = SX[b * C::BN + n0 + l32];
+                ndx[c] = -MAGIC_F * dx[c];
+            }
+            // Software pipeline over the TM*TN tiles of this k-block: the MFMA of tile i+1 is issued before the
+            // 32 scaling operations of tile i, so the matrix unit works underneath the vector unit.
+            i32x16 d_cur = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0], bf[0], magic, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < TM * TN; i++) {
+                const int a = i / TN, c = i % TN;
+                i32x16 d_next = d_cur;
+                if (i + 1 < TM * TN) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[(i + 1) / TN], bf[(i + 1) % TN], magic, 0, 0, 0);
+                const uint32_t swd[8] = {sw[a][0].x, sw[a][0].y, sw[a][0].z, sw[a][0].w,
+                                         sw[a][1].x, sw[a][1].y, sw[a][1].z, sw[a][1].w};
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float t = __builtin_fmaf(__int_as_float(d_cur[v]), dx[c], ndx[c]);
+                    const __half hw = __ushort_as_half((unsigned short)((v & 1) ? (swd[v >> 1] >> 16) : (swd[v >> 1] & 0xffffu)));
+                    acc[a][c][v] = __builtin_fmaf(t, __half2float(hw), acc[a][c][v]);
+                }
+                d_cur = d_next;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+
+        if (s + 1 < nstages) commit(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: register v of tile (a, c) is row 8*(v/4) + 4*half + v%4, token l32 ----
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int c = 0; c < TN; c++) {
+            const int64_t tok = tok_base + (wc * TN + c) * 32 + l32;
+            if (tok >= M) continue;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int64_t row = row_base + (wr * TM + a) * 32 + 8 * g + 4 * half;
+                float *dst = y + (size_t)tok * ldy + row;
+                if (row + 3 < N && (((uintptr_t)dst) & 15) == 0) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(acc[a][c][4 * g], acc[a][c][4 * g + 1], acc[a][c][4 * g + 2], acc[a][c][4 * g + 3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (row + e < N) dst[e] = acc[a][c][4 * g + e];
+                }
+            }
+        }
+}
+
+bool gemm_q4_0_supported(int64_t K, int64_t N, int64_t n) { return K % (32 * GEMM_KB) == 0 && N >= 1 && n >= 1; }
+
+template <int TM, int TN, int WR, int WC>
+static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
+                             float *y, int64_t ldy, hipStream_t st) {
+    using C = GemmCfg<TM, TN, WR, WC>;
+    const size_t lds_bytes = 2 * C::STAGE;
+    auto kfn = gemm_q4_0_kernel<TM, TN, WR, WC>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    dim3 grid((unsigned)ceil_div(N, C::BM), (unsigned)ceil_div(M, C::BN));
+    hipLaunchKernelGGL(kfn, grid, dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws, ws_stride,
+                       M, y, ldy);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
+                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    if (M <= 0 || N <= 0) return hipSuccess;
+    const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    // pick the largest workgroup tile that still leaves about two workgroups' worth of work per CU
+    const int64_t big = ceil_div(N, 128) * ceil_div(M, 256);
+    const int64_t mid = ceil_div(N, 128) * ceil_div(M, 128);
+    if (big >= 2 * cus) return launch_cfg<2, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+    if (mid >= 2 * cus) return launch_cfg<2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+    return launch_cfg<1, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+}
+
+}  // namespace chip

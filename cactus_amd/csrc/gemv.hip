@@ -1,0 +1,510 @@
+// Decode GEMV for gfx950: y[t][r] = vec_dot(W row r, quantized activation t) for 1..8 tokens, over GGUF
+// Q4_0 / Q8_0 / Q4_K / Q6_K rows kept in their on-disk block layout.  Restates the work of
+// lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K} (reference ggml-cpu/ggml-cpu-quants.c:1906,
+// 3591,6772,8520) driven by lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449).
+//
+// Shape of the kernel (HBM-bound: every weight byte is read exactly once):
+//   * a wave owns a tile of R consecutive weight rows and walks along K; lane l handles "unit" u = l + 64*it
+//     of every row, a unit being the smallest piece that carries whole scales (two 32-blocks for Q4_0/Q8_0,
+//     1/8 of a Q4_K super-block, 1/4 of a Q6_K super-block).  Consecutive lanes read consecutive bytes, so a
+//     wave's loads cover one contiguous span of each row;
+//   * the R rows' loads of an iteration are issued back to back before any use (R x 36..68 bytes per lane in
+//     flight), which is what keeps HBM busy;
+//   * quantized activations are staged once per workgroup into LDS, transposed so that lane l's 16-byte
+//     chunks are adjacent to lane l+1's (conflict-free ds_read_b128), and are re-read per row tile from LDS,
+//     never from global memory;
+//   * integer dots use v_dot4_i32_i8; each lane keeps fp32 partial sums per (row, token) and the 64 lanes are
+//     combined at the end with a fixed DPP butterfly (no LDS round trip, deterministic order).
+#include "dev_common.h"
+#include "act_layout.h"
+#include "kernels.h"
+
+namespace chip {
+
+// ------------------------------------------------------------------------------------------------ traits
+// For each weight type: how a lane's unit maps to weight bytes and to activation planes.
+//   UNIT_ELEMS : K elements covered by one lane-unit
+//   QCH        : 16-byte activation chunks per unit
+//   AUX        : bytes of per-unit activation side data (scales, sums) kept in LDS
+template <int WT> struct Traits;
+
+template <> struct Traits<T_Q8_0> {
+    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
+    struct W { uint32_t q[16]; float d0, d1; };
+    struct A { uint32_t q[16]; float d0, d1; };
+
+    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *p = row + (size_t)u * 68;                       // two 34-byte blocks, 4-byte aligned
+        const u32x4 a = *reinterpret_cast<const u32x4_a4 *>(p);
+        const u32x4 b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        const u32x4 c = *reinterpret_cast<const u32x4_a4 *>(p + 32);
+        const u32x4 e = *reinterpret_cast<const u32x4_a4 *>(p + 48);
+        const uint32_t f = *reinterpret_cast<const uint32_t *>(p + 64);
+        // block 0: d at byte 0, quants at bytes 2..33 -> re-slice by 16 bits; block 1: d at 34, quants at 36..67
+        w.d0 = h2f(a.x);
+        w.q[0] = shr16(a.y, a.x); w.q[1] = shr16(a.z, a.y); w.q[2] = shr16(a.w, a.z); w.q[3] = shr16(b.x, a.w);
+        w.q[4] = shr16(b.y, b.x); w.q[5] = shr16(b.z, b.y); w.q[6] = shr16(b.w, b.z); w.q[7] = shr16(c.x, b.w);
+        w.d1 = h2f(c.x >> 16);
+        w.q[8] = c.y; w.q[9] = c.z; w.q[10] = c.w; w.q[11] = e.x;
+        w.q[12] = e.y; w.q[13] = e.z; w.q[14] = e.w; w.q[15] = f;
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
+        const float2 d = reinterpret_cast<const float2 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
+        a.d0 = d.x; a.d1 = d.y;
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
+        i0 = 0; i1 = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { i0 = dot4(w.q[i], a.q[i], i0); i1 = dot4(w.q[8 + i], a.q[8 + i], i1); }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int i0, i1;
+        isums(w, a, i0, i1);
+        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
+        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
+    }
+    // staging: where unit u's chunk j and side data live in the split workspace planes of one token
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
+    __device__ static __forceinline__ void stage_aux(uint8_t *dst, const uint8_t *ws, int64_t K, int u, bool valid) {
+        float2 d = make_float2(0.f, 0.f);
+        if (valid) d = reinterpret_cast<const float2 *>(ws + q8_0_off_d(K))[u];
+        *reinterpret_cast<float2 *>(dst) = d;
+    }
+};
+
+template <> struct Traits<T_Q4_0> {
+    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
+    struct W { uint32_t lo[8], hi[8]; float d0, d1; };          // nibbles spread to bytes, 0..15
+    struct A { uint32_t q[16]; float d0, d1; int s0, s1; };
+
+    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *p = row + (size_t)u * 36;                       // two 18-byte blocks, 4-byte aligned
+        const u32x4 a = *reinterpret_cast<const u32x4_a4 *>(p);
+        const u32x4 b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        const uint32_t c = *reinterpret_cast<const uint32_t *>(p + 32);
+        uint32_t q[8];
+        w.d0 = h2f(a.x);
+        q[0] = shr16(a.y, a.x); q[1] = shr16(a.z, a.y); q[2] = shr16(a.w, a.z); q[3] = shr16(b.x, a.w);
+        w.d1 = h2f(b.x >> 16);
+        q[4] = b.y; q[5] = b.z; q[6] = b.w; q[7] = c;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { w.lo[i] = q[i] & 0x0f0f0f0fu; w.hi[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
+        const u32x4 x = reinterpret_cast<const u32x4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
+        a.d0 = __uint_as_float(x.x); a.d1 = __uint_as_float(x.y); a.s0 = (int)x.z; a.s1 = (int)x.w;
+    }
+    // byte i of qs holds element i (low nibble) and element i+16 (high nibble); value = nibble - 8
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
+        i0 = -8 * a.s0; i1 = -8 * a.s1;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            i0 = dot4(w.lo[i], a.q[i], i0);         i0 = dot4(w.hi[i], a.q[4 + i], i0);
+            i1 = dot4(w.lo[4 + i], a.q[8 + i], i1); i1 = dot4(w.hi[4 + i], a.q[12 + i], i1);
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int i0, i1;
+        isums(w, a, i0, i1);
+        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
+        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
+    __device__ static __forceinline__ void stage_aux(uint8_t *dst, const uint8_t *ws, int64_t K, int u, bool valid) {
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (valid) {
+            const u32x2 d = reinterpret_cast<const u32x2 *>(ws + q8_0_off_d(K))[u];
+            const u32x2 s = reinterpret_cast<const u32x2 *>(ws + q8_0_off_sum(K))[u];
+            x.x = d.x; x.y = d.y; x.z = s.x; x.w = s.y;
+        }
+        *reinterpret_cast<u32x4 *>(dst) = x;
+    }
+};
+
+template <> struct Traits<T_Q4_K> {
+    // unit = (super-block sb, chunk c of 8): qs bytes 16c..16c+15, i.e. elements 64*(c/2) + 16*(c%2) + [0,16)
+    // from the low nibbles (sub-block 2*(c/2)) and the same + 32 from the high nibbles (sub-block 2*(c/2)+1)
+    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 32, QCH = 2, AUX = 8;
+    struct W { uint32_t lo[4], hi[4]; float d, dmin; int sc0, sc1, m0, m1; };
+    struct A { uint32_t q[8]; float d; int s0, s1; };
+
+    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const int sb = u >> 3, c = u & 7;
+        const uint8_t *p = row + (size_t)sb * BYTES_Q4_K;              // 144-byte super-block, 16-byte aligned
+        const u32x4 h = *reinterpret_cast<const u32x4 *>(p);
+        const u32x4 q = *reinterpret_cast<const u32x4 *>(p + 16 + 16 * c);
+        w.d = h2f(h.x); w.dmin = h2f(h.x >> 16);
+        // 6-bit scale/min of sub-blocks (2jp, 2jp+1), jp = c/2 (reference ggml-quants.c:625-632)
+        const int jp = c >> 1, sh = 16 * (jp & 1);
+        const uint32_t a1 = h.y >> sh, a2 = h.z >> sh, a3 = h.w >> sh;
+        uint32_t sc, mn;
+        if (jp < 2) { sc = a1 & 0x3f3fu; mn = a2 & 0x3f3fu; }
+        else        { sc = (a3 & 0x0f0fu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
+        w.sc0 = sc & 0xff; w.sc1 = sc >> 8; w.m0 = mn & 0xff; w.m1 = mn >> 8;
+        w.lo[0] = q.x & 0x0f0f0f0fu; w.lo[1] = q.y & 0x0f0f0f0fu; w.lo[2] = q.z & 0x0f0f0f0fu; w.lo[3] = q.w & 0x0f0f0f0fu;
+        w.hi[0] = (q.x >> 4) & 0x0f0f0f0fu; w.hi[1] = (q.y >> 4) & 0x0f0f0f0fu;
+        w.hi[2] = (q.z >> 4) & 0x0f0f0f0fu; w.hi[3] = (q.w >> 4) & 0x0f0f0f0fu;
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+        const u32x4 v0 = q[0], v1 = q[64];
+        a.q[0] = v0.x; a.q[1] = v0.y; a.q[2] = v0.z; a.q[3] = v0.w;
+        a.q[4] = v1.x; a.q[5] = v1.y; a.q[6] = v1.z; a.q[7] = v1.w;
+        const u32x2 x = reinterpret_cast<const u32x2 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
+        a.d = __uint_as_float(x.x);
+        a.s0 = (int)(int16_t)(x.y & 0xffff); a.s1 = (int)(int16_t)(x.y >> 16);
+    }
+    // this unit's share of the super-block sums: isum = sum_j sc_j * dot_j, imin = sum_j m_j * bsum_j
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &im) {
+        int dl = 0, dh = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { dl = dot4(w.lo[i], a.q[i], dl); dh = dot4(w.hi[i], a.q[4 + i], dh); }
+        is = w.sc0 * dl + w.sc1 * dh;
+        im = w.m0 * a.s0 + w.m1 * a.s1;
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int is, im;
+        isums(w, a, is, im);
+        acc = __builtin_fmaf(w.d * a.d, (float)is, acc);
+        return __builtin_fmaf(-(w.dmin * a.d), (float)im, acc);
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) {
+        const int sb = u >> 3, c = u & 7;
+        return (size_t)sb * 256 + 64 * (c >> 1) + 16 * (c & 1) + 32 * j;
+    }
+    __device__ static __forceinline__ void stage_aux(uint8_t *dst, const uint8_t *ws, int64_t K, int u, bool valid) {
+        u32x2 x = {0u, 0u};
+        if (valid) {
+            const int sb = u >> 3, c = u & 7;
+            const int16_t *bs = reinterpret_cast<const int16_t *>(ws + q8_K_off_bsums(K)) + sb * 16 + 4 * (c >> 1) + (c & 1);
+            x.x = reinterpret_cast<const uint32_t *>(ws + q8_K_off_d(K))[sb];
+            x.y = (uint32_t)(uint16_t)bs[0] | ((uint32_t)(uint16_t)bs[2] << 16);
+        }
+        *reinterpret_cast<u32x2 *>(dst) = x;
+    }
+};
+
+template <> struct Traits<T_Q6_K> {
+    // unit = (super-block sb, half h, ip): 16 consecutive l = 16*ip + [0,16) of half h, i.e. the four
+    // 16-element groups {128h + 32v + 16ip + [0,16) : v = 0..3}; scale of group v is scales[8h + 2v + ip]
+    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
+    struct W { uint32_t q[16]; float d; int sc[4]; };            // q[4v + k]: 6-bit values 0..63 of group v
+    struct A { uint32_t q[16]; float d; int bs[4]; };
+
+    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
+        const uint8_t *p = row + (size_t)sb * BYTES_Q6_K;              // 210-byte super-block, 2-byte aligned
+        const u32x4 l0 = *reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 16 * ip);
+        const u32x4 l1 = *reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 32 + 16 * ip);
+        const u32x4 qh = *reinterpret_cast<const u32x4_a2 *>(p + 128 + 32 * h + 16 * ip);
+        const u32x2 s  = *reinterpret_cast<const u32x2_a2 *>(p + 192 + 8 * h);
+        w.d = h2f(*reinterpret_cast<const unsigned short *>(p + 208));
+        const uint32_t ql0[4] = {l0.x, l0.y, l0.z, l0.w}, ql1[4] = {l1.x, l1.y, l1.z, l1.w}, hh[4] = {qh.x, qh.y, qh.z, qh.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {                                   // reference ggml-quants.c:1695-1711
+            w.q[k]      = (ql0[k] & 0x0f0f0f0fu)        | ((hh[k] << 4) & 0x30303030u);
+            w.q[4 + k]  = (ql1[k] & 0x0f0f0f0fu)        | ((hh[k] << 2) & 0x30303030u);
+            w.q[8 + k]  = ((ql0[k] >> 4) & 0x0f0f0f0fu) | (hh[k] & 0x30303030u);
+            w.q[12 + k] = ((ql1[k] >> 4) & 0x0f0f0f0fu) | ((hh[k] >> 2) & 0x30303030u);
+        }
+        const int b = 8 * ip;                                           // scales[8h + 2v + ip]: byte ip / ip+2 of each dword
+        w.sc[0] = (int)(int8_t)(s.x >> b); w.sc[1] = (int)(int8_t)(s.x >> (b + 16));
+        w.sc[2] = (int)(int8_t)(s.y >> b); w.sc[3] = (int)(int8_t)(s.y >> (b + 16));
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
+        const u32x4 x = reinterpret_cast<const u32x4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
+        a.d = __uint_as_float(x.x);
+        a.bs[0] = (int)(int16_t)(x.y & 0xffff); a.bs[1] = (int)(int16_t)(x.y >> 16);
+        a.bs[2] = (int)(int16_t)(x.z & 0xffff); a.bs[3] = (int)(int16_t)(x.z >> 16);
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &unused) {
+        is = 0; unused = 0;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            int dv = -32 * a.bs[v];                                     // sum (q-32)*a = sum q*a - 32*sum a
+#pragma unroll
+            for (int k = 0; k < 4; k++) dv = dot4(w.q[4 * v + k], a.q[4 * v + k], dv);
+            is += w.sc[v] * dv;
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int is, unused;
+        isums(w, a, is, unused);
+        return __builtin_fmaf(w.d * a.d, (float)is, acc);
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) {
+        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
+        return (size_t)sb * 256 + 128 * h + 32 * j + 16 * ip;
+    }
+    __device__ static __forceinline__ void stage_aux(uint8_t *dst, const uint8_t *ws, int64_t K, int u, bool valid) {
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (valid) {
+            const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
+            const int16_t *bs = reinterpret_cast<const int16_t *>(ws + q8_K_off_bsums(K)) + sb * 16 + 8 * h + ip;
+            x.x = reinterpret_cast<const uint32_t *>(ws + q8_K_off_d(K))[sb];
+            x.y = (uint32_t)(uint16_t)bs[0] | ((uint32_t)(uint16_t)bs[2] << 16);
+            x.z = (uint32_t)(uint16_t)bs[4] | ((uint32_t)(uint16_t)bs[6] << 16);
+        }
+        *reinterpret_cast<u32x4 *>(dst) = x;
+    }
+};
+
+template <int WT> __host__ __device__ constexpr int units_per_row(int64_t K) { return (int)(K / Traits<WT>::UNIT_ELEMS); }
+template <int WT> __host__ __device__ constexpr int iters_per_row(int64_t K) { return (int)ceil_div(K / Traits<WT>::UNIT_ELEMS, 64); }
+template <int WT> __host__ __device__ constexpr size_t lds_image_bytes(int64_t K) {
+    return (size_t)iters_per_row<WT>(K) * (Traits<WT>::QCH * 1024 + 64 * Traits<WT>::AUX);
+}
+
+// ------------------------------------------------------------------------------------------------ kernel
+template <int WT, int NTOK, int R, int WGS>
+__global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
+                                                   const uint8_t *__restrict__ ws, size_t ws_stride,
+                                                   float *__restrict__ y, int64_t ldy) {
+    using T = Traits<WT>;
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int NI = iters_per_row<WT>(K);
+    const int units = units_per_row<WT>(K);
+    const size_t img = lds_image_bytes<WT>(K);
+
+    // ---- stage the NTOK quantized activations, transposed to [it][chunk][lane] ----
+    {
+        const int nq = NI * T::QCH * 64;                                // 16-byte chunks per token
+        for (int idx = threadIdx.x; idx < NTOK * nq; idx += WGS) {
+            const int t = idx / nq, r = idx - t * nq;
+            const int lane = r & 63, j = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
+            const int u = it * 64 + lane;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (u < units) v = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + T::src_chunk(K, u, j));
+            reinterpret_cast<u32x4 *>(lds + t * img)[r] = v;
+        }
+        const int na = NI * 64;
+        for (int idx = threadIdx.x; idx < NTOK * na; idx += WGS) {
+            const int t = idx / na, u = idx - t * na;
+            T::stage_aux(lds + t * img + (size_t)NI * T::QCH * 1024 + (size_t)u * T::AUX, ws + t * ws_stride, K, u, u < units);
+        }
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (WGS / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (WGS / 64);
+    const int64_t tiles = ceil_div(N, R);
+
+    for (int64_t tile = wave; tile < tiles; tile += nwaves) {
+        const int64_t row0 = tile * R;
+        float acc[R][NTOK];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < NTOK; t++) acc[r][t] = 0.f;
+
+        for (int it = 0; it < NI; it++) {
+            const int u = it * 64 + lane;
+            if (u < units) {
+                typename T::W w[R];
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int64_t row = min(row0 + r, N - 1);           // tail tile: re-read the last row, never store it
+                    T::load_w(w[r], W + (size_t)row * nb01, u);
+                }
+#pragma unroll
+                for (int t = 0; t < NTOK; t++) {
+                    typename T::A a;
+                    T::load_a(a, lds + t * img, NI, it, lane);
+#pragma unroll
+                    for (int r = 0; r < R; r++) acc[r][t] = T::dot(w[r], a, acc[r][t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < NTOK; t++) {
+                const float s = wave_sum_to_lane63(acc[r][t]);
+                if (lane == 63 && row0 + r < N) y[(size_t)t * ldy + row0 + r] = s;
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ launch
+template <int WT, int NTOK>
+static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                               float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
+    if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    // Small LDS images: 256-thread groups, several per CU, 4 rows per wave.  Large images leave room for a
+    // single group per CU, so make it 16 waves wide and use 2 rows per wave to stay within 128 VGPRs.
+    if (lds_bytes <= 40 * 1024) {
+        constexpr int R = 4, WGS = 256;
+        const int64_t tiles = ceil_div(N, R);
+        int64_t groups = ceil_div(tiles, WGS / 64);                     // one tile per wave ...
+        const int64_t cap = (int64_t)cus * 8;                           // ... until the grid is ~2 waves of groups deep
+        if (groups > cap) groups = cap;
+        auto kfn = gemv_kernel<WT, NTOK, R, WGS>;
+        if (lds_bytes > 48 * 1024) (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                           (const uint8_t *)ws, ws_stride, y, ldy);
+    } else {
+        constexpr int R = 2, WGS = 1024;
+        const int64_t tiles = ceil_div(N, R);
+        int64_t groups = ceil_div(tiles, WGS / 64);
+        if (groups > cus) groups = cus;
+        auto kfn = gemv_kernel<WT, NTOK, R, WGS>;
+        hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                           (const uint8_t *)ws, ws_stride, y, ldy);
+    }
+    return hipGetLastError();
+}
+
+template <int WT>
+static hipError_t launch_ntok(int n, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    switch (n) {
+        case 1: return launch_typed<WT, 1>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 2: return launch_typed<WT, 2>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 3: return launch_typed<WT, 3>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 4: return launch_typed<WT, 4>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 5: return launch_typed<WT, 5>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 6: return launch_typed<WT, 6>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 7: return launch_typed<WT, 7>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case 8: return launch_typed<WT, 8>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <int WT> static int max_tokens_typed(int64_t K, const DeviceLimits &lim) {
+    const size_t img = lds_image_bytes<WT>(K);
+    int64_t m = img ? (int64_t)(lim.max_lds_per_block / img) : 0;
+    return (int)(m > 8 ? 8 : m);
+}
+
+int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
+    switch (wtype) {
+        case T_Q4_0: return max_tokens_typed<T_Q4_0>(K, lim);
+        case T_Q8_0: return max_tokens_typed<T_Q8_0>(K, lim);
+        case T_Q4_K: return max_tokens_typed<T_Q4_K>(K, lim);
+        case T_Q6_K: return max_tokens_typed<T_Q6_K>(K, lim);
+        default: return 0;
+    }
+}
+
+hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                       int n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    if (N <= 0 || n <= 0) return hipSuccess;
+    switch (wtype) {
+        case T_Q4_0: return launch_ntok<T_Q4_0>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case T_Q8_0: return launch_ntok<T_Q8_0>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case T_Q4_K: return launch_ntok<T_Q4_K>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case T_Q6_K: return launch_ntok<T_Q6_K>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ isum hook
+// Per-block integer sums through the same load_w / isums device code.  One wave per (token, row); activations
+// come from reference-layout blocks and are converted to the unit form on the fly (slow path, tests only).
+template <int WT>
+__global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
+                                                        const uint8_t *__restrict__ aq, int32_t *__restrict__ isum,
+                                                        int32_t *__restrict__ imin) {
+    using T = Traits<WT>;
+    const int64_t row = blockIdx.x, t = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int units = units_per_row<WT>(K);
+    const int64_t nblk = K / (T::ACT == T_Q8_0 ? 32 : 256);
+    const size_t a_row = (size_t)(T::ACT == T_Q8_0 ? (K / 32) * BYTES_Q8_0 : (K / 256) * BYTES_Q8_K);
+    const uint8_t *arow = aq + t * a_row;
+    int32_t *out = isum + ((size_t)t * N + row) * nblk;
+    int32_t *outm = imin ? imin + ((size_t)t * N + row) * nblk : nullptr;
+    for (int u0 = 0; u0 < units; u0 += 64) {
+        const int u = u0 + lane;
+        int v0 = 0, v1 = 0;
+        if (u < units) {
+            typename T::W w;
+            T::load_w(w, W + (size_t)row * nb01, u);
+            typename T::A a;
+            // gather this unit's activation bytes from reference blocks
+            if constexpr (T::ACT == T_Q8_0) {
+                for (int b = 0; b < 2; b++) {
+                    const uint8_t *blk = arow + (size_t)(2 * u + b) * BYTES_Q8_0;
+                    int s = 0;
+                    for (int i = 0; i < 8; i++) {
+                        uint32_t d = blk[2 + 4 * i] | (blk[3 + 4 * i] << 8) | (blk[4 + 4 * i] << 16) | ((uint32_t)blk[5 + 4 * i] << 24);
+                        a.q[8 * b + i] = d;
+                        s = dot4(d, 0x01010101u, s);
+                    }
+                    if constexpr (WT == T_Q4_0) { if (b == 0) a.s0 = s; else a.s1 = s; }
+                }
+                a.d0 = a.d1 = 1.f;
+            } else {
+                const int sb = (WT == T_Q4_K) ? (u >> 3) : (u >> 2);
+                const uint8_t *blk = arow + (size_t)sb * BYTES_Q8_K;
+                const int16_t *bs = reinterpret_cast<const int16_t *>(blk + 260);
+                for (int j = 0; j < T::QCH; j++) {
+                    const size_t off = T::src_chunk(K, u, j) - (size_t)sb * 256;
+                    for (int i = 0; i < 4; i++) {
+                        const uint8_t *p = blk + 4 + off + 4 * i;
+                        a.q[4 * j + i] = p[0] | (p[1] << 8) | (p[2] << 16) | ((uint32_t)p[3] << 24);
+                    }
+                }
+                a.d = 1.f;
+                if constexpr (WT == T_Q4_K) {
+                    const int c = u & 7;
+                    a.s0 = bs[4 * (c >> 1) + (c & 1)]; a.s1 = bs[4 * (c >> 1) + 2 + (c & 1)];
+                } else {
+                    const int h = (u >> 1) & 1, ip = u & 1;
+                    for (int v = 0; v < 4; v++) a.bs[v] = bs[8 * h + 2 * v + ip];
+                }
+            }
+            T::isums(w, a, v0, v1);
+        }
+        if constexpr (T::ACT == T_Q8_0) {
+            if (u < units) { out[2 * u] = v0; out[2 * u + 1] = v1; }
+        } else {
+            // sum the units of each super-block (8 lanes for Q4_K, 4 for Q6_K) in integer arithmetic
+            constexpr int G = (WT == T_Q4_K) ? 8 : 4;
+            for (int m = 1; m < G; m <<= 1) { v0 += __shfl_xor(v0, m); v1 += __shfl_xor(v1, m); }
+            if (u < units && (lane % G) == 0) {
+                out[u / G] = v0;
+                if (outm) outm[u / G] = v1;
+            }
+        }
+    }
+}
+
+hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
+                              int32_t *isum, int32_t *imin, hipStream_t st) {
+    if (N <= 0 || n <= 0) return hipSuccess;
+    dim3 grid((unsigned)N, (unsigned)n);
+    switch (wtype) {
+        case T_Q4_0: hipLaunchKernelGGL(block_isums_kernel<T_Q4_0>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q8_0: hipLaunchKernelGGL(block_isums_kernel<T_Q8_0>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q4_K: hipLaunchKernelGGL(block_isums_kernel<T_Q4_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q6_K: hipLaunchKernelGGL(block_isums_kernel<T_Q6_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace chip

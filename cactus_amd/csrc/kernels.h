@@ -1,0 +1,33 @@
+// Internal launch interface between the C-ABI layer (capi.hip) and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+namespace chip {
+
+struct DeviceLimits {
+    int compute_units;
+    int max_lds_per_block;   // bytes one workgroup may allocate (static + dynamic)
+};
+
+// quantize.hip
+hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx, int64_t n, int64_t K, void *y,
+                           size_t y_stride, hipStream_t st);
+hipError_t launch_split_to_blocks(int act_type, const void *ws, size_t ws_stride, int64_t n, int64_t K, void *y,
+                                  size_t y_stride, hipStream_t st);
+
+// gemv.hip: y[t][r] for t < n (n <= 8 per launch), activations in the split workspace layout.
+// Returns hipErrorInvalidValue if the shape does not fit the kernel (caller splits the token range).
+int        gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim);   // tokens one launch can take (<= 8)
+hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                       int n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
+                              int32_t *isum, int32_t *imin, hipStream_t st);
+
+// gemm_q4_0.hip: int8-MFMA prefill GEMM over Q4_0 weights, activations in the split Q8_0 workspace layout.
+bool       gemm_q4_0_supported(int64_t K, int64_t N, int64_t n);
+hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                            int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+
+}  // namespace chip

@@ -1,0 +1,174 @@
+// On-the-fly activation quantizers for gfx950: fp32 rows -> Q8_0 / Q8_K, bit-identical to the reference's
+// x86 AVX2 build (reference ggml-cpu/ggml-cpu-quants.c:802-885 for Q8_0; ggml-quants.c:2473-2510 for Q8_K).
+//
+// Both kernels are pure streaming work: each lane loads one float4 (16-byte coalesced), block maxima are
+// combined with DPP moves inside the 8 (Q8_0) or 64 (Q8_K) lanes that share a block, and each lane stores
+// one packed dword of four int8 quants.  Output goes either to the reference block layout (SPLIT = false,
+// the public quantize entry points) or to the workspace planes of act_layout.h (SPLIT = true).
+//
+// Exactness notes: fp32 division is the correctly rounded one, denormals are kept, and the file is compiled
+// with -ffp-contract=off so `iscale*x + 12582912.f` rounds twice, as the C source of the reference says.
+#include "dev_common.h"
+#include "act_layout.h"
+#include "kernels.h"
+
+namespace chip {
+
+// x86 cvtps2dq semantics followed by two saturating packs: NaN or |r| >= 2^31 becomes INT_MIN -> -128.
+__device__ __forceinline__ int to_i8_x86(float r) {
+    int q = (fabsf(r) < 2147483648.f) ? (int)r : INT32_MIN;
+    return max(-128, min(127, q));
+}
+
+template <bool SPLIT>
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, int64_t ldx, int64_t K,
+                                                           uint8_t *__restrict__ y, size_t y_stride) {
+    const int64_t t = blockIdx.y;
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;      // first of this lane's 4 elements
+    const bool live = e0 < K;                                             // K % 32 == 0: whole 8-lane groups agree
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live) v = *reinterpret_cast<const float4 *>(x + t * ldx + e0);
+
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, dpp_get<0xB1>(amax));
+    amax = fmaxf(amax, dpp_get<0x4E>(amax));
+    amax = fmaxf(amax, dpp_get<0x141>(amax));                              // max over the block's 8 lanes
+
+    const float d = amax / 127.f;
+    const float id = (amax != 0.0f) ? 127.f / amax : 0.0f;
+    const int q0 = to_i8_x86(__builtin_rintf(v.x * id));
+    const int q1 = to_i8_x86(__builtin_rintf(v.y * id));
+    const int q2 = to_i8_x86(__builtin_rintf(v.z * id));
+    const int q3 = to_i8_x86(__builtin_rintf(v.w * id));
+    const uint32_t packed = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
+                            ((uint32_t)(q3 & 0xff) << 24);
+    const unsigned short dh = f2h_rne(d);
+    const int64_t blk = e0 / 32;
+    const int sub = threadIdx.x & 7;
+
+    if (SPLIT) {
+        int s = q0 + q1 + q2 + q3;
+        s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xf, 0xf, true);
+        s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xf, 0xf, true);
+        s += __builtin_amdgcn_update_dpp(0, s, 0x141, 0xf, 0xf, true);
+        if (live) {
+            uint8_t *base = y + t * y_stride;
+            *reinterpret_cast<uint32_t *>(base + e0) = packed;
+            if (sub == 0) {
+                reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = h2f(dh);
+                reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = s;
+            }
+        }
+    } else if (live) {
+        uint8_t *b = y + t * y_stride + blk * BYTES_Q8_0;
+        *reinterpret_cast<u32_a2 *>(b + 2 + 4 * sub) = packed;
+        if (sub == 0) *reinterpret_cast<unsigned short *>(b) = dh;
+    }
+}
+
+template <bool SPLIT>
+__global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float *__restrict__ x, int64_t ldx, int64_t K,
+                                                           uint8_t *__restrict__ y, size_t y_stride) {
+    const int64_t t = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);       // one wave per 256-value super-block
+    if (sb * QK_K >= K) return;                                           // whole wave leaves together
+    const float4 v = *reinterpret_cast<const float4 *>(x + t * ldx + sb * QK_K + lane * 4);
+
+    // (amax, max): the first element with the largest magnitude decides, sign kept (strict > in index order)
+    float cand = v.x;
+    if (fabsf(v.y) > fabsf(cand)) cand = v.y;
+    if (fabsf(v.z) > fabsf(cand)) cand = v.z;
+    if (fabsf(v.w) > fabsf(cand)) cand = v.w;
+    const float amax = wave_max_all(fabsf(cand));
+    const unsigned long long holders = __ballot(fabsf(cand) == amax);
+    const int first = __builtin_ctzll(holders);
+    const float mx = __shfl(cand, first);
+
+    int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+    float d = 0.f;
+    if (amax != 0.0f) {
+        const float iscale = -127.f / mx;
+        auto nearest = [](float f) {
+            const float m = f + 12582912.f;
+            return (int)(__float_as_uint(m) & 0x007fffffu) - 0x00400000;
+        };
+        q0 = min(127, nearest(iscale * v.x));
+        q1 = min(127, nearest(iscale * v.y));
+        q2 = min(127, nearest(iscale * v.z));
+        q3 = min(127, nearest(iscale * v.w));
+        d = 1.0f / iscale;
+    }
+    const uint32_t packed = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
+                            ((uint32_t)(q3 & 0xff) << 24);
+    int s = q0 + q1 + q2 + q3;                                             // 16 values = 4 lanes
+    s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xf, 0xf, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xf, 0xf, true);
+
+    if (SPLIT) {
+        uint8_t *base = y + t * y_stride;
+        *reinterpret_cast<uint32_t *>(base + sb * QK_K + lane * 4) = packed;
+        if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(K))[sb] = d;
+        if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(K))[sb * 16 + (lane >> 2)] = (int16_t)s;
+    } else {
+        uint8_t *b = y + t * y_stride + sb * BYTES_Q8_K;
+        *reinterpret_cast<uint32_t *>(b + 4 + lane * 4) = packed;
+        if (lane == 0) *reinterpret_cast<float *>(b) = d;
+        if ((lane & 3) == 0) *reinterpret_cast<int16_t *>(b + 260 + 2 * (lane >> 2)) = (int16_t)s;
+    }
+}
+
+// Inverse of the split layout: rebuild reference blocks from workspace planes (verification only).
+__global__ void split_to_blocks_q8_0_kernel(const uint8_t *__restrict__ ws, size_t ws_stride, int64_t K,
+                                            uint8_t *__restrict__ y, size_t y_stride) {
+    const int64_t t = blockIdx.y;
+    const int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (blk >= K / 32) return;
+    const uint8_t *base = ws + t * ws_stride;
+    uint8_t *b = y + t * y_stride + blk * BYTES_Q8_0;
+    *reinterpret_cast<unsigned short *>(b) = f2h_rne(reinterpret_cast<const float *>(base + q8_0_off_d(K))[blk]);
+    for (int i = 0; i < 32; i++) b[2 + i] = base[blk * 32 + i];
+}
+__global__ void split_to_blocks_q8_K_kernel(const uint8_t *__restrict__ ws, size_t ws_stride, int64_t K,
+                                            uint8_t *__restrict__ y, size_t y_stride) {
+    const int64_t t = blockIdx.y;
+    const int64_t sb = blockIdx.x;
+    const int i = threadIdx.x;                                             // 256 threads
+    const uint8_t *base = ws + t * ws_stride;
+    uint8_t *b = y + t * y_stride + sb * BYTES_Q8_K;
+    b[4 + i] = base[sb * QK_K + i];
+    if (i == 0) *reinterpret_cast<float *>(b) = reinterpret_cast<const float *>(base + q8_K_off_d(K))[sb];
+    if (i < 16)
+        *reinterpret_cast<int16_t *>(b + 260 + 2 * i) = reinterpret_cast<const int16_t *>(base + q8_K_off_bsums(K))[sb * 16 + i];
+}
+
+hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx, int64_t n, int64_t K, void *y,
+                           size_t y_stride, hipStream_t st) {
+    if (n <= 0 || K <= 0) return hipSuccess;
+    dim3 grid((unsigned)ceil_div(K, 1024), (unsigned)n);
+    if (act_type == T_Q8_0) {
+        if (split) hipLaunchKernelGGL(quantize_q8_0_kernel<true>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+        else       hipLaunchKernelGGL(quantize_q8_0_kernel<false>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+    } else {
+        if (split) hipLaunchKernelGGL(quantize_q8_K_kernel<true>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+        else       hipLaunchKernelGGL(quantize_q8_K_kernel<false>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_split_to_blocks(int act_type, const void *ws, size_t ws_stride, int64_t n, int64_t K, void *y,
+                                  size_t y_stride, hipStream_t st) {
+    if (n <= 0 || K <= 0) return hipSuccess;
+    if (act_type == T_Q8_0) {
+        dim3 grid((unsigned)ceil_div(K / 32, 256), (unsigned)n);
+        hipLaunchKernelGGL(split_to_blocks_q8_0_kernel, grid, dim3(256), 0, st, (const uint8_t *)ws, ws_stride, K,
+                           (uint8_t *)y, y_stride);
+    } else {
+        dim3 grid((unsigned)(K / 256), (unsigned)n);
+        hipLaunchKernelGGL(split_to_blocks_q8_K_kernel, grid, dim3(256), 0, st, (const uint8_t *)ws, ws_stride, K,
+                           (uint8_t *)y, y_stride);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace chip

@@ -1,0 +1,133 @@
+/*
+ * cactus_hip.h -- C-ABI of libcactus_hip.so: the MI355X (gfx950) kernels for the quantized MUL_MAT path.
+ *
+ * Plain pointers, sizes and integer return codes only; no ggml, torch or C++ types.  The ggml backend
+ * (ggml_backend_hip.h / libggml-hip.so) sits on top of this layer; tests and benchmarks bind it with ctypes.
+ *
+ * Every entry point names the reference interface it replaces (paths relative to the reference's cactus/
+ * directory).  All device pointers are plain HIP device addresses; `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  Calls are asynchronous with respect to the host unless stated otherwise.
+ *
+ * Return value: 0 on success, a negative CHIP_E* code on a rejected argument, a positive hipError_t value
+ * if the HIP runtime failed.  chip_error_string() renders either.
+ */
+#ifndef CACTUS_HIP_H
+#define CACTUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CHIP_API __attribute__((visibility("default")))
+
+/* weight / activation type ids: the reference's lm_ggml_type values (ggml.h:351-391) */
+enum chip_type {
+    CHIP_TYPE_F32  = 0,
+    CHIP_TYPE_Q4_0 = 2,
+    CHIP_TYPE_Q8_0 = 8,
+    CHIP_TYPE_Q4_K = 12,
+    CHIP_TYPE_Q6_K = 14,
+    CHIP_TYPE_Q8_K = 15,
+};
+
+enum chip_status {
+    CHIP_OK            = 0,
+    CHIP_EINVAL        = -1,   /* NULL pointer, negative size, misaligned pointer or stride */
+    CHIP_EUNSUPPORTED  = -2,   /* type or shape outside what the kernels implement */
+    CHIP_ENOMEM        = -3,   /* workspace too small */
+    CHIP_ENODEVICE     = -4,   /* no gfx950 device visible */
+};
+
+typedef struct chip_device_info {
+    int    device;             /* HIP ordinal */
+    int    compute_units;
+    int    wavefront_size;
+    int    max_lds_per_block;  /* bytes a single workgroup may use */
+    int    clock_khz;
+    int    xcd_count;          /* 0 if the runtime does not say */
+    size_t hbm_total;
+    size_t hbm_free;
+    char   name[128];
+    char   arch[64];
+} chip_device_info;
+
+/* ---- device and memory plumbing (what a ggml device/buffer needs; replaces nothing in the CPU path) ---- */
+CHIP_API int         chip_init(int device);                    /* selects the device, checks it is gfx950 */
+CHIP_API int         chip_device_count(void);
+CHIP_API int         chip_get_device_info(chip_device_info *out);
+CHIP_API const char *chip_error_string(int code);
+CHIP_API int         chip_malloc(void **dptr, size_t bytes);
+CHIP_API int         chip_free(void *dptr);
+CHIP_API int         chip_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);   /* synchronous if stream == NULL */
+CHIP_API int         chip_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
+CHIP_API int         chip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+CHIP_API int         chip_memset(void *dst, int value, size_t bytes, void *stream);
+CHIP_API int         chip_stream_create(void **stream);
+CHIP_API int         chip_stream_destroy(void *stream);
+CHIP_API int         chip_stream_synchronize(void *stream);
+
+/* ---- layout facts ---- */
+/* lm_ggml_blck_size / lm_ggml_type_size / lm_ggml_row_size (ggml.c:1186-1200) for the types above; 0 if unknown */
+CHIP_API int    chip_block_elems(int type);
+CHIP_API size_t chip_block_bytes(int type);
+CHIP_API size_t chip_row_size(int type, int64_t k);
+/* type_traits_cpu[type].vec_dot_type (ggml-cpu/ggml-cpu.c:198-367): Q8_0 for Q4_0/Q8_0, Q8_K for Q4_K/Q6_K */
+CHIP_API int    chip_vec_dot_type(int type);
+/* 1 if chip_mul_mat accepts this weight type and K (K must be a multiple of 256) */
+CHIP_API int    chip_mul_mat_supported(int type, int64_t K);
+
+/* ---- activation quantizers ----
+ * quantize_row_q8_0, AVX2 branch (ggml-cpu/ggml-cpu-quants.c:732-738,802-885) and quantize_row_q8_K
+ * (ggml-cpu/ggml-cpu-quants.c:1740,1819-1821 -> ggml-quants.c:2473-2510), for n rows at once.
+ *   x       : n rows of k floats, row t at x + t*ldx (ldx in elements, >= k)
+ *   y       : n rows of chip_row_size(type, k) bytes, packed, in the reference's block layout
+ * Output bytes equal the reference's bit for bit (an all-zero Q8_K block gets zero bsums, which the
+ * reference leaves unwritten). */
+CHIP_API int chip_quantize_q8_0(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
+CHIP_API int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
+
+/* ---- the op: LM_GGML_OP_MUL_MAT over block-quantized weights ----
+ * lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449) with src0 = W (type, [K, N], row stride
+ * nb01 bytes, GGUF block layout untouched), src1 = x (F32 [K, n], row stride ldx elements), dst = y
+ * (F32 [N, n], row stride ldy elements):  y[t][r] = vec_dot(W row r, quantize(x row t)).
+ *
+ *   workspace : device scratch of at least chip_mul_mat_workspace_size(type, K, n) bytes (params->wdata in the
+ *               reference, sized by lm_ggml_graph_plan, ggml-cpu/ggml-cpu.c:2697-2704); holds the quantized
+ *               activations in a kernel-private layout
+ * n <= 8 runs the bandwidth-bound GEMV; larger n runs the int8-MFMA GEMM (Q4_0) or the GEMV in token groups.
+ * K must be a multiple of 256.  W must be 16-byte aligned and nb01 a multiple of 16 (2 and 2 for Q6_K, whose
+ * 210-byte blocks allow no more); x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
+ */
+CHIP_API size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n);
+CHIP_API int    chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N,
+                             const float *x, int64_t ldx, int64_t n,
+                             float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+
+/* The two phases of chip_mul_mat separately (Phase A / Phase B of the reference op, ggml-cpu/ggml-cpu.c:1319-1354
+ * and :1380-1448), so one quantized activation can feed several matmuls (wq/wk/wv share an input, as do
+ * ffn_up/ffn_gate).  chip_mul_mat_prepare fills `workspace` from x; chip_mul_mat_run consumes it.
+ * The workspace contents depend on (vec_dot_type of `type`, K, n) only. */
+CHIP_API int chip_mul_mat_prepare(int type, int64_t K, const float *x, int64_t ldx, int64_t n,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,
+                              const void *workspace, float *y, int64_t ldy, void *stream);
+
+/* ---- verification hooks ----
+ * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K}
+ * (ggml-cpu/ggml-cpu-quants.c:1906,3591,6772,8520), computed with the same device code the GEMV uses.
+ *   aq   : n rows of activations in the reference block layout (chip_quantize_q8_0 / _q8_K output)
+ *   isum : [n][N][K/block] int32; for Q4_K/Q6_K one value per 256-block (sum over sub-blocks of scale*dot)
+ *   imin : Q4_K only, [n][N][K/256] int32 (sum of min_j * bsum pairs); NULL otherwise */
+CHIP_API int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
+                              const void *aq, int64_t n, int32_t *isum, int32_t *imin, void *stream);
+/* Rebuilds the reference block layout from a prepared workspace (inverse of the kernel-private layout), so
+ * tests can check that the fused prepare step quantizes bit-identically to chip_quantize_q8_0/_q8_K. */
+CHIP_API int chip_workspace_to_blocks(int type, int64_t K, int64_t n, const void *workspace, void *y, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -636,7 +636,6 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
     if (!be) return NAN;
     const int64_t nb = k / be;
     int32_t *is = (int32_t *)malloc(sizeof(int32_t) * (size_t)(nb > 0 ? nb : 1) * 2);
-    int32_t *im = is + (nb > 0 ? nb : 1);
     if (type == ORC_TYPE_Q4_0 || type == ORC_TYPE_Q8_0) {
         if (type == ORC_TYPE_Q4_0) orc_vec_dot_q4_0_q8_0(k, vx, vy, is);
         else                       orc_vec_dot_q8_0_q8_0(k, vx, vy, is);
@@ -647,22 +646,44 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
             s += t; sa += fabs(t);
         }
     } else if (type == ORC_TYPE_Q4_K) {
-        orc_vec_dot_q4_K_q8_K(k, vx, vy, is, im);
+        /* terms at sub-block granularity (32 values with their own 6-bit scale and min) */
         const blk_q4_K *x = (const blk_q4_K *)vx;
         const blk_q8_K *y = (const blk_q8_K *)vy;
         for (int64_t b = 0; b < nb; b++) {
-            const double t1 = (double)y[b].d * (double)H2F(x[b].d) * (double)is[b];
-            const double t2 = (double)y[b].d * (double)H2F(x[b].dmin) * (double)im[b];
-            s += t1 - t2; sa += fabs(t1) + fabs(t2);
+            const double d = (double)y[b].d * (double)H2F(x[b].d), dm = (double)y[b].d * (double)H2F(x[b].dmin);
+            for (int j = 0; j < 8; j++) {
+                uint8_t sc, m;
+                unpack_sc_m(j, x[b].scales, &sc, &m);
+                const uint8_t *q4 = x[b].qs + 32 * (j / 2);
+                const int8_t *q8 = y[b].qs + 32 * j;
+                int64_t dot = 0;
+                for (int l = 0; l < 32; l++) dot += (int64_t)((j & 1) ? (q4[l] >> 4) : (q4[l] & 0xF)) * q8[l];
+                const double t1 = d * (double)sc * (double)dot;
+                const double t2 = dm * (double)m * (double)(y[b].bsums[2 * j] + y[b].bsums[2 * j + 1]);
+                s += t1 - t2; sa += fabs(t1) + fabs(t2);
+            }
         }
     } else if (type == ORC_TYPE_Q6_K) {
-        orc_vec_dot_q6_K_q8_K(k, vx, vy, is);
+        /* terms at sub-block granularity (16 values with their own int8 scale) */
+        const int64_t n6 = k;
+        float *wi = (float *)malloc(sizeof(float) * (size_t)(n6 > 0 ? n6 : 1));
+        blk_q6_K *tmp = (blk_q6_K *)malloc(sizeof(blk_q6_K) * (size_t)(nb > 0 ? nb : 1));
         const blk_q6_K *x = (const blk_q6_K *)vx;
         const blk_q8_K *y = (const blk_q8_K *)vy;
+        /* dequantize with d = 1 and unit scales to recover the integers q-32 in element order */
+        memcpy(tmp, x, sizeof(blk_q6_K) * (size_t)nb);
+        for (int64_t b = 0; b < nb; b++) { tmp[b].d = 0x3c00; for (int g = 0; g < 16; g++) tmp[b].scales[g] = 1; }
+        orc_dequantize_row(ORC_TYPE_Q6_K, tmp, wi, k);
         for (int64_t b = 0; b < nb; b++) {
-            const double t = (double)y[b].d * (double)H2F(x[b].d) * (double)is[b];
-            s += t; sa += fabs(t);
+            const double d = (double)y[b].d * (double)H2F(x[b].d);
+            for (int g = 0; g < 16; g++) {
+                int64_t dot = 0;
+                for (int l = 0; l < 16; l++) dot += (int64_t)wi[256 * b + 16 * g + l] * y[b].qs[16 * g + l];
+                const double t = d * (double)x[b].scales[g] * (double)dot;
+                s += t; sa += fabs(t);
+            }
         }
+        free(wi); free(tmp);
     } else { s = NAN; }
     free(is);
     if (sum_abs) *sum_abs = sa;

@@ -84,8 +84,11 @@ float orc_vec_dot_q4_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *
 float orc_vec_dot_q6_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
 
-/* fp64 evaluation of sum_b scale_b*isum_b (returned) and of sum_b |scale_b*isum_b| (*sum_abs; for Q4_K the
- * |dmin term| is included): the tolerance yardstick 1e-5 * sum_abs and an order-free reference value. */
+/* fp64 evaluation of sum_b scale_b*isum_b (returned) and of sum_b |scale_b*isum_b| (*sum_abs): the tolerance
+ * yardstick 1e-5 * sum_abs and an order-free reference value.  A "block" is the smallest group of values that
+ * carries its own scale: 32 values for Q4_0/Q8_0, a 32-value sub-block for Q4_K (terms d*sc_j*dot_j and
+ * dmin*m_j*bsum_j, both counted), a 16-value sub-block for Q6_K (d*sc_j*dot_j).  Coarser terms (whole
+ * super-blocks) would cancel internally and make a bound that the reference's own AVX2 result misses. */
 double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, double *sum_abs);
 
 /*

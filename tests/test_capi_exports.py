@@ -1,0 +1,39 @@
+"""CPU-only: the C-ABI library is present, loads, and exports every symbol include/cactus_hip.h declares.
+No compute call is made (there is no GPU here)."""
+import ctypes
+import os
+import re
+
+import cactus_amd
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    return sorted(set(re.findall(r"CHIP_API\s+[\w\s\*]+?\b(chip_\w+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_symbols("cactus_hip.h") == sorted(cactus_amd.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(cactus_amd.KERNEL_LIB)
+    for name in declared_symbols("cactus_hip.h"):
+        assert hasattr(lib, name), name
+
+
+def test_layout_queries_need_no_gpu():
+    lib = cactus_amd.load_library()
+    assert [lib.chip_block_bytes(t) for t in (2, 8, 12, 14, 15)] == [18, 34, 144, 210, 292]
+    assert lib.chip_row_size(cactus_amd.Q4_0, 4096) == 2304
+    assert lib.chip_row_size(cactus_amd.Q4_K, 4096) == 2304
+    assert lib.chip_row_size(cactus_amd.Q6_K, 14336) == 11760
+    assert lib.chip_vec_dot_type(cactus_amd.Q4_0) == cactus_amd.Q8_0
+    assert lib.chip_vec_dot_type(cactus_amd.Q6_K) == cactus_amd.Q8_K
+    assert lib.chip_mul_mat_supported(cactus_amd.Q4_K, 4096) == 1
+    assert lib.chip_mul_mat_supported(cactus_amd.Q4_K, 4000) == 0
+    assert lib.chip_mul_mat_supported(1, 4096) == 0           # F16 weights are not on this path
+    assert lib.chip_mul_mat_workspace_size(cactus_amd.Q8_0, 4096, 3) == 3 * (4096 + 8 * 128)
+    assert lib.chip_error_string(-2).decode().startswith("unsupported")
