@@ -1,0 +1,355 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized MUL_MAT hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): Q8_0 x Q8_0 decode GEMV at Llama FFN shapes, W[11008 x 4096]
+and W[4096 x 11008], token batch n in {1, 2, 4, 8}.  One "step" = the eight ops (2 shapes x 4 batch sizes),
+each op being what LM_GGML_OP_MUL_MAT does: quantize the fp32 activations to Q8_0 on the GPU, then the GEMV.
+Inputs are resident in HBM before the timed region; weights rotate through > 512 MB of distinct copies per
+shape so that the 256 MB Infinity Cache cannot serve them (cold numbers).
+
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a step (HIP events on the launch
+stream).  `roofline` is for the dominant kernel, the n = 1 GEMV, timed with its own HIP event pairs inside the
+timed region.  `cpu_baseline` times the reference's own ggml-cpu MUL_MAT (oracle/_ref, when it travelled) or the
+oracle port on the host cores for a bounded sample of the same workload.  `extra` carries the other BASELINE
+configurations (Q4_0 mat-vec, Q4_K GEMV, prefill GEMM TOPS, Llama-3-8B-shaped decode trace).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+class Hip:
+    """The few HIP runtime calls the harness needs beyond the C-ABI: events and graph capture."""
+
+    def __init__(self):
+        self.lib = L = C.CDLL("libamdhip64.so")
+        L.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        L.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        L.hipEventSynchronize.argtypes = [C.c_void_p]
+        L.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        L.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        L.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        L.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        L.hipDeviceSynchronize.argtypes = []
+
+    def event(self):
+        e = C.c_void_p()
+        assert self.lib.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.lib.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.lib.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.lib.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return ms.value
+
+
+def synth_weights(dev, wtype, N, K, rng):
+    """Random-init weights directly in block form: random quants, a fixed small fp16 scale per block."""
+    L = dev.lib
+    be, bb = L.chip_block_elems(wtype), L.chip_block_bytes(wtype)
+    w = rng.integers(0, 256, (N, K // be, bb), dtype=np.uint8)
+    d = np.array([0.0107], np.float16).view(np.uint8)
+    if wtype in (2, 8):
+        w[..., 0:2] = d
+    elif wtype == 12:
+        w[..., 0:2] = d
+        w[..., 2:4] = d
+    else:
+        w[..., 208:210] = d
+    return w.reshape(N, -1)
+
+
+class RotatingWeights:
+    """`copies` distinct copies of one weight matrix in HBM, handed out round robin (cold-cache reads)."""
+
+    def __init__(self, dev, wtype, N, K, rng, min_bytes=640e6, host=None):
+        self.dev, self.wtype, self.N, self.K = dev, wtype, N, K
+        self.nb01 = dev.row_size(wtype, K)
+        self.bytes = N * self.nb01
+        self.copies = max(2, int(min_bytes // self.bytes) + 1)
+        self.host = synth_weights(dev, wtype, N, K, rng) if host is None else host
+        self.buf = dev.alloc(self.copies * self.bytes)
+        self.buf.upload(self.host)
+        for c in range(1, self.copies):
+            dev.check(dev.lib.chip_memcpy_d2d(self.buf.ptr + c * self.bytes, self.buf.ptr, self.bytes, None))
+        dev.sync()
+        self.i = 0
+
+    def next(self):
+        p = self.buf.ptr + (self.i % self.copies) * self.bytes
+        self.i += 1
+        return p
+
+
+def algorithmic_bytes(wbytes, K, N, n):
+    return wbytes + 4 * n * (K + N)            # weights once + fp32 activations in + fp32 outputs out
+
+
+def bench_headline(dev, hip, steps, warmup):
+    import cactus_amd as ca
+    L = dev.lib
+    rng = np.random.default_rng(2)
+    shapes = [(11008, 4096), (4096, 11008)]
+    batches = [1, 2, 4, 8]
+    mats = [RotatingWeights(dev, ca.Q8_0, N, K, rng) for (N, K) in shapes]
+    xs = {K: dev.to_device(rng.standard_normal((8, K)).astype(np.float32)) for (_, K) in shapes}
+    ys = dev.alloc(8 * 11008 * 4)
+    wsz = max(L.chip_mul_mat_workspace_size(ca.Q8_0, K, 8) for (_, K) in shapes)
+    ws = dev.alloc(wsz)
+    st = C.c_void_p()
+    dev.check(L.chip_stream_create(C.byref(st)))
+
+    n1_events = []
+
+    def step(timed):
+        for m in mats:
+            for n in batches:
+                dev.check(L.chip_mul_mat_prepare(ca.Q8_0, m.K, xs[m.K].ptr, m.K, n, ws.ptr, wsz, st))
+                if timed and n == 1:
+                    a, b = hip.event(), hip.event()
+                    hip.record(a, st)
+                dev.check(L.chip_mul_mat_run(ca.Q8_0, m.next(), m.nb01, m.K, m.N, n, ws.ptr, ys.ptr, m.N, st))
+                if timed and n == 1:
+                    hip.record(b, st)
+                    n1_events.append((a, b))
+
+    for _ in range(warmup):
+        step(False)
+    dev.sync(st)
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, st)
+    for _ in range(steps):
+        step(True)
+    hip.record(e1, st)
+    ms = hip.elapsed_ms(e0, e1)
+    dev.sync(st)
+
+    step_bytes = sum(algorithmic_bytes(m.bytes, m.K, m.N, n) for m in mats for n in batches)
+    ms_per_step = ms / steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    k_us = float(np.mean([hip.elapsed_ms(a, b) for a, b in n1_events])) * 1e3
+    k_bytes = algorithmic_bytes(mats[0].bytes, 4096, 11008, 1)      # both shapes move the same byte count
+    achieved = k_bytes / (k_us * 1e-6) / 1e9
+    roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "gemv_kernel<Q8_0, n=1> (W[11008x4096] and W[4096x11008], cold weights)",
+            "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 2)}
+    return value, ms_per_step, step_bytes, roof, {"copies_per_shape": [m.copies for m in mats]}
+
+
+def time_runs(dev, hip, st, fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    dev.sync(st)
+    a, b = hip.event(), hip.event()
+    hip.record(a, st)
+    for _ in range(iters):
+        fn()
+    hip.record(b, st)
+    return hip.elapsed_ms(a, b) * 1e3 / iters          # microseconds per call
+
+
+def bench_extra(dev, hip):
+    import cactus_amd as ca
+    L = dev.lib
+    rng = np.random.default_rng(5)
+    st = C.c_void_p()
+    dev.check(L.chip_stream_create(C.byref(st)))
+    out = {}
+
+    def gemv_case(name, wt, N, K, n, iters=200):
+        m = RotatingWeights(dev, wt, N, K, rng)
+        x = dev.to_device(rng.standard_normal((n, K)).astype(np.float32))
+        y = dev.alloc(n * N * 4)
+        wsz = L.chip_mul_mat_workspace_size(wt, K, n)
+        ws = dev.alloc(wsz)
+        dev.check(L.chip_mul_mat_prepare(wt, K, x.ptr, K, n, ws.ptr, wsz, st))
+        us_run = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run(wt, m.next(), m.nb01, K, N, n, ws.ptr, y.ptr, N, st), iters)
+        us_op = time_runs(dev, hip, st, lambda: L.chip_mul_mat(wt, m.next(), m.nb01, K, N, x.ptr, K, n, y.ptr, N, ws.ptr, wsz, st), iters)
+        b = algorithmic_bytes(m.bytes, K, N, n)
+        out[name] = {"us_gemv": round(us_run, 2), "us_op": round(us_op, 2), "GBps_gemv": round(b / us_run / 1e3, 1),
+                     "GBps_op": round(b / us_op / 1e3, 1), "hbm_frac_gemv": round(b / us_run / 1e3 / HBM_PEAK_GBS, 4),
+                     "bytes": b, "cold_copies": m.copies}
+        m.buf.free()
+
+    gemv_case("config1_q4_0_4096x4096_n1", ca.Q4_0, 4096, 4096, 1)
+    gemv_case("config3_q4_K_14336x4096_n1", ca.Q4_K, 14336, 4096, 1)
+
+    # config 4: prefill GEMM on int8 MFMA
+    for (N, M) in ((4096, 512), (4096, 2048), (14336, 512), (14336, 2048)):
+        K = 4096
+        w = dev.to_device(synth_weights(dev, ca.Q4_0, N, K, rng))
+        x = dev.to_device(rng.standard_normal((M, K)).astype(np.float32))
+        y = dev.alloc(M * N * 4)
+        wsz = L.chip_mul_mat_workspace_size(ca.Q4_0, K, M)
+        ws = dev.alloc(wsz)
+        nb01 = dev.row_size(ca.Q4_0, K)
+        dev.check(L.chip_mul_mat_prepare(ca.Q4_0, K, x.ptr, K, M, ws.ptr, wsz, st))
+        us_g = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run(ca.Q4_0, w.ptr, nb01, K, N, M, ws.ptr, y.ptr, N, st), 20)
+        us_o = time_runs(dev, hip, st, lambda: L.chip_mul_mat(ca.Q4_0, w.ptr, nb01, K, N, x.ptr, K, M, y.ptr, N, ws.ptr, wsz, st), 20)
+        ops = 2.0 * M * N * K
+        out["config4_q4_0_%dx4096_M%d" % (N, M)] = {
+            "us_gemm": round(us_g, 1), "us_op": round(us_o, 1), "TOPS_gemm": round(ops / us_g / 1e6, 1),
+            "TOPS_op": round(ops / us_o / 1e6, 1), "int8_frac_gemm": round(ops / us_g / 1e6 / INT8_PEAK_TOPS, 4)}
+        for b in (w, x, y, ws):
+            b.free()
+
+    out.update(bench_trace(dev, hip, st, rng))
+    return out
+
+
+def bench_trace(dev, hip, st, rng):
+    """config 5: every weight matmul of one decode step of a Llama-3-8B-shaped Q4_K_M model (32 layers, 225
+    matmuls; attn_v / ffn_down / output head in Q6_K, the rest Q4_K), replayed as a HIP graph."""
+    import cactus_amd as ca
+    L = dev.lib
+    H, FF, KV, V, NL = 4096, 14336, 1024, 128256, 32
+    layer = [("wq", ca.Q4_K, H, H, "attn"), ("wk", ca.Q4_K, KV, H, "attn"), ("wv", ca.Q6_K, KV, H, "attn"),
+             ("wo", ca.Q4_K, H, H, "wo"), ("up", ca.Q4_K, FF, H, "ffn"), ("gate", ca.Q4_K, FF, H, "ffn"),
+             ("down", ca.Q6_K, H, FF, "down")]
+    sizes = [N * dev.row_size(t, K) for (_, t, N, K, _) in layer]
+    layer_bytes = sum(sizes)
+    head_bytes = V * dev.row_size(ca.Q6_K, H)
+    total = NL * layer_bytes + head_bytes
+    arena = dev.alloc(total)
+    off = 0
+    first = []
+    for (name, t, N, K, _), sz in zip(layer, sizes):
+        arena.upload(synth_weights(dev, t, N, K, rng), offset=off)
+        first.append(off)
+        off += sz
+    for l in range(1, NL):
+        dev.check(L.chip_memcpy_d2d(arena.ptr + l * layer_bytes, arena.ptr, layer_bytes, None))
+    head_off = NL * layer_bytes
+    part = V // 8
+    arena.upload(synth_weights(dev, ca.Q6_K, part, H, rng), offset=head_off)
+    for i in range(1, 8):
+        dev.check(L.chip_memcpy_d2d(arena.ptr + head_off + i * (head_bytes // 8), arena.ptr + head_off, head_bytes // 8, None))
+    dev.sync()
+
+    res = {}
+    for n in (1, 8):
+        x_h = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
+        x_ff = dev.to_device(rng.standard_normal((n, FF)).astype(np.float32))
+        y = dev.alloc(n * V * 4)
+        wsz = max(L.chip_mul_mat_workspace_size(ca.Q6_K, FF, n), L.chip_mul_mat_workspace_size(ca.Q4_K, H, n))
+        ws = dev.alloc(wsz)
+
+        def one_step():
+            for l in range(NL):
+                base = arena.ptr + l * layer_bytes
+                prepared = None
+                for (name, t, N, K, grp), o in zip(layer, first):
+                    if grp != prepared:            # wq/wk/wv share one quantized input, as do up/gate
+                        src = x_ff if K == FF else x_h
+                        dev.check(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, ws.ptr, wsz, st))
+                        prepared = grp
+                    dev.check(L.chip_mul_mat_run(t, base + o, dev.row_size(t, K), K, N, n, ws.ptr, y.ptr, N, st))
+            dev.check(L.chip_mul_mat_prepare(ca.Q6_K, H, x_h.ptr, H, n, ws.ptr, wsz, st))
+            dev.check(L.chip_mul_mat_run(ca.Q6_K, arena.ptr + head_off, dev.row_size(ca.Q6_K, H), H, V, n, ws.ptr, y.ptr, V, st))
+
+        one_step()
+        dev.sync(st)
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.lib.hipStreamBeginCapture(st, 0) == 0
+        one_step()
+        assert hip.lib.hipStreamEndCapture(st, C.byref(graph)) == 0
+        assert hip.lib.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        us = time_runs(dev, hip, st, lambda: hip.lib.hipGraphLaunch(gexec, st), 20, warm=2)
+        b = total + 4 * n * (NL * sum(K + N for (_, _, N, K, _) in layer) + H + V)
+        res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = {
+            "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1), "weight_bytes": total,
+            "GBps": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4), "matmuls": 7 * NL + 1}
+        for bf in (x_h, x_ff, y, ws):
+            bf.free()
+    arena.free()
+    return res
+
+
+def cpu_baseline(step_bytes_n):
+    """Reference ggml-cpu MUL_MAT (oracle/_ref) or the oracle port on the host cores, bounded sample:
+    the two headline shapes at n = 1 and n = 8."""
+    import oracle as O
+    cores = min(16, os.cpu_count() or 1)
+    rng = np.random.default_rng(2)
+    use_ref = O.Reference.available()
+    eng = O.Reference() if use_ref else O.Oracle()
+    t_total, b_total, budget = 0.0, 0, 20.0
+    t_start = time.perf_counter()
+    for (N, K) in ((11008, 4096), (4096, 11008)):
+        w = rng.integers(0, 256, (N, K // 32, 34), dtype=np.uint8)
+        w[..., 0:2] = np.array([0.0107], np.float16).view(np.uint8)
+        w = w.reshape(N, -1)
+        for n in (1, 8):
+            x = rng.standard_normal((n, K)).astype(np.float32)
+            if use_ref:
+                _, times = eng.mul_mat_graph(O.Q8_0, w, x, nthreads=cores, repeat=12)
+                t = float(np.median(times[2:]))
+            else:
+                t0 = time.perf_counter()
+                eng.mul_mat(O.Q8_0, w, x, nthreads=cores)
+                t = time.perf_counter() - t0
+            t_total += t
+            b_total += w.size + 4 * n * (K + N)
+            if time.perf_counter() - t_start > budget:
+                break
+    return {"value": round(b_total / t_total / 1e9, 2), "unit": "GB/s", "cores": cores,
+            "kind": "reference" if use_ref else "port",
+            "sample": "Q8_0 W[11008x4096] and W[4096x11008] at n=1 and n=8, median of 10 calls each, "
+                      "%s with a persistent %d-thread pool" % ("reference ggml-cpu MUL_MAT graph (AVX2 build)" if use_ref
+                                                               else "oracle restatement", cores)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (every figure is single-GPU)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import cactus_amd as ca
+    dev = ca.Device(0)
+    hip = Hip()
+    value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, args.steps, args.warmup)
+    extra = {} if args.no_extra else bench_extra(dev, hip)
+    cpu = None if args.no_cpu else cpu_baseline(step_bytes)
+    line = {
+        "metric": "quant mul_mat GEMV HBM GB/s & prefill int8 TOPS (% of roofline), 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: Q8_0 x Q8_0 decode GEMV, W[11008x4096] and W[4096x11008], "
+                               "n in {1,2,4,8}; step = 8 ops (GPU Q8_0 activation quantize + GEMV each); cold weights",
+                   "bytes_per_step": step_bytes, "device": dev.info.arch.decode(), **info},
+        "roofline": roof, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
