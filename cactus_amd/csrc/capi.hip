@@ -262,6 +262,20 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
 
 int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
                  float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (n >= 1 && n <= 4 && N > 0 && chip_mul_mat_supported(type, K)) {
+        // decode: one launch that quantizes in the GEMV prologue (argument checks as in prepare + run)
+        DeviceLimits lim;
+        int rc0 = current_limits(lim);
+        if (rc0) return rc0;
+        if (gemv_fused_applicable(type, K, (int)n, lim)) {
+            if (!x || !workspace || ldx < K || !W || !y || ldy < N) return CHIP_EINVAL;
+            if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0) return CHIP_EINVAL;
+            if (!weights_aligned(type, W, nb01) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
+            if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+            return hip_rc(launch_gemv_fused(type, W, nb01, K, N, x, ldx, (int)n, workspace,
+                                            act_stride(chip_vec_dot_type(type), K), y, ldy, lim, (hipStream_t)stream));
+        }
+    }
     int rc = chip_mul_mat_prepare(type, K, x, ldx, n, workspace, workspace_bytes, stream);
     if (rc) return rc;
     return chip_mul_mat_run(type, W, nb01, K, N, n, workspace, y, ldy, stream);

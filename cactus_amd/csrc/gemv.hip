@@ -8,15 +8,19 @@
 //     of every row, a unit being the smallest piece that carries whole scales (two 32-blocks for Q4_0/Q8_0,
 //     1/8 of a Q4_K super-block, 1/4 of a Q6_K super-block).  Consecutive lanes read consecutive bytes, so a
 //     wave's loads cover one contiguous span of each row;
-//   * the R rows' loads of an iteration are issued back to back before any use (R x 36..68 bytes per lane in
-//     flight), which is what keeps HBM busy;
+//   * the R rows' loads of an iteration are issued back to back before any use (about 128..144 bytes per lane
+//     in flight, the depth at which a plain read kernel with the same access pattern peaks on this GPU), and
+//     the first tile's loads are issued before the activation prologue so HBM latency overlaps it;
 //   * quantized activations are staged once per workgroup into LDS, transposed so that lane l's 16-byte
 //     chunks are adjacent to lane l+1's (conflict-free ds_read_b128), and are re-read per row tile from LDS,
-//     never from global memory;
+//     never from global memory.  For small token counts the prologue quantizes the fp32 activations itself
+//     (same device functions as the stand-alone quantize kernels), which removes a kernel launch per op;
+//     workgroup 0 then also writes the quantized activations to the workspace in the split layout;
 //   * integer dots use v_dot4_i32_i8; each lane keeps fp32 partial sums per (row, token) and the 64 lanes are
 //     combined at the end with a fixed DPP butterfly (no LDS round trip, deterministic order).
 #include "dev_common.h"
 #include "act_layout.h"
+#include "quant_dev.h"
 #include "kernels.h"
 
 namespace chip {
@@ -32,14 +36,19 @@ template <> struct Traits<T_Q8_0> {
     static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
     struct W { uint32_t q[16]; float d0, d1; };
     struct A { uint32_t q[16]; float d0, d1; };
+    struct Raw { u32x4 a, b, c, e; uint32_t f; };
 
-    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
         const uint8_t *p = row + (size_t)u * 68;                       // two 34-byte blocks, 4-byte aligned
-        const u32x4 a = *reinterpret_cast<const u32x4_a4 *>(p);
-        const u32x4 b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
-        const u32x4 c = *reinterpret_cast<const u32x4_a4 *>(p + 32);
-        const u32x4 e = *reinterpret_cast<const u32x4_a4 *>(p + 48);
-        const uint32_t f = *reinterpret_cast<const uint32_t *>(p + 64);
+        r.a = *reinterpret_cast<const u32x4_a4 *>(p);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        r.c = *reinterpret_cast<const u32x4_a4 *>(p + 32);
+        r.e = *reinterpret_cast<const u32x4_a4 *>(p + 48);
+        r.f = *reinterpret_cast<const uint32_t *>(p + 64);
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
+        const u32x4 a = r.a, b = r.b, c = r.c, e = r.e;
+        const uint32_t f = r.f;
         // block 0: d at byte 0, quants at bytes 2..33 -> re-slice by 16 bits; block 1: d at 34, quants at 36..67
         w.d0 = h2f(a.x);
         w.q[0] = shr16(a.y, a.x); w.q[1] = shr16(a.z, a.y); w.q[2] = shr16(a.w, a.z); w.q[3] = shr16(b.x, a.w);
@@ -76,6 +85,14 @@ template <> struct Traits<T_Q8_0> {
         if (valid) d = reinterpret_cast<const float2 *>(ws + q8_0_off_d(K))[u];
         *reinterpret_cast<float2 *>(dst) = d;
     }
+    // fused prologue: where the dword of elements e..e+3 and the side data of 32-block blk go in the LDS image
+    __device__ static __forceinline__ size_t img_qs(int, int e) {
+        const int b = e >> 5, u = b >> 1, off = 32 * (b & 1) + (e & 31);
+        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
+    }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int) {
+        reinterpret_cast<float *>(img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX)[blk & 1] = d;
+    }
 };
 
 template <> struct Traits<T_Q4_0> {
@@ -83,11 +100,16 @@ template <> struct Traits<T_Q4_0> {
     struct W { uint32_t lo[8], hi[8]; float d0, d1; };          // nibbles spread to bytes, 0..15
     struct A { uint32_t q[16]; float d0, d1; int s0, s1; };
 
-    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+    struct Raw { u32x4 a, b; uint32_t c; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
         const uint8_t *p = row + (size_t)u * 36;                       // two 18-byte blocks, 4-byte aligned
-        const u32x4 a = *reinterpret_cast<const u32x4_a4 *>(p);
-        const u32x4 b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
-        const uint32_t c = *reinterpret_cast<const uint32_t *>(p + 32);
+        r.a = *reinterpret_cast<const u32x4_a4 *>(p);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        r.c = *reinterpret_cast<const uint32_t *>(p + 32);
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
+        const u32x4 a = r.a, b = r.b;
+        const uint32_t c = r.c;
         uint32_t q[8];
         w.d0 = h2f(a.x);
         q[0] = shr16(a.y, a.x); q[1] = shr16(a.z, a.y); q[2] = shr16(a.w, a.z); q[3] = shr16(b.x, a.w);
@@ -131,6 +153,15 @@ template <> struct Traits<T_Q4_0> {
         }
         *reinterpret_cast<u32x4 *>(dst) = x;
     }
+    __device__ static __forceinline__ size_t img_qs(int, int e) {
+        const int b = e >> 5, u = b >> 1, off = 32 * (b & 1) + (e & 31);
+        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
+    }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum) {
+        uint8_t *a = img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX;
+        reinterpret_cast<float *>(a)[blk & 1] = d;
+        reinterpret_cast<int *>(a)[2 + (blk & 1)] = sum;
+    }
 };
 
 template <> struct Traits<T_Q4_K> {
@@ -140,11 +171,16 @@ template <> struct Traits<T_Q4_K> {
     struct W { uint32_t lo[4], hi[4]; float d, dmin; int sc0, sc1, m0, m1; };
     struct A { uint32_t q[8]; float d; int s0, s1; };
 
-    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+    struct Raw { u32x4 h, q; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
         const int sb = u >> 3, c = u & 7;
         const uint8_t *p = row + (size_t)sb * BYTES_Q4_K;              // 144-byte super-block, 16-byte aligned
-        const u32x4 h = *reinterpret_cast<const u32x4 *>(p);
-        const u32x4 q = *reinterpret_cast<const u32x4 *>(p + 16 + 16 * c);
+        r.h = *reinterpret_cast<const u32x4 *>(p);
+        r.q = *reinterpret_cast<const u32x4 *>(p + 16 + 16 * c);
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+        const int c = u & 7;
+        const u32x4 h = r.h, q = r.q;
         w.d = h2f(h.x); w.dmin = h2f(h.x >> 16);
         // 6-bit scale/min of sub-blocks (2jp, 2jp+1), jp = c/2 (reference ggml-quants.c:625-632)
         const int jp = c >> 1, sh = 16 * (jp & 1);
@@ -194,6 +230,20 @@ template <> struct Traits<T_Q4_K> {
         }
         *reinterpret_cast<u32x2 *>(dst) = x;
     }
+    // fused prologue (one wave per super-block sb; lane holds elements 4*lane..4*lane+3 of it)
+    static constexpr int UNITS_PER_SB = 8;
+    __device__ static __forceinline__ size_t img_qs(int, int e) {
+        const int sb = e >> 8, o = e & 255;
+        const int jp = o >> 6, j = (o >> 5) & 1, cc = (o >> 4) & 1, w = o & 15;
+        const int u = sb * 8 + 2 * jp + cc;
+        return ((size_t)((u >> 6) * QCH + j) * 64 + (u & 63)) * 16 + w;
+    }
+    __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return img + (size_t)NI * QCH * 1024 + (size_t)u * AUX; }
+    // bsum of 16-value group g of super-block sb: group g = 4*jp + 2*j + cc feeds unit 2*jp + cc, slot j
+    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int g, int s) {
+        const int u = sb * 8 + 2 * (g >> 2) + (g & 1);
+        reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 1] = (int16_t)s;
+    }
 };
 
 template <> struct Traits<T_Q6_K> {
@@ -203,14 +253,21 @@ template <> struct Traits<T_Q6_K> {
     struct W { uint32_t q[16]; float d; int sc[4]; };            // q[4v + k]: 6-bit values 0..63 of group v
     struct A { uint32_t q[16]; float d; int bs[4]; };
 
-    __device__ static __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+    struct Raw { u32x4 l0, l1, qh; u32x2 s; uint32_t d; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
         const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
         const uint8_t *p = row + (size_t)sb * BYTES_Q6_K;              // 210-byte super-block, 2-byte aligned
-        const u32x4 l0 = *reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 16 * ip);
-        const u32x4 l1 = *reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 32 + 16 * ip);
-        const u32x4 qh = *reinterpret_cast<const u32x4_a2 *>(p + 128 + 32 * h + 16 * ip);
-        const u32x2 s  = *reinterpret_cast<const u32x2_a2 *>(p + 192 + 8 * h);
-        w.d = h2f(*reinterpret_cast<const unsigned short *>(p + 208));
+        r.l0 = *reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 16 * ip);
+        r.l1 = *reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 32 + 16 * ip);
+        r.qh = *reinterpret_cast<const u32x4_a2 *>(p + 128 + 32 * h + 16 * ip);
+        r.s  = *reinterpret_cast<const u32x2_a2 *>(p + 192 + 8 * h);
+        r.d  = *reinterpret_cast<const unsigned short *>(p + 208);
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+        const int ip = u & 1;
+        const u32x4 l0 = r.l0, l1 = r.l1, qh = r.qh;
+        const u32x2 s = r.s;
+        w.d = h2f(r.d);
         const uint32_t ql0[4] = {l0.x, l0.y, l0.z, l0.w}, ql1[4] = {l1.x, l1.y, l1.z, l1.w}, hh[4] = {qh.x, qh.y, qh.z, qh.w};
 #pragma unroll
         for (int k = 0; k < 4; k++) {                                   // reference ggml-quants.c:1695-1711
@@ -265,6 +322,19 @@ template <> struct Traits<T_Q6_K> {
         }
         *reinterpret_cast<u32x4 *>(dst) = x;
     }
+    static constexpr int UNITS_PER_SB = 4;
+    __device__ static __forceinline__ size_t img_qs(int, int e) {
+        const int sb = e >> 8, o = e & 255;
+        const int h = o >> 7, v = (o >> 5) & 3, ip = (o >> 4) & 1, w = o & 15;
+        const int u = sb * 4 + 2 * h + ip;
+        return ((size_t)((u >> 6) * QCH + v) * 64 + (u & 63)) * 16 + w;
+    }
+    __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return img + (size_t)NI * QCH * 1024 + (size_t)u * AUX; }
+    // bsum of 16-value group g = 8*h + 2*v + ip feeds unit 2*h + ip, slot v
+    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int g, int s) {
+        const int u = sb * 4 + 2 * (g >> 3) + (g & 1);
+        reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 3] = (int16_t)s;
+    }
 };
 
 template <int WT> __host__ __device__ constexpr int units_per_row(int64_t K) { return (int)(K / Traits<WT>::UNIT_ELEMS); }
@@ -274,40 +344,111 @@ template <int WT> __host__ __device__ constexpr size_t lds_image_bytes(int64_t K
 }
 
 // ------------------------------------------------------------------------------------------------ kernel
-template <int WT, int NTOK, int R, int WGS>
+// Fused prologue: quantize NTOK fp32 rows straight into the LDS image; workgroup 0 also writes the split
+// workspace planes so the quantized activations exist in memory as the reference's wdata does.
+template <int WT, int NTOK, int WGS>
+__device__ __forceinline__ void quantize_into_image(uint8_t *lds, size_t img, int NI, const float *__restrict__ x,
+                                                    int64_t ldx, int64_t K, uint8_t *__restrict__ ws, size_t ws_stride) {
+    using T = Traits<WT>;
+    const bool dump = blockIdx.x == 0 && ws != nullptr;
+    if constexpr (T::ACT == T_Q8_0) {
+        // 8 lanes per 32-block; K % 256 == 0 keeps every 64-lane group either fully inside or fully outside
+        const int nchunk = (int)(K / 4);
+        for (int t = 0; t < NTOK; t++) {
+            uint8_t *im = lds + t * img;
+            for (int c0 = 0; c0 < nchunk; c0 += WGS) {
+                const int c = c0 + threadIdx.x;
+                const bool live = c < nchunk;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (live) v = *reinterpret_cast<const float4 *>(x + t * ldx + 4 * (int64_t)c);
+                const Q8_0Lane q = quantize_q8_0_lane(v);
+                if (live) {
+                    const int e = 4 * c, blk = e >> 5;
+                    *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, e)) = q.packed;
+                    const float d = h2f(q.dh);
+                    if ((threadIdx.x & 7) == 0) T::img_block_aux(im, NI, blk, d, q.sum);
+                    if (dump) {
+                        uint8_t *base = ws + t * ws_stride;
+                        *reinterpret_cast<uint32_t *>(base + e) = q.packed;
+                        if ((threadIdx.x & 7) == 0) {
+                            reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = d;
+                            reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q.sum;
+                        }
+                    }
+                }
+            }
+        }
+    } else {
+        // one wave per 256-value super-block
+        const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+        const int nsb = (int)(K / 256);
+        for (int t = 0; t < NTOK; t++) {
+            uint8_t *im = lds + t * img;
+            for (int sb = wv; sb < nsb; sb += WGS / 64) {
+                const float4 v = *reinterpret_cast<const float4 *>(x + t * ldx + (int64_t)sb * 256 + 4 * lane);
+                const Q8_KLane q = quantize_q8_K_lane(v);
+                *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, sb * 256 + 4 * lane)) = q.packed;
+                if (lane < T::UNITS_PER_SB) *reinterpret_cast<float *>(T::img_aux(im, NI, sb * T::UNITS_PER_SB + lane)) = q.d;
+                if ((lane & 3) == 0) T::img_bsum(im, NI, sb, lane >> 2, q.bsum);
+                if (dump) {
+                    uint8_t *base = ws + t * ws_stride;
+                    *reinterpret_cast<uint32_t *>(base + (size_t)sb * 256 + 4 * lane) = q.packed;
+                    if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(K))[sb] = q.d;
+                    if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(K))[sb * 16 + (lane >> 2)] = (int16_t)q.bsum;
+                }
+            }
+        }
+    }
+}
+
+// Staging from an already quantized workspace: transpose the split planes to [it][chunk][lane].
+template <int WT, int NTOK, int WGS>
+__device__ __forceinline__ void stage_from_workspace(uint8_t *lds, size_t img, int NI, int units, int64_t K,
+                                                     const uint8_t *__restrict__ ws, size_t ws_stride) {
+    using T = Traits<WT>;
+    const int nq = NI * T::QCH * 64;                                    // 16-byte chunks per token
+    for (int idx = threadIdx.x; idx < NTOK * nq; idx += WGS) {
+        const int t = idx / nq, r = idx - t * nq;
+        const int lane = r & 63, j = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
+        const int u = it * 64 + lane;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (u < units) v = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + T::src_chunk(K, u, j));
+        reinterpret_cast<u32x4 *>(lds + t * img)[r] = v;
+    }
+    const int na = NI * 64;
+    for (int idx = threadIdx.x; idx < NTOK * na; idx += WGS) {
+        const int t = idx / na, u = idx - t * na;
+        T::stage_aux(lds + t * img + (size_t)NI * T::QCH * 1024 + (size_t)u * T::AUX, ws + t * ws_stride, K, u, u < units);
+    }
+}
+
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
 __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
-                                                   const uint8_t *__restrict__ ws, size_t ws_stride,
+                                                   const float *__restrict__ x, int64_t ldx,
+                                                   uint8_t *__restrict__ ws, size_t ws_stride,
                                                    float *__restrict__ y, int64_t ldy) {
     using T = Traits<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int NI = iters_per_row<WT>(K);
     const int units = units_per_row<WT>(K);
     const size_t img = lds_image_bytes<WT>(K);
-
-    // ---- stage the NTOK quantized activations, transposed to [it][chunk][lane] ----
-    {
-        const int nq = NI * T::QCH * 64;                                // 16-byte chunks per token
-        for (int idx = threadIdx.x; idx < NTOK * nq; idx += WGS) {
-            const int t = idx / nq, r = idx - t * nq;
-            const int lane = r & 63, j = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
-            const int u = it * 64 + lane;
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (u < units) v = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + T::src_chunk(K, u, j));
-            reinterpret_cast<u32x4 *>(lds + t * img)[r] = v;
-        }
-        const int na = NI * 64;
-        for (int idx = threadIdx.x; idx < NTOK * na; idx += WGS) {
-            const int t = idx / na, u = idx - t * na;
-            T::stage_aux(lds + t * img + (size_t)NI * T::QCH * 1024 + (size_t)u * T::AUX, ws + t * ws_stride, K, u, u < units);
-        }
-    }
-    __syncthreads();
-
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (WGS / 64) + (threadIdx.x >> 6);
     const int64_t nwaves = (int64_t)gridDim.x * (WGS / 64);
     const int64_t tiles = ceil_div(N, R);
 
+    // ---- issue the first tile's weight loads, then build the activation image while they fly ----
+    typename T::Raw raw[R];
+    const bool first_valid = wave < tiles && lane < units;
+    if (first_valid) {
+#pragma unroll
+        for (int r = 0; r < R; r++) T::load_raw(raw[r], W + (size_t)min(wave * R + r, N - 1) * nb01, lane);
+    }
+    if constexpr (FUSEQ) quantize_into_image<WT, NTOK, WGS>(lds, img, NI, x, ldx, K, ws, ws_stride);
+    else                 stage_from_workspace<WT, NTOK, WGS>(lds, img, NI, units, K, ws, ws_stride);
+    __syncthreads();
+
+    bool preloaded = true;
     for (int64_t tile = wave; tile < tiles; tile += nwaves) {
         const int64_t row0 = tile * R;
         float acc[R][NTOK];
@@ -319,12 +460,14 @@ __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W
         for (int it = 0; it < NI; it++) {
             const int u = it * 64 + lane;
             if (u < units) {
+                if (!preloaded) {
+#pragma unroll
+                    for (int r = 0; r < R; r++)                          // tail tile: re-read the last row, never store it
+                        T::load_raw(raw[r], W + (size_t)min(row0 + r, N - 1) * nb01, u);
+                }
                 typename T::W w[R];
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    const int64_t row = min(row0 + r, N - 1);           // tail tile: re-read the last row, never store it
-                    T::load_w(w[r], W + (size_t)row * nb01, u);
-                }
+                for (int r = 0; r < R; r++) T::decode(w[r], raw[r], u);
 #pragma unroll
                 for (int t = 0; t < NTOK; t++) {
                     typename T::A a;
@@ -333,6 +476,7 @@ __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W
                     for (int r = 0; r < R; r++) acc[r][t] = T::dot(w[r], a, acc[r][t]);
                 }
             }
+            preloaded = false;
         }
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -345,57 +489,67 @@ __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W
 }
 
 // ------------------------------------------------------------------------------------------------ launch
-template <int WT, int NTOK>
-static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                               float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
-    if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
-    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    // Small LDS images: 256-thread groups, several per CU, 4 rows per wave.  Large images leave room for a
-    // single group per CU, so make it 16 waves wide and use 2 rows per wave to stay within 128 VGPRs.
-    if (lds_bytes <= 40 * 1024) {
-        constexpr int R = 4, WGS = 256;
-        const int64_t tiles = ceil_div(N, R);
-        int64_t groups = ceil_div(tiles, WGS / 64);                     // one tile per wave ...
-        const int64_t cap = (int64_t)cus * 8;                           // ... until the grid is ~2 waves of groups deep
-        if (groups > cap) groups = cap;
-        auto kfn = gemv_kernel<WT, NTOK, R, WGS>;
-        if (lds_bytes > 48 * 1024) (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
-                           (const uint8_t *)ws, ws_stride, y, ldy);
-    } else {
-        constexpr int R = 2, WGS = 1024;
-        const int64_t tiles = ceil_div(N, R);
-        int64_t groups = ceil_div(tiles, WGS / 64);
-        if (groups > cus) groups = cus;
-        auto kfn = gemv_kernel<WT, NTOK, R, WGS>;
+// Rows per wave: units of 32..36 bytes take 4 rows (128..144 bytes per lane in flight), 52..68-byte units take 2.
+template <int WT> struct RowsPerWave { static constexpr int BIG = (WT == T_Q8_0 || WT == T_Q6_K) ? 2 : 4; };
+
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
+static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
+                             size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, hipStream_t st) {
+    const int64_t tiles = ceil_div(N, R);
+    int64_t groups = ceil_div(tiles, WGS / 64);
+    if (groups > max_groups) groups = max_groups;
+    auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ>;
+    if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
-                           (const uint8_t *)ws, ws_stride, y, ldy);
     }
+    hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
+                       (uint8_t *)ws, ws_stride, y, ldy);
     return hipGetLastError();
 }
 
-template <int WT>
-static hipError_t launch_ntok(int n, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    switch (n) {
-        case 1: return launch_typed<WT, 1>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 2: return launch_typed<WT, 2>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 3: return launch_typed<WT, 3>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 4: return launch_typed<WT, 4>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 5: return launch_typed<WT, 5>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 6: return launch_typed<WT, 6>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 7: return launch_typed<WT, 7>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case 8: return launch_typed<WT, 8>(W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        default: return hipErrorInvalidValue;
+template <int WT, int NTOK, bool FUSEQ>
+static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
+                               size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
+    if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    constexpr int RB = RowsPerWave<WT>::BIG, RS = RB / 2;
+    if (lds_bytes <= 40 * 1024) {
+        // 256-thread groups, several per CU.  Matrices with few rows take half the rows per wave so that the
+        // grid still has about 8 waves per CU.
+        const int64_t cap = (int64_t)cus * 8;
+        if (ceil_div(N, RB) >= (int64_t)cus * 8)
+            return launch_one<WT, NTOK, RB, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, st);
+        return launch_one<WT, NTOK, RS, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, st);
     }
+    if constexpr (!FUSEQ) {
+        // large images leave room for one group per CU: make it 16 waves wide
+        return launch_one<WT, NTOK, RS, 1024, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, st);
+    }
+    return hipErrorInvalidValue;
+}
+
+template <int WT, bool FUSEQ>
+static hipError_t launch_ntok(int n, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
+                              size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    switch (n) {
+        case 1: return launch_typed<WT, 1, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case 2: return launch_typed<WT, 2, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case 3: if constexpr (!FUSEQ) return launch_typed<WT, 3, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
+        case 4: return launch_typed<WT, 4, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case 5: if constexpr (!FUSEQ) return launch_typed<WT, 5, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
+        case 6: if constexpr (!FUSEQ) return launch_typed<WT, 6, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
+        case 7: if constexpr (!FUSEQ) return launch_typed<WT, 7, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
+        case 8: if constexpr (!FUSEQ) return launch_typed<WT, 8, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
+        default: break;
+    }
+    return hipErrorInvalidValue;
 }
 
 template <int WT> static int max_tokens_typed(int64_t K, const DeviceLimits &lim) {
     const size_t img = lds_image_bytes<WT>(K);
-    int64_t m = img ? (int64_t)(lim.max_lds_per_block / img) : 0;
+    const int64_t m = img ? (int64_t)(lim.max_lds_per_block / img) : 0;
     return (int)(m > 8 ? 8 : m);
 }
 
@@ -412,11 +566,39 @@ int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
 hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                        int n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     if (N <= 0 || n <= 0) return hipSuccess;
+    void *w = const_cast<void *>(ws);
     switch (wtype) {
-        case T_Q4_0: return launch_ntok<T_Q4_0>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case T_Q8_0: return launch_ntok<T_Q8_0>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case T_Q4_K: return launch_ntok<T_Q4_K>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
-        case T_Q6_K: return launch_ntok<T_Q6_K>(n, W, nb01, K, N, ws, ws_stride, y, ldy, lim, st);
+        case T_Q4_0: return launch_ntok<T_Q4_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q8_0: return launch_ntok<T_Q8_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q4_K: return launch_ntok<T_Q4_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q6_K: return launch_ntok<T_Q6_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// One launch for the whole op: quantize in the prologue.  Worth it while a workgroup's share of that work stays
+// small: n * K <= 16384 values (64 KB of fp32 per workgroup) and n in {1, 2, 4}.
+bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
+    if (!(n == 1 || n == 2 || n == 4) || (int64_t)n * K > 16384) return false;
+    size_t img = 0;
+    switch (wtype) {
+        case T_Q4_0: img = lds_image_bytes<T_Q4_0>(K); break;
+        case T_Q8_0: img = lds_image_bytes<T_Q8_0>(K); break;
+        case T_Q4_K: img = lds_image_bytes<T_Q4_K>(K); break;
+        case T_Q6_K: img = lds_image_bytes<T_Q6_K>(K); break;
+        default: return false;
+    }
+    return (size_t)n * img <= 40 * 1024 && (size_t)n * img <= (size_t)lim.max_lds_per_block;
+}
+
+hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                             int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    if (N <= 0 || n <= 0) return hipSuccess;
+    switch (wtype) {
+        case T_Q4_0: return launch_ntok<T_Q4_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q8_0: return launch_ntok<T_Q8_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q4_K: return launch_ntok<T_Q4_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q6_K: return launch_ntok<T_Q6_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
@@ -441,8 +623,10 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
         const int u = u0 + lane;
         int v0 = 0, v1 = 0;
         if (u < units) {
+            typename T::Raw raw;
+            T::load_raw(raw, W + (size_t)row * nb01, u);
             typename T::W w;
-            T::load_w(w, W + (size_t)row * nb01, u);
+            T::decode(w, raw, u);
             typename T::A a;
             // gather this unit's activation bytes from reference blocks
             if constexpr (T::ACT == T_Q8_0) {

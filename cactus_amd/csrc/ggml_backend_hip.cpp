@@ -1,0 +1,317 @@
+// libggml-hip.so: the reference's ggml backend interface (ggml-backend-impl.h:17-207) implemented on top of the
+// C-ABI of include/cactus_hip.h.  Host C++ only; every GPU action goes through chip_* calls.
+//
+//   reg "HIP"  ->  device "HIP0" (ACCEL by default: a weights-only co-processor, like the AMX extra buffer type,
+//                  reference ggml-cpu/amx/amx.cpp:141-174; CACTUS_HIP_DEVICE_TYPE=GPU switches)
+//              ->  buffer type "HIP": hipMalloc'd buffers, tensors at base + offset, GGUF blocks kept verbatim
+//              ->  backend "HIP": one stream; graph_compute runs MUL_MAT (F32 activations x Q4_0/Q8_0/Q4_K/Q6_K
+//                  weights living in a HIP buffer) and skips view ops.
+// No C++ exception crosses the vtables; failures are NULL returns or LM_GGML_STATUS_FAILED.
+#include "../../include/cactus_hip.h"
+#include "../../include/ggml_abi_mirror.h"
+#include "../../include/ggml_backend_hip.h"
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+namespace {
+
+std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0};
+
+#define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
+
+struct buffer_ctx { void *base; size_t size; };
+struct backend_ctx { void *stream; void *workspace; size_t workspace_size; };
+
+lm_ggml_backend_buffer_type_t hip_buffer_type();
+lm_ggml_backend_dev_t hip_device();
+
+bool device_ok() {
+    static int ok = -1;
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lk(mu);
+    if (ok < 0) ok = (chip_device_count() > 0 && chip_init(0) == CHIP_OK) ? 1 : 0;
+    return ok == 1;
+}
+
+bool is_host_buffer(const lm_ggml_backend_buffer *b) {
+    return b && b->buft && b->buft->iface.is_host && b->buft->iface.is_host(b->buft);
+}
+bool is_hip_buffer(const lm_ggml_backend_buffer *b) { return b && b->buft == hip_buffer_type(); }
+
+// ------------------------------------------------------------------------------------------------ buffer
+void buf_free(lm_ggml_backend_buffer_t buffer) {
+    buffer_ctx *c = (buffer_ctx *)buffer->context;
+    chip_free(c->base);
+    delete c;
+}
+void *buf_get_base(lm_ggml_backend_buffer_t buffer) { return ((buffer_ctx *)buffer->context)->base; }
+void buf_memset_tensor(lm_ggml_backend_buffer_t, lm_ggml_tensor *t, uint8_t value, size_t offset, size_t size) {
+    chip_memset((char *)t->data + offset, value, size, nullptr);
+    chip_stream_synchronize(nullptr);
+}
+void buf_set_tensor(lm_ggml_backend_buffer_t, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
+    chip_memcpy_h2d((char *)t->data + offset, data, size, nullptr);          // synchronous
+    g_uploaded += size;
+}
+void buf_get_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *t, void *data, size_t offset, size_t size) {
+    chip_stream_synchronize(nullptr);
+    chip_memcpy_d2h(data, (const char *)t->data + offset, size, nullptr);    // synchronous
+}
+bool buf_cpy_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *src, lm_ggml_tensor *dst) {
+    const size_t n = lm_ggml_nbytes(src);
+    if (is_host_buffer(src->buffer)) {
+        chip_memcpy_h2d(dst->data, src->data, n, nullptr);
+        return true;
+    }
+    if (is_hip_buffer(src->buffer)) {
+        chip_memcpy_d2d(dst->data, src->data, n, nullptr);
+        chip_stream_synchronize(nullptr);
+        return true;
+    }
+    return false;
+}
+void buf_clear(lm_ggml_backend_buffer_t buffer, uint8_t value) {
+    buffer_ctx *c = (buffer_ctx *)buffer->context;
+    chip_memset(c->base, value, c->size, nullptr);
+    chip_stream_synchronize(nullptr);
+}
+const lm_ggml_backend_buffer_i k_buffer_i = {
+    /* free_buffer   */ buf_free,
+    /* get_base      */ buf_get_base,
+    /* init_tensor   */ nullptr,
+    /* memset_tensor */ buf_memset_tensor,
+    /* set_tensor    */ buf_set_tensor,
+    /* get_tensor    */ buf_get_tensor,
+    /* cpy_tensor    */ buf_cpy_tensor,
+    /* clear         */ buf_clear,
+    /* reset         */ nullptr,
+};
+
+// ------------------------------------------------------------------------------------------------ buffer type
+const char *buft_name(lm_ggml_backend_buffer_type_t) { return "HIP"; }
+lm_ggml_backend_buffer_t buft_alloc(lm_ggml_backend_buffer_type_t buft, size_t size) {
+    if (!device_ok()) return nullptr;
+    void *p = nullptr;
+    if (chip_malloc(&p, size) != CHIP_OK || !p) {
+        HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: hipMalloc of %zu bytes failed\n", __func__, size);
+        return nullptr;
+    }
+    buffer_ctx *c = new (std::nothrow) buffer_ctx{p, size};
+    if (!c) { chip_free(p); return nullptr; }
+    return lm_ggml_backend_buffer_init(buft, k_buffer_i, c, size);
+}
+size_t buft_alignment(lm_ggml_backend_buffer_type_t) { return 256; }       // rows stay 16-byte aligned for the kernels
+bool buft_is_host(lm_ggml_backend_buffer_type_t) { return false; }
+
+// ------------------------------------------------------------------------------------------------ backend
+lm_ggml_guid_t hip_guid() {
+    static lm_ggml_guid g = {0x63, 0x61, 0x63, 0x74, 0x75, 0x73, 0x2d, 0x68, 0x69, 0x70, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35};
+    return &g;
+}
+const char *backend_name(lm_ggml_backend_t) { return "HIP"; }
+void backend_free(lm_ggml_backend_t backend) {
+    backend_ctx *c = (backend_ctx *)backend->context;
+    chip_stream_synchronize(c->stream);
+    chip_free(c->workspace);
+    chip_stream_destroy(c->stream);
+    delete c;
+    delete backend;
+}
+void backend_synchronize(lm_ggml_backend_t backend) { chip_stream_synchronize(((backend_ctx *)backend->context)->stream); }
+
+bool is_view_op(int op) {
+    return op == LM_GGML_OP_NONE || op == LM_GGML_OP_RESHAPE || op == LM_GGML_OP_VIEW || op == LM_GGML_OP_PERMUTE ||
+           op == LM_GGML_OP_TRANSPOSE;
+}
+
+// The MUL_MAT shapes the kernels take: weights [K, N] of a supported block type with whole-row strides, F32
+// activations [K, n] and F32 result [N, n] with element-contiguous rows, no batch dimensions.
+bool mul_mat_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *w = op->src[0], *x = op->src[1];
+    if (!w || !x) return false;
+    if (!chip_mul_mat_supported(w->type, w->ne[0])) return false;
+    if (x->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32) return false;
+    if (w->ne[2] != 1 || w->ne[3] != 1 || x->ne[2] != 1 || x->ne[3] != 1) return false;
+    if (x->ne[0] != w->ne[0] || op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1]) return false;
+    if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, w->ne[0])) return false;
+    if (w->nb[1] % (w->type == LM_GGML_TYPE_Q6_K ? 2 : 16) != 0) return false;
+    if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)x->ne[0] * 4) return false;
+    if (op->nb[0] != sizeof(float) || op->nb[1] % 4 != 0 || op->nb[1] < (size_t)op->ne[0] * 4) return false;
+    return true;
+}
+
+int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
+    backend_ctx *c = (backend_ctx *)backend->context;
+    for (int i = 0; i < cgraph->n_nodes; i++) {
+        lm_ggml_tensor *node = cgraph->nodes[i];
+        if (is_view_op(node->op)) continue;
+        if (node->op != LM_GGML_OP_MUL_MAT || !mul_mat_shape_ok(node)) {
+            HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: node %d (%s, op %d) is not supported by the HIP backend\n", __func__, i, node->name, node->op);
+            return LM_GGML_STATUS_FAILED;
+        }
+        const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
+        const int64_t K = w->ne[0], N = w->ne[1], n = x->ne[1];
+        if (N == 0 || n == 0) continue;
+        const size_t need = chip_mul_mat_workspace_size(w->type, K, n);
+        if (need > c->workspace_size) {                                    // grow the activation scratch (wdata)
+            chip_stream_synchronize(c->stream);
+            chip_free(c->workspace);
+            c->workspace = nullptr;
+            c->workspace_size = 0;
+            const size_t want = need + need / 4;
+            if (chip_malloc(&c->workspace, want) != CHIP_OK) return LM_GGML_STATUS_ALLOC_FAILED;
+            c->workspace_size = want;
+        }
+        const int rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, (int64_t)(x->nb[1] / 4), n,
+                                    (float *)node->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
+        if (rc != CHIP_OK) {
+            HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+            return LM_GGML_STATUS_FAILED;
+        }
+        g_mul_mat_nodes++;
+    }
+    return LM_GGML_STATUS_SUCCESS;
+}
+
+const lm_ggml_backend_i k_backend_i = {
+    /* get_name           */ backend_name,
+    /* free               */ backend_free,
+    /* set_tensor_async   */ nullptr,
+    /* get_tensor_async   */ nullptr,
+    /* cpy_tensor_async   */ nullptr,
+    /* synchronize        */ backend_synchronize,
+    /* graph_plan_create  */ nullptr,
+    /* graph_plan_free    */ nullptr,
+    /* graph_plan_update  */ nullptr,
+    /* graph_plan_compute */ nullptr,
+    /* graph_compute      */ backend_graph_compute,
+    /* event_record       */ nullptr,
+    /* event_wait         */ nullptr,
+};
+
+// ------------------------------------------------------------------------------------------------ device
+char g_description[160] = "AMD gfx950";
+
+const char *dev_name(lm_ggml_backend_dev_t) { return "HIP0"; }
+const char *dev_description(lm_ggml_backend_dev_t) { return g_description; }
+void dev_memory(lm_ggml_backend_dev_t, size_t *free_b, size_t *total_b) {
+    chip_device_info info;
+    *free_b = *total_b = 0;
+    if (device_ok() && chip_get_device_info(&info) == CHIP_OK) { *free_b = info.hbm_free; *total_b = info.hbm_total; }
+}
+int dev_type(lm_ggml_backend_dev_t) {
+    // ACCEL: weights of supported matmuls move to the device, every other tensor (KV cache included) stays in
+    // host buffers, so a backend that only implements MUL_MAT is safe (reference llama-model.cpp:277-287).
+    const char *e = std::getenv("CACTUS_HIP_DEVICE_TYPE");
+    return (e && std::strcmp(e, "GPU") == 0) ? LM_GGML_BACKEND_DEVICE_TYPE_GPU : LM_GGML_BACKEND_DEVICE_TYPE_ACCEL;
+}
+void dev_props(lm_ggml_backend_dev_t dev, lm_ggml_backend_dev_props *props) {
+    props->name = dev_name(dev);
+    props->description = dev_description(dev);
+    props->type = dev_type(dev);
+    dev_memory(dev, &props->memory_free, &props->memory_total);
+    props->caps = {/* async */ false, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false};
+}
+lm_ggml_backend_t dev_init_backend(lm_ggml_backend_dev_t dev, const char *) {
+    if (!device_ok()) return nullptr;
+    backend_ctx *c = new (std::nothrow) backend_ctx{nullptr, nullptr, 0};
+    if (!c) return nullptr;
+    if (chip_stream_create(&c->stream) != CHIP_OK) { delete c; return nullptr; }
+    lm_ggml_backend *b = new (std::nothrow) lm_ggml_backend{hip_guid(), k_backend_i, dev, c};
+    if (!b) { chip_stream_destroy(c->stream); delete c; return nullptr; }
+    return b;
+}
+lm_ggml_backend_buffer_type_t dev_buffer_type(lm_ggml_backend_dev_t) { return hip_buffer_type(); }
+
+bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
+    if (is_view_op(op->op)) return true;
+    if (op->op != LM_GGML_OP_MUL_MAT) return false;
+    // Only weights that already live in a HIP buffer: claiming host-resident weights would make the scheduler
+    // copy the whole matrix to the device on every call.  At model load the probe tensor carries a zero-size
+    // dummy buffer of the candidate buffer type and NULL data (reference llama-model.cpp:161-165,246-251).
+    const lm_ggml_tensor *w = op->src[0];
+    if (!w || !w->buffer || !is_hip_buffer(w->buffer)) return false;
+    return mul_mat_shape_ok(op);
+}
+bool dev_supports_buft(lm_ggml_backend_dev_t, lm_ggml_backend_buffer_type_t buft) { return buft == hip_buffer_type(); }
+
+const lm_ggml_backend_device_i k_device_i = {
+    /* get_name             */ dev_name,
+    /* get_description      */ dev_description,
+    /* get_memory           */ dev_memory,
+    /* get_type             */ dev_type,
+    /* get_props            */ dev_props,
+    /* init_backend         */ dev_init_backend,
+    /* get_buffer_type      */ dev_buffer_type,
+    /* get_host_buffer_type */ nullptr,
+    /* buffer_from_host_ptr */ nullptr,
+    /* supports_op          */ dev_supports_op,
+    /* supports_buft        */ dev_supports_buft,
+    /* offload_op           */ nullptr,
+    /* event_new            */ nullptr,
+    /* event_free           */ nullptr,
+    /* event_synchronize    */ nullptr,
+};
+
+// ------------------------------------------------------------------------------------------------ reg
+const char *reg_name(lm_ggml_backend_reg_t) { return "HIP"; }
+size_t reg_device_count(lm_ggml_backend_reg_t) { return device_ok() ? 1 : 0; }
+lm_ggml_backend_dev_t reg_get_device(lm_ggml_backend_reg_t, size_t index) { return (index == 0 && device_ok()) ? hip_device() : nullptr; }
+void *reg_get_proc_address(lm_ggml_backend_reg_t, const char *name) {
+    if (std::strcmp(name, "lm_ggml_backend_hip_get_stats") == 0) return (void *)lm_ggml_backend_hip_get_stats;
+    return nullptr;         // no n_threads, no extra buffer types, no split buffer type, no feature list
+}
+const lm_ggml_backend_reg_i k_reg_i = {reg_name, reg_device_count, reg_get_device, reg_get_proc_address};
+
+lm_ggml_backend_dev_t hip_device() {
+    static lm_ggml_backend_device dev = {k_device_i, lm_ggml_backend_hip_reg(), nullptr};
+    return &dev;
+}
+lm_ggml_backend_buffer_type_t hip_buffer_type() {
+    static lm_ggml_backend_buffer_type buft = {
+        {buft_name, buft_alloc, buft_alignment, /* get_max_size */ nullptr, /* get_alloc_size */ nullptr, buft_is_host},
+        /* device  */ nullptr,
+        /* context */ nullptr,
+    };
+    static std::once_flag once;
+    std::call_once(once, [] { buft.device = hip_device(); });
+    return &buft;
+}
+
+}  // namespace
+
+extern "C" {
+
+lm_ggml_backend_reg *lm_ggml_backend_hip_reg(void) {
+    static lm_ggml_backend_reg reg = {LM_GGML_BACKEND_API_VERSION, k_reg_i, nullptr};
+    static std::once_flag once;
+    std::call_once(once, [] {
+        chip_device_info info;
+        if (device_ok() && chip_get_device_info(&info) == CHIP_OK)
+            std::snprintf(g_description, sizeof(g_description), "%.60s (%.40s, %d CUs)", info.name[0] ? info.name : "AMD Instinct", info.arch, info.compute_units);
+    });
+    return &reg;
+}
+lm_ggml_backend_reg *lm_ggml_backend_init(void) { return lm_ggml_backend_hip_reg(); }
+int lm_ggml_backend_score(void) { return device_ok() ? 100 : 0; }
+
+lm_ggml_backend *lm_ggml_backend_hip_init(void) {
+    lm_ggml_backend_hip_reg();
+    return dev_init_backend(hip_device(), nullptr);
+}
+lm_ggml_backend_buffer_type *lm_ggml_backend_hip_buffer_type(void) {
+    lm_ggml_backend_hip_reg();
+    return hip_buffer_type();
+}
+int lm_ggml_backend_is_hip(lm_ggml_backend *backend) { return backend && backend->guid == hip_guid(); }
+void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned long long *uploaded_bytes) {
+    if (mul_mat_nodes) *mul_mat_nodes = g_mul_mat_nodes.load();
+    if (uploaded_bytes) *uploaded_bytes = g_uploaded.load();
+}
+
+}  // extern "C"

@@ -22,6 +22,11 @@ hipError_t launch_split_to_blocks(int act_type, const void *ws, size_t ws_stride
 int        gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim);   // tokens one launch can take (<= 8)
 hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                        int n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+// One launch for quantize + GEMV (n in {1,2,4}, small n*K): x is fp32; ws receives the split-layout quantized
+// activations from workgroup 0.
+bool       gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim);
+hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                             int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                               int32_t *isum, int32_t *imin, hipStream_t st);
 

@@ -10,15 +10,10 @@
 // with -ffp-contract=off so `iscale*x + 12582912.f` rounds twice, as the C source of the reference says.
 #include "dev_common.h"
 #include "act_layout.h"
+#include "quant_dev.h"
 #include "kernels.h"
 
 namespace chip {
-
-// x86 cvtps2dq semantics followed by two saturating packs: NaN or |r| >= 2^31 becomes INT_MIN -> -128.
-__device__ __forceinline__ int to_i8_x86(float r) {
-    int q = (fabsf(r) < 2147483648.f) ? (int)r : INT32_MIN;
-    return max(-128, min(127, q));
-}
 
 template <bool SPLIT>
 __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, int64_t ldx, int64_t K,
@@ -28,41 +23,21 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     const bool live = e0 < K;                                             // K % 32 == 0: whole 8-lane groups agree
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (live) v = *reinterpret_cast<const float4 *>(x + t * ldx + e0);
-
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, dpp_get<0xB1>(amax));
-    amax = fmaxf(amax, dpp_get<0x4E>(amax));
-    amax = fmaxf(amax, dpp_get<0x141>(amax));                              // max over the block's 8 lanes
-
-    const float d = amax / 127.f;
-    const float id = (amax != 0.0f) ? 127.f / amax : 0.0f;
-    const int q0 = to_i8_x86(__builtin_rintf(v.x * id));
-    const int q1 = to_i8_x86(__builtin_rintf(v.y * id));
-    const int q2 = to_i8_x86(__builtin_rintf(v.z * id));
-    const int q3 = to_i8_x86(__builtin_rintf(v.w * id));
-    const uint32_t packed = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
-                            ((uint32_t)(q3 & 0xff) << 24);
-    const unsigned short dh = f2h_rne(d);
+    const Q8_0Lane q = quantize_q8_0_lane(v);
     const int64_t blk = e0 / 32;
     const int sub = threadIdx.x & 7;
-
+    if (!live) return;
     if (SPLIT) {
-        int s = q0 + q1 + q2 + q3;
-        s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xf, 0xf, true);
-        s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xf, 0xf, true);
-        s += __builtin_amdgcn_update_dpp(0, s, 0x141, 0xf, 0xf, true);
-        if (live) {
-            uint8_t *base = y + t * y_stride;
-            *reinterpret_cast<uint32_t *>(base + e0) = packed;
-            if (sub == 0) {
-                reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = h2f(dh);
-                reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = s;
-            }
+        uint8_t *base = y + t * y_stride;
+        *reinterpret_cast<uint32_t *>(base + e0) = q.packed;
+        if (sub == 0) {
+            reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = h2f(q.dh);
+            reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q.sum;
         }
-    } else if (live) {
+    } else {
         uint8_t *b = y + t * y_stride + blk * BYTES_Q8_0;
-        *reinterpret_cast<u32_a2 *>(b + 2 + 4 * sub) = packed;
-        if (sub == 0) *reinterpret_cast<unsigned short *>(b) = dh;
+        *reinterpret_cast<u32_a2 *>(b + 2 + 4 * sub) = q.packed;
+        if (sub == 0) *reinterpret_cast<unsigned short *>(b) = q.dh;
     }
 }
 
@@ -74,47 +49,17 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float *__restr
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);       // one wave per 256-value super-block
     if (sb * QK_K >= K) return;                                           // whole wave leaves together
     const float4 v = *reinterpret_cast<const float4 *>(x + t * ldx + sb * QK_K + lane * 4);
-
-    // (amax, max): the first element with the largest magnitude decides, sign kept (strict > in index order)
-    float cand = v.x;
-    if (fabsf(v.y) > fabsf(cand)) cand = v.y;
-    if (fabsf(v.z) > fabsf(cand)) cand = v.z;
-    if (fabsf(v.w) > fabsf(cand)) cand = v.w;
-    const float amax = wave_max_all(fabsf(cand));
-    const unsigned long long holders = __ballot(fabsf(cand) == amax);
-    const int first = __builtin_ctzll(holders);
-    const float mx = __shfl(cand, first);
-
-    int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
-    float d = 0.f;
-    if (amax != 0.0f) {
-        const float iscale = -127.f / mx;
-        auto nearest = [](float f) {
-            const float m = f + 12582912.f;
-            return (int)(__float_as_uint(m) & 0x007fffffu) - 0x00400000;
-        };
-        q0 = min(127, nearest(iscale * v.x));
-        q1 = min(127, nearest(iscale * v.y));
-        q2 = min(127, nearest(iscale * v.z));
-        q3 = min(127, nearest(iscale * v.w));
-        d = 1.0f / iscale;
-    }
-    const uint32_t packed = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
-                            ((uint32_t)(q3 & 0xff) << 24);
-    int s = q0 + q1 + q2 + q3;                                             // 16 values = 4 lanes
-    s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xf, 0xf, true);
-    s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xf, 0xf, true);
-
+    const Q8_KLane q = quantize_q8_K_lane(v);
     if (SPLIT) {
         uint8_t *base = y + t * y_stride;
-        *reinterpret_cast<uint32_t *>(base + sb * QK_K + lane * 4) = packed;
-        if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(K))[sb] = d;
-        if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(K))[sb * 16 + (lane >> 2)] = (int16_t)s;
+        *reinterpret_cast<uint32_t *>(base + sb * QK_K + lane * 4) = q.packed;
+        if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(K))[sb] = q.d;
+        if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(K))[sb * 16 + (lane >> 2)] = (int16_t)q.bsum;
     } else {
         uint8_t *b = y + t * y_stride + sb * BYTES_Q8_K;
-        *reinterpret_cast<uint32_t *>(b + 4 + lane * 4) = packed;
-        if (lane == 0) *reinterpret_cast<float *>(b) = d;
-        if ((lane & 3) == 0) *reinterpret_cast<int16_t *>(b + 260 + 2 * (lane >> 2)) = (int16_t)s;
+        *reinterpret_cast<uint32_t *>(b + 4 + lane * 4) = q.packed;
+        if (lane == 0) *reinterpret_cast<float *>(b) = q.d;
+        if ((lane & 3) == 0) *reinterpret_cast<int16_t *>(b + 260 + 2 * (lane >> 2)) = (int16_t)q.bsum;
     }
 }
 

@@ -1,0 +1,51 @@
+/*
+ * ggml_backend_hip.h -- entry points of libggml-hip.so, the ggml backend that runs LM_GGML_OP_MUL_MAT over
+ * block-quantized weights on an MI355X through the C-ABI of cactus_hip.h.
+ *
+ * It implements the reference's backend interface (ggml-backend-impl.h:17-207): a registry entry with one
+ * device, a buffer type that keeps GGUF blocks in their on-disk layout in HBM, and a backend (stream) whose
+ * graph_compute handles MUL_MAT and the view ops.  Everything else stays on the CPU backend; the reference's
+ * scheduler splits the graph accordingly (ggml-backend.cpp:730-785).
+ *
+ * Three ways to make it visible to llama.cpp / cactus_context (reference ggml-backend-reg.cpp:162-193,305,401):
+ *   - dynamic:  lm_ggml_backend_load("libggml-hip.so")  (or LM_GGML_BACKEND_PATH) -> calls lm_ggml_backend_init()
+ *   - explicit: lm_ggml_backend_register(lm_ggml_backend_hip_reg()) before the first model load
+ *   - built in: an `#ifdef LM_GGML_USE_HIP  register_backend(lm_ggml_backend_hip_reg());` line in the registry
+ * The library resolves lm_ggml_backend_buffer_init, lm_ggml_nbytes and lm_ggml_log_internal from the process
+ * that loads it.
+ */
+#ifndef CACTUS_GGML_BACKEND_HIP_H
+#define CACTUS_GGML_BACKEND_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+struct lm_ggml_backend_reg;
+struct lm_ggml_backend;
+struct lm_ggml_backend_buffer_type;
+
+#define CACTUS_GGML_API __attribute__((visibility("default")))
+
+/* The registry entry ("HIP", one device "HIP0").  Counterpart of lm_ggml_backend_cpu_reg()
+ * (ggml-cpu/ggml-cpu.cpp:658-669).  Returns a reg with zero devices if no gfx950 GPU is usable. */
+CACTUS_GGML_API struct lm_ggml_backend_reg *lm_ggml_backend_hip_reg(void);
+
+/* Dynamic-loading entry points looked up by lm_ggml_backend_load (ggml-backend-impl.h:215-246,
+ * ggml-backend-reg.cpp:227-271): score 0 means "not usable on this machine". */
+CACTUS_GGML_API struct lm_ggml_backend_reg *lm_ggml_backend_init(void);
+CACTUS_GGML_API int lm_ggml_backend_score(void);
+
+/* Direct construction, like lm_ggml_backend_cpu_init() (ggml-cpu/ggml-cpu.cpp:195-225) and
+ * lm_ggml_backend_cpu_buffer_type() (ggml-backend.cpp:1985). */
+CACTUS_GGML_API struct lm_ggml_backend *lm_ggml_backend_hip_init(void);
+CACTUS_GGML_API struct lm_ggml_backend_buffer_type *lm_ggml_backend_hip_buffer_type(void);
+CACTUS_GGML_API int lm_ggml_backend_is_hip(struct lm_ggml_backend *backend);
+
+/* Counters for tests and tracing: MUL_MAT nodes executed on the GPU and bytes uploaded by set_tensor. */
+CACTUS_GGML_API void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned long long *uploaded_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,224 @@
+"""The ggml backend (libggml-hip.so) driven the way llama.cpp drives a backend, with the reference's own ggml
+(oracle/_ref) as the host framework: dynamic load + registration, weight upload into the HIP buffer type,
+one-node and multi-node MUL_MAT graphs, the reference scheduler splitting a mixed graph between HIP and CPU,
+and lm_ggml_backend_compare_graph_backend node-by-node against the reference CPU backend."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import common
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def host():
+    if not O.Reference.available():
+        pytest.skip("oracle/_ref/libggml_ref.so not present: no ggml host framework to load the backend into")
+    from ggml_host import Host
+    h = Host()
+    h.reg = h.load_hip()
+    return h
+
+
+def test_registration_and_device(host):
+    L = host.L
+    assert L.lm_ggml_backend_reg_name(host.reg) == b"HIP"
+    assert L.lm_ggml_backend_reg_by_name(b"HIP") == host.reg            # it is in the reference's registry now
+    assert L.lm_ggml_backend_reg_dev_count(host.reg) == 1
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    assert L.lm_ggml_backend_dev_name(dev) == b"HIP0"
+    assert b"gfx950" in L.lm_ggml_backend_dev_description(dev)
+    assert L.lm_ggml_backend_dev_type(dev) == 2                         # ACCEL
+    fr, tot = C.c_size_t(), C.c_size_t()
+    L.lm_ggml_backend_dev_memory(dev, C.byref(fr), C.byref(tot))
+    assert tot.value > 200 << 30 and 0 < fr.value <= tot.value
+    buft = L.lm_ggml_backend_dev_buffer_type(dev)
+    assert L.lm_ggml_backend_buft_name(buft) == b"HIP"
+    assert not L.lm_ggml_backend_buft_is_host(buft)
+    assert L.lm_ggml_backend_dev_supports_buft(dev, buft)
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    assert be and L.lm_ggml_backend_name(be) == b"HIP"
+    assert L.lm_ggml_backend_get_default_buffer_type(be) == buft
+    L.lm_ggml_backend_free(be)
+
+
+@pytest.mark.parametrize("wt", O.WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("n", [1, 7, 40])
+def test_one_node_graph(host, orc, wt, n):
+    """Weights and activations allocated in the HIP buffer type, one MUL_MAT node, direct graph_compute."""
+    L = host.L
+    K, N = 1024, 200
+    wq = orc.quantize_weights(wt, common.weights_f32(wt + n, N, K))
+    x = common.activations_f32(wt + n, n, K)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    ctx = host.context()
+    a = host.tensor_2d(ctx, wt, K, N, "w")
+    b = host.tensor_2d(ctx, O.F32, K, n, "x")
+    c = L.lm_ggml_mul_mat(ctx, a, b)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, c)
+    assert L.lm_ggml_backend_dev_supports_op(dev, c) is False            # weights not in a HIP buffer yet
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    assert buf and L.lm_ggml_backend_buffer_get_size(buf) >= wq.size + x.nbytes + 4 * n * N
+    assert L.lm_ggml_backend_dev_supports_op(dev, c) is True
+    host.set(a, wq)
+    host.set(b, x)
+    assert np.array_equal(host.get(a, np.uint8, wq.shape), wq)           # set_tensor / get_tensor round trip
+    assert L.lm_ggml_backend_graph_compute(be, g) == 0
+    y = host.get(c, np.float32, (n, N))
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("sum_abs",))
+    assert (np.abs(y.astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all()
+    # memset_tensor / clear
+    L.lm_ggml_backend_tensor_memset(c, 0x7f, 0, 4 * n * N)
+    assert (host.get(c, np.uint8, (4 * n * N,)) == 0x7f).all()
+    L.lm_ggml_backend_buffer_clear(buf, 0)
+    assert not host.get(a, np.uint8, wq.shape).any()
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_free(ctx)
+
+
+def test_unsupported_ops_are_declined(host):
+    L = host.L
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    ctx = host.context()
+    w = host.tensor_2d(ctx, O.Q4_0, 256, 8)
+    wf = host.tensor_2d(ctx, O.F32, 256, 8)
+    x = host.tensor_2d(ctx, O.F32, 256, 2)
+    k96 = host.tensor_2d(ctx, O.Q8_0, 96, 8)
+    x96 = host.tensor_2d(ctx, O.F32, 96, 2)
+    mm = L.lm_ggml_mul_mat(ctx, w, x)
+    mm_f32 = L.lm_ggml_mul_mat(ctx, wf, x)
+    mm_96 = L.lm_ggml_mul_mat(ctx, k96, x96)
+    add = L.lm_ggml_add(ctx, x, x)
+    view = L.lm_ggml_reshape_2d(ctx, x, 128, 4)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    assert L.lm_ggml_backend_dev_supports_op(dev, mm) is True
+    assert L.lm_ggml_backend_dev_supports_op(dev, mm_f32) is False       # F32 weights: not this path
+    assert L.lm_ggml_backend_dev_supports_op(dev, mm_96) is False        # K not a multiple of 256
+    assert L.lm_ggml_backend_dev_supports_op(dev, add) is False
+    assert L.lm_ggml_backend_dev_supports_op(dev, view) is True
+    # graph_compute on a node the device declined reports failure, it does not compute on the host
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, add)
+    assert L.lm_ggml_backend_graph_compute(be, g) == -1                  # LM_GGML_STATUS_FAILED
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_free(ctx)
+
+
+def test_scheduler_splits_between_hip_and_cpu(host, orc):
+    """llama.cpp's flow: weights in a HIP buffer tagged USAGE_WEIGHTS, activations produced on the CPU; the
+    reference scheduler assigns the MUL_MATs to HIP, the ADD to the CPU, and copies inputs across."""
+    L = host.L
+    K, N1, N2, n = 2048, 512, 256, 3
+    w1 = orc.quantize_weights(O.Q4_K, common.weights_f32(11, N1, K))
+    w2 = orc.quantize_weights(O.Q6_K, common.weights_f32(12, N2, K))
+    w3 = orc.quantize_weights(O.Q8_0, common.weights_f32(13, N2, 512))
+    x = common.activations_f32(11, n, K)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    # weights
+    wctx = host.context(with_graph=False)
+    tw1 = host.tensor_2d(wctx, O.Q4_K, K, N1, "w1")
+    tw2 = host.tensor_2d(wctx, O.Q6_K, K, N2, "w2")
+    tw3 = host.tensor_2d(wctx, O.Q8_0, 512, N2, "w3")
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
+    host.set(tw1, w1); host.set(tw2, w2); host.set(tw3, w3)
+    # graph: y = w3 @ (w1 @ x)[:512]... keep shapes simple: h = w1 x ; z = w2 x ; s = w3 h + z
+    ctx = host.context()
+    tx = host.tensor_2d(ctx, O.F32, K, n, "x")
+    L.lm_ggml_set_input(tx)
+    h = L.lm_ggml_mul_mat(ctx, tw1, tx)          # [N1=512, n]
+    z = L.lm_ggml_mul_mat(ctx, tw2, tx)          # [N2, n]
+    s = L.lm_ggml_mul_mat(ctx, tw3, h)           # [N2, n]   (K = 512 = N1)
+    out = L.lm_ggml_add(ctx, s, z)
+    L.lm_ggml_set_output(out)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, out)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 64, False, True)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(tx, x)
+    before = (C.c_ulonglong(), C.c_ulonglong())
+    import cactus_amd
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_stats(C.byref(before[0]), C.byref(before[1]))
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    after = (C.c_ulonglong(), C.c_ulonglong())
+    blib.lm_ggml_backend_hip_get_stats(C.byref(after[0]), C.byref(after[1]))
+    assert after[0].value - before[0].value == 3                       # the three MUL_MATs ran on the GPU
+    assert L.lm_ggml_backend_sched_get_tensor_backend(sched, h) == hip
+    assert L.lm_ggml_backend_sched_get_tensor_backend(sched, out) == cpu
+    assert L.lm_ggml_backend_sched_get_n_splits(sched) >= 2
+    y = host.get(out, np.float32, (n, N2))
+    # reference: same graph entirely on the reference CPU path (through the oracle, bit-identical to it)
+    hh = orc.mul_mat(O.Q4_K, w1, x)["y"]
+    zz = orc.mul_mat(O.Q6_K, w2, x, want=("sum_abs",))
+    ss = orc.mul_mat(O.Q8_0, w3, hh, want=("sum_abs",))
+    want = ss["y"] + zz["y"]
+    # h itself carries the GPU's rounding (<= 1e-5 relative), which the Q8_0 requantization of h passes on:
+    # compare at a tolerance that reflects two chained ops
+    scale = ss["sum_abs"] + zz["sum_abs"]
+    assert (np.abs(y - want) <= 2e-3 * scale).all()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(wbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(wctx)
+
+
+def test_compare_graph_backend_against_reference_cpu(host, orc):
+    """The reference's own node-by-node comparison engine (ggml-backend.cpp:1821-1857): graph built on the CPU
+    backend, copied to HIP, each node evaluated on both and handed to a callback."""
+    L = host.L
+    from ggml_host import EVAL_CB
+    K, n = 1024, 5
+    specs = [(O.Q4_0, 300), (O.Q8_0, 64), (O.Q4_K, 257), (O.Q6_K, 130)]
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    ctx = host.context(n_tensors=64)
+    tx = host.tensor_2d(ctx, O.F32, K, n, "x")
+    tws, outs = [], []
+    for i, (wt, N) in enumerate(specs):
+        tw = host.tensor_2d(ctx, wt, K, N, "w%d" % i)
+        tws.append(tw)
+        outs.append(L.lm_ggml_mul_mat(ctx, tw, tx))
+    g = L.lm_ggml_new_graph(ctx)
+    for o in outs:
+        L.lm_ggml_build_forward_expand(g, o)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors(ctx, cpu)
+    x = common.activations_f32(31, n, K)
+    host.set(tx, x)
+    weights = []
+    for (wt, N), tw in zip(specs, tws):
+        wq = orc.quantize_weights(wt, common.weights_f32(31 + wt, N, K))
+        weights.append(wq)
+        host.set(tw, wq)
+    seen = []
+
+    def cb(idx, t1, t2, ud):
+        wt, N = specs[idx]
+        y1 = host.get(t1, np.float32, (n, N))          # reference CPU backend
+        y2 = host.get(t2, np.float32, (n, N))          # HIP backend
+        sa = orc.mul_mat(wt, weights[idx], x, nthreads=8, want=("sum_abs",))["sum_abs"]
+        seen.append(bool((np.abs(y1.astype(np.float64) - y2) <= REL_TOL * sa).all()))
+        return True
+
+    ok = L.lm_ggml_backend_compare_graph_backend(cpu, hip, g, EVAL_CB(cb), None)
+    assert ok and seen == [True] * len(specs)
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
