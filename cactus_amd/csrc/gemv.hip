@@ -6,7 +6,7 @@
 // Shape of the kernel (HBM-bound: every weight byte is read exactly once):
 //   * a wave owns a tile of R consecutive weight rows and walks along K; lane l handles "unit" u = l + 64*it
 //     of every row, a unit being the smallest piece that carries whole scales (two 32-blocks for Q4_0/Q8_0,
-//     1/8 of a Q4_K super-block, 1/4 of a Q6_K super-block).  Consecutive lanes read consecutive bytes, so a
+//     1/4 of a Q4_K or Q6_K super-block).  Consecutive lanes read consecutive bytes, so a
 //     wave's loads cover one contiguous span of each row;
 //   * the R rows' loads of an iteration are issued back to back before any use (about 128..144 bytes per lane
 //     in flight, the depth at which a plain read kernel with the same access pattern peaks on this GPU), and
@@ -22,6 +22,7 @@
 #include "act_layout.h"
 #include "quant_dev.h"
 #include "kernels.h"
+#include <cstdlib>
 
 namespace chip {
 
@@ -165,48 +166,52 @@ template <> struct Traits<T_Q4_0> {
 };
 
 template <> struct Traits<T_Q4_K> {
-    // unit = (super-block sb, chunk c of 8): qs bytes 16c..16c+15, i.e. elements 64*(c/2) + 16*(c%2) + [0,16)
-    // from the low nibbles (sub-block 2*(c/2)) and the same + 32 from the high nibbles (sub-block 2*(c/2)+1)
-    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 32, QCH = 2, AUX = 8;
-    struct W { uint32_t lo[4], hi[4]; float d, dmin; int sc0, sc1, m0, m1; };
-    struct A { uint32_t q[8]; float d; int s0, s1; };
+    // unit = (super-block sb, 64-value group jp of 4): the 32 qs bytes 32*jp..32*jp+31, whose low nibbles are
+    // elements 64*jp + [0,32) (sub-block 2*jp) and whose high nibbles are elements 64*jp + 32 + [0,32)
+    // (sub-block 2*jp+1).  The matching activations are the 64 contiguous quants 64*jp..64*jp+63.
+    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
+    struct W { uint32_t lo[8], hi[8]; float d, dmin; int sc0, sc1, m0, m1; };
+    struct A { uint32_t q[16]; float d; int s0, s1; };
+    struct Raw { u32x4 h, q0, q1; };
 
-    struct Raw { u32x4 h, q; };
     __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const int sb = u >> 3, c = u & 7;
+        const int sb = u >> 2, jp = u & 3;
         const uint8_t *p = row + (size_t)sb * BYTES_Q4_K;              // 144-byte super-block, 16-byte aligned
         r.h = *reinterpret_cast<const u32x4 *>(p);
-        r.q = *reinterpret_cast<const u32x4 *>(p + 16 + 16 * c);
+        r.q0 = *reinterpret_cast<const u32x4 *>(p + 16 + 32 * jp);
+        r.q1 = *reinterpret_cast<const u32x4 *>(p + 32 + 32 * jp);
     }
     __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
-        const int c = u & 7;
-        const u32x4 h = r.h, q = r.q;
+        const int jp = u & 3;
+        const u32x4 h = r.h;
         w.d = h2f(h.x); w.dmin = h2f(h.x >> 16);
-        // 6-bit scale/min of sub-blocks (2jp, 2jp+1), jp = c/2 (reference ggml-quants.c:625-632)
-        const int jp = c >> 1, sh = 16 * (jp & 1);
+        // 6-bit scale/min of sub-blocks (2jp, 2jp+1) (reference ggml-quants.c:625-632)
+        const int sh = 16 * (jp & 1);
         const uint32_t a1 = h.y >> sh, a2 = h.z >> sh, a3 = h.w >> sh;
         uint32_t sc, mn;
         if (jp < 2) { sc = a1 & 0x3f3fu; mn = a2 & 0x3f3fu; }
         else        { sc = (a3 & 0x0f0fu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
         w.sc0 = sc & 0xff; w.sc1 = sc >> 8; w.m0 = mn & 0xff; w.m1 = mn >> 8;
-        w.lo[0] = q.x & 0x0f0f0f0fu; w.lo[1] = q.y & 0x0f0f0f0fu; w.lo[2] = q.z & 0x0f0f0f0fu; w.lo[3] = q.w & 0x0f0f0f0fu;
-        w.hi[0] = (q.x >> 4) & 0x0f0f0f0fu; w.hi[1] = (q.y >> 4) & 0x0f0f0f0fu;
-        w.hi[2] = (q.z >> 4) & 0x0f0f0f0fu; w.hi[3] = (q.w >> 4) & 0x0f0f0f0fu;
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) { w.lo[i] = q[i] & 0x0f0f0f0fu; w.hi[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
     }
     __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
         const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-        const u32x4 v0 = q[0], v1 = q[64];
-        a.q[0] = v0.x; a.q[1] = v0.y; a.q[2] = v0.z; a.q[3] = v0.w;
-        a.q[4] = v1.x; a.q[5] = v1.y; a.q[6] = v1.z; a.q[7] = v1.w;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
         const u32x2 x = reinterpret_cast<const u32x2 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
         a.d = __uint_as_float(x.x);
         a.s0 = (int)(int16_t)(x.y & 0xffff); a.s1 = (int)(int16_t)(x.y >> 16);
     }
-    // this unit's share of the super-block sums: isum = sum_j sc_j * dot_j, imin = sum_j m_j * bsum_j
+    // this unit's share of the super-block sums: isum = sum_j sc_j * dot_j, imin = sum_j m_j * (sum of sub-block j)
     __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &im) {
         int dl = 0, dh = 0;
 #pragma unroll
-        for (int i = 0; i < 4; i++) { dl = dot4(w.lo[i], a.q[i], dl); dh = dot4(w.hi[i], a.q[4 + i], dh); }
+        for (int i = 0; i < 8; i++) { dl = dot4(w.lo[i], a.q[i], dl); dh = dot4(w.hi[i], a.q[8 + i], dh); }
         is = w.sc0 * dl + w.sc1 * dh;
         im = w.m0 * a.s0 + w.m1 * a.s1;
     }
@@ -216,33 +221,31 @@ template <> struct Traits<T_Q4_K> {
         acc = __builtin_fmaf(w.d * a.d, (float)is, acc);
         return __builtin_fmaf(-(w.dmin * a.d), (float)im, acc);
     }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) {
-        const int sb = u >> 3, c = u & 7;
-        return (size_t)sb * 256 + 64 * (c >> 1) + 16 * (c & 1) + 32 * j;
-    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
     __device__ static __forceinline__ void stage_aux(uint8_t *dst, const uint8_t *ws, int64_t K, int u, bool valid) {
         u32x2 x = {0u, 0u};
         if (valid) {
-            const int sb = u >> 3, c = u & 7;
-            const int16_t *bs = reinterpret_cast<const int16_t *>(ws + q8_K_off_bsums(K)) + sb * 16 + 4 * (c >> 1) + (c & 1);
+            const int sb = u >> 2, jp = u & 3;
+            const int16_t *bs = reinterpret_cast<const int16_t *>(ws + q8_K_off_bsums(K)) + sb * 16 + 4 * jp;
             x.x = reinterpret_cast<const uint32_t *>(ws + q8_K_off_d(K))[sb];
-            x.y = (uint32_t)(uint16_t)bs[0] | ((uint32_t)(uint16_t)bs[2] << 16);
+            x.y = (uint32_t)(uint16_t)(bs[0] + bs[1]) | ((uint32_t)(uint16_t)(bs[2] + bs[3]) << 16);
         }
         *reinterpret_cast<u32x2 *>(dst) = x;
     }
     // fused prologue (one wave per super-block sb; lane holds elements 4*lane..4*lane+3 of it)
-    static constexpr int UNITS_PER_SB = 8;
+    static constexpr int UNITS_PER_SB = 4;
     __device__ static __forceinline__ size_t img_qs(int, int e) {
-        const int sb = e >> 8, o = e & 255;
-        const int jp = o >> 6, j = (o >> 5) & 1, cc = (o >> 4) & 1, w = o & 15;
-        const int u = sb * 8 + 2 * jp + cc;
-        return ((size_t)((u >> 6) * QCH + j) * 64 + (u & 63)) * 16 + w;
+        const int u = e >> 6, off = e & 63;
+        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
     }
     __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return img + (size_t)NI * QCH * 1024 + (size_t)u * AUX; }
-    // bsum of 16-value group g of super-block sb: group g = 4*jp + 2*j + cc feeds unit 2*jp + cc, slot j
-    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int g, int s) {
-        const int u = sb * 8 + 2 * (g >> 2) + (g & 1);
-        reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 1] = (int16_t)s;
+    // called by all 64 lanes with the sum of their 16-value group: sub-block sums are two groups (8 lanes)
+    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int lane, int s16) {
+        const int s32 = s16 + __builtin_amdgcn_update_dpp(0, s16, 0x141, 0xf, 0xf, true);
+        if ((lane & 7) == 0) {
+            const int g32 = lane >> 3;                                  // sub-block index 0..7
+            reinterpret_cast<int16_t *>(img_aux(img, NI, sb * 4 + (g32 >> 1)) + 4)[g32 & 1] = (int16_t)s32;
+        }
     }
 };
 
@@ -330,10 +333,13 @@ template <> struct Traits<T_Q6_K> {
         return ((size_t)((u >> 6) * QCH + v) * 64 + (u & 63)) * 16 + w;
     }
     __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return img + (size_t)NI * QCH * 1024 + (size_t)u * AUX; }
-    // bsum of 16-value group g = 8*h + 2*v + ip feeds unit 2*h + ip, slot v
-    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int g, int s) {
-        const int u = sb * 4 + 2 * (g >> 3) + (g & 1);
-        reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 3] = (int16_t)s;
+    // called by all 64 lanes with the sum of their 16-value group g = lane/4 = 8*h + 2*v + ip: unit 2*h + ip, slot v
+    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int lane, int s16) {
+        if ((lane & 3) == 0) {
+            const int g = lane >> 2;
+            const int u = sb * 4 + 2 * (g >> 3) + (g & 1);
+            reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 3] = (int16_t)s16;
+        }
     }
 };
 
@@ -346,34 +352,67 @@ template <int WT> __host__ __device__ constexpr size_t lds_image_bytes(int64_t K
 // ------------------------------------------------------------------------------------------------ kernel
 // Fused prologue: quantize NTOK fp32 rows straight into the LDS image; workgroup 0 also writes the split
 // workspace planes so the quantized activations exist in memory as the reference's wdata does.
+// The fp32 loads are split from their use (xload_* issues them, quantize_* consumes them) so that the caller
+// can put the weight prefetch between the two: all of a thread's loads are then in flight together and the
+// quantization waits only for the activations, which were issued first.
+constexpr int FUSE_MAX_VALUES = 16384;                     // n * K limit of the fused prologue
+
+template <int NTOK, int WGS> struct XRegs { float4 v[FUSE_MAX_VALUES / 4 / WGS]; };
+
 template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void quantize_into_image(uint8_t *lds, size_t img, int NI, const float *__restrict__ x,
-                                                    int64_t ldx, int64_t K, uint8_t *__restrict__ ws, size_t ws_stride) {
+__device__ __forceinline__ void xload(XRegs<NTOK, WGS> &xr, const float *__restrict__ x, int64_t ldx, int64_t K) {
     using T = Traits<WT>;
+    constexpr int SLOTS = FUSE_MAX_VALUES / 4 / WGS;
+    if constexpr (T::ACT == T_Q8_0) {
+        const int nchunk = (int)(K / 4);                                // float4 chunks per token
+        const int per_tok = (nchunk + WGS - 1) / WGS;                   // slots per token
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            const int t = s / per_tok, c = (s - t * per_tok) * WGS + threadIdx.x;
+            xr.v[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (t < NTOK && c < nchunk) xr.v[s] = *reinterpret_cast<const float4 *>(x + t * ldx + 4 * (int64_t)c);
+        }
+    } else {
+        const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+        const int nsb = (int)(K / 256);
+        const int per_tok = (nsb + WGS / 64 - 1) / (WGS / 64);
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            const int t = s / per_tok, sb = (s - t * per_tok) * (WGS / 64) + wv;
+            xr.v[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (t < NTOK && sb < nsb) xr.v[s] = *reinterpret_cast<const float4 *>(x + t * ldx + (int64_t)sb * 256 + 4 * lane);
+        }
+    }
+}
+
+template <int WT, int NTOK, int WGS>
+__device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, uint8_t *lds, size_t img, int NI, int64_t K,
+                                                    uint8_t *__restrict__ ws, size_t ws_stride) {
+    using T = Traits<WT>;
+    constexpr int SLOTS = FUSE_MAX_VALUES / 4 / WGS;
     const bool dump = blockIdx.x == 0 && ws != nullptr;
     if constexpr (T::ACT == T_Q8_0) {
         // 8 lanes per 32-block; K % 256 == 0 keeps every 64-lane group either fully inside or fully outside
         const int nchunk = (int)(K / 4);
-        for (int t = 0; t < NTOK; t++) {
-            uint8_t *im = lds + t * img;
-            for (int c0 = 0; c0 < nchunk; c0 += WGS) {
-                const int c = c0 + threadIdx.x;
-                const bool live = c < nchunk;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (live) v = *reinterpret_cast<const float4 *>(x + t * ldx + 4 * (int64_t)c);
-                const Q8_0Lane q = quantize_q8_0_lane(v);
-                if (live) {
-                    const int e = 4 * c, blk = e >> 5;
-                    *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, e)) = q.packed;
-                    const float d = h2f(q.dh);
-                    if ((threadIdx.x & 7) == 0) T::img_block_aux(im, NI, blk, d, q.sum);
-                    if (dump) {
-                        uint8_t *base = ws + t * ws_stride;
-                        *reinterpret_cast<uint32_t *>(base + e) = q.packed;
-                        if ((threadIdx.x & 7) == 0) {
-                            reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = d;
-                            reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q.sum;
-                        }
+        const int per_tok = (nchunk + WGS - 1) / WGS;
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            const int t = s / per_tok, c = (s - t * per_tok) * WGS + threadIdx.x;
+            if (s >= NTOK * per_tok) break;                             // uniform
+            const bool live = c < nchunk;
+            const Q8_0Lane q = quantize_q8_0_lane(xr.v[s]);
+            if (live) {
+                uint8_t *im = lds + t * img;
+                const int e = 4 * c, blk = e >> 5;
+                *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, e)) = q.packed;
+                const float d = h2f(q.dh);
+                if ((threadIdx.x & 7) == 0) T::img_block_aux(im, NI, blk, d, q.sum);
+                if (dump) {
+                    uint8_t *base = ws + t * ws_stride;
+                    *reinterpret_cast<uint32_t *>(base + e) = q.packed;
+                    if ((threadIdx.x & 7) == 0) {
+                        reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = d;
+                        reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q.sum;
                     }
                 }
             }
@@ -382,14 +421,17 @@ __device__ __forceinline__ void quantize_into_image(uint8_t *lds, size_t img, in
         // one wave per 256-value super-block
         const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
         const int nsb = (int)(K / 256);
-        for (int t = 0; t < NTOK; t++) {
-            uint8_t *im = lds + t * img;
-            for (int sb = wv; sb < nsb; sb += WGS / 64) {
-                const float4 v = *reinterpret_cast<const float4 *>(x + t * ldx + (int64_t)sb * 256 + 4 * lane);
-                const Q8_KLane q = quantize_q8_K_lane(v);
+        const int per_tok = (nsb + WGS / 64 - 1) / (WGS / 64);
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            const int t = s / per_tok, sb = (s - t * per_tok) * (WGS / 64) + wv;
+            if (s >= NTOK * per_tok) break;                             // uniform
+            if (sb < nsb) {                                             // wave-uniform
+                uint8_t *im = lds + t * img;
+                const Q8_KLane q = quantize_q8_K_lane(xr.v[s]);
                 *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, sb * 256 + 4 * lane)) = q.packed;
                 if (lane < T::UNITS_PER_SB) *reinterpret_cast<float *>(T::img_aux(im, NI, sb * T::UNITS_PER_SB + lane)) = q.d;
-                if ((lane & 3) == 0) T::img_bsum(im, NI, sb, lane >> 2, q.bsum);
+                T::img_bsum(im, NI, sb, lane, q.bsum);
                 if (dump) {
                     uint8_t *base = ws + t * ws_stride;
                     *reinterpret_cast<uint32_t *>(base + (size_t)sb * 256 + 4 * lane) = q.packed;
@@ -401,19 +443,35 @@ __device__ __forceinline__ void quantize_into_image(uint8_t *lds, size_t img, in
     }
 }
 
-// Staging from an already quantized workspace: transpose the split planes to [it][chunk][lane].
+// Staging from an already quantized workspace: transpose the split planes to [it][chunk][lane].  Loads are
+// issued eight at a time before their LDS stores so that their latencies overlap.
 template <int WT, int NTOK, int WGS>
 __device__ __forceinline__ void stage_from_workspace(uint8_t *lds, size_t img, int NI, int units, int64_t K,
                                                      const uint8_t *__restrict__ ws, size_t ws_stride) {
     using T = Traits<WT>;
+    constexpr int UN = 8;
     const int nq = NI * T::QCH * 64;                                    // 16-byte chunks per token
-    for (int idx = threadIdx.x; idx < NTOK * nq; idx += WGS) {
-        const int t = idx / nq, r = idx - t * nq;
-        const int lane = r & 63, j = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
-        const int u = it * 64 + lane;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (u < units) v = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + T::src_chunk(K, u, j));
-        reinterpret_cast<u32x4 *>(lds + t * img)[r] = v;
+    for (int base = 0; base < NTOK * nq; base += UN * WGS) {
+        u32x4 v[UN];
+#pragma unroll
+        for (int k = 0; k < UN; k++) {
+            const int idx = base + k * WGS + threadIdx.x;
+            v[k] = u32x4{0u, 0u, 0u, 0u};
+            if (idx < NTOK * nq) {
+                const int t = idx / nq, r = idx - t * nq;
+                const int lane = r & 63, j = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
+                const int u = it * 64 + lane;
+                if (u < units) v[k] = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + T::src_chunk(K, u, j));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < UN; k++) {
+            const int idx = base + k * WGS + threadIdx.x;
+            if (idx < NTOK * nq) {
+                const int t = idx / nq, r = idx - t * nq;
+                reinterpret_cast<u32x4 *>(lds + t * img)[r] = v[k];
+            }
+        }
     }
     const int na = NI * 64;
     for (int idx = threadIdx.x; idx < NTOK * na; idx += WGS) {
@@ -437,60 +495,87 @@ __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W
     const int64_t nwaves = (int64_t)gridDim.x * (WGS / 64);
     const int64_t tiles = ceil_div(N, R);
 
-    // ---- issue the first tile's weight loads, then build the activation image while they fly ----
+    // ---- prologue: activation loads first, then the first tile's weight loads, then the activation image is
+    //      built while the weights are still in flight ----
     typename T::Raw raw[R];
     const bool first_valid = wave < tiles && lane < units;
-    if (first_valid) {
+    if constexpr (FUSEQ) {
+        XRegs<NTOK, WGS> xr;
+        xload<WT, NTOK, WGS>(xr, x, ldx, K);
+        if (first_valid) {
 #pragma unroll
-        for (int r = 0; r < R; r++) T::load_raw(raw[r], W + (size_t)min(wave * R + r, N - 1) * nb01, lane);
+            for (int r = 0; r < R; r++) T::load_raw(raw[r], W + (size_t)min(wave * R + r, N - 1) * nb01, lane);
+        }
+        quantize_into_image<WT, NTOK, WGS>(xr, lds, img, NI, K, ws, ws_stride);
+    } else {
+        if (first_valid) {
+#pragma unroll
+            for (int r = 0; r < R; r++) T::load_raw(raw[r], W + (size_t)min(wave * R + r, N - 1) * nb01, lane);
+        }
+        stage_from_workspace<WT, NTOK, WGS>(lds, img, NI, units, K, ws, ws_stride);
     }
-    if constexpr (FUSEQ) quantize_into_image<WT, NTOK, WGS>(lds, img, NI, x, ldx, K, ws, ws_stride);
-    else                 stage_from_workspace<WT, NTOK, WGS>(lds, img, NI, units, K, ws, ws_stride);
     __syncthreads();
 
-    bool preloaded = true;
-    for (int64_t tile = wave; tile < tiles; tile += nwaves) {
-        const int64_t row0 = tile * R;
-        float acc[R][NTOK];
+    // ---- main loop over this wave's (tile, iteration) steps; the next step's weights are requested right
+    //      after the current step's registers have been decoded, so two steps are in flight per wave ----
+    int64_t tile = wave;
+    int it = 0;
+    bool have = tile < tiles;                                          // wave-uniform
+    float acc[R][NTOK];
 #pragma unroll
-        for (int r = 0; r < R; r++)
+    for (int r = 0; r < R; r++)
 #pragma unroll
-            for (int t = 0; t < NTOK; t++) acc[r][t] = 0.f;
+        for (int t = 0; t < NTOK; t++) acc[r][t] = 0.f;
 
-        for (int it = 0; it < NI; it++) {
-            const int u = it * 64 + lane;
-            if (u < units) {
-                if (!preloaded) {
+    while (have) {
+        const int u = it * 64 + lane;
+        const bool active = u < units;
+        typename T::W w[R];
+        if (active) {
 #pragma unroll
-                    for (int r = 0; r < R; r++)                          // tail tile: re-read the last row, never store it
-                        T::load_raw(raw[r], W + (size_t)min(row0 + r, N - 1) * nb01, u);
-                }
-                typename T::W w[R];
-#pragma unroll
-                for (int r = 0; r < R; r++) T::decode(w[r], raw[r], u);
-#pragma unroll
-                for (int t = 0; t < NTOK; t++) {
-                    typename T::A a;
-                    T::load_a(a, lds + t * img, NI, it, lane);
-#pragma unroll
-                    for (int r = 0; r < R; r++) acc[r][t] = T::dot(w[r], a, acc[r][t]);
-                }
-            }
-            preloaded = false;
+            for (int r = 0; r < R; r++) T::decode(w[r], raw[r], u);
         }
+        const bool last_it = it + 1 == NI;
+        const int64_t ntile = last_it ? tile + nwaves : tile;
+        const int nit = last_it ? 0 : it + 1;
+        const bool nhave = ntile < tiles;
+        if (nhave && nit * 64 + lane < units) {
 #pragma unroll
-        for (int r = 0; r < R; r++)
+            for (int r = 0; r < R; r++)                                  // tail tile: re-read the last row, never store it
+                T::load_raw(raw[r], W + (size_t)min(ntile * R + r, N - 1) * nb01, nit * 64 + lane);
+        }
+        if (active) {
 #pragma unroll
             for (int t = 0; t < NTOK; t++) {
-                const float s = wave_sum_to_lane63(acc[r][t]);
-                if (lane == 63 && row0 + r < N) y[(size_t)t * ldy + row0 + r] = s;
+                typename T::A a;
+                T::load_a(a, lds + t * img, NI, it, lane);
+#pragma unroll
+                for (int r = 0; r < R; r++) acc[r][t] = T::dot(w[r], a, acc[r][t]);
             }
+        }
+        if (last_it) {
+            const int64_t row0 = tile * R;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int t = 0; t < NTOK; t++) {
+                    const float s = wave_sum_to_lane63(acc[r][t]);
+                    if (lane == 63 && row0 + r < N) y[(size_t)t * ldy + row0 + r] = s;
+                    acc[r][t] = 0.f;
+                }
+        }
+        tile = ntile;
+        it = nit;
+        have = nhave;
     }
 }
 
 // ------------------------------------------------------------------------------------------------ launch
-// Rows per wave: units of 32..36 bytes take 4 rows (128..144 bytes per lane in flight), 52..68-byte units take 2.
-template <int WT> struct RowsPerWave { static constexpr int BIG = (WT == T_Q8_0 || WT == T_Q6_K) ? 2 : 4; };
+// Rows per wave step.  Two steps are in flight per wave (the next step's loads are issued before the current
+// step's arithmetic), so one row of a 48..68-byte unit (Q4_K, Q6_K, Q8_0) or two rows of a 36-byte unit (Q4_0)
+// keep about 100..140 bytes per lane outstanding, the depth at which a plain read kernel with the same access
+// pattern peaks on this GPU; measured sweeps over rows x group size x groups per CU agree.
+template <int WT> struct RowsPerWave { static constexpr int R = (WT == T_Q4_0) ? 2 : 1; };
 
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
 static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
@@ -514,20 +599,27 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
     const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    constexpr int RB = RowsPerWave<WT>::BIG, RS = RB / 2;
-    if (lds_bytes <= 40 * 1024) {
-        // 256-thread groups, several per CU.  Matrices with few rows take half the rows per wave so that the
-        // grid still has about 8 waves per CU.
-        const int64_t cap = (int64_t)cus * 8;
-        if (ceil_div(N, RB) >= (int64_t)cus * 8)
-            return launch_one<WT, NTOK, RB, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, st);
-        return launch_one<WT, NTOK, RS, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, st);
+    constexpr int R = RowsPerWave<WT>::R;
+#ifdef CHIP_TUNE
+    if constexpr (NTOK == 1 || NTOK == 4 || NTOK == 8) {
+        const char *ew = getenv("CHIP_TUNE_WGS"), *er = getenv("CHIP_TUNE_R"), *ec = getenv("CHIP_TUNE_CAP");
+        if (ew && er && ec) {
+            const int w = atoi(ew), r = atoi(er); const int64_t cap = (int64_t)cus * atoi(ec);
+#define TUNE_CASE(WW, RR) if (w == WW && r == RR) return launch_one<WT, NTOK, RR, WW, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, st);
+            TUNE_CASE(256, 1) TUNE_CASE(256, 2) TUNE_CASE(256, 4) TUNE_CASE(512, 1) TUNE_CASE(512, 2) TUNE_CASE(512, 4)
+            TUNE_CASE(1024, 1) TUNE_CASE(1024, 2) TUNE_CASE(1024, 4)
+#undef TUNE_CASE
+        }
     }
-    if constexpr (!FUSEQ) {
-        // large images leave room for one group per CU: make it 16 waves wide
-        return launch_one<WT, NTOK, RS, 1024, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, st);
-    }
-    return hipErrorInvalidValue;
+#endif
+    // The activation prologue (staging, or quantizing in the fused variant) is paid once per workgroup, so the
+    // grid is persistent: one or two 8-wave groups per CU, each wave striding over the row tiles.  Matrices with
+    // too few rows to give every CU an 8-wave group use 4-wave groups instead.
+    const int64_t per_cu = (lds_bytes <= 24 * 1024) ? 2 : 1;
+    const int64_t tiles = ceil_div(N, R);
+    if (ceil_div(tiles, 8) >= cus)
+        return launch_one<WT, NTOK, R, 512, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, st);
+    return launch_one<WT, NTOK, R, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, st);
 }
 
 template <int WT, bool FUSEQ>
@@ -579,7 +671,7 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
 // One launch for the whole op: quantize in the prologue.  Worth it while a workgroup's share of that work stays
 // small: n * K <= 16384 values (64 KB of fp32 per workgroup) and n in {1, 2, 4}.
 bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
-    if (!(n == 1 || n == 2 || n == 4) || (int64_t)n * K > 16384) return false;
+    if (!(n == 1 || n == 2 || n == 4) || (int64_t)n * K > FUSE_MAX_VALUES) return false;
     size_t img = 0;
     switch (wtype) {
         case T_Q4_0: img = lds_image_bytes<T_Q4_0>(K); break;
@@ -588,7 +680,7 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
         case T_Q6_K: img = lds_image_bytes<T_Q6_K>(K); break;
         default: return false;
     }
-    return (size_t)n * img <= 40 * 1024 && (size_t)n * img <= (size_t)lim.max_lds_per_block;
+    return (size_t)n * img <= (size_t)lim.max_lds_per_block;
 }
 
 hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
@@ -642,7 +734,7 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
                 }
                 a.d0 = a.d1 = 1.f;
             } else {
-                const int sb = (WT == T_Q4_K) ? (u >> 3) : (u >> 2);
+                const int sb = u >> 2;
                 const uint8_t *blk = arow + (size_t)sb * BYTES_Q8_K;
                 const int16_t *bs = reinterpret_cast<const int16_t *>(blk + 260);
                 for (int j = 0; j < T::QCH; j++) {
@@ -654,8 +746,8 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
                 }
                 a.d = 1.f;
                 if constexpr (WT == T_Q4_K) {
-                    const int c = u & 7;
-                    a.s0 = bs[4 * (c >> 1) + (c & 1)]; a.s1 = bs[4 * (c >> 1) + 2 + (c & 1)];
+                    const int jp = u & 3;
+                    a.s0 = bs[4 * jp] + bs[4 * jp + 1]; a.s1 = bs[4 * jp + 2] + bs[4 * jp + 3];
                 } else {
                     const int h = (u >> 1) & 1, ip = u & 1;
                     for (int v = 0; v < 4; v++) a.bs[v] = bs[8 * h + 2 * v + ip];
@@ -666,8 +758,8 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
         if constexpr (T::ACT == T_Q8_0) {
             if (u < units) { out[2 * u] = v0; out[2 * u + 1] = v1; }
         } else {
-            // sum the units of each super-block (8 lanes for Q4_K, 4 for Q6_K) in integer arithmetic
-            constexpr int G = (WT == T_Q4_K) ? 8 : 4;
+            // sum the four units of each super-block in integer arithmetic
+            constexpr int G = 4;
             for (int m = 1; m < G; m <<= 1) { v0 += __shfl_xor(v0, m); v1 += __shfl_xor(v1, m); }
             if (u < units && (lane % G) == 0) {
                 out[u / G] = v0;
