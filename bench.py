@@ -125,41 +125,47 @@ def bench_headline(dev, hip, steps, warmup):
     st = C.c_void_p()
     dev.check(L.chip_stream_create(C.byref(st)))
 
-    n1_events = []
-
-    def step(timed):
+    def step():
         for m in mats:
             for n in batches:
-                dev.check(L.chip_mul_mat_prepare(ca.Q8_0, m.K, xs[m.K].ptr, m.K, n, ws.ptr, wsz, st))
-                if timed and n == 1:
-                    a, b = hip.event(), hip.event()
-                    hip.record(a, st)
-                dev.check(L.chip_mul_mat_run(ca.Q8_0, m.next(), m.nb01, m.K, m.N, n, ws.ptr, ys.ptr, m.N, st))
-                if timed and n == 1:
-                    hip.record(b, st)
-                    n1_events.append((a, b))
+                dev.check(L.chip_mul_mat(ca.Q8_0, m.next(), m.nb01, m.K, m.N, xs[m.K].ptr, m.K, n, ys.ptr, m.N, ws.ptr, wsz, st))
 
     for _ in range(warmup):
-        step(False)
+        step()
     dev.sync(st)
     e0, e1 = hip.event(), hip.event()
     hip.record(e0, st)
     for _ in range(steps):
-        step(True)
+        step()
     hip.record(e1, st)
     ms = hip.elapsed_ms(e0, e1)
-    dev.sync(st)
 
     step_bytes = sum(algorithmic_bytes(m.bytes, m.K, m.N, n) for m in mats for n in batches)
     ms_per_step = ms / steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    k_us = float(np.mean([hip.elapsed_ms(a, b) for a, b in n1_events])) * 1e3
+
+    # Dominant kernel: the n = 1 GEMV (one launch per op: activation quantization happens in its prologue).
+    # Its own timed region: the same two shapes, cold weights, launches back to back on the same stream between
+    # one HIP event pair (an event between every launch would cost more than the kernel itself).
+    def n1_pass():
+        for m in mats:
+            dev.check(L.chip_mul_mat(ca.Q8_0, m.next(), m.nb01, m.K, m.N, xs[m.K].ptr, m.K, 1, ys.ptr, m.N, ws.ptr, wsz, st))
+
+    reps = max(20, 2 * steps)
+    n1_pass()
+    dev.sync(st)
+    hip.record(e0, st)
+    for _ in range(reps):
+        n1_pass()
+    hip.record(e1, st)
+    k_us = hip.elapsed_ms(e0, e1) * 1e3 / (2 * reps)
+    dev.sync(st)
     k_bytes = algorithmic_bytes(mats[0].bytes, 4096, 11008, 1)      # both shapes move the same byte count
     achieved = k_bytes / (k_us * 1e-6) / 1e9
     roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-            "kernel": "gemv_kernel<Q8_0, n=1> (W[11008x4096] and W[4096x11008], cold weights)",
-            "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 2)}
+            "kernel": "gemv_kernel<Q8_0, n=1, fused activation quantize> (W[11008x4096] and W[4096x11008], cold weights)",
+            "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 2), "launches_timed": 2 * reps}
     return value, ms_per_step, step_bytes, roof, {"copies_per_shape": [m.copies for m in mats]}
 
 

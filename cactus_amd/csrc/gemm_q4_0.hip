@@ -25,6 +25,7 @@
 #include "dev_common.h"
 #include "act_layout.h"
 #include "kernels.h"
+#include <cstdlib>
 
 namespace chip {
 
@@ -45,8 +46,12 @@ struct GemmCfg {
     static constexpr int NW = WR * WC, NT = NW * 64;
     static constexpr int BM = 32 * TM * WR;                        // weight rows per workgroup
     static constexpr int BN = 32 * TN * WC;                        // tokens per workgroup
-    static constexpr int A_CELLS = GEMM_KB * 2 * BM;               // 16-byte cells
-    static constexpr int B_CELLS = GEMM_KB * 2 * BN;
+    // Each (k-block, half) plane of 16-byte cells is padded by two cells: the staging threads that write one
+    // stage walk the planes fastest, and a plane stride that is 2 mod 16 cells puts 16 consecutive writers on
+    // 16 different bank groups (unpadded, all of them hit the same banks).
+    static constexpr int A_PLANE = BM + 2, B_PLANE = BN + 2;
+    static constexpr int A_CELLS = GEMM_KB * 2 * A_PLANE;          // 16-byte cells
+    static constexpr int B_CELLS = GEMM_KB * 2 * B_PLANE;
     static constexpr size_t OFF_A = 0;
     static constexpr size_t OFF_B = OFF_A + (size_t)A_CELLS * 16;
     static constexpr size_t OFF_SW = OFF_B + (size_t)B_CELLS * 16;                 // fp16 [KB][BM], permuted per 32 rows
@@ -60,8 +65,8 @@ struct GemmCfg {
     static constexpr int S_PER_T = (S_ITEMS + NT - 1) / NT;
 };
 
-template <int TM, int TN, int WR, int WC>
-__global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
+template <int TM, int TN, int WR, int WC, int OCC>
+__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_q4_0_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
                                                                 int64_t N, const uint8_t *__restrict__ ws,
                                                                 size_t ws_stride, int64_t M, float *__restrict__ y,
                                                                 int64_t ldy) {
@@ -130,8 +135,8 @@ __global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *_
                 lo.y = nib_to_i8(wq[i].y & 0x0f0f0f0fu); hi.y = nib_to_i8((wq[i].y >> 4) & 0x0f0f0f0fu);
                 lo.z = nib_to_i8(wq[i].z & 0x0f0f0f0fu); hi.z = nib_to_i8((wq[i].z >> 4) & 0x0f0f0f0fu);
                 lo.w = nib_to_i8(wq[i].w & 0x0f0f0f0fu); hi.w = nib_to_i8((wq[i].w >> 4) & 0x0f0f0f0fu);
-                A[(b * 2 + 0) * C::BM + r] = lo;
-                A[(b * 2 + 1) * C::BM + r] = hi;
+                A[(b * 2 + 0) * C::A_PLANE + r] = lo;
+                A[(b * 2 + 1) * C::A_PLANE + r] = hi;
                 // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4;
                 // store the scale of row i at half*16 + (i/8)*4 + i%4 so each lane reads its 16 scales contiguously
                 const int i32 = r & 31;
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *_
             const int item = tid + i * C::NT;
             if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
                 const int c = item % (GEMM_KB * 2), n = item / (GEMM_KB * 2);
-                B[c * C::BN + n] = xq[i];
+                B[c * C::B_PLANE + n] = xq[i];
             }
         }
 #pragma unroll
@@ -197,7 +202,7 @@ __global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *_
 #pragma unroll
             for (int a = 0; a < TM; a++) {
                 const int r0 = (wr * TM + a) * 32;
-                const u32x4 t = A[(b * 2 + half) * C::BM + r0 + l32];
+                const u32x4 t = A[(b * 2 + half) * C::A_PLANE + r0 + l32];
                 af[a] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
                 const u32x4 *sp = SW + ((size_t)b * C::BM + r0 + half * 16) / 8;    // 8 halves per 16-byte cell
                 sw[a][0] = sp[0];
@@ -206,29 +211,46 @@ __global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *_
 #pragma unroll
             for (int c = 0; c < TN; c++) {
                 const int n0 = (wc * TN + c) * 32;
-                const u32x4 t = B[(b * 2 + half) * C::BN + n0 + l32];
+                const u32x4 t = B[(b * 2 + half) * C::B_PLANE + n0 + l32];
                 bf[c] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
                 dx[c] = SX[b * C::BN + n0 + l32];
                 ndx[c] = -MAGIC_F * dx[c];
             }
-            // Software pipeline over the TM*TN tiles of this k-block: the MFMA of tile i+1 is issued before the
-            // 32 scaling operations of tile i, so the matrix unit works underneath the vector unit.
-            i32x16 d_cur = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0], bf[0], magic, 0, 0, 0);
+            if constexpr (OCC >= 4) {
+                // enough waves per SIMD to cover the MFMA latency: consume each result right away (16 fewer VGPRs)
 #pragma unroll
-            for (int i = 0; i < TM * TN; i++) {
-                const int a = i / TN, c = i % TN;
-                i32x16 d_next = d_cur;
-                if (i + 1 < TM * TN) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[(i + 1) / TN], bf[(i + 1) % TN], magic, 0, 0, 0);
-                const uint32_t swd[8] = {sw[a][0].x, sw[a][0].y, sw[a][0].z, sw[a][0].w,
-                                         sw[a][1].x, sw[a][1].y, sw[a][1].z, sw[a][1].w};
+                for (int i = 0; i < TM * TN; i++) {
+                    const int a = i / TN, c = i % TN;
+                    const i32x16 d = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bf[c], magic, 0, 0, 0);
+                    const uint32_t swd[8] = {sw[a][0].x, sw[a][0].y, sw[a][0].z, sw[a][0].w,
+                                             sw[a][1].x, sw[a][1].y, sw[a][1].z, sw[a][1].w};
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const float t = __builtin_fmaf(__int_as_float(d_cur[v]), dx[c], ndx[c]);
-                    const __half hw = __ushort_as_half((unsigned short)((v & 1) ? (swd[v >> 1] >> 16) : (swd[v >> 1] & 0xffffu)));
-                    acc[a][c][v] = __builtin_fmaf(t, __half2float(hw), acc[a][c][v]);
+                    for (int v = 0; v < 16; v++) {
+                        const float t = __builtin_fmaf(__int_as_float(d[v]), dx[c], ndx[c]);
+                        const __half hw = __ushort_as_half((unsigned short)((v & 1) ? (swd[v >> 1] >> 16) : (swd[v >> 1] & 0xffffu)));
+                        acc[a][c][v] = __builtin_fmaf(t, __half2float(hw), acc[a][c][v]);
+                    }
                 }
-                d_cur = d_next;
-                __builtin_amdgcn_sched_barrier(0);
+            } else {
+                // Software pipeline over the TM*TN tiles of this k-block: the MFMA of tile i+1 is issued before
+                // the 32 scaling operations of tile i.
+                i32x16 d_cur = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0], bf[0], magic, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < TM * TN; i++) {
+                    const int a = i / TN, c = i % TN;
+                    i32x16 d_next = d_cur;
+                    if (i + 1 < TM * TN) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[(i + 1) / TN], bf[(i + 1) % TN], magic, 0, 0, 0);
+                    const uint32_t swd[8] = {sw[a][0].x, sw[a][0].y, sw[a][0].z, sw[a][0].w,
+                                             sw[a][1].x, sw[a][1].y, sw[a][1].z, sw[a][1].w};
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const float t = __builtin_fmaf(__int_as_float(d_cur[v]), dx[c], ndx[c]);
+                        const __half hw = __ushort_as_half((unsigned short)((v & 1) ? (swd[v >> 1] >> 16) : (swd[v >> 1] & 0xffffu)));
+                        acc[a][c][v] = __builtin_fmaf(t, __half2float(hw), acc[a][c][v]);
+                    }
+                    d_cur = d_next;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
 
@@ -260,12 +282,12 @@ __global__ __launch_bounds__(WR *WC * 64) void gemm_q4_0_kernel(const uint8_t *_
 
 bool gemm_q4_0_supported(int64_t K, int64_t N, int64_t n) { return K % (32 * GEMM_KB) == 0 && N >= 1 && n >= 1; }
 
-template <int TM, int TN, int WR, int WC>
+template <int TM, int TN, int WR, int WC, int OCC>
 static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
                              float *y, int64_t ldy, hipStream_t st) {
     using C = GemmCfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
-    auto kfn = gemm_q4_0_kernel<TM, TN, WR, WC>;
+    auto kfn = gemm_q4_0_kernel<TM, TN, WR, WC, OCC>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
@@ -280,12 +302,20 @@ hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, co
                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     if (M <= 0 || N <= 0) return hipSuccess;
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    // pick the largest workgroup tile that still leaves about two workgroups' worth of work per CU
-    const int64_t big = ceil_div(N, 128) * ceil_div(M, 256);
-    const int64_t mid = ceil_div(N, 128) * ceil_div(M, 128);
-    if (big >= 2 * cus) return launch_cfg<2, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-    if (mid >= 2 * cus) return launch_cfg<2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-    return launch_cfg<1, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+    // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
+    // every CU such a group fall back to 64 x 128 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
+    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
+    const char *force = getenv("CHIP_GEMM_CFG");
+    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
+    switch (cfg) {
+        case 0: return launch_cfg<1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        case 1: return launch_cfg<1, 2, 2, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        case 2: return launch_cfg<2, 2, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        case 3: return launch_cfg<2, 2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        case 4: return launch_cfg<1, 2, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        case 5: return launch_cfg<2, 1, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace chip

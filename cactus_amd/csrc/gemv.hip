@@ -617,6 +617,11 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
     // too few rows to give every CU an 8-wave group use 4-wave groups instead.
     const int64_t per_cu = (lds_bytes <= 24 * 1024) ? 2 : 1;
     const int64_t tiles = ceil_div(N, R);
+    if constexpr (FUSEQ) {
+        // quantizing a long row costs every group the same work: spread it over 16 waves, one group per CU
+        if ((int64_t)NTOK * K > 8192 && ceil_div(tiles, 16) >= cus)
+            return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, st);
+    }
     if (ceil_div(tiles, 8) >= cus)
         return launch_one<WT, NTOK, R, 512, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, st);
     return launch_one<WT, NTOK, R, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, st);
