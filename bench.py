@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
+# HBM bytes per launch of the n = 1 Q8_0 GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
+# counters read for a device-to-device copy of known size (profiles/gemv_q8_0_n1_hbm_traffic_pmc.md): mean of the
+# two headline shapes.  Algorithmic bytes per launch: 47 967 232.
+N1_GEMV_HBM_TRAFFIC_BYTES = 48334680
 
 
 def parse():
@@ -163,7 +167,7 @@ def bench_headline(dev, hip, steps, warmup):
     k_bytes = algorithmic_bytes(mats[0].bytes, 4096, 11008, 1)      # both shapes move the same byte count
     achieved = k_bytes / (k_us * 1e-6) / 1e9
     roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": N1_GEMV_HBM_TRAFFIC_BYTES,
             "kernel": "gemv_kernel<Q8_0, n=1, fused activation quantize> (W[11008x4096] and W[4096x11008], cold weights)",
             "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 2), "launches_timed": 2 * reps}
     return value, ms_per_step, step_bytes, roof, {"copies_per_shape": [m.copies for m in mats]}
@@ -227,7 +231,29 @@ def bench_extra(dev, hip):
             b.free()
 
     out.update(bench_trace(dev, hip, st, rng))
+    out["mfma_i8_measured_peak"] = measured_mfma_peak()
     return out
+
+
+def measured_mfma_peak():
+    """Runs the issue-rate probe (a child process) and returns the best device-wide rate it saw for the MFMA
+    form the GEMM uses, so TOPS can be read against the measured matrix peak as well as the datasheet one."""
+    import re
+    import subprocess
+    exe = os.path.join(ROOT, "cactus_amd", "lib", "probe_issue_rates")
+    if not os.path.exists(exe):
+        return None
+    try:
+        txt = subprocess.run([exe], capture_output=True, text=True, timeout=60).stdout
+    except Exception:
+        return None
+    best = 0.0
+    for line in txt.splitlines():
+        if line.startswith("mfma_i32_32x32x32_i8"):
+            m = re.search(r";\s*([\d.]+) Tops/s", line)
+            if m:
+                best = max(best, float(m.group(1)))
+    return {"instruction": "v_mfma_i32_32x32x32_i8", "TOPS": best, "datasheet_TOPS": INT8_PEAK_TOPS} if best else None
 
 
 def bench_trace(dev, hip, st, rng):
