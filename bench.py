@@ -258,7 +258,8 @@ def measured_mfma_peak():
 
 def bench_trace(dev, hip, st, rng):
     """config 5: every weight matmul of one decode step of a Llama-3-8B-shaped Q4_K_M model (32 layers, 225
-    matmuls; attn_v / ffn_down / output head in Q6_K, the rest Q4_K), replayed as a HIP graph."""
+    matmuls; attn_v / ffn_down / output head in Q6_K, the rest Q4_K), replayed as a HIP graph, once as a serial
+    chain and once with the independent matmuls of a layer as concurrent graph branches."""
     import cactus_amd as ca
     L = dev.lib
     H, FF, KV, V, NL = 4096, 14336, 1024, 128256, 32
@@ -285,40 +286,86 @@ def bench_trace(dev, hip, st, rng):
         dev.check(L.chip_memcpy_d2d(arena.ptr + head_off + i * (head_bytes // 8), arena.ptr + head_off, head_bytes // 8, None))
     dev.sync()
 
+    hl = hip.lib
+    hl.hipStreamWaitEvent.argtypes = [C.c_void_p, C.c_void_p, C.c_uint]
+    side = [C.c_void_p(), C.c_void_p()]
+    for s_ in side:
+        dev.check(L.chip_stream_create(C.byref(s_)))
+
     res = {}
     for n in (1, 8):
         x_h = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
         x_ff = dev.to_device(rng.standard_normal((n, FF)).astype(np.float32))
-        y = dev.alloc(n * V * 4)
+        y = dev.alloc(3 * n * V * 4)                                   # one output region per concurrent branch
         wsz = max(L.chip_mul_mat_workspace_size(ca.Q6_K, FF, n), L.chip_mul_mat_workspace_size(ca.Q4_K, H, n))
-        ws = dev.alloc(wsz)
+        wss = [dev.alloc(wsz) for _ in range(3)]
+        fused = n <= 4            # chip_mul_mat quantizes in the GEMV prologue: one launch per matmul
 
-        def one_step():
+        def matmul(t, wptr, N, K, src, stream, lane, prepared):
+            yp = y.ptr + lane * n * V * 4
+            if fused:
+                dev.check(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, yp, N, wss[lane].ptr, wsz, stream))
+            else:
+                if not prepared:
+                    dev.check(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, wss[lane].ptr, wsz, stream))
+                dev.check(L.chip_mul_mat_run(t, wptr, dev.row_size(t, K), K, N, n, wss[lane].ptr, yp, N, stream))
+
+        def fork(streams):
+            e = hip.event()
+            hip.record(e, st)
+            for s_ in streams:
+                assert hl.hipStreamWaitEvent(s_, e, 0) == 0
+
+        def join(streams):
+            for s_ in streams:
+                e = hip.event()
+                hip.record(e, s_)
+                assert hl.hipStreamWaitEvent(st, e, 0) == 0
+
+        def one_step(parallel):
+            """serial: the 225 matmuls back to back on one stream (what a one-stream ggml backend issues).
+            parallel: matmuls of a layer that share an input and do not depend on each other (wq/wk/wv; up/gate)
+            run as concurrent branches of the graph; wo and down wait for them."""
             for l in range(NL):
                 base = arena.ptr + l * layer_bytes
-                prepared = None
-                for (name, t, N, K, grp), o in zip(layer, first):
-                    if grp != prepared:            # wq/wk/wv share one quantized input, as do up/gate
-                        src = x_ff if K == FF else x_h
-                        dev.check(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, ws.ptr, wsz, st))
-                        prepared = grp
-                    dev.check(L.chip_mul_mat_run(t, base + o, dev.row_size(t, K), K, N, n, ws.ptr, y.ptr, N, st))
-            dev.check(L.chip_mul_mat_prepare(ca.Q6_K, H, x_h.ptr, H, n, ws.ptr, wsz, st))
-            dev.check(L.chip_mul_mat_run(ca.Q6_K, arena.ptr + head_off, dev.row_size(ca.Q6_K, H), H, V, n, ws.ptr, y.ptr, V, st))
+                W = {name: (t, base + o, N, K) for (name, t, N, K, _), o in zip(layer, first)}
+                if parallel:
+                    fork(side)
+                    matmul(*W["wq"], x_h, st, 0, False)
+                    matmul(*W["wk"], x_h, side[0], 1, False)
+                    matmul(*W["wv"], x_h, side[1], 2, False)
+                    join(side)
+                    matmul(*W["wo"], x_h, st, 0, False)
+                    fork(side[:1])
+                    matmul(*W["up"], x_h, st, 0, False)
+                    matmul(*W["gate"], x_h, side[0], 1, False)
+                    join(side[:1])
+                    matmul(*W["down"], x_ff, st, 0, False)
+                else:
+                    matmul(*W["wq"], x_h, st, 0, False)
+                    matmul(*W["wk"], x_h, st, 0, True)          # wq/wk share the quantized input (both Q8_K planes)
+                    matmul(*W["wv"], x_h, st, 0, True)
+                    matmul(*W["wo"], x_h, st, 0, False)
+                    matmul(*W["up"], x_h, st, 0, False)
+                    matmul(*W["gate"], x_h, st, 0, True)
+                    matmul(*W["down"], x_ff, st, 0, False)
+            matmul(ca.Q6_K, arena.ptr + head_off, V, H, x_h, st, 0, False)
 
-        one_step()
-        dev.sync(st)
-        graph, gexec = C.c_void_p(), C.c_void_p()
-        assert hip.lib.hipStreamBeginCapture(st, 0) == 0
-        one_step()
-        assert hip.lib.hipStreamEndCapture(st, C.byref(graph)) == 0
-        assert hip.lib.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
-        us = time_runs(dev, hip, st, lambda: hip.lib.hipGraphLaunch(gexec, st), 20, warm=2)
         b = total + 4 * n * (NL * sum(K + N for (_, _, N, K, _) in layer) + H + V)
-        res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = {
-            "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1), "weight_bytes": total,
-            "GBps": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4), "matmuls": 7 * NL + 1}
-        for bf in (x_h, x_ff, y, ws):
+        entry = {"weight_bytes": total, "matmuls": 7 * NL + 1}
+        for mode in ("serial", "parallel"):
+            one_step(mode == "parallel")
+            dev.sync(st)
+            graph, gexec = C.c_void_p(), C.c_void_p()
+            assert hl.hipStreamBeginCapture(st, 0) == 0
+            one_step(mode == "parallel")
+            assert hl.hipStreamEndCapture(st, C.byref(graph)) == 0
+            assert hl.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+            us = time_runs(dev, hip, st, lambda: hl.hipGraphLaunch(gexec, st), 20, warm=2)
+            entry[mode] = {"us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
+                           "GBps": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+        res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = entry
+        for bf in [x_h, x_ff, y] + wss:
             bf.free()
     arena.free()
     return res

@@ -24,7 +24,7 @@ struct Q8_0Lane {
     int sum;                // sum of the block's 32 quants (same in the 8 lanes)
 };
 // Eight consecutive lanes hold one 32-value block, four consecutive values each.  All 64 lanes must be active.
-__device__ __forceinline__ Q8_0Lane quantize_q8_0_lane(float4 v) {
+__device__ __forceinline__ Q8_0Lane quantize_q8_0_lane_general(float4 v) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = fmaxf(amax, dpp_get<0xB1>(amax));
     amax = fmaxf(amax, dpp_get<0x4E>(amax));
@@ -52,7 +52,7 @@ struct Q8_KLane {
     int bsum;               // sum of the 16 quants of this lane's group of 4 lanes
 };
 // One wave holds one 256-value super-block, four consecutive values per lane.  All 64 lanes must be active.
-__device__ __forceinline__ Q8_KLane quantize_q8_K_lane(float4 v) {
+__device__ __forceinline__ Q8_KLane quantize_q8_K_lane_general(float4 v) {
     // (amax, max): the first element with the largest magnitude decides, sign kept (strict > in index order)
     float cand = v.x;
     if (fabsf(v.y) > fabsf(cand)) cand = v.y;
@@ -61,7 +61,7 @@ __device__ __forceinline__ Q8_KLane quantize_q8_K_lane(float4 v) {
     const float amax = wave_max_all(fabsf(cand));
     const unsigned long long holders = __ballot(fabsf(cand) == amax);
     const int first = __builtin_ctzll(holders);
-    const float mx = __shfl(cand, first);
+    const float mx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cand), first));
     int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
     Q8_KLane r;
     r.d = 0.f;
@@ -82,6 +82,95 @@ __device__ __forceinline__ Q8_KLane quantize_q8_K_lane(float4 v) {
     s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xf, 0xf, true);
     s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xf, 0xf, true);
     r.bsum = s;
+    return r;
+}
+
+// ---- fast paths -------------------------------------------------------------------------------------------
+// When every input of the wave is finite and the scale cannot overflow, |x * iscale| <= 127.00002, so
+//   * rounding is one add of 1.5 * 2^23 (ties to even, the same result as rint / the reference's magic add),
+//   * the quant is the low byte of that sum's bit pattern, no clamp and no x86 "integer indefinite" case,
+//   * |x| orders like its bit pattern, so the max reduction runs on integers (one DPP instruction per step).
+// Anything else (NaN, infinity, a sum that overflows, a maximum below 1e-30) takes the general functions above;
+// the choice is made per wave, so both paths see full waves.
+template <int CTRL, int ROW_MASK = 0xf, bool BOUND = true>
+__device__ __forceinline__ uint32_t umax_dpp(uint32_t v) {
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, BOUND);
+    return v > o ? v : o;
+}
+__device__ __forceinline__ uint32_t abs_bits(float f) { return __float_as_uint(f) & 0x7fffffffu; }
+__device__ __forceinline__ uint32_t umax4(float4 v) {
+    const uint32_t a = abs_bits(v.x), b = abs_bits(v.y), c = abs_bits(v.z), d = abs_bits(v.w);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+// low bytes of four magic-add sums -> one dword; the sum of the four quants
+__device__ __forceinline__ uint32_t pack_low_bytes(float m0, float m1, float m2, float m3) {
+    const uint32_t lo = __builtin_amdgcn_perm(__float_as_uint(m1), __float_as_uint(m0), 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm(__float_as_uint(m3), __float_as_uint(m2), 0x04000c0cu);
+    return lo | hi;
+}
+constexpr float QUANT_MAGIC = 12582912.f;
+constexpr float QUANT_MIN_AMAX = 1e-30f;
+
+__device__ __forceinline__ Q8_0Lane quantize_q8_0_lane(float4 v) {
+    const float s = (v.x + v.y) + (v.z + v.w);
+    uint32_t am = umax4(v);
+    am = umax_dpp<0xB1>(am);
+    am = umax_dpp<0x4E>(am);
+    am = umax_dpp<0x141>(am);
+    const float amax = __uint_as_float(am);
+    const bool odd = !(fabsf(s) < __builtin_inff()) || (am != 0u && amax < QUANT_MIN_AMAX);
+    if (__ballot(odd) != 0ull) return quantize_q8_0_lane_general(v);
+    const float d = amax / 127.f;
+    const float id = (am != 0u) ? 127.f / amax : 0.0f;
+    const float m0 = v.x * id + QUANT_MAGIC, m1 = v.y * id + QUANT_MAGIC;
+    const float m2 = v.z * id + QUANT_MAGIC, m3 = v.w * id + QUANT_MAGIC;
+    Q8_0Lane r;
+    r.packed = pack_low_bytes(m0, m1, m2, m3);
+    int sum = dot4(r.packed, 0x01010101u, 0);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xf, 0xf, true);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xf, 0xf, true);
+    r.dh = f2h_rne(d);
+    r.sum = sum;
+    return r;
+}
+
+__device__ __forceinline__ Q8_KLane quantize_q8_K_lane(float4 v) {
+    const float s = (v.x + v.y) + (v.z + v.w);
+    // first element with the largest magnitude, sign kept (strict > in index order)
+    float cand = v.x;
+    uint32_t cb = abs_bits(v.x);
+    if (abs_bits(v.y) > cb) { cand = v.y; cb = abs_bits(v.y); }
+    if (abs_bits(v.z) > cb) { cand = v.z; cb = abs_bits(v.z); }
+    if (abs_bits(v.w) > cb) { cand = v.w; cb = abs_bits(v.w); }
+    uint32_t am = cb;
+    am = umax_dpp<0xB1>(am);
+    am = umax_dpp<0x4E>(am);
+    am = umax_dpp<0x141>(am);
+    am = umax_dpp<0x140>(am);                      // every lane of a 16-lane row holds the row maximum
+    am = umax_dpp<0x142, 0xa, false>(am);          // rows 1 and 3 take in rows 0 and 2
+    am = umax_dpp<0x143, 0xc, false>(am);          // lane 63 holds the wave maximum
+    am = (uint32_t)__builtin_amdgcn_readlane((int)am, 63);
+    const bool odd = !(fabsf(s) < __builtin_inff()) || (am != 0u && __uint_as_float(am) < QUANT_MIN_AMAX);
+    if (__ballot(odd) != 0ull) return quantize_q8_K_lane_general(v);
+    Q8_KLane r;
+    if (am == 0u) {                                // wave-uniform
+        r.packed = 0u; r.d = 0.f; r.bsum = 0;
+        return r;
+    }
+    const unsigned long long holders = __ballot(cb == am);
+    const int first = __builtin_ctzll(holders);
+    const float mx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cand), first));
+    const float iscale = -127.f / mx;
+    const float m0 = iscale * v.x + QUANT_MAGIC, m1 = iscale * v.y + QUANT_MAGIC;
+    const float m2 = iscale * v.z + QUANT_MAGIC, m3 = iscale * v.w + QUANT_MAGIC;
+    r.packed = pack_low_bytes(m0, m1, m2, m3);
+    r.d = 1.0f / iscale;
+    int sum = dot4(r.packed, 0x01010101u, 0);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xf, 0xf, true);
+    r.bsum = sum;
     return r;
 }
 
