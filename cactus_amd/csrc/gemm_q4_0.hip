@@ -284,14 +284,12 @@ bool gemm_q4_0_supported(int64_t K, int64_t N, int64_t n) { return K % (32 * GEM
 
 template <int TM, int TN, int WR, int WC, int OCC>
 static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                             float *y, int64_t ldy, hipStream_t st) {
+                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     using C = GemmCfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
     auto kfn = gemm_q4_0_kernel<TM, TN, WR, WC, OCC>;
-    if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return e;
-    }
+    static LdsGrant grant;                                               // one per kernel instantiation
+    if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     dim3 grid((unsigned)ceil_div(N, C::BM), (unsigned)ceil_div(M, C::BN));
     hipLaunchKernelGGL(kfn, grid, dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws, ws_stride,
                        M, y, ldy);
@@ -308,12 +306,12 @@ hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, co
     const char *force = getenv("CHIP_GEMM_CFG");
     const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
     switch (cfg) {
-        case 0: return launch_cfg<1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-        case 1: return launch_cfg<1, 2, 2, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-        case 2: return launch_cfg<2, 2, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-        case 3: return launch_cfg<2, 2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-        case 4: return launch_cfg<1, 2, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
-        case 5: return launch_cfg<2, 1, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, st);
+        case 0: return launch_cfg<1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 1: return launch_cfg<1, 2, 2, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 2: return launch_cfg<2, 2, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 3: return launch_cfg<2, 2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 4: return launch_cfg<1, 2, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 5: return launch_cfg<2, 1, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }

@@ -672,15 +672,14 @@ template <int WT> struct RowsPerWave { static constexpr int R = (WT == T_Q4_0) ?
 #endif
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
 static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
-                             size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, hipStream_t st) {
+                             size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, const DeviceLimits &lim,
+                             hipStream_t st) {
     const int64_t tiles = ceil_div(N, R);
     int64_t groups = ceil_div(tiles, WGS / 64);
     if (groups > max_groups) groups = max_groups;
     auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, GEMV_DEPTH>;
-    if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return e;
-    }
+    static LdsGrant grant;                                               // one per kernel instantiation
+    if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
                        (uint8_t *)ws, ws_stride, y, ldy);
     return hipGetLastError();
@@ -698,7 +697,7 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         const char *ew = getenv("CHIP_TUNE_WGS"), *er = getenv("CHIP_TUNE_R"), *ec = getenv("CHIP_TUNE_CAP");
         if (ew && er && ec) {
             const int w = atoi(ew), r = atoi(er); const int64_t cap = (int64_t)cus * atoi(ec);
-#define TUNE_CASE(WW, RR) if (w == WW && r == RR) return launch_one<WT, NTOK, RR, WW, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, st);
+#define TUNE_CASE(WW, RR) if (w == WW && r == RR) return launch_one<WT, NTOK, RR, WW, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, lim, st);
             TUNE_CASE(256, 1) TUNE_CASE(256, 2) TUNE_CASE(256, 4) TUNE_CASE(512, 1) TUNE_CASE(512, 2) TUNE_CASE(512, 4)
             TUNE_CASE(1024, 1) TUNE_CASE(1024, 2) TUNE_CASE(1024, 4)
 #undef TUNE_CASE
@@ -717,11 +716,11 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         const bool one_tile_per_wave = tiles <= 16 * (int64_t)cus && tiles > 8 * (int64_t)cus;
         const bool long_q8_0_row = Traits<WT>::ACT == T_Q8_0 && NTOK == 1 && K > 8192;
         if (one_tile_per_wave && !long_q8_0_row)
-            return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, st);
+            return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st);
     }
     if (ceil_div(tiles, 8) >= cus)
-        return launch_one<WT, NTOK, R, 512, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, st);
-    return launch_one<WT, NTOK, R, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, st);
+        return launch_one<WT, NTOK, R, 512, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, lim, st);
+    return launch_one<WT, NTOK, R, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, lim, st);
 }
 
 template <int WT, bool FUSEQ>

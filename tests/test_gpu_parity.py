@@ -137,6 +137,22 @@ def test_mul_mat_token_groups(dev, orc, wt):
     check_outputs(dev.mul_mat(wt, wq, x), ref["y"], ref["sum_abs"], "token groups")
 
 
+@pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (14336, 4096)])
+@pytest.mark.parametrize("n", [5, 8, 9, 16, 17, 37])
+def test_mul_mat_q8_0_matrix_core_gemv(dev, orc, K, N, n):
+    # enough 16-row tiles for every CU and 5+ tokens: the integer sums come from v_mfma_i32_16x16x64_i8;
+    # ragged N (last tile partly outside), token counts on both sides of the 8- and 16-token images
+    print("mmv q8_0 K", K, "N", N, "n", n, flush=True)
+    wq = orc.quantize_weights(O.Q8_0, common.weights_f32(K + N, N, K))
+    x = common.activations_f32(K + n, n, K)
+    x[2] = 0
+    x[3] *= 250
+    ref = orc.mul_mat(O.Q8_0, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(O.Q8_0, wq, x, want_workspace_blocks=True)
+    assert np.array_equal(blocks, ref["wdata"])
+    check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv")
+
+
 # ------------------------------------------------------------------------------------------ BASELINE sizes
 def test_config1_q4_0_4096(dev, orc):
     K = N = 4096
