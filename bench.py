@@ -30,7 +30,7 @@ INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
 # HBM bytes per launch of the n = 1 Q8_0 GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a device-to-device copy of known size (profiles/gemv_q8_0_n1_hbm_traffic_pmc.md): mean of the
 # two headline shapes.  Algorithmic bytes per launch: 47 967 232.
-N1_GEMV_HBM_TRAFFIC_BYTES = 48334680
+N1_GEMV_HBM_TRAFFIC_BYTES = 48350573
 
 
 def parse():
