@@ -19,8 +19,10 @@ KERNEL_LIB = os.path.join(LIB_DIR, "libcactus_hip.so")
 BACKEND_LIB = os.path.join(LIB_DIR, "libggml-hip.so")
 
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
-TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K"}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K)
+Q5_0, Q5_K, IQ4_NL = 6, 13, 20
+TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
+              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl"}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL)
 
 # every symbol include/cactus_hip.h declares
 EXPORTS = (
@@ -192,7 +194,7 @@ class Device:
         return y
 
     def block_isums(self, wtype, W, aq, k):
-        """Per-block integer sums [n, N, K/block] (and imin for Q4_K) from reference-layout activation blocks."""
+        """Per-block integer sums [n, N, K/block] (and imin for Q4_K / Q5_K) from reference-layout activation blocks."""
         W = np.ascontiguousarray(W, np.uint8)
         aq = np.ascontiguousarray(aq, np.uint8)
         N, n = W.shape[0], aq.shape[0]
@@ -203,5 +205,5 @@ class Device:
         self.check(self.lib.chip_block_isums(wtype, dW.ptr, W.shape[1], k, N, da.ptr, n, di.ptr, dm.ptr, None))
         self.sync()
         isum = di.download(np.int32, n * N * nblk).reshape(n, N, nblk)
-        imin = dm.download(np.int32, n * N * nblk).reshape(n, N, nblk) if wtype == Q4_K else None
+        imin = dm.download(np.int32, n * N * nblk).reshape(n, N, nblk) if wtype in (Q4_K, Q5_K) else None
         return isum, imin

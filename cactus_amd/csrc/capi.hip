@@ -49,7 +49,9 @@ int current_limits(DeviceLimits &out) {
     return CHIP_OK;
 }
 
-bool is_weight_type(int t) { return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K; }
+bool is_weight_type(int t) {
+    return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K || t == T_Q5_0 || t == T_Q5_K || t == T_IQ4_NL;
+}
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // Q4_0 / Q8_0 / Q4_K rows of K % 256 == 0 elements are multiples of 16 bytes and the kernels load them with
@@ -164,8 +166,8 @@ int chip_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((
 int chip_block_elems(int type) {
     switch (type) {
         case T_F32: return 1;
-        case T_Q4_0: case T_Q8_0: return 32;
-        case T_Q4_K: case T_Q6_K: case T_Q8_K: return 256;
+        case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return 32;
+        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: return 256;
         default: return 0;
     }
 }
@@ -177,6 +179,9 @@ size_t chip_block_bytes(int type) {
         case T_Q4_K: return BYTES_Q4_K;
         case T_Q6_K: return BYTES_Q6_K;
         case T_Q8_K: return BYTES_Q8_K;
+        case T_Q5_0: return BYTES_Q5_0;
+        case T_Q5_K: return BYTES_Q5_K;
+        case T_IQ4_NL: return BYTES_IQ4_NL;
         default: return 0;
     }
 }
@@ -186,8 +191,8 @@ size_t chip_row_size(int type, int64_t k) {
 }
 int chip_vec_dot_type(int type) {
     switch (type) {
-        case T_Q4_0: case T_Q8_0: return T_Q8_0;
-        case T_Q4_K: case T_Q6_K: return T_Q8_K;
+        case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return T_Q8_0;
+        case T_Q4_K: case T_Q6_K: case T_Q5_K: return T_Q8_K;
         default: return -1;
     }
 }
@@ -303,7 +308,7 @@ int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     if (N == 0 || n == 0) return CHIP_OK;
     if (!W || !aq || !isum) return CHIP_EINVAL;
     if (!weights_aligned(type, W, nb01) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;
-    return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, type == T_Q4_K ? imin : nullptr, (hipStream_t)stream));
+    return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, (type == T_Q4_K || type == T_Q5_K) ? imin : nullptr, (hipStream_t)stream));
 }
 
 int chip_workspace_to_blocks(int type, int64_t K, int64_t n, const void *workspace, void *y, void *stream) {

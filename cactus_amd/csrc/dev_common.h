@@ -12,8 +12,9 @@ namespace chip {
 constexpr int QK_SMALL = 32;     // elements per Q4_0 / Q8_0 block
 constexpr int QK_K     = 256;    // elements per K-quant super-block
 constexpr int BYTES_Q4_0 = 18, BYTES_Q8_0 = 34, BYTES_Q4_K = 144, BYTES_Q6_K = 210, BYTES_Q8_K = 292;
+constexpr int BYTES_Q5_0 = 22, BYTES_Q5_K = 176, BYTES_IQ4_NL = 18;
 
-enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15 };
+enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15, T_Q5_0 = 6, T_Q5_K = 13, T_IQ4_NL = 20 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -22,6 +23,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
 typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
+typedef u32x2 u32x2_a4 __attribute__((aligned(4)));
 typedef uint32_t u32_a2 __attribute__((aligned(2)));
 
 __device__ __forceinline__ float h2f(uint32_t h16) {

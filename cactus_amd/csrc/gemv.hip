@@ -44,6 +44,7 @@ template <int WT> struct Traits;
 
 template <> struct Traits<T_Q8_0> {
     static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
+    static constexpr bool A_HAS_SUMS = false;                   // A carries the per-block activation sums
     struct W { uint32_t q[16]; float d0, d1; };
     struct A { uint32_t q[16]; float d0, d1; };
     struct Raw { u32x4 a, b, c, e; uint32_t f; };
@@ -108,6 +109,7 @@ template <> struct Traits<T_Q8_0> {
 
 template <> struct Traits<T_Q4_0> {
     static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
+    static constexpr bool A_HAS_SUMS = true;
     struct W { uint32_t lo[8], hi[8]; float d0, d1; };          // nibbles spread to bytes, 0..15
     struct A { uint32_t q[16]; float d0, d1; int s0, s1; };
 
@@ -181,6 +183,7 @@ template <> struct Traits<T_Q4_K> {
     // elements 64*jp + [0,32) (sub-block 2*jp) and whose high nibbles are elements 64*jp + 32 + [0,32)
     // (sub-block 2*jp+1).  The matching activations are the 64 contiguous quants 64*jp..64*jp+63.
     static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
+    static constexpr int KQ_STYLE = 0;                          // activation side data: two 32-value sub-block sums
     struct W { uint32_t lo[8], hi[8]; float d, dmin; int sc0, sc1, m0, m1; };
     struct A { uint32_t q[16]; float d; int s0, s1; };
     struct Raw { u32x4 h, q0, q1; };
@@ -265,6 +268,7 @@ template <> struct Traits<T_Q6_K> {
     // unit = (super-block sb, half h, ip): 16 consecutive l = 16*ip + [0,16) of half h, i.e. the four
     // 16-element groups {128h + 32v + 16ip + [0,16) : v = 0..3}; scale of group v is scales[8h + 2v + ip]
     static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
+    static constexpr int KQ_STYLE = 1;                          // four 16-value group sums
     struct W { uint32_t q[16]; float d; int sc[4]; };            // q[4v + k]: 6-bit values 0..63 of group v
     struct A { uint32_t q[16]; float d; int bs[4]; };
 
@@ -354,6 +358,168 @@ template <> struct Traits<T_Q6_K> {
             reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 3] = (int16_t)s16;
         }
     }
+};
+
+// ---- further weight types (reference type_traits_cpu[], ggml-cpu/ggml-cpu.c:198-367): same activation formats
+template <> struct Traits<T_Q5_0> {
+    // block_q5_0 (ggml-common.h:187-193): fp16 d, 32 high bits qh, 16 nibble bytes; value = d * (q5 - 16),
+    // q5 = nibble | bit << 4, bit j of qh for element j (low nibbles), bit j + 16 for element j + 16 (high nibbles)
+    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
+    static constexpr bool A_HAS_SUMS = true;
+    struct W { uint32_t lo[8], hi[8]; float d0, d1; };          // 5-bit values spread to bytes, 0..31
+    struct A { uint32_t q[16]; float d0, d1; int s0, s1; };
+    struct Raw { u32x4 a, b; u32x2 c; uint32_t e; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        const uint8_t *p = row + (size_t)u * 44;                       // two 22-byte blocks, 4-byte aligned
+        r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
+        r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
+        r.c = WLOAD(reinterpret_cast<const u32x2_a4 *>(p + 32));
+        r.e = WLOAD(reinterpret_cast<const uint32_t *>(p + 40));
+    }
+    // four high bits -> bit 4 of four bytes
+    __device__ static __forceinline__ uint32_t spread4(uint32_t bits) { return (((bits & 0xFu) * 0x00204081u) & 0x01010101u) << 4; }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
+        const uint32_t d[11] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y, r.e};
+        // block 0: d at bytes 0..1, qh at 2..5, qs at 6..21; block 1: d at 22..23, qh at 24..27, qs at 28..43
+        w.d0 = h2f(d[0]);
+        w.d1 = h2f(d[5] >> 16);
+        const uint32_t qh0 = shr16(d[1], d[0]), qh1 = d[6];
+        const uint32_t q0[4] = {shr16(d[2], d[1]), shr16(d[3], d[2]), shr16(d[4], d[3]), shr16(d[5], d[4])};
+        const uint32_t q1[4] = {d[7], d[8], d[9], d[10]};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w.lo[i]     = (q0[i] & 0x0f0f0f0fu)        | spread4(qh0 >> (4 * i));
+            w.hi[i]     = ((q0[i] >> 4) & 0x0f0f0f0fu) | spread4(qh0 >> (16 + 4 * i));
+            w.lo[4 + i] = (q1[i] & 0x0f0f0f0fu)        | spread4(qh1 >> (4 * i));
+            w.hi[4 + i] = ((q1[i] >> 4) & 0x0f0f0f0fu) | spread4(qh1 >> (16 + 4 * i));
+        }
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
+        const u32x4 x = reinterpret_cast<const u32x4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
+        a.d0 = __uint_as_float(x.x); a.d1 = __uint_as_float(x.y); a.s0 = (int)x.z; a.s1 = (int)x.w;
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
+        i0 = -16 * a.s0; i1 = -16 * a.s1;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            i0 = dot4(w.lo[i], a.q[i], i0);         i0 = dot4(w.hi[i], a.q[4 + i], i0);
+            i1 = dot4(w.lo[4 + i], a.q[8 + i], i1); i1 = dot4(w.hi[4 + i], a.q[12 + i], i1);
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int i0, i1;
+        isums(w, a, i0, i1);
+        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
+        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
+    using AuxT = u32x4;
+    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q4_0>::aux_load(ws, K, u, valid); }
+    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_0>::img_qs(NI, e); }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum) { Traits<T_Q4_0>::img_block_aux(img, NI, blk, d, sum); }
+};
+
+template <> struct Traits<T_IQ4_NL> {
+    // block_iq4_nl (ggml-common.h:405-410): fp16 d, 16 nibble bytes; value = d * codebook[nibble]
+    // (ggml-quants.c:2428), low nibbles are elements 0..15, high nibbles 16..31
+    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
+    static constexpr bool A_HAS_SUMS = false;
+    struct W { uint32_t q[16]; float d0, d1; };                 // signed code points, element order
+    using A = Traits<T_Q8_0>::A;
+    using Raw = Traits<T_Q4_0>::Raw;
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) { Traits<T_Q4_0>::load_raw(r, row, u); }
+    // four code indices (one per byte, 0..15) -> four code points, through two byte permutes of the 16-entry table
+    __device__ static __forceinline__ uint32_t lookup4(uint32_t idx) {
+        constexpr uint32_t T0 = 0xbfad9881u, T1 = 0xf6eaddcfu, T2 = 0x26190d01u, T3 = 0x71594535u;
+        const uint32_t sel = idx & 0x07070707u;
+        const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel), hi = __builtin_amdgcn_perm(T3, T2, sel);
+        const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xffu;
+        return (lo & ~m) | (hi & m);
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
+        const u32x4 a = r.a, b = r.b;
+        const uint32_t c = r.c;
+        uint32_t q[8];
+        w.d0 = h2f(a.x);
+        q[0] = shr16(a.y, a.x); q[1] = shr16(a.z, a.y); q[2] = shr16(a.w, a.z); q[3] = shr16(b.x, a.w);
+        w.d1 = h2f(b.x >> 16);
+        q[4] = b.y; q[5] = b.z; q[6] = b.w; q[7] = c;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w.q[i]      = lookup4(q[i] & 0x0f0f0f0fu);        w.q[4 + i]  = lookup4((q[i] >> 4) & 0x0f0f0f0fu);
+            w.q[8 + i]  = lookup4(q[4 + i] & 0x0f0f0f0fu);    w.q[12 + i] = lookup4((q[4 + i] >> 4) & 0x0f0f0f0fu);
+        }
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) { Traits<T_Q8_0>::load_a(a, tok, NI, it, lane); }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
+        i0 = 0; i1 = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { i0 = dot4(w.q[i], a.q[i], i0); i1 = dot4(w.q[8 + i], a.q[8 + i], i1); }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int i0, i1;
+        isums(w, a, i0, i1);
+        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
+        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
+    using AuxT = float2;
+    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q8_0>::aux_load(ws, K, u, valid); }
+    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q8_0>::img_qs(NI, e); }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum) { Traits<T_Q8_0>::img_block_aux(img, NI, blk, d, sum); }
+};
+
+template <> struct Traits<T_Q5_K> {
+    // block_q5_K (ggml-common.h:303-314): as q4_K plus qh[32]: bit 2jp of qh[l] is the fifth bit of element l of
+    // sub-block 2jp (low nibbles of the group's 32 qs bytes), bit 2jp+1 that of sub-block 2jp+1 (high nibbles)
+    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
+    static constexpr int KQ_STYLE = 0;
+    using W = Traits<T_Q4_K>::W;
+    using A = Traits<T_Q4_K>::A;
+    struct Raw { u32x4 h, qh0, qh1, q0, q1; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        const int sb = u >> 2, jp = u & 3;
+        const uint8_t *p = row + (size_t)sb * BYTES_Q5_K;              // 176-byte super-block, 16-byte aligned
+        r.h = WLOAD(reinterpret_cast<const u32x4 *>(p));
+        r.qh0 = WLOAD(reinterpret_cast<const u32x4 *>(p + 16));
+        r.qh1 = WLOAD(reinterpret_cast<const u32x4 *>(p + 32));
+        r.q0 = WLOAD(reinterpret_cast<const u32x4 *>(p + 48 + 32 * jp));
+        r.q1 = WLOAD(reinterpret_cast<const u32x4 *>(p + 64 + 32 * jp));
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+        const int jp = u & 3;
+        const u32x4 h = r.h;
+        w.d = h2f(h.x); w.dmin = h2f(h.x >> 16);
+        const int sh = 16 * (jp & 1);
+        const uint32_t a1 = h.y >> sh, a2 = h.z >> sh, a3 = h.w >> sh;
+        uint32_t sc, mn;
+        if (jp < 2) { sc = a1 & 0x3f3fu; mn = a2 & 0x3f3fu; }
+        else        { sc = (a3 & 0x0f0fu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
+        w.sc0 = sc & 0xff; w.sc1 = sc >> 8; w.m0 = mn & 0xff; w.m1 = mn >> 8;
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t hb[8] = {r.qh0.x, r.qh0.y, r.qh0.z, r.qh0.w, r.qh1.x, r.qh1.y, r.qh1.z, r.qh1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            w.lo[i] = (q[i] & 0x0f0f0f0fu)        | (((hb[i] >> (2 * jp)) & 0x01010101u) << 4);
+            w.hi[i] = ((q[i] >> 4) & 0x0f0f0f0fu) | (((hb[i] >> (2 * jp + 1)) & 0x01010101u) << 4);
+        }
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) { Traits<T_Q4_K>::load_a(a, tok, NI, it, lane); }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &im) { Traits<T_Q4_K>::isums(w, a, is, im); }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) { return Traits<T_Q4_K>::dot(w, a, acc); }
+    __device__ static __forceinline__ size_t src_chunk(int64_t K, int u, int j) { return Traits<T_Q4_K>::src_chunk(K, u, j); }
+    using AuxT = u32x2;
+    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q4_K>::aux_load(ws, K, u, valid); }
+    static constexpr int UNITS_PER_SB = 4;
+    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_K>::img_qs(NI, e); }
+    __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return Traits<T_Q4_K>::img_aux(img, NI, u); }
+    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int lane, int s16) { Traits<T_Q4_K>::img_bsum(img, NI, sb, lane, s16); }
 };
 
 template <int WT> __host__ __device__ constexpr int units_per_row(int64_t K) { return (int)(K / Traits<WT>::UNIT_ELEMS); }
@@ -752,6 +918,9 @@ int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
         case T_Q8_0: return max_tokens_typed<T_Q8_0>(K, lim);
         case T_Q4_K: return max_tokens_typed<T_Q4_K>(K, lim);
         case T_Q6_K: return max_tokens_typed<T_Q6_K>(K, lim);
+        case T_Q5_0: return max_tokens_typed<T_Q5_0>(K, lim);
+        case T_Q5_K: return max_tokens_typed<T_Q5_K>(K, lim);
+        case T_IQ4_NL: return max_tokens_typed<T_IQ4_NL>(K, lim);
         default: return 0;
     }
 }
@@ -765,6 +934,9 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
         case T_Q8_0: return launch_ntok<T_Q8_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q4_K: return launch_ntok<T_Q4_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q6_K: return launch_ntok<T_Q6_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q5_0: return launch_ntok<T_Q5_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_IQ4_NL: return launch_ntok<T_IQ4_NL, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
@@ -779,6 +951,9 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
         case T_Q8_0: img = lds_image_bytes<T_Q8_0>(K); break;
         case T_Q4_K: img = lds_image_bytes<T_Q4_K>(K); break;
         case T_Q6_K: img = lds_image_bytes<T_Q6_K>(K); break;
+        case T_Q5_0: img = lds_image_bytes<T_Q5_0>(K); break;
+        case T_Q5_K: img = lds_image_bytes<T_Q5_K>(K); break;
+        case T_IQ4_NL: img = lds_image_bytes<T_IQ4_NL>(K); break;
         default: return false;
     }
     return (size_t)n * img <= (size_t)lim.max_lds_per_block;
@@ -792,6 +967,9 @@ hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, i
         case T_Q8_0: return launch_ntok<T_Q8_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         case T_Q4_K: return launch_ntok<T_Q4_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         case T_Q6_K: return launch_ntok<T_Q6_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q5_0: return launch_ntok<T_Q5_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q5_K: return launch_ntok<T_Q5_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_IQ4_NL: return launch_ntok<T_IQ4_NL, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
@@ -831,7 +1009,7 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
                         a.q[8 * b + i] = d;
                         s = dot4(d, 0x01010101u, s);
                     }
-                    if constexpr (WT == T_Q4_0) { if (b == 0) a.s0 = s; else a.s1 = s; }
+                    if constexpr (T::A_HAS_SUMS) { if (b == 0) a.s0 = s; else a.s1 = s; }
                 }
                 a.d0 = a.d1 = 1.f;
             } else {
@@ -846,7 +1024,7 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
                     }
                 }
                 a.d = 1.f;
-                if constexpr (WT == T_Q4_K) {
+                if constexpr (T::KQ_STYLE == 0) {
                     const int jp = u & 3;
                     a.s0 = bs[4 * jp] + bs[4 * jp + 1]; a.s1 = bs[4 * jp + 2] + bs[4 * jp + 3];
                 } else {
@@ -879,6 +1057,9 @@ hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, 
         case T_Q8_0: hipLaunchKernelGGL(block_isums_kernel<T_Q8_0>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q4_K: hipLaunchKernelGGL(block_isums_kernel<T_Q4_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q6_K: hipLaunchKernelGGL(block_isums_kernel<T_Q6_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q5_0: hipLaunchKernelGGL(block_isums_kernel<T_Q5_0>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q5_K: hipLaunchKernelGGL(block_isums_kernel<T_Q5_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_IQ4_NL: hipLaunchKernelGGL(block_isums_kernel<T_IQ4_NL>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

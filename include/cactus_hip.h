@@ -31,6 +31,10 @@ enum chip_type {
     CHIP_TYPE_Q4_K = 12,
     CHIP_TYPE_Q6_K = 14,
     CHIP_TYPE_Q8_K = 15,
+    /* further weight types of type_traits_cpu[] (ggml-cpu/ggml-cpu.c:229,278,340) */
+    CHIP_TYPE_Q5_0   = 6,
+    CHIP_TYPE_Q5_K   = 13,
+    CHIP_TYPE_IQ4_NL = 20,
 };
 
 enum chip_status {
@@ -74,7 +78,8 @@ CHIP_API int         chip_stream_synchronize(void *stream);
 CHIP_API int    chip_block_elems(int type);
 CHIP_API size_t chip_block_bytes(int type);
 CHIP_API size_t chip_row_size(int type, int64_t k);
-/* type_traits_cpu[type].vec_dot_type (ggml-cpu/ggml-cpu.c:198-367): Q8_0 for Q4_0/Q8_0, Q8_K for Q4_K/Q6_K */
+/* type_traits_cpu[type].vec_dot_type (ggml-cpu/ggml-cpu.c:198-367): Q8_0 for Q4_0/Q8_0/Q5_0/IQ4_NL, Q8_K for
+ * Q4_K/Q5_K/Q6_K */
 CHIP_API int    chip_vec_dot_type(int type);
 /* 1 if chip_mul_mat accepts this weight type and K (K must be a multiple of 256) */
 CHIP_API int    chip_mul_mat_supported(int type, int64_t K);
@@ -97,7 +102,8 @@ CHIP_API int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t 
  *   workspace : device scratch of at least chip_mul_mat_workspace_size(type, K, n) bytes (params->wdata in the
  *               reference, sized by lm_ggml_graph_plan, ggml-cpu/ggml-cpu.c:2697-2704); holds the quantized
  *               activations in a kernel-private layout
- * n <= 8 runs the bandwidth-bound GEMV; larger n runs the int8-MFMA GEMM (Q4_0) or the GEMV in token groups.
+ * n <= 4 runs the dot-product GEMV with the quantizer in its prologue; Q8_0 with n >= 5 the matrix-core GEMV
+ * (16 tokens per pass over W); Q4_0 with n >= 16 the int8-MFMA GEMM; everything else the GEMV in token groups.
  * K must be a multiple of 256.  W must be 16-byte aligned and nb01 a multiple of 16 (2 and 2 for Q6_K, whose
  * 210-byte blocks allow no more); x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
  */
@@ -116,11 +122,12 @@ CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, i
                               const void *workspace, float *y, int64_t ldy, void *stream);
 
 /* ---- verification hooks ----
- * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K}
- * (ggml-cpu/ggml-cpu-quants.c:1906,3591,6772,8520), computed with the same device code the GEMV uses.
+ * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,
+ * iq4_nl_q8_0} (ggml-cpu/ggml-cpu-quants.c:1906,3591,6772,8520,2924,7699,12751), computed with the same device
+ * code the GEMV uses.
  *   aq   : n rows of activations in the reference block layout (chip_quantize_q8_0 / _q8_K output)
- *   isum : [n][N][K/block] int32; for Q4_K/Q6_K one value per 256-block (sum over sub-blocks of scale*dot)
- *   imin : Q4_K only, [n][N][K/256] int32 (sum of min_j * bsum pairs); NULL otherwise */
+ *   isum : [n][N][K/block] int32; for Q4_K/Q5_K/Q6_K one value per 256-block (sum over sub-blocks of scale*dot)
+ *   imin : Q4_K and Q5_K only, [n][N][K/256] int32 (sum of min_j * bsum pairs); NULL otherwise */
 CHIP_API int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
                               const void *aq, int64_t n, int32_t *isum, int32_t *imin, void *stream);
 /* Rebuilds the reference block layout from a prepared workspace (inverse of the kernel-private layout), so

@@ -16,11 +16,50 @@ REF_SO = os.path.join(HERE, "_ref", "libggml_ref.so")
 
 # lm_ggml_type values (reference ggml.h:351-391)
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
-TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K"}
-BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256}
-BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292}
-VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K)
+Q5_0, Q5_K, IQ4_NL = 6, 13, 20
+TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
+              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl"}
+BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32}
+BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18}
+VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL)
+# types whose weight quantizer is restated in the oracle (IQ4_NL weights come from the reference build, from the
+# golden fixture, or are random bytes: any byte string is a valid block)
+ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K)
+
+
+IQ4_NL_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
+
+
+def nearest_iq4_nl_rows(w):
+    """fp32 [N, K] -> IQ4_NL rows: per 32-block d = max|x| / 127 (sign of the largest element, as fp16), index =
+    nearest code point of x / d.  Not the reference's quantizer."""
+    w = np.ascontiguousarray(w, np.float32)
+    n, k = w.shape
+    nb = k // 32
+    blk = w.reshape(n, nb, 32)
+    imax = np.abs(blk).argmax(-1)
+    mx = np.take_along_axis(blk, imax[..., None], -1)[..., 0]
+    d = (mx / np.float32(-127)).astype(np.float16)
+    df = d.astype(np.float32)
+    inv = np.where(df != 0, 1.0 / np.where(df != 0, df, 1), 0).astype(np.float32)
+    idx = np.abs((blk * inv[..., None])[..., None] - IQ4_NL_VALUES).argmin(-1).astype(np.uint8)
+    out = np.zeros((n, nb, 18), np.uint8)
+    out[..., :2] = d.view(np.uint8).reshape(n, nb, 2)
+    out[..., 2:] = idx[..., :16] | (idx[..., 16:] << 4)
+    return out.reshape(n, nb * 18)
+
+
+def random_iq4_nl_rows(seed, n, k):
+    """Random but plausible IQ4_NL rows: uniform code indices, fp16 scales around 2e-4 (weights ~ N(0, 0.02))."""
+    rng = np.random.default_rng(seed)
+    nb = k // 32
+    blk = np.zeros((n, nb, 18), np.uint8)
+    d = (2e-4 * np.exp(rng.uniform(-1.0, 1.0, (n, nb)))).astype(np.float16)
+    d[rng.random((n, nb)) < 0.05] *= np.float16(-1)
+    blk[..., :2] = d.view(np.uint8).reshape(n, nb, 2)
+    blk[..., 2:] = rng.integers(0, 256, (n, nb, 16), dtype=np.uint8)
+    return blk.reshape(n, nb * 18)
 
 
 def row_size(t, k):
@@ -58,7 +97,7 @@ class Oracle:
         L.orc_fp16_to_fp32.argtypes = [C.c_uint16]
         L.orc_fp32_to_fp16.restype = C.c_uint16
         L.orc_fp32_to_fp16.argtypes = [C.c_float]
-        for n in ("q8_0", "q8_K", "q4_0_ref", "q8_0_ref", "q4_K_ref", "q6_K_ref"):
+        for n in ("q8_0", "q8_K", "q4_0_ref", "q8_0_ref", "q4_K_ref", "q6_K_ref", "q5_0_ref", "q5_K_ref"):
             f = getattr(L, "orc_quantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
@@ -66,12 +105,14 @@ class Oracle:
         L.orc_quantize_rows.argtypes = [_i32, _vp, _vp, _i64, _i64]
         L.orc_dequantize_row.restype = None
         L.orc_dequantize_row.argtypes = [_i32, _vp, _vp, _i64]
-        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K"):
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0"):
             f = getattr(L, "orc_vec_dot_" + n)
             f.restype = C.c_float
             f.argtypes = [_i64, _vp, _vp, _vp]
-        L.orc_vec_dot_q4_K_q8_K.restype = C.c_float
-        L.orc_vec_dot_q4_K_q8_K.argtypes = [_i64, _vp, _vp, _vp, _vp]
+        for n in ("q4_K_q8_K", "q5_K_q8_K"):
+            f = getattr(L, "orc_vec_dot_" + n)
+            f.restype = C.c_float
+            f.argtypes = [_i64, _vp, _vp, _vp, _vp]
         L.orc_vec_dot_exact.restype = C.c_double
         L.orc_vec_dot_exact.argtypes = [_i32, _i64, _vp, _vp, _vp]
         L.orc_mul_mat.restype = None
@@ -103,9 +144,13 @@ class Oracle:
         return out
 
     def quantize_weights(self, wtype, w):
-        """w [N, K] fp32 -> uint8 [N, row_size] with the reference's *_ref weight quantizer."""
+        """w [N, K] fp32 -> uint8 [N, row_size] with the reference's *_ref weight quantizer.
+        IQ4_NL: a plain nearest-code-point quantizer (NOT the reference's search; it only makes meaningful bytes,
+        the op's parity surface starts at the bytes)."""
         w = _f32(w)
         n, k = w.shape
+        if wtype == IQ4_NL:
+            return nearest_iq4_nl_rows(w)
         out = np.zeros((n, row_size(wtype, k)), np.uint8)
         got = self.lib.orc_quantize_rows(wtype, _ptr(w), _ptr(out), n, k)
         assert got == out.size
@@ -134,6 +179,12 @@ class Oracle:
             v = self.lib.orc_vec_dot_q4_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
         elif wtype == Q6_K:
             v = self.lib.orc_vec_dot_q6_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == Q5_0:
+            v = self.lib.orc_vec_dot_q5_0_q8_0(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == IQ4_NL:
+            v = self.lib.orc_vec_dot_iq4_nl_q8_0(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == Q5_K:
+            v = self.lib.orc_vec_dot_q5_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
         else:
             raise ValueError(wtype)
         v = np.float32(v)
@@ -191,15 +242,16 @@ class Reference:
         ctx = L.lm_ggml_init(_InitParams(1 << 20, None, False))
         L.lm_ggml_free(ctx)
         for n in ("quantize_row_q8_0", "quantize_row_q8_K", "quantize_row_q4_0_ref", "quantize_row_q8_0_ref",
-                  "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref"):
+                  "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref",
+                  "quantize_row_q5_0_ref", "quantize_row_q5_K_ref", "quantize_row_iq4_nl_ref"):
             f = getattr(L, n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
-        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K"):
+        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl"):
             f = getattr(L, "dequantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
-        for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K"):
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "q5_0_q8_0", "q5_K_q8_K", "iq4_nl_q8_0"):
             f = getattr(L, "lm_ggml_vec_dot_" + n)
             f.restype = None
             f.argtypes = [C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, _vp, C.c_size_t, C.c_int]
@@ -234,9 +286,11 @@ class Reference:
 
     _ACT = {Q8_0: "quantize_row_q8_0", Q8_K: "quantize_row_q8_K"}
     _WQ = {Q4_0: "quantize_row_q4_0_ref", Q8_0: "quantize_row_q8_0_ref",
-           Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref"}
+           Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref",
+           Q5_0: "quantize_row_q5_0_ref", Q5_K: "quantize_row_q5_K_ref", IQ4_NL: "quantize_row_iq4_nl_ref"}
     _DOT = {Q4_0: "lm_ggml_vec_dot_q4_0_q8_0", Q8_0: "lm_ggml_vec_dot_q8_0_q8_0",
-            Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K"}
+            Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K",
+            Q5_0: "lm_ggml_vec_dot_q5_0_q8_0", Q5_K: "lm_ggml_vec_dot_q5_K_q8_K", IQ4_NL: "lm_ggml_vec_dot_iq4_nl_q8_0"}
 
     def quantize_activation(self, act_type, x):
         x = _f32(x)

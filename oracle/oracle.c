@@ -20,6 +20,10 @@ typedef struct { uint16_t d; int8_t qs[32]; } blk_q8_0;
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[128]; } blk_q4_K;
 typedef struct { uint8_t ql[128]; uint8_t qh[64]; int8_t scales[16]; uint16_t d; } blk_q6_K;
 typedef struct { float d; int8_t qs[256]; int16_t bsums[16]; } blk_q8_K;
+/* further weight types: ggml-common.h:187-193 (q5_0), :303-314 (q5_K), :405-410 (iq4_nl) */
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_0;
+typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qh[32]; uint8_t qs[128]; } blk_q5_K;
+typedef struct { uint16_t d; uint8_t qs[16]; } blk_iq4_nl;
 #pragma pack(pop)
 
 _Static_assert(sizeof(blk_q4_0) == 18, "q4_0");
@@ -27,12 +31,18 @@ _Static_assert(sizeof(blk_q8_0) == 34, "q8_0");
 _Static_assert(sizeof(blk_q4_K) == 144, "q4_K");
 _Static_assert(sizeof(blk_q6_K) == 210, "q6_K");
 _Static_assert(sizeof(blk_q8_K) == 292, "q8_K");
+_Static_assert(sizeof(blk_q5_0) == 22, "q5_0");
+_Static_assert(sizeof(blk_q5_K) == 176, "q5_K");
+_Static_assert(sizeof(blk_iq4_nl) == 18, "iq4_nl");
+
+/* ggml-quants.c:2428: the 16 code points of the non-linear 4-bit types. */
+static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
 int orc_block_elems(int type) {
     switch (type) {
         case ORC_TYPE_F32: return 1;
-        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: return 32;
-        case ORC_TYPE_Q4_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
+        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return 32;
+        case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
         default: return 0;
     }
 }
@@ -44,6 +54,9 @@ size_t orc_block_bytes(int type) {
         case ORC_TYPE_Q4_K: return 144;
         case ORC_TYPE_Q6_K: return 210;
         case ORC_TYPE_Q8_K: return 292;
+        case ORC_TYPE_Q5_0: return 22;
+        case ORC_TYPE_Q5_K: return 176;
+        case ORC_TYPE_IQ4_NL: return 18;
         default: return 0;
     }
 }
@@ -52,9 +65,9 @@ size_t orc_row_size(int type, int64_t k) {
     return be ? (size_t)(k / be) * orc_block_bytes(type) : 0;
 }
 int orc_vec_dot_type(int type) {
-    switch (type) { /* ggml-cpu/ggml-cpu.c:213,245,272,284 */
-        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: return ORC_TYPE_Q8_0;
-        case ORC_TYPE_Q4_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
+    switch (type) { /* ggml-cpu/ggml-cpu.c:213,245,272,284; :229 (q5_0), :278 (q5_K), :340 (iq4_nl) */
+        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return ORC_TYPE_Q8_0;
+        case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
         default: return -1;
     }
 }
@@ -190,11 +203,12 @@ void orc_quantize_row_q4_0_ref(const float *x, void *vy, int64_t k) {
     }
 }
 
-/* ggml-quants.c:544-623 with the arguments quantize_row_q4_K_ref passes (n=32, nmax=15, rmin=-1,
- * rdelta=0.1, nstep=20, use_mad=false).  Returns the scale, writes -min to *neg_min. */
-static float fit_scale_min_32(const float *x, const float *w, uint8_t *L, float *neg_min, uint8_t *Laux) {
-    const int n = 32, nmax = 15, nstep = 20;
-    const float rmin = -1.f, rdelta = 0.1f;
+/* ggml-quants.c:544-623 with n=32, use_mad=false.  quantize_row_q4_K_ref passes nmax=15, rmin=-1, rdelta=0.1,
+ * nstep=20 (:1221); quantize_row_q5_K_ref passes nmax=31, rmin=-0.5, rdelta=0.1, nstep=15 (:1409).
+ * Returns the scale, writes -min to *neg_min. */
+static float fit_scale_min_32(const float *x, const float *w, uint8_t *L, float *neg_min, uint8_t *Laux,
+                              int nmax, float rmin, float rdelta, int nstep) {
+    const int n = 32;
     float lo = x[0], hi = x[0];
     float sum_w = w[0];
     float sum_x = sum_w * x[0];
@@ -274,7 +288,7 @@ void orc_quantize_row_q4_K_ref(const float *x, void *vy, int64_t k) {
             for (int l = 0; l < 32; l++) sum_x2 += xs[l] * xs[l];
             float av = sqrtf(sum_x2 / 32);
             for (int l = 0; l < 32; l++) w[l] = av + fabsf(xs[l]);
-            scales[j] = fit_scale_min_32(xs, w, L + 32 * j, &mins[j], Laux);
+            scales[j] = fit_scale_min_32(xs, w, L + 32 * j, &mins[j], Laux, 15, -1.f, 0.1f, 20);
             if (scales[j] > max_scale) max_scale = scales[j];
             if (mins[j] > max_min) max_min = mins[j];
         }
@@ -308,6 +322,89 @@ void orc_quantize_row_q4_K_ref(const float *x, void *vy, int64_t k) {
         uint8_t *q = y[b].qs;
         for (int j = 0; j < 256; j += 64, q += 32)
             for (int l = 0; l < 32; l++) q[l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
+    }
+}
+
+/* ggml-quants.c:1389-1474. */
+void orc_quantize_row_q5_K_ref(const float *x, void *vy, int64_t k) {
+    blk_q5_K *y = (blk_q5_K *)vy;
+    uint8_t L[256], Laux[32];
+    float w[32], mins[8], scales[8];
+    for (int64_t b = 0; b < k / 256; b++, x += 256) {
+        float max_scale = 0, max_min = 0;
+        for (int j = 0; j < 8; j++) {
+            const float *xs = x + 32 * j;
+            float sum_x2 = 0;
+            for (int l = 0; l < 32; l++) sum_x2 += xs[l] * xs[l];
+            float av = sqrtf(sum_x2 / 32);
+            for (int l = 0; l < 32; l++) w[l] = av + fabsf(xs[l]);
+            scales[j] = fit_scale_min_32(xs, w, L + 32 * j, &mins[j], Laux, 31, -0.5f, 0.1f, 15);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+        const float inv_min   = max_min   > 0 ? 63.f / max_min   : 0.f;
+        for (int j = 0; j < 8; j++) {
+            uint8_t ls = (uint8_t)nearest_i(inv_scale * scales[j]);
+            uint8_t lm = (uint8_t)nearest_i(inv_min * mins[j]);
+            if (ls > 63) ls = 63;
+            if (lm > 63) lm = 63;
+            if (j < 4) { y[b].scales[j] = ls; y[b].scales[j + 4] = lm; }
+            else {
+                y[b].scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                y[b].scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                y[b].scales[j]     |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        y[b].d    = F2H(max_scale / 63.f);
+        y[b].dmin = F2H(max_min / 63.f);
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            unpack_sc_m(j, y[b].scales, &sc, &m);
+            const float d = H2F(y[b].d) * sc;
+            if (!d) continue;
+            const float dm = H2F(y[b].dmin) * m;
+            for (int i = 0; i < 32; i++) {
+                int l = nearest_i((x[32 * j + i] + dm) / d);
+                L[32 * j + i] = (uint8_t)imax_(0, imin_(31, l));
+            }
+        }
+        memset(y[b].qh, 0, 32);
+        uint8_t *ql = y[b].qs;
+        uint8_t m1 = 1, m2 = 2;
+        for (int n = 0; n < 256; n += 64, ql += 32) {
+            for (int j = 0; j < 32; j++) {
+                int l1 = L[n + j], l2 = L[n + j + 32];
+                if (l1 > 15) { l1 -= 16; y[b].qh[j] |= m1; }
+                if (l2 > 15) { l2 -= 16; y[b].qh[j] |= m2; }
+                ql[j] = (uint8_t)(l1 | (l2 << 4));
+            }
+            m1 = (uint8_t)(m1 << 2); m2 = (uint8_t)(m2 << 2);
+        }
+    }
+}
+
+/* ggml-quants.c:99-141. */
+void orc_quantize_row_q5_0_ref(const float *x, void *vy, int64_t k) {
+    blk_q5_0 *y = (blk_q5_0 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float amax = 0.f, mx = 0.f;
+        for (int j = 0; j < 32; j++) {
+            if (amax < fabsf(x[j])) { amax = fabsf(x[j]); mx = x[j]; }
+        }
+        const float d = mx / -16;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = F2H(d);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            const float x0 = x[j] * id, x1 = x[16 + j] * id;
+            const uint8_t xi0 = (uint8_t)imin_(31, (int8_t)(x0 + 16.5f));
+            const uint8_t xi1 = (uint8_t)imin_(31, (int8_t)(x1 + 16.5f));
+            y[b].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= ((xi0 & 0x10u) >> 4) << (j + 0);
+            qh |= ((xi1 & 0x10u) >> 4) << (j + 16);
+        }
+        memcpy(y[b].qh, &qh, 4);
     }
 }
 
@@ -407,6 +504,8 @@ size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64
             case ORC_TYPE_Q8_0: orc_quantize_row_q8_0_ref(src, dst, k); break;
             case ORC_TYPE_Q4_K: orc_quantize_row_q4_K_ref(src, dst, k); break;
             case ORC_TYPE_Q6_K: orc_quantize_row_q6_K_ref(src, dst, k); break;
+            case ORC_TYPE_Q5_K: orc_quantize_row_q5_K_ref(src, dst, k); break;
+            case ORC_TYPE_Q5_0: orc_quantize_row_q5_0_ref(src, dst, k); break;
             default: return 0;
         }
     }
@@ -470,6 +569,67 @@ void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
         const blk_q8_K *x = (const blk_q8_K *)vx;
         for (int64_t b = 0; b < k / 256; b++)
             for (int j = 0; j < 256; j++) *y++ = x[b].d * x[b].qs[j];
+    } else if (type == ORC_TYPE_Q5_0) {                 /* ggml-quants.c:290-313 */
+        const blk_q5_0 *x = (const blk_q5_0 *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d);
+            uint32_t qh;
+            memcpy(&qh, x[b].qh, 4);
+            for (int j = 0; j < 16; j++) {
+                const uint8_t xh0 = (uint8_t)(((qh >> (j + 0)) << 4) & 0x10);
+                const uint8_t xh1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+                y[j]      = (float)(((x[b].qs[j] & 0x0F) | xh0) - 16) * d;
+                y[j + 16] = (float)(((x[b].qs[j] >> 4) | xh1) - 16) * d;
+            }
+        }
+    } else if (type == ORC_TYPE_Q5_K) {                 /* ggml-quants.c:1476-1501 */
+        const blk_q5_K *x = (const blk_q5_K *)vx;
+        for (int64_t b = 0; b < k / 256; b++) {
+            const float d = H2F(x[b].d), mn = H2F(x[b].dmin);
+            const uint8_t *ql = x[b].qs, *qh = x[b].qh;
+            uint8_t u1 = 1, u2 = 2;
+            for (int j = 0; j < 4; j++, ql += 32) {
+                uint8_t sc, m;
+                unpack_sc_m(2 * j, x[b].scales, &sc, &m);
+                const float d1 = d * sc, m1 = mn * m;
+                unpack_sc_m(2 * j + 1, x[b].scales, &sc, &m);
+                const float d2 = d * sc, m2 = mn * m;
+                for (int l = 0; l < 32; l++) *y++ = d1 * ((ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0)) - m1;
+                for (int l = 0; l < 32; l++) *y++ = d2 * ((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
+                u1 = (uint8_t)(u1 << 2); u2 = (uint8_t)(u2 << 2);
+            }
+        }
+    } else if (type == ORC_TYPE_IQ4_NL) {               /* ggml-quants.c:2430-2446 */
+        const blk_iq4_nl *x = (const blk_iq4_nl *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d);
+            for (int j = 0; j < 16; j++) {
+                y[j]      = d * iq4nl_values[x[b].qs[j] & 0xf];
+                y[j + 16] = d * iq4nl_values[x[b].qs[j] >> 4];
+            }
+        }
+    }
+}
+
+/* The 32 signed weights of one block of the 32-element types in element order (what the SIMD paths put into
+ * one 256-bit register before multiplying with the Q8_0 quants). */
+static void block32_ints(int type, const void *vx, int64_t b, int8_t w[32], uint16_t *dh) {
+    if (type == ORC_TYPE_Q5_0) {                        /* ggml-cpu/ggml-cpu-quants.c:70-80 + q5_0 AVX2 branch */
+        const blk_q5_0 *x = (const blk_q5_0 *)vx + b;
+        uint32_t qh;
+        memcpy(&qh, x->qh, 4);
+        for (int j = 0; j < 16; j++) {
+            w[j]      = (int8_t)(((x->qs[j] & 0xF) | (((qh >> j) & 1) << 4)) - 16);
+            w[j + 16] = (int8_t)(((x->qs[j] >> 4) | (((qh >> (j + 16)) & 1) << 4)) - 16);
+        }
+        *dh = x->d;
+    } else {                                            /* ORC_TYPE_IQ4_NL */
+        const blk_iq4_nl *x = (const blk_iq4_nl *)vx + b;
+        for (int j = 0; j < 16; j++) {
+            w[j]      = iq4nl_values[x->qs[j] & 0xf];
+            w[j + 16] = iq4nl_values[x->qs[j] >> 4];
+        }
+        *dh = x->d;
     }
 }
 
@@ -620,12 +780,122 @@ float orc_vec_dot_q6_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *
     return hsum8(acc);
 }
 
+/* q5_0: ggml-cpu/ggml-cpu-quants.c AVX2 branch of lm_ggml_vec_dot_q5_0_q8_0 (:2924...): one 8-lane accumulator,
+ * lane j takes the four products of elements 4j..4j+3, fmadd with d = dx * dy. */
+float orc_vec_dot_q5_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q8_0 *y = (const blk_q8_0 *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 32; b++) {
+        int8_t w[32];
+        uint16_t dh;
+        block32_ints(ORC_TYPE_Q5_0, vx, b, w, &dh);
+        const float d = H2F(dh) * H2F(y[b].d);
+        int32_t tot = 0;
+        for (int j = 0; j < 8; j++) {
+            int32_t p = 0;
+            for (int t = 0; t < 4; t++) p += (int32_t)w[4 * j + t] * y[b].qs[4 * j + t];
+            tot += p;
+            acc[j] = fmaf(d, (float)p, acc[j]);
+        }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc);
+}
+
+/* iq4_nl: AVX2 branch of lm_ggml_vec_dot_iq4_nl_q8_0 (ggml-cpu/ggml-cpu-quants.c:12798-12826): blocks are taken
+ * two at a time into two 8-lane accumulators (d = dy * dx), added lane-wise at the end; an odd last block
+ * goes through the scalar tail (:12869-12878: sumf += d * (sumi1 + sumi2)). */
+float orc_vec_dot_iq4_nl_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q8_0 *y = (const blk_q8_0 *)vy;
+    const int64_t nb = k / 32;
+    float acc1[8] = {0}, acc2[8] = {0};
+    int64_t b = 0;
+    for (; b + 1 < nb; b += 2) {
+        for (int h = 0; h < 2; h++) {
+            int8_t w[32];
+            uint16_t dh;
+            block32_ints(ORC_TYPE_IQ4_NL, vx, b + h, w, &dh);
+            const float d = H2F(y[b + h].d) * H2F(dh);
+            float *acc = h ? acc2 : acc1;
+            int32_t tot = 0;
+            for (int j = 0; j < 8; j++) {
+                int32_t p = 0;
+                for (int t = 0; t < 4; t++) p += (int32_t)w[4 * j + t] * y[b + h].qs[4 * j + t];
+                tot += p;
+                acc[j] = fmaf(d, (float)p, acc[j]);
+            }
+            if (isum) isum[b + h] = tot;
+        }
+    }
+    float s8[8];
+    for (int j = 0; j < 8; j++) s8[j] = acc1[j] + acc2[j];
+    float sumf = hsum8(s8);
+    for (; b < nb; b++) {
+        int8_t w[32];
+        uint16_t dh;
+        block32_ints(ORC_TYPE_IQ4_NL, vx, b, w, &dh);
+        const float d = H2F(y[b].d) * H2F(dh);
+        int32_t s1 = 0, s2 = 0;
+        for (int j = 0; j < 16; j++) { s1 += y[b].qs[j] * w[j]; s2 += y[b].qs[j + 16] * w[j + 16]; }
+        if (isum) isum[b] = s1 + s2;
+        sumf += d * (float)(s1 + s2);
+    }
+    return sumf;
+}
+
+/* q5_K: AVX2 branch of lm_ggml_vec_dot_q5_K_q8_K (ggml-cpu/ggml-cpu-quants.c:7786-7860): as q4_K for the d term
+ * (one integer 8-lane sum per super-block, one fmadd), but the min term is a scalar
+ * `summs += dmin * hsum` (separate multiply and add) added after the horizontal sum. */
+float orc_vec_dot_q5_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin) {
+    const blk_q5_K *x = (const blk_q5_K *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    float acc[8] = {0};
+    float summs = 0.f;
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float d = y[b].d * H2F(x[b].d);
+        const float dmin = -y[b].d * H2F(x[b].dmin);
+        uint8_t sm[16];
+        unpack_scales_kmask(x[b].scales, sm);
+        const uint8_t *sc = sm, *mn = sm + 8;
+        int32_t mtot = 0;
+        for (int j = 0; j < 8; j++)
+            mtot += (int32_t)mn[j] * (int16_t)(y[b].bsums[2 * j] + y[b].bsums[2 * j + 1]);
+        const float prod = dmin * (float)mtot;
+        summs = summs + prod;
+
+        int32_t lane[8] = {0};
+        const uint8_t *q5 = x[b].qs, *qh = x[b].qh;
+        const int8_t *q8 = y[b].qs;
+        for (int j = 0; j < 4; j++, q5 += 32, q8 += 64) {
+            for (int m = 0; m < 8; m++) {
+                int32_t pl = 0, ph = 0;
+                for (int t = 0; t < 4; t++) {
+                    const int e = 4 * m + t;
+                    const int lo = (q5[e] & 0xF) + (((qh[e] >> (2 * j)) & 1) << 4);
+                    const int hi = (q5[e] >> 4) + (((qh[e] >> (2 * j + 1)) & 1) << 4);
+                    pl += lo * q8[e];
+                    ph += hi * q8[32 + e];
+                }
+                lane[m] += (int32_t)sc[2 * j] * pl + (int32_t)sc[2 * j + 1] * ph;
+            }
+        }
+        int32_t tot = 0;
+        for (int m = 0; m < 8; m++) { tot += lane[m]; acc[m] = fmaf(d, (float)lane[m], acc[m]); }
+        if (isum) isum[b] = tot;
+        if (imin) imin[b] = mtot;
+    }
+    return hsum8(acc) + summs;
+}
+
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
     switch (type) {
         case ORC_TYPE_Q4_0: return orc_vec_dot_q4_0_q8_0(k, vx, vy, NULL);
         case ORC_TYPE_Q8_0: return orc_vec_dot_q8_0_q8_0(k, vx, vy, NULL);
         case ORC_TYPE_Q4_K: return orc_vec_dot_q4_K_q8_K(k, vx, vy, NULL, NULL);
         case ORC_TYPE_Q6_K: return orc_vec_dot_q6_K_q8_K(k, vx, vy, NULL);
+        case ORC_TYPE_Q5_0: return orc_vec_dot_q5_0_q8_0(k, vx, vy, NULL);
+        case ORC_TYPE_IQ4_NL: return orc_vec_dot_iq4_nl_q8_0(k, vx, vy, NULL);
+        case ORC_TYPE_Q5_K: return orc_vec_dot_q5_K_q8_K(k, vx, vy, NULL, NULL);
         default: return NAN;
     }
 }
@@ -644,6 +914,35 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
             const uint16_t hx = type == ORC_TYPE_Q4_0 ? ((const blk_q4_0 *)vx)[b].d : ((const blk_q8_0 *)vx)[b].d;
             const double t = (double)H2F(hx) * (double)H2F(y[b].d) * (double)is[b];
             s += t; sa += fabs(t);
+        }
+    } else if (type == ORC_TYPE_Q5_0 || type == ORC_TYPE_IQ4_NL) {
+        if (type == ORC_TYPE_Q5_0) orc_vec_dot_q5_0_q8_0(k, vx, vy, is);
+        else                       orc_vec_dot_iq4_nl_q8_0(k, vx, vy, is);
+        const blk_q8_0 *y = (const blk_q8_0 *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const uint16_t hx = type == ORC_TYPE_Q5_0 ? ((const blk_q5_0 *)vx)[b].d : ((const blk_iq4_nl *)vx)[b].d;
+            const double t = (double)H2F(hx) * (double)H2F(y[b].d) * (double)is[b];
+            s += t; sa += fabs(t);
+        }
+    } else if (type == ORC_TYPE_Q5_K) {
+        const blk_q5_K *x = (const blk_q5_K *)vx;
+        const blk_q8_K *y = (const blk_q8_K *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const double d = (double)y[b].d * (double)H2F(x[b].d), dm = (double)y[b].d * (double)H2F(x[b].dmin);
+            for (int j = 0; j < 8; j++) {
+                uint8_t sc, m;
+                unpack_sc_m(j, x[b].scales, &sc, &m);
+                const uint8_t *q5 = x[b].qs + 32 * (j / 2);
+                const int8_t *q8 = y[b].qs + 32 * j;
+                int64_t dot = 0;
+                for (int l = 0; l < 32; l++) {
+                    const int q = ((j & 1) ? (q5[l] >> 4) : (q5[l] & 0xF)) + (((x[b].qh[l] >> j) & 1) << 4);
+                    dot += (int64_t)q * q8[l];
+                }
+                const double t1 = d * (double)sc * (double)dot;
+                const double t2 = dm * (double)m * (double)(y[b].bsums[2 * j] + y[b].bsums[2 * j + 1]);
+                s += t1 - t2; sa += fabs(t1) + fabs(t2);
+            }
         }
     } else if (type == ORC_TYPE_Q4_K) {
         /* terms at sub-block granularity (32 values with their own 6-bit scale and min) */

@@ -18,6 +18,9 @@
  *   orc_quantize_row_q4_0_ref        bit-exact vs oracle/_ref + golden; dequant closed form d*(nib-8)
  *   orc_quantize_row_q4_K_ref        bit-exact vs oracle/_ref + golden (iterative search: only the oracle run
  *   orc_quantize_row_q6_K_ref          pins the bytes); reconstruction-error bound as a sanity invariant
+ *   orc_quantize_row_q5_0_ref/_q5_K_ref  bit-exact vs oracle/_ref + golden; dequant closed forms
+ *   (iq4_nl has no quantizer here: its weights come from oracle/_ref, committed in the golden fixture, or
+ *    are random code indices with a random fp16 scale -- any byte string is a valid iq4_nl block)
  *   orc_dequantize_row_*             closed forms; vs oracle/_ref + golden
  *   orc_vec_dot_*                    integer sums: brute force from dequantised integers; float result: bit-exact
  *                                    vs oracle/_ref (the AVX2 lane structure is restated) + golden; fp64 identity
@@ -44,6 +47,10 @@ enum orc_type {
     ORC_TYPE_Q4_K = 12,
     ORC_TYPE_Q6_K = 14,
     ORC_TYPE_Q8_K = 15,
+    /* further weight types (same activation quantizers) */
+    ORC_TYPE_Q5_0 = 6,
+    ORC_TYPE_Q5_K = 13,
+    ORC_TYPE_IQ4_NL = 20,
 };
 
 /* elements per block / bytes per block / bytes per row of k elements; 0 for an unknown type */
@@ -65,6 +72,8 @@ void orc_quantize_row_q4_0_ref(const float *x, void *y, int64_t k);
 void orc_quantize_row_q8_0_ref(const float *x, void *y, int64_t k);
 void orc_quantize_row_q4_K_ref(const float *x, void *y, int64_t k);
 void orc_quantize_row_q6_K_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q5_0_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q5_K_ref(const float *x, void *y, int64_t k);
 /* dispatch on weight type, nrows rows of k elements, rows packed back to back; returns bytes written */
 size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64_t k);
 
@@ -82,12 +91,17 @@ float orc_vec_dot_q4_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *
 float orc_vec_dot_q8_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot_q4_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin);
 float orc_vec_dot_q6_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum);
+/* q5_0, iq4_nl: isum[k/32] = sum (q5-16)*aq resp. sum codebook[nib]*aq ; q5_K: as q4_K with 5-bit quants */
+float orc_vec_dot_q5_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot_iq4_nl_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot_q5_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin);
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
 
 /* fp64 evaluation of sum_b scale_b*isum_b (returned) and of sum_b |scale_b*isum_b| (*sum_abs): the tolerance
  * yardstick 1e-5 * sum_abs and an order-free reference value.  A "block" is the smallest group of values that
  * carries its own scale: 32 values for Q4_0/Q8_0, a 32-value sub-block for Q4_K (terms d*sc_j*dot_j and
- * dmin*m_j*bsum_j, both counted), a 16-value sub-block for Q6_K (d*sc_j*dot_j).  Coarser terms (whole
+ * dmin*m_j*bsum_j, both counted), a 16-value sub-block for Q6_K (d*sc_j*dot_j); Q5_0 and
+ * IQ4_NL as Q4_0, Q5_K as Q4_K.  Coarser terms (whole
  * super-blocks) would cancel internally and make a bound that the reference's own AVX2 result misses. */
 double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, double *sum_abs);
 

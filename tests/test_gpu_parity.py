@@ -84,7 +84,7 @@ SHAPES = [(256, 1), (512, 7), (2048, 130), (4096, 257), (11008, 40), (14336, 33)
 @pytest.mark.parametrize("n", [1, 2, 3, 5, 8])
 def test_mul_mat_vs_oracle(dev, orc, wt, K, N, n):
     print("mul_mat", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
-    wq = orc.quantize_weights(wt, common.weights_f32(K + N + wt, N, K, outliers=(wt == O.Q4_K)))
+    wq = orc.quantize_weights(wt, common.weights_f32(K + N + wt, N, K, outliers=(wt in (O.Q4_K, O.Q5_K))))
     x = common.activations_f32(K + n, n, K)
     if n >= 3:
         x[1] = 0                                    # an all-zero token
@@ -104,7 +104,7 @@ def test_block_integer_sums_bit_exact(dev, orc, wt):
         for i in range(N):
             _, ri, rm = orc.vec_dot(wt, K, wq[i], aq[t], want_sums=True)
             assert np.array_equal(isum[t, i], ri)
-            if wt == O.Q4_K:
+            if wt in (O.Q4_K, O.Q5_K):
                 assert np.array_equal(imin[t, i], rm)
 
 

@@ -20,8 +20,9 @@ def test_mul_mat_golden(orc, wt):
     g = gold("mul_mat_%s.npz" % O.TYPE_NAMES[wt])
     K = int(g["K"])
     assert int(g["wtype"]) == wt
-    # weight quantizer bytes
-    assert np.array_equal(orc.quantize_weights(wt, g["w"]), g["wq"])
+    # weight quantizer bytes (IQ4_NL's quantizer is not restated: its golden bytes come from the reference build)
+    if wt in O.ORACLE_QUANTIZED:
+        assert np.array_equal(orc.quantize_weights(wt, g["w"]), g["wq"])
     # dequantizer closed form
     assert np.array_equal(orc.dequantize(wt, g["wq"], K), g["w_deq"])
     # on-the-fly activation quantizer bytes

@@ -37,8 +37,9 @@ def test_weight_quantizers_and_dots(orc, ref, wt):
     w[5] = 0
     w[6, :256] = 0
     x = common.activations_f32(wt, n, K)
-    a, b = orc.quantize_weights(wt, w), ref.quantize_weights(wt, w)
-    assert np.array_equal(a, b)
+    b = ref.quantize_weights(wt, w)
+    if wt in O.ORACLE_QUANTIZED:
+        assert np.array_equal(orc.quantize_weights(wt, w), b)
     assert np.array_equal(orc.dequantize(wt, b, K), ref.dequantize(wt, b, K))
     xq = ref.quantize_activation(O.VEC_DOT_TYPE[wt], x)
     for t in range(n):
