@@ -9,6 +9,8 @@
 //       d   float [K/32]     at +K                 the block scale after rounding to fp16 (exactly as stored
 //                                                  in block_q8_0.d), widened back to fp32
 //       sum int32 [K/32]     at +K + 4*(K/32)      sum of the 32 quants of the block (Q4_0's -8 offset)
+//       s   float [K/32]     at +K + 8*(K/32)      block_q8_1.s (fp16(d * sum), widened): the min term of Q4_1 / Q5_1,
+//                                                  whose activation format Q8_1 is Q8_0 plus this number
 //
 //   Q8_K activations (for Q4_K and Q6_K weights), token stride = q8_K_stride(K):
 //       qs    int8  [K]      at +0
@@ -26,7 +28,8 @@ __host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~(siz
 
 __host__ __device__ constexpr size_t q8_0_off_d(int64_t K)   { return (size_t)K; }
 __host__ __device__ constexpr size_t q8_0_off_sum(int64_t K) { return (size_t)K + 4 * (size_t)(K / 32); }
-__host__ __device__ constexpr size_t q8_0_stride(int64_t K)  { return align16((size_t)K + 8 * (size_t)(K / 32)); }
+__host__ __device__ constexpr size_t q8_0_off_s(int64_t K)   { return (size_t)K + 8 * (size_t)(K / 32); }
+__host__ __device__ constexpr size_t q8_0_stride(int64_t K)  { return align16((size_t)K + 12 * (size_t)(K / 32)); }
 
 __host__ __device__ constexpr size_t q8_K_off_d(int64_t K)     { return (size_t)K; }
 __host__ __device__ constexpr size_t q8_K_off_bsums(int64_t K) { return (size_t)K + 4 * (size_t)(K / 256); }

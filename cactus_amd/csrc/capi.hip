@@ -50,7 +50,8 @@ int current_limits(DeviceLimits &out) {
 }
 
 bool is_weight_type(int t) {
-    return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K || t == T_Q5_0 || t == T_Q5_K || t == T_IQ4_NL;
+    return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K || t == T_Q5_0 || t == T_Q5_K || t == T_IQ4_NL ||
+           t == T_Q4_1 || t == T_Q5_1;
 }
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -62,7 +63,8 @@ bool weights_aligned(int type, const void *W, size_t nb01) {
     return ((uintptr_t)W % a) == 0 && (nb01 % a) == 0;
 }
 
-size_t act_stride(int act_type, int64_t K) { return act_type == T_Q8_0 ? q8_0_stride(K) : q8_K_stride(K); }
+// Q8_1 activations live in the Q8_0 workspace planes (which carry block_q8_1.s as well)
+size_t act_stride(int act_type, int64_t K) { return (act_type == T_Q8_0 || act_type == T_Q8_1) ? q8_0_stride(K) : q8_K_stride(K); }
 
 }  // namespace
 
@@ -166,7 +168,7 @@ int chip_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((
 int chip_block_elems(int type) {
     switch (type) {
         case T_F32: return 1;
-        case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return 32;
+        case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: case T_Q8_1: return 32;
         case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: return 256;
         default: return 0;
     }
@@ -182,6 +184,9 @@ size_t chip_block_bytes(int type) {
         case T_Q5_0: return BYTES_Q5_0;
         case T_Q5_K: return BYTES_Q5_K;
         case T_IQ4_NL: return BYTES_IQ4_NL;
+        case T_Q4_1: return BYTES_Q4_1;
+        case T_Q5_1: return BYTES_Q5_1;
+        case T_Q8_1: return BYTES_Q8_1;
         default: return 0;
     }
 }
@@ -193,6 +198,7 @@ int chip_vec_dot_type(int type) {
     switch (type) {
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return T_Q8_0;
         case T_Q4_K: case T_Q6_K: case T_Q5_K: return T_Q8_K;
+        case T_Q4_1: case T_Q5_1: return T_Q8_1;
         default: return -1;
     }
 }
@@ -213,6 +219,9 @@ int chip_quantize_q8_0(const float *x, int64_t ldx, int64_t n, int64_t k, void *
 }
 int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
     return quantize_public(T_Q8_K, x, ldx, n, k, y, stream);
+}
+int chip_quantize_q8_1(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
+    return quantize_public(T_Q8_1, x, ldx, n, k, y, stream);
 }
 
 size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n) {

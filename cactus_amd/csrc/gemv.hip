@@ -102,7 +102,7 @@ template <> struct Traits<T_Q8_0> {
         const int b = e >> 5, u = b >> 1, off = 32 * (b & 1) + (e & 31);
         return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
     }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int) {
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int, float) {
         reinterpret_cast<float *>(img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX)[blk & 1] = d;
     }
 };
@@ -171,7 +171,7 @@ template <> struct Traits<T_Q4_0> {
         const int b = e >> 5, u = b >> 1, off = 32 * (b & 1) + (e & 31);
         return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
     }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum) {
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float) {
         uint8_t *a = img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX;
         reinterpret_cast<float *>(a)[blk & 1] = d;
         reinterpret_cast<int *>(a)[2 + (blk & 1)] = sum;
@@ -422,7 +422,7 @@ template <> struct Traits<T_Q5_0> {
     using AuxT = u32x4;
     __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q4_0>::aux_load(ws, K, u, valid); }
     __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_0>::img_qs(NI, e); }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum) { Traits<T_Q4_0>::img_block_aux(img, NI, blk, d, sum); }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float s) { Traits<T_Q4_0>::img_block_aux(img, NI, blk, d, sum, s); }
 };
 
 template <> struct Traits<T_IQ4_NL> {
@@ -472,8 +472,108 @@ template <> struct Traits<T_IQ4_NL> {
     using AuxT = float2;
     __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q8_0>::aux_load(ws, K, u, valid); }
     __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q8_0>::img_qs(NI, e); }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum) { Traits<T_Q8_0>::img_block_aux(img, NI, blk, d, sum); }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float s) { Traits<T_Q8_0>::img_block_aux(img, NI, blk, d, sum, s); }
 };
+
+// Q4_1 / Q5_1 (ggml-common.h:175-185,196-207): value = d * u + m with an unsigned 4- or 5-bit u.  Their activation
+// format Q8_1 is Q8_0 plus s = fp16(d * sum q) per block (kept in the Q8_0 workspace planes), so
+// y += (dw * dx) * sum(u * q) + m * s (reference lm_ggml_vec_dot_q4_1_q8_1 / _q5_1_q8_1, AVX2 branches).
+template <int WT> struct TraitsMin32 {
+    static constexpr bool FIVE = (WT == T_Q5_1);
+    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
+    static constexpr bool A_HAS_SUMS = false;
+    static constexpr int ABLK_BYTES = BYTES_Q8_1, ABLK_QOFF = 4;          // reference activation records (block_isums)
+    struct W { uint32_t lo[8], hi[8]; float d0, d1, m0, m1; };
+    struct A { uint32_t q[16]; float d0, d1, s0, s1; };
+    struct Raw { u32x4 a, b; u32x2 c; uint32_t e[2]; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        if constexpr (!FIVE) {
+            const uint8_t *p = row + (size_t)u * 40;                   // two 20-byte blocks, 4-byte aligned
+            r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
+            r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
+            r.c = WLOAD(reinterpret_cast<const u32x2_a4 *>(p + 32));
+        } else {
+            const uint8_t *p = row + (size_t)u * 48;                   // two 24-byte blocks, 4-byte aligned
+            r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
+            r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
+            r.c = WLOAD(reinterpret_cast<const u32x2_a4 *>(p + 32));
+            r.e[0] = WLOAD(reinterpret_cast<const uint32_t *>(p + 40));
+            r.e[1] = WLOAD(reinterpret_cast<const uint32_t *>(p + 44));
+        }
+    }
+    __device__ static __forceinline__ uint32_t spread4(uint32_t bits) { return (((bits & 0xFu) * 0x00204081u) & 0x01010101u) << 4; }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
+        if constexpr (!FIVE) {
+            // block: d, m (one dword), 16 qs bytes
+            const uint32_t d[10] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y};
+            w.d0 = h2f(d[0]); w.m0 = h2f(d[0] >> 16);
+            w.d1 = h2f(d[5]); w.m1 = h2f(d[5] >> 16);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                w.lo[i]     = d[1 + i] & 0x0f0f0f0fu; w.hi[i]     = (d[1 + i] >> 4) & 0x0f0f0f0fu;
+                w.lo[4 + i] = d[6 + i] & 0x0f0f0f0fu; w.hi[4 + i] = (d[6 + i] >> 4) & 0x0f0f0f0fu;
+            }
+        } else {
+            // block: d, m (one dword), qh (one dword), 16 qs bytes
+            const uint32_t d[12] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y, r.e[0], r.e[1]};
+            w.d0 = h2f(d[0]); w.m0 = h2f(d[0] >> 16);
+            w.d1 = h2f(d[6]); w.m1 = h2f(d[6] >> 16);
+            const uint32_t qh0 = d[1], qh1 = d[7];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                w.lo[i]     = (d[2 + i] & 0x0f0f0f0fu)        | spread4(qh0 >> (4 * i));
+                w.hi[i]     = ((d[2 + i] >> 4) & 0x0f0f0f0fu) | spread4(qh0 >> (16 + 4 * i));
+                w.lo[4 + i] = (d[8 + i] & 0x0f0f0f0fu)        | spread4(qh1 >> (4 * i));
+                w.hi[4 + i] = ((d[8 + i] >> 4) & 0x0f0f0f0fu) | spread4(qh1 >> (16 + 4 * i));
+            }
+        }
+    }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
+        const float4 x = reinterpret_cast<const float4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
+        a.d0 = x.x; a.d1 = x.y; a.s0 = x.z; a.s1 = x.w;
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
+        i0 = 0; i1 = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            i0 = dot4(w.lo[i], a.q[i], i0);         i0 = dot4(w.hi[i], a.q[4 + i], i0);
+            i1 = dot4(w.lo[4 + i], a.q[8 + i], i1); i1 = dot4(w.hi[4 + i], a.q[12 + i], i1);
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int i0, i1;
+        isums(w, a, i0, i1);
+        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
+        acc = __builtin_fmaf(w.m0, a.s0, acc);
+        acc = __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
+        return __builtin_fmaf(w.m1, a.s1, acc);
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
+    using AuxT = float4;
+    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) {
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (valid) {
+            const float2 d = reinterpret_cast<const float2 *>(ws + q8_0_off_d(K))[u];
+            const float2 s = reinterpret_cast<const float2 *>(ws + q8_0_off_s(K))[u];
+            x = make_float4(d.x, d.y, s.x, s.y);
+        }
+        return x;
+    }
+    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_0>::img_qs(NI, e); }
+    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int, float s) {
+        float *a = reinterpret_cast<float *>(img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX);
+        a[blk & 1] = d;
+        a[2 + (blk & 1)] = s;
+    }
+};
+template <> struct Traits<T_Q4_1> : TraitsMin32<T_Q4_1> {};
+template <> struct Traits<T_Q5_1> : TraitsMin32<T_Q5_1> {};
 
 template <> struct Traits<T_Q5_K> {
     // block_q5_K (ggml-common.h:303-314): as q4_K plus qh[32]: bit 2jp of qh[l] is the fifth bit of element l of
@@ -603,13 +703,14 @@ __device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, 
                         const int e = 4 * c, blk = e >> 5;
                         *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, e)) = q[u].packed;
                         const float d = h2f(q[u].dh);
-                        if ((threadIdx.x & 7) == 0) T::img_block_aux(im, NI, blk, d, q[u].sum);
+                        if ((threadIdx.x & 7) == 0) T::img_block_aux(im, NI, blk, d, q[u].sum, h2f(q[u].sh));
                         if (dump) {
                             uint8_t *base = ws + t * ws_stride;
                             *reinterpret_cast<uint32_t *>(base + e) = q[u].packed;
                             if ((threadIdx.x & 7) == 0) {
                                 reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = d;
                                 reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q[u].sum;
+                                reinterpret_cast<float *>(base + q8_0_off_s(K))[blk] = h2f(q[u].sh);
                             }
                         }
                     }
@@ -921,6 +1022,8 @@ int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
         case T_Q5_0: return max_tokens_typed<T_Q5_0>(K, lim);
         case T_Q5_K: return max_tokens_typed<T_Q5_K>(K, lim);
         case T_IQ4_NL: return max_tokens_typed<T_IQ4_NL>(K, lim);
+        case T_Q4_1: return max_tokens_typed<T_Q4_1>(K, lim);
+        case T_Q5_1: return max_tokens_typed<T_Q5_1>(K, lim);
         default: return 0;
     }
 }
@@ -937,6 +1040,8 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
         case T_Q5_0: return launch_ntok<T_Q5_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q4_1: return launch_ntok<T_Q4_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q5_1: return launch_ntok<T_Q5_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
@@ -954,6 +1059,8 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
         case T_Q5_0: img = lds_image_bytes<T_Q5_0>(K); break;
         case T_Q5_K: img = lds_image_bytes<T_Q5_K>(K); break;
         case T_IQ4_NL: img = lds_image_bytes<T_IQ4_NL>(K); break;
+        case T_Q4_1: img = lds_image_bytes<T_Q4_1>(K); break;
+        case T_Q5_1: img = lds_image_bytes<T_Q5_1>(K); break;
         default: return false;
     }
     return (size_t)n * img <= (size_t)lim.max_lds_per_block;
@@ -970,11 +1077,20 @@ hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, i
         case T_Q5_0: return launch_ntok<T_Q5_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         case T_Q5_K: return launch_ntok<T_Q5_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q4_1: return launch_ntok<T_Q4_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q5_1: return launch_ntok<T_Q5_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
 
 // ------------------------------------------------------------------------------------------------ isum hook
+// Reference activation record of a 32-element type: block_q8_0 (34 bytes, quants at +2) unless the traits say
+// block_q8_1 (36 bytes, quants at +4).
+template <typename T, typename = void> struct ActBlock { static constexpr int BYTES = BYTES_Q8_0, QOFF = 2; };
+template <typename T> struct ActBlock<T, decltype((void)T::ABLK_BYTES)> { static constexpr int BYTES = T::ABLK_BYTES, QOFF = T::ABLK_QOFF; };
+template <typename T> __host__ __device__ constexpr int act_block_bytes() { return ActBlock<T>::BYTES; }
+template <typename T> __host__ __device__ constexpr int act_block_qoff() { return ActBlock<T>::QOFF; }
+
 // Per-block integer sums through the same load_w / isums device code.  One wave per (token, row); activations
 // come from reference-layout blocks and are converted to the unit form on the fly (slow path, tests only).
 template <int WT>
@@ -986,7 +1102,7 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
     const int lane = threadIdx.x;
     const int units = units_per_row<WT>(K);
     const int64_t nblk = K / (T::ACT == T_Q8_0 ? 32 : 256);
-    const size_t a_row = (size_t)(T::ACT == T_Q8_0 ? (K / 32) * BYTES_Q8_0 : (K / 256) * BYTES_Q8_K);
+    const size_t a_row = (size_t)(T::ACT == T_Q8_0 ? (K / 32) * act_block_bytes<T>() : (K / 256) * BYTES_Q8_K);
     const uint8_t *arow = aq + t * a_row;
     int32_t *out = isum + ((size_t)t * N + row) * nblk;
     int32_t *outm = imin ? imin + ((size_t)t * N + row) * nblk : nullptr;
@@ -1002,7 +1118,7 @@ __global__ __launch_bounds__(64) void block_isums_kernel(const uint8_t *__restri
             // gather this unit's activation bytes from reference blocks
             if constexpr (T::ACT == T_Q8_0) {
                 for (int b = 0; b < 2; b++) {
-                    const uint8_t *blk = arow + (size_t)(2 * u + b) * BYTES_Q8_0;
+                    const uint8_t *blk = arow + (size_t)(2 * u + b) * act_block_bytes<T>() + (act_block_qoff<T>() - 2);
                     int s = 0;
                     for (int i = 0; i < 8; i++) {
                         uint32_t d = blk[2 + 4 * i] | (blk[3 + 4 * i] << 8) | (blk[4 + 4 * i] << 16) | ((uint32_t)blk[5 + 4 * i] << 24);
@@ -1060,6 +1176,8 @@ hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, 
         case T_Q5_0: hipLaunchKernelGGL(block_isums_kernel<T_Q5_0>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q5_K: hipLaunchKernelGGL(block_isums_kernel<T_Q5_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_IQ4_NL: hipLaunchKernelGGL(block_isums_kernel<T_IQ4_NL>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q4_1: hipLaunchKernelGGL(block_isums_kernel<T_Q4_1>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_Q5_1: hipLaunchKernelGGL(block_isums_kernel<T_Q5_1>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

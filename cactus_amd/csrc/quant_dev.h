@@ -21,9 +21,20 @@ __device__ __forceinline__ uint32_t pack_i8x4(int q0, int q1, int q2, int q3) {
 struct Q8_0Lane {
     uint32_t packed;        // this lane's four quants
     unsigned short dh;      // block scale as fp16 bits (same in the 8 lanes of the block)
+    unsigned short sh;      // block_q8_1.s as fp16 bits: fp16(d * sum) with the unrounded d and the sum of the int32
+                            // conversion results before saturation (reference ggml-cpu/ggml-cpu-quants.c:1094)
     int sum;                // sum of the block's 32 quants (same in the 8 lanes)
 };
 // Eight consecutive lanes hold one 32-value block, four consecutive values each.  All 64 lanes must be active.
+// fp16(a * b) with the product rounded to fp32 first, as the C source of the reference computes it; the empty asm
+// keeps the compiler from folding the multiply into a single-rounding mixed-precision instruction
+__device__ __forceinline__ unsigned short f2h_of_product(float a, float b) {
+    float p = a * b;
+    asm volatile("" : "+v"(p));
+    return f2h_rne(p);
+}
+__device__ __forceinline__ int to_i32_x86(float r) { return (fabsf(r) < 2147483648.f) ? (int)r : INT32_MIN; }
+__device__ __forceinline__ int clamp_i8(int q) { return max(-128, min(127, q)); }
 __device__ __forceinline__ Q8_0Lane quantize_q8_0_lane_general(float4 v) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = fmaxf(amax, dpp_get<0xB1>(amax));
@@ -31,17 +42,22 @@ __device__ __forceinline__ Q8_0Lane quantize_q8_0_lane_general(float4 v) {
     amax = fmaxf(amax, dpp_get<0x141>(amax));
     const float d = amax / 127.f;
     const float id = (amax != 0.0f) ? 127.f / amax : 0.0f;
-    const int q0 = to_i8_x86(__builtin_rintf(v.x * id));
-    const int q1 = to_i8_x86(__builtin_rintf(v.y * id));
-    const int q2 = to_i8_x86(__builtin_rintf(v.z * id));
-    const int q3 = to_i8_x86(__builtin_rintf(v.w * id));
+    const int w0 = to_i32_x86(__builtin_rintf(v.x * id)), w1 = to_i32_x86(__builtin_rintf(v.y * id));
+    const int w2 = to_i32_x86(__builtin_rintf(v.z * id)), w3 = to_i32_x86(__builtin_rintf(v.w * id));
+    const int q0 = clamp_i8(w0), q1 = clamp_i8(w1), q2 = clamp_i8(w2), q3 = clamp_i8(w3);
     int s = q0 + q1 + q2 + q3;
     s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xf, 0xf, true);
     s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xf, 0xf, true);
     s += __builtin_amdgcn_update_dpp(0, s, 0x141, 0xf, 0xf, true);
+    // the unsaturated sum wraps like the 32-bit vector adds of the reference
+    unsigned us = (unsigned)w0 + (unsigned)w1 + (unsigned)w2 + (unsigned)w3;
+    us += (unsigned)__builtin_amdgcn_update_dpp(0, (int)us, 0xB1, 0xf, 0xf, true);
+    us += (unsigned)__builtin_amdgcn_update_dpp(0, (int)us, 0x4E, 0xf, 0xf, true);
+    us += (unsigned)__builtin_amdgcn_update_dpp(0, (int)us, 0x141, 0xf, 0xf, true);
     Q8_0Lane r;
     r.packed = pack_i8x4(q0, q1, q2, q3);
     r.dh = f2h_rne(d);
+    r.sh = f2h_of_product(d, (float)(int)us);
     r.sum = s;
     return r;
 }
@@ -132,6 +148,7 @@ __device__ __forceinline__ Q8_0Lane quantize_q8_0_lane(float4 v) {
     sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xf, 0xf, true);
     sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xf, 0xf, true);
     r.dh = f2h_rne(d);
+    r.sh = f2h_of_product(d, (float)sum);
     r.sum = sum;
     return r;
 }

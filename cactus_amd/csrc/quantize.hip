@@ -15,7 +15,8 @@
 
 namespace chip {
 
-template <bool SPLIT>
+// FMT: 0 = workspace planes, 1 = block_q8_0 records, 2 = block_q8_1 records (reference ggml-common.h:216-227)
+template <int FMT>
 __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, int64_t ldx, int64_t K,
                                                            uint8_t *__restrict__ y, size_t y_stride) {
     const int64_t t = blockIdx.y;
@@ -27,17 +28,22 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     const int64_t blk = e0 / 32;
     const int sub = threadIdx.x & 7;
     if (!live) return;
-    if (SPLIT) {
+    if (FMT == 0) {
         uint8_t *base = y + t * y_stride;
         *reinterpret_cast<uint32_t *>(base + e0) = q.packed;
         if (sub == 0) {
             reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = h2f(q.dh);
             reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q.sum;
+            reinterpret_cast<float *>(base + q8_0_off_s(K))[blk] = h2f(q.sh);
         }
-    } else {
+    } else if (FMT == 1) {
         uint8_t *b = y + t * y_stride + blk * BYTES_Q8_0;
         *reinterpret_cast<u32_a2 *>(b + 2 + 4 * sub) = q.packed;
         if (sub == 0) *reinterpret_cast<unsigned short *>(b) = q.dh;
+    } else {
+        uint8_t *b = y + t * y_stride + blk * BYTES_Q8_1;
+        *reinterpret_cast<uint32_t *>(b + 4 + 4 * sub) = q.packed;
+        if (sub == 0) *reinterpret_cast<uint32_t *>(b) = (uint32_t)q.dh | ((uint32_t)q.sh << 16);
     }
 }
 
@@ -74,6 +80,17 @@ __global__ void split_to_blocks_q8_0_kernel(const uint8_t *__restrict__ ws, size
     *reinterpret_cast<unsigned short *>(b) = f2h_rne(reinterpret_cast<const float *>(base + q8_0_off_d(K))[blk]);
     for (int i = 0; i < 32; i++) b[2 + i] = base[blk * 32 + i];
 }
+__global__ void split_to_blocks_q8_1_kernel(const uint8_t *__restrict__ ws, size_t ws_stride, int64_t K,
+                                            uint8_t *__restrict__ y, size_t y_stride) {
+    const int64_t t = blockIdx.y;
+    const int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (blk >= K / 32) return;
+    const uint8_t *base = ws + t * ws_stride;
+    uint8_t *b = y + t * y_stride + blk * BYTES_Q8_1;
+    reinterpret_cast<unsigned short *>(b)[0] = f2h_rne(reinterpret_cast<const float *>(base + q8_0_off_d(K))[blk]);
+    reinterpret_cast<unsigned short *>(b)[1] = f2h_rne(reinterpret_cast<const float *>(base + q8_0_off_s(K))[blk]);
+    for (int i = 0; i < 32; i++) b[4 + i] = base[blk * 32 + i];
+}
 __global__ void split_to_blocks_q8_K_kernel(const uint8_t *__restrict__ ws, size_t ws_stride, int64_t K,
                                             uint8_t *__restrict__ y, size_t y_stride) {
     const int64_t t = blockIdx.y;
@@ -91,9 +108,11 @@ hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx
                            size_t y_stride, hipStream_t st) {
     if (n <= 0 || K <= 0) return hipSuccess;
     dim3 grid((unsigned)ceil_div(K, 1024), (unsigned)n);
-    if (act_type == T_Q8_0) {
-        if (split) hipLaunchKernelGGL(quantize_q8_0_kernel<true>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
-        else       hipLaunchKernelGGL(quantize_q8_0_kernel<false>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+    if (act_type == T_Q8_0 || act_type == T_Q8_1) {
+        // Q8_1 shares the Q8_0 workspace planes (which carry its s); only the block records differ
+        if (split)                  hipLaunchKernelGGL(quantize_q8_0_kernel<0>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+        else if (act_type == T_Q8_0) hipLaunchKernelGGL(quantize_q8_0_kernel<1>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+        else                        hipLaunchKernelGGL(quantize_q8_0_kernel<2>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
     } else {
         if (split) hipLaunchKernelGGL(quantize_q8_K_kernel<true>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
         else       hipLaunchKernelGGL(quantize_q8_K_kernel<false>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
@@ -104,10 +123,14 @@ hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx
 hipError_t launch_split_to_blocks(int act_type, const void *ws, size_t ws_stride, int64_t n, int64_t K, void *y,
                                   size_t y_stride, hipStream_t st) {
     if (n <= 0 || K <= 0) return hipSuccess;
-    if (act_type == T_Q8_0) {
+    if (act_type == T_Q8_0 || act_type == T_Q8_1) {
         dim3 grid((unsigned)ceil_div(K / 32, 256), (unsigned)n);
-        hipLaunchKernelGGL(split_to_blocks_q8_0_kernel, grid, dim3(256), 0, st, (const uint8_t *)ws, ws_stride, K,
-                           (uint8_t *)y, y_stride);
+        if (act_type == T_Q8_0)
+            hipLaunchKernelGGL(split_to_blocks_q8_0_kernel, grid, dim3(256), 0, st, (const uint8_t *)ws, ws_stride, K,
+                               (uint8_t *)y, y_stride);
+        else
+            hipLaunchKernelGGL(split_to_blocks_q8_1_kernel, grid, dim3(256), 0, st, (const uint8_t *)ws, ws_stride, K,
+                               (uint8_t *)y, y_stride);
     } else {
         dim3 grid((unsigned)(K / 256), (unsigned)n);
         hipLaunchKernelGGL(split_to_blocks_q8_K_kernel, grid, dim3(256), 0, st, (const uint8_t *)ws, ws_stride, K,

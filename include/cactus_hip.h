@@ -35,6 +35,9 @@ enum chip_type {
     CHIP_TYPE_Q5_0   = 6,
     CHIP_TYPE_Q5_K   = 13,
     CHIP_TYPE_IQ4_NL = 20,
+    CHIP_TYPE_Q4_1   = 3,
+    CHIP_TYPE_Q5_1   = 7,
+    CHIP_TYPE_Q8_1   = 9,    /* activation format of Q4_1 / Q5_1 (ggml-cpu/ggml-cpu.c:221,237) */
 };
 
 enum chip_status {
@@ -79,7 +82,7 @@ CHIP_API int    chip_block_elems(int type);
 CHIP_API size_t chip_block_bytes(int type);
 CHIP_API size_t chip_row_size(int type, int64_t k);
 /* type_traits_cpu[type].vec_dot_type (ggml-cpu/ggml-cpu.c:198-367): Q8_0 for Q4_0/Q8_0/Q5_0/IQ4_NL, Q8_K for
- * Q4_K/Q5_K/Q6_K */
+ * Q4_K/Q5_K/Q6_K, Q8_1 for Q4_1/Q5_1 */
 CHIP_API int    chip_vec_dot_type(int type);
 /* 1 if chip_mul_mat accepts this weight type and K (K must be a multiple of 256) */
 CHIP_API int    chip_mul_mat_supported(int type, int64_t K);
@@ -93,6 +96,9 @@ CHIP_API int    chip_mul_mat_supported(int type, int64_t K);
  * reference leaves unwritten). */
 CHIP_API int chip_quantize_q8_0(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
 CHIP_API int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
+/* quantize_row_q8_1, AVX2 branch (ggml-cpu/ggml-cpu-quants.c:1047-1140): the activation format of Q4_1 / Q5_1;
+ * quants and d as Q8_0, plus s = fp16(d * sum of quants) */
+CHIP_API int chip_quantize_q8_1(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
 
 /* ---- the op: LM_GGML_OP_MUL_MAT over block-quantized weights ----
  * lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449) with src0 = W (type, [K, N], row stride

@@ -17,15 +17,19 @@ REF_SO = os.path.join(HERE, "_ref", "libggml_ref.so")
 # lm_ggml_type values (reference ggml.h:351-391)
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
+Q4_1, Q5_1, Q8_1 = 3, 7, 9
 TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
-              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl"}
-BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32}
-BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18}
-VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL)
+              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1"}
+BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32,
+               Q4_1: 32, Q5_1: 32, Q8_1: 32}
+BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18,
+               Q4_1: 20, Q5_1: 24, Q8_1: 36}
+VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0,
+                Q4_1: Q8_1, Q5_1: Q8_1}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1)
 # types whose weight quantizer is restated in the oracle (IQ4_NL weights come from the reference build, from the
 # golden fixture, or are random bytes: any byte string is a valid block)
-ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K)
+ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, Q4_1, Q5_1)
 
 
 IQ4_NL_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
@@ -97,7 +101,8 @@ class Oracle:
         L.orc_fp16_to_fp32.argtypes = [C.c_uint16]
         L.orc_fp32_to_fp16.restype = C.c_uint16
         L.orc_fp32_to_fp16.argtypes = [C.c_float]
-        for n in ("q8_0", "q8_K", "q4_0_ref", "q8_0_ref", "q4_K_ref", "q6_K_ref", "q5_0_ref", "q5_K_ref"):
+        for n in ("q8_0", "q8_K", "q8_1", "q4_0_ref", "q8_0_ref", "q4_K_ref", "q6_K_ref", "q5_0_ref", "q5_K_ref",
+                  "q4_1_ref", "q5_1_ref"):
             f = getattr(L, "orc_quantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
@@ -105,7 +110,7 @@ class Oracle:
         L.orc_quantize_rows.argtypes = [_i32, _vp, _vp, _i64, _i64]
         L.orc_dequantize_row.restype = None
         L.orc_dequantize_row.argtypes = [_i32, _vp, _vp, _i64]
-        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0"):
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0", "q4_1_q8_1", "q5_1_q8_1"):
             f = getattr(L, "orc_vec_dot_" + n)
             f.restype = C.c_float
             f.argtypes = [_i64, _vp, _vp, _vp]
@@ -132,7 +137,8 @@ class Oracle:
         k = x.shape[-1]
         rows = x.reshape(-1, k)
         out = np.zeros((rows.shape[0], row_size(act_type, k)), np.uint8)
-        fn = {Q8_0: self.lib.orc_quantize_row_q8_0, Q8_K: self.lib.orc_quantize_row_q8_K}[act_type]
+        fn = {Q8_0: self.lib.orc_quantize_row_q8_0, Q8_K: self.lib.orc_quantize_row_q8_K,
+              Q8_1: self.lib.orc_quantize_row_q8_1}[act_type]
         for r in range(rows.shape[0]):
             fn(_ptr(rows[r]), _ptr(out[r]), k)
         return out.reshape(x.shape[:-1] + (out.shape[1],))
@@ -185,6 +191,10 @@ class Oracle:
             v = self.lib.orc_vec_dot_iq4_nl_q8_0(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q5_K:
             v = self.lib.orc_vec_dot_q5_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
+        elif wtype == Q4_1:
+            v = self.lib.orc_vec_dot_q4_1_q8_1(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == Q5_1:
+            v = self.lib.orc_vec_dot_q5_1_q8_1(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         else:
             raise ValueError(wtype)
         v = np.float32(v)
@@ -243,15 +253,17 @@ class Reference:
         L.lm_ggml_free(ctx)
         for n in ("quantize_row_q8_0", "quantize_row_q8_K", "quantize_row_q4_0_ref", "quantize_row_q8_0_ref",
                   "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref",
-                  "quantize_row_q5_0_ref", "quantize_row_q5_K_ref", "quantize_row_iq4_nl_ref"):
+                  "quantize_row_q5_0_ref", "quantize_row_q5_K_ref", "quantize_row_iq4_nl_ref",
+                  "quantize_row_q4_1_ref", "quantize_row_q5_1_ref", "quantize_row_q8_1"):
             f = getattr(L, n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
-        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl"):
+        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl", "q4_1", "q5_1"):
             f = getattr(L, "dequantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
-        for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "q5_0_q8_0", "q5_K_q8_K", "iq4_nl_q8_0"):
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "q5_0_q8_0", "q5_K_q8_K", "iq4_nl_q8_0",
+                  "q4_1_q8_1", "q5_1_q8_1"):
             f = getattr(L, "lm_ggml_vec_dot_" + n)
             f.restype = None
             f.argtypes = [C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, _vp, C.c_size_t, C.c_int]
@@ -284,13 +296,15 @@ class Reference:
         L.lm_ggml_threadpool_free.argtypes = [_vp]
         L.lm_ggml_threadpool_params_init.argtypes = [_vp, _i32]
 
-    _ACT = {Q8_0: "quantize_row_q8_0", Q8_K: "quantize_row_q8_K"}
+    _ACT = {Q8_0: "quantize_row_q8_0", Q8_K: "quantize_row_q8_K", Q8_1: "quantize_row_q8_1"}
     _WQ = {Q4_0: "quantize_row_q4_0_ref", Q8_0: "quantize_row_q8_0_ref",
            Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref",
-           Q5_0: "quantize_row_q5_0_ref", Q5_K: "quantize_row_q5_K_ref", IQ4_NL: "quantize_row_iq4_nl_ref"}
+           Q5_0: "quantize_row_q5_0_ref", Q5_K: "quantize_row_q5_K_ref", IQ4_NL: "quantize_row_iq4_nl_ref",
+           Q4_1: "quantize_row_q4_1_ref", Q5_1: "quantize_row_q5_1_ref"}
     _DOT = {Q4_0: "lm_ggml_vec_dot_q4_0_q8_0", Q8_0: "lm_ggml_vec_dot_q8_0_q8_0",
             Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K",
-            Q5_0: "lm_ggml_vec_dot_q5_0_q8_0", Q5_K: "lm_ggml_vec_dot_q5_K_q8_K", IQ4_NL: "lm_ggml_vec_dot_iq4_nl_q8_0"}
+            Q5_0: "lm_ggml_vec_dot_q5_0_q8_0", Q5_K: "lm_ggml_vec_dot_q5_K_q8_K", IQ4_NL: "lm_ggml_vec_dot_iq4_nl_q8_0",
+            Q4_1: "lm_ggml_vec_dot_q4_1_q8_1", Q5_1: "lm_ggml_vec_dot_q5_1_q8_1"}
 
     def quantize_activation(self, act_type, x):
         x = _f32(x)

@@ -24,6 +24,10 @@ typedef struct { float d; int8_t qs[256]; int16_t bsums[16]; } blk_q8_K;
 typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_0;
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qh[32]; uint8_t qs[128]; } blk_q5_K;
 typedef struct { uint16_t d; uint8_t qs[16]; } blk_iq4_nl;
+/* min-based types and their activation format: ggml-common.h:175-185 (q4_1), :196-207 (q5_1), :216-227 (q8_1) */
+typedef struct { uint16_t d; uint16_t m; uint8_t qs[16]; } blk_q4_1;
+typedef struct { uint16_t d; uint16_t m; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_1;
+typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } blk_q8_1;
 #pragma pack(pop)
 
 _Static_assert(sizeof(blk_q4_0) == 18, "q4_0");
@@ -34,6 +38,9 @@ _Static_assert(sizeof(blk_q8_K) == 292, "q8_K");
 _Static_assert(sizeof(blk_q5_0) == 22, "q5_0");
 _Static_assert(sizeof(blk_q5_K) == 176, "q5_K");
 _Static_assert(sizeof(blk_iq4_nl) == 18, "iq4_nl");
+_Static_assert(sizeof(blk_q4_1) == 20, "q4_1");
+_Static_assert(sizeof(blk_q5_1) == 24, "q5_1");
+_Static_assert(sizeof(blk_q8_1) == 36, "q8_1");
 
 /* ggml-quants.c:2428: the 16 code points of the non-linear 4-bit types. */
 static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
@@ -41,7 +48,8 @@ static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10
 int orc_block_elems(int type) {
     switch (type) {
         case ORC_TYPE_F32: return 1;
-        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return 32;
+        case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL:
+        case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: case ORC_TYPE_Q8_1: return 32;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
         default: return 0;
     }
@@ -57,6 +65,9 @@ size_t orc_block_bytes(int type) {
         case ORC_TYPE_Q5_0: return 22;
         case ORC_TYPE_Q5_K: return 176;
         case ORC_TYPE_IQ4_NL: return 18;
+        case ORC_TYPE_Q4_1: return 20;
+        case ORC_TYPE_Q5_1: return 24;
+        case ORC_TYPE_Q8_1: return 36;
         default: return 0;
     }
 }
@@ -68,6 +79,7 @@ int orc_vec_dot_type(int type) {
     switch (type) { /* ggml-cpu/ggml-cpu.c:213,245,272,284; :229 (q5_0), :278 (q5_K), :340 (iq4_nl) */
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return ORC_TYPE_Q8_0;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
+        case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: return ORC_TYPE_Q8_1;   /* ggml-cpu/ggml-cpu.c:221,237 */
         default: return -1;
     }
 }
@@ -143,6 +155,28 @@ void orc_quantize_row_q8_0(const float *x, void *vy, int64_t k) {
             const int q = fabsf(r) < 2147483648.f ? (int)r : INT32_MIN;
             y[b].qs[j] = (int8_t)imax_(-128, imin_(127, q));
         }
+    }
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:1047-1140 (AVX2 branch of quantize_row_q8_1): the quants and d are those of
+ * quantize_row_q8_0; s = fp16(d * sum) with the *unrounded* fp32 d and the sum of the 32 int32 conversion
+ * results before the saturating packs (wrapping 32-bit adds), :1094. */
+void orc_quantize_row_q8_1(const float *x, void *vy, int64_t k) {
+    blk_q8_1 *y = (blk_q8_1 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) { float a = fabsf(x[j]); if (a > amax) amax = a; }
+        const float d = amax / 127.f;
+        const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+        y[b].d = F2H(d);
+        uint32_t sum = 0;
+        for (int j = 0; j < 32; j++) {
+            const float r = nearbyintf(x[j] * id);
+            const int q = fabsf(r) < 2147483648.f ? (int)r : INT32_MIN;
+            sum += (uint32_t)q;
+            y[b].qs[j] = (int8_t)imax_(-128, imin_(127, q));
+        }
+        y[b].s = F2H(d * (float)(int32_t)sum);
     }
 }
 
@@ -384,6 +418,47 @@ void orc_quantize_row_q5_K_ref(const float *x, void *vy, int64_t k) {
     }
 }
 
+/* ggml-quants.c:62-97. */
+void orc_quantize_row_q4_1_ref(const float *x, void *vy, int64_t k) {
+    blk_q4_1 *y = (blk_q4_1 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+        for (int j = 0; j < 32; j++) { if (x[j] < mn) mn = x[j]; if (x[j] > mx) mx = x[j]; }
+        const float d = (mx - mn) / 15;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = F2H(d);
+        y[b].m = F2H(mn);
+        for (int j = 0; j < 16; j++) {
+            const float x0 = (x[j] - mn) * id, x1 = (x[16 + j] - mn) * id;
+            const uint8_t xi0 = (uint8_t)imin_(15, (int8_t)(x0 + 0.5f));
+            const uint8_t xi1 = (uint8_t)imin_(15, (int8_t)(x1 + 0.5f));
+            y[b].qs[j] = (uint8_t)(xi0 | (xi1 << 4));
+        }
+    }
+}
+
+/* ggml-quants.c:143-186. */
+void orc_quantize_row_q5_1_ref(const float *x, void *vy, int64_t k) {
+    blk_q5_1 *y = (blk_q5_1 *)vy;
+    for (int64_t b = 0; b < k / 32; b++, x += 32) {
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+        for (int j = 0; j < 32; j++) { if (x[j] < mn) mn = x[j]; if (x[j] > mx) mx = x[j]; }
+        const float d = (mx - mn) / 31;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = F2H(d);
+        y[b].m = F2H(mn);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            const float x0 = (x[j] - mn) * id, x1 = (x[16 + j] - mn) * id;
+            const uint8_t xi0 = (uint8_t)(x0 + 0.5f), xi1 = (uint8_t)(x1 + 0.5f);
+            y[b].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= ((xi0 & 0x10u) >> 4) << (j + 0);
+            qh |= ((xi1 & 0x10u) >> 4) << (j + 16);
+        }
+        memcpy(y[b].qh, &qh, 4);
+    }
+}
+
 /* ggml-quants.c:99-141. */
 void orc_quantize_row_q5_0_ref(const float *x, void *vy, int64_t k) {
     blk_q5_0 *y = (blk_q5_0 *)vy;
@@ -506,6 +581,8 @@ size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64
             case ORC_TYPE_Q6_K: orc_quantize_row_q6_K_ref(src, dst, k); break;
             case ORC_TYPE_Q5_K: orc_quantize_row_q5_K_ref(src, dst, k); break;
             case ORC_TYPE_Q5_0: orc_quantize_row_q5_0_ref(src, dst, k); break;
+            case ORC_TYPE_Q4_1: orc_quantize_row_q4_1_ref(src, dst, k); break;
+            case ORC_TYPE_Q5_1: orc_quantize_row_q5_1_ref(src, dst, k); break;
             default: return 0;
         }
     }
@@ -598,6 +675,34 @@ void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
                 for (int l = 0; l < 32; l++) *y++ = d2 * ((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
                 u1 = (uint8_t)(u1 << 2); u2 = (uint8_t)(u2 << 2);
             }
+        }
+    } else if (type == ORC_TYPE_Q4_1) {                 /* ggml-quants.c:269-288 */
+        const blk_q4_1 *x = (const blk_q4_1 *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d), m = H2F(x[b].m);
+            for (int j = 0; j < 16; j++) {
+                y[j]      = (x[b].qs[j] & 0x0F) * d + m;
+                y[j + 16] = (x[b].qs[j] >> 4) * d + m;
+            }
+        }
+    } else if (type == ORC_TYPE_Q5_1) {                 /* ggml-quants.c:315-341 */
+        const blk_q5_1 *x = (const blk_q5_1 *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d), m = H2F(x[b].m);
+            uint32_t qh;
+            memcpy(&qh, x[b].qh, 4);
+            for (int j = 0; j < 16; j++) {
+                const uint8_t xh0 = (uint8_t)(((qh >> (j + 0)) << 4) & 0x10);
+                const uint8_t xh1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+                y[j]      = (float)((x[b].qs[j] & 0x0F) | xh0) * d + m;
+                y[j + 16] = (float)((x[b].qs[j] >> 4) | xh1) * d + m;
+            }
+        }
+    } else if (type == ORC_TYPE_Q8_1) {
+        const blk_q8_1 *x = (const blk_q8_1 *)vx;
+        for (int64_t b = 0; b < k / 32; b++, y += 32) {
+            const float d = H2F(x[b].d);
+            for (int j = 0; j < 32; j++) y[j] = x[b].qs[j] * d;
         }
     } else if (type == ORC_TYPE_IQ4_NL) {               /* ggml-quants.c:2430-2446 */
         const blk_iq4_nl *x = (const blk_iq4_nl *)vx;
@@ -843,6 +948,48 @@ float orc_vec_dot_iq4_nl_q8_0(int64_t k, const void *vx, const void *vy, int32_t
     return sumf;
 }
 
+/* q4_1 / q5_1 x q8_1: AVX2 branches of lm_ggml_vec_dot_q4_1_q8_1 and lm_ggml_vec_dot_q5_1_q8_1
+ * (ggml-cpu/ggml-cpu-quants.c): unsigned weights u (nibble, or nibble | bit << 4), lane j takes the four
+ * products of elements 4j..4j+3, acc = fmadd(dx*dy, float(p), acc); the min term is the scalar
+ * summs += m * s (separate multiply and add), added after the horizontal sum. */
+static float dot_min32(int type, int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q8_1 *y = (const blk_q8_1 *)vy;
+    float acc[8] = {0};
+    float summs = 0.f;
+    for (int64_t b = 0; b < k / 32; b++) {
+        uint8_t w[32];
+        uint16_t dh, mh;
+        if (type == ORC_TYPE_Q4_1) {
+            const blk_q4_1 *x = (const blk_q4_1 *)vx + b;
+            for (int j = 0; j < 16; j++) { w[j] = x->qs[j] & 0xF; w[j + 16] = x->qs[j] >> 4; }
+            dh = x->d; mh = x->m;
+        } else {
+            const blk_q5_1 *x = (const blk_q5_1 *)vx + b;
+            uint32_t qh;
+            memcpy(&qh, x->qh, 4);
+            for (int j = 0; j < 16; j++) {
+                w[j]      = (uint8_t)((x->qs[j] & 0xF) | (((qh >> j) & 1) << 4));
+                w[j + 16] = (uint8_t)((x->qs[j] >> 4) | (((qh >> (j + 16)) & 1) << 4));
+            }
+            dh = x->d; mh = x->m;
+        }
+        const float prod = H2F(mh) * H2F(y[b].s);
+        summs = summs + prod;
+        const float d = H2F(dh) * H2F(y[b].d);
+        int32_t tot = 0;
+        for (int j = 0; j < 8; j++) {
+            int32_t p = 0;
+            for (int t = 0; t < 4; t++) p += (int32_t)w[4 * j + t] * y[b].qs[4 * j + t];
+            tot += p;
+            acc[j] = fmaf(d, (float)p, acc[j]);
+        }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc) + summs;
+}
+float orc_vec_dot_q4_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *isum) { return dot_min32(ORC_TYPE_Q4_1, k, vx, vy, isum); }
+float orc_vec_dot_q5_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *isum) { return dot_min32(ORC_TYPE_Q5_1, k, vx, vy, isum); }
+
 /* q5_K: AVX2 branch of lm_ggml_vec_dot_q5_K_q8_K (ggml-cpu/ggml-cpu-quants.c:7786-7860): as q4_K for the d term
  * (one integer 8-lane sum per super-block, one fmadd), but the min term is a scalar
  * `summs += dmin * hsum` (separate multiply and add) added after the horizontal sum. */
@@ -896,6 +1043,8 @@ float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
         case ORC_TYPE_Q5_0: return orc_vec_dot_q5_0_q8_0(k, vx, vy, NULL);
         case ORC_TYPE_IQ4_NL: return orc_vec_dot_iq4_nl_q8_0(k, vx, vy, NULL);
         case ORC_TYPE_Q5_K: return orc_vec_dot_q5_K_q8_K(k, vx, vy, NULL, NULL);
+        case ORC_TYPE_Q4_1: return orc_vec_dot_q4_1_q8_1(k, vx, vy, NULL);
+        case ORC_TYPE_Q5_1: return orc_vec_dot_q5_1_q8_1(k, vx, vy, NULL);
         default: return NAN;
     }
 }
@@ -923,6 +1072,16 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
             const uint16_t hx = type == ORC_TYPE_Q5_0 ? ((const blk_q5_0 *)vx)[b].d : ((const blk_iq4_nl *)vx)[b].d;
             const double t = (double)H2F(hx) * (double)H2F(y[b].d) * (double)is[b];
             s += t; sa += fabs(t);
+        }
+    } else if (type == ORC_TYPE_Q4_1 || type == ORC_TYPE_Q5_1) {
+        dot_min32(type, k, vx, vy, is);
+        const blk_q8_1 *y = (const blk_q8_1 *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const uint16_t dh = type == ORC_TYPE_Q4_1 ? ((const blk_q4_1 *)vx)[b].d : ((const blk_q5_1 *)vx)[b].d;
+            const uint16_t mh = type == ORC_TYPE_Q4_1 ? ((const blk_q4_1 *)vx)[b].m : ((const blk_q5_1 *)vx)[b].m;
+            const double t1 = (double)H2F(dh) * (double)H2F(y[b].d) * (double)is[b];
+            const double t2 = (double)H2F(mh) * (double)H2F(y[b].s);
+            s += t1 + t2; sa += fabs(t1) + fabs(t2);
         }
     } else if (type == ORC_TYPE_Q5_K) {
         const blk_q5_K *x = (const blk_q5_K *)vx;
@@ -1017,8 +1176,9 @@ void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const
     const size_t ars = orc_row_size(vdt, K);
     char *wd = wdata ? (char *)wdata : (char *)malloc(ars * (size_t)(n > 0 ? n : 1));
     for (int64_t t = 0; t < n; t++) {
-        if (vdt == ORC_TYPE_Q8_0) orc_quantize_row_q8_0(x + t * K, wd + (size_t)t * ars, K);
-        else                      orc_quantize_row_q8_K(x + t * K, wd + (size_t)t * ars, K);
+        if (vdt == ORC_TYPE_Q8_0)      orc_quantize_row_q8_0(x + t * K, wd + (size_t)t * ars, K);
+        else if (vdt == ORC_TYPE_Q8_1) orc_quantize_row_q8_1(x + t * K, wd + (size_t)t * ars, K);
+        else                           orc_quantize_row_q8_K(x + t * K, wd + (size_t)t * ars, K);
     }
     if (nthreads < 1) nthreads = 1;
     if (nthreads > 256) nthreads = 256;

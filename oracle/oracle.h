@@ -19,6 +19,9 @@
  *   orc_quantize_row_q4_K_ref        bit-exact vs oracle/_ref + golden (iterative search: only the oracle run
  *   orc_quantize_row_q6_K_ref          pins the bytes); reconstruction-error bound as a sanity invariant
  *   orc_quantize_row_q5_0_ref/_q5_K_ref  bit-exact vs oracle/_ref + golden; dequant closed forms
+ *   orc_quantize_row_q4_1_ref/_q5_1_ref  bit-exact vs oracle/_ref + golden; dequant closed form d*u + m
+ *   orc_quantize_row_q8_1            bit-exact vs oracle/_ref on seeded data + golden edge rows; quants and d
+ *                                    equal orc_quantize_row_q8_0's, s == fp16(d * sum q) on finite rows
  *   (iq4_nl has no quantizer here: its weights come from oracle/_ref, committed in the golden fixture, or
  *    are random code indices with a random fp16 scale -- any byte string is a valid iq4_nl block)
  *   orc_dequantize_row_*             closed forms; vs oracle/_ref + golden
@@ -51,6 +54,9 @@ enum orc_type {
     ORC_TYPE_Q5_0 = 6,
     ORC_TYPE_Q5_K = 13,
     ORC_TYPE_IQ4_NL = 20,
+    ORC_TYPE_Q4_1 = 3,
+    ORC_TYPE_Q5_1 = 7,
+    ORC_TYPE_Q8_1 = 9,      /* activation format of Q4_1 / Q5_1 */
 };
 
 /* elements per block / bytes per block / bytes per row of k elements; 0 for an unknown type */
@@ -66,6 +72,7 @@ uint16_t orc_fp32_to_fp16(float f);
 /* activation quantizers (the two the MUL_MAT op calls on the fly) */
 void orc_quantize_row_q8_0(const float *x, void *y, int64_t k);      /* AVX2 semantics */
 void orc_quantize_row_q8_K(const float *x, void *y, int64_t k);
+void orc_quantize_row_q8_1(const float *x, void *y, int64_t k);      /* AVX2 semantics */
 
 /* weight quantizers (offline; their output bytes are the op's input) */
 void orc_quantize_row_q4_0_ref(const float *x, void *y, int64_t k);
@@ -74,6 +81,8 @@ void orc_quantize_row_q4_K_ref(const float *x, void *y, int64_t k);
 void orc_quantize_row_q6_K_ref(const float *x, void *y, int64_t k);
 void orc_quantize_row_q5_0_ref(const float *x, void *y, int64_t k);
 void orc_quantize_row_q5_K_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q4_1_ref(const float *x, void *y, int64_t k);
+void orc_quantize_row_q5_1_ref(const float *x, void *y, int64_t k);
 /* dispatch on weight type, nrows rows of k elements, rows packed back to back; returns bytes written */
 size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64_t k);
 
@@ -95,13 +104,17 @@ float orc_vec_dot_q6_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *
 float orc_vec_dot_q5_0_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot_iq4_nl_q8_0(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot_q5_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin);
+/* q4_1, q5_1: isum[k/32] = sum u*aq with the unsigned weight u; the min term m*s is not part of isum */
+float orc_vec_dot_q4_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot_q5_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
 
 /* fp64 evaluation of sum_b scale_b*isum_b (returned) and of sum_b |scale_b*isum_b| (*sum_abs): the tolerance
  * yardstick 1e-5 * sum_abs and an order-free reference value.  A "block" is the smallest group of values that
  * carries its own scale: 32 values for Q4_0/Q8_0, a 32-value sub-block for Q4_K (terms d*sc_j*dot_j and
  * dmin*m_j*bsum_j, both counted), a 16-value sub-block for Q6_K (d*sc_j*dot_j); Q5_0 and
- * IQ4_NL as Q4_0, Q5_K as Q4_K.  Coarser terms (whole
+ * IQ4_NL as Q4_0, Q5_K as Q4_K;
+ * Q4_1 / Q5_1: d*dy*isum and m*s per 32-block, both counted.  Coarser terms (whole
  * super-blocks) would cancel internally and make a bound that the reference's own AVX2 result misses. */
 double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, double *sum_abs);
 

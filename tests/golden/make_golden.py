@@ -40,6 +40,7 @@ def main():
         np.savez_compressed(os.path.join(HERE, "quantize_q8_0_edges.npz"), x=e0,
                             q_avx2=r.quantize_activation(O.Q8_0, e0),
                             q_ref=np.stack([r.quantize_q8_0_ref(row) for row in e0]))
+        np.savez_compressed(os.path.join(HERE, "quantize_q8_1_edges.npz"), x=e0, q=r.quantize_activation(O.Q8_1, e0))
         ek = common.q8_K_edge_rows()
         np.savez_compressed(os.path.join(HERE, "quantize_q8_K_edges.npz"), x=ek,
                             q=r.quantize_activation(O.Q8_K, ek))

@@ -27,6 +27,8 @@ def test_library_exports_every_declared_symbol():
 def test_layout_queries_need_no_gpu():
     lib = cactus_amd.load_library()
     assert [lib.chip_block_bytes(t) for t in (2, 8, 12, 14, 15)] == [18, 34, 144, 210, 292]
+    assert [lib.chip_block_bytes(t) for t in (6, 13, 20, 3, 7, 9)] == [22, 176, 18, 20, 24, 36]
+    assert lib.chip_vec_dot_type(cactus_amd.Q4_1) == cactus_amd.Q8_1 and lib.chip_vec_dot_type(cactus_amd.Q5_K) == cactus_amd.Q8_K
     assert lib.chip_row_size(cactus_amd.Q4_0, 4096) == 2304
     assert lib.chip_row_size(cactus_amd.Q4_K, 4096) == 2304
     assert lib.chip_row_size(cactus_amd.Q6_K, 14336) == 11760
@@ -35,5 +37,5 @@ def test_layout_queries_need_no_gpu():
     assert lib.chip_mul_mat_supported(cactus_amd.Q4_K, 4096) == 1
     assert lib.chip_mul_mat_supported(cactus_amd.Q4_K, 4000) == 0
     assert lib.chip_mul_mat_supported(1, 4096) == 0           # F16 weights are not on this path
-    assert lib.chip_mul_mat_workspace_size(cactus_amd.Q8_0, 4096, 3) == 3 * (4096 + 8 * 128)
+    assert lib.chip_mul_mat_workspace_size(cactus_amd.Q8_0, 4096, 3) == 3 * (4096 + 12 * 128)   # qs, d, sum, s planes
     assert lib.chip_error_string(-2).decode().startswith("unsupported")

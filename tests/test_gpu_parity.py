@@ -41,7 +41,7 @@ def test_quantizers_bit_exact(dev, orc, K):
     x[2] *= 300
     x[3, : K // 2] = 0
     x[4] = 0
-    for at in (O.Q8_0, O.Q8_K):
+    for at in (O.Q8_0, O.Q8_K, O.Q8_1):
         print("quantize", O.TYPE_NAMES[at], "K", K, flush=True)
         assert np.array_equal(dev.quantize(at, x), orc.quantize_activation(at, x))
 
@@ -49,7 +49,7 @@ def test_quantizers_bit_exact(dev, orc, K):
 def test_quantizers_many_blocks(dev, orc):
     rng = np.random.default_rng(42)
     x = (rng.standard_normal((64, 16384)) * np.exp(rng.uniform(-6, 6, (64, 1)))).astype(np.float32)
-    for at in (O.Q8_0, O.Q8_K):
+    for at in (O.Q8_0, O.Q8_K, O.Q8_1):
         assert np.array_equal(dev.quantize(at, x), orc.quantize_activation(at, x))
 
 
@@ -61,6 +61,10 @@ def test_quantizer_edge_vectors(dev):
     assert np.array_equal(got, g["q_avx2"])
     g = np.load(os.path.join(GOLD, "quantize_q8_K_edges.npz"))
     assert np.array_equal(dev.quantize(O.Q8_K, g["x"]), g["q"])
+    g = np.load(os.path.join(GOLD, "quantize_q8_1_edges.npz"))
+    x = np.zeros((g["x"].shape[0], 256), np.float32)
+    x[:, :32] = g["x"]
+    assert np.array_equal(dev.quantize(O.Q8_1, x)[:, :36], g["q"])
 
 
 # ------------------------------------------------------------------------------------------ the op

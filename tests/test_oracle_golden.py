@@ -52,6 +52,18 @@ def test_quantize_q8_0_edges(orc):
     assert not np.array_equal(g["q_avx2"][1], g["q_ref"][1])
 
 
+def test_quantize_q8_1_edges(orc):
+    g = gold("quantize_q8_1_edges.npz")
+    with np.errstate(all="ignore"):
+        got = orc.quantize_activation(O.Q8_1, g["x"])
+    assert np.array_equal(got, g["q"])
+    # same quants and d as Q8_0 on the same rows
+    g0 = gold("quantize_q8_0_edges.npz")
+    b1 = g["q"].reshape(g["q"].shape[0], -1, 36)
+    b0 = g0["q_avx2"].reshape(g0["q_avx2"].shape[0], -1, 34)
+    assert np.array_equal(b1[..., 4:], b0[..., 2:]) and np.array_equal(b1[..., :2], b0[..., :2])
+
+
 def test_quantize_q8_K_edges(orc):
     g = gold("quantize_q8_K_edges.npz")
     got = orc.quantize_activation(O.Q8_K, g["x"])
