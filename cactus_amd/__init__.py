@@ -21,9 +21,10 @@ BACKEND_LIB = os.path.join(LIB_DIR, "libggml-hip.so")
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
+F16 = 1
 TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
-              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1"}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1)
+              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16"}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, F16)
 
 # every symbol include/cactus_hip.h declares
 EXPORTS = (
@@ -31,7 +32,7 @@ EXPORTS = (
     "chip_memcpy_h2d", "chip_memcpy_d2h", "chip_memcpy_d2d", "chip_memset", "chip_stream_create",
     "chip_stream_destroy", "chip_stream_synchronize", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
-    "chip_quantize_q8_1",
+    "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -82,6 +83,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_quantize_q8_0.argtypes = [vp, i64, i64, i64, vp, vp]
     L.chip_quantize_q8_K.argtypes = [vp, i64, i64, i64, vp, vp]
     L.chip_quantize_q8_1.argtypes = [vp, i64, i64, i64, vp, vp]
+    L.chip_convert_f32_to_f16.argtypes = [vp, i64, i64, i64, vp, vp]
     L.chip_mul_mat_workspace_size.restype = sz
     L.chip_mul_mat_workspace_size.argtypes = [i32, i64, i64]
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
@@ -165,7 +167,7 @@ class Device:
         rs = self.row_size(act_type, k)
         dy = self.alloc(n * rs)
         fn = {Q8_0: self.lib.chip_quantize_q8_0, Q8_K: self.lib.chip_quantize_q8_K,
-              Q8_1: self.lib.chip_quantize_q8_1}[act_type]
+              Q8_1: self.lib.chip_quantize_q8_1, F16: self.lib.chip_convert_f32_to_f16}[act_type]
         self.check(fn(dx.ptr, k, n, k, dy.ptr, None))
         self.sync()
         return dy.download(np.uint8, n * rs).reshape(n, rs)

@@ -17,6 +17,8 @@
 //       d     float [K/256]  at +K
 //       bsums int16 [K/16]   at +K + 4*(K/256)     block_q8_K.bsums
 //
+//   F16 activations (for F16 weights), token stride = f16_stride(K): K halves, nothing else.
+//
 // K is a multiple of 256, so every plane starts 16-byte aligned.
 #pragma once
 #include <stdint.h>
@@ -30,6 +32,8 @@ __host__ __device__ constexpr size_t q8_0_off_d(int64_t K)   { return (size_t)K;
 __host__ __device__ constexpr size_t q8_0_off_sum(int64_t K) { return (size_t)K + 4 * (size_t)(K / 32); }
 __host__ __device__ constexpr size_t q8_0_off_s(int64_t K)   { return (size_t)K + 8 * (size_t)(K / 32); }
 __host__ __device__ constexpr size_t q8_0_stride(int64_t K)  { return align16((size_t)K + 12 * (size_t)(K / 32)); }
+
+__host__ __device__ constexpr size_t f16_stride(int64_t K)   { return align16(2 * (size_t)K); }
 
 __host__ __device__ constexpr size_t q8_K_off_d(int64_t K)     { return (size_t)K; }
 __host__ __device__ constexpr size_t q8_K_off_bsums(int64_t K) { return (size_t)K + 4 * (size_t)(K / 256); }

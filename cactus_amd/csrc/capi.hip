@@ -51,7 +51,7 @@ int current_limits(DeviceLimits &out) {
 
 bool is_weight_type(int t) {
     return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K || t == T_Q5_0 || t == T_Q5_K || t == T_IQ4_NL ||
-           t == T_Q4_1 || t == T_Q5_1;
+           t == T_Q4_1 || t == T_Q5_1 || t == T_F16;
 }
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -64,7 +64,10 @@ bool weights_aligned(int type, const void *W, size_t nb01) {
 }
 
 // Q8_1 activations live in the Q8_0 workspace planes (which carry block_q8_1.s as well)
-size_t act_stride(int act_type, int64_t K) { return (act_type == T_Q8_0 || act_type == T_Q8_1) ? q8_0_stride(K) : q8_K_stride(K); }
+size_t act_stride(int act_type, int64_t K) {
+    if (act_type == T_F16) return f16_stride(K);
+    return (act_type == T_Q8_0 || act_type == T_Q8_1) ? q8_0_stride(K) : q8_K_stride(K);
+}
 
 }  // namespace
 
@@ -167,7 +170,7 @@ int chip_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((
 
 int chip_block_elems(int type) {
     switch (type) {
-        case T_F32: return 1;
+        case T_F32: case T_F16: return 1;
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: case T_Q8_1: return 32;
         case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: return 256;
         default: return 0;
@@ -176,6 +179,7 @@ int chip_block_elems(int type) {
 size_t chip_block_bytes(int type) {
     switch (type) {
         case T_F32: return 4;
+        case T_F16: return 2;
         case T_Q4_0: return BYTES_Q4_0;
         case T_Q8_0: return BYTES_Q8_0;
         case T_Q4_K: return BYTES_Q4_K;
@@ -199,6 +203,7 @@ int chip_vec_dot_type(int type) {
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return T_Q8_0;
         case T_Q4_K: case T_Q6_K: case T_Q5_K: return T_Q8_K;
         case T_Q4_1: case T_Q5_1: return T_Q8_1;
+        case T_F16: return T_F16;
         default: return -1;
     }
 }
@@ -222,6 +227,10 @@ int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t k, void *
 }
 int chip_quantize_q8_1(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
     return quantize_public(T_Q8_1, x, ldx, n, k, y, stream);
+}
+int chip_convert_f32_to_f16(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
+    if (k % 4 != 0) return CHIP_EUNSUPPORTED;
+    return quantize_public(T_F16, x, ldx, n, k, y, stream);
 }
 
 size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n) {
@@ -313,7 +322,7 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                      int32_t *isum, int32_t *imin, void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;
-    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (!chip_mul_mat_supported(type, K) || type == T_F16) return CHIP_EUNSUPPORTED;   // F16 has no integer sums
     if (N == 0 || n == 0) return CHIP_OK;
     if (!W || !aq || !isum) return CHIP_EINVAL;
     if (!weights_aligned(type, W, nb01) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;

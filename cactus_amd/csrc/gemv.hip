@@ -475,6 +475,52 @@ template <> struct Traits<T_IQ4_NL> {
     __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float s) { Traits<T_Q8_0>::img_block_aux(img, NI, blk, d, sum, s); }
 };
 
+// F16 weights (type_traits_cpu[LM_GGML_TYPE_F16], ggml-cpu/ggml-cpu.c:204-209): the activations are rounded to fp16
+// (lm_ggml_cpu_fp32_to_fp16) and lm_ggml_vec_dot_f16 (ggml-cpu/vec.cpp:122-162) accumulates the products of the
+// widened halves in fp32.  A unit is 32 elements = 64 weight bytes and 64 activation bytes; no side data.
+template <> struct Traits<T_F16> {
+    static constexpr int ACT = T_F16, UNIT_ELEMS = 32, QCH = 4, AUX = 0;
+    struct Raw { u32x4 q[4]; };
+    using W = Raw;
+    struct A { uint32_t q[16]; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(row + (size_t)u * 64);  // rows are multiples of 512 bytes
+#pragma unroll
+        for (int j = 0; j < 4; j++) r.q[j] = WLOAD(p + j);
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) { w = r; }
+    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int, int it, int lane) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < QCH; j++) {
+            const u32x4 v = q[j * 64];
+            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t wq[4] = {w.q[j].x, w.q[j].y, w.q[j].z, w.q[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const half2_t wv = __builtin_bit_cast(half2_t, wq[i]), av = __builtin_bit_cast(half2_t, a.q[4 * j + i]);
+                acc = __builtin_fmaf((float)wv.x, (float)av.x, acc);      // v_fma_mix_f32: fp16 operands, fp32 accumulate
+                acc = __builtin_fmaf((float)wv.y, (float)av.y, acc);
+            }
+        }
+        return acc;
+    }
+    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
+    using AuxT = uint32_t;                                       // unused (AUX == 0)
+    __device__ static __forceinline__ AuxT aux_load(const uint8_t *, int64_t, int, bool) { return 0u; }
+    // fused prologue: byte position of element e (an fp16) in the LDS image
+    __device__ static __forceinline__ size_t img_h(int, int e) {
+        const int u = e >> 5, off = (e & 31) * 2;
+        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
+    }
+};
+
 // Q4_1 / Q5_1 (ggml-common.h:175-185,196-207): value = d * u + m with an unsigned 4- or 5-bit u.  Their activation
 // format Q8_1 is Q8_0 plus s = fp16(d * sum q) per block (kept in the Q8_0 workspace planes), so
 // y += (dw * dx) * sum(u * q) + m * s (reference lm_ggml_vec_dot_q4_1_q8_1 / _q5_1_q8_1, AVX2 branches).
@@ -651,7 +697,7 @@ template <int WT, int NTOK, int WGS>
 __device__ __forceinline__ void xload(XRegs<NTOK, WGS> &xr, const float *__restrict__ x, int64_t ldx, int64_t K) {
     using T = Traits<WT>;
     constexpr int PER = XRegs<NTOK, WGS>::PER;
-    if constexpr (T::ACT == T_Q8_0) {
+    if constexpr (T::ACT == T_Q8_0 || T::ACT == T_F16) {
         const int nchunk = (int)(K / 4);                                // float4 chunks per token
 #pragma unroll
         for (int t = 0; t < NTOK; t++)
@@ -681,7 +727,26 @@ __device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, 
     using T = Traits<WT>;
     constexpr int PER = XRegs<NTOK, WGS>::PER;
     const bool dump = blockIdx.x == 0 && ws != nullptr;
-    if constexpr (T::ACT == T_Q8_0) {
+    if constexpr (T::ACT == T_F16) {
+        // plain conversion: four floats -> four halves (round to nearest even), 8 bytes into the image
+        const int nchunk = (int)(K / 4);
+#pragma unroll
+        for (int t = 0; t < NTOK; t++) {
+            uint8_t *im = lds + t * img;
+#pragma unroll
+            for (int j = 0; j < PER; j++) {
+                const int c = j * WGS + (int)threadIdx.x;
+                if (c < nchunk) {
+                    const float4 v = xr.v[t][j];
+                    u32x2 h;
+                    h.x = (uint32_t)f2h_rne(v.x) | ((uint32_t)f2h_rne(v.y) << 16);
+                    h.y = (uint32_t)f2h_rne(v.z) | ((uint32_t)f2h_rne(v.w) << 16);
+                    *reinterpret_cast<u32x2 *>(im + T::img_h(NI, 4 * c)) = h;
+                    if (dump) *reinterpret_cast<u32x2 *>(ws + t * ws_stride + 8 * (size_t)c) = h;
+                }
+            }
+        }
+    } else if constexpr (T::ACT == T_Q8_0) {
         // 8 lanes per 32-block; K % 256 == 0 keeps every 64-lane group either fully inside or fully outside.
         // Slots are quantized FUSE_ILP at a time so their dependent chains (DPP max, two divisions, DPP sum) overlap.
         const int nchunk = (int)(K / 4);
@@ -784,7 +849,7 @@ __device__ __forceinline__ void stage_issue(StageRegs<WT, NTOK> &sr, int NI, int
     }
     const int u = (int)threadIdx.x;
 #pragma unroll
-    for (int t = 0; t < NTOK; t++) sr.a[t] = T::aux_load(ws + t * ws_stride, K, u, u < units);
+    for (int t = 0; t < NTOK; t++) sr.a[t] = T::aux_load(ws + t * ws_stride, K, u, u < units);   // no-op when AUX == 0
 }
 
 template <int WT, int NTOK, int WGS>
@@ -803,9 +868,11 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
             for (int t = 0; t < NTOK; t++) reinterpret_cast<u32x4 *>(lds + t * img)[r] = sr.v[t][j];
         }
     }
-    if ((int)threadIdx.x < na) {
+    if constexpr (T::AUX > 0) {
+        if ((int)threadIdx.x < na) {
 #pragma unroll
-        for (int t = 0; t < NTOK; t++) *reinterpret_cast<AuxT *>(lds + t * img + aux0 + (size_t)threadIdx.x * T::AUX) = sr.a[t];
+            for (int t = 0; t < NTOK; t++) *reinterpret_cast<AuxT *>(lds + t * img + aux0 + (size_t)threadIdx.x * T::AUX) = sr.a[t];
+        }
     }
     // rows longer than the register slots
     for (int r = PQ * WGS + (int)threadIdx.x; r < nq; r += WGS) {
@@ -819,10 +886,12 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
             reinterpret_cast<u32x4 *>(lds + t * img)[r] = v;
         }
     }
-    for (int u = WGS + (int)threadIdx.x; u < na; u += WGS) {
+    if constexpr (T::AUX > 0) {
+        for (int u = WGS + (int)threadIdx.x; u < na; u += WGS) {
 #pragma unroll
-        for (int t = 0; t < NTOK; t++)
-            *reinterpret_cast<AuxT *>(lds + t * img + aux0 + (size_t)u * T::AUX) = T::aux_load(ws + t * ws_stride, K, u, u < units);
+            for (int t = 0; t < NTOK; t++)
+                *reinterpret_cast<AuxT *>(lds + t * img + aux0 + (size_t)u * T::AUX) = T::aux_load(ws + t * ws_stride, K, u, u < units);
+        }
     }
 }
 
@@ -1024,6 +1093,7 @@ int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
         case T_IQ4_NL: return max_tokens_typed<T_IQ4_NL>(K, lim);
         case T_Q4_1: return max_tokens_typed<T_Q4_1>(K, lim);
         case T_Q5_1: return max_tokens_typed<T_Q5_1>(K, lim);
+        case T_F16: return max_tokens_typed<T_F16>(K, lim);
         default: return 0;
     }
 }
@@ -1042,6 +1112,7 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q4_1: return launch_ntok<T_Q4_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q5_1: return launch_ntok<T_Q5_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_F16: return launch_ntok<T_F16, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1061,6 +1132,7 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
         case T_IQ4_NL: img = lds_image_bytes<T_IQ4_NL>(K); break;
         case T_Q4_1: img = lds_image_bytes<T_Q4_1>(K); break;
         case T_Q5_1: img = lds_image_bytes<T_Q5_1>(K); break;
+        case T_F16: img = lds_image_bytes<T_F16>(K); break;
         default: return false;
     }
     return (size_t)n * img <= (size_t)lim.max_lds_per_block;
@@ -1079,6 +1151,7 @@ hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, i
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         case T_Q4_1: return launch_ntok<T_Q4_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         case T_Q5_1: return launch_ntok<T_Q5_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_F16: return launch_ntok<T_F16, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }

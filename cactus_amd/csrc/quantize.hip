@@ -69,6 +69,20 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float *__restr
     }
 }
 
+// fp32 -> fp16 rows, round to nearest even (reference lm_ggml_cpu_fp32_to_fp16, ggml-cpu/ggml-cpu.c:3161-3190): the
+// activation format of F16 weights.  The workspace layout and the reference layout are the same K halves.
+__global__ __launch_bounds__(256) void convert_f16_kernel(const float *__restrict__ x, int64_t ldx, int64_t K,
+                                                        uint8_t *__restrict__ y, size_t y_stride) {
+    const int64_t t = blockIdx.y;
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e0 >= K) return;
+    const float4 v = *reinterpret_cast<const float4 *>(x + t * ldx + e0);
+    u32x2 h;
+    h.x = (uint32_t)f2h_rne(v.x) | ((uint32_t)f2h_rne(v.y) << 16);
+    h.y = (uint32_t)f2h_rne(v.z) | ((uint32_t)f2h_rne(v.w) << 16);
+    *reinterpret_cast<u32x2 *>(y + t * y_stride + 2 * e0) = h;
+}
+
 // Inverse of the split layout: rebuild reference blocks from workspace planes (verification only).
 __global__ void split_to_blocks_q8_0_kernel(const uint8_t *__restrict__ ws, size_t ws_stride, int64_t K,
                                             uint8_t *__restrict__ y, size_t y_stride) {
@@ -108,7 +122,9 @@ hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx
                            size_t y_stride, hipStream_t st) {
     if (n <= 0 || K <= 0) return hipSuccess;
     dim3 grid((unsigned)ceil_div(K, 1024), (unsigned)n);
-    if (act_type == T_Q8_0 || act_type == T_Q8_1) {
+    if (act_type == T_F16) {
+        hipLaunchKernelGGL(convert_f16_kernel, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
+    } else if (act_type == T_Q8_0 || act_type == T_Q8_1) {
         // Q8_1 shares the Q8_0 workspace planes (which carry its s); only the block records differ
         if (split)                  hipLaunchKernelGGL(quantize_q8_0_kernel<0>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
         else if (act_type == T_Q8_0) hipLaunchKernelGGL(quantize_q8_0_kernel<1>, grid, dim3(256), 0, st, x, ldx, K, (uint8_t *)y, y_stride);
@@ -123,6 +139,8 @@ hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx
 hipError_t launch_split_to_blocks(int act_type, const void *ws, size_t ws_stride, int64_t n, int64_t K, void *y,
                                   size_t y_stride, hipStream_t st) {
     if (n <= 0 || K <= 0) return hipSuccess;
+    if (act_type == T_F16)
+        return hipMemcpy2DAsync(y, y_stride, ws, ws_stride, 2 * (size_t)K, (size_t)n, hipMemcpyDeviceToDevice, st);
     if (act_type == T_Q8_0 || act_type == T_Q8_1) {
         dim3 grid((unsigned)ceil_div(K / 32, 256), (unsigned)n);
         if (act_type == T_Q8_0)

@@ -26,6 +26,7 @@ extern "C" {
 /* weight / activation type ids: the reference's lm_ggml_type values (ggml.h:351-391) */
 enum chip_type {
     CHIP_TYPE_F32  = 0,
+    CHIP_TYPE_F16  = 1,      /* weight type and its own activation format (ggml-cpu/ggml-cpu.c:204-209) */
     CHIP_TYPE_Q4_0 = 2,
     CHIP_TYPE_Q8_0 = 8,
     CHIP_TYPE_Q4_K = 12,
@@ -82,7 +83,7 @@ CHIP_API int    chip_block_elems(int type);
 CHIP_API size_t chip_block_bytes(int type);
 CHIP_API size_t chip_row_size(int type, int64_t k);
 /* type_traits_cpu[type].vec_dot_type (ggml-cpu/ggml-cpu.c:198-367): Q8_0 for Q4_0/Q8_0/Q5_0/IQ4_NL, Q8_K for
- * Q4_K/Q5_K/Q6_K, Q8_1 for Q4_1/Q5_1 */
+ * Q4_K/Q5_K/Q6_K, Q8_1 for Q4_1/Q5_1, F16 for F16 */
 CHIP_API int    chip_vec_dot_type(int type);
 /* 1 if chip_mul_mat accepts this weight type and K (K must be a multiple of 256) */
 CHIP_API int    chip_mul_mat_supported(int type, int64_t K);
@@ -99,6 +100,9 @@ CHIP_API int chip_quantize_q8_K(const float *x, int64_t ldx, int64_t n, int64_t 
 /* quantize_row_q8_1, AVX2 branch (ggml-cpu/ggml-cpu-quants.c:1047-1140): the activation format of Q4_1 / Q5_1;
  * quants and d as Q8_0, plus s = fp16(d * sum of quants) */
 CHIP_API int chip_quantize_q8_1(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
+/* lm_ggml_cpu_fp32_to_fp16 (ggml-cpu/ggml-cpu.c:3161-3190): fp32 rows -> fp16 rows, round to nearest even; the
+ * activation format of F16 weights (k a multiple of 4) */
+CHIP_API int chip_convert_f32_to_f16(const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream);
 
 /* ---- the op: LM_GGML_OP_MUL_MAT over block-quantized weights ----
  * lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449) with src0 = W (type, [K, N], row stride

@@ -18,18 +18,20 @@ REF_SO = os.path.join(HERE, "_ref", "libggml_ref.so")
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
+F16 = 1
 TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
-              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1"}
+              Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16"}
 BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32,
-               Q4_1: 32, Q5_1: 32, Q8_1: 32}
+               Q4_1: 32, Q5_1: 32, Q8_1: 32, F16: 1}
 BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18,
-               Q4_1: 20, Q5_1: 24, Q8_1: 36}
+               Q4_1: 20, Q5_1: 24, Q8_1: 36, F16: 2}
 VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0,
-                Q4_1: Q8_1, Q5_1: Q8_1}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1)
+                Q4_1: Q8_1, Q5_1: Q8_1, F16: F16}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, F16)
+BLOCK_WEIGHT_TYPES = WEIGHT_TYPES[:-1]        # the types with per-block integer sums
 # types whose weight quantizer is restated in the oracle (IQ4_NL weights come from the reference build, from the
 # golden fixture, or are random bytes: any byte string is a valid block)
-ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, Q4_1, Q5_1)
+ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, Q4_1, Q5_1, F16)
 
 
 IQ4_NL_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
@@ -106,6 +108,10 @@ class Oracle:
             f = getattr(L, "orc_quantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
+        L.orc_fp32_to_fp16_row.restype = None
+        L.orc_fp32_to_fp16_row.argtypes = [_vp, _vp, _i64]
+        L.orc_vec_dot_f16.restype = C.c_float
+        L.orc_vec_dot_f16.argtypes = [_i64, _vp, _vp]
         L.orc_quantize_rows.restype = C.c_size_t
         L.orc_quantize_rows.argtypes = [_i32, _vp, _vp, _i64, _i64]
         L.orc_dequantize_row.restype = None
@@ -138,7 +144,7 @@ class Oracle:
         rows = x.reshape(-1, k)
         out = np.zeros((rows.shape[0], row_size(act_type, k)), np.uint8)
         fn = {Q8_0: self.lib.orc_quantize_row_q8_0, Q8_K: self.lib.orc_quantize_row_q8_K,
-              Q8_1: self.lib.orc_quantize_row_q8_1}[act_type]
+              Q8_1: self.lib.orc_quantize_row_q8_1, F16: self.lib.orc_fp32_to_fp16_row}[act_type]
         for r in range(rows.shape[0]):
             fn(_ptr(rows[r]), _ptr(out[r]), k)
         return out.reshape(x.shape[:-1] + (out.shape[1],))
@@ -191,6 +197,8 @@ class Oracle:
             v = self.lib.orc_vec_dot_iq4_nl_q8_0(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q5_K:
             v = self.lib.orc_vec_dot_q5_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
+        elif wtype == F16:
+            v = self.lib.orc_vec_dot_f16(k, _ptr(wrow), _ptr(arow))
         elif wtype == Q4_1:
             v = self.lib.orc_vec_dot_q4_1_q8_1(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q5_1:
@@ -254,7 +262,8 @@ class Reference:
         for n in ("quantize_row_q8_0", "quantize_row_q8_K", "quantize_row_q4_0_ref", "quantize_row_q8_0_ref",
                   "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref",
                   "quantize_row_q5_0_ref", "quantize_row_q5_K_ref", "quantize_row_iq4_nl_ref",
-                  "quantize_row_q4_1_ref", "quantize_row_q5_1_ref", "quantize_row_q8_1"):
+                  "quantize_row_q4_1_ref", "quantize_row_q5_1_ref", "quantize_row_q8_1",
+                  "lm_ggml_fp32_to_fp16_row", "lm_ggml_cpu_fp32_to_fp16", "lm_ggml_fp16_to_fp32_row"):
             f = getattr(L, n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
@@ -263,7 +272,7 @@ class Reference:
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
         for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "q5_0_q8_0", "q5_K_q8_K", "iq4_nl_q8_0",
-                  "q4_1_q8_1", "q5_1_q8_1"):
+                  "q4_1_q8_1", "q5_1_q8_1", "f16"):
             f = getattr(L, "lm_ggml_vec_dot_" + n)
             f.restype = None
             f.argtypes = [C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, _vp, C.c_size_t, C.c_int]
@@ -296,15 +305,16 @@ class Reference:
         L.lm_ggml_threadpool_free.argtypes = [_vp]
         L.lm_ggml_threadpool_params_init.argtypes = [_vp, _i32]
 
-    _ACT = {Q8_0: "quantize_row_q8_0", Q8_K: "quantize_row_q8_K", Q8_1: "quantize_row_q8_1"}
+    _ACT = {Q8_0: "quantize_row_q8_0", Q8_K: "quantize_row_q8_K", Q8_1: "quantize_row_q8_1",
+            F16: "lm_ggml_cpu_fp32_to_fp16"}
     _WQ = {Q4_0: "quantize_row_q4_0_ref", Q8_0: "quantize_row_q8_0_ref",
            Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref",
            Q5_0: "quantize_row_q5_0_ref", Q5_K: "quantize_row_q5_K_ref", IQ4_NL: "quantize_row_iq4_nl_ref",
-           Q4_1: "quantize_row_q4_1_ref", Q5_1: "quantize_row_q5_1_ref"}
+           Q4_1: "quantize_row_q4_1_ref", Q5_1: "quantize_row_q5_1_ref", F16: "lm_ggml_fp32_to_fp16_row"}
     _DOT = {Q4_0: "lm_ggml_vec_dot_q4_0_q8_0", Q8_0: "lm_ggml_vec_dot_q8_0_q8_0",
             Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K",
             Q5_0: "lm_ggml_vec_dot_q5_0_q8_0", Q5_K: "lm_ggml_vec_dot_q5_K_q8_K", IQ4_NL: "lm_ggml_vec_dot_iq4_nl_q8_0",
-            Q4_1: "lm_ggml_vec_dot_q4_1_q8_1", Q5_1: "lm_ggml_vec_dot_q5_1_q8_1"}
+            Q4_1: "lm_ggml_vec_dot_q4_1_q8_1", Q5_1: "lm_ggml_vec_dot_q5_1_q8_1", F16: "lm_ggml_vec_dot_f16"}
 
     def quantize_activation(self, act_type, x):
         x = _f32(x)
@@ -336,7 +346,7 @@ class Reference:
         q = np.ascontiguousarray(q, np.uint8)
         rows = q.reshape(-1, row_size(t, k))
         out = np.zeros((rows.shape[0], k), np.float32)
-        fn = getattr(self.lib, "dequantize_row_" + TYPE_NAMES[t])
+        fn = getattr(self.lib, "lm_ggml_fp16_to_fp32_row" if t == F16 else "dequantize_row_" + TYPE_NAMES[t])
         for r in range(rows.shape[0]):
             fn(_ptr(rows[r]), _ptr(out[r]), k)
         return out.reshape(q.shape[:-1] + (k,))

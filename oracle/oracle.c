@@ -47,7 +47,7 @@ static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10
 
 int orc_block_elems(int type) {
     switch (type) {
-        case ORC_TYPE_F32: return 1;
+        case ORC_TYPE_F32: case ORC_TYPE_F16: return 1;
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL:
         case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: case ORC_TYPE_Q8_1: return 32;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
@@ -57,6 +57,7 @@ int orc_block_elems(int type) {
 size_t orc_block_bytes(int type) {
     switch (type) {
         case ORC_TYPE_F32: return 4;
+        case ORC_TYPE_F16: return 2;
         case ORC_TYPE_Q4_0: return 18;
         case ORC_TYPE_Q8_0: return 34;
         case ORC_TYPE_Q4_K: return 144;
@@ -80,6 +81,7 @@ int orc_vec_dot_type(int type) {
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return ORC_TYPE_Q8_0;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
         case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: return ORC_TYPE_Q8_1;   /* ggml-cpu/ggml-cpu.c:221,237 */
+        case ORC_TYPE_F16: return ORC_TYPE_F16;                        /* ggml-cpu/ggml-cpu.c:204-209 */
         default: return -1;
     }
 }
@@ -178,6 +180,14 @@ void orc_quantize_row_q8_1(const float *x, void *vy, int64_t k) {
         }
         y[b].s = F2H(d * (float)(int32_t)sum);
     }
+}
+
+/* F16 weights: activations are converted to fp16, round to nearest even (lm_ggml_cpu_fp32_to_fp16,
+ * ggml-cpu/ggml-cpu.c:3161-3190: F16C _mm256_cvtps_ph / _mm_cvtps_ph with _MM_FROUND_TO_NEAREST_INT); weights made
+ * from fp32 the same way (lm_ggml_fp32_to_fp16_row, ggml.c:417-422). */
+void orc_fp32_to_fp16_row(const float *x, void *vy, int64_t k) {
+    uint16_t *y = (uint16_t *)vy;
+    for (int64_t i = 0; i < k; i++) y[i] = F2H(x[i]);
 }
 
 /* ggml-quants.c:188-211 (scalar reference, used for Q8_0 *weights*). */
@@ -583,6 +593,7 @@ size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64
             case ORC_TYPE_Q5_0: orc_quantize_row_q5_0_ref(src, dst, k); break;
             case ORC_TYPE_Q4_1: orc_quantize_row_q4_1_ref(src, dst, k); break;
             case ORC_TYPE_Q5_1: orc_quantize_row_q5_1_ref(src, dst, k); break;
+            case ORC_TYPE_F16: orc_fp32_to_fp16_row(src, dst, k); break;
             default: return 0;
         }
     }
@@ -676,6 +687,9 @@ void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
                 u1 = (uint8_t)(u1 << 2); u2 = (uint8_t)(u2 << 2);
             }
         }
+    } else if (type == ORC_TYPE_F16) {
+        const uint16_t *x = (const uint16_t *)vx;
+        for (int64_t i = 0; i < k; i++) y[i] = H2F(x[i]);
     } else if (type == ORC_TYPE_Q4_1) {                 /* ggml-quants.c:269-288 */
         const blk_q4_1 *x = (const blk_q4_1 *)vx;
         for (int64_t b = 0; b < k / 32; b++, y += 32) {
@@ -948,6 +962,27 @@ float orc_vec_dot_iq4_nl_q8_0(int64_t k, const void *vx, const void *vy, int32_t
     return sumf;
 }
 
+/* F16 x F16: lm_ggml_vec_dot_f16 (ggml-cpu/vec.cpp:122-162) with the AVX2 mapping of ggml-cpu/simd-mappings.h
+ * (LM_GGML_F16_STEP 32, four 8-lane fp32 accumulators, fmadd of the widened halves; reduction :251-269:
+ * acc0 += acc2, acc1 += acc3, acc0 += acc1, low half + high half, two horizontal adds).  Elements past the last
+ * multiple of 32 are added in double precision (:152-154). */
+float orc_vec_dot_f16(int64_t k, const void *vx, const void *vy) {
+    const uint16_t *x = (const uint16_t *)vx, *y = (const uint16_t *)vy;
+    float acc[4][8] = {{0}};
+    const int64_t np = k & ~(int64_t)31;
+    for (int64_t i = 0; i < np; i += 32)
+        for (int j = 0; j < 4; j++)
+            for (int l = 0; l < 8; l++) acc[j][l] = fmaf(H2F(x[i + 8 * j + l]), H2F(y[i + 8 * j + l]), acc[j][l]);
+    float t[4];
+    for (int l = 0; l < 8; l++) { acc[0][l] = acc[0][l] + acc[2][l]; acc[1][l] = acc[1][l] + acc[3][l]; }
+    for (int l = 0; l < 8; l++) acc[0][l] = acc[0][l] + acc[1][l];
+    for (int l = 0; l < 4; l++) t[l] = acc[0][l] + acc[0][l + 4];
+    const float h0 = t[0] + t[1], h1 = t[2] + t[3];
+    double sumf = (double)(h0 + h1);
+    for (int64_t i = np; i < k; i++) sumf += (double)(H2F(x[i]) * H2F(y[i]));
+    return (float)sumf;
+}
+
 /* q4_1 / q5_1 x q8_1: AVX2 branches of lm_ggml_vec_dot_q4_1_q8_1 and lm_ggml_vec_dot_q5_1_q8_1
  * (ggml-cpu/ggml-cpu-quants.c): unsigned weights u (nibble, or nibble | bit << 4), lane j takes the four
  * products of elements 4j..4j+3, acc = fmadd(dx*dy, float(p), acc); the min term is the scalar
@@ -1045,6 +1080,7 @@ float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
         case ORC_TYPE_Q5_K: return orc_vec_dot_q5_K_q8_K(k, vx, vy, NULL, NULL);
         case ORC_TYPE_Q4_1: return orc_vec_dot_q4_1_q8_1(k, vx, vy, NULL);
         case ORC_TYPE_Q5_1: return orc_vec_dot_q5_1_q8_1(k, vx, vy, NULL);
+        case ORC_TYPE_F16: return orc_vec_dot_f16(k, vx, vy);
         default: return NAN;
     }
 }
@@ -1071,6 +1107,12 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
         for (int64_t b = 0; b < nb; b++) {
             const uint16_t hx = type == ORC_TYPE_Q5_0 ? ((const blk_q5_0 *)vx)[b].d : ((const blk_iq4_nl *)vx)[b].d;
             const double t = (double)H2F(hx) * (double)H2F(y[b].d) * (double)is[b];
+            s += t; sa += fabs(t);
+        }
+    } else if (type == ORC_TYPE_F16) {
+        const uint16_t *x = (const uint16_t *)vx, *y = (const uint16_t *)vy;
+        for (int64_t i = 0; i < k; i++) {
+            const double t = (double)H2F(x[i]) * (double)H2F(y[i]);
             s += t; sa += fabs(t);
         }
     } else if (type == ORC_TYPE_Q4_1 || type == ORC_TYPE_Q5_1) {
@@ -1178,6 +1220,7 @@ void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const
     for (int64_t t = 0; t < n; t++) {
         if (vdt == ORC_TYPE_Q8_0)      orc_quantize_row_q8_0(x + t * K, wd + (size_t)t * ars, K);
         else if (vdt == ORC_TYPE_Q8_1) orc_quantize_row_q8_1(x + t * K, wd + (size_t)t * ars, K);
+        else if (vdt == ORC_TYPE_F16)  orc_fp32_to_fp16_row(x + t * K, wd + (size_t)t * ars, K);
         else                           orc_quantize_row_q8_K(x + t * K, wd + (size_t)t * ars, K);
     }
     if (nthreads < 1) nthreads = 1;

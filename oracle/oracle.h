@@ -28,6 +28,8 @@
  *   orc_vec_dot_*                    integer sums: brute force from dequantised integers; float result: bit-exact
  *                                    vs oracle/_ref (the AVX2 lane structure is restated) + golden; fp64 identity
  *                                    sum(dequant(x)*dequant(y))
+ *   orc_fp32_to_fp16_row, orc_vec_dot_f16  conversion: the exhaustive fp16 checks above; dot: bit-exact vs oracle/_ref
+ *                                    (lane structure restated) + golden; fp64 identity sum w_i * x_i
  *   orc_mul_mat                      == n*N independent vec_dots; vs oracle/_ref's LM_GGML_OP_MUL_MAT graph
  *
  * No function here is "parity unpinned".
@@ -45,6 +47,7 @@ extern "C" {
 /* type ids are the reference's lm_ggml_type values (ggml.h:351-391) */
 enum orc_type {
     ORC_TYPE_F32  = 0,
+    ORC_TYPE_F16  = 1,      /* as a weight type and as its own activation format */
     ORC_TYPE_Q4_0 = 2,
     ORC_TYPE_Q8_0 = 8,
     ORC_TYPE_Q4_K = 12,
@@ -73,6 +76,7 @@ uint16_t orc_fp32_to_fp16(float f);
 void orc_quantize_row_q8_0(const float *x, void *y, int64_t k);      /* AVX2 semantics */
 void orc_quantize_row_q8_K(const float *x, void *y, int64_t k);
 void orc_quantize_row_q8_1(const float *x, void *y, int64_t k);      /* AVX2 semantics */
+void orc_fp32_to_fp16_row(const float *x, void *y, int64_t k);       /* fp16 round to nearest even */
 
 /* weight quantizers (offline; their output bytes are the op's input) */
 void orc_quantize_row_q4_0_ref(const float *x, void *y, int64_t k);
@@ -107,6 +111,7 @@ float orc_vec_dot_q5_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *
 /* q4_1, q5_1: isum[k/32] = sum u*aq with the unsigned weight u; the min term m*s is not part of isum */
 float orc_vec_dot_q4_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot_q5_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *isum);
+float orc_vec_dot_f16(int64_t k, const void *vx, const void *vy);   /* both operands fp16, fp32 fmadd lanes */
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
 
 /* fp64 evaluation of sum_b scale_b*isum_b (returned) and of sum_b |scale_b*isum_b| (*sum_abs): the tolerance
@@ -114,7 +119,7 @@ float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
  * carries its own scale: 32 values for Q4_0/Q8_0, a 32-value sub-block for Q4_K (terms d*sc_j*dot_j and
  * dmin*m_j*bsum_j, both counted), a 16-value sub-block for Q6_K (d*sc_j*dot_j); Q5_0 and
  * IQ4_NL as Q4_0, Q5_K as Q4_K;
- * Q4_1 / Q5_1: d*dy*isum and m*s per 32-block, both counted.  Coarser terms (whole
+ * Q4_1 / Q5_1: d*dy*isum and m*s per 32-block, both counted; F16: every product w_i * x_i.  Coarser terms (whole
  * super-blocks) would cancel internally and make a bound that the reference's own AVX2 result misses. */
 double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, double *sum_abs);
 

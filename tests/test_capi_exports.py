@@ -36,6 +36,7 @@ def test_layout_queries_need_no_gpu():
     assert lib.chip_vec_dot_type(cactus_amd.Q6_K) == cactus_amd.Q8_K
     assert lib.chip_mul_mat_supported(cactus_amd.Q4_K, 4096) == 1
     assert lib.chip_mul_mat_supported(cactus_amd.Q4_K, 4000) == 0
-    assert lib.chip_mul_mat_supported(1, 4096) == 0           # F16 weights are not on this path
+    assert lib.chip_mul_mat_supported(cactus_amd.F16, 4096) == 1 and lib.chip_vec_dot_type(cactus_amd.F16) == cactus_amd.F16
+    assert lib.chip_mul_mat_supported(30, 4096) == 0          # BF16 weights are not on this path
     assert lib.chip_mul_mat_workspace_size(cactus_amd.Q8_0, 4096, 3) == 3 * (4096 + 12 * 128)   # qs, d, sum, s planes
     assert lib.chip_error_string(-2).decode().startswith("unsupported")

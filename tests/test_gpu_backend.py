@@ -185,7 +185,7 @@ def test_compare_graph_backend_against_reference_cpu(host, orc):
     from ggml_host import EVAL_CB
     K, n = 1024, 5
     specs = [(O.Q4_0, 300), (O.Q8_0, 64), (O.Q4_K, 257), (O.Q6_K, 130), (O.Q5_0, 77), (O.Q5_K, 96), (O.IQ4_NL, 45),
-             (O.Q4_1, 51), (O.Q5_1, 38)]
+             (O.Q4_1, 51), (O.Q5_1, 38), (O.F16, 29)]
     dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
     hip = L.lm_ggml_backend_dev_init(dev, None)
     cpu = L.lm_ggml_backend_cpu_init()

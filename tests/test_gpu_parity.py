@@ -41,7 +41,7 @@ def test_quantizers_bit_exact(dev, orc, K):
     x[2] *= 300
     x[3, : K // 2] = 0
     x[4] = 0
-    for at in (O.Q8_0, O.Q8_K, O.Q8_1):
+    for at in (O.Q8_0, O.Q8_K, O.Q8_1, O.F16):
         print("quantize", O.TYPE_NAMES[at], "K", K, flush=True)
         assert np.array_equal(dev.quantize(at, x), orc.quantize_activation(at, x))
 
@@ -98,7 +98,7 @@ def test_mul_mat_vs_oracle(dev, orc, wt, K, N, n):
     check_outputs(y, ref["y"], ref["sum_abs"], "mul_mat")
 
 
-@pytest.mark.parametrize("wt", O.WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("wt", O.BLOCK_WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_block_integer_sums_bit_exact(dev, orc, wt):
     K, N, n = 2048, 9, 2
     wq = orc.quantize_weights(wt, common.weights_f32(300 + wt, N, K, outliers=True))
@@ -205,7 +205,7 @@ def test_argument_errors(dev):
     ws = dev.alloc(1 << 16)
     # K not a multiple of 256, unknown type
     assert L.chip_mul_mat(O.Q4_0, buf.ptr, 18, 32, 1, buf.ptr, 32, 1, buf.ptr, 1, ws.ptr, 1 << 16, None) == -2
-    assert L.chip_mul_mat(1, buf.ptr, 512, 256, 1, buf.ptr, 256, 1, buf.ptr, 1, ws.ptr, 1 << 16, None) == -2
+    assert L.chip_mul_mat(30, buf.ptr, 512, 256, 1, buf.ptr, 256, 1, buf.ptr, 1, ws.ptr, 1 << 16, None) == -2    # BF16
     # workspace too small, null pointers, misaligned weights, row stride below the row size
     assert L.chip_mul_mat(O.Q4_0, buf.ptr, 144, 256, 1, buf.ptr, 256, 1, buf.ptr, 1, ws.ptr, 16, None) == -3
     assert L.chip_mul_mat(O.Q4_0, None, 144, 256, 1, buf.ptr, 256, 1, buf.ptr, 1, ws.ptr, 1 << 16, None) == -1
