@@ -7,7 +7,8 @@
 //     its K extent is exactly one 32-value quantization block, so each of the 1024 int32 results is one
 //     per-block integer sum isum[t][r][b], bit-exact.
 //   * Weight tiles are staged through LDS once per workgroup and k-stage: the Q4_0 nibbles are split into the
-//     low-nibble half (elements 0..15) and the high-nibble half (16..31) and turned into signed int8 (nib - 8);
+//     low-nibble half (elements 0..15) and the high-nibble half (16..31) and turned into signed int8
+//     16 * (nib - 8), the 16 being undone by the activation scale;
 //     activations arrive as int8 from the split workspace layout.  Both sit in LDS as [k-block][half][row]
 //     16-byte cells, which is exactly what one lane feeds the MFMA (row = lane % 32, half = lane / 32).
 //   * Per-block scales are applied in fp32 after the integer accumulate.  The MFMA's C input is a register
@@ -36,10 +37,12 @@ constexpr int GEMM_KB = 4;                    // 32-value blocks per LDS stage
 constexpr float MAGIC_F = 12582912.f;         // 1.5 * 2^23
 constexpr int MAGIC_I = 0x4B400000;
 
-// nibbles 0..15 in the four bytes of x  ->  signed bytes (nibble - 8)
-__device__ __forceinline__ uint32_t nib_to_i8(uint32_t x) {
-    return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-}
+// The weight operand holds 16 * (nibble - 8): a nibble moved to the high half of its byte with its top bit flipped
+// is that number as a signed byte (two or three operations per dword instead of four); the factor 16 is taken
+// back through the activation scale (dx / 16 is exact), and |16 * isum| <= 16 * 32 * 8 * 127 < 2^22 still fits
+// the magic-constant conversion.
+__device__ __forceinline__ uint32_t lo_nib_x16(uint32_t q) { return ((q << 4) & 0xf0f0f0f0u) ^ 0x80808080u; }
+__device__ __forceinline__ uint32_t hi_nib_x16(uint32_t q) { return (q & 0xf0f0f0f0u) ^ 0x80808080u; }
 
 template <int TM, int TN, int WR, int WC>
 struct GemmCfg {
@@ -131,10 +134,10 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
             if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
                 const int r = item / GEMM_KB, b = item % GEMM_KB;
                 u32x4 lo, hi;
-                lo.x = nib_to_i8(wq[i].x & 0x0f0f0f0fu); hi.x = nib_to_i8((wq[i].x >> 4) & 0x0f0f0f0fu);
-                lo.y = nib_to_i8(wq[i].y & 0x0f0f0f0fu); hi.y = nib_to_i8((wq[i].y >> 4) & 0x0f0f0f0fu);
-                lo.z = nib_to_i8(wq[i].z & 0x0f0f0f0fu); hi.z = nib_to_i8((wq[i].z >> 4) & 0x0f0f0f0fu);
-                lo.w = nib_to_i8(wq[i].w & 0x0f0f0f0fu); hi.w = nib_to_i8((wq[i].w >> 4) & 0x0f0f0f0fu);
+                lo.x = lo_nib_x16(wq[i].x); hi.x = hi_nib_x16(wq[i].x);
+                lo.y = lo_nib_x16(wq[i].y); hi.y = hi_nib_x16(wq[i].y);
+                lo.z = lo_nib_x16(wq[i].z); hi.z = hi_nib_x16(wq[i].z);
+                lo.w = lo_nib_x16(wq[i].w); hi.w = hi_nib_x16(wq[i].w);
                 A[(b * 2 + 0) * C::A_PLANE + r] = lo;
                 A[(b * 2 + 1) * C::A_PLANE + r] = hi;
                 // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4;
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
             const int item = tid + i * C::NT;
             if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
                 const int b = item % GEMM_KB, n = item / GEMM_KB;
-                SX[b * C::BN + n] = xs[i];
+                SX[b * C::BN + n] = xs[i] * 0.0625f;                       // takes back the 16 of the weight operand
             }
         }
     };
@@ -301,17 +304,17 @@ hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, co
     if (M <= 0 || N <= 0) return hipSuccess;
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
     // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
-    // every CU such a group fall back to 64 x 128 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
+    // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_CFG");
-    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
+    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 6);
     switch (cfg) {
         case 0: return launch_cfg<1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         case 1: return launch_cfg<1, 2, 2, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         case 2: return launch_cfg<2, 2, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         case 3: return launch_cfg<2, 2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 4: return launch_cfg<1, 2, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         case 5: return launch_cfg<2, 1, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 6: return launch_cfg<1, 1, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }

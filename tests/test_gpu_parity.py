@@ -276,3 +276,99 @@ def test_config4_prefill_sampled(dev, orc, N, M):
     # the same weights reversed must give the same numbers reversed
     y2 = dev.mul_mat(O.Q4_0, wq[::-1].copy(), x[:64])
     assert np.array_equal(y2[:, ::-1], y[:64])
+
+
+# ------------------------------------------------------------------------------------------ K-quant prefill GEMM
+KQ_TYPES = (O.Q4_K, O.Q5_K, O.Q6_K)
+
+
+@pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N,n", [(256, 1, 16), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257)])
+def test_gemm_kquant_vs_oracle(dev, orc, wt, K, N, n):
+    print("gemm", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
+    wq = orc.quantize_weights(wt, common.weights_f32(K + N + wt, N, K, outliers=True))
+    x = common.activations_f32(K + n + wt, n, K)
+    x[3] = 0
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(wt, wq, x, want_workspace_blocks=True)
+    assert np.array_equal(blocks, ref["wdata"])
+    check_outputs(y, ref["y"], ref["sum_abs"], "k-quant gemm")
+
+
+def random_kquant_rows(wt, rng, N, nsb, extreme_rows=0):
+    """Raw super-blocks with every super-block scale (d, dmin) equal to 1 and random bytes everywhere else, so all
+    6-bit / 8-bit sub-block scales and quants occur; the first `extreme_rows` rows use saturating bytes."""
+    one = np.array([1.0], np.float16).view(np.uint8)
+    bb = O.BLOCK_BYTES[wt]
+    w = rng.integers(0, 256, (N, nsb, bb), dtype=np.uint8)
+    fills = (0xFF, 0x00, 0x80, 0x7F)
+    for r in range(extreme_rows):
+        w[r] = fills[r % 4]
+    if wt == O.Q6_K:
+        w[..., 208:210] = one
+    else:
+        w[..., 0:2] = one
+        w[..., 2:4] = one
+    return w.reshape(N, -1)
+
+
+def exact_q8_K_inputs(rng, n, K):
+    """Integer activations whose first largest-magnitude value per super-block is -127: Q8_K then has
+    iscale = -127 / max = 1, so d = 1 and q = x."""
+    x = rng.integers(-127, 128, (n, K)).astype(np.float32)
+    x[:, ::256] = -127.0
+    return x
+
+
+@pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+def test_gemm_kquant_integer_sums_bit_exact(dev, orc, wt):
+    """With d = dmin = 1 and activation scale 1 the fp32 output of a one-super-block product is sumi - summ itself
+    (below 2^24), so the digit planes folded into the MFMA operand are compared bit for bit with the reference's
+    integer sums, over random scale and quant bytes."""
+    K, N, n = 256, 150, 48
+    rng = np.random.default_rng(77 + wt)
+    w = random_kquant_rows(wt, rng, N, 1)
+    x = exact_q8_K_inputs(rng, n, K)
+    x[7, 1:] = 0.0
+    aq = orc.quantize_activation(O.Q8_K, x)
+    assert np.array_equal(aq[:, 4:4 + K].view(np.int8).astype(np.float32), x) and (aq[:, :4].view(np.float32) == 1).all()
+    y = dev.mul_mat(wt, w, x)
+    want = np.zeros((n, N), np.int64)
+    for t in range(n):
+        for i in range(N):
+            _, isum, imin = orc.vec_dot(wt, K, w[i], aq[t], want_sums=True)
+            want[t, i] = int(isum.sum()) - int(imin.sum())
+    assert np.abs(want).max() < 2 ** 24
+    assert np.array_equal(y.astype(np.int64), want)
+
+
+@pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+def test_gemm_kquant_extreme_bytes(dev, orc, wt):
+    # saturating scale / quant bytes in the first rows, activations pinned at +-127: the operand digits at their limits
+    K, N, n = 1024, 64, 32
+    rng = np.random.default_rng(5 + wt)
+    w = random_kquant_rows(wt, rng, N, K // 256, extreme_rows=8)
+    x = exact_q8_K_inputs(rng, n, K)
+    x[0, :] = 127.0
+    x[1, :] = -127.0
+    x[0:2, ::256] = -127.0
+    ref = orc.mul_mat(wt, w, x, nthreads=8, want=("sum_abs",))
+    check_outputs(dev.mul_mat(wt, w, x), ref["y"], ref["sum_abs"], "extreme bytes")
+
+
+@pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+def test_gemm_kquant_prefill_shape_sampled(dev, orc, wt):
+    """A full prefill shape on the GPU, the oracle on a sample of rows and tokens, and row-order independence."""
+    K, N, M = 4096, 4096, 512
+    rng = np.random.default_rng(wt)
+    wq = orc.quantize_weights(wt, common.weights_f32(40 + wt, N, K))
+    x = common.activations_f32(40 + wt, M, K)
+    y = dev.mul_mat(wt, wq, x)
+    rows = np.sort(rng.choice(N, 64, replace=False))
+    rows[:2] = [0, 1]; rows[-1] = N - 1
+    toks = np.sort(rng.choice(M, 16, replace=False))
+    toks[0] = 0; toks[-1] = M - 1
+    ref = orc.mul_mat(wt, wq[rows], x[toks], nthreads=8, want=("sum_abs",))
+    check_outputs(y[np.ix_(toks, rows)], ref["y"], ref["sum_abs"], "k-quant prefill")
+    y2 = dev.mul_mat(wt, wq[::-1].copy(), x[:64])
+    assert np.array_equal(y2[:, ::-1], y[:64])
