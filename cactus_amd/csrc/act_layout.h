@@ -19,7 +19,8 @@
 //
 //   F16 activations (for F16 weights), token stride = f16_stride(K): K halves, nothing else.
 //
-// K is a multiple of 256, so every plane starts 16-byte aligned.
+// K is a multiple of 256, so every plane starts 16-byte aligned.  Token strides are multiples of 128 bytes: a token's
+// 128-byte stretches of quants then coincide with cache lines, which halves the lines the GEMM kernels touch.
 #pragma once
 #include <stdint.h>
 #include <stddef.h>
@@ -27,16 +28,17 @@
 namespace chip {
 
 __host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
+__host__ __device__ constexpr size_t align128(size_t v) { return (v + 127) & ~(size_t)127; }
 
 __host__ __device__ constexpr size_t q8_0_off_d(int64_t K)   { return (size_t)K; }
 __host__ __device__ constexpr size_t q8_0_off_sum(int64_t K) { return (size_t)K + 4 * (size_t)(K / 32); }
 __host__ __device__ constexpr size_t q8_0_off_s(int64_t K)   { return (size_t)K + 8 * (size_t)(K / 32); }
-__host__ __device__ constexpr size_t q8_0_stride(int64_t K)  { return align16((size_t)K + 12 * (size_t)(K / 32)); }
+__host__ __device__ constexpr size_t q8_0_stride(int64_t K)  { return align128((size_t)K + 12 * (size_t)(K / 32)); }
 
-__host__ __device__ constexpr size_t f16_stride(int64_t K)   { return align16(2 * (size_t)K); }
+__host__ __device__ constexpr size_t f16_stride(int64_t K)   { return align128(2 * (size_t)K); }
 
 __host__ __device__ constexpr size_t q8_K_off_d(int64_t K)     { return (size_t)K; }
 __host__ __device__ constexpr size_t q8_K_off_bsums(int64_t K) { return (size_t)K + 4 * (size_t)(K / 256); }
-__host__ __device__ constexpr size_t q8_K_stride(int64_t K)    { return align16((size_t)K + 4 * (size_t)(K / 256) + 2 * (size_t)(K / 16)); }
+__host__ __device__ constexpr size_t q8_K_stride(int64_t K)    { return align128((size_t)K + 4 * (size_t)(K / 256) + 2 * (size_t)(K / 16)); }
 
 }  // namespace chip

@@ -17,7 +17,6 @@ namespace {
 
 // From this many tokens on the matrix-core GEMV beats the dot-product GEMV (measured on Q8_0 4096x11008).
 constexpr int MMV_MIN_TOKENS = 5;
-constexpr int GEMM_KQ_MIN_TOKENS = 16;
 
 std::mutex g_mu;
 bool g_limits_ready[64] = {};
@@ -273,9 +272,9 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     const size_t stride = act_stride(chip_vec_dot_type(type), K);
     hipStream_t st = (hipStream_t)stream;
 
-    if (type == T_Q4_0 && n >= 16 && gemm_q4_0_supported(K, N, n))
+    if (type == T_Q4_0 && gemm_q4_0_supported(K, N, n))
         return hip_rc(launch_gemm_q4_0(W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
-    if (n >= GEMM_KQ_MIN_TOKENS && gemm_kq_supported(type, K, N, n))
+    if (gemm_kq_supported(type, K, N, n))
         return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
 
     // 5 tokens or more: integer sums on the matrix cores, up to 16 tokens per pass over the weights

@@ -7,23 +7,23 @@
 // with 6-bit (Q4_K, Q5_K: 32-value sub-blocks) or 8-bit signed (Q6_K: 16-value sub-blocks) integer sub-block
 // scales, and applies the fp16 super-block scales d, dmin and the fp32 activation scale once per super-block.
 // Applying an integer scale after each 32-value MFMA would cost vector work per integer sum, which is what bounds
-// the Q4_0 GEMM.  Here the integer scales are folded into the int8 MFMA operand instead:
+// the Q4_0 GEMM.  Here the integer scales are folded into the int8 MFMA operand instead, as two digit planes:
 //
 //   Q4_K   sc = 8*sh + sl (3-bit digits): planes q*sh and q*sl (both <= 105), sumi = 8*P0 + P1
-//   Q5_K   sc = 16*s2 + 4*s1 + s0 (2-bit digits): planes q*s2, q*s1, q*s0 (<= 93), sumi = 16*P0 + 4*P1 + P2
-//   Q6_K   (q - 32)*sc + 4064 = 64*hi + lo with hi in 0..127, lo in 0..63: two digit planes of the biased product,
+//   Q5_K   the same digits on (q - 16) in -16..15 (products in -112..105), sumi = 8*P0 + P1 + 16 * sum_j sc_j * bsum_j
+//   Q6_K   (q - 32)*sc + 4064 = 64*hi + lo with hi in 0..127, lo in 0..63: the digits of the biased product,
 //          sumi = 64*P0 + P1 - 4064 * (sum of the token's 256 quants, i.e. of its 16 bsums)
-//   mins   summ = sum_k m_j(k) * a_k: one more MFMA whose weight operand is the sub-block's m_j in all 32 positions
-//          (built in registers from one byte, never stored per element)
 //
-// so every plane accumulates in the MFMA's own int32 accumulator over the 8 k-blocks of a super-block and the
-// vector unit only works once per super-block and output (6-7 operations per 256 values instead of 16).  All
-// sums are exact integers, equal to the reference's sumi and summ.
+// so both planes accumulate in the MFMA's own int32 accumulator over the 8 k-blocks of a super-block.  The sums
+// against the activation block sums, summ (and Q5_K's sum_j sc_j * bsum_j), are a product with inner dimension 16
+// per super-block - the 16 bsums of block_q8_K, each |bsum| <= 2048, against m_j (sc_j) <= 63 taken twice - which
+// is exact in fp16 inputs with fp32 accumulation: one v_mfma_f32_32x32x16_f16 per super-block and tile.  The vector
+// unit works only once per super-block and output (5-6 operations per 256 values instead of 16).  All sums are
+// exact integers, equal to the reference's sumi and summ.
 //
 // Structure: a workgroup of WR x WC waves owns 32*WR rows x 64*WC tokens; each wave owns one 32-row tile by two
-// 32-token tiles.  LDS is double buffered over stages of 4 k-blocks (half a super-block), one barrier per stage,
-// the next stage's global loads in flight during the current stage's MFMAs.  Operand cells are 16 bytes
-// ([plane][k-block][k-half][row]), exactly what one lane feeds v_mfma_i32_32x32x32_i8.
+// 32-token tiles.  LDS is double buffered over stages of 4 k-blocks (half a super-block), one barrier per stage.
+// Operand cells are 16 bytes ([plane][k-block][k-half][row]), exactly what one lane feeds v_mfma_i32_32x32x32_i8.
 #include "dev_common.h"
 #include "act_layout.h"
 #include "kernels.h"
@@ -34,10 +34,13 @@ namespace chip {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int KQ_KB = 4;                      // 32-value k-blocks per LDS stage
 constexpr int KQ_TN = 2;                      // 32-token tiles per wave
+constexpr int KQ_NPL = 2;                     // int8 digit planes per weight type
 constexpr int Q6_BIAS = 4064;                 // 32 * 127: makes (q - 32) * sc + bias >= 0 for every int8 sc
 
 // two independent 16-bit products / multiply-adds per dword (v_pk_mul_lo_u16, v_pk_mad_u16)
@@ -55,26 +58,52 @@ __device__ __forceinline__ void scale_min_pair(const u32x4 &h, int jp, uint32_t 
     const int sh = 16 * (jp & 1);
     const uint32_t a1 = h.y >> sh, a2 = h.z >> sh, a3 = h.w >> sh;
     if (jp < 2) { sc = a1 & 0x3f3fu; mn = a2 & 0x3f3fu; }
-    else        { sc = (a3 & 0x0f0fu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
+    else        { sc = (a3 & 0x0f0f0f0fu & 0xffffu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
+}
+// the same for four sub-blocks at once, one per byte: sub-blocks 0..3 (g = 0) or 4..7 (g = 1)
+__device__ __forceinline__ void scale_min_quad(const u32x4 &h, int g, uint32_t &sc, uint32_t &mn) {
+    if (g == 0) { sc = h.y & 0x3f3f3f3fu; mn = h.z & 0x3f3f3f3fu; }
+    else        { sc = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u); mn = ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u); }
+}
+// four small integers (one per byte) -> the fp16 operand cell {b0, b0, b1, b1, b2, b2, b3, b3}: sub-block j stands
+// against the two 16-value bsums 2j and 2j+1
+__device__ __forceinline__ u32x4 bytes_to_f16_pairs(uint32_t v) {
+    u32x4 c;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t hbits = (uint32_t)__half_as_ushort(__float2half_rn((float)((v >> (8 * i)) & 0xffu)));   // exact
+        c[i] = hbits | (hbits << 16);
+    }
+    return c;
+}
+// eight int16 -> eight fp16 (exact for |v| <= 2048)
+__device__ __forceinline__ u32x4 i16x8_to_f16(const u32x4 &v) {
+    u32x4 c;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const _Float16 lo = (_Float16)(int16_t)(v[i] & 0xffffu), hi = (_Float16)(int16_t)(v[i] >> 16);
+        c[i] = (uint32_t)__builtin_bit_cast(unsigned short, lo) | ((uint32_t)__builtin_bit_cast(unsigned short, hi) << 16);
+    }
+    return c;
 }
 
 // One staging item = (row, x) of a stage h (half of a super-block): 16 bytes of packed quants that expand into
-// the 16-value k-half hf = x & 1 of two k-blocks kb0(x), kb1(x) of the stage, for every stored plane.
+// the 16-value k-half hf = x & 1 of two k-blocks kb0(x), kb1(x) of the stage, for both digit planes.
 struct Emit {
-    u32x4 cell[3][2];      // [plane][0: k-block kb0, 1: k-block kb1]
-    uint32_t mins;         // m of kb0 | m of kb1 << 8
-    uint32_t dd;           // d | dmin << 16 (fp16 bits)
+    u32x4 cell[KQ_NPL][2]; // [plane][0: k-block kb0, 1: k-block kb1]
 };
 
 template <int WT> struct KQ;
 
 template <> struct KQ<T_Q4_K> {
-    static constexpr int BYTES = BYTES_Q4_K, NPL = 2, NACC = 3;
-    static constexpr bool HAS_MIN = true, HAS_BSUM = false;
-    struct Raw { u32x4 hdr, q; };
-    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *blk, int h, int x) {
+    static constexpr int BYTES = BYTES_Q4_K, NF16 = 1;             // fp16 products: summ
+    static constexpr bool HAS_BSUM = false;
+    // what item x of a row needs from one super-block: the 16 header bytes and 16 quant bytes per half
+    struct Raw { u32x4 hdr, q[2]; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *blk, int x) {
         r.hdr = *reinterpret_cast<const u32x4 *>(blk);
-        r.q = *reinterpret_cast<const u32x4 *>(blk + 16 + 64 * h + 16 * x);       // qs[32*jp + 16*hf], jp = 2h + x/2
+        r.q[0] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * x);             // qs[32*jp + 16*hf], jp = 2h + x/2
+        r.q[1] = *reinterpret_cast<const u32x4 *>(blk + 80 + 16 * x);
     }
     __device__ static __forceinline__ int kb0(int x) { return x & 2; }            // low nibbles: sub-block 2*jp
     __device__ static __forceinline__ int kb1(int x) { return (x & 2) + 1; }      // high nibbles: sub-block 2*jp + 1
@@ -83,28 +112,35 @@ template <> struct KQ<T_Q4_K> {
         scale_min_pair(r.hdr, 2 * h + (x >> 1), sc, mn);
         const uint32_t sc0 = sc & 0xff, sc1 = sc >> 8;
         const uint32_t sh0 = splat16(sc0 >> 3), sl0 = splat16(sc0 & 7), sh1 = splat16(sc1 >> 3), sl1 = splat16(sc1 & 7);
+        const u32x4 q = r.q[h];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t lo = r.q[i] & 0x0f0f0f0fu, hi = (r.q[i] >> 4) & 0x0f0f0f0fu;
+            const uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
             e.cell[0][0][i] = pk_mul16(lo, sh0); e.cell[1][0][i] = pk_mul16(lo, sl0);   // byte products < 256: no carries
             e.cell[0][1][i] = pk_mul16(hi, sh1); e.cell[1][1][i] = pk_mul16(hi, sl1);
         }
-        e.mins = mn;
-        e.dd = r.hdr.x;
     }
-    __device__ static __forceinline__ float value(const int (&p)[NACC], uint32_t dd, int) {
-        return h2f(dd) * (float)((p[0] << 3) + p[1]) - h2f(dd >> 16) * (float)p[2];
+    __device__ static __forceinline__ uint32_t scales(const Raw &r) { return r.hdr.x; }        // d | dmin << 16
+    // fp16 operand cell of item x < 2: mins of sub-blocks 4x .. 4x+3
+    __device__ static __forceinline__ u32x4 f16_cell(const Raw &r, int x) {
+        uint32_t sc, mn;
+        scale_min_quad(r.hdr, x & 1, sc, mn);
+        return bytes_to_f16_pairs(mn);
+    }
+    __device__ static __forceinline__ float value(int p0, int p1, const float (&f)[2], uint32_t dd, int) {
+        return __builtin_fmaf(-h2f(dd >> 16), f[0], __builtin_fmaf(h2f(dd), (float)((p0 << 3) + p1), 0.f));
     }
 };
 
 template <> struct KQ<T_Q5_K> {
-    static constexpr int BYTES = BYTES_Q5_K, NPL = 3, NACC = 4;
-    static constexpr bool HAS_MIN = true, HAS_BSUM = false;
-    struct Raw { u32x4 hdr, q, qh; };
-    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *blk, int h, int x) {
+    static constexpr int BYTES = BYTES_Q5_K, NF16 = 2;             // fp16 products: summ, sum_j sc_j * bsum_j
+    static constexpr bool HAS_BSUM = false;
+    struct Raw { u32x4 hdr, qh, q[2]; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *blk, int x) {
         r.hdr = *reinterpret_cast<const u32x4 *>(blk);
         r.qh = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (x & 1));          // qh[l], l = 16*hf + [0,16)
-        r.q = *reinterpret_cast<const u32x4 *>(blk + 48 + 64 * h + 16 * x);
+        r.q[0] = *reinterpret_cast<const u32x4 *>(blk + 48 + 16 * x);
+        r.q[1] = *reinterpret_cast<const u32x4 *>(blk + 112 + 16 * x);
     }
     __device__ static __forceinline__ int kb0(int x) { return x & 2; }
     __device__ static __forceinline__ int kb1(int x) { return (x & 2) + 1; }
@@ -113,40 +149,53 @@ template <> struct KQ<T_Q5_K> {
         uint32_t sc, mn;
         scale_min_pair(r.hdr, jp, sc, mn);
         const uint32_t sc0 = sc & 0xff, sc1 = sc >> 8;
-        const uint32_t a2 = splat16(sc0 >> 4), a1 = splat16((sc0 >> 2) & 3), a0 = splat16(sc0 & 3);
-        const uint32_t b2 = splat16(sc1 >> 4), b1 = splat16((sc1 >> 2) & 3), b0 = splat16(sc1 & 3);
+        // byte = q*s + (128 - 16*s) lies in 16..233 for q in 0..31, s in 0..7: no carries between the bytes of a
+        // 16-bit lane, and flipping bit 7 turns it into the signed byte (q - 16)*s
+        const uint32_t sh0 = sc0 >> 3, sl0 = sc0 & 7, sh1 = sc1 >> 3, sl1 = sc1 & 7;
+        const uint32_t mh0 = splat16(sh0), ml0 = splat16(sl0), mh1 = splat16(sh1), ml1 = splat16(sl1);
+        const uint32_t ah0 = splat16((128 - 16 * sh0) * 0x101u), al0 = splat16((128 - 16 * sl0) * 0x101u);
+        const uint32_t ah1 = splat16((128 - 16 * sh1) * 0x101u), al1 = splat16((128 - 16 * sl1) * 0x101u);
+        const u32x4 q = r.q[h];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             // bit 2*jp of qh[l] is the fifth bit of element 64*jp + l, bit 2*jp + 1 that of 64*jp + 32 + l
             // (reference ggml-quants.c:1460-1478)
             const uint32_t hb = r.qh[i] >> (2 * jp);
-            const uint32_t lo = (r.q[i] & 0x0f0f0f0fu) | ((hb << 4) & 0x10101010u);
-            const uint32_t hi = ((r.q[i] >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
-            e.cell[0][0][i] = pk_mul16(lo, a2); e.cell[1][0][i] = pk_mul16(lo, a1); e.cell[2][0][i] = pk_mul16(lo, a0);
-            e.cell[0][1][i] = pk_mul16(hi, b2); e.cell[1][1][i] = pk_mul16(hi, b1); e.cell[2][1][i] = pk_mul16(hi, b0);
+            const uint32_t lo = (q[i] & 0x0f0f0f0fu) | ((hb << 4) & 0x10101010u);
+            const uint32_t hi = ((q[i] >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
+            e.cell[0][0][i] = pk_mad16(lo, mh0, ah0) ^ 0x80808080u; e.cell[1][0][i] = pk_mad16(lo, ml0, al0) ^ 0x80808080u;
+            e.cell[0][1][i] = pk_mad16(hi, mh1, ah1) ^ 0x80808080u; e.cell[1][1][i] = pk_mad16(hi, ml1, al1) ^ 0x80808080u;
         }
-        e.mins = mn;
-        e.dd = r.hdr.x;
     }
-    __device__ static __forceinline__ float value(const int (&p)[NACC], uint32_t dd, int) {
-        return h2f(dd) * (float)((p[0] << 4) + (p[1] << 2) + p[2]) - h2f(dd >> 16) * (float)p[3];
+    __device__ static __forceinline__ uint32_t scales(const Raw &r) { return r.hdr.x; }
+    // item x: x / 2 = 0 mins, 1 scales; x & 1 = sub-blocks 0..3 or 4..7
+    __device__ static __forceinline__ u32x4 f16_cell(const Raw &r, int x) {
+        uint32_t sc, mn;
+        scale_min_quad(r.hdr, x & 1, sc, mn);
+        return bytes_to_f16_pairs((x & 2) ? sc : mn);
+    }
+    __device__ static __forceinline__ float value(int p0, int p1, const float (&f)[2], uint32_t dd, int) {
+        const int sumi = (p0 << 3) + p1 + ((int)f[1] << 4);                 // f[1] is an exact integer below 2^24
+        return __builtin_fmaf(-h2f(dd >> 16), f[0], __builtin_fmaf(h2f(dd), (float)sumi, 0.f));
     }
 };
 
 template <> struct KQ<T_Q6_K> {
-    static constexpr int BYTES = BYTES_Q6_K, NPL = 2, NACC = 2;
-    static constexpr bool HAS_MIN = false, HAS_BSUM = true;
-    struct Raw { u32x4 ql, qh; int s0, s1; uint32_t d; };
+    static constexpr int BYTES = BYTES_Q6_K, NF16 = 0;
+    static constexpr bool HAS_BSUM = true;
+    struct Raw { u32x4 ql[2], qh[2], sc; uint32_t d; };
     // Half h of a super-block holds, for l = 0..31, the elements 128h + 32b + l of k-blocks b = 0..3 as
     //   low / high nibble of ql[64h + l] (b = 0 / 2) and of ql[64h + 32 + l] (b = 1 / 3), two more bits from
     //   qh[32h + l] >> 2b, scale scales[8h + 2b + l/16]                       (reference ggml-quants.c:1695-1711)
     // item x: p = x / 2 picks the ql half (k-blocks p and p + 2), hf = x & 1 the 16 values l = 16*hf + [0,16).
-    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *blk, int h, int x) {
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *blk, int x) {
         const int p = x >> 1, hf = x & 1;
-        r.ql = *reinterpret_cast<const u32x4_a2 *>(blk + 64 * h + 32 * p + 16 * hf);
-        r.qh = *reinterpret_cast<const u32x4_a2 *>(blk + 128 + 32 * h + 16 * hf);
-        r.s0 = *reinterpret_cast<const int8_t *>(blk + 192 + 8 * h + 2 * p + hf);
-        r.s1 = *reinterpret_cast<const int8_t *>(blk + 192 + 8 * h + 2 * p + 4 + hf);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            r.ql[h] = *reinterpret_cast<const u32x4_a2 *>(blk + 64 * h + 32 * p + 16 * hf);
+            r.qh[h] = *reinterpret_cast<const u32x4_a2 *>(blk + 128 + 32 * h + 16 * hf);
+        }
+        r.sc = *reinterpret_cast<const u32x4_a2 *>(blk + 192);
         r.d = *reinterpret_cast<const unsigned short *>(blk + 208);
     }
     __device__ static __forceinline__ int kb0(int x) { return x >> 1; }
@@ -158,180 +207,252 @@ template <> struct KQ<T_Q6_K> {
         hi = ((ue >> 6) & 0x007f007fu) | (((uo >> 6) & 0x007f007fu) << 8);
         lo = (ue & 0x003f003fu) | ((uo & 0x003f003fu) << 8);
     }
-    __device__ static __forceinline__ void emit(Emit &e, const Raw &r, int, int x) {
-        const int p = x >> 1;
-        const uint32_t sa = splat16((uint32_t)r.s0), ba = splat16((uint32_t)(Q6_BIAS - 32 * r.s0));
-        const uint32_t sb = splat16((uint32_t)r.s1), bb = splat16((uint32_t)(Q6_BIAS - 32 * r.s1));
+    __device__ static __forceinline__ void emit(Emit &e, const Raw &r, int h, int x) {
+        const int p = x >> 1, hf = x & 1;
+        // scales[8h + 2p + hf] and scales[8h + 2p + 4 + hf]: byte 2p + hf of dwords 2h and 2h + 1
+        const int s0 = __builtin_amdgcn_sbfe((int)r.sc[2 * h], 8 * (2 * p + hf), 8);
+        const int s1 = __builtin_amdgcn_sbfe((int)r.sc[2 * h + 1], 8 * (2 * p + hf), 8);
+        const uint32_t sa = splat16((uint32_t)s0), ba = splat16((uint32_t)(Q6_BIAS - 32 * s0));
+        const uint32_t sb = splat16((uint32_t)s1), bb = splat16((uint32_t)(Q6_BIAS - 32 * s1));
+        const u32x4 ql = r.ql[h], qh = r.qh[h];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t hb = r.qh[i] >> (2 * p);
-            const uint32_t q0 = (r.ql[i] & 0x0f0f0f0fu) | ((hb << 4) & 0x30303030u);            // k-block p
-            const uint32_t q1 = ((r.ql[i] >> 4) & 0x0f0f0f0fu) | (hb & 0x30303030u);            // k-block p + 2
+            const uint32_t hb = qh[i] >> (2 * p);
+            const uint32_t q0 = (ql[i] & 0x0f0f0f0fu) | ((hb << 4) & 0x30303030u);            // k-block p
+            const uint32_t q1 = ((ql[i] >> 4) & 0x0f0f0f0fu) | (hb & 0x30303030u);            // k-block p + 2
             uint32_t hi, lo;
             digits(q0, sa, ba, hi, lo);
             e.cell[0][0][i] = hi; e.cell[1][0][i] = lo;
             digits(q1, sb, bb, hi, lo);
             e.cell[0][1][i] = hi; e.cell[1][1][i] = lo;
         }
-        e.mins = 0;
-        e.dd = r.d;
     }
-    __device__ static __forceinline__ float value(const int (&p)[NACC], uint32_t dd, int corr) {
-        return h2f(dd) * (float)((p[0] << 6) + p[1] + corr);
+    __device__ static __forceinline__ uint32_t scales(const Raw &r) { return r.d; }
+    __device__ static __forceinline__ u32x4 f16_cell(const Raw &, int) { return u32x4{0u, 0u, 0u, 0u}; }
+    __device__ static __forceinline__ float value(int p0, int p1, const float (&)[2], uint32_t dd, int corr) {
+        return __builtin_fmaf(h2f(dd), (float)((p0 << 6) + p1 + corr), 0.f);
     }
 };
+
+constexpr int KQ_PRODUCERS = 4;               // staging waves per workgroup, one per SIMD
 
 template <int WT, int WR, int WC>
 struct KqCfg {
     using T = KQ<WT>;
-    static constexpr int NW = WR * WC, NT = NW * 64;
+    static constexpr int NC = WR * WC;                             // MFMA waves
+    static constexpr int NW = NC + KQ_PRODUCERS, NT = NW * 64;
+    static constexpr int NPT = KQ_PRODUCERS * 64;                  // staging threads
     static constexpr int BM = 32 * WR;                             // weight rows per workgroup
     static constexpr int BN = 32 * KQ_TN * WC;                     // tokens per workgroup
+    static constexpr int NF = T::NF16 > 0 ? T::NF16 : 1;
     // plane stride 2 mod 16 cells: the staging threads of one wave spread over the bank groups
     static constexpr int A_PLANE = BM + 2, B_PLANE = BN + 2;
-    static constexpr int A_CELLS = T::NPL * KQ_KB * 2 * A_PLANE;   // 16-byte cells
+    static constexpr int A_CELLS = KQ_NPL * KQ_KB * 2 * A_PLANE;   // 16-byte cells
     static constexpr int B_CELLS = KQ_KB * 2 * B_PLANE;
+    // one stage buffer (two of them, by stage parity)
     static constexpr size_t OFF_A = 0;
     static constexpr size_t OFF_B = OFF_A + (size_t)A_CELLS * 16;
-    static constexpr size_t OFF_SD = OFF_B + (size_t)B_CELLS * 16;          // u32 [BM]: d | dmin << 16, permuted per 32 rows
-    static constexpr size_t OFF_SM = OFF_SD + (size_t)BM * 4;               // u8  [BM][4]: m of the stage's 4 k-blocks
-    static constexpr size_t OFF_SX = OFF_SM + (size_t)BM * 4;               // f32 [BN]: activation scale of the super-block
+    static constexpr size_t STAGE = OFF_B + (size_t)B_CELLS * 16;
+    // one super-block buffer (two of them, by super-block parity)
+    static constexpr size_t OFF_FA = 0;                                     // fp16 cells [NF16][k-half][BM]: m_j (sc_j) twice
+    static constexpr size_t OFF_FB = OFF_FA + (size_t)NF * 2 * BM * 16;     // fp16 cells [k-half][BN]: the token's 16 bsums
+    static constexpr size_t OFF_SD = OFF_FB + (size_t)2 * BN * 16;          // u32 [BM]: d | dmin << 16, permuted per 32 rows
+    static constexpr size_t OFF_SX = OFF_SD + (size_t)BM * 4;               // f32 [BN]: activation scale of the super-block
     static constexpr size_t OFF_SC = OFF_SX + (size_t)BN * 4;               // i32 [BN]: -4064 * sum of the token's quants
-    static constexpr size_t STAGE = OFF_SC + (size_t)BN * 4;
+    static constexpr size_t SBLK = OFF_SC + (size_t)BN * 4;
+    static constexpr size_t OFF_STAGES = 0;
+    static constexpr size_t OFF_SBLK = 2 * STAGE;
+    static constexpr size_t OFF_DUMP = OFF_SBLK + 2 * SBLK;                 // 16 bytes per staging thread: where stores that do not apply go
+    static constexpr size_t TOTAL = OFF_DUMP + (size_t)NPT * 16;
     static constexpr int W_ITEMS = BM * 4;
-    static constexpr int W_PER_T = (W_ITEMS + NT - 1) / NT;
+    static constexpr int W_PER_T = W_ITEMS / NPT;
     static constexpr int X_ITEMS = BN * KQ_KB * 2;
-    static constexpr int X_PER_T = (X_ITEMS + NT - 1) / NT;
-    static_assert(BN <= NT, "one thread per token stages the activation scale");
-    static_assert(STAGE % 16 == 0, "stage buffers keep 16-byte alignment");
+    static constexpr int X_PER_T = X_ITEMS / NPT;
+    static_assert(2 * BN <= NPT, "two staging threads per token convert its block sums");
+    static_assert(W_ITEMS % NPT == 0 && X_ITEMS % NPT == 0, "staging items divide evenly over the staging threads");
+    static_assert(STAGE % 16 == 0 && SBLK % 16 == 0, "buffers keep 16-byte alignment");
 };
 
+// A workgroup is WR x WC MFMA waves plus four staging waves (one per SIMD).  Per stage (4 k-blocks = half a
+// super-block; LDS double buffered; one barrier per stage):
+//
+//     staging waves : global loads of stage s+3 | expand stage s+1 (loaded two stages ago) into the other buffer
+//     MFMA waves    : 4 k-blocks of MFMAs from the current buffer | after a super-block's second half: fold
+//
+// The two kinds of wave run side by side on every SIMD, so operand expansion (vector pipe, LDS writes, memory
+// latency) overlaps the matrix pipe by construction instead of by instruction scheduling.  Nothing in the loops is
+// conditional: loads past the last stage repeat it, and stores that do not apply go to a per-thread dump slot.
 template <int WT, int WR, int WC, int OCC>
-__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+__global__ __launch_bounds__((WR * WC + KQ_PRODUCERS) * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
-                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy) {
+                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map) {
     using T = KQ<WT>;
     using C = KqCfg<WT, WR, WC>;
     constexpr int TN = KQ_TN;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave / WC, wc = wave % WC;
-    const int half = lane >> 5, l32 = lane & 31;
-    const int64_t row_base = (int64_t)blockIdx.x * C::BM;
-    const int64_t tok_base = (int64_t)blockIdx.y * C::BN;
     const int nstages = (int)(K / QK_K) * 2;
-    const size_t off_d = q8_K_off_d(K), off_bs = q8_K_off_bsums(K);
+    const TileCoord tc = xcd_tile(blockIdx.x, map);
+    if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;        // padding of the tile map
+    const int64_t row_base = (int64_t)tc.row_tile * C::BM;
+    const int64_t tok_base = (int64_t)tc.tok_tile * C::BN;
 
-    // ---- per-thread prefetch registers for one stage ----
-    typename T::Raw wraw[C::W_PER_T];
-    u32x4 xq[C::X_PER_T];
-    float xs = 0.f;
-    int xc = 0;
+    if (wave >= C::NC) {
+        // ------------------------------------------------------------------------------------ staging waves
+        const int pt = tid - C::NC * 64;
+        const size_t off_d = q8_K_off_d(K), off_bs = q8_K_off_bsums(K);
+        uint8_t *const dump = lds + C::OFF_DUMP + pt * 16;
+        struct Acts {
+            u32x4 x[C::X_PER_T];
+            u32x4 bs;          // 8 of the token's bsums (threads 2*token + k-half)
+            float xs;
+            int xc;
+        };
+        struct Wts { typename T::Raw w[C::W_PER_T]; };
+        Acts E, O;             // activations of an even / odd stage
+        Wts W0, W1;            // weights of an even / odd super-block (both halves: every cache line is fetched once)
+        // per-thread source addresses of stage 0 (they advance by a constant per stage / super-block)
+        const uint8_t *wsrc[C::W_PER_T], *xsrc[C::X_PER_T];
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; i++) wsrc[i] = W + (size_t)min(row_base + ((pt + i * C::NPT) >> 2), N - 1) * nb01;
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; i++)
+            xsrc[i] = ws + (size_t)min(tok_base + ((pt + i * C::NPT) >> 3), M - 1) * ws_stride + 16 * ((pt + i * C::NPT) & 7);
+        // activation scale: thread t < BN for token t; block sums: thread t < 2*BN for token t/2, half t&1
+        const uint8_t *ssrc = ws + (size_t)min(tok_base + min(pt, C::BN - 1), M - 1) * ws_stride;
+        const uint8_t *bsrc = ws + (size_t)min(tok_base + min(pt >> 1, C::BN - 1), M - 1) * ws_stride + off_bs + 16 * (pt & 1);
+        const int nsb = nstages >> 1;
 
-    auto fetch = [&](int stage) {
-        const int sb = stage >> 1, h = stage & 1;
+        auto fetch_w = [&](Wts &R, int sb_wanted) {
+            const int sb = min(sb_wanted, nsb - 1);
 #pragma unroll
-        for (int i = 0; i < C::W_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
-                const int64_t row = min(row_base + (item >> 2), N - 1);
-                T::fetch(wraw[i], W + (size_t)row * nb01 + (size_t)sb * T::BYTES, h, item & 3);
-            }
-        }
+            for (int i = 0; i < C::W_PER_T; i++) T::fetch(R.w[i], wsrc[i] + (size_t)sb * T::BYTES, (pt + i * C::NPT) & 3);
+        };
+        auto fetch_x = [&](Acts &R, int stage_wanted, auto even_tag) {
+            constexpr bool even = decltype(even_tag)::value;
+            const int stage = min(stage_wanted, nstages - 1);
+            const int sb = stage >> 1;
 #pragma unroll
-        for (int i = 0; i < C::X_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
-                const int64_t tok = min(tok_base + (item >> 3), M - 1);
-                xq[i] = *reinterpret_cast<const u32x4 *>(ws + (size_t)tok * ws_stride + (size_t)stage * (32 * KQ_KB) + 16 * (item & 7));
-            }
-        }
-        if (tid < C::BN) {
-            const uint8_t *t = ws + (size_t)min(tok_base + tid, M - 1) * ws_stride;
-            xs = reinterpret_cast<const float *>(t + off_d)[sb];
-            if constexpr (T::HAS_BSUM) {
-                const u32x4 *bp = reinterpret_cast<const u32x4 *>(t + off_bs + (size_t)sb * 32);
-                const u32x4 b0 = bp[0], b1 = bp[1];
-                const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
-                int sum = 0;
+            for (int i = 0; i < C::X_PER_T; i++) R.x[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + (size_t)stage * (32 * KQ_KB));
+            if constexpr (even) {
+                R.xs = reinterpret_cast<const float *>(ssrc + off_d)[sb];
+                if constexpr (T::NF16 > 0) R.bs = *reinterpret_cast<const u32x4 *>(bsrc + (size_t)sb * 32);
+                if constexpr (T::HAS_BSUM) {
+                    const u32x4 *bp = reinterpret_cast<const u32x4 *>(ssrc + off_bs + (size_t)sb * 32);
+                    const u32x4 b0 = bp[0], b1 = bp[1];
+                    const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+                    int sum = 0;
 #pragma unroll
-                for (int j = 0; j < 8; j++) sum += (int)(int16_t)(w[j] & 0xffffu) + ((int)w[j] >> 16);
-                xc = -Q6_BIAS * sum;
+                    for (int j = 0; j < 8; j++) sum += (int)(int16_t)(w[j] & 0xffffu) + ((int)w[j] >> 16);
+                    R.xc = -Q6_BIAS * sum;
+                }
             }
-        }
-    };
+        };
 
-    auto commit = [&](int stage, int buf) {
-        const int h = stage & 1;
-        uint8_t *base = lds + (size_t)buf * C::STAGE;
-        u32x4 *A = reinterpret_cast<u32x4 *>(base + C::OFF_A);
-        u32x4 *B = reinterpret_cast<u32x4 *>(base + C::OFF_B);
+        // expand a prefetched stage into LDS buffer `buf`; even stages also carry the super-block's scales
+        auto commit = [&](const Wts &RW, const Acts &R, int buf, int sbp, auto even_tag) {
+            constexpr bool even = decltype(even_tag)::value;
+            constexpr int h = even ? 0 : 1;
+            uint8_t *base = lds + C::OFF_STAGES + (size_t)buf * C::STAGE;
+            uint8_t *sblk = lds + C::OFF_SBLK + (size_t)sbp * C::SBLK;
+            u32x4 *A = reinterpret_cast<u32x4 *>(base + C::OFF_A);
+            u32x4 *B = reinterpret_cast<u32x4 *>(base + C::OFF_B);
 #pragma unroll
-        for (int i = 0; i < C::W_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
+            for (int i = 0; i < C::W_PER_T; i++) {
+                const int item = pt + i * C::NPT;
                 const int r = item >> 2, x = item & 3, hf = x & 1;
                 Emit e;
-                T::emit(e, wraw[i], h, x);
+                T::emit(e, RW.w[i], h, x);
                 const int k0 = T::kb0(x), k1 = T::kb1(x);
 #pragma unroll
-                for (int pl = 0; pl < T::NPL; pl++) {
+                for (int pl = 0; pl < KQ_NPL; pl++) {
                     A[((pl * KQ_KB + k0) * 2 + hf) * C::A_PLANE + r] = e.cell[pl][0];
                     A[((pl * KQ_KB + k1) * 2 + hf) * C::A_PLANE + r] = e.cell[pl][1];
                 }
-                if constexpr (T::HAS_MIN) {
-                    // sub-blocks kb0, kb1 = kb0 + 1 of this row: two adjacent bytes, written by the hf = 0 item
-                    if (hf == 0) *reinterpret_cast<unsigned short *>(base + C::OFF_SM + r * 4 + k0) = (unsigned short)e.mins;
-                }
-                if (x == 0) {
+                if constexpr (even) {
                     // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4:
                     // keep the scale of row i at half*16 + (i/8)*4 + i%4 so a lane reads its 16 scales contiguously
                     const int i32 = r & 31;
                     const int pos = ((i32 >> 2) & 1) * 16 + (i32 >> 3) * 4 + (i32 & 3);
-                    reinterpret_cast<uint32_t *>(base + C::OFF_SD)[(r & ~31) + pos] = e.dd;
+                    uint8_t *dst = (x == 0) ? sblk + C::OFF_SD + ((r & ~31) + pos) * 4 : dump;
+                    *reinterpret_cast<uint32_t *>(dst) = T::scales(RW.w[i]);
+                    if constexpr (T::NF16 > 0) {
+                        // items x < 2*NF16 of a row each build one fp16 operand cell [x/2][x&1][row]
+                        uint8_t *fd = (x < 2 * T::NF16) ? sblk + C::OFF_FA + (size_t)(x * C::BM + r) * 16 : dump;
+                        *reinterpret_cast<u32x4 *>(fd) = T::f16_cell(RW.w[i], x);
+                    }
                 }
             }
-        }
 #pragma unroll
-        for (int i = 0; i < C::X_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) B[(item & 7) * C::B_PLANE + (item >> 3)] = xq[i];
-        }
-        if (tid < C::BN) {
-            reinterpret_cast<float *>(base + C::OFF_SX)[tid] = xs;
-            if constexpr (T::HAS_BSUM) reinterpret_cast<int *>(base + C::OFF_SC)[tid] = xc;
-        }
-    };
+            for (int i = 0; i < C::X_PER_T; i++) {
+                const int item = pt + i * C::NPT;
+                B[(item & 7) * C::B_PLANE + (item >> 3)] = R.x[i];
+            }
+            if constexpr (even) {
+                uint8_t *dx = (pt < C::BN) ? sblk + C::OFF_SX + pt * 4 : dump;
+                *reinterpret_cast<float *>(dx) = R.xs;
+                if constexpr (T::HAS_BSUM) {
+                    uint8_t *dc = (pt < C::BN) ? sblk + C::OFF_SC + pt * 4 : dump;
+                    *reinterpret_cast<int *>(dc) = R.xc;
+                }
+                if constexpr (T::NF16 > 0) {
+                    uint8_t *fb = (pt < 2 * C::BN) ? sblk + C::OFF_FB + (size_t)((pt & 1) * C::BN + (pt >> 1)) * 16 : dump;
+                    *reinterpret_cast<u32x4 *>(fb) = i16x8_to_f16(R.bs);
+                }
+            }
+        };
 
-    i32x16 P[T::NACC][TN];
+        // the two staging steps that run while the MFMA waves work on super-block j (weights in `cur`); `nxt` holds
+        // super-block j + 1, and `cur` is refilled with super-block j + 2 once its second half has been expanded
+        auto steps = [&](Wts &cur, Wts &nxt, int j) {
+            fetch_x(E, 2 * j + 2, std::true_type{});
+            commit(cur, O, 1, j & 1, std::false_type{});                  // stage 2j + 1, during stage 2j
+            __syncthreads();
+            fetch_x(O, 2 * j + 3, std::false_type{});
+            fetch_w(cur, j + 2);
+            commit(nxt, E, 0, (j + 1) & 1, std::true_type{});             // stage 2j + 2, during stage 2j + 1 and the fold
+            __syncthreads();
+        };
+
+        fetch_w(W0, 0);
+        fetch_x(E, 0, std::true_type{});
+        fetch_x(O, 1, std::false_type{});
+        fetch_w(W1, 1);
+        commit(W0, E, 0, 0, std::true_type{});
+        __syncthreads();
+        for (int j = 0; j < nsb; j += 2) {
+            steps(W0, W1, j);
+            if (j + 1 < nsb) steps(W1, W0, j + 1);
+        }
+        return;
+    }
+
+    // ------------------------------------------------------------------------------------------ MFMA waves
+    const int wr = wave / WC, wc = wave % WC;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int r0 = wr * 32, n0 = wc * TN * 32;
+
+    i32x16 P[KQ_NPL][TN];
     float out[TN][16];
 #pragma unroll
     for (int c = 0; c < TN; c++)
 #pragma unroll
         for (int v = 0; v < 16; v++) out[c][v] = 0.f;
 
-    const int r0 = wr * 32, n0 = wc * TN * 32;
-
     // 4 k-blocks of one stage; `first` starts the super-block's accumulators from zero
     auto compute = [&](int buf, auto first_tag) {
         constexpr bool first = decltype(first_tag)::value;
-        const uint8_t *base = lds + (size_t)buf * C::STAGE;
+        const uint8_t *base = lds + C::OFF_STAGES + (size_t)buf * C::STAGE;
         const u32x4 *A = reinterpret_cast<const u32x4 *>(base + C::OFF_A);
         const u32x4 *B = reinterpret_cast<const u32x4 *>(base + C::OFF_B);
-        uint32_t mw = 0;
-        if constexpr (T::HAS_MIN) mw = reinterpret_cast<const uint32_t *>(base + C::OFF_SM)[r0 + l32];
 #pragma unroll
         for (int b = 0; b < KQ_KB; b++) {
-            i32x4 af[T::NACC], bf[TN];
+            i32x4 af[KQ_NPL], bf[TN];
 #pragma unroll
-            for (int pl = 0; pl < T::NPL; pl++) {
+            for (int pl = 0; pl < KQ_NPL; pl++) {
                 const u32x4 t = A[((pl * KQ_KB + b) * 2 + half) * C::A_PLANE + r0 + l32];
                 af[pl] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
-            }
-            if constexpr (T::HAS_MIN) {
-                const int m4 = (int)__builtin_amdgcn_perm(mw, mw, 0x01010101u * (uint32_t)b);   // byte b in all four bytes
-                af[T::NPL] = i32x4{m4, m4, m4, m4};
             }
 #pragma unroll
             for (int c = 0; c < TN; c++) {
@@ -339,57 +460,60 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
                 bf[c] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
             }
 #pragma unroll
-            for (int pl = 0; pl < T::NACC; pl++)
+            for (int pl = 0; pl < KQ_NPL; pl++)
 #pragma unroll
                 for (int c = 0; c < TN; c++) {
-                    if constexpr (first) {
-                        if (b == 0) {
-                            const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                            P[pl][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[pl], bf[c], zero, 0, 0, 0);
-                            continue;
-                        }
+                    if (first && b == 0) {
+                        const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        P[pl][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[pl], bf[c], zero, 0, 0, 0);
+                    } else {
+                        P[pl][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[pl], bf[c], P[pl][c], 0, 0, 0);
                     }
-                    P[pl][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[pl], bf[c], P[pl][c], 0, 0, 0);
                 }
         }
     };
 
-    // once per super-block: fold the planes and apply d, dmin and the activation scale
-    auto finish = [&](int buf) {
-        const uint8_t *base = lds + (size_t)buf * C::STAGE;
-        const u32x4 *sp = reinterpret_cast<const u32x4 *>(base + C::OFF_SD) + (r0 + half * 16) / 4;
+    // once per super-block: the fp16 products against the block sums, then fold the planes and apply d, dmin and
+    // the activation scale
+    auto fold = [&](int sbp) {
+        const uint8_t *sblk = lds + C::OFF_SBLK + (size_t)sbp * C::SBLK;
+        const u32x4 *sp = reinterpret_cast<const u32x4 *>(sblk + C::OFF_SD) + (r0 + half * 16) / 4;
         const u32x4 s0 = sp[0], s1 = sp[1], s2 = sp[2], s3 = sp[3];
         const uint32_t sd[16] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w, s2.x, s2.y, s2.z, s2.w, s3.x, s3.y, s3.z, s3.w};
+        f16x8 fa[C::NF];
+        if constexpr (T::NF16 > 0) {
+#pragma unroll
+            for (int f = 0; f < T::NF16; f++)
+                fa[f] = *reinterpret_cast<const f16x8 *>(sblk + C::OFF_FA + (size_t)((2 * f + half) * C::BM + r0 + l32) * 16);
+        }
 #pragma unroll
         for (int c = 0; c < TN; c++) {
-            const float dx = reinterpret_cast<const float *>(base + C::OFF_SX)[n0 + c * 32 + l32];
+            f32x16 F[2];
+            if constexpr (T::NF16 > 0) {
+                const f16x8 fb = *reinterpret_cast<const f16x8 *>(sblk + C::OFF_FB + (size_t)(half * C::BN + n0 + c * 32 + l32) * 16);
+                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int f = 0; f < T::NF16; f++) F[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[f], fb, zero, 0, 0, 0);
+            }
+            const float dx = reinterpret_cast<const float *>(sblk + C::OFF_SX)[n0 + c * 32 + l32];
             int corr = 0;
-            if constexpr (T::HAS_BSUM) corr = reinterpret_cast<const int *>(base + C::OFF_SC)[n0 + c * 32 + l32];
+            if constexpr (T::HAS_BSUM) corr = reinterpret_cast<const int *>(sblk + C::OFF_SC)[n0 + c * 32 + l32];
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                int p[T::NACC];
+                float f[2] = {0.f, 0.f};
 #pragma unroll
-                for (int pl = 0; pl < T::NACC; pl++) p[pl] = P[pl][c][v];
-                out[c][v] = __builtin_fmaf(T::value(p, sd[v], corr), dx, out[c][v]);
+                for (int j = 0; j < T::NF16; j++) f[j] = F[j][v];
+                out[c][v] = __builtin_fmaf(T::value(P[0][c][v], P[1][c][v], f, sd[v], corr), dx, out[c][v]);
             }
         }
     };
 
-    fetch(0);
-    commit(0, 0);
-    __syncthreads();
-
+    __syncthreads();                                                    // stage 0 is in LDS
     for (int s = 0; s < nstages; s += 2) {
-        // first half of the super-block (buffer 0), second half (buffer 1)
-        fetch(s + 1);
         compute(0, std::true_type{});
-        commit(s + 1, 1);
         __syncthreads();
-
-        if (s + 2 < nstages) fetch(s + 2);
         compute(1, std::false_type{});
-        finish(1);
-        if (s + 2 < nstages) commit(s + 2, 0);
+        fold((s >> 1) & 1);
         __syncthreads();
     }
 
@@ -413,22 +537,26 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     }
 }
 
+// The GEMM pays off once the token count outweighs its fixed cost of about 2 us per super-block of K: from 16
+// tokens on large matrices, from 32 on small ones (below that the GEMV passes over the weights are faster).
 bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n) {
-    return (wtype == T_Q4_K || wtype == T_Q5_K || wtype == T_Q6_K) && K >= QK_K && K % QK_K == 0 && N >= 1 && n >= 1;
+    if (!(wtype == T_Q4_K || wtype == T_Q5_K || wtype == T_Q6_K) || K < QK_K || K % QK_K != 0 || N < 1) return false;
+    return n >= ((N * K >= (int64_t)48 << 20) ? 16 : 32);
 }
 
 template <int WT, int WR, int WC, int OCC>
 static hipError_t launch_kq(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     using C = KqCfg<WT, WR, WC>;
-    const size_t lds_bytes = 2 * C::STAGE;
+    const size_t lds_bytes = C::TOTAL;
     if ((int64_t)lds_bytes > lim.max_lds_per_block) return hipErrorInvalidValue;
     auto kfn = gemm_kq_kernel<WT, WR, WC, OCC>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
-    dim3 grid((unsigned)ceil_div(N, C::BM), (unsigned)ceil_div(M, C::BN));
-    hipLaunchKernelGGL(kfn, grid, dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws, ws_stride,
-                       M, y, ldy);
+    // one workgroup per CU: 32 workgroups run on an XCD at a time
+    const TileMap map = make_tile_map(ceil_div(N, C::BM), ceil_div(M, C::BN), 32);
+    hipLaunchKernelGGL(kfn, dim3(map.grid), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws,
+                       ws_stride, M, y, ldy, map);
     return hipGetLastError();
 }
 
@@ -436,14 +564,15 @@ template <int WT>
 static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                                  int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    // 128 rows x 128 tokens per workgroup when that gives every CU one, else 64 x 128.  (CHIP_GEMM_KQ_CFG selects a
+    // shape by hand.)
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_KQ_CFG");
-    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
+    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 2);
     switch (cfg) {
-        case 0: return launch_kq<WT, 4, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 128 x 128, 8 waves
-        case 1: return launch_kq<WT, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 64 x 128, 4 waves
-        case 2: return launch_kq<WT, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 64 x 256, 8 waves
-        case 3: return launch_kq<WT, 2, 1, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 64 x 64, 2 waves
+        case 0: return launch_kq<WT, 4, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 128 x 128, 8 + 4 waves
+        case 1: return launch_kq<WT, 4, 1, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 128 x 64, 4 + 4 waves
+        case 2: return launch_kq<WT, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 64 x 128, 4 + 4 waves
         default: return hipErrorInvalidValue;
     }
 }

@@ -72,14 +72,16 @@ template <int TM, int TN, int WR, int WC, int OCC>
 __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_q4_0_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
                                                                 int64_t N, const uint8_t *__restrict__ ws,
                                                                 size_t ws_stride, int64_t M, float *__restrict__ y,
-                                                                int64_t ldy) {
+                                                                int64_t ldy, TileMap map) {
     using C = GemmCfg<TM, TN, WR, WC>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave / WC, wc = wave % WC;
     const int half = lane >> 5, l32 = lane & 31;
-    const int64_t row_base = (int64_t)blockIdx.x * C::BM;
-    const int64_t tok_base = (int64_t)blockIdx.y * C::BN;
+    const TileCoord tc = xcd_tile(blockIdx.x, map);
+    if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;        // padding of the tile map
+    const int64_t row_base = (int64_t)tc.row_tile * C::BM;
+    const int64_t tok_base = (int64_t)tc.tok_tile * C::BN;
     const int nstages = (int)(K / (32 * GEMM_KB));
     const size_t off_d = q8_0_off_d(K);
 
@@ -283,7 +285,12 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         }
 }
 
-bool gemm_q4_0_supported(int64_t K, int64_t N, int64_t n) { return K % (32 * GEMM_KB) == 0 && N >= 1 && n >= 1; }
+// The GEMM has a fixed cost of about 0.35 us per 32-value block of K; below 32 tokens (48 on small matrices) the
+// GEMV passes over the weights are faster.
+bool gemm_q4_0_supported(int64_t K, int64_t N, int64_t n) {
+    if (K % (32 * GEMM_KB) != 0 || N < 1) return false;
+    return n >= ((N * K >= (int64_t)48 << 20) ? 32 : 48);
+}
 
 template <int TM, int TN, int WR, int WC, int OCC>
 static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
@@ -293,9 +300,10 @@ static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, c
     auto kfn = gemm_q4_0_kernel<TM, TN, WR, WC, OCC>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
-    dim3 grid((unsigned)ceil_div(N, C::BM), (unsigned)ceil_div(M, C::BN));
-    hipLaunchKernelGGL(kfn, grid, dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws, ws_stride,
-                       M, y, ldy);
+    // workgroups that share an XCD (OCC waves per SIMD, 32 CUs) take a compact block of output tiles
+    const TileMap map = make_tile_map(ceil_div(N, C::BM), ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
+    hipLaunchKernelGGL(kfn, dim3(map.grid), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws,
+                       ws_stride, M, y, ldy, map);
     return hipGetLastError();
 }
 

@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <atomic>
+#include "dev_common.h"
 
 namespace chip {
 
@@ -25,6 +26,53 @@ template <typename F> inline hipError_t grant_dynamic_lds(F kfn, size_t need, co
     e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lim.max_lds_per_block);
     if (e == hipSuccess) g.devices.fetch_or(bit, std::memory_order_release);
     return e;
+}
+
+// Output-tile order for the GEMM kernels.  The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and each
+// XCD has its own L2.  Tiles are numbered block by block (sr x sc tiles per block, about as many as run on one XCD at a
+// time; blocks at the far edges are smaller), the numbering is cut into 8 equal stretches, and XCD x walks stretch x:
+// workgroup id L -> XCD L % 8, its (L / 8)-th tile.  The workgroups that share an L2 then read the same few weight
+// rows and tokens, every XCD gets the same number of tiles, and no XCD streams the whole weight matrix.
+constexpr int XCDS = 8;
+struct TileMap {
+    int row_tiles, tok_tiles;      // output tiles in each direction
+    int sr, sc;                    // tiles per full block
+    int blocks_r, blocks_c;
+    unsigned tiles, per_xcd;       // tiles in all, tiles per XCD (rounded up)
+    unsigned grid;                 // workgroups to launch; those numbered past the last tile exit at once
+};
+struct TileCoord { int row_tile, tok_tile; };
+inline TileMap make_tile_map(int64_t row_tiles, int64_t tok_tiles, int concurrent_per_xcd) {
+    TileMap m;
+    m.row_tiles = (int)row_tiles;
+    m.tok_tiles = (int)tok_tiles;
+    m.blocks_c = (int)ceil_div(tok_tiles, 8);
+    m.sc = (int)ceil_div(tok_tiles, m.blocks_c);
+    int sr = concurrent_per_xcd / m.sc;
+    if (sr < 1) sr = 1;
+    m.blocks_r = (int)ceil_div(row_tiles, sr);
+    m.sr = (int)ceil_div(row_tiles, m.blocks_r);
+    m.tiles = (unsigned)(row_tiles * tok_tiles);
+    m.per_xcd = (unsigned)ceil_div(m.tiles, XCDS);
+    m.grid = m.per_xcd * XCDS;
+    return m;
+}
+__device__ __forceinline__ TileCoord xcd_tile(unsigned wg, const TileMap &m) {
+    unsigned g = (wg % XCDS) * m.per_xcd + wg / XCDS;
+    TileCoord t;
+    if (wg / XCDS >= m.per_xcd || g >= m.tiles) { t.row_tile = m.row_tiles; t.tok_tile = m.tok_tiles; return t; }
+    const unsigned col_block = (unsigned)(m.row_tiles * m.sc);                  // tiles in a full column of blocks
+    unsigned cb = g / col_block;
+    if (cb > (unsigned)m.blocks_c - 1) cb = m.blocks_c - 1;
+    g -= cb * col_block;
+    const unsigned wc = (cb < (unsigned)m.blocks_c - 1) ? m.sc : m.tok_tiles - (m.blocks_c - 1) * m.sc;
+    unsigned rb = g / (m.sr * wc);
+    if (rb > (unsigned)m.blocks_r - 1) rb = m.blocks_r - 1;
+    g -= rb * m.sr * wc;
+    const unsigned hr = (rb < (unsigned)m.blocks_r - 1) ? m.sr : m.row_tiles - (m.blocks_r - 1) * m.sr;
+    t.row_tile = (int)(rb * m.sr + g % hr);
+    t.tok_tile = (int)(cb * m.sc + g / hr);
+    return t;
 }
 
 // quantize.hip

@@ -39,4 +39,6 @@ def test_layout_queries_need_no_gpu():
     assert lib.chip_mul_mat_supported(cactus_amd.F16, 4096) == 1 and lib.chip_vec_dot_type(cactus_amd.F16) == cactus_amd.F16
     assert lib.chip_mul_mat_supported(30, 4096) == 0          # BF16 weights are not on this path
     assert lib.chip_mul_mat_workspace_size(cactus_amd.Q8_0, 4096, 3) == 3 * (4096 + 12 * 128)   # qs, d, sum, s planes
+    # Q8_K planes (qs, d, bsums) of K = 4096 take 4672 bytes; token strides are multiples of 128
+    assert lib.chip_mul_mat_workspace_size(cactus_amd.Q4_K, 4096, 3) == 3 * 4736
     assert lib.chip_error_string(-2).decode().startswith("unsupported")

@@ -221,7 +221,8 @@ def test_argument_errors(dev):
 
 
 # ------------------------------------------------------------------------------------------ prefill GEMM (int8 MFMA)
-@pytest.mark.parametrize("K,N,n", [(256, 1, 16), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257)])
+@pytest.mark.parametrize("K,N,n", [(256, 1, 48), (512, 40, 49), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
+                                   (4096, 12300, 33)])
 def test_gemm_q4_0_vs_oracle(dev, orc, K, N, n):
     print("gemm q4_0 K", K, "N", N, "n", n, flush=True)
     wq = orc.quantize_weights(O.Q4_0, common.weights_f32(K + N, N, K))
@@ -283,7 +284,8 @@ KQ_TYPES = (O.Q4_K, O.Q5_K, O.Q6_K)
 
 
 @pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N,n", [(256, 1, 16), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257)])
+@pytest.mark.parametrize("K,N,n", [(256, 1, 32), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
+                                   (4096, 12300, 17)])
 def test_gemm_kquant_vs_oracle(dev, orc, wt, K, N, n):
     print("gemm", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
     wq = orc.quantize_weights(wt, common.weights_f32(K + N + wt, N, K, outliers=True))
