@@ -272,8 +272,8 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     const size_t stride = act_stride(chip_vec_dot_type(type), K);
     hipStream_t st = (hipStream_t)stream;
 
-    if (type == T_Q4_0 && gemm_q4_0_supported(K, N, n))
-        return hip_rc(launch_gemm_q4_0(W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
+    if (gemm_blk32_supported(type, K, N, n))
+        return hip_rc(launch_gemm_blk32(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
     if (gemm_kq_supported(type, K, N, n))
         return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
 

@@ -1,14 +1,15 @@
-// Prefill GEMM for gfx950: Y[t][r] = sum_b dw[r][b] * dx[t][b] * isum[t][r][b] over Q4_0 weights and Q8_0
-// activations, the batched form of lm_ggml_vec_dot_q4_0_q8_0 (reference ggml-cpu/ggml-cpu-quants.c:1906-2602)
-// as driven by lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449).
+// Prefill GEMM for gfx950 over weights in 32-value blocks with one fp16 scale each (Q4_0, Q8_0, Q5_0, IQ4_NL) and Q8_0
+// activations: Y[t][r] = sum_b dw[r][b] * dx[t][b] * isum[t][r][b], the batched form of lm_ggml_vec_dot_q4_0_q8_0,
+// _q8_0_q8_0, _q5_0_q8_0 and _iq4_nl_q8_0 (reference ggml-cpu/ggml-cpu-quants.c) as driven by
+// lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449).
 //
 // Structure
 //   * One v_mfma_i32_32x32x32_i8 multiplies a 32-row x 32-k weight tile by a 32-k x 32-token activation tile:
 //     its K extent is exactly one 32-value quantization block, so each of the 1024 int32 results is one
 //     per-block integer sum isum[t][r][b], bit-exact.
-//   * Weight tiles are staged through LDS once per workgroup and k-stage: the Q4_0 nibbles are split into the
-//     low-nibble half (elements 0..15) and the high-nibble half (16..31) and turned into signed int8
-//     16 * (nib - 8), the 16 being undone by the activation scale;
+//   * Weight tiles are staged through LDS once per workgroup and k-stage: a block's packed quants are expanded into
+//     two 16-byte cells of signed int8 (elements 0..15 and 16..31), possibly times a power of two that the
+//     activation scale takes back (Q4_0: 16 * (nib - 8), Q5_0: 8 * (q - 16); IQ4_NL: the code point; Q8_0: as is);
 //     activations arrive as int8 from the split workspace layout.  Both sit in LDS as [k-block][half][row]
 //     16-byte cells, which is exactly what one lane feeds the MFMA (row = lane % 32, half = lane / 32).
 //   * Per-block scales are applied in fp32 after the integer accumulate.  The MFMA's C input is a register
@@ -37,12 +38,80 @@ constexpr int GEMM_KB = 4;                    // 32-value blocks per LDS stage
 constexpr float MAGIC_F = 12582912.f;         // 1.5 * 2^23
 constexpr int MAGIC_I = 0x4B400000;
 
-// The weight operand holds 16 * (nibble - 8): a nibble moved to the high half of its byte with its top bit flipped
-// is that number as a signed byte (two or three operations per dword instead of four); the factor 16 is taken
-// back through the activation scale (dx / 16 is exact), and |16 * isum| <= 16 * 32 * 8 * 127 < 2^22 still fits
-// the magic-constant conversion.
-__device__ __forceinline__ uint32_t lo_nib_x16(uint32_t q) { return ((q << 4) & 0xf0f0f0f0u) ^ 0x80808080u; }
-__device__ __forceinline__ uint32_t hi_nib_x16(uint32_t q) { return (q & 0xf0f0f0f0u) ^ 0x80808080u; }
+// How a weight type's block becomes two MFMA operand cells.  MULT is the power of two the cells carry on top of the
+// quant (taken back through the activation scale, exactly); MULT * |isum| stays below 2^22 for every type.
+template <int WT> struct Blk32;
+
+template <> struct Blk32<T_Q4_0> {
+    static constexpr int BYTES = BYTES_Q4_0;
+    static constexpr float INV_MULT = 1.f / 16.f;
+    struct Raw { u32x4 q; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) { r.q = *reinterpret_cast<const u32x4_a2 *>(p + 2); }
+    // a nibble moved to the high half of its byte with its top bit flipped is 16 * (nibble - 8) as a signed byte
+    __device__ static __forceinline__ void emit(const Raw &r, u32x4 &lo, u32x4 &hi) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            lo[i] = ((r.q[i] << 4) & 0xf0f0f0f0u) ^ 0x80808080u;
+            hi[i] = (r.q[i] & 0xf0f0f0f0u) ^ 0x80808080u;
+        }
+    }
+};
+
+template <> struct Blk32<T_IQ4_NL> {
+    static constexpr int BYTES = BYTES_IQ4_NL;
+    static constexpr float INV_MULT = 1.f;
+    using Raw = Blk32<T_Q4_0>::Raw;
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) { Blk32<T_Q4_0>::fetch(r, p); }
+    // four code indices (one per byte, 0..15) -> four code points of kvalues_iq4nl (reference ggml-common.h), through
+    // two byte permutes of the 16-entry table
+    __device__ static __forceinline__ uint32_t lookup4(uint32_t idx) {
+        constexpr uint32_t T0 = 0xbfad9881u, T1 = 0xf6eaddcfu, T2 = 0x26190d01u, T3 = 0x71594535u;
+        const uint32_t sel = idx & 0x07070707u;
+        const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel), hi = __builtin_amdgcn_perm(T3, T2, sel);
+        const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xffu;
+        return (lo & ~m) | (hi & m);
+    }
+    __device__ static __forceinline__ void emit(const Raw &r, u32x4 &lo, u32x4 &hi) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            lo[i] = lookup4(r.q[i] & 0x0f0f0f0fu);
+            hi[i] = lookup4((r.q[i] >> 4) & 0x0f0f0f0fu);
+        }
+    }
+};
+
+template <> struct Blk32<T_Q8_0> {
+    static constexpr int BYTES = BYTES_Q8_0;
+    static constexpr float INV_MULT = 1.f;
+    struct Raw { u32x4 lo, hi; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) {
+        r.lo = *reinterpret_cast<const u32x4_a2 *>(p + 2);
+        r.hi = *reinterpret_cast<const u32x4_a2 *>(p + 18);
+    }
+    __device__ static __forceinline__ void emit(const Raw &r, u32x4 &lo, u32x4 &hi) { lo = r.lo; hi = r.hi; }
+};
+
+template <> struct Blk32<T_Q5_0> {
+    static constexpr int BYTES = BYTES_Q5_0;
+    static constexpr float INV_MULT = 1.f / 8.f;
+    struct Raw { u32x4 q; uint32_t qh; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) {
+        r.qh = *reinterpret_cast<const u32_a2 *>(p + 2);
+        r.q = *reinterpret_cast<const u32x4_a2 *>(p + 6);
+    }
+    // element j < 16: low nibble of qs[j] with bit j of qh on top, element 16 + j: high nibble with bit 16 + j
+    // (reference ggml-quants.c:290-310).  The cell byte is 8 * (q - 16): q << 3 with the top bit flipped.
+    __device__ static __forceinline__ void emit(const Raw &r, u32x4 &lo, u32x4 &hi) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            // 4 bits -> bit 0 of each byte: bit k lands at 7k + k = 8k
+            const uint32_t bl = (((r.qh >> (4 * i)) & 0xfu) * 0x00204081u) & 0x01010101u;
+            const uint32_t bh = (((r.qh >> (16 + 4 * i)) & 0xfu) * 0x00204081u) & 0x01010101u;
+            lo[i] = (((r.q[i] << 3) & 0x78787878u) | (bl << 7)) ^ 0x80808080u;
+            hi[i] = (((r.q[i] >> 1) & 0x78787878u) | (bh << 7)) ^ 0x80808080u;
+        }
+    }
+};
 
 template <int TM, int TN, int WR, int WC>
 struct GemmCfg {
@@ -68,12 +137,13 @@ struct GemmCfg {
     static constexpr int S_PER_T = (S_ITEMS + NT - 1) / NT;
 };
 
-template <int TM, int TN, int WR, int WC, int OCC>
-__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_q4_0_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
+template <int WT, int TM, int TN, int WR, int WC, int OCC>
+__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_blk32_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
                                                                 int64_t N, const uint8_t *__restrict__ ws,
                                                                 size_t ws_stride, int64_t M, float *__restrict__ y,
                                                                 int64_t ldy, TileMap map) {
     using C = GemmCfg<TM, TN, WR, WC>;
+    using T = Blk32<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave / WC, wc = wave % WC;
@@ -86,7 +156,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
     const size_t off_d = q8_0_off_d(K);
 
     // ---- per-thread prefetch registers for one stage ----
-    u32x4 wq[C::W_PER_T];
+    typename T::Raw wq[C::W_PER_T];
     uint32_t wd[C::W_PER_T];
     u32x4 xq[C::X_PER_T];
     float xs[C::S_PER_T];
@@ -99,9 +169,9 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
             if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
                 const int r = item / GEMM_KB, b = item % GEMM_KB;
                 const int64_t row = min(row_base + r, N - 1);
-                const uint8_t *p = W + (size_t)row * nb01 + (size_t)(kb0 + b) * BYTES_Q4_0;
+                const uint8_t *p = W + (size_t)row * nb01 + (size_t)(kb0 + b) * T::BYTES;
                 wd[i] = *reinterpret_cast<const unsigned short *>(p);
-                wq[i] = *reinterpret_cast<const u32x4_a2 *>(p + 2);
+                T::fetch(wq[i], p);
             }
         }
 #pragma unroll
@@ -136,10 +206,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
             if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
                 const int r = item / GEMM_KB, b = item % GEMM_KB;
                 u32x4 lo, hi;
-                lo.x = lo_nib_x16(wq[i].x); hi.x = hi_nib_x16(wq[i].x);
-                lo.y = lo_nib_x16(wq[i].y); hi.y = hi_nib_x16(wq[i].y);
-                lo.z = lo_nib_x16(wq[i].z); hi.z = hi_nib_x16(wq[i].z);
-                lo.w = lo_nib_x16(wq[i].w); hi.w = hi_nib_x16(wq[i].w);
+                T::emit(wq[i], lo, hi);
                 A[(b * 2 + 0) * C::A_PLANE + r] = lo;
                 A[(b * 2 + 1) * C::A_PLANE + r] = hi;
                 // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4;
@@ -162,7 +229,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
             const int item = tid + i * C::NT;
             if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
                 const int b = item % GEMM_KB, n = item / GEMM_KB;
-                SX[b * C::BN + n] = xs[i] * 0.0625f;                       // takes back the 16 of the weight operand
+                SX[b * C::BN + n] = xs[i] * T::INV_MULT;                   // takes back the power of two in the weight cells
             }
         }
     };
@@ -287,17 +354,18 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
 
 // The GEMM has a fixed cost of about 0.35 us per 32-value block of K; below 32 tokens (48 on small matrices) the
 // GEMV passes over the weights are faster.
-bool gemm_q4_0_supported(int64_t K, int64_t N, int64_t n) {
+bool gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n) {
+    if (!(wtype == T_Q4_0 || wtype == T_Q8_0 || wtype == T_Q5_0 || wtype == T_IQ4_NL)) return false;
     if (K % (32 * GEMM_KB) != 0 || N < 1) return false;
     return n >= ((N * K >= (int64_t)48 << 20) ? 32 : 48);
 }
 
-template <int TM, int TN, int WR, int WC, int OCC>
+template <int WT, int TM, int TN, int WR, int WC, int OCC>
 static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     using C = GemmCfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
-    auto kfn = gemm_q4_0_kernel<TM, TN, WR, WC, OCC>;
+    auto kfn = gemm_blk32_kernel<WT, TM, TN, WR, WC, OCC>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     // workgroups that share an XCD (OCC waves per SIMD, 32 CUs) take a compact block of output tiles
@@ -307,22 +375,30 @@ static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, c
     return hipGetLastError();
 }
 
-hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (M <= 0 || N <= 0) return hipSuccess;
+template <int WT>
+static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
+                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
     // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
     // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_CFG");
-    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 6);
+    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
     switch (cfg) {
-        case 0: return launch_cfg<1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 1: return launch_cfg<1, 2, 2, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 2: return launch_cfg<2, 2, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 3: return launch_cfg<2, 2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 5: return launch_cfg<2, 1, 2, 4, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 6: return launch_cfg<1, 1, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 0: return launch_cfg<WT, 1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 1: return launch_cfg<WT, 1, 1, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                             int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    if (M <= 0 || N <= 0) return hipSuccess;
+    switch (wtype) {
+        case T_Q4_0:   return launch_type<T_Q4_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_Q8_0:   return launch_type<T_Q8_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_Q5_0:   return launch_type<T_Q5_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_IQ4_NL: return launch_type<T_IQ4_NL>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }

@@ -100,10 +100,11 @@ int        mmv_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &l
 hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                       int n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 
-// gemm_q4_0.hip: int8-MFMA prefill GEMM over Q4_0 weights, activations in the split Q8_0 workspace layout.
-bool       gemm_q4_0_supported(int64_t K, int64_t N, int64_t n);
-hipError_t launch_gemm_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                            int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+// gemm_block32.hip: int8-MFMA prefill GEMM over weights in 32-value blocks with one fp16 scale (Q4_0, Q8_0, Q5_0,
+// IQ4_NL), activations in the split Q8_0 workspace layout.  _supported includes the token count from which it pays.
+bool       gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n);
+hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                             int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 
 // gemm_kquant.hip: int8-MFMA prefill GEMM over Q4_K / Q5_K / Q6_K weights, activations in the split Q8_K workspace
 // layout; the integer sub-block scales ride in the MFMA operand.

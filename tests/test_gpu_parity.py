@@ -221,39 +221,46 @@ def test_argument_errors(dev):
 
 
 # ------------------------------------------------------------------------------------------ prefill GEMM (int8 MFMA)
+B32_TYPES = (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL)
+
+
+@pytest.mark.parametrize("wt", B32_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N,n", [(256, 1, 48), (512, 40, 49), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
                                    (4096, 12300, 33)])
-def test_gemm_q4_0_vs_oracle(dev, orc, K, N, n):
-    print("gemm q4_0 K", K, "N", N, "n", n, flush=True)
-    wq = orc.quantize_weights(O.Q4_0, common.weights_f32(K + N, N, K))
+def test_gemm_block32_vs_oracle(dev, orc, wt, K, N, n):
+    print("gemm", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
+    wq = orc.quantize_weights(wt, common.weights_f32(K + N, N, K))
     x = common.activations_f32(K + n, n, K)
     x[3] = 0
-    ref = orc.mul_mat(O.Q4_0, wq, x, nthreads=8, want=("wdata", "sum_abs"))
-    y, blocks = dev.mul_mat(O.Q4_0, wq, x, want_workspace_blocks=True)
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(wt, wq, x, want_workspace_blocks=True)
     assert np.array_equal(blocks, ref["wdata"])
     check_outputs(y, ref["y"], ref["sum_abs"], "gemm")
 
 
-def test_gemm_q4_0_integer_sums_bit_exact(dev, orc):
+@pytest.mark.parametrize("wt", B32_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+def test_gemm_block32_integer_sums_bit_exact(dev, orc, wt):
     """With every scale equal to 1 the fp32 output is the integer sum itself, so the MFMA path's per-block
-    integer dot sums can be compared bit for bit: one block at a time (all other weight scales zero), then all."""
+    integer dot sums can be compared bit for bit: one block at a time (all other weight scales zero), then all.
+    The weight bytes are random, so every nibble / fifth bit / code index / int8 value occurs."""
     K, N, n = 256, 70, 48
-    rng = np.random.default_rng(9)
+    rng = np.random.default_rng(9 + wt)
+    bb = O.BLOCK_BYTES[wt]
     x = rng.integers(-127, 128, (n, K)).astype(np.float32)
     x[:, ::32] = 127.0                                   # amax = 127 in every block -> d = 1, q = x
     x[5, 64:96] = 0.0                                    # one all-zero activation block
     aq = orc.quantize_activation(O.Q8_0, x)
     for only in list(range(K // 32)) + [None]:
-        w = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+        w = rng.integers(0, 256, (N, K // 32, bb), dtype=np.uint8)
         w[..., :2] = 0
         sel = slice(None) if only is None else only
         w[:, sel, :2] = np.array([1.0], np.float16).view(np.uint8)
         w = w.reshape(N, -1)
-        y = dev.mul_mat(O.Q4_0, w, x)
+        y = dev.mul_mat(wt, w, x)
         want = np.zeros((n, N), np.int64)
         for t in range(n):
             for i in range(N):
-                _, isum, _ = orc.vec_dot(O.Q4_0, K, w[i], aq[t], want_sums=True)
+                _, isum, _ = orc.vec_dot(wt, K, w[i], aq[t], want_sums=True)
                 want[t, i] = isum.sum() if only is None else isum[only]
         assert np.array_equal(y.astype(np.int64), want) and np.array_equal(y, want.astype(np.float32))
 
