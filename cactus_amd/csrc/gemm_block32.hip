@@ -1,5 +1,5 @@
-// Prefill GEMM for gfx950 over weights in 32-value blocks with one fp16 scale each (Q4_0, Q8_0, Q5_0, IQ4_NL) and Q8_0
-// activations: Y[t][r] = sum_b dw[r][b] * dx[t][b] * isum[t][r][b], the batched form of lm_ggml_vec_dot_q4_0_q8_0,
+// Prefill GEMM for gfx950 over weights in 32-value blocks with one fp16 scale each (Q4_0, Q8_0, Q5_0, IQ4_NL; Q4_1 and
+// Q5_1 with a minimum on top) and Q8_0 / Q8_1 activations: Y[t][r] = sum_b dw[r][b] * dx[t][b] * isum[t][r][b], the batched form of lm_ggml_vec_dot_q4_0_q8_0,
 // _q8_0_q8_0, _q5_0_q8_0 and _iq4_nl_q8_0 (reference ggml-cpu/ggml-cpu-quants.c) as driven by
 // lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449).
 //
@@ -21,6 +21,9 @@
 //     i.e. two VALU operations per integer sum, 32 per MFMA.  That VALU work, not the matrix pipe, bounds this
 //     kernel: an MFMA occupies the matrix unit for 32 cycles, 32 wave-wide fp32 operations occupy the vector
 //     unit for 128.
+//   * Q4_1 and Q5_1 add m * s per block (the weight block's minimum times the activation block's d * sum, the s of
+//     block_q8_1).  Both factors are fp16 numbers, so sum_b m[r][b] * s[t][b] over the 4 blocks of a stage is one
+//     v_mfma_f32_32x32x8f16 that adds straight into the fp32 accumulators: no vector work.
 //   * A workgroup is WR x WC waves, each wave owns TM x TN MFMA tiles (32*TM rows x 32*TN tokens); LDS is
 //     double buffered over stages of KB = 4 blocks with one barrier per stage and the next stage's global
 //     loads in flight during the current stage's arithmetic.
@@ -33,6 +36,8 @@ namespace chip {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GEMM_KB = 4;                    // 32-value blocks per LDS stage
 constexpr float MAGIC_F = 12582912.f;         // 1.5 * 2^23
@@ -44,6 +49,7 @@ template <int WT> struct Blk32;
 
 template <> struct Blk32<T_Q4_0> {
     static constexpr int BYTES = BYTES_Q4_0;
+    static constexpr bool HAS_MIN = false;
     static constexpr float INV_MULT = 1.f / 16.f;
     struct Raw { u32x4 q; };
     __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) { r.q = *reinterpret_cast<const u32x4_a2 *>(p + 2); }
@@ -59,6 +65,7 @@ template <> struct Blk32<T_Q4_0> {
 
 template <> struct Blk32<T_IQ4_NL> {
     static constexpr int BYTES = BYTES_IQ4_NL;
+    static constexpr bool HAS_MIN = false;
     static constexpr float INV_MULT = 1.f;
     using Raw = Blk32<T_Q4_0>::Raw;
     __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) { Blk32<T_Q4_0>::fetch(r, p); }
@@ -82,6 +89,7 @@ template <> struct Blk32<T_IQ4_NL> {
 
 template <> struct Blk32<T_Q8_0> {
     static constexpr int BYTES = BYTES_Q8_0;
+    static constexpr bool HAS_MIN = false;
     static constexpr float INV_MULT = 1.f;
     struct Raw { u32x4 lo, hi; };
     __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) {
@@ -93,6 +101,7 @@ template <> struct Blk32<T_Q8_0> {
 
 template <> struct Blk32<T_Q5_0> {
     static constexpr int BYTES = BYTES_Q5_0;
+    static constexpr bool HAS_MIN = false;
     static constexpr float INV_MULT = 1.f / 8.f;
     struct Raw { u32x4 q; uint32_t qh; };
     __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) {
@@ -113,6 +122,42 @@ template <> struct Blk32<T_Q5_0> {
     }
 };
 
+// Q4_1 / Q5_1: unsigned quants, block = d, m (fp16), [qh,] qs; value = d * q + m
+template <> struct Blk32<T_Q4_1> {
+    static constexpr int BYTES = BYTES_Q4_1;
+    static constexpr bool HAS_MIN = true;
+    static constexpr float INV_MULT = 1.f / 8.f;
+    struct Raw { u32x4 q; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) { r.q = *reinterpret_cast<const u32x4_a4 *>(p + 4); }
+    __device__ static __forceinline__ void emit(const Raw &r, u32x4 &lo, u32x4 &hi) {      // 8 * nibble, 0..120
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            lo[i] = (r.q[i] << 3) & 0x78787878u;
+            hi[i] = (r.q[i] >> 1) & 0x78787878u;
+        }
+    }
+};
+
+template <> struct Blk32<T_Q5_1> {
+    static constexpr int BYTES = BYTES_Q5_1;
+    static constexpr bool HAS_MIN = true;
+    static constexpr float INV_MULT = 1.f / 4.f;
+    struct Raw { u32x4 q; uint32_t qh; };
+    __device__ static __forceinline__ void fetch(Raw &r, const uint8_t *p) {
+        r.qh = *reinterpret_cast<const uint32_t *>(p + 4);
+        r.q = *reinterpret_cast<const u32x4_a4 *>(p + 8);
+    }
+    __device__ static __forceinline__ void emit(const Raw &r, u32x4 &lo, u32x4 &hi) {      // 4 * q, 0..124
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t bl = (((r.qh >> (4 * i)) & 0xfu) * 0x00204081u) & 0x01010101u;
+            const uint32_t bh = (((r.qh >> (16 + 4 * i)) & 0xfu) * 0x00204081u) & 0x01010101u;
+            lo[i] = ((r.q[i] << 2) & 0x3c3c3c3cu) | (bl << 6);
+            hi[i] = ((r.q[i] >> 2) & 0x3c3c3c3cu) | (bh << 6);
+        }
+    }
+};
+
 template <int TM, int TN, int WR, int WC>
 struct GemmCfg {
     static constexpr int NW = WR * WC, NT = NW * 64;
@@ -128,7 +173,9 @@ struct GemmCfg {
     static constexpr size_t OFF_B = OFF_A + (size_t)A_CELLS * 16;
     static constexpr size_t OFF_SW = OFF_B + (size_t)B_CELLS * 16;                 // fp16 [KB][BM], permuted per 32 rows
     static constexpr size_t OFF_SX = OFF_SW + (size_t)GEMM_KB * BM * 2;            // fp32 [KB][BN]
-    static constexpr size_t STAGE = OFF_SX + (size_t)GEMM_KB * BN * 4;
+    static constexpr size_t OFF_MW = OFF_SX + (size_t)GEMM_KB * BN * 4;            // fp16 [BM][KB]: block minimum (Q4_1, Q5_1)
+    static constexpr size_t OFF_MX = OFF_MW + (size_t)BM * GEMM_KB * 2;            // fp16 [BN][KB]: block_q8_1.s
+    static constexpr size_t STAGE = OFF_MX + (size_t)BN * GEMM_KB * 2;
     static constexpr int W_ITEMS = BM * GEMM_KB;                   // (row, block) pairs per stage
     static constexpr int W_PER_T = (W_ITEMS + NT - 1) / NT;
     static constexpr int X_ITEMS = BN * GEMM_KB * 2;               // 16-byte activation cells per stage
@@ -160,6 +207,8 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
     uint32_t wd[C::W_PER_T];
     u32x4 xq[C::X_PER_T];
     float xs[C::S_PER_T];
+    float xm[C::S_PER_T];                         // block_q8_1.s, for the types with a minimum
+    const size_t off_s = q8_0_off_s(K);
 
     auto fetch = [&](int stage) {
         const int64_t kb0 = (int64_t)stage * GEMM_KB;
@@ -170,7 +219,8 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
                 const int r = item / GEMM_KB, b = item % GEMM_KB;
                 const int64_t row = min(row_base + r, N - 1);
                 const uint8_t *p = W + (size_t)row * nb01 + (size_t)(kb0 + b) * T::BYTES;
-                wd[i] = *reinterpret_cast<const unsigned short *>(p);
+                if constexpr (T::HAS_MIN) wd[i] = *reinterpret_cast<const uint32_t *>(p);          // d | m << 16
+                else wd[i] = *reinterpret_cast<const unsigned short *>(p);
                 T::fetch(wq[i], p);
             }
         }
@@ -190,6 +240,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
                 const int b = item % GEMM_KB, n = item / GEMM_KB;
                 const int64_t tok = min(tok_base + n, M - 1);
                 xs[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_d)[kb0 + b];
+                if constexpr (T::HAS_MIN) xm[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_s)[kb0 + b];
             }
         }
     };
@@ -214,6 +265,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
                 const int i32 = r & 31;
                 const int pos = ((i32 >> 2) & 1) * 16 + (i32 >> 3) * 4 + (i32 & 3);
                 SW[b * C::BM + (r & ~31) + pos] = (unsigned short)wd[i];
+                if constexpr (T::HAS_MIN) reinterpret_cast<unsigned short *>(base + C::OFF_MW)[r * GEMM_KB + b] = (unsigned short)(wd[i] >> 16);
             }
         }
 #pragma unroll
@@ -230,11 +282,12 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
             if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
                 const int b = item % GEMM_KB, n = item / GEMM_KB;
                 SX[b * C::BN + n] = xs[i] * T::INV_MULT;                   // takes back the power of two in the weight cells
+                if constexpr (T::HAS_MIN) reinterpret_cast<unsigned short *>(base + C::OFF_MX)[n * GEMM_KB + b] = f2h_rne(xm[i]);   // exact: s is an fp16 number
             }
         }
     };
 
-    float acc[TM][TN][16];
+    f32x16 acc[TM][TN];
 #pragma unroll
     for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -266,6 +319,24 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         const u32x4 *SW = reinterpret_cast<const u32x4 *>(base + C::OFF_SW);
         const float *SX = reinterpret_cast<const float *>(base + C::OFF_SX);
 
+        if constexpr (T::HAS_MIN) {
+            // sum over the stage's 4 blocks of m[row][b] * s[token][b]: k = 0..3 live in lanes 0..31, k = 4..7 are zero
+            f16x4 ma[TM], sb[TN];
+#pragma unroll
+            for (int a = 0; a < TM; a++) {
+                const u32x2 t = reinterpret_cast<const u32x2 *>(base + C::OFF_MW)[(wr * TM + a) * 32 + l32];
+                ma[a] = __builtin_bit_cast(f16x4, half ? u32x2{0u, 0u} : t);
+            }
+#pragma unroll
+            for (int c = 0; c < TN; c++) {
+                const u32x2 t = reinterpret_cast<const u32x2 *>(base + C::OFF_MX)[(wc * TN + c) * 32 + l32];
+                sb[c] = __builtin_bit_cast(f16x4, half ? u32x2{0u, 0u} : t);
+            }
+#pragma unroll
+            for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int c = 0; c < TN; c++) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x8f16(ma[a], sb[c], acc[a][c], 0, 0, 0);
+        }
 #pragma unroll 1
         for (int b = 0; b < GEMM_KB; b++) {
             i32x4 af[TM], bf[TN];
@@ -355,7 +426,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
 // The GEMM has a fixed cost of about 0.35 us per 32-value block of K; below 32 tokens (48 on small matrices) the
 // GEMV passes over the weights are faster.
 bool gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n) {
-    if (!(wtype == T_Q4_0 || wtype == T_Q8_0 || wtype == T_Q5_0 || wtype == T_IQ4_NL)) return false;
+    if (!(wtype == T_Q4_0 || wtype == T_Q8_0 || wtype == T_Q5_0 || wtype == T_IQ4_NL || wtype == T_Q4_1 || wtype == T_Q5_1)) return false;
     if (K % (32 * GEMM_KB) != 0 || N < 1) return false;
     return n >= ((N * K >= (int64_t)48 << 20) ? 32 : 48);
 }
@@ -399,6 +470,8 @@ hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, i
         case T_Q8_0:   return launch_type<T_Q8_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         case T_Q5_0:   return launch_type<T_Q5_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         case T_IQ4_NL: return launch_type<T_IQ4_NL>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_Q4_1:   return launch_type<T_Q4_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_Q5_1:   return launch_type<T_Q5_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
 }

@@ -221,7 +221,7 @@ def test_argument_errors(dev):
 
 
 # ------------------------------------------------------------------------------------------ prefill GEMM (int8 MFMA)
-B32_TYPES = (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL)
+B32_TYPES = (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL, O.Q4_1, O.Q5_1)
 
 
 @pytest.mark.parametrize("wt", B32_TYPES, ids=lambda t: O.TYPE_NAMES[t])
@@ -250,9 +250,12 @@ def test_gemm_block32_integer_sums_bit_exact(dev, orc, wt):
     x[:, ::32] = 127.0                                   # amax = 127 in every block -> d = 1, q = x
     x[5, 64:96] = 0.0                                    # one all-zero activation block
     aq = orc.quantize_activation(O.Q8_0, x)
+    aq1 = orc.quantize_activation(O.Q8_1, x)
     for only in list(range(K // 32)) + [None]:
         w = rng.integers(0, 256, (N, K // 32, bb), dtype=np.uint8)
         w[..., :2] = 0
+        if wt in (O.Q4_1, O.Q5_1):
+            w[..., 2:4] = 0                              # block minimum 0: the output is the integer sums alone
         sel = slice(None) if only is None else only
         w[:, sel, :2] = np.array([1.0], np.float16).view(np.uint8)
         w = w.reshape(N, -1)
@@ -260,7 +263,7 @@ def test_gemm_block32_integer_sums_bit_exact(dev, orc, wt):
         want = np.zeros((n, N), np.int64)
         for t in range(n):
             for i in range(N):
-                _, isum, _ = orc.vec_dot(wt, K, w[i], aq[t], want_sums=True)
+                _, isum, _ = orc.vec_dot(wt, K, w[i], aq1[t] if wt in (O.Q4_1, O.Q5_1) else aq[t], want_sums=True)
                 want[t, i] = isum.sum() if only is None else isum[only]
         assert np.array_equal(y.astype(np.int64), want) and np.array_equal(y, want.astype(np.float32))
 
