@@ -274,6 +274,8 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
 
     if (gemm_blk32_supported(type, K, N, n))
         return hip_rc(launch_gemm_blk32(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
+    if (type == T_F16 && gemm_f16_supported(K, N, n))
+        return hip_rc(launch_gemm_f16(W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
     if (gemm_kq_supported(type, K, N, n))
         return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
 

@@ -106,6 +106,11 @@ bool       gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n);
 hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                              int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 
+// gemm_f16.hip: fp16-MFMA prefill GEMM over F16 weights, activations as fp16 in the workspace.
+bool       gemm_f16_supported(int64_t K, int64_t N, int64_t n);
+hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t n,
+                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+
 // gemm_kquant.hip: int8-MFMA prefill GEMM over Q4_K / Q5_K / Q6_K weights, activations in the split Q8_K workspace
 // layout; the integer sub-block scales ride in the MFMA operand.
 bool       gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n);

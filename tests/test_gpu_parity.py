@@ -289,6 +289,31 @@ def test_config4_prefill_sampled(dev, orc, N, M):
     assert np.array_equal(y2[:, ::-1], y[:64])
 
 
+@pytest.mark.parametrize("K,N,n", [(256, 1, 32), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257), (64, 70, 40)])
+def test_gemm_f16_vs_oracle(dev, orc, K, N, n):
+    print("gemm f16 K", K, "N", N, "n", n, flush=True)
+    if K % 256:
+        pytest.skip("the C-ABI takes K in multiples of 256")
+    wq = orc.quantize_weights(O.F16, common.weights_f32(K + N, N, K, outliers=True))
+    x = common.activations_f32(K + n, n, K)
+    x[3] = 0
+    ref = orc.mul_mat(O.F16, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(O.F16, wq, x, want_workspace_blocks=True)
+    assert np.array_equal(blocks, ref["wdata"])
+    check_outputs(y, ref["y"], ref["sum_abs"], "f16 gemm")
+
+
+def test_gemm_f16_exact_small_integers(dev, orc):
+    """Small integer weights and activations: every product and partial sum is an integer below 2^24, so the fp16 MFMA
+    with fp32 accumulation must give the exact dot products whatever its summation order."""
+    K, N, n = 512, 100, 64
+    rng = np.random.default_rng(3)
+    w = rng.integers(-64, 65, (N, K)).astype(np.float32)
+    x = rng.integers(-64, 65, (n, K)).astype(np.float32)
+    y = dev.mul_mat(O.F16, w.astype(np.float16).view(np.uint8).reshape(N, -1), x)
+    assert np.array_equal(y, x @ w.T)
+
+
 # ------------------------------------------------------------------------------------------ K-quant prefill GEMM
 KQ_TYPES = (O.Q4_K, O.Q5_K, O.Q6_K)
 
