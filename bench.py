@@ -27,6 +27,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
+F16_PEAK_TFLOPS = 2500.0       # MI355X published dense fp16 MFMA rate
 # HBM bytes per launch of the n = 1 Q8_0 GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a device-to-device copy of known size (profiles/gemv_q8_0_n1_hbm_traffic_pmc.md): mean of the
 # two headline shapes.  Algorithmic bytes per launch: 47 967 232.
@@ -79,13 +80,15 @@ def synth_weights(dev, wtype, N, K, rng):
     be, bb = L.chip_block_elems(wtype), L.chip_block_bytes(wtype)
     w = rng.integers(0, 256, (N, K // be, bb), dtype=np.uint8)
     d = np.array([0.0107], np.float16).view(np.uint8)
-    if wtype in (2, 8):
-        w[..., 0:2] = d
-    elif wtype == 12:
-        w[..., 0:2] = d
-        w[..., 2:4] = d
-    else:
+    import cactus_amd as ca
+    if wtype == ca.F16:
+        return rng.standard_normal((N, K)).astype(np.float16).view(np.uint8).reshape(N, -1)
+    if wtype == ca.Q6_K:
         w[..., 208:210] = d
+    else:
+        w[..., 0:2] = d                                   # d first in every other block format
+        if wtype in (ca.Q4_K, ca.Q5_K, ca.Q4_1, ca.Q5_1):
+            w[..., 2:4] = d                               # dmin / m follow it
     return w.reshape(N, -1)
 
 
@@ -211,24 +214,30 @@ def bench_extra(dev, hip):
     gemv_case("config1_q4_0_4096x4096_n1", ca.Q4_0, 4096, 4096, 1)
     gemv_case("config3_q4_K_14336x4096_n1", ca.Q4_K, 14336, 4096, 1)
 
-    # config 4: prefill GEMM on int8 MFMA
-    for (N, M) in ((4096, 512), (4096, 2048), (14336, 512), (14336, 2048)):
-        K = 4096
-        w = dev.to_device(synth_weights(dev, ca.Q4_0, N, K, rng))
+    # config 4: prefill GEMM on int8 MFMA (Q4_0 is the configuration BASELINE names; the other weight types run the
+    # same shapes through their own GEMM kernels: block-32 types, K-quants with digit-plane operands, F16 on fp16 MFMA)
+    def gemm_case(key, wt, N, M, K=4096):
+        w = dev.to_device(synth_weights(dev, wt, N, K, rng))
         x = dev.to_device(rng.standard_normal((M, K)).astype(np.float32))
         y = dev.alloc(M * N * 4)
-        wsz = L.chip_mul_mat_workspace_size(ca.Q4_0, K, M)
+        wsz = L.chip_mul_mat_workspace_size(wt, K, M)
         ws = dev.alloc(wsz)
-        nb01 = dev.row_size(ca.Q4_0, K)
-        dev.check(L.chip_mul_mat_prepare(ca.Q4_0, K, x.ptr, K, M, ws.ptr, wsz, st))
-        us_g = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run(ca.Q4_0, w.ptr, nb01, K, N, M, ws.ptr, y.ptr, N, st), 20)
-        us_o = time_runs(dev, hip, st, lambda: L.chip_mul_mat(ca.Q4_0, w.ptr, nb01, K, N, x.ptr, K, M, y.ptr, N, ws.ptr, wsz, st), 20)
+        nb01 = dev.row_size(wt, K)
+        dev.check(L.chip_mul_mat_prepare(wt, K, x.ptr, K, M, ws.ptr, wsz, st))
+        us_g = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run(wt, w.ptr, nb01, K, N, M, ws.ptr, y.ptr, N, st), 20)
+        us_o = time_runs(dev, hip, st, lambda: L.chip_mul_mat(wt, w.ptr, nb01, K, N, x.ptr, K, M, y.ptr, N, ws.ptr, wsz, st), 20)
         ops = 2.0 * M * N * K
-        out["config4_q4_0_%dx4096_M%d" % (N, M)] = {
-            "us_gemm": round(us_g, 1), "us_op": round(us_o, 1), "TOPS_gemm": round(ops / us_g / 1e6, 1),
-            "TOPS_op": round(ops / us_o / 1e6, 1), "int8_frac_gemm": round(ops / us_g / 1e6 / INT8_PEAK_TOPS, 4)}
+        peak = F16_PEAK_TFLOPS if wt == ca.F16 else INT8_PEAK_TOPS
+        out[key] = {"us_gemm": round(us_g, 1), "us_op": round(us_o, 1), "TOPS_gemm": round(ops / us_g / 1e6, 1),
+                    "TOPS_op": round(ops / us_o / 1e6, 1), "mfma_frac_gemm": round(ops / us_g / 1e6 / peak, 4)}
         for b in (w, x, y, ws):
             b.free()
+
+    for (N, M) in ((4096, 512), (4096, 2048), (14336, 512), (14336, 2048)):
+        gemm_case("config4_q4_0_%dx4096_M%d" % (N, M), ca.Q4_0, N, M)
+    for wt in (ca.Q8_0, ca.Q4_K, ca.Q5_K, ca.Q6_K, ca.F16):
+        for (N, M) in ((4096, 512), (14336, 2048)):
+            gemm_case("prefill_%s_%dx4096_M%d" % (ca.TYPE_NAMES[wt], N, M), wt, N, M)
 
     out.update(bench_trace(dev, hip, st, rng))
     out["mfma_i8_measured_peak"] = measured_mfma_peak()
@@ -259,7 +268,8 @@ def measured_mfma_peak():
 def bench_trace(dev, hip, st, rng):
     """config 5: every weight matmul of one decode step of a Llama-3-8B-shaped Q4_K_M model (32 layers, 225
     matmuls; attn_v / ffn_down / output head in Q6_K, the rest Q4_K), replayed as a HIP graph, once as a serial
-    chain and once with the independent matmuls of a layer as concurrent graph branches."""
+    chain and once with the independent matmuls of a layer as concurrent graph branches; and the same matmuls for
+    one 512-token prefill chunk (serial only)."""
     import cactus_amd as ca
     L = dev.lib
     H, FF, KV, V, NL = 4096, 14336, 1024, 128256, 32
@@ -293,7 +303,7 @@ def bench_trace(dev, hip, st, rng):
         dev.check(L.chip_stream_create(C.byref(s_)))
 
     res = {}
-    for n in (1, 8):
+    for n in (1, 8, 512):                                              # decode, small batch, one prefill chunk
         x_h = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
         x_ff = dev.to_device(rng.standard_normal((n, FF)).astype(np.float32))
         y = dev.alloc(3 * n * V * 4)                                   # one output region per concurrent branch
@@ -353,7 +363,7 @@ def bench_trace(dev, hip, st, rng):
 
         b = total + 4 * n * (NL * sum(K + N for (_, _, N, K, _) in layer) + H + V)
         entry = {"weight_bytes": total, "matmuls": 7 * NL + 1}
-        for mode in ("serial", "parallel"):
+        for mode in (("serial", "parallel") if n <= 8 else ("serial",)):
             one_step(mode == "parallel")
             dev.sync(st)
             graph, gexec = C.c_void_p(), C.c_void_p()
@@ -364,6 +374,10 @@ def bench_trace(dev, hip, st, rng):
             us = time_runs(dev, hip, st, lambda: hl.hipGraphLaunch(gexec, st), 20, warm=2)
             entry[mode] = {"us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
                            "GBps": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+            if n > 8:                                                   # prefill: the matrix pipe is the yardstick
+                ops = 2.0 * n * (NL * sum(N * K for (_, _, N, K, _) in layer) + V * H)
+                entry[mode]["TOPS"] = round(ops / us / 1e6, 1)
+                entry[mode]["int8_frac"] = round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)
         res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = entry
         for bf in [x_h, x_ff, y] + wss:
             bf.free()
