@@ -113,7 +113,8 @@ CHIP_API int chip_convert_f32_to_f16(const float *x, int64_t ldx, int64_t n, int
  *               reference, sized by lm_ggml_graph_plan, ggml-cpu/ggml-cpu.c:2697-2704); holds the quantized
  *               activations in a kernel-private layout
  * n <= 4 runs the dot-product GEMV with the quantizer in its prologue; Q8_0 with n >= 5 the matrix-core GEMV
- * (16 tokens per pass over W); Q4_0 with n >= 16 the int8-MFMA GEMM; everything else the GEMV in token groups.
+ * (16 tokens per pass over W); from 16 to 48 tokens on (by type and matrix size) the MFMA GEMM of the weight type;
+ * everything else the GEMV in token groups.
  * K must be a multiple of 256.  W must be 16-byte aligned and nb01 a multiple of 16 (2 and 2 for Q6_K, whose
  * 210-byte blocks allow no more); x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
  */
