@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-trace", action="store_true",
+                    help="skip the model-shaped HIP-graph trace and the issue-rate probe (for runs under a profiler)")
     return ap.parse_args()
 
 
@@ -188,7 +190,7 @@ def time_runs(dev, hip, st, fn, iters, warm=3):
     return hip.elapsed_ms(a, b) * 1e3 / iters          # microseconds per call
 
 
-def bench_extra(dev, hip):
+def bench_extra(dev, hip, trace=True):
     import cactus_amd as ca
     L = dev.lib
     rng = np.random.default_rng(5)
@@ -239,8 +241,9 @@ def bench_extra(dev, hip):
         for (N, M) in ((4096, 512), (14336, 2048)):
             gemm_case("prefill_%s_%dx4096_M%d" % (ca.TYPE_NAMES[wt], N, M), wt, N, M)
 
-    out.update(bench_trace(dev, hip, st, rng))
-    out["mfma_i8_measured_peak"] = measured_mfma_peak()
+    if trace:
+        out.update(bench_trace(dev, hip, st, rng))
+        out["mfma_i8_measured_peak"] = measured_mfma_peak()
     return out
 
 
@@ -429,7 +432,7 @@ def main():
     dev = ca.Device(0)
     hip = Hip()
     value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, args.steps, args.warmup)
-    extra = {} if args.no_extra else bench_extra(dev, hip)
+    extra = {} if args.no_extra else bench_extra(dev, hip, trace=not args.no_trace)
     cpu = None if args.no_cpu else cpu_baseline(step_bytes)
     line = {
         "metric": "quant mul_mat GEMV HBM GB/s & prefill int8 TOPS (% of roofline), 1 GPU",
