@@ -241,6 +241,37 @@ def bench_extra(dev, hip, trace=True):
         for (N, M) in ((4096, 512), (14336, 2048)):
             gemm_case("prefill_%s_%dx4096_M%d" % (ca.TYPE_NAMES[wt], N, M), wt, N, M)
 
+    # MUL_MAT_ID (mixture-of-experts matmul), decode: one token, every (token, slot) pair a GEMV on its expert
+    def moe_case(key, wt, n_as, n_used, N, K, n_tokens=1):
+        nb01 = dev.row_size(wt, K)
+        one = synth_weights(dev, wt, N, K, rng)
+        w = dev.alloc(n_as * N * nb01)
+        w.upload(one)
+        for e in range(1, n_as):
+            dev.check(L.chip_memcpy_d2d(w.ptr + e * N * nb01, w.ptr, N * nb01, None))
+        x = dev.to_device(rng.standard_normal((n_tokens, K)).astype(np.float32))
+        y = dev.alloc(n_tokens * n_used * N * 4)
+        wsz = L.chip_mul_mat_workspace_size(wt, K, n_tokens)
+        ws = dev.alloc(wsz)
+        # a different set of experts on every call, so the weights come from HBM like in a real layer stack
+        sets = [np.stack([rng.permutation(n_as)[:n_used] for _ in range(n_tokens)]).astype(np.int32) for _ in range(16)]
+        ids = [dev.to_device(s_) for s_ in sets]
+        state = {"i": 0}
+
+        def call():
+            state["i"] += 1
+            return L.chip_mul_mat_id(wt, w.ptr, nb01, N * nb01, K, N, n_as, x.ptr, K, 1, ids[state["i"] % 16].ptr, n_used,
+                                     n_used, n_tokens, y.ptr, N, ws.ptr, wsz, st)
+        us = time_runs(dev, hip, st, call, 100)
+        b = n_tokens * n_used * N * nb01 + 4 * n_tokens * (K + n_used * N)
+        out[key] = {"us_op": round(us, 2), "GBps_op": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4),
+                    "bytes": b, "experts": n_as, "used": n_used}
+        for bf in [w, x, y, ws] + ids:
+            bf.free()
+
+    moe_case("moe_q4_K_128x8_768x2048_n1", ca.Q4_K, 128, 8, 768, 2048)          # Qwen3-30B-A3B-shaped expert up/gate
+    moe_case("moe_q4_K_8x2_14336x4096_n1", ca.Q4_K, 8, 2, 14336, 4096)          # Mixtral-8x7B-shaped expert up/gate
+
     if trace:
         out.update(bench_trace(dev, hip, st, rng))
         out["mfma_i8_measured_peak"] = measured_mfma_peak()

@@ -33,7 +33,8 @@ EXPORTS = (
     "chip_stream_destroy", "chip_stream_synchronize", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_block_isums",
+    "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
+    "chip_block_isums",
     "chip_workspace_to_blocks",
 )
 
@@ -89,6 +90,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
+    L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
     L.chip_block_isums.argtypes = [i32, vp, sz, i64, i64, vp, i64, vp, vp, vp]
     L.chip_workspace_to_blocks.argtypes = [i32, i64, i64, vp, vp, vp]
     return L
@@ -198,6 +200,26 @@ class Device:
             self.sync()
             return y, db.download(np.uint8, n * rs).reshape(n, rs)
         return y
+
+    def mul_mat_id(self, wtype, W, x, ids):
+        """LM_GGML_OP_MUL_MAT_ID: W uint8 [n_as, N, row_size], x fp32 [n_tokens, ne11, K], ids int32 [n_tokens, n_used]
+        -> y [n_tokens, n_used, N]."""
+        W = np.ascontiguousarray(W, np.uint8)
+        x = np.ascontiguousarray(x, np.float32)
+        ids = np.ascontiguousarray(ids, np.int32)
+        n_tokens, ne11, k = x.shape
+        n_as, N = W.shape[0], W.shape[1]
+        n_used = ids.shape[1]
+        nb01 = self.row_size(wtype, k)
+        dW, dx, di = self.to_device(W), self.to_device(x), self.to_device(ids)
+        dy = self.alloc(n_tokens * n_used * N * 4)
+        self.check(self.lib.chip_memset(dy.ptr, 0xFF, max(n_tokens * n_used * N * 4, 16), None))   # NaN: unwritten rows show
+        wsz = self.lib.chip_mul_mat_workspace_size(wtype, k, n_tokens * ne11)
+        ws = self.alloc(wsz)
+        self.check(self.lib.chip_mul_mat_id(wtype, dW.ptr, nb01, N * nb01, k, N, n_as, dx.ptr, k, ne11, di.ptr, n_used,
+                                            n_used, n_tokens, dy.ptr, N, ws.ptr, wsz, None))
+        self.sync()
+        return dy.download(np.float32, n_tokens * n_used * N).reshape(n_tokens, n_used, N)
 
     def block_isums(self, wtype, W, aq, k):
         """Per-block integer sums [n, N, K/block] (and imin for Q4_K / Q5_K) from reference-layout activation blocks."""

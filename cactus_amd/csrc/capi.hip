@@ -323,6 +323,37 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
     return chip_mul_mat_run(type, W, nb01, K, N, n, workspace, y, ldy, stream);
 }
 
+int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t n_as, const float *x,
+                    int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride, int64_t n_used, int64_t n_tokens,
+                    float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (N < 0 || n_as < 0 || n_used < 0 || n_tokens < 0 || ne11 < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n_used == 0 || n_tokens == 0) return CHIP_OK;
+    if (n_as == 0 || !(ne11 == 1 || ne11 == n_used)) return CHIP_EINVAL;
+    if (!W || !x || !ids || !y || !workspace || ldx < K || ldy < N || ids_stride < n_used) return CHIP_EINVAL;
+    if (!weights_aligned(type, W, nb01) || !weights_aligned(type, W, nb02) || nb01 < chip_row_size(type, K) ||
+        nb02 < (size_t)N * nb01)
+        return CHIP_EINVAL;
+    if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0 || (((uintptr_t)ids) & 3) != 0)
+        return CHIP_EINVAL;
+    const int64_t rows = n_tokens * ne11;
+    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, rows)) return CHIP_ENOMEM;
+    DeviceLimits lim;
+    int rc = current_limits(lim);
+    if (rc) return rc;
+    const size_t stride = act_stride(chip_vec_dot_type(type), K);
+    hipStream_t st = (hipStream_t)stream;
+    // few pairs: quantize in the GEMV prologue (one launch); many pairs would each repeat that work, so the rows are
+    // quantized once up front instead
+    const bool fused = n_tokens * n_used <= 16 && gemv_fused_applicable(type, K, 1, lim);
+    if (!fused) {
+        rc = chip_mul_mat_prepare(type, K, x, ldx, rows, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+    }
+    return hip_rc(launch_gemv_id(type, fused, W, nb01, nb02, n_as, K, N, x, ldx, ne11, ids, ids_stride, n_used, n_tokens,
+                                 workspace, stride, y, ldy, lim, st));
+}
+
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                      int32_t *isum, int32_t *imin, void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;

@@ -897,10 +897,10 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
 
 
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
-__global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
-                                                   const float *__restrict__ x, int64_t ldx,
-                                                   uint8_t *__restrict__ ws, size_t ws_stride,
-                                                   float *__restrict__ y, int64_t ldy) {
+__device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
+                                          const float *__restrict__ x, int64_t ldx,
+                                          uint8_t *__restrict__ ws, size_t ws_stride,
+                                          float *__restrict__ y, int64_t ldy) {
     using T = Traits<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int NI = iters_per_row<WT>(K);
@@ -993,6 +993,39 @@ __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W
             advance(cc);
         }
     }
+}
+
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
+__global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
+                                                   const float *__restrict__ x, int64_t ldx,
+                                                   uint8_t *__restrict__ ws, size_t ws_stride,
+                                                   float *__restrict__ y, int64_t ldy) {
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy);
+}
+
+// LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
+// ids[token][slot] picks the weight matrix W + id * nb02, its activation is row token * ne11 + slot % ne11 of x (of
+// the workspace), its output row `pair` of y.  Every pair is a one-token GEMV of the kind above.  A pair whose id is
+// outside [0, n_as) is skipped (the reference asserts).
+struct MoeArgs {
+    const int32_t *ids;
+    int64_t ids_stride;      // elements between the ids of consecutive tokens
+    int64_t n_used, ne11, n_as;
+    size_t nb02;
+    int64_t pair0;           // first pair of this launch
+};
+template <int WT, int R, int WGS, bool FUSEQ, int DEPTH>
+__global__ __launch_bounds__(WGS) void gemv_id_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
+                                                      const float *__restrict__ x, int64_t ldx,
+                                                      uint8_t *__restrict__ ws, size_t ws_stride,
+                                                      float *__restrict__ y, int64_t ldy, MoeArgs m) {
+    const int64_t pair = m.pair0 + blockIdx.y;
+    const int64_t t = pair / m.n_used, s = pair % m.n_used;
+    const int64_t e = m.ids[t * m.ids_stride + s];
+    if (e < 0 || e >= m.n_as) return;
+    const int64_t xrow = t * m.ne11 + s % m.ne11;
+    gemv_body<WT, 1, R, WGS, FUSEQ, DEPTH>(W + (size_t)e * m.nb02, nb01, K, N, FUSEQ ? x + xrow * ldx : x, ldx,
+                                          ws + (size_t)xrow * ws_stride, ws_stride, y + pair * ldy, ldy);
 }
 
 // ------------------------------------------------------------------------------------------------ launch
@@ -1154,6 +1187,51 @@ hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, i
         case T_F16: return launch_ntok<T_F16, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
         default: return hipErrorInvalidValue;
     }
+}
+
+// MUL_MAT_ID: one launch of (groups, pairs) workgroups, each pair a one-token GEMV on its expert's rows.  `fused`
+// quantizes the pair's activation row in the prologue (x is fp32); otherwise ws holds the quantized rows already.
+template <int WT, bool FUSEQ>
+static hipError_t launch_id_typed(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
+                                  size_t ws_stride, float *y, int64_t ldy, MoeArgs m, int64_t pairs, const DeviceLimits &lim,
+                                  hipStream_t st) {
+    const size_t lds_bytes = lds_image_bytes<WT>(K);
+    if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    constexpr int R = RowsPerWave<WT>::R, WGS = 256;
+    const int64_t tiles = ceil_div(N, R);
+    auto kfn = gemv_id_kernel<WT, R, WGS, FUSEQ, GEMV_DEPTH>;
+    static LdsGrant grant;
+    if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
+    for (int64_t p0 = 0; p0 < pairs; p0 += 32768) {
+        const int64_t np = pairs - p0 < 32768 ? pairs - p0 : 32768;
+        // about two 4-wave groups per CU over all pairs of the launch, at least one group per pair
+        int64_t groups = ceil_div(tiles, WGS / 64);
+        const int64_t cap = ceil_div((int64_t)cus * 4, np);
+        if (groups > cap) groups = cap;
+        m.pair0 = p0;
+        hipLaunchKernelGGL(kfn, dim3((unsigned)groups, (unsigned)np), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                           x, ldx, (uint8_t *)ws, ws_stride, y, ldy, m);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_gemv_id(int wtype, bool fused, const void *W, size_t nb01, size_t nb02, int64_t n_as, int64_t K, int64_t N,
+                          const float *x, int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride, int64_t n_used,
+                          int64_t n_tokens, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim,
+                          hipStream_t st) {
+    const int64_t pairs = n_tokens * n_used;
+    if (N <= 0 || pairs <= 0) return hipSuccess;
+    const MoeArgs m{ids, ids_stride, n_used, ne11, n_as, nb02, 0};
+#define ID_CASE(TT) case TT: return fused ? launch_id_typed<TT, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, m, pairs, lim, st) \
+                                          : launch_id_typed<TT, false>(W, nb01, K, N, nullptr, 0, ws, ws_stride, y, ldy, m, pairs, lim, st);
+    switch (wtype) {
+        ID_CASE(T_Q4_0) ID_CASE(T_Q8_0) ID_CASE(T_Q4_K) ID_CASE(T_Q6_K) ID_CASE(T_Q5_0) ID_CASE(T_Q5_K) ID_CASE(T_IQ4_NL)
+        ID_CASE(T_Q4_1) ID_CASE(T_Q5_1) ID_CASE(T_F16)
+        default: return hipErrorInvalidValue;
+    }
+#undef ID_CASE
 }
 
 // ------------------------------------------------------------------------------------------------ isum hook

@@ -145,11 +145,60 @@ bool mul_mat_shape_ok(const lm_ggml_tensor *op) {
     return true;
 }
 
+// The MUL_MAT_ID shapes: experts [K, N, n_as] stored one matrix after the other, F32 activations [K, ne11, n_tokens]
+// with ne11 = 1 or n_used and the rows of a token adjacent, I32 ids [n_used, n_tokens], F32 result
+// [N, n_used, n_tokens] with adjacent rows (reference ggml.c lm_ggml_mul_mat_id, ggml-cpu/ggml-cpu.c:1531-1710).
+bool mul_mat_id_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *w = op->src[0], *x = op->src[1], *ids = op->src[2];
+    if (!w || !x || !ids) return false;
+    if (!chip_mul_mat_supported(w->type, w->ne[0])) return false;
+    if (x->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32 || ids->type != LM_GGML_TYPE_I32) return false;
+    const int64_t K = w->ne[0], N = w->ne[1], n_used = ids->ne[0], n_tokens = ids->ne[1];
+    if (w->ne[3] != 1 || x->ne[3] != 1 || op->ne[3] != 1 || ids->ne[2] != 1 || ids->ne[3] != 1) return false;
+    if (x->ne[0] != K || x->ne[2] != n_tokens || !(x->ne[1] == 1 || x->ne[1] == n_used)) return false;
+    if (op->ne[0] != N || op->ne[1] != n_used || op->ne[2] != n_tokens) return false;
+    const size_t a = (w->type == LM_GGML_TYPE_Q6_K) ? 2 : 16;
+    if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, K) || w->nb[1] % a != 0) return false;
+    if (w->nb[2] < (size_t)N * w->nb[1] || w->nb[2] % a != 0) return false;
+    if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)K * 4 || x->nb[2] != (size_t)x->ne[1] * x->nb[1]) return false;
+    if (ids->nb[0] != sizeof(int32_t) || ids->nb[1] % 4 != 0 || ids->nb[1] < (size_t)n_used * 4) return false;
+    if (op->nb[0] != sizeof(float) || op->nb[1] % 4 != 0 || op->nb[1] < (size_t)N * 4 || op->nb[2] != (size_t)n_used * op->nb[1]) return false;
+    return true;
+}
+
+static bool grow_workspace(backend_ctx *c, size_t need) {
+    if (need <= c->workspace_size) return true;
+    chip_stream_synchronize(c->stream);
+    chip_free(c->workspace);
+    c->workspace = nullptr;
+    c->workspace_size = 0;
+    const size_t want = need + need / 4;
+    if (chip_malloc(&c->workspace, want) != CHIP_OK) return false;
+    c->workspace_size = want;
+    return true;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        if (node->op == LM_GGML_OP_MUL_MAT_ID && mul_mat_id_shape_ok(node)) {
+            const lm_ggml_tensor *w = node->src[0], *x = node->src[1], *ids = node->src[2];
+            const int64_t K = w->ne[0], N = w->ne[1], n_used = ids->ne[0], n_tokens = ids->ne[1];
+            if (N == 0 || n_used == 0 || n_tokens == 0) continue;
+            if (!grow_workspace(c, chip_mul_mat_workspace_size(w->type, K, n_tokens * x->ne[1]))) return LM_GGML_STATUS_ALLOC_FAILED;
+            const int rc = chip_mul_mat_id(w->type, w->data, w->nb[1], w->nb[2], K, N, w->ne[2], (const float *)x->data,
+                                           (int64_t)(x->nb[1] / 4), x->ne[1], (const int32_t *)ids->data, (int64_t)(ids->nb[1] / 4),
+                                           n_used, n_tokens, (float *)node->data, (int64_t)(node->nb[1] / 4), c->workspace,
+                                           c->workspace_size, c->stream);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT_ID %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            g_mul_mat_nodes++;
+            continue;
+        }
         if (node->op != LM_GGML_OP_MUL_MAT || !mul_mat_shape_ok(node)) {
             HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: node %d (%s, op %d) is not supported by the HIP backend\n", __func__, i, node->name, node->op);
             return LM_GGML_STATUS_FAILED;
@@ -157,16 +206,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
         const int64_t K = w->ne[0], N = w->ne[1], n = x->ne[1];
         if (N == 0 || n == 0) continue;
-        const size_t need = chip_mul_mat_workspace_size(w->type, K, n);
-        if (need > c->workspace_size) {                                    // grow the activation scratch (wdata)
-            chip_stream_synchronize(c->stream);
-            chip_free(c->workspace);
-            c->workspace = nullptr;
-            c->workspace_size = 0;
-            const size_t want = need + need / 4;
-            if (chip_malloc(&c->workspace, want) != CHIP_OK) return LM_GGML_STATUS_ALLOC_FAILED;
-            c->workspace_size = want;
-        }
+        if (!grow_workspace(c, chip_mul_mat_workspace_size(w->type, K, n))) return LM_GGML_STATUS_ALLOC_FAILED;   // wdata
         const int rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, (int64_t)(x->nb[1] / 4), n,
                                     (float *)node->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
         if (rc != CHIP_OK) {
@@ -230,13 +270,13 @@ lm_ggml_backend_buffer_type_t dev_buffer_type(lm_ggml_backend_dev_t) { return hi
 
 bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     if (is_view_op(op->op)) return true;
-    if (op->op != LM_GGML_OP_MUL_MAT) return false;
+    if (op->op != LM_GGML_OP_MUL_MAT && op->op != LM_GGML_OP_MUL_MAT_ID) return false;
     // Only weights that already live in a HIP buffer: claiming host-resident weights would make the scheduler
     // copy the whole matrix to the device on every call.  At model load the probe tensor carries a zero-size
     // dummy buffer of the candidate buffer type and NULL data (reference llama-model.cpp:161-165,246-251).
     const lm_ggml_tensor *w = op->src[0];
     if (!w || !w->buffer || !is_hip_buffer(w->buffer)) return false;
-    return mul_mat_shape_ok(op);
+    return op->op == LM_GGML_OP_MUL_MAT ? mul_mat_shape_ok(op) : mul_mat_id_shape_ok(op);
 }
 bool dev_supports_buft(lm_ggml_backend_dev_t, lm_ggml_backend_buffer_type_t buft) { return buft == hip_buffer_type(); }
 

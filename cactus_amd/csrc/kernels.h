@@ -91,6 +91,13 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
 bool       gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim);
 hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
                              int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+// MUL_MAT_ID: every (token, slot) pair is a one-token GEMV on the expert ids[token][slot] names (W + id * nb02), its
+// activation row token * ne11 + slot % ne11, its output row token * n_used + slot.  fused: x is fp32 and is quantized in
+// the prologue; otherwise ws already holds the quantized rows.
+hipError_t launch_gemv_id(int wtype, bool fused, const void *W, size_t nb01, size_t nb02, int64_t n_as, int64_t K, int64_t N,
+                          const float *x, int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride, int64_t n_used,
+                          int64_t n_tokens, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim,
+                          hipStream_t st);
 hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                               int32_t *isum, int32_t *imin, hipStream_t st);
 

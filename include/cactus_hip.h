@@ -132,6 +132,21 @@ CHIP_API int chip_mul_mat_prepare(int type, int64_t K, const float *x, int64_t l
 CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,
                               const void *workspace, float *y, int64_t ldy, void *stream);
 
+/* ---- LM_GGML_OP_MUL_MAT_ID: the expert matmul of mixture-of-experts layers ----
+ * lm_ggml_compute_forward_mul_mat_id (ggml-cpu/ggml-cpu.c:1460-1710) with src0 = W (type, [K, N, n_as]: n_as expert
+ * matrices, row stride nb01 and matrix stride nb02 bytes), src1 = x (F32 [K, ne11, n_tokens], row stride ldx
+ * elements, the ne11 rows of a token adjacent: nb12 = ne11 * nb11), ids (I32 [n_used, n_tokens] in device memory,
+ * ids_stride elements between tokens), dst = y (F32 [N, n_used, n_tokens], row stride ldy elements, rows adjacent):
+ *     y[t][s][r] = vec_dot(row r of expert ids[t][s], quantize(x[t][s % ne11]))
+ * ne11 is 1 (all slots of a token share one activation row) or n_used.  Every id must lie in [0, n_as); a pair
+ * with an id outside is left unwritten (the reference asserts).  The workspace holds the n_tokens * ne11 quantized
+ * rows: at least chip_mul_mat_workspace_size(type, K, n_tokens * ne11) bytes.  Alignment rules as chip_mul_mat;
+ * nb02 obeys the rule of nb01.  Each (token, slot) pair runs as a one-token GEMV on its expert. */
+CHIP_API int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t n_as,
+                             const float *x, int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride,
+                             int64_t n_used, int64_t n_tokens, float *y, int64_t ldy,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,
  * iq4_nl_q8_0} (ggml-cpu/ggml-cpu-quants.c:1906,3591,6772,8520,2924,7699,12751), computed with the same device

@@ -34,10 +34,10 @@ extern "C" {
 /* enum values used on this path (the enums themselves are plain ints in the ABI) */
 enum {
     LM_GGML_TYPE_F32 = 0, LM_GGML_TYPE_F16 = 1, LM_GGML_TYPE_Q4_0 = 2, LM_GGML_TYPE_Q8_0 = 8,
-    LM_GGML_TYPE_Q4_K = 12, LM_GGML_TYPE_Q6_K = 14, LM_GGML_TYPE_Q8_K = 15,
+    LM_GGML_TYPE_Q4_K = 12, LM_GGML_TYPE_Q6_K = 14, LM_GGML_TYPE_Q8_K = 15, LM_GGML_TYPE_I32 = 26,
 };
 enum {
-    LM_GGML_OP_NONE = 0, LM_GGML_OP_MUL_MAT = 27,
+    LM_GGML_OP_NONE = 0, LM_GGML_OP_MUL_MAT = 27, LM_GGML_OP_MUL_MAT_ID = 28,
     LM_GGML_OP_RESHAPE = 34, LM_GGML_OP_VIEW = 35, LM_GGML_OP_PERMUTE = 36, LM_GGML_OP_TRANSPOSE = 37,
     LM_GGML_OP_COUNT = 82,
 };

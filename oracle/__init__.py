@@ -128,6 +128,8 @@ class Oracle:
         L.orc_vec_dot_exact.argtypes = [_i32, _i64, _vp, _vp, _vp]
         L.orc_mul_mat.restype = None
         L.orc_mul_mat.argtypes = [_i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i32]
+        L.orc_mul_mat_id.restype = _i32
+        L.orc_mul_mat_id.argtypes = [_i32, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i32]
 
     # -- scalars
     def h2f(self, h):
@@ -234,6 +236,27 @@ class Oracle:
             out["sum_abs"] = sa
         return out
 
+    def mul_mat_id(self, wtype, W, x, ids, nthreads=1, want=()):
+        """LM_GGML_OP_MUL_MAT_ID: W uint8 [n_as, N, row_size], x fp32 [n_tokens, ne11, K] (ne11 = 1 or n_used),
+        ids int32 [n_tokens, n_used] -> y fp32 [n_tokens, n_used, N]."""
+        W = np.ascontiguousarray(W, np.uint8)
+        x = _f32(x)
+        ids = np.ascontiguousarray(ids, np.int32)
+        n_tokens, ne11, k = x.shape
+        n_as, N = W.shape[0], W.shape[1]
+        n_used = ids.shape[1]
+        assert W.shape[2] == row_size(wtype, k) and ids.shape[0] == n_tokens
+        y = np.zeros((n_tokens, n_used, N), np.float32)
+        sa = np.zeros((n_tokens, n_used, N), np.float64) if "sum_abs" in want else None
+        rc = self.lib.orc_mul_mat_id(wtype, k, N, n_as, _ptr(W), _ptr(x), ne11, _ptr(ids), n_used, n_tokens, _ptr(y),
+                                     _ptr(sa), nthreads)
+        if rc:
+            raise ValueError("orc_mul_mat_id: %d" % rc)
+        out = {"y": y}
+        if sa is not None:
+            out["sum_abs"] = sa
+        return out
+
 
 class _InitParams(C.Structure):
     _fields_ = [("mem_size", C.c_size_t), ("mem_buffer", C.c_void_p), ("no_alloc", C.c_bool)]
@@ -283,6 +306,10 @@ class Reference:
         L.lm_ggml_new_tensor_2d.argtypes = [_vp, _i32, _i64, _i64]
         L.lm_ggml_mul_mat.restype = _vp
         L.lm_ggml_mul_mat.argtypes = [_vp, _vp, _vp]
+        L.lm_ggml_new_tensor_3d.restype = _vp
+        L.lm_ggml_new_tensor_3d.argtypes = [_vp, _i32, _i64, _i64, _i64]
+        L.lm_ggml_mul_mat_id.restype = _vp
+        L.lm_ggml_mul_mat_id.argtypes = [_vp, _vp, _vp, _vp]
         L.lm_ggml_new_graph.restype = _vp
         L.lm_ggml_new_graph.argtypes = [_vp]
         L.lm_ggml_build_forward_expand.restype = None
@@ -395,3 +422,36 @@ class Reference:
         L.lm_ggml_threadpool_free(tp)
         L.lm_ggml_free(ctx)
         return y, times
+
+    def mul_mat_id_graph(self, wtype, W, x, ids, nthreads=1):
+        """LM_GGML_OP_MUL_MAT_ID on the reference CPU backend: W uint8 [n_as, N, row_size], x fp32
+        [n_tokens, ne11, K], ids int32 [n_tokens, n_used] -> y fp32 [n_tokens, n_used, N]."""
+        L = self.lib
+        W = np.ascontiguousarray(W, np.uint8)
+        x = _f32(x)
+        ids = np.ascontiguousarray(ids, np.int32)
+        n_tokens, ne11, k = x.shape
+        n_as, N = W.shape[0], W.shape[1]
+        n_used = ids.shape[1]
+        I32 = 26                                                   # LM_GGML_TYPE_I32 (ggml.h)
+        ctx = L.lm_ggml_init(_InitParams(L.lm_ggml_tensor_overhead() * 8 + L.lm_ggml_graph_overhead() + 4096,
+                                         None, True))
+        a = L.lm_ggml_new_tensor_3d(ctx, wtype, k, N, n_as)
+        b = L.lm_ggml_new_tensor_3d(ctx, F32, k, ne11, n_tokens)
+        i = L.lm_ggml_new_tensor_2d(ctx, I32, n_used, n_tokens)
+        c = L.lm_ggml_mul_mat_id(ctx, a, b, i)
+        g = L.lm_ggml_new_graph(ctx)
+        L.lm_ggml_build_forward_expand(g, c)
+        be = L.lm_ggml_backend_cpu_init()
+        L.lm_ggml_backend_cpu_set_n_threads(be, nthreads)
+        buf = L.lm_ggml_backend_alloc_ctx_tensors(ctx, be)
+        L.lm_ggml_backend_tensor_set(a, _ptr(W), 0, W.size)
+        L.lm_ggml_backend_tensor_set(b, _ptr(x), 0, x.size * 4)
+        L.lm_ggml_backend_tensor_set(i, _ptr(ids), 0, ids.size * 4)
+        assert L.lm_ggml_backend_graph_compute(be, g) == 0
+        y = np.zeros((n_tokens, n_used, N), np.float32)
+        L.lm_ggml_backend_tensor_get(c, _ptr(y), 0, y.size * 4)
+        L.lm_ggml_backend_buffer_free(buf)
+        L.lm_ggml_backend_free(be)
+        L.lm_ggml_free(ctx)
+        return y

@@ -1236,3 +1236,24 @@ void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const
     for (int i = 1; i < nthreads; i++) pthread_join(th[i], NULL);
     if (!wdata) free(wd);
 }
+
+/* LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): n_as expert matrices of N rows each, stored one
+ * after the other; for token t and slot s the expert is ids[t][s], the activation row is x[t][s % ne11] (quantized to
+ * the weight type's vec_dot type like in MUL_MAT), and y[t][s][r] = vec_dot(expert row r, that activation row).  The
+ * reference groups the (token, slot) pairs by expert only to schedule them; every output is this one vec_dot. */
+int orc_mul_mat_id(int type, int64_t K, int64_t N, int64_t n_as, const void *W, const float *x, int64_t ne11,
+                   const int32_t *ids, int64_t n_used, int64_t n_tokens, float *y, double *sum_abs, int nthreads) {
+    const size_t rs = orc_row_size(type, K);
+    if (orc_vec_dot_type(type) < 0 || ne11 < 1) return -1;
+    for (int64_t t = 0; t < n_tokens; t++)
+        for (int64_t s = 0; s < n_used; s++) {
+            const int32_t e = ids[t * n_used + s];
+            if (e < 0 || e >= n_as) return -2;                     /* the reference asserts */
+            const float *xr = x + (size_t)(t * ne11 + s % ne11) * K;
+            const size_t o = (size_t)(t * n_used + s) * N;
+            orc_mul_mat(type, K, N, 1, (const char *)W + (size_t)e * N * rs, xr, y + o, NULL, sum_abs ? sum_abs + o : NULL,
+                        nthreads);
+        }
+    return 0;
+}
+

@@ -31,6 +31,8 @@
  *   orc_fp32_to_fp16_row, orc_vec_dot_f16  conversion: the exhaustive fp16 checks above; dot: bit-exact vs oracle/_ref
  *                                    (lane structure restated) + golden; fp64 identity sum w_i * x_i
  *   orc_mul_mat                      == n*N independent vec_dots; vs oracle/_ref's LM_GGML_OP_MUL_MAT graph
+ *   orc_mul_mat_id                   == orc_mul_mat per (token, slot) on the expert the id names; vs oracle/_ref's
+ *                                       LM_GGML_OP_MUL_MAT_ID graph (bit-exact, tests/test_oracle_vs_ref.py)
  *
  * No function here is "parity unpinned".
  */
@@ -134,6 +136,10 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
  */
 void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const float *x, float *y,
                  void *wdata, double *sum_abs, int nthreads);
+/* LM_GGML_OP_MUL_MAT_ID: W holds n_as expert matrices [N][row_size] back to back, x is [n_tokens][ne11][K], ids is
+ * [n_tokens][n_used], y (and sum_abs, may be NULL) [n_tokens][n_used][N].  Returns 0, or -2 for an id out of range. */
+int orc_mul_mat_id(int type, int64_t K, int64_t N, int64_t n_as, const void *W, const float *x, int64_t ne11,
+                   const int32_t *ids, int64_t n_used, int64_t n_tokens, float *y, double *sum_abs, int nthreads);
 
 #ifdef __cplusplus
 }

@@ -23,8 +23,10 @@ namespace mirror {
 #define LM_GGML_TYPE_Q4_K M_TYPE_Q4_K
 #define LM_GGML_TYPE_Q6_K M_TYPE_Q6_K
 #define LM_GGML_TYPE_Q8_K M_TYPE_Q8_K
+#define LM_GGML_TYPE_I32 M_TYPE_I32
 #define LM_GGML_OP_NONE M_OP_NONE
 #define LM_GGML_OP_MUL_MAT M_OP_MUL_MAT
+#define LM_GGML_OP_MUL_MAT_ID M_OP_MUL_MAT_ID
 #define LM_GGML_OP_RESHAPE M_OP_RESHAPE
 #define LM_GGML_OP_VIEW M_OP_VIEW
 #define LM_GGML_OP_PERMUTE M_OP_PERMUTE
@@ -56,8 +58,10 @@ constexpr int k_max_dims = LM_GGML_MAX_DIMS, k_max_src = LM_GGML_MAX_SRC, k_max_
 #undef LM_GGML_TYPE_Q4_K
 #undef LM_GGML_TYPE_Q6_K
 #undef LM_GGML_TYPE_Q8_K
+#undef LM_GGML_TYPE_I32
 #undef LM_GGML_OP_NONE
 #undef LM_GGML_OP_MUL_MAT
+#undef LM_GGML_OP_MUL_MAT_ID
 #undef LM_GGML_OP_RESHAPE
 #undef LM_GGML_OP_VIEW
 #undef LM_GGML_OP_PERMUTE
@@ -116,10 +120,10 @@ static_assert(mirror::k_max_op_params == LM_GGML_MAX_OP_PARAMS && mirror::k_max_
 static_assert(mirror::k_api == LM_GGML_BACKEND_API_VERSION, "api version");
 static_assert(mirror::M_TYPE_F32 == LM_GGML_TYPE_F32 && mirror::M_TYPE_F16 == LM_GGML_TYPE_F16 && mirror::M_TYPE_Q4_0 == LM_GGML_TYPE_Q4_0 &&
               mirror::M_TYPE_Q8_0 == LM_GGML_TYPE_Q8_0 && mirror::M_TYPE_Q4_K == LM_GGML_TYPE_Q4_K && mirror::M_TYPE_Q6_K == LM_GGML_TYPE_Q6_K &&
-              mirror::M_TYPE_Q8_K == LM_GGML_TYPE_Q8_K, "type ids");
+              mirror::M_TYPE_Q8_K == LM_GGML_TYPE_Q8_K && mirror::M_TYPE_I32 == LM_GGML_TYPE_I32, "type ids");
 static_assert(mirror::M_OP_NONE == LM_GGML_OP_NONE && mirror::M_OP_MUL_MAT == LM_GGML_OP_MUL_MAT && mirror::M_OP_RESHAPE == LM_GGML_OP_RESHAPE &&
               mirror::M_OP_VIEW == LM_GGML_OP_VIEW && mirror::M_OP_PERMUTE == LM_GGML_OP_PERMUTE && mirror::M_OP_TRANSPOSE == LM_GGML_OP_TRANSPOSE &&
-              mirror::M_OP_COUNT == LM_GGML_OP_COUNT, "op ids");
+              mirror::M_OP_COUNT == LM_GGML_OP_COUNT && mirror::M_OP_MUL_MAT_ID == LM_GGML_OP_MUL_MAT_ID, "op ids");
 static_assert(mirror::M_STATUS_ALLOC_FAILED == LM_GGML_STATUS_ALLOC_FAILED && mirror::M_STATUS_FAILED == LM_GGML_STATUS_FAILED &&
               mirror::M_STATUS_SUCCESS == LM_GGML_STATUS_SUCCESS && mirror::M_STATUS_ABORTED == LM_GGML_STATUS_ABORTED, "status");
 static_assert(mirror::M_DEV_CPU == LM_GGML_BACKEND_DEVICE_TYPE_CPU && mirror::M_DEV_GPU == LM_GGML_BACKEND_DEVICE_TYPE_GPU &&

@@ -95,6 +95,12 @@ class Host:
             self.L.lm_ggml_set_name(p, name.encode())
         return p
 
+    def tensor_3d(self, ctx, t, ne0, ne1, ne2, name=None):
+        p = self.L.lm_ggml_new_tensor_3d(ctx, t, ne0, ne1, ne2)
+        if name:
+            self.L.lm_ggml_set_name(p, name.encode())
+        return p
+
     def set(self, tensor, arr):
         arr = np.ascontiguousarray(arr)
         self.L.lm_ggml_backend_tensor_set(tensor, arr.ctypes.data_as(vp), 0, arr.nbytes)

@@ -223,3 +223,63 @@ def test_compare_graph_backend_against_reference_cpu(host, orc):
     L.lm_ggml_backend_free(hip)
     L.lm_ggml_backend_free(cpu)
     L.lm_ggml_free(ctx)
+
+
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q6_K, O.F16), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("n_tokens,ne11", [(1, 1), (6, 4)])
+def test_mul_mat_id_node(host, orc, wt, n_tokens, ne11):
+    """LM_GGML_OP_MUL_MAT_ID (mixture-of-experts matmul) through the backend: supports_op, direct graph_compute, and
+    the reference's node-by-node comparison against its CPU backend."""
+    L = host.L
+    from ggml_host import EVAL_CB
+    K, N, n_as, n_used = 512, 130, 6, 4
+    I32 = 26
+    rng = np.random.default_rng(5 + wt + n_tokens)
+    W = np.stack([orc.quantize_weights(wt, common.weights_f32(60 + wt + e, N, K)) for e in range(n_as)])
+    x = common.activations_f32(61 + wt, n_tokens * ne11, K).reshape(n_tokens, ne11, K)
+    ids = np.stack([rng.permutation(n_as)[:n_used] for _ in range(n_tokens)]).astype(np.int32)
+    ref = orc.mul_mat_id(wt, W, x, ids, nthreads=8, want=("sum_abs",))
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+
+    def build(ctx):
+        a = host.tensor_3d(ctx, wt, K, N, n_as, "experts")
+        b = host.tensor_3d(ctx, O.F32, K, ne11, n_tokens, "x")
+        i = host.tensor_2d(ctx, I32, n_used, n_tokens, "ids")
+        c = L.lm_ggml_mul_mat_id(ctx, a, b, i)
+        g = L.lm_ggml_new_graph(ctx)
+        L.lm_ggml_build_forward_expand(g, c)
+        return a, b, i, c, g
+
+    # direct: everything in the HIP buffer type
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    ctx = host.context()
+    a, b, i, c, g = build(ctx)
+    assert L.lm_ggml_backend_dev_supports_op(dev, c) is False            # experts not in a HIP buffer yet
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    assert L.lm_ggml_backend_dev_supports_op(dev, c) is True
+    host.set(a, W); host.set(b, x); host.set(i, ids)
+    assert L.lm_ggml_backend_graph_compute(be, g) == 0
+    y = host.get(c, np.float32, (n_tokens, n_used, N))
+    assert (np.abs(y.astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all()
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_free(ctx)
+
+    # node by node against the reference CPU backend
+    cpu = L.lm_ggml_backend_cpu_init()
+    ctx = host.context()
+    a, b, i, c, g = build(ctx)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors(ctx, cpu)
+    host.set(a, W); host.set(b, x); host.set(i, ids)
+    seen = []
+
+    def cb(idx, t1, t2, ud):
+        y1 = host.get(t1, np.float32, (n_tokens, n_used, N))
+        y2 = host.get(t2, np.float32, (n_tokens, n_used, N))
+        seen.append(bool(np.array_equal(y1, ref["y"]) and (np.abs(y1.astype(np.float64) - y2) <= REL_TOL * ref["sum_abs"]).all()))
+        return True
+
+    assert L.lm_ggml_backend_compare_graph_backend(cpu, be, g, EVAL_CB(cb), None) and seen == [True]
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_free(ctx)

@@ -409,3 +409,61 @@ def test_gemm_kquant_prefill_shape_sampled(dev, orc, wt):
     check_outputs(y[np.ix_(toks, rows)], ref["y"], ref["sum_abs"], "k-quant prefill")
     y2 = dev.mul_mat(wt, wq[::-1].copy(), x[:64])
     assert np.array_equal(y2[:, ::-1], y[:64])
+
+
+# ------------------------------------------------------------------------------------------ MUL_MAT_ID (expert matmul)
+def moe_case(orc, wt, K, N, n_as, n_used, n_tokens, ne11, seed):
+    rng = np.random.default_rng(seed)
+    W = np.stack([orc.quantize_weights(wt, common.weights_f32(seed + e, N, K)) for e in range(n_as)])
+    x = common.activations_f32(seed + 100, n_tokens * ne11, K).reshape(n_tokens, ne11, K)
+    ids = np.stack([rng.permutation(n_as)[:n_used] for _ in range(n_tokens)]).astype(np.int32)
+    return W, x, ids
+
+
+@pytest.mark.parametrize("wt", O.WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("n_tokens,ne11", [(1, 1), (2, 4), (9, 1)])
+def test_mul_mat_id_vs_oracle(dev, orc, wt, n_tokens, ne11):
+    # decode (one token, fused quantize), per-slot activations, and more pairs than the fused path takes
+    K, N, n_as, n_used = 1024, 200, 8, 4
+    W, x, ids = moe_case(orc, wt, K, N, n_as, n_used, n_tokens, ne11, 700 + wt)
+    ref = orc.mul_mat_id(wt, W, x, ids, nthreads=8, want=("sum_abs",))
+    y = dev.mul_mat_id(wt, W, x, ids)
+    check_outputs(y, ref["y"], ref["sum_abs"], "mul_mat_id")
+
+
+def test_mul_mat_id_is_mul_mat_on_the_chosen_expert(dev, orc):
+    """Same device code as MUL_MAT: each (token, slot) output equals chip_mul_mat on that expert, bit for bit; repeated
+    experts and a long K (activation quantized ahead of the GEMV) included."""
+    wt, K, N, n_as, n_used, n_tokens = O.Q4_K, 8192, 96, 5, 3, 4
+    W, x, ids = moe_case(orc, wt, K, N, n_as, n_used, n_tokens, 1, 41)
+    ids[1] = [2, 2, 2]
+    y = dev.mul_mat_id(wt, W, x, ids)
+    for t in range(n_tokens):
+        for s in range(n_used):
+            one = dev.mul_mat(wt, W[ids[t, s]], x[t])
+            assert np.array_equal(y[t, s], one[0])
+
+
+def test_mul_mat_id_argument_errors(dev, orc):
+    import cactus_amd as ca
+    L = dev.lib
+    wt, K, N = O.Q8_0, 256, 8
+    W, x, ids = moe_case(orc, wt, K, N, 2, 2, 1, 1, 5)
+    nb01 = dev.row_size(wt, K)
+    dW, dx, di, dy = dev.to_device(W), dev.to_device(x), dev.to_device(ids), dev.alloc(2 * N * 4)
+    wsz = L.chip_mul_mat_workspace_size(wt, K, 1)
+    ws = dev.alloc(wsz)
+    call = lambda **kw: L.chip_mul_mat_id(*[kw.get(k, v) for k, v in (
+        ("type", wt), ("W", dW.ptr), ("nb01", nb01), ("nb02", N * nb01), ("K", K), ("N", N), ("n_as", 2), ("x", dx.ptr),
+        ("ldx", K), ("ne11", 1), ("ids", di.ptr), ("ids_stride", 2), ("n_used", 2), ("n_tokens", 1), ("y", dy.ptr),
+        ("ldy", N), ("ws", ws.ptr), ("wsz", wsz), ("stream", None))])
+    assert call() == 0
+    assert call(type=30) != 0 and call(ne11=3) != 0 and call(ids=None) != 0 and call(wsz=16) != 0
+    assert call(nb02=nb01) != 0 and call(ldy=N - 1) != 0 and call(n_tokens=0) == 0
+    # an id outside [0, n_as) leaves its output row unwritten and does not touch memory outside the experts
+    bad = dev.to_device(np.array([[1, 7]], np.int32))
+    dev.check(L.chip_memset(dy.ptr, 0xFF, 2 * N * 4, None))
+    assert call(ids=bad.ptr) == 0
+    dev.sync()
+    out = dy.download(np.float32, 2 * N).reshape(2, N)
+    assert np.isfinite(out[0]).all() and np.isnan(out[1]).all()

@@ -56,3 +56,22 @@ def test_mul_mat_graph(orc, ref, wt, n, threads):
     y_ref, _ = ref.mul_mat_graph(wt, wq, x, nthreads=threads)
     y = orc.mul_mat(wt, wq, x, nthreads=threads)["y"]
     assert np.array_equal(y, y_ref)
+
+
+@pytest.mark.parametrize("wt", (O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K, O.Q5_K, O.Q4_1, O.F16), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("n_tokens,ne11,threads", [(1, 1, 1), (3, 4, 2), (5, 1, 3)])
+def test_mul_mat_id_graph(orc, ref, wt, n_tokens, ne11, threads):
+    """MUL_MAT_ID against the reference CPU backend: 6 experts, 4 used per token, activations either shared by the
+    slots of a token (ne11 = 1) or one row per slot; bit-exact."""
+    K, N, n_as, n_used = 512, 37, 6, 4
+    rng = np.random.default_rng(21 + wt + n_tokens)
+    W = np.stack([orc.quantize_weights(wt, common.weights_f32(30 + wt + e, N, K)) for e in range(n_as)])
+    x = common.activations_f32(31 + wt, n_tokens * ne11, K).reshape(n_tokens, ne11, K)
+    ids = np.stack([rng.permutation(n_as)[:n_used] for _ in range(n_tokens)]).astype(np.int32)
+    y_ref = ref.mul_mat_id_graph(wt, W, x, ids, nthreads=threads)
+    y = orc.mul_mat_id(wt, W, x, ids, nthreads=threads)["y"]
+    assert np.array_equal(y, y_ref)
+    # the op is MUL_MAT on the selected expert, pair by pair
+    t, s = n_tokens - 1, n_used - 1
+    one = orc.mul_mat(wt, W[ids[t, s]], x[t, s % ne11][None, :])["y"][0]
+    assert np.array_equal(y[t, s], one)
