@@ -35,6 +35,17 @@ def main():
         np.savez_compressed(os.path.join(HERE, "mul_mat_%s.npz" % name),
                             wtype=np.int32(wt), K=np.int32(K), w=w, x=x, wq=wq, xq=xq,
                             w_deq=r.dequantize(wt, wq, K), y_dot=y_dot, y_graph=y_graph)
+    # LM_GGML_OP_MUL_MAT_ID from the reference's CPU graph: 5 experts, 3 used per token, per-slot activations for one
+    # type and activations shared by a token's slots for the other
+    for wt, ne11 in ((O.Q4_K, 1), (O.Q8_0, 3)):
+        K, N, n_as, n_used, n_tokens = 512, 5, 5, 3, 3
+        rng = np.random.default_rng(200 + wt)
+        W = np.stack([r.quantize_weights(wt, common.weights_f32(200 + wt + e, N, K)) for e in range(n_as)])
+        x = common.activations_f32(200 + wt, n_tokens * ne11, K).reshape(n_tokens, ne11, K)
+        ids = np.stack([rng.permutation(n_as)[:n_used] for _ in range(n_tokens)]).astype(np.int32)
+        ids[1] = ids[1, 0]                                   # one token sends all its slots to the same expert
+        np.savez_compressed(os.path.join(HERE, "mul_mat_id_%s.npz" % O.TYPE_NAMES[wt]), wtype=np.int32(wt), W=W, x=x,
+                            ids=ids, y_graph=r.mul_mat_id_graph(wt, W, x, ids, nthreads=2))
     e0 = common.q8_0_edge_rows()
     with np.errstate(all="ignore"):
         np.savez_compressed(os.path.join(HERE, "quantize_q8_0_edges.npz"), x=e0,

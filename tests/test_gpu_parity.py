@@ -431,6 +431,13 @@ def test_mul_mat_id_vs_oracle(dev, orc, wt, n_tokens, ne11):
     check_outputs(y, ref["y"], ref["sum_abs"], "mul_mat_id")
 
 
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0), ids=lambda t: O.TYPE_NAMES[t])
+def test_mul_mat_id_golden(dev, orc, wt):
+    g = np.load(os.path.join(GOLD, "mul_mat_id_%s.npz" % O.TYPE_NAMES[wt]))
+    sa = orc.mul_mat_id(wt, g["W"], g["x"], g["ids"], want=("sum_abs",))["sum_abs"]
+    check_outputs(dev.mul_mat_id(wt, g["W"], g["x"], g["ids"]), g["y_graph"], sa, "mul_mat_id golden")
+
+
 def test_mul_mat_id_is_mul_mat_on_the_chosen_expert(dev, orc):
     """Same device code as MUL_MAT: each (token, slot) output equals chip_mul_mat on that expert, bit for bit; repeated
     experts and a long K (activation quantized ahead of the GEMV) included."""

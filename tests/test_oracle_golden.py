@@ -41,6 +41,16 @@ def test_mul_mat_golden(orc, wt):
     assert (out["sum_abs"] > 0).all()
 
 
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0), ids=lambda t: O.TYPE_NAMES[t])
+def test_mul_mat_id_golden(orc, wt):
+    g = gold("mul_mat_id_%s.npz" % O.TYPE_NAMES[wt])
+    assert int(g["wtype"]) == wt
+    out = orc.mul_mat_id(wt, g["W"], g["x"], g["ids"], nthreads=2)
+    assert np.array_equal(out["y"], g["y_graph"])
+    with pytest.raises(ValueError):                          # the reference asserts on ids outside [0, n_as)
+        orc.mul_mat_id(wt, g["W"], g["x"], g["ids"] + 3)
+
+
 def test_quantize_q8_0_edges(orc):
     g = gold("quantize_q8_0_edges.npz")
     with np.errstate(all="ignore"):
