@@ -251,7 +251,7 @@ def bench_extra(dev, hip, trace=True):
             dev.check(L.chip_memcpy_d2d(w.ptr + e * N * nb01, w.ptr, N * nb01, None))
         x = dev.to_device(rng.standard_normal((n_tokens, K)).astype(np.float32))
         y = dev.alloc(n_tokens * n_used * N * 4)
-        wsz = L.chip_mul_mat_workspace_size(wt, K, n_tokens)
+        wsz = L.chip_mul_mat_id_workspace_size(wt, K, n_as, n_used, n_tokens, 1)
         ws = dev.alloc(wsz)
         # a different set of experts on every call, so the weights come from HBM like in a real layer stack
         sets = [np.stack([rng.permutation(n_as)[:n_used] for _ in range(n_tokens)]).astype(np.int32) for _ in range(16)]
@@ -262,15 +262,22 @@ def bench_extra(dev, hip, trace=True):
             state["i"] += 1
             return L.chip_mul_mat_id(wt, w.ptr, nb01, N * nb01, K, N, n_as, x.ptr, K, 1, ids[state["i"] % 16].ptr, n_used,
                                      n_used, n_tokens, y.ptr, N, ws.ptr, wsz, st)
-        us = time_runs(dev, hip, st, call, 100)
-        b = n_tokens * n_used * N * nb01 + 4 * n_tokens * (K + n_used * N)
-        out[key] = {"us_op": round(us, 2), "GBps_op": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4),
-                    "bytes": b, "experts": n_as, "used": n_used}
+        us = time_runs(dev, hip, st, call, 100 if n_tokens == 1 else 20)
+        if n_tokens == 1:
+            b = n_used * N * nb01 + 4 * (K + n_used * N)
+            out[key] = {"us_op": round(us, 2), "GBps_op": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "bytes": b, "experts": n_as, "used": n_used}
+        else:                                                       # prefill: pairs grouped by expert, MFMA GEMMs
+            ops = 2.0 * n_tokens * n_used * N * K
+            out[key] = {"us_op": round(us, 1), "TOPS_op": round(ops / us / 1e6, 1), "tokens": n_tokens, "experts": n_as,
+                        "used": n_used}
         for bf in [w, x, y, ws] + ids:
             bf.free()
 
     moe_case("moe_q4_K_128x8_768x2048_n1", ca.Q4_K, 128, 8, 768, 2048)          # Qwen3-30B-A3B-shaped expert up/gate
     moe_case("moe_q4_K_8x2_14336x4096_n1", ca.Q4_K, 8, 2, 14336, 4096)          # Mixtral-8x7B-shaped expert up/gate
+    moe_case("moe_q4_K_128x8_768x2048_n512", ca.Q4_K, 128, 8, 768, 2048, 512)
+    moe_case("moe_q4_K_8x2_14336x4096_n512", ca.Q4_K, 8, 2, 14336, 4096, 512)
 
     if trace:
         out.update(bench_trace(dev, hip, st, rng))

@@ -34,6 +34,7 @@ EXPORTS = (
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
+    "chip_mul_mat_id_workspace_size",
     "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -90,6 +91,8 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
+    L.chip_mul_mat_id_workspace_size.restype = sz
+    L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
     L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
     L.chip_block_isums.argtypes = [i32, vp, sz, i64, i64, vp, i64, vp, vp, vp]
     L.chip_workspace_to_blocks.argtypes = [i32, i64, i64, vp, vp, vp]
@@ -214,7 +217,7 @@ class Device:
         dW, dx, di = self.to_device(W), self.to_device(x), self.to_device(ids)
         dy = self.alloc(n_tokens * n_used * N * 4)
         self.check(self.lib.chip_memset(dy.ptr, 0xFF, max(n_tokens * n_used * N * 4, 16), None))   # NaN: unwritten rows show
-        wsz = self.lib.chip_mul_mat_workspace_size(wtype, k, n_tokens * ne11)
+        wsz = self.lib.chip_mul_mat_id_workspace_size(wtype, k, n_as, n_used, n_tokens, ne11)
         ws = self.alloc(wsz)
         self.check(self.lib.chip_mul_mat_id(wtype, dW.ptr, nb01, N * nb01, k, N, n_as, dx.ptr, k, ne11, di.ptr, n_used,
                                             n_used, n_tokens, dy.ptr, N, ws.ptr, wsz, None))

@@ -323,6 +323,19 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
     return chip_mul_mat_run(type, W, nb01, K, N, n, workspace, y, ldy, stream);
 }
 
+// MUL_MAT_ID workspace: the quantized activation rows, then the expert offsets and the pair list of the grouped path
+static size_t moe_rows_bytes(int type, int64_t K, int64_t rows) { return align16(act_stride(chip_vec_dot_type(type), K) * (size_t)rows); }
+size_t chip_mul_mat_id_workspace_size(int type, int64_t K, int64_t n_as, int64_t n_used, int64_t n_tokens, int64_t ne11) {
+    if (!chip_mul_mat_supported(type, K) || n_as <= 0 || n_used <= 0 || n_tokens <= 0 || ne11 <= 0) return 0;
+    const size_t pairs = (size_t)(n_tokens * n_used);
+    return moe_rows_bytes(type, K, n_tokens * ne11) + align16(4 * (size_t)(n_as + 1)) + align16(4 * pairs) +
+           align16(4 * (pairs / 64 + (size_t)n_as + 2));                // pair list, then the tile list (tiles of >= 64 pairs)
+}
+
+// from this many (token, slot) pairs on, the pairs are grouped by expert and run through the GEMM of the weight type
+// (one-token GEMVs re-read an expert's matrix for every pair)
+constexpr int64_t MOE_GEMM_MIN_PAIRS = 64;
+
 int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t n_as, const float *x,
                     int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride, int64_t n_used, int64_t n_tokens,
                     float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
@@ -336,16 +349,35 @@ int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K
         return CHIP_EINVAL;
     if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0 || (((uintptr_t)ids) & 3) != 0)
         return CHIP_EINVAL;
-    const int64_t rows = n_tokens * ne11;
-    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, rows)) return CHIP_ENOMEM;
+    const int64_t rows = n_tokens * ne11, pairs = n_tokens * n_used;
+    if (workspace_bytes < chip_mul_mat_id_workspace_size(type, K, n_as, n_used, n_tokens, ne11)) return CHIP_ENOMEM;
     DeviceLimits lim;
     int rc = current_limits(lim);
     if (rc) return rc;
     const size_t stride = act_stride(chip_vec_dot_type(type), K);
     hipStream_t st = (hipStream_t)stream;
-    // few pairs: quantize in the GEMV prologue (one launch); many pairs would each repeat that work, so the rows are
-    // quantized once up front instead
-    const bool fused = n_tokens * n_used <= 16 && gemv_fused_applicable(type, K, 1, lim);
+
+    const bool kq = type == T_Q4_K || type == T_Q5_K || type == T_Q6_K;
+    const bool have_gemm = type == T_F16 ? K % 64 == 0 : (kq ? true : K % 128 == 0);
+    if (pairs >= MOE_GEMM_MIN_PAIRS && have_gemm && moe_group_supported(n_as, pairs)) {
+        rc = chip_mul_mat_prepare(type, K, x, ldx, rows, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+        int32_t *offsets = reinterpret_cast<int32_t *>((uint8_t *)workspace + moe_rows_bytes(type, K, rows));
+        int32_t *perm = offsets + align16(4 * (size_t)(n_as + 1)) / 4;
+        int32_t *tiles = perm + align16(4 * (size_t)pairs) / 4;
+        const int bn = type == T_F16 ? gemm_f16_moe_tile_tokens() : (kq ? gemm_kq_moe_tile_tokens() : gemm_blk32_moe_tile_tokens());
+        if (hipError_t e = launch_moe_group(ids, ids_stride, n_used, pairs, n_as, bn, offsets, perm, tiles, st); e != hipSuccess)
+            return (int)e;
+        const RowGather rg{perm, offsets, tiles, (int32_t)n_used, (int32_t)ne11, nb02};
+        // the grid provides a slot for every token tile the list can have; slots past its length exit at once
+        const int64_t slots = pairs / bn + n_as;
+        if (type == T_F16) return hip_rc(launch_gemm_f16(W, nb01, K, N, workspace, stride, pairs, y, ldy, lim, st, &rg, slots));
+        if (kq) return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, pairs, y, ldy, lim, st, &rg, slots));
+        return hip_rc(launch_gemm_blk32(type, W, nb01, K, N, workspace, stride, pairs, y, ldy, lim, st, &rg, slots));
+    }
+
+    // few pairs: one-token GEMVs, quantizing in the prologue (one launch) while that repeats little work
+    const bool fused = pairs <= 16 && gemv_fused_applicable(type, K, 1, lim);
     if (!fused) {
         rc = chip_mul_mat_prepare(type, K, x, ldx, rows, workspace, workspace_bytes, stream);
         if (rc) return rc;

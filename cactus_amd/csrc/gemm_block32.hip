@@ -184,11 +184,11 @@ struct GemmCfg {
     static constexpr int S_PER_T = (S_ITEMS + NT - 1) / NT;
 };
 
-template <int WT, int TM, int TN, int WR, int WC, int OCC>
+template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
 __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_blk32_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
                                                                 int64_t N, const uint8_t *__restrict__ ws,
                                                                 size_t ws_stride, int64_t M, float *__restrict__ y,
-                                                                int64_t ldy, TileMap map) {
+                                                                int64_t ldy, TileMap map, RowGather rg) {
     using C = GemmCfg<TM, TN, WR, WC>;
     using T = Blk32<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -198,7 +198,12 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
     const TileCoord tc = xcd_tile(blockIdx.x, map);
     if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;        // padding of the tile map
     const int64_t row_base = (int64_t)tc.row_tile * C::BM;
-    const int64_t tok_base = (int64_t)tc.tok_tile * C::BN;
+    size_t w_offset;
+    const GatherView gv = resolve_gather<GATHER>(rg, w_offset, M);                   // MUL_MAT_ID: this expert's rows
+    W += w_offset;
+    if (gv.tok_tile < 0) return;
+    const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
+    if (tok_base >= M) return;
     const int nstages = (int)(K / (32 * GEMM_KB));
     const size_t off_d = q8_0_off_d(K);
 
@@ -209,6 +214,12 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
     float xs[C::S_PER_T];
     float xm[C::S_PER_T];                         // block_q8_1.s, for the types with a minimum
     const size_t off_s = q8_0_off_s(K);
+    // activation rows of this thread's staging items (looked up once: with a gather they come from the pair list)
+    int64_t xrow[C::X_PER_T], srow[C::S_PER_T];
+#pragma unroll
+    for (int i = 0; i < C::X_PER_T; i++) xrow[i] = gv.act_row(min(tok_base + (tid + i * C::NT) / (GEMM_KB * 2), M - 1));
+#pragma unroll
+    for (int i = 0; i < C::S_PER_T; i++) srow[i] = gv.act_row(min(tok_base + (tid + i * C::NT) / GEMM_KB, M - 1));
 
     auto fetch = [&](int stage) {
         const int64_t kb0 = (int64_t)stage * GEMM_KB;
@@ -228,8 +239,8 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         for (int i = 0; i < C::X_PER_T; i++) {
             const int item = tid + i * C::NT;
             if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
-                const int c = item % (GEMM_KB * 2), n = item / (GEMM_KB * 2);       // c = 2*b + half
-                const int64_t tok = min(tok_base + n, M - 1);
+                const int c = item % (GEMM_KB * 2);                                 // c = 2*b + half
+                const int64_t tok = xrow[i];
                 xq[i] = *reinterpret_cast<const u32x4 *>(ws + (size_t)tok * ws_stride + (size_t)kb0 * 32 + 16 * c);
             }
         }
@@ -237,8 +248,8 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         for (int i = 0; i < C::S_PER_T; i++) {
             const int item = tid + i * C::NT;
             if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
-                const int b = item % GEMM_KB, n = item / GEMM_KB;
-                const int64_t tok = min(tok_base + n, M - 1);
+                const int b = item % GEMM_KB;
+                const int64_t tok = srow[i];
                 xs[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_d)[kb0 + b];
                 if constexpr (T::HAS_MIN) xm[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_s)[kb0 + b];
             }
@@ -408,10 +419,11 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         for (int c = 0; c < TN; c++) {
             const int64_t tok = tok_base + (wc * TN + c) * 32 + l32;
             if (tok >= M) continue;
+            const int64_t orow = gv.out_row(tok);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int64_t row = row_base + (wr * TM + a) * 32 + 8 * g + 4 * half;
-                float *dst = y + (size_t)tok * ldy + row;
+                float *dst = y + (size_t)orow * ldy + row;
                 if (row + 3 < N && (((uintptr_t)dst) & 15) == 0) {
                     *reinterpret_cast<float4 *>(dst) = make_float4(acc[a][c][4 * g], acc[a][c][4 * g + 1], acc[a][c][4 * g + 2], acc[a][c][4 * g + 3]);
                 } else {
@@ -431,47 +443,53 @@ bool gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n) {
     return n >= ((N * K >= (int64_t)48 << 20) ? 32 : 48);
 }
 
-template <int WT, int TM, int TN, int WR, int WC, int OCC>
+template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
 static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
     using C = GemmCfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
-    auto kfn = gemm_blk32_kernel<WT, TM, TN, WR, WC, OCC>;
+    auto kfn = gemm_blk32_kernel<WT, TM, TN, WR, WC, OCC, GATHER>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     // workgroups that share an XCD (OCC waves per SIMD, 32 CUs) take a compact block of output tiles
-    const TileMap map = make_tile_map(ceil_div(N, C::BM), ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
-    hipLaunchKernelGGL(kfn, dim3(map.grid), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws,
-                       ws_stride, M, y, ldy, map);
+    const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
+    hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg);
     return hipGetLastError();
 }
 
 template <int WT>
 static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
     // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
     // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
+    if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
+        return launch_cfg<WT, 1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_CFG");
     const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
     switch (cfg) {
-        case 0: return launch_cfg<WT, 1, 2, 4, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case 1: return launch_cfg<WT, 1, 1, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case 0: return launch_cfg<WT, 1, 2, 4, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case 1: return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
         default: return hipErrorInvalidValue;
     }
 }
 
+int gemm_blk32_moe_tile_tokens() { return GemmCfg<1, 1, 2, 2>::BN; }   // the 64 x 64 shape serves the expert groups
+
 hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                             int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (M <= 0 || N <= 0) return hipSuccess;
+                             int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp,
+                             int64_t n_as) {
+    if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
+    const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     switch (wtype) {
-        case T_Q4_0:   return launch_type<T_Q4_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_Q8_0:   return launch_type<T_Q8_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_Q5_0:   return launch_type<T_Q5_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_IQ4_NL: return launch_type<T_IQ4_NL>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_Q4_1:   return launch_type<T_Q4_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_Q5_1:   return launch_type<T_Q5_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_Q4_0:   return launch_type<T_Q4_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q8_0:   return launch_type<T_Q8_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q5_0:   return launch_type<T_Q5_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_IQ4_NL: return launch_type<T_IQ4_NL>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q4_1:   return launch_type<T_Q4_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q5_1:   return launch_type<T_Q5_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
         default: return hipErrorInvalidValue;
     }
 }

@@ -36,10 +36,10 @@ struct F16Cfg {
     static_assert(W_ITEMS % NT == 0 && X_ITEMS % NT == 0, "staging items divide evenly over the threads");
 };
 
-template <int TM, int TN, int WR, int WC, int OCC>
+template <int TM, int TN, int WR, int WC, int OCC, bool GATHER>
 __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
-                     size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map) {
+                     size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg) {
     using C = F16Cfg<TM, TN, WR, WC>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -49,7 +49,12 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
     const TileCoord tc = xcd_tile(blockIdx.x, map);
     if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;
     const int64_t row_base = (int64_t)tc.row_tile * C::BM;
-    const int64_t tok_base = (int64_t)tc.tok_tile * C::BN;
+    size_t w_offset;
+    const GatherView gv = resolve_gather<GATHER>(rg, w_offset, M);                   // MUL_MAT_ID: this expert's rows
+    W += w_offset;
+    if (gv.tok_tile < 0) return;
+    const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
+    if (tok_base >= M) return;
     const int nstages = (int)(K / (16 * F16_KG));
     constexpr int STAGE_BYTES = 16 * F16_KG * 2;                   // bytes of one row per stage
 
@@ -63,7 +68,7 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
 #pragma unroll
     for (int i = 0; i < C::X_PER_T; i++) {
         const int item = tid + i * C::NT;
-        xsrc[i] = ws + (size_t)min(tok_base + item / C::CELLS, M - 1) * ws_stride + 16 * (item % C::CELLS);
+        xsrc[i] = ws + (size_t)gv.act_row(min(tok_base + item / C::CELLS, M - 1)) * ws_stride + 16 * (item % C::CELLS);
     }
     u32x4 wq[C::W_PER_T], xq[C::X_PER_T];
 
@@ -128,10 +133,11 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
         for (int c = 0; c < TN; c++) {
             const int64_t tok = tok_base + (wc * TN + c) * 32 + l32;
             if (tok >= M) continue;
+            const int64_t orow = gv.out_row(tok);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int64_t row = row_base + (wr * TM + a) * 32 + 8 * g + 4 * half;
-                float *dst = y + (size_t)tok * ldy + row;
+                float *dst = y + (size_t)orow * ldy + row;
                 if (row + 3 < N && (((uintptr_t)dst) & 15) == 0) {
                     *reinterpret_cast<float4 *>(dst) = make_float4(acc[a][c][4 * g], acc[a][c][4 * g + 1], acc[a][c][4 * g + 2], acc[a][c][4 * g + 3]);
                 } else {
@@ -146,32 +152,37 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
 // rows must be 16-byte aligned (the weight alignment rule of the C-ABI) and K a multiple of the 64-value stage
 bool gemm_f16_supported(int64_t K, int64_t N, int64_t n) { return K >= 64 && K % (16 * F16_KG) == 0 && N >= 1 && n >= 32; }
 
-template <int TM, int TN, int WR, int WC, int OCC>
+template <int TM, int TN, int WR, int WC, int OCC, bool GATHER>
 static hipError_t launch_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
     using C = F16Cfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
-    auto kfn = gemm_f16_kernel<TM, TN, WR, WC, OCC>;
+    auto kfn = gemm_f16_kernel<TM, TN, WR, WC, OCC, GATHER>;
     static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
-    const TileMap map = make_tile_map(ceil_div(N, C::BM), ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
-    hipLaunchKernelGGL(kfn, dim3(map.grid), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws,
-                       ws_stride, M, y, ldy, map);
+    const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
+    hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg);
     return hipGetLastError();
 }
 
+int gemm_f16_moe_tile_tokens() { return F16Cfg<1, 1, 2, 2>::BN; }      // the 64 x 64 shape serves the expert groups
+
 hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (M <= 0 || N <= 0) return hipSuccess;
+                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as) {
+    if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
+    const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
+        return launch_f16<1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_F16_CFG");
     const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
     switch (cfg) {
-        case 0: return launch_f16<2, 2, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);       // 128 x 128, 4 waves
-        case 1: return launch_f16<1, 1, 2, 2, 4>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);       // 64 x 64, 4 waves
-        case 2: return launch_f16<2, 2, 2, 4, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);       // 128 x 256, 8 waves
-        case 3: return launch_f16<2, 4, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);       // 128 x 256, 4 waves
+        case 0: return launch_f16<2, 2, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 128, 4 waves
+        case 1: return launch_f16<1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 64 x 64, 4 waves
+        case 2: return launch_f16<2, 2, 2, 4, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 256, 8 waves
+        case 3: return launch_f16<2, 4, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 256, 4 waves
         default: return hipErrorInvalidValue;
     }
 }

@@ -282,10 +282,10 @@ struct KqCfg {
 // The two kinds of wave run side by side on every SIMD, so operand expansion (vector pipe, LDS writes, memory
 // latency) overlaps the matrix pipe by construction instead of by instruction scheduling.  Nothing in the loops is
 // conditional: loads past the last stage repeat it, and stores that do not apply go to a per-thread dump slot.
-template <int WT, int WR, int WC, int OCC>
+template <int WT, int WR, int WC, int OCC, bool GATHER>
 __global__ __launch_bounds__((WR * WC + KQ_PRODUCERS) * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
-                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map) {
+                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg) {
     using T = KQ<WT>;
     using C = KqCfg<WT, WR, WC>;
     constexpr int TN = KQ_TN;
@@ -295,8 +295,13 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     const int nstages = (int)(K / QK_K) * 2;
     const TileCoord tc = xcd_tile(blockIdx.x, map);
     if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;        // padding of the tile map
+    size_t w_offset;
+    const GatherView gv = resolve_gather<GATHER>(rg, w_offset, M);                   // MUL_MAT_ID: this expert's rows
+    W += w_offset;
     const int64_t row_base = (int64_t)tc.row_tile * C::BM;
-    const int64_t tok_base = (int64_t)tc.tok_tile * C::BN;
+    if (gv.tok_tile < 0) return;
+    const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
+    if (tok_base >= M) return;
 
     if (wave >= C::NC) {
         // ------------------------------------------------------------------------------------ staging waves
@@ -318,10 +323,10 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
         for (int i = 0; i < C::W_PER_T; i++) wsrc[i] = W + (size_t)min(row_base + ((pt + i * C::NPT) >> 2), N - 1) * nb01;
 #pragma unroll
         for (int i = 0; i < C::X_PER_T; i++)
-            xsrc[i] = ws + (size_t)min(tok_base + ((pt + i * C::NPT) >> 3), M - 1) * ws_stride + 16 * ((pt + i * C::NPT) & 7);
+            xsrc[i] = ws + (size_t)gv.act_row(min(tok_base + ((pt + i * C::NPT) >> 3), M - 1)) * ws_stride + 16 * ((pt + i * C::NPT) & 7);
         // activation scale: thread t < BN for token t; block sums: thread t < 2*BN for token t/2, half t&1
-        const uint8_t *ssrc = ws + (size_t)min(tok_base + min(pt, C::BN - 1), M - 1) * ws_stride;
-        const uint8_t *bsrc = ws + (size_t)min(tok_base + min(pt >> 1, C::BN - 1), M - 1) * ws_stride + off_bs + 16 * (pt & 1);
+        const uint8_t *ssrc = ws + (size_t)gv.act_row(min(tok_base + min(pt, C::BN - 1), M - 1)) * ws_stride;
+        const uint8_t *bsrc = ws + (size_t)gv.act_row(min(tok_base + min(pt >> 1, C::BN - 1), M - 1)) * ws_stride + off_bs + 16 * (pt & 1);
         const int nsb = nstages >> 1;
 
         auto fetch_w = [&](Wts &R, int sb_wanted) {
@@ -522,10 +527,11 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     for (int c = 0; c < TN; c++) {
         const int64_t tok = tok_base + n0 + c * 32 + l32;
         if (tok >= M) continue;
+        const int64_t orow = gv.out_row(tok);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const int64_t row = row_base + r0 + 8 * g + 4 * half;
-            float *dst = y + (size_t)tok * ldy + row;
+            float *dst = y + (size_t)orow * ldy + row;
             if (row + 3 < N && (((uintptr_t)dst) & 15) == 0) {
                 *reinterpret_cast<float4 *>(dst) = make_float4(out[c][4 * g], out[c][4 * g + 1], out[c][4 * g + 2], out[c][4 * g + 3]);
             } else {
@@ -544,46 +550,52 @@ bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n) {
     return n >= ((N * K >= (int64_t)48 << 20) ? 16 : 32);
 }
 
-template <int WT, int WR, int WC, int OCC>
+template <int WT, int WR, int WC, int OCC, bool GATHER>
 static hipError_t launch_kq(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
     using C = KqCfg<WT, WR, WC>;
     const size_t lds_bytes = C::TOTAL;
     if ((int64_t)lds_bytes > lim.max_lds_per_block) return hipErrorInvalidValue;
-    auto kfn = gemm_kq_kernel<WT, WR, WC, OCC>;
+    auto kfn = gemm_kq_kernel<WT, WR, WC, OCC, GATHER>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     // one workgroup per CU: 32 workgroups run on an XCD at a time
-    const TileMap map = make_tile_map(ceil_div(N, C::BM), ceil_div(M, C::BN), 32);
-    hipLaunchKernelGGL(kfn, dim3(map.grid), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)ws,
-                       ws_stride, M, y, ldy, map);
+    const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32);
+    hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg);
     return hipGetLastError();
 }
 
 template <int WT>
 static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                                 int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                                 int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg,
+                                 int64_t n_as) {
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
     // 128 rows x 128 tokens per workgroup when that gives every CU one, else 64 x 128.  (CHIP_GEMM_KQ_CFG selects a
     // shape by hand.)
+    if (rg.perm)                                                                     // expert groups: 64 x 128 tiles
+        return launch_kq<WT, 2, 2, 2, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_KQ_CFG");
     const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 2);
     switch (cfg) {
-        case 0: return launch_kq<WT, 4, 2, 3>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 128 x 128, 8 + 4 waves
-        case 1: return launch_kq<WT, 4, 1, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 128 x 64, 4 + 4 waves
-        case 2: return launch_kq<WT, 2, 2, 2>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);      // 64 x 128, 4 + 4 waves
+        case 0: return launch_kq<WT, 4, 2, 3, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 128 x 128, 8 + 4 waves
+        case 1: return launch_kq<WT, 4, 1, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 128 x 64, 4 + 4 waves
+        case 2: return launch_kq<WT, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 64 x 128, 4 + 4 waves
         default: return hipErrorInvalidValue;
     }
 }
 
+int gemm_kq_moe_tile_tokens() { return KqCfg<T_Q4_K, 2, 2>::BN; }      // the 64 x 128 shape serves the expert groups
+
 hipError_t launch_gemm_kq(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                          int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (M <= 0 || N <= 0) return hipSuccess;
+                          int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as) {
+    if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
+    const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     switch (wtype) {
-        case T_Q4_K: return launch_kq_type<T_Q4_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_Q5_K: return launch_kq_type<T_Q5_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
-        case T_Q6_K: return launch_kq_type<T_Q6_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);
+        case T_Q4_K: return launch_kq_type<T_Q4_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q5_K: return launch_kq_type<T_Q5_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q6_K: return launch_kq_type<T_Q6_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
         default: return hipErrorInvalidValue;
     }
 }

@@ -187,7 +187,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             const lm_ggml_tensor *w = node->src[0], *x = node->src[1], *ids = node->src[2];
             const int64_t K = w->ne[0], N = w->ne[1], n_used = ids->ne[0], n_tokens = ids->ne[1];
             if (N == 0 || n_used == 0 || n_tokens == 0) continue;
-            if (!grow_workspace(c, chip_mul_mat_workspace_size(w->type, K, n_tokens * x->ne[1]))) return LM_GGML_STATUS_ALLOC_FAILED;
+            if (!grow_workspace(c, chip_mul_mat_id_workspace_size(w->type, K, w->ne[2], n_used, n_tokens, x->ne[1]))) return LM_GGML_STATUS_ALLOC_FAILED;
             const int rc = chip_mul_mat_id(w->type, w->data, w->nb[1], w->nb[2], K, N, w->ne[2], (const float *)x->data,
                                            (int64_t)(x->nb[1] / 4), x->ne[1], (const int32_t *)ids->data, (int64_t)(ids->nb[1] / 4),
                                            n_used, n_tokens, (float *)node->data, (int64_t)(node->nb[1] / 4), c->workspace,

@@ -75,6 +75,48 @@ __device__ __forceinline__ TileCoord xcd_tile(unsigned wg, const TileMap &m) {
     return t;
 }
 
+// Row gather of LM_GGML_OP_MUL_MAT_ID for the GEMM kernels (reference ggml-cpu/ggml-cpu.c:1460-1710 groups the (token,
+// slot) pairs by expert the same way: matrix_rows / matrix_row_counts).  With perm set, blockIdx.y walks a list of
+// token tiles built on the device: entry i = expert | tile << 12 says "pairs perm[offsets[e] + tile * BN ...] of expert
+// e"; entries past tiles[-1] (the count, stored in front of the list) do not exist.  The expert's matrix is
+// W + e * nb02; pair p reads activation row (p / n_used) * ne11 + (p % n_used) % ne11 and writes output row p.
+// perm == nullptr: plain MUL_MAT.
+constexpr int MOE_EXPERT_BITS = 12;
+struct RowGather {
+    const int32_t *perm, *offsets, *tiles;     // tiles[0] = number of entries, entries from tiles[1]
+    int32_t n_used, ne11;
+    size_t nb02;
+};
+struct GatherView {                // resolved once per workgroup
+    const int32_t *list;           // this expert's pairs, or nullptr
+    int32_t n_used, ne11;
+    int32_t tok_tile;              // grouped mode: the token tile of this workgroup, -1 = nothing to do
+    __device__ __forceinline__ int64_t act_row(int64_t tok) const {
+        if (!list) return tok;
+        const int32_t p = list[tok];
+        return (int64_t)(p / n_used) * ne11 + (p % n_used) % ne11;
+    }
+    __device__ __forceinline__ int64_t out_row(int64_t tok) const { return list ? (int64_t)list[tok] : tok; }
+};
+// Sets the token count M and the byte offset of the weight matrix to the expert's and returns its view.  GATHER is a
+// template argument of the kernels so that the plain MUL_MAT instantiations carry none of this.
+template <bool GATHER>
+__device__ __forceinline__ GatherView resolve_gather(const RowGather &rg, size_t &w_offset, int64_t &M) {
+    GatherView v{nullptr, rg.n_used, rg.ne11, 0};
+    w_offset = 0;
+    if constexpr (GATHER) {
+        if ((int)blockIdx.y >= rg.tiles[0]) { v.tok_tile = -1; return v; }
+        const int32_t d = rg.tiles[1 + blockIdx.y];
+        const int e = d & ((1 << MOE_EXPERT_BITS) - 1);
+        const int32_t off = rg.offsets[e];
+        M = rg.offsets[e + 1] - off;
+        v.list = rg.perm + off;
+        v.tok_tile = d >> MOE_EXPERT_BITS;
+        w_offset = (size_t)e * rg.nb02;
+    }
+    return v;
+}
+
 // quantize.hip
 hipError_t launch_quantize(int act_type, bool split, const float *x, int64_t ldx, int64_t n, int64_t K, void *y,
                            size_t y_stride, hipStream_t st);
@@ -111,17 +153,31 @@ hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t 
 // IQ4_NL), activations in the split Q8_0 workspace layout.  _supported includes the token count from which it pays.
 bool       gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n);
 hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                             int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+                             int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st,
+                             const RowGather *rg = nullptr, int64_t n_as = 1);
 
 // gemm_f16.hip: fp16-MFMA prefill GEMM over F16 weights, activations as fp16 in the workspace.
 bool       gemm_f16_supported(int64_t K, int64_t N, int64_t n);
 hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t n,
-                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rg = nullptr,
+                           int64_t n_as = 1);
 
 // gemm_kquant.hip: int8-MFMA prefill GEMM over Q4_K / Q5_K / Q6_K weights, activations in the split Q8_K workspace
 // layout; the integer sub-block scales ride in the MFMA operand.
 bool       gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n);
 hipError_t launch_gemm_kq(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                          int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+                          int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rg = nullptr,
+                          int64_t n_as = 1);
+// In the three GEMM launchers: with rg, n_as is the number of token-tile slots the grid provides in y (an upper bound
+// of the tile list's length) and n is ignored; gemm_*_moe_tile_tokens gives the tile height the list must be built for.
+
+// moe_group.hip: counting sort of MUL_MAT_ID's (token, slot) pairs by expert into offsets[n_as + 1] / perm[pairs].
+// tiles[0] = number of token tiles, tiles[1 + i] = expert | tile << 12 for tiles of `tile_tokens` pairs.
+bool       moe_group_supported(int64_t n_as, int64_t pairs);
+hipError_t launch_moe_group(const int32_t *ids, int64_t ids_stride, int64_t n_used, int64_t pairs, int64_t n_as,
+                            int tile_tokens, int32_t *offsets, int32_t *perm, int32_t *tiles, hipStream_t st);
+int        gemm_blk32_moe_tile_tokens();
+int        gemm_kq_moe_tile_tokens();
+int        gemm_f16_moe_tile_tokens();
 
 }  // namespace chip

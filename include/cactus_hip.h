@@ -139,9 +139,13 @@ CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, i
  * ids_stride elements between tokens), dst = y (F32 [N, n_used, n_tokens], row stride ldy elements, rows adjacent):
  *     y[t][s][r] = vec_dot(row r of expert ids[t][s], quantize(x[t][s % ne11]))
  * ne11 is 1 (all slots of a token share one activation row) or n_used.  Every id must lie in [0, n_as); a pair
- * with an id outside is left unwritten (the reference asserts).  The workspace holds the n_tokens * ne11 quantized
- * rows: at least chip_mul_mat_workspace_size(type, K, n_tokens * ne11) bytes.  Alignment rules as chip_mul_mat;
- * nb02 obeys the rule of nb01.  Each (token, slot) pair runs as a one-token GEMV on its expert. */
+ * with an id outside is left unwritten (the reference asserts).  The workspace (at least
+ * chip_mul_mat_id_workspace_size bytes) holds the n_tokens * ne11 quantized rows and the pair lists.  Alignment rules
+ * as chip_mul_mat; nb02 obeys the rule of nb01.  Below 64 (token, slot) pairs each pair runs as a one-token GEMV on
+ * its expert; from 64 on the pairs are grouped by expert on the device (the reference's matrix_rows) and every
+ * expert's group runs through the MFMA GEMM of the weight type. */
+CHIP_API size_t chip_mul_mat_id_workspace_size(int type, int64_t K, int64_t n_as, int64_t n_used, int64_t n_tokens,
+                                               int64_t ne11);
 CHIP_API int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t n_as,
                              const float *x, int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride,
                              int64_t n_used, int64_t n_tokens, float *y, int64_t ldy,

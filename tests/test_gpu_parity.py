@@ -451,6 +451,40 @@ def test_mul_mat_id_is_mul_mat_on_the_chosen_expert(dev, orc):
             assert np.array_equal(y[t, s], one[0])
 
 
+@pytest.mark.parametrize("wt", O.WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("n_tokens,ne11,n_as", [(16, 1, 8), (50, 4, 6), (130, 1, 32)])
+def test_mul_mat_id_prefill_grouped_by_expert(dev, orc, wt, n_tokens, ne11, n_as):
+    """64 (token, slot) pairs and more: grouped by expert on the device and run through the GEMMs.  Uneven loads: one
+    expert gets a pair from every token, some get none."""
+    K, N, n_used = 512, 150, 4
+    rng = np.random.default_rng(900 + wt + n_tokens)
+    W = np.stack([orc.quantize_weights(wt, common.weights_f32(900 + wt + e, N, K)) for e in range(n_as)])
+    x = common.activations_f32(901 + wt, n_tokens * ne11, K).reshape(n_tokens, ne11, K)
+    pool = np.arange(1, n_as - 2)                                    # experts n_as-2 and n_as-1 stay idle
+    ids = np.stack([np.concatenate(([0], rng.permutation(pool)[:n_used - 1])) for _ in range(n_tokens)]).astype(np.int32)
+    ref = orc.mul_mat_id(wt, W, x, ids, nthreads=8, want=("sum_abs",))
+    y = dev.mul_mat_id(wt, W, x, ids)
+    check_outputs(y, ref["y"], ref["sum_abs"], "mul_mat_id grouped")
+
+
+def test_mul_mat_id_grouped_matches_pairwise_and_skips_bad_ids(dev, orc):
+    """The grouped GEMM path and the pair-by-pair GEMV path agree within the tolerance on the same inputs (first 15
+    tokens alone take the GEMV path), and an id outside [0, n_as) leaves exactly its own output row unwritten."""
+    wt, K, N, n_as, n_used, n_tokens = O.Q4_K, 1024, 96, 8, 4, 40
+    W, x, ids = moe_case(orc, wt, K, N, n_as, n_used, n_tokens, 1, 77)
+    ids[7, 2] = n_as + 5
+    ids[9, 0] = -1
+    y = dev.mul_mat_id(wt, W, x, ids)
+    bad = np.zeros((n_tokens, n_used), bool)
+    bad[7, 2] = bad[9, 0] = True
+    assert np.isnan(y[bad]).all() and np.isfinite(y[~bad]).all()
+    y15 = dev.mul_mat_id(wt, W, x[:15], ids[:15])
+    good = ~bad[:15]
+    ok_ids = np.where(bad, 0, ids)
+    sa = orc.mul_mat_id(wt, W, x, ok_ids, nthreads=8, want=("sum_abs",))["sum_abs"]
+    assert (np.abs(y[:15][good].astype(np.float64) - y15[good]) <= 2 * REL_TOL * sa[:15][good]).all()
+
+
 def test_mul_mat_id_argument_errors(dev, orc):
     import cactus_amd as ca
     L = dev.lib
@@ -458,7 +492,8 @@ def test_mul_mat_id_argument_errors(dev, orc):
     W, x, ids = moe_case(orc, wt, K, N, 2, 2, 1, 1, 5)
     nb01 = dev.row_size(wt, K)
     dW, dx, di, dy = dev.to_device(W), dev.to_device(x), dev.to_device(ids), dev.alloc(2 * N * 4)
-    wsz = L.chip_mul_mat_workspace_size(wt, K, 1)
+    wsz = L.chip_mul_mat_id_workspace_size(wt, K, 2, 2, 1, 1)
+    assert wsz > L.chip_mul_mat_workspace_size(wt, K, 1)
     ws = dev.alloc(wsz)
     call = lambda **kw: L.chip_mul_mat_id(*[kw.get(k, v) for k, v in (
         ("type", wt), ("W", dW.ptr), ("nb01", nb01), ("nb02", N * nb01), ("K", K), ("N", N), ("n_as", 2), ("x", dx.ptr),
