@@ -279,6 +279,41 @@ def bench_extra(dev, hip, trace=True):
     moe_case("moe_q4_K_128x8_768x2048_n512", ca.Q4_K, 128, 8, 768, 2048, 512)
     moe_case("moe_q4_K_8x2_14336x4096_n512", ca.Q4_K, 8, 2, 14336, 4096, 512)
 
+    # weight upload: one synchronous copy from pageable memory (what set_tensor does) against the loader's protocol of
+    # four pinned 1 MB staging buffers with an event each (chunked set_tensor_async)
+    def upload_case():
+        total, chunk, nbuf = 256 << 20, 1 << 20, 4
+        src = rng.integers(0, 256, total, dtype=np.uint8)
+        dst = dev.alloc(total)
+        t0 = time.perf_counter()
+        dev.check(L.chip_memcpy_h2d(dst.ptr, src.ctypes.data, total, None))
+        t_sync = time.perf_counter() - t0
+        pins, evs = [], []
+        for _ in range(nbuf):
+            p_, e_ = C.c_void_p(), C.c_void_p()
+            dev.check(L.chip_host_malloc(C.byref(p_), chunk))
+            dev.check(L.chip_event_create(C.byref(e_)))
+            pins.append(p_)
+            evs.append(e_)
+        t0 = time.perf_counter()
+        for i, off in enumerate(range(0, total, chunk)):
+            b_ = i % nbuf
+            dev.check(L.chip_event_synchronize(evs[b_]))
+            C.memmove(pins[b_], src.ctypes.data + off, chunk)                     # the loader's file read
+            dev.check(L.chip_memcpy_h2d(dst.ptr + off, pins[b_], chunk, st))
+            dev.check(L.chip_event_record(evs[b_], st))
+        dev.sync(st)
+        t_async = time.perf_counter() - t0
+        ok = bool(np.array_equal(dst.download(np.uint8, 1 << 20, total - (1 << 20)), src[-(1 << 20):]))
+        for p_, e_ in zip(pins, evs):
+            L.chip_host_free(p_)
+            L.chip_event_destroy(e_)
+        dst.free()
+        out["upload_256MB"] = {"sync_pageable_GBps": round(total / t_sync / 1e9, 2),
+                               "async_pinned_chunks_GBps": round(total / t_async / 1e9, 2), "verified": ok}
+
+    upload_case()
+
     if trace:
         out.update(bench_trace(dev, hip, st, rng))
         out["mfma_i8_measured_peak"] = measured_mfma_peak()

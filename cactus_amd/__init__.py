@@ -30,7 +30,8 @@ WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, F16)
 EXPORTS = (
     "chip_init", "chip_device_count", "chip_get_device_info", "chip_error_string", "chip_malloc", "chip_free",
     "chip_memcpy_h2d", "chip_memcpy_d2h", "chip_memcpy_d2d", "chip_memset", "chip_stream_create",
-    "chip_stream_destroy", "chip_stream_synchronize", "chip_block_elems", "chip_block_bytes", "chip_row_size",
+    "chip_stream_destroy", "chip_stream_synchronize", "chip_host_malloc", "chip_host_free", "chip_event_create",
+    "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
@@ -75,6 +76,13 @@ def load_library(path=KERNEL_LIB):
     L.chip_stream_create.argtypes = [C.POINTER(vp)]
     L.chip_stream_destroy.argtypes = [vp]
     L.chip_stream_synchronize.argtypes = [vp]
+    L.chip_host_malloc.argtypes = [C.POINTER(vp), sz]
+    L.chip_host_free.argtypes = [vp]
+    L.chip_event_create.argtypes = [C.POINTER(vp)]
+    L.chip_event_destroy.argtypes = [vp]
+    L.chip_event_record.argtypes = [vp, vp]
+    L.chip_event_synchronize.argtypes = [vp]
+    L.chip_stream_wait_event.argtypes = [vp, vp]
     L.chip_block_elems.argtypes = [i32]
     L.chip_block_bytes.restype = sz
     L.chip_block_bytes.argtypes = [i32]

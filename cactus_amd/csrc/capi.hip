@@ -168,6 +168,28 @@ int chip_stream_create(void **stream) {
 int chip_stream_destroy(void *stream) { return stream ? hip_rc(hipStreamDestroy((hipStream_t)stream)) : CHIP_OK; }
 int chip_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((hipStream_t)stream)); }
 
+int chip_host_malloc(void **ptr, size_t bytes) {
+    if (!ptr) return CHIP_EINVAL;
+    *ptr = nullptr;
+    return hip_rc(hipHostMalloc(ptr, bytes ? bytes : 16, hipHostMallocDefault));        // pinned, allocated (never registered)
+}
+int chip_host_free(void *ptr) { return ptr ? hip_rc(hipHostFree(ptr)) : CHIP_OK; }
+int chip_event_create(void **event) {
+    if (!event) return CHIP_EINVAL;
+    hipEvent_t e = nullptr;
+    hipError_t rc = hipEventCreateWithFlags(&e, hipEventDisableTiming);
+    *event = (void *)e;
+    return hip_rc(rc);
+}
+int chip_event_destroy(void *event) { return event ? hip_rc(hipEventDestroy((hipEvent_t)event)) : CHIP_OK; }
+int chip_event_record(void *event, void *stream) {
+    return event ? hip_rc(hipEventRecord((hipEvent_t)event, (hipStream_t)stream)) : CHIP_EINVAL;
+}
+int chip_event_synchronize(void *event) { return event ? hip_rc(hipEventSynchronize((hipEvent_t)event)) : CHIP_EINVAL; }
+int chip_stream_wait_event(void *stream, void *event) {
+    return event ? hip_rc(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0)) : CHIP_EINVAL;
+}
+
 int chip_block_elems(int type) {
     switch (type) {
         case T_F32: case T_F16: return 1;

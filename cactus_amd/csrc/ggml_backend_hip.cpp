@@ -4,8 +4,10 @@
 //   reg "HIP"  ->  device "HIP0" (ACCEL by default: a weights-only co-processor, like the AMX extra buffer type,
 //                  reference ggml-cpu/amx/amx.cpp:141-174; CACTUS_HIP_DEVICE_TYPE=GPU switches)
 //              ->  buffer type "HIP": hipMalloc'd buffers, tensors at base + offset, GGUF blocks kept verbatim
-//              ->  backend "HIP": one stream; graph_compute runs MUL_MAT (F32 activations x Q4_0/Q8_0/Q4_K/Q6_K
-//                  weights living in a HIP buffer) and skips view ops.
+//              ->  buffer type "HIP_Host": pinned host memory (the staging buffers of the loader's async upload)
+//              ->  backend "HIP": one stream; graph_compute runs MUL_MAT / MUL_MAT_ID (F32 activations x block-quantized
+//                  or F16 weights living in a HIP buffer) and skips view ops; set/get_tensor_async and events on
+//                  that stream.
 // No C++ exception crosses the vtables; failures are NULL returns or LM_GGML_STATUS_FAILED.
 #include "../../include/cactus_hip.h"
 #include "../../include/ggml_abi_mirror.h"
@@ -108,6 +110,59 @@ lm_ggml_backend_buffer_t buft_alloc(lm_ggml_backend_buffer_type_t buft, size_t s
 size_t buft_alignment(lm_ggml_backend_buffer_type_t) { return 256; }       // rows stay 16-byte aligned for the kernels
 bool buft_is_host(lm_ggml_backend_buffer_type_t) { return false; }
 
+// ------------------------------------------------------------------------------------------------ pinned host buffer type
+// What lm_ggml_backend_dev_host_buffer_type returns: host memory the GPU can copy from without staging, so that
+// set_tensor_async overlaps with the caller (the loader reads the next chunk of the file meanwhile).
+lm_ggml_backend_buffer_type_t hip_host_buffer_type();
+void hbuf_free(lm_ggml_backend_buffer_t buffer) {
+    buffer_ctx *c = (buffer_ctx *)buffer->context;
+    chip_host_free(c->base);
+    delete c;
+}
+void hbuf_memset_tensor(lm_ggml_backend_buffer_t, lm_ggml_tensor *t, uint8_t value, size_t offset, size_t size) {
+    std::memset((char *)t->data + offset, value, size);
+}
+void hbuf_set_tensor(lm_ggml_backend_buffer_t, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
+    std::memcpy((char *)t->data + offset, data, size);
+}
+void hbuf_get_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *t, void *data, size_t offset, size_t size) {
+    std::memcpy(data, (const char *)t->data + offset, size);
+}
+bool hbuf_cpy_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *src, lm_ggml_tensor *dst) {
+    if (!is_host_buffer(src->buffer)) return false;
+    std::memcpy(dst->data, src->data, lm_ggml_nbytes(src));
+    return true;
+}
+void hbuf_clear(lm_ggml_backend_buffer_t buffer, uint8_t value) {
+    buffer_ctx *c = (buffer_ctx *)buffer->context;
+    std::memset(c->base, value, c->size);
+}
+const lm_ggml_backend_buffer_i k_host_buffer_i = {
+    /* free_buffer   */ hbuf_free,
+    /* get_base      */ buf_get_base,
+    /* init_tensor   */ nullptr,
+    /* memset_tensor */ hbuf_memset_tensor,
+    /* set_tensor    */ hbuf_set_tensor,
+    /* get_tensor    */ hbuf_get_tensor,
+    /* cpy_tensor    */ hbuf_cpy_tensor,
+    /* clear         */ hbuf_clear,
+    /* reset         */ nullptr,
+};
+const char *hbuft_name(lm_ggml_backend_buffer_type_t) { return "HIP_Host"; }
+lm_ggml_backend_buffer_t hbuft_alloc(lm_ggml_backend_buffer_type_t buft, size_t size) {
+    if (!device_ok()) return nullptr;
+    void *p = nullptr;
+    if (chip_host_malloc(&p, size) != CHIP_OK || !p) {
+        HIP_LOG(LM_GGML_LOG_LEVEL_WARN, "%s: pinned allocation of %zu bytes failed\n", __func__, size);
+        return nullptr;
+    }
+    buffer_ctx *c = new (std::nothrow) buffer_ctx{p, size};
+    if (!c) { chip_host_free(p); return nullptr; }
+    return lm_ggml_backend_buffer_init(buft, k_host_buffer_i, c, size);
+}
+size_t hbuft_alignment(lm_ggml_backend_buffer_type_t) { return 64; }
+bool hbuft_is_host(lm_ggml_backend_buffer_type_t) { return true; }
+
 // ------------------------------------------------------------------------------------------------ backend
 lm_ggml_guid_t hip_guid() {
     static lm_ggml_guid g = {0x63, 0x61, 0x63, 0x74, 0x75, 0x73, 0x2d, 0x68, 0x69, 0x70, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35};
@@ -123,6 +178,21 @@ void backend_free(lm_ggml_backend_t backend) {
     delete backend;
 }
 void backend_synchronize(lm_ggml_backend_t backend) { chip_stream_synchronize(((backend_ctx *)backend->context)->stream); }
+// Asynchronous on the backend's stream, ordered with graph_compute; the host memory must stay untouched until the
+// stream (or an event recorded after the call) has been waited for.
+void backend_set_tensor_async(lm_ggml_backend_t backend, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
+    chip_memcpy_h2d((char *)t->data + offset, data, size, ((backend_ctx *)backend->context)->stream);
+    g_uploaded += size;
+}
+void backend_get_tensor_async(lm_ggml_backend_t backend, const lm_ggml_tensor *t, void *data, size_t offset, size_t size) {
+    chip_memcpy_d2h(data, (const char *)t->data + offset, size, ((backend_ctx *)backend->context)->stream);
+}
+void backend_event_record(lm_ggml_backend_t backend, lm_ggml_backend_event_t event) {
+    chip_event_record(event->context, ((backend_ctx *)backend->context)->stream);
+}
+void backend_event_wait(lm_ggml_backend_t backend, lm_ggml_backend_event_t event) {
+    chip_stream_wait_event(((backend_ctx *)backend->context)->stream, event->context);
+}
 
 bool is_view_op(int op) {
     return op == LM_GGML_OP_NONE || op == LM_GGML_OP_RESHAPE || op == LM_GGML_OP_VIEW || op == LM_GGML_OP_PERMUTE ||
@@ -221,8 +291,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
 const lm_ggml_backend_i k_backend_i = {
     /* get_name           */ backend_name,
     /* free               */ backend_free,
-    /* set_tensor_async   */ nullptr,
-    /* get_tensor_async   */ nullptr,
+    /* set_tensor_async   */ backend_set_tensor_async,
+    /* get_tensor_async   */ backend_get_tensor_async,
     /* cpy_tensor_async   */ nullptr,
     /* synchronize        */ backend_synchronize,
     /* graph_plan_create  */ nullptr,
@@ -230,8 +300,8 @@ const lm_ggml_backend_i k_backend_i = {
     /* graph_plan_update  */ nullptr,
     /* graph_plan_compute */ nullptr,
     /* graph_compute      */ backend_graph_compute,
-    /* event_record       */ nullptr,
-    /* event_wait         */ nullptr,
+    /* event_record       */ backend_event_record,
+    /* event_wait         */ backend_event_wait,
 };
 
 // ------------------------------------------------------------------------------------------------ device
@@ -255,7 +325,7 @@ void dev_props(lm_ggml_backend_dev_t dev, lm_ggml_backend_dev_props *props) {
     props->description = dev_description(dev);
     props->type = dev_type(dev);
     dev_memory(dev, &props->memory_free, &props->memory_total);
-    props->caps = {/* async */ false, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false};
+    props->caps = {/* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ true};
 }
 lm_ggml_backend_t dev_init_backend(lm_ggml_backend_dev_t dev, const char *) {
     if (!device_ok()) return nullptr;
@@ -267,6 +337,21 @@ lm_ggml_backend_t dev_init_backend(lm_ggml_backend_dev_t dev, const char *) {
     return b;
 }
 lm_ggml_backend_buffer_type_t dev_buffer_type(lm_ggml_backend_dev_t) { return hip_buffer_type(); }
+lm_ggml_backend_buffer_type_t dev_host_buffer_type(lm_ggml_backend_dev_t) { return hip_host_buffer_type(); }
+lm_ggml_backend_event_t dev_event_new(lm_ggml_backend_dev_t dev) {
+    if (!device_ok()) return nullptr;
+    void *e = nullptr;
+    if (chip_event_create(&e) != CHIP_OK || !e) return nullptr;
+    lm_ggml_backend_event *ev = new (std::nothrow) lm_ggml_backend_event{dev, e};
+    if (!ev) chip_event_destroy(e);
+    return ev;
+}
+void dev_event_free(lm_ggml_backend_dev_t, lm_ggml_backend_event_t event) {
+    if (!event) return;
+    chip_event_destroy(event->context);
+    delete event;
+}
+void dev_event_synchronize(lm_ggml_backend_dev_t, lm_ggml_backend_event_t event) { chip_event_synchronize(event->context); }
 
 bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     if (is_view_op(op->op)) return true;
@@ -288,14 +373,14 @@ const lm_ggml_backend_device_i k_device_i = {
     /* get_props            */ dev_props,
     /* init_backend         */ dev_init_backend,
     /* get_buffer_type      */ dev_buffer_type,
-    /* get_host_buffer_type */ nullptr,
+    /* get_host_buffer_type */ dev_host_buffer_type,
     /* buffer_from_host_ptr */ nullptr,
     /* supports_op          */ dev_supports_op,
     /* supports_buft        */ dev_supports_buft,
     /* offload_op           */ nullptr,
-    /* event_new            */ nullptr,
-    /* event_free           */ nullptr,
-    /* event_synchronize    */ nullptr,
+    /* event_new            */ dev_event_new,
+    /* event_free           */ dev_event_free,
+    /* event_synchronize    */ dev_event_synchronize,
 };
 
 // ------------------------------------------------------------------------------------------------ reg
@@ -311,6 +396,16 @@ const lm_ggml_backend_reg_i k_reg_i = {reg_name, reg_device_count, reg_get_devic
 lm_ggml_backend_dev_t hip_device() {
     static lm_ggml_backend_device dev = {k_device_i, lm_ggml_backend_hip_reg(), nullptr};
     return &dev;
+}
+lm_ggml_backend_buffer_type_t hip_host_buffer_type() {
+    static lm_ggml_backend_buffer_type buft = {
+        {hbuft_name, hbuft_alloc, hbuft_alignment, /* get_max_size */ nullptr, /* get_alloc_size */ nullptr, hbuft_is_host},
+        /* device  */ nullptr,
+        /* context */ nullptr,
+    };
+    static std::once_flag once;
+    std::call_once(once, [] { buft.device = hip_device(); });
+    return &buft;
 }
 lm_ggml_backend_buffer_type_t hip_buffer_type() {
     static lm_ggml_backend_buffer_type buft = {

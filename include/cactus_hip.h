@@ -77,6 +77,18 @@ CHIP_API int         chip_stream_create(void **stream);
 CHIP_API int         chip_stream_destroy(void *stream);
 CHIP_API int         chip_stream_synchronize(void *stream);
 
+/* ---- what a ggml device with async uploads needs (reference ggml-backend-impl.h:100-116 set/get_tensor_async,
+ * event_record/event_wait; :160 get_host_buffer_type; :176-178 event_new/free/synchronize; used by the model loader's
+ * chunked upload, llama-model-loader.cpp:905-1064) ----
+ * chip_memcpy_h2d / _d2h with a stream are asynchronous; they overlap with the host only from pinned memory. */
+CHIP_API int chip_host_malloc(void **ptr, size_t bytes);          /* pinned host memory (hipHostMalloc) */
+CHIP_API int chip_host_free(void *ptr);
+CHIP_API int chip_event_create(void **event);
+CHIP_API int chip_event_destroy(void *event);
+CHIP_API int chip_event_record(void *event, void *stream);        /* the event completes when the stream reaches this point */
+CHIP_API int chip_event_synchronize(void *event);                 /* host waits */
+CHIP_API int chip_stream_wait_event(void *stream, void *event);   /* later work of the stream waits */
+
 /* ---- layout facts ---- */
 /* lm_ggml_blck_size / lm_ggml_type_size / lm_ggml_row_size (ggml.c:1186-1200) for the types above; 0 if unknown */
 CHIP_API int    chip_block_elems(int type);

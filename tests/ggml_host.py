@@ -13,6 +13,15 @@ vp, i64, i32, sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
 EVAL_CB = C.CFUNCTYPE(C.c_bool, C.c_int, vp, vp, vp)
 
 
+class DevCaps(C.Structure):
+    _fields_ = [("async_", C.c_bool), ("host_buffer", C.c_bool), ("buffer_from_host_ptr", C.c_bool), ("events", C.c_bool)]
+
+
+class DevProps(C.Structure):            # struct lm_ggml_backend_dev_props (reference ggml-backend.h:152-159)
+    _fields_ = [("name", C.c_char_p), ("description", C.c_char_p), ("memory_free", C.c_size_t),
+                ("memory_total", C.c_size_t), ("type", C.c_int), ("caps", DevCaps)]
+
+
 class Host:
     def __init__(self):
         self.ref = O.Reference()                       # RTLD_GLOBAL, fp16 table initialised
@@ -73,6 +82,27 @@ class Host:
         L.lm_ggml_backend_sched_reset.argtypes = [vp]
         L.lm_ggml_backend_compare_graph_backend.restype = C.c_bool
         L.lm_ggml_backend_compare_graph_backend.argtypes = [vp, vp, vp, EVAL_CB, vp]
+        L.lm_ggml_backend_dev_get_props.argtypes = [vp, C.POINTER(DevProps)]
+        L.lm_ggml_backend_dev_host_buffer_type.restype = vp
+        L.lm_ggml_backend_dev_host_buffer_type.argtypes = [vp]
+        L.lm_ggml_backend_buft_alloc_buffer.restype = vp
+        L.lm_ggml_backend_buft_alloc_buffer.argtypes = [vp, sz]
+        L.lm_ggml_backend_buft_get_device.restype = vp
+        L.lm_ggml_backend_buft_get_device.argtypes = [vp]
+        L.lm_ggml_backend_buffer_get_base.restype = vp
+        L.lm_ggml_backend_buffer_get_base.argtypes = [vp]
+        L.lm_ggml_backend_buffer_get_type.restype = vp
+        L.lm_ggml_backend_buffer_get_type.argtypes = [vp]
+        L.lm_ggml_backend_buffer_is_host.restype = C.c_bool
+        L.lm_ggml_backend_buffer_is_host.argtypes = [vp]
+        L.lm_ggml_backend_event_new.restype = vp
+        L.lm_ggml_backend_event_new.argtypes = [vp]
+        L.lm_ggml_backend_event_free.argtypes = [vp]
+        L.lm_ggml_backend_event_record.argtypes = [vp, vp]
+        L.lm_ggml_backend_event_synchronize.argtypes = [vp]
+        L.lm_ggml_backend_event_wait.argtypes = [vp, vp]
+        L.lm_ggml_backend_tensor_set_async.argtypes = [vp, vp, vp, sz, sz]
+        L.lm_ggml_backend_tensor_get_async.argtypes = [vp, vp, vp, sz, sz]
         L.lm_ggml_add.restype = vp
         L.lm_ggml_add.argtypes = [vp, vp, vp]
         L.lm_ggml_set_name.restype = vp

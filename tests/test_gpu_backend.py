@@ -283,3 +283,79 @@ def test_mul_mat_id_node(host, orc, wt, n_tokens, ne11):
     L.lm_ggml_backend_free(cpu)
     L.lm_ggml_backend_free(be)
     L.lm_ggml_free(ctx)
+
+
+def test_async_upload_protocol_of_the_model_loader(host, orc):
+    """What llama_model_loader::load_all_data does when a device reports async + host_buffer + events
+    (reference llama-model-loader.cpp:905-1064): four pinned 1 MB staging buffers with one event each, the tensor
+    uploaded chunk by chunk with set_tensor_async, the event of a buffer waited for before the buffer is refilled."""
+    from ggml_host import DevProps
+    L = host.L
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    props = DevProps()
+    L.lm_ggml_backend_dev_get_props(dev, C.byref(props))
+    assert props.caps.async_ and props.caps.host_buffer and props.caps.events and not props.caps.buffer_from_host_ptr
+    assert props.name == b"HIP0" and props.memory_total > 200 << 30
+    host_buft = L.lm_ggml_backend_dev_host_buffer_type(dev)
+    assert host_buft and L.lm_ggml_backend_buft_name(host_buft) == b"HIP_Host" and L.lm_ggml_backend_buft_is_host(host_buft)
+    assert L.lm_ggml_backend_buft_get_device(host_buft) == dev
+    assert not L.lm_ggml_backend_dev_supports_buft(dev, host_buft)      # operands of the kernels live in device memory
+
+    wt, K, N, n = O.Q4_K, 4096, 3000, 3                                  # 6.9 MB of weights: 7 chunks
+    wq = orc.quantize_weights(wt, common.weights_f32(77, N, K))
+    x = common.activations_f32(78, n, K)
+    ctx = host.context()
+    a = host.tensor_2d(ctx, wt, K, N, "w")
+    b = host.tensor_2d(ctx, O.F32, K, n, "x")
+    c = L.lm_ggml_mul_mat(ctx, a, b)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, c)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    assert L.lm_ggml_backend_buffer_get_type(buf) == L.lm_ggml_backend_dev_buffer_type(dev)
+
+    n_buffers, chunk = 4, 1 << 20
+    bufs = [L.lm_ggml_backend_buft_alloc_buffer(host_buft, chunk) for _ in range(n_buffers)]
+    assert all(bufs) and all(L.lm_ggml_backend_buffer_is_host(hb) for hb in bufs)
+    ptrs = [L.lm_ggml_backend_buffer_get_base(hb) for hb in bufs]
+    events = [L.lm_ggml_backend_event_new(dev) for _ in range(n_buffers)]
+    assert all(events)
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    raw = wq.reshape(-1)
+    done, idx = 0, 0
+    while done < raw.size:
+        size = min(chunk, raw.size - done)
+        L.lm_ggml_backend_event_synchronize(events[idx])                 # the buffer's previous upload has finished
+        C.memmove(ptrs[idx], raw[done:done + size].ctypes.data, size)    # "file->read_raw" into pinned memory
+        L.lm_ggml_backend_tensor_set_async(be, a, ptrs[idx], done, size)
+        L.lm_ggml_backend_event_record(events[idx], be)
+        done += size
+        idx = (idx + 1) % n_buffers
+    for ev in events:
+        L.lm_ggml_backend_event_synchronize(ev)
+    assert np.array_equal(host.get(a, np.uint8, wq.shape), wq)
+
+    # activations through the async path too, compute on the same stream, result read back asynchronously
+    xin = np.ascontiguousarray(x)
+    L.lm_ggml_backend_tensor_set_async(be, b, xin.ctypes.data_as(C.c_void_p), 0, xin.nbytes)
+    assert L.lm_ggml_backend_graph_compute(be, g) == 0
+    y = np.empty((n, N), np.float32)
+    L.lm_ggml_backend_tensor_get_async(be, c, y.ctypes.data_as(C.c_void_p), 0, y.nbytes)
+    # a second backend (stream) waits for the first one's event before it reads the result
+    be2 = L.lm_ggml_backend_dev_init(dev, None)
+    L.lm_ggml_backend_event_record(events[0], be)
+    L.lm_ggml_backend_event_wait(be2, events[0])
+    y2 = np.empty((n, N), np.float32)
+    L.lm_ggml_backend_tensor_get_async(be2, c, y2.ctypes.data_as(C.c_void_p), 0, y2.nbytes)
+    L.lm_ggml_backend_synchronize(be)
+    L.lm_ggml_backend_synchronize(be2)
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("sum_abs",))
+    assert (np.abs(y.astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all() and np.array_equal(y, y2)
+
+    for ev in events:
+        L.lm_ggml_backend_event_free(ev)
+    for hb in bufs:
+        L.lm_ggml_backend_buffer_free(hb)
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_free(be2)
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_free(ctx)
