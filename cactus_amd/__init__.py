@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
-    "chip_mul_mat_id_workspace_size",
+    "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu",
     "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -99,6 +99,10 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
+    L.chip_rms_norm.argtypes = [vp, i64, i64, i64, C.c_float, vp, i64, vp]
+    L.chip_add.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
+    L.chip_mul.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
+    L.chip_silu.argtypes = [vp, i64, i64, i64, vp, i64, vp]
     L.chip_mul_mat_id_workspace_size.restype = sz
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
     L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
@@ -211,6 +215,34 @@ class Device:
             self.sync()
             return y, db.download(np.uint8, n * rs).reshape(n, rs)
         return y
+
+    # -- element-wise ops next to the matmuls ---------------------------------------------------------------
+    def rms_norm(self, x, eps):
+        x = np.ascontiguousarray(x, np.float32)
+        n, ne0 = x.shape
+        dx, dy = self.to_device(x), self.alloc(x.nbytes)
+        self.check(self.lib.chip_rms_norm(dx.ptr, ne0, n, ne0, eps, dy.ptr, ne0, None))
+        self.sync()
+        return dy.download(np.float32, n * ne0).reshape(n, ne0)
+
+    def silu(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        n, ne0 = x.shape
+        dx, dy = self.to_device(x), self.alloc(x.nbytes)
+        self.check(self.lib.chip_silu(dx.ptr, ne0, n, ne0, dy.ptr, ne0, None))
+        self.sync()
+        return dy.download(np.float32, n * ne0).reshape(n, ne0)
+
+    def binary(self, op, a, b):
+        """op "add" or "mul"; b has the shape of a or is one row."""
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(b, np.float32).reshape(-1, a.shape[1])
+        n, ne0 = a.shape
+        da, db, dy = self.to_device(a), self.to_device(b), self.alloc(a.nbytes)
+        fn = self.lib.chip_add if op == "add" else self.lib.chip_mul
+        self.check(fn(da.ptr, ne0, db.ptr, ne0, b.shape[0], n, ne0, dy.ptr, ne0, None))
+        self.sync()
+        return dy.download(np.float32, n * ne0).reshape(n, ne0)
 
     def mul_mat_id(self, wtype, W, x, ids):
         """LM_GGML_OP_MUL_MAT_ID: W uint8 [n_as, N, row_size], x fp32 [n_tokens, ne11, K], ids int32 [n_tokens, n_used]

@@ -408,6 +408,37 @@ int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K
                                  workspace, stride, y, ldy, lim, st));
 }
 
+// ---- element-wise ops next to the matmuls ----
+static bool rows_ok(const float *p, int64_t ld, int64_t ne0) { return p && ld >= ne0 && (((uintptr_t)p) & 3) == 0; }
+int chip_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0 || !(eps >= 0.0f)) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0)) return CHIP_EINVAL;
+    return hip_rc(launch_rms_norm(x, ldx, n, ne0, eps, y, ldy, (hipStream_t)stream));
+}
+static int binary_checked(bool mul, const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0,
+                          float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!(n_b == 1 || n_b == n)) return CHIP_EUNSUPPORTED;               // src1: the shape of src0, or one row for all
+    if (!rows_ok(a, lda, ne0) || !rows_ok(y, ldy, ne0) || !b || (((uintptr_t)b) & 3) != 0 || (n_b == n && n > 1 && ldb < ne0))
+        return CHIP_EINVAL;
+    const int64_t step = (n_b == 1) ? 0 : ldb;
+    return hip_rc(mul ? launch_mul(a, lda, b, step, ne0, n, y, ldy, (hipStream_t)stream)
+                      : launch_add(a, lda, b, step, ne0, n, y, ldy, (hipStream_t)stream));
+}
+int chip_add(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0, float *y, int64_t ldy,
+             void *stream) { return binary_checked(false, a, lda, b, ldb, n_b, n, ne0, y, ldy, stream); }
+int chip_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0, float *y, int64_t ldy,
+             void *stream) { return binary_checked(true, a, lda, b, ldb, n_b, n, ne0, y, ldy, stream); }
+int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (ne0 % 8 != 0) return CHIP_EUNSUPPORTED;                            // the reference's row tail uses the C library's expf
+    if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0)) return CHIP_EINVAL;
+    return hip_rc(launch_silu(x, ldx, ne0, n, y, ldy, (hipStream_t)stream));
+}
+
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                      int32_t *isum, int32_t *imin, void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;

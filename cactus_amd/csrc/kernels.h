@@ -171,6 +171,12 @@ hipError_t launch_gemm_kq(int wtype, const void *W, size_t nb01, int64_t K, int6
 // In the three GEMM launchers: with rg, n_as is the number of token-tile slots the grid provides in y (an upper bound
 // of the tile list's length) and n is ignored; gemm_*_moe_tile_tokens gives the tile height the list must be built for.
 
+// ops.hip: RMS_NORM, ADD, MUL, SILU over F32 rows (ldb = 0 broadcasts one row of b over all rows of a).
+hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, float *y, int64_t ldy, hipStream_t st);
+hipError_t launch_add(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
+hipError_t launch_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
+hipError_t launch_silu(const float *x, int64_t ldx, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
+
 // moe_group.hip: counting sort of MUL_MAT_ID's (token, slot) pairs by expert into offsets[n_as + 1] / perm[pairs].
 // tiles[0] = number of token tiles, tiles[1 + i] = expert | tile << 12 for tiles of `tile_tokens` pairs.
 bool       moe_group_supported(int64_t n_as, int64_t pairs);

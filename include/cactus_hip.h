@@ -163,6 +163,22 @@ CHIP_API int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, 
                              int64_t n_used, int64_t n_tokens, float *y, int64_t ldy,
                              void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- the element-wise ops between the matmuls of an FFN block (F32 rows; row strides in elements) ----
+ * So that norm -> up/gate -> activation -> down -> residual stays on the device.  In-place use (y == x / a) is allowed.
+ *   chip_rms_norm : LM_GGML_OP_RMS_NORM, lm_ggml_compute_forward_rms_norm_f32 (ggml-cpu/ops.cpp:3270-3316):
+ *                   y = x / sqrt(mean(x^2) + eps) per row; squares summed in double.
+ *   chip_add/_mul : LM_GGML_OP_ADD / LM_GGML_OP_MUL (ggml-cpu/binary-ops.cpp) for src1 of the shape of src0 (n_b == n) or
+ *                   one row broadcast over all rows (n_b == 1: norm weights, biases); other broadcasts are declined.
+ *   chip_silu     : LM_GGML_UNARY_OP_SILU, lm_ggml_vec_silu_f32 (ggml-cpu/vec.cpp:164-186) in its AVX2 + FMA form
+ *                   (lm_ggml_v_expf, ggml-cpu/vec.h:615-656), bit for bit; ne0 must be a multiple of 8 (the reference
+ *                   finishes other rows with the C library's expf). */
+CHIP_API int chip_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, float *y, int64_t ldy, void *stream);
+CHIP_API int chip_add(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0,
+                      float *y, int64_t ldy, void *stream);
+CHIP_API int chip_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0,
+                      float *y, int64_t ldy, void *stream);
+CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream);
+
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,
  * iq4_nl_q8_0} (ggml-cpu/ggml-cpu-quants.c:1906,3591,6772,8520,2924,7699,12751), computed with the same device

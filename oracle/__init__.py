@@ -128,6 +128,10 @@ class Oracle:
         L.orc_vec_dot_exact.argtypes = [_i32, _i64, _vp, _vp, _vp]
         L.orc_mul_mat.restype = None
         L.orc_mul_mat.argtypes = [_i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i32]
+        L.orc_rms_norm_f32.restype = None
+        L.orc_rms_norm_f32.argtypes = [_vp, _vp, _i64, _i64, C.c_float]
+        L.orc_silu_f32.restype = None
+        L.orc_silu_f32.argtypes = [_vp, _vp, _i64, _i64]
         L.orc_mul_mat_id.restype = _i32
         L.orc_mul_mat_id.argtypes = [_i32, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i32]
 
@@ -236,6 +240,20 @@ class Oracle:
             out["sum_abs"] = sa
         return out
 
+    def rms_norm(self, x, eps):
+        """LM_GGML_OP_RMS_NORM over the rows of x fp32 [n, ne0]."""
+        x = _f32(x)
+        y = np.empty_like(x)
+        self.lib.orc_rms_norm_f32(_ptr(x), _ptr(y), x.shape[0], x.shape[1], eps)
+        return y
+
+    def silu(self, x):
+        """LM_GGML_UNARY_OP_SILU over the rows of x fp32 [n, ne0] (AVX2 build of the reference)."""
+        x = _f32(x)
+        y = np.empty_like(x)
+        self.lib.orc_silu_f32(_ptr(x), _ptr(y), x.shape[0], x.shape[1])
+        return y
+
     def mul_mat_id(self, wtype, W, x, ids, nthreads=1, want=()):
         """LM_GGML_OP_MUL_MAT_ID: W uint8 [n_as, N, row_size], x fp32 [n_tokens, ne11, K] (ne11 = 1 or n_used),
         ids int32 [n_tokens, n_used] -> y fp32 [n_tokens, n_used, N]."""
@@ -308,6 +326,13 @@ class Reference:
         L.lm_ggml_mul_mat.argtypes = [_vp, _vp, _vp]
         L.lm_ggml_new_tensor_3d.restype = _vp
         L.lm_ggml_new_tensor_3d.argtypes = [_vp, _i32, _i64, _i64, _i64]
+        for n_ in ("lm_ggml_add", "lm_ggml_mul"):
+            getattr(L, n_).restype = _vp
+            getattr(L, n_).argtypes = [_vp, _vp, _vp]
+        L.lm_ggml_silu.restype = _vp
+        L.lm_ggml_silu.argtypes = [_vp, _vp]
+        L.lm_ggml_rms_norm.restype = _vp
+        L.lm_ggml_rms_norm.argtypes = [_vp, _vp, C.c_float]
         L.lm_ggml_mul_mat_id.restype = _vp
         L.lm_ggml_mul_mat_id.argtypes = [_vp, _vp, _vp, _vp]
         L.lm_ggml_new_graph.restype = _vp
@@ -422,6 +447,40 @@ class Reference:
         L.lm_ggml_threadpool_free(tp)
         L.lm_ggml_free(ctx)
         return y, times
+
+    def op_graph(self, op, x, b=None, eps=0.0, nthreads=1):
+        """One element-wise node on the reference CPU backend: op in {"rms_norm", "silu", "add", "mul"}; x fp32
+        [n, ne0]; b fp32 [n, ne0] or [1, ne0] for the binary ops."""
+        L = self.lib
+        x = _f32(x)
+        n, ne0 = x.shape
+        ctx = L.lm_ggml_init(_InitParams(L.lm_ggml_tensor_overhead() * 8 + L.lm_ggml_graph_overhead() + 4096,
+                                         None, True))
+        tx = L.lm_ggml_new_tensor_2d(ctx, F32, ne0, n)
+        tb = None
+        if op == "rms_norm":
+            c = L.lm_ggml_rms_norm(ctx, tx, eps)
+        elif op == "silu":
+            c = L.lm_ggml_silu(ctx, tx)
+        else:
+            b = _f32(b)
+            tb = L.lm_ggml_new_tensor_2d(ctx, F32, ne0, b.shape[0])
+            c = (L.lm_ggml_add if op == "add" else L.lm_ggml_mul)(ctx, tx, tb)
+        g = L.lm_ggml_new_graph(ctx)
+        L.lm_ggml_build_forward_expand(g, c)
+        be = L.lm_ggml_backend_cpu_init()
+        L.lm_ggml_backend_cpu_set_n_threads(be, nthreads)
+        buf = L.lm_ggml_backend_alloc_ctx_tensors(ctx, be)
+        L.lm_ggml_backend_tensor_set(tx, _ptr(x), 0, x.size * 4)
+        if tb is not None:
+            L.lm_ggml_backend_tensor_set(tb, _ptr(b), 0, b.size * 4)
+        assert L.lm_ggml_backend_graph_compute(be, g) == 0
+        y = np.zeros((n, ne0), np.float32)
+        L.lm_ggml_backend_tensor_get(c, _ptr(y), 0, y.size * 4)
+        L.lm_ggml_backend_buffer_free(buf)
+        L.lm_ggml_backend_free(be)
+        L.lm_ggml_free(ctx)
+        return y
 
     def mul_mat_id_graph(self, wtype, W, x, ids, nthreads=1):
         """LM_GGML_OP_MUL_MAT_ID on the reference CPU backend: W uint8 [n_as, N, row_size], x fp32

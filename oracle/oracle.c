@@ -1257,3 +1257,61 @@ int orc_mul_mat_id(int type, int64_t K, int64_t N, int64_t n_as, const void *W, 
     return 0;
 }
 
+/* ---- the element-wise ops next to the matmuls of an FFN block ---- */
+
+/* lm_ggml_compute_forward_rms_norm_f32 (reference ggml-cpu/ops.cpp:3270-3316): per row, the sum of the float squares
+ * in double, in element order; mean and scale in float; y = x * scale (lm_ggml_vec_scale_f32: one float multiply). */
+void orc_rms_norm_f32(const float *x, float *y, int64_t n_rows, int64_t ne0, float eps) {
+    for (int64_t r = 0; r < n_rows; r++) {
+        const float *xr = x + r * ne0;
+        double sum = 0.0;
+        for (int64_t i = 0; i < ne0; i++) sum += (double)(xr[i] * xr[i]);
+        const float mean = (float)(sum / (double)ne0);
+        const float scale = 1.0f / sqrtf(mean + eps);
+        for (int64_t i = 0; i < ne0; i++) y[r * ne0 + i] = xr[i] * scale;
+    }
+}
+
+/* One lane of lm_ggml_v_expf, AVX2 + FMA form (reference ggml-cpu/vec.h:615-656): round-to-nearest via the 1.5 * 2^23
+ * shift, two-step range reduction, degree-5 polynomial, exponent assembled in the integer domain; |n| > 126 takes the
+ * two-factor scaling path, |n| > 192 saturates through s1 * s1.  The lanes of a vector do not interact (the early
+ * return computes the same value as the select). */
+static float v_expf_lane(float x) {
+    const float r = 0x1.8p23f;
+    const float z = fmaf(x, 0x1.715476p+0f, r);
+    const float n = z - r;
+    const float b = fmaf(-n, 0x1.7f7d1cp-20f, fmaf(-n, 0x1.62e4p-1f, x));
+    uint32_t zb, one_b;
+    memcpy(&zb, &z, 4);
+    const float one = 1.0f;
+    memcpy(&one_b, &one, 4);
+    const uint32_t e = zb << 23;
+    const uint32_t kb = e + one_b;
+    float k;
+    memcpy(&k, &kb, 4);
+    const float u = b * b;
+    const float j = fmaf(fmaf(fmaf(0x1.0e4020p-7f, b, 0x1.573e2ep-5f), u, fmaf(0x1.555e66p-3f, b, 0x1.fffdb6p-2f)), u,
+                         0x1.ffffecp-1f * b);
+    if (!(fabsf(n) > 126.0f)) return fmaf(j, k, k);
+    const uint32_t g = (n <= 0.0f) ? 0x82000000u : 0u;
+    const uint32_t s1b = g + 0x7f000000u, s2b = e - g;
+    float s1, s2;
+    memcpy(&s1, &s1b, 4);
+    memcpy(&s2, &s2b, 4);
+    if (fabsf(n) > 192.0f) return s1 * s1;
+    return fmaf(s2, j, s2) * s1;
+}
+
+/* lm_ggml_vec_silu_f32 (reference ggml-cpu/vec.cpp:164-186), AVX2 build: x / (1 + v_expf(-x)) for the first
+ * n - n % 8 elements of a row, x / (1 + expf(-x)) with the C library's expf for the rest. */
+void orc_silu_f32(const float *x, float *y, int64_t n_rows, int64_t ne0) {
+    for (int64_t r = 0; r < n_rows; r++) {
+        const float *xr = x + r * ne0;
+        float *yr = y + r * ne0;
+        int64_t i = 0;
+        for (; i + 7 < ne0; i += 8)
+            for (int l = 0; l < 8; l++) yr[i + l] = xr[i + l] / (1.0f + v_expf_lane(0.0f - xr[i + l]));
+        for (; i < ne0; i++) yr[i] = xr[i] / (1.0f + expf(-xr[i]));
+    }
+}
+

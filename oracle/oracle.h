@@ -141,6 +141,12 @@ void orc_mul_mat(int type, int64_t K, int64_t N, int64_t n, const void *W, const
 int orc_mul_mat_id(int type, int64_t K, int64_t N, int64_t n_as, const void *W, const float *x, int64_t ne11,
                    const int32_t *ids, int64_t n_used, int64_t n_tokens, float *y, double *sum_abs, int nthreads);
 
+/* Element-wise ops of an FFN block, restated from ggml-cpu/ops.cpp and ggml-cpu/vec.{h,cpp} (AVX2 + FMA build);
+ * rows are contiguous.  Pinned bit-exact on oracle/_ref's graphs (tests/test_oracle_vs_ref.py).  ADD and MUL are
+ * single IEEE operations per element and need no restatement. */
+void orc_rms_norm_f32(const float *x, float *y, int64_t n_rows, int64_t ne0, float eps);
+void orc_silu_f32(const float *x, float *y, int64_t n_rows, int64_t ne0);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,106 @@
+"""GPU parity of the element-wise ops next to the matmuls (RMS_NORM, ADD, MUL, SILU), through the C-ABI, against the
+CPU oracle (pinned bit-exact on the reference build).
+
+Bars: ADD, MUL and SILU bit-exact; RMS_NORM within one fp32 ulp per element, and bit-exact in practice (the sum of
+squares is a double: only its last bits depend on the order of the additions)."""
+import numpy as np
+import pytest
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import cactus_amd
+    return cactus_amd.Device(0)
+
+
+def inputs(seed, n, ne0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((n, ne0)) * rng.choice([0.01, 1.0, 8.0, 40.0], (n, 1))).astype(np.float32)
+    special = np.array([0.0, -0.0, 1e-30, -1e-30, 87.0, -87.0, 88.5, -88.5, 89.0, -104.0, 130.0, -130.0, 133.0, -140.0, 1e4, -1e4],
+                       np.float32)
+    m = min(special.size, ne0)
+    x[0, :m] = special[:m]
+    return x
+
+
+SHAPES = [(1, 256), (1, 4096), (7, 4096), (3, 40), (2, 11008), (130, 14336), (5, 1000)]
+
+
+@pytest.mark.parametrize("n,ne0", SHAPES)
+def test_rms_norm(dev, orc, n, ne0):
+    x = inputs(n + ne0, n, ne0)
+    for eps in (1e-5, 1e-6):
+        ref = orc.rms_norm(x, eps)
+        y = dev.rms_norm(x, eps)
+        ulp = np.spacing(np.abs(ref))
+        assert (np.abs(y.astype(np.float64) - ref) <= ulp).all()
+        assert (y.view(np.uint32) == ref.view(np.uint32)).mean() > 0.999
+    z = np.zeros((2, ne0), np.float32)
+    assert np.array_equal(dev.rms_norm(z, 1e-5), orc.rms_norm(z, 1e-5))          # all-zero rows: 0 * 1/sqrt(eps)
+
+
+@pytest.mark.parametrize("n,ne0", [s for s in SHAPES if s[1] % 8 == 0])
+def test_silu_bit_exact(dev, orc, n, ne0):
+    x = inputs(2 * n + ne0, n, ne0)
+    with np.errstate(all="ignore"):
+        ref = orc.silu(x)
+    assert dev.silu(x).tobytes() == ref.tobytes()
+
+
+def test_silu_every_exponent_range(dev, orc):
+    # a sweep through the whole input range of the exponential, including the thresholds of its scaling branches
+    x = np.concatenate([np.linspace(-150, 150, 8192, dtype=np.float32), np.float32([87.3, 88.0, 88.72, 88.73, 103.9, 104.1]),
+                        -np.float32([87.3, 88.0, 88.72, 88.73, 103.9, 104.1]), np.float32([np.inf, -np.inf, np.nan, 3e38]),
+                        np.zeros(8, np.float32)]).reshape(1, -1)
+    assert x.shape[1] % 8 == 0
+    with np.errstate(all="ignore"):
+        ref = orc.silu(x)
+    y = dev.silu(x)
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    assert y[~np.isnan(y)].tobytes() == ref[~np.isnan(ref)].tobytes()
+
+
+@pytest.mark.parametrize("n,ne0", SHAPES)
+def test_add_mul_bit_exact(dev, n, ne0):
+    a, b, w = inputs(3 * n + ne0, n, ne0), inputs(4 * n + ne0, n, ne0), inputs(5 + ne0, 1, ne0)
+    with np.errstate(all="ignore"):
+        assert dev.binary("add", a, b).tobytes() == (a + b).tobytes()
+        assert dev.binary("mul", a, b).tobytes() == (a * b).tobytes()
+        assert dev.binary("mul", a, w).tobytes() == (a * w).tobytes()             # one row over all rows: norm weight
+        assert dev.binary("add", a, w).tobytes() == (a + w).tobytes()             # bias
+
+
+def test_strided_rows_in_place_and_errors(dev, orc):
+    import cactus_amd as ca
+    L = dev.lib
+    n, ne0, ld = 5, 512, 640
+    x = np.zeros((n, ld), np.float32)
+    x[:, :ne0] = inputs(1, n, ne0)
+    dx = dev.to_device(x)
+    dev.check(L.chip_rms_norm(dx.ptr, ld, n, ne0, 1e-5, dx.ptr, ld, None))             # in place, padded rows
+    dev.sync()
+    out = dx.download(np.float32, n * ld).reshape(n, ld)
+    assert np.array_equal(out[:, :ne0], orc.rms_norm(x[:, :ne0].copy(), 1e-5)) and not out[:, ne0:].any()
+    dev.check(L.chip_silu(dx.ptr, ld, n, ne0, dx.ptr, ld, None))
+    dev.sync()
+    assert np.array_equal(dx.download(np.float32, n * ld).reshape(n, ld)[:, :ne0], orc.silu(out[:, :ne0].copy()))
+    assert L.chip_silu(dx.ptr, ld, n, 12, dx.ptr, ld, None) == -2                      # row tail: unsupported
+    assert L.chip_rms_norm(dx.ptr, 100, n, ne0, 1e-5, dx.ptr, ld, None) != 0           # stride shorter than the row
+    assert L.chip_rms_norm(dx.ptr, ld, n, ne0, -1.0, dx.ptr, ld, None) != 0
+    assert L.chip_add(dx.ptr, ld, dx.ptr, ld, 2, n, ne0, dx.ptr, ld, None) == -2       # src1 neither 1 nor n rows
+    assert L.chip_mul(dx.ptr, ld, None, ld, 1, n, ne0, dx.ptr, ld, None) != 0
+    assert L.chip_add(dx.ptr, ld, dx.ptr, ld, n, 0, ne0, dx.ptr, ld, None) == 0
+    # unaligned base pointer: the scalar path
+    y = dev.alloc(n * ld * 4 + 16)
+    dev.check(L.chip_mul(dx.ptr + 4, ld, dx.ptr + 4, ld, n - 1, n - 1, ne0 - 3, y.ptr + 4, ld, None))
+    dev.sync()
+    cur = dx.download(np.float32, n * ld)
+    want = np.stack([cur[1 + r * ld: 1 + r * ld + ne0 - 3] for r in range(n - 1)])
+    got = y.download(np.float32, n * ld + 4)
+    got = np.stack([got[1 + r * ld: 1 + r * ld + ne0 - 3] for r in range(n - 1)])
+    with np.errstate(all="ignore"):
+        assert got.tobytes() == (want * want).tobytes()

@@ -75,3 +75,43 @@ def test_mul_mat_id_graph(orc, ref, wt, n_tokens, ne11, threads):
     t, s = n_tokens - 1, n_used - 1
     one = orc.mul_mat(wt, W[ids[t, s]], x[t, s % ne11][None, :])["y"][0]
     assert np.array_equal(y[t, s], one)
+
+
+def elementwise_inputs(seed, n, ne0):
+    """Activations with the magnitudes that occur next to the matmuls, plus the values that exercise every branch of
+    the exponential: large |x| (beyond the two-factor scaling thresholds), zeros, tiny values."""
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((n, ne0)) * rng.choice([0.01, 1.0, 8.0, 40.0], (n, 1))).astype(np.float32)
+    special = np.array([0.0, -0.0, 1e-30, -1e-30, 87.0, -87.0, 88.5, -88.5, 89.0, -104.0, 130.0, -130.0, 133.0, -140.0, 1e4, -1e4],
+                       np.float32)
+    m = min(special.size, ne0)
+    x[0, :m] = special[:m]
+    return x
+
+
+@pytest.mark.parametrize("n,ne0,threads", [(1, 256, 1), (7, 4096, 3), (3, 40, 2), (2, 11008, 2)])
+def test_rms_norm_and_silu_graph(orc, ref, n, ne0, threads):
+    x = elementwise_inputs(n + ne0, n, ne0)
+    for eps in (1e-5, 1e-6):
+        assert orc.rms_norm(x, eps).tobytes() == ref.op_graph("rms_norm", x, eps=eps, nthreads=threads).tobytes()
+    with np.errstate(all="ignore"):
+        a, b = orc.silu(x), ref.op_graph("silu", x, nthreads=threads)
+    assert a.tobytes() == b.tobytes()
+
+
+def test_rms_norm_and_silu_rows_with_a_tail(orc, ref):
+    # 13 = 8 + 5: the last 5 elements of a row take the reference's scalar expf path
+    x = elementwise_inputs(5, 4, 13)
+    assert orc.silu(x).tobytes() == ref.op_graph("silu", x).tobytes()
+    assert orc.rms_norm(x, 1e-5).tobytes() == ref.op_graph("rms_norm", x, eps=1e-5).tobytes()
+
+
+def test_add_and_mul_are_single_ieee_operations(ref):
+    x = elementwise_inputs(9, 6, 512)
+    y = elementwise_inputs(10, 6, 512)
+    w = elementwise_inputs(11, 1, 512)
+    with np.errstate(all="ignore"):
+        assert ref.op_graph("add", x, y).tobytes() == (x + y).tobytes()
+        assert ref.op_graph("mul", x, y).tobytes() == (x * y).tobytes()
+        assert ref.op_graph("mul", x, w).tobytes() == (x * w).tobytes()        # one row broadcast over all rows
+        assert ref.op_graph("add", x, w).tobytes() == (x + w).tobytes()
