@@ -279,6 +279,23 @@ def bench_extra(dev, hip, trace=True):
     moe_case("moe_q4_K_128x8_768x2048_n512", ca.Q4_K, 128, 8, 768, 2048, 512)
     moe_case("moe_q4_K_8x2_14336x4096_n512", ca.Q4_K, 8, 2, 14336, 4096, 512)
 
+    # the element-wise ops between the matmuls (F32 rows): HBM-bound streams, bytes = reads + writes
+    def ew_case(key, fn, n, ne0, streams):
+        a = dev.to_device(rng.standard_normal((n, ne0)).astype(np.float32))
+        b = dev.to_device(rng.standard_normal((n, ne0)).astype(np.float32))
+        y = dev.alloc(n * ne0 * 4)
+        us = time_runs(dev, hip, st, lambda: fn(a, b, y, n, ne0), 50)
+        byts = streams * n * ne0 * 4
+        out[key] = {"us": round(us, 2), "GBps": round(byts / us / 1e3, 1), "hbm_frac": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+        for bf in (a, b, y):
+            bf.free()
+
+    for (n, ne0) in ((1, 4096), (512, 4096), (512, 14336)):
+        ew_case("rms_norm_%dx%d" % (n, ne0), lambda a, b, y, n_, e: L.chip_rms_norm(a.ptr, e, n_, e, 1e-5, y.ptr, e, st), n, ne0, 2)
+        ew_case("silu_%dx%d" % (n, ne0), lambda a, b, y, n_, e: L.chip_silu(a.ptr, e, n_, e, y.ptr, e, st), n, ne0, 2)
+        ew_case("mul_%dx%d" % (n, ne0), lambda a, b, y, n_, e: L.chip_mul(a.ptr, e, b.ptr, e, n_, n_, e, y.ptr, e, st), n, ne0, 3)
+        ew_case("add_%dx%d" % (n, ne0), lambda a, b, y, n_, e: L.chip_add(a.ptr, e, b.ptr, e, n_, n_, e, y.ptr, e, st), n, ne0, 3)
+
     # weight upload: one synchronous copy from pageable memory (what set_tensor does) against the loader's protocol of
     # four pinned 1 MB staging buffers with an event each (chunked set_tensor_async)
     def upload_case():

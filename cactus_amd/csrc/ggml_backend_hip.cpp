@@ -22,7 +22,7 @@
 
 namespace {
 
-std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0};
+std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -236,6 +236,60 @@ bool mul_mat_id_shape_ok(const lm_ggml_tensor *op) {
     return true;
 }
 
+// ---- the element-wise ops between the matmuls (RMS_NORM, ADD, MUL, UNARY SILU; F32) ----
+// A tensor as rows: element-contiguous rows at one uniform stride across the higher dimensions.
+bool as_rows(const lm_ggml_tensor *t, int64_t &rows, int64_t &ld) {
+    if (t->type != LM_GGML_TYPE_F32 || t->nb[0] != sizeof(float) || t->nb[1] % 4 != 0 || t->nb[1] < (size_t)t->ne[0] * 4) return false;
+    if (t->ne[2] > 1 && t->nb[2] != (size_t)t->ne[1] * t->nb[1]) return false;
+    if (t->ne[3] > 1 && t->nb[3] != (size_t)t->ne[2] * t->ne[1] * t->nb[1]) return false;
+    rows = t->ne[1] * t->ne[2] * t->ne[3];
+    ld = (int64_t)(t->nb[1] / 4);
+    return true;
+}
+bool same_shape(const lm_ggml_tensor *a, const lm_ggml_tensor *b) {
+    return a->ne[0] == b->ne[0] && a->ne[1] == b->ne[1] && a->ne[2] == b->ne[2] && a->ne[3] == b->ne[3];
+}
+bool elementwise_enabled() {
+    static const bool on = [] { const char *e = std::getenv("CACTUS_HIP_ELEMENTWISE"); return !(e && std::strcmp(e, "0") == 0); }();
+    return on;
+}
+bool elementwise_shape_ok(const lm_ggml_tensor *op) {
+    if (!elementwise_enabled()) return false;
+    const lm_ggml_tensor *a = op->src[0], *b = op->src[1];
+    int64_t r, ld;
+    if (!a || !as_rows(op, r, ld) || !as_rows(a, r, ld) || !same_shape(op, a)) return false;
+    switch (op->op) {
+        case LM_GGML_OP_RMS_NORM: return true;
+        case LM_GGML_OP_UNARY:    return op->op_params[0] == LM_GGML_UNARY_OP_SILU && a->ne[0] % 8 == 0;
+        case LM_GGML_OP_ADD:
+        case LM_GGML_OP_MUL:
+            // src1: the shape of src0, or one row broadcast over all rows (norm weights, biases)
+            if (!b || !as_rows(b, r, ld) || b->ne[0] != a->ne[0]) return false;
+            return same_shape(a, b) || (b->ne[1] == 1 && b->ne[2] == 1 && b->ne[3] == 1);
+        default: return false;
+    }
+}
+int run_elementwise(backend_ctx *c, lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0], *b = op->src[1];
+    int64_t rows, lda, ldy, rb = 0, ldb = 0;
+    as_rows(a, rows, lda);
+    as_rows(op, rows, ldy);
+    const int64_t ne0 = a->ne[0];
+    switch (op->op) {
+        case LM_GGML_OP_RMS_NORM: {
+            float eps;
+            std::memcpy(&eps, op->op_params, sizeof(float));
+            return chip_rms_norm((const float *)a->data, lda, rows, ne0, eps, (float *)op->data, ldy, c->stream);
+        }
+        case LM_GGML_OP_UNARY:
+            return chip_silu((const float *)a->data, lda, rows, ne0, (float *)op->data, ldy, c->stream);
+        default:
+            as_rows(b, rb, ldb);
+            return (op->op == LM_GGML_OP_ADD ? chip_add : chip_mul)((const float *)a->data, lda, (const float *)b->data, ldb, rb, rows,
+                                                                 ne0, (float *)op->data, ldy, c->stream);
+    }
+}
+
 static bool grow_workspace(backend_ctx *c, size_t need) {
     if (need <= c->workspace_size) return true;
     chip_stream_synchronize(c->stream);
@@ -253,6 +307,16 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_ADD || node->op == LM_GGML_OP_MUL || node->op == LM_GGML_OP_UNARY) &&
+            elementwise_shape_ok(node)) {
+            const int rc = run_elementwise(c, node);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            g_elementwise_nodes++;
+            continue;
+        }
         if (node->op == LM_GGML_OP_MUL_MAT_ID && mul_mat_id_shape_ok(node)) {
             const lm_ggml_tensor *w = node->src[0], *x = node->src[1], *ids = node->src[2];
             const int64_t K = w->ne[0], N = w->ne[1], n_used = ids->ne[0], n_tokens = ids->ne[1];
@@ -355,6 +419,9 @@ void dev_event_synchronize(lm_ggml_backend_dev_t, lm_ggml_backend_event_t event)
 
 bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     if (is_view_op(op->op)) return true;
+    // element-wise F32 ops run wherever their operands are put: the scheduler keeps them with the matmuls around them
+    if (op->op == LM_GGML_OP_RMS_NORM || op->op == LM_GGML_OP_ADD || op->op == LM_GGML_OP_MUL || op->op == LM_GGML_OP_UNARY)
+        return elementwise_shape_ok(op);
     if (op->op != LM_GGML_OP_MUL_MAT && op->op != LM_GGML_OP_MUL_MAT_ID) return false;
     // Only weights that already live in a HIP buffer: claiming host-resident weights would make the scheduler
     // copy the whole matrix to the device on every call.  At model load the probe tensor carries a zero-size

@@ -26,6 +26,11 @@ namespace mirror {
 #define LM_GGML_TYPE_I32 M_TYPE_I32
 #define LM_GGML_OP_NONE M_OP_NONE
 #define LM_GGML_OP_MUL_MAT M_OP_MUL_MAT
+#define LM_GGML_UNARY_OP_SILU M_UNARY_OP_SILU
+#define LM_GGML_OP_UNARY M_OP_UNARY
+#define LM_GGML_OP_RMS_NORM M_OP_RMS_NORM
+#define LM_GGML_OP_MUL M_OP_MUL
+#define LM_GGML_OP_ADD M_OP_ADD
 #define LM_GGML_OP_MUL_MAT_ID M_OP_MUL_MAT_ID
 #define LM_GGML_OP_RESHAPE M_OP_RESHAPE
 #define LM_GGML_OP_VIEW M_OP_VIEW
@@ -61,6 +66,11 @@ constexpr int k_max_dims = LM_GGML_MAX_DIMS, k_max_src = LM_GGML_MAX_SRC, k_max_
 #undef LM_GGML_TYPE_I32
 #undef LM_GGML_OP_NONE
 #undef LM_GGML_OP_MUL_MAT
+#undef LM_GGML_UNARY_OP_SILU
+#undef LM_GGML_OP_UNARY
+#undef LM_GGML_OP_RMS_NORM
+#undef LM_GGML_OP_MUL
+#undef LM_GGML_OP_ADD
 #undef LM_GGML_OP_MUL_MAT_ID
 #undef LM_GGML_OP_RESHAPE
 #undef LM_GGML_OP_VIEW
@@ -123,7 +133,9 @@ static_assert(mirror::M_TYPE_F32 == LM_GGML_TYPE_F32 && mirror::M_TYPE_F16 == LM
               mirror::M_TYPE_Q8_K == LM_GGML_TYPE_Q8_K && mirror::M_TYPE_I32 == LM_GGML_TYPE_I32, "type ids");
 static_assert(mirror::M_OP_NONE == LM_GGML_OP_NONE && mirror::M_OP_MUL_MAT == LM_GGML_OP_MUL_MAT && mirror::M_OP_RESHAPE == LM_GGML_OP_RESHAPE &&
               mirror::M_OP_VIEW == LM_GGML_OP_VIEW && mirror::M_OP_PERMUTE == LM_GGML_OP_PERMUTE && mirror::M_OP_TRANSPOSE == LM_GGML_OP_TRANSPOSE &&
-              mirror::M_OP_COUNT == LM_GGML_OP_COUNT && mirror::M_OP_MUL_MAT_ID == LM_GGML_OP_MUL_MAT_ID, "op ids");
+              mirror::M_OP_COUNT == LM_GGML_OP_COUNT && mirror::M_OP_MUL_MAT_ID == LM_GGML_OP_MUL_MAT_ID &&
+              mirror::M_OP_ADD == LM_GGML_OP_ADD && mirror::M_OP_MUL == LM_GGML_OP_MUL && mirror::M_OP_RMS_NORM == LM_GGML_OP_RMS_NORM &&
+              mirror::M_OP_UNARY == LM_GGML_OP_UNARY && mirror::M_UNARY_OP_SILU == LM_GGML_UNARY_OP_SILU, "op ids");
 static_assert(mirror::M_STATUS_ALLOC_FAILED == LM_GGML_STATUS_ALLOC_FAILED && mirror::M_STATUS_FAILED == LM_GGML_STATUS_FAILED &&
               mirror::M_STATUS_SUCCESS == LM_GGML_STATUS_SUCCESS && mirror::M_STATUS_ABORTED == LM_GGML_STATUS_ABORTED, "status");
 static_assert(mirror::M_DEV_CPU == LM_GGML_BACKEND_DEVICE_TYPE_CPU && mirror::M_DEV_GPU == LM_GGML_BACKEND_DEVICE_TYPE_GPU &&

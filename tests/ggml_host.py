@@ -105,6 +105,16 @@ class Host:
         L.lm_ggml_backend_tensor_get_async.argtypes = [vp, vp, vp, sz, sz]
         L.lm_ggml_add.restype = vp
         L.lm_ggml_add.argtypes = [vp, vp, vp]
+        L.lm_ggml_mul.restype = vp
+        L.lm_ggml_mul.argtypes = [vp, vp, vp]
+        L.lm_ggml_silu.restype = vp
+        L.lm_ggml_silu.argtypes = [vp, vp]
+        L.lm_ggml_rms_norm.restype = vp
+        L.lm_ggml_rms_norm.argtypes = [vp, vp, C.c_float]
+        L.lm_ggml_soft_max.restype = vp
+        L.lm_ggml_soft_max.argtypes = [vp, vp]
+        L.lm_ggml_new_tensor_1d.restype = vp
+        L.lm_ggml_new_tensor_1d.argtypes = [vp, i32, i64]
         L.lm_ggml_set_name.restype = vp
         L.lm_ggml_set_name.argtypes = [vp, C.c_char_p]
         L.lm_ggml_set_input.argtypes = [vp]

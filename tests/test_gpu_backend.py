@@ -97,17 +97,28 @@ def test_unsupported_ops_are_declined(host):
     mm_f32 = L.lm_ggml_mul_mat(ctx, wf, x)
     mm_96 = L.lm_ggml_mul_mat(ctx, k96, x96)
     add = L.lm_ggml_add(ctx, x, x)
+    x12 = host.tensor_2d(ctx, O.F32, 12, 2)
+    silu12 = L.lm_ggml_silu(ctx, x12)
+    wide = host.tensor_2d(ctx, O.F32, 256, 4)
+    add_bcast = L.lm_ggml_add(ctx, wide, x)                              # src1 [256, 2] repeated over [256, 4]
+    soft = L.lm_ggml_soft_max(ctx, x)
     view = L.lm_ggml_reshape_2d(ctx, x, 128, 4)
     buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
     assert L.lm_ggml_backend_dev_supports_op(dev, mm) is True
     assert L.lm_ggml_backend_dev_supports_op(dev, mm_f32) is False       # F32 weights: not this path
     assert L.lm_ggml_backend_dev_supports_op(dev, mm_96) is False        # K not a multiple of 256
-    assert L.lm_ggml_backend_dev_supports_op(dev, add) is False
+    assert L.lm_ggml_backend_dev_supports_op(dev, add) is True           # element-wise F32 ops next to the matmuls
+    assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_mul(ctx, x, x)) is True
+    assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_rms_norm(ctx, x, 1e-5)) is True
+    assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_silu(ctx, x)) is True
+    assert L.lm_ggml_backend_dev_supports_op(dev, silu12) is False       # row tail: the reference uses libm's expf there
+    assert L.lm_ggml_backend_dev_supports_op(dev, add_bcast) is False    # a broadcast other than one row
+    assert L.lm_ggml_backend_dev_supports_op(dev, soft) is False
     assert L.lm_ggml_backend_dev_supports_op(dev, view) is True
     # graph_compute on a node the device declined reports failure, it does not compute on the host
     be = L.lm_ggml_backend_dev_init(dev, None)
     g = L.lm_ggml_new_graph(ctx)
-    L.lm_ggml_build_forward_expand(g, add)
+    L.lm_ggml_build_forward_expand(g, soft)
     assert L.lm_ggml_backend_graph_compute(be, g) == -1                  # LM_GGML_STATUS_FAILED
     L.lm_ggml_backend_free(be)
     L.lm_ggml_backend_buffer_free(buf)
@@ -116,7 +127,8 @@ def test_unsupported_ops_are_declined(host):
 
 def test_scheduler_splits_between_hip_and_cpu(host, orc):
     """llama.cpp's flow: weights in a HIP buffer tagged USAGE_WEIGHTS, activations produced on the CPU; the
-    reference scheduler assigns the MUL_MATs to HIP, the ADD to the CPU, and copies inputs across."""
+    reference scheduler assigns the MUL_MATs and the ADD between them to HIP, the SOFT_MAX to the CPU, and copies
+    tensors across."""
     L = host.L
     K, N1, N2, n = 2048, 512, 256, 3
     w1 = orc.quantize_weights(O.Q4_K, common.weights_f32(11, N1, K))
@@ -141,7 +153,9 @@ def test_scheduler_splits_between_hip_and_cpu(host, orc):
     h = L.lm_ggml_mul_mat(ctx, tw1, tx)          # [N1=512, n]
     z = L.lm_ggml_mul_mat(ctx, tw2, tx)          # [N2, n]
     s = L.lm_ggml_mul_mat(ctx, tw3, h)           # [N2, n]   (K = 512 = N1)
-    out = L.lm_ggml_add(ctx, s, z)
+    out_add = L.lm_ggml_add(ctx, s, z)
+    L.lm_ggml_set_output(out_add)
+    out = L.lm_ggml_soft_max(ctx, out_add)
     L.lm_ggml_set_output(out)
     g = L.lm_ggml_new_graph(ctx)
     L.lm_ggml_build_forward_expand(g, out)
@@ -158,9 +172,12 @@ def test_scheduler_splits_between_hip_and_cpu(host, orc):
     blib.lm_ggml_backend_hip_get_stats(C.byref(after[0]), C.byref(after[1]))
     assert after[0].value - before[0].value == 3                       # the three MUL_MATs ran on the GPU
     assert L.lm_ggml_backend_sched_get_tensor_backend(sched, h) == hip
+    assert L.lm_ggml_backend_sched_get_tensor_backend(sched, out_add) == hip
     assert L.lm_ggml_backend_sched_get_tensor_backend(sched, out) == cpu
     assert L.lm_ggml_backend_sched_get_n_splits(sched) >= 2
-    y = host.get(out, np.float32, (n, N2))
+    y = host.get(out_add, np.float32, (n, N2))
+    sm = host.get(out, np.float32, (n, N2))
+    assert np.allclose(sm.sum(axis=1), 1.0, atol=1e-5)
     # reference: same graph entirely on the reference CPU path (through the oracle, bit-identical to it)
     hh = orc.mul_mat(O.Q4_K, w1, x)["y"]
     zz = orc.mul_mat(O.Q6_K, w2, x, want=("sum_abs",))
@@ -359,3 +376,67 @@ def test_async_upload_protocol_of_the_model_loader(host, orc):
     L.lm_ggml_backend_free(be2)
     L.lm_ggml_backend_free(be)
     L.lm_ggml_free(ctx)
+
+
+def test_ffn_block_stays_on_the_device(host, orc):
+    """norm -> up / gate -> SiLU * up -> down -> residual, the FFN half of a transformer layer as llama.cpp builds it
+    (reference llama-graph.cpp build_norm / build_ffn): with the element-wise ops on the device the reference scheduler
+    puts the whole block into one HIP split."""
+    import cactus_amd
+    L = host.L
+    H, FF, n = 1024, 2816, 5
+    eps = 1e-5
+    rng = np.random.default_rng(3)
+    wn = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    wu = orc.quantize_weights(O.Q4_K, common.weights_f32(21, FF, H))
+    wg = orc.quantize_weights(O.Q4_K, common.weights_f32(22, FF, H))
+    wd = orc.quantize_weights(O.Q6_K, common.weights_f32(23, H, FF))
+    x = common.activations_f32(24, n, H)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    wctx = host.context(with_graph=False)
+    tn = L.lm_ggml_new_tensor_1d(wctx, O.F32, H)
+    tu = host.tensor_2d(wctx, O.Q4_K, H, FF, "up")
+    tg = host.tensor_2d(wctx, O.Q4_K, H, FF, "gate")
+    td = host.tensor_2d(wctx, O.Q6_K, FF, H, "down")
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
+    host.set(tn, wn); host.set(tu, wu); host.set(tg, wg); host.set(td, wd)
+    ctx = host.context()
+    tx = host.tensor_2d(ctx, O.F32, H, n, "x")
+    L.lm_ggml_set_input(tx)
+    cur = L.lm_ggml_mul(ctx, L.lm_ggml_rms_norm(ctx, tx, eps), tn)
+    up = L.lm_ggml_mul_mat(ctx, tu, cur)
+    gate = L.lm_ggml_mul_mat(ctx, tg, cur)
+    act = L.lm_ggml_mul(ctx, L.lm_ggml_silu(ctx, gate), up)
+    down = L.lm_ggml_mul_mat(ctx, td, act)
+    out = L.lm_ggml_add(ctx, down, tx)
+    L.lm_ggml_set_output(out)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, out)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 64, False, True)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(tx, x)
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
+    for t in (cur, up, gate, act, down, out):
+        assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
+    y = host.get(out, np.float32, (n, H))
+    # the same chain on the oracle (the reference's CPU arithmetic)
+    c0 = orc.rms_norm(x, eps) * wn
+    u = orc.mul_mat(O.Q4_K, wu, c0)["y"]
+    gt = orc.mul_mat(O.Q4_K, wg, c0)["y"]
+    a = orc.silu(gt) * u
+    d = orc.mul_mat(O.Q6_K, wd, a, want=("sum_abs",))
+    want = d["y"] + x
+    # up / gate carry the GPU's summation order (<= 1e-5 of their yardstick); the Q8_K requantization of `act` passes
+    # that on, so compare at a tolerance for two chained matmuls
+    assert (np.abs(y - want) <= 2e-3 * d["sum_abs"] + 1e-6).all()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(wbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(wctx)
