@@ -57,7 +57,7 @@ inline TileMap make_tile_map(int64_t row_tiles, int64_t tok_tiles, int concurren
     m.grid = m.per_xcd * XCDS;
     return m;
 }
-__device__ __forceinline__ TileCoord xcd_tile(unsigned wg, const TileMap &m) {
+__host__ __device__ __forceinline__ TileCoord xcd_tile(unsigned wg, const TileMap &m) {
     unsigned g = (wg % XCDS) * m.per_xcd + wg / XCDS;
     TileCoord t;
     if (wg / XCDS >= m.per_xcd || g >= m.tiles) { t.row_tile = m.row_tiles; t.tok_tile = m.tok_tiles; return t; }
