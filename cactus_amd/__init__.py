@@ -22,6 +22,7 @@ F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
 F16 = 1
+CHIP_OK, CHIP_EINVAL, CHIP_EUNSUPPORTED = 0, -1, -2        # include/cactus_hip.h
 TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
               Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16"}
 WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, F16)
@@ -36,6 +37,7 @@ EXPORTS = (
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu",
+    "chip_soft_max", "chip_cpy", "chip_rope",
     "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -103,6 +105,9 @@ def load_library(path=KERNEL_LIB):
     L.chip_add.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
     L.chip_mul.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
     L.chip_silu.argtypes = [vp, i64, i64, i64, vp, i64, vp]
+    L.chip_soft_max.argtypes = [vp, i64, vp, i32, i64, i64, i64, C.c_float, C.c_float, vp, i64, vp]
+    L.chip_cpy.argtypes = [vp, i32, vp, i32, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64), vp]
+    L.chip_rope.argtypes = [vp, i64, i64, vp, vp, i64, i64, i64, i32, i32, i32] + [C.c_float] * 6 + [vp, i64, i64, vp]
     L.chip_mul_mat_id_workspace_size.restype = sz
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
     L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
@@ -243,6 +248,63 @@ class Device:
         self.check(fn(da.ptr, ne0, db.ptr, ne0, b.shape[0], n, ne0, dy.ptr, ne0, None))
         self.sync()
         return dy.download(np.float32, n * ne0).reshape(n, ne0)
+
+    # -- attention-side ops ---------------------------------------------------------------------------------
+    def soft_max(self, x, mask=None, scale=1.0, max_bias=0.0):
+        """x fp32 [n_head, ne01, ne00]; mask fp32 / fp16 [>= ne01, ne00] or None."""
+        x = np.ascontiguousarray(x, np.float32)
+        n_head, ne01, ne00 = x.shape
+        dx, dy = self.to_device(x), self.alloc(x.nbytes)
+        dm, mt = None, F32
+        if mask is not None:
+            mask = np.ascontiguousarray(mask)
+            mt = F16 if mask.dtype == np.float16 else F32
+            dm = self.to_device(mask)
+        self.check(self.lib.chip_soft_max(dx.ptr, ne00, dm.ptr if dm else None, mt, ne00, ne01, n_head * ne01, scale, max_bias,
+                                          dy.ptr, ne00, None))
+        self.sync()
+        return dy.download(np.float32, x.size).reshape(x.shape)
+
+    def cpy(self, x, dst_dtype, dst_strides=None, dst_elems=None):
+        """Copies the numpy array (or strided view) x, at most 4-D, into a destination of dst_dtype: dense, or with the
+        given byte strides (numpy order, slowest first) inside a zeroed region of dst_elems elements.  The source is
+        uploaded with the view's own strides.  Returns the destination region as a flat array."""
+        base = x
+        while isinstance(base.base, np.ndarray):
+            base = base.base
+        base = np.ascontiguousarray(base) if not base.flags.c_contiguous else base
+        off = x.__array_interface__["data"][0] - base.__array_interface__["data"][0]
+        types = {np.dtype(np.float32): F32, np.dtype(np.float16): F16}
+        dst_dtype = np.dtype(dst_dtype)
+        pad = 4 - x.ndim
+        ne = [1] * pad + list(x.shape)
+        nbs = [0] * pad + list(x.strides)
+        if dst_strides is None:
+            dst_strides = list(np.empty(x.shape, dst_dtype).strides)
+            dst_elems = x.size
+        nbd = [0] * pad + list(dst_strides)
+        A = C.c_int64 * 4
+        dsrc = self.to_device(base.reshape(-1).view(np.uint8))
+        ddst = self.alloc(dst_elems * dst_dtype.itemsize)
+        ddst.upload(np.zeros(dst_elems * dst_dtype.itemsize, np.uint8))
+        self.check(self.lib.chip_cpy(dsrc.ptr + off, types[x.dtype], ddst.ptr, types[dst_dtype], A(*ne[::-1]), A(*nbs[::-1]),
+                                     A(*nbd[::-1]), None))
+        self.sync()
+        return ddst.download(dst_dtype, dst_elems)
+
+    def rope(self, x, pos, n_dims, mode, freq_factors=None, n_ctx_orig=4096, freq_base=10000.0, freq_scale=1.0,
+             ext_factor=0.0, attn_factor=1.0, beta_fast=32.0, beta_slow=1.0):
+        """x fp32 [n_tokens, n_head, ne0], pos int32 [n_tokens]."""
+        x = np.ascontiguousarray(x, np.float32)
+        ne2, ne1, ne0 = x.shape
+        dx, dy = self.to_device(x), self.alloc(x.nbytes)
+        dp = self.to_device(np.ascontiguousarray(pos, np.int32))
+        df = self.to_device(np.ascontiguousarray(freq_factors, np.float32)) if freq_factors is not None else None
+        self.check(self.lib.chip_rope(dx.ptr, ne0, ne0 * ne1, dp.ptr, df.ptr if df else None, ne0, ne1, ne2, n_dims, mode,
+                                      n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow,
+                                      dy.ptr, ne0, ne0 * ne1, None))
+        self.sync()
+        return dy.download(np.float32, x.size).reshape(x.shape)
 
     def mul_mat_id(self, wtype, W, x, ids):
         """LM_GGML_OP_MUL_MAT_ID: W uint8 [n_as, N, row_size], x fp32 [n_tokens, ne11, K], ids int32 [n_tokens, n_used]

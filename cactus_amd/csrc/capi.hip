@@ -4,6 +4,7 @@
 #include "../../include/cactus_hip.h"
 #include "act_layout.h"
 #include "dev_common.h"
+#include <math.h>
 #include "kernels.h"
 
 #include <atomic>
@@ -437,6 +438,62 @@ int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int
     if (ne0 % 8 != 0) return CHIP_EUNSUPPORTED;                            // the reference's row tail uses the C library's expf
     if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0)) return CHIP_EINVAL;
     return hip_rc(launch_silu(x, ldx, ne0, n, y, ldy, (hipStream_t)stream));
+}
+
+// ---- attention-side ops ----
+int chip_soft_max(const float *x, int64_t ldx, const void *mask, int mask_type, int64_t ne00, int64_t ne01, int64_t n_rows,
+                  float scale, float max_bias, float *y, int64_t ldy, void *stream) {
+    if (ne00 < 0 || ne01 <= 0 || n_rows < 0) return CHIP_EINVAL;
+    if (n_rows == 0 || ne00 == 0) return CHIP_OK;
+    if (max_bias != 0.0f) return CHIP_EUNSUPPORTED;                          // ALiBi slopes
+    if (ne00 % 8 != 0) return CHIP_EUNSUPPORTED;                             // the reference's row tail uses the C library's expf
+    if (mask && mask_type != T_F32 && mask_type != T_F16) return CHIP_EUNSUPPORTED;
+    if (!x || !y || ldx < ne00 || ldy < ne00 || n_rows > 0x7fffffff) return CHIP_EINVAL;
+    if (((ldx | ldy) & 3) != 0 || ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)mask)) & 15) != 0) return CHIP_EINVAL;
+    return hip_rc(launch_soft_max(x, ldx, mask, mask_type == T_F16, ne00, ne01, n_rows, scale, y, ldy, (hipStream_t)stream));
+}
+
+int chip_cpy(const void *src, int src_type, void *dst, int dst_type, const int64_t ne[4], const int64_t nb_src[4],
+             const int64_t nb_dst[4], void *stream) {
+    if ((src_type != T_F32 && src_type != T_F16) || (dst_type != T_F32 && dst_type != T_F16)) return CHIP_EUNSUPPORTED;
+    if (!ne || !nb_src || !nb_dst) return CHIP_EINVAL;
+    const int64_t es = src_type == T_F16 ? 2 : 4, ed = dst_type == T_F16 ? 2 : 4;
+    int64_t total = 1;
+    for (int k = 0; k < 4; k++) {
+        if (ne[k] < 0 || nb_src[k] < 0 || nb_dst[k] < 0) return CHIP_EINVAL;
+        if (nb_src[k] % es != 0 || nb_dst[k] % ed != 0) return CHIP_EINVAL;
+        total *= ne[k];
+    }
+    if (total == 0) return CHIP_OK;
+    if (!src || !dst || (((uintptr_t)src) % es) != 0 || (((uintptr_t)dst) % ed) != 0) return CHIP_EINVAL;
+    return hip_rc(launch_cpy(src, src_type == T_F16, dst, dst_type == T_F16, ne, nb_src, nb_dst, (hipStream_t)stream));
+}
+
+int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1,
+              int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
+              float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1, int64_t ldy2, void *stream) {
+    if (ne0 < 0 || ne1 < 0 || ne2 < 0 || n_dims < 0 || n_dims > ne0 || (n_dims & 1)) return CHIP_EINVAL;
+    if (mode != 0 && mode != 2) return CHIP_EUNSUPPORTED;                   // multi-section and vision layouts
+    if (n_dims / 2 > 256) return CHIP_EUNSUPPORTED;
+    if (ne0 == 0 || ne1 == 0 || ne2 == 0) return CHIP_OK;
+    if (!x || !y || !pos || ldx1 < ne0 || ldy1 < ne0 || ne2 > 0x7fffffff) return CHIP_EINVAL;
+    if ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)pos) | ((uintptr_t)freq_factors)) & 3) return CHIP_EINVAL;
+    RopeArgs a;
+    a.ne0 = ne0; a.ne1 = ne1; a.ne2 = ne2;
+    a.ldx1 = ldx1; a.ldx2 = ldx2; a.ldy1 = ldy1; a.ldy2 = ldy2;
+    a.n_dims = n_dims; a.neox = (mode & 2) != 0;
+    // constants of the op, computed like the reference's host code computes them (ggml-cpu/ops.cpp:5229-5232, ggml.c:3749-3761)
+    a.theta_scale = powf(freq_base, -2.0f / n_dims);
+    a.freq_scale = freq_scale;
+    a.ext_factor = ext_factor;
+    const float lo = n_dims * logf(n_ctx_orig / (beta_fast * 2 * (float)M_PI)) / (2 * logf(freq_base));
+    const float hi = n_dims * logf(n_ctx_orig / (beta_slow * 2 * (float)M_PI)) / (2 * logf(freq_base));
+    const float start = floorf(lo), end = ceilf(hi);
+    a.corr0 = 0 > start ? 0 : start;
+    a.corr1 = (n_dims - 1) < end ? (float)(n_dims - 1) : end;
+    a.mscale = attn_factor;
+    if (ext_factor != 0.0f) a.mscale *= 1.0f + 0.1f * logf(1.0f / freq_scale);
+    return hip_rc(launch_rope(x, pos, freq_factors, a, y, (hipStream_t)stream));
 }
 
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,

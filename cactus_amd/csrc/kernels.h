@@ -176,6 +176,19 @@ hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, 
 hipError_t launch_add(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
 hipError_t launch_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
 hipError_t launch_silu(const float *x, int64_t ldx, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
+// SOFT_MAX over n_rows rows of ne00 values (a multiple of 8); row r adds row r % ne01 of the mask (fp32 or fp16, dense).
+hipError_t launch_soft_max(const float *x, int64_t ldx, const void *mask, int mask_f16, int64_t ne00, int64_t ne01, int64_t n_rows,
+                           float scale, float *y, int64_t ldy, hipStream_t st);
+// Same-shape copy between F32 / F16 tensors; ne in elements, strides in bytes.
+hipError_t launch_cpy(const void *src, int src_f16, void *dst, int dst_f16, const int64_t *ne, const int64_t *nb_src,
+                      const int64_t *nb_dst, hipStream_t st);
+struct RopeArgs {
+    int64_t ne0, ne1, ne2;
+    int64_t ldx1, ldx2, ldy1, ldy2;        // head and token strides in floats
+    int n_dims, neox;
+    float theta_scale, freq_scale, ext_factor, corr0, corr1, mscale;
+};
+hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, hipStream_t st);
 
 // moe_group.hip: counting sort of MUL_MAT_ID's (token, slot) pairs by expert into offsets[n_as + 1] / perm[pairs].
 // tiles[0] = number of token tiles, tiles[1 + i] = expert | tile << 12 for tiles of `tile_tokens` pairs.

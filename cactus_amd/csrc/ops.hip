@@ -11,8 +11,22 @@
 //             lm_ggml_v_expf (ggml-cpu/vec.h:615-656) restated operation by operation, so that the result is bit-exact
 //             for rows whose length is a multiple of 8 (the reference finishes other rows with the C library's expf:
 //             those rows are declined).
+//   SOFT_MAX  lm_ggml_compute_forward_soft_max_f32 (ggml-cpu/ops.cpp:4731-4827) with the AVX2 branch of
+//             lm_ggml_vec_soft_max_f32 (ggml-cpu/vec.cpp:198-208): w = x * scale + mask, e = lm_ggml_v_expf(w - max), groups
+//             of 8 summed in float in the reference's shuffle order, the groups in double (a tree here, in row order
+//             there: same remark as RMS_NORM), y = e * (float)(1 / sum).  Rows of a multiple of 8 values, no ALiBi.
+//   CPY, CONT lm_ggml_compute_forward_dup (ggml-cpu/ops.cpp): element i of the source in its logical order becomes element
+//             i of the destination; F32 -> F16 rounds to nearest even.  Bit-exact.
+//   ROPE      lm_ggml_compute_forward_rope_f32 (ggml-cpu/ops.cpp:5178-5361), modes 0 and NEOX: the angle of pair i at
+//             position p follows the reference's float recurrence theta_0 = p, theta_{i+1} = theta_i * theta_scale; cos
+//             and sin are computed in double here and rounded once (the reference calls the C library's cosf / sinf,
+//             which may differ from that by one unit in the last place), the rotation itself is unfused float
+//             arithmetic as in the reference.
 #include "dev_common.h"
 #include "kernels.h"
+
+// One rounding per written operation, as in the reference's C code; the fused operations of this file are explicit fmaf calls.
+#pragma clang fp contract(off)
 
 namespace chip {
 
@@ -104,6 +118,281 @@ __global__ __launch_bounds__(EW_THREADS) void elementwise_kernel(const float *__
                 yr[i] = ew_apply<OP>(ar[i], OP == EW_SILU ? 0.f : br[i]);
         }
     }
+}
+
+// ---- SOFT_MAX: one workgroup per row; thread t owns the groups of 8 values t, t + 256, ... ----
+// G > 0: the row fits 8 * G * EW_THREADS values and stays in registers.  G == 0: any length, y holds e between passes.
+enum { MASK_NONE = 0, MASK_F32 = 1, MASK_F16 = 2 };
+template <int MASK>
+__device__ __forceinline__ void soft_max_load(const float *xr, const void *mrow, int64_t i, float scale, float (&w)[8]) {
+    const float4 a = *reinterpret_cast<const float4 *>(xr + i), b = *reinterpret_cast<const float4 *>(xr + i + 4);
+    w[0] = a.x * scale; w[1] = a.y * scale; w[2] = a.z * scale; w[3] = a.w * scale;
+    w[4] = b.x * scale; w[5] = b.y * scale; w[6] = b.z * scale; w[7] = b.w * scale;
+    if constexpr (MASK == MASK_F32) {
+        const float *m = reinterpret_cast<const float *>(mrow) + i;
+        const float4 c = *reinterpret_cast<const float4 *>(m), d = *reinterpret_cast<const float4 *>(m + 4);
+        w[0] += c.x; w[1] += c.y; w[2] += c.z; w[3] += c.w; w[4] += d.x; w[5] += d.y; w[6] += d.z; w[7] += d.w;
+    } else if constexpr (MASK == MASK_F16) {
+        const u32x4 h = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint16_t *>(mrow) + i);
+#pragma unroll
+        for (int k = 0; k < 4; k++) { w[2 * k] += h2f(h[k]); w[2 * k + 1] += h2f(h[k] >> 16); }
+    }
+}
+__device__ __forceinline__ float group_sum8(const float (&e)[8]) {
+    return ((e[0] + e[4]) + (e[2] + e[6])) + ((e[1] + e[5]) + (e[3] + e[7]));
+}
+template <int MASK, int G>
+__global__ __launch_bounds__(EW_THREADS) void soft_max_kernel(const float *__restrict__ x, int64_t ldx, const void *__restrict__ mask,
+                                                              int64_t ne00, int64_t ne01, float scale, float *__restrict__ y,
+                                                              int64_t ldy) {
+    __shared__ float wmax[EW_THREADS / 64];
+    __shared__ double wsum[EW_THREADS / 64];
+    const int64_t row = blockIdx.x;
+    const float *xr = x + row * ldx;
+    float *yr = y + row * ldy;
+    const void *mrow = nullptr;
+    if constexpr (MASK == MASK_F32) mrow = reinterpret_cast<const float *>(mask) + (row % ne01) * ne00;
+    if constexpr (MASK == MASK_F16) mrow = reinterpret_cast<const uint16_t *>(mask) + (row % ne01) * ne00;
+    const int tid = threadIdx.x;
+    const int64_t groups = ne00 / 8;
+    constexpr int GR = G > 0 ? G : 1;
+    float w[GR][8];
+    float mx = -INFINITY;
+    if constexpr (G > 0) {
+#pragma unroll
+        for (int j = 0; j < G; j++) {
+            const int64_t g = tid + (int64_t)j * EW_THREADS;
+            if (g < groups) {
+                soft_max_load<MASK>(xr, mrow, 8 * g, scale, w[j]);
+#pragma unroll
+                for (int k = 0; k < 8; k++) mx = fmaxf(mx, w[j][k]);
+            }
+        }
+    } else {
+        for (int64_t g = tid; g < groups; g += EW_THREADS) {
+            soft_max_load<MASK>(xr, mrow, 8 * g, scale, w[0]);
+#pragma unroll
+            for (int k = 0; k < 8; k++) mx = fmaxf(mx, w[0][k]);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((tid & 63) == 0) wmax[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    static_assert(EW_THREADS == 256, "four waves");
+
+    double sum = 0.0;
+    if constexpr (G > 0) {
+#pragma unroll
+        for (int j = 0; j < G; j++) {
+            const int64_t g = tid + (int64_t)j * EW_THREADS;
+            if (g < groups) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) w[j][k] = v_expf_lane(w[j][k] - mx);
+                sum += (double)group_sum8(w[j]);
+            }
+        }
+    } else {
+        for (int64_t g = tid; g < groups; g += EW_THREADS) {
+            soft_max_load<MASK>(xr, mrow, 8 * g, scale, w[0]);
+#pragma unroll
+            for (int k = 0; k < 8; k++) w[0][k] = v_expf_lane(w[0][k] - mx);
+            sum += (double)group_sum8(w[0]);
+            *reinterpret_cast<float4 *>(yr + 8 * g) = make_float4(w[0][0], w[0][1], w[0][2], w[0][3]);
+            *reinterpret_cast<float4 *>(yr + 8 * g + 4) = make_float4(w[0][4], w[0][5], w[0][6], w[0][7]);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if ((tid & 63) == 0) wsum[tid >> 6] = sum;
+    __syncthreads();
+    const float inv = (float)(1.0 / ((wsum[0] + wsum[1]) + (wsum[2] + wsum[3])));
+    if constexpr (G > 0) {
+#pragma unroll
+        for (int j = 0; j < G; j++) {
+            const int64_t g = tid + (int64_t)j * EW_THREADS;
+            if (g < groups) {
+                *reinterpret_cast<float4 *>(yr + 8 * g) = make_float4(w[j][0] * inv, w[j][1] * inv, w[j][2] * inv, w[j][3] * inv);
+                *reinterpret_cast<float4 *>(yr + 8 * g + 4) = make_float4(w[j][4] * inv, w[j][5] * inv, w[j][6] * inv, w[j][7] * inv);
+            }
+        }
+    } else {
+        for (int64_t g = tid; g < groups; g += EW_THREADS) {           // each thread re-reads what it wrote itself
+            float4 a = *reinterpret_cast<float4 *>(yr + 8 * g), b = *reinterpret_cast<float4 *>(yr + 8 * g + 4);
+            a.x *= inv; a.y *= inv; a.z *= inv; a.w *= inv; b.x *= inv; b.y *= inv; b.z *= inv; b.w *= inv;
+            *reinterpret_cast<float4 *>(yr + 8 * g) = a;
+            *reinterpret_cast<float4 *>(yr + 8 * g + 4) = b;
+        }
+    }
+}
+
+template <int MASK>
+static void launch_soft_max_masked(const float *x, int64_t ldx, const void *mask, int64_t ne00, int64_t ne01, int64_t n_rows,
+                                   float scale, float *y, int64_t ldy, hipStream_t st) {
+    const int64_t per = 8 * EW_THREADS;
+    const unsigned rows = (unsigned)n_rows;
+#define SM_GO(G) hipLaunchKernelGGL((soft_max_kernel<MASK, G>), dim3(rows), dim3(EW_THREADS), 0, st, x, ldx, mask, ne00, ne01, scale, y, ldy)
+    if (ne00 <= per) SM_GO(1);
+    else if (ne00 <= 2 * per) SM_GO(2);
+    else if (ne00 <= 4 * per) SM_GO(4);
+    else SM_GO(0);
+#undef SM_GO
+}
+hipError_t launch_soft_max(const float *x, int64_t ldx, const void *mask, int mask_f16, int64_t ne00, int64_t ne01, int64_t n_rows,
+                           float scale, float *y, int64_t ldy, hipStream_t st) {
+    if (n_rows <= 0 || ne00 <= 0) return hipSuccess;
+    if (n_rows > 0x7fffffff || ne00 % 8 != 0) return hipErrorInvalidValue;
+    if (!mask) launch_soft_max_masked<MASK_NONE>(x, ldx, nullptr, ne00, ne01, n_rows, scale, y, ldy, st);
+    else if (mask_f16) launch_soft_max_masked<MASK_F16>(x, ldx, mask, ne00, ne01, n_rows, scale, y, ldy, st);
+    else launch_soft_max_masked<MASK_F32>(x, ldx, mask, ne00, ne01, n_rows, scale, y, ldy, st);
+    return hipGetLastError();
+}
+
+// ---- CPY / CONT: same-shape strided copy with conversion; strides in bytes ----
+struct CopyShape { int64_t ne[4]; int64_t nbs[4]; int64_t nbd[4]; };
+template <typename S, typename D> __device__ __forceinline__ D cpy_conv(S v) {
+    if constexpr (sizeof(S) == sizeof(D)) return v;                              // same type: the bits
+    else if constexpr (sizeof(D) == 2) return f2h_rne(v);                        // F32 -> F16, nearest even
+    else return h2f(v);                                                          // F16 -> F32, exact
+}
+template <typename S, typename D> __device__ __forceinline__ void cpy_one(const char *s, char *d) {
+    *reinterpret_cast<D *>(d) = cpy_conv<S, D>(*reinterpret_cast<const S *>(s));
+}
+// one thread per element, destination-logical order (i0 fastest)
+template <typename S, typename D>
+__global__ __launch_bounds__(EW_THREADS) void cpy_kernel(const char *__restrict__ src, char *__restrict__ dst, CopyShape sh, int64_t total) {
+    for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (int64_t)gridDim.x * EW_THREADS) {
+        const int64_t i0 = i % sh.ne[0], r0 = i / sh.ne[0];
+        const int64_t i1 = r0 % sh.ne[1], r1 = r0 / sh.ne[1];
+        const int64_t i2 = r1 % sh.ne[2], i3 = r1 / sh.ne[2];
+        cpy_one<S, D>(src + i0 * sh.nbs[0] + i1 * sh.nbs[1] + i2 * sh.nbs[2] + i3 * sh.nbs[3],
+                      dst + i0 * sh.nbd[0] + i1 * sh.nbd[1] + i2 * sh.nbd[2] + i3 * sh.nbd[3]);
+    }
+}
+// both sides dense in the same order: four elements per thread
+template <typename S, typename D>
+__global__ __launch_bounds__(EW_THREADS) void cpy_flat_kernel(const S *__restrict__ src, D *__restrict__ dst, int64_t total) {
+    const int64_t i = 4 * ((int64_t)blockIdx.x * EW_THREADS + threadIdx.x);
+    if (i + 3 < total) {
+        if constexpr (sizeof(S) == 4 && sizeof(D) == 2) {
+            const float4 v = *reinterpret_cast<const float4 *>(src + i);
+            u32x2 o;
+            o[0] = (uint32_t)f2h_rne(v.x) | ((uint32_t)f2h_rne(v.y) << 16);
+            o[1] = (uint32_t)f2h_rne(v.z) | ((uint32_t)f2h_rne(v.w) << 16);
+            *reinterpret_cast<u32x2 *>(dst + i) = o;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; k++) cpy_one<S, D>(reinterpret_cast<const char *>(src + i + k), reinterpret_cast<char *>(dst + i + k));
+        }
+    } else {
+        for (int64_t k = i; k < total; k++) cpy_one<S, D>(reinterpret_cast<const char *>(src + k), reinterpret_cast<char *>(dst + k));
+    }
+}
+// the source runs fastest along i1, the destination along i0: 32 x 32 tiles through LDS so that both sides see
+// consecutive lanes on consecutive addresses
+template <typename S, typename D>
+__global__ __launch_bounds__(EW_THREADS) void cpy_transpose_kernel(const char *__restrict__ src, char *__restrict__ dst, CopyShape sh) {
+    __shared__ S tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int64_t t0 = (int64_t)blockIdx.x * 32, t1 = (int64_t)blockIdx.y * 32;
+    const int64_t i2 = blockIdx.z % sh.ne[2], i3 = blockIdx.z / sh.ne[2];
+    const char *s = src + i2 * sh.nbs[2] + i3 * sh.nbs[3];
+    char *d = dst + i2 * sh.nbd[2] + i3 * sh.nbd[3];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int64_t i0 = t0 + ty + 8 * r, i1 = t1 + tx;
+        if (i0 < sh.ne[0] && i1 < sh.ne[1]) tile[ty + 8 * r][tx] = *reinterpret_cast<const S *>(s + i0 * sh.nbs[0] + i1 * sh.nbs[1]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int64_t i0 = t0 + tx, i1 = t1 + ty + 8 * r;
+        if (i0 < sh.ne[0] && i1 < sh.ne[1])
+            *reinterpret_cast<D *>(d + i0 * sh.nbd[0] + i1 * sh.nbd[1]) = cpy_conv<S, D>(tile[tx][ty + 8 * r]);
+    }
+}
+template <typename S, typename D>
+static hipError_t launch_cpy_typed(const void *src, void *dst, const CopyShape &sh, hipStream_t st) {
+    const int64_t total = sh.ne[0] * sh.ne[1] * sh.ne[2] * sh.ne[3];
+    bool dense_s = true, dense_d = true;
+    int64_t es = sizeof(S), ed = sizeof(D);
+    for (int k = 0; k < 4; k++) {
+        if (sh.ne[k] != 1 && sh.nbs[k] != es) dense_s = false;
+        if (sh.ne[k] != 1 && sh.nbd[k] != ed) dense_d = false;
+        es *= sh.ne[k]; ed *= sh.ne[k];
+    }
+    if (dense_s && dense_d && (((uintptr_t)src) & 15) == 0 && (((uintptr_t)dst) & 7) == 0) {
+        hipLaunchKernelGGL((cpy_flat_kernel<S, D>), dim3((unsigned)ceil_div(total, 4 * EW_THREADS)), dim3(EW_THREADS), 0, st,
+                           (const S *)src, (D *)dst, total);
+    } else if (sh.nbs[1] == (int64_t)sizeof(S) && sh.nbd[0] == (int64_t)sizeof(D) && sh.ne[0] >= 16 && sh.ne[1] >= 16 &&
+               sh.ne[2] * sh.ne[3] <= 65535) {
+        hipLaunchKernelGGL((cpy_transpose_kernel<S, D>), dim3((unsigned)ceil_div(sh.ne[0], 32), (unsigned)ceil_div(sh.ne[1], 32),
+                                                               (unsigned)(sh.ne[2] * sh.ne[3])),
+                           dim3(EW_THREADS), 0, st, (const char *)src, (char *)dst, sh);
+    } else {
+        const int64_t want = ceil_div(total, EW_THREADS);
+        hipLaunchKernelGGL((cpy_kernel<S, D>), dim3((unsigned)(want < (1 << 20) ? want : (1 << 20))), dim3(EW_THREADS), 0, st,
+                           (const char *)src, (char *)dst, sh, total);
+    }
+    return hipGetLastError();
+}
+hipError_t launch_cpy(const void *src, int src_f16, void *dst, int dst_f16, const int64_t *ne, const int64_t *nb_src,
+                      const int64_t *nb_dst, hipStream_t st) {
+    CopyShape sh;
+    for (int k = 0; k < 4; k++) { sh.ne[k] = ne[k]; sh.nbs[k] = nb_src[k]; sh.nbd[k] = nb_dst[k]; if (ne[k] <= 0) return hipSuccess; }
+    if (!src_f16 && !dst_f16) return launch_cpy_typed<float, float>(src, dst, sh, st);
+    if (!src_f16 && dst_f16) return launch_cpy_typed<float, uint16_t>(src, dst, sh, st);
+    if (src_f16 && dst_f16) return launch_cpy_typed<uint16_t, uint16_t>(src, dst, sh, st);
+    return launch_cpy_typed<uint16_t, float>(src, dst, sh, st);
+}
+
+// ---- ROPE: one workgroup per token; the first n_dims / 2 threads build that position's cos / sin table ----
+constexpr int ROPE_MAX_PAIRS = 256;
+__global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restrict__ x, const int32_t *__restrict__ pos,
+                                                          const float *__restrict__ freq_factors, RopeArgs a, float *__restrict__ y) {
+    __shared__ float cs[ROPE_MAX_PAIRS], sn[ROPE_MAX_PAIRS];
+    const int64_t tok = blockIdx.x;
+    const int half = a.n_dims / 2;
+    for (int p = threadIdx.x; p < half; p += EW_THREADS) {
+        float theta = (float)(int64_t)pos[tok];
+        for (int k = 0; k < p; k++) theta *= a.theta_scale;
+        const float ff = freq_factors ? freq_factors[p] : 1.0f;
+        const float extrap = theta / ff;
+        const float interp = a.freq_scale * extrap;
+        float th = interp;
+        if (a.ext_factor != 0.0f) {
+            const float d = a.corr1 - a.corr0;
+            const float yv = ((float)p - a.corr0) / fmaxf(0.001f, d);
+            const float ramp_mix = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * a.ext_factor;
+            th = interp * (1.0f - ramp_mix) + extrap * ramp_mix;
+        }
+        cs[p] = (float)cos((double)th) * a.mscale;
+        sn[p] = (float)sin((double)th) * a.mscale;
+    }
+    __syncthreads();
+    const float *xt = x + tok * a.ldx2;
+    float *yt = y + tok * a.ldy2;
+    const int64_t per_head = a.ne0 - half;                       // one item per rotated pair or per passed-through value
+    for (int64_t i = threadIdx.x; i < a.ne1 * per_head; i += EW_THREADS) {
+        const int64_t h = i / per_head, j = i % per_head;
+        const float *xr = xt + h * a.ldx1;
+        float *yr = yt + h * a.ldy1;
+        if (j < half) {
+            const int64_t ia = a.neox ? j : 2 * j, ib = a.neox ? j + half : 2 * j + 1;
+            const float x0 = xr[ia], x1 = xr[ib], c = cs[j], s = sn[j];
+            yr[ia] = x0 * c - x1 * s;
+            yr[ib] = x0 * s + x1 * c;
+        } else {
+            yr[j + half] = xr[j + half];
+        }
+    }
+}
+hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, hipStream_t st) {
+    if (a.ne0 <= 0 || a.ne1 <= 0 || a.ne2 <= 0) return hipSuccess;
+    if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a.ne2), dim3(EW_THREADS), 0, st, x, pos, freq_factors, a, y);
+    return hipGetLastError();
 }
 
 hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, float *y, int64_t ldy, hipStream_t st) {

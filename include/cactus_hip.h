@@ -179,6 +179,34 @@ CHIP_API int chip_mul(const float *a, int64_t lda, const float *b, int64_t ldb, 
                       float *y, int64_t ldy, void *stream);
 CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream);
 
+/* ---- the attention-side ops around the KV cache ----
+ *   chip_soft_max : LM_GGML_OP_SOFT_MAX (lm_ggml_soft_max_ext), lm_ggml_compute_forward_soft_max_f32 (ggml-cpu/ops.cpp:4731-4827):
+ *                   y[r] = softmax(x[r] * scale + mask[r % ne01]) over n_rows rows of ne00 values; mask NULL, or a dense
+ *                   [>= ne01][ne00] matrix of mask_type LM_GGML_TYPE_F32 / _F16 shared by all heads.  Bit for bit the AVX2
+ *                   build (lm_ggml_v_expf, groups of 8 summed in the reference's order); ne00 must be a multiple of 8 (the
+ *                   reference finishes other rows with the C library's expf) and max_bias 0 (ALiBi slopes are declined).
+ *                   x, y, mask 16-byte aligned, ldx and ldy multiples of 4.  In place (y == x) is allowed.
+ *   chip_cpy      : LM_GGML_OP_CPY / LM_GGML_OP_CONT / LM_GGML_OP_DUP, lm_ggml_compute_forward_dup (ggml-cpu/ops.cpp), between
+ *                   F32 and F16 tensors of one shape ne[4] with byte strides nb_src[4] / nb_dst[4] (a contiguous tensor of
+ *                   another shape is passed as {total, 1, 1, 1}): the K-cache store (F32 -> F16, dense), the transposed
+ *                   V-cache store (transposed source, strided destination), the permuted attention output made dense.
+ *                   F32 -> F16 rounds to nearest even like LM_GGML_FP32_TO_FP16's F16C conversion.
+ *   chip_rope     : LM_GGML_OP_ROPE (lm_ggml_rope_ext), lm_ggml_compute_forward_rope_f32 (ggml-cpu/ops.cpp:5178-5361), modes 0
+ *                   (adjacent pairs) and LM_GGML_ROPE_TYPE_NEOX = 2; x, y F32 [ne2 tokens][ne1 heads][ne0] with head stride
+ *                   ld?1 and token stride ld?2 in elements, pos I32 [ne2], freq_factors F32 [n_dims / 2] or NULL; YaRN
+ *                   parameters as in the reference.  The angles follow the reference's float recurrence; cos and sin are
+ *                   computed in double and rounded once, where the reference calls the C library's cosf / sinf: results
+ *                   agree to one unit in the last place of cos / sin (|dy| <= 4e-7 * (|x0| + |x1|) * mscale).  Multi-section
+ *                   and vision modes are declined.  In place is allowed. */
+CHIP_API int chip_soft_max(const float *x, int64_t ldx, const void *mask, int mask_type, int64_t ne00, int64_t ne01,
+                           int64_t n_rows, float scale, float max_bias, float *y, int64_t ldy, void *stream);
+CHIP_API int chip_cpy(const void *src, int src_type, void *dst, int dst_type, const int64_t ne[4], const int64_t nb_src[4],
+                      const int64_t nb_dst[4], void *stream);
+CHIP_API int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0,
+                       int64_t ne1, int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                       float ext_factor, float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1,
+                       int64_t ldy2, void *stream);
+
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,
  * iq4_nl_q8_0} (ggml-cpu/ggml-cpu-quants.c:1906,3591,6772,8520,2924,7699,12751), computed with the same device

@@ -132,6 +132,10 @@ class Oracle:
         L.orc_rms_norm_f32.argtypes = [_vp, _vp, _i64, _i64, C.c_float]
         L.orc_silu_f32.restype = None
         L.orc_silu_f32.argtypes = [_vp, _vp, _i64, _i64]
+        L.orc_soft_max_f32.restype = None
+        L.orc_soft_max_f32.argtypes = [_vp, _vp, _i32, _i64, _i64, _i64, _i64, C.c_float, C.c_float, _vp]
+        L.orc_rope_f32.restype = None
+        L.orc_rope_f32.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _i32] + [C.c_float] * 6 + [_vp]
         L.orc_mul_mat_id.restype = _i32
         L.orc_mul_mat_id.argtypes = [_i32, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i32]
 
@@ -254,6 +258,42 @@ class Oracle:
         self.lib.orc_silu_f32(_ptr(x), _ptr(y), x.shape[0], x.shape[1])
         return y
 
+    def soft_max(self, x, mask=None, scale=1.0, max_bias=0.0):
+        """LM_GGML_OP_SOFT_MAX (lm_ggml_soft_max_ext): x fp32 [n_head, ne01, ne00]; mask fp32 or fp16 [>= ne01, ne00] or
+        None, shared by the heads."""
+        x = _f32(x)
+        n_head, ne01, ne00 = x.shape
+        y = np.empty_like(x)
+        if mask is not None:
+            mask = np.ascontiguousarray(mask)
+            assert mask.dtype in (np.float32, np.float16) and mask.shape[1] == ne00 and mask.shape[0] >= ne01
+        self.lib.orc_soft_max_f32(_ptr(x), _ptr(mask) if mask is not None else None,
+                                  int(mask is not None and mask.dtype == np.float16), ne00, ne01, n_head,
+                                  n_head * ne01, scale, max_bias, _ptr(y))
+        return y
+
+    def rope(self, x, pos, n_dims, mode, freq_factors=None, n_ctx_orig=4096, freq_base=10000.0, freq_scale=1.0,
+             ext_factor=0.0, attn_factor=1.0, beta_fast=32.0, beta_slow=1.0):
+        """LM_GGML_OP_ROPE (lm_ggml_rope_ext), text modes 0 and 2 (NEOX): x fp32 [n_tokens, n_head, ne0], pos int32
+        [n_tokens], freq_factors fp32 [n_dims / 2] or None."""
+        x = _f32(x)
+        pos = np.ascontiguousarray(pos, np.int32)
+        ne2, ne1, ne0 = x.shape
+        assert pos.shape == (ne2,) and n_dims % 2 == 0 and n_dims <= ne0 and mode in (0, 2)
+        ff = _f32(freq_factors) if freq_factors is not None else None
+        y = np.empty_like(x)
+        self.lib.orc_rope_f32(_ptr(x), _ptr(pos), _ptr(ff) if ff is not None else None, ne0, ne1, ne2, n_dims, mode,
+                              n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, _ptr(y))
+        return y
+
+    @staticmethod
+    def cpy(x, dst_dtype):
+        """LM_GGML_OP_CPY / CONT between F32 and F16 (reference ggml-cpu/ops.cpp lm_ggml_compute_forward_dup): element i of
+        the source, in the source's logical order, becomes element i of the destination; F32 -> F16 rounds to nearest
+        even (the F16C conversion of LM_GGML_FP32_TO_FP16), F16 -> F32 is exact.  x is a numpy array (or view) in the
+        source's logical order; the result is the destination's contents in its logical order."""
+        return np.ascontiguousarray(x).astype(dst_dtype)
+
     def mul_mat_id(self, wtype, W, x, ids, nthreads=1, want=()):
         """LM_GGML_OP_MUL_MAT_ID: W uint8 [n_as, N, row_size], x fp32 [n_tokens, ne11, K] (ne11 = 1 or n_used),
         ids int32 [n_tokens, n_used] -> y fp32 [n_tokens, n_used, N]."""
@@ -335,6 +375,24 @@ class Reference:
         L.lm_ggml_rms_norm.argtypes = [_vp, _vp, C.c_float]
         L.lm_ggml_mul_mat_id.restype = _vp
         L.lm_ggml_mul_mat_id.argtypes = [_vp, _vp, _vp, _vp]
+        L.lm_ggml_new_tensor_1d.restype = _vp
+        L.lm_ggml_new_tensor_1d.argtypes = [_vp, _i32, _i64]
+        L.lm_ggml_new_tensor_4d.restype = _vp
+        L.lm_ggml_new_tensor_4d.argtypes = [_vp, _i32, _i64, _i64, _i64, _i64]
+        L.lm_ggml_soft_max_ext.restype = _vp
+        L.lm_ggml_soft_max_ext.argtypes = [_vp, _vp, _vp, C.c_float, C.c_float]
+        L.lm_ggml_rope_ext.restype = _vp
+        L.lm_ggml_rope_ext.argtypes = [_vp, _vp, _vp, _vp, _i32, _i32, _i32] + [C.c_float] * 6
+        for n_ in ("lm_ggml_cpy",):
+            getattr(L, n_).restype = _vp
+            getattr(L, n_).argtypes = [_vp, _vp, _vp]
+        for n_ in ("lm_ggml_cont", "lm_ggml_transpose"):
+            getattr(L, n_).restype = _vp
+            getattr(L, n_).argtypes = [_vp, _vp]
+        L.lm_ggml_permute.restype = _vp
+        L.lm_ggml_permute.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32]
+        L.lm_ggml_view_2d.restype = _vp
+        L.lm_ggml_view_2d.argtypes = [_vp, _vp, _i64, _i64, C.c_size_t, C.c_size_t]
         L.lm_ggml_new_graph.restype = _vp
         L.lm_ggml_new_graph.argtypes = [_vp]
         L.lm_ggml_build_forward_expand.restype = None
@@ -481,6 +539,90 @@ class Reference:
         L.lm_ggml_backend_free(be)
         L.lm_ggml_free(ctx)
         return y
+
+    def _run_graph(self, build, inputs, out_shape, out_dtype, nthreads=1, n_tensors=16):
+        """Builds a graph with build(ctx) -> (result node, {name: tensor}), uploads inputs[name], computes on the reference
+        CPU backend and returns the result node's bytes as an array of out_shape / out_dtype."""
+        L = self.lib
+        ctx = L.lm_ggml_init(_InitParams(L.lm_ggml_tensor_overhead() * n_tensors + L.lm_ggml_graph_overhead() + 4096,
+                                         None, True))
+        c, tensors = build(ctx)
+        g = L.lm_ggml_new_graph(ctx)
+        L.lm_ggml_build_forward_expand(g, c)
+        be = L.lm_ggml_backend_cpu_init()
+        L.lm_ggml_backend_cpu_set_n_threads(be, nthreads)
+        buf = L.lm_ggml_backend_alloc_ctx_tensors(ctx, be)
+        for name, t in tensors.items():
+            a = np.ascontiguousarray(inputs[name])
+            L.lm_ggml_backend_tensor_set(t, _ptr(a), 0, a.nbytes)
+        assert L.lm_ggml_backend_graph_compute(be, g) == 0
+        y = np.zeros(out_shape, out_dtype)
+        L.lm_ggml_backend_tensor_get(c, _ptr(y), 0, y.nbytes)
+        L.lm_ggml_backend_buffer_free(buf)
+        L.lm_ggml_backend_free(be)
+        L.lm_ggml_free(ctx)
+        return y
+
+    def soft_max_graph(self, x, mask=None, scale=1.0, max_bias=0.0, nthreads=1):
+        """lm_ggml_soft_max_ext on the reference CPU backend: x fp32 [n_head, ne01, ne00], mask fp32 / fp16 [>= ne01, ne00]."""
+        L = self.lib
+        x = _f32(x)
+        n_head, ne01, ne00 = x.shape
+        F16 = 1
+
+        def build(ctx):
+            tx = L.lm_ggml_new_tensor_3d(ctx, F32, ne00, ne01, n_head)
+            ts = {"x": tx}
+            tm = None
+            if mask is not None:
+                tm = L.lm_ggml_new_tensor_2d(ctx, F16 if mask.dtype == np.float16 else F32, ne00, mask.shape[0])
+                ts["mask"] = tm
+            return L.lm_ggml_soft_max_ext(ctx, tx, tm, scale, max_bias), ts
+        return self._run_graph(build, {"x": x, "mask": mask}, x.shape, np.float32, nthreads)
+
+    def rope_graph(self, x, pos, n_dims, mode, freq_factors=None, n_ctx_orig=4096, freq_base=10000.0, freq_scale=1.0,
+                   ext_factor=0.0, attn_factor=1.0, beta_fast=32.0, beta_slow=1.0, nthreads=1):
+        """lm_ggml_rope_ext on the reference CPU backend: x fp32 [n_tokens, n_head, ne0], pos int32 [n_tokens]."""
+        L = self.lib
+        x = _f32(x)
+        ne2, ne1, ne0 = x.shape
+        I32 = 26
+
+        def build(ctx):
+            tx = L.lm_ggml_new_tensor_3d(ctx, F32, ne0, ne1, ne2)
+            tp = L.lm_ggml_new_tensor_1d(ctx, I32, ne2)
+            ts = {"x": tx, "pos": tp}
+            tf = None
+            if freq_factors is not None:
+                tf = L.lm_ggml_new_tensor_1d(ctx, F32, len(freq_factors))
+                ts["ff"] = tf
+            return L.lm_ggml_rope_ext(ctx, tx, tp, tf, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor,
+                                      attn_factor, beta_fast, beta_slow), ts
+        return self._run_graph(build, {"x": x, "pos": np.ascontiguousarray(pos, np.int32),
+                                       "ff": _f32(freq_factors) if freq_factors is not None else None},
+                               x.shape, np.float32, nthreads)
+
+    def cpy_graph(self, x, dst_dtype, kind, nthreads=1):
+        """lm_ggml_cpy / lm_ggml_cont on the reference CPU backend.  x [ne1, ne0] fp32 or fp16.  kind:
+          "flat"       contiguous source into a 1-D destination of dst_dtype (the K-cache store);
+          "transpose"  the transposed source into a [ne0, ne1] destination (the transposed V-cache store);
+          "cont"       lm_ggml_cont of the transposed source (same type).
+        Returns the destination in its logical order."""
+        L = self.lib
+        x = np.ascontiguousarray(x)
+        ne1, ne0 = x.shape
+        tt = {np.dtype(np.float32): F32, np.dtype(np.float16): 1}
+        st, dt = tt[x.dtype], tt[np.dtype(dst_dtype)]
+
+        def build(ctx):
+            tx = L.lm_ggml_new_tensor_2d(ctx, st, ne0, ne1)
+            if kind == "flat":
+                return L.lm_ggml_cpy(ctx, tx, L.lm_ggml_new_tensor_1d(ctx, dt, ne0 * ne1)), {"x": tx}
+            if kind == "transpose":
+                return L.lm_ggml_cpy(ctx, L.lm_ggml_transpose(ctx, tx), L.lm_ggml_new_tensor_2d(ctx, dt, ne1, ne0)), {"x": tx}
+            return L.lm_ggml_cont(ctx, L.lm_ggml_transpose(ctx, tx)), {"x": tx}
+        shape = (ne0 * ne1,) if kind == "flat" else (ne0, ne1)
+        return self._run_graph(build, {"x": x}, shape, np.dtype(dst_dtype) if kind != "cont" else x.dtype, nthreads)
 
     def mul_mat_id_graph(self, wtype, W, x, ids, nthreads=1):
         """LM_GGML_OP_MUL_MAT_ID on the reference CPU backend: W uint8 [n_as, N, row_size], x fp32

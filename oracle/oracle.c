@@ -1315,3 +1315,100 @@ void orc_silu_f32(const float *x, float *y, int64_t n_rows, int64_t ne0) {
     }
 }
 
+/* lm_ggml_compute_forward_soft_max_f32 (reference ggml-cpu/ops.cpp:4731-4827) with lm_ggml_vec_soft_max_f32's AVX2 branch
+ * (ggml-cpu/vec.cpp:198-208, 233-238).  Row i1 of x [n_rows][ne00]: w = x * scale + slope * mask[i1 % ne01] (mask fp32
+ * or fp16, one [ne01][ne00] matrix shared by all heads), max over the row, e = lm_ggml_v_expf(w - max) in groups of 8
+ * with the group summed in float as ((e0+e4)+(e2+e6)) + ((e1+e5)+(e3+e7)) and the groups added in double in row
+ * order, the tail (ne00 % 8) through the C library's expf; y = e * (float)(1.0 / sum).  ALiBi: head h = (i1 / ne01) %
+ * n_head gets slope m0^(h+1) or m1^(2(h - n_head_log2) + 1); max_bias == 0 means slope 1. */
+void orc_soft_max_f32(const float *x, const void *mask, int mask_is_f16, int64_t ne00, int64_t ne01, int64_t n_head,
+                      int64_t n_rows, float scale, float max_bias, float *y) {
+    const uint32_t n_head_log2 = 1u << (uint32_t)floor(log2((double)n_head));
+    const float m0 = powf(2.0f, -(max_bias) / n_head_log2);
+    const float m1 = powf(2.0f, -(max_bias / 2.0f) / n_head_log2);
+    float *w = (float *)malloc(sizeof(float) * (size_t)(ne00 > 0 ? ne00 : 1));
+    for (int64_t i1 = 0; i1 < n_rows; i1++) {
+        const uint32_t h = (uint32_t)((i1 / ne01) % n_head);
+        const float slope = (max_bias > 0.0f) ? (h < n_head_log2 ? powf(m0, h + 1) : powf(m1, 2 * (h - n_head_log2) + 1)) : 1.0f;
+        const float *xr = x + i1 * ne00;
+        float *yr = y + i1 * ne00;
+        for (int64_t i = 0; i < ne00; i++) w[i] = xr[i] * scale;
+        if (mask) {
+            const int64_t mr = (i1 % ne01) * ne00;
+            if (mask_is_f16) for (int64_t i = 0; i < ne00; i++) w[i] += slope * H2F(((const uint16_t *)mask)[mr + i]);
+            else             for (int64_t i = 0; i < ne00; i++) w[i] += slope * ((const float *)mask)[mr + i];
+        }
+        float mx = -INFINITY;
+        for (int64_t i = 0; i < ne00; i++) mx = mx > w[i] ? mx : w[i];
+        double sum = 0.0;
+        int64_t i = 0;
+        for (; i + 7 < ne00; i += 8) {
+            float e[8];
+            for (int l = 0; l < 8; l++) e[l] = yr[i + l] = v_expf_lane(w[i + l] - mx);
+            const float a0 = e[0] + e[4], a1 = e[1] + e[5], a2 = e[2] + e[6], a3 = e[3] + e[7];
+            sum += (double)((a0 + a2) + (a1 + a3));
+        }
+        for (; i < ne00; i++) {
+            const float v = expf(w[i] - mx);
+            sum += (double)v;
+            yr[i] = v;
+        }
+        const float inv = (float)(1.0 / sum);
+        for (int64_t k = 0; k < ne00; k++) yr[k] *= inv;
+    }
+    free(w);
+}
+
+/* lm_ggml_compute_forward_rope_f32 (reference ggml-cpu/ops.cpp:5178-5361) for the text modes (mode 0: adjacent pairs,
+ * LM_GGML_ROPE_TYPE_NEOX = 2: pairs half a rotation apart), with lm_ggml_rope_cache_init / rope_yarn (ops.cpp:5080-5118)
+ * and lm_ggml_rope_yarn_corr_dims (ggml.c:3749-3761).  x, y [ne2][ne1][ne0] contiguous (token, head, channel); pos
+ * [ne2]; freq_factors [n_dims / 2] or NULL.  theta runs through the float recurrence theta *= theta_scale from
+ * theta = pos; cosf / sinf are the C library's. */
+void orc_rope_f32(const float *x, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1, int64_t ne2,
+                  int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
+                  float attn_factor, float beta_fast, float beta_slow, float *y) {
+    const float theta_scale = powf(freq_base, -2.0f / n_dims);
+    float corr[2];
+    {
+        const float lo = n_dims * logf(n_ctx_orig / (beta_fast * 2 * (float)M_PI)) / (2 * logf(freq_base));
+        const float hi = n_dims * logf(n_ctx_orig / (beta_slow * 2 * (float)M_PI)) / (2 * logf(freq_base));
+        const float start = floorf(lo), end = ceilf(hi);
+        corr[0] = 0 > start ? 0 : start;
+        corr[1] = (n_dims - 1) < end ? (float)(n_dims - 1) : end;
+    }
+    const int neox = mode & 2;
+    float *cache = (float *)malloc(sizeof(float) * (size_t)(ne0 + 2));
+    for (int64_t i2 = 0; i2 < ne2; i2++) {
+        float theta = (float)(int64_t)pos[i2];
+        for (int64_t i0 = 0; i0 < ne0; i0 += 2) {
+            const float ff = freq_factors ? freq_factors[i0 / 2] : 1.0f;
+            const float theta_extrap = theta / ff;
+            const float theta_interp = freq_scale * theta_extrap;
+            float th = theta_interp, mscale = attn_factor;
+            if (ext_factor != 0.0f) {
+                const float d = corr[1] - corr[0];
+                const float yv = ((int)i0 / 2 - corr[0]) / (0.001f > d ? 0.001f : d);
+                const float ramp = 1 - (1 < (0 > yv ? 0 : yv) ? 1 : (0 > yv ? 0 : yv));
+                const float ramp_mix = ramp * ext_factor;
+                th = theta_interp * (1 - ramp_mix) + theta_extrap * ramp_mix;
+                mscale *= 1.0f + 0.1f * logf(1.0f / freq_scale);
+            }
+            cache[i0 + 0] = cosf(th) * mscale;
+            cache[i0 + 1] = sinf(th) * mscale;
+            theta *= theta_scale;
+        }
+        for (int64_t i1 = 0; i1 < ne1; i1++) {
+            const float *src = x + (i2 * ne1 + i1) * ne0;
+            float *dst = y + (i2 * ne1 + i1) * ne0;
+            for (int64_t i0 = 0; i0 < n_dims; i0 += 2) {
+                const float c = cache[i0], sn = cache[i0 + 1];
+                const int64_t a = neox ? i0 / 2 : i0, b = neox ? i0 / 2 + n_dims / 2 : i0 + 1;
+                const float x0 = src[a], x1 = src[b];
+                dst[a] = x0 * c - x1 * sn;
+                dst[b] = x0 * sn + x1 * c;
+            }
+            for (int64_t i0 = n_dims; i0 < ne0; i0++) dst[i0] = src[i0];
+        }
+    }
+    free(cache);
+}

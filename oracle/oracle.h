@@ -147,6 +147,16 @@ int orc_mul_mat_id(int type, int64_t K, int64_t N, int64_t n_as, const void *W, 
 void orc_rms_norm_f32(const float *x, float *y, int64_t n_rows, int64_t ne0, float eps);
 void orc_silu_f32(const float *x, float *y, int64_t n_rows, int64_t ne0);
 
+/* Attention-side ops (ggml-cpu/ops.cpp), contiguous rows.  orc_soft_max_f32: pinned bit-exact on oracle/_ref's
+ * lm_ggml_soft_max_ext graphs.  orc_rope_f32: pinned bit-exact on oracle/_ref's lm_ggml_rope_ext graphs on this host (both
+ * call the same C library cosf / sinf); a device computes those two functions itself, so its parity with this function
+ * is a tolerance, stated in the GPU test. */
+void orc_soft_max_f32(const float *x, const void *mask, int mask_is_f16, int64_t ne00, int64_t ne01, int64_t n_head,
+                      int64_t n_rows, float scale, float max_bias, float *y);
+void orc_rope_f32(const float *x, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1, int64_t ne2,
+                  int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
+                  float attn_factor, float beta_fast, float beta_slow, float *y);
+
 #ifdef __cplusplus
 }
 #endif

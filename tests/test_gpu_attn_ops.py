@@ -1,0 +1,220 @@
+"""GPU parity of the attention-side ops (SOFT_MAX, CPY / CONT, ROPE), through the C-ABI, against the CPU oracle (pinned
+bit-exact on the reference build).
+
+Bars: CPY / CONT bit-exact; SOFT_MAX within one fp32 ulp per element and bit-exact in practice (the exponentials and the
+group sums are the reference's operation by operation; only the double sum over the groups is ordered differently);
+ROPE |dy| <= 4e-7 * (|x0| + |x1|) * mscale per rotated pair (cos and sin may differ from the C library's by one unit in
+the last place), pass-through channels bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import cactus_amd
+    return cactus_amd.Device(0)
+
+
+def causal_mask(ne01, ne00, n_past, dtype, pad_rows=0):
+    m = np.full((ne01 + pad_rows, ne00), -np.inf, np.float32)
+    for i in range(ne01):
+        m[i, : min(ne00, n_past + i + 1)] = 0.0
+    return m.astype(dtype)
+
+
+def assert_soft_max_close(y, ref):
+    ulp = np.spacing(np.abs(ref))
+    assert (np.abs(y.astype(np.float64) - ref) <= ulp).all()
+    assert (y.view(np.uint32) == ref.view(np.uint32)).mean() > 0.999
+
+
+# (n_head, ne01, ne00): register-resident rows of 1, 2 and 4 groups per thread, and the streaming path beyond 8192 values
+SOFT_MAX_SHAPES = [(1, 1, 32), (4, 3, 256), (8, 5, 1000), (32, 1, 2048), (2, 16, 4096), (3, 2, 8192), (2, 3, 8200), (1, 2, 40000)]
+
+
+@pytest.mark.parametrize("n_head,ne01,ne00", SOFT_MAX_SHAPES)
+def test_soft_max(dev, orc, n_head, ne01, ne00):
+    rng = np.random.default_rng(n_head * 1000 + ne00)
+    x = (rng.standard_normal((n_head, ne01, ne00)) * 6).astype(np.float32)
+    x[0, 0, :8] = [30.0, -30.0, 88.0, -104.0, 0.0, 1e-3, -200.0, 50.0]
+    assert_soft_max_close(dev.soft_max(x), orc.soft_max(x))
+    for dt in (np.float32, np.float16):
+        mask = causal_mask(ne01, ne00, max(0, ne00 - ne01 - 3), dt, pad_rows=3)
+        for scale in (1.0, 0.08838834764831845):
+            ref = orc.soft_max(x, mask, scale)
+            y = dev.soft_max(x, mask, scale)
+            assert_soft_max_close(y, ref)
+            assert np.all(y[np.broadcast_to(np.isinf(mask[:ne01]), y.shape)] == 0.0)
+    bias = (rng.standard_normal((ne01, ne00)) * 2).astype(np.float32)
+    assert_soft_max_close(dev.soft_max(x, bias, 0.5), orc.soft_max(x, bias, 0.5))
+
+
+def test_soft_max_in_place_and_strided(dev, orc):
+    import cactus_amd as ca
+    rng = np.random.default_rng(2)
+    n_rows, ne00, ld = 6, 264, 272
+    buf = np.zeros((n_rows, ld), np.float32)
+    buf[:, :ne00] = rng.standard_normal((n_rows, ne00)) * 3
+    d = dev.to_device(buf)
+    dev.check(dev.lib.chip_soft_max(d.ptr, ld, None, ca.F32, ne00, n_rows, n_rows, 0.3, 0.0, d.ptr, ld, None))
+    dev.sync()
+    out = d.download(np.float32, buf.size).reshape(n_rows, ld)
+    assert_soft_max_close(np.ascontiguousarray(out[:, :ne00]), orc.soft_max(buf[None, :, :ne00], None, 0.3)[0])
+    assert np.array_equal(out[:, ne00:], buf[:, ne00:])                      # the padding between rows is untouched
+
+
+def test_soft_max_declines_what_it_does_not_restate(dev):
+    import cactus_amd as ca
+    x = dev.to_device(np.zeros((2, 64), np.float32))
+    L = dev.lib
+    assert L.chip_soft_max(x.ptr, 64, None, ca.F32, 60, 1, 2, 1.0, 0.0, x.ptr, 64, None) == ca.CHIP_EUNSUPPORTED   # row tail
+    assert L.chip_soft_max(x.ptr, 64, x.ptr, ca.F32, 64, 1, 2, 1.0, 8.0, x.ptr, 64, None) == ca.CHIP_EUNSUPPORTED  # ALiBi
+    assert L.chip_soft_max(x.ptr, 64, x.ptr, ca.Q8_0, 64, 1, 2, 1.0, 0.0, x.ptr, 64, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_soft_max(x.ptr, 62, None, ca.F32, 64, 1, 2, 1.0, 0.0, x.ptr, 64, None) == ca.CHIP_EINVAL
+    assert L.chip_soft_max(x.ptr, 64, None, ca.F32, 64, 1, 0, 1.0, 0.0, x.ptr, 64, None) == ca.CHIP_OK
+
+
+def cpy_inputs(shape, seed):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    x.reshape(-1)[:6] = [65504.0, 65520.0, 1e-8, -6.1e-5, 2049.0, 2051.0]         # fp16 max, overflow, underflow, ties
+    return x
+
+
+@pytest.mark.parametrize("ne1,ne0", [(1, 1024), (7, 96), (33, 130), (512, 1024), (5, 3)])
+def test_cpy_flat_and_transposed(dev, orc, ne1, ne0):
+    x = cpy_inputs((ne1, ne0), ne1 + ne0)
+    with np.errstate(all="ignore"):
+        h = x.astype(np.float16)
+        # the K-cache store: dense F32 -> dense F16
+        assert dev.cpy(x, np.float16).tobytes() == orc.cpy(x, np.float16).tobytes()
+        # CONT of a transposed view, every type pair
+        assert dev.cpy(x.T, np.float16).tobytes() == orc.cpy(x.T, np.float16).tobytes()
+        assert dev.cpy(x.T, np.float32).tobytes() == orc.cpy(x.T, np.float32).tobytes()
+        assert dev.cpy(h.T, np.float16).tobytes() == orc.cpy(h.T, np.float16).tobytes()
+        assert dev.cpy(h.T, np.float32).tobytes() == orc.cpy(h.T, np.float32).tobytes()
+        assert dev.cpy(h, np.float32).tobytes() == orc.cpy(h, np.float32).tobytes()
+
+
+@pytest.mark.parametrize("n_tokens,n_embd,kv_size,head", [(1, 1024, 4096, 77), (33, 256, 512, 100), (512, 1024, 2048, 1024)])
+def test_cpy_into_the_transposed_v_cache(dev, orc, n_tokens, n_embd, kv_size, head):
+    # reference llama-kv-cache.cpp:631-656: v_cur [n_tokens][n_embd] transposed into the view [n_embd rows of kv_size] at column `head`
+    x = cpy_inputs((n_tokens, n_embd), n_tokens)
+    with np.errstate(all="ignore"):
+        got = dev.cpy(x.T, np.float16, dst_strides=(kv_size * 2, 2), dst_elems=n_embd * kv_size).reshape(n_embd, kv_size)
+        want = np.zeros((n_embd, kv_size), np.float16)
+        want[:, :n_tokens] = orc.cpy(x.T, np.float16)
+    assert got.tobytes() == want.tobytes()
+    # placed at column `head` through the destination pointer: same bytes, shifted
+    import cactus_amd as ca
+    A = C.c_int64 * 4
+    dsrc = dev.to_device(x)
+    ddst = dev.alloc(n_embd * kv_size * 2)
+    ddst.upload(np.zeros(n_embd * kv_size, np.float16))
+    if head + n_tokens <= kv_size:
+        dev.check(dev.lib.chip_cpy(dsrc.ptr, ca.F32, ddst.ptr + 2 * head, ca.F16, A(n_tokens, n_embd, 1, 1), A(n_embd * 4, 4, 0, 0),
+                                   A(2, kv_size * 2, 0, 0), None))
+        dev.sync()
+        got = ddst.download(np.float16, n_embd * kv_size).reshape(n_embd, kv_size)
+        want = np.zeros((n_embd, kv_size), np.float16)
+        with np.errstate(all="ignore"):
+            want[:, head:head + n_tokens] = orc.cpy(x.T, np.float16)
+        assert got.tobytes() == want.tobytes()
+
+
+def test_cont_of_the_permuted_attention_output(dev, orc):
+    # reference llama-graph.cpp:1161-1163: kqv [n_head][n_tokens][head_dim] permuted to [n_tokens][n_head][head_dim] and made dense
+    rng = np.random.default_rng(4)
+    kqv = rng.standard_normal((8, 37, 64)).astype(np.float32)
+    view = kqv.transpose(1, 0, 2)
+    assert dev.cpy(view, np.float32).tobytes() == orc.cpy(view, np.float32).tobytes()
+    big = rng.standard_normal((2, 3, 5, 16)).astype(np.float32)
+    for perm in ((0, 2, 1, 3), (1, 0, 3, 2), (3, 2, 1, 0), (2, 3, 0, 1)):
+        v = big.transpose(perm)
+        assert dev.cpy(v, np.float32).tobytes() == orc.cpy(v, np.float32).tobytes()
+        assert dev.cpy(v, np.float16).tobytes() == orc.cpy(v, np.float16).tobytes()
+
+
+def test_cpy_rejects_bad_arguments(dev):
+    import cactus_amd as ca
+    A = C.c_int64 * 4
+    d = dev.alloc(1024)
+    L = dev.lib
+    ne, nb4, nb2 = A(16, 4, 1, 1), A(4, 64, 256, 256), A(2, 32, 128, 128)
+    assert L.chip_cpy(d.ptr, ca.Q8_0, d.ptr, ca.F16, ne, nb4, nb2, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_cpy(d.ptr, ca.F32, d.ptr, ca.Q8_0, ne, nb4, nb2, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_cpy(d.ptr, ca.F32, d.ptr + 512, ca.F16, ne, A(3, 64, 256, 256), nb2, None) == ca.CHIP_EINVAL
+    assert L.chip_cpy(d.ptr + 2, ca.F32, d.ptr + 512, ca.F16, ne, nb4, nb2, None) == ca.CHIP_EINVAL
+    assert L.chip_cpy(None, ca.F32, d.ptr, ca.F16, ne, nb4, nb2, None) == ca.CHIP_EINVAL
+    assert L.chip_cpy(None, ca.F32, None, ca.F16, A(0, 4, 1, 1), nb4, nb2, None) == ca.CHIP_OK
+
+
+def rope_tolerance(x, n_dims, mode, mscale):
+    half = n_dims // 2
+    tol = np.zeros_like(x, dtype=np.float64)
+    ax = np.abs(x.astype(np.float64))
+    if mode == 0:
+        pair = ax[..., 0:n_dims:2] + ax[..., 1:n_dims:2]
+        tol[..., 0:n_dims:2] = pair
+        tol[..., 1:n_dims:2] = pair
+    else:
+        pair = ax[..., :half] + ax[..., half:n_dims]
+        tol[..., :half] = pair
+        tol[..., half:n_dims] = pair
+    return 4e-7 * abs(mscale) * tol
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("ne0,n_dims,n_head,n_tokens", [(128, 128, 32, 1), (128, 128, 8, 7), (64, 32, 3, 2), (128, 64, 2, 7), (256, 256, 4, 3)])
+def test_rope(dev, orc, mode, ne0, n_dims, n_head, n_tokens):
+    rng = np.random.default_rng(ne0 + n_dims + mode)
+    x = rng.standard_normal((n_tokens, n_head, ne0)).astype(np.float32)
+    pos = np.array([0, 1, 17, 4095, 100000, 31, 2][:n_tokens], np.int32)
+    ff = (1.0 + rng.random(n_dims // 2) * 7).astype(np.float32)
+    cases = [({}, 1.0), (dict(freq_base=500000.0, freq_scale=0.25), 1.0), (dict(freq_factors=ff), 1.0),
+             (dict(freq_scale=0.25, ext_factor=1.0, attn_factor=1.2, n_ctx_orig=2048), 1.2 * (1.0 + 0.1 * np.log(4.0)))]
+    for kw, mscale in cases:
+        ref = orc.rope(x, pos, n_dims, mode, **kw)
+        y = dev.rope(x, pos, n_dims, mode, **kw)
+        assert (np.abs(y.astype(np.float64) - ref) <= rope_tolerance(x, n_dims, mode, mscale)).all(), kw
+        assert y[..., n_dims:].tobytes() == x[..., n_dims:].tobytes()
+        assert y[pos == 0].tobytes() == ref[pos == 0].tobytes()               # angle 0: cos 1, sin 0 exactly
+        assert (y.view(np.uint32) == ref.view(np.uint32)).mean() > 0.9        # most values agree to the bit
+
+
+def test_rope_strided_in_place(dev, orc):
+    # rope over the Q part of a fused QKV activation: head stride ne0, token stride 3 * n_head * ne0
+    import cactus_amd as ca
+    rng = np.random.default_rng(9)
+    n_tokens, n_head, ne0 = 5, 4, 64
+    qkv = rng.standard_normal((n_tokens, 3, n_head, ne0)).astype(np.float32)
+    pos = np.arange(10, 10 + n_tokens, dtype=np.int32)
+    d, dp = dev.to_device(qkv), dev.to_device(pos)
+    tok = 3 * n_head * ne0
+    dev.check(dev.lib.chip_rope(d.ptr, ne0, tok, dp.ptr, None, ne0, n_head, n_tokens, ne0, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0,
+                                d.ptr, ne0, tok, None))
+    dev.sync()
+    out = d.download(np.float32, qkv.size).reshape(qkv.shape)
+    ref = orc.rope(qkv[:, 0], pos, ne0, 2)
+    assert (np.abs(out[:, 0].astype(np.float64) - ref) <= rope_tolerance(qkv[:, 0], ne0, 2, 1.0)).all()
+    assert out[:, 1:].tobytes() == qkv[:, 1:].tobytes()
+
+
+def test_rope_declines_multi_section_modes(dev):
+    import cactus_amd as ca
+    d = dev.alloc(4096)
+    L = dev.lib
+    args = (None, 64, 1, 1, 64)
+    for mode in (8, 24):
+        assert L.chip_rope(d.ptr, 64, 64, d.ptr, None, 64, 1, 1, 64, mode, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, d.ptr, 64, 64,
+                           None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_rope(d.ptr, 64, 64, d.ptr, None, 64, 1, 1, 63, 0, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, d.ptr, 64, 64,
+                       None) == ca.CHIP_EINVAL
+    assert L.chip_rope(d.ptr, 64, 64, None, None, 64, 1, 1, 64, 0, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, d.ptr, 64, 64,
+                       None) == ca.CHIP_EINVAL

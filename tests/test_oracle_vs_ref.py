@@ -115,3 +115,87 @@ def test_add_and_mul_are_single_ieee_operations(ref):
         assert ref.op_graph("mul", x, y).tobytes() == (x * y).tobytes()
         assert ref.op_graph("mul", x, w).tobytes() == (x * w).tobytes()        # one row broadcast over all rows
         assert ref.op_graph("add", x, w).tobytes() == (x + w).tobytes()
+
+
+def causal_mask(ne01, ne00, n_past, dtype, pad_rows=0):
+    """The attention mask of a causal decoder: token i (of ne01 new ones after n_past cached) sees keys 0 .. n_past + i."""
+    m = np.full((ne01 + pad_rows, ne00), -np.inf, np.float32)
+    for i in range(ne01):
+        m[i, : min(ne00, n_past + i + 1)] = 0.0
+    return m.astype(dtype)
+
+
+@pytest.mark.parametrize("n_head,ne01,ne00,threads", [(1, 1, 32, 1), (4, 3, 256, 2), (8, 5, 1000, 3), (2, 16, 4096, 2), (3, 2, 13, 1)])
+def test_soft_max_graph(orc, ref, n_head, ne01, ne00, threads):
+    rng = np.random.default_rng(n_head * 1000 + ne00)
+    x = (rng.standard_normal((n_head, ne01, ne00)) * 6).astype(np.float32)
+    x[0, 0, : min(8, ne00)] = [30.0, -30.0, 88.0, -104.0, 0.0, 1e-3, -200.0, 50.0][: min(8, ne00)]
+    assert orc.soft_max(x).tobytes() == ref.soft_max_graph(x, nthreads=threads).tobytes()
+    for dt in (np.float32, np.float16):
+        mask = causal_mask(ne01, ne00, max(0, ne00 - ne01 - 3), dt, pad_rows=3)
+        for scale in (1.0, 0.08838834764831845):
+            a = orc.soft_max(x, mask, scale)
+            b = ref.soft_max_graph(x, mask, scale, nthreads=threads)
+            assert a.tobytes() == b.tobytes()
+            assert np.all(a[:, :, :][np.broadcast_to(np.isinf(mask[:ne01]), a.shape)] == 0.0)
+    # a finite additive mask (relative position bias) and ALiBi slopes
+    bias = (rng.standard_normal((ne01, ne00)) * 2).astype(np.float32)
+    assert orc.soft_max(x, bias, 0.5).tobytes() == ref.soft_max_graph(x, bias, 0.5, nthreads=threads).tobytes()
+    assert orc.soft_max(x, bias, 0.5, 8.0).tobytes() == ref.soft_max_graph(x, bias, 0.5, 8.0, nthreads=threads).tobytes()
+
+
+def test_soft_max_rows_sum_to_one(orc):
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((2, 4, 512)) * 4).astype(np.float32)
+    y = orc.soft_max(x, None, 0.7)
+    assert np.allclose(y.sum(-1, dtype=np.float64), 1.0, atol=1e-6)
+    ref64 = np.exp((x * np.float32(0.7)).astype(np.float64) - (x * np.float32(0.7)).max(-1, keepdims=True))
+    ref64 /= ref64.sum(-1, keepdims=True)
+    assert np.allclose(y, ref64, rtol=3e-6, atol=1e-12)
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("ne0,n_dims,n_head,n_tokens", [(128, 128, 4, 5), (64, 32, 3, 2), (128, 64, 2, 7)])
+def test_rope_graph(orc, ref, mode, ne0, n_dims, n_head, n_tokens):
+    rng = np.random.default_rng(ne0 + n_dims + mode)
+    x = rng.standard_normal((n_tokens, n_head, ne0)).astype(np.float32)
+    pos = np.array([0, 1, 17, 4095, 100000, 31, 2][:n_tokens], np.int32)
+    assert orc.rope(x, pos, n_dims, mode).tobytes() == ref.rope_graph(x, pos, n_dims, mode).tobytes()
+    kw = dict(freq_base=500000.0, freq_scale=0.25)
+    assert orc.rope(x, pos, n_dims, mode, **kw).tobytes() == ref.rope_graph(x, pos, n_dims, mode, **kw).tobytes()
+    ff = (1.0 + rng.random(n_dims // 2) * 7).astype(np.float32)
+    assert orc.rope(x, pos, n_dims, mode, ff).tobytes() == ref.rope_graph(x, pos, n_dims, mode, ff).tobytes()
+    yarn = dict(freq_scale=0.25, ext_factor=1.0, attn_factor=1.2, n_ctx_orig=2048)
+    assert orc.rope(x, pos, n_dims, mode, **yarn).tobytes() == ref.rope_graph(x, pos, n_dims, mode, **yarn).tobytes()
+
+
+def test_rope_is_a_rotation(orc):
+    # what the mathematics fixes: position 0 is the identity, pair norms are preserved, the angle of pair i at position
+    # p is p * base^(-2i / n_dims)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((3, 2, 64)).astype(np.float32)
+    pos = np.array([0, 5, 77], np.int32)
+    for mode in (0, 2):
+        y = orc.rope(x, pos, 64, mode)
+        assert y[0].tobytes() == x[0].tobytes()
+        pair = (lambda a: (a[..., 0::2], a[..., 1::2])) if mode == 0 else (lambda a: (a[..., :32], a[..., 32:]))
+        x0, x1 = pair(x.astype(np.float64))
+        y0, y1 = pair(y.astype(np.float64))
+        assert np.allclose(x0 ** 2 + x1 ** 2, y0 ** 2 + y1 ** 2, rtol=1e-5)
+        theta = pos[:, None, None].astype(np.float64) * 10000.0 ** (-2.0 * np.arange(32) / 64)
+        assert np.allclose(y0, x0 * np.cos(theta) - x1 * np.sin(theta), atol=2e-4)
+        assert np.allclose(y1, x0 * np.sin(theta) + x1 * np.cos(theta), atol=2e-4)
+
+
+@pytest.mark.parametrize("ne1,ne0", [(1, 1024), (7, 96), (33, 130)])
+def test_cpy_graphs(orc, ref, ne1, ne0):
+    rng = np.random.default_rng(ne1 + ne0)
+    x = (rng.standard_normal((ne1, ne0)) * 3).astype(np.float32)
+    x.reshape(-1)[:6] = [65504.0, 65520.0, 1e-8, -6.1e-5, 2049.0, 2051.0]     # fp16 max, overflow, underflow, ties
+    with np.errstate(all="ignore"):
+        assert orc.cpy(x, np.float16).reshape(-1).tobytes() == ref.cpy_graph(x, np.float16, "flat").tobytes()
+        assert orc.cpy(x.T, np.float16).tobytes() == ref.cpy_graph(x, np.float16, "transpose").tobytes()
+        assert orc.cpy(x.T, np.float32).tobytes() == ref.cpy_graph(x, np.float32, "cont").tobytes()
+        h = x.astype(np.float16)
+        assert orc.cpy(h.T, np.float16).tobytes() == ref.cpy_graph(h, np.float16, "cont").tobytes()
+        assert orc.cpy(h, np.float32).reshape(-1).tobytes() == ref.cpy_graph(h, np.float32, "flat").tobytes()
