@@ -296,6 +296,39 @@ def bench_extra(dev, hip, trace=True):
         ew_case("mul_%dx%d" % (n, ne0), lambda a, b, y, n_, e: L.chip_mul(a.ptr, e, b.ptr, e, n_, n_, e, y.ptr, e, st), n, ne0, 3)
         ew_case("add_%dx%d" % (n, ne0), lambda a, b, y, n_, e: L.chip_add(a.ptr, e, b.ptr, e, n_, n_, e, y.ptr, e, st), n, ne0, 3)
 
+    # attention-side ops at LLaMA-3-8B shapes (32 heads, 8 KV heads of 128): decode over 4096 cached keys, prefill of 512 tokens
+    def attn_side_cases():
+        A = C.c_int64 * 4
+        hd, n_head, n_head_kv, kv_size = 128, 32, 8, 8192
+        n_embd_kv = hd * n_head_kv
+        for n_tok, n_kv in ((1, 4096), (512, 512)):
+            rows = n_head * n_tok
+            kq = dev.to_device((rng.standard_normal((rows, n_kv)) * 4).astype(np.float32))
+            mask = dev.to_device(np.zeros((max(n_tok, 8), n_kv), np.float16))
+            us = time_runs(dev, hip, st, lambda: L.chip_soft_max(kq.ptr, n_kv, mask.ptr, ca.F16, n_kv, n_tok, rows, 0.088, 0.0,
+                                                                  kq.ptr, n_kv, st), 50)
+            byts = rows * n_kv * 8 + n_tok * n_kv * 2
+            out["soft_max_%dx%d" % (rows, n_kv)] = {"us": round(us, 2), "GBps": round(byts / us / 1e3, 1)}
+            q = dev.to_device(rng.standard_normal((n_tok, n_head, hd)).astype(np.float32))
+            pos = dev.to_device(np.arange(n_tok, dtype=np.int32))
+            us = time_runs(dev, hip, st, lambda: L.chip_rope(q.ptr, hd, hd * n_head, pos.ptr, None, hd, n_head, n_tok, hd, 2, 8192,
+                                                              500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, q.ptr, hd, hd * n_head, st), 50)
+            out["rope_%dx%dx%d" % (n_tok, n_head, hd)] = {"us": round(us, 2), "GBps": round(n_tok * n_head * hd * 8 / us / 1e3, 1)}
+            k = dev.to_device(rng.standard_normal((n_tok, n_embd_kv)).astype(np.float32))
+            cache = dev.alloc(kv_size * n_embd_kv * 2)
+            flat, one = A(n_tok * n_embd_kv, 1, 1, 1), n_tok * n_embd_kv
+            us = time_runs(dev, hip, st, lambda: L.chip_cpy(k.ptr, ca.F32, flat, A(4, 4 * one, 4 * one, 4 * one), cache.ptr, ca.F16, flat,
+                                                             A(2, 2 * one, 2 * one, 2 * one), st), 50)
+            out["k_store_%dx%d" % (n_tok, n_embd_kv)] = {"us": round(us, 2), "GBps": round(one * 6 / us / 1e3, 1)}
+            shape = A(n_tok, n_embd_kv, 1, 1)
+            us = time_runs(dev, hip, st, lambda: L.chip_cpy(k.ptr, ca.F32, shape, A(n_embd_kv * 4, 4, 0, 0), cache.ptr, ca.F16, shape,
+                                                             A(2, kv_size * 2, 0, 0), st), 50)
+            out["v_store_transposed_%dx%d" % (n_tok, n_embd_kv)] = {"us": round(us, 2), "GBps": round(one * 6 / us / 1e3, 1)}
+            for bf in (kq, mask, q, pos, k, cache):
+                bf.free()
+
+    attn_side_cases()
+
     # weight upload: one synchronous copy from pageable memory (what set_tensor does) against the loader's protocol of
     # four pinned 1 MB staging buffers with an event each (chunked set_tensor_async)
     def upload_case():

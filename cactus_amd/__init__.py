@@ -106,7 +106,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
     L.chip_silu.argtypes = [vp, i64, i64, i64, vp, i64, vp]
     L.chip_soft_max.argtypes = [vp, i64, vp, i32, i64, i64, i64, C.c_float, C.c_float, vp, i64, vp]
-    L.chip_cpy.argtypes = [vp, i32, vp, i32, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64), vp]
+    L.chip_cpy.argtypes = [vp, i32, C.POINTER(i64), C.POINTER(i64), vp, i32, C.POINTER(i64), C.POINTER(i64), vp]
     L.chip_rope.argtypes = [vp, i64, i64, vp, vp, i64, i64, i64, i32, i32, i32] + [C.c_float] * 6 + [vp, i64, i64, vp]
     L.chip_mul_mat_id_workspace_size.restype = sz
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
@@ -265,10 +265,11 @@ class Device:
         self.sync()
         return dy.download(np.float32, x.size).reshape(x.shape)
 
-    def cpy(self, x, dst_dtype, dst_strides=None, dst_elems=None):
-        """Copies the numpy array (or strided view) x, at most 4-D, into a destination of dst_dtype: dense, or with the
-        given byte strides (numpy order, slowest first) inside a zeroed region of dst_elems elements.  The source is
-        uploaded with the view's own strides.  Returns the destination region as a flat array."""
+    def cpy(self, x, dst_dtype, dst_strides=None, dst_elems=None, dst_shape=None):
+        """Copies the numpy array (or strided view) x, at most 4-D, into a destination of dst_dtype: dense (of x's shape,
+        or of dst_shape with the same element count), or with the given byte strides (numpy order, slowest first) inside
+        a zeroed region of dst_elems elements.  The source is uploaded with the view's own strides.  Returns the
+        destination region as a flat array."""
         base = x
         while isinstance(base.base, np.ndarray):
             base = base.base
@@ -279,16 +280,18 @@ class Device:
         pad = 4 - x.ndim
         ne = [1] * pad + list(x.shape)
         nbs = [0] * pad + list(x.strides)
+        dshape = list(dst_shape if dst_shape is not None else x.shape)
         if dst_strides is None:
-            dst_strides = list(np.empty(x.shape, dst_dtype).strides)
+            dst_strides = list(np.empty(dshape, dst_dtype).strides)
             dst_elems = x.size
-        nbd = [0] * pad + list(dst_strides)
+        ned = [1] * (4 - len(dshape)) + dshape
+        nbd = [0] * (4 - len(dshape)) + list(dst_strides)
         A = C.c_int64 * 4
         dsrc = self.to_device(base.reshape(-1).view(np.uint8))
         ddst = self.alloc(dst_elems * dst_dtype.itemsize)
         ddst.upload(np.zeros(dst_elems * dst_dtype.itemsize, np.uint8))
-        self.check(self.lib.chip_cpy(dsrc.ptr + off, types[x.dtype], ddst.ptr, types[dst_dtype], A(*ne[::-1]), A(*nbs[::-1]),
-                                     A(*nbd[::-1]), None))
+        self.check(self.lib.chip_cpy(dsrc.ptr + off, types[x.dtype], A(*ne[::-1]), A(*nbs[::-1]), ddst.ptr, types[dst_dtype],
+                                     A(*ned[::-1]), A(*nbd[::-1]), None))
         self.sync()
         return ddst.download(dst_dtype, dst_elems)
 

@@ -453,20 +453,22 @@ int chip_soft_max(const float *x, int64_t ldx, const void *mask, int mask_type, 
     return hip_rc(launch_soft_max(x, ldx, mask, mask_type == T_F16, ne00, ne01, n_rows, scale, y, ldy, (hipStream_t)stream));
 }
 
-int chip_cpy(const void *src, int src_type, void *dst, int dst_type, const int64_t ne[4], const int64_t nb_src[4],
-             const int64_t nb_dst[4], void *stream) {
+int chip_cpy(const void *src, int src_type, const int64_t ne_src[4], const int64_t nb_src[4], void *dst, int dst_type,
+             const int64_t ne_dst[4], const int64_t nb_dst[4], void *stream) {
     if ((src_type != T_F32 && src_type != T_F16) || (dst_type != T_F32 && dst_type != T_F16)) return CHIP_EUNSUPPORTED;
-    if (!ne || !nb_src || !nb_dst) return CHIP_EINVAL;
+    if (!ne_src || !nb_src || !ne_dst || !nb_dst) return CHIP_EINVAL;
     const int64_t es = src_type == T_F16 ? 2 : 4, ed = dst_type == T_F16 ? 2 : 4;
-    int64_t total = 1;
+    int64_t total_s = 1, total_d = 1;
     for (int k = 0; k < 4; k++) {
-        if (ne[k] < 0 || nb_src[k] < 0 || nb_dst[k] < 0) return CHIP_EINVAL;
+        if (ne_src[k] < 0 || ne_dst[k] < 0 || nb_src[k] < 0 || nb_dst[k] < 0) return CHIP_EINVAL;
         if (nb_src[k] % es != 0 || nb_dst[k] % ed != 0) return CHIP_EINVAL;
-        total *= ne[k];
+        total_s *= ne_src[k];
+        total_d *= ne_dst[k];
     }
-    if (total == 0) return CHIP_OK;
+    if (total_s != total_d) return CHIP_EINVAL;
+    if (total_s == 0) return CHIP_OK;
     if (!src || !dst || (((uintptr_t)src) % es) != 0 || (((uintptr_t)dst) % ed) != 0) return CHIP_EINVAL;
-    return hip_rc(launch_cpy(src, src_type == T_F16, dst, dst_type == T_F16, ne, nb_src, nb_dst, (hipStream_t)stream));
+    return hip_rc(launch_cpy(src, src_type == T_F16, ne_src, nb_src, dst, dst_type == T_F16, ne_dst, nb_dst, (hipStream_t)stream));
 }
 
 int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1,

@@ -290,6 +290,83 @@ int run_elementwise(backend_ctx *c, lm_ggml_tensor *op) {
     }
 }
 
+// ---- the attention-side ops around the KV cache (SOFT_MAX, ROPE, CPY / CONT / DUP) ----
+bool is_attn_side_op(int op) {
+    return op == LM_GGML_OP_SOFT_MAX || op == LM_GGML_OP_ROPE || op == LM_GGML_OP_CPY || op == LM_GGML_OP_CONT || op == LM_GGML_OP_DUP;
+}
+bool dense(const lm_ggml_tensor *t) {                   // lm_ggml_is_contiguous for the unquantized types
+    size_t want = (t->type == LM_GGML_TYPE_F16) ? 2 : 4;
+    for (int k = 0; k < LM_GGML_MAX_DIMS; k++) {
+        if (t->ne[k] != 1 && t->nb[k] != want) return false;
+        want *= (size_t)t->ne[k];
+    }
+    return true;
+}
+bool f32_or_f16(const lm_ggml_tensor *t) { return t->type == LM_GGML_TYPE_F32 || t->type == LM_GGML_TYPE_F16; }
+int64_t n_elements(const lm_ggml_tensor *t) { return t->ne[0] * t->ne[1] * t->ne[2] * t->ne[3]; }
+
+bool soft_max_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0], *m = op->src[1];
+    if (!a || a->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32 || !dense(a) || !dense(op) || !same_shape(a, op)) return false;
+    float max_bias;
+    std::memcpy(&max_bias, (const float *)op->op_params + 1, sizeof(float));
+    if (max_bias != 0.0f || a->ne[0] % 8 != 0 || a->ne[1] < 1) return false;            // no ALiBi; the AVX2 row tail
+    if (m && (!f32_or_f16(m) || !dense(m) || m->ne[0] != a->ne[0] || m->ne[1] < a->ne[1] || m->ne[2] != 1 || m->ne[3] != 1)) return false;
+    return true;
+}
+bool rope_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0], *pos = op->src[1], *ff = op->src[2];
+    if (!a || !pos || a->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32 || !same_shape(a, op) || a->ne[3] != 1) return false;
+    if (pos->type != LM_GGML_TYPE_I32 || pos->nb[0] != 4 || pos->ne[0] != a->ne[2]) return false;   // multi-section modes carry 4 * ne2 positions
+    const int n_dims = op->op_params[1], mode = op->op_params[2];
+    if ((mode != 0 && mode != 2) || n_dims <= 0 || (n_dims & 1) || n_dims > a->ne[0] || n_dims > 512) return false;
+    if (ff && (ff->type != LM_GGML_TYPE_F32 || ff->nb[0] != 4 || ff->ne[0] < n_dims / 2)) return false;
+    for (const lm_ggml_tensor *t : {a, (const lm_ggml_tensor *)op})
+        if (t->nb[0] != 4 || t->nb[1] % 4 != 0 || t->nb[2] % 4 != 0 || t->nb[1] < (size_t)t->ne[0] * 4) return false;
+    return true;
+}
+// CPY / CONT / DUP: node->data and node->nb are the destination's (for CPY the node is a view of src[1]).
+bool cpy_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0];
+    if (!a || !f32_or_f16(a) || !f32_or_f16(op) || n_elements(a) != n_elements(op)) return false;
+    return true;                                       // shapes may differ: element i of one logical order to element i of the other
+}
+bool attn_side_shape_ok(const lm_ggml_tensor *op) {
+    if (!elementwise_enabled()) return false;
+    switch (op->op) {
+        case LM_GGML_OP_SOFT_MAX: return soft_max_shape_ok(op);
+        case LM_GGML_OP_ROPE:     return rope_shape_ok(op);
+        default:               return cpy_shape_ok(op);
+    }
+}
+int run_attn_side(backend_ctx *c, lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0];
+    switch (op->op) {
+        case LM_GGML_OP_SOFT_MAX: {
+            const lm_ggml_tensor *m = op->src[1];
+            float scale, max_bias;
+            std::memcpy(&scale, (const float *)op->op_params + 0, sizeof(float));
+            std::memcpy(&max_bias, (const float *)op->op_params + 1, sizeof(float));
+            return chip_soft_max((const float *)a->data, a->ne[0], m ? m->data : nullptr, m ? (int)m->type : (int)LM_GGML_TYPE_F32, a->ne[0],
+                                 a->ne[1], a->ne[1] * a->ne[2] * a->ne[3], scale, max_bias, (float *)op->data, op->ne[0], c->stream);
+        }
+        case LM_GGML_OP_ROPE: {
+            const lm_ggml_tensor *pos = op->src[1], *ff = op->src[2];
+            float f[6];
+            std::memcpy(f, op->op_params + 5, sizeof(f));        // freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow
+            return chip_rope((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), (const int32_t *)pos->data,
+                             ff ? (const float *)ff->data : nullptr, a->ne[0], a->ne[1], a->ne[2], op->op_params[1], op->op_params[2],
+                             op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], (float *)op->data, (int64_t)(op->nb[1] / 4),
+                             (int64_t)(op->nb[2] / 4), c->stream);
+        }
+        default: {
+            int64_t nes[4], nbs[4], ned[4], nbd[4];
+            for (int k = 0; k < 4; k++) { nes[k] = a->ne[k]; nbs[k] = (int64_t)a->nb[k]; ned[k] = op->ne[k]; nbd[k] = (int64_t)op->nb[k]; }
+            return chip_cpy(a->data, a->type, nes, nbs, op->data, op->type, ned, nbd, c->stream);
+        }
+    }
+}
+
 static bool grow_workspace(backend_ctx *c, size_t need) {
     if (need <= c->workspace_size) return true;
     chip_stream_synchronize(c->stream);
@@ -310,6 +387,15 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_ADD || node->op == LM_GGML_OP_MUL || node->op == LM_GGML_OP_UNARY) &&
             elementwise_shape_ok(node)) {
             const int rc = run_elementwise(c, node);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            g_elementwise_nodes++;
+            continue;
+        }
+        if (is_attn_side_op(node->op) && attn_side_shape_ok(node)) {
+            const int rc = run_attn_side(c, node);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
                 return LM_GGML_STATUS_FAILED;
@@ -422,6 +508,7 @@ bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     // element-wise F32 ops run wherever their operands are put: the scheduler keeps them with the matmuls around them
     if (op->op == LM_GGML_OP_RMS_NORM || op->op == LM_GGML_OP_ADD || op->op == LM_GGML_OP_MUL || op->op == LM_GGML_OP_UNARY)
         return elementwise_shape_ok(op);
+    if (is_attn_side_op(op->op)) return attn_side_shape_ok(op);
     if (op->op != LM_GGML_OP_MUL_MAT && op->op != LM_GGML_OP_MUL_MAT_ID) return false;
     // Only weights that already live in a HIP buffer: claiming host-resident weights would make the scheduler
     // copy the whole matrix to the device on every call.  At model load the probe tensor carries a zero-size

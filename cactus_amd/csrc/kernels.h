@@ -179,9 +179,10 @@ hipError_t launch_silu(const float *x, int64_t ldx, int64_t ne0, int64_t n, floa
 // SOFT_MAX over n_rows rows of ne00 values (a multiple of 8); row r adds row r % ne01 of the mask (fp32 or fp16, dense).
 hipError_t launch_soft_max(const float *x, int64_t ldx, const void *mask, int mask_f16, int64_t ne00, int64_t ne01, int64_t n_rows,
                            float scale, float *y, int64_t ldy, hipStream_t st);
-// Same-shape copy between F32 / F16 tensors; ne in elements, strides in bytes.
-hipError_t launch_cpy(const void *src, int src_f16, void *dst, int dst_f16, const int64_t *ne, const int64_t *nb_src,
-                      const int64_t *nb_dst, hipStream_t st);
+// Copy between F32 / F16 tensors of one element count, element i of the source's logical order to element i of the
+// destination's; shapes in elements, strides in bytes.
+hipError_t launch_cpy(const void *src, int src_f16, const int64_t *ne_src, const int64_t *nb_src, void *dst, int dst_f16,
+                      const int64_t *ne_dst, const int64_t *nb_dst, hipStream_t st);
 struct RopeArgs {
     int64_t ne0, ne1, ne2;
     int64_t ldx1, ldx2, ldy1, ldy2;        // head and token strides in floats

@@ -250,7 +250,7 @@ hipError_t launch_soft_max(const float *x, int64_t ldx, const void *mask, int ma
 }
 
 // ---- CPY / CONT: same-shape strided copy with conversion; strides in bytes ----
-struct CopyShape { int64_t ne[4]; int64_t nbs[4]; int64_t nbd[4]; };
+struct CopyShape { int64_t ne[4]; int64_t nbs[4]; int64_t ned[4]; int64_t nbd[4]; };   // source shape / strides, destination shape / strides
 template <typename S, typename D> __device__ __forceinline__ D cpy_conv(S v) {
     if constexpr (sizeof(S) == sizeof(D)) return v;                              // same type: the bits
     else if constexpr (sizeof(D) == 2) return f2h_rne(v);                        // F32 -> F16, nearest even
@@ -259,16 +259,17 @@ template <typename S, typename D> __device__ __forceinline__ D cpy_conv(S v) {
 template <typename S, typename D> __device__ __forceinline__ void cpy_one(const char *s, char *d) {
     *reinterpret_cast<D *>(d) = cpy_conv<S, D>(*reinterpret_cast<const S *>(s));
 }
-// one thread per element, destination-logical order (i0 fastest)
+// one thread per element in logical order (i0 fastest); the two sides may have different shapes of one element count
+__device__ __forceinline__ int64_t cpy_offset(int64_t i, const int64_t (&ne)[4], const int64_t (&nb)[4]) {
+    const int64_t i0 = i % ne[0], r0 = i / ne[0];
+    const int64_t i1 = r0 % ne[1], r1 = r0 / ne[1];
+    const int64_t i2 = r1 % ne[2], i3 = r1 / ne[2];
+    return i0 * nb[0] + i1 * nb[1] + i2 * nb[2] + i3 * nb[3];
+}
 template <typename S, typename D>
 __global__ __launch_bounds__(EW_THREADS) void cpy_kernel(const char *__restrict__ src, char *__restrict__ dst, CopyShape sh, int64_t total) {
-    for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (int64_t)gridDim.x * EW_THREADS) {
-        const int64_t i0 = i % sh.ne[0], r0 = i / sh.ne[0];
-        const int64_t i1 = r0 % sh.ne[1], r1 = r0 / sh.ne[1];
-        const int64_t i2 = r1 % sh.ne[2], i3 = r1 / sh.ne[2];
-        cpy_one<S, D>(src + i0 * sh.nbs[0] + i1 * sh.nbs[1] + i2 * sh.nbs[2] + i3 * sh.nbs[3],
-                      dst + i0 * sh.nbd[0] + i1 * sh.nbd[1] + i2 * sh.nbd[2] + i3 * sh.nbd[3]);
-    }
+    for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (int64_t)gridDim.x * EW_THREADS)
+        cpy_one<S, D>(src + cpy_offset(i, sh.ne, sh.nbs), dst + cpy_offset(i, sh.ned, sh.nbd));
 }
 // both sides dense in the same order: four elements per thread
 template <typename S, typename D>
@@ -315,17 +316,18 @@ __global__ __launch_bounds__(EW_THREADS) void cpy_transpose_kernel(const char *_
 template <typename S, typename D>
 static hipError_t launch_cpy_typed(const void *src, void *dst, const CopyShape &sh, hipStream_t st) {
     const int64_t total = sh.ne[0] * sh.ne[1] * sh.ne[2] * sh.ne[3];
-    bool dense_s = true, dense_d = true;
+    bool dense_s = true, dense_d = true, same = true;
     int64_t es = sizeof(S), ed = sizeof(D);
     for (int k = 0; k < 4; k++) {
         if (sh.ne[k] != 1 && sh.nbs[k] != es) dense_s = false;
-        if (sh.ne[k] != 1 && sh.nbd[k] != ed) dense_d = false;
-        es *= sh.ne[k]; ed *= sh.ne[k];
+        if (sh.ned[k] != 1 && sh.nbd[k] != ed) dense_d = false;
+        if (sh.ne[k] != sh.ned[k]) same = false;
+        es *= sh.ne[k]; ed *= sh.ned[k];
     }
     if (dense_s && dense_d && (((uintptr_t)src) & 15) == 0 && (((uintptr_t)dst) & 7) == 0) {
         hipLaunchKernelGGL((cpy_flat_kernel<S, D>), dim3((unsigned)ceil_div(total, 4 * EW_THREADS)), dim3(EW_THREADS), 0, st,
                            (const S *)src, (D *)dst, total);
-    } else if (sh.nbs[1] == (int64_t)sizeof(S) && sh.nbd[0] == (int64_t)sizeof(D) && sh.ne[0] >= 16 && sh.ne[1] >= 16 &&
+    } else if (same && sh.nbs[1] == (int64_t)sizeof(S) && sh.nbd[0] == (int64_t)sizeof(D) && sh.ne[0] >= 16 && sh.ne[1] >= 16 &&
                sh.ne[2] * sh.ne[3] <= 65535) {
         hipLaunchKernelGGL((cpy_transpose_kernel<S, D>), dim3((unsigned)ceil_div(sh.ne[0], 32), (unsigned)ceil_div(sh.ne[1], 32),
                                                                (unsigned)(sh.ne[2] * sh.ne[3])),
@@ -337,10 +339,13 @@ static hipError_t launch_cpy_typed(const void *src, void *dst, const CopyShape &
     }
     return hipGetLastError();
 }
-hipError_t launch_cpy(const void *src, int src_f16, void *dst, int dst_f16, const int64_t *ne, const int64_t *nb_src,
-                      const int64_t *nb_dst, hipStream_t st) {
+hipError_t launch_cpy(const void *src, int src_f16, const int64_t *ne_src, const int64_t *nb_src, void *dst, int dst_f16,
+                      const int64_t *ne_dst, const int64_t *nb_dst, hipStream_t st) {
     CopyShape sh;
-    for (int k = 0; k < 4; k++) { sh.ne[k] = ne[k]; sh.nbs[k] = nb_src[k]; sh.nbd[k] = nb_dst[k]; if (ne[k] <= 0) return hipSuccess; }
+    for (int k = 0; k < 4; k++) {
+        sh.ne[k] = ne_src[k]; sh.nbs[k] = nb_src[k]; sh.ned[k] = ne_dst[k]; sh.nbd[k] = nb_dst[k];
+        if (ne_src[k] <= 0 || ne_dst[k] <= 0) return hipSuccess;
+    }
     if (!src_f16 && !dst_f16) return launch_cpy_typed<float, float>(src, dst, sh, st);
     if (!src_f16 && dst_f16) return launch_cpy_typed<float, uint16_t>(src, dst, sh, st);
     if (src_f16 && dst_f16) return launch_cpy_typed<uint16_t, uint16_t>(src, dst, sh, st);

@@ -187,9 +187,10 @@ CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, floa
  *                   reference finishes other rows with the C library's expf) and max_bias 0 (ALiBi slopes are declined).
  *                   x, y, mask 16-byte aligned, ldx and ldy multiples of 4.  In place (y == x) is allowed.
  *   chip_cpy      : LM_GGML_OP_CPY / LM_GGML_OP_CONT / LM_GGML_OP_DUP, lm_ggml_compute_forward_dup (ggml-cpu/ops.cpp), between
- *                   F32 and F16 tensors of one shape ne[4] with byte strides nb_src[4] / nb_dst[4] (a contiguous tensor of
- *                   another shape is passed as {total, 1, 1, 1}): the K-cache store (F32 -> F16, dense), the transposed
- *                   V-cache store (transposed source, strided destination), the permuted attention output made dense.
+ *                   F32 and F16 tensors of one element count: element i of the source in its logical order (shape
+ *                   ne_src[4], byte strides nb_src[4]) becomes element i of the destination (ne_dst[4], nb_dst[4]).  The
+ *                   K-cache store (F32 -> F16, both dense), the transposed V-cache store (transposed source, strided
+ *                   destination), the permuted attention output made dense under a new shape.
  *                   F32 -> F16 rounds to nearest even like LM_GGML_FP32_TO_FP16's F16C conversion.
  *   chip_rope     : LM_GGML_OP_ROPE (lm_ggml_rope_ext), lm_ggml_compute_forward_rope_f32 (ggml-cpu/ops.cpp:5178-5361), modes 0
  *                   (adjacent pairs) and LM_GGML_ROPE_TYPE_NEOX = 2; x, y F32 [ne2 tokens][ne1 heads][ne0] with head stride
@@ -200,8 +201,8 @@ CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, floa
  *                   and vision modes are declined.  In place is allowed. */
 CHIP_API int chip_soft_max(const float *x, int64_t ldx, const void *mask, int mask_type, int64_t ne00, int64_t ne01,
                            int64_t n_rows, float scale, float max_bias, float *y, int64_t ldy, void *stream);
-CHIP_API int chip_cpy(const void *src, int src_type, void *dst, int dst_type, const int64_t ne[4], const int64_t nb_src[4],
-                      const int64_t nb_dst[4], void *stream);
+CHIP_API int chip_cpy(const void *src, int src_type, const int64_t ne_src[4], const int64_t nb_src[4], void *dst, int dst_type,
+                      const int64_t ne_dst[4], const int64_t nb_dst[4], void *stream);
 CHIP_API int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0,
                        int64_t ne1, int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                        float ext_factor, float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1,

@@ -80,6 +80,7 @@ class Host:
         L.lm_ggml_backend_sched_get_tensor_backend.restype = vp
         L.lm_ggml_backend_sched_get_tensor_backend.argtypes = [vp, vp]
         L.lm_ggml_backend_sched_reset.argtypes = [vp]
+        L.lm_ggml_backend_sched_set_tensor_backend.argtypes = [vp, vp, vp]
         L.lm_ggml_backend_compare_graph_backend.restype = C.c_bool
         L.lm_ggml_backend_compare_graph_backend.argtypes = [vp, vp, vp, EVAL_CB, vp]
         L.lm_ggml_backend_dev_get_props.argtypes = [vp, C.POINTER(DevProps)]
@@ -113,6 +114,8 @@ class Host:
         L.lm_ggml_rms_norm.argtypes = [vp, vp, C.c_float]
         L.lm_ggml_soft_max.restype = vp
         L.lm_ggml_soft_max.argtypes = [vp, vp]
+        L.lm_ggml_sqr.restype = vp
+        L.lm_ggml_sqr.argtypes = [vp, vp]
         L.lm_ggml_new_tensor_1d.restype = vp
         L.lm_ggml_new_tensor_1d.argtypes = [vp, i32, i64]
         L.lm_ggml_set_name.restype = vp
@@ -123,6 +126,14 @@ class Host:
         L.lm_ggml_nbytes.argtypes = [vp]
         L.lm_ggml_reshape_2d.restype = vp
         L.lm_ggml_reshape_2d.argtypes = [vp, vp, i64, i64]
+        L.lm_ggml_reshape_3d.restype = vp
+        L.lm_ggml_reshape_3d.argtypes = [vp, vp, i64, i64, i64]
+        L.lm_ggml_view_1d.restype = vp
+        L.lm_ggml_view_1d.argtypes = [vp, vp, i64, sz]
+        L.lm_ggml_view_3d.restype = vp
+        L.lm_ggml_view_3d.argtypes = [vp, vp, i64, i64, i64, sz, sz, sz]
+        L.lm_ggml_cont_2d.restype = vp
+        L.lm_ggml_cont_2d.argtypes = [vp, vp, i64, i64]
 
     def context(self, n_tensors=32, with_graph=True):
         L = self.L

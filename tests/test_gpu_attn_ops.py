@@ -118,7 +118,8 @@ def test_cpy_into_the_transposed_v_cache(dev, orc, n_tokens, n_embd, kv_size, he
     ddst = dev.alloc(n_embd * kv_size * 2)
     ddst.upload(np.zeros(n_embd * kv_size, np.float16))
     if head + n_tokens <= kv_size:
-        dev.check(dev.lib.chip_cpy(dsrc.ptr, ca.F32, ddst.ptr + 2 * head, ca.F16, A(n_tokens, n_embd, 1, 1), A(n_embd * 4, 4, 0, 0),
+        shape = A(n_tokens, n_embd, 1, 1)
+        dev.check(dev.lib.chip_cpy(dsrc.ptr, ca.F32, shape, A(n_embd * 4, 4, 0, 0), ddst.ptr + 2 * head, ca.F16, shape,
                                    A(2, kv_size * 2, 0, 0), None))
         dev.sync()
         got = ddst.download(np.float16, n_embd * kv_size).reshape(n_embd, kv_size)
@@ -134,6 +135,8 @@ def test_cont_of_the_permuted_attention_output(dev, orc):
     kqv = rng.standard_normal((8, 37, 64)).astype(np.float32)
     view = kqv.transpose(1, 0, 2)
     assert dev.cpy(view, np.float32).tobytes() == orc.cpy(view, np.float32).tobytes()
+    assert dev.cpy(view, np.float32, dst_shape=(37, 8 * 64)).tobytes() == orc.cpy(view, np.float32).tobytes()    # lm_ggml_cont_2d
+    assert dev.cpy(view, np.float16, dst_shape=(37 * 8, 64)).tobytes() == orc.cpy(view, np.float16).tobytes()
     big = rng.standard_normal((2, 3, 5, 16)).astype(np.float32)
     for perm in ((0, 2, 1, 3), (1, 0, 3, 2), (3, 2, 1, 0), (2, 3, 0, 1)):
         v = big.transpose(perm)
@@ -147,12 +150,14 @@ def test_cpy_rejects_bad_arguments(dev):
     d = dev.alloc(1024)
     L = dev.lib
     ne, nb4, nb2 = A(16, 4, 1, 1), A(4, 64, 256, 256), A(2, 32, 128, 128)
-    assert L.chip_cpy(d.ptr, ca.Q8_0, d.ptr, ca.F16, ne, nb4, nb2, None) == ca.CHIP_EUNSUPPORTED
-    assert L.chip_cpy(d.ptr, ca.F32, d.ptr, ca.Q8_0, ne, nb4, nb2, None) == ca.CHIP_EUNSUPPORTED
-    assert L.chip_cpy(d.ptr, ca.F32, d.ptr + 512, ca.F16, ne, A(3, 64, 256, 256), nb2, None) == ca.CHIP_EINVAL
-    assert L.chip_cpy(d.ptr + 2, ca.F32, d.ptr + 512, ca.F16, ne, nb4, nb2, None) == ca.CHIP_EINVAL
-    assert L.chip_cpy(None, ca.F32, d.ptr, ca.F16, ne, nb4, nb2, None) == ca.CHIP_EINVAL
-    assert L.chip_cpy(None, ca.F32, None, ca.F16, A(0, 4, 1, 1), nb4, nb2, None) == ca.CHIP_OK
+    assert L.chip_cpy(d.ptr, ca.Q8_0, ne, nb4, d.ptr, ca.F16, ne, nb2, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_cpy(d.ptr, ca.F32, ne, nb4, d.ptr, ca.Q8_0, ne, nb2, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_cpy(d.ptr, ca.F32, ne, A(3, 64, 256, 256), d.ptr + 512, ca.F16, ne, nb2, None) == ca.CHIP_EINVAL
+    assert L.chip_cpy(d.ptr + 2, ca.F32, ne, nb4, d.ptr + 512, ca.F16, ne, nb2, None) == ca.CHIP_EINVAL
+    assert L.chip_cpy(None, ca.F32, ne, nb4, d.ptr, ca.F16, ne, nb2, None) == ca.CHIP_EINVAL
+    assert L.chip_cpy(d.ptr, ca.F32, ne, nb4, d.ptr + 512, ca.F16, A(16, 5, 1, 1), nb2, None) == ca.CHIP_EINVAL   # element counts differ
+    zero = A(0, 4, 1, 1)
+    assert L.chip_cpy(None, ca.F32, zero, nb4, None, ca.F16, zero, nb2, None) == ca.CHIP_OK
 
 
 def rope_tolerance(x, n_dims, mode, mscale):

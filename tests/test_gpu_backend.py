@@ -101,7 +101,7 @@ def test_unsupported_ops_are_declined(host):
     silu12 = L.lm_ggml_silu(ctx, x12)
     wide = host.tensor_2d(ctx, O.F32, 256, 4)
     add_bcast = L.lm_ggml_add(ctx, wide, x)                              # src1 [256, 2] repeated over [256, 4]
-    soft = L.lm_ggml_soft_max(ctx, x)
+    sqr = L.lm_ggml_sqr(ctx, x)
     view = L.lm_ggml_reshape_2d(ctx, x, 128, 4)
     buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
     assert L.lm_ggml_backend_dev_supports_op(dev, mm) is True
@@ -113,12 +113,12 @@ def test_unsupported_ops_are_declined(host):
     assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_silu(ctx, x)) is True
     assert L.lm_ggml_backend_dev_supports_op(dev, silu12) is False       # row tail: the reference uses libm's expf there
     assert L.lm_ggml_backend_dev_supports_op(dev, add_bcast) is False    # a broadcast other than one row
-    assert L.lm_ggml_backend_dev_supports_op(dev, soft) is False
+    assert L.lm_ggml_backend_dev_supports_op(dev, sqr) is False         # an op outside the path
     assert L.lm_ggml_backend_dev_supports_op(dev, view) is True
     # graph_compute on a node the device declined reports failure, it does not compute on the host
     be = L.lm_ggml_backend_dev_init(dev, None)
     g = L.lm_ggml_new_graph(ctx)
-    L.lm_ggml_build_forward_expand(g, soft)
+    L.lm_ggml_build_forward_expand(g, sqr)
     assert L.lm_ggml_backend_graph_compute(be, g) == -1                  # LM_GGML_STATUS_FAILED
     L.lm_ggml_backend_free(be)
     L.lm_ggml_backend_buffer_free(buf)
@@ -127,7 +127,7 @@ def test_unsupported_ops_are_declined(host):
 
 def test_scheduler_splits_between_hip_and_cpu(host, orc):
     """llama.cpp's flow: weights in a HIP buffer tagged USAGE_WEIGHTS, activations produced on the CPU; the
-    reference scheduler assigns the MUL_MATs and the ADD between them to HIP, the SOFT_MAX to the CPU, and copies
+    reference scheduler assigns the MUL_MATs and the ADD between them to HIP, the SQR (an op outside the path) to the CPU, and copies
     tensors across."""
     L = host.L
     K, N1, N2, n = 2048, 512, 256, 3
@@ -155,7 +155,7 @@ def test_scheduler_splits_between_hip_and_cpu(host, orc):
     s = L.lm_ggml_mul_mat(ctx, tw3, h)           # [N2, n]   (K = 512 = N1)
     out_add = L.lm_ggml_add(ctx, s, z)
     L.lm_ggml_set_output(out_add)
-    out = L.lm_ggml_soft_max(ctx, out_add)
+    out = L.lm_ggml_sqr(ctx, out_add)
     L.lm_ggml_set_output(out)
     g = L.lm_ggml_new_graph(ctx)
     L.lm_ggml_build_forward_expand(g, out)
@@ -176,8 +176,8 @@ def test_scheduler_splits_between_hip_and_cpu(host, orc):
     assert L.lm_ggml_backend_sched_get_tensor_backend(sched, out) == cpu
     assert L.lm_ggml_backend_sched_get_n_splits(sched) >= 2
     y = host.get(out_add, np.float32, (n, N2))
-    sm = host.get(out, np.float32, (n, N2))
-    assert np.allclose(sm.sum(axis=1), 1.0, atol=1e-5)
+    sq = host.get(out, np.float32, (n, N2))
+    assert sq.tobytes() == (y * y).tobytes()
     # reference: same graph entirely on the reference CPU path (through the oracle, bit-identical to it)
     hh = orc.mul_mat(O.Q4_K, w1, x)["y"]
     zz = orc.mul_mat(O.Q6_K, w2, x, want=("sum_abs",))
@@ -440,3 +440,122 @@ def test_ffn_block_stays_on_the_device(host, orc):
     L.lm_ggml_backend_free(cpu)
     L.lm_ggml_free(ctx)
     L.lm_ggml_free(wctx)
+
+
+def test_attention_side_nodes_run_on_the_device(host, orc):
+    """The nodes llama.cpp puts around the KV cache (reference llama-graph.cpp:1060-1166, llama-kv-cache.cpp:617-656): RoPE of
+    Q and K, the K store (F32 -> F16 into a 1-D view of the cache), the transposed V store, the masked soft-max and the
+    permuted attention output made dense.  With the caches in a HIP buffer the reference scheduler gives the stores
+    (and the RoPE that feeds them) to the HIP backend by itself; results against the oracle."""
+    L = host.L
+    hd, n_head, n_head_kv, n_tokens, kv_size, head, n_kv = 64, 8, 2, 5, 256, 37, 64
+    n_embd_kv = hd * n_head_kv
+    rng = np.random.default_rng(12)
+    q_in = rng.standard_normal((n_tokens, n_head * hd)).astype(np.float32)
+    k_in = rng.standard_normal((n_tokens, n_embd_kv)).astype(np.float32)
+    v_in = rng.standard_normal((n_tokens, n_embd_kv)).astype(np.float32)
+    kq_in = (rng.standard_normal((n_head, n_tokens, n_kv)) * 4).astype(np.float32)
+    kqv_in = rng.standard_normal((n_head, n_tokens, hd)).astype(np.float32)
+    pos = np.arange(head, head + n_tokens, dtype=np.int32)
+    mask = np.full((8, n_kv), -np.inf, np.float32)                       # token rows padded to 8
+    for i in range(n_tokens):
+        mask[i, : head + i + 1] = 0.0
+    mask16 = mask.astype(np.float16)
+    scale = 1.0 / np.sqrt(hd)
+
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    cctx = host.context(with_graph=False)
+    kc = host.tensor_2d(cctx, O.F16, n_embd_kv, kv_size, "cache_k")
+    vc = host.tensor_2d(cctx, O.F16, kv_size, n_embd_kv, "cache_v")       # transposed V cache
+    cbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(cctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_clear(cbuf, 0)
+
+    ctx = host.context(n_tensors=64)
+    tq = host.tensor_2d(ctx, O.F32, n_head * hd, n_tokens, "q_in")
+    tk = host.tensor_2d(ctx, O.F32, n_embd_kv, n_tokens, "k_in")
+    tv = host.tensor_2d(ctx, O.F32, n_embd_kv, n_tokens, "v_in")
+    tkq = host.tensor_3d(ctx, O.F32, n_kv, n_tokens, n_head, "kq_in")
+    tkqv = host.tensor_3d(ctx, O.F32, hd, n_tokens, n_head, "kqv_in")
+    tpos = L.lm_ggml_new_tensor_1d(ctx, 26, n_tokens)
+    tmask = host.tensor_2d(ctx, O.F16, n_kv, 8, "mask")
+    for t in (tq, tk, tv, tkq, tkqv, tpos, tmask):
+        L.lm_ggml_set_input(t)
+    rope = lambda t, nh: L.lm_ggml_rope_ext(ctx, L.lm_ggml_reshape_3d(ctx, t, hd, nh, n_tokens), tpos, None, hd, 2, 4096, 10000.0, 1.0,
+                                         0.0, 1.0, 32.0, 1.0)
+    q = rope(tq, n_head)
+    k = rope(tk, n_head_kv)
+    k_store = L.lm_ggml_cpy(ctx, k, L.lm_ggml_view_1d(ctx, kc, n_tokens * n_embd_kv, 2 * n_embd_kv * head))
+    v_store = L.lm_ggml_cpy(ctx, L.lm_ggml_transpose(ctx, tv), L.lm_ggml_view_2d(ctx, vc, n_tokens, n_embd_kv, kv_size * 2, head * 2))
+    sm = L.lm_ggml_soft_max_ext(ctx, tkq, tmask, scale, 0.0)
+    out = L.lm_ggml_cont_2d(ctx, L.lm_ggml_permute(ctx, tkqv, 0, 2, 1, 3), hd * n_head, n_tokens)
+    g = L.lm_ggml_new_graph(ctx)
+    for t in (q, k_store, v_store, sm, out):
+        L.lm_ggml_set_output(t)
+        L.lm_ggml_build_forward_expand(g, t)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 128, False, True)
+    # in a model these nodes sit between HIP matmuls; here their inputs come from the host, so pin them like the reference
+    # pins its attention nodes (llama-graph.cpp:1165-1168)
+    for t in (q, sm, out):
+        L.lm_ggml_backend_sched_set_tensor_backend(sched, t, hip)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    for t, a in ((tq, q_in), (tk, k_in), (tv, v_in), (tkq, kq_in), (tkqv, kqv_in), (tpos, pos), (tmask, mask16)):
+        host.set(t, a)
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    for t in (k_store, v_store):
+        assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip     # stores into a HIP buffer must run there
+    y_q = host.get(q, np.float32, (n_tokens, n_head, hd))
+    y_sm = host.get(sm, np.float32, (n_head, n_tokens, n_kv))
+    y_out = host.get(out, np.float32, (n_tokens, n_head * hd))
+    y_kc = host.get(kc, np.float16, (kv_size, n_embd_kv))
+    y_vc = host.get(vc, np.float16, (n_embd_kv, kv_size))
+
+    q3 = q_in.reshape(n_tokens, n_head, hd)
+    want_q = orc.rope(q3, pos, hd, 2)
+    tol = 4e-7 * (np.abs(q3[..., : hd // 2]) + np.abs(q3[..., hd // 2:]))
+    assert (np.abs(y_q - want_q) <= np.concatenate([tol, tol], -1)).all()
+    want_k = orc.rope(k_in.reshape(n_tokens, n_head_kv, hd), pos, hd, 2).reshape(n_tokens, n_embd_kv)
+    want_kc = np.zeros((kv_size, n_embd_kv), np.float16)
+    want_kc[head:head + n_tokens] = want_k.astype(np.float16)
+    # the stored K went through the device's RoPE: equal to the oracle's within one fp16 step where the fp32 values straddle a tie
+    assert (np.abs(y_kc.astype(np.float32) - want_kc.astype(np.float32)) <= np.spacing(np.abs(want_kc)).astype(np.float32)).all()
+    assert (y_kc[:head] == 0).all() and (y_kc[head + n_tokens:] == 0).all()
+    want_vc = np.zeros((n_embd_kv, kv_size), np.float16)
+    want_vc[:, head:head + n_tokens] = v_in.T.astype(np.float16)
+    assert y_vc.tobytes() == want_vc.tobytes()
+    want_sm = orc.soft_max(kq_in, mask16, scale)
+    assert y_sm.tobytes() == want_sm.tobytes()
+    assert y_out.tobytes() == np.ascontiguousarray(kqv_in.transpose(1, 0, 2)).tobytes()
+    for t in (q, k, sm, out):
+        assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(cbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(cctx)
+
+
+def test_attention_side_ops_outside_the_restated_cases_are_declined(host):
+    """supports_op says no to what the kernels do not restate: ALiBi slopes, rows that are not a multiple of 8 values,
+    multi-section RoPE, copies into quantized tensors."""
+    L = host.L
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    ctx = host.context()
+    x = host.tensor_3d(ctx, O.F32, 64, 4, 2)
+    m = host.tensor_2d(ctx, O.F32, 64, 4)
+    assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_soft_max_ext(ctx, x, m, 1.0, 0.0))
+    assert not L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_soft_max_ext(ctx, x, m, 1.0, 8.0))
+    x2 = host.tensor_3d(ctx, O.F32, 60, 4, 2)
+    assert not L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_soft_max_ext(ctx, x2, None, 1.0, 0.0))
+    pos = L.lm_ggml_new_tensor_1d(ctx, 26, 2)
+    assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_rope_ext(ctx, x, pos, None, 64, 0, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0))
+    assert not L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_rope_ext(ctx, x, pos, None, 32, 24, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0))
+    q = host.tensor_2d(ctx, O.Q8_0, 64, 8)
+    x3 = host.tensor_2d(ctx, O.F32, 64, 8)
+    assert not L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_cpy(ctx, x3, q))
+    h = host.tensor_2d(ctx, O.F16, 64, 8)
+    assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_cpy(ctx, x3, h))
+    L.lm_ggml_free(ctx)
