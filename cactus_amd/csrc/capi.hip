@@ -440,6 +440,23 @@ int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int
     return hip_rc(launch_silu(x, ldx, ne0, n, y, ldy, (hipStream_t)stream));
 }
 
+// ---- attention matmuls over an F16 cache ----
+int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
+                             int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y, int64_t ldy1, int64_t ldy2,
+                             void *stream) {
+    if (K < 0 || N < 0 || n < 0 || ne02 < 0 || ne12 < 0) return CHIP_EINVAL;
+    if (ne02 > 0 && ne12 % ne02 != 0) return CHIP_EINVAL;                   // src1's batch must be a multiple of src0's
+    if (N == 0 || n == 0 || ne12 == 0) return CHIP_OK;
+    if (K == 0 || K % 8 != 0 || ne02 > 65535) return CHIP_EUNSUPPORTED;
+    if (!W || !x || !y) return CHIP_EINVAL;
+    if (!aligned16(W) || nb01 % 16 != 0 || nb02 % 16 != 0 || nb01 < (size_t)K * 2) return CHIP_EINVAL;
+    if (!aligned16(x) || ((ldx1 | ldx2) & 3) != 0 || (((uintptr_t)y) & 3) != 0 || ldy1 < N) return CHIP_EINVAL;
+    DeviceLimits lim;
+    if (int rc = current_limits(lim); rc != CHIP_OK) return rc;
+    return hip_rc(launch_mul_mat_f16_batched(W, nb01, nb02, K, N, ne02, x, ldx1, ldx2, n, ne12 / ne02, y, ldy1, ldy2, lim,
+                                             (hipStream_t)stream));
+}
+
 // ---- attention-side ops ----
 int chip_soft_max(const float *x, int64_t ldx, const void *mask, int mask_type, int64_t ne00, int64_t ne01, int64_t n_rows,
                   float scale, float max_bias, float *y, int64_t ldy, void *stream) {

@@ -215,6 +215,23 @@ bool mul_mat_shape_ok(const lm_ggml_tensor *op) {
     return true;
 }
 
+// The attention matmuls: F16 src0 [K, N, ne02] that is a strided view of the KV cache, F32 src1 [K, n, ne12] with ne12 a
+// multiple of ne02 (reference llama-graph.cpp:1120, 1154).  Anything the plain 2-D path takes goes there first.
+bool elementwise_enabled();
+bool mul_mat_f16_batched_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *w = op->src[0], *x = op->src[1];
+    if (!w || !x || w->type != LM_GGML_TYPE_F16 || x->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32) return false;
+    if (!elementwise_enabled()) return false;
+    const int64_t K = w->ne[0], N = w->ne[1];
+    if (K <= 0 || K % 8 != 0 || w->ne[3] != 1 || x->ne[3] != 1 || op->ne[3] != 1) return false;
+    if (w->ne[2] < 1 || w->ne[2] > 65535 || x->ne[2] % w->ne[2] != 0) return false;
+    if (x->ne[0] != K || op->ne[0] != N || op->ne[1] != x->ne[1] || op->ne[2] != x->ne[2]) return false;
+    if (w->nb[0] != 2 || w->nb[1] % 16 != 0 || w->nb[2] % 16 != 0 || w->nb[1] < (size_t)K * 2) return false;
+    if (x->nb[0] != 4 || x->nb[1] % 16 != 0 || x->nb[2] % 16 != 0) return false;
+    if (op->nb[0] != 4 || op->nb[1] % 4 != 0 || op->nb[2] % 4 != 0 || op->nb[1] < (size_t)N * 4) return false;
+    return true;
+}
+
 // The MUL_MAT_ID shapes: experts [K, N, n_as] stored one matrix after the other, F32 activations [K, ne11, n_tokens]
 // with ne11 = 1 or n_used and the rows of a token adjacent, I32 ids [n_used, n_tokens], F32 result
 // [N, n_used, n_tokens] with adjacent rows (reference ggml.c lm_ggml_mul_mat_id, ggml-cpu/ggml-cpu.c:1531-1710).
@@ -419,6 +436,18 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             g_mul_mat_nodes++;
             continue;
         }
+        if (node->op == LM_GGML_OP_MUL_MAT && !mul_mat_shape_ok(node) && mul_mat_f16_batched_shape_ok(node)) {
+            const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
+            const int rc = chip_mul_mat_f16_batched(w->data, w->nb[1], w->nb[2], w->ne[0], w->ne[1], w->ne[2], (const float *)x->data,
+                                                    (int64_t)(x->nb[1] / 4), (int64_t)(x->nb[2] / 4), x->ne[1], x->ne[2],
+                                                    (float *)node->data, (int64_t)(node->nb[1] / 4), (int64_t)(node->nb[2] / 4), c->stream);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: batched F16 MUL_MAT %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            g_mul_mat_nodes++;
+            continue;
+        }
         if (node->op != LM_GGML_OP_MUL_MAT || !mul_mat_shape_ok(node)) {
             HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: node %d (%s, op %d) is not supported by the HIP backend\n", __func__, i, node->name, node->op);
             return LM_GGML_STATUS_FAILED;
@@ -513,9 +542,11 @@ bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     // Only weights that already live in a HIP buffer: claiming host-resident weights would make the scheduler
     // copy the whole matrix to the device on every call.  At model load the probe tensor carries a zero-size
     // dummy buffer of the candidate buffer type and NULL data (reference llama-model.cpp:161-165,246-251).
+    // A view (the cache views of attention) answers with the buffer of the tensor it views, as the scheduler does.
     const lm_ggml_tensor *w = op->src[0];
-    if (!w || !w->buffer || !is_hip_buffer(w->buffer)) return false;
-    return op->op == LM_GGML_OP_MUL_MAT ? mul_mat_shape_ok(op) : mul_mat_id_shape_ok(op);
+    const lm_ggml_backend_buffer_t wbuf = !w ? nullptr : (w->view_src ? w->view_src->buffer : w->buffer);
+    if (!wbuf || !is_hip_buffer(wbuf)) return false;
+    return op->op == LM_GGML_OP_MUL_MAT ? (mul_mat_shape_ok(op) || mul_mat_f16_batched_shape_ok(op)) : mul_mat_id_shape_ok(op);
 }
 bool dev_supports_buft(lm_ggml_backend_dev_t, lm_ggml_backend_buffer_type_t buft) { return buft == hip_buffer_type(); }
 

@@ -179,6 +179,19 @@ CHIP_API int chip_mul(const float *a, int64_t lda, const float *b, int64_t ldb, 
                       float *y, int64_t ldy, void *stream);
 CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream);
 
+/* ---- the attention matmuls over an F16 KV cache ----
+ * LM_GGML_OP_MUL_MAT whose src0 is an F16, batched, strided view and whose src1 is F32 (reference llama-graph.cpp:1120
+ * kq = mul_mat(k, q) and :1154 kqv = mul_mat(v, kq); CPU path ggml-cpu/ggml-cpu.c:1177-1456 with
+ * type_traits_cpu[LM_GGML_TYPE_F16]: src1 rounded to fp16, lm_ggml_vec_dot_f16, ggml-cpu/vec.cpp:122-162):
+ *     y[b][t][r] = sum_k W[b / (ne12 / ne02)][r][k] * fp16(x[b][t][k])       b < ne12, t < n, r < N
+ * W: F16, rows of K halves at nb01 bytes, batches (KV heads) at nb02 bytes; x: F32 rows of K at ldx1 floats (tokens) and
+ * ldx2 floats (batches: query heads); y likewise, rows of N.  ne12 must be a multiple of ne02 (grouped-query broadcast,
+ * the reference's r2); a fourth dimension is not taken.  K a multiple of 8; W, nb01, nb02, x 16-byte aligned, ldx1 and
+ * ldx2 multiples of 4.  No workspace: the activations are rounded on the fly. */
+CHIP_API int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02,
+                                      const float *x, int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y,
+                                      int64_t ldy1, int64_t ldy2, void *stream);
+
 /* ---- the attention-side ops around the KV cache ----
  *   chip_soft_max : LM_GGML_OP_SOFT_MAX (lm_ggml_soft_max_ext), lm_ggml_compute_forward_soft_max_f32 (ggml-cpu/ops.cpp:4731-4827):
  *                   y[r] = softmax(x[r] * scale + mask[r % ne01]) over n_rows rows of ne00 values; mask NULL, or a dense

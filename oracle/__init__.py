@@ -244,6 +244,21 @@ class Oracle:
             out["sum_abs"] = sa
         return out
 
+    def mul_mat_f16_batched(self, W, x, want=()):
+        """LM_GGML_OP_MUL_MAT with a batched F16 src0 (ggml-cpu/ggml-cpu.c:1177-1456: src0's batch = src1's batch / r2):
+        W fp16 [ne02, N, K] (any view), x fp32 [ne12, n, K] (any view) -> y fp32 [ne12, n, N]."""
+        ne02, N, K = W.shape
+        ne12, n, _ = x.shape
+        assert ne12 % ne02 == 0
+        r2 = ne12 // ne02
+        y = np.zeros((ne12, n, N), np.float32)
+        sa = np.zeros((ne12, n, N), np.float64)
+        for b in range(ne12):
+            wb = np.ascontiguousarray(W[b // r2]).view(np.uint8).reshape(N, 2 * K)
+            o = self.mul_mat(F16, wb, np.ascontiguousarray(x[b]), want=("sum_abs",))
+            y[b], sa[b] = o["y"], o["sum_abs"]
+        return {"y": y, "sum_abs": sa} if "sum_abs" in want else {"y": y}
+
     def rms_norm(self, x, eps):
         """LM_GGML_OP_RMS_NORM over the rows of x fp32 [n, ne0]."""
         x = _f32(x)
@@ -623,6 +638,29 @@ class Reference:
             return L.lm_ggml_cont(ctx, L.lm_ggml_transpose(ctx, tx)), {"x": tx}
         shape = (ne0 * ne1,) if kind == "flat" else (ne0, ne1)
         return self._run_graph(build, {"x": x}, shape, np.dtype(dst_dtype) if kind != "cont" else x.dtype, nthreads)
+
+    def attention_matmul_graphs(self, k_cache, vt_cache, q, p, nthreads=1):
+        """The two attention matmuls as the reference builds them (llama-graph.cpp:1069-1071, 1120, 1154):
+        k_cache fp16 [n_kv, n_head_kv, hd] and q fp32 [n_tokens, n_head, hd], both permuted (0, 2, 1, 3) -> kq fp32
+        [n_head, n_tokens, n_kv]; vt_cache fp16 [hd, n_head_kv, n_kv] (the transposed V cache: positions fastest)
+        permuted likewise and p fp32 [n_head, n_tokens, n_kv] -> kqv fp32 [n_head, n_tokens, hd]."""
+        L = self.lib
+        n_kv, n_head_kv, hd = k_cache.shape
+        n_tokens, n_head, _ = q.shape
+        F16_ = 1
+
+        def build_kq(ctx):
+            tk = L.lm_ggml_new_tensor_3d(ctx, F16_, hd, n_head_kv, n_kv)
+            tq = L.lm_ggml_new_tensor_3d(ctx, F32, hd, n_head, n_tokens)
+            return L.lm_ggml_mul_mat(ctx, L.lm_ggml_permute(ctx, tk, 0, 2, 1, 3), L.lm_ggml_permute(ctx, tq, 0, 2, 1, 3)), {"k": tk, "q": tq}
+
+        def build_kqv(ctx):
+            tv = L.lm_ggml_new_tensor_3d(ctx, F16_, n_kv, n_head_kv, hd)
+            tp = L.lm_ggml_new_tensor_3d(ctx, F32, n_kv, n_tokens, n_head)
+            return L.lm_ggml_mul_mat(ctx, L.lm_ggml_permute(ctx, tv, 0, 2, 1, 3), tp), {"v": tv, "p": tp}
+        kq = self._run_graph(build_kq, {"k": k_cache, "q": _f32(q)}, (n_head, n_tokens, n_kv), np.float32, nthreads)
+        kqv = self._run_graph(build_kqv, {"v": vt_cache, "p": _f32(p)}, (n_head, n_tokens, hd), np.float32, nthreads)
+        return kq, kqv
 
     def mul_mat_id_graph(self, wtype, W, x, ids, nthreads=1):
         """LM_GGML_OP_MUL_MAT_ID on the reference CPU backend: W uint8 [n_as, N, row_size], x fp32

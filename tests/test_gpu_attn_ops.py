@@ -223,3 +223,84 @@ def test_rope_declines_multi_section_modes(dev):
                        None) == ca.CHIP_EINVAL
     assert L.chip_rope(d.ptr, 64, 64, None, None, 64, 1, 1, 64, 0, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, d.ptr, 64, 64,
                        None) == ca.CHIP_EINVAL
+
+
+def attn_case(seed, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
+    """An F16 KV cache laid out like the reference's (K: [kv_size][n_head_kv * hd]; V transposed: [n_head_kv * hd][kv_size])
+    with n_kv positions in use, new queries and a probability tensor."""
+    rng = np.random.default_rng(seed)
+    k_cache = np.zeros((kv_size, n_head_kv, hd), np.float16)
+    k_cache[:n_kv] = rng.standard_normal((n_kv, n_head_kv, hd)).astype(np.float16)
+    vt_cache = np.zeros((n_head_kv, hd, kv_size), np.float16)
+    vt_cache[:, :, :n_kv] = rng.standard_normal((n_head_kv, hd, n_kv)).astype(np.float16)
+    q = rng.standard_normal((n_tokens, n_head, hd)).astype(np.float32)
+    p = rng.random((n_head, n_tokens, n_kv)).astype(np.float32)
+    p /= p.sum(-1, keepdims=True)
+    return k_cache, vt_cache, q, p
+
+
+# (hd, n_head, n_head_kv, n_tokens, n_kv, kv_size): LLaMA-3-8B decode and a short prefill, multi-head attention, head sizes
+# that use 8 / 16 / 32 lanes per cache row, a GQA ratio that is no power of two, positions that are no multiple of 64
+ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8, 3, 96, 128), (256, 4, 2, 2, 160, 160),
+               (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128)]
+
+
+@pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", ATTN_SHAPES)
+def test_attention_matmuls_over_the_cache(dev, orc, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
+    k_cache, vt_cache, q, p = attn_case(hd + n_kv, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size)
+    # kq = mul_mat(k, q): the K cache as [n_head_kv][n_kv][hd] (rows one position apart), q as [n_head][n_tokens][hd]
+    kv = k_cache[:n_kv].transpose(1, 0, 2)
+    qv = q.transpose(1, 0, 2)
+    want = orc.mul_mat_f16_batched(kv, qv, want=("sum_abs",))
+    got = dev.mul_mat_f16_batched(kv, qv)
+    assert got.shape == (n_head, n_tokens, n_kv)
+    assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
+    # kqv = mul_mat(v, p): the transposed V cache as [n_head_kv][hd][n_kv] (rows kv_size apart)
+    vv = vt_cache[:, :, :n_kv]
+    want = orc.mul_mat_f16_batched(vv, p, want=("sum_abs",))
+    got = dev.mul_mat_f16_batched(vv, p)
+    assert got.shape == (n_head, n_tokens, hd)
+    assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
+
+
+def test_attention_matmul_exact_small_integers(dev):
+    # halves and activations that are small integers: every product and partial sum is exact in fp32, so any summation
+    # order gives the same bits, and a wrong index or a dropped term shows
+    rng = np.random.default_rng(8)
+    W = rng.integers(-8, 9, (3, 50, 72)).astype(np.float16)
+    x = rng.integers(-8, 9, (6, 4, 72)).astype(np.float32)
+    want = np.einsum("bnk,btk->btn", W.astype(np.float64)[np.arange(6) // 2], x.astype(np.float64)).astype(np.float32)
+    assert dev.mul_mat_f16_batched(W, x).tobytes() == want.tobytes()
+
+
+def test_attention_matmul_rounds_activations_to_fp16(dev, orc):
+    # 1 + 2^-11 is a tie in fp16 (rounds to 1), 1 + 2^-11 + 2^-20 rounds up to 1 + 2^-10; 65520 overflows to inf
+    W = np.ones((1, 1, 8), np.float16)
+    x = np.zeros((1, 3, 8), np.float32)
+    x[0, 0, 0] = 1 + 2.0 ** -11
+    x[0, 1, 0] = 1 + 2.0 ** -11 + 2.0 ** -20
+    x[0, 2, 0] = 65520.0
+    with np.errstate(all="ignore"):
+        got = dev.mul_mat_f16_batched(W, x)[0, :, 0]
+    assert got[0] == 1.0 and got[1] == np.float32(1 + 2.0 ** -10) and np.isinf(got[2])
+    assert got.tobytes() == orc.mul_mat_f16_batched(W, x)["y"][0, :, 0].tobytes()
+
+
+def test_attention_matmul_rejects_bad_arguments(dev):
+    import cactus_amd as ca
+    d = dev.alloc(1 << 16)
+    L = dev.lib
+    ok = (d.ptr, 256, 256 * 16, 128, 16, 2, d.ptr, 128, 512, 1, 4, d.ptr, 16, 16, None)
+    assert L.chip_mul_mat_f16_batched(*ok) == ca.CHIP_OK
+    dev.sync()
+
+    def call(i, v):
+        a = list(ok); a[i] = v
+        return L.chip_mul_mat_f16_batched(*a)
+    assert call(10, 3) == ca.CHIP_EINVAL              # ne12 not a multiple of ne02
+    assert call(3, 100) == ca.CHIP_EUNSUPPORTED       # K not a multiple of 8
+    assert call(1, 250) == ca.CHIP_EINVAL             # row stride not 16-byte aligned
+    assert call(0, d.ptr + 2) == ca.CHIP_EINVAL
+    assert call(7, 126) == ca.CHIP_EINVAL             # activation stride not a multiple of 4
+    assert call(6, None) == ca.CHIP_EINVAL
+    assert call(9, 0) == ca.CHIP_OK                   # no tokens

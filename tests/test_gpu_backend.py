@@ -559,3 +559,121 @@ def test_attention_side_ops_outside_the_restated_cases_are_declined(host):
     h = host.tensor_2d(ctx, O.F16, 64, 8)
     assert L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_cpy(ctx, x3, h))
     L.lm_ggml_free(ctx)
+
+
+def test_attention_block_stays_on_the_device(host, orc):
+    """A whole attention block as llama.cpp builds it without flash attention (reference llama-graph.cpp build_attn /
+    build_attn_mha :1060-1170, llama-kv-cache.cpp get_k / get_v / cpy_k / cpy_v): q/k/v projections, RoPE, the cache stores,
+    kq over the F16 K cache, masked soft-max, kqv over the transposed F16 V cache, the merge of the heads, the output
+    projection and the residual.  Weights and caches live in HIP buffers: the reference scheduler puts everything into
+    one HIP split."""
+    L = host.L
+    H, hd, n_head, n_head_kv, n_tokens, kv_size, head, n_kv = 1024, 64, 16, 4, 5, 256, 59, 64
+    n_embd_kv = hd * n_head_kv
+    rng = np.random.default_rng(31)
+    wq = orc.quantize_weights(O.Q4_K, common.weights_f32(41, n_head * hd, H))
+    wk = orc.quantize_weights(O.Q4_K, common.weights_f32(42, n_embd_kv, H))
+    wv = orc.quantize_weights(O.Q6_K, common.weights_f32(43, n_embd_kv, H))
+    wo = orc.quantize_weights(O.Q4_K, common.weights_f32(44, H, n_head * hd))
+    x = common.activations_f32(45, n_tokens, H)
+    pos = np.arange(head, head + n_tokens, dtype=np.int32)
+    mask = np.full((8, n_kv), -np.inf, np.float32)
+    for i in range(n_tokens):
+        mask[i, : head + i + 1] = 0.0
+    mask16 = mask.astype(np.float16)
+    scale = 1.0 / np.sqrt(hd)
+    # what the cache holds from earlier tokens
+    k_old = (rng.standard_normal((head, n_embd_kv)) * 0.5).astype(np.float16)
+    v_old = (rng.standard_normal((head, n_embd_kv)) * 0.5).astype(np.float16)
+    kc0 = np.zeros((kv_size, n_embd_kv), np.float16)
+    kc0[:head] = k_old
+    vc0 = np.zeros((n_embd_kv, kv_size), np.float16)
+    vc0[:, :head] = v_old.T
+
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    wctx = host.context(with_graph=False)
+    twq = host.tensor_2d(wctx, O.Q4_K, H, n_head * hd, "wq")
+    twk = host.tensor_2d(wctx, O.Q4_K, H, n_embd_kv, "wk")
+    twv = host.tensor_2d(wctx, O.Q6_K, H, n_embd_kv, "wv")
+    two = host.tensor_2d(wctx, O.Q4_K, n_head * hd, H, "wo")
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
+    for t, a in ((twq, wq), (twk, wk), (twv, wv), (two, wo)):
+        host.set(t, a)
+    cctx = host.context(with_graph=False)
+    kc = host.tensor_2d(cctx, O.F16, n_embd_kv, kv_size, "cache_k")
+    vc = host.tensor_2d(cctx, O.F16, n_embd_kv, kv_size, "cache_v")       # allocated like the reference; used transposed
+    cbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(cctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    host.set(kc, kc0)
+    host.set(vc, vc0)
+
+    ctx = host.context(n_tensors=96)
+    tx = host.tensor_2d(ctx, O.F32, H, n_tokens, "x")
+    tpos = L.lm_ggml_new_tensor_1d(ctx, 26, n_tokens)
+    tmask = host.tensor_2d(ctx, O.F16, n_kv, 8, "mask")
+    for t in (tx, tpos, tmask):
+        L.lm_ggml_set_input(t)
+    rope = lambda t, nh: L.lm_ggml_rope_ext(ctx, L.lm_ggml_reshape_3d(ctx, t, hd, nh, n_tokens), tpos, None, hd, 2, 4096, 10000.0, 1.0,
+                                         0.0, 1.0, 32.0, 1.0)
+    q = rope(L.lm_ggml_mul_mat(ctx, twq, tx), n_head)
+    k = rope(L.lm_ggml_mul_mat(ctx, twk, tx), n_head_kv)
+    v = L.lm_ggml_mul_mat(ctx, twv, tx)
+    k_store = L.lm_ggml_cpy(ctx, k, L.lm_ggml_view_1d(ctx, kc, n_tokens * n_embd_kv, 2 * n_embd_kv * head))
+    v_store = L.lm_ggml_cpy(ctx, L.lm_ggml_transpose(ctx, v), L.lm_ggml_view_2d(ctx, vc, n_tokens, n_embd_kv, kv_size * 2, head * 2))
+    kview = L.lm_ggml_view_3d(ctx, kc, hd, n_head_kv, n_kv, 2 * hd, 2 * n_embd_kv, 0)
+    vview = L.lm_ggml_view_3d(ctx, vc, n_kv, n_head_kv, hd, 2 * kv_size * hd, 2 * kv_size, 0)
+    qp = L.lm_ggml_permute(ctx, q, 0, 2, 1, 3)
+    kp = L.lm_ggml_permute(ctx, kview, 0, 2, 1, 3)
+    vp = L.lm_ggml_permute(ctx, vview, 0, 2, 1, 3)
+    kq = L.lm_ggml_mul_mat(ctx, kp, qp)
+    sm = L.lm_ggml_soft_max_ext(ctx, kq, tmask, scale, 0.0)
+    kqv = L.lm_ggml_mul_mat(ctx, vp, sm)
+    merged = L.lm_ggml_cont_2d(ctx, L.lm_ggml_permute(ctx, kqv, 0, 2, 1, 3), hd * n_head, n_tokens)
+    out = L.lm_ggml_add(ctx, L.lm_ggml_mul_mat(ctx, two, merged), tx)
+    L.lm_ggml_set_output(out)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, k_store)          # the stores first, as the reference builds its graph
+    L.lm_ggml_build_forward_expand(g, v_store)
+    L.lm_ggml_build_forward_expand(g, out)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 128, False, True)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(tx, x); host.set(tpos, pos); host.set(tmask, mask16)
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
+    for t in (q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
+        assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
+    y = host.get(out, np.float32, (n_tokens, H))
+    y_kc = host.get(kc, np.float16, (kv_size, n_embd_kv))
+    y_vc = host.get(vc, np.float16, (n_embd_kv, kv_size))
+
+    # the same chain on the oracle
+    q_ = orc.rope(orc.mul_mat(O.Q4_K, wq, x)["y"].reshape(n_tokens, n_head, hd), pos, hd, 2)
+    k_ = orc.rope(orc.mul_mat(O.Q4_K, wk, x)["y"].reshape(n_tokens, n_head_kv, hd), pos, hd, 2)
+    v_ = orc.mul_mat(O.Q6_K, wv, x)["y"]
+    kc_ = kc0.copy()
+    kc_[head:head + n_tokens] = k_.reshape(n_tokens, n_embd_kv).astype(np.float16)
+    vc_ = vc0.copy()
+    vc_[:, head:head + n_tokens] = v_.T.astype(np.float16)
+    # the stored rows went through the device's matmul and RoPE (tolerances of their own): within two fp16 steps
+    step = lambda a: 2 * np.spacing(np.abs(a).astype(np.float16)).astype(np.float32) + 1e-3
+    assert (np.abs(y_kc.astype(np.float32) - kc_.astype(np.float32)) <= step(kc_)).all()
+    assert (np.abs(y_vc.astype(np.float32) - vc_.astype(np.float32)) <= step(vc_)).all()
+    assert y_kc[:head].tobytes() == kc0[:head].tobytes() and (y_kc[head + n_tokens:] == 0).all()
+    kq_ = orc.mul_mat_f16_batched(kc_[:n_kv].reshape(n_kv, n_head_kv, hd).transpose(1, 0, 2), q_.transpose(1, 0, 2))["y"]
+    sm_ = orc.soft_max(kq_, mask16, scale)
+    kqv_ = orc.mul_mat_f16_batched(vc_.reshape(n_head_kv, hd, kv_size)[:, :, :n_kv], sm_)["y"]
+    merged_ = np.ascontiguousarray(kqv_.transpose(1, 0, 2)).reshape(n_tokens, n_head * hd)
+    o = orc.mul_mat(O.Q4_K, wo, merged_, want=("sum_abs",))
+    want = o["y"] + x
+    assert (np.abs(y - want) <= 5e-3 * o["sum_abs"] + 1e-5).all()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(cbuf)
+    L.lm_ggml_backend_buffer_free(wbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(cctx)
+    L.lm_ggml_free(wctx)

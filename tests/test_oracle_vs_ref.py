@@ -199,3 +199,18 @@ def test_cpy_graphs(orc, ref, ne1, ne0):
         h = x.astype(np.float16)
         assert orc.cpy(h.T, np.float16).tobytes() == ref.cpy_graph(h, np.float16, "cont").tobytes()
         assert orc.cpy(h, np.float32).reshape(-1).tobytes() == ref.cpy_graph(h, np.float32, "flat").tobytes()
+
+
+@pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,threads", [(128, 8, 2, 3, 96, 2), (64, 4, 4, 1, 40, 1), (96, 6, 2, 5, 33, 3)])
+def test_attention_matmuls_over_an_f16_cache(orc, ref, hd, n_head, n_head_kv, n_tokens, n_kv, threads):
+    """The batched, broadcast F16 MUL_MAT of the oracle against the reference's graph over permuted cache views."""
+    rng = np.random.default_rng(hd + n_kv)
+    k_cache = rng.standard_normal((n_kv, n_head_kv, hd)).astype(np.float16)
+    vt_cache = rng.standard_normal((hd, n_head_kv, n_kv)).astype(np.float16)
+    q = rng.standard_normal((n_tokens, n_head, hd)).astype(np.float32)
+    p = rng.random((n_head, n_tokens, n_kv)).astype(np.float32)
+    kq_ref, kqv_ref = ref.attention_matmul_graphs(k_cache, vt_cache, q, p, nthreads=threads)
+    kq = orc.mul_mat_f16_batched(k_cache.transpose(1, 0, 2), q.transpose(1, 0, 2))["y"]
+    kqv = orc.mul_mat_f16_batched(vt_cache.transpose(1, 0, 2), p)["y"]
+    assert kq.tobytes() == kq_ref.tobytes()
+    assert kqv.tobytes() == kqv_ref.tobytes()
