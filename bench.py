@@ -324,7 +324,27 @@ def bench_extra(dev, hip, trace=True):
             us = time_runs(dev, hip, st, lambda: L.chip_cpy(k.ptr, ca.F32, shape, A(n_embd_kv * 4, 4, 0, 0), cache.ptr, ca.F16, shape,
                                                              A(2, kv_size * 2, 0, 0), st), 50)
             out["v_store_transposed_%dx%d" % (n_tok, n_embd_kv)] = {"us": round(us, 2), "GBps": round(one * 6 / us / 1e3, 1)}
-            for bf in (kq, mask, q, pos, k, cache):
+            # kq = mul_mat(K cache, q) and kqv = mul_mat(transposed V cache, probabilities), F16 caches of kv_size positions
+            kcache = dev.to_device((rng.standard_normal((kv_size, n_embd_kv)) * 0.5).astype(np.float16))
+            vcache = dev.to_device((rng.standard_normal((n_embd_kv, kv_size)) * 0.5).astype(np.float16))
+            kq_out = dev.alloc(n_head * n_tok * n_kv * 4)
+            kqv_out = dev.alloc(n_head * n_tok * hd * 4)
+            aws_bytes = max(L.chip_mul_mat_f16_batched_workspace_size(hd, n_kv, n_head_kv, n_head, n_tok),
+                            L.chip_mul_mat_f16_batched_workspace_size(n_kv, hd, n_head_kv, n_head, n_tok), 256)
+            aws = dev.alloc(aws_bytes)
+            us = time_runs(dev, hip, st, lambda: L.chip_mul_mat_f16_batched(kcache.ptr, 2 * n_embd_kv, 2 * hd, hd, n_kv, n_head_kv, q.ptr,
+                                                                             hd * n_head, hd, n_tok, n_head, kq_out.ptr, n_kv, n_kv * n_tok,
+                                                                             aws.ptr, aws_bytes, st), 30)
+            cache_bytes = n_kv * n_embd_kv * 2
+            flops = 2.0 * n_head * n_tok * n_kv * hd
+            out["attn_kq_%dtok_%dkv" % (n_tok, n_kv)] = {"us": round(us, 2), "cache_GBps": round(cache_bytes / us / 1e3, 1),
+                                                          "TFLOPs": round(flops / us / 1e6, 2)}
+            us = time_runs(dev, hip, st, lambda: L.chip_mul_mat_f16_batched(vcache.ptr, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv,
+                                                                             kq.ptr, n_kv, n_kv * n_tok, n_tok, n_head, kqv_out.ptr, hd,
+                                                                             hd * n_tok, aws.ptr, aws_bytes, st), 30)
+            out["attn_kqv_%dtok_%dkv" % (n_tok, n_kv)] = {"us": round(us, 2), "cache_GBps": round(cache_bytes / us / 1e3, 1),
+                                                           "TFLOPs": round(flops / us / 1e6, 2)}
+            for bf in (kq, mask, q, pos, k, cache, kcache, vcache, kq_out, kqv_out, aws):
                 bf.free()
 
     attn_side_cases()

@@ -37,7 +37,7 @@ EXPORTS = (
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu",
-    "chip_soft_max", "chip_cpy", "chip_rope", "chip_mul_mat_f16_batched",
+    "chip_soft_max", "chip_cpy", "chip_rope", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -108,7 +108,9 @@ def load_library(path=KERNEL_LIB):
     L.chip_soft_max.argtypes = [vp, i64, vp, i32, i64, i64, i64, C.c_float, C.c_float, vp, i64, vp]
     L.chip_cpy.argtypes = [vp, i32, C.POINTER(i64), C.POINTER(i64), vp, i32, C.POINTER(i64), C.POINTER(i64), vp]
     L.chip_rope.argtypes = [vp, i64, i64, vp, vp, i64, i64, i64, i32, i32, i32] + [C.c_float] * 6 + [vp, i64, i64, vp]
-    L.chip_mul_mat_f16_batched.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp]
+    L.chip_mul_mat_f16_batched.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp, sz, vp]
+    L.chip_mul_mat_f16_batched_workspace_size.restype = sz
+    L.chip_mul_mat_f16_batched_workspace_size.argtypes = [i64, i64, i64, i64, i64]
     L.chip_mul_mat_id_workspace_size.restype = sz
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
     L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
@@ -310,9 +312,10 @@ class Device:
         self.sync()
         return dy.download(np.float32, x.size).reshape(x.shape)
 
-    def mul_mat_f16_batched(self, W, x):
+    def mul_mat_f16_batched(self, W, x, workspace=True):
         """W fp16 array or view [ne02, N, K] (K contiguous), x fp32 array or view [ne12, n, K] (K contiguous) ->
-        y fp32 [ne12, n, N]; the views are uploaded with their own strides."""
+        y fp32 [ne12, n, N]; the views are uploaded with their own strides.  workspace=False withholds the workspace
+        (dot-product kernels only)."""
         def upload(v):
             base = v
             while isinstance(base.base, np.ndarray):
@@ -325,8 +328,11 @@ class Device:
         dw, woff = upload(W)
         dx, xoff = upload(x)
         dy = self.alloc(ne12 * n * N * 4)
+        wsz = self.lib.chip_mul_mat_f16_batched_workspace_size(K, N, ne02, ne12, n) if workspace else 0
+        ws = self.alloc(wsz) if wsz else None
         self.check(self.lib.chip_mul_mat_f16_batched(dw.ptr + woff, W.strides[1], W.strides[0], K, N, ne02, dx.ptr + xoff,
-                                                     x.strides[1] // 4, x.strides[0] // 4, n, ne12, dy.ptr, N, n * N, None))
+                                                     x.strides[1] // 4, x.strides[0] // 4, n, ne12, dy.ptr, N, n * N,
+                                                     ws.ptr if ws else None, wsz, None))
         self.sync()
         return dy.download(np.float32, ne12 * n * N).reshape(ne12, n, N)
 

@@ -7,36 +7,51 @@
 //   y[b][t][r] = sum_k  W[b / r2][r][k] * fp16(x[b][t][k])        b < ne12 = ne02 * r2, t < n, r < N
 //
 // kq:  W = the K cache seen as [head_dim, n_kv, n_head_kv]: rows of head_dim halves, row stride one cache position.
-//      K = head_dim is small: LPR = K / 8 lanes (8, 16 or 32) share a row, a wave reads 64 / LPR rows per load.
-// kqv: W = the transposed V cache seen as [n_kv, head_dim, n_head_kv]: rows of n_kv halves.  K is long: a wave per row.
+// kqv: W = the transposed V cache seen as [n_kv, head_dim, n_head_kv]: rows of n_kv halves.
 //
 // A workgroup handles one src0 batch (KV head) and with it the r2 src1 batches (query heads) that share it, so a row of
-// the cache is read once for all of them.  The (query head, token) pairs of the KV head are "columns"; a pass keeps COLS
-// fp32 accumulators per lane and walks the row once.  Activations are rounded to fp16 on the fly (v_cvt_f16_f32, round
-// to nearest even) and fed to v_fma_mix_f32 as halves.  Both kernels are bound by the cache bytes (HBM) for few tokens
-// and by the vector pipe for many; the summation order differs from the reference's 4 x 8-lane accumulators, so parity
-// is a tolerance (1e-5 of sum |terms|), as for the other fp32-accumulating kernels.
+// the cache is read once for all of them.  The (query head, token) pairs of the KV head are its "columns".
+//
+// Few columns (decode) - bound: the cache bytes (HBM), in practice launch and memory latency:
+//   short rows (K <= 256, kq): LPR = 8, 16 or 32 lanes share a row and a wave reads 64 / LPR rows per load; the lane's
+//     slice of every column is rounded to fp16 once and stays in registers while the wave walks the rows.
+//   long rows (kqv): a workgroup takes four rows, its four waves a quarter of K each; the activations are read once for
+//     the four rows; partial sums meet in LDS.
+// Many columns (prefill): the columns of a KV head are the token rows of a GEMM against that head's cache rows, so
+//   the work goes to the fp16 MFMA GEMM in its row-gather mode (the mode MUL_MAT_ID uses): activations rounded to fp16
+//   into a workspace, one (KV head, 64-column tile) list entry per workgroup column.
+// Activations are rounded with v_cvt_f16_f32 (nearest even) and multiplied as halves by v_fma_mix_f32 with an fp32
+// accumulator.  The summation order differs from the reference's 4 x 8-lane accumulators, so parity is a tolerance
+// (1e-5 of sum |terms|), as for the other fp32-accumulating kernels.
 #include "dev_common.h"
 #include "kernels.h"
+#include "act_layout.h"
 
 namespace chip {
 
 namespace {
 
 constexpr int AM_THREADS = 256;
-constexpr int AM_COLS = 8;
+constexpr int AM_WAVES = AM_THREADS / 64;
+constexpr int AM_COLS = 4;                   // columns per pass: r2 = 4 with one token is one pass
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ float dot8(const u32x4 w, const float4 a, const float4 b, float acc) {
-    const float xs[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+__device__ __forceinline__ u32x4 round8(const float4 a, const float4 b) {
+    const half2_t h0 = {(_Float16)a.x, (_Float16)a.y}, h1 = {(_Float16)a.z, (_Float16)a.w};       // round to nearest even
+    const half2_t h2 = {(_Float16)b.x, (_Float16)b.y}, h3 = {(_Float16)b.z, (_Float16)b.w};
+    u32x4 r;
+    r.x = __builtin_bit_cast(uint32_t, h0); r.y = __builtin_bit_cast(uint32_t, h1);
+    r.z = __builtin_bit_cast(uint32_t, h2); r.w = __builtin_bit_cast(uint32_t, h3);
+    return r;
+}
+__device__ __forceinline__ float dot8(const u32x4 w, const u32x4 x, float acc) {
+    const uint32_t ws[4] = {w.x, w.y, w.z, w.w}, xs[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const half2_t wv = __builtin_bit_cast(half2_t, ws[i]);
-        const _Float16 x0 = (_Float16)xs[2 * i], x1 = (_Float16)xs[2 * i + 1];          // round to nearest even
-        acc = __builtin_fmaf((float)wv.x, (float)x0, acc);
-        acc = __builtin_fmaf((float)wv.y, (float)x1, acc);
+        const half2_t wv = __builtin_bit_cast(half2_t, ws[i]), xv = __builtin_bit_cast(half2_t, xs[i]);
+        acc = __builtin_fmaf((float)wv.x, (float)xv.x, acc);
+        acc = __builtin_fmaf((float)wv.y, (float)xv.y, acc);
     }
     return acc;
 }
@@ -48,75 +63,212 @@ struct BatchedArgs {
     int64_t n, r2;
     float *y; int64_t ldy1, ldy2;            // token and batch strides of dst, in floats
 };
+// Column c of KV head b0: query head c % r2 of its group, token c / r2.
+__device__ __forceinline__ const float *col_x(const BatchedArgs &a, int64_t b0, int64_t c) {
+    return a.x + (b0 * a.r2 + c % a.r2) * a.ldx2 + (c / a.r2) * a.ldx1;
+}
+__device__ __forceinline__ float *col_y(const BatchedArgs &a, int64_t b0, int64_t c) {
+    return a.y + (b0 * a.r2 + c % a.r2) * a.ldy2 + (c / a.r2) * a.ldy1;
+}
 
-// LPR lanes per row.  Column c of a KV head: query head c % r2 of the group, token c / r2.
+// ---- short rows: K <= 8 * LPR, one 16-byte chunk per lane ----
 template <int LPR>
-__global__ __launch_bounds__(AM_THREADS) void mul_mat_f16_batched_kernel(BatchedArgs a) {
+__global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedArgs a) {
     constexpr int RPS = 64 / LPR;                                    // rows per wave step
+    constexpr int UNROLL = 4;                                        // row steps in flight
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPR, grp = lane / LPR;
     const int64_t b0 = blockIdx.y;
     const uint8_t *Wb = a.W + b0 * a.nb02;
-    const int64_t chunks = a.K / 8;
+    const bool has_chunk = sub < a.K / 8;
     const int64_t cols = a.r2 * a.n;
-    const int64_t row_step = (int64_t)gridDim.x * (AM_THREADS / 64) * RPS;
-    for (int64_t row = ((int64_t)blockIdx.x * (AM_THREADS / 64) + wave) * RPS + grp; row < a.N; row += row_step) {
-        const u32x4 *wrow = reinterpret_cast<const u32x4 *>(Wb + row * a.nb01);
-        for (int64_t c0 = 0; c0 < cols; c0 += AM_COLS) {
-            float acc[AM_COLS];
-            const float *xc[AM_COLS];
+    const int64_t row_step = (int64_t)gridDim.x * AM_WAVES * RPS;
+    const int64_t row0 = ((int64_t)blockIdx.x * AM_WAVES + wave) * RPS + grp;
+    for (int64_t c0 = 0; c0 < cols; c0 += AM_COLS) {
+        u32x4 xh[AM_COLS];
 #pragma unroll
-            for (int j = 0; j < AM_COLS; j++) {
-                acc[j] = 0.0f;
-                const int64_t c = c0 + j < cols ? c0 + j : cols - 1;               // clamped: loads stay in bounds, result unused
-                xc[j] = a.x + (b0 * a.r2 + c % a.r2) * a.ldx2 + (c / a.r2) * a.ldx1;
+        for (int j = 0; j < AM_COLS; j++) {
+            const int64_t c = c0 + j < cols ? c0 + j : cols - 1;                  // clamped: the load stays in bounds, the result is unused
+            xh[j] = u32x4{0u, 0u, 0u, 0u};
+            if (has_chunk) {
+                const float4 *xp = reinterpret_cast<const float4 *>(col_x(a, b0, c) + 8 * sub);
+                xh[j] = round8(xp[0], xp[1]);
             }
-            for (int64_t ch = sub; ch < chunks; ch += LPR) {
-                const u32x4 w = wrow[ch];
+        }
+        for (int64_t rbase = row0; rbase < a.N; rbase += UNROLL * row_step) {
+            u32x4 w[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const int64_t row = rbase + u * row_step;
+                w[u] = u32x4{0u, 0u, 0u, 0u};
+                if (row < a.N && has_chunk) w[u] = *reinterpret_cast<const u32x4 *>(Wb + row * a.nb01 + 16 * sub);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const int64_t row = rbase + u * row_step;
+                float acc[AM_COLS];
 #pragma unroll
                 for (int j = 0; j < AM_COLS; j++) {
-                    const float4 *xp = reinterpret_cast<const float4 *>(xc[j] + 8 * ch);
-                    acc[j] = dot8(w, xp[0], xp[1], acc[j]);
+                    acc[j] = dot8(w[u], xh[j], 0.0f);
+#pragma unroll
+                    for (int o = LPR / 2; o > 0; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
                 }
-            }
+                if (sub == 0 && row < a.N) {
 #pragma unroll
-            for (int j = 0; j < AM_COLS; j++) {
-#pragma unroll
-                for (int o = LPR / 2; o > 0; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
-            }
-            if (sub == 0) {
-#pragma unroll
-                for (int j = 0; j < AM_COLS; j++) {
-                    const int64_t c = c0 + j;
-                    if (c < cols) a.y[(b0 * a.r2 + c % a.r2) * a.ldy2 + (c / a.r2) * a.ldy1 + row] = acc[j];
+                    for (int j = 0; j < AM_COLS; j++)
+                        if (c0 + j < cols) col_y(a, b0, c0 + j)[row] = acc[j];
                 }
             }
         }
     }
 }
 
+// ---- long rows: a workgroup takes AM_ROWS rows, wave w the chunks w * 64 + lane, + 256, ... of each ----
+constexpr int AM_ROWS = 4;
+__global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArgs a) {
+    __shared__ float part[AM_WAVES][AM_ROWS][AM_COLS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t b0 = blockIdx.y;
+    const uint8_t *Wb = a.W + b0 * a.nb02;
+    const int64_t chunks = a.K / 8;
+    const int64_t cols = a.r2 * a.n;
+    for (int64_t r0 = (int64_t)blockIdx.x * AM_ROWS; r0 < a.N; r0 += (int64_t)gridDim.x * AM_ROWS) {
+        const uint8_t *wrow[AM_ROWS];
+#pragma unroll
+        for (int r = 0; r < AM_ROWS; r++) wrow[r] = Wb + (r0 + r < a.N ? r0 + r : a.N - 1) * a.nb01;      // clamped, unused past N
+        for (int64_t c0 = 0; c0 < cols; c0 += AM_COLS) {
+            const float *xc[AM_COLS];
+#pragma unroll
+            for (int j = 0; j < AM_COLS; j++) xc[j] = col_x(a, b0, c0 + j < cols ? c0 + j : cols - 1);
+            float acc[AM_ROWS][AM_COLS];
+#pragma unroll
+            for (int r = 0; r < AM_ROWS; r++)
+#pragma unroll
+                for (int j = 0; j < AM_COLS; j++) acc[r][j] = 0.0f;
+            for (int64_t ch = wave * 64 + lane; ch < chunks; ch += AM_THREADS) {
+                u32x4 w[AM_ROWS], xh[AM_COLS];
+#pragma unroll
+                for (int r = 0; r < AM_ROWS; r++) w[r] = *reinterpret_cast<const u32x4 *>(wrow[r] + 16 * ch);
+#pragma unroll
+                for (int j = 0; j < AM_COLS; j++) {
+                    const float4 *xp = reinterpret_cast<const float4 *>(xc[j] + 8 * ch);
+                    xh[j] = round8(xp[0], xp[1]);
+                }
+#pragma unroll
+                for (int r = 0; r < AM_ROWS; r++)
+#pragma unroll
+                    for (int j = 0; j < AM_COLS; j++) acc[r][j] = dot8(w[r], xh[j], acc[r][j]);
+            }
+#pragma unroll
+            for (int r = 0; r < AM_ROWS; r++)
+#pragma unroll
+                for (int j = 0; j < AM_COLS; j++) {
+                    float v = acc[r][j];
+#pragma unroll
+                    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+                    if (lane == 0) part[wave][r][j] = v;
+                }
+            __syncthreads();
+            if (threadIdx.x < AM_ROWS * AM_COLS) {
+                const int r = threadIdx.x / AM_COLS, j = threadIdx.x % AM_COLS;
+                if (r0 + r < a.N && c0 + j < cols)
+                    col_y(a, b0, c0 + j)[r0 + r] = (part[0][r][j] + part[1][r][j]) + (part[2][r][j] + part[3][r][j]);
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// ---- many columns: fp16 rows for the GEMM and its (KV head, tile) list ----
+// Row R = b * n + t of the workspace and of y is column (query head b, token t); the pairs of KV head e are the rows
+// e * r2 * n ... (e + 1) * r2 * n - 1, in order.
+__global__ __launch_bounds__(AM_THREADS) void mm_f16_round_rows_kernel(const float *__restrict__ x, int64_t ldx1, int64_t ldx2,
+                                                                       int64_t n, int64_t K, uint8_t *__restrict__ ws, size_t ws_stride) {
+    const int64_t t = blockIdx.x, b = blockIdx.y;
+    const float *xr = x + b * ldx2 + t * ldx1;
+    u32x4 *out = reinterpret_cast<u32x4 *>(ws + (size_t)(b * n + t) * ws_stride);
+    for (int64_t ch = threadIdx.x; ch < K / 8; ch += AM_THREADS) {
+        const float4 *xp = reinterpret_cast<const float4 *>(xr + 8 * ch);
+        out[ch] = round8(xp[0], xp[1]);
+    }
+}
+__global__ __launch_bounds__(AM_THREADS) void mm_f16_tile_list_kernel(int64_t ne02, int64_t per_head, int tile_tokens,
+                                                                      int32_t *__restrict__ perm, int32_t *__restrict__ offsets,
+                                                                      int32_t *__restrict__ tiles) {
+    const int64_t i0 = (int64_t)blockIdx.x * AM_THREADS + threadIdx.x, step = (int64_t)gridDim.x * AM_THREADS;
+    const int64_t tiles_per_head = ceil_div(per_head, (int64_t)tile_tokens);
+    for (int64_t i = i0; i < ne02 * per_head; i += step) perm[i] = (int32_t)i;
+    for (int64_t i = i0; i <= ne02; i += step) offsets[i] = (int32_t)(i * per_head);
+    for (int64_t i = i0; i < ne02 * tiles_per_head; i += step)
+        tiles[1 + i] = (int32_t)(i / tiles_per_head) | (int32_t)((i % tiles_per_head) << MOE_EXPERT_BITS);
+    if (i0 == 0) tiles[0] = (int32_t)(ne02 * tiles_per_head);
+}
+
+constexpr int64_t GEMM_MIN_COLS = 64;        // columns per KV head from which the GEMM route is taken
+
+struct GemmPlan { bool use; size_t act_stride, off_perm, off_offsets, off_tiles, bytes; int64_t n_tiles; };
+GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
+    GemmPlan p{};
+    const int64_t per_head = r2 * n;
+    p.use = K % 64 == 0 && N >= 32 && per_head >= GEMM_MIN_COLS && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
+    if (!p.use) return p;
+    p.act_stride = f16_stride(K);
+    p.n_tiles = ne02 * ceil_div(per_head, (int64_t)gemm_f16_moe_tile_tokens());
+    if (p.n_tiles > 65535) { p.use = false; return p; }                  // one grid row per list entry
+    p.off_perm = align128((size_t)(ne02 * per_head) * p.act_stride);
+    p.off_offsets = p.off_perm + align128((size_t)(ne02 * per_head) * 4);
+    p.off_tiles = p.off_offsets + align128((size_t)(ne02 + 1) * 4);
+    p.bytes = p.off_tiles + align128((size_t)(1 + p.n_tiles) * 4);
+    return p;
+}
+
 }  // namespace
 
 bool mul_mat_f16_batched_supported(int64_t K) { return K > 0 && K % 8 == 0; }
 
+size_t mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
+    if (K <= 0 || N <= 0 || ne02 <= 0 || r2 <= 0 || n <= 0) return 0;
+    return gemm_plan(K, N, ne02, r2, n).bytes;
+}
+
 hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
                                       int64_t ldx1, int64_t ldx2, int64_t n, int64_t r2, float *y, int64_t ldy1, int64_t ldy2,
-                                      const DeviceLimits &lim, hipStream_t st) {
+                                      void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st) {
     if (N <= 0 || n <= 0 || ne02 <= 0 || r2 <= 0) return hipSuccess;
     if (!mul_mat_f16_batched_supported(K) || ne02 > 65535) return hipErrorInvalidValue;
+    const GemmPlan plan = gemm_plan(K, N, ne02, r2, n);
+    // the GEMM writes row R of y at R * ldy1: the batches of y must follow each other without a gap
+    if (plan.use && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {
+        uint8_t *ws = (uint8_t *)workspace;
+        int32_t *perm = (int32_t *)(ws + plan.off_perm), *offsets = (int32_t *)(ws + plan.off_offsets), *tiles = (int32_t *)(ws + plan.off_tiles);
+        hipLaunchKernelGGL(mm_f16_round_rows_kernel, dim3((unsigned)n, (unsigned)(ne02 * r2)), dim3(AM_THREADS), 0, st, x, ldx1, ldx2, n, K,
+                           ws, plan.act_stride);
+        hipLaunchKernelGGL(mm_f16_tile_list_kernel, dim3(64), dim3(AM_THREADS), 0, st, ne02, r2 * n, gemm_f16_moe_tile_tokens(), perm,
+                           offsets, tiles);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        const RowGather rg{perm, offsets, tiles, 1, 1, nb02};
+        return launch_gemm_f16(W, nb01, K, N, ws, plan.act_stride, ne02 * r2 * n, y, ldy1, lim, st, &rg, plan.n_tiles);
+    }
     const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    const int lpr = K <= 64 ? 8 : K <= 128 ? 16 : K <= 256 ? 32 : 64;
-    const int64_t rows_per_wg = (AM_THREADS / 64) * (64 / lpr);
-    int64_t gx = ceil_div(N, rows_per_wg);
-    const int64_t cap = ceil_div((int64_t)cus * 8, ne02);               // about eight workgroups per CU over all KV heads
-    if (gx > cap) gx = cap;
-    const dim3 grid((unsigned)gx, (unsigned)ne02);
-    switch (lpr) {
-        case 8:  hipLaunchKernelGGL(mul_mat_f16_batched_kernel<8>, grid, dim3(AM_THREADS), 0, st, a); break;
-        case 16: hipLaunchKernelGGL(mul_mat_f16_batched_kernel<16>, grid, dim3(AM_THREADS), 0, st, a); break;
-        case 32: hipLaunchKernelGGL(mul_mat_f16_batched_kernel<32>, grid, dim3(AM_THREADS), 0, st, a); break;
-        default: hipLaunchKernelGGL(mul_mat_f16_batched_kernel<64>, grid, dim3(AM_THREADS), 0, st, a); break;
+    if (K <= 256) {
+        const int lpr = K <= 64 ? 8 : K <= 128 ? 16 : 32;
+        // a wave walks at least four row steps (its loads in flight together); about four workgroups per CU over all KV heads
+        const int64_t rows_per_wg = AM_WAVES * (64 / lpr) * 4;
+        int64_t gx = ceil_div(N, rows_per_wg);
+        const int64_t cap = ceil_div((int64_t)cus * 4, ne02);
+        if (gx > cap) gx = cap;
+        const dim3 grid((unsigned)gx, (unsigned)ne02);
+        switch (lpr) {
+            case 8:  hipLaunchKernelGGL(mm_f16_short_rows_kernel<8>, grid, dim3(AM_THREADS), 0, st, a); break;
+            case 16: hipLaunchKernelGGL(mm_f16_short_rows_kernel<16>, grid, dim3(AM_THREADS), 0, st, a); break;
+            default: hipLaunchKernelGGL(mm_f16_short_rows_kernel<32>, grid, dim3(AM_THREADS), 0, st, a); break;
+        }
+    } else {
+        int64_t gx = ceil_div(N, (int64_t)AM_ROWS);
+        const int64_t cap = ceil_div((int64_t)cus * 8, ne02);
+        if (gx > cap) gx = cap;
+        hipLaunchKernelGGL(mm_f16_long_rows_kernel, dim3((unsigned)gx, (unsigned)ne02), dim3(AM_THREADS), 0, st, a);
     }
     return hipGetLastError();
 }

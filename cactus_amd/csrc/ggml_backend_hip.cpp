@@ -438,9 +438,13 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         }
         if (node->op == LM_GGML_OP_MUL_MAT && !mul_mat_shape_ok(node) && mul_mat_f16_batched_shape_ok(node)) {
             const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
+            if (w->ne[1] == 0 || x->ne[1] == 0 || x->ne[2] == 0) continue;
+            if (!grow_workspace(c, chip_mul_mat_f16_batched_workspace_size(w->ne[0], w->ne[1], w->ne[2], x->ne[2], x->ne[1])))
+                return LM_GGML_STATUS_ALLOC_FAILED;
             const int rc = chip_mul_mat_f16_batched(w->data, w->nb[1], w->nb[2], w->ne[0], w->ne[1], w->ne[2], (const float *)x->data,
                                                     (int64_t)(x->nb[1] / 4), (int64_t)(x->nb[2] / 4), x->ne[1], x->ne[2],
-                                                    (float *)node->data, (int64_t)(node->nb[1] / 4), (int64_t)(node->nb[2] / 4), c->stream);
+                                                    (float *)node->data, (int64_t)(node->nb[1] / 4), (int64_t)(node->nb[2] / 4),
+                                                    c->workspace, c->workspace_size, c->stream);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: batched F16 MUL_MAT %s failed: %s\n", __func__, node->name, chip_error_string(rc));
                 return LM_GGML_STATUS_FAILED;

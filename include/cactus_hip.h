@@ -187,10 +187,13 @@ CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, floa
  * W: F16, rows of K halves at nb01 bytes, batches (KV heads) at nb02 bytes; x: F32 rows of K at ldx1 floats (tokens) and
  * ldx2 floats (batches: query heads); y likewise, rows of N.  ne12 must be a multiple of ne02 (grouped-query broadcast,
  * the reference's r2); a fourth dimension is not taken.  K a multiple of 8; W, nb01, nb02, x 16-byte aligned, ldx1 and
- * ldx2 multiples of 4.  No workspace: the activations are rounded on the fly. */
+ * ldx2 multiples of 4.  The workspace is optional (NULL, 0): with chip_mul_mat_f16_batched_workspace_size bytes of it,
+ * 64 or more (query head, token) pairs per KV head go through the fp16 MFMA GEMM (K a multiple of 64, y's batches
+ * adjacent: ldy2 == n * ldy1); without it, and for fewer pairs, dot-product kernels round the activations on the fly. */
+CHIP_API size_t chip_mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne02, int64_t ne12, int64_t n);
 CHIP_API int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02,
                                       const float *x, int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y,
-                                      int64_t ldy1, int64_t ldy2, void *stream);
+                                      int64_t ldy1, int64_t ldy2, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- the attention-side ops around the KV cache ----
  *   chip_soft_max : LM_GGML_OP_SOFT_MAX (lm_ggml_soft_max_ext), lm_ggml_compute_forward_soft_max_f32 (ggml-cpu/ops.cpp:4731-4827):

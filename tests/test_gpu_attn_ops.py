@@ -241,8 +241,10 @@ def attn_case(seed, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
 
 # (hd, n_head, n_head_kv, n_tokens, n_kv, kv_size): LLaMA-3-8B decode and a short prefill, multi-head attention, head sizes
 # that use 8 / 16 / 32 lanes per cache row, a GQA ratio that is no power of two, positions that are no multiple of 64
+# the last three have 64 or more (head, token) pairs per KV head: with a workspace they take the GEMM route
 ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8, 3, 96, 128), (256, 4, 2, 2, 160, 160),
-               (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128)]
+               (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128), (128, 32, 8, 130, 320, 512),
+               (64, 4, 4, 100, 192, 256)]
 
 
 @pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", ATTN_SHAPES)
@@ -261,6 +263,12 @@ def test_attention_matmuls_over_the_cache(dev, orc, hd, n_head, n_head_kv, n_tok
     got = dev.mul_mat_f16_batched(vv, p)
     assert got.shape == (n_head, n_tokens, hd)
     assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
+    if n_tokens * (n_head // n_head_kv) >= 64:                                  # the same without a workspace: dot-product kernels
+        got = dev.mul_mat_f16_batched(vv, p, workspace=False)
+        assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
+        want = orc.mul_mat_f16_batched(kv, qv, want=("sum_abs",))
+        got = dev.mul_mat_f16_batched(kv, qv, workspace=False)
+        assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
 
 
 def test_attention_matmul_exact_small_integers(dev):
@@ -290,7 +298,7 @@ def test_attention_matmul_rejects_bad_arguments(dev):
     import cactus_amd as ca
     d = dev.alloc(1 << 16)
     L = dev.lib
-    ok = (d.ptr, 256, 256 * 16, 128, 16, 2, d.ptr, 128, 512, 1, 4, d.ptr, 16, 16, None)
+    ok = (d.ptr, 256, 256 * 16, 128, 16, 2, d.ptr, 128, 512, 1, 4, d.ptr, 16, 16, None, 0, None)
     assert L.chip_mul_mat_f16_batched(*ok) == ca.CHIP_OK
     dev.sync()
 
