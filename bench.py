@@ -448,6 +448,78 @@ def bench_trace(dev, hip, st, rng):
     for s_ in side:
         dev.check(L.chip_stream_create(C.byref(s_)))
 
+    def full_layers(n, n_kv, ws, wsz):
+        """Every node of the 32 layers as llama.cpp builds them without flash attention (norms, projections, RoPE, cache
+        stores, kq, soft-max, kqv, head merge, residuals, SiLU * up), n new tokens against n_kv cached positions, as one
+        HIP graph on one stream: what a decode step costs when no activation leaves the device."""
+        hd, n_head, n_head_kv, kv_size = 128, 32, 8, 4096
+        A4 = C.c_int64 * 4
+        f32 = lambda *shape: dev.alloc(int(np.prod(shape)) * 4)
+        resid = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
+        wn = dev.to_device((1 + 0.1 * rng.standard_normal(H)).astype(np.float32))
+        pos = dev.to_device(np.arange(n_kv - n, n_kv, dtype=np.int32))
+        mask = dev.to_device(np.zeros((max(n, 8), n_kv), np.float16))
+        cur, q, k, v, merged, att = f32(n, H), f32(n, H), f32(n, KV), f32(n, KV), f32(n, H), f32(n, H)
+        kq, kqv = f32(n_head, n, n_kv), f32(n_head, n, hd)
+        up, gate = f32(n, FF), f32(n, FF)
+        caches = dev.alloc(NL * 2 * kv_size * KV * 2)
+        dev.check(L.chip_memset(caches.ptr, 0, caches.nbytes, None))
+        aws_bytes = max(L.chip_mul_mat_f16_batched_workspace_size(hd, n_kv, n_head_kv, n_head, n),
+                        L.chip_mul_mat_f16_batched_workspace_size(n_kv, hd, n_head_kv, n_head, n), 256)
+        aws = dev.alloc(aws_bytes)
+        ck = dev.check
+
+        def mm(t, wptr, N, K, src, dst):
+            ck(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, dst.ptr, N, ws.ptr, wsz, st))
+
+        def step():
+            for l in range(NL):
+                base = arena.ptr + l * layer_bytes
+                W = {name: (t, base + o, N, K) for (name, t, N, K, _), o in zip(layer, first)}
+                kc = caches.ptr + (2 * l) * kv_size * KV * 2
+                vc = kc + kv_size * KV * 2
+                ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))     # norm + weight: one kernel, as the backend fuses them
+                mm(*W["wq"], cur, q); mm(*W["wk"], cur, k); mm(*W["wv"], cur, v)
+                for t_, nh in ((q, n_head), (k, n_head_kv)):
+                    ck(L.chip_rope(t_.ptr, hd, hd * nh, pos.ptr, None, hd, nh, n, hd, 2, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0,
+                                   t_.ptr, hd, hd * nh, st))
+                flat, one = A4(n * KV, 1, 1, 1), n * KV
+                ck(L.chip_cpy(k.ptr, ca.F32, flat, A4(4, 4 * one, 4 * one, 4 * one), kc + 2 * KV * (n_kv - n), ca.F16, flat,
+                              A4(2, 2 * one, 2 * one, 2 * one), st))
+                shp = A4(n, KV, 1, 1)
+                ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))
+                ck(L.chip_mul_mat_f16_batched(kc, 2 * KV, 2 * hd, hd, n_kv, n_head_kv, q.ptr, hd * n_head, hd, n, n_head, kq.ptr, n_kv,
+                                              n_kv * n, aws.ptr, aws_bytes, st))
+                ck(L.chip_soft_max(kq.ptr, n_kv, mask.ptr, ca.F16, n_kv, n, n_head * n, 0.0884, 0.0, kq.ptr, n_kv, st))
+                ck(L.chip_mul_mat_f16_batched(vc, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv, kq.ptr, n_kv, n_kv * n, n, n_head,
+                                              kqv.ptr, hd, hd * n, aws.ptr, aws_bytes, st))
+                ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
+                              A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
+                mm(*W["wo"], merged, att)
+                ck(L.chip_add(att.ptr, H, resid.ptr, H, n, n, H, resid.ptr, H, st))
+                ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))     # norm + weight: one kernel, as the backend fuses them
+                mm(*W["up"], cur, up); mm(*W["gate"], cur, gate)
+                ck(L.chip_silu(gate.ptr, FF, n, FF, gate.ptr, FF, st))
+                ck(L.chip_mul(gate.ptr, FF, up.ptr, FF, n, n, FF, gate.ptr, FF, st))
+                mm(*W["down"], gate, att)
+                ck(L.chip_add(att.ptr, H, resid.ptr, H, n, n, H, resid.ptr, H, st))
+            ck(L.chip_rms_norm(resid.ptr, H, n, H, 1e-5, cur.ptr, H, st))
+            ck(L.chip_mul_mat(ca.Q6_K, arena.ptr + head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
+
+        step()
+        dev.sync(st)
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hl.hipStreamBeginCapture(st, 0) == 0
+        step()
+        assert hl.hipStreamEndCapture(st, C.byref(graph)) == 0
+        assert hl.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        us = time_runs(dev, hip, st, lambda: hl.hipGraphLaunch(gexec, st), 10, warm=2)
+        for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws):
+            bf.free()
+        cache_bytes = NL * 2 * n_kv * KV * 2
+        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "kernels": 22 * NL + 2, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
+                "weight_and_cache_GBps": round((total + cache_bytes) / us / 1e3, 1)}
+
     res = {}
     for n in (1, 8, 512):                                              # decode, small batch, one prefill chunk
         x_h = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
@@ -524,6 +596,8 @@ def bench_trace(dev, hip, st, rng):
                 ops = 2.0 * n * (NL * sum(N * K for (_, _, N, K, _) in layer) + V * H)
                 entry[mode]["TOPS"] = round(ops / us / 1e6, 1)
                 entry[mode]["int8_frac"] = round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)
+        if n in (1, 512):
+            entry["whole_layers"] = full_layers(n, 4096 if n == 1 else 512, wss[0], wsz)
         res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = entry
         for bf in [x_h, x_ff, y] + wss:
             bf.free()

@@ -56,6 +56,17 @@ __device__ __forceinline__ float dot8(const u32x4 w, const u32x4 x, float acc) {
     return acc;
 }
 
+// Sum over the LPR lanes that share a row (LPR consecutive lanes, LPR in {8, 16, 32, 64}); every lane of the group gets it.
+template <int LPR> __device__ __forceinline__ float group_sum(float v) {
+    v += dpp_get<0xB1>(v);                                   // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E>(v);                                   // quad_perm [2,3,0,1]
+    v += dpp_get<0x141>(v);                                  // row_half_mirror: sums of 8
+    if constexpr (LPR >= 16) v += dpp_get<0x140>(v);         // row_mirror: sums of 16
+    if constexpr (LPR >= 32) v += __shfl_xor(v, 16);
+    if constexpr (LPR >= 64) v += __shfl_xor(v, 32);
+    return v;
+}
+
 struct BatchedArgs {
     const uint8_t *W; size_t nb01, nb02;
     int64_t K, N;
@@ -63,12 +74,14 @@ struct BatchedArgs {
     int64_t n, r2;
     float *y; int64_t ldy1, ldy2;            // token and batch strides of dst, in floats
 };
-// Column c of KV head b0: query head c % r2 of its group, token c / r2.
+// Column c of KV head b0: query head c % r2 of its group, token c / r2 (32-bit division: 64-bit is a long software routine).
 __device__ __forceinline__ const float *col_x(const BatchedArgs &a, int64_t b0, int64_t c) {
-    return a.x + (b0 * a.r2 + c % a.r2) * a.ldx2 + (c / a.r2) * a.ldx1;
+    const uint32_t r2 = (uint32_t)a.r2, t = (uint32_t)c / r2, h = (uint32_t)c - t * r2;
+    return a.x + (b0 * a.r2 + h) * a.ldx2 + (int64_t)t * a.ldx1;
 }
 __device__ __forceinline__ float *col_y(const BatchedArgs &a, int64_t b0, int64_t c) {
-    return a.y + (b0 * a.r2 + c % a.r2) * a.ldy2 + (c / a.r2) * a.ldy1;
+    const uint32_t r2 = (uint32_t)a.r2, t = (uint32_t)c / r2, h = (uint32_t)c - t * r2;
+    return a.y + (b0 * a.r2 + h) * a.ldy2 + (int64_t)t * a.ldy1;
 }
 
 // ---- short rows: K <= 8 * LPR, one 16-byte chunk per lane ----
@@ -109,9 +122,7 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedAr
                 float acc[AM_COLS];
 #pragma unroll
                 for (int j = 0; j < AM_COLS; j++) {
-                    acc[j] = dot8(w[u], xh[j], 0.0f);
-#pragma unroll
-                    for (int o = LPR / 2; o > 0; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
+                    acc[j] = group_sum<LPR>(dot8(w[u], xh[j], 0.0f));
                 }
                 if (sub == 0 && row < a.N) {
 #pragma unroll
@@ -163,9 +174,7 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArg
             for (int r = 0; r < AM_ROWS; r++)
 #pragma unroll
                 for (int j = 0; j < AM_COLS; j++) {
-                    float v = acc[r][j];
-#pragma unroll
-                    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+                    const float v = group_sum<64>(acc[r][j]);
                     if (lane == 0) part[wave][r][j] = v;
                 }
             __syncthreads();
@@ -235,7 +244,7 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
                                       int64_t ldx1, int64_t ldx2, int64_t n, int64_t r2, float *y, int64_t ldy1, int64_t ldy2,
                                       void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st) {
     if (N <= 0 || n <= 0 || ne02 <= 0 || r2 <= 0) return hipSuccess;
-    if (!mul_mat_f16_batched_supported(K) || ne02 > 65535) return hipErrorInvalidValue;
+    if (!mul_mat_f16_batched_supported(K) || ne02 > 65535 || r2 * n > 0x7fffffff) return hipErrorInvalidValue;
     const GemmPlan plan = gemm_plan(K, N, ne02, r2, n);
     // the GEMM writes row R of y at R * ldy1: the batches of y must follow each other without a gap
     if (plan.use && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {

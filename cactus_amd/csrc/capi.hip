@@ -432,6 +432,21 @@ int chip_add(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n
              void *stream) { return binary_checked(false, a, lda, b, ldb, n_b, n, ne0, y, ldy, stream); }
 int chip_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0, float *y, int64_t ldy,
              void *stream) { return binary_checked(true, a, lda, b, ldb, n_b, n, ne0, y, ldy, stream); }
+int chip_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, const float *w, float *y_norm, int64_t ld_norm,
+                      float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0 || !(eps >= 0.0f)) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0) || !w || (((uintptr_t)w) & 3) != 0 || n > 0x7fffffff) return CHIP_EINVAL;
+    if (y_norm && !rows_ok(y_norm, ld_norm, ne0)) return CHIP_EINVAL;
+    return hip_rc(launch_rms_norm_mul(x, ldx, n, ne0, eps, w, y_norm, ld_norm, y, ldy, (hipStream_t)stream));
+}
+int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (ne0 % 8 != 0) return CHIP_EUNSUPPORTED;                            // as chip_silu
+    if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0) || !rows_ok(b, ldb, ne0)) return CHIP_EINVAL;
+    return hip_rc(launch_silu_mul(x, ldx, b, ldb, ne0, n, y, ldy, (hipStream_t)stream));
+}
 int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream) {
     if (n < 0 || ne0 < 0) return CHIP_EINVAL;
     if (n == 0 || ne0 == 0) return CHIP_OK;
@@ -470,7 +485,7 @@ int chip_soft_max(const float *x, int64_t ldx, const void *mask, int mask_type, 
     if (max_bias != 0.0f) return CHIP_EUNSUPPORTED;                          // ALiBi slopes
     if (ne00 % 8 != 0) return CHIP_EUNSUPPORTED;                             // the reference's row tail uses the C library's expf
     if (mask && mask_type != T_F32 && mask_type != T_F16) return CHIP_EUNSUPPORTED;
-    if (!x || !y || ldx < ne00 || ldy < ne00 || n_rows > 0x7fffffff) return CHIP_EINVAL;
+    if (!x || !y || ldx < ne00 || ldy < ne00 || n_rows > 0x7fffffff || ne01 > 0x7fffffff) return CHIP_EINVAL;
     if (((ldx | ldy) & 3) != 0 || ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)mask)) & 15) != 0) return CHIP_EINVAL;
     return hip_rc(launch_soft_max(x, ldx, mask, mask_type == T_F16, ne00, ne01, n_rows, scale, y, ldy, (hipStream_t)stream));
 }

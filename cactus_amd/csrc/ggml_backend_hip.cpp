@@ -22,7 +22,7 @@
 
 namespace {
 
-std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0};
+std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -270,6 +270,10 @@ bool elementwise_enabled() {
     static const bool on = [] { const char *e = std::getenv("CACTUS_HIP_ELEMENTWISE"); return !(e && std::strcmp(e, "0") == 0); }();
     return on;
 }
+bool fusion_enabled() {
+    static const bool on = [] { const char *e = std::getenv("CACTUS_HIP_FUSE"); return !(e && std::strcmp(e, "0") == 0); }();
+    return on;
+}
 bool elementwise_shape_ok(const lm_ggml_tensor *op) {
     if (!elementwise_enabled()) return false;
     const lm_ggml_tensor *a = op->src[0], *b = op->src[1];
@@ -396,11 +400,55 @@ static bool grow_workspace(backend_ctx *c, size_t need) {
     return true;
 }
 
+// RMS_NORM or SILU directly followed by the MUL that consumes it, the MUL written over the first node's output: the
+// allocator reuses a node's memory for its consumer only when nothing else reads it (reference ggml-alloc.c in-place
+// rule: one child, no views), so the first node's own result is not needed and the pair runs as one kernel.
+// Returns CHIP_OK and sets fused, or leaves fused false.
+int try_fused_pair(backend_ctx *c, const lm_ggml_tensor *node, const lm_ggml_tensor *next, bool &fused) {
+    fused = false;
+    if (!next || next->op != LM_GGML_OP_MUL || next->data != node->data || !elementwise_shape_ok(next)) return CHIP_OK;
+    const lm_ggml_tensor *other = next->src[0] == node ? next->src[1] : (next->src[1] == node ? next->src[0] : nullptr);
+    if (!other || other == node || !same_shape(next, node)) return CHIP_OK;
+    const lm_ggml_tensor *a = node->src[0];
+    int64_t rows, lda, ldy, rb, ldb;
+    if (!as_rows(a, rows, lda) || !as_rows(next, rows, ldy) || !as_rows(other, rb, ldb)) return CHIP_OK;
+    if (node->op == LM_GGML_OP_RMS_NORM) {
+        if (rb != 1) return CHIP_OK;                                       // the norm weight: one row
+        float eps;
+        std::memcpy(&eps, node->op_params, sizeof(float));
+        fused = true;
+        return chip_rms_norm_mul((const float *)a->data, lda, rows, a->ne[0], eps, (const float *)other->data, nullptr, 0,
+                                 (float *)next->data, ldy, c->stream);
+    }
+    if (node->op == LM_GGML_OP_UNARY && node->op_params[0] == LM_GGML_UNARY_OP_SILU) {
+        if (!same_shape(other, node)) return CHIP_OK;
+        fused = true;
+        return chip_silu_mul((const float *)a->data, lda, (const float *)other->data, ldb, rows, a->ne[0], (float *)next->data, ldy,
+                             c->stream);
+    }
+    return CHIP_OK;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_UNARY) && elementwise_shape_ok(node) && fusion_enabled()) {
+            bool fused = false;
+            const int rc = try_fused_pair(c, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d, fused with the next node) failed: %s\n", __func__, node->name, node->op,
+                        chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            if (fused) {
+                g_elementwise_nodes += 2;
+                g_fused_pairs++;
+                i++;
+                continue;
+            }
+        }
         if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_ADD || node->op == LM_GGML_OP_MUL || node->op == LM_GGML_OP_UNARY) &&
             elementwise_shape_ok(node)) {
             const int rc = run_elementwise(c, node);
@@ -578,6 +626,7 @@ size_t reg_device_count(lm_ggml_backend_reg_t) { return device_ok() ? 1 : 0; }
 lm_ggml_backend_dev_t reg_get_device(lm_ggml_backend_reg_t, size_t index) { return (index == 0 && device_ok()) ? hip_device() : nullptr; }
 void *reg_get_proc_address(lm_ggml_backend_reg_t, const char *name) {
     if (std::strcmp(name, "lm_ggml_backend_hip_get_stats") == 0) return (void *)lm_ggml_backend_hip_get_stats;
+    if (std::strcmp(name, "lm_ggml_backend_hip_get_fused_pairs") == 0) return (void *)lm_ggml_backend_hip_get_fused_pairs;
     return nullptr;         // no n_threads, no extra buffer types, no split buffer type, no feature list
 }
 const lm_ggml_backend_reg_i k_reg_i = {reg_name, reg_device_count, reg_get_device, reg_get_proc_address};
@@ -637,5 +686,6 @@ void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned l
     if (mul_mat_nodes) *mul_mat_nodes = g_mul_mat_nodes.load();
     if (uploaded_bytes) *uploaded_bytes = g_uploaded.load();
 }
+unsigned long long lm_ggml_backend_hip_get_fused_pairs(void) { return g_fused_pairs.load(); }
 
 }  // extern "C"

@@ -53,8 +53,11 @@ __device__ __forceinline__ float v_expf_lane(float x) {
 __device__ __forceinline__ float silu1(float x) { return x / (1.0f + v_expf_lane(0.0f - x)); }
 
 // ---- RMS_NORM: one workgroup per row ----
+// With w, the row is also multiplied by the weight row w (the MUL node that follows a norm): y = (x * scale) * w, two
+// roundings as in the two separate ops; yn (may be NULL) then receives the norm itself.
 __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *__restrict__ x, int64_t ldx, int64_t ne0, float eps,
-                                                              float *__restrict__ y, int64_t ldy) {
+                                                              float *__restrict__ y, int64_t ldy, const float *__restrict__ w,
+                                                              float *__restrict__ yn, int64_t ldyn) {
     __shared__ double part[EW_THREADS / 64];
     const float *xr = x + (size_t)blockIdx.x * ldx;
     float *yr = y + (size_t)blockIdx.x * ldy;
@@ -78,22 +81,37 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *__res
     for (int w = 0; w < EW_THREADS / 64; w++) total += part[w];
     const float mean = (float)(total / (double)ne0);
     const float scale = 1.0f / sqrtf(mean + eps);
-    if (vec) {
+    float *ynr = yn ? yn + (size_t)blockIdx.x * ldyn : nullptr;
+    const bool vecw = vec && (!w || ((uintptr_t)w & 15) == 0) && (!yn || ((ldyn & 3) == 0 && ((uintptr_t)yn & 15) == 0));
+    if (vecw) {
         for (int64_t i = 4 * tid; i < ne0; i += 4 * EW_THREADS) {
             float4 v = *reinterpret_cast<const float4 *>(xr + i);
             v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+            if (w) {
+                if (ynr) *reinterpret_cast<float4 *>(ynr + i) = v;
+                const float4 g = *reinterpret_cast<const float4 *>(w + i);
+                v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w;
+            }
             *reinterpret_cast<float4 *>(yr + i) = v;
         }
     } else {
-        for (int64_t i = tid; i < ne0; i += EW_THREADS) yr[i] = xr[i] * scale;
+        for (int64_t i = tid; i < ne0; i += EW_THREADS) {
+            float v = xr[i] * scale;
+            if (w) {
+                if (ynr) ynr[i] = v;
+                v *= w[i];
+            }
+            yr[i] = v;
+        }
     }
 }
 
 // ---- element-wise: grid.y walks the rows, grid.x the row in chunks of 4 * EW_THREADS values ----
-enum { EW_ADD = 0, EW_MUL = 1, EW_SILU = 2 };
+enum { EW_ADD = 0, EW_MUL = 1, EW_SILU = 2, EW_SILU_MUL = 3 };      // SILU_MUL: silu(a) * b, the two nodes of a gated FFN in one pass
 template <int OP> __device__ __forceinline__ float ew_apply(float a, float b) {
     if constexpr (OP == EW_ADD) return a + b;
     else if constexpr (OP == EW_MUL) return a * b;
+    else if constexpr (OP == EW_SILU_MUL) return silu1(a) * b;
     else return silu1(a);
 }
 template <int OP, bool VEC>
@@ -151,8 +169,9 @@ __global__ __launch_bounds__(EW_THREADS) void soft_max_kernel(const float *__res
     const float *xr = x + row * ldx;
     float *yr = y + row * ldy;
     const void *mrow = nullptr;
-    if constexpr (MASK == MASK_F32) mrow = reinterpret_cast<const float *>(mask) + (row % ne01) * ne00;
-    if constexpr (MASK == MASK_F16) mrow = reinterpret_cast<const uint16_t *>(mask) + (row % ne01) * ne00;
+    const int64_t mask_row = (uint32_t)blockIdx.x % (uint32_t)ne01;          // 32-bit: the 64-bit remainder is a long software routine
+    if constexpr (MASK == MASK_F32) mrow = reinterpret_cast<const float *>(mask) + mask_row * ne00;
+    if constexpr (MASK == MASK_F16) mrow = reinterpret_cast<const uint16_t *>(mask) + mask_row * ne00;
     const int tid = threadIdx.x;
     const int64_t groups = ne00 / 8;
     constexpr int GR = G > 0 ? G : 1;
@@ -259,17 +278,21 @@ template <typename S, typename D> __device__ __forceinline__ D cpy_conv(S v) {
 template <typename S, typename D> __device__ __forceinline__ void cpy_one(const char *s, char *d) {
     *reinterpret_cast<D *>(d) = cpy_conv<S, D>(*reinterpret_cast<const S *>(s));
 }
-// one thread per element in logical order (i0 fastest); the two sides may have different shapes of one element count
-__device__ __forceinline__ int64_t cpy_offset(int64_t i, const int64_t (&ne)[4], const int64_t (&nb)[4]) {
-    const int64_t i0 = i % ne[0], r0 = i / ne[0];
-    const int64_t i1 = r0 % ne[1], r1 = r0 / ne[1];
-    const int64_t i2 = r1 % ne[2], i3 = r1 / ne[2];
-    return i0 * nb[0] + i1 * nb[1] + i2 * nb[2] + i3 * nb[3];
+// one thread per element in logical order (i0 fastest); the two sides may have different shapes of one element count.
+// IDX is uint32_t whenever the element count allows: 64-bit division is a long software routine.
+template <typename IDX>
+__device__ __forceinline__ int64_t cpy_offset(IDX i, const int64_t (&ne)[4], const int64_t (&nb)[4]) {
+    const IDX n0 = (IDX)ne[0], n1 = (IDX)ne[1], n2 = (IDX)ne[2];
+    const IDX r0 = i / n0, i0 = i - r0 * n0;
+    const IDX r1 = r0 / n1, i1 = r0 - r1 * n1;
+    const IDX i3 = r1 / n2, i2 = r1 - i3 * n2;
+    return (int64_t)i0 * nb[0] + (int64_t)i1 * nb[1] + (int64_t)i2 * nb[2] + (int64_t)i3 * nb[3];
 }
-template <typename S, typename D>
+template <typename S, typename D, typename IDX, bool DENSE_DST>
 __global__ __launch_bounds__(EW_THREADS) void cpy_kernel(const char *__restrict__ src, char *__restrict__ dst, CopyShape sh, int64_t total) {
     for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (int64_t)gridDim.x * EW_THREADS)
-        cpy_one<S, D>(src + cpy_offset(i, sh.ne, sh.nbs), dst + cpy_offset(i, sh.ned, sh.nbd));
+        cpy_one<S, D>(src + cpy_offset<IDX>((IDX)i, sh.ne, sh.nbs),
+                      dst + (DENSE_DST ? i * (int64_t)sizeof(D) : cpy_offset<IDX>((IDX)i, sh.ned, sh.nbd)));
 }
 // both sides dense in the same order: four elements per thread
 template <typename S, typename D>
@@ -297,7 +320,7 @@ __global__ __launch_bounds__(EW_THREADS) void cpy_transpose_kernel(const char *_
     __shared__ S tile[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int64_t t0 = (int64_t)blockIdx.x * 32, t1 = (int64_t)blockIdx.y * 32;
-    const int64_t i2 = blockIdx.z % sh.ne[2], i3 = blockIdx.z / sh.ne[2];
+    const int64_t i3 = (uint32_t)blockIdx.z / (uint32_t)sh.ne[2], i2 = (uint32_t)blockIdx.z - (uint32_t)i3 * (uint32_t)sh.ne[2];
     const char *s = src + i2 * sh.nbs[2] + i3 * sh.nbs[3];
     char *d = dst + i2 * sh.nbd[2] + i3 * sh.nbd[3];
 #pragma unroll
@@ -334,8 +357,14 @@ static hipError_t launch_cpy_typed(const void *src, void *dst, const CopyShape &
                            dim3(EW_THREADS), 0, st, (const char *)src, (char *)dst, sh);
     } else {
         const int64_t want = ceil_div(total, EW_THREADS);
-        hipLaunchKernelGGL((cpy_kernel<S, D>), dim3((unsigned)(want < (1 << 20) ? want : (1 << 20))), dim3(EW_THREADS), 0, st,
-                           (const char *)src, (char *)dst, sh, total);
+        const dim3 grid((unsigned)(want < (1 << 20) ? want : (1 << 20)));
+        const bool small = total < (1LL << 31);
+#define CPY_GO(IDX, DD) hipLaunchKernelGGL((cpy_kernel<S, D, IDX, DD>), grid, dim3(EW_THREADS), 0, st, (const char *)src, (char *)dst, sh, total)
+        if (small && dense_d) CPY_GO(uint32_t, true);
+        else if (small) CPY_GO(uint32_t, false);
+        else if (dense_d) CPY_GO(int64_t, true);
+        else CPY_GO(int64_t, false);
+#undef CPY_GO
     }
     return hipGetLastError();
 }
@@ -352,42 +381,117 @@ hipError_t launch_cpy(const void *src, int src_f16, const int64_t *ne_src, const
     return launch_cpy_typed<uint16_t, float>(src, dst, sh, st);
 }
 
+// cos and sin of a float angle, evaluated in double and rounded once.  |th| < 1e6: two-term Cody-Waite reduction by pi/2
+// (the first term has 33 significant bits, so its product with the quadrant count < 2^20 is exact) and the classic
+// degree-13 / degree-14 minimax polynomials on [-pi/4, pi/4]; absolute error near 1e-16, far below half a unit of the
+// float result.  Larger angles go through the library's full-range reduction.
+__device__ __forceinline__ void sincos_rounded(float th, float &sn, float &cs) {
+    const double x = (double)th;
+    if (!(fabs(x) < 1.0e6)) {
+        double sd, cd;
+        sincos(x, &sd, &cd);
+        sn = (float)sd; cs = (float)cd;
+        return;
+    }
+    const double fn = rint(x * 6.36619772367581382433e-01);
+    const double r = fma(-fn, 1.57079632673412561417e+00, x);
+    const double y = fma(-fn, 6.07710050650619224932e-11, r);
+    const double z = y * y;
+    const double ps = fma(z, fma(z, fma(z, fma(z, fma(z, 1.58969099521155010221e-10, -2.50507602534068634195e-08),
+                                               2.75573137070700676789e-06), -1.98412698298579493134e-04),
+                                 8.33333333332248946124e-03), -1.66666666666666324348e-01);
+    const double s = fma(y * z, ps, y);
+    const double pc = fma(z, fma(z, fma(z, fma(z, fma(z, -1.13596475577881948265e-11, 2.08757232129817482790e-09),
+                                               -2.75573143513906633035e-07), 2.48015872894767294178e-05),
+                                 -1.38888888888741095749e-03), 4.16666666666666019037e-02);
+    const double c = fma(z * z, pc, fma(z, -0.5, 1.0));
+    const int q = (int)fn & 3;
+    const double ss = (q & 1) ? c : s, cc = (q & 1) ? s : c;
+    sn = (float)((q & 2) ? -ss : ss);
+    cs = (float)(((q + 1) & 2) ? -cc : cc);
+}
+
 // ---- ROPE: one workgroup per token; the first n_dims / 2 threads build that position's cos / sin table ----
 constexpr int ROPE_MAX_PAIRS = 256;
 __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restrict__ x, const int32_t *__restrict__ pos,
                                                           const float *__restrict__ freq_factors, RopeArgs a, float *__restrict__ y) {
     __shared__ float cs[ROPE_MAX_PAIRS], sn[ROPE_MAX_PAIRS];
+    constexpr int PRE = 8;                                       // items per thread whose loads are issued before the table is built
     const int64_t tok = blockIdx.x;
     const int half = a.n_dims / 2;
-    for (int p = threadIdx.x; p < half; p += EW_THREADS) {
-        float theta = (float)(int64_t)pos[tok];
-        for (int k = 0; k < p; k++) theta *= a.theta_scale;
-        const float ff = freq_factors ? freq_factors[p] : 1.0f;
-        const float extrap = theta / ff;
-        const float interp = a.freq_scale * extrap;
-        float th = interp;
-        if (a.ext_factor != 0.0f) {
-            const float d = a.corr1 - a.corr0;
-            const float yv = ((float)p - a.corr0) / fmaxf(0.001f, d);
-            const float ramp_mix = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * a.ext_factor;
-            th = interp * (1.0f - ramp_mix) + extrap * ramp_mix;
-        }
-        cs[p] = (float)cos((double)th) * a.mscale;
-        sn[p] = (float)sin((double)th) * a.mscale;
-    }
-    __syncthreads();
     const float *xt = x + tok * a.ldx2;
     float *yt = y + tok * a.ldy2;
-    const int64_t per_head = a.ne0 - half;                       // one item per rotated pair or per passed-through value
-    for (int64_t i = threadIdx.x; i < a.ne1 * per_head; i += EW_THREADS) {
-        const int64_t h = i / per_head, j = i % per_head;
+    const uint32_t per_head = (uint32_t)(a.ne0 - half);          // one item per rotated pair or per passed-through value
+    const uint32_t items = (uint32_t)a.ne1 * per_head;           // 32-bit division: the 64-bit one is a long software routine
+    // the operands of the first PRE * EW_THREADS items do not depend on the table: fetch them first
+    float x0[PRE], x1[PRE];
+    uint32_t ia[PRE], ib[PRE], jj[PRE];
+#pragma unroll
+    for (int u = 0; u < PRE; u++) {
+        const uint32_t i = threadIdx.x + u * EW_THREADS;
+        jj[u] = 0xffffffffu;                                     // no item
+        if (i < items) {
+            const uint32_t h = i / per_head, j = i - h * per_head;
+            const uint32_t base = h * (uint32_t)a.ldx1;
+            jj[u] = j;
+            if (j < (uint32_t)half) { ia[u] = a.neox ? j : 2 * j; ib[u] = a.neox ? j + half : 2 * j + 1; }
+            else                    { ia[u] = j + half; ib[u] = j + half; }
+            x0[u] = xt[base + ia[u]];
+            x1[u] = xt[base + ib[u]];
+            ia[u] += h * (uint32_t)a.ldy1;
+            ib[u] += h * (uint32_t)a.ldy1;
+        }
+    }
+    if ((int)threadIdx.x < half || half > EW_THREADS) {
+        // every lane walks the same chain theta_0 = pos, theta_{k+1} = theta_k * theta_scale and keeps its own step
+        float theta = (float)(int64_t)pos[tok];
+        for (int p0 = 0; p0 < half; p0 += EW_THREADS) {
+            const int p = p0 + threadIdx.x;
+            float mine = theta;
+            const int steps = half - p0 < EW_THREADS ? half - p0 : EW_THREADS;
+            for (int k = 0; k < steps; k++) {
+                mine = (k == (int)threadIdx.x) ? theta : mine;
+                theta *= a.theta_scale;
+            }
+            if (p < half) {
+                const float ff = freq_factors ? freq_factors[p] : 1.0f;
+                const float extrap = mine / ff;
+                const float interp = a.freq_scale * extrap;
+                float th = interp;
+                if (a.ext_factor != 0.0f) {
+                    const float d = a.corr1 - a.corr0;
+                    const float yv = ((float)p - a.corr0) / fmaxf(0.001f, d);
+                    const float ramp_mix = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * a.ext_factor;
+                    th = interp * (1.0f - ramp_mix) + extrap * ramp_mix;
+                }
+                float sf, cf;
+                sincos_rounded(th, sf, cf);
+                cs[p] = cf * a.mscale;
+                sn[p] = sf * a.mscale;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < PRE; u++) {
+        if (jj[u] == 0xffffffffu) continue;
+        if (jj[u] < (uint32_t)half) {
+            const float c = cs[jj[u]], s = sn[jj[u]];
+            yt[ia[u]] = x0[u] * c - x1[u] * s;
+            yt[ib[u]] = x0[u] * s + x1[u] * c;
+        } else {
+            yt[ia[u]] = x0[u];
+        }
+    }
+    for (uint32_t i = threadIdx.x + PRE * EW_THREADS; i < items; i += EW_THREADS) {
+        const uint32_t h = i / per_head, j = i - h * per_head;
         const float *xr = xt + h * a.ldx1;
         float *yr = yt + h * a.ldy1;
-        if (j < half) {
-            const int64_t ia = a.neox ? j : 2 * j, ib = a.neox ? j + half : 2 * j + 1;
-            const float x0 = xr[ia], x1 = xr[ib], c = cs[j], s = sn[j];
-            yr[ia] = x0 * c - x1 * s;
-            yr[ib] = x0 * s + x1 * c;
+        if (j < (uint32_t)half) {
+            const int64_t ka = a.neox ? j : 2 * j, kb = a.neox ? j + half : 2 * j + 1;
+            const float v0 = xr[ka], v1 = xr[kb], c = cs[j], s = sn[j];
+            yr[ka] = v0 * c - v1 * s;
+            yr[kb] = v0 * s + v1 * c;
         } else {
             yr[j + half] = xr[j + half];
         }
@@ -395,7 +499,8 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
 }
 hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, hipStream_t st) {
     if (a.ne0 <= 0 || a.ne1 <= 0 || a.ne2 <= 0) return hipSuccess;
-    if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff) return hipErrorInvalidValue;
+    if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff || a.ne0 * a.ne1 > 0x7fffffff) return hipErrorInvalidValue;
+    if (a.ne1 * a.ldx1 > 0x7fffffff || a.ne1 * a.ldy1 > 0x7fffffff) return hipErrorInvalidValue;       // 32-bit offsets inside a token
     hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a.ne2), dim3(EW_THREADS), 0, st, x, pos, freq_factors, a, y);
     return hipGetLastError();
 }
@@ -405,8 +510,15 @@ hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, 
     for (int64_t r0 = 0; r0 < n; r0 += 1 << 30) {
         const int64_t rows = n - r0 < (1 << 30) ? n - r0 : (1 << 30);
         hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(EW_THREADS), 0, st, x + r0 * ldx, ldx, ne0, eps,
-                           y + r0 * ldy, ldy);
+                           y + r0 * ldy, ldy, (const float *)nullptr, (float *)nullptr, (int64_t)0);
     }
+    return hipGetLastError();
+}
+hipError_t launch_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, const float *w, float *yn, int64_t ldyn,
+                               float *y, int64_t ldy, hipStream_t st) {
+    if (n <= 0 || ne0 <= 0) return hipSuccess;
+    if (n > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)n), dim3(EW_THREADS), 0, st, x, ldx, ne0, eps, y, ldy, w, yn, ldyn);
     return hipGetLastError();
 }
 
@@ -431,6 +543,8 @@ hipError_t launch_add(const float *a, int64_t lda, const float *b, int64_t ldb, 
                       hipStream_t st) { return launch_ew<EW_ADD>(a, lda, b, ldb, ne0, n, y, ldy, st); }
 hipError_t launch_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy,
                       hipStream_t st) { return launch_ew<EW_MUL>(a, lda, b, ldb, ne0, n, y, ldy, st); }
+hipError_t launch_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy,
+                           hipStream_t st) { return launch_ew<EW_SILU_MUL>(x, ldx, b, ldb, ne0, n, y, ldy, st); }
 hipError_t launch_silu(const float *x, int64_t ldx, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st) {
     return launch_ew<EW_SILU>(x, ldx, nullptr, 0, ne0, n, y, ldy, st);
 }

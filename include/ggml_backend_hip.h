@@ -44,6 +44,8 @@ CACTUS_GGML_API int lm_ggml_backend_is_hip(struct lm_ggml_backend *backend);
 
 /* Counters for tests and tracing: MUL_MAT nodes executed on the GPU and bytes uploaded by set_tensor. */
 CACTUS_GGML_API void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned long long *uploaded_bytes);
+/* Pairs of adjacent nodes (RMS_NORM + MUL, SILU + MUL) that graph_compute ran as one kernel. */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_fused_pairs(void);
 
 #ifdef __cplusplus
 }

@@ -180,7 +180,7 @@ def rope_tolerance(x, n_dims, mode, mscale):
 def test_rope(dev, orc, mode, ne0, n_dims, n_head, n_tokens):
     rng = np.random.default_rng(ne0 + n_dims + mode)
     x = rng.standard_normal((n_tokens, n_head, ne0)).astype(np.float32)
-    pos = np.array([0, 1, 17, 4095, 100000, 31, 2][:n_tokens], np.int32)
+    pos = np.array([0, 1, 17, 4095, 100000, 31, 3000000][:n_tokens], np.int32)   # the last one takes the full-range reduction
     ff = (1.0 + rng.random(n_dims // 2) * 7).astype(np.float32)
     cases = [({}, 1.0), (dict(freq_base=500000.0, freq_scale=0.25), 1.0), (dict(freq_factors=ff), 1.0),
              (dict(freq_scale=0.25, ext_factor=1.0, attn_factor=1.2, n_ctx_orig=2048), 1.2 * (1.0 + 0.1 * np.log(4.0)))]

@@ -419,7 +419,13 @@ def test_ffn_block_stays_on_the_device(host, orc):
     sched = L.lm_ggml_backend_sched_new(backends, None, 2, 64, False, True)
     assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
     host.set(tx, x)
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_fused_pairs.restype = C.c_ulonglong
+    fused_before = blib.lm_ggml_backend_hip_get_fused_pairs()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    # norm + weight ran as one kernel (the allocator writes the MUL over its only producer); SiLU and its MUL are not
+    # neighbours in the node order (the up projection sits between them), so they stay two kernels
+    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == 1
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (cur, up, gate, act, down, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip

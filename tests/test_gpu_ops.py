@@ -104,3 +104,33 @@ def test_strided_rows_in_place_and_errors(dev, orc):
     got = np.stack([got[1 + r * ld: 1 + r * ld + ne0 - 3] for r in range(n - 1)])
     with np.errstate(all="ignore"):
         assert got.tobytes() == (want * want).tobytes()
+
+
+@pytest.mark.parametrize("n,ne0", [(1, 4096), (7, 4096), (3, 40), (130, 14336), (5, 1000)])
+def test_fused_pairs_equal_the_separate_ops(dev, orc, n, ne0):
+    """chip_rms_norm_mul and chip_silu_mul against the two separate device calls (bit for bit) and the oracle."""
+    x = inputs(3 * n + ne0, n, ne0)
+    w = (1.0 + 0.1 * np.random.default_rng(ne0).standard_normal(ne0)).astype(np.float32)
+    dx, dw = dev.to_device(x), dev.to_device(w)
+    dy, dn = dev.alloc(x.nbytes), dev.alloc(x.nbytes)
+    dev.check(dev.lib.chip_rms_norm_mul(dx.ptr, ne0, n, ne0, 1e-5, dw.ptr, dn.ptr, ne0, dy.ptr, ne0, None))
+    dev.sync()
+    y = dy.download(np.float32, x.size).reshape(n, ne0)
+    yn = dn.download(np.float32, x.size).reshape(n, ne0)
+    sep = dev.rms_norm(x, 1e-5)
+    assert yn.tobytes() == sep.tobytes()
+    assert y.tobytes() == dev.binary("mul", sep, w).tobytes() == (sep * w).tobytes()
+    dev.check(dev.lib.chip_rms_norm_mul(dx.ptr, ne0, n, ne0, 1e-5, dw.ptr, None, 0, dx.ptr, ne0, None))      # in place, no norm output
+    dev.sync()
+    assert dx.download(np.float32, x.size).tobytes() == y.tobytes()
+    if ne0 % 8 == 0:
+        b = inputs(5 * n + ne0, n, ne0)
+        da, db = dev.to_device(x), dev.to_device(b)
+        dev.check(dev.lib.chip_silu_mul(da.ptr, ne0, db.ptr, ne0, n, ne0, da.ptr, ne0, None))
+        dev.sync()
+        with np.errstate(all="ignore"):
+            want = orc.silu(x) * b
+        assert da.download(np.float32, x.size).tobytes() == want.tobytes()
+    else:
+        import cactus_amd as ca
+        assert dev.lib.chip_silu_mul(dx.ptr, ne0, dx.ptr, ne0, n, ne0, dy.ptr, ne0, None) == ca.CHIP_EUNSUPPORTED
