@@ -193,12 +193,16 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArg
 // e * r2 * n ... (e + 1) * r2 * n - 1, in order.
 __global__ __launch_bounds__(AM_THREADS) void mm_f16_round_rows_kernel(const float *__restrict__ x, int64_t ldx1, int64_t ldx2,
                                                                        int64_t n, int64_t K, uint8_t *__restrict__ ws, size_t ws_stride) {
-    const int64_t t = blockIdx.x, b = blockIdx.y;
-    const float *xr = x + b * ldx2 + t * ldx1;
-    u32x4 *out = reinterpret_cast<u32x4 *>(ws + (size_t)(b * n + t) * ws_stride);
-    for (int64_t ch = threadIdx.x; ch < K / 8; ch += AM_THREADS) {
-        const float4 *xp = reinterpret_cast<const float4 *>(xr + 8 * ch);
-        out[ch] = round8(xp[0], xp[1]);
+    // a workgroup takes as many tokens of one batch as its threads cover with one 8-value chunk each (16 for K = 128)
+    const uint32_t chunks = (uint32_t)(K / 8);
+    const uint32_t per = chunks >= AM_THREADS ? 1u : AM_THREADS / chunks;
+    const int64_t b = blockIdx.y;
+    for (uint32_t i = threadIdx.x; i < per * chunks; i += AM_THREADS) {
+        const uint32_t r = i / chunks, ch = i - r * chunks;
+        const int64_t t = (int64_t)blockIdx.x * per + r;
+        if (t >= n) continue;
+        const float4 *xp = reinterpret_cast<const float4 *>(x + b * ldx2 + t * ldx1 + 8 * ch);
+        reinterpret_cast<u32x4 *>(ws + (size_t)(b * n + t) * ws_stride)[ch] = round8(xp[0], xp[1]);
     }
 }
 __global__ __launch_bounds__(AM_THREADS) void mm_f16_tile_list_kernel(int64_t ne02, int64_t per_head, int tile_tokens,
@@ -250,8 +254,9 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
     if (plan.use && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {
         uint8_t *ws = (uint8_t *)workspace;
         int32_t *perm = (int32_t *)(ws + plan.off_perm), *offsets = (int32_t *)(ws + plan.off_offsets), *tiles = (int32_t *)(ws + plan.off_tiles);
-        hipLaunchKernelGGL(mm_f16_round_rows_kernel, dim3((unsigned)n, (unsigned)(ne02 * r2)), dim3(AM_THREADS), 0, st, x, ldx1, ldx2, n, K,
-                           ws, plan.act_stride);
+        const int64_t chunks = K / 8, per = chunks >= AM_THREADS ? 1 : AM_THREADS / chunks;
+        hipLaunchKernelGGL(mm_f16_round_rows_kernel, dim3((unsigned)ceil_div(n, per), (unsigned)(ne02 * r2)), dim3(AM_THREADS), 0, st, x,
+                           ldx1, ldx2, n, K, ws, plan.act_stride);
         hipLaunchKernelGGL(mm_f16_tile_list_kernel, dim3(64), dim3(AM_THREADS), 0, st, ne02, r2 * n, gemm_f16_moe_tile_tokens(), perm,
                            offsets, tiles);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
