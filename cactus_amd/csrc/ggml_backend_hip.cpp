@@ -6,8 +6,9 @@
 //              ->  buffer type "HIP": hipMalloc'd buffers, tensors at base + offset, GGUF blocks kept verbatim
 //              ->  buffer type "HIP_Host": pinned host memory (the staging buffers of the loader's async upload)
 //              ->  backend "HIP": one stream; graph_compute runs MUL_MAT / MUL_MAT_ID (F32 activations x block-quantized
-//                  or F16 weights living in a HIP buffer) and skips view ops; set/get_tensor_async and events on
-//                  that stream.
+//                  or F16 weights living in a HIP buffer), the ops around them in a transformer layer (RMS_NORM, ADD,
+//                  MUL, SILU, ROPE, CPY / CONT / DUP, SOFT_MAX, the batched F16 matmuls over the KV cache) and skips
+//                  view ops; set/get_tensor_async and events on that stream.
 // No C++ exception crosses the vtables; failures are NULL returns or LM_GGML_STATUS_FAILED.
 #include "../../include/cactus_hip.h"
 #include "../../include/ggml_abi_mirror.h"
