@@ -37,7 +37,7 @@ EXPORTS = (
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul",
-    "chip_soft_max", "chip_cpy", "chip_rope", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
+    "chip_soft_max", "chip_cpy", "chip_rope", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -110,6 +110,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_soft_max.argtypes = [vp, i64, vp, i32, i64, i64, i64, C.c_float, C.c_float, vp, i64, vp]
     L.chip_cpy.argtypes = [vp, i32, C.POINTER(i64), C.POINTER(i64), vp, i32, C.POINTER(i64), C.POINTER(i64), vp]
     L.chip_rope.argtypes = [vp, i64, i64, vp, vp, i64, i64, i64, i32, i32, i32] + [C.c_float] * 6 + [vp, i64, i64, vp]
+    L.chip_get_rows.argtypes = [i32, vp, sz, sz, sz, i64, i64, vp, i64, i64, i64, i64, i64, vp, i64, i64, i64, vp]
     L.chip_mul_mat_f16_batched.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_f16_batched_workspace_size.restype = sz
     L.chip_mul_mat_f16_batched_workspace_size.argtypes = [i64, i64, i64, i64, i64]
@@ -313,6 +314,21 @@ class Device:
                                       dy.ptr, ne0, ne0 * ne1, None))
         self.sync()
         return dy.download(np.float32, x.size).reshape(x.shape)
+
+    def get_rows(self, t, table, nc, ids):
+        """table uint8 [ne01, row_size(t, nc)] (or float32 / float16 [ne01, nc] for F32 / F16), ids int32 [n] -> fp32 [n, nc];
+        rows of ids outside the table come back as NaN (left unwritten)."""
+        table = np.ascontiguousarray(table)
+        ids = np.ascontiguousarray(ids, np.int32)
+        ne01 = table.shape[0]
+        nb01 = table.strides[0]
+        dt, di = self.to_device(table.reshape(-1).view(np.uint8)), self.to_device(ids)
+        dy = self.alloc(max(ids.size * nc * 4, 16))
+        self.check(self.lib.chip_memset(dy.ptr, 0xFF, max(ids.size * nc * 4, 16), None))
+        self.check(self.lib.chip_get_rows(t, dt.ptr, nb01, nb01 * ne01, nb01 * ne01, nc, ne01, di.ptr, ids.size, 1, 1, ids.size,
+                                          ids.size, dy.ptr, nc, nc * ids.size, nc * ids.size, None))
+        self.sync()
+        return dy.download(np.float32, ids.size * nc).reshape(ids.size, nc)
 
     def mul_mat_f16_batched(self, W, x, workspace=True):
         """W fp16 array or view [ne02, N, K] (K contiguous), x fp32 array or view [ne12, n, K] (K contiguous) ->

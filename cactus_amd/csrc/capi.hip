@@ -508,6 +508,21 @@ int chip_cpy(const void *src, int src_type, const int64_t ne_src[4], const int64
     return hip_rc(launch_cpy(src, src_type == T_F16, ne_src, nb_src, dst, dst_type == T_F16, ne_dst, nb_dst, (hipStream_t)stream));
 }
 
+int chip_get_rows(int type, const void *src, size_t nb01, size_t nb02, size_t nb03, int64_t nc, int64_t ne01, const int32_t *ids,
+                  int64_t ne10, int64_t ne11, int64_t ne12, int64_t ldi1, int64_t ldi2, float *dst, int64_t ld1, int64_t ld2, int64_t ld3,
+                  void *stream) {
+    if (nc < 0 || ne01 < 0 || ne10 < 0 || ne11 < 0 || ne12 < 0) return CHIP_EINVAL;
+    if (!(type == T_F32 || is_weight_type(type))) return CHIP_EUNSUPPORTED;
+    const int be = (type == T_F32 || type == T_F16) ? 1 : chip_block_elems(type);
+    if (nc % be != 0) return CHIP_EINVAL;                                    // whole blocks
+    if (nc == 0 || ne10 * ne11 * ne12 == 0) return CHIP_OK;
+    if (!src || !ids || !dst || ld1 < nc) return CHIP_EINVAL;
+    const size_t al = type == T_F32 ? 4 : 2;                                 // the dequantizers read 2-byte pieces
+    if (((uintptr_t)src | nb01 | nb02 | nb03) % al != 0 || ((uintptr_t)ids & 3) != 0 || ((uintptr_t)dst & 3) != 0) return CHIP_EINVAL;
+    const GetRowsArgs a{(const uint8_t *)src, nb01, nb02, nb03, nc, ne01, ids, ne10, ne11, ne12, ldi1, ldi2, dst, ld1, ld2, ld3};
+    return hip_rc(launch_get_rows(type, a, (hipStream_t)stream));
+}
+
 int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1,
               int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
               float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1, int64_t ldy2, void *stream) {

@@ -314,7 +314,8 @@ int run_elementwise(backend_ctx *c, lm_ggml_tensor *op) {
 
 // ---- the attention-side ops around the KV cache (SOFT_MAX, ROPE, CPY / CONT / DUP) ----
 bool is_attn_side_op(int op) {
-    return op == LM_GGML_OP_SOFT_MAX || op == LM_GGML_OP_ROPE || op == LM_GGML_OP_CPY || op == LM_GGML_OP_CONT || op == LM_GGML_OP_DUP;
+    return op == LM_GGML_OP_SOFT_MAX || op == LM_GGML_OP_ROPE || op == LM_GGML_OP_CPY || op == LM_GGML_OP_CONT || op == LM_GGML_OP_DUP ||
+           op == LM_GGML_OP_GET_ROWS;
 }
 bool dense(const lm_ggml_tensor *t) {                   // lm_ggml_is_contiguous for the unquantized types
     size_t want = (t->type == LM_GGML_TYPE_F16) ? 2 : 4;
@@ -353,11 +354,27 @@ bool cpy_shape_ok(const lm_ggml_tensor *op) {
     if (!a || !f32_or_f16(a) || !f32_or_f16(op) || n_elements(a) != n_elements(op)) return false;
     return true;                                       // shapes may differ: element i of one logical order to element i of the other
 }
+// GET_ROWS: a table that lives in a HIP buffer (any type the matmuls take, or F32), or an F32 / F16 activation.
+bool get_rows_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0], *ids = op->src[1];
+    if (!a || !ids || ids->type != LM_GGML_TYPE_I32 || op->type != LM_GGML_TYPE_F32) return false;
+    const bool plain = a->type == LM_GGML_TYPE_F32 || a->type == LM_GGML_TYPE_F16;
+    if (!plain && !chip_mul_mat_supported(a->type, 256)) return false;
+    const lm_ggml_backend_buffer_t abuf = a->view_src ? a->view_src->buffer : a->buffer;
+    if (abuf ? !is_hip_buffer(abuf) : !plain) return false;                   // a host-resident table stays with the CPU backend
+    if (a->nb[0] != (plain ? (a->type == LM_GGML_TYPE_F16 ? 2u : 4u) : chip_block_bytes(a->type))) return false;
+    if (!plain && a->ne[0] % chip_block_elems(a->type) != 0) return false;
+    if (ids->nb[0] != 4 || ids->nb[1] % 4 != 0 || ids->nb[2] % 4 != 0 || ids->ne[3] != 1) return false;
+    if (a->ne[2] != ids->ne[1] || a->ne[3] != ids->ne[2]) return false;       // the reference's batch rule (ne02 == ne11)
+    if (op->nb[0] != 4 || op->nb[1] % 4 != 0 || op->nb[2] % 4 != 0 || op->nb[3] % 4 != 0 || op->nb[1] < (size_t)a->ne[0] * 4) return false;
+    return op->ne[0] == a->ne[0] && op->ne[1] == ids->ne[0] && op->ne[2] == ids->ne[1] && op->ne[3] == ids->ne[2];
+}
 bool attn_side_shape_ok(const lm_ggml_tensor *op) {
     if (!elementwise_enabled()) return false;
     switch (op->op) {
         case LM_GGML_OP_SOFT_MAX: return soft_max_shape_ok(op);
         case LM_GGML_OP_ROPE:     return rope_shape_ok(op);
+        case LM_GGML_OP_GET_ROWS: return get_rows_shape_ok(op);
         default:               return cpy_shape_ok(op);
     }
 }
@@ -380,6 +397,12 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op) {
                              ff ? (const float *)ff->data : nullptr, a->ne[0], a->ne[1], a->ne[2], op->op_params[1], op->op_params[2],
                              op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], (float *)op->data, (int64_t)(op->nb[1] / 4),
                              (int64_t)(op->nb[2] / 4), c->stream);
+        }
+        case LM_GGML_OP_GET_ROWS: {
+            const lm_ggml_tensor *ids = op->src[1];
+            return chip_get_rows(a->type, a->data, a->nb[1], a->nb[2], a->nb[3], a->ne[0], a->ne[1], (const int32_t *)ids->data, ids->ne[0],
+                                 ids->ne[1], ids->ne[2], (int64_t)(ids->nb[1] / 4), (int64_t)(ids->nb[2] / 4), (float *)op->data,
+                                 (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), (int64_t)(op->nb[3] / 4), c->stream);
         }
         default: {
             int64_t nes[4], nbs[4], ned[4], nbd[4];

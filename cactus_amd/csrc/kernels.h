@@ -203,6 +203,13 @@ struct RopeArgs {
     int n_dims, neox;
     float theta_scale, freq_scale, ext_factor, corr0, corr1, mscale;
 };
+// LM_GGML_OP_GET_ROWS: dst row (i10, i11, i12) = row ids[i10, i11, i12] of matrix (i11, i12) of src, dequantized to F32.
+struct GetRowsArgs {
+    const uint8_t *src; size_t nb01, nb02, nb03; int64_t nc, ne01;
+    const int32_t *ids; int64_t ne10, ne11, ne12, ldi1, ldi2;                 // ids strides in elements
+    float *dst; int64_t ld1, ld2, ld3;                                         // dst strides in floats
+};
+hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st);
 hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, hipStream_t st);
 
 // moe_group.hip: counting sort of MUL_MAT_ID's (token, slot) pairs by expert into offsets[n_as + 1] / perm[pairs].

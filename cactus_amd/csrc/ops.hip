@@ -22,6 +22,8 @@
 //             and sin are computed in double here and rounded once (the reference calls the C library's cosf / sinf,
 //             which may differ from that by one unit in the last place), the rotation itself is unfused float
 //             arithmetic as in the reference.
+//   GET_ROWS  lm_ggml_compute_forward_get_rows (ggml-cpu/ops.cpp:4236-4453): selected rows of a table converted to F32 with
+//             the type's dequantize_row_* expression (ggml-quants.c).  Bit-exact.
 #include "dev_common.h"
 #include "kernels.h"
 
@@ -409,6 +411,97 @@ __device__ __forceinline__ void sincos_rounded(float th, float &sn, float &cs) {
     const double ss = (q & 1) ? c : s, cc = (q & 1) ? s : c;
     sn = (float)((q & 2) ? -ss : ss);
     cs = (float)(((q + 1) & 2) ? -cc : cc);
+}
+
+// ---- GET_ROWS: one thread per output value; element i of a row in the row's block format ----
+// The expressions are those of the reference's dequantize_row_* (ggml-quants.c:249-341, 1274-1296, 1476-1501, 1684-1713,
+// 2430-2446), one rounding per operation, so the values are bit-identical to the CPU's.
+__device__ __forceinline__ void k_scale_min(int j, const uint8_t *q, int &sc, int &m) {        // get_scale_min_k4
+    if (j < 4) { sc = q[j] & 63; m = q[j + 4] & 63; }
+    else { sc = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4); m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4); }
+}
+__device__ __constant__ int8_t k_iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+__device__ __forceinline__ uint32_t load_u32_unaligned2(const uint8_t *p) {
+    return (uint32_t)reinterpret_cast<const uint16_t *>(p)[0] | ((uint32_t)reinterpret_cast<const uint16_t *>(p)[1] << 16);
+}
+template <int WT> __device__ __forceinline__ float dequant_at(const uint8_t *row, uint32_t i) {
+    if constexpr (WT == T_F32) return reinterpret_cast<const float *>(row)[i];
+    else if constexpr (WT == T_F16) return h2f(reinterpret_cast<const uint16_t *>(row)[i]);
+    else if constexpr (WT == T_Q4_0 || WT == T_Q4_1 || WT == T_IQ4_NL) {
+        constexpr int BYTES = WT == T_Q4_1 ? BYTES_Q4_1 : BYTES_Q4_0, QS = WT == T_Q4_1 ? 4 : 2;
+        const uint8_t *b = row + (size_t)(i >> 5) * BYTES;
+        const uint32_t j = i & 31;
+        const float d = h2f(reinterpret_cast<const uint16_t *>(b)[0]);
+        const int q = b[QS + (j & 15)], nib = j < 16 ? (q & 0xF) : (q >> 4);
+        if constexpr (WT == T_Q4_0) return (float)(nib - 8) * d;
+        else if constexpr (WT == T_Q4_1) return (float)nib * d + h2f(reinterpret_cast<const uint16_t *>(b)[1]);
+        else return d * (float)k_iq4nl_values[nib];
+    } else if constexpr (WT == T_Q8_0) {
+        const uint8_t *b = row + (size_t)(i >> 5) * BYTES_Q8_0;
+        return (float)(int8_t)b[2 + (i & 31)] * h2f(reinterpret_cast<const uint16_t *>(b)[0]);
+    } else if constexpr (WT == T_Q5_0 || WT == T_Q5_1) {
+        constexpr int BYTES = WT == T_Q5_1 ? BYTES_Q5_1 : BYTES_Q5_0, QH = WT == T_Q5_1 ? 4 : 2;
+        const uint8_t *b = row + (size_t)(i >> 5) * BYTES;
+        const uint32_t j = i & 31;
+        const float d = h2f(reinterpret_cast<const uint16_t *>(b)[0]);
+        const uint32_t qh = load_u32_unaligned2(b + QH);
+        const int q = b[QH + 4 + (j & 15)];
+        const int v = j < 16 ? ((q & 0xF) | (int)(((qh >> j) << 4) & 0x10)) : ((q >> 4) | (int)((qh >> (j - 16 + 12)) & 0x10));
+        if constexpr (WT == T_Q5_0) return (float)(v - 16) * d;
+        else return (float)v * d + h2f(reinterpret_cast<const uint16_t *>(b)[1]);
+    } else if constexpr (WT == T_Q4_K || WT == T_Q5_K) {
+        constexpr int BYTES = WT == T_Q5_K ? BYTES_Q5_K : BYTES_Q4_K, QS = WT == T_Q5_K ? 48 : 16;
+        const uint8_t *b = row + (size_t)(i >> 8) * BYTES;
+        const uint32_t r = i & 255, j64 = r >> 6, l = r & 63, hi = l >> 5, ll = l & 31;
+        const float d = h2f(reinterpret_cast<const uint16_t *>(b)[0]), mn = h2f(reinterpret_cast<const uint16_t *>(b)[1]);
+        int sc, m;
+        k_scale_min((int)(2 * j64 + hi), b + 4, sc, m);
+        const float d1 = d * (float)sc, m1 = mn * (float)m;
+        const int q = b[QS + 32 * j64 + ll];
+        int v = hi ? (q >> 4) : (q & 0xF);
+        if constexpr (WT == T_Q5_K) v += (b[16 + ll] & (1u << (2 * j64 + hi))) ? 16 : 0;
+        return d1 * (float)v - m1;
+    } else {                                                            // T_Q6_K: ql[128] qh[64] scales[16] d
+        const uint8_t *b = row + (size_t)(i >> 8) * BYTES_Q6_K;
+        const uint32_t r = i & 255, h = r >> 7, rr = r & 127, quarter = rr >> 5, l = rr & 31;
+        const uint8_t *ql = b + 64 * h, *qh = b + 128 + 32 * h;
+        const int8_t *sc = reinterpret_cast<const int8_t *>(b + 192 + 8 * h);
+        const float d = h2f(reinterpret_cast<const uint16_t *>(b + 208)[0]);
+        const int lo = (quarter & 1) ? ql[l + 32] : ql[l];
+        const int nib = (quarter & 2) ? (lo >> 4) : (lo & 0xF);
+        const int q = (int)(int8_t)(nib | (((qh[l] >> (2 * quarter)) & 3) << 4)) - 32;
+        return d * (float)sc[(l >> 4) + 2 * quarter] * (float)q;
+    }
+}
+template <int WT>
+__global__ __launch_bounds__(EW_THREADS) void get_rows_kernel(GetRowsArgs a) {
+    const uint32_t per = (uint32_t)(a.ne11 * a.ne10), rows = per * (uint32_t)a.ne12;
+    for (uint32_t r = blockIdx.y; r < rows; r += gridDim.y) {                   // row of dst: (i12, i11, i10), i10 fastest
+        const uint32_t i12 = r / per, rem = r - i12 * per, i11 = rem / (uint32_t)a.ne10, i10 = rem - i11 * (uint32_t)a.ne10;
+        const int64_t id = a.ids[i10 + i11 * a.ldi1 + i12 * a.ldi2];
+        if (id < 0 || id >= a.ne01) continue;                                   // the reference asserts; the row stays unwritten
+        const uint8_t *row = a.src + id * a.nb01 + i11 * a.nb02 + i12 * a.nb03;
+        float *out = a.dst + i10 * a.ld1 + i11 * a.ld2 + i12 * a.ld3;
+        for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < a.nc; i += (int64_t)gridDim.x * EW_THREADS)
+            out[i] = dequant_at<WT>(row, (uint32_t)i);
+    }
+}
+hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st) {
+    const int64_t rows = a.ne10 * a.ne11 * a.ne12;
+    if (rows <= 0 || a.nc <= 0) return hipSuccess;
+    if (a.nc > 0x7fffffff) return hipErrorInvalidValue;
+    const int64_t want = ceil_div(a.nc, EW_THREADS);
+    const unsigned gx = (unsigned)(want < 64 ? want : 64);
+    if (rows > 0x7fffffff) return hipErrorInvalidValue;
+    const dim3 grid(gx, (unsigned)(rows < 65535 ? rows : 65535));
+#define GR_CASE(TT) case TT: hipLaunchKernelGGL(get_rows_kernel<TT>, grid, dim3(EW_THREADS), 0, st, a); break;
+    switch (type) {
+        GR_CASE(T_F32) GR_CASE(T_F16) GR_CASE(T_Q4_0) GR_CASE(T_Q4_1) GR_CASE(T_Q5_0) GR_CASE(T_Q5_1) GR_CASE(T_Q8_0)
+        GR_CASE(T_Q4_K) GR_CASE(T_Q5_K) GR_CASE(T_Q6_K) GR_CASE(T_IQ4_NL)
+        default: return hipErrorInvalidValue;
+    }
+#undef GR_CASE
+    return hipGetLastError();
 }
 
 // ---- ROPE: one workgroup per token; the first n_dims / 2 threads build that position's cos / sin table ----

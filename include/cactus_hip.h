@@ -228,6 +228,15 @@ CHIP_API int chip_soft_max(const float *x, int64_t ldx, const void *mask, int ma
                            int64_t n_rows, float scale, float max_bias, float *y, int64_t ldy, void *stream);
 CHIP_API int chip_cpy(const void *src, int src_type, const int64_t ne_src[4], const int64_t nb_src[4], void *dst, int dst_type,
                       const int64_t ne_dst[4], const int64_t nb_dst[4], void *stream);
+/*   chip_get_rows : LM_GGML_OP_GET_ROWS, lm_ggml_compute_forward_get_rows (ggml-cpu/ops.cpp:4236-4453): dst row (i10, i11, i12) =
+ *                   row ids[i10, i11, i12] of matrix (i11, i12) of src, converted to F32 with the type's dequantize_row_*
+ *                   (ggml-quants.c) - bit for bit.  src: F32, F16 or any weight type of this library, rows of nc values
+ *                   (whole blocks) at nb01 bytes, matrices at nb02 / nb03 bytes; ids I32 with strides ldi1 / ldi2 in
+ *                   elements; dst strides in floats.  An id outside [0, ne01) leaves its row unwritten (the reference
+ *                   asserts). */
+CHIP_API int chip_get_rows(int type, const void *src, size_t nb01, size_t nb02, size_t nb03, int64_t nc, int64_t ne01,
+                           const int32_t *ids, int64_t ne10, int64_t ne11, int64_t ne12, int64_t ldi1, int64_t ldi2, float *dst,
+                           int64_t ld1, int64_t ld2, int64_t ld3, void *stream);
 CHIP_API int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0,
                        int64_t ne1, int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                        float ext_factor, float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1,

@@ -259,6 +259,15 @@ class Oracle:
             y[b], sa[b] = o["y"], o["sum_abs"]
         return {"y": y, "sum_abs": sa} if "sum_abs" in want else {"y": y}
 
+    def get_rows(self, t, table, nc, ids):
+        """LM_GGML_OP_GET_ROWS (ggml-cpu/ops.cpp:4236-4453): the rows ids of a table of type t, dequantized to fp32 with the
+        type's dequantize_row (F32: copied).  table: uint8 [ne01, row_size] for block types and F16, fp32 [ne01, nc] for F32."""
+        ids = np.asarray(ids, np.int64)
+        if t == F32:
+            return np.ascontiguousarray(np.asarray(table, np.float32)[ids])
+        tb = np.ascontiguousarray(table).view(np.uint8).reshape(len(table), -1)
+        return self.dequantize(t, tb[ids], nc)
+
     def rms_norm(self, x, eps):
         """LM_GGML_OP_RMS_NORM over the rows of x fp32 [n, ne0]."""
         x = _f32(x)
@@ -661,6 +670,21 @@ class Reference:
         kq = self._run_graph(build_kq, {"k": k_cache, "q": _f32(q)}, (n_head, n_tokens, n_kv), np.float32, nthreads)
         kqv = self._run_graph(build_kqv, {"v": vt_cache, "p": _f32(p)}, (n_head, n_tokens, hd), np.float32, nthreads)
         return kq, kqv
+
+    def get_rows_graph(self, t, table, nc, ids, nthreads=1):
+        """lm_ggml_get_rows on the reference CPU backend: table as Oracle.get_rows takes it, ids int32 [n] -> fp32 [n, nc]."""
+        L = self.lib
+        L.lm_ggml_get_rows.restype = _vp
+        L.lm_ggml_get_rows.argtypes = [_vp, _vp, _vp]
+        table = np.ascontiguousarray(table)
+        ids = np.ascontiguousarray(ids, np.int32)
+        ne01 = table.shape[0]
+
+        def build(ctx):
+            ta = L.lm_ggml_new_tensor_2d(ctx, t, nc, ne01)
+            ti = L.lm_ggml_new_tensor_1d(ctx, 26, ids.size)
+            return L.lm_ggml_get_rows(ctx, ta, ti), {"a": ta, "i": ti}
+        return self._run_graph(build, {"a": table, "i": ids}, (ids.size, nc), np.float32, nthreads)
 
     def mul_mat_id_graph(self, wtype, W, x, ids, nthreads=1):
         """LM_GGML_OP_MUL_MAT_ID on the reference CPU backend: W uint8 [n_as, N, row_size], x fp32

@@ -33,6 +33,7 @@ namespace mirror {
 #define LM_GGML_OP_ADD M_OP_ADD
 #define LM_GGML_OP_MUL_MAT_ID M_OP_MUL_MAT_ID
 #define LM_GGML_OP_DUP M_OP_DUP
+#define LM_GGML_OP_GET_ROWS M_OP_GET_ROWS
 #define LM_GGML_OP_CPY M_OP_CPY
 #define LM_GGML_OP_CONT M_OP_CONT
 #define LM_GGML_OP_SOFT_MAX M_OP_SOFT_MAX
@@ -78,6 +79,7 @@ constexpr int k_max_dims = LM_GGML_MAX_DIMS, k_max_src = LM_GGML_MAX_SRC, k_max_
 #undef LM_GGML_OP_ADD
 #undef LM_GGML_OP_MUL_MAT_ID
 #undef LM_GGML_OP_DUP
+#undef LM_GGML_OP_GET_ROWS
 #undef LM_GGML_OP_CPY
 #undef LM_GGML_OP_CONT
 #undef LM_GGML_OP_SOFT_MAX
@@ -146,7 +148,7 @@ static_assert(mirror::M_OP_NONE == LM_GGML_OP_NONE && mirror::M_OP_MUL_MAT == LM
               mirror::M_OP_COUNT == LM_GGML_OP_COUNT && mirror::M_OP_MUL_MAT_ID == LM_GGML_OP_MUL_MAT_ID &&
               mirror::M_OP_ADD == LM_GGML_OP_ADD && mirror::M_OP_MUL == LM_GGML_OP_MUL && mirror::M_OP_RMS_NORM == LM_GGML_OP_RMS_NORM &&
               mirror::M_OP_UNARY == LM_GGML_OP_UNARY && mirror::M_UNARY_OP_SILU == LM_GGML_UNARY_OP_SILU &&
-              mirror::M_OP_DUP == LM_GGML_OP_DUP && mirror::M_OP_CPY == LM_GGML_OP_CPY && mirror::M_OP_CONT == LM_GGML_OP_CONT && mirror::M_OP_SOFT_MAX == LM_GGML_OP_SOFT_MAX && mirror::M_OP_ROPE == LM_GGML_OP_ROPE, "op ids");
+              mirror::M_OP_DUP == LM_GGML_OP_DUP && mirror::M_OP_GET_ROWS == LM_GGML_OP_GET_ROWS && mirror::M_OP_CPY == LM_GGML_OP_CPY && mirror::M_OP_CONT == LM_GGML_OP_CONT && mirror::M_OP_SOFT_MAX == LM_GGML_OP_SOFT_MAX && mirror::M_OP_ROPE == LM_GGML_OP_ROPE, "op ids");
 static_assert(mirror::M_STATUS_ALLOC_FAILED == LM_GGML_STATUS_ALLOC_FAILED && mirror::M_STATUS_FAILED == LM_GGML_STATUS_FAILED &&
               mirror::M_STATUS_SUCCESS == LM_GGML_STATUS_SUCCESS && mirror::M_STATUS_ABORTED == LM_GGML_STATUS_ABORTED, "status");
 static_assert(mirror::M_DEV_CPU == LM_GGML_BACKEND_DEVICE_TYPE_CPU && mirror::M_DEV_GPU == LM_GGML_BACKEND_DEVICE_TYPE_GPU &&

@@ -312,3 +312,61 @@ def test_attention_matmul_rejects_bad_arguments(dev):
     assert call(7, 126) == ca.CHIP_EINVAL             # activation stride not a multiple of 4
     assert call(6, None) == ca.CHIP_EINVAL
     assert call(9, 0) == ca.CHIP_OK                   # no tokens
+
+
+@pytest.mark.parametrize("wt", [O.F32] + list(O.WEIGHT_TYPES))
+def test_get_rows_every_type(dev, orc, wt):
+    nc, ne01 = 1024, 53
+    rng = np.random.default_rng(wt + 3)
+    w = (rng.standard_normal((ne01, nc)) * 0.3).astype(np.float32)
+    w[0, :4] = [0.0, -0.0, 3.0, -3.0]
+    if wt == O.F32:
+        table = w
+    elif wt == O.F16:
+        table = w.astype(np.float16).view(np.uint8).reshape(ne01, -1)
+    else:
+        table = orc.quantize_weights(wt, w)
+    ids = rng.integers(0, ne01, 40).astype(np.int32)
+    ids[:3] = [0, ne01 - 1, 0]
+    got = dev.get_rows(wt, table, nc, ids)
+    assert got.tobytes() == orc.get_rows(wt, table, nc, ids).tobytes()
+    # ids outside the table leave their rows unwritten (the wrapper pre-fills with NaN)
+    bad = np.array([1, -1, ne01, 2], np.int32)
+    got = dev.get_rows(wt, table, nc, bad)
+    assert np.isnan(got[1]).all() and np.isnan(got[2]).all()
+    assert got[[0, 3]].tobytes() == orc.get_rows(wt, table, nc, bad[[0, 3]]).tobytes()
+
+
+def test_get_rows_batched_like_the_expert_weights(dev):
+    # reference llama-graph.cpp:746: the router probabilities as [1, n_expert, n_tokens] picked by ids [n_used, n_tokens]
+    import cactus_amd as ca
+    n_expert, n_tokens, n_used = 8, 5, 2
+    rng = np.random.default_rng(6)
+    probs = rng.random((n_tokens, n_expert, 1)).astype(np.float32)
+    ids = np.stack([rng.permutation(n_expert)[:n_used] for _ in range(n_tokens)]).astype(np.int32)
+    dp, di, dy = dev.to_device(probs), dev.to_device(ids), dev.alloc(n_tokens * n_used * 4)
+    dev.check(dev.lib.chip_get_rows(ca.F32, dp.ptr, 4, 4 * n_expert, 4 * n_expert * n_tokens, 1, n_expert, di.ptr, n_used, n_tokens, 1,
+                                    n_used, n_used * n_tokens, dy.ptr, 1, n_used, n_used * n_tokens, None))
+    dev.sync()
+    got = dy.download(np.float32, n_tokens * n_used).reshape(n_tokens, n_used)
+    assert np.array_equal(got, np.take_along_axis(probs[:, :, 0], ids, axis=1))
+
+
+def test_get_rows_rejects_bad_arguments(dev):
+    import cactus_amd as ca
+    d = dev.alloc(1 << 14)
+    L = dev.lib
+    ok = [ca.Q4_K, d.ptr, 144, 144 * 4, 144 * 4, 256, 4, d.ptr, 2, 1, 1, 2, 2, d.ptr + 8192, 256, 512, 512, None]
+    dev.check(L.chip_memset(d.ptr, 0, 1 << 14, None))
+    assert L.chip_get_rows(*ok) == ca.CHIP_OK
+    dev.sync()
+
+    def call(i, v):
+        a = list(ok); a[i] = v
+        return L.chip_get_rows(*a)
+    assert call(0, ca.Q8_K) == ca.CHIP_EUNSUPPORTED
+    assert call(5, 200) == ca.CHIP_EINVAL              # not whole blocks
+    assert call(1, d.ptr + 1) == ca.CHIP_EINVAL
+    assert call(7, None) == ca.CHIP_EINVAL
+    assert call(14, 100) == ca.CHIP_EINVAL             # dst row stride shorter than a row
+    assert call(8, 0) == ca.CHIP_OK

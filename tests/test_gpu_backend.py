@@ -683,3 +683,46 @@ def test_attention_block_stays_on_the_device(host, orc):
     L.lm_ggml_free(ctx)
     L.lm_ggml_free(cctx)
     L.lm_ggml_free(wctx)
+
+
+def test_get_rows_from_a_device_resident_table(host, orc):
+    """LM_GGML_OP_GET_ROWS over a quantized table in a HIP buffer (an embedding matrix kept on the device) runs on the HIP
+    backend, bit for bit the reference's dequantized rows; a table in host memory is declined."""
+    L = host.L
+    L.lm_ggml_get_rows.restype = C.c_void_p
+    L.lm_ggml_get_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    nc, ne01, n = 512, 64, 9
+    table = orc.quantize_weights(O.Q6_K, common.weights_f32(71, ne01, nc))
+    ids = np.array([3, 0, 63, 17, 17, 5, 44, 1, 2], np.int32)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    wctx = host.context(with_graph=False)
+    tt = host.tensor_2d(wctx, O.Q6_K, nc, ne01, "table")
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
+    host.set(tt, table)
+    ctx = host.context()
+    ti = L.lm_ggml_new_tensor_1d(ctx, 26, n)
+    L.lm_ggml_set_input(ti)
+    rows = L.lm_ggml_get_rows(ctx, tt, ti)
+    L.lm_ggml_set_output(rows)
+    host_table = host.tensor_2d(ctx, O.Q6_K, nc, ne01, "host_table")        # no buffer yet, not F32 / F16: stays with the CPU
+    assert L.lm_ggml_backend_dev_supports_op(dev, rows)
+    assert not L.lm_ggml_backend_dev_supports_op(dev, L.lm_ggml_get_rows(ctx, host_table, ti))
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, rows)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 64, False, True)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(ti, ids)
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    assert L.lm_ggml_backend_sched_get_tensor_backend(sched, rows) == hip
+    y = host.get(rows, np.float32, (n, nc))
+    assert y.tobytes() == orc.get_rows(O.Q6_K, table, nc, ids).tobytes()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(wbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(wctx)

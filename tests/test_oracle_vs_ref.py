@@ -214,3 +214,21 @@ def test_attention_matmuls_over_an_f16_cache(orc, ref, hd, n_head, n_head_kv, n_
     kqv = orc.mul_mat_f16_batched(vt_cache.transpose(1, 0, 2), p)["y"]
     assert kq.tobytes() == kq_ref.tobytes()
     assert kqv.tobytes() == kqv_ref.tobytes()
+
+
+@pytest.mark.parametrize("wt", [O.F32] + list(O.WEIGHT_TYPES))
+def test_get_rows_graph(orc, ref, wt):
+    nc, ne01 = 512, 37
+    rng = np.random.default_rng(wt + 1)
+    ids = rng.integers(0, ne01, 11).astype(np.int32)
+    ids[:3] = [0, ne01 - 1, 5]
+    w = (rng.standard_normal((ne01, nc)) * 0.3).astype(np.float32)
+    if wt == O.F32:
+        table = w
+    elif wt == O.F16:
+        table = w.astype(np.float16).view(np.uint8).reshape(ne01, -1)
+    else:
+        table = orc.quantize_weights(wt, w)
+    a = orc.get_rows(wt, table, nc, ids)
+    b = ref.get_rows_graph(wt, table, nc, ids, nthreads=2)
+    assert a.shape == (11, nc) and a.tobytes() == b.tobytes()
