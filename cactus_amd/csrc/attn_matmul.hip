@@ -223,7 +223,7 @@ struct GemmPlan { bool use; size_t act_stride, off_perm, off_offsets, off_tiles,
 GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
     GemmPlan p{};
     const int64_t per_head = r2 * n;
-    p.use = K % 64 == 0 && N >= 32 && per_head >= GEMM_MIN_COLS && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
+    p.use = K >= 64 && K % 8 == 0 && N >= 32 && per_head >= GEMM_MIN_COLS && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
     if (!p.use) return p;
     p.act_stride = f16_stride(K);
     p.n_tiles = ne02 * ceil_div(per_head, (int64_t)gemm_f16_moe_tile_tokens());

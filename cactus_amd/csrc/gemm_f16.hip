@@ -55,8 +55,13 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
     if (gv.tok_tile < 0) return;
     const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
     if (tok_base >= M) return;
-    const int nstages = (int)(K / (16 * F16_KG));
+    // The row-gather instantiation also takes K that is not a multiple of the 64-value stage (the attention matmul over
+    // n_kv cache positions, a multiple of 8): cells of the last stage that lie past K are zeroed on both sides.
+    constexpr bool KTAIL = GATHER;
+    const int nstages = (int)(KTAIL ? ceil_div(K, (int64_t)(16 * F16_KG)) : K / (16 * F16_KG));
     constexpr int STAGE_BYTES = 16 * F16_KG * 2;                   // bytes of one row per stage
+    static_assert(C::NT % C::CELLS == 0, "a thread's items all have the same cell index");
+    const int my_cell = tid % C::CELLS;
 
     // item = (row, cell): 8 consecutive threads copy 128 contiguous bytes of one row
     const uint8_t *wsrc[C::W_PER_T], *xsrc[C::X_PER_T];
@@ -73,10 +78,19 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
     u32x4 wq[C::W_PER_T], xq[C::X_PER_T];
 
     auto fetch = [&](int stage) {
+        const bool live = !KTAIL || (int64_t)stage * (16 * F16_KG) + 8 * my_cell < K;
+        const size_t off = live ? (size_t)stage * STAGE_BYTES : 0;                   // a dead cell re-reads stage 0 (in bounds) and is zeroed
+        const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int i = 0; i < C::W_PER_T; i++) wq[i] = *reinterpret_cast<const u32x4 *>(wsrc[i] + (size_t)stage * STAGE_BYTES);
+        for (int i = 0; i < C::W_PER_T; i++) {
+            wq[i] = *reinterpret_cast<const u32x4 *>(wsrc[i] + off);
+            if (KTAIL && !live) wq[i] = z;
+        }
 #pragma unroll
-        for (int i = 0; i < C::X_PER_T; i++) xq[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + (size_t)stage * STAGE_BYTES);
+        for (int i = 0; i < C::X_PER_T; i++) {
+            xq[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + off);
+            if (KTAIL && !live) xq[i] = z;
+        }
     };
     auto commit = [&](int buf) {
         u32x4 *A = reinterpret_cast<u32x4 *>(lds + (size_t)buf * C::STAGE + C::OFF_A);

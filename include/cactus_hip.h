@@ -197,8 +197,8 @@ CHIP_API int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t 
  * ldx2 floats (batches: query heads); y likewise, rows of N.  ne12 must be a multiple of ne02 (grouped-query broadcast,
  * the reference's r2); a fourth dimension is not taken.  K a multiple of 8; W, nb01, nb02, x 16-byte aligned, ldx1 and
  * ldx2 multiples of 4.  The workspace is optional (NULL, 0): with chip_mul_mat_f16_batched_workspace_size bytes of it,
- * 64 or more (query head, token) pairs per KV head go through the fp16 MFMA GEMM (K a multiple of 64, y's batches
- * adjacent: ldy2 == n * ldy1); without it, and for fewer pairs, dot-product kernels round the activations on the fly. */
+ * 64 or more (query head, token) pairs per KV head go through the fp16 MFMA GEMM (K >= 64, y's batches adjacent:
+ * ldy2 == n * ldy1); without it, and for fewer pairs, dot-product kernels round the activations on the fly. */
 CHIP_API size_t chip_mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne02, int64_t ne12, int64_t n);
 CHIP_API int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02,
                                       const float *x, int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y,

@@ -241,10 +241,11 @@ def attn_case(seed, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
 
 # (hd, n_head, n_head_kv, n_tokens, n_kv, kv_size): LLaMA-3-8B decode and a short prefill, multi-head attention, head sizes
 # that use 8 / 16 / 32 lanes per cache row, a GQA ratio that is no power of two, positions that are no multiple of 64
-# the last three have 64 or more (head, token) pairs per KV head: with a workspace they take the GEMM route
+# the last five have 64 or more (head, token) pairs per KV head: with a workspace they take the GEMM route, the last two
+# with K (head size 96; 104 and 1056 cache positions) that is no multiple of the GEMM's 64-value stage
 ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8, 3, 96, 128), (256, 4, 2, 2, 160, 160),
                (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128), (128, 32, 8, 130, 320, 512),
-               (64, 4, 4, 100, 192, 256)]
+               (64, 4, 4, 100, 192, 256), (96, 6, 2, 40, 104, 128), (128, 32, 8, 512, 1056, 2048)]
 
 
 @pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", ATTN_SHAPES)
