@@ -303,11 +303,13 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
         return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
 
     // 5 tokens or more: integer sums on the matrix cores, up to 16 tokens per pass over the weights
-    const int mgroup = (n >= MMV_MIN_TOKENS) ? mmv_max_tokens(type, K, N, lim) : 0;
+    // (Q4_K on a small matrix: the dot-product GEMV is still ahead at 5 and 6 tokens)
+    const int mmv_min = (type == T_Q4_K && N * K < (32LL << 20)) ? 7 : MMV_MIN_TOKENS;
+    const int mgroup = (n >= mmv_min) ? mmv_max_tokens(type, K, N, lim) : 0;
     if (mgroup > 0) {
         for (int64_t t0 = 0; t0 < n; t0 += mgroup) {
             const int nt = (int)((n - t0 < mgroup) ? n - t0 : mgroup);
-            hipError_t e = (nt >= MMV_MIN_TOKENS || nt > gemv_max_tokens(type, K, lim))
+            hipError_t e = (nt >= mmv_min || nt > gemv_max_tokens(type, K, lim))
                 ? launch_mmv(type, W, nb01, K, N, (const uint8_t *)workspace + t0 * stride, stride, nt, y + t0 * ldy, ldy, lim, st)
                 : launch_gemv(type, W, nb01, K, N, (const uint8_t *)workspace + t0 * stride, stride, nt, y + t0 * ldy, ldy, lim, st);
             if (e != hipSuccess) return (int)e;

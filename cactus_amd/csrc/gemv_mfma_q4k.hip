@@ -1,0 +1,361 @@
+// Multi-token GEMV on the matrix cores for Q4_K weights, 5..16 tokens: the Q8_0 kernel's structure (gemv_mfma.hip)
+// with the K-quant arithmetic of lm_ggml_vec_dot_q4_K_q8_K (reference ggml-cpu/ggml-cpu-quants.c:6772-7085) as driven by
+// lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449):
+//
+//   y[t][r] = sum over super-blocks b of  d[r][b] * dx[t][b] * sum_j sc[r][b][j] * isum[t][r][b][j]
+//                                       - dmin[r][b] * dx[t][b] * sum_j m[r][b][j] * bsum[t][b][j]
+//
+// with j the eight 32-value sub-blocks, isum the integer dot of the 4-bit quants with the Q8_K quants and bsum the sum of
+// the 32 activation quants (block_q8_K.bsums, two per sub-block).  Both inner sums are integers and are accumulated as
+// integers, so they are exact; the fp32 part is two fused multiply-adds per super-block and (row, token).
+//
+// One v_mfma_i32_16x16x64_i8 covers 64 values of 16 rows: the 32 bytes qs[32p .. 32p+31] of a super-block hold sub-block
+// 2p in their low nibbles and sub-block 2p+1 in their high nibbles.  Lane (x = lane % 16, g = lane / 16) of the weight
+// operand holds 16 values of row x: the low (g < 2) or high (g >= 2) nibbles of bytes 32p + 16(g & 1) ... + 15, which puts
+// sub-block 2p into k = 0..31 and sub-block 2p+1 into k = 32..63, the order of the activation quants.  The two
+// sub-blocks have different scales, so their sums are separated as in the Q8_0 kernel: with 9..16 tokens the activation
+// operand is issued twice with the other half of the lane groups zeroed; with 8 tokens or fewer rows 8..15 of the
+// operand carry the same tokens again, rows 0..7 real only in the lane groups of sub-block 2p and rows 8..15 only in
+// those of sub-block 2p+1, and one MFMA returns both.
+//
+// A wave fetches a macro tile of 16 rows x 144 bytes (one super-block per row) with row-contiguous 16-byte loads,
+// passes it through a private LDS buffer and reads header and operands back from there; the next macro tile's loads
+// are in flight meanwhile.  Bound: the weight stream (HBM).
+#include "kernels.h"
+#include "dev_common.h"
+#include "act_layout.h"
+#include <cstdlib>
+
+namespace chip {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int KQ_ROW_BYTES = BYTES_Q4_K;                        // 144 = 9 chunks of 16 bytes
+constexpr int KQ_MACRO_BYTES = 16 * KQ_ROW_BYTES;               // 2304 per wave; also holds the wave's partial sums
+constexpr int KQ_CHUNKS = KQ_MACRO_BYTES / 16;                  // 144
+
+// LDS: quant image [NT tokens][K + 16] bytes | dx image [K/256][16 tokens] float | bsum image [K/32][16 tokens] int32 |
+// 256 zero bytes | [NW waves] macro-tile buffers
+template <int NT, int NW> __host__ __device__ constexpr size_t mmv_q4k_lds_bytes(int64_t K) {
+    return (size_t)(K + 16) * NT + (size_t)(K / 256) * 64 + (size_t)(K / 32) * 64 + 256 + NW * (size_t)KQ_MACRO_BYTES;
+}
+
+template <int NT, int NW, int OCC>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
+                    size_t ws_stride, int n, float *__restrict__ y, int64_t ldy) {
+    constexpr int WGS = NW * 64;
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int np = (int)(K / 256);                                      // macro steps (super-blocks) per row
+    const uint32_t q_stride = (uint32_t)K + 16u, q_bytes = q_stride * NT;
+    const uint32_t dx_base = q_bytes, bs_base = dx_base + (uint32_t)(K / 256) * 64u;
+    const uint32_t zero_off = bs_base + (uint32_t)(K / 32) * 64u, buf_off = zero_off + 256u;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int x = lane & 15, g = lane >> 4;
+
+    // this lane's three chunks of a macro tile: chunk qi -> row qi / 9, byte 16 * (qi % 9)
+    int crow[3];
+    uint32_t coff[3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        int qi = 64 * j + lane;
+        if (qi > KQ_CHUNKS - 1) qi = KQ_CHUNKS - 1;
+        crow[j] = qi / 9;
+        coff[j] = 16u * (uint32_t)(qi % 9);
+    }
+    const bool tail_chunk = lane < KQ_CHUNKS - 128;                     // chunk 128 + lane exists
+
+    // tiles of 16 rows: a contiguous range per workgroup, in rounds of TC <= 4 tiles whose (tile, macro step) items are
+    // split evenly over the waves; a wave's share touches at most two tiles
+    const uint32_t tiles = (uint32_t)ceil_div(N, 16);
+    const uint32_t t_begin = tiles * blockIdx.x / gridDim.x, t_end = tiles * (blockIdx.x + 1) / gridDim.x;
+    const int T = (int)(t_end - t_begin);
+    const int rounds = (T + 3) / 4;
+    const int TCmax = rounds ? (T + rounds - 1) / rounds : 0;
+    struct Seg { uint32_t tile; int m0, m1; };
+    auto segment = [&](int rd, int seg) {
+        const uint32_t t0 = t_begin + (uint32_t)(rd * TCmax);
+        const int TC = min((int)(t_end - t0), TCmax);
+        const int items = TC * np;
+        const int i0 = items * wv / NW, i1 = items * (wv + 1) / NW;
+        const int k = i0 / np + seg;
+        const int lo = seg == 0 ? i0 : (k * np < i1 ? k * np : i1);
+        const int hi = (k + 1) * np < i1 ? (k + 1) * np : i1;
+        Seg r;
+        r.tile = t0 + k;
+        r.m0 = lo - k * np;
+        r.m1 = (seg == 0 || lo < i1) ? hi - k * np : r.m0;
+        return r;
+    };
+    auto macro_offsets = [&](uint32_t (&co)[3], uint32_t tile) {
+        const int last = (int)min((int64_t)15, N - 1 - (int64_t)tile * 16);
+#pragma unroll
+        for (int j = 0; j < 3; j++) co[j] = (uint32_t)min(crow[j], last) * (uint32_t)nb01 + coff[j];
+    };
+
+    // ---- prologue: activation loads, then the first macro tile's weight loads, then the LDS images ----
+    u32x4 v[3];
+    {
+        const int nchunk = (int)(K / 16), nsb = (int)(K / 256), nsub = (int)(K / 32);
+        u32x4 qv[8][2];
+        float dv[8];
+        uint32_t bv[8];
+        auto load_batch = [&](int tb) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint8_t *tokp = ws + (size_t)min(tb + i, n - 1) * ws_stride;
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int c = min(j * WGS + (int)threadIdx.x, nchunk - 1);       // unconditional, clamped
+                    qv[i][j] = *reinterpret_cast<const u32x4 *>(tokp + 16 * (size_t)c);
+                }
+                dv[i] = reinterpret_cast<const float *>(tokp + q8_K_off_d(K))[min((int)threadIdx.x, nsb - 1)];
+                bv[i] = reinterpret_cast<const uint32_t *>(tokp + q8_K_off_bsums(K))[min((int)threadIdx.x, nsub - 1)];   // two int16 bsums
+            }
+        };
+        auto store_batch = [&](int tb) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int c = j * WGS + (int)threadIdx.x;
+                    const u32x4 z = {0u, 0u, 0u, 0u};
+                    // a thread past the end of a row dumps its clamped duplicate into the idle macro-tile buffers
+                    const uint32_t dst = c < nchunk ? (uint32_t)(tb + i) * q_stride + 16u * c : buf_off + 16u * (threadIdx.x % (NW * KQ_CHUNKS));
+                    *reinterpret_cast<u32x4 *>(lds + dst) = (tb + i < n) ? qv[i][j] : z;
+                }
+                if ((int)threadIdx.x < nsb) reinterpret_cast<float *>(lds + dx_base)[threadIdx.x * 16 + tb + i] = (tb + i < n) ? dv[i] : 0.f;
+                if ((int)threadIdx.x < nsub) {
+                    const int s = (int)(int16_t)(bv[i] & 0xffffu) + (int)(int16_t)(bv[i] >> 16);
+                    reinterpret_cast<int *>(lds + bs_base)[threadIdx.x * 16 + tb + i] = (tb + i < n) ? s : 0;
+                }
+            }
+            for (int c = 2 * WGS + (int)threadIdx.x; c < nchunk; c += WGS)
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    u32x4 t = {0u, 0u, 0u, 0u};
+                    if (tb + i < n) t = *reinterpret_cast<const u32x4 *>(ws + (size_t)(tb + i) * ws_stride + 16 * (size_t)c);
+                    *reinterpret_cast<u32x4 *>(lds + (uint32_t)(tb + i) * q_stride + 16u * c) = t;
+                }
+            for (int b = WGS + (int)threadIdx.x; b < nsub; b += WGS)
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    int s = 0;
+                    if (tb + i < n) {
+                        const uint32_t p = reinterpret_cast<const uint32_t *>(ws + (size_t)(tb + i) * ws_stride + q8_K_off_bsums(K))[b];
+                        s = (int)(int16_t)(p & 0xffffu) + (int)(int16_t)(p >> 16);
+                    }
+                    reinterpret_cast<int *>(lds + bs_base)[b * 16 + tb + i] = s;
+                }
+        };
+        load_batch(0);
+        __builtin_amdgcn_sched_barrier(0);                               // activations are requested before weights
+        {
+            Seg s0 = segment(0, 0);
+            s0.tile = min(s0.tile, tiles - 1);
+            s0.m0 = max(0, min(s0.m0, np - 1));
+            uint32_t co[3];
+            macro_offsets(co, s0.tile);
+            const uint8_t *tb = W + (size_t)s0.tile * 16 * nb01 + (size_t)s0.m0 * KQ_ROW_BYTES;
+#pragma unroll
+            for (int j = 0; j < 3; j++) v[j] = *reinterpret_cast<const u32x4 *>(tb + co[j]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        store_batch(0);
+        if constexpr (NT == 16) {
+            load_batch(8);
+            store_batch(8);
+        }
+        if (threadIdx.x < 64) reinterpret_cast<uint32_t *>(lds + zero_off)[threadIdx.x] = 0u;
+    }
+    __syncthreads();
+
+    // ---- per-lane LDS addressing ----
+    // NT == 16: operand a0 is real in lane groups g < 2 (sub-block 2p), a1 in g >= 2 (sub-block 2p+1).
+    // NT == 8 : one operand; row x < 8 is token x, real in g < 2; row x >= 8 is token x - 8, real in g >= 2.
+    const int tokx = NT == 16 ? x : (x & 7);
+    const bool real0 = NT == 16 ? g < 2 : ((x < 8) == (g < 2));
+    const bool real1 = NT == 16 && g >= 2;
+    const uint32_t a_real = (uint32_t)tokx * q_stride + 16u * g;
+    const uint32_t a0_off = real0 ? a_real : zero_off, a0_step = real0 ? 256u : 0u;
+    const uint32_t a1_off = real1 ? a_real : zero_off, a1_step = real1 ? 256u : 0u;
+    // result rows 4g..4g+3 of this lane: NT == 16: tokens 4g..4g+3 of both sub-blocks;
+    // NT == 8: tokens 4(g&1)..4(g&1)+3 of sub-block 2p + (g >> 1)
+    const int par = g >> 1;                                             // NT == 8: the sub-block parity of this lane's results
+    const uint32_t tok4 = NT == 16 ? 4u * g : 4u * (g & 1);             // first of the lane's four tokens
+    uint8_t *mybuf = lds + buf_off + (uint32_t)wv * KQ_MACRO_BYTES;
+    const uint32_t hdr = (uint32_t)x * KQ_ROW_BYTES;                    // row x of the macro tile: d, dmin, scales[12], qs[128]
+    const uint32_t b_off = hdr + 16u + 16u * (g & 1);                   // + 32 * p
+    const uint32_t nib_shift = 4u * (g >> 1);
+
+    for (int rd = 0; rd < rounds; rd++) {
+        float4 part[2];
+#pragma unroll
+        for (int seg = 0; seg < 2; seg++) {
+            const Seg sg = segment(rd, seg);
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            if (sg.m0 < sg.m1) {                                         // wave-uniform
+                uint32_t co[3];
+                macro_offsets(co, sg.tile);
+                const uint8_t *tb = W + (size_t)sg.tile * 16 * nb01;
+                if (rd != 0 || seg != 0) {
+#pragma unroll
+                    for (int j = 0; j < 3; j++) v[j] = *reinterpret_cast<const u32x4 *>(tb + (size_t)sg.m0 * KQ_ROW_BYTES + co[j]);
+                }
+                u32x4 v2[3];
+                {
+                    const int mn = min(sg.m0 + 1, sg.m1 - 1);
+#pragma unroll
+                    for (int j = 0; j < 3; j++) v2[j] = *reinterpret_cast<const u32x4 *>(tb + (size_t)mn * KQ_ROW_BYTES + co[j]);
+                }
+                auto step = [&](u32x4 (&r)[3], int m, int mnext, bool live) {
+                    // registers -> LDS (the wave's LDS operations execute in order), then the same registers
+                    // receive macro tile mnext
+                    reinterpret_cast<u32x4 *>(mybuf)[lane] = r[0];
+                    reinterpret_cast<u32x4 *>(mybuf)[64 + lane] = r[1];
+                    if (tail_chunk) reinterpret_cast<u32x4 *>(mybuf)[128 + lane] = r[2];
+                    const uint8_t *nb = tb + (size_t)min(mnext, sg.m1 - 1) * KQ_ROW_BYTES;
+#pragma unroll
+                    for (int j = 0; j < 3; j++) r[j] = *reinterpret_cast<const u32x4 *>(nb + co[j]);
+                    if (!live) return;                                   // wave-uniform
+                    // header of row x: d | dmin, then the 12 scale bytes (get_scale_min_k4, ggml-quants.c)
+                    const u32x4 h = *reinterpret_cast<const u32x4 *>(mybuf + hdr);
+                    const float d = h2f(h.x), dmin = h2f(h.x >> 16);
+                    const uint32_t s0 = h.y, s1 = h.z, s2 = h.w;         // scales[0..3], [4..7], [8..11]
+                    // sub-block j < 4: sc = s0.byte[j] & 63, m = s1.byte[j] & 63;
+                    // j >= 4: sc = (s2.byte[j-4] & 15) | (s0.byte[j-4] >> 6 << 4), m = (s2.byte[j-4] >> 4) | (s1.byte[j-4] >> 6 << 4)
+                    auto sc_of = [&](int j) -> int {
+                        return j < 4 ? (int)((s0 >> (8 * j)) & 63u)
+                                     : (int)(((s2 >> (8 * (j - 4))) & 15u) | ((((s0 >> (8 * (j - 4))) >> 6) & 3u) << 4));
+                    };
+                    auto m_of = [&](int j) -> int {
+                        return j < 4 ? (int)((s1 >> (8 * j)) & 63u)
+                                     : (int)((((s2 >> (8 * (j - 4))) >> 4) & 15u) | ((((s1 >> (8 * (j - 4))) >> 6) & 3u) << 4));
+                    };
+                    const uint8_t *pa0 = lds + a0_off + (uint32_t)m * a0_step;
+                    const uint8_t *pa1 = lds + a1_off + (uint32_t)m * a1_step;
+                    const int *pbs = reinterpret_cast<const int *>(lds + bs_base) + ((uint32_t)m * 8u) * 16u + tok4;
+                    int isc[4] = {0, 0, 0, 0}, imn[4] = {0, 0, 0, 0};
+#pragma unroll
+                    for (int pi = 0; pi < 4; pi++) {
+                        const u32x4 wq = *reinterpret_cast<const u32x4 *>(mybuf + b_off + 32u * pi);
+                        const v4i b = {(int)((wq.x >> nib_shift) & 0x0f0f0f0fu), (int)((wq.y >> nib_shift) & 0x0f0f0f0fu),
+                                       (int)((wq.z >> nib_shift) & 0x0f0f0f0fu), (int)((wq.w >> nib_shift) & 0x0f0f0f0fu)};
+                        const v4i zero = {0, 0, 0, 0};
+                        const v4i a0 = *reinterpret_cast<const v4i *>(pa0 + 64 * pi);
+                        const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, zero, 0, 0, 0);
+                        if constexpr (NT == 8) {
+                            // the lane's results belong to sub-block 2 pi + par
+                            const int sc = par ? sc_of(2 * pi + 1) : sc_of(2 * pi);
+                            const int mn = par ? m_of(2 * pi + 1) : m_of(2 * pi);
+                            const v4i bs = *reinterpret_cast<const v4i *>(pbs + (2 * pi + par) * 16);
+                            isc[0] += sc * r0.x; isc[1] += sc * r0.y; isc[2] += sc * r0.z; isc[3] += sc * r0.w;
+                            imn[0] += mn * bs.x; imn[1] += mn * bs.y; imn[2] += mn * bs.z; imn[3] += mn * bs.w;
+                        } else {
+                            const v4i a1 = *reinterpret_cast<const v4i *>(pa1 + 64 * pi);
+                            const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, zero, 0, 0, 0);
+                            const int sc0 = sc_of(2 * pi), sc1 = sc_of(2 * pi + 1), mn0 = m_of(2 * pi), mn1 = m_of(2 * pi + 1);
+                            const v4i bs0 = *reinterpret_cast<const v4i *>(pbs + (2 * pi) * 16);
+                            const v4i bs1 = *reinterpret_cast<const v4i *>(pbs + (2 * pi + 1) * 16);
+                            isc[0] += sc0 * r0.x + sc1 * r1.x; isc[1] += sc0 * r0.y + sc1 * r1.y;
+                            isc[2] += sc0 * r0.z + sc1 * r1.z; isc[3] += sc0 * r0.w + sc1 * r1.w;
+                            imn[0] += mn0 * bs0.x + mn1 * bs1.x; imn[1] += mn0 * bs0.y + mn1 * bs1.y;
+                            imn[2] += mn0 * bs0.z + mn1 * bs1.z; imn[3] += mn0 * bs0.w + mn1 * bs1.w;
+                        }
+                    }
+                    const float4 dx = *reinterpret_cast<const float4 *>(lds + dx_base + ((uint32_t)m * 16u + tok4) * 4u);
+                    acc[0] = __builtin_fmaf(d * dx.x, (float)isc[0], acc[0]); acc[0] = __builtin_fmaf(-(dmin * dx.x), (float)imn[0], acc[0]);
+                    acc[1] = __builtin_fmaf(d * dx.y, (float)isc[1], acc[1]); acc[1] = __builtin_fmaf(-(dmin * dx.y), (float)imn[1], acc[1]);
+                    acc[2] = __builtin_fmaf(d * dx.z, (float)isc[2], acc[2]); acc[2] = __builtin_fmaf(-(dmin * dx.z), (float)imn[2], acc[2]);
+                    acc[3] = __builtin_fmaf(d * dx.w, (float)isc[3], acc[3]); acc[3] = __builtin_fmaf(-(dmin * dx.w), (float)imn[3], acc[3]);
+                };
+                for (int m = sg.m0; m < sg.m1; m += 2) {
+                    step(v, m, m + 2, true);
+                    step(v2, m + 1, m + 3, m + 1 < sg.m1);
+                }
+            }
+            part[seg] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        }
+        // partial sums go to the wave's own (now idle) macro-tile buffer
+        reinterpret_cast<float4 *>(mybuf)[lane] = part[0];
+        reinterpret_cast<float4 *>(mybuf)[64 + lane] = part[1];
+        __syncthreads();
+
+        // wave k adds up tile k's partial sums in wave order and stores 16 rows x n tokens
+        const uint32_t t0 = t_begin + (uint32_t)(rd * TCmax);
+        const int TC = min((int)(t_end - t0), TCmax);
+        const int items = TC * np;
+        if (wv < TC) {
+            const int k = wv;
+            float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int w = 0; w < NW; w++) {
+                const int wi0 = items * w / NW, wi1 = items * (w + 1) / NW;
+                if (wi1 <= k * np || wi0 >= (k + 1) * np || wi0 == wi1) continue;
+                const int seg = (wi0 / np == k) ? 0 : 1;
+                const float4 pv = reinterpret_cast<const float4 *>(lds + buf_off + (uint32_t)w * KQ_MACRO_BYTES)[seg * 64 + lane];
+                s.x += pv.x; s.y += pv.y; s.z += pv.z; s.w += pv.w;
+            }
+            if constexpr (NT == 8) {
+                // lanes (x, g) and (x, g + 2) hold the even and odd sub-blocks' halves of the same (row, token) sums
+                s.x += __shfl_xor(s.x, 32); s.y += __shfl_xor(s.y, 32);
+                s.z += __shfl_xor(s.z, 32); s.w += __shfl_xor(s.w, 32);
+            }
+            const int64_t row = (int64_t)(t0 + k) * 16 + x;
+            if (row < N && (NT == 16 || g < 2)) {
+                const int tk = 4 * g;
+                if (tk + 0 < n) y[(size_t)(tk + 0) * ldy + row] = s.x;
+                if (tk + 1 < n) y[(size_t)(tk + 1) * ldy + row] = s.y;
+                if (tk + 2 < n) y[(size_t)(tk + 2) * ldy + row] = s.z;
+                if (tk + 3 < n) y[(size_t)(tk + 3) * ldy + row] = s.w;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int NT, int NW, int OCC>
+hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
+                      int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    const size_t lds_bytes = mmv_q4k_lds_bytes<NT, NW>(K);
+    auto kfn = mmv_q4k_kernel<NT, NW, OCC>;
+    static LdsGrant grant;
+    if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    const int64_t tiles = ceil_div(N, 16);
+    constexpr int per_cu = OCC * 4 / NW;
+    const int64_t groups = tiles < (int64_t)cus * per_cu ? tiles : (int64_t)cus * per_cu;
+    hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(NW * 64), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                       (const uint8_t *)ws, ws_stride, n, y, ldy);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// Tokens one launch takes for this shape: 16 if the 16-token image fits in LDS, else 8, else 0 (use the dot-product GEMV).
+int mmv_q4k_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim) {
+    static const bool off = [] { const char *e = getenv("CHIP_MMV_Q4K"); return e && e[0] == '0'; }();      // tuning: dot-product GEMV instead
+    if (off || K % 256 != 0) return 0;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
+    if (N > (1 << 24) || K > (1 << 20) || K > 32 * 512) return 0;        // 32-bit tile arithmetic; two quant chunks per thread in the prologue
+    if (mmv_q4k_lds_bytes<16, 8>(K) <= (size_t)lim.max_lds_per_block) return 16;
+    if (mmv_q4k_lds_bytes<8, 8>(K) <= (size_t)lim.max_lds_per_block) return 8;
+    return 0;
+}
+
+hipError_t launch_mmv_q4k(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
+                          int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    if (n < 1 || n > 16) return hipErrorInvalidValue;
+    if (N <= 0) return hipSuccess;
+    if (n <= 8) {
+        if (mmv_q4k_lds_bytes<8, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+        return launch_cfg<8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+    }
+    if (mmv_q4k_lds_bytes<16, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+    return launch_cfg<16, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+}
+
+}  // namespace chip
