@@ -173,6 +173,38 @@ def test_mul_mat_q4_K_matrix_core_gemv(dev, orc, K, N, n):
     check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv q4_K")
 
 
+@pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (14336, 4096)])
+@pytest.mark.parametrize("n", [5, 8, 9, 16, 17, 31])
+def test_mul_mat_q4_0_matrix_core_gemv(dev, orc, K, N, n):
+    # the Q4_0 form of the matrix-core GEMV: operands 16 * (nibble - 8), scale d / 16
+    print("mmv q4_0 K", K, "N", N, "n", n, flush=True)
+    wq = orc.quantize_weights(O.Q4_0, common.weights_f32(K + N + 2, N, K))
+    x = common.activations_f32(K + n + 2, n, K)
+    x[2] = 0
+    x[3] *= 250
+    ref = orc.mul_mat(O.Q4_0, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(O.Q4_0, wq, x, want_workspace_blocks=True)
+    assert np.array_equal(blocks, ref["wdata"])
+    check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv q4_0")
+
+
+def test_matrix_core_gemv_integer_sums_are_exact(dev, orc):
+    # all scales 1 and activations that quantize to themselves: the fp32 result is the integer sum itself, so a wrong
+    # nibble plane, sign or scale factor in the operand form of the Q4_0 kernel shows as a different integer
+    K, N, n = 512, 4096, 8
+    rng = np.random.default_rng(77)
+    xi = rng.integers(-127, 128, (n, K)).astype(np.float32)
+    xi[:, 0::32] = 127.0                                                   # every 32-block's maximum: d = 1 for Q8_0
+    w4 = np.zeros((N, K // 32, 18), np.uint8)
+    w4[..., 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w4[..., 2:] = rng.integers(0, 256, (N, K // 32, 16), dtype=np.uint8)
+    w4 = w4.reshape(N, -1)
+    ref = orc.mul_mat(O.Q4_0, w4, xi)
+    got = dev.mul_mat(O.Q4_0, w4, xi)
+    assert got.tobytes() == ref["y"].tobytes()
+    assert np.array_equal(got, np.round(got))
+
+
 # ------------------------------------------------------------------------------------------ BASELINE sizes
 def test_config1_q4_0_4096(dev, orc):
     K = N = 4096
