@@ -303,7 +303,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OC
 
 // Tokens one launch takes for this shape: 16 if the 16-token image fits in LDS, else 8, else 0 (not supported).
 int mmv_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim) {
-    if (wtype == T_Q4_K) return mmv_q4k_max_tokens(K, N, lim);
+    if (wtype == T_Q4_K || wtype == T_Q5_K) return mmv_q4k_max_tokens(wtype, K, N, lim);
     if (wtype == T_Q4_0) return mmv_q4_0_max_tokens(K, N, lim);
     if (wtype != T_Q8_0 || K % 256 != 0) return 0;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
@@ -341,7 +341,7 @@ static hipError_t launch_mmv_nt(const void *W, size_t nb01, int64_t K, int64_t N
 
 hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
                       float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (wtype == T_Q4_K) return launch_mmv_q4k(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+    if (wtype == T_Q4_K || wtype == T_Q5_K) return launch_mmv_q4k(wtype, W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
     if (wtype == T_Q4_0) return launch_mmv_q4_0(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
     if (wtype != T_Q8_0 || n < 1 || n > 16) return hipErrorInvalidValue;
     if (N <= 0) return hipSuccess;

@@ -1,4 +1,4 @@
-// Multi-token GEMV on the matrix cores for Q4_K weights, 5..16 tokens: the Q8_0 kernel's structure (gemv_mfma.hip)
+// Multi-token GEMV on the matrix cores for Q4_K and Q5_K weights, 5..16 tokens: the Q8_0 kernel's structure (gemv_mfma.hip)
 // with the K-quant arithmetic of lm_ggml_vec_dot_q4_K_q8_K (reference ggml-cpu/ggml-cpu-quants.c:6772-7085) as driven by
 // lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449):
 //
@@ -32,21 +32,32 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int KQ_ROW_BYTES = BYTES_Q4_K;                        // 144 = 9 chunks of 16 bytes
-constexpr int KQ_MACRO_BYTES = 16 * KQ_ROW_BYTES;               // 2304 per wave; also holds the wave's partial sums
-constexpr int KQ_CHUNKS = KQ_MACRO_BYTES / 16;                  // 144
+// Q4_K: 144-byte super-blocks = 9 chunks of 16 bytes: d | dmin | scales[12] | qs[128].
+// Q5_K: 176 bytes = 11 chunks: d | dmin | scales[12] | qh[32] | qs[128]; bit j of qh[l] is the fifth bit of element l of
+// sub-block j, so the operand byte is nibble + 16 * bit and everything after the operand is the same as for Q4_K
+// (lm_ggml_vec_dot_q5_K_q8_K, reference ggml-cpu/ggml-cpu-quants.c:7699-8150).
+template <int WT> struct KqGeom {
+    static constexpr int ROW_BYTES = WT == T_Q5_K ? BYTES_Q5_K : BYTES_Q4_K;
+    static constexpr int CHUNKS_PER_ROW = ROW_BYTES / 16;
+    static constexpr int MACRO_BYTES = 16 * ROW_BYTES;          // per wave; also holds the wave's partial sums
+    static constexpr int CHUNKS = MACRO_BYTES / 16;             // 144 or 176: three loads per lane
+    static constexpr int QS_OFF = WT == T_Q5_K ? 48 : 16;
+    static_assert(ROW_BYTES % 16 == 0 && CHUNKS <= 192 && MACRO_BYTES >= 2048, "macro tile geometry");
+};
 
 // LDS: quant image [NT tokens][K + 16] bytes | dx image [K/256][16 tokens] float | bsum image [K/32][16 tokens] int32 |
 // 256 zero bytes | [NW waves] macro-tile buffers
-template <int NT, int NW> __host__ __device__ constexpr size_t mmv_q4k_lds_bytes(int64_t K) {
-    return (size_t)(K + 16) * NT + (size_t)(K / 256) * 64 + (size_t)(K / 32) * 64 + 256 + NW * (size_t)KQ_MACRO_BYTES;
+template <int WT, int NT, int NW> __host__ __device__ constexpr size_t mmv_q4k_lds_bytes(int64_t K) {
+    return (size_t)(K + 16) * NT + (size_t)(K / 256) * 64 + (size_t)(K / 32) * 64 + 256 + NW * (size_t)KqGeom<WT>::MACRO_BYTES;
 }
 
-template <int NT, int NW, int OCC>
+template <int WT, int NT, int NW, int OCC>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
                     size_t ws_stride, int n, float *__restrict__ y, int64_t ldy) {
     constexpr int WGS = NW * 64;
+    constexpr int KQ_ROW_BYTES = KqGeom<WT>::ROW_BYTES, KQ_MACRO_BYTES = KqGeom<WT>::MACRO_BYTES, KQ_CHUNKS = KqGeom<WT>::CHUNKS;
+    constexpr int CPR = KqGeom<WT>::CHUNKS_PER_ROW;
     extern __shared__ __align__(16) uint8_t lds[];
     const int np = (int)(K / 256);                                      // macro steps (super-blocks) per row
     const uint32_t q_stride = (uint32_t)K + 16u, q_bytes = q_stride * NT;
@@ -56,17 +67,17 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int x = lane & 15, g = lane >> 4;
 
-    // this lane's three chunks of a macro tile: chunk qi -> row qi / 9, byte 16 * (qi % 9)
+    // this lane's three chunks of a macro tile: chunk qi -> row qi / CPR, byte 16 * (qi % CPR)
     int crow[3];
     uint32_t coff[3];
 #pragma unroll
     for (int j = 0; j < 3; j++) {
         int qi = 64 * j + lane;
         if (qi > KQ_CHUNKS - 1) qi = KQ_CHUNKS - 1;
-        crow[j] = qi / 9;
-        coff[j] = 16u * (uint32_t)(qi % 9);
+        crow[j] = qi / CPR;
+        coff[j] = 16u * (uint32_t)(qi % CPR);
     }
-    const bool tail_chunk = lane < KQ_CHUNKS - 128;                     // chunk 128 + lane exists
+    const bool tail_chunk = lane < KQ_CHUNKS - 128;                     // chunk 128 + lane exists (16 or 48 lanes)
 
     // tiles of 16 rows: a contiguous range per workgroup, in rounds of TC <= 4 tiles whose (tile, macro step) items are
     // split evenly over the waves; a wave's share touches at most two tiles
@@ -188,7 +199,8 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     const uint32_t tok4 = NT == 16 ? 4u * g : 4u * (g & 1);             // first of the lane's four tokens
     uint8_t *mybuf = lds + buf_off + (uint32_t)wv * KQ_MACRO_BYTES;
     const uint32_t hdr = (uint32_t)x * KQ_ROW_BYTES;                    // row x of the macro tile: d, dmin, scales[12], qs[128]
-    const uint32_t b_off = hdr + 16u + 16u * (g & 1);                   // + 32 * p
+    const uint32_t b_off = hdr + (uint32_t)KqGeom<WT>::QS_OFF + 16u * (g & 1);     // + 32 * p
+    const uint32_t qh_off = hdr + 16u + 16u * (g & 1);                  // Q5_K: the fifth bits of the same 16 elements
     const uint32_t nib_shift = 4u * (g >> 1);
 
     for (int rd = 0; rd < rounds; rd++) {
@@ -239,11 +251,18 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
                     const uint8_t *pa1 = lds + a1_off + (uint32_t)m * a1_step;
                     const int *pbs = reinterpret_cast<const int *>(lds + bs_base) + ((uint32_t)m * 8u) * 16u + tok4;
                     int isc[4] = {0, 0, 0, 0}, imn[4] = {0, 0, 0, 0};
+                    u32x4 qh = {0u, 0u, 0u, 0u};
+                    if constexpr (WT == T_Q5_K) qh = *reinterpret_cast<const u32x4 *>(mybuf + qh_off);
 #pragma unroll
                     for (int pi = 0; pi < 4; pi++) {
                         const u32x4 wq = *reinterpret_cast<const u32x4 *>(mybuf + b_off + 32u * pi);
-                        const v4i b = {(int)((wq.x >> nib_shift) & 0x0f0f0f0fu), (int)((wq.y >> nib_shift) & 0x0f0f0f0fu),
-                                       (int)((wq.z >> nib_shift) & 0x0f0f0f0fu), (int)((wq.w >> nib_shift) & 0x0f0f0f0fu)};
+                        v4i b = {(int)((wq.x >> nib_shift) & 0x0f0f0f0fu), (int)((wq.y >> nib_shift) & 0x0f0f0f0fu),
+                                 (int)((wq.z >> nib_shift) & 0x0f0f0f0fu), (int)((wq.w >> nib_shift) & 0x0f0f0f0fu)};
+                        if constexpr (WT == T_Q5_K) {
+                            const uint32_t hb = 2u * pi + (g >> 1);                   // the sub-block = the bit of qh
+                            b.x |= (int)(((qh.x >> hb) & 0x01010101u) << 4); b.y |= (int)(((qh.y >> hb) & 0x01010101u) << 4);
+                            b.z |= (int)(((qh.z >> hb) & 0x01010101u) << 4); b.w |= (int)(((qh.w >> hb) & 0x01010101u) << 4);
+                        }
                         const v4i zero = {0, 0, 0, 0};
                         const v4i a0 = *reinterpret_cast<const v4i *>(pa0 + 64 * pi);
                         const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, zero, 0, 0, 0);
@@ -316,11 +335,11 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     }
 }
 
-template <int NT, int NW, int OCC>
+template <int WT, int NT, int NW, int OCC>
 hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
                       int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    const size_t lds_bytes = mmv_q4k_lds_bytes<NT, NW>(K);
-    auto kfn = mmv_q4k_kernel<NT, NW, OCC>;
+    const size_t lds_bytes = mmv_q4k_lds_bytes<WT, NT, NW>(K);
+    auto kfn = mmv_q4k_kernel<WT, NT, NW, OCC>;
     static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
@@ -332,30 +351,41 @@ hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const vo
     return hipGetLastError();
 }
 
-}  // namespace
-
-// Tokens one launch takes for this shape: 16 if the 16-token image fits in LDS, else 8, else 0 (use the dot-product GEMV).
-int mmv_q4k_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim) {
-    static const bool off = [] { const char *e = getenv("CHIP_MMV_Q4K"); return e && e[0] == '0'; }();      // tuning: dot-product GEMV instead
-    if (off || K % 256 != 0) return 0;
-    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
-    if (N > (1 << 24) || K > (1 << 20) || K > 32 * 512) return 0;        // 32-bit tile arithmetic; two quant chunks per thread in the prologue
-    if (mmv_q4k_lds_bytes<16, 8>(K) <= (size_t)lim.max_lds_per_block) return 16;
-    if (mmv_q4k_lds_bytes<8, 8>(K) <= (size_t)lim.max_lds_per_block) return 8;
+template <int WT> int max_tokens_typed(int64_t K, const DeviceLimits &lim) {
+    if (mmv_q4k_lds_bytes<WT, 16, 8>(K) <= (size_t)lim.max_lds_per_block) return 16;
+    if (mmv_q4k_lds_bytes<WT, 8, 8>(K) <= (size_t)lim.max_lds_per_block) return 8;
     return 0;
 }
-
-hipError_t launch_mmv_q4k(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
-                          int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (n < 1 || n > 16) return hipErrorInvalidValue;
-    if (N <= 0) return hipSuccess;
+template <int WT>
+hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
+                        int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     if (n <= 8) {
-        if (mmv_q4k_lds_bytes<8, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
-        return launch_cfg<8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+        if (mmv_q4k_lds_bytes<WT, 8, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+        return launch_cfg<WT, 8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
     }
-    if (mmv_q4k_lds_bytes<16, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
-    return launch_cfg<16, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+    if (mmv_q4k_lds_bytes<WT, 16, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+    return launch_cfg<WT, 16, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+}
+
+}  // namespace
+
+// Tokens one launch takes for this shape and type (Q4_K or Q5_K): 16 if the 16-token image fits in LDS, else 8, else 0
+// (use the dot-product GEMV).
+int mmv_q4k_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim) {
+    static const bool off = [] { const char *e = getenv("CHIP_MMV_Q4K"); return e && e[0] == '0'; }();      // tuning: dot-product GEMV instead
+    if (off || K % 256 != 0 || (wtype != T_Q4_K && wtype != T_Q5_K)) return 0;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
+    if (N > (1 << 24) || K > (1 << 20)) return 0;                        // 32-bit tile arithmetic
+    return wtype == T_Q4_K ? max_tokens_typed<T_Q4_K>(K, lim) : max_tokens_typed<T_Q5_K>(K, lim);
+}
+
+hipError_t launch_mmv_q4k(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
+                          float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    if (n < 1 || n > 16 || (wtype != T_Q4_K && wtype != T_Q5_K)) return hipErrorInvalidValue;
+    if (N <= 0) return hipSuccess;
+    return wtype == T_Q4_K ? launch_typed<T_Q4_K>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st)
+                           : launch_typed<T_Q5_K>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
 }
 
 }  // namespace chip

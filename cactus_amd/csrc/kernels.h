@@ -146,10 +146,10 @@ hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, 
 // gemv_mfma.hip: the same product for up to 16 tokens per launch with the integer sums on the matrix cores.
 // mmv_max_tokens returns 16, 8 or 0 (shape or type not covered: use launch_gemv).
 int        mmv_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim);
-// gemv_mfma_q4k.hip: the Q4_K form (activations in the split Q8_K layout); reached through the two functions above.
-int        mmv_q4k_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim);
-hipError_t launch_mmv_q4k(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
-                          int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+// gemv_mfma_q4k.hip: the Q4_K / Q5_K form (activations in the split Q8_K layout); reached through the two functions above.
+int        mmv_q4k_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim);
+hipError_t launch_mmv_q4k(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
+                          float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 // gemv_mfma_q4_0.hip: the Q4_0 form (activations in the split Q8_0 layout).
 int        mmv_q4_0_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim);
 hipError_t launch_mmv_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,

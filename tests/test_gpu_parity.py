@@ -157,20 +157,22 @@ def test_mul_mat_q8_0_matrix_core_gemv(dev, orc, K, N, n):
     check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv")
 
 
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q5_K), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (8192, 4128)])
 @pytest.mark.parametrize("n", [5, 8, 9, 15, 16])
-def test_mul_mat_q4_K_matrix_core_gemv(dev, orc, K, N, n):
-    # the Q4_K form of the matrix-core GEMV: 6-bit sub-block scales and mins applied to exact integer sums; ragged N,
-    # token counts on both sides of the 8-token image, outlier weights (large dmin), a zero row and a large row of activations
-    print("mmv q4_K K", K, "N", N, "n", n, flush=True)
-    wq = orc.quantize_weights(O.Q4_K, common.weights_f32(K + N + 1, N, K, outliers=True))
+def test_mul_mat_q4_K_q5_K_matrix_core_gemv(dev, orc, wt, K, N, n):
+    # the K-quant form of the matrix-core GEMV: 6-bit sub-block scales and mins applied to exact integer sums (Q5_K: the
+    # fifth bit from qh); ragged N, token counts on both sides of the 8-token image, outlier weights (large dmin), a
+    # zero row and a large row of activations
+    print("mmv", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
+    wq = orc.quantize_weights(wt, common.weights_f32(K + N + 1, N, K, outliers=True))
     x = common.activations_f32(K + n + 1, n, K)
     x[2] = 0
     x[3] *= 250
-    ref = orc.mul_mat(O.Q4_K, wq, x, nthreads=8, want=("wdata", "sum_abs"))
-    y, blocks = dev.mul_mat(O.Q4_K, wq, x, want_workspace_blocks=True)
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(wt, wq, x, want_workspace_blocks=True)
     assert np.array_equal(blocks, ref["wdata"])
-    check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv q4_K")
+    check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv " + O.TYPE_NAMES[wt])
 
 
 @pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (14336, 4096)])
