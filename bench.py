@@ -467,6 +467,7 @@ def bench_trace(dev, hip, st, rng):
         aws_bytes = max(L.chip_mul_mat_f16_batched_workspace_size(hd, n_kv, n_head_kv, n_head, n),
                         L.chip_mul_mat_f16_batched_workspace_size(n_kv, hd, n_head_kv, n_head, n), 256)
         aws = dev.alloc(aws_bytes)
+        rope_tab = dev.alloc(n * hd * 4)
         ck = dev.check
 
         def mm(t, wptr, N, K, src, dst):
@@ -480,9 +481,10 @@ def bench_trace(dev, hip, st, rng):
                 vc = kc + kv_size * KV * 2
                 ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))     # norm + weight: one kernel, as the backend fuses them
                 mm(*W["wq"], cur, q); mm(*W["wk"], cur, k); mm(*W["wv"], cur, v)
+                if l == 0:                                                # one cos / sin table per step, as the backend keeps it
+                    ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
                 for t_, nh in ((q, n_head), (k, n_head_kv)):
-                    ck(L.chip_rope(t_.ptr, hd, hd * nh, pos.ptr, None, hd, nh, n, hd, 2, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0,
-                                   t_.ptr, hd, hd * nh, st))
+                    ck(L.chip_rope_apply(t_.ptr, hd, hd * nh, rope_tab.ptr, hd, nh, n, hd, 2, t_.ptr, hd, hd * nh, st))
                 flat, one = A4(n * KV, 1, 1, 1), n * KV
                 ck(L.chip_cpy(k.ptr, ca.F32, flat, A4(4, 4 * one, 4 * one, 4 * one), kc + 2 * KV * (n_kv - n), ca.F16, flat,
                               A4(2, 2 * one, 2 * one, 2 * one), st))
@@ -514,10 +516,10 @@ def bench_trace(dev, hip, st, rng):
         assert hl.hipStreamEndCapture(st, C.byref(graph)) == 0
         assert hl.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
         us = time_runs(dev, hip, st, lambda: hl.hipGraphLaunch(gexec, st), 10, warm=2)
-        for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws):
+        for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws, rope_tab):
             bf.free()
         cache_bytes = NL * 2 * n_kv * KV * 2
-        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "kernels": 22 * NL + 2, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
+        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "kernels": 22 * NL + 3, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
                 "weight_and_cache_GBps": round((total + cache_bytes) / us / 1e3, 1)}
 
     res = {}

@@ -525,20 +525,11 @@ int chip_get_rows(int type, const void *src, size_t nb01, size_t nb02, size_t nb
     return hip_rc(launch_get_rows(type, a, (hipStream_t)stream));
 }
 
-int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1,
-              int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
-              float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1, int64_t ldy2, void *stream) {
-    if (ne0 < 0 || ne1 < 0 || ne2 < 0 || n_dims < 0 || n_dims > ne0 || (n_dims & 1)) return CHIP_EINVAL;
-    if (mode != 0 && mode != 2) return CHIP_EUNSUPPORTED;                   // multi-section and vision layouts
-    if (n_dims / 2 > 256) return CHIP_EUNSUPPORTED;
-    if (ne0 == 0 || ne1 == 0 || ne2 == 0) return CHIP_OK;
-    if (!x || !y || !pos || ldx1 < ne0 || ldy1 < ne0 || ne2 > 0x7fffffff) return CHIP_EINVAL;
-    if ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)pos) | ((uintptr_t)freq_factors)) & 3) return CHIP_EINVAL;
-    RopeArgs a;
-    a.ne0 = ne0; a.ne1 = ne1; a.ne2 = ne2;
-    a.ldx1 = ldx1; a.ldx2 = ldx2; a.ldy1 = ldy1; a.ldy2 = ldy2;
+// The constants of a ROPE node, computed like the reference's host code computes them (ggml-cpu/ops.cpp:5229-5232,
+// ggml.c:3749-3761).
+static void rope_constants(RopeArgs &a, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
+                           float attn_factor, float beta_fast, float beta_slow) {
     a.n_dims = n_dims; a.neox = (mode & 2) != 0;
-    // constants of the op, computed like the reference's host code computes them (ggml-cpu/ops.cpp:5229-5232, ggml.c:3749-3761)
     a.theta_scale = powf(freq_base, -2.0f / n_dims);
     a.freq_scale = freq_scale;
     a.ext_factor = ext_factor;
@@ -549,7 +540,56 @@ int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, co
     a.corr1 = (n_dims - 1) < end ? (float)(n_dims - 1) : end;
     a.mscale = attn_factor;
     if (ext_factor != 0.0f) a.mscale *= 1.0f + 0.1f * logf(1.0f / freq_scale);
-    return hip_rc(launch_rope(x, pos, freq_factors, a, y, (hipStream_t)stream));
+}
+static int rope_dims_checked(int64_t ne0, int64_t ne1, int64_t ne2, int n_dims, int mode) {
+    if (ne0 < 0 || ne1 < 0 || ne2 < 0 || n_dims <= 0 || n_dims > ne0 || (n_dims & 1)) return CHIP_EINVAL;
+    if (mode != 0 && mode != 2) return CHIP_EUNSUPPORTED;                   // multi-section and vision layouts
+    if (n_dims / 2 > 256) return CHIP_EUNSUPPORTED;
+    return CHIP_OK;
+}
+
+int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t *pos, const float *freq_factors, int64_t ne0, int64_t ne1,
+              int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
+              float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1, int64_t ldy2, void *stream) {
+    if (ne0 == 0 && n_dims == 0) return CHIP_OK;
+    if (int rc = rope_dims_checked(ne0, ne1, ne2, n_dims, mode); rc != CHIP_OK) return rc;
+    if (ne0 == 0 || ne1 == 0 || ne2 == 0) return CHIP_OK;
+    if (!x || !y || !pos || ldx1 < ne0 || ldy1 < ne0 || ne2 > 0x7fffffff) return CHIP_EINVAL;
+    if ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)pos) | ((uintptr_t)freq_factors)) & 3) return CHIP_EINVAL;
+    RopeArgs a;
+    a.ne0 = ne0; a.ne1 = ne1; a.ne2 = ne2;
+    a.ldx1 = ldx1; a.ldx2 = ldx2; a.ldy1 = ldy1; a.ldy2 = ldy2;
+    rope_constants(a, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+    return hip_rc(launch_rope(x, pos, freq_factors, a, y, nullptr, false, (hipStream_t)stream));
+}
+
+int chip_rope_table(const int32_t *pos, const float *freq_factors, int64_t ne2, int n_dims, int n_ctx_orig, float freq_base,
+                    float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, float *table,
+                    void *stream) {
+    if (int rc = rope_dims_checked(n_dims, 1, ne2, n_dims, 0); rc != CHIP_OK) return rc;
+    if (ne2 == 0) return CHIP_OK;
+    if (!pos || !table || ne2 > 0x7fffffff) return CHIP_EINVAL;
+    if ((((uintptr_t)table) | ((uintptr_t)pos) | ((uintptr_t)freq_factors)) & 3) return CHIP_EINVAL;
+    RopeArgs a;
+    a.ne0 = n_dims; a.ne1 = 1; a.ne2 = ne2;
+    a.ldx1 = a.ldx2 = a.ldy1 = a.ldy2 = 0;
+    rope_constants(a, n_dims, 0, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+    return hip_rc(launch_rope(nullptr, pos, freq_factors, a, nullptr, table, true, (hipStream_t)stream));
+}
+
+int chip_rope_apply(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1, int64_t ne2,
+                    int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, void *stream) {
+    if (ne0 == 0 && n_dims == 0) return CHIP_OK;
+    if (int rc = rope_dims_checked(ne0, ne1, ne2, n_dims, mode); rc != CHIP_OK) return rc;
+    if (ne0 == 0 || ne1 == 0 || ne2 == 0) return CHIP_OK;
+    if (!x || !y || !table || ldx1 < ne0 || ldy1 < ne0 || ne2 > 0x7fffffff) return CHIP_EINVAL;
+    if ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)table)) & 3) return CHIP_EINVAL;
+    RopeArgs a;
+    a.ne0 = ne0; a.ne1 = ne1; a.ne2 = ne2;
+    a.ldx1 = ldx1; a.ldx2 = ldx2; a.ldy1 = ldy1; a.ldy2 = ldy2;
+    a.n_dims = n_dims; a.neox = (mode & 2) != 0;
+    a.theta_scale = a.freq_scale = a.ext_factor = a.corr0 = a.corr1 = a.mscale = 0.0f;       // all in the table
+    return hip_rc(launch_rope(x, nullptr, nullptr, a, y, const_cast<float *>(table), false, (hipStream_t)stream));
 }
 
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,

@@ -23,12 +23,25 @@
 
 namespace {
 
-std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0};
+std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
 struct buffer_ctx { void *base; size_t size; };
-struct backend_ctx { void *stream; void *workspace; size_t workspace_size; };
+// The cos / sin table of the ROPE nodes of one graph_compute call: Q and K of every layer are rotated by the same
+// positions, so the first ROPE node of a call builds the table and the others apply it.  The key is only valid inside
+// the call (the position tensor keeps its address from call to call while its contents change).
+struct rope_table_key {
+    const void *pos, *ff;
+    int64_t ne2;
+    int32_t params[11];        // op_params 1..10 without the mode: n_dims, n_ctx, n_ctx_orig and the six floats
+    bool valid;
+};
+struct backend_ctx {
+    void *stream; void *workspace; size_t workspace_size;
+    float *rope_table = nullptr; size_t rope_table_bytes = 0;
+    rope_table_key rope_key = {};
+};
 
 lm_ggml_backend_buffer_type_t hip_buffer_type();
 lm_ggml_backend_dev_t hip_device();
@@ -174,6 +187,7 @@ void backend_free(lm_ggml_backend_t backend) {
     backend_ctx *c = (backend_ctx *)backend->context;
     chip_stream_synchronize(c->stream);
     chip_free(c->workspace);
+    chip_free(c->rope_table);
     chip_stream_destroy(c->stream);
     delete c;
     delete backend;
@@ -393,6 +407,36 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op) {
             const lm_ggml_tensor *pos = op->src[1], *ff = op->src[2];
             float f[6];
             std::memcpy(f, op->op_params + 5, sizeof(f));        // freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow
+            if (fusion_enabled()) {
+                // the table of this call, built by its first ROPE node (or by the first one with other parameters)
+                rope_table_key k = {pos->data, ff ? ff->data : nullptr, a->ne[2], {}, true};
+                k.params[0] = op->op_params[1];
+                std::memcpy(k.params + 1, op->op_params + 3, 8 * sizeof(int32_t));
+                const size_t need = (size_t)a->ne[2] * (size_t)op->op_params[1] * sizeof(float);
+                bool have = c->rope_key.valid && c->rope_key.pos == k.pos && c->rope_key.ff == k.ff && c->rope_key.ne2 == k.ne2 &&
+                            std::memcmp(c->rope_key.params, k.params, sizeof(k.params)) == 0;
+                if (!have) {
+                    if (need > c->rope_table_bytes) {
+                        chip_stream_synchronize(c->stream);          // earlier nodes of this call may still read the old table
+                        chip_free(c->rope_table);
+                        c->rope_table = nullptr;
+                        c->rope_table_bytes = 0;
+                        void *p = nullptr;
+                        if (chip_malloc(&p, need + need / 2) != CHIP_OK) return CHIP_ENOMEM;
+                        c->rope_table = (float *)p;
+                        c->rope_table_bytes = need + need / 2;
+                    }
+                    const int rc = chip_rope_table((const int32_t *)pos->data, ff ? (const float *)ff->data : nullptr, a->ne[2],
+                                                   op->op_params[1], op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], c->rope_table,
+                                                   c->stream);
+                    if (rc != CHIP_OK) return rc;
+                    c->rope_key = k;
+                    g_rope_tables++;
+                }
+                return chip_rope_apply((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table, a->ne[0],
+                                       a->ne[1], a->ne[2], op->op_params[1], op->op_params[2], (float *)op->data,
+                                       (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), c->stream);
+            }
             return chip_rope((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), (const int32_t *)pos->data,
                              ff ? (const float *)ff->data : nullptr, a->ne[0], a->ne[1], a->ne[2], op->op_params[1], op->op_params[2],
                              op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], (float *)op->data, (int64_t)(op->nb[1] / 4),
@@ -455,6 +499,7 @@ int try_fused_pair(backend_ctx *c, const lm_ggml_tensor *node, const lm_ggml_ten
 
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
+    c->rope_key.valid = false;                        // positions may have changed since the last call
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -584,7 +629,7 @@ void dev_props(lm_ggml_backend_dev_t dev, lm_ggml_backend_dev_props *props) {
 }
 lm_ggml_backend_t dev_init_backend(lm_ggml_backend_dev_t dev, const char *) {
     if (!device_ok()) return nullptr;
-    backend_ctx *c = new (std::nothrow) backend_ctx{nullptr, nullptr, 0};
+    backend_ctx *c = new (std::nothrow) backend_ctx{};
     if (!c) return nullptr;
     if (chip_stream_create(&c->stream) != CHIP_OK) { delete c; return nullptr; }
     lm_ggml_backend *b = new (std::nothrow) lm_ggml_backend{hip_guid(), k_backend_i, dev, c};
@@ -651,6 +696,7 @@ lm_ggml_backend_dev_t reg_get_device(lm_ggml_backend_reg_t, size_t index) { retu
 void *reg_get_proc_address(lm_ggml_backend_reg_t, const char *name) {
     if (std::strcmp(name, "lm_ggml_backend_hip_get_stats") == 0) return (void *)lm_ggml_backend_hip_get_stats;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_fused_pairs") == 0) return (void *)lm_ggml_backend_hip_get_fused_pairs;
+    if (std::strcmp(name, "lm_ggml_backend_hip_get_rope_tables") == 0) return (void *)lm_ggml_backend_hip_get_rope_tables;
     return nullptr;         // no n_threads, no extra buffer types, no split buffer type, no feature list
 }
 const lm_ggml_backend_reg_i k_reg_i = {reg_name, reg_device_count, reg_get_device, reg_get_proc_address};
@@ -711,5 +757,6 @@ void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned l
     if (uploaded_bytes) *uploaded_bytes = g_uploaded.load();
 }
 unsigned long long lm_ggml_backend_hip_get_fused_pairs(void) { return g_fused_pairs.load(); }
+unsigned long long lm_ggml_backend_hip_get_rope_tables(void) { return g_rope_tables.load(); }
 
 }  // extern "C"

@@ -218,7 +218,8 @@ struct GetRowsArgs {
     float *dst; int64_t ld1, ld2, ld3;                                         // dst strides in floats
 };
 hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st);
-hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, hipStream_t st);
+hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, float *table,
+                       bool build, hipStream_t st);
 
 // moe_group.hip: counting sort of MUL_MAT_ID's (token, slot) pairs by expert into offsets[n_as + 1] / perm[pairs].
 // tiles[0] = number of token tiles, tiles[1 + i] = expert | tile << 12 for tiles of `tile_tokens` pairs.

@@ -505,9 +505,16 @@ hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st) {
 }
 
 // ---- ROPE: one workgroup per token; the first n_dims / 2 threads build that position's cos / sin table ----
+// The table depends on the positions and the op's parameters only, and a graph applies the same one to Q and K of every
+// layer: ROPE_BUILD writes it to memory ([token][cos of the n_dims / 2 pairs | sin of the pairs], scaled by mscale) and
+// ROPE_APPLY reads it back, which leaves a kernel with no serial part.  ROPE_FULL does both in one launch.  The three give
+// the same bits.
+enum { ROPE_FULL = 0, ROPE_BUILD = 1, ROPE_APPLY = 2 };
 constexpr int ROPE_MAX_PAIRS = 256;
+template <int MODE>
 __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restrict__ x, const int32_t *__restrict__ pos,
-                                                          const float *__restrict__ freq_factors, RopeArgs a, float *__restrict__ y) {
+                                                          const float *__restrict__ freq_factors, RopeArgs a, float *__restrict__ y,
+                                                          float *__restrict__ table) {
     __shared__ float cs[ROPE_MAX_PAIRS], sn[ROPE_MAX_PAIRS];
     constexpr int PRE = 8;                                       // items per thread whose loads are issued before the table is built
     const int64_t tok = blockIdx.x;
@@ -519,11 +526,15 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
     // the operands of the first PRE * EW_THREADS items do not depend on the table: fetch them first
     float x0[PRE], x1[PRE];
     uint32_t ia[PRE], ib[PRE], jj[PRE];
+    float *tab = table + tok * a.n_dims;                         // this token's cos | sin
+    if constexpr (MODE == ROPE_APPLY) {
+        for (int p = threadIdx.x; p < half; p += EW_THREADS) { cs[p] = tab[p]; sn[p] = tab[half + p]; }
+    }
 #pragma unroll
     for (int u = 0; u < PRE; u++) {
         const uint32_t i = threadIdx.x + u * EW_THREADS;
         jj[u] = 0xffffffffu;                                     // no item
-        if (i < items) {
+        if (MODE != ROPE_BUILD && i < items) {
             const uint32_t h = i / per_head, j = i - h * per_head;
             const uint32_t base = h * (uint32_t)a.ldx1;
             jj[u] = j;
@@ -535,7 +546,7 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
             ib[u] += h * (uint32_t)a.ldy1;
         }
     }
-    if ((int)threadIdx.x < half || half > EW_THREADS) {
+    if (MODE != ROPE_APPLY && ((int)threadIdx.x < half || half > EW_THREADS)) {
         // every lane walks the same chain theta_0 = pos, theta_{k+1} = theta_k * theta_scale and keeps its own step
         float theta = (float)(int64_t)pos[tok];
         for (int p0 = 0; p0 < half; p0 += EW_THREADS) {
@@ -561,9 +572,11 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
                 sincos_rounded(th, sf, cf);
                 cs[p] = cf * a.mscale;
                 sn[p] = sf * a.mscale;
+                if constexpr (MODE == ROPE_BUILD) { tab[p] = cs[p]; tab[half + p] = sn[p]; }
             }
         }
     }
+    if constexpr (MODE == ROPE_BUILD) return;
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < PRE; u++) {
@@ -590,11 +603,16 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
         }
     }
 }
-hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, hipStream_t st) {
-    if (a.ne0 <= 0 || a.ne1 <= 0 || a.ne2 <= 0) return hipSuccess;
+// table == nullptr: one launch.  Otherwise build (x, y unused) or apply (pos, freq_factors unused) against table.
+hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, float *table,
+                       bool build, hipStream_t st) {
+    if (a.ne2 <= 0 || (!build && (a.ne0 <= 0 || a.ne1 <= 0))) return hipSuccess;
     if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff || a.ne0 * a.ne1 > 0x7fffffff) return hipErrorInvalidValue;
     if (a.ne1 * a.ldx1 > 0x7fffffff || a.ne1 * a.ldy1 > 0x7fffffff) return hipErrorInvalidValue;       // 32-bit offsets inside a token
-    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a.ne2), dim3(EW_THREADS), 0, st, x, pos, freq_factors, a, y);
+    const dim3 grid((unsigned)a.ne2), block(EW_THREADS);
+    if (!table) hipLaunchKernelGGL(rope_kernel<ROPE_FULL>, grid, block, 0, st, x, pos, freq_factors, a, y, (float *)nullptr);
+    else if (build) hipLaunchKernelGGL(rope_kernel<ROPE_BUILD>, grid, block, 0, st, x, pos, freq_factors, a, y, table);
+    else hipLaunchKernelGGL(rope_kernel<ROPE_APPLY>, grid, block, 0, st, x, pos, freq_factors, a, y, table);
     return hipGetLastError();
 }
 

@@ -241,6 +241,15 @@ CHIP_API int chip_rope(const float *x, int64_t ldx1, int64_t ldx2, const int32_t
                        int64_t ne1, int64_t ne2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                        float ext_factor, float attn_factor, float beta_fast, float beta_slow, float *y, int64_t ldy1,
                        int64_t ldy2, void *stream);
+/* chip_rope in two steps, for graphs that rotate many tensors by the same positions (Q and K of every layer): the
+ * reference rebuilds its cos / sin cache per row block (lm_ggml_rope_cache_init, ggml-cpu/ops.cpp:5104-5118); here
+ * chip_rope_table writes it once - table[token][cos of the n_dims / 2 pairs | sin of the pairs], n_dims floats per token,
+ * already scaled - and chip_rope_apply rotates with it.  Results are bit-identical to chip_rope. */
+CHIP_API int chip_rope_table(const int32_t *pos, const float *freq_factors, int64_t ne2, int n_dims, int n_ctx_orig,
+                             float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast,
+                             float beta_slow, float *table, void *stream);
+CHIP_API int chip_rope_apply(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1,
+                             int64_t ne2, int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, void *stream);
 
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,

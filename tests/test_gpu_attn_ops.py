@@ -191,6 +191,7 @@ def test_rope(dev, orc, mode, ne0, n_dims, n_head, n_tokens):
         assert y[..., n_dims:].tobytes() == x[..., n_dims:].tobytes()
         assert y[pos == 0].tobytes() == ref[pos == 0].tobytes()               # angle 0: cos 1, sin 0 exactly
         assert (y.view(np.uint32) == ref.view(np.uint32)).mean() > 0.9        # most values agree to the bit
+        assert dev.rope(x, pos, n_dims, mode, two_step=True, **kw).tobytes() == y.tobytes()   # table + apply: the same bits
 
 
 def test_rope_strided_in_place(dev, orc):

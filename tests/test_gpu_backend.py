@@ -647,7 +647,12 @@ def test_attention_block_stays_on_the_device(host, orc):
     sched = L.lm_ggml_backend_sched_new(backends, None, 2, 128, False, True)
     assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
     host.set(tx, x); host.set(tpos, pos); host.set(tmask, mask16)
+    import cactus_amd
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_rope_tables.restype = C.c_ulonglong
+    tables_before = blib.lm_ggml_backend_hip_get_rope_tables()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    assert blib.lm_ggml_backend_hip_get_rope_tables() - tables_before == 1      # Q and K share one cos / sin table
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
