@@ -301,7 +301,7 @@ def bench_extra(dev, hip, trace=True):
         A = C.c_int64 * 4
         hd, n_head, n_head_kv, kv_size = 128, 32, 8, 8192
         n_embd_kv = hd * n_head_kv
-        for n_tok, n_kv in ((1, 4096), (512, 512)):
+        for n_tok, n_kv in ((1, 4096), (512, 512), (512, 4096)):
             rows = n_head * n_tok
             kq = dev.to_device((rng.standard_normal((rows, n_kv)) * 4).astype(np.float32))
             mask = dev.to_device(np.zeros((max(n_tok, 8), n_kv), np.float16))

@@ -26,6 +26,7 @@
 #include "dev_common.h"
 #include "kernels.h"
 #include "act_layout.h"
+#include <cstdlib>
 
 namespace chip {
 
@@ -219,14 +220,18 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_tile_list_kernel(int64_t ne
 
 constexpr int64_t GEMM_MIN_COLS = 64;        // columns per KV head from which the GEMM route is taken
 
-struct GemmPlan { bool use; size_t act_stride, off_perm, off_offsets, off_tiles, bytes; int64_t n_tiles; };
+struct GemmPlan { bool use; size_t act_stride, off_perm, off_offsets, off_tiles, bytes; int64_t n_tiles; int tile; };
 GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
     GemmPlan p{};
     const int64_t per_head = r2 * n;
     p.use = K >= 64 && K % 8 == 0 && N >= 32 && per_head >= GEMM_MIN_COLS && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
     if (!p.use) return p;
     p.act_stride = f16_stride(K);
-    p.n_tiles = ne02 * ceil_div(per_head, (int64_t)gemm_f16_moe_tile_tokens());
+    // 128 x 128 tiles once they still give every CU four workgroups, else 64 x 64 (CHIP_ATTN_TILE forces one, for tuning)
+    static const int forced = [] { const char *e = getenv("CHIP_ATTN_TILE"); return e ? atoi(e) : 0; }();
+    p.tile = (N >= 128 && per_head >= 128 && ne02 * ceil_div(per_head, (int64_t)128) * ceil_div(N, (int64_t)128) >= 1024) ? 128 : 64;
+    if (forced == 64 || forced == 128) p.tile = forced;
+    p.n_tiles = ne02 * ceil_div(per_head, (int64_t)p.tile);
     if (p.n_tiles > 65535) { p.use = false; return p; }                  // one grid row per list entry
     p.off_perm = align128((size_t)(ne02 * per_head) * p.act_stride);
     p.off_offsets = p.off_perm + align128((size_t)(ne02 * per_head) * 4);
@@ -257,11 +262,10 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
         const int64_t chunks = K / 8, per = chunks >= AM_THREADS ? 1 : AM_THREADS / chunks;
         hipLaunchKernelGGL(mm_f16_round_rows_kernel, dim3((unsigned)ceil_div(n, per), (unsigned)(ne02 * r2)), dim3(AM_THREADS), 0, st, x,
                            ldx1, ldx2, n, K, ws, plan.act_stride);
-        hipLaunchKernelGGL(mm_f16_tile_list_kernel, dim3(64), dim3(AM_THREADS), 0, st, ne02, r2 * n, gemm_f16_moe_tile_tokens(), perm,
-                           offsets, tiles);
+        hipLaunchKernelGGL(mm_f16_tile_list_kernel, dim3(64), dim3(AM_THREADS), 0, st, ne02, r2 * n, plan.tile, perm, offsets, tiles);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
         const RowGather rg{perm, offsets, tiles, 1, 1, nb02};
-        return launch_gemm_f16(W, nb01, K, N, ws, plan.act_stride, ne02 * r2 * n, y, ldy1, lim, st, &rg, plan.n_tiles);
+        return launch_gemm_f16(W, nb01, K, N, ws, plan.act_stride, ne02 * r2 * n, y, ldy1, lim, st, &rg, plan.n_tiles, plan.tile);
     }
     const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;

@@ -183,12 +183,16 @@ static hipError_t launch_f16(const void *W, size_t nb01, int64_t K, int64_t N, c
 int gemm_f16_moe_tile_tokens() { return F16Cfg<1, 1, 2, 2>::BN; }      // the 64 x 64 shape serves the expert groups
 
 hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as) {
+                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as,
+                           int gather_tile) {
     if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
     const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
+    if (rg.perm) {                                                                   // row groups: the tile list was built for 64 or 128 tokens
+        if (gather_tile == 128) return launch_f16<2, 2, 2, 2, 2, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        if (gather_tile != 64) return hipErrorInvalidValue;
         return launch_f16<1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+    }
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_F16_CFG");
     const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);

@@ -168,7 +168,7 @@ hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, i
 bool       gemm_f16_supported(int64_t K, int64_t N, int64_t n);
 hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t n,
                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rg = nullptr,
-                           int64_t n_as = 1);
+                           int64_t n_as = 1, int gather_tile = 64);       // gather_tile: tokens per list entry, 64 or 128
 
 // gemm_kquant.hip: int8-MFMA prefill GEMM over Q4_K / Q5_K / Q6_K weights, activations in the split Q8_K workspace
 // layout; the integer sub-block scales ride in the MFMA operand.
