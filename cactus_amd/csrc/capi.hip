@@ -304,7 +304,9 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
 
     // 5 tokens or more: integer sums on the matrix cores, up to 16 tokens per pass over the weights
     // (4-bit weights on a small matrix: the dot-product GEMV is still ahead up to 6 or 7 tokens)
-    const int mmv_min = ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7) : MMV_MIN_TOKENS;
+    // (and Q4_K rows so wide that the kernel runs with six waves: from 7 tokens)
+    const int mmv_min = ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7)
+                        : (type == T_Q4_K && K > 13312) ? 7 : MMV_MIN_TOKENS;
     const int mgroup = (n >= mmv_min) ? mmv_max_tokens(type, K, N, lim) : 0;
     if (mgroup > 0) {
         for (int64_t t0 = 0; t0 < n; t0 += mgroup) {

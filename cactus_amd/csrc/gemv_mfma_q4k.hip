@@ -351,17 +351,22 @@ hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const vo
     return hipGetLastError();
 }
 
+// Eight waves per workgroup; six when that is what makes the 8-token image of a wide row fit (K = 14336).
 template <int WT> int max_tokens_typed(int64_t K, const DeviceLimits &lim) {
     if (mmv_q4k_lds_bytes<WT, 16, 8>(K) <= (size_t)lim.max_lds_per_block) return 16;
     if (mmv_q4k_lds_bytes<WT, 8, 8>(K) <= (size_t)lim.max_lds_per_block) return 8;
+    if (mmv_q4k_lds_bytes<WT, 8, 6>(K) <= (size_t)lim.max_lds_per_block) return 8;
     return 0;
 }
 template <int WT>
 hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
                         int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     if (n <= 8) {
-        if (mmv_q4k_lds_bytes<WT, 8, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
-        return launch_cfg<WT, 8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+        if (mmv_q4k_lds_bytes<WT, 8, 8>(K) <= (size_t)lim.max_lds_per_block)
+            return launch_cfg<WT, 8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+        if (mmv_q4k_lds_bytes<WT, 8, 6>(K) <= (size_t)lim.max_lds_per_block)
+            return launch_cfg<WT, 8, 6, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+        return hipErrorInvalidValue;
     }
     if (mmv_q4k_lds_bytes<WT, 16, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     return launch_cfg<WT, 16, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);

@@ -158,7 +158,7 @@ def test_mul_mat_q8_0_matrix_core_gemv(dev, orc, K, N, n):
 
 
 @pytest.mark.parametrize("wt", (O.Q4_K, O.Q5_K), ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (8192, 4128)])
+@pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (8192, 4128), (14336, 4096)])
 @pytest.mark.parametrize("n", [5, 8, 9, 15, 16])
 def test_mul_mat_q4_K_q5_K_matrix_core_gemv(dev, orc, wt, K, N, n):
     # the K-quant form of the matrix-core GEMV: 6-bit sub-block scales and mins applied to exact integer sums (Q5_K: the
