@@ -536,6 +536,14 @@ def test_attention_side_nodes_run_on_the_device(host, orc):
     assert y_out.tobytes() == np.ascontiguousarray(kqv_in.transpose(1, 0, 2)).tobytes()
     for t in (q, k, sm, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
+    # the next step: the same graph and the same tensors at the same addresses, other positions - the cos / sin table of
+    # the previous call must not be used again
+    pos2 = pos + 1000
+    host.set(tpos, pos2)
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    y_q2 = host.get(q, np.float32, (n_tokens, n_head, hd))
+    assert (np.abs(y_q2 - orc.rope(q3, pos2, hd, 2)) <= np.concatenate([tol, tol], -1)).all()
+    assert not np.array_equal(y_q2, y_q)
     L.lm_ggml_backend_sched_free(sched)
     L.lm_ggml_backend_buffer_free(cbuf)
     L.lm_ggml_backend_free(hip)
