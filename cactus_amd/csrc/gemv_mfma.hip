@@ -305,6 +305,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OC
 int mmv_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim) {
     if (wtype == T_Q4_K || wtype == T_Q5_K) return mmv_q4k_max_tokens(wtype, K, N, lim);
     if (wtype == T_Q4_0) return mmv_q4_0_max_tokens(K, N, lim);
+    if (wtype == T_Q6_K) return mmv_q6k_max_tokens(K, N, lim);
     if (wtype != T_Q8_0 || K % 256 != 0) return 0;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
@@ -343,6 +344,7 @@ hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t 
                       float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
     if (wtype == T_Q4_K || wtype == T_Q5_K) return launch_mmv_q4k(wtype, W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
     if (wtype == T_Q4_0) return launch_mmv_q4_0(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+    if (wtype == T_Q6_K) return launch_mmv_q6k(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
     if (wtype != T_Q8_0 || n < 1 || n > 16) return hipErrorInvalidValue;
     if (N <= 0) return hipSuccess;
     if (n <= 8) return launch_mmv_nt<8>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);

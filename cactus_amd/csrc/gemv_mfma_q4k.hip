@@ -271,18 +271,19 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
                             const int sc = par ? sc_of(2 * pi + 1) : sc_of(2 * pi);
                             const int mn = par ? m_of(2 * pi + 1) : m_of(2 * pi);
                             const v4i bs = *reinterpret_cast<const v4i *>(pbs + (2 * pi + par) * 16);
-                            isc[0] += sc * r0.x; isc[1] += sc * r0.y; isc[2] += sc * r0.z; isc[3] += sc * r0.w;
-                            imn[0] += mn * bs.x; imn[1] += mn * bs.y; imn[2] += mn * bs.z; imn[3] += mn * bs.w;
+                            // 24-bit multiplies (full rate): scales and mins < 2^6, sums < 2^17
+                            isc[0] += __mul24(sc, r0.x); isc[1] += __mul24(sc, r0.y); isc[2] += __mul24(sc, r0.z); isc[3] += __mul24(sc, r0.w);
+                            imn[0] += __mul24(mn, bs.x); imn[1] += __mul24(mn, bs.y); imn[2] += __mul24(mn, bs.z); imn[3] += __mul24(mn, bs.w);
                         } else {
                             const v4i a1 = *reinterpret_cast<const v4i *>(pa1 + 64 * pi);
                             const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, zero, 0, 0, 0);
                             const int sc0 = sc_of(2 * pi), sc1 = sc_of(2 * pi + 1), mn0 = m_of(2 * pi), mn1 = m_of(2 * pi + 1);
                             const v4i bs0 = *reinterpret_cast<const v4i *>(pbs + (2 * pi) * 16);
                             const v4i bs1 = *reinterpret_cast<const v4i *>(pbs + (2 * pi + 1) * 16);
-                            isc[0] += sc0 * r0.x + sc1 * r1.x; isc[1] += sc0 * r0.y + sc1 * r1.y;
-                            isc[2] += sc0 * r0.z + sc1 * r1.z; isc[3] += sc0 * r0.w + sc1 * r1.w;
-                            imn[0] += mn0 * bs0.x + mn1 * bs1.x; imn[1] += mn0 * bs0.y + mn1 * bs1.y;
-                            imn[2] += mn0 * bs0.z + mn1 * bs1.z; imn[3] += mn0 * bs0.w + mn1 * bs1.w;
+                            isc[0] += __mul24(sc0, r0.x) + __mul24(sc1, r1.x); isc[1] += __mul24(sc0, r0.y) + __mul24(sc1, r1.y);
+                            isc[2] += __mul24(sc0, r0.z) + __mul24(sc1, r1.z); isc[3] += __mul24(sc0, r0.w) + __mul24(sc1, r1.w);
+                            imn[0] += __mul24(mn0, bs0.x) + __mul24(mn1, bs1.x); imn[1] += __mul24(mn0, bs0.y) + __mul24(mn1, bs1.y);
+                            imn[2] += __mul24(mn0, bs0.z) + __mul24(mn1, bs1.z); imn[3] += __mul24(mn0, bs0.w) + __mul24(mn1, bs1.w);
                         }
                     }
                     const float4 dx = *reinterpret_cast<const float4 *>(lds + dx_base + ((uint32_t)m * 16u + tok4) * 4u);

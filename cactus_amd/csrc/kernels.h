@@ -154,6 +154,10 @@ hipError_t launch_mmv_q4k(int wtype, const void *W, size_t nb01, int64_t K, int6
 int        mmv_q4_0_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim);
 hipError_t launch_mmv_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
                            int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+// gemv_mfma_q6k.hip: the Q6_K form (8 tokens per launch; activations in the split Q8_K layout).
+int        mmv_q6k_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim);
+hipError_t launch_mmv_q6k(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
+                          int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                       int n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
 

@@ -8,8 +8,17 @@ import os
 import numpy as np
 import pytest
 
+import functools
+
 import common
 import oracle as O
+
+
+@functools.lru_cache(maxsize=12)
+def quantized_weights(wt, seed, N, K, outliers=False):
+    """Seeded weights quantized by the oracle; kept for the other token counts of the same shape (the quantizer search
+    of a 4099 x 11008 matrix costs seconds of CPU)."""
+    return O.Oracle().quantize_weights(wt, common.weights_f32(seed, N, K, outliers=outliers))
 
 pytestmark = pytest.mark.gpu
 
@@ -147,7 +156,7 @@ def test_mul_mat_q8_0_matrix_core_gemv(dev, orc, K, N, n):
     # enough 16-row tiles for every CU and 5+ tokens: the integer sums come from v_mfma_i32_16x16x64_i8;
     # ragged N (last tile partly outside), token counts on both sides of the 8- and 16-token images
     print("mmv q8_0 K", K, "N", N, "n", n, flush=True)
-    wq = orc.quantize_weights(O.Q8_0, common.weights_f32(K + N, N, K))
+    wq = quantized_weights(O.Q8_0, K + N, N, K)
     x = common.activations_f32(K + n, n, K)
     x[2] = 0
     x[3] *= 250
@@ -165,7 +174,7 @@ def test_mul_mat_q4_K_q5_K_matrix_core_gemv(dev, orc, wt, K, N, n):
     # fifth bit from qh); ragged N, token counts on both sides of the 8-token image, outlier weights (large dmin), a
     # zero row and a large row of activations
     print("mmv", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
-    wq = orc.quantize_weights(wt, common.weights_f32(K + N + 1, N, K, outliers=True))
+    wq = quantized_weights(wt, K + N + 1, N, K, True)
     x = common.activations_f32(K + n + 1, n, K)
     x[2] = 0
     x[3] *= 250
@@ -180,7 +189,7 @@ def test_mul_mat_q4_K_q5_K_matrix_core_gemv(dev, orc, wt, K, N, n):
 def test_mul_mat_q4_0_matrix_core_gemv(dev, orc, K, N, n):
     # the Q4_0 form of the matrix-core GEMV: operands 16 * (nibble - 8), scale d / 16
     print("mmv q4_0 K", K, "N", N, "n", n, flush=True)
-    wq = orc.quantize_weights(O.Q4_0, common.weights_f32(K + N + 2, N, K))
+    wq = quantized_weights(O.Q4_0, K + N + 2, N, K)
     x = common.activations_f32(K + n + 2, n, K)
     x[2] = 0
     x[3] *= 250
@@ -188,6 +197,22 @@ def test_mul_mat_q4_0_matrix_core_gemv(dev, orc, K, N, n):
     y, blocks = dev.mul_mat(O.Q4_0, wq, x, want_workspace_blocks=True)
     assert np.array_equal(blocks, ref["wdata"])
     check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv q4_0")
+
+
+@pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (14336, 4096)])
+@pytest.mark.parametrize("n", [5, 8, 9, 16, 21])
+def test_mul_mat_q6_K_matrix_core_gemv(dev, orc, K, N, n):
+    # the Q6_K form: unsigned 6-bit operands, int8 sub-block scales, the -32 taken out through the activation block sums;
+    # rows that are only 2-byte aligned (210-byte super-blocks), ragged N, several launches of 8 tokens
+    print("mmv q6_K K", K, "N", N, "n", n, flush=True)
+    wq = quantized_weights(O.Q6_K, K + N + 3, N, K)
+    x = common.activations_f32(K + n + 3, n, K)
+    x[2] = 0
+    x[3] *= 250
+    ref = orc.mul_mat(O.Q6_K, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(O.Q6_K, wq, x, want_workspace_blocks=True)
+    assert np.array_equal(blocks, ref["wdata"])
+    check_outputs(y, ref["y"], ref["sum_abs"], "matrix-core gemv q6_K")
 
 
 def test_matrix_core_gemv_integer_sums_are_exact(dev, orc):
