@@ -215,6 +215,9 @@ def bench_extra(dev, hip, trace=True):
 
     gemv_case("config1_q4_0_4096x4096_n1", ca.Q4_0, 4096, 4096, 1)
     gemv_case("config3_q4_K_14336x4096_n1", ca.Q4_K, 14336, 4096, 1)
+    # 8 tokens (a small serving batch): the matrix-core GEMV of each weight type that has one, the dot-product GEMV otherwise
+    for wt in (ca.Q8_0, ca.Q4_0, ca.Q4_K, ca.Q5_K, ca.Q6_K):
+        gemv_case("batch8_%s_14336x4096" % ca.TYPE_NAMES[wt], wt, 14336, 4096, 8, iters=100)
 
     # config 4: prefill GEMM on int8 MFMA (Q4_0 is the configuration BASELINE names; the other weight types run the
     # same shapes through their own GEMM kernels: block-32 types, K-quants with digit-plane operands, F16 on fp16 MFMA)
