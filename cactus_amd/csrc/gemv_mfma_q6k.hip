@@ -199,14 +199,10 @@ void mmv_q6k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
                         }
                     }
                     const float4 dx = *reinterpret_cast<const float4 *>(lds + dx_base + ((uint32_t)m * NT + tok4) * 4u);
-#ifdef Q6_DEBUG
-                    acc[0] += (float)isc[0]; acc[1] += (float)ibs[0]; acc[2] += d; acc[3] += dx.x;
-#else
                     acc[0] = __builtin_fmaf(d * dx.x, (float)(isc[0] - 32 * ibs[0]), acc[0]);
                     acc[1] = __builtin_fmaf(d * dx.y, (float)(isc[1] - 32 * ibs[1]), acc[1]);
                     acc[2] = __builtin_fmaf(d * dx.z, (float)(isc[2] - 32 * ibs[2]), acc[2]);
                     acc[3] = __builtin_fmaf(d * dx.w, (float)(isc[3] - 32 * ibs[3]), acc[3]);
-#endif
                 };
                 for (int m = sg.m0; m < sg.m1; m += 2) {
                     step(v, m, m + 2, true);
