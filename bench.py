@@ -482,7 +482,8 @@ def bench_trace(dev, hip, st, rng):
                 W = {name: (t, base + o, N, K) for (name, t, N, K, _), o in zip(layer, first)}
                 kc = caches.ptr + (2 * l) * kv_size * KV * 2
                 vc = kc + kv_size * KV * 2
-                ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))     # norm + weight: one kernel, as the backend fuses them
+                if l == 0:
+                    ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))  # norm + weight: one kernel, as the backend fuses them
                 mm(*W["wq"], cur, q); mm(*W["wk"], cur, k); mm(*W["wv"], cur, v)
                 if l == 0:                                                # one cos / sin table per step, as the backend keeps it
                     ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
@@ -501,14 +502,14 @@ def bench_trace(dev, hip, st, rng):
                 ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
                               A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
                 mm(*W["wo"], merged, att)
-                ck(L.chip_add(att.ptr, H, resid.ptr, H, n, n, H, resid.ptr, H, st))
-                ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))     # norm + weight: one kernel, as the backend fuses them
+                # residual + norm + weight: one kernel, as the backend fuses the three nodes
+                ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
                 mm(*W["up"], cur, up); mm(*W["gate"], cur, gate)
                 ck(L.chip_silu(gate.ptr, FF, n, FF, gate.ptr, FF, st))
                 ck(L.chip_mul(gate.ptr, FF, up.ptr, FF, n, n, FF, gate.ptr, FF, st))
                 mm(*W["down"], gate, att)
-                ck(L.chip_add(att.ptr, H, resid.ptr, H, n, n, H, resid.ptr, H, st))
-            ck(L.chip_rms_norm(resid.ptr, H, n, H, 1e-5, cur.ptr, H, st))
+                # the layer's second residual with the next layer's (or the final) norm
+                ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
             ck(L.chip_mul_mat(ca.Q6_K, arena.ptr + head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
 
         step()
@@ -522,7 +523,7 @@ def bench_trace(dev, hip, st, rng):
         for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws, rope_tab):
             bf.free()
         cache_bytes = NL * 2 * n_kv * KV * 2
-        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "kernels": 22 * NL + 3, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
+        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "kernels": 20 * NL + 3, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
                 "weight_and_cache_GBps": round((total + cache_bytes) / us / 1e3, 1)}
 
     res = {}

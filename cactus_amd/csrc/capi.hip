@@ -444,6 +444,15 @@ int chip_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t ne0, float
     if (y_norm && !rows_ok(y_norm, ld_norm, ne0)) return CHIP_EINVAL;
     return hip_rc(launch_rms_norm_mul(x, ldx, n, ne0, eps, w, y_norm, ld_norm, y, ldy, (hipStream_t)stream));
 }
+int chip_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n, int64_t ne0,
+                          float eps, const float *w, float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0 || !(eps >= 0.0f)) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!rows_ok(a, lda, ne0) || !rows_ok(b, ldb, ne0) || !rows_ok(sum, ld_sum, ne0) || !rows_ok(y, ldy, ne0) || n > 0x7fffffff ||
+        (w && (((uintptr_t)w) & 3) != 0) || (const float *)y == sum)
+        return CHIP_EINVAL;
+    return hip_rc(launch_add_rms_norm_mul(a, lda, b, ldb, sum, ld_sum, n, ne0, eps, w, nullptr, 0, y, ldy, (hipStream_t)stream));
+}
 int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream) {
     if (n < 0 || ne0 < 0) return CHIP_EINVAL;
     if (n == 0 || ne0 == 0) return CHIP_OK;

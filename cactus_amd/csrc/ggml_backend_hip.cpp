@@ -497,12 +497,70 @@ int try_fused_pair(backend_ctx *c, const lm_ggml_tensor *node, const lm_ggml_ten
     return CHIP_OK;
 }
 
+// Row blocks [p, p + rows * ld) of two tensors: the same block, or no element in common.
+bool same_or_disjoint(const void *p, int64_t ldp, const void *q, int64_t ldq, int64_t rows, int64_t ne0) {
+    if (p == q) return ldp == ldq;
+    const uintptr_t a = (uintptr_t)p, b = (uintptr_t)q;
+    const uintptr_t ea = a + (uintptr_t)(((rows - 1) * ldp + ne0) * 4), eb = b + (uintptr_t)(((rows - 1) * ldq + ne0) * 4);
+    return ea <= b || eb <= a;
+}
+
+// A residual ADD directly followed by the RMS_NORM of its result (and that, as above, by the MUL with the norm weight):
+// the sum is still written, since the next residual reads it, but the norm reads it back in the same kernel. The
+// allocator may have placed any of the outputs over a dead operand, so every output block is the same block as, or
+// apart from, every block read. Sets used to the number of nodes run (0: not this pattern).
+int try_fused_add_norm(backend_ctx *c, const lm_ggml_cgraph *g, int i, int &used) {
+    used = 0;
+    const lm_ggml_tensor *add = g->nodes[i];
+    const lm_ggml_tensor *norm = i + 1 < g->n_nodes ? g->nodes[i + 1] : nullptr;
+    if (!norm || norm->op != LM_GGML_OP_RMS_NORM || norm->src[0] != add || !elementwise_shape_ok(norm)) return CHIP_OK;
+    const lm_ggml_tensor *a = add->src[0], *b = add->src[1];
+    if (!same_shape(a, b)) return CHIP_OK;
+    const lm_ggml_tensor *mul = i + 2 < g->n_nodes ? g->nodes[i + 2] : nullptr, *wt = nullptr;
+    if (mul && mul->op == LM_GGML_OP_MUL && mul->data == norm->data && elementwise_shape_ok(mul) && same_shape(mul, norm)) {
+        wt = mul->src[0] == norm ? mul->src[1] : (mul->src[1] == norm ? mul->src[0] : nullptr);
+        int64_t rw, ldw;
+        if (!wt || wt == norm || !as_rows(wt, rw, ldw) || rw != 1) wt = nullptr;
+    }
+    const lm_ggml_tensor *out = wt ? mul : norm;
+    int64_t rows, lda, ldb, lds, ldy;
+    if (!as_rows(a, rows, lda) || !as_rows(b, rows, ldb) || !as_rows(add, rows, lds) || !as_rows(out, rows, ldy)) return CHIP_OK;
+    const int64_t ne0 = a->ne[0];
+    if (rows == 0 || ne0 == 0) return CHIP_OK;
+    if (!same_or_disjoint(add->data, lds, a->data, lda, rows, ne0) || !same_or_disjoint(add->data, lds, b->data, ldb, rows, ne0) ||
+        !same_or_disjoint(out->data, ldy, a->data, lda, rows, ne0) || !same_or_disjoint(out->data, ldy, b->data, ldb, rows, ne0) ||
+        out->data == add->data || !same_or_disjoint(out->data, ldy, add->data, lds, rows, ne0))
+        return CHIP_OK;
+    if (wt && !same_or_disjoint(out->data, ldy, wt->data, ne0, 1, ne0)) return CHIP_OK;
+    if (wt && out->data == wt->data) return CHIP_OK;
+    float eps;
+    std::memcpy(&eps, norm->op_params, sizeof(float));
+    used = wt ? 3 : 2;
+    return chip_add_rms_norm_mul((const float *)a->data, lda, (const float *)b->data, ldb, (float *)add->data, lds, rows, ne0, eps,
+                                 wt ? (const float *)wt->data : nullptr, (float *)out->data, ldy, c->stream);
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        if (node->op == LM_GGML_OP_ADD && elementwise_shape_ok(node) && fusion_enabled()) {
+            int used = 0;
+            const int rc = try_fused_add_norm(c, cgraph, i, used);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (ADD fused with the norm that follows) failed: %s\n", __func__, node->name,
+                        chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            if (used) {
+                g_elementwise_nodes += used;
+                g_fused_pairs += used - 1;
+                i += used - 1;
+                continue;
+            }
+        }
         if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_UNARY) && elementwise_shape_ok(node) && fusion_enabled()) {
             bool fused = false;
             const int rc = try_fused_pair(c, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused);

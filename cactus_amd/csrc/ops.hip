@@ -57,16 +57,41 @@ __device__ __forceinline__ float silu1(float x) { return x / (1.0f + v_expf_lane
 // ---- RMS_NORM: one workgroup per row ----
 // With w, the row is also multiplied by the weight row w (the MUL node that follows a norm): y = (x * scale) * w, two
 // roundings as in the two separate ops; yn (may be NULL) then receives the norm itself.
-__global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *__restrict__ x, int64_t ldx, int64_t ne0, float eps,
+// With ADD, the row normalised is a + b (the residual ADD node in front of a norm): the sum is stored to xs, which may be a
+// or b themselves (every thread reads an element of a and b before it writes that element of xs, and reads back only its
+// own elements), and the norm then runs over the stored sum.
+template <bool ADD>
+__global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, int64_t ldx, int64_t ne0, float eps,
                                                               float *__restrict__ y, int64_t ldy, const float *__restrict__ w,
-                                                              float *__restrict__ yn, int64_t ldyn) {
+                                                              float *__restrict__ yn, int64_t ldyn, const float *b, int64_t ldb,
+                                                              float *xs, int64_t ldxs) {
     __shared__ double part[EW_THREADS / 64];
     const float *xr = x + (size_t)blockIdx.x * ldx;
     float *yr = y + (size_t)blockIdx.x * ldy;
     const int tid = threadIdx.x;
-    const bool vec = ((ne0 | ldx | ldy) & 3) == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
+    bool vec = ((ne0 | ldx | ldy) & 3) == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
+    if (ADD) vec = vec && ((ldb | ldxs) & 3) == 0 && ((((uintptr_t)b) | ((uintptr_t)xs)) & 15) == 0;
     double sum = 0.0;
-    if (vec) {
+    if (ADD) {
+        const float *br = b + (size_t)blockIdx.x * ldb;
+        float *sr = xs + (size_t)blockIdx.x * ldxs;
+        if (vec) {
+            for (int64_t i = 4 * tid; i < ne0; i += 4 * EW_THREADS) {
+                float4 v = *reinterpret_cast<const float4 *>(xr + i);
+                const float4 u = *reinterpret_cast<const float4 *>(br + i);
+                v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+                *reinterpret_cast<float4 *>(sr + i) = v;
+                sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+            }
+        } else {
+            for (int64_t i = tid; i < ne0; i += EW_THREADS) {
+                const float v = xr[i] + br[i];
+                sr[i] = v;
+                sum += (double)(v * v);
+            }
+        }
+        xr = sr;
+    } else if (vec) {
         for (int64_t i = 4 * tid; i < ne0; i += 4 * EW_THREADS) {
             const float4 v = *reinterpret_cast<const float4 *>(xr + i);
             sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
@@ -620,8 +645,9 @@ hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, 
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     for (int64_t r0 = 0; r0 < n; r0 += 1 << 30) {
         const int64_t rows = n - r0 < (1 << 30) ? n - r0 : (1 << 30);
-        hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(EW_THREADS), 0, st, x + r0 * ldx, ldx, ne0, eps,
-                           y + r0 * ldy, ldy, (const float *)nullptr, (float *)nullptr, (int64_t)0);
+        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)rows), dim3(EW_THREADS), 0, st, x + r0 * ldx, ldx, ne0, eps,
+                           y + r0 * ldy, ldy, (const float *)nullptr, (float *)nullptr, (int64_t)0, (const float *)nullptr,
+                           (int64_t)0, (float *)nullptr, (int64_t)0);
     }
     return hipGetLastError();
 }
@@ -629,7 +655,17 @@ hipError_t launch_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t n
                                float *y, int64_t ldy, hipStream_t st) {
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     if (n > 0x7fffffff) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)n), dim3(EW_THREADS), 0, st, x, ldx, ne0, eps, y, ldy, w, yn, ldyn);
+    hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, x, ldx, ne0, eps, y, ldy, w, yn, ldyn,
+                       (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0);
+    return hipGetLastError();
+}
+hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *xs, int64_t ldxs, int64_t n,
+                                   int64_t ne0, float eps, const float *w, float *yn, int64_t ldyn, float *y, int64_t ldy,
+                                   hipStream_t st) {
+    if (n <= 0 || ne0 <= 0) return hipSuccess;
+    if (n > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rms_norm_kernel<true>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, yn, ldyn, b,
+                       ldb, xs, ldxs);
     return hipGetLastError();
 }
 

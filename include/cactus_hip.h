@@ -178,15 +178,20 @@ CHIP_API int chip_add(const float *a, int64_t lda, const float *b, int64_t ldb, 
 CHIP_API int chip_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t n_b, int64_t n, int64_t ne0,
                       float *y, int64_t ldy, void *stream);
 CHIP_API int chip_silu(const float *x, int64_t ldx, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream);
-/* Two adjacent graph nodes in one launch; every element goes through the same operations in the same order as in the
+/* Two or three adjacent graph nodes in one launch; every element goes through the same operations in the same order as in the
  * separate calls, so the results are bit-identical to them:
  *   chip_rms_norm_mul : y = chip_rms_norm(x) * w, w one row of ne0 (build_norm's weight, llama-graph.cpp:527-560); y_norm
  *                       (may be NULL) receives the norm itself.
- *   chip_silu_mul     : y = chip_silu(x) * b, b of the shape of x (the gated FFN, llama-graph.cpp:562-690). */
+ *   chip_silu_mul     : y = chip_silu(x) * b, b of the shape of x (the gated FFN, llama-graph.cpp:562-690).
+ *   chip_add_rms_norm_mul : sum = a + b (the residual, llama-model.cpp build_llama: "ffn_inp", "l_out"), y = chip_rms_norm(sum)
+ *                       [* w when w is not NULL]. sum is always written (the next residual reads it) and may be a or b;
+ *                       y may be a or b (with their row stride) but not sum; otherwise the blocks must not overlap. */
 CHIP_API int chip_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, const float *w, float *y_norm,
                                int64_t ld_norm, float *y, int64_t ldy, void *stream);
 CHIP_API int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy,
                            void *stream);
+CHIP_API int chip_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
+                                   int64_t ne0, float eps, const float *w, float *y, int64_t ldy, void *stream);
 
 /* ---- the attention matmuls over an F16 KV cache ----
  * LM_GGML_OP_MUL_MAT whose src0 is an F16, batched, strided view and whose src1 is F32 (reference llama-graph.cpp:1120

@@ -448,6 +448,61 @@ def test_ffn_block_stays_on_the_device(host, orc):
     L.lm_ggml_free(wctx)
 
 
+def test_residual_add_runs_with_the_norm_that_follows(host, orc):
+    """ADD -> RMS_NORM -> MUL (a residual and the next block's norm, reference llama-model.cpp build_llama: "ffn_inp" / "l_out"
+    followed by build_norm) runs as one kernel, ADD -> RMS_NORM as one kernel, and the sums stay available to the later
+    residuals; all element-wise, so the result equals the CPU arithmetic bit for bit."""
+    import cactus_amd
+    L = host.L
+    H, n = 2048, 6
+    eps = 1e-5
+    rng = np.random.default_rng(8)
+    wn = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    x, z = common.activations_f32(31, n, H), common.activations_f32(32, n, H)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    wctx = host.context(with_graph=False)
+    tn = L.lm_ggml_new_tensor_1d(wctx, O.F32, H)
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
+    host.set(tn, wn)
+    ctx = host.context()
+    tx = host.tensor_2d(ctx, O.F32, H, n, "x")
+    tz = host.tensor_2d(ctx, O.F32, H, n, "z")
+    L.lm_ggml_set_input(tx); L.lm_ggml_set_input(tz)
+    h1 = L.lm_ggml_add(ctx, tx, tz)
+    c1 = L.lm_ggml_mul(ctx, L.lm_ggml_rms_norm(ctx, h1, eps), tn)
+    h2 = L.lm_ggml_add(ctx, c1, h1)
+    o = L.lm_ggml_rms_norm(ctx, h2, eps)
+    out = L.lm_ggml_add(ctx, o, h2)
+    L.lm_ggml_set_output(out)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, out)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 64, False, True)
+    for t in (h1, c1, h2, o, out):
+        L.lm_ggml_backend_sched_set_tensor_backend(sched, t, hip)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(tx, x); host.set(tz, z)
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_fused_pairs.restype = C.c_ulonglong
+    fused_before = blib.lm_ggml_backend_hip_get_fused_pairs()
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == 3          # (add, norm, mul) = 2 joins, (add, norm) = 1
+    y = host.get(out, np.float32, (n, H))
+    s1 = x + z
+    s2 = orc.rms_norm(s1, eps) * wn + s1
+    want = orc.rms_norm(s2, eps) + s2
+    assert y.tobytes() == want.tobytes()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(wbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(wctx)
+
+
 def test_attention_side_nodes_run_on_the_device(host, orc):
     """The nodes llama.cpp puts around the KV cache (reference llama-graph.cpp:1060-1166, llama-kv-cache.cpp:617-656): RoPE of
     Q and K, the K store (F32 -> F16 into a 1-D view of the cache), the transposed V store, the masked soft-max and the

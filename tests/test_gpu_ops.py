@@ -134,3 +134,34 @@ def test_fused_pairs_equal_the_separate_ops(dev, orc, n, ne0):
     else:
         import cactus_amd as ca
         assert dev.lib.chip_silu_mul(dx.ptr, ne0, dx.ptr, ne0, n, ne0, dy.ptr, ne0, None) == ca.CHIP_EUNSUPPORTED
+
+
+@pytest.mark.parametrize("n,ne0", [(1, 4096), (8, 4096), (3, 40), (130, 14336), (5, 1001)])
+@pytest.mark.parametrize("with_w", [True, False])
+def test_fused_add_norm_equals_the_separate_ops(dev, n, ne0, with_w):
+    """chip_add_rms_norm_mul against chip_add, chip_rms_norm and chip_mul run one after the other (bit for bit), with the sum
+    written over either operand and the result over the other."""
+    a, b = inputs(7 * n + ne0, n, ne0), inputs(11 * n + ne0, n, ne0)
+    w = (1.0 + 0.1 * np.random.default_rng(ne0).standard_normal(ne0)).astype(np.float32)
+    with np.errstate(all="ignore"):
+        s_want = dev.binary("add", a, b)
+        y_want = dev.rms_norm(s_want, 1e-6)
+        if with_w:
+            y_want = dev.binary("mul", y_want, w)
+    dw = dev.to_device(w)
+    wp = dw.ptr if with_w else None
+    for sum_over, y_over in (("new", "new"), ("a", "new"), ("b", "new"), ("b", "a"), ("a", "b"), ("new", "a")):
+        da, db = dev.to_device(a), dev.to_device(b)
+        ds, dy = dev.alloc(a.nbytes), dev.alloc(a.nbytes)
+        sp = {"new": ds, "a": da, "b": db}[sum_over]
+        yp = {"new": dy, "a": da, "b": db}[y_over]
+        dev.check(dev.lib.chip_add_rms_norm_mul(da.ptr, ne0, db.ptr, ne0, sp.ptr, ne0, n, ne0, 1e-6, wp, yp.ptr, ne0, None))
+        dev.sync()
+        assert sp.download(np.float32, a.size).tobytes() == s_want.tobytes(), (sum_over, y_over)
+        assert yp.download(np.float32, a.size).tobytes() == y_want.tobytes(), (sum_over, y_over)
+        for t in (da, db, ds, dy):
+            t.free()
+    import cactus_amd as ca
+    da = dev.to_device(a)
+    assert dev.lib.chip_add_rms_norm_mul(da.ptr, ne0, da.ptr, ne0, da.ptr, ne0, n, ne0, 1e-6, wp, da.ptr, ne0, None) == ca.CHIP_EINVAL
+    da.free(); dw.free()
