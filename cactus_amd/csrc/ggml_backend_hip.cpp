@@ -540,12 +540,51 @@ int try_fused_add_norm(backend_ctx *c, const lm_ggml_cgraph *g, int i, int &used
                                  wt ? (const float *)wt->data : nullptr, (float *)out->data, ldy, c->stream);
 }
 
+bool disjoint(const lm_ggml_tensor *p, const lm_ggml_tensor *q) {
+    const uintptr_t a = (uintptr_t)p->data, b = (uintptr_t)q->data;
+    return a + lm_ggml_nbytes(p) <= b || b + lm_ggml_nbytes(q) <= a;
+}
+
+// The gated FFN in llama.cpp's node order: gate matmul, SILU, up matmul, MUL(silu, up) (reference llama-graph.cpp:562-690;
+// the up projection is the MUL's second operand and is visited after the first). When the matmul between the two
+// writes nothing the SILU reads, the SILU can wait for it and run inside the MUL's kernel. True: silu is to be skipped
+// now and nodes[i + 2] run as chip_silu_mul.
+bool silu_can_wait_for_its_mul(const lm_ggml_cgraph *g, int i) {
+    const lm_ggml_tensor *silu = g->nodes[i];
+    if (i + 2 >= g->n_nodes) return false;
+    const lm_ggml_tensor *mm = g->nodes[i + 1], *mul = g->nodes[i + 2];
+    if (mm->op != LM_GGML_OP_MUL_MAT || !mul_mat_shape_ok(mm) || mm->src[0] == silu || mm->src[1] == silu) return false;
+    if (mul->op != LM_GGML_OP_MUL || mul->data != silu->data || !elementwise_shape_ok(mul) || !same_shape(mul, silu)) return false;
+    const lm_ggml_tensor *other = mul->src[0] == silu ? mul->src[1] : (mul->src[1] == silu ? mul->src[0] : nullptr);
+    int64_t r, ld;
+    if (!other || other == silu || !same_shape(other, silu) || !as_rows(other, r, ld)) return false;
+    return disjoint(mm, silu->src[0]) && disjoint(mm, silu);
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
+    const lm_ggml_tensor *waiting_silu = nullptr;     // a SILU held back for the MUL two nodes on
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        if (waiting_silu && node->op == LM_GGML_OP_MUL) {
+            const lm_ggml_tensor *silu = waiting_silu, *other = node->src[0] == silu ? node->src[1] : node->src[0];
+            waiting_silu = nullptr;
+            int64_t rows, lda, ldb, ldy;
+            as_rows(silu->src[0], rows, lda);
+            as_rows(other, rows, ldb);
+            as_rows(node, rows, ldy);
+            const int rc = chip_silu_mul((const float *)silu->src[0]->data, lda, (const float *)other->data, ldb, rows, silu->ne[0],
+                                         (float *)node->data, ldy, c->stream);
+            if (rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (SILU run with its MUL) failed: %s\n", __func__, node->name, chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+            g_elementwise_nodes += 2;
+            g_fused_pairs++;
+            continue;
+        }
         if (node->op == LM_GGML_OP_ADD && elementwise_shape_ok(node) && fusion_enabled()) {
             int used = 0;
             const int rc = try_fused_add_norm(c, cgraph, i, used);
@@ -573,6 +612,10 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 g_elementwise_nodes += 2;
                 g_fused_pairs++;
                 i++;
+                continue;
+            }
+            if (node->op == LM_GGML_OP_UNARY && silu_can_wait_for_its_mul(cgraph, i)) {
+                waiting_silu = node;                   // nodes[i + 1] is a weight matmul (it runs next), nodes[i + 2] the MUL
                 continue;
             }
         }
