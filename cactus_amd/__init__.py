@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums",
@@ -98,6 +98,8 @@ def load_library(path=KERNEL_LIB):
     L.chip_convert_f32_to_f16.argtypes = [vp, i64, i64, i64, vp, vp]
     L.chip_mul_mat_workspace_size.restype = sz
     L.chip_mul_mat_workspace_size.argtypes = [i32, i64, i64]
+    L.chip_mul_mat_workspace_size_n.restype = sz
+    L.chip_mul_mat_workspace_size_n.argtypes = [i32, i64, i64, i64]
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
@@ -203,8 +205,9 @@ class Device:
         self.sync()
         return dy.download(np.uint8, n * rs).reshape(n, rs)
 
-    def mul_mat(self, wtype, W, x, dW=None, want_workspace_blocks=False):
-        """LM_GGML_OP_MUL_MAT: W uint8 [N, row_size(wtype, K)] (or a DeviceBuffer via dW), x fp32 [n, K] -> y [n, N]."""
+    def mul_mat(self, wtype, W, x, dW=None, want_workspace_blocks=False, split_k=True):
+        """LM_GGML_OP_MUL_MAT: W uint8 [N, row_size(wtype, K)] (or a DeviceBuffer via dW), x fp32 [n, K] -> y [n, N].
+        split_k=False gives the library only the activation workspace, so a GEMM never splits K."""
         x = np.ascontiguousarray(x, np.float32)
         n, k = x.shape
         if dW is None:
@@ -216,7 +219,7 @@ class Device:
         nb01 = self.row_size(wtype, k)
         dx = self.to_device(x)
         dy = self.alloc(n * N * 4)
-        wsz = self.lib.chip_mul_mat_workspace_size(wtype, k, n)
+        wsz = self.lib.chip_mul_mat_workspace_size_n(wtype, k, N, n) if split_k else self.lib.chip_mul_mat_workspace_size(wtype, k, n)
         ws = self.alloc(wsz)
         self.check(self.lib.chip_mul_mat(wtype, dW.ptr, nb01, k, N, dx.ptr, k, n, dy.ptr, N, ws.ptr, wsz, None))
         self.sync()

@@ -189,6 +189,191 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArg
     }
 }
 
+// ---- 5 to 63 columns (a few tokens per step): 16 rows x 16 columns x 32 halves per MFMA ----
+// Operand layout of v_mfma_f32_16x16x32_f16: lane (i = lane % 16, g = lane / 16) gives the 8 halves k = 8g .. 8g + 7 of row i
+// (A, a cache row) or of column i (B, an activation column), i.e. 16-byte chunk 4 * step + g of that row; it receives
+// D[4g .. 4g + 3][i], four consecutive rows of column i, which are four consecutive floats of that column's output.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f16x8 as_halves(const u32x4 v) { return __builtin_bit_cast(f16x8, v); }
+__device__ __forceinline__ void store_rows4(float *yp, int64_t row, int64_t N, const f32x4 d) {
+    if (row + 3 < N && (((uintptr_t)(yp + row)) & 15) == 0) {
+        *reinterpret_cast<f32x4 *>(yp + row) = d;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            if (row + r < N) yp[row + r] = d[r];
+    }
+}
+
+// short rows (kq): K <= 32 * KS; the rounded activation columns stay in registers (KS * CG operands), a wave walks 16-row tiles
+template <int KS, int CG>
+__global__ __launch_bounds__(AM_THREADS) void mm_f16_mfma_short_kernel(BatchedArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int64_t b0 = blockIdx.y;
+    const uint8_t *Wb = a.W + b0 * a.nb02;
+    const int64_t cols = a.r2 * a.n, chunks = a.K / 8;
+    u32x4 bx[CG][KS];
+    float *yp[CG];
+#pragma unroll
+    for (int cg = 0; cg < CG; cg++) {
+        const int64_t c = cg * 16 + i;
+        const float *xc = col_x(a, b0, c < cols ? c : cols - 1);
+        yp[cg] = c < cols ? col_y(a, b0, c) : nullptr;
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            const int ch = 4 * s + g;
+            bx[cg][s] = u32x4{0u, 0u, 0u, 0u};
+            if (c < cols && ch < chunks) {
+                const float4 *xp = reinterpret_cast<const float4 *>(xc + 8 * ch);
+                bx[cg][s] = round8(xp[0], xp[1]);
+            }
+        }
+    }
+    const int64_t tiles = ceil_div(a.N, (int64_t)16);
+    for (int64_t t = (int64_t)blockIdx.x * AM_WAVES + wave; t < tiles; t += (int64_t)gridDim.x * AM_WAVES) {
+        const int64_t row = t * 16 + i;
+        u32x4 aw[KS];
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            const int ch = 4 * s + g;
+            aw[s] = u32x4{0u, 0u, 0u, 0u};
+            if (row < a.N && ch < chunks) aw[s] = *reinterpret_cast<const u32x4 *>(Wb + row * a.nb01 + 16 * ch);
+        }
+#pragma unroll
+        for (int cg = 0; cg < CG; cg++) {
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < KS; s++) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_halves(aw[s]), as_halves(bx[cg][s]), acc, 0, 0, 0);
+            if (yp[cg]) store_rows4(yp[cg], t * 16 + 4 * g, a.N, acc);
+        }
+    }
+}
+
+// long rows (kqv): a workgroup of AL_WAVES waves takes 16 rows of one KV head; wave w takes the 32-half steps w, w + AL_WAVES, ...
+// of K for all columns; the partial tiles meet in LDS and are added in wave order.
+constexpr int AL_WAVES = 16;
+template <int CG>
+__global__ __launch_bounds__(AL_WAVES * 64) void mm_f16_mfma_long_kernel(BatchedArgs a) {
+    __shared__ f32x4 part[AL_WAVES][CG][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int64_t b0 = blockIdx.y, t = blockIdx.x;
+    const uint8_t *Wb = a.W + b0 * a.nb02;
+    const int64_t cols = a.r2 * a.n, chunks = a.K / 8, steps = ceil_div(chunks, (int64_t)4);
+    const int64_t row = t * 16 + i;
+    const uint8_t *wrow = Wb + (row < a.N ? row : a.N - 1) * a.nb01;
+    const float *xc[CG];
+#pragma unroll
+    for (int cg = 0; cg < CG; cg++) {
+        const int64_t c = cg * 16 + i;
+        xc[cg] = col_x(a, b0, c < cols ? c : cols - 1);
+    }
+    f32x4 acc[CG];
+#pragma unroll
+    for (int cg = 0; cg < CG; cg++) acc[cg] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int UN = CG == 1 ? 8 : CG == 2 ? 4 : 2;                 // steps whose loads are in flight together (128 registers per lane)
+    for (int64_t q0 = wave; q0 < steps; q0 += UN * AL_WAVES) {
+        u32x4 aw[UN];
+        float4 xr[UN][CG][2];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int64_t ch = 4 * (q0 + u * AL_WAVES) + g;
+            const bool in = ch < chunks;
+            aw[u] = u32x4{0u, 0u, 0u, 0u};
+            if (in && row < a.N) aw[u] = *reinterpret_cast<const u32x4 *>(wrow + 16 * ch);
+#pragma unroll
+            for (int cg = 0; cg < CG; cg++) {
+                xr[u][cg][0] = xr[u][cg][1] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (in && cg * 16 + i < cols) {
+                    const float4 *xp = reinterpret_cast<const float4 *>(xc[cg] + 8 * ch);
+                    xr[u][cg][0] = xp[0];
+                    xr[u][cg][1] = xp[1];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++)
+#pragma unroll
+            for (int cg = 0; cg < CG; cg++)
+                acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_halves(aw[u]), as_halves(round8(xr[u][cg][0], xr[u][cg][1])), acc[cg], 0, 0, 0);
+    }
+#pragma unroll
+    for (int cg = 0; cg < CG; cg++) part[wave][cg][lane] = acc[cg];
+    __syncthreads();
+    // element e of the tile: column group, lane, row within the lane's four
+    for (int e = threadIdx.x; e < CG * 64 * 4; e += AL_WAVES * 64) {
+        const int cg = e >> 8, ln = (e >> 2) & 63, r = e & 3;
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < AL_WAVES; w++) v += part[w][cg][ln][r];
+        const int64_t c = cg * 16 + (ln & 15), rr = t * 16 + 4 * (ln >> 4) + r;
+        if (c < cols && rr < a.N) col_y(a, b0, c)[rr] = v;
+    }
+}
+
+// long rows, K split over workgroups (kqv with 5 to 128 columns): workgroup (slice, KV head) takes AS_SLICE values of K for
+// every row and column of the head.  The slice of the activations is rounded to fp16 once into LDS and shared by the
+// waves, each of which owns 16-row tiles; the cache and the activations are each read once overall.  The partial
+// sums go to the workspace as [slice][KV head][column][row] and a second kernel adds the slices in order.
+constexpr int AS_SLICE = 256, AS_WAVES = 8, AS_STEPS = AS_SLICE / 32;
+constexpr int AS_XSTRIDE = AS_SLICE * 2 + 16;                       // bytes per column in LDS
+constexpr int64_t AS_MAX_COLS = 128, AS_MAX_ROWS = 256;
+template <int CG>
+__global__ __launch_bounds__(AS_WAVES * 64) void mm_f16_mfma_slice_kernel(BatchedArgs a, float *__restrict__ part) {
+    __shared__ __attribute__((aligned(16))) uint8_t xb[CG * 16 * AS_XSTRIDE];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int64_t slice = blockIdx.x, b0 = blockIdx.y;
+    const int64_t cols = a.r2 * a.n, chunks = a.K / 8, ch0 = slice * (AS_SLICE / 8);
+    for (int e = threadIdx.x; e < CG * 16 * (AS_SLICE / 8); e += AS_WAVES * 64) {
+        const int c = e / (AS_SLICE / 8), ch = e % (AS_SLICE / 8);
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (c < cols && ch0 + ch < chunks) {
+            const float4 *xp = reinterpret_cast<const float4 *>(col_x(a, b0, c) + 8 * (ch0 + ch));
+            v = round8(xp[0], xp[1]);
+        }
+        *reinterpret_cast<u32x4 *>(xb + c * AS_XSTRIDE + 16 * ch) = v;
+    }
+    __syncthreads();
+    const uint8_t *Wb = a.W + b0 * a.nb02;
+    float *pbase = part + ((slice * gridDim.y + b0) * cols) * a.N;
+    for (int64_t t = wave; t * 16 < a.N; t += AS_WAVES) {
+        const int64_t row = t * 16 + i;
+        u32x4 aw[AS_STEPS];
+#pragma unroll
+        for (int s = 0; s < AS_STEPS; s++) {
+            const int64_t ch = ch0 + 4 * s + g;
+            aw[s] = u32x4{0u, 0u, 0u, 0u};
+            if (row < a.N && ch < chunks) aw[s] = *reinterpret_cast<const u32x4 *>(Wb + row * a.nb01 + 16 * ch);
+        }
+#pragma unroll
+        for (int cg = 0; cg < CG; cg++) {
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < AS_STEPS; s++) {
+                const u32x4 b = *reinterpret_cast<const u32x4 *>(xb + (cg * 16 + i) * AS_XSTRIDE + 16 * (4 * s + g));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_halves(aw[s]), as_halves(b), acc, 0, 0, 0);
+            }
+            const int64_t c = cg * 16 + i;
+            if (c < cols) store_rows4(pbase + c * a.N, t * 16 + 4 * g, a.N, acc);
+        }
+    }
+}
+__global__ __launch_bounds__(AM_THREADS) void mm_f16_slice_sum_kernel(BatchedArgs a, const float *__restrict__ part, int64_t slices,
+                                                                      int64_t ne02) {
+    const int64_t cols = a.r2 * a.n, per_slice = ne02 * cols * a.N;
+    const int64_t e = (int64_t)blockIdx.x * AM_THREADS + threadIdx.x;
+    if (e >= per_slice) return;
+    float v = 0.0f;
+    for (int64_t sl = 0; sl < slices; sl++) v += part[sl * per_slice + e];
+    const uint32_t N = (uint32_t)a.N, cr = (uint32_t)(e / N), row = (uint32_t)(e - (int64_t)cr * N);     // e < 2^31 (checked by the launcher)
+    const uint32_t b0 = cr / (uint32_t)cols, c = cr - b0 * (uint32_t)cols;
+    col_y(a, b0, c)[row] = v;
+}
+
 // ---- many columns: fp16 rows for the GEMM and its (KV head, tile) list ----
 // Row R = b * n + t of the workspace and of y is column (query head b, token t); the pairs of KV head e are the rows
 // e * r2 * n ... (e + 1) * r2 * n - 1, in order.
@@ -224,7 +409,8 @@ struct GemmPlan { bool use; size_t act_stride, off_perm, off_offsets, off_tiles,
 GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
     GemmPlan p{};
     const int64_t per_head = r2 * n;
-    p.use = K >= 64 && K % 8 == 0 && N >= 32 && per_head >= GEMM_MIN_COLS && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
+    static const int64_t min_cols = [] { const char *e = getenv("CHIP_ATTN_GEMM_MIN"); return e ? (int64_t)atoi(e) : GEMM_MIN_COLS; }();
+    p.use = K >= 64 && K % 8 == 0 && N >= 32 && per_head >= min_cols && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
     if (!p.use) return p;
     p.act_stride = f16_stride(K);
     // 128 x 128 tiles once they still give every CU four workgroups, else 64 x 64 (CHIP_ATTN_TILE forces one, for tuning)
@@ -244,9 +430,17 @@ GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
 
 bool mul_mat_f16_batched_supported(int64_t K) { return K > 0 && K % 8 == 0; }
 
+// the split-K pair: 5 to AS_MAX_COLS columns per KV head, long rows, up to AS_MAX_ROWS rows (head sizes)
+static size_t slice_plan_bytes(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
+    const int64_t cols = r2 * n, slices = ceil_div(K, (int64_t)AS_SLICE);
+    if (K <= 256 || K % 8 != 0 || cols <= AM_COLS || cols > AS_MAX_COLS || N > AS_MAX_ROWS || ne02 > 65535 || ne02 * cols * N >= (1LL << 31)) return 0;
+    return (size_t)(slices * ne02 * cols * N) * sizeof(float);
+}
+
 size_t mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
     if (K <= 0 || N <= 0 || ne02 <= 0 || r2 <= 0 || n <= 0) return 0;
-    return gemm_plan(K, N, ne02, r2, n).bytes;
+    const size_t g = gemm_plan(K, N, ne02, r2, n).bytes, sp = slice_plan_bytes(K, N, ne02, r2, n);
+    return g > sp ? g : sp;
 }
 
 hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
@@ -254,6 +448,22 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
                                       void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st) {
     if (N <= 0 || n <= 0 || ne02 <= 0 || r2 <= 0) return hipSuccess;
     if (!mul_mat_f16_batched_supported(K) || ne02 > 65535 || r2 * n > 0x7fffffff) return hipErrorInvalidValue;
+    static const bool mfma_rows = [] { const char *e = getenv("CHIP_ATTN_MFMA"); return !(e && e[0] == '0'); }();
+    if (const size_t sp = slice_plan_bytes(K, N, ne02, r2, n); mfma_rows && sp > 0 && workspace && workspace_bytes >= sp &&
+                                                              (((uintptr_t)workspace) & 15) == 0) {
+        const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
+        const int64_t cols = r2 * n, slices = ceil_div(K, (int64_t)AS_SLICE);
+        const dim3 grid((unsigned)slices, (unsigned)ne02), block(AS_WAVES * 64);
+        float *part = (float *)workspace;
+        if (cols <= 16)      hipLaunchKernelGGL(mm_f16_mfma_slice_kernel<1>, grid, block, 0, st, a, part);
+        else if (cols <= 32) hipLaunchKernelGGL(mm_f16_mfma_slice_kernel<2>, grid, block, 0, st, a, part);
+        else if (cols <= 64) hipLaunchKernelGGL(mm_f16_mfma_slice_kernel<4>, grid, block, 0, st, a, part);
+        else                 hipLaunchKernelGGL(mm_f16_mfma_slice_kernel<8>, grid, block, 0, st, a, part);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        hipLaunchKernelGGL(mm_f16_slice_sum_kernel, dim3((unsigned)ceil_div(ne02 * cols * N, (int64_t)AM_THREADS)), dim3(AM_THREADS), 0, st,
+                           a, part, slices, ne02);
+        return hipGetLastError();
+    }
     const GemmPlan plan = gemm_plan(K, N, ne02, r2, n);
     // the GEMM writes row R of y at R * ldy1: the batches of y must follow each other without a gap
     if (plan.use && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {
@@ -269,6 +479,31 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
     }
     const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    const int64_t cols = r2 * n;
+    if (mfma_rows && cols > AM_COLS && cols <= 64 && N <= 16LL * 0x7fffffff) {
+        const int cg = cols <= 16 ? 1 : cols <= 32 ? 2 : 4;
+        const int64_t tiles = ceil_div(N, (int64_t)16);
+        if (K <= 256 && (K <= 128 || cg <= 2)) {
+            int64_t gx = ceil_div(tiles, (int64_t)AM_WAVES);
+            const int64_t cap = ceil_div((int64_t)cus * 4, ne02);
+            if (gx > cap) gx = cap;
+            const dim3 grid((unsigned)gx, (unsigned)ne02), block(AM_THREADS);
+            const int ks = K <= 64 ? 2 : K <= 128 ? 4 : 8;
+#define SHORT_CASE(KS, CG) hipLaunchKernelGGL((mm_f16_mfma_short_kernel<KS, CG>), grid, block, 0, st, a)
+            if (ks == 2)      { if (cg == 1) SHORT_CASE(2, 1); else if (cg == 2) SHORT_CASE(2, 2); else SHORT_CASE(2, 4); }
+            else if (ks == 4) { if (cg == 1) SHORT_CASE(4, 1); else if (cg == 2) SHORT_CASE(4, 2); else SHORT_CASE(4, 4); }
+            else              { if (cg == 1) SHORT_CASE(8, 1); else SHORT_CASE(8, 2); }
+#undef SHORT_CASE
+            return hipGetLastError();
+        }
+        if (K > 256) {
+            const dim3 grid((unsigned)tiles, (unsigned)ne02), block(AL_WAVES * 64);
+            if (cg == 1)      hipLaunchKernelGGL(mm_f16_mfma_long_kernel<1>, grid, block, 0, st, a);
+            else if (cg == 2) hipLaunchKernelGGL(mm_f16_mfma_long_kernel<2>, grid, block, 0, st, a);
+            else              hipLaunchKernelGGL(mm_f16_mfma_long_kernel<4>, grid, block, 0, st, a);
+            return hipGetLastError();
+        }
+    }
     if (K <= 256) {
         const int lpr = K <= 64 ? 8 : K <= 128 ? 16 : 32;
         // a wave walks at least four row steps (its loads in flight together); about four workgroups per CU over all KV heads

@@ -281,8 +281,30 @@ int chip_mul_mat_prepare(int type, int64_t K, const float *x, int64_t ldx, int64
     return CHIP_OK;
 }
 
+// bytes of the activation rows in the workspace, rounded so that what follows them is 256-byte aligned
+static size_t act_rows_bytes(int type, int64_t K, int64_t n) { return (chip_mul_mat_workspace_size(type, K, n) + 255) & ~(size_t)255; }
+static int split_slices(int type, int64_t K, int64_t N, int64_t n, int cus) {
+    const int a = gemm_blk32_slices(type, K, N, n, cus), b = gemm_kq_slices(type, K, N, n, cus);
+    return a > b ? a : b;
+}
+size_t chip_mul_mat_workspace_size_n(int type, int64_t K, int64_t N, int64_t n) {
+    const size_t act = chip_mul_mat_workspace_size(type, K, n);
+    if (act == 0 || N <= 0) return act;
+    DeviceLimits lim;
+    const int cus = current_limits(lim) == CHIP_OK ? lim.compute_units : 256;
+    const int slices = split_slices(type, K, N, n, cus);
+    return slices > 1 ? act_rows_bytes(type, K, n) + (size_t)slices * (size_t)n * (size_t)N * sizeof(float) : act;
+}
+
+static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
+                       size_t workspace_bytes, float *y, int64_t ldy, void *stream);
 int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
                      float *y, int64_t ldy, void *stream) {
+    return mul_mat_run(type, W, nb01, K, N, n, workspace, 0, y, ldy, stream);
+}
+// workspace_bytes: what the caller says lies behind `workspace` (0 = the activation rows only, no room for split-K partials)
+static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
+                       size_t workspace_bytes, float *y, int64_t ldy, void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;
     if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
     if (N == 0 || n == 0) return CHIP_OK;
@@ -295,17 +317,26 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     const size_t stride = act_stride(chip_vec_dot_type(type), K);
     hipStream_t st = (hipStream_t)stream;
 
-    if (gemm_blk32_supported(type, K, N, n))
-        return hip_rc(launch_gemm_blk32(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
+    SplitK split{nullptr, 0};
+    if (const size_t act = act_rows_bytes(type, K, n); workspace_bytes > act)
+        split = SplitK{reinterpret_cast<float *>((uint8_t *)const_cast<void *>(workspace) + act), workspace_bytes - act};
+    // K is split only with room for every slice's partial output behind the activation rows
+    const int want_slices = split.part ? split_slices(type, K, N, n, lim.compute_units) : 1;
+    const bool can_split = want_slices > 1 && split.bytes >= (size_t)want_slices * (size_t)n * (size_t)N * sizeof(float);
+    if (!can_split) split = SplitK{nullptr, 0};
+    if (gemm_blk32_supported(type, K, N, n, can_split))
+        return hip_rc(launch_gemm_blk32(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st, nullptr, 1, split));
     if (type == T_F16 && gemm_f16_supported(K, N, n))
         return hip_rc(launch_gemm_f16(W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
-    if (gemm_kq_supported(type, K, N, n))
-        return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st));
+    if (gemm_kq_supported(type, K, N, n, can_split))
+        return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st, nullptr, 1, split));
 
     // 5 tokens or more: integer sums on the matrix cores, up to 16 tokens per pass over the weights
     // (4-bit weights on a small matrix: the dot-product GEMV is still ahead up to 6 or 7 tokens)
     // (and Q4_K rows so wide that the kernel runs with six waves: from 7 tokens)
-    const int mmv_min = ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7)
+    static const int mmv_forced = [] { const char *e = getenv("CHIP_MMV_MIN"); return e ? atoi(e) : 0; }();
+    const int mmv_min = mmv_forced > 0 ? mmv_forced
+                        : ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7)
                         : (type == T_Q4_K && K > 13312) ? 7 : MMV_MIN_TOKENS;
     const int mgroup = (n >= mmv_min) ? mmv_max_tokens(type, K, N, lim) : 0;
     if (mgroup > 0) {
@@ -331,7 +362,8 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
 
 int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
                  float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
-    if (n >= 1 && n <= 4 && N > 0 && chip_mul_mat_supported(type, K)) {
+    static const int mmv_forced = [] { const char *e = getenv("CHIP_MMV_MIN"); return e ? atoi(e) : 0; }();
+    if (n >= 1 && n <= 4 && !(mmv_forced > 0 && n >= mmv_forced) && N > 0 && chip_mul_mat_supported(type, K)) {
         // decode: one launch that quantizes in the GEMV prologue (argument checks as in prepare + run)
         DeviceLimits lim;
         int rc0 = current_limits(lim);
@@ -347,7 +379,7 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
     }
     int rc = chip_mul_mat_prepare(type, K, x, ldx, n, workspace, workspace_bytes, stream);
     if (rc) return rc;
-    return chip_mul_mat_run(type, W, nb01, K, N, n, workspace, y, ldy, stream);
+    return mul_mat_run(type, W, nb01, K, N, n, workspace, workspace_bytes, y, ldy, stream);
 }
 
 // MUL_MAT_ID workspace: the quantized activation rows, then the expert offsets and the pair list of the grouped path

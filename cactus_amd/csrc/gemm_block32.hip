@@ -188,7 +188,7 @@ template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
 __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_blk32_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
                                                                 int64_t N, const uint8_t *__restrict__ ws,
                                                                 size_t ws_stride, int64_t M, float *__restrict__ y,
-                                                                int64_t ldy, TileMap map, RowGather rg) {
+                                                                int64_t ldy, TileMap map, RowGather rg, int slice_stages) {
     using C = GemmCfg<TM, TN, WR, WC>;
     using T = Blk32<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -204,7 +204,14 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
     if (gv.tok_tile < 0) return;
     const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
     if (tok_base >= M) return;
-    const int nstages = (int)(K / (32 * GEMM_KB));
+    // split K (never with a gather, whose grid rows are the experts): grid row s takes the stages stage0 .. of every row and
+    // writes its partial tile to slice s of y
+    int stage0 = 0, nstages = (int)(K / (32 * GEMM_KB));
+    if (!GATHER && slice_stages > 0) {
+        stage0 = (int)blockIdx.y * slice_stages;
+        nstages = min(slice_stages, nstages - stage0);
+        y += (size_t)blockIdx.y * (size_t)M * (size_t)ldy;
+    }
     const size_t off_d = q8_0_off_d(K);
 
     // ---- per-thread prefetch registers for one stage ----
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
     for (int i = 0; i < C::S_PER_T; i++) srow[i] = gv.act_row(min(tok_base + (tid + i * C::NT) / GEMM_KB, M - 1));
 
     auto fetch = [&](int stage) {
-        const int64_t kb0 = (int64_t)stage * GEMM_KB;
+        const int64_t kb0 = (int64_t)(stage0 + stage) * GEMM_KB;
 #pragma unroll
         for (int i = 0; i < C::W_PER_T; i++) {
             const int item = tid + i * C::NT;
@@ -435,17 +442,97 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         }
 }
 
-// The GEMM has a fixed cost of about 0.35 us per 32-value block of K; below 32 tokens (48 on small matrices) the
-// GEMV passes over the weights are faster.
-bool gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n) {
+// With few tokens the GEMM's time is its walk over K, about 0.25 us per 32-value block whatever the token count
+// (33 - 37 us at K = 4096, 110 - 120 us at K = 14336), while the GEMV forms pass over the weights once per 8 or 16
+// tokens at memory speed.  Up to 128 tokens on a matrix with few row tiles the walk is cut into slices
+// (blk32_slices_for below: 17 - 20 us at K = 4096, 28 - 39 us at K = 14336).  The token count from which the GEMM is
+// ahead, measured on 4096 x 4096, 14336 x 4096 and 4096 x 14336 (Q8_0 and Q4_0 have the matrix-core GEMV of 16 tokens
+// a pass, 8 on very long rows; the other types pass once per 8 tokens or fewer):
+static bool blk32_splittable(int64_t N) { return ceil_div(N, (int64_t)64) <= 384; }
+static int64_t gemm_blk32_min_tokens(int wtype, int64_t K, int64_t N, bool can_split) {
+    const bool long_rows = K > 8192, big = N * K >= ((int64_t)48 << 20);
+    if (can_split && blk32_splittable(N)) return (wtype == T_Q8_0 && long_rows) ? 9 : 17;
+    // too many row tiles to split, or no room for the partial outputs in the caller's workspace: the unsplit walk
+    switch (wtype) {
+        case T_Q8_0: return long_rows ? 49 : big ? 17 : 49;
+        case T_Q4_0: return long_rows ? 65 : big ? 33 : 49;
+        default:     return big ? 32 : 48;
+    }
+}
+bool gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_split) {
     if (!(wtype == T_Q4_0 || wtype == T_Q8_0 || wtype == T_Q5_0 || wtype == T_IQ4_NL || wtype == T_Q4_1 || wtype == T_Q5_1)) return false;
     if (K % (32 * GEMM_KB) != 0 || N < 1) return false;
-    return n >= ((N * K >= (int64_t)48 << 20) ? 32 : 48);
+    static const int64_t forced = [] { const char *e = getenv("CHIP_GEMM_MIN_TOKENS"); return e ? (int64_t)atoll(e) : (int64_t)0; }();
+    if (forced > 0) return n >= forced;
+    return n >= gemm_blk32_min_tokens(wtype, K, N, can_split);
+}
+
+// ---- split K: the partial outputs [slice][token][row] added in slice order ----
+__global__ __launch_bounds__(256) void sum_slices_kernel(const float *__restrict__ part, int slices, int64_t per_slice, int64_t n,
+                                                         int64_t N, float *__restrict__ y, int64_t ldy) {
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;                // four consecutive rows of one token
+    if (e0 >= n * N) return;
+    const uint32_t t = (uint32_t)(e0 / N);
+    const int64_t r = e0 - (int64_t)t * N;
+    const bool vec = (N & 3) == 0 && (((uintptr_t)part) & 15) == 0;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < slices; s0 += 8) {
+        float4 p[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            p[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (s0 + j < slices) {
+                const float *src = part + (size_t)(s0 + j) * per_slice + e0;
+                if (vec) p[j] = *reinterpret_cast<const float4 *>(src);
+                else {
+                    p[j].x = src[0];
+                    if (r + 1 < N) p[j].y = src[1];
+                    if (r + 2 < N) p[j].z = src[2];
+                    if (r + 3 < N) p[j].w = src[3];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (s0 + j < slices) { v[0] += p[j].x; v[1] += p[j].y; v[2] += p[j].z; v[3] += p[j].w; }
+    }
+    float *dst = y + (size_t)t * ldy + r;
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (r + k < N) dst[k] = v[k];
+}
+hipError_t launch_sum_slices(const float *part, int slices, int64_t n, int64_t N, float *y, int64_t ldy, hipStream_t st) {
+    if (n <= 0 || N <= 0 || slices <= 0) return hipSuccess;
+    // a token's rows in fours: with N not a multiple of 4 a group of four would straddle two tokens, so pad per token
+    if ((N & 3) != 0) {
+        for (int64_t t = 0; t < n; t++) {
+            hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)ceil_div(N, (int64_t)1024)), dim3(256), 0, st, part + t * N, slices, n * N,
+                               (int64_t)1, N, y + t * ldy, ldy);
+        }
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)ceil_div(n * N, (int64_t)1024)), dim3(256), 0, st, part, slices, n * N, n, N, y, ldy);
+    return hipGetLastError();
+}
+
+// Slices of K for the 64 x 64 shape with at most two token tiles: about three workgroups per CU, at least eight stages each.
+static int blk32_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
+    static const int forced = [] { const char *e = getenv("CHIP_GEMM_SLICES"); return e ? atoi(e) : 0; }();
+    const int64_t units = K / (32 * GEMM_KB), tiles = ceil_div(N, (int64_t)64) * ceil_div(M, (int64_t)64);
+    if (M > 128 || units < 16 || !blk32_splittable(N)) return 1;
+    int64_t s = 3 * cus / tiles;
+    if (s > units / 8) s = units / 8;
+    if (s > 16) s = 16;
+    if (forced > 0) s = forced < units ? forced : units;
+    if (s < 2) return 1;
+    const int64_t per = ceil_div(units, s);
+    return (int)ceil_div(units, per);                                   // no empty slice
 }
 
 template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
 static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
+                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
+                             int slices = 1, float *part = nullptr) {
     using C = GemmCfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
     auto kfn = gemm_blk32_kernel<WT, TM, TN, WR, WC, OCC, GATHER>;
@@ -453,15 +540,28 @@ static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, c
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     // workgroups that share an XCD (OCC waves per SIMD, 32 CUs) take a compact block of output tiles
     const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
+    if (!GATHER && slices > 1) {
+        const int slice_stages = (int)ceil_div(K / (32 * GEMM_KB), (int64_t)slices);
+        hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)slices), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                           (const uint8_t *)ws, ws_stride, M, part, N, map, rg, slice_stages);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        return launch_sum_slices(part, slices, M, N, y, ldy, st);
+    }
     hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
-                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg);
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg, 0);
     return hipGetLastError();
 }
 
 template <int WT>
 static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
+                              float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
+                              SplitK split) {
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    if (!rg.perm && split.part) {
+        const int slices = blk32_slices_for(K, N, M, cus);
+        if (slices > 1 && split.bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (((uintptr_t)split.part) & 15) == 0)
+            return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, slices, split.part);
+    }
     // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
     // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
     if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
@@ -476,20 +576,25 @@ static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, 
     }
 }
 
+int gemm_blk32_slices(int wtype, int64_t K, int64_t N, int64_t n, int compute_units) {
+    if (!gemm_blk32_supported(wtype, K, N, n, true)) return 1;
+    return blk32_slices_for(K, N, n, compute_units > 0 ? compute_units : 256);
+}
+
 int gemm_blk32_moe_tile_tokens() { return GemmCfg<1, 1, 2, 2>::BN; }   // the 64 x 64 shape serves the expert groups
 
 hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                              int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp,
-                             int64_t n_as) {
+                             int64_t n_as, SplitK split) {
     if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
     const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     switch (wtype) {
-        case T_Q4_0:   return launch_type<T_Q4_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_Q8_0:   return launch_type<T_Q8_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_Q5_0:   return launch_type<T_Q5_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_IQ4_NL: return launch_type<T_IQ4_NL>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_Q4_1:   return launch_type<T_Q4_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_Q5_1:   return launch_type<T_Q5_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q4_0:   return launch_type<T_Q4_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_Q8_0:   return launch_type<T_Q8_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_Q5_0:   return launch_type<T_Q5_0>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_IQ4_NL: return launch_type<T_IQ4_NL>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_Q4_1:   return launch_type<T_Q4_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_Q5_1:   return launch_type<T_Q5_1>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
         default: return hipErrorInvalidValue;
     }
 }

@@ -285,14 +285,21 @@ struct KqCfg {
 template <int WT, int WR, int WC, int OCC, bool GATHER>
 __global__ __launch_bounds__((WR * WC + KQ_PRODUCERS) * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
-                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg) {
+                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg, int slice_sb) {
     using T = KQ<WT>;
     using C = KqCfg<WT, WR, WC>;
     constexpr int TN = KQ_TN;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nstages = (int)(K / QK_K) * 2;
+    // split K (never with a gather, whose grid rows are the experts): grid row s takes super-blocks sb0 .. of every row
+    // and writes its partial tile to slice s of y
+    int sb0 = 0, nstages = (int)(K / QK_K) * 2;
+    if (!GATHER && slice_sb > 0) {
+        sb0 = (int)blockIdx.y * slice_sb;
+        nstages = 2 * min(slice_sb, (int)(K / QK_K) - sb0);
+        y += (size_t)blockIdx.y * (size_t)M * (size_t)ldy;
+    }
     const TileCoord tc = xcd_tile(blockIdx.x, map);
     if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;        // padding of the tile map
     size_t w_offset;
@@ -332,19 +339,19 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
         auto fetch_w = [&](Wts &R, int sb_wanted) {
             const int sb = min(sb_wanted, nsb - 1);
 #pragma unroll
-            for (int i = 0; i < C::W_PER_T; i++) T::fetch(R.w[i], wsrc[i] + (size_t)sb * T::BYTES, (pt + i * C::NPT) & 3);
+            for (int i = 0; i < C::W_PER_T; i++) T::fetch(R.w[i], wsrc[i] + (size_t)(sb0 + sb) * T::BYTES, (pt + i * C::NPT) & 3);
         };
         auto fetch_x = [&](Acts &R, int stage_wanted, auto even_tag) {
             constexpr bool even = decltype(even_tag)::value;
             const int stage = min(stage_wanted, nstages - 1);
             const int sb = stage >> 1;
 #pragma unroll
-            for (int i = 0; i < C::X_PER_T; i++) R.x[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + (size_t)stage * (32 * KQ_KB));
+            for (int i = 0; i < C::X_PER_T; i++) R.x[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + (size_t)(2 * sb0 + stage) * (32 * KQ_KB));
             if constexpr (even) {
-                R.xs = reinterpret_cast<const float *>(ssrc + off_d)[sb];
-                if constexpr (T::NF16 > 0) R.bs = *reinterpret_cast<const u32x4 *>(bsrc + (size_t)sb * 32);
+                R.xs = reinterpret_cast<const float *>(ssrc + off_d)[sb0 + sb];
+                if constexpr (T::NF16 > 0) R.bs = *reinterpret_cast<const u32x4 *>(bsrc + (size_t)(sb0 + sb) * 32);
                 if constexpr (T::HAS_BSUM) {
-                    const u32x4 *bp = reinterpret_cast<const u32x4 *>(ssrc + off_bs + (size_t)sb * 32);
+                    const u32x4 *bp = reinterpret_cast<const u32x4 *>(ssrc + off_bs + (size_t)(sb0 + sb) * 32);
                     const u32x4 b0 = bp[0], b1 = bp[1];
                     const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
                     int sum = 0;
@@ -543,16 +550,54 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     }
 }
 
-// The GEMM pays off once the token count outweighs its fixed cost of about 2 us per super-block of K: from 16
-// tokens on large matrices, from 32 on small ones (below that the GEMV passes over the weights are faster).
-bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n) {
+// With few tokens the GEMM's time is its walk over K (about 1.5 - 2 us per super-block, whatever the token count:
+// 28 - 35 us at K = 4096, 88 - 112 us at K = 14336), while the GEMV forms pass over the weights once per 8 or 16 tokens at
+// memory speed.  Up to 128 tokens on a matrix with few row tiles the walk is cut into slices (kq_slices_for below:
+// 16 - 19 us at K = 4096, 36 - 41 us at K = 14336).  The token count from which the GEMM is ahead, measured on 4096 x 4096,
+// 14336 x 4096 (too many row tiles to split) and 4096 x 14336:
+static bool kq_splittable(int64_t N) { return ceil_div(N, (int64_t)64) <= 128; }
+static int64_t gemm_kq_min_tokens(int wtype, int64_t K, int64_t N, bool can_split) {
+    if (can_split || !kq_splittable(N)) {
+        if (wtype == T_Q6_K) return 9;                               // its GEMV passes take 8 tokens
+        return kq_splittable(N) ? 17 : 33;                           // Q4_K, Q5_K: passes of 16 tokens
+    }
+    // the caller's workspace has no room for the partial outputs: the unsplit walk
+    const bool long_rows = K > 8192;
+    switch (wtype) {
+        case T_Q4_K: return long_rows ? 33 : 49;
+        case T_Q5_K: return long_rows ? 33 : 49;
+        default:     return long_rows ? 41 : 25;
+    }
+}
+bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_split) {
     if (!(wtype == T_Q4_K || wtype == T_Q5_K || wtype == T_Q6_K) || K < QK_K || K % QK_K != 0 || N < 1) return false;
-    return n >= ((N * K >= (int64_t)48 << 20) ? 16 : 32);
+    static const int64_t forced = [] { const char *e = getenv("CHIP_GEMM_MIN_TOKENS"); return e ? (int64_t)atoll(e) : (int64_t)0; }();
+    if (forced > 0) return n >= forced;
+    return n >= gemm_kq_min_tokens(wtype, K, N, can_split);
+}
+
+// Slices of K for the 64 x 128 shape with one token tile: up to two workgroups per CU, at least four super-blocks each.
+static int kq_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
+    static const int forced = [] { const char *e = getenv("CHIP_GEMM_SLICES"); return e ? atoi(e) : 0; }();
+    const int64_t units = K / QK_K, tiles = ceil_div(N, (int64_t)64);
+    if (M > 128 || units < 8 || !kq_splittable(N)) return 1;
+    int64_t s = 2 * cus / tiles;
+    if (s > units / 4) s = units / 4;
+    if (s > 16) s = 16;
+    if (forced > 0) s = forced < units ? forced : units;
+    if (s < 2) return 1;
+    const int64_t per = ceil_div(units, s);
+    return (int)ceil_div(units, per);                                   // no empty slice
+}
+int gemm_kq_slices(int wtype, int64_t K, int64_t N, int64_t n, int compute_units) {
+    if (!gemm_kq_supported(wtype, K, N, n, true)) return 1;
+    return kq_slices_for(K, N, n, compute_units > 0 ? compute_units : 256);
 }
 
 template <int WT, int WR, int WC, int OCC, bool GATHER>
 static hipError_t launch_kq(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
+                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
+                            int slices = 1, float *part = nullptr) {
     using C = KqCfg<WT, WR, WC>;
     const size_t lds_bytes = C::TOTAL;
     if ((int64_t)lds_bytes > lim.max_lds_per_block) return hipErrorInvalidValue;
@@ -561,16 +606,28 @@ static hipError_t launch_kq(const void *W, size_t nb01, int64_t K, int64_t N, co
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     // one workgroup per CU: 32 workgroups run on an XCD at a time
     const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32);
+    if (!GATHER && slices > 1) {
+        const int slice_sb = (int)ceil_div(K / QK_K, (int64_t)slices);
+        hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)slices), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                           (const uint8_t *)ws, ws_stride, M, part, N, map, rg, slice_sb);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        return launch_sum_slices(part, slices, M, N, y, ldy, st);
+    }
     hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
-                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg);
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg, 0);
     return hipGetLastError();
 }
 
 template <int WT>
 static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                                  int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg,
-                                 int64_t n_as) {
+                                 int64_t n_as, SplitK split) {
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    if (!rg.perm && split.part) {
+        const int slices = kq_slices_for(K, N, M, cus);
+        if (slices > 1 && split.bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (((uintptr_t)split.part) & 15) == 0)
+            return launch_kq<WT, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, slices, split.part);
+    }
     // 128 rows x 128 tokens per workgroup when that gives every CU one, else 64 x 128.  (CHIP_GEMM_KQ_CFG selects a
     // shape by hand.)
     if (rg.perm)                                                                     // expert groups: 64 x 128 tiles
@@ -589,13 +646,14 @@ static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t 
 int gemm_kq_moe_tile_tokens() { return KqCfg<T_Q4_K, 2, 2>::BN; }      // the 64 x 128 shape serves the expert groups
 
 hipError_t launch_gemm_kq(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
-                          int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as) {
+                          int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as,
+                          SplitK split) {
     if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
     const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     switch (wtype) {
-        case T_Q4_K: return launch_kq_type<T_Q4_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_Q5_K: return launch_kq_type<T_Q5_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case T_Q6_K: return launch_kq_type<T_Q6_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case T_Q4_K: return launch_kq_type<T_Q4_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_Q5_K: return launch_kq_type<T_Q5_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
+        case T_Q6_K: return launch_kq_type<T_Q6_K>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, split);
         default: return hipErrorInvalidValue;
     }
 }

@@ -677,7 +677,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
         const int64_t K = w->ne[0], N = w->ne[1], n = x->ne[1];
         if (N == 0 || n == 0) continue;
-        if (!grow_workspace(c, chip_mul_mat_workspace_size(w->type, K, n))) return LM_GGML_STATUS_ALLOC_FAILED;   // wdata
+        if (!grow_workspace(c, chip_mul_mat_workspace_size_n(w->type, K, N, n))) return LM_GGML_STATUS_ALLOC_FAILED;   // wdata
         const int rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, (int64_t)(x->nb[1] / 4), n,
                                     (float *)node->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
         if (rc != CHIP_OK) {

@@ -163,10 +163,18 @@ hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t 
 
 // gemm_block32.hip: int8-MFMA prefill GEMM over weights in 32-value blocks with one fp16 scale (Q4_0, Q8_0, Q5_0,
 // IQ4_NL), activations in the split Q8_0 workspace layout.  _supported includes the token count from which it pays.
-bool       gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n);
+// Split K: with one token tile and fewer row tiles than the machine holds workgroups, K is cut into slices that run as
+// separate workgroups; their partial outputs [slice][token][row] go to `part` and launch_sum_slices adds them in slice
+// order (same result on every run).  gemm_*_slices: the number of slices the launcher would use (1 = no split), and so
+// the size of `part`: slices * n * N floats.
+struct SplitK { float *part; size_t bytes; };
+int        gemm_blk32_slices(int wtype, int64_t K, int64_t N, int64_t n, int compute_units);
+int        gemm_kq_slices(int wtype, int64_t K, int64_t N, int64_t n, int compute_units);
+hipError_t launch_sum_slices(const float *part, int slices, int64_t n, int64_t N, float *y, int64_t ldy, hipStream_t st);
+bool       gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_split = false);
 hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                              int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st,
-                             const RowGather *rg = nullptr, int64_t n_as = 1);
+                             const RowGather *rg = nullptr, int64_t n_as = 1, SplitK split = SplitK{nullptr, 0});
 
 // gemm_f16.hip: fp16-MFMA prefill GEMM over F16 weights, activations as fp16 in the workspace.
 bool       gemm_f16_supported(int64_t K, int64_t N, int64_t n);
@@ -176,10 +184,10 @@ hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, con
 
 // gemm_kquant.hip: int8-MFMA prefill GEMM over Q4_K / Q5_K / Q6_K weights, activations in the split Q8_K workspace
 // layout; the integer sub-block scales ride in the MFMA operand.
-bool       gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n);
+bool       gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_split = false);
 hipError_t launch_gemm_kq(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                           int64_t n, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rg = nullptr,
-                          int64_t n_as = 1);
+                          int64_t n_as = 1, SplitK split = SplitK{nullptr, 0});
 // In the three GEMM launchers: with rg, n_as is the number of token-tile slots the grid provides in y (an upper bound
 // of the tile list's length) and n is ignored; gemm_*_moe_tile_tokens gives the tile height the list must be built for.
 

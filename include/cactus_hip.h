@@ -131,6 +131,10 @@ CHIP_API int chip_convert_f32_to_f16(const float *x, int64_t ldx, int64_t n, int
  * 210-byte blocks allow no more); x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
  */
 CHIP_API size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n);
+/* The same plus room for the partial outputs of a GEMM whose K is split over workgroups (up to 128 tokens on a matrix
+ * with fewer row tiles than the device holds workgroups: the partial tiles are added in a fixed order by a second
+ * kernel).  chip_mul_mat splits K only when workspace_bytes is at least this; with the smaller size it runs unsplit. */
+CHIP_API size_t chip_mul_mat_workspace_size_n(int type, int64_t K, int64_t N, int64_t n);
 CHIP_API int    chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N,
                              const float *x, int64_t ldx, int64_t n,
                              float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);

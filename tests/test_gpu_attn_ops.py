@@ -246,7 +246,12 @@ def attn_case(seed, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
 # with K (head size 96; 104 and 1056 cache positions) that is no multiple of the GEMM's 64-value stage
 ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8, 3, 96, 128), (256, 4, 2, 2, 160, 160),
                (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128), (128, 32, 8, 130, 320, 512),
-               (64, 4, 4, 100, 192, 256), (96, 6, 2, 40, 104, 128), (128, 32, 8, 512, 1056, 2048)]
+               (64, 4, 4, 100, 192, 256), (96, 6, 2, 40, 104, 128), (128, 32, 8, 512, 1056, 2048),
+               # 5 to 63 (head, token) pairs per KV head: the 16 x 16 x 32 matrix-core kernels, one to four column groups
+               (128, 32, 8, 8, 1040, 2048), (128, 32, 8, 15, 520, 1024), (256, 8, 2, 4, 296, 512), (256, 8, 2, 8, 296, 512),
+               (256, 16, 2, 5, 264, 512), (64, 16, 2, 6, 1032, 2048), (128, 32, 8, 2, 4096, 4096), (80, 8, 1, 3, 24, 32),
+               # 65 to 128 pairs: kqv with K split over workgroups (eight column groups), kq through the GEMM
+               (128, 32, 8, 32, 1048, 2048), (96, 12, 2, 17, 520, 1024)]
 
 
 @pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", ATTN_SHAPES)
@@ -265,7 +270,7 @@ def test_attention_matmuls_over_the_cache(dev, orc, hd, n_head, n_head_kv, n_tok
     got = dev.mul_mat_f16_batched(vv, p)
     assert got.shape == (n_head, n_tokens, hd)
     assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
-    if n_tokens * (n_head // n_head_kv) >= 64:                                  # the same without a workspace: dot-product kernels
+    if n_tokens * (n_head // n_head_kv) > 4:                                    # the same without a workspace: the one-launch kernels
         got = dev.mul_mat_f16_batched(vv, p, workspace=False)
         assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
         want = orc.mul_mat_f16_batched(kv, qv, want=("sum_abs",))

@@ -300,7 +300,7 @@ B32_TYPES = (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL, O.Q4_1, O.Q5_1)
 
 
 @pytest.mark.parametrize("wt", B32_TYPES, ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N,n", [(256, 1, 48), (512, 40, 49), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
+@pytest.mark.parametrize("K,N,n", [(256, 1, 49), (512, 40, 50), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
                                    (4096, 12300, 33)])
 def test_gemm_block32_vs_oracle(dev, orc, wt, K, N, n):
     print("gemm", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
@@ -318,7 +318,7 @@ def test_gemm_block32_integer_sums_bit_exact(dev, orc, wt):
     """With every scale equal to 1 the fp32 output is the integer sum itself, so the MFMA path's per-block
     integer dot sums can be compared bit for bit: one block at a time (all other weight scales zero), then all.
     The weight bytes are random, so every nibble / fifth bit / code index / int8 value occurs."""
-    K, N, n = 256, 70, 48
+    K, N, n = 256, 70, 56                                 # from 49 tokens on every block-32 type takes the GEMM
     rng = np.random.default_rng(9 + wt)
     bb = O.BLOCK_BYTES[wt]
     x = rng.integers(-127, 128, (n, K)).astype(np.float32)
@@ -360,7 +360,7 @@ def test_config4_prefill_sampled(dev, orc, N, M):
     check_outputs(y[np.ix_(toks, rows)], ref["y"], ref["sum_abs"], "config 4")
     # linearity across tokens is not available (quantization is per row), but row order independence is:
     # the same weights reversed must give the same numbers reversed
-    y2 = dev.mul_mat(O.Q4_0, wq[::-1].copy(), x[:64])
+    y2 = dev.mul_mat(O.Q4_0, wq[::-1].copy(), x[:64], split_k=False)    # the same walk over K as y: the same bits
     assert np.array_equal(y2[:, ::-1], y[:64])
 
 
@@ -394,8 +394,8 @@ KQ_TYPES = (O.Q4_K, O.Q5_K, O.Q6_K)
 
 
 @pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N,n", [(256, 1, 32), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
-                                   (4096, 12300, 17)])
+@pytest.mark.parametrize("K,N,n", [(256, 1, 49), (512, 40, 50), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257),
+                                   (4096, 12300, 33)])
 def test_gemm_kquant_vs_oracle(dev, orc, wt, K, N, n):
     print("gemm", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
     wq = orc.quantize_weights(wt, common.weights_f32(K + N + wt, N, K, outliers=True))
@@ -432,12 +432,31 @@ def exact_q8_K_inputs(rng, n, K):
     return x
 
 
+@pytest.mark.parametrize("wt", KQ_TYPES + B32_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N,n", [(4096, 300, 64), (2304, 131, 70), (14336, 200, 128), (4096, 8000, 50)])
+def test_gemm_split_k_vs_oracle(dev, orc, wt, K, N, n):
+    """Few tokens on a matrix with few row tiles: K is cut into slices run by separate workgroups and a second kernel adds
+    the partial outputs in slice order (uneven slices at K = 2304; N = 131 is no multiple of the adder's four rows).
+    Against the oracle, against the unsplit GEMM, and the same bits on a second run."""
+    import cactus_amd as ca
+    print("split-k gemm", O.TYPE_NAMES[wt], "K", K, "N", N, "n", n, flush=True)
+    act = dev.lib.chip_mul_mat_workspace_size(wt, K, n)
+    assert dev.lib.chip_mul_mat_workspace_size_n(wt, K, N, n) > act                   # this case does split
+    wq = quantized_weights(wt, K + N, N, K)
+    x = common.activations_f32(K + n, n, K)
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("sum_abs",))
+    y = dev.mul_mat(wt, wq, x)
+    check_outputs(y, ref["y"], ref["sum_abs"], "split-k gemm")
+    check_outputs(dev.mul_mat(wt, wq, x, split_k=False), ref["y"], ref["sum_abs"], "unsplit gemm")
+    assert dev.mul_mat(wt, wq, x).tobytes() == y.tobytes()
+
+
 @pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_gemm_kquant_integer_sums_bit_exact(dev, orc, wt):
     """With d = dmin = 1 and activation scale 1 the fp32 output of a one-super-block product is sumi - summ itself
     (below 2^24), so the digit planes folded into the MFMA operand are compared bit for bit with the reference's
     integer sums, over random scale and quant bytes."""
-    K, N, n = 256, 150, 48
+    K, N, n = 256, 150, 56                                # from 49 tokens on every K-quant takes the GEMM
     rng = np.random.default_rng(77 + wt)
     w = random_kquant_rows(wt, rng, N, 1)
     x = exact_q8_K_inputs(rng, n, K)
@@ -457,7 +476,7 @@ def test_gemm_kquant_integer_sums_bit_exact(dev, orc, wt):
 @pytest.mark.parametrize("wt", KQ_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_gemm_kquant_extreme_bytes(dev, orc, wt):
     # saturating scale / quant bytes in the first rows, activations pinned at +-127: the operand digits at their limits
-    K, N, n = 1024, 64, 32
+    K, N, n = 1024, 64, 64
     rng = np.random.default_rng(5 + wt)
     w = random_kquant_rows(wt, rng, N, K // 256, extreme_rows=8)
     x = exact_q8_K_inputs(rng, n, K)
@@ -482,7 +501,7 @@ def test_gemm_kquant_prefill_shape_sampled(dev, orc, wt):
     toks[0] = 0; toks[-1] = M - 1
     ref = orc.mul_mat(wt, wq[rows], x[toks], nthreads=8, want=("sum_abs",))
     check_outputs(y[np.ix_(toks, rows)], ref["y"], ref["sum_abs"], "k-quant prefill")
-    y2 = dev.mul_mat(wt, wq[::-1].copy(), x[:64])
+    y2 = dev.mul_mat(wt, wq[::-1].copy(), x[:64], split_k=False)      # the same walk over K: the same bits, whatever the tile
     assert np.array_equal(y2[:, ::-1], y[:64])
 
 
