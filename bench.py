@@ -202,10 +202,10 @@ def bench_extra(dev, hip, trace=True):
         m = RotatingWeights(dev, wt, N, K, rng)
         x = dev.to_device(rng.standard_normal((n, K)).astype(np.float32))
         y = dev.alloc(n * N * 4)
-        wsz = L.chip_mul_mat_workspace_size(wt, K, n)
+        wsz = L.chip_mul_mat_workspace_size_n(wt, K, N, n)
         ws = dev.alloc(wsz)
         dev.check(L.chip_mul_mat_prepare(wt, K, x.ptr, K, n, ws.ptr, wsz, st))
-        us_run = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run(wt, m.next(), m.nb01, K, N, n, ws.ptr, y.ptr, N, st), iters)
+        us_run = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run_ws(wt, m.next(), m.nb01, K, N, n, ws.ptr, wsz, y.ptr, N, st), iters)
         us_op = time_runs(dev, hip, st, lambda: L.chip_mul_mat(wt, m.next(), m.nb01, K, N, x.ptr, K, n, y.ptr, N, ws.ptr, wsz, st), iters)
         b = algorithmic_bytes(m.bytes, K, N, n)
         out[name] = {"us_gemv": round(us_run, 2), "us_op": round(us_op, 2), "GBps_gemv": round(b / us_run / 1e3, 1),
@@ -225,11 +225,11 @@ def bench_extra(dev, hip, trace=True):
         w = dev.to_device(synth_weights(dev, wt, N, K, rng))
         x = dev.to_device(rng.standard_normal((M, K)).astype(np.float32))
         y = dev.alloc(M * N * 4)
-        wsz = L.chip_mul_mat_workspace_size(wt, K, M)
+        wsz = L.chip_mul_mat_workspace_size_n(wt, K, N, M)
         ws = dev.alloc(wsz)
         nb01 = dev.row_size(wt, K)
         dev.check(L.chip_mul_mat_prepare(wt, K, x.ptr, K, M, ws.ptr, wsz, st))
-        us_g = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run(wt, w.ptr, nb01, K, N, M, ws.ptr, y.ptr, N, st), 20)
+        us_g = time_runs(dev, hip, st, lambda: L.chip_mul_mat_run_ws(wt, w.ptr, nb01, K, N, M, ws.ptr, wsz, y.ptr, N, st), 20)
         us_o = time_runs(dev, hip, st, lambda: L.chip_mul_mat(wt, w.ptr, nb01, K, N, x.ptr, K, M, y.ptr, N, ws.ptr, wsz, st), 20)
         ops = 2.0 * M * N * K
         peak = F16_PEAK_TFLOPS if wt == ca.F16 else INT8_PEAK_TOPS
@@ -530,7 +530,7 @@ def bench_trace(dev, hip, st, rng):
         x_h = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
         x_ff = dev.to_device(rng.standard_normal((n, FF)).astype(np.float32))
         y = dev.alloc(3 * n * V * 4)                                   # one output region per concurrent branch
-        wsz = max(L.chip_mul_mat_workspace_size(ca.Q6_K, FF, n), L.chip_mul_mat_workspace_size(ca.Q4_K, H, n))
+        wsz = max([L.chip_mul_mat_workspace_size_n(t, K, N, n) for (_, t, N, K, _) in layer] + [L.chip_mul_mat_workspace_size_n(ca.Q6_K, H, V, n)])
         wss = [dev.alloc(wsz) for _ in range(3)]
         fused = n <= 4            # chip_mul_mat quantizes in the GEMV prologue: one launch per matmul
 
@@ -541,7 +541,7 @@ def bench_trace(dev, hip, st, rng):
             else:
                 if not prepared:
                     dev.check(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, wss[lane].ptr, wsz, stream))
-                dev.check(L.chip_mul_mat_run(t, wptr, dev.row_size(t, K), K, N, n, wss[lane].ptr, yp, N, stream))
+                dev.check(L.chip_mul_mat_run_ws(t, wptr, dev.row_size(t, K), K, N, n, wss[lane].ptr, wsz, yp, N, stream))
 
         def fork(streams):
             e = hip.event()

@@ -302,6 +302,11 @@ int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N,
                      float *y, int64_t ldy, void *stream) {
     return mul_mat_run(type, W, nb01, K, N, n, workspace, 0, y, ldy, stream);
 }
+int chip_mul_mat_run_ws(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, void *workspace, size_t workspace_bytes,
+                        float *y, int64_t ldy, void *stream) {
+    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+    return mul_mat_run(type, W, nb01, K, N, n, workspace, workspace_bytes, y, ldy, stream);
+}
 // workspace_bytes: what the caller says lies behind `workspace` (0 = the activation rows only, no room for split-K partials)
 static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
                        size_t workspace_bytes, float *y, int64_t ldy, void *stream) {

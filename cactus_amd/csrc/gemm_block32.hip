@@ -515,15 +515,19 @@ hipError_t launch_sum_slices(const float *part, int slices, int64_t n, int64_t N
     return hipGetLastError();
 }
 
-// Slices of K for the 64 x 64 shape with at most two token tiles: about three workgroups per CU, at least eight stages each.
+// Slices of K for the 64 x 64 shape: about three workgroups per CU up to 128 tokens, two with more (the partial outputs
+// grow with the token count), at least eight stages each.
 static int blk32_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
     static const int forced = [] { const char *e = getenv("CHIP_GEMM_SLICES"); return e ? atoi(e) : 0; }();
     const int64_t units = K / (32 * GEMM_KB), tiles = ceil_div(N, (int64_t)64) * ceil_div(M, (int64_t)64);
-    if (M > 128 || units < 16 || !blk32_splittable(N)) return 1;
-    int64_t s = 3 * cus / tiles;
+    if (forced > 0) {
+        const int64_t per = ceil_div(units, (int64_t)(forced < units ? forced : units));
+        return (int)ceil_div(units, per);
+    }
+    if (units < 16 || (M <= 128 && !blk32_splittable(N))) return 1;
+    int64_t s = (M <= 128 ? 3 : 2) * cus / tiles;
     if (s > units / 8) s = units / 8;
     if (s > 16) s = 16;
-    if (forced > 0) s = forced < units ? forced : units;
     if (s < 2) return 1;
     const int64_t per = ceil_div(units, s);
     return (int)ceil_div(units, per);                                   // no empty slice

@@ -576,15 +576,19 @@ bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_spli
     return n >= gemm_kq_min_tokens(wtype, K, N, can_split);
 }
 
-// Slices of K for the 64 x 128 shape with one token tile: up to two workgroups per CU, at least four super-blocks each.
+// Slices of K for the 64 x 128 shape: up to two workgroups per CU with one token tile, one per CU with more (the partial
+// outputs grow with the token count), at least four super-blocks each.
 static int kq_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
     static const int forced = [] { const char *e = getenv("CHIP_GEMM_SLICES"); return e ? atoi(e) : 0; }();
-    const int64_t units = K / QK_K, tiles = ceil_div(N, (int64_t)64);
-    if (M > 128 || units < 8 || !kq_splittable(N)) return 1;
-    int64_t s = 2 * cus / tiles;
+    const int64_t units = K / QK_K, tiles = ceil_div(N, (int64_t)64) * ceil_div(M, (int64_t)128);
+    if (forced > 0) {
+        const int64_t per = ceil_div(units, (int64_t)(forced < units ? forced : units));
+        return (int)ceil_div(units, per);
+    }
+    if (units < 8 || (M <= 128 && !kq_splittable(N))) return 1;
+    int64_t s = (M <= 128 ? 2 : 1) * cus / tiles;
     if (s > units / 4) s = units / 4;
     if (s > 16) s = 16;
-    if (forced > 0) s = forced < units ? forced : units;
     if (s < 2) return 1;
     const int64_t per = ceil_div(units, s);
     return (int)ceil_div(units, per);                                   // no empty slice

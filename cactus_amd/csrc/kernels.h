@@ -163,7 +163,7 @@ hipError_t launch_mmv(int wtype, const void *W, size_t nb01, int64_t K, int64_t 
 
 // gemm_block32.hip: int8-MFMA prefill GEMM over weights in 32-value blocks with one fp16 scale (Q4_0, Q8_0, Q5_0,
 // IQ4_NL), activations in the split Q8_0 workspace layout.  _supported includes the token count from which it pays.
-// Split K: with one token tile and fewer row tiles than the machine holds workgroups, K is cut into slices that run as
+// Split K: with fewer output tiles than the machine holds workgroups, K is cut into slices that run as
 // separate workgroups; their partial outputs [slice][token][row] go to `part` and launch_sum_slices adds them in slice
 // order (same result on every run).  gemm_*_slices: the number of slices the launcher would use (1 = no split), and so
 // the size of `part`: slices * n * N floats.

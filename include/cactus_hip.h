@@ -131,9 +131,10 @@ CHIP_API int chip_convert_f32_to_f16(const float *x, int64_t ldx, int64_t n, int
  * 210-byte blocks allow no more); x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
  */
 CHIP_API size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n);
-/* The same plus room for the partial outputs of a GEMM whose K is split over workgroups (up to 128 tokens on a matrix
- * with fewer row tiles than the device holds workgroups: the partial tiles are added in a fixed order by a second
- * kernel).  chip_mul_mat splits K only when workspace_bytes is at least this; with the smaller size it runs unsplit. */
+/* The same plus room for the partial outputs of a GEMM whose K is split over workgroups (when the output has fewer
+ * tiles than the device holds workgroups: a few hundred tokens at most; the partial tiles are added in a fixed order by
+ * a second kernel).  chip_mul_mat splits K only when workspace_bytes is at least this; with the smaller size it runs
+ * unsplit, and takes the GEMM from a larger token count on. */
 CHIP_API size_t chip_mul_mat_workspace_size_n(int type, int64_t K, int64_t N, int64_t n);
 CHIP_API int    chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N,
                              const float *x, int64_t ldx, int64_t n,
@@ -147,6 +148,10 @@ CHIP_API int chip_mul_mat_prepare(int type, int64_t K, const float *x, int64_t l
                                   void *workspace, size_t workspace_bytes, void *stream);
 CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,
                               const void *workspace, float *y, int64_t ldy, void *stream);
+/* chip_mul_mat_run told how large the workspace is: with chip_mul_mat_workspace_size_n(type, K, N, n) bytes a GEMM may
+ * split K (the partial outputs go behind the activation rows, which stay valid for the next matmul). */
+CHIP_API int chip_mul_mat_run_ws(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,
+                                 void *workspace, size_t workspace_bytes, float *y, int64_t ldy, void *stream);
 
 /* ---- LM_GGML_OP_MUL_MAT_ID: the expert matmul of mixture-of-experts layers ----
  * lm_ggml_compute_forward_mul_mat_id (ggml-cpu/ggml-cpu.c:1460-1710) with src0 = W (type, [K, N, n_as]: n_as expert
