@@ -328,14 +328,24 @@ __global__ __launch_bounds__(AS_WAVES * 64) void mm_f16_mfma_slice_kernel(Batche
     const int i = lane & 15, g = lane >> 4;
     const int64_t slice = blockIdx.x, b0 = blockIdx.y;
     const int64_t cols = a.r2 * a.n, chunks = a.K / 8, ch0 = slice * (AS_SLICE / 8);
-    for (int e = threadIdx.x; e < CG * 16 * (AS_SLICE / 8); e += AS_WAVES * 64) {
+    static_assert(16 * (AS_SLICE / 8) == AS_WAVES * 64, "one column group per staging round");
+    float4 raw[CG][2];
+#pragma unroll
+    for (int it = 0; it < CG; it++) {                                   // all loads first, then the rounding and the LDS writes
+        const int e = it * (AS_WAVES * 64) + threadIdx.x;
         const int c = e / (AS_SLICE / 8), ch = e % (AS_SLICE / 8);
-        u32x4 v = {0u, 0u, 0u, 0u};
+        raw[it][0] = raw[it][1] = float4{0.0f, 0.0f, 0.0f, 0.0f};
         if (c < cols && ch0 + ch < chunks) {
             const float4 *xp = reinterpret_cast<const float4 *>(col_x(a, b0, c) + 8 * (ch0 + ch));
-            v = round8(xp[0], xp[1]);
+            raw[it][0] = xp[0];
+            raw[it][1] = xp[1];
         }
-        *reinterpret_cast<u32x4 *>(xb + c * AS_XSTRIDE + 16 * ch) = v;
+    }
+#pragma unroll
+    for (int it = 0; it < CG; it++) {
+        const int e = it * (AS_WAVES * 64) + threadIdx.x;
+        const int c = e / (AS_SLICE / 8), ch = e % (AS_SLICE / 8);
+        *reinterpret_cast<u32x4 *>(xb + c * AS_XSTRIDE + 16 * ch) = round8(raw[it][0], raw[it][1]);
     }
     __syncthreads();
     const uint8_t *Wb = a.W + b0 * a.nb02;
@@ -368,7 +378,14 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_slice_sum_kernel(BatchedArg
     const int64_t e = (int64_t)blockIdx.x * AM_THREADS + threadIdx.x;
     if (e >= per_slice) return;
     float v = 0.0f;
-    for (int64_t sl = 0; sl < slices; sl++) v += part[sl * per_slice + e];
+    for (int64_t sl0 = 0; sl0 < slices; sl0 += 8) {                     // eight loads in flight, added in slice order
+        float t[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = sl0 + j < slices ? part[(sl0 + j) * per_slice + e] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (sl0 + j < slices) v += t[j];
+    }
     const uint32_t N = (uint32_t)a.N, cr = (uint32_t)(e / N), row = (uint32_t)(e - (int64_t)cr * N);     // e < 2^31 (checked by the launcher)
     const uint32_t b0 = cr / (uint32_t)cols, c = cr - b0 * (uint32_t)cols;
     col_y(a, b0, c)[row] = v;

@@ -23,7 +23,8 @@
 
 namespace {
 
-std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0};
+std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
+    g_quantizers_skipped{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -37,10 +38,20 @@ struct rope_table_key {
     int32_t params[11];        // op_params 1..10 without the mode: n_dims, n_ctx, n_ctx_orig and the six floats
     bool valid;
 };
+// What the workspace's activation rows were quantized from: wq / wk / wv (and ffn_up / ffn_gate) read the same tensor, so
+// the later ones skip the quantizer.  Dropped when anything else uses the workspace or writes over the source.
+struct quantized_key {
+    bool valid = false;
+    const void *src = nullptr; size_t src_bytes = 0;
+    int64_t K = 0, n = 0, ldx = 0;
+    int vec_dot_type = -1;
+};
+
 struct backend_ctx {
     void *stream; void *workspace; size_t workspace_size;
     float *rope_table = nullptr; size_t rope_table_bytes = 0;
     rope_table_key rope_key = {};
+    quantized_key quantized = {};
 };
 
 lm_ggml_backend_buffer_type_t hip_buffer_type();
@@ -458,6 +469,7 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op) {
 
 static bool grow_workspace(backend_ctx *c, size_t need) {
     if (need <= c->workspace_size) return true;
+    c->quantized.valid = false;
     chip_stream_synchronize(c->stream);
     chip_free(c->workspace);
     c->workspace = nullptr;
@@ -564,10 +576,20 @@ bool silu_can_wait_for_its_mul(const lm_ggml_cgraph *g, int i) {
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
+    c->quantized.valid = false;                       // and so may any activation
     const lm_ggml_tensor *waiting_silu = nullptr;     // a SILU held back for the MUL two nodes on
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        // a node that writes into the tensor the workspace was quantized from, or that uses the workspace itself, ends
+        // the reuse of the quantized rows (every node is seen here, also those run inside a neighbour's kernel)
+        auto writes = [c](const lm_ggml_tensor *t) {
+            if (!c->quantized.valid) return;
+            const uintptr_t a = (uintptr_t)t->data, b = (uintptr_t)c->quantized.src;
+            const bool apart = a + lm_ggml_nbytes(t) <= b || b + c->quantized.src_bytes <= a;
+            if (!apart || t->op == LM_GGML_OP_MUL_MAT_ID || (t->op == LM_GGML_OP_MUL_MAT && !mul_mat_shape_ok(t))) c->quantized.valid = false;
+        };
+        writes(node);
         if (waiting_silu && node->op == LM_GGML_OP_MUL) {
             const lm_ggml_tensor *silu = waiting_silu, *other = node->src[0] == silu ? node->src[1] : node->src[0];
             waiting_silu = nullptr;
@@ -594,6 +616,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 return LM_GGML_STATUS_FAILED;
             }
             if (used) {
+                for (int k = 1; k < used; k++) writes(cgraph->nodes[i + k]);
                 g_elementwise_nodes += used;
                 g_fused_pairs += used - 1;
                 i += used - 1;
@@ -609,6 +632,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 return LM_GGML_STATUS_FAILED;
             }
             if (fused) {
+                writes(cgraph->nodes[i + 1]);
                 g_elementwise_nodes += 2;
                 g_fused_pairs++;
                 i++;
@@ -678,8 +702,28 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         const int64_t K = w->ne[0], N = w->ne[1], n = x->ne[1];
         if (N == 0 || n == 0) continue;
         if (!grow_workspace(c, chip_mul_mat_workspace_size_n(w->type, K, N, n))) return LM_GGML_STATUS_ALLOC_FAILED;   // wdata
-        const int rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, (int64_t)(x->nb[1] / 4), n,
-                                    (float *)node->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
+        int rc;
+        const int64_t ldx = (int64_t)(x->nb[1] / 4);
+        if (n > 4 && fusion_enabled()) {
+            // quantize once per source tensor: the matmuls that share an input follow each other closely
+            quantized_key &q = c->quantized;
+            const int vt = chip_vec_dot_type(w->type);
+            if (!(q.valid && q.src == x->data && q.K == K && q.n == n && q.ldx == ldx && q.vec_dot_type == vt)) {
+                q.valid = false;
+                rc = chip_mul_mat_prepare(w->type, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                if (rc == CHIP_OK) q = quantized_key{true, x->data, lm_ggml_nbytes(x), K, n, ldx, vt};
+            } else {
+                rc = CHIP_OK;
+                g_quantizers_skipped++;
+            }
+            if (rc == CHIP_OK)
+                rc = chip_mul_mat_run_ws(w->type, w->data, w->nb[1], K, N, n, c->workspace, c->workspace_size, (float *)node->data,
+                                         (int64_t)(node->nb[1] / 4), c->stream);
+        } else {
+            c->quantized.valid = false;               // up to 4 tokens the GEMV quantizes in its own prologue, into the workspace
+            rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
+                              (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
+        }
         if (rc != CHIP_OK) {
             HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT %s failed: %s\n", __func__, node->name, chip_error_string(rc));
             return LM_GGML_STATUS_FAILED;
@@ -797,6 +841,7 @@ lm_ggml_backend_dev_t reg_get_device(lm_ggml_backend_reg_t, size_t index) { retu
 void *reg_get_proc_address(lm_ggml_backend_reg_t, const char *name) {
     if (std::strcmp(name, "lm_ggml_backend_hip_get_stats") == 0) return (void *)lm_ggml_backend_hip_get_stats;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_fused_pairs") == 0) return (void *)lm_ggml_backend_hip_get_fused_pairs;
+    if (std::strcmp(name, "lm_ggml_backend_hip_get_quantizers_skipped") == 0) return (void *)lm_ggml_backend_hip_get_quantizers_skipped;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_rope_tables") == 0) return (void *)lm_ggml_backend_hip_get_rope_tables;
     return nullptr;         // no n_threads, no extra buffer types, no split buffer type, no feature list
 }
@@ -858,6 +903,7 @@ void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned l
     if (uploaded_bytes) *uploaded_bytes = g_uploaded.load();
 }
 unsigned long long lm_ggml_backend_hip_get_fused_pairs(void) { return g_fused_pairs.load(); }
+unsigned long long lm_ggml_backend_hip_get_quantizers_skipped(void) { return g_quantizers_skipped.load(); }
 unsigned long long lm_ggml_backend_hip_get_rope_tables(void) { return g_rope_tables.load(); }
 
 }  // extern "C"

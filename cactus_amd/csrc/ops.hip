@@ -71,8 +71,31 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
     const int tid = threadIdx.x;
     bool vec = ((ne0 | ldx | ldy) & 3) == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
     if (ADD) vec = vec && ((ldb | ldxs) & 3) == 0 && ((((uintptr_t)b) | ((uintptr_t)xs)) & 15) == 0;
+    float *ynr = yn ? yn + (size_t)blockIdx.x * ldyn : nullptr;
+    const bool vecw = vec && (!w || ((uintptr_t)w & 15) == 0) && (!yn || ((ldyn & 3) == 0 && ((uintptr_t)yn & 15) == 0));
     double sum = 0.0;
-    if (ADD) {
+    // rows of up to 8192 values stay in registers between the two passes (same order of additions as the loops below)
+    constexpr int RC = 8;
+    const bool cached = vecw && ne0 <= 4 * EW_THREADS * RC;
+    float4 keep[RC];
+    if (cached) {
+        const float *br = ADD ? b + (size_t)blockIdx.x * ldb : nullptr;
+        float *sr = ADD ? xs + (size_t)blockIdx.x * ldxs : nullptr;
+#pragma unroll
+        for (int k = 0; k < RC; k++) {
+            const int64_t i = 4 * tid + (int64_t)k * 4 * EW_THREADS;
+            if (i < ne0) {
+                float4 v = *reinterpret_cast<const float4 *>(xr + i);
+                if (ADD) {
+                    const float4 u = *reinterpret_cast<const float4 *>(br + i);
+                    v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+                    *reinterpret_cast<float4 *>(sr + i) = v;
+                }
+                keep[k] = v;
+                sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+            }
+        }
+    } else if (ADD) {
         const float *br = b + (size_t)blockIdx.x * ldb;
         float *sr = xs + (size_t)blockIdx.x * ldxs;
         if (vec) {
@@ -108,9 +131,22 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
     for (int w = 0; w < EW_THREADS / 64; w++) total += part[w];
     const float mean = (float)(total / (double)ne0);
     const float scale = 1.0f / sqrtf(mean + eps);
-    float *ynr = yn ? yn + (size_t)blockIdx.x * ldyn : nullptr;
-    const bool vecw = vec && (!w || ((uintptr_t)w & 15) == 0) && (!yn || ((ldyn & 3) == 0 && ((uintptr_t)yn & 15) == 0));
-    if (vecw) {
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; k++) {
+            const int64_t i = 4 * tid + (int64_t)k * 4 * EW_THREADS;
+            if (i < ne0) {
+                float4 v = keep[k];
+                v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+                if (w) {
+                    if (ynr) *reinterpret_cast<float4 *>(ynr + i) = v;
+                    const float4 g = *reinterpret_cast<const float4 *>(w + i);
+                    v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w;
+                }
+                *reinterpret_cast<float4 *>(yr + i) = v;
+            }
+        }
+    } else if (vecw) {
         for (int64_t i = 4 * tid; i < ne0; i += 4 * EW_THREADS) {
             float4 v = *reinterpret_cast<const float4 *>(xr + i);
             v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;

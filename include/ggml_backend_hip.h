@@ -46,6 +46,7 @@ CACTUS_GGML_API int lm_ggml_backend_is_hip(struct lm_ggml_backend *backend);
 CACTUS_GGML_API void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned long long *uploaded_bytes);
 /* Pairs of adjacent nodes (RMS_NORM + MUL, SILU + MUL) that graph_compute ran as one kernel. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_fused_pairs(void);
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_quantizers_skipped(void);   /* matmuls that reused the previous one's quantized input */
 /* cos / sin tables built for ROPE nodes (one per graph_compute call and set of parameters; the other ROPE nodes apply it). */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_tables(void);
 

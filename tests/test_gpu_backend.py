@@ -422,11 +422,15 @@ def test_ffn_block_stays_on_the_device(host, orc):
     blib = C.CDLL(cactus_amd.BACKEND_LIB)
     blib.lm_ggml_backend_hip_get_fused_pairs.restype = C.c_ulonglong
     fused_before = blib.lm_ggml_backend_hip_get_fused_pairs()
+    blib.lm_ggml_backend_hip_get_quantizers_skipped.restype = C.c_ulonglong
+    skipped_before = blib.lm_ggml_backend_hip_get_quantizers_skipped()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     # norm + weight ran as one kernel (the allocator writes the MUL over its only producer); SiLU and its MUL are not
     # neighbours in the node order (the up projection sits between them): the SiLU waits for that matmul and runs in the
     # MUL's kernel
     assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == 2
+    # up and gate read the same tensor: the second one reuses the first one's quantized rows
+    assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - skipped_before == 1
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (cur, up, gate, act, down, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
