@@ -473,8 +473,14 @@ def bench_trace(dev, hip, st, rng):
         rope_tab = dev.alloc(n * hd * 4)
         ck = dev.check
 
-        def mm(t, wptr, N, K, src, dst):
-            ck(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, dst.ptr, N, ws.ptr, wsz, st))
+        def mm(t, wptr, N, K, src, dst, shared=False):
+            """shared: src was quantized by the previous matmul (same tensor, same activation type), as the backend reuses it"""
+            if n <= 4:                                                    # the GEMV quantizes in its prologue
+                ck(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, dst.ptr, N, ws.ptr, wsz, st))
+                return
+            if not shared:
+                ck(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, ws.ptr, wsz, st))
+            ck(L.chip_mul_mat_run_ws(t, wptr, dev.row_size(t, K), K, N, n, ws.ptr, wsz, dst.ptr, N, st))
 
         def step():
             for l in range(NL):
@@ -484,7 +490,7 @@ def bench_trace(dev, hip, st, rng):
                 vc = kc + kv_size * KV * 2
                 if l == 0:
                     ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))  # norm + weight: one kernel, as the backend fuses them
-                mm(*W["wq"], cur, q); mm(*W["wk"], cur, k); mm(*W["wv"], cur, v)
+                mm(*W["wq"], cur, q); mm(*W["wk"], cur, k, True); mm(*W["wv"], cur, v, True)
                 if l == 0:                                                # one cos / sin table per step, as the backend keeps it
                     ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
                 for t_, nh in ((q, n_head), (k, n_head_kv)):
@@ -504,7 +510,7 @@ def bench_trace(dev, hip, st, rng):
                 mm(*W["wo"], merged, att)
                 # residual + norm + weight: one kernel, as the backend fuses the three nodes
                 ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
-                mm(*W["up"], cur, up); mm(*W["gate"], cur, gate)
+                mm(*W["up"], cur, up); mm(*W["gate"], cur, gate, True)
                 ck(L.chip_silu_mul(gate.ptr, FF, up.ptr, FF, n, FF, gate.ptr, FF, st))                 # SiLU in its MUL's kernel, as the backend runs the pair
                 mm(*W["down"], gate, att)
                 # the layer's second residual with the next layer's (or the final) norm
@@ -522,7 +528,7 @@ def bench_trace(dev, hip, st, rng):
         for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws, rope_tab):
             bf.free()
         cache_bytes = NL * 2 * n_kv * KV * 2
-        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "kernels": 18 * NL + 3, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
+        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
                 "weight_and_cache_GBps": round((total + cache_bytes) / us / 1e3, 1)}
 
     res = {}
@@ -601,8 +607,7 @@ def bench_trace(dev, hip, st, rng):
                 ops = 2.0 * n * (NL * sum(N * K for (_, _, N, K, _) in layer) + V * H)
                 entry[mode]["TOPS"] = round(ops / us / 1e6, 1)
                 entry[mode]["int8_frac"] = round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)
-        if n in (1, 512):
-            entry["whole_layers"] = full_layers(n, 4096 if n == 1 else 512, wss[0], wsz)
+        entry["whole_layers"] = full_layers(n, 512 if n == 512 else 4096, wss[0], wsz)      # decode and the 8-token batch over 4096 cached positions
         res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = entry
         for bf in [x_h, x_ff, y] + wss:
             bf.free()
