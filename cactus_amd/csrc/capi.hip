@@ -59,8 +59,12 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 // Q4_0 / Q8_0 / Q4_K rows of K % 256 == 0 elements are multiples of 16 bytes and the kernels load them with
 // 4- and 16-byte aligned vectors.  Q6_K rows are multiples of 210 bytes: only 2-byte alignment can be asked for,
 // and that kernel loads with 2-byte aligned vectors throughout.
-bool weights_aligned(int type, const void *W, size_t nb01) {
-    const size_t a = (type == T_Q6_K) ? 2 : 16;
+// The types of 32-value blocks also come with rows of K % 64 == 0 elements (hidden sizes such as 576, 896, 960): such
+// rows are multiples of 4 bytes only, and only the kernels that load with 4-byte aligned vectors take them (the
+// dot-product GEMV; the GEMM, whose staging reads single blocks, when K % 128 == 0).
+bool is_block32_type(int t) { return t == T_Q4_0 || t == T_Q8_0 || t == T_Q5_0 || t == T_IQ4_NL || t == T_Q4_1 || t == T_Q5_1; }
+bool weights_aligned(int type, const void *W, size_t nb01, int64_t K = 256) {
+    const size_t a = (type == T_Q6_K) ? 2 : (is_block32_type(type) && K % 256 != 0) ? 4 : 16;
     return ((uintptr_t)W % a) == 0 && (nb01 % a) == 0;
 }
 
@@ -230,7 +234,9 @@ int chip_vec_dot_type(int type) {
         default: return -1;
     }
 }
-int chip_mul_mat_supported(int type, int64_t K) { return is_weight_type(type) && K > 0 && K % 256 == 0 && K <= (1 << 20); }
+int chip_mul_mat_supported(int type, int64_t K) {
+    return is_weight_type(type) && K > 0 && K % (is_block32_type(type) ? 64 : 256) == 0 && K <= (1 << 20);
+}
 
 static int quantize_public(int act_type, const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
     if (n < 0 || k < 0) return CHIP_EINVAL;
@@ -314,7 +320,7 @@ static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t 
     if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
     if (N == 0 || n == 0) return CHIP_OK;
     if (!W || !workspace || !y || ldy < N) return CHIP_EINVAL;
-    if (!weights_aligned(type, W, nb01) || nb01 < chip_row_size(type, K) || !aligned16(workspace)) return CHIP_EINVAL;
+    if (!weights_aligned(type, W, nb01, K) || nb01 < chip_row_size(type, K) || !aligned16(workspace)) return CHIP_EINVAL;
     if (((uintptr_t)y & 3) != 0) return CHIP_EINVAL;
     DeviceLimits lim;
     int rc = current_limits(lim);
@@ -376,7 +382,7 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
         if (gemv_fused_applicable(type, K, (int)n, lim)) {
             if (!x || !workspace || ldx < K || !W || !y || ldy < N) return CHIP_EINVAL;
             if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0) return CHIP_EINVAL;
-            if (!weights_aligned(type, W, nb01) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
+            if (!weights_aligned(type, W, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
             if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
             return hip_rc(launch_gemv_fused(type, W, nb01, K, N, x, ldx, (int)n, workspace,
                                             act_stride(chip_vec_dot_type(type), K), y, ldy, lim, (hipStream_t)stream));
@@ -404,11 +410,11 @@ int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K
                     int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride, int64_t n_used, int64_t n_tokens,
                     float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
     if (N < 0 || n_as < 0 || n_used < 0 || n_tokens < 0 || ne11 < 0) return CHIP_EINVAL;
-    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (!chip_mul_mat_supported(type, K) || K % 256 != 0) return CHIP_EUNSUPPORTED;
     if (N == 0 || n_used == 0 || n_tokens == 0) return CHIP_OK;
     if (n_as == 0 || !(ne11 == 1 || ne11 == n_used)) return CHIP_EINVAL;
     if (!W || !x || !ids || !y || !workspace || ldx < K || ldy < N || ids_stride < n_used) return CHIP_EINVAL;
-    if (!weights_aligned(type, W, nb01) || !weights_aligned(type, W, nb02) || nb01 < chip_row_size(type, K) ||
+    if (!weights_aligned(type, W, nb01, K) || !weights_aligned(type, W, nb02, K) || nb01 < chip_row_size(type, K) ||
         nb02 < (size_t)N * nb01)
         return CHIP_EINVAL;
     if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0 || (((uintptr_t)ids) & 3) != 0)
@@ -646,7 +652,7 @@ int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     if (!chip_mul_mat_supported(type, K) || type == T_F16) return CHIP_EUNSUPPORTED;   // F16 has no integer sums
     if (N == 0 || n == 0) return CHIP_OK;
     if (!W || !aq || !isum) return CHIP_EINVAL;
-    if (!weights_aligned(type, W, nb01) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;
+    if (!weights_aligned(type, W, nb01, K) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;
     return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, (type == T_Q4_K || type == T_Q5_K) ? imin : nullptr, (hipStream_t)stream));
 }
 

@@ -235,7 +235,8 @@ bool mul_mat_shape_ok(const lm_ggml_tensor *op) {
     if (w->ne[2] != 1 || w->ne[3] != 1 || x->ne[2] != 1 || x->ne[3] != 1) return false;
     if (x->ne[0] != w->ne[0] || op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1]) return false;
     if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, w->ne[0])) return false;
-    if (w->nb[1] % (w->type == LM_GGML_TYPE_Q6_K ? 2 : 16) != 0) return false;
+    // rows of K % 256 != 0 (32-value block types only) are multiples of 4 bytes
+    if (w->nb[1] % (w->type == LM_GGML_TYPE_Q6_K ? 2 : (w->ne[0] % 256 != 0 ? 4 : 16)) != 0) return false;
     if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)x->ne[0] * 4) return false;
     if (op->nb[0] != sizeof(float) || op->nb[1] % 4 != 0 || op->nb[1] < (size_t)op->ne[0] * 4) return false;
     return true;
@@ -267,6 +268,7 @@ bool mul_mat_id_shape_ok(const lm_ggml_tensor *op) {
     if (!chip_mul_mat_supported(w->type, w->ne[0])) return false;
     if (x->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32 || ids->type != LM_GGML_TYPE_I32) return false;
     const int64_t K = w->ne[0], N = w->ne[1], n_used = ids->ne[0], n_tokens = ids->ne[1];
+    if (K % 256 != 0) return false;                                     // the expert kernels assume 16-byte aligned rows
     if (w->ne[3] != 1 || x->ne[3] != 1 || op->ne[3] != 1 || ids->ne[2] != 1 || ids->ne[3] != 1) return false;
     if (x->ne[0] != K || x->ne[2] != n_tokens || !(x->ne[1] == 1 || x->ne[1] == n_used)) return false;
     if (op->ne[0] != N || op->ne[1] != n_used || op->ne[2] != n_tokens) return false;

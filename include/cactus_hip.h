@@ -127,8 +127,10 @@ CHIP_API int chip_convert_f32_to_f16(const float *x, int64_t ldx, int64_t n, int
  * n <= 4 runs the dot-product GEMV with the quantizer in its prologue; Q8_0 with n >= 5 the matrix-core GEMV
  * (16 tokens per pass over W); from 16 to 48 tokens on (by type and matrix size) the MFMA GEMM of the weight type;
  * everything else the GEMV in token groups.
- * K must be a multiple of 256.  W must be 16-byte aligned and nb01 a multiple of 16 (2 and 2 for Q6_K, whose
- * 210-byte blocks allow no more); x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
+ * K must be a multiple of 256; for the types of 32-value blocks (Q4_0, Q8_0, Q5_0, IQ4_NL, Q4_1, Q5_1) a multiple of 64
+ * is enough (hidden sizes such as 576, 896, 960: the GEMV, and the GEMM when K % 128 == 0).  W must be 16-byte aligned
+ * and nb01 a multiple of 16 (2 and 2 for Q6_K, whose 210-byte blocks allow no more; 4 and 4 for rows of K % 256 != 0);
+ * x 16-byte aligned with ldx a multiple of 4; y 4-byte aligned.
  */
 CHIP_API size_t chip_mul_mat_workspace_size(int type, int64_t K, int64_t n);
 /* The same plus room for the partial outputs of a GEMM whose K is split over workgroups (when the output has fewer

@@ -84,6 +84,36 @@ def test_one_node_graph(host, orc, wt, n):
     L.lm_ggml_free(ctx)
 
 
+@pytest.mark.parametrize("wt", (O.Q8_0, O.Q4_0, O.Q5_1), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,n", [(576, 1), (960, 9), (896, 40)])
+def test_one_node_graph_with_a_hidden_size_that_is_no_multiple_of_256(host, orc, wt, K, n):
+    """Small models have hidden sizes such as 576, 896 or 960: rows of the 32-value block types that are multiples of 4
+    bytes only.  The backend takes them (GEMV; the GEMM at K = 896 with 40 tokens)."""
+    L = host.L
+    N = 300
+    wq = orc.quantize_weights(wt, common.weights_f32(wt + K, N, K))
+    x = common.activations_f32(wt + K + n, n, K)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    ctx = host.context()
+    a = host.tensor_2d(ctx, wt, K, N, "w")
+    b = host.tensor_2d(ctx, O.F32, K, n, "x")
+    c = L.lm_ggml_mul_mat(ctx, a, b)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, c)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    assert L.lm_ggml_backend_dev_supports_op(dev, c) is True
+    host.set(a, wq)
+    host.set(b, x)
+    assert L.lm_ggml_backend_graph_compute(be, g) == 0
+    y = host.get(c, np.float32, (n, N))
+    ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("sum_abs",))
+    assert (np.abs(y.astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all()
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_free(ctx)
+
+
 def test_unsupported_ops_are_declined(host):
     L = host.L
     dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)

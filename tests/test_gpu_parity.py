@@ -295,6 +295,27 @@ def test_argument_errors(dev):
     dev.sync()
 
 
+# ------------------------------------------------------------------------------------------ rows of K % 256 != 0
+@pytest.mark.parametrize("wt", (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL, O.Q4_1, O.Q5_1), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N", [(576, 1536), (896, 151), (960, 2560), (4160, 300), (64, 5)])
+def test_block32_rows_of_k_not_a_multiple_of_256(dev, orc, wt, K, N):
+    """Hidden sizes such as 576, 896 and 960 (K % 64 == 0): the rows of the 32-value block types are then multiples of 4
+    bytes only.  Every token count class: prologue-quantizing GEMV (1, 2, 4), GEMV over the workspace (3, 5, 8), several
+    passes (11, 20), and from 17 tokens the GEMM where K % 128 == 0 (896, 960 is not: passes)."""
+    import cactus_amd as ca
+    assert dev.lib.chip_mul_mat_supported(wt, K) == 1
+    wq = quantized_weights(wt, 7 * K + N, N, K)
+    for n in (1, 2, 3, 4, 5, 8, 11, 20, 70):
+        x = common.activations_f32(K + n, n, K)
+        ref = orc.mul_mat(wt, wq, x, nthreads=8, want=("wdata", "sum_abs"))
+        y, blocks = dev.mul_mat(wt, wq, x, want_workspace_blocks=True)
+        assert np.array_equal(blocks, ref["wdata"]), n
+        check_outputs(y, ref["y"], ref["sum_abs"], "K %% 256 != 0, n = %d" % n)
+    for t in (O.Q4_K, O.Q5_K, O.Q6_K):
+        assert dev.lib.chip_mul_mat_supported(t, K) == 0                 # super-blocks of 256 values
+    assert dev.lib.chip_mul_mat_supported(wt, K + 32) == 0              # an odd number of blocks: rows of 2-byte alignment
+
+
 # ------------------------------------------------------------------------------------------ prefill GEMM (int8 MFMA)
 B32_TYPES = (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL, O.Q4_1, O.Q5_1)
 
