@@ -496,6 +496,63 @@ int chip_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t l
         return CHIP_EINVAL;
     return hip_rc(launch_add_rms_norm_mul(a, lda, b, ldb, sum, ld_sum, n, ne0, eps, w, nullptr, 0, y, ldy, (hipStream_t)stream));
 }
+int chip_scale(const float *x, int64_t ldx, int64_t n, int64_t ne0, float scale, float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0)) return CHIP_EINVAL;
+    return hip_rc(launch_scale(x, ldx, ne0, n, scale, y, ldy, (hipStream_t)stream));
+}
+// fp16 <-> fp32 on the host, round to nearest even (the conversions lm_ggml_cpu_init uses for its tables)
+static float half_bits_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 31u, man = h & 0x3ffu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) bits = sign;
+        else {                                                           // subnormal half: man * 2^-24
+            float f = (float)man * 5.9604644775390625e-8f;
+            std::memcpy(&bits, &f, 4);
+            bits |= sign;
+        }
+    } else if (exp == 31) bits = sign | 0x7f800000u | (man << 13);
+    else bits = sign | ((exp + 112u) << 23) | (man << 13);
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+static uint16_t float_to_half_bits(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u, ax = x & 0x7fffffffu;
+    if (ax > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((ax & 0x7fffffu) >> 13));   // NaN: quiet, payload kept (as vcvtps2ph does)
+    if (ax >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);                          // rounds to 65536 or more, or inf
+    if (ax < 0x33000001u) return (uint16_t)sign;                                       // at most half the smallest subnormal
+    const int e = (int)(ax >> 23) - 127;
+    uint32_t man = (ax & 0x7fffffu) | 0x800000u;
+    if (e < -14) {                                                                     // subnormal half: units of 2^-24
+        const int shift = -e - 1;                                                      // 14 .. 24
+        const uint32_t q = man >> shift, rem = man & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+        return (uint16_t)(sign | (q + ((rem > halfway || (rem == halfway && (q & 1u))) ? 1u : 0u)));
+    }
+    uint32_t h = ((uint32_t)(e + 15) << 10) | ((man >> 13) & 0x3ffu);
+    const uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;                            // a carry moves into the exponent as it should
+    return (uint16_t)(sign | h);
+}
+int chip_gelu_table(uint16_t *table) {
+    if (!table) return CHIP_EINVAL;
+    const float coef_a = 0.044715f, sqrt_2_over_pi = 0.79788456080286535587989211986876f;
+    for (uint32_t i = 0; i < 65536u; i++) {
+        const float x = half_bits_to_float((uint16_t)i);
+        table[i] = float_to_half_bits(0.5f * x * (1.0f + tanhf(sqrt_2_over_pi * x * (1.0f + coef_a * x * x))));
+    }
+    return CHIP_OK;
+}
+int chip_gelu(const float *x, int64_t ldx, int64_t n, int64_t ne0, const uint16_t *table, float *y, int64_t ldy, void *stream) {
+    if (n < 0 || ne0 < 0) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0) || !table || (((uintptr_t)table) & 1) != 0) return CHIP_EINVAL;
+    return hip_rc(launch_gelu(x, ldx, ne0, n, table, y, ldy, (hipStream_t)stream));
+}
 int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream) {
     if (n < 0 || ne0 < 0) return CHIP_EINVAL;
     if (n == 0 || ne0 == 0) return CHIP_OK;

@@ -15,6 +15,7 @@
 #include "../../include/ggml_backend_hip.h"
 
 #include <atomic>
+#include <dlfcn.h>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -52,6 +53,7 @@ struct backend_ctx {
     float *rope_table = nullptr; size_t rope_table_bytes = 0;
     rope_table_key rope_key = {};
     quantized_key quantized = {};
+    uint16_t *gelu_table = nullptr;                  // device copy of the 65536-entry fp16 GELU table
 };
 
 lm_ggml_backend_buffer_type_t hip_buffer_type();
@@ -199,6 +201,7 @@ void backend_free(lm_ggml_backend_t backend) {
     chip_stream_synchronize(c->stream);
     chip_free(c->workspace);
     chip_free(c->rope_table);
+    chip_free(c->gelu_table);
     chip_stream_destroy(c->stream);
     delete c;
     delete backend;
@@ -309,7 +312,8 @@ bool elementwise_shape_ok(const lm_ggml_tensor *op) {
     if (!a || !as_rows(op, r, ld) || !as_rows(a, r, ld) || !same_shape(op, a)) return false;
     switch (op->op) {
         case LM_GGML_OP_RMS_NORM: return true;
-        case LM_GGML_OP_UNARY:    return op->op_params[0] == LM_GGML_UNARY_OP_SILU && a->ne[0] % 8 == 0;
+        case LM_GGML_OP_SCALE:    return true;
+        case LM_GGML_OP_UNARY:    return (op->op_params[0] == LM_GGML_UNARY_OP_SILU && a->ne[0] % 8 == 0) || op->op_params[0] == LM_GGML_UNARY_OP_GELU;
         case LM_GGML_OP_ADD:
         case LM_GGML_OP_MUL:
             // src1: the shape of src0, or one row broadcast over all rows (norm weights, biases)
@@ -318,6 +322,28 @@ bool elementwise_shape_ok(const lm_ggml_tensor *op) {
         default: return false;
     }
 }
+// The table of LM_GGML_UNARY_OP_GELU on the device.  The host framework's own table (lm_ggml_table_gelu_f16, filled by
+// lm_ggml_cpu_init, reference ggml-cpu/ggml-cpu.c:3474-3481) is taken when this process exports it and it is filled: the
+// device then returns exactly what that framework's CPU backend returns, whatever compiler and C library built it.
+// Otherwise the same formula is evaluated here.
+bool ensure_gelu_table(backend_ctx *c) {
+    if (c->gelu_table) return true;
+    static uint16_t host_table[65536];
+    const uint16_t *src = (const uint16_t *)dlsym(RTLD_DEFAULT, "lm_ggml_table_gelu_f16");
+    if (!src || src[0x3c00] == 0) {                                     // gelu(1.0) is 0.84: a zero entry means "not initialised"
+        if (chip_gelu_table(host_table) != CHIP_OK) return false;
+        src = host_table;
+    }
+    void *dev = nullptr;
+    if (chip_malloc(&dev, sizeof(host_table)) != CHIP_OK) return false;
+    if (chip_memcpy_h2d(dev, src, sizeof(host_table), c->stream) != CHIP_OK || chip_stream_synchronize(c->stream) != CHIP_OK) {
+        chip_free(dev);
+        return false;
+    }
+    c->gelu_table = (uint16_t *)dev;
+    return true;
+}
+
 int run_elementwise(backend_ctx *c, lm_ggml_tensor *op) {
     const lm_ggml_tensor *a = op->src[0], *b = op->src[1];
     int64_t rows, lda, ldy, rb = 0, ldb = 0;
@@ -330,7 +356,16 @@ int run_elementwise(backend_ctx *c, lm_ggml_tensor *op) {
             std::memcpy(&eps, op->op_params, sizeof(float));
             return chip_rms_norm((const float *)a->data, lda, rows, ne0, eps, (float *)op->data, ldy, c->stream);
         }
+        case LM_GGML_OP_SCALE: {
+            float v;
+            std::memcpy(&v, op->op_params, sizeof(float));
+            return chip_scale((const float *)a->data, lda, rows, ne0, v, (float *)op->data, ldy, c->stream);
+        }
         case LM_GGML_OP_UNARY:
+            if (op->op_params[0] == LM_GGML_UNARY_OP_GELU) {
+                if (!ensure_gelu_table(c)) return CHIP_ENOMEM;
+                return chip_gelu((const float *)a->data, lda, rows, ne0, c->gelu_table, (float *)op->data, ldy, c->stream);
+            }
             return chip_silu((const float *)a->data, lda, rows, ne0, (float *)op->data, ldy, c->stream);
         default:
             as_rows(b, rb, ldb);
@@ -625,7 +660,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 continue;
             }
         }
-        if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_UNARY) && elementwise_shape_ok(node) && fusion_enabled()) {
+        if ((node->op == LM_GGML_OP_RMS_NORM || (node->op == LM_GGML_OP_UNARY && node->op_params[0] == LM_GGML_UNARY_OP_SILU)) &&
+            elementwise_shape_ok(node) && fusion_enabled()) {
             bool fused = false;
             const int rc = try_fused_pair(c, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused);
             if (rc != CHIP_OK) {
@@ -645,8 +681,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 continue;
             }
         }
-        if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_ADD || node->op == LM_GGML_OP_MUL || node->op == LM_GGML_OP_UNARY) &&
-            elementwise_shape_ok(node)) {
+        if ((node->op == LM_GGML_OP_RMS_NORM || node->op == LM_GGML_OP_ADD || node->op == LM_GGML_OP_MUL || node->op == LM_GGML_OP_UNARY ||
+             node->op == LM_GGML_OP_SCALE) && elementwise_shape_ok(node)) {
             const int rc = run_elementwise(c, node);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
@@ -803,7 +839,8 @@ void dev_event_synchronize(lm_ggml_backend_dev_t, lm_ggml_backend_event_t event)
 bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     if (is_view_op(op->op)) return true;
     // element-wise F32 ops run wherever their operands are put: the scheduler keeps them with the matmuls around them
-    if (op->op == LM_GGML_OP_RMS_NORM || op->op == LM_GGML_OP_ADD || op->op == LM_GGML_OP_MUL || op->op == LM_GGML_OP_UNARY)
+    if (op->op == LM_GGML_OP_RMS_NORM || op->op == LM_GGML_OP_ADD || op->op == LM_GGML_OP_MUL || op->op == LM_GGML_OP_UNARY ||
+        op->op == LM_GGML_OP_SCALE)
         return elementwise_shape_ok(op);
     if (is_attn_side_op(op->op)) return attn_side_shape_ok(op);
     if (op->op != LM_GGML_OP_MUL_MAT && op->op != LM_GGML_OP_MUL_MAT_ID) return false;

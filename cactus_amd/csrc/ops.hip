@@ -201,6 +201,39 @@ __global__ __launch_bounds__(EW_THREADS) void elementwise_kernel(const float *__
     }
 }
 
+// ---- SCALE and GELU: one value in, one value out ----
+// GELU is the reference's table form (ggml-cpu/vec.h:452-466): 0 at or below -10, x at or above 10, else entry fp16(x) of
+// a 65536-entry fp16 table built on the host with the C library's tanhf (the caller uploads it).
+enum { UN_SCALE = 0, UN_GELU = 1 };
+template <int OP> __device__ __forceinline__ float unary_apply(float x, float s, const unsigned short *__restrict__ table) {
+    if constexpr (OP == UN_SCALE) return x * s;
+    else {
+        if (x <= -10.0f) return 0.0f;
+        if (x >= 10.0f) return x;
+        return h2f(table[f2h_rne(x)]);
+    }
+}
+template <int OP, bool VEC>
+__global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restrict__ x, int64_t ldx, int64_t ne0, int64_t n,
+                                                           float *__restrict__ y, int64_t ldy, float s,
+                                                           const unsigned short *__restrict__ table) {
+    for (int64_t row = blockIdx.y; row < n; row += gridDim.y) {
+        const float *xr = x + (size_t)row * ldx;
+        float *yr = y + (size_t)row * ldy;
+        if constexpr (VEC) {
+            const int64_t i = 4 * ((int64_t)blockIdx.x * EW_THREADS + threadIdx.x);
+            if (i < ne0) {
+                const float4 v = *reinterpret_cast<const float4 *>(xr + i);
+                *reinterpret_cast<float4 *>(yr + i) = make_float4(unary_apply<OP>(v.x, s, table), unary_apply<OP>(v.y, s, table),
+                                                                  unary_apply<OP>(v.z, s, table), unary_apply<OP>(v.w, s, table));
+            }
+        } else {
+            for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < ne0; i += (int64_t)gridDim.x * EW_THREADS)
+                yr[i] = unary_apply<OP>(xr[i], s, table);
+        }
+    }
+}
+
 // ---- SOFT_MAX: one workgroup per row; thread t owns the groups of 8 values t, t + 256, ... ----
 // G > 0: the row fits 8 * G * EW_THREADS values and stays in registers.  G == 0: any length, y holds e between passes.
 enum { MASK_NONE = 0, MASK_F32 = 1, MASK_F16 = 2 };
@@ -730,6 +763,30 @@ hipError_t launch_silu_mul(const float *x, int64_t ldx, const float *b, int64_t 
                            hipStream_t st) { return launch_ew<EW_SILU_MUL>(x, ldx, b, ldb, ne0, n, y, ldy, st); }
 hipError_t launch_silu(const float *x, int64_t ldx, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st) {
     return launch_ew<EW_SILU>(x, ldx, nullptr, 0, ne0, n, y, ldy, st);
+}
+
+template <int OP>
+static hipError_t launch_unary(const float *x, int64_t ldx, int64_t ne0, int64_t n, float *y, int64_t ldy, float s,
+                               const unsigned short *table, hipStream_t st) {
+    if (n <= 0 || ne0 <= 0) return hipSuccess;
+    const bool vec = ((ne0 | ldx | ldy) & 3) == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
+    const unsigned gy = (unsigned)(n < 32768 ? n : 32768);
+    if (vec) {
+        hipLaunchKernelGGL((unary_kernel<OP, true>), dim3((unsigned)ceil_div(ne0, 4 * EW_THREADS), gy), dim3(EW_THREADS), 0, st, x, ldx,
+                           ne0, n, y, ldy, s, table);
+    } else {
+        const int64_t want = ceil_div(ne0, EW_THREADS);
+        hipLaunchKernelGGL((unary_kernel<OP, false>), dim3((unsigned)(want < 64 ? want : 64), gy), dim3(EW_THREADS), 0, st, x, ldx, ne0,
+                           n, y, ldy, s, table);
+    }
+    return hipGetLastError();
+}
+hipError_t launch_scale(const float *x, int64_t ldx, int64_t ne0, int64_t n, float s, float *y, int64_t ldy, hipStream_t st) {
+    return launch_unary<UN_SCALE>(x, ldx, ne0, n, y, ldy, s, nullptr, st);
+}
+hipError_t launch_gelu(const float *x, int64_t ldx, int64_t ne0, int64_t n, const unsigned short *table, float *y, int64_t ldy,
+                       hipStream_t st) {
+    return launch_unary<UN_GELU>(x, ldx, ne0, n, y, ldy, 0.0f, table, st);
 }
 
 }  // namespace chip

@@ -201,6 +201,16 @@ CHIP_API int chip_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t n
                                int64_t ld_norm, float *y, int64_t ldy, void *stream);
 CHIP_API int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy,
                            void *stream);
+/* LM_GGML_OP_SCALE (lm_ggml_compute_forward_scale_f32, ggml-cpu/ops.cpp:3930-3968): y = x * scale, one fp32 multiply.
+ * LM_GGML_UNARY_OP_GELU on F32 (lm_ggml_vec_gelu_f32 with LM_GGML_GELU_FP16, ggml-cpu/vec.h:16,452-466): 0 at or below -10,
+ * x at or above 10, else entry fp16(x) of the 65536-entry fp16 table of lm_ggml_cpu_init (ggml-cpu/ggml-cpu.c:3474-3481).
+ * `table` is that table in device memory (128 KiB): chip_gelu_table computes it on the host, with this process's tanhf,
+ * for the caller to upload - or the caller uploads the host framework's own lm_ggml_table_gelu_f16, as the ggml
+ * backend does, and is then bit-identical to that framework's CPU path whatever it was compiled with. */
+CHIP_API int chip_scale(const float *x, int64_t ldx, int64_t n, int64_t ne0, float scale, float *y, int64_t ldy, void *stream);
+CHIP_API int chip_gelu_table(uint16_t *table_host_65536);
+CHIP_API int chip_gelu(const float *x, int64_t ldx, int64_t n, int64_t ne0, const uint16_t *table, float *y, int64_t ldy,
+                       void *stream);
 CHIP_API int chip_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
                                    int64_t ne0, float eps, const float *w, float *y, int64_t ldy, void *stream);
 

@@ -38,12 +38,12 @@ enum {
 };
 enum {
     LM_GGML_OP_NONE = 0, LM_GGML_OP_ADD = 2, LM_GGML_OP_MUL = 6, LM_GGML_OP_RMS_NORM = 23,
-    LM_GGML_OP_MUL_MAT = 27, LM_GGML_OP_MUL_MAT_ID = 28, LM_GGML_OP_UNARY = 74,
+    LM_GGML_OP_MUL_MAT = 27, LM_GGML_OP_MUL_MAT_ID = 28, LM_GGML_OP_SCALE = 30, LM_GGML_OP_UNARY = 74,
     LM_GGML_OP_DUP = 1, LM_GGML_OP_GET_ROWS = 38, LM_GGML_OP_CPY = 32, LM_GGML_OP_CONT = 33, LM_GGML_OP_SOFT_MAX = 43, LM_GGML_OP_ROPE = 45,
     LM_GGML_OP_RESHAPE = 34, LM_GGML_OP_VIEW = 35, LM_GGML_OP_PERMUTE = 36, LM_GGML_OP_TRANSPOSE = 37,
     LM_GGML_OP_COUNT = 82,
 };
-enum { LM_GGML_UNARY_OP_SILU = 10 };
+enum { LM_GGML_UNARY_OP_GELU = 8, LM_GGML_UNARY_OP_SILU = 10 };
 enum { LM_GGML_STATUS_ALLOC_FAILED = -2, LM_GGML_STATUS_FAILED = -1, LM_GGML_STATUS_SUCCESS = 0, LM_GGML_STATUS_ABORTED = 1 };
 enum { LM_GGML_BACKEND_DEVICE_TYPE_CPU = 0, LM_GGML_BACKEND_DEVICE_TYPE_GPU = 1, LM_GGML_BACKEND_DEVICE_TYPE_ACCEL = 2 };
 enum { LM_GGML_BACKEND_BUFFER_USAGE_ANY = 0, LM_GGML_BACKEND_BUFFER_USAGE_WEIGHTS = 1, LM_GGML_BACKEND_BUFFER_USAGE_COMPUTE = 2 };

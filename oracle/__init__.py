@@ -132,6 +132,10 @@ class Oracle:
         L.orc_rms_norm_f32.argtypes = [_vp, _vp, _i64, _i64, C.c_float]
         L.orc_silu_f32.restype = None
         L.orc_silu_f32.argtypes = [_vp, _vp, _i64, _i64]
+        L.orc_gelu_f32.restype = None
+        L.orc_gelu_f32.argtypes = [_vp, _vp, _i64]
+        L.orc_gelu_table.restype = None
+        L.orc_gelu_table.argtypes = [_vp]
         L.orc_soft_max_f32.restype = None
         L.orc_soft_max_f32.argtypes = [_vp, _vp, _i32, _i64, _i64, _i64, _i64, C.c_float, C.c_float, _vp]
         L.orc_rope_f32.restype = None
@@ -281,6 +285,25 @@ class Oracle:
         y = np.empty_like(x)
         self.lib.orc_silu_f32(_ptr(x), _ptr(y), x.shape[0], x.shape[1])
         return y
+
+    def gelu(self, x):
+        """LM_GGML_UNARY_OP_GELU over x fp32 (any shape): the reference's fp16-table form."""
+        x = _f32(x)
+        y = np.empty_like(x)
+        self.lib.orc_gelu_f32(_ptr(x), _ptr(y), x.size)
+        return y
+
+    def gelu_table(self):
+        """The 65536 fp16 entries lm_ggml_cpu_init computes (as uint16 bit patterns)."""
+        t = np.empty(65536, np.uint16)
+        self.lib.orc_gelu_table(_ptr(t))
+        return t
+
+    @staticmethod
+    def scale(x, v):
+        """LM_GGML_OP_SCALE (lm_ggml_compute_forward_scale_f32, reference ggml-cpu/ops.cpp:3930-3968): one fp32 multiply
+        per element (lm_ggml_vec_scale_f32, ggml-cpu/vec.h:264-293)."""
+        return _f32(x) * np.float32(v)
 
     def soft_max(self, x, mask=None, scale=1.0, max_bias=0.0):
         """LM_GGML_OP_SOFT_MAX (lm_ggml_soft_max_ext): x fp32 [n_head, ne01, ne00]; mask fp32 or fp16 [>= ne01, ne00] or
@@ -586,6 +609,31 @@ class Reference:
         L.lm_ggml_backend_free(be)
         L.lm_ggml_free(ctx)
         return y
+
+    def unary_graph(self, name, x, nthreads=1):
+        """lm_ggml_gelu / lm_ggml_silu (name) on the reference CPU backend: x fp32 [n, ne0]."""
+        L = self.lib
+        x = _f32(x)
+        fn = getattr(L, "lm_ggml_" + name)
+        fn.restype = _vp
+        fn.argtypes = [_vp, _vp]
+
+        def build(ctx):
+            tx = L.lm_ggml_new_tensor_2d(ctx, F32, x.shape[1], x.shape[0])
+            return fn(ctx, tx), {"x": tx}
+        return self._run_graph(build, {"x": x}, x.shape, np.float32, nthreads)
+
+    def scale_graph(self, x, v, nthreads=1):
+        """lm_ggml_scale on the reference CPU backend: x fp32 [n, ne0]."""
+        L = self.lib
+        x = _f32(x)
+        L.lm_ggml_scale.restype = _vp
+        L.lm_ggml_scale.argtypes = [_vp, _vp, C.c_float]
+
+        def build(ctx):
+            tx = L.lm_ggml_new_tensor_2d(ctx, F32, x.shape[1], x.shape[0])
+            return L.lm_ggml_scale(ctx, tx, v), {"x": tx}
+        return self._run_graph(build, {"x": x}, x.shape, np.float32, nthreads)
 
     def soft_max_graph(self, x, mask=None, scale=1.0, max_bias=0.0, nthreads=1):
         """lm_ggml_soft_max_ext on the reference CPU backend: x fp32 [n_head, ne01, ne00], mask fp32 / fp16 [>= ne01, ne00]."""

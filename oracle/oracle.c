@@ -1315,6 +1315,28 @@ void orc_silu_f32(const float *x, float *y, int64_t n_rows, int64_t ne0) {
     }
 }
 
+/* LM_GGML_UNARY_OP_GELU on F32 rows: lm_ggml_vec_gelu_f32 in its LM_GGML_GELU_FP16 form (reference ggml-cpu/vec.h:16, 452-466):
+ * 0 at or below -10, x at or above 10, else the entry fp16(x) of a 65536-entry fp16 table, widened.  The table is what
+ * lm_ggml_cpu_init fills (ggml-cpu/ggml-cpu.c:3474-3481): entry h = fp16(lm_ggml_gelu_f32(fp32(h))) with
+ * lm_ggml_gelu_f32(x) = 0.5 x (1 + tanhf(sqrt(2/pi) x (1 + 0.044715 x x))) (vec.h:428-435) and the C library's tanhf. */
+void orc_gelu_table(uint16_t *table) {
+    static const float coef_a = 0.044715f, sqrt_2_over_pi = 0.79788456080286535587989211986876f;
+    for (uint32_t i = 0; i < 65536u; i++) {
+        const float x = H2F((uint16_t)i);
+        table[i] = F2H(0.5f * x * (1.0f + tanhf(sqrt_2_over_pi * x * (1.0f + coef_a * x * x))));
+    }
+}
+void orc_gelu_f32(const float *x, float *y, int64_t n) {
+    static uint16_t table[65536];
+    static int ready = 0;
+    if (!ready) { orc_gelu_table(table); ready = 1; }
+    for (int64_t i = 0; i < n; i++) {
+        if (x[i] <= -10.0f) y[i] = 0.0f;
+        else if (x[i] >= 10.0f) y[i] = x[i];
+        else y[i] = H2F(table[F2H(x[i])]);
+    }
+}
+
 /* lm_ggml_compute_forward_soft_max_f32 (reference ggml-cpu/ops.cpp:4731-4827) with lm_ggml_vec_soft_max_f32's AVX2 branch
  * (ggml-cpu/vec.cpp:198-208, 233-238).  Row i1 of x [n_rows][ne00]: w = x * scale + slope * mask[i1 % ne01] (mask fp32
  * or fp16, one [ne01][ne00] matrix shared by all heads), max over the row, e = lm_ggml_v_expf(w - max) in groups of 8

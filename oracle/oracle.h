@@ -146,6 +146,10 @@ int orc_mul_mat_id(int type, int64_t K, int64_t N, int64_t n_as, const void *W, 
  * single IEEE operations per element and need no restatement. */
 void orc_rms_norm_f32(const float *x, float *y, int64_t n_rows, int64_t ne0, float eps);
 void orc_silu_f32(const float *x, float *y, int64_t n_rows, int64_t ne0);
+/* LM_GGML_UNARY_OP_GELU through the reference's fp16 table (ggml-cpu/vec.h:452-466, table of ggml-cpu/ggml-cpu.c:3474-3481);
+ * pinned bit-exact on oracle/_ref's lm_ggml_gelu graph, and by gelu(0) = 0, gelu(x) = x from 10 on, 0 down from -10. */
+void orc_gelu_table(uint16_t *table);
+void orc_gelu_f32(const float *x, float *y, int64_t n);
 
 /* Attention-side ops (ggml-cpu/ops.cpp), contiguous rows.  orc_soft_max_f32: pinned bit-exact on oracle/_ref's
  * lm_ggml_soft_max_ext graphs.  orc_rope_f32: pinned bit-exact on oracle/_ref's lm_ggml_rope_ext graphs on this host (both

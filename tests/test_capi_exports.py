@@ -42,3 +42,17 @@ def test_layout_queries_need_no_gpu():
     # Q8_K planes (qs, d, bsums) of K = 4096 take 4672 bytes; token strides are multiples of 128
     assert lib.chip_mul_mat_workspace_size(cactus_amd.Q4_K, 4096, 3) == 3 * 4736
     assert lib.chip_error_string(-2).decode().startswith("unsupported")
+
+
+def test_gelu_table_is_the_reference_table():
+    """chip_gelu_table runs on the host (no GPU): the 65536 fp16 entries equal the oracle's restatement of lm_ggml_cpu_init's
+    loop (pinned on the reference build in test_oracle_vs_ref), NaN entries included."""
+    import ctypes as C
+    import numpy as np
+    import cactus_amd
+    import oracle as O
+    lib = C.CDLL(cactus_amd.KERNEL_LIB)
+    t = np.zeros(65536, np.uint16)
+    assert lib.chip_gelu_table(t.ctypes.data_as(C.c_void_p)) == 0
+    assert np.array_equal(t, O.Oracle().gelu_table())
+    assert t[0x3c00] != 0 and t[0] == 0                                  # gelu(1) = 0.84, gelu(0) = 0

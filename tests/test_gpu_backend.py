@@ -538,6 +538,48 @@ def test_residual_add_runs_with_the_norm_that_follows(host, orc):
     L.lm_ggml_free(wctx)
 
 
+def test_gelu_and_scale_nodes(host, orc):
+    """A GELU-gated FFN entry and a SCALE (Gemma-style graphs: lm_ggml_gelu, lm_ggml_scale): both run on the device, and the
+    GELU goes through the host framework's own table, so the result equals the reference CPU backend bit for bit."""
+    L = host.L
+    L.lm_ggml_gelu.restype = C.c_void_p
+    L.lm_ggml_gelu.argtypes = [C.c_void_p, C.c_void_p]
+    L.lm_ggml_scale.restype = C.c_void_p
+    L.lm_ggml_scale.argtypes = [C.c_void_p, C.c_void_p, C.c_float]
+    n, ne0 = 5, 1152
+    x = (common.activations_f32(77, n, ne0) * 3).astype(np.float32)
+    u = common.activations_f32(78, n, ne0)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    ctx = host.context()
+    tx = host.tensor_2d(ctx, O.F32, ne0, n, "x")
+    tu = host.tensor_2d(ctx, O.F32, ne0, n, "u")
+    L.lm_ggml_set_input(tx); L.lm_ggml_set_input(tu)
+    gl = L.lm_ggml_gelu(ctx, tx)
+    act = L.lm_ggml_mul(ctx, gl, tu)
+    out = L.lm_ggml_scale(ctx, act, 0.0625)
+    L.lm_ggml_set_output(out)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, out)
+    for t in (gl, act, out):
+        assert L.lm_ggml_backend_dev_supports_op(dev, t) is True
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 64, False, True)
+    for t in (gl, act, out):
+        L.lm_ggml_backend_sched_set_tensor_backend(sched, t, hip)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(tx, x); host.set(tu, u)
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    y = host.get(out, np.float32, (n, ne0))
+    want = orc.scale(orc.gelu(x) * u, 0.0625)
+    assert y.tobytes() == want.tobytes()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+
+
 def test_attention_side_nodes_run_on_the_device(host, orc):
     """The nodes llama.cpp puts around the KV cache (reference llama-graph.cpp:1060-1166, llama-kv-cache.cpp:617-656): RoPE of
     Q and K, the K store (F32 -> F16 into a 1-D view of the cache), the transposed V store, the masked soft-max and the

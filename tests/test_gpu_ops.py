@@ -165,3 +165,38 @@ def test_fused_add_norm_equals_the_separate_ops(dev, n, ne0, with_w):
     da = dev.to_device(a)
     assert dev.lib.chip_add_rms_norm_mul(da.ptr, ne0, da.ptr, ne0, da.ptr, ne0, n, ne0, 1e-6, wp, da.ptr, ne0, None) == ca.CHIP_EINVAL
     da.free(); dw.free()
+
+
+def test_scale_and_gelu_equal_the_oracle(dev, orc):
+    """chip_scale: one multiply per element.  chip_gelu: the reference's fp16-table form, over every finite fp16 value, random
+    values that round to either neighbour, and the two cut-offs; rows with a stride, and a length that is no multiple of 4."""
+    import ctypes as C
+    rng = np.random.default_rng(21)
+    table = np.zeros(65536, np.uint16)
+    dev.check(dev.lib.chip_gelu_table(table.ctypes.data_as(C.c_void_p)))
+    dt = dev.to_device(table)
+    h = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    h = h[np.isfinite(h)]
+    edge = np.array([-10.0, np.nextafter(np.float32(-10), np.float32(0)), 10.0, np.nextafter(np.float32(10), np.float32(0)), 0.0, -0.0,
+                     1.0 + 2.0 ** -11, 1.0 + 2.0 ** -11 + 2.0 ** -20, 65519.0, 1e-8, -1e-8, 3e38, -3e38], np.float32)
+    flat = np.concatenate([h, (rng.standard_normal(20000) * 4).astype(np.float32), edge])
+    for ne0 in (64, 1001):
+        x = flat[: flat.size // ne0 * ne0].reshape(-1, ne0)
+        n = x.shape[0]
+        dx, dy = dev.to_device(x), dev.alloc(x.nbytes)
+        dev.check(dev.lib.chip_gelu(dx.ptr, ne0, n, ne0, dt.ptr, dy.ptr, ne0, None))
+        dev.sync()
+        with np.errstate(all="ignore"):
+            assert dy.download(np.float32, x.size).tobytes() == orc.gelu(x).tobytes()
+        for v in (0.125, 0.08838834764831845, -3.7):
+            dev.check(dev.lib.chip_scale(dx.ptr, ne0, n, ne0, v, dy.ptr, ne0, None))
+            dev.sync()
+            with np.errstate(all="ignore"):
+                assert dy.download(np.float32, x.size).tobytes() == orc.scale(x, v).tobytes()
+        dev.check(dev.lib.chip_scale(dx.ptr, ne0, n, ne0, 2.0, dx.ptr, ne0, None))                 # in place
+        dev.sync()
+        with np.errstate(all="ignore"):
+            assert dx.download(np.float32, x.size).tobytes() == (x * np.float32(2)).tobytes()
+        for t in (dx, dy):
+            t.free()
+    dt.free()

@@ -144,6 +144,39 @@ def test_soft_max_graph(orc, ref, n_head, ne01, ne00, threads):
     assert orc.soft_max(x, bias, 0.5, 8.0).tobytes() == ref.soft_max_graph(x, bias, 0.5, 8.0, nthreads=threads).tobytes()
 
 
+def test_gelu_graph(orc, ref):
+    """Every fp16 value (each entry of the reference's table), values that round to fp16 ties, and the two cut-offs."""
+    h = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    h = h[np.isfinite(h)]
+    rng = np.random.default_rng(12)
+    r = (rng.standard_normal(8192) * 4).astype(np.float32)
+    edge = np.array([-10.0, np.nextafter(np.float32(-10), np.float32(0)), 10.0, np.nextafter(np.float32(10), np.float32(0)), 0.0, -0.0,
+                     1.0 + 2.0 ** -11, 1.0 + 2.0 ** -11 + 2.0 ** -20, 65519.0, 1e-8, -1e-8, 3e38, -3e38], np.float32)
+    x = np.concatenate([h, r, edge])
+    x = np.concatenate([x, np.zeros(-x.size % 64, np.float32)]).reshape(-1, 64)
+    with np.errstate(all="ignore"):
+        assert orc.gelu(x).tobytes() == ref.unary_graph("gelu", x, nthreads=2).tobytes()
+
+
+def test_gelu_known_values(orc):
+    x = np.array([[0.0, 10.0, 25.0, -10.0, -30.0, 1.0, -1.0, 3.0]], np.float32)
+    y = orc.gelu(x)[0]
+    assert y[0] == 0.0 and y[1] == 10.0 and y[2] == 25.0 and y[3] == 0.0 and y[4] == 0.0
+    # the table holds fp16 values of 0.5 x (1 + tanh(...)): 0.8413 / -0.1587 / 2.996 to fp16 precision
+    want = [0.5 * v * (1 + np.tanh(np.sqrt(2 / np.pi) * v * (1 + 0.044715 * v * v))) for v in (1.0, -1.0, 3.0)]
+    assert np.allclose(y[5:], want, rtol=1e-3)
+    assert (orc.gelu(x).view(np.uint32) & 0x1fff == 0).all()             # every output is an fp16 number
+
+
+def test_scale_graph(orc, ref):
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((7, 96)) * 50).astype(np.float32)
+    x[0, :4] = [0.0, -0.0, 3e38, 1e-40]
+    for v in (0.125, 0.08838834764831845, -3.7, 1e30):
+        with np.errstate(all="ignore"):
+            assert orc.scale(x, v).tobytes() == ref.scale_graph(x, v).tobytes()
+
+
 def test_soft_max_rows_sum_to_one(orc):
     rng = np.random.default_rng(5)
     x = (rng.standard_normal((2, 4, 512)) * 4).astype(np.float32)
