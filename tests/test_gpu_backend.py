@@ -538,6 +538,47 @@ def test_residual_add_runs_with_the_norm_that_follows(host, orc):
     L.lm_ggml_free(wctx)
 
 
+def test_shared_quantized_input_is_dropped_when_the_input_is_overwritten(host, orc):
+    """Two matmuls read the same tensor, but an in-place SCALE rewrites it between them: the second matmul must quantize
+    again (same data pointer, same shape - only the write in between tells).  A third one after it reuses the new rows."""
+    import cactus_amd
+    L = host.L
+    L.lm_ggml_scale_inplace.restype = C.c_void_p
+    L.lm_ggml_scale_inplace.argtypes = [C.c_void_p, C.c_void_p, C.c_float]
+    K, N, n = 1024, 300, 6
+    w1 = orc.quantize_weights(O.Q4_K, common.weights_f32(91, N, K))
+    w2 = orc.quantize_weights(O.Q6_K, common.weights_f32(92, N, K))
+    x = common.activations_f32(93, n, K)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    ctx = host.context()
+    t1 = host.tensor_2d(ctx, O.Q4_K, K, N, "w1")
+    t2 = host.tensor_2d(ctx, O.Q6_K, K, N, "w2")
+    tx = host.tensor_2d(ctx, O.F32, K, n, "x")
+    y1 = L.lm_ggml_mul_mat(ctx, t1, tx)
+    xs = L.lm_ggml_scale_inplace(ctx, tx, 3.0)
+    y2 = L.lm_ggml_mul_mat(ctx, t2, xs)
+    y3 = L.lm_ggml_mul_mat(ctx, t1, xs)
+    g = L.lm_ggml_new_graph(ctx)
+    for t in (y1, y2, y3):
+        L.lm_ggml_build_forward_expand(g, t)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    host.set(t1, w1); host.set(t2, w2); host.set(tx, x)
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_quantizers_skipped.restype = C.c_ulonglong
+    before = blib.lm_ggml_backend_hip_get_quantizers_skipped()
+    assert L.lm_ggml_backend_graph_compute(be, g) == 0
+    assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - before == 1                 # y3 only
+    x3 = x * np.float32(3.0)
+    for t, wt, w, xin in ((y1, O.Q4_K, w1, x), (y2, O.Q6_K, w2, x3), (y3, O.Q4_K, w1, x3)):
+        ref = orc.mul_mat(wt, w, xin, nthreads=8, want=("sum_abs",))
+        y = host.get(t, np.float32, (n, N))
+        assert (np.abs(y.astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all()
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_free(ctx)
+
+
 def test_gelu_and_scale_nodes(host, orc):
     """A GELU-gated FFN entry and a SCALE (Gemma-style graphs: lm_ggml_gelu, lm_ggml_scale): both run on the device, and the
     GELU goes through the host framework's own table, so the result equals the reference CPU backend bit for bit."""
