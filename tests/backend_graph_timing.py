@@ -131,6 +131,17 @@ for it in range(20):
     t0 = time.perf_counter()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     ts.append(time.perf_counter() - t0)
+# the same split in two: how long the host needs to issue the launches, and the wait for the device after that
+L.lm_ggml_backend_sched_graph_compute_async.restype = C.c_int
+L.lm_ggml_backend_sched_graph_compute_async.argtypes = [C.c_void_p, C.c_void_p]
+L.lm_ggml_backend_sched_synchronize.argtypes = [C.c_void_p]
+issue = []
+for it in range(10):
+    t0 = time.perf_counter()
+    assert L.lm_ggml_backend_sched_graph_compute_async(sched, g) == 0
+    issue.append(time.perf_counter() - t0)
+    L.lm_ggml_backend_sched_synchronize(sched)
+print(f"NL={NL} n={n}: host time to issue one graph us: median {np.median(issue) * 1e6:.0f}", flush=True)
 ts = np.array(ts) * 1e6
 print(f"NL={NL} n={n}: graph_compute wall us: min {ts.min():.0f} median {np.median(ts):.0f} max {ts.max():.0f}", flush=True)
 y = host.get(out, np.float32, (n, H))
