@@ -493,11 +493,10 @@ def bench_trace(dev, hip, st, rng):
                 mm(*W["wq"], cur, q); mm(*W["wk"], cur, k, True); mm(*W["wv"], cur, v, True)
                 if l == 0:                                                # one cos / sin table per step, as the backend keeps it
                     ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
-                for t_, nh in ((q, n_head), (k, n_head_kv)):
-                    ck(L.chip_rope_apply(t_.ptr, hd, hd * nh, rope_tab.ptr, hd, nh, n, hd, 2, t_.ptr, hd, hd * nh, st))
-                flat, one = A4(n * KV, 1, 1, 1), n * KV
-                ck(L.chip_cpy(k.ptr, ca.F32, flat, A4(4, 4 * one, 4 * one, 4 * one), kc + 2 * KV * (n_kv - n), ca.F16, flat,
-                              A4(2, 2 * one, 2 * one, 2 * one), st))
+                ck(L.chip_rope_apply(q.ptr, hd, hd * n_head, rope_tab.ptr, hd, n_head, n, hd, 2, q.ptr, hd, hd * n_head, st))
+                # K: RoPE and the store into the F16 cache in one launch, as the backend runs the two nodes
+                ck(L.chip_rope_apply_store(k.ptr, hd, KV, rope_tab.ptr, hd, n_head_kv, n, hd, 2, k.ptr, hd, KV,
+                                           kc + 2 * KV * (n_kv - n), hd, KV, st))
                 shp = A4(n, KV, 1, 1)
                 ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))
                 ck(L.chip_mul_mat_f16_batched(kc, 2 * KV, 2 * hd, hd, n_kv, n_head_kv, q.ptr, hd * n_head, hd, n, n_head, kq.ptr, n_kv,

@@ -37,7 +37,7 @@ EXPORTS = (
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_scale", "chip_gelu_table", "chip_gelu",
-    "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
+    "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums",
     "chip_workspace_to_blocks",
 )
@@ -119,6 +119,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_rope.argtypes = [vp, i64, i64, vp, vp, i64, i64, i64, i32, i32, i32] + [C.c_float] * 6 + [vp, i64, i64, vp]
     L.chip_rope_table.argtypes = [vp, vp, i64, i32, i32] + [C.c_float] * 6 + [vp, vp]
     L.chip_rope_apply.argtypes = [vp, i64, i64, vp, i64, i64, i64, i32, i32, vp, i64, i64, vp]
+    L.chip_rope_apply_store.argtypes = [vp, i64, i64, vp, i64, i64, i64, i32, i32, vp, i64, i64, vp, i64, i64, vp]
     L.chip_get_rows.argtypes = [i32, vp, sz, sz, sz, i64, i64, vp, i64, i64, i64, i64, i64, vp, i64, i64, i64, vp]
     L.chip_mul_mat_f16_batched.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_f16_batched_workspace_size.restype = sz
@@ -312,13 +313,22 @@ class Device:
         return ddst.download(dst_dtype, dst_elems)
 
     def rope(self, x, pos, n_dims, mode, freq_factors=None, n_ctx_orig=4096, freq_base=10000.0, freq_scale=1.0,
-             ext_factor=0.0, attn_factor=1.0, beta_fast=32.0, beta_slow=1.0, two_step=False):
-        """x fp32 [n_tokens, n_head, ne0], pos int32 [n_tokens].  two_step: chip_rope_table + chip_rope_apply."""
+             ext_factor=0.0, attn_factor=1.0, beta_fast=32.0, beta_slow=1.0, two_step=False, store_f16=False):
+        """x fp32 [n_tokens, n_head, ne0], pos int32 [n_tokens].  two_step: chip_rope_table + chip_rope_apply.
+        store_f16: chip_rope_table + chip_rope_apply_store; returns (y fp32, y fp16)."""
         x = np.ascontiguousarray(x, np.float32)
         ne2, ne1, ne0 = x.shape
         dx, dy = self.to_device(x), self.alloc(x.nbytes)
         dp = self.to_device(np.ascontiguousarray(pos, np.int32))
         df = self.to_device(np.ascontiguousarray(freq_factors, np.float32)) if freq_factors is not None else None
+        if store_f16:
+            dt, dh = self.alloc(ne2 * n_dims * 4), self.alloc(x.size * 2)
+            self.check(self.lib.chip_rope_table(dp.ptr, df.ptr if df else None, ne2, n_dims, n_ctx_orig, freq_base, freq_scale,
+                                                ext_factor, attn_factor, beta_fast, beta_slow, dt.ptr, None))
+            self.check(self.lib.chip_rope_apply_store(dx.ptr, ne0, ne0 * ne1, dt.ptr, ne0, ne1, ne2, n_dims, mode, dy.ptr, ne0,
+                                                      ne0 * ne1, dh.ptr, ne0, ne0 * ne1, None))
+            self.sync()
+            return dy.download(np.float32, x.size).reshape(x.shape), dh.download(np.float16, x.size).reshape(x.shape)
         if two_step:
             dt = self.alloc(ne2 * n_dims * 4)
             self.check(self.lib.chip_rope_table(dp.ptr, df.ptr if df else None, ne2, n_dims, n_ctx_orig, freq_base, freq_scale,

@@ -688,19 +688,32 @@ int chip_rope_table(const int32_t *pos, const float *freq_factors, int64_t ne2, 
     return hip_rc(launch_rope(nullptr, pos, freq_factors, a, nullptr, table, true, (hipStream_t)stream));
 }
 
-int chip_rope_apply(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1, int64_t ne2,
-                    int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, void *stream) {
+static int rope_apply_checked(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1, int64_t ne2,
+                              int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, uint16_t *y16, int64_t ld16_1,
+                              int64_t ld16_2, void *stream) {
     if (ne0 == 0 && n_dims == 0) return CHIP_OK;
     if (int rc = rope_dims_checked(ne0, ne1, ne2, n_dims, mode); rc != CHIP_OK) return rc;
     if (ne0 == 0 || ne1 == 0 || ne2 == 0) return CHIP_OK;
     if (!x || !y || !table || ldx1 < ne0 || ldy1 < ne0 || ne2 > 0x7fffffff) return CHIP_EINVAL;
     if ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)table)) & 3) return CHIP_EINVAL;
+    if (y16 && (ld16_1 < ne0 || (((uintptr_t)y16) & 1) != 0)) return CHIP_EINVAL;
     RopeArgs a;
     a.ne0 = ne0; a.ne1 = ne1; a.ne2 = ne2;
     a.ldx1 = ldx1; a.ldx2 = ldx2; a.ldy1 = ldy1; a.ldy2 = ldy2;
     a.n_dims = n_dims; a.neox = (mode & 2) != 0;
     a.theta_scale = a.freq_scale = a.ext_factor = a.corr0 = a.corr1 = a.mscale = 0.0f;       // all in the table
+    a.y16 = y16; a.ld16_1 = ld16_1; a.ld16_2 = ld16_2;
     return hip_rc(launch_rope(x, nullptr, nullptr, a, y, const_cast<float *>(table), false, (hipStream_t)stream));
+}
+int chip_rope_apply(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1, int64_t ne2,
+                    int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, void *stream) {
+    return rope_apply_checked(x, ldx1, ldx2, table, ne0, ne1, ne2, n_dims, mode, y, ldy1, ldy2, nullptr, 0, 0, stream);
+}
+int chip_rope_apply_store(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1, int64_t ne2,
+                          int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, uint16_t *y_f16, int64_t ld16_1,
+                          int64_t ld16_2, void *stream) {
+    if (!y_f16) return CHIP_EINVAL;
+    return rope_apply_checked(x, ldx1, ldx2, table, ne0, ne1, ne2, n_dims, mode, y, ldy1, ldy2, y_f16, ld16_1, ld16_2, stream);
 }
 
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,

@@ -440,7 +440,8 @@ bool attn_side_shape_ok(const lm_ggml_tensor *op) {
         default:               return cpy_shape_ok(op);
     }
 }
-int run_attn_side(backend_ctx *c, lm_ggml_tensor *op) {
+// store: the F32 -> F16 CPY of the RoPE's result into a dense destination (the K cache store), run in the RoPE's kernel
+int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *store = nullptr) {
     const lm_ggml_tensor *a = op->src[0];
     switch (op->op) {
         case LM_GGML_OP_SOFT_MAX: {
@@ -481,6 +482,11 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op) {
                     c->rope_key = k;
                     g_rope_tables++;
                 }
+                if (store)
+                    return chip_rope_apply_store((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table,
+                                                 a->ne[0], a->ne[1], a->ne[2], op->op_params[1], op->op_params[2], (float *)op->data,
+                                                 (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), (uint16_t *)store->data, a->ne[0],
+                                                 a->ne[0] * a->ne[1], c->stream);
                 return chip_rope_apply((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table, a->ne[0],
                                        a->ne[1], a->ne[2], op->op_params[1], op->op_params[2], (float *)op->data,
                                        (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), c->stream);
@@ -610,11 +616,26 @@ bool silu_can_wait_for_its_mul(const lm_ggml_cgraph *g, int i) {
     return disjoint(mm, silu->src[0]) && disjoint(mm, silu);
 }
 
+// The RoPE of K followed (views aside) by the CPY of its result into the F16 cache (reference llama-kv-cache.cpp cpy_k:
+// a dense 1-D view of the cache): index of that CPY node, or -1.  The RoPE still writes its own F32 result.
+int rope_store_index(const lm_ggml_cgraph *g, int i) {
+    const lm_ggml_tensor *rope = g->nodes[i];
+    int j = i + 1;
+    while (j < g->n_nodes && is_view_op(g->nodes[j]->op)) j++;
+    if (j >= g->n_nodes) return -1;
+    const lm_ggml_tensor *cp = g->nodes[j];
+    if (cp->op != LM_GGML_OP_CPY || cp->src[0] != rope || cp->type != LM_GGML_TYPE_F16 || rope->type != LM_GGML_TYPE_F32) return -1;
+    if (!attn_side_shape_ok(cp) || !dense(cp) || !dense(rope) || n_elements(cp) != n_elements(rope)) return -1;
+    if (!disjoint(cp, rope) || !disjoint(cp, rope->src[0])) return -1;
+    return j;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
     c->quantized.valid = false;                       // and so may any activation
     const lm_ggml_tensor *waiting_silu = nullptr;     // a SILU held back for the MUL two nodes on
+    int stored_by_rope = -1;                          // index of a CPY node that ran inside the RoPE before it
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -691,8 +712,22 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             g_elementwise_nodes++;
             continue;
         }
+        if (i == stored_by_rope) {                    // this CPY ran in the kernel of the RoPE before it
+            stored_by_rope = -1;
+            continue;
+        }
         if (is_attn_side_op(node->op) && attn_side_shape_ok(node)) {
-            const int rc = run_attn_side(c, node);
+            const lm_ggml_tensor *store = nullptr;
+            if (node->op == LM_GGML_OP_ROPE && fusion_enabled()) {
+                stored_by_rope = rope_store_index(cgraph, i);
+                if (stored_by_rope >= 0) {
+                    store = cgraph->nodes[stored_by_rope];
+                    writes(store);
+                    g_elementwise_nodes++;
+                    g_fused_pairs++;
+                }
+            }
+            const int rc = run_attn_side(c, node, store);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
                 return LM_GGML_STATUS_FAILED;

@@ -228,6 +228,8 @@ struct RopeArgs {
     int64_t ldx1, ldx2, ldy1, ldy2;        // head and token strides in floats
     int n_dims, neox;
     float theta_scale, freq_scale, ext_factor, corr0, corr1, mscale;
+    unsigned short *y16 = nullptr;         // optional second output: y rounded to fp16 (the K cache store that follows a RoPE)
+    int64_t ld16_1 = 0, ld16_2 = 0;        // its head and token strides in halves
 };
 // LM_GGML_OP_GET_ROWS: dst row (i10, i11, i12) = row ids[i10, i11, i12] of matrix (i11, i12) of src, dequantized to F32.
 struct GetRowsArgs {

@@ -619,7 +619,7 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
     const uint32_t items = (uint32_t)a.ne1 * per_head;           // 32-bit division: the 64-bit one is a long software routine
     // the operands of the first PRE * EW_THREADS items do not depend on the table: fetch them first
     float x0[PRE], x1[PRE];
-    uint32_t ia[PRE], ib[PRE], jj[PRE];
+    uint32_t ia[PRE], ib[PRE], jj[PRE], ha[PRE], hb[PRE];       // ha / hb: where the two values go in the fp16 copy
     float *tab = table + tok * a.n_dims;                         // this token's cos | sin
     if constexpr (MODE == ROPE_APPLY) {
         for (int p = threadIdx.x; p < half; p += EW_THREADS) { cs[p] = tab[p]; sn[p] = tab[half + p]; }
@@ -636,6 +636,8 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
             else                    { ia[u] = j + half; ib[u] = j + half; }
             x0[u] = xt[base + ia[u]];
             x1[u] = xt[base + ib[u]];
+            ha[u] = ia[u] + h * (uint32_t)a.ld16_1;
+            hb[u] = ib[u] + h * (uint32_t)a.ld16_1;
             ia[u] += h * (uint32_t)a.ldy1;
             ib[u] += h * (uint32_t)a.ldy1;
         }
@@ -672,28 +674,36 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restric
     }
     if constexpr (MODE == ROPE_BUILD) return;
     __syncthreads();
+    unsigned short *ht = a.y16 ? a.y16 + tok * a.ld16_2 : nullptr;
 #pragma unroll
     for (int u = 0; u < PRE; u++) {
         if (jj[u] == 0xffffffffu) continue;
         if (jj[u] < (uint32_t)half) {
             const float c = cs[jj[u]], s = sn[jj[u]];
-            yt[ia[u]] = x0[u] * c - x1[u] * s;
-            yt[ib[u]] = x0[u] * s + x1[u] * c;
+            const float r0 = x0[u] * c - x1[u] * s, r1 = x0[u] * s + x1[u] * c;
+            yt[ia[u]] = r0;
+            yt[ib[u]] = r1;
+            if (ht) { ht[ha[u]] = f2h_rne(r0); ht[hb[u]] = f2h_rne(r1); }
         } else {
             yt[ia[u]] = x0[u];
+            if (ht) ht[ha[u]] = f2h_rne(x0[u]);
         }
     }
     for (uint32_t i = threadIdx.x + PRE * EW_THREADS; i < items; i += EW_THREADS) {
         const uint32_t h = i / per_head, j = i - h * per_head;
         const float *xr = xt + h * a.ldx1;
         float *yr = yt + h * a.ldy1;
+        unsigned short *hr = ht ? ht + h * a.ld16_1 : nullptr;
         if (j < (uint32_t)half) {
             const int64_t ka = a.neox ? j : 2 * j, kb = a.neox ? j + half : 2 * j + 1;
             const float v0 = xr[ka], v1 = xr[kb], c = cs[j], s = sn[j];
-            yr[ka] = v0 * c - v1 * s;
-            yr[kb] = v0 * s + v1 * c;
+            const float r0 = v0 * c - v1 * s, r1 = v0 * s + v1 * c;
+            yr[ka] = r0;
+            yr[kb] = r1;
+            if (hr) { hr[ka] = f2h_rne(r0); hr[kb] = f2h_rne(r1); }
         } else {
             yr[j + half] = xr[j + half];
+            if (hr) hr[j + half] = f2h_rne(xr[j + half]);
         }
     }
 }
@@ -702,7 +712,7 @@ hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_fac
                        bool build, hipStream_t st) {
     if (a.ne2 <= 0 || (!build && (a.ne0 <= 0 || a.ne1 <= 0))) return hipSuccess;
     if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff || a.ne0 * a.ne1 > 0x7fffffff) return hipErrorInvalidValue;
-    if (a.ne1 * a.ldx1 > 0x7fffffff || a.ne1 * a.ldy1 > 0x7fffffff) return hipErrorInvalidValue;       // 32-bit offsets inside a token
+    if (a.ne1 * a.ldx1 > 0x7fffffff || a.ne1 * a.ldy1 > 0x7fffffff || a.ne1 * a.ld16_1 > 0x7fffffff) return hipErrorInvalidValue;   // 32-bit offsets inside a token
     const dim3 grid((unsigned)a.ne2), block(EW_THREADS);
     if (!table) hipLaunchKernelGGL(rope_kernel<ROPE_FULL>, grid, block, 0, st, x, pos, freq_factors, a, y, (float *)nullptr);
     else if (build) hipLaunchKernelGGL(rope_kernel<ROPE_BUILD>, grid, block, 0, st, x, pos, freq_factors, a, y, table);

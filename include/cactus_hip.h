@@ -276,6 +276,13 @@ CHIP_API int chip_rope_table(const int32_t *pos, const float *freq_factors, int6
                              float beta_slow, float *table, void *stream);
 CHIP_API int chip_rope_apply(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1,
                              int64_t ne2, int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, void *stream);
+/* chip_rope_apply that also stores the result rounded to fp16 (round to nearest even, as lm_ggml_cpu_fp32_to_fp16 does):
+ * the RoPE of K and the CPY into the F16 cache that follows it (llama-kv-cache.cpp cpy_k) in one launch.  y_f16 takes
+ * the element at (i0, head, token) at i0 + head * ld16_1 + token * ld16_2 halves.  Bit-identical to chip_rope_apply
+ * followed by chip_cpy F32 -> F16. */
+CHIP_API int chip_rope_apply_store(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1,
+                                   int64_t ne2, int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, uint16_t *y_f16,
+                                   int64_t ld16_1, int64_t ld16_2, void *stream);
 
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,

@@ -244,6 +244,19 @@ def attn_case(seed, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
 # that use 8 / 16 / 32 lanes per cache row, a GQA ratio that is no power of two, positions that are no multiple of 64
 # the last five have 64 or more (head, token) pairs per KV head: with a workspace they take the GEMM route, the last two
 # with K (head size 96; 104 and 1056 cache positions) that is no multiple of the GEMM's 64-value stage
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("ne0,n_dims,n_head,n_tokens", [(128, 128, 8, 1), (128, 128, 8, 7), (64, 32, 3, 2), (256, 256, 40, 3)])
+def test_rope_with_the_cache_store_in_one_launch(dev, mode, ne0, n_dims, n_head, n_tokens):
+    """chip_rope_apply_store: the fp32 result equals chip_rope's bit for bit, the fp16 copy equals chip_cpy of that result
+    (round to nearest even), for rotated and passed-through values, also past the first 2048 items of a token."""
+    rng = np.random.default_rng(ne0 + n_head + mode)
+    x = (rng.standard_normal((n_tokens, n_head, ne0)) * 3).astype(np.float32)
+    pos = np.array([5, 0, 4095, 17, 100000, 31, 2][:n_tokens], np.int32)
+    y, h = dev.rope(x, pos, n_dims, mode, freq_base=500000.0, store_f16=True)
+    assert y.tobytes() == dev.rope(x, pos, n_dims, mode, freq_base=500000.0).tobytes()
+    assert h.tobytes() == dev.cpy(y.reshape(-1, ne0), np.float16).tobytes() == y.astype(np.float16).tobytes()
+
+
 ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8, 3, 96, 128), (256, 4, 2, 2, 160, 160),
                (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128), (128, 32, 8, 130, 320, 512),
                (64, 4, 4, 100, 192, 256), (96, 6, 2, 40, 104, 128), (128, 32, 8, 512, 1056, 2048),

@@ -832,8 +832,11 @@ def test_attention_block_stays_on_the_device(host, orc):
     blib = C.CDLL(cactus_amd.BACKEND_LIB)
     blib.lm_ggml_backend_hip_get_rope_tables.restype = C.c_ulonglong
     tables_before = blib.lm_ggml_backend_hip_get_rope_tables()
+    blib.lm_ggml_backend_hip_get_fused_pairs.restype = C.c_ulonglong
+    fused_before = blib.lm_ggml_backend_hip_get_fused_pairs()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     assert blib.lm_ggml_backend_hip_get_rope_tables() - tables_before == 1      # Q and K share one cos / sin table
+    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before >= 1       # the K store ran in the kernel of K's RoPE
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
