@@ -509,7 +509,11 @@ def bench_trace(dev, hip, st, rng):
                 mm(*W["wo"], merged, att)
                 # residual + norm + weight: one kernel, as the backend fuses the three nodes
                 ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
-                mm(*W["up"], cur, up); mm(*W["gate"], cur, gate, True)
+                if n <= 4:                                                # gate and up in one launch, as the backend pairs them
+                    (t_, wg, N_, K_), (_, wu, _, _) = W["gate"], W["up"]
+                    ck(L.chip_mul_mat_pair(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, up.ptr, N_, ws.ptr, wsz, st))
+                else:
+                    mm(*W["up"], cur, up); mm(*W["gate"], cur, gate, True)
                 ck(L.chip_silu_mul(gate.ptr, FF, up.ptr, FF, n, FF, gate.ptr, FF, st))                 # SiLU in its MUL's kernel, as the backend runs the pair
                 mm(*W["down"], gate, att)
                 # the layer's second residual with the next layer's (or the final) norm

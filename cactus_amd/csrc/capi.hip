@@ -393,6 +393,27 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
     return mul_mat_run(type, W, nb01, K, N, n, workspace, workspace_bytes, y, ldy, stream);
 }
 
+// Two matmuls on one activation (ffn_gate / ffn_up).  Up to 4 tokens: one launch of the prologue-quantizing GEMV over
+// both matrices; more tokens: one quantizer, then each matrix on its own path.
+int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                      int64_t n, float *y1, float *y2, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (N < 0 || n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n == 0) return CHIP_OK;
+    if (!W1 || !W2 || !x || !y1 || !y2 || !workspace || ldx < K || ldy < N) return CHIP_EINVAL;
+    if (!weights_aligned(type, W1, nb01, K) || !weights_aligned(type, W2, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
+    if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || ((((uintptr_t)y1) | ((uintptr_t)y2)) & 3) != 0) return CHIP_EINVAL;
+    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+    DeviceLimits lim;
+    if (int rc = current_limits(lim); rc) return rc;
+    if (n <= 4 && 2 * N <= 0x7fffffff && gemv_fused_applicable(type, K, (int)n, lim))
+        return hip_rc(launch_gemv_fused_pair(type, W1, W2, nb01, K, N, x, ldx, (int)n, workspace,
+                                             act_stride(chip_vec_dot_type(type), K), y1, y2, ldy, lim, (hipStream_t)stream));
+    if (int rc = chip_mul_mat_prepare(type, K, x, ldx, n, workspace, workspace_bytes, stream); rc) return rc;
+    if (int rc = mul_mat_run(type, W1, nb01, K, N, n, workspace, workspace_bytes, y1, ldy, stream); rc) return rc;
+    return mul_mat_run(type, W2, nb01, K, N, n, workspace, workspace_bytes, y2, ldy, stream);
+}
+
 // MUL_MAT_ID workspace: the quantized activation rows, then the expert offsets and the pair list of the grouped path
 static size_t moe_rows_bytes(int type, int64_t K, int64_t rows) { return align16(act_stride(chip_vec_dot_type(type), K) * (size_t)rows); }
 size_t chip_mul_mat_id_workspace_size(int type, int64_t K, int64_t n_as, int64_t n_used, int64_t n_tokens, int64_t ne11) {

@@ -896,11 +896,17 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
 }
 
 
+// Two matrices of one shape and type that read the same activation (ffn_gate and ffn_up) as one launch: rows
+// [0, n_first) are the first matrix, rows [n_first, N) the second one, whose weights and outputs lie w_off bytes / y_off
+// floats away from where the first matrix's row and output of that index would be.  One matrix: n_first = N.
+struct SecondMatrix { int64_t n_first, w_off, y_off; };
+constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0};
+
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                           const float *__restrict__ x, int64_t ldx,
                                           uint8_t *__restrict__ ws, size_t ws_stride,
-                                          float *__restrict__ y, int64_t ldy) {
+                                          float *__restrict__ y, int64_t ldy, const SecondMatrix sec) {
     using T = Traits<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int NI = iters_per_row<WT>(K);
@@ -926,8 +932,10 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
             const int u = lc.it * 64 + lane;
             if (u < units) {
 #pragma unroll
-                for (int r = 0; r < R; r++)                              // tail tile: re-read the last row, never store it
-                    T::load_raw(slot[r], W + (size_t)min(lc.tile * R + r, N - 1) * nb01, u);
+                for (int r = 0; r < R; r++) {                            // tail tile: re-read the last row, never store it
+                    const int64_t row = min(lc.tile * R + r, N - 1);
+                    T::load_raw(slot[r], W + (size_t)row * nb01 + (row >= sec.n_first ? sec.w_off : (int64_t)0), u);
+                }
             }
             advance(lc);
         }
@@ -986,7 +994,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
 #pragma unroll
                     for (int t = 0; t < NTOK; t++) {
                         const float s = wave_sum_to_lane63(acc[r][t]);
-                        if (lane == 63 && row0 + r < N) y[(size_t)t * ldy + row0 + r] = s;
+                        if (lane == 63 && row0 + r < N) y[(int64_t)t * ldy + row0 + r + (row0 + r >= sec.n_first ? sec.y_off : (int64_t)0)] = s;
                         acc[r][t] = 0.f;
                     }
             }
@@ -999,8 +1007,8 @@ template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
 __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                                    const float *__restrict__ x, int64_t ldx,
                                                    uint8_t *__restrict__ ws, size_t ws_stride,
-                                                   float *__restrict__ y, int64_t ldy) {
-    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy);
+                                                   float *__restrict__ y, int64_t ldy, SecondMatrix sec) {
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec);
 }
 
 // LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
@@ -1025,7 +1033,7 @@ __global__ __launch_bounds__(WGS) void gemv_id_kernel(const uint8_t *__restrict_
     if (e < 0 || e >= m.n_as) return;
     const int64_t xrow = t * m.ne11 + s % m.ne11;
     gemv_body<WT, 1, R, WGS, FUSEQ, DEPTH>(W + (size_t)e * m.nb02, nb01, K, N, FUSEQ ? x + xrow * ldx : x, ldx,
-                                          ws + (size_t)xrow * ws_stride, ws_stride, y + pair * ldy, ldy);
+                                          ws + (size_t)xrow * ws_stride, ws_stride, y + pair * ldy, ldy, kNoSecond);
 }
 
 // ------------------------------------------------------------------------------------------------ launch
@@ -1042,7 +1050,7 @@ template <int WT> struct RowsPerWave { static constexpr int R = (WT == T_Q4_0) ?
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
 static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
                              size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, const DeviceLimits &lim,
-                             hipStream_t st) {
+                             hipStream_t st, const SecondMatrix &sec) {
     const int64_t tiles = ceil_div(N, R);
     int64_t groups = ceil_div(tiles, WGS / 64);
     if (groups > max_groups) groups = max_groups;
@@ -1050,13 +1058,14 @@ static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, c
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
-                       (uint8_t *)ws, ws_stride, y, ldy);
+                       (uint8_t *)ws, ws_stride, y, ldy, sec);
     return hipGetLastError();
 }
 
 template <int WT, int NTOK, bool FUSEQ>
 static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
-                               size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                               size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st,
+                               const SecondMatrix &sec = kNoSecond) {
     const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
@@ -1066,7 +1075,7 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         const char *ew = getenv("CHIP_TUNE_WGS"), *er = getenv("CHIP_TUNE_R"), *ec = getenv("CHIP_TUNE_CAP");
         if (ew && er && ec) {
             const int w = atoi(ew), r = atoi(er); const int64_t cap = (int64_t)cus * atoi(ec);
-#define TUNE_CASE(WW, RR) if (w == WW && r == RR) return launch_one<WT, NTOK, RR, WW, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, lim, st);
+#define TUNE_CASE(WW, RR) if (w == WW && r == RR) return launch_one<WT, NTOK, RR, WW, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, lim, st, sec);
             TUNE_CASE(256, 1) TUNE_CASE(256, 2) TUNE_CASE(256, 4) TUNE_CASE(512, 1) TUNE_CASE(512, 2) TUNE_CASE(512, 4)
             TUNE_CASE(1024, 1) TUNE_CASE(1024, 2) TUNE_CASE(1024, 4)
 #undef TUNE_CASE
@@ -1085,25 +1094,26 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         const bool one_tile_per_wave = tiles <= 16 * (int64_t)cus && tiles > 8 * (int64_t)cus;
         const bool long_q8_0_row = Traits<WT>::ACT == T_Q8_0 && NTOK == 1 && K > 8192;
         if (one_tile_per_wave && !long_q8_0_row)
-            return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st);
+            return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
     }
     if (ceil_div(tiles, 8) >= cus)
-        return launch_one<WT, NTOK, R, 512, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, lim, st);
-    return launch_one<WT, NTOK, R, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, lim, st);
+        return launch_one<WT, NTOK, R, 512, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, lim, st, sec);
+    return launch_one<WT, NTOK, R, 256, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus * per_cu, lim, st, sec);
 }
 
 template <int WT, bool FUSEQ>
 static hipError_t launch_ntok(int n, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
-                              size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                              size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st,
+                              const SecondMatrix &sec = kNoSecond) {
     switch (n) {
-        case 1: return launch_typed<WT, 1, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case 2: return launch_typed<WT, 2, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case 3: if constexpr (!FUSEQ) return launch_typed<WT, 3, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
-        case 4: return launch_typed<WT, 4, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case 5: if constexpr (!FUSEQ) return launch_typed<WT, 5, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
-        case 6: if constexpr (!FUSEQ) return launch_typed<WT, 6, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
-        case 7: if constexpr (!FUSEQ) return launch_typed<WT, 7, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
-        case 8: if constexpr (!FUSEQ) return launch_typed<WT, 8, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st); break;
+        case 1: return launch_typed<WT, 1, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case 2: return launch_typed<WT, 2, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case 3: if constexpr (!FUSEQ) return launch_typed<WT, 3, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec); break;
+        case 4: return launch_typed<WT, 4, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case 5: if constexpr (!FUSEQ) return launch_typed<WT, 5, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec); break;
+        case 6: if constexpr (!FUSEQ) return launch_typed<WT, 6, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec); break;
+        case 7: if constexpr (!FUSEQ) return launch_typed<WT, 7, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec); break;
+        case 8: if constexpr (!FUSEQ) return launch_typed<WT, 8, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec); break;
         default: break;
     }
     return hipErrorInvalidValue;
@@ -1171,20 +1181,35 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
     return (size_t)n * img <= (size_t)lim.max_lds_per_block;
 }
 
+static hipError_t launch_gemv_fused_sec(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                                        int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim,
+                                        hipStream_t st, const SecondMatrix &sec);
 hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
                              int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    return launch_gemv_fused_sec(wtype, W, nb01, K, N, x, ldx, n, ws, ws_stride, y, ldy, lim, st, kNoSecond);
+}
+// W2 / y2: a second matrix of the same type, shape and row stride on the same activation; both outputs have stride ldy
+hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
+                                  int64_t ldx, int n, void *ws, size_t ws_stride, float *y1, float *y2, int64_t ldy,
+                                  const DeviceLimits &lim, hipStream_t st) {
+    const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, (int64_t)(y2 - y1) - N};
+    return launch_gemv_fused_sec(wtype, W1, nb01, K, 2 * N, x, ldx, n, ws, ws_stride, y1, ldy, lim, st, sec);
+}
+static hipError_t launch_gemv_fused_sec(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                                        int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim,
+                                        hipStream_t st, const SecondMatrix &sec) {
     if (N <= 0 || n <= 0) return hipSuccess;
     switch (wtype) {
-        case T_Q4_0: return launch_ntok<T_Q4_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q8_0: return launch_ntok<T_Q8_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q4_K: return launch_ntok<T_Q4_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q6_K: return launch_ntok<T_Q6_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q5_0: return launch_ntok<T_Q5_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q5_K: return launch_ntok<T_Q5_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_IQ4_NL: return launch_ntok<T_IQ4_NL, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q4_1: return launch_ntok<T_Q4_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_Q5_1: return launch_ntok<T_Q5_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
-        case T_F16: return launch_ntok<T_F16, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st);
+        case T_Q4_0: return launch_ntok<T_Q4_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q8_0: return launch_ntok<T_Q8_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q4_K: return launch_ntok<T_Q4_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q6_K: return launch_ntok<T_Q6_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q5_0: return launch_ntok<T_Q5_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q5_K: return launch_ntok<T_Q5_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_IQ4_NL: return launch_ntok<T_IQ4_NL, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q4_1: return launch_ntok<T_Q4_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q5_1: return launch_ntok<T_Q5_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_F16: return launch_ntok<T_F16, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         default: return hipErrorInvalidValue;
     }
 }

@@ -630,12 +630,30 @@ int rope_store_index(const lm_ggml_cgraph *g, int i) {
     return j;
 }
 
+// ffn_gate and ffn_up in llama.cpp's node order: gate matmul, SILU, up matmul, MUL.  With up to 4 tokens the two matmuls
+// (same activation tensor, weight type and shape) run as one launch when the SILU between them is one that waits for
+// its MUL anyway and the up projection's output overlaps nothing that is read before its own node: the activation, the
+// gate's output (which the SILU reads) and the SILU's output.  Index of the up matmul, or -1.
+int paired_matmul_index(const lm_ggml_cgraph *g, int i) {
+    if (i + 3 >= g->n_nodes) return -1;
+    const lm_ggml_tensor *gate = g->nodes[i], *silu = g->nodes[i + 1], *up = g->nodes[i + 2];
+    if (silu->op != LM_GGML_OP_UNARY || silu->op_params[0] != LM_GGML_UNARY_OP_SILU || silu->src[0] != gate) return -1;
+    if (!elementwise_shape_ok(silu) || !silu_can_wait_for_its_mul(g, i + 1)) return -1;
+    if (up->op != LM_GGML_OP_MUL_MAT || !mul_mat_shape_ok(up) || up->src[1] != gate->src[1]) return -1;
+    const lm_ggml_tensor *wg = gate->src[0], *wu = up->src[0], *x = gate->src[1];
+    if (x->ne[1] > 4 || wg->type != wu->type || wg->ne[0] != wu->ne[0] || wg->ne[1] != wu->ne[1] || wg->nb[1] != wu->nb[1]) return -1;
+    if (up->nb[1] != gate->nb[1]) return -1;
+    if (!disjoint(up, x) || !disjoint(up, gate) || !disjoint(up, silu)) return -1;
+    return i + 2;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
     c->quantized.valid = false;                       // and so may any activation
     const lm_ggml_tensor *waiting_silu = nullptr;     // a SILU held back for the MUL two nodes on
     int stored_by_rope = -1;                          // index of a CPY node that ran inside the RoPE before it
+    int paired_matmul = -1;                           // index of an up projection that ran with its gate projection
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -716,6 +734,10 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             stored_by_rope = -1;
             continue;
         }
+        if (i == paired_matmul) {                     // this matmul ran in the launch of the one two nodes before it
+            paired_matmul = -1;
+            continue;
+        }
         if (is_attn_side_op(node->op) && attn_side_shape_ok(node)) {
             const lm_ggml_tensor *store = nullptr;
             if (node->op == LM_GGML_OP_ROPE && fusion_enabled()) {
@@ -777,7 +799,15 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         if (!grow_workspace(c, chip_mul_mat_workspace_size_n(w->type, K, N, n))) return LM_GGML_STATUS_ALLOC_FAILED;   // wdata
         int rc;
         const int64_t ldx = (int64_t)(x->nb[1] / 4);
-        if (n > 4 && fusion_enabled()) {
+        if (n <= 4 && fusion_enabled() && (paired_matmul = paired_matmul_index(cgraph, i)) >= 0) {
+            lm_ggml_tensor *up = cgraph->nodes[paired_matmul];
+            writes(up);
+            c->quantized.valid = false;
+            rc = chip_mul_mat_pair(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
+                                   (float *)up->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
+            g_mul_mat_nodes++;
+            g_fused_pairs++;
+        } else if (n > 4 && fusion_enabled()) {
             // quantize once per source tensor: the matmuls that share an input follow each other closely
             quantized_key &q = c->quantized;
             const int vt = chip_vec_dot_type(w->type);

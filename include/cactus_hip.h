@@ -150,6 +150,12 @@ CHIP_API int chip_mul_mat_prepare(int type, int64_t K, const float *x, int64_t l
                                   void *workspace, size_t workspace_bytes, void *stream);
 CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,
                               const void *workspace, float *y, int64_t ldy, void *stream);
+/* Two matmuls of one type, shape and row stride on the same activation (ffn_gate and ffn_up, llama-graph.cpp:562-690):
+ * up to 4 tokens both run in one launch of the GEMV that quantizes in its prologue; with more tokens the activation is
+ * quantized once and each matrix takes its usual path.  Results as from two chip_mul_mat calls. */
+CHIP_API int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
+                               int64_t ldx, int64_t n, float *y1, float *y2, int64_t ldy, void *workspace, size_t workspace_bytes,
+                               void *stream);
 /* chip_mul_mat_run told how large the workspace is: with chip_mul_mat_workspace_size_n(type, K, N, n) bytes a GEMM may
  * split K (the partial outputs go behind the activation rows, which stay valid for the next matmul). */
 CHIP_API int chip_mul_mat_run_ws(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,

@@ -295,6 +295,23 @@ def test_argument_errors(dev):
     dev.sync()
 
 
+# ------------------------------------------------------------------------------------------ two matrices, one activation
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N", [(1024, 333), (4096, 1030)])
+def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
+    """chip_mul_mat_pair (ffn_gate and ffn_up in one launch up to 4 tokens; an odd row count puts a two-row tile of Q4_0
+    across the two matrices): each output equals the single call's bit for bit, and the oracle within the tolerance."""
+    w1 = quantized_weights(wt, K + N, N, K)
+    w2 = quantized_weights(wt, K + N + 1, N, K)
+    for n in (1, 2, 4, 3, 7):
+        x = common.activations_f32(K + n, n, K)
+        y1, y2 = dev.mul_mat_pair(wt, w1, w2, x)
+        assert y1.tobytes() == dev.mul_mat(wt, w1, x).tobytes(), n
+        assert y2.tobytes() == dev.mul_mat(wt, w2, x).tobytes(), n
+        ref = orc.mul_mat(wt, w2, x, nthreads=8, want=("sum_abs",))
+        check_outputs(y2, ref["y"], ref["sum_abs"], "second matrix of the pair, n = %d" % n)
+
+
 # ------------------------------------------------------------------------------------------ rows of K % 256 != 0
 @pytest.mark.parametrize("wt", (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL, O.Q4_1, O.Q5_1), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(576, 1536), (896, 151), (960, 2560), (4160, 300), (64, 5)])
