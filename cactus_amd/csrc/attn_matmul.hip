@@ -486,13 +486,25 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
     if (plan.use && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {
         uint8_t *ws = (uint8_t *)workspace;
         int32_t *perm = (int32_t *)(ws + plan.off_perm), *offsets = (int32_t *)(ws + plan.off_offsets), *tiles = (int32_t *)(ws + plan.off_tiles);
-        const int64_t chunks = K / 8, per = chunks >= AM_THREADS ? 1 : AM_THREADS / chunks;
-        hipLaunchKernelGGL(mm_f16_round_rows_kernel, dim3((unsigned)ceil_div(n, per), (unsigned)(ne02 * r2)), dim3(AM_THREADS), 0, st, x,
-                           ldx1, ldx2, n, K, ws, plan.act_stride);
+        // one row tile, or two with at most 1024 columns per KV head (kqv: a head's rows): the GEMM reads the fp32 activations
+        // itself and rounds them while staging (measured: 1.3 % of a 128-token step over 4096 positions; with 2048 columns and two
+        // row tiles the doubled staging traffic costs more than the rounding pass, and kq, with thousands of cache positions
+        // as rows, reads the activations back once per row tile): the others get an fp16 copy first
+        static const bool f32_direct = [] { const char *e = getenv("CHIP_ATTN_F32_ROWS"); return !(e && e[0] == '0'); }();
+        const int64_t row_tiles = ceil_div(N, (int64_t)plan.tile);
+        const bool direct = f32_direct && (row_tiles == 1 || (row_tiles == 2 && r2 * n <= 1024)) && n <= 0x7fffffff &&
+                            ne02 * r2 * n <= 0x7fffffff;
+        if (!direct) {
+            const int64_t chunks = K / 8, per = chunks >= AM_THREADS ? 1 : AM_THREADS / chunks;
+            hipLaunchKernelGGL(mm_f16_round_rows_kernel, dim3((unsigned)ceil_div(n, per), (unsigned)(ne02 * r2)), dim3(AM_THREADS), 0, st, x,
+                               ldx1, ldx2, n, K, ws, plan.act_stride);
+        }
         hipLaunchKernelGGL(mm_f16_tile_list_kernel, dim3(64), dim3(AM_THREADS), 0, st, ne02, r2 * n, plan.tile, perm, offsets, tiles);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
         const RowGather rg{perm, offsets, tiles, 1, 1, nb02};
-        return launch_gemm_f16(W, nb01, K, N, ws, plan.act_stride, ne02 * r2 * n, y, ldy1, lim, st, &rg, plan.n_tiles, plan.tile);
+        const F32Rows fr{x, ldx1, ldx2, n};
+        return launch_gemm_f16(W, nb01, K, N, ws, plan.act_stride, ne02 * r2 * n, y, ldy1, lim, st, &rg, plan.n_tiles, plan.tile,
+                               direct ? &fr : nullptr);
     }
     const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;

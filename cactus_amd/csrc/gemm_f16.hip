@@ -36,10 +36,25 @@ struct F16Cfg {
     static_assert(W_ITEMS % NT == 0 && X_ITEMS % NT == 0, "staging items divide evenly over the threads");
 };
 
-template <int TM, int TN, int WR, int WC, int OCC, bool GATHER>
+// XF32 (row-gather mode only): the activations are read as fp32 from their own tensor - row R of the gather is token
+// R % n of batch R / n - and rounded to fp16 (nearest even) on their way into LDS, instead of from an fp16 copy in the
+// workspace.  Pays when the output has one or two row tiles (kqv: a head's 64 - 256 rows), so that the fp32 rows are read
+// once or twice; with many row tiles the fp16 copy, read back many times, is the cheaper source.
+__device__ __forceinline__ u32x4 round8_f16(const float4 a, const float4 b) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 h0 = {(_Float16)a.x, (_Float16)a.y}, h1 = {(_Float16)a.z, (_Float16)a.w};
+    const h2 h2v = {(_Float16)b.x, (_Float16)b.y}, h3 = {(_Float16)b.z, (_Float16)b.w};
+    u32x4 r;
+    r.x = __builtin_bit_cast(uint32_t, h0); r.y = __builtin_bit_cast(uint32_t, h1);
+    r.z = __builtin_bit_cast(uint32_t, h2v); r.w = __builtin_bit_cast(uint32_t, h3);
+    return r;
+}
+
+template <int TM, int TN, int WR, int WC, int OCC, bool GATHER, bool XF32 = false>
 __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
-                     size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg) {
+                     size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg, F32Rows fs) {
+    static_assert(!XF32 || GATHER, "fp32 activation rows come with the row-gather mode");
     using C = F16Cfg<TM, TN, WR, WC>;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -73,7 +88,13 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
 #pragma unroll
     for (int i = 0; i < C::X_PER_T; i++) {
         const int item = tid + i * C::NT;
-        xsrc[i] = ws + (size_t)gv.act_row(min(tok_base + item / C::CELLS, M - 1)) * ws_stride + 16 * (item % C::CELLS);
+        const int64_t arow = gv.act_row(min(tok_base + item / C::CELLS, M - 1));
+        if constexpr (XF32) {
+            const uint32_t b = (uint32_t)arow / (uint32_t)fs.n, t = (uint32_t)arow - b * (uint32_t)fs.n;
+            xsrc[i] = reinterpret_cast<const uint8_t *>(fs.x + (int64_t)b * fs.ldx2 + (int64_t)t * fs.ldx1) + 32 * (item % C::CELLS);
+        } else {
+            xsrc[i] = ws + (size_t)arow * ws_stride + 16 * (item % C::CELLS);
+        }
     }
     u32x4 wq[C::W_PER_T], xq[C::X_PER_T];
 
@@ -88,7 +109,12 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
         }
 #pragma unroll
         for (int i = 0; i < C::X_PER_T; i++) {
-            xq[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + off);
+            if constexpr (XF32) {
+                const float4 *xp = reinterpret_cast<const float4 *>(xsrc[i] + 2 * off);      // a stage is twice the bytes in fp32
+                xq[i] = round8_f16(xp[0], xp[1]);
+            } else {
+                xq[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + off);
+            }
             if (KTAIL && !live) xq[i] = z;
         }
     };
@@ -166,17 +192,18 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
 // rows must be 16-byte aligned (the weight alignment rule of the C-ABI) and K a multiple of the 64-value stage
 bool gemm_f16_supported(int64_t K, int64_t N, int64_t n) { return K >= 64 && K % (16 * F16_KG) == 0 && N >= 1 && n >= 32; }
 
-template <int TM, int TN, int WR, int WC, int OCC, bool GATHER>
+template <int TM, int TN, int WR, int WC, int OCC, bool GATHER, bool XF32 = false>
 static hipError_t launch_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as) {
+                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
+                             const F32Rows &fs = F32Rows{nullptr, 0, 0, 1}) {
     using C = F16Cfg<TM, TN, WR, WC>;
     const size_t lds_bytes = 2 * C::STAGE;
-    auto kfn = gemm_f16_kernel<TM, TN, WR, WC, OCC, GATHER>;
+    auto kfn = gemm_f16_kernel<TM, TN, WR, WC, OCC, GATHER, XF32>;
     static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
     hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
-                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg);
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg, fs);
     return hipGetLastError();
 }
 
@@ -184,15 +211,21 @@ int gemm_f16_moe_tile_tokens() { return F16Cfg<1, 1, 2, 2>::BN; }      // the 64
 
 hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp, int64_t n_as,
-                           int gather_tile) {
+                           int gather_tile, const F32Rows *f32_rows) {
     if (M <= 0 || N <= 0 || n_as <= 0) return hipSuccess;
     const RowGather rg = rgp ? *rgp : RowGather{nullptr, nullptr, nullptr, 1, 1, 0};
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if (rg.perm) {                                                                   // row groups: the tile list was built for 64 or 128 tokens
+        if (f32_rows) {
+            if (gather_tile == 128) return launch_f16<2, 2, 2, 2, 2, true, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, *f32_rows);
+            if (gather_tile != 64) return hipErrorInvalidValue;
+            return launch_f16<1, 1, 2, 2, 4, true, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, *f32_rows);
+        }
         if (gather_tile == 128) return launch_f16<2, 2, 2, 2, 2, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
         if (gather_tile != 64) return hipErrorInvalidValue;
         return launch_f16<1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     }
+    if (f32_rows) return hipErrorInvalidValue;
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
     const char *force = getenv("CHIP_GEMM_F16_CFG");
     const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);

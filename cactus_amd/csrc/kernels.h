@@ -181,9 +181,13 @@ hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, i
 
 // gemm_f16.hip: fp16-MFMA prefill GEMM over F16 weights, activations as fp16 in the workspace.
 bool       gemm_f16_supported(int64_t K, int64_t N, int64_t n);
+// f32_rows (with rg only): the activation rows as fp32, gather row R = token R % n of batch R / n, rounded to fp16 in the
+// kernel's staging instead of being read from the fp16 workspace
+struct F32Rows { const float *x; int64_t ldx1, ldx2, n; };
 hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t n,
                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rg = nullptr,
-                           int64_t n_as = 1, int gather_tile = 64);       // gather_tile: tokens per list entry, 64 or 128
+                           int64_t n_as = 1, int gather_tile = 64,        // gather_tile: tokens per list entry, 64 or 128
+                           const F32Rows *f32_rows = nullptr);
 
 // gemm_kquant.hip: int8-MFMA prefill GEMM over Q4_K / Q5_K / Q6_K weights, activations in the split Q8_K workspace
 // layout; the integer sub-block scales ride in the MFMA operand.
