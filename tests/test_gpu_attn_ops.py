@@ -264,7 +264,9 @@ ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8
                (128, 32, 8, 8, 1040, 2048), (128, 32, 8, 15, 520, 1024), (256, 8, 2, 4, 296, 512), (256, 8, 2, 8, 296, 512),
                (256, 16, 2, 5, 264, 512), (64, 16, 2, 6, 1032, 2048), (128, 32, 8, 2, 4096, 4096), (80, 8, 1, 3, 24, 32),
                # 65 to 128 pairs: kqv with K split over workgroups (eight column groups), kq through the GEMM
-               (128, 32, 8, 32, 1048, 2048), (96, 12, 2, 17, 520, 1024)]
+               (128, 32, 8, 32, 1048, 2048), (96, 12, 2, 17, 520, 1024),
+               # more than 128 pairs over a long cache (K not a multiple of the GEMM's 64-value stage)
+               (128, 8, 2, 40, 2056, 4096), (64, 8, 2, 64, 4104, 4352)]
 
 
 @pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", ATTN_SHAPES)
