@@ -490,15 +490,22 @@ def bench_trace(dev, hip, st, rng):
                 vc = kc + kv_size * KV * 2
                 if l == 0:
                     ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))  # norm + weight: one kernel, as the backend fuses them
-                mm(*W["wq"], cur, q); mm(*W["wk"], cur, k, True); mm(*W["wv"], cur, v, True)
+                mm(*W["wq"], cur, q); mm(*W["wk"], cur, k, True)
+                if n <= 4:                                                # V projection and its transposed store in one launch
+                    t_, wv_, N_, K_ = W["wv"]
+                    ck(L.chip_mul_mat_store_t(t_, wv_, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, v.ptr, N_, vc + 2 * (n_kv - n), kv_size,
+                                              ws.ptr, wsz, st))
+                else:
+                    mm(*W["wv"], cur, v, True)
                 if l == 0:                                                # one cos / sin table per step, as the backend keeps it
                     ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
                 ck(L.chip_rope_apply(q.ptr, hd, hd * n_head, rope_tab.ptr, hd, n_head, n, hd, 2, q.ptr, hd, hd * n_head, st))
                 # K: RoPE and the store into the F16 cache in one launch, as the backend runs the two nodes
                 ck(L.chip_rope_apply_store(k.ptr, hd, KV, rope_tab.ptr, hd, n_head_kv, n, hd, 2, k.ptr, hd, KV,
                                            kc + 2 * KV * (n_kv - n), hd, KV, st))
-                shp = A4(n, KV, 1, 1)
-                ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))
+                if n > 4:
+                    shp = A4(n, KV, 1, 1)
+                    ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))
                 ck(L.chip_mul_mat_f16_batched(kc, 2 * KV, 2 * hd, hd, n_kv, n_head_kv, q.ptr, hd * n_head, hd, n, n_head, kq.ptr, n_kv,
                                               n_kv * n, aws.ptr, aws_bytes, st))
                 ck(L.chip_soft_max(kq.ptr, n_kv, mask.ptr, ca.F16, n_kv, n, n_head * n, 0.0884, 0.0, kq.ptr, n_kv, st))

@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums",
@@ -105,6 +105,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
     L.chip_mul_mat_run_ws.argtypes = [i32, vp, sz, i64, i64, i64, vp, sz, vp, i64, vp]
     L.chip_mul_mat_pair.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, vp, i64, vp, sz, vp]
+    L.chip_mul_mat_store_t.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, i64, vp, sz, vp]
     L.chip_rms_norm.argtypes = [vp, i64, i64, i64, C.c_float, vp, i64, vp]
     L.chip_add.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
     L.chip_mul.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
@@ -240,6 +241,22 @@ class Device:
         return y
 
     # -- element-wise ops next to the matmuls ---------------------------------------------------------------
+    def mul_mat_store_t(self, wtype, W, x, ld16):
+        """chip_mul_mat_store_t: returns (y fp32 [n, N], the fp16 matrix [N, ld16] whose first n columns hold y transposed;
+        the other columns keep the 0x7bff pattern they were filled with)."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, k = x.shape
+        W = np.ascontiguousarray(W, np.uint8)
+        N = W.shape[0]
+        dW, dx, dy = self.to_device(W), self.to_device(x), self.alloc(n * N * 4)
+        dh = self.to_device(np.full(N * ld16, 0x7bff, np.uint16))
+        wsz = self.lib.chip_mul_mat_workspace_size_n(wtype, k, N, n)
+        ws = self.alloc(wsz)
+        self.check(self.lib.chip_mul_mat_store_t(wtype, dW.ptr, self.row_size(wtype, k), k, N, dx.ptr, k, n, dy.ptr, N, dh.ptr, ld16,
+                                                 ws.ptr, wsz, None))
+        self.sync()
+        return dy.download(np.float32, n * N).reshape(n, N), dh.download(np.uint16, N * ld16).reshape(N, ld16)
+
     def mul_mat_pair(self, wtype, W1, W2, x):
         """Two matrices of one shape on the same activation (chip_mul_mat_pair): returns (y1, y2), each fp32 [n, N]."""
         x = np.ascontiguousarray(x, np.float32)

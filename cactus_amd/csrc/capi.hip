@@ -414,6 +414,30 @@ int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int
     return mul_mat_run(type, W2, nb01, K, N, n, workspace, workspace_bytes, y2, ldy, stream);
 }
 
+// A matmul whose result is also stored transposed as fp16 (the V projection and the store into the transposed F16 V cache).
+int chip_mul_mat_store_t(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
+                         float *y, int64_t ldy, uint16_t *y16t, int64_t ld16, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!y16t || ld16 < n || (((uintptr_t)y16t) & 1) != 0) return CHIP_EINVAL;
+    if (n >= 1 && n <= 4 && N > 0 && chip_mul_mat_supported(type, K)) {
+        DeviceLimits lim;
+        if (int rc = current_limits(lim); rc) return rc;
+        if (gemv_fused_applicable(type, K, (int)n, lim)) {
+            if (!x || !workspace || ldx < K || !W || !y || ldy < N) return CHIP_EINVAL;
+            if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0) return CHIP_EINVAL;
+            if (!weights_aligned(type, W, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
+            if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+            return hip_rc(launch_gemv_fused_store_t(type, W, nb01, K, N, x, ldx, (int)n, workspace, act_stride(chip_vec_dot_type(type), K),
+                                                    y, ldy, y16t, ld16, lim, (hipStream_t)stream));
+        }
+    }
+    if (int rc = chip_mul_mat(type, W, nb01, K, N, x, ldx, n, y, ldy, workspace, workspace_bytes, stream); rc) return rc;
+    if (N == 0 || n == 0) return CHIP_OK;
+    // y [n tokens][N] read as a matrix of n values per row r (stride 1 token = ldy floats), written as halves with rows ld16 apart
+    const int64_t ne[4] = {n, N, 1, 1};
+    const int64_t nbs[4] = {ldy * 4, 4, N * 4, N * 4}, nbd[4] = {2, ld16 * 2, N * ld16 * 2, N * ld16 * 2};
+    return hip_rc(launch_cpy(y, 0, ne, nbs, y16t, 1, ne, nbd, (hipStream_t)stream));
+}
+
 // MUL_MAT_ID workspace: the quantized activation rows, then the expert offsets and the pair list of the grouped path
 static size_t moe_rows_bytes(int type, int64_t K, int64_t rows) { return align16(act_stride(chip_vec_dot_type(type), K) * (size_t)rows); }
 size_t chip_mul_mat_id_workspace_size(int type, int64_t K, int64_t n_as, int64_t n_used, int64_t n_tokens, int64_t ne11) {

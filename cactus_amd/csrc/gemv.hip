@@ -899,8 +899,10 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
 // Two matrices of one shape and type that read the same activation (ffn_gate and ffn_up) as one launch: rows
 // [0, n_first) are the first matrix, rows [n_first, N) the second one, whose weights and outputs lie w_off bytes / y_off
 // floats away from where the first matrix's row and output of that index would be.  One matrix: n_first = N.
-struct SecondMatrix { int64_t n_first, w_off, y_off; };
-constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0};
+// t16 (one matrix only): the outputs also go, rounded to fp16, to t16[row * t16_ld + token] - the transposed store of V
+// into the F16 cache that follows the V projection (reference llama-kv-cache.cpp cpy_v without flash attention).
+struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; };
+constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0};
 
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
@@ -994,7 +996,10 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
 #pragma unroll
                     for (int t = 0; t < NTOK; t++) {
                         const float s = wave_sum_to_lane63(acc[r][t]);
-                        if (lane == 63 && row0 + r < N) y[(int64_t)t * ldy + row0 + r + (row0 + r >= sec.n_first ? sec.y_off : (int64_t)0)] = s;
+                        if (lane == 63 && row0 + r < N) {
+                            y[(int64_t)t * ldy + row0 + r + (row0 + r >= sec.n_first ? sec.y_off : (int64_t)0)] = s;
+                            if (sec.t16) sec.t16[(row0 + r) * sec.t16_ld + t] = f2h_rne(s);
+                        }
                         acc[r][t] = 0.f;
                     }
             }
@@ -1192,8 +1197,15 @@ hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, i
 hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                   int64_t ldx, int n, void *ws, size_t ws_stride, float *y1, float *y2, int64_t ldy,
                                   const DeviceLimits &lim, hipStream_t st) {
-    const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, (int64_t)(y2 - y1) - N};
+    const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, (int64_t)(y2 - y1) - N, nullptr, 0};
     return launch_gemv_fused_sec(wtype, W1, nb01, K, 2 * N, x, ldx, n, ws, ws_stride, y1, ldy, lim, st, sec);
+}
+// y16t: element (token t, row r) of the result also goes to y16t[r * ld16 + t] as fp16
+hipError_t launch_gemv_fused_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int n,
+                                     void *ws, size_t ws_stride, float *y, int64_t ldy, unsigned short *y16t, int64_t ld16,
+                                     const DeviceLimits &lim, hipStream_t st) {
+    const SecondMatrix sec{INT64_MAX, 0, 0, y16t, ld16};
+    return launch_gemv_fused_sec(wtype, W, nb01, K, N, x, ldx, n, ws, ws_stride, y, ldy, lim, st, sec);
 }
 static hipError_t launch_gemv_fused_sec(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
                                         int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim,

@@ -647,12 +647,31 @@ int paired_matmul_index(const lm_ggml_cgraph *g, int i) {
     return i + 2;
 }
 
+// The V projection followed (views aside) by the CPY of its transpose into the transposed F16 V cache (reference
+// llama-kv-cache.cpp cpy_v without flash attention: dst is a 2-D view [n_tokens, n_embd_v] with rows kv_size apart).
+// Index of that CPY node, or -1.  The matmul still writes its own F32 result.
+int transposed_store_index(const lm_ggml_cgraph *g, int i) {
+    const lm_ggml_tensor *mm = g->nodes[i];
+    int j = i + 1;
+    while (j < g->n_nodes && is_view_op(g->nodes[j]->op)) j++;
+    if (j >= g->n_nodes) return -1;
+    const lm_ggml_tensor *cp = g->nodes[j], *tr = cp->src[0];
+    if (cp->op != LM_GGML_OP_CPY || !tr || tr->op != LM_GGML_OP_TRANSPOSE || tr->src[0] != mm || cp->type != LM_GGML_TYPE_F16) return -1;
+    const int64_t N = mm->ne[0], n = mm->ne[1];
+    if (cp->ne[0] != n || cp->ne[1] != N || cp->ne[2] != 1 || cp->ne[3] != 1 || cp->nb[0] != 2 || cp->nb[1] % 2 != 0 ||
+        cp->nb[1] < (size_t)n * 2)
+        return -1;
+    if (!is_hip_buffer(cp->view_src ? cp->view_src->buffer : cp->buffer)) return -1;
+    if (!disjoint(cp, mm) || !disjoint(cp, mm->src[1])) return -1;
+    return j;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
     c->quantized.valid = false;                       // and so may any activation
     const lm_ggml_tensor *waiting_silu = nullptr;     // a SILU held back for the MUL two nodes on
-    int stored_by_rope = -1;                          // index of a CPY node that ran inside the RoPE before it
+    int stored_by_rope = -1;                          // index of a CPY node that ran inside the RoPE (or the matmul) before it
     int paired_matmul = -1;                           // index of an up projection that ran with its gate projection
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
@@ -799,7 +818,18 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         if (!grow_workspace(c, chip_mul_mat_workspace_size_n(w->type, K, N, n))) return LM_GGML_STATUS_ALLOC_FAILED;   // wdata
         int rc;
         const int64_t ldx = (int64_t)(x->nb[1] / 4);
-        if (n <= 4 && fusion_enabled() && (paired_matmul = paired_matmul_index(cgraph, i)) >= 0) {
+        int store_t = -1;
+        if (n <= 4 && fusion_enabled() && (store_t = transposed_store_index(cgraph, i)) >= 0) {
+            lm_ggml_tensor *cp = cgraph->nodes[store_t];
+            writes(cp);
+            c->quantized.valid = false;
+            stored_by_rope = store_t;                  // skipped like the CPY that ran inside a RoPE
+            rc = chip_mul_mat_store_t(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
+                                      (int64_t)(node->nb[1] / 4), (uint16_t *)cp->data, (int64_t)(cp->nb[1] / 2), c->workspace,
+                                      c->workspace_size, c->stream);
+            g_elementwise_nodes++;
+            g_fused_pairs++;
+        } else if (n <= 4 && fusion_enabled() && (paired_matmul = paired_matmul_index(cgraph, i)) >= 0) {
             lm_ggml_tensor *up = cgraph->nodes[paired_matmul];
             writes(up);
             c->quantized.valid = false;

@@ -133,6 +133,9 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
 bool       gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim);
 hipError_t launch_gemv_fused(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
                              int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+hipError_t launch_gemv_fused_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int n,
+                                     void *ws, size_t ws_stride, float *y, int64_t ldy, unsigned short *y16t, int64_t ld16,
+                                     const DeviceLimits &lim, hipStream_t st);
 hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                   int64_t ldx, int n, void *ws, size_t ws_stride, float *y1, float *y2, int64_t ldy,
                                   const DeviceLimits &lim, hipStream_t st);

@@ -156,6 +156,12 @@ CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, i
 CHIP_API int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                int64_t ldx, int64_t n, float *y1, float *y2, int64_t ldy, void *workspace, size_t workspace_bytes,
                                void *stream);
+/* chip_mul_mat whose result also goes, rounded to fp16 (nearest even), to y_f16_t[row * ld16 + token]: the V projection
+ * and its store into the transposed F16 V cache (llama-kv-cache.cpp cpy_v without flash attention) - one launch up to 4
+ * tokens, otherwise the matmul followed by the copy.  Results as from chip_mul_mat and chip_cpy. */
+CHIP_API int chip_mul_mat_store_t(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
+                                  float *y, int64_t ldy, uint16_t *y_f16_t, int64_t ld16, void *workspace, size_t workspace_bytes,
+                                  void *stream);
 /* chip_mul_mat_run told how large the workspace is: with chip_mul_mat_workspace_size_n(type, K, N, n) bytes a GEMM may
  * split K (the partial outputs go behind the activation rows, which stay valid for the next matmul). */
 CHIP_API int chip_mul_mat_run_ws(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,

@@ -312,6 +312,21 @@ def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
         check_outputs(y2, ref["y"], ref["sum_abs"], "second matrix of the pair, n = %d" % n)
 
 
+@pytest.mark.parametrize("wt", (O.Q6_K, O.Q4_K, O.Q8_0, O.Q4_0), ids=lambda t: O.TYPE_NAMES[t])
+def test_mul_mat_with_transposed_fp16_store(dev, wt):
+    """chip_mul_mat_store_t (the V projection and its store into the transposed F16 cache): y equals chip_mul_mat's bit for
+    bit, the fp16 matrix holds y transposed and rounded to nearest even in its first n columns and is untouched elsewhere;
+    1, 2, 4 tokens in one launch, 3 and 9 through the matmul and the copy."""
+    K, N, ld16 = 1024, 515, 24
+    w = quantized_weights(wt, K + N + 5, N, K)
+    for n in (1, 2, 4, 3, 9):
+        x = common.activations_f32(K + n, n, K)
+        y, h = dev.mul_mat_store_t(wt, w, x, ld16)
+        assert y.tobytes() == dev.mul_mat(wt, w, x).tobytes(), n
+        assert h[:, :n].tobytes() == np.ascontiguousarray(y.T.astype(np.float16)).view(np.uint16).tobytes(), n
+        assert (h[:, n:] == 0x7bff).all(), n
+
+
 # ------------------------------------------------------------------------------------------ rows of K % 256 != 0
 @pytest.mark.parametrize("wt", (O.Q4_0, O.Q8_0, O.Q5_0, O.IQ4_NL, O.Q4_1, O.Q5_1), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(576, 1536), (896, 151), (960, 2560), (4160, 300), (64, 5)])
