@@ -77,7 +77,7 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
     // rows of up to 8192 values stay in registers between the two passes (same order of additions as the loops below)
     constexpr int RC = 8;
     const bool cached = vecw && ne0 <= 4 * EW_THREADS * RC;
-    float4 keep[RC];
+    float4 keep[RC], wk[RC];                                     // wk: the weight row, asked for before the reduction
     if (cached) {
         const float *br = ADD ? b + (size_t)blockIdx.x * ldb : nullptr;
         float *sr = ADD ? xs + (size_t)blockIdx.x * ldxs : nullptr;
@@ -92,6 +92,7 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
                     *reinterpret_cast<float4 *>(sr + i) = v;
                 }
                 keep[k] = v;
+                if (w) wk[k] = *reinterpret_cast<const float4 *>(w + i);
                 sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
             }
         }
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
                 v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
                 if (w) {
                     if (ynr) *reinterpret_cast<float4 *>(ynr + i) = v;
-                    const float4 g = *reinterpret_cast<const float4 *>(w + i);
+                    const float4 g = wk[k];
                     v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w;
                 }
                 *reinterpret_cast<float4 *>(yr + i) = v;
