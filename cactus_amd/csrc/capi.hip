@@ -598,6 +598,25 @@ int chip_gelu(const float *x, int64_t ldx, int64_t n, int64_t ne0, const uint16_
     if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0) || !table || (((uintptr_t)table) & 1) != 0) return CHIP_EINVAL;
     return hip_rc(launch_gelu(x, ldx, ne0, n, table, y, ldy, (hipStream_t)stream));
 }
+// The norm in front of a group of matmuls, leaving the quantized rows in their workspace (what chip_mul_mat_prepare would
+// write from y afterwards).
+int chip_rms_norm_quantized(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
+                            int64_t ne0, float eps, const float *w, float *y, int64_t ldy, int wtype, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+    if (n < 0 || ne0 < 0 || !(eps >= 0.0f)) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(wtype, ne0)) return CHIP_EUNSUPPORTED;
+    const int at = chip_vec_dot_type(wtype);
+    const int kind = (at == T_Q8_0 || at == T_Q8_1) ? 1 : (at == T_Q8_K ? 2 : 0);
+    if (kind == 0) return CHIP_EUNSUPPORTED;                               // F16 weights: plain fp16 rows, not done here
+    if (n == 0 || ne0 == 0) return CHIP_OK;
+    if (!rows_ok(a, lda, ne0) || !rows_ok(y, ldy, ne0) || (w && (((uintptr_t)w) & 3) != 0) || n > 0x7fffffff) return CHIP_EINVAL;
+    if (b && (!rows_ok(b, ldb, ne0) || !rows_ok(sum, ld_sum, ne0) || (const float *)y == sum)) return CHIP_EINVAL;
+    if (!workspace || !aligned16(workspace)) return CHIP_EINVAL;
+    if (workspace_bytes < chip_mul_mat_workspace_size(wtype, ne0, n)) return CHIP_ENOMEM;
+    if (!norm_quantized_applicable(a, lda, b, ldb, sum, ld_sum, ne0, w, y, ldy)) return CHIP_EUNSUPPORTED;
+    return hip_rc(launch_norm_quantized(a, lda, b, ldb, sum, ld_sum, n, ne0, eps, w, y, ldy, (uint8_t *)workspace, act_stride(at, ne0),
+                                        kind, (hipStream_t)stream));
+}
 int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy, void *stream) {
     if (n < 0 || ne0 < 0) return CHIP_EINVAL;
     if (n == 0 || ne0 == 0) return CHIP_OK;

@@ -224,6 +224,11 @@ hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, 
 hipError_t launch_scale(const float *x, int64_t ldx, int64_t ne0, int64_t n, float s, float *y, int64_t ldy, hipStream_t st);
 hipError_t launch_gelu(const float *x, int64_t ldx, int64_t ne0, int64_t n, const unsigned short *table, float *y, int64_t ldy,
                        hipStream_t st);
+bool norm_quantized_applicable(const float *a, int64_t lda, const float *b, int64_t ldb, const float *xs, int64_t ldxs, int64_t ne0,
+                               const float *w, const float *y, int64_t ldy);
+hipError_t launch_norm_quantized(const float *a, int64_t lda, const float *b, int64_t ldb, float *xs, int64_t ldxs, int64_t n,
+                                 int64_t ne0, float eps, const float *w, float *y, int64_t ldy, uint8_t *qws, size_t qstride,
+                                 int act_kind, hipStream_t st);
 hipError_t launch_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy,
                            hipStream_t st);
 // SOFT_MAX over n_rows rows of ne00 values (a multiple of 8); row r adds row r % ne01 of the mask (fp32 or fp16, dense).

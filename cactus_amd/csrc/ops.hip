@@ -26,6 +26,8 @@
 //             the type's dequantize_row_* expression (ggml-quants.c).  Bit-exact.
 #include "dev_common.h"
 #include "kernels.h"
+#include "quant_dev.h"
+#include "act_layout.h"
 
 // One rounding per written operation, as in the reference's C code; the fused operations of this file are explicit fmaf calls.
 #pragma clang fp contract(off)
@@ -64,7 +66,8 @@ template <bool ADD>
 __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, int64_t ldx, int64_t ne0, float eps,
                                                               float *__restrict__ y, int64_t ldy, const float *__restrict__ w,
                                                               float *__restrict__ yn, int64_t ldyn, const float *b, int64_t ldb,
-                                                              float *xs, int64_t ldxs) {
+                                                              float *xs, int64_t ldxs, uint8_t *__restrict__ qws, size_t qstride,
+                                                              int qkind) {
     __shared__ double part[EW_THREADS / 64];
     const float *xr = x + (size_t)blockIdx.x * ldx;
     float *yr = y + (size_t)blockIdx.x * ldy;
@@ -145,6 +148,27 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
                     v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w;
                 }
                 *reinterpret_cast<float4 *>(yr + i) = v;
+                // the row as the next matmuls want it: quantized into the workspace planes of token blockIdx.x (ne0 is a
+                // multiple of 256 here, so a wave is inside the row with all its lanes or not at all)
+                if (qkind == 2) {
+                    const Q8_KLane q = quantize_q8_K_lane(v);
+                    uint8_t *base = qws + (size_t)blockIdx.x * qstride;
+                    const int64_t sb = i >> 8;
+                    const int lane = tid & 63;
+                    *reinterpret_cast<uint32_t *>(base + i) = q.packed;
+                    if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(ne0))[sb] = q.d;
+                    if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(ne0))[sb * 16 + (lane >> 2)] = (int16_t)q.bsum;
+                } else if (qkind == 1) {
+                    const Q8_0Lane q = quantize_q8_0_lane(v);
+                    uint8_t *base = qws + (size_t)blockIdx.x * qstride;
+                    const int64_t blk = i >> 5;
+                    *reinterpret_cast<uint32_t *>(base + i) = q.packed;
+                    if ((tid & 7) == 0) {
+                        reinterpret_cast<float *>(base + q8_0_off_d(ne0))[blk] = h2f(q.dh);
+                        reinterpret_cast<int32_t *>(base + q8_0_off_sum(ne0))[blk] = q.sum;
+                        reinterpret_cast<float *>(base + q8_0_off_s(ne0))[blk] = h2f(q.sh);
+                    }
+                }
             }
         }
     } else if (vecw) {
@@ -727,7 +751,7 @@ hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, 
         const int64_t rows = n - r0 < (1 << 30) ? n - r0 : (1 << 30);
         hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)rows), dim3(EW_THREADS), 0, st, x + r0 * ldx, ldx, ne0, eps,
                            y + r0 * ldy, ldy, (const float *)nullptr, (float *)nullptr, (int64_t)0, (const float *)nullptr,
-                           (int64_t)0, (float *)nullptr, (int64_t)0);
+                           (int64_t)0, (float *)nullptr, (int64_t)0, (uint8_t *)nullptr, (size_t)0, 0);
     }
     return hipGetLastError();
 }
@@ -736,7 +760,7 @@ hipError_t launch_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t n
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     if (n > 0x7fffffff) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, x, ldx, ne0, eps, y, ldy, w, yn, ldyn,
-                       (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0);
+                       (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0, (uint8_t *)nullptr, (size_t)0, 0);
     return hipGetLastError();
 }
 hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *xs, int64_t ldxs, int64_t n,
@@ -745,7 +769,30 @@ hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, 
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     if (n > 0x7fffffff) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rms_norm_kernel<true>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, yn, ldyn, b,
-                       ldb, xs, ldxs);
+                       ldb, xs, ldxs, (uint8_t *)nullptr, (size_t)0, 0);
+    return hipGetLastError();
+}
+// The norm (with or without the residual ADD in front: b may be NULL) whose result also goes, quantized as the activation
+// type act_kind (1 = Q8_0 / Q8_1 planes, 2 = Q8_K planes), into the matmul workspace.  Rows of up to 8192 values that
+// are a multiple of 256 and meet the vector alignment (the register-resident path of the kernel); false otherwise.
+bool norm_quantized_applicable(const float *a, int64_t lda, const float *b, int64_t ldb, const float *xs, int64_t ldxs, int64_t ne0,
+                               const float *w, const float *y, int64_t ldy) {
+    if (ne0 <= 0 || ne0 % 256 != 0 || ne0 > 4 * EW_THREADS * 8) return false;
+    bool vec = ((lda | ldy) & 3) == 0 && ((((uintptr_t)a) | ((uintptr_t)y) | ((uintptr_t)w)) & 15) == 0;
+    if (b) vec = vec && ((ldb | ldxs) & 3) == 0 && ((((uintptr_t)b) | ((uintptr_t)xs)) & 15) == 0;
+    return vec;
+}
+hipError_t launch_norm_quantized(const float *a, int64_t lda, const float *b, int64_t ldb, float *xs, int64_t ldxs, int64_t n,
+                                 int64_t ne0, float eps, const float *w, float *y, int64_t ldy, uint8_t *qws, size_t qstride,
+                                 int act_kind, hipStream_t st) {
+    if (n <= 0 || ne0 <= 0) return hipSuccess;
+    if (n > 0x7fffffff || !norm_quantized_applicable(a, lda, b, ldb, xs, ldxs, ne0, w, y, ldy)) return hipErrorInvalidValue;
+    if (b)
+        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, (float *)nullptr,
+                           (int64_t)0, b, ldb, xs, ldxs, qws, qstride, act_kind);
+    else
+        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, (float *)nullptr,
+                           (int64_t)0, (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0, qws, qstride, act_kind);
     return hipGetLastError();
 }
 

@@ -223,6 +223,14 @@ CHIP_API int chip_scale(const float *x, int64_t ldx, int64_t n, int64_t ne0, flo
 CHIP_API int chip_gelu_table(uint16_t *table_host_65536);
 CHIP_API int chip_gelu(const float *x, int64_t ldx, int64_t n, int64_t ne0, const uint16_t *table, float *y, int64_t ldy,
                        void *stream);
+/* The norm in front of a group of matmuls: y = chip_rms_norm(a [+ b, the sum stored to `sum` as in chip_add_rms_norm_mul])
+ * [* w], and y quantized as the activation type of weight type `wtype` into `workspace`, exactly what chip_mul_mat_prepare
+ * (wtype, K = ne0, y, ...) would leave there - the matmuls that read y can go straight to chip_mul_mat_run.  Rows of up to
+ * 8192 values, a multiple of 256, 16-byte aligned with strides that are multiples of 4; CHIP_EUNSUPPORTED otherwise (and
+ * for F16 weights), in which case nothing has been written. */
+CHIP_API int chip_rms_norm_quantized(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
+                                     int64_t ne0, float eps, const float *w, float *y, int64_t ldy, int wtype, void *workspace,
+                                     size_t workspace_bytes, void *stream);
 CHIP_API int chip_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
                                    int64_t ne0, float eps, const float *w, float *y, int64_t ldy, void *stream);
 

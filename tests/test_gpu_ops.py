@@ -200,3 +200,44 @@ def test_scale_and_gelu_equal_the_oracle(dev, orc):
         for t in (dx, dy):
             t.free()
     dt.free()
+
+
+@pytest.mark.parametrize("wt", ["Q4_K", "Q6_K", "Q8_0", "Q4_1"])
+@pytest.mark.parametrize("n,ne0", [(1, 4096), (9, 4096), (3, 256), (5, 8192), (40, 1024)])
+@pytest.mark.parametrize("with_add", [False, True])
+def test_norm_that_leaves_quantized_rows(dev, orc, wt, n, ne0, with_add):
+    """chip_rms_norm_quantized: y equals the unquantizing entry points bit for bit, and the workspace holds what
+    chip_mul_mat_prepare writes from y (compared as the reference's activation blocks, and against the oracle's quantizer)."""
+    import cactus_amd as ca
+    import oracle as O
+    t = getattr(ca, wt)
+    a, b = inputs(13 * n + ne0, n, ne0), inputs(17 * n + ne0, n, ne0)
+    w = (1.0 + 0.1 * np.random.default_rng(ne0).standard_normal(ne0)).astype(np.float32)
+    da, db, dw = dev.to_device(a), dev.to_device(b), dev.to_device(w)
+    ds, dy = dev.alloc(a.nbytes), dev.alloc(a.nbytes)
+    wsz = dev.lib.chip_mul_mat_workspace_size(t, ne0, n)
+    ws = dev.alloc(wsz)
+    dev.check(dev.lib.chip_rms_norm_quantized(da.ptr, ne0, db.ptr if with_add else None, ne0, ds.ptr if with_add else None, ne0, n, ne0,
+                                              1e-5, dw.ptr, dy.ptr, ne0, t, ws.ptr, wsz, None))
+    dev.sync()
+    y = dy.download(np.float32, a.size).reshape(n, ne0)
+    with np.errstate(all="ignore"):
+        x0 = dev.binary("add", a, b) if with_add else a
+        want = dev.binary("mul", dev.rms_norm(x0, 1e-5), w)
+    assert y.tobytes() == want.tobytes()
+    if with_add:
+        assert ds.download(np.float32, a.size).tobytes() == x0.tobytes()
+    at = dev.lib.chip_vec_dot_type(t)
+    rs = dev.row_size(at, ne0)
+    blk = dev.alloc(n * rs)
+    dev.check(dev.lib.chip_workspace_to_blocks(t, ne0, n, ws.ptr, blk.ptr, None))
+    dev.sync()
+    got = blk.download(np.uint8, n * rs).reshape(n, rs)
+    assert np.array_equal(got, orc.quantize_activation(at, y))
+    for tt in (da, db, dw, ds, dy, ws, blk):
+        tt.free()
+    # rows that are no multiple of 256 are declined, nothing written
+    dx = dev.to_device(inputs(3, 2, 320))
+    dyy, ws2 = dev.alloc(2 * 320 * 4), dev.alloc(4096)
+    assert dev.lib.chip_rms_norm_quantized(dx.ptr, 320, None, 0, None, 0, 2, 320, 1e-5, None, dyy.ptr, 320, ca.Q8_0, ws2.ptr, 4096, None) \
+        == ca.CHIP_EUNSUPPORTED
