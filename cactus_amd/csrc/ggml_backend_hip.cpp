@@ -523,11 +523,40 @@ static bool grow_workspace(backend_ctx *c, size_t need) {
     return true;
 }
 
+// The first node (views aside) after index `last` when it is a quantized weight matmul of more than 4 tokens that reads
+// `out`: the norm in front of it can then leave the quantized rows in the workspace.  NULL otherwise.
+const lm_ggml_tensor *quantized_consumer(const lm_ggml_cgraph *g, int last, const lm_ggml_tensor *out) {
+    int j = last + 1;
+    while (j < g->n_nodes && is_view_op(g->nodes[j]->op)) j++;
+    if (j >= g->n_nodes) return nullptr;
+    const lm_ggml_tensor *mm = g->nodes[j];
+    if (mm->op != LM_GGML_OP_MUL_MAT || mm->src[1] != out || !mul_mat_shape_ok(mm) || out->ne[1] <= 4) return nullptr;
+    if (mm->src[0]->type == LM_GGML_TYPE_F16 || out->ne[2] != 1 || out->ne[3] != 1) return nullptr;
+    return mm;
+}
+// Runs the norm (a [+ b -> sum]) [* w] -> out with the quantized rows going to the workspace when the next node is such a
+// matmul; sets key to what the workspace then holds.  CHIP_EUNSUPPORTED: not done, the caller runs the plain kernel.
+int norm_for_quantized_consumer(backend_ctx *c, const lm_ggml_cgraph *g, int last, const float *a, int64_t lda, const float *b,
+                                int64_t ldb, float *sum, int64_t lds, int64_t rows, int64_t ne0, float eps, const float *w,
+                                const lm_ggml_tensor *out, int64_t ldy, quantized_key &key) {
+    const lm_ggml_tensor *mm = quantized_consumer(g, last, out);
+    if (!mm) return CHIP_EUNSUPPORTED;
+    const int wtype = mm->src[0]->type;
+    if (!grow_workspace(c, chip_mul_mat_workspace_size_n(wtype, ne0, mm->src[0]->ne[1], rows))) return CHIP_EUNSUPPORTED;
+    const int rc = chip_rms_norm_quantized(a, lda, b, ldb, sum, lds, rows, ne0, eps, w, (float *)out->data, ldy, wtype, c->workspace,
+                                           c->workspace_size, c->stream);
+    if (rc == CHIP_OK) {
+        key = quantized_key{true, out->data, lm_ggml_nbytes(out), ne0, rows, ldy, chip_vec_dot_type(wtype)};
+    }
+    return rc;
+}
+
 // RMS_NORM or SILU directly followed by the MUL that consumes it, the MUL written over the first node's output: the
 // allocator reuses a node's memory for its consumer only when nothing else reads it (reference ggml-alloc.c in-place
 // rule: one child, no views), so the first node's own result is not needed and the pair runs as one kernel.
 // Returns CHIP_OK and sets fused, or leaves fused false.
-int try_fused_pair(backend_ctx *c, const lm_ggml_tensor *node, const lm_ggml_tensor *next, bool &fused) {
+int try_fused_pair(backend_ctx *c, const lm_ggml_cgraph *g, int i, const lm_ggml_tensor *node, const lm_ggml_tensor *next, bool &fused,
+                   quantized_key &key) {
     fused = false;
     if (!next || next->op != LM_GGML_OP_MUL || next->data != node->data || !elementwise_shape_ok(next)) return CHIP_OK;
     const lm_ggml_tensor *other = next->src[0] == node ? next->src[1] : (next->src[1] == node ? next->src[0] : nullptr);
@@ -540,6 +569,10 @@ int try_fused_pair(backend_ctx *c, const lm_ggml_tensor *node, const lm_ggml_ten
         float eps;
         std::memcpy(&eps, node->op_params, sizeof(float));
         fused = true;
+        if (const int rc = norm_for_quantized_consumer(c, g, i + 1, (const float *)a->data, lda, nullptr, 0, nullptr, 0, rows, a->ne[0], eps,
+                                                       (const float *)other->data, next, ldy, key);
+            rc != CHIP_EUNSUPPORTED)
+            return rc;
         return chip_rms_norm_mul((const float *)a->data, lda, rows, a->ne[0], eps, (const float *)other->data, nullptr, 0,
                                  (float *)next->data, ldy, c->stream);
     }
@@ -564,7 +597,7 @@ bool same_or_disjoint(const void *p, int64_t ldp, const void *q, int64_t ldq, in
 // the sum is still written, since the next residual reads it, but the norm reads it back in the same kernel. The
 // allocator may have placed any of the outputs over a dead operand, so every output block is the same block as, or
 // apart from, every block read. Sets used to the number of nodes run (0: not this pattern).
-int try_fused_add_norm(backend_ctx *c, const lm_ggml_cgraph *g, int i, int &used) {
+int try_fused_add_norm(backend_ctx *c, const lm_ggml_cgraph *g, int i, int &used, quantized_key &key) {
     used = 0;
     const lm_ggml_tensor *add = g->nodes[i];
     const lm_ggml_tensor *norm = i + 1 < g->n_nodes ? g->nodes[i + 1] : nullptr;
@@ -591,6 +624,11 @@ int try_fused_add_norm(backend_ctx *c, const lm_ggml_cgraph *g, int i, int &used
     float eps;
     std::memcpy(&eps, norm->op_params, sizeof(float));
     used = wt ? 3 : 2;
+    if (const int rc = norm_for_quantized_consumer(c, g, i + used - 1, (const float *)a->data, lda, (const float *)b->data, ldb,
+                                                   (float *)add->data, lds, rows, ne0, eps, wt ? (const float *)wt->data : nullptr, out,
+                                                   ldy, key);
+        rc != CHIP_EUNSUPPORTED)
+        return rc;
     return chip_add_rms_norm_mul((const float *)a->data, lda, (const float *)b->data, ldb, (float *)add->data, lds, rows, ne0, eps,
                                  wt ? (const float *)wt->data : nullptr, (float *)out->data, ldy, c->stream);
 }
@@ -704,7 +742,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         }
         if (node->op == LM_GGML_OP_ADD && elementwise_shape_ok(node) && fusion_enabled()) {
             int used = 0;
-            const int rc = try_fused_add_norm(c, cgraph, i, used);
+            quantized_key key;
+            const int rc = try_fused_add_norm(c, cgraph, i, used, key);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (ADD fused with the norm that follows) failed: %s\n", __func__, node->name,
                         chip_error_string(rc));
@@ -712,6 +751,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             }
             if (used) {
                 for (int k = 1; k < used; k++) writes(cgraph->nodes[i + k]);
+                if (key.valid) c->quantized = key;      // after the group's own writes: the workspace holds the group's result
                 g_elementwise_nodes += used;
                 g_fused_pairs += used - 1;
                 i += used - 1;
@@ -721,7 +761,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         if ((node->op == LM_GGML_OP_RMS_NORM || (node->op == LM_GGML_OP_UNARY && node->op_params[0] == LM_GGML_UNARY_OP_SILU)) &&
             elementwise_shape_ok(node) && fusion_enabled()) {
             bool fused = false;
-            const int rc = try_fused_pair(c, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused);
+            quantized_key key;
+            const int rc = try_fused_pair(c, cgraph, i, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused, key);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d, fused with the next node) failed: %s\n", __func__, node->name, node->op,
                         chip_error_string(rc));
@@ -729,6 +770,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             }
             if (fused) {
                 writes(cgraph->nodes[i + 1]);
+                if (key.valid) c->quantized = key;
                 g_elementwise_nodes += 2;
                 g_fused_pairs++;
                 i++;
