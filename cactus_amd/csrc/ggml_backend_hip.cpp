@@ -654,18 +654,43 @@ bool silu_can_wait_for_its_mul(const lm_ggml_cgraph *g, int i) {
     return disjoint(mm, silu->src[0]) && disjoint(mm, silu);
 }
 
-// The RoPE of K followed (views aside) by the CPY of its result into the F16 cache (reference llama-kv-cache.cpp cpy_k:
-// a dense 1-D view of the cache): index of that CPY node, or -1.  The RoPE still writes its own F32 result.
+// A cache store that is run early, inside the kernel that produces what it stores.  The reference builds q, k, v of a layer
+// first and the two stores after them (llama-graph.cpp:1265-1277), so between a producer and its CPY lie views, the
+// projections of the other tensors and the other store.  Running the CPY at the producer's place is safe when none of
+// the nodes in between reads or writes the destination region.  Finds, within the next STORE_LOOKAHEAD nodes after i, the
+// CPY node that `wanted` accepts; -1 if there is none or a node in between touches its destination.
+constexpr int STORE_LOOKAHEAD = 16;
+bool ranges_apart(const lm_ggml_tensor *p, const lm_ggml_tensor *q) {
+    if (!p->data || !q->data) return true;            // no memory behind it (an unallocated leaf cannot alias the destination)
+    return disjoint(p, q);
+}
+template <typename F>
+int early_store_index(const lm_ggml_cgraph *g, int i, F wanted) {
+    const int end = i + 1 + STORE_LOOKAHEAD < g->n_nodes ? i + 1 + STORE_LOOKAHEAD : g->n_nodes;
+    for (int j = i + 1; j < end; j++) {
+        const lm_ggml_tensor *cp = g->nodes[j];
+        if (cp->op != LM_GGML_OP_CPY || !wanted(cp)) continue;
+        for (int m = i + 1; m < j; m++) {
+            const lm_ggml_tensor *t = g->nodes[m];
+            if (is_view_op(t->op)) continue;
+            if (!ranges_apart(t, cp)) return -1;
+            for (int k = 0; k < LM_GGML_MAX_SRC; k++)
+                if (t->src[k] && !ranges_apart(t->src[k], cp)) return -1;
+        }
+        return j;
+    }
+    return -1;
+}
+
+// The RoPE of K and the CPY of its result into the F16 cache (reference llama-kv-cache.cpp cpy_k: a dense 1-D view of the
+// cache): index of that CPY node, or -1.  The RoPE still writes its own F32 result.
 int rope_store_index(const lm_ggml_cgraph *g, int i) {
     const lm_ggml_tensor *rope = g->nodes[i];
-    int j = i + 1;
-    while (j < g->n_nodes && is_view_op(g->nodes[j]->op)) j++;
-    if (j >= g->n_nodes) return -1;
-    const lm_ggml_tensor *cp = g->nodes[j];
-    if (cp->op != LM_GGML_OP_CPY || cp->src[0] != rope || cp->type != LM_GGML_TYPE_F16 || rope->type != LM_GGML_TYPE_F32) return -1;
-    if (!attn_side_shape_ok(cp) || !dense(cp) || !dense(rope) || n_elements(cp) != n_elements(rope)) return -1;
-    if (!disjoint(cp, rope) || !disjoint(cp, rope->src[0])) return -1;
-    return j;
+    if (rope->type != LM_GGML_TYPE_F32 || !dense(rope)) return -1;
+    return early_store_index(g, i, [rope](const lm_ggml_tensor *cp) {
+        return cp->src[0] == rope && cp->type == LM_GGML_TYPE_F16 && attn_side_shape_ok(cp) && dense(cp) &&
+               n_elements(cp) == n_elements(rope) && disjoint(cp, rope) && disjoint(cp, rope->src[0]);
+    });
 }
 
 // ffn_gate and ffn_up in llama.cpp's node order: gate matmul, SILU, up matmul, MUL.  With up to 4 tokens the two matmuls
@@ -690,18 +715,18 @@ int paired_matmul_index(const lm_ggml_cgraph *g, int i) {
 // Index of that CPY node, or -1.  The matmul still writes its own F32 result.
 int transposed_store_index(const lm_ggml_cgraph *g, int i) {
     const lm_ggml_tensor *mm = g->nodes[i];
-    int j = i + 1;
-    while (j < g->n_nodes && is_view_op(g->nodes[j]->op)) j++;
-    if (j >= g->n_nodes) return -1;
-    const lm_ggml_tensor *cp = g->nodes[j], *tr = cp->src[0];
-    if (cp->op != LM_GGML_OP_CPY || !tr || tr->op != LM_GGML_OP_TRANSPOSE || tr->src[0] != mm || cp->type != LM_GGML_TYPE_F16) return -1;
     const int64_t N = mm->ne[0], n = mm->ne[1];
-    if (cp->ne[0] != n || cp->ne[1] != N || cp->ne[2] != 1 || cp->ne[3] != 1 || cp->nb[0] != 2 || cp->nb[1] % 2 != 0 ||
-        cp->nb[1] < (size_t)n * 2)
-        return -1;
-    if (!is_hip_buffer(cp->view_src ? cp->view_src->buffer : cp->buffer)) return -1;
-    if (!disjoint(cp, mm) || !disjoint(cp, mm->src[1])) return -1;
-    return j;
+    return early_store_index(g, i, [mm, N, n](const lm_ggml_tensor *cp) {
+        // the source: a TRANSPOSE of the projection's result (through reshapes: views collapse onto the tensor that owns the memory)
+        const lm_ggml_tensor *tr = cp->src[0];
+        if (!tr || tr->op != LM_GGML_OP_TRANSPOSE || (tr->view_src != mm && tr->src[0] != mm) || tr->view_offs != 0) return false;
+        if (tr->ne[0] != n || tr->ne[1] != N || tr->ne[2] != 1 || tr->ne[3] != 1 || tr->nb[0] != mm->nb[1] || tr->nb[1] != mm->nb[0]) return false;
+        if (cp->type != LM_GGML_TYPE_F16 || cp->ne[0] != n || cp->ne[1] != N || cp->ne[2] != 1 || cp->ne[3] != 1 || cp->nb[0] != 2 ||
+            cp->nb[1] % 2 != 0 || cp->nb[1] < (size_t)n * 2)
+            return false;
+        if (!is_hip_buffer(cp->view_src ? cp->view_src->buffer : cp->buffer)) return false;
+        return disjoint(cp, mm) && disjoint(cp, mm->src[1]);
+    });
 }
 
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
@@ -709,7 +734,12 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     c->rope_key.valid = false;                        // positions may have changed since the last call
     c->quantized.valid = false;                       // and so may any activation
     const lm_ggml_tensor *waiting_silu = nullptr;     // a SILU held back for the MUL two nodes on
-    int stored_by_rope = -1;                          // index of a CPY node that ran inside the RoPE (or the matmul) before it
+    int stored_early[4] = {-1, -1, -1, -1};           // CPY nodes that already ran inside the RoPE / the projection before them
+    auto remember_store = [&stored_early](int j) {
+        for (int &slot : stored_early)
+            if (slot < 0) { slot = j; return true; }
+        return false;
+    };
     int paired_matmul = -1;                           // index of an up projection that ran with its gate projection
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
@@ -791,9 +821,11 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             g_elementwise_nodes++;
             continue;
         }
-        if (i == stored_by_rope) {                    // this CPY ran in the kernel of the RoPE before it
-            stored_by_rope = -1;
-            continue;
+        {
+            bool done = false;                        // this CPY ran in the kernel of the RoPE / the projection before it
+            for (int &slot : stored_early)
+                if (slot == i) { slot = -1; done = true; }
+            if (done) continue;
         }
         if (i == paired_matmul) {                     // this matmul ran in the launch of the one two nodes before it
             paired_matmul = -1;
@@ -802,9 +834,9 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         if (is_attn_side_op(node->op) && attn_side_shape_ok(node)) {
             const lm_ggml_tensor *store = nullptr;
             if (node->op == LM_GGML_OP_ROPE && fusion_enabled()) {
-                stored_by_rope = rope_store_index(cgraph, i);
-                if (stored_by_rope >= 0) {
-                    store = cgraph->nodes[stored_by_rope];
+                const int j = rope_store_index(cgraph, i);
+                if (j >= 0 && remember_store(j)) {
+                    store = cgraph->nodes[j];
                     writes(store);
                     g_elementwise_nodes++;
                     g_fused_pairs++;
@@ -861,11 +893,10 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         int rc;
         const int64_t ldx = (int64_t)(x->nb[1] / 4);
         int store_t = -1;
-        if (n <= 4 && fusion_enabled() && (store_t = transposed_store_index(cgraph, i)) >= 0) {
+        if (n <= 4 && fusion_enabled() && (store_t = transposed_store_index(cgraph, i)) >= 0 && remember_store(store_t)) {
             lm_ggml_tensor *cp = cgraph->nodes[store_t];
             writes(cp);
             c->quantized.valid = false;
-            stored_by_rope = store_t;                  // skipped like the CPY that ran inside a RoPE
             rc = chip_mul_mat_store_t(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
                                       (int64_t)(node->nb[1] / 4), (uint16_t *)cp->data, (int64_t)(cp->nb[1] / 2), c->workspace,
                                       c->workspace_size, c->stream);

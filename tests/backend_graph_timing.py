@@ -86,8 +86,8 @@ for l in range(NL):
     v = L.lm_ggml_mul_mat(ctx, w["wv"], cur)
     k_store = L.lm_ggml_cpy(ctx, k, L.lm_ggml_view_1d(ctx, kc, n * KV, 2 * KV * head))
     v_store = L.lm_ggml_cpy(ctx, L.lm_ggml_transpose(ctx, v), L.lm_ggml_view_2d(ctx, vc, n, KV, kv_size * 2, head * 2))
-    L.lm_ggml_build_forward_expand(g, k_store)
-    L.lm_ggml_build_forward_expand(g, v_store)
+    for t in (q, k, v, k_store, v_store):                # the reference's order (llama-graph.cpp:1265-1277): q, k, v, then the stores
+        L.lm_ggml_build_forward_expand(g, t)
     kview = L.lm_ggml_view_3d(ctx, kc, hd, n_head_kv, n_kv, 2 * hd, 2 * KV, 0)
     vview = L.lm_ggml_view_3d(ctx, vc, n_kv, n_head_kv, hd, 2 * kv_size * hd, 2 * kv_size, 0)
     qp = L.lm_ggml_permute(ctx, q, 0, 2, 1, 3)

@@ -824,9 +824,8 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     out = L.lm_ggml_add(ctx, L.lm_ggml_mul_mat(ctx, two, merged), tx)
     L.lm_ggml_set_output(out)
     g = L.lm_ggml_new_graph(ctx)
-    L.lm_ggml_build_forward_expand(g, k_store)          # the stores first, as the reference builds its graph
-    L.lm_ggml_build_forward_expand(g, v_store)
-    L.lm_ggml_build_forward_expand(g, out)
+    for t in (q, k, v, k_store, v_store, out):           # q, k, v first, then the two stores, as the reference builds its graph
+        L.lm_ggml_build_forward_expand(g, t)              # (llama-graph.cpp:1265-1277)
     backends = (C.c_void_p * 2)(hip, cpu)
     sched = L.lm_ggml_backend_sched_new(backends, None, 2, 128, False, True)
     assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
