@@ -581,6 +581,48 @@ def test_shared_quantized_input_is_dropped_when_the_input_is_overwritten(host, o
     L.lm_ggml_free(ctx)
 
 
+def test_cache_store_is_not_run_early_past_a_reader_of_its_destination(host, orc):
+    """Between a RoPE and the CPY of its result into the cache lies a node that reads that cache region: the store must
+    stay where it is (the reader sees the old contents).  Without the reader the same store runs in the RoPE's kernel."""
+    import cactus_amd
+    L = host.L
+    hd, n_head, n_tok = 64, 4, 3
+    E = hd * n_head * n_tok
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((n_tok, n_head, hd)).astype(np.float32)
+    pos = np.array([3, 4, 5], np.int32)
+    old = (rng.standard_normal(E) * 0.5).astype(np.float16)
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_fused_pairs.restype = C.c_ulonglong
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    for with_reader in (True, False):
+        be = L.lm_ggml_backend_dev_init(dev, None)
+        ctx = host.context()
+        tx = host.tensor_3d(ctx, O.F32, hd, n_head, n_tok, "x")
+        tp = L.lm_ggml_new_tensor_1d(ctx, 26, n_tok)
+        kc = L.lm_ggml_new_tensor_1d(ctx, O.F16, E)
+        seen = L.lm_ggml_new_tensor_1d(ctx, O.F32, E)
+        r = L.lm_ggml_rope_ext(ctx, tx, tp, None, hd, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+        reader = L.lm_ggml_cpy(ctx, L.lm_ggml_view_1d(ctx, kc, E, 0), seen)
+        store = L.lm_ggml_cpy(ctx, r, L.lm_ggml_view_1d(ctx, kc, E, 0))
+        g = L.lm_ggml_new_graph(ctx)
+        for t in ((r, reader, store) if with_reader else (r, store)):
+            L.lm_ggml_build_forward_expand(g, t)
+        buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+        host.set(tx, x); host.set(tp, pos); host.set(kc, old)
+        before = blib.lm_ggml_backend_hip_get_fused_pairs()
+        assert L.lm_ggml_backend_graph_compute(be, g) == 0
+        assert blib.lm_ggml_backend_hip_get_fused_pairs() - before == (0 if with_reader else 1)
+        want = orc.rope(x, pos, hd, 2)
+        got = host.get(kc, np.float16, (E,)).astype(np.float32)
+        assert (np.abs(got - want.reshape(-1)) <= 2 * np.spacing(np.abs(want.reshape(-1)).astype(np.float16)).astype(np.float32) + 1e-3).all()
+        if with_reader:
+            assert host.get(seen, np.float32, (E,)).tobytes() == old.astype(np.float32).tobytes()
+        L.lm_ggml_backend_buffer_free(buf)
+        L.lm_ggml_backend_free(be)
+        L.lm_ggml_free(ctx)
+
+
 def test_gelu_and_scale_nodes(host, orc):
     """A GELU-gated FFN entry and a SCALE (Gemma-style graphs: lm_ggml_gelu, lm_ggml_scale): both run on the device, and the
     GELU goes through the host framework's own table, so the result equals the reference CPU backend bit for bit."""
