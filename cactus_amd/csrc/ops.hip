@@ -62,12 +62,12 @@ __device__ __forceinline__ float silu1(float x) { return x / (1.0f + v_expf_lane
 // With ADD, the row normalised is a + b (the residual ADD node in front of a norm): the sum is stored to xs, which may be a
 // or b themselves (every thread reads an element of a and b before it writes that element of xs, and reads back only its
 // own elements), and the norm then runs over the stored sum.
-template <bool ADD>
+template <bool ADD, int QKIND = 0>
 __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, int64_t ldx, int64_t ne0, float eps,
                                                               float *__restrict__ y, int64_t ldy, const float *__restrict__ w,
                                                               float *__restrict__ yn, int64_t ldyn, const float *b, int64_t ldb,
-                                                              float *xs, int64_t ldxs, uint8_t *__restrict__ qws, size_t qstride,
-                                                              int qkind) {
+                                                              float *xs, int64_t ldxs, uint8_t *__restrict__ qws, size_t qstride) {
+    constexpr int qkind = QKIND;                                 // 0: no quantized copy; 1: Q8_0 / Q8_1 planes; 2: Q8_K planes
     __shared__ double part[EW_THREADS / 64];
     const float *xr = x + (size_t)blockIdx.x * ldx;
     float *yr = y + (size_t)blockIdx.x * ldy;
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
                 *reinterpret_cast<float4 *>(yr + i) = v;
                 // the row as the next matmuls want it: quantized into the workspace planes of token blockIdx.x (ne0 is a
                 // multiple of 256 here, so a wave is inside the row with all its lanes or not at all)
-                if (qkind == 2) {
+                if constexpr (qkind == 2) {
                     const Q8_KLane q = quantize_q8_K_lane(v);
                     uint8_t *base = qws + (size_t)blockIdx.x * qstride;
                     const int64_t sb = i >> 8;
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
                     *reinterpret_cast<uint32_t *>(base + i) = q.packed;
                     if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(ne0))[sb] = q.d;
                     if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(ne0))[sb * 16 + (lane >> 2)] = (int16_t)q.bsum;
-                } else if (qkind == 1) {
+                } else if constexpr (qkind == 1) {
                     const Q8_0Lane q = quantize_q8_0_lane(v);
                     uint8_t *base = qws + (size_t)blockIdx.x * qstride;
                     const int64_t blk = i >> 5;
@@ -751,7 +751,7 @@ hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, 
         const int64_t rows = n - r0 < (1 << 30) ? n - r0 : (1 << 30);
         hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)rows), dim3(EW_THREADS), 0, st, x + r0 * ldx, ldx, ne0, eps,
                            y + r0 * ldy, ldy, (const float *)nullptr, (float *)nullptr, (int64_t)0, (const float *)nullptr,
-                           (int64_t)0, (float *)nullptr, (int64_t)0, (uint8_t *)nullptr, (size_t)0, 0);
+                           (int64_t)0, (float *)nullptr, (int64_t)0, (uint8_t *)nullptr, (size_t)0);
     }
     return hipGetLastError();
 }
@@ -760,7 +760,7 @@ hipError_t launch_rms_norm_mul(const float *x, int64_t ldx, int64_t n, int64_t n
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     if (n > 0x7fffffff) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, x, ldx, ne0, eps, y, ldy, w, yn, ldyn,
-                       (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0, (uint8_t *)nullptr, (size_t)0, 0);
+                       (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0, (uint8_t *)nullptr, (size_t)0);
     return hipGetLastError();
 }
 hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *xs, int64_t ldxs, int64_t n,
@@ -769,7 +769,7 @@ hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, 
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     if (n > 0x7fffffff) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rms_norm_kernel<true>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, yn, ldyn, b,
-                       ldb, xs, ldxs, (uint8_t *)nullptr, (size_t)0, 0);
+                       ldb, xs, ldxs, (uint8_t *)nullptr, (size_t)0);
     return hipGetLastError();
 }
 // The norm (with or without the residual ADD in front: b may be NULL) whose result also goes, quantized as the activation
@@ -787,12 +787,15 @@ hipError_t launch_norm_quantized(const float *a, int64_t lda, const float *b, in
                                  int act_kind, hipStream_t st) {
     if (n <= 0 || ne0 <= 0) return hipSuccess;
     if (n > 0x7fffffff || !norm_quantized_applicable(a, lda, b, ldb, xs, ldxs, ne0, w, y, ldy)) return hipErrorInvalidValue;
-    if (b)
-        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, (float *)nullptr,
-                           (int64_t)0, b, ldb, xs, ldxs, qws, qstride, act_kind);
-    else
-        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3((unsigned)n), dim3(EW_THREADS), 0, st, a, lda, ne0, eps, y, ldy, w, (float *)nullptr,
-                           (int64_t)0, (const float *)nullptr, (int64_t)0, (float *)nullptr, (int64_t)0, qws, qstride, act_kind);
+    if (act_kind != 1 && act_kind != 2) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)n), block(EW_THREADS);
+    const float *nob = nullptr;
+    float *nos = nullptr, *noyn = nullptr;
+    const int64_t z = 0;
+    if (b && act_kind == 1)  hipLaunchKernelGGL((rms_norm_kernel<true, 1>), grid, block, 0, st, a, lda, ne0, eps, y, ldy, w, noyn, z, b, ldb, xs, ldxs, qws, qstride);
+    else if (b)              hipLaunchKernelGGL((rms_norm_kernel<true, 2>), grid, block, 0, st, a, lda, ne0, eps, y, ldy, w, noyn, z, b, ldb, xs, ldxs, qws, qstride);
+    else if (act_kind == 1)  hipLaunchKernelGGL((rms_norm_kernel<false, 1>), grid, block, 0, st, a, lda, ne0, eps, y, ldy, w, noyn, z, nob, z, nos, z, qws, qstride);
+    else                     hipLaunchKernelGGL((rms_norm_kernel<false, 2>), grid, block, 0, st, a, lda, ne0, eps, y, ldy, w, noyn, z, nob, z, nos, z, qws, qstride);
     return hipGetLastError();
 }
 
