@@ -1,17 +1,21 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized MUL_MAT hot path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): Q8_0 x Q8_0 decode GEMV at Llama FFN shapes, W[11008 x 4096]
-and W[4096 x 11008], token batch n in {1, 2, 4, 8}.  One "step" = the eight ops (2 shapes x 4 batch sizes),
-each op being what LM_GGML_OP_MUL_MAT does: quantize the fp32 activations to Q8_0 on the GPU, then the GEMV.
-Inputs are resident in HBM before the timed region; weights rotate through > 512 MB of distinct copies per
-shape so that the 256 MB Infinity Cache cannot serve them (cold numbers).
+Headline workload (BASELINE configs[4], the largest single-GPU configuration): every weight matmul of one decode step of a
+random-init Llama-3-8B-shaped Q4_K_M model - 32 layers of wq / wk / wv(Q6_K) / wo / ffn_gate / ffn_up / ffn_down(Q6_K) plus
+the Q6_K output head, 225 matmuls over 4 875 853 824 weight bytes - at one token.  One "step" = that serial chain, issued
+through the C-ABI the way the ggml backend issues it (matmuls that share an activation in one launch), each op doing what
+LM_GGML_OP_MUL_MAT does: quantize the fp32 activation on the GPU, then the GEMV.  The weights of a step (4.9 GB) exceed the
+256 MB Infinity Cache many times over, so every read is cold.  The step is replayed as a HIP graph (the host cannot issue
+225 launches from Python in the time the GPU needs for them); --eager issues the same launches one by one, for runs under a
+profiler.
 
-Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a step (HIP events on the launch
-stream).  `roofline` is for the dominant kernel, the n = 1 GEMV, timed with its own HIP event pairs inside the
-timed region.  `cpu_baseline` times the reference's own ggml-cpu MUL_MAT (oracle/_ref, when it travelled) or the
-oracle port on the host cores for a bounded sample of the same workload.  `extra` carries the other BASELINE
-configurations (Q4_0 mat-vec, Q4_K GEMV, prefill GEMM TOPS, Llama-3-8B-shaped decode trace).
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a step (HIP events on the launch stream, K steps
+between one pair of events).  `roofline` is for the kernel with the largest share of the step, timed with its own HIP event
+pair over back-to-back launches on distinct (cold) weights.  `cpu_baseline` times the reference's own ggml-cpu MUL_MAT
+(oracle/_ref, when it travelled) or the oracle port on the host cores for a bounded sample of the same workload.  `extra`
+carries the other BASELINE configurations (Q4_0 mat-vec, Q8_0 FFN GEMVs, Q4_K GEMV, prefill GEMM TOPS, the trace at 8 tokens
+and as a 512-token prefill chunk).
 """
 import argparse
 import ctypes as C
@@ -28,10 +32,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
 F16_PEAK_TFLOPS = 2500.0       # MI355X published dense fp16 MFMA rate
-# HBM bytes per launch of the n = 1 Q8_0 GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
-# counters read for a device-to-device copy of known size (profiles/gemv_q8_0_n1_hbm_traffic_pmc.md): mean of the
-# two headline shapes.  Algorithmic bytes per launch: 47 967 232.
-N1_GEMV_HBM_TRAFFIC_BYTES = 48350573
+# HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the
+# same counters read for a device-to-device copy of known size.  The summary of those runs is a committed text file; its
+# line "traffic_bytes_per_launch: <kernel key> <bytes>" is read here, so the figure in the JSON is the profile's.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemv_trace_dominant_kernel_hbm_traffic_pmc.md")
 
 
 def parse():
@@ -41,8 +45,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-trace", action="store_true",
-                    help="skip the model-shaped HIP-graph trace and the issue-rate probe (for runs under a profiler)")
+    ap.add_argument("--eager", action="store_true",
+                    help="issue every launch of the trace directly instead of replaying a HIP graph, and skip everything that "
+                         "replays one (for runs under rocprofv3 --kernel-trace; the host then bounds the step time)")
+    ap.add_argument("--no-backend", action="store_true", help="skip the ggml-backend graph timing (a child process)")
     return ap.parse_args()
 
 
@@ -59,6 +65,9 @@ class Hip:
         L.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         L.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
         L.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        L.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        L.hipGraphDestroy.argtypes = [C.c_void_p]
+        L.hipStreamWaitEvent.argtypes = [C.c_void_p, C.c_void_p, C.c_uint]
         L.hipDeviceSynchronize.argtypes = []
 
     def event(self):
@@ -68,6 +77,20 @@ class Hip:
 
     def record(self, e, stream):
         assert self.lib.hipEventRecord(e, stream) == 0
+
+    def capture(self, stream, fn):
+        """Runs fn() under stream capture and returns a replay function and a destroy function."""
+        L = self.lib
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert L.hipStreamBeginCapture(stream, 0) == 0
+        fn()
+        assert L.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert L.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+
+        def destroy():
+            L.hipGraphExecDestroy(gexec)
+            L.hipGraphDestroy(graph)
+        return (lambda: L.hipGraphLaunch(gexec, stream)), destroy
 
     def elapsed_ms(self, a, b):
         assert self.lib.hipEventSynchronize(b) == 0
@@ -120,7 +143,8 @@ def algorithmic_bytes(wbytes, K, N, n):
     return wbytes + 4 * n * (K + N)            # weights once + fp32 activations in + fp32 outputs out
 
 
-def bench_headline(dev, hip, steps, warmup):
+def bench_config2(dev, hip, steps=20, warmup=3):
+    """BASELINE configs[1]: Q8_0 FFN-shaped GEMVs at 1, 2, 4, 8 tokens, cold weights (rotating copies)."""
     import cactus_amd as ca
     L = dev.lib
     rng = np.random.default_rng(2)
@@ -171,11 +195,11 @@ def bench_headline(dev, hip, steps, warmup):
     dev.sync(st)
     k_bytes = algorithmic_bytes(mats[0].bytes, 4096, 11008, 1)      # both shapes move the same byte count
     achieved = k_bytes / (k_us * 1e-6) / 1e9
-    roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": N1_GEMV_HBM_TRAFFIC_BYTES,
-            "kernel": "gemv_kernel<Q8_0, n=1, fused activation quantize> (W[11008x4096] and W[4096x11008], cold weights)",
-            "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 2), "launches_timed": 2 * reps}
-    return value, ms_per_step, step_bytes, roof, {"copies_per_shape": [m.copies for m in mats]}
+    for m in mats:
+        m.buf.free()
+    return {"step_8_ops_us": round(ms_per_step * 1e3, 2), "step_GBps": round(value, 1), "bytes_per_step": step_bytes,
+            "n1_us_per_launch": round(k_us, 2), "n1_GBps": round(achieved, 1), "n1_hbm_frac": round(achieved / HBM_PEAK_GBS, 4),
+            "n1_bytes_per_launch": k_bytes, "copies_per_shape": [m.copies for m in mats]}
 
 
 def time_runs(dev, hip, st, fn, iters, warm=3):
@@ -190,7 +214,7 @@ def time_runs(dev, hip, st, fn, iters, warm=3):
     return hip.elapsed_ms(a, b) * 1e3 / iters          # microseconds per call
 
 
-def bench_extra(dev, hip, trace=True):
+def bench_extra(dev, hip):
     import cactus_amd as ca
     L = dev.lib
     rng = np.random.default_rng(5)
@@ -387,9 +411,6 @@ def bench_extra(dev, hip, trace=True):
 
     upload_case()
 
-    if trace:
-        out.update(bench_trace(dev, hip, st, rng))
-        out["mfma_i8_measured_peak"] = measured_mfma_peak()
     return out
 
 
@@ -398,7 +419,7 @@ def measured_mfma_peak():
     form the GEMM uses, so TOPS can be read against the measured matrix peak as well as the datasheet one."""
     import re
     import subprocess
-    exe = os.path.join(ROOT, "cactus_amd", "lib", "probe_issue_rates")
+    exe = os.path.join(ROOT, "cactus_amd", "probes", "bin", "issue_rates")
     if not os.path.exists(exe):
         return None
     try:
@@ -414,249 +435,440 @@ def measured_mfma_peak():
     return {"instruction": "v_mfma_i32_32x32x32_i8", "TOPS": best, "datasheet_TOPS": INT8_PEAK_TOPS} if best else None
 
 
-def bench_trace(dev, hip, st, rng):
-    """config 5: every weight matmul of one decode step of a Llama-3-8B-shaped Q4_K_M model (32 layers, 225
-    matmuls; attn_v / ffn_down / output head in Q6_K, the rest Q4_K), replayed as a HIP graph, once as a serial
-    chain and once with the independent matmuls of a layer as concurrent graph branches; and the same matmuls for
-    one 512-token prefill chunk (serial only)."""
-    import cactus_amd as ca
-    L = dev.lib
+class Trace:
+    """BASELINE configs[4]: the weight matmuls of a Llama-3-8B-shaped Q4_K_M model (32 layers; attn_v / ffn_down / the
+    output head in Q6_K, the rest Q4_K) as random-init weights in one arena, and the launches of one step over them."""
     H, FF, KV, V, NL = 4096, 14336, 1024, 128256, 32
-    layer = [("wq", ca.Q4_K, H, H, "attn"), ("wk", ca.Q4_K, KV, H, "attn"), ("wv", ca.Q6_K, KV, H, "attn"),
-             ("wo", ca.Q4_K, H, H, "wo"), ("up", ca.Q4_K, FF, H, "ffn"), ("gate", ca.Q4_K, FF, H, "ffn"),
-             ("down", ca.Q6_K, H, FF, "down")]
-    sizes = [N * dev.row_size(t, K) for (_, t, N, K, _) in layer]
-    layer_bytes = sum(sizes)
-    head_bytes = V * dev.row_size(ca.Q6_K, H)
-    total = NL * layer_bytes + head_bytes
-    arena = dev.alloc(total)
-    off = 0
-    first = []
-    for (name, t, N, K, _), sz in zip(layer, sizes):
-        arena.upload(synth_weights(dev, t, N, K, rng), offset=off)
-        first.append(off)
-        off += sz
-    for l in range(1, NL):
-        dev.check(L.chip_memcpy_d2d(arena.ptr + l * layer_bytes, arena.ptr, layer_bytes, None))
-    head_off = NL * layer_bytes
-    part = V // 8
-    arena.upload(synth_weights(dev, ca.Q6_K, part, H, rng), offset=head_off)
-    for i in range(1, 8):
-        dev.check(L.chip_memcpy_d2d(arena.ptr + head_off + i * (head_bytes // 8), arena.ptr + head_off, head_bytes // 8, None))
-    dev.sync()
 
-    hl = hip.lib
-    hl.hipStreamWaitEvent.argtypes = [C.c_void_p, C.c_void_p, C.c_uint]
-    side = [C.c_void_p(), C.c_void_p()]
-    for s_ in side:
-        dev.check(L.chip_stream_create(C.byref(s_)))
+    def __init__(self, dev, hip, rng):
+        import cactus_amd as ca
+        self.dev, self.hip, self.ca = dev, hip, ca
+        L = dev.lib
+        H, FF, KV, V, NL = self.H, self.FF, self.KV, self.V, self.NL
+        self.layer = [("wq", ca.Q4_K, H, H), ("wk", ca.Q4_K, KV, H), ("wv", ca.Q6_K, KV, H), ("wo", ca.Q4_K, H, H),
+                      ("up", ca.Q4_K, FF, H), ("gate", ca.Q4_K, FF, H), ("down", ca.Q6_K, H, FF)]
+        sizes = [N * dev.row_size(t, K) for (_, t, N, K) in self.layer]
+        self.layer_bytes = sum(sizes)
+        self.head_bytes = V * dev.row_size(ca.Q6_K, H)
+        self.total = NL * self.layer_bytes + self.head_bytes
+        self.arena = dev.alloc(self.total)
+        off, self.first = 0, []
+        for (name, t, N, K), sz in zip(self.layer, sizes):
+            self.arena.upload(synth_weights(dev, t, N, K, rng), offset=off)
+            self.first.append(off)
+            off += sz
+        for l in range(1, NL):
+            dev.check(L.chip_memcpy_d2d(self.arena.ptr + l * self.layer_bytes, self.arena.ptr, self.layer_bytes, None))
+        self.head_off = NL * self.layer_bytes
+        self.arena.upload(synth_weights(dev, ca.Q6_K, V // 8, H, rng), offset=self.head_off)
+        for i in range(1, 8):
+            dev.check(L.chip_memcpy_d2d(self.arena.ptr + self.head_off + i * (self.head_bytes // 8), self.arena.ptr + self.head_off,
+                                        self.head_bytes // 8, None))
+        dev.sync()
+        self.st = C.c_void_p()
+        dev.check(L.chip_stream_create(C.byref(self.st)))
+        self.bufs = {}
 
-    def full_layers(n, n_kv, ws, wsz):
-        """Every node of the 32 layers as llama.cpp builds them without flash attention (norms, projections, RoPE, cache
-        stores, kq, soft-max, kqv, head merge, residuals, SiLU * up), n new tokens against n_kv cached positions, as one
-        HIP graph on one stream: what a decode step costs when no activation leaves the device."""
-        hd, n_head, n_head_kv, kv_size = 128, 32, 8, 4096
-        A4 = C.c_int64 * 4
-        f32 = lambda *shape: dev.alloc(int(np.prod(shape)) * 4)
-        resid = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
-        wn = dev.to_device((1 + 0.1 * rng.standard_normal(H)).astype(np.float32))
-        pos = dev.to_device(np.arange(n_kv - n, n_kv, dtype=np.int32))
-        mask = dev.to_device(np.zeros((max(n, 8), n_kv), np.float16))
-        cur, q, k, v, merged, att = f32(n, H), f32(n, H), f32(n, KV), f32(n, KV), f32(n, H), f32(n, H)
-        kq, kqv = f32(n_head, n, n_kv), f32(n_head, n, hd)
-        up, gate = f32(n, FF), f32(n, FF)
-        caches = dev.alloc(NL * 2 * kv_size * KV * 2)
-        dev.check(L.chip_memset(caches.ptr, 0, caches.nbytes, None))
-        aws_bytes = max(L.chip_mul_mat_f16_batched_workspace_size(hd, n_kv, n_head_kv, n_head, n),
-                        L.chip_mul_mat_f16_batched_workspace_size(n_kv, hd, n_head_kv, n_head, n), 256)
-        aws = dev.alloc(aws_bytes)
-        rope_tab = dev.alloc(n * hd * 4)
+    def weights(self, l):
+        base = self.arena.ptr + l * self.layer_bytes
+        return {name: (t, base + o, N, K) for (name, t, N, K), o in zip(self.layer, self.first)}
+
+    def io(self, n):
+        """Activations, outputs and workspace for n tokens (kept for the life of the trace)."""
+        if n not in self.bufs:
+            dev, L, ca = self.dev, self.dev.lib, self.ca
+            rng = np.random.default_rng(11 + n)
+            wsz = max([L.chip_mul_mat_workspace_size_n(t, K, N, n) for (_, t, N, K) in self.layer] +
+                      [L.chip_mul_mat_workspace_size_n(ca.Q6_K, self.H, self.V, n)])
+            self.bufs[n] = {"x_h": dev.to_device(rng.standard_normal((n, self.H)).astype(np.float32)),
+                            "x_ff": dev.to_device(rng.standard_normal((n, self.FF)).astype(np.float32)),
+                            "y": dev.alloc(4 * n * self.V * 4), "ws": dev.alloc(wsz), "wsz": wsz}
+        return self.bufs[n]
+
+    def step_bytes(self, n):
+        return self.total + 4 * n * (self.NL * sum(K + N for (_, _, N, K) in self.layer) + self.H + self.V)
+
+    # ---- the launches, per class of op (one entry of OPS = what the backend issues as one call)
+    def op_calls(self, n):
+        """name -> function(layer index) that issues that op of that layer; 'head' ignores the index."""
+        dev, L, ca, st = self.dev, self.dev.lib, self.ca, self.st
+        b = self.io(n)
+        ws, wsz, y = b["ws"].ptr, b["wsz"], b["y"].ptr
+        xh, xff = b["x_h"].ptr, b["x_ff"].ptr
+        V, H = self.V, self.H
+        nV = n * V * 4
         ck = dev.check
 
-        def mm(t, wptr, N, K, src, dst, shared=False):
-            """shared: src was quantized by the previous matmul (same tensor, same activation type), as the backend reuses it"""
-            if n <= 4:                                                    # the GEMV quantizes in its prologue
-                ck(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, dst.ptr, N, ws.ptr, wsz, st))
-                return
-            if not shared:
-                ck(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, ws.ptr, wsz, st))
-            ck(L.chip_mul_mat_run_ws(t, wptr, dev.row_size(t, K), K, N, n, ws.ptr, wsz, dst.ptr, N, st))
+        def qkv(l):                      # three matrices on one activation: one call (one launch up to 4 tokens)
+            W = self.weights(l)
+            arr = (ca.Mat * 3)()
+            for i, nm in enumerate(("wq", "wk", "wv")):
+                t, p, N, K = W[nm]
+                arr[i] = ca.Mat(t, p, dev.row_size(t, K), N, y + i * nV, N, None, 0)
+            ck(L.chip_mul_mat_group(arr, 3, H, xh, H, n, ws, wsz, st))
 
-        def step():
-            for l in range(NL):
-                base = arena.ptr + l * layer_bytes
-                W = {name: (t, base + o, N, K) for (name, t, N, K, _), o in zip(layer, first)}
-                kc = caches.ptr + (2 * l) * kv_size * KV * 2
-                vc = kc + kv_size * KV * 2
-                if l == 0:
-                    ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))  # norm + weight: one kernel, as the backend fuses them
-                mm(*W["wq"], cur, q); mm(*W["wk"], cur, k, True)
-                if n <= 4:                                                # V projection and its transposed store in one launch
-                    t_, wv_, N_, K_ = W["wv"]
-                    ck(L.chip_mul_mat_store_t(t_, wv_, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, v.ptr, N_, vc + 2 * (n_kv - n), kv_size,
-                                              ws.ptr, wsz, st))
-                else:
-                    mm(*W["wv"], cur, v, True)
-                if l == 0:                                                # one cos / sin table per step, as the backend keeps it
-                    ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
-                ck(L.chip_rope_apply(q.ptr, hd, hd * n_head, rope_tab.ptr, hd, n_head, n, hd, 2, q.ptr, hd, hd * n_head, st))
-                # K: RoPE and the store into the F16 cache in one launch, as the backend runs the two nodes
-                ck(L.chip_rope_apply_store(k.ptr, hd, KV, rope_tab.ptr, hd, n_head_kv, n, hd, 2, k.ptr, hd, KV,
-                                           kc + 2 * KV * (n_kv - n), hd, KV, st))
-                if n > 4:
-                    shp = A4(n, KV, 1, 1)
-                    ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))
-                ck(L.chip_mul_mat_f16_batched(kc, 2 * KV, 2 * hd, hd, n_kv, n_head_kv, q.ptr, hd * n_head, hd, n, n_head, kq.ptr, n_kv,
-                                              n_kv * n, aws.ptr, aws_bytes, st))
-                ck(L.chip_soft_max(kq.ptr, n_kv, mask.ptr, ca.F16, n_kv, n, n_head * n, 0.0884, 0.0, kq.ptr, n_kv, st))
-                ck(L.chip_mul_mat_f16_batched(vc, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv, kq.ptr, n_kv, n_kv * n, n, n_head,
-                                              kqv.ptr, hd, hd * n, aws.ptr, aws_bytes, st))
-                ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
-                              A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
-                mm(*W["wo"], merged, att)
-                # residual + norm + weight: one kernel, as the backend fuses the three nodes
-                ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
-                if n <= 4:                                                # gate and up in one launch, as the backend pairs them
-                    (t_, wg, N_, K_), (_, wu, _, _) = W["gate"], W["up"]
-                    ck(L.chip_mul_mat_pair(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, up.ptr, N_, ws.ptr, wsz, st))
-                else:
-                    mm(*W["up"], cur, up); mm(*W["gate"], cur, gate, True)
-                ck(L.chip_silu_mul(gate.ptr, FF, up.ptr, FF, n, FF, gate.ptr, FF, st))                 # SiLU in its MUL's kernel, as the backend runs the pair
-                mm(*W["down"], gate, att)
-                # the layer's second residual with the next layer's (or the final) norm
-                ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
-            ck(L.chip_mul_mat(ca.Q6_K, arena.ptr + head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
+        def single(nm, x):
+            def f(l):
+                t, p, N, K = self.weights(l)[nm]
+                ck(L.chip_mul_mat(t, p, dev.row_size(t, K), K, N, x, K, n, y, N, ws, wsz, st))
+            return f
 
-        step()
+        def gate_up(l):                  # two matrices of one shape on one activation: one call
+            W = self.weights(l)
+            (t, pg, N, K), (_, pu, _, _) = W["gate"], W["up"]
+            ck(L.chip_mul_mat_pair(t, pg, pu, dev.row_size(t, K), K, N, xh, K, n, y, y + nV, N, ws, wsz, st))
+
+        def head(_l):
+            ck(L.chip_mul_mat(ca.Q6_K, self.arena.ptr + self.head_off, dev.row_size(ca.Q6_K, H), H, V, xh, H, n, y, V, ws, wsz, st))
+
+        return {"qkv": qkv, "wo": single("wo", xh), "gate_up": gate_up, "down": single("down", xff), "head": head}
+
+    def op_bytes(self, n):
+        """Algorithmic bytes of one call of each op class: its weights once, fp32 activations in, fp32 outputs out."""
+        sz = {nm: N * self.dev.row_size(t, K) for (nm, t, N, K) in self.layer}
+        H, FF, KV, V = self.H, self.FF, self.KV, self.V
+        return {"qkv": sz["wq"] + sz["wk"] + sz["wv"] + 4 * n * (H + H + 2 * KV), "wo": sz["wo"] + 4 * n * 2 * H,
+                "gate_up": sz["gate"] + sz["up"] + 4 * n * (H + 2 * FF), "down": sz["down"] + 4 * n * (FF + H),
+                "head": self.head_bytes + 4 * n * (H + V)}
+
+    ORDER = ("qkv", "wo", "gate_up", "down")
+
+    def step(self, n):
+        calls = self.op_calls(n)
+
+        def run():
+            for l in range(self.NL):
+                for nm in self.ORDER:
+                    calls[nm](l)
+            calls["head"](0)
+        return run
+
+    def free(self):
+        for b in self.bufs.values():
+            for k in ("x_h", "x_ff", "y", "ws"):
+                b[k].free()
+        self.arena.free()
+
+
+def percentiles(xs):
+    xs = np.sort(np.asarray(xs, np.float64))
+    return {"median": round(float(np.median(xs)), 2), "p10": round(float(np.percentile(xs, 10)), 2),
+            "p90": round(float(np.percentile(xs, 90)), 2)}
+
+
+def time_steps(dev, hip, st, launch, steps, warmup):
+    """W untimed steps, a synchronization, exactly K steps between one pair of events (the figure reported), and an event
+    after every step for the spread.  Returns (ms per step, per-step microseconds)."""
+    for _ in range(warmup):
+        launch()
+    dev.sync(st)
+    marks = [hip.event() for _ in range(steps + 1)]
+    hip.record(marks[0], st)
+    for i in range(steps):
+        launch()
+        hip.record(marks[i + 1], st)
+    total_ms = hip.elapsed_ms(marks[0], marks[steps])
+    dev.sync(st)
+    per = [hip.elapsed_ms(marks[i], marks[i + 1]) * 1e3 for i in range(steps)]
+    return total_ms / steps, per
+
+
+def traffic_from_profile(key):
+    """HBM bytes per launch of kernel `key` as the committed counter summary states them, or None."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            p = line.split()
+            if len(p) >= 3 and p[0] == "traffic_bytes_per_launch:" and p[1] == key:
+                return int(p[2])
+    except OSError:
+        pass
+    return None
+
+
+def bench_headline(dev, hip, trace, steps, warmup, eager):
+    """One-token decode step over the trace; then each op class alone (32 back-to-back launches on the 32 layers' distinct
+    weights between one event pair) to find the kernel with the largest share and its roofline figure."""
+    st = trace.st
+    run = trace.step(1)
+    run()
+    dev.sync(st)
+    if eager:
+        launch, destroy = run, (lambda: None)
+    else:
+        launch, destroy = hip.capture(st, run)
+    ms_per_step, per = time_steps(dev, hip, st, launch, steps, warmup)
+    destroy()
+    b = trace.step_bytes(1)
+    value = b / (ms_per_step * 1e-3) / 1e9
+
+    calls, ob = trace.op_calls(1), trace.op_bytes(1)
+    per_op = {}
+    for nm in ("qkv", "wo", "gate_up", "down", "head"):
+        reps = 4 if nm == "head" else 3
+
+        def sweep(nm=nm):
+            for l in range(1 if nm == "head" else trace.NL):
+                calls[nm](l)
+        launches = reps * (1 if nm == "head" else trace.NL)
+        if eager:
+            one, kill = sweep, (lambda: None)
+        else:
+            one, kill = hip.capture(st, sweep)
+        one()
         dev.sync(st)
-        graph, gexec = C.c_void_p(), C.c_void_p()
-        assert hl.hipStreamBeginCapture(st, 0) == 0
-        step()
-        assert hl.hipStreamEndCapture(st, C.byref(graph)) == 0
-        assert hl.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
-        us = time_runs(dev, hip, st, lambda: hl.hipGraphLaunch(gexec, st), 10, warm=2)
-        for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws, rope_tab):
-            bf.free()
-        cache_bytes = NL * 2 * n_kv * KV * 2
-        return {"n_kv": n_kv, "nodes": 24 * NL + 2, "us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
-                "weight_and_cache_GBps": round((total + cache_bytes) / us / 1e3, 1)}
+        e0, e1 = hip.event(), hip.event()
+        hip.record(e0, st)
+        for _ in range(reps):
+            one()
+        hip.record(e1, st)
+        us = hip.elapsed_ms(e0, e1) * 1e3 / launches
+        kill()
+        count = 1 if nm == "head" else trace.NL
+        per_op[nm] = {"us_per_launch": round(us, 2), "bytes_per_launch": ob[nm], "GBps": round(ob[nm] / us / 1e3, 1),
+                      "hbm_frac": round(ob[nm] / us / 1e3 / HBM_PEAK_GBS, 4), "launches_per_step": count,
+                      "share_of_step": round(count * us / (ms_per_step * 1e3), 3), "launches_timed": launches}
+    dom = max(per_op, key=lambda k: per_op[k]["share_of_step"])
+    d = per_op[dom]
+    kernel_names = {"qkv": "gemv_group_kernel<K-quants, n=1> (wq Q4_K 4096x4096 + wk Q4_K 1024x4096 + wv Q6_K 1024x4096)",
+                    "wo": "gemv_kernel<Q4_K, n=1, fused quantize> (4096x4096)",
+                    "gate_up": "gemv_kernel<Q4_K, n=1, fused quantize> over ffn_gate + ffn_up (2 x 14336x4096, one launch)",
+                    "down": "gemv_kernel<Q6_K, n=1, fused quantize> (4096x14336)",
+                    "head": "gemv_kernel<Q6_K, n=1, fused quantize> (128256x4096)"}
+    roof = {"bound": "hbm", "achieved": d["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": d["hbm_frac"],
+            "traffic": traffic_from_profile(dom), "kernel": kernel_names[dom], "op": dom,
+            "bytes_per_launch": d["bytes_per_launch"], "us_per_launch": d["us_per_launch"],
+            "launches_timed": d["launches_timed"], "share_of_step": d["share_of_step"]}
+    info = {"step_us": percentiles(per), "tokens_per_s": round(1e3 / ms_per_step, 1), "launches_per_step": 4 * trace.NL + 1,
+            "matmuls_per_step": 7 * trace.NL + 1, "replay": "eager launches" if eager else "HIP graph",
+            "per_op": per_op}
+    return value, ms_per_step, b, roof, info
 
+
+def bench_whole_layers(dev, hip, trace, n, n_kv):
+    """Every node of the 32 layers as llama.cpp builds them without flash attention (norms, projections, RoPE, cache
+    stores, kq, soft-max, kqv, head merge, residuals, SiLU * up), n new tokens against n_kv cached positions, as one
+    HIP graph on one stream: what a decode step costs when no activation leaves the device."""
+    ca, L, st = trace.ca, dev.lib, trace.st
+    H, FF, KV, V, NL = trace.H, trace.FF, trace.KV, trace.V, trace.NL
+    hd, n_head, n_head_kv, kv_size = 128, 32, 8, 4096
+    rng = np.random.default_rng(17)
+    A4 = C.c_int64 * 4
+    f32 = lambda *shape: dev.alloc(int(np.prod(shape)) * 4)
+    b = trace.io(n)
+    ws, wsz, y = b["ws"], b["wsz"], b["y"]
+    resid = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
+    wn = dev.to_device((1 + 0.1 * rng.standard_normal(H)).astype(np.float32))
+    pos = dev.to_device(np.arange(n_kv - n, n_kv, dtype=np.int32))
+    mask = dev.to_device(np.zeros((max(n, 8), n_kv), np.float16))
+    cur, q, k, v, merged, att = f32(n, H), f32(n, H), f32(n, KV), f32(n, KV), f32(n, H), f32(n, H)
+    kq, kqv = f32(n_head, n, n_kv), f32(n_head, n, hd)
+    up, gate = f32(n, FF), f32(n, FF)
+    caches = dev.alloc(NL * 2 * kv_size * KV * 2)
+    dev.check(L.chip_memset(caches.ptr, 0, caches.nbytes, None))
+    aws_bytes = max(L.chip_mul_mat_f16_batched_workspace_size(hd, n_kv, n_head_kv, n_head, n),
+                    L.chip_mul_mat_f16_batched_workspace_size(n_kv, hd, n_head_kv, n_head, n), 256)
+    aws = dev.alloc(aws_bytes)
+    rope_tab = dev.alloc(n * hd * 4)
+    ck = dev.check
+
+    def mm(t, wptr, N, K, src, dst, shared=False):
+        """shared: src was quantized by the previous matmul (same tensor, same activation type), as the backend reuses it"""
+        if n <= 4:                                                    # the GEMV quantizes in its prologue
+            ck(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, dst.ptr, N, ws.ptr, wsz, st))
+            return
+        if not shared:
+            ck(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, ws.ptr, wsz, st))
+        ck(L.chip_mul_mat_run_ws(t, wptr, dev.row_size(t, K), K, N, n, ws.ptr, wsz, dst.ptr, N, st))
+
+    def step():
+        for l in range(NL):
+            W = trace.weights(l)
+            kc = caches.ptr + (2 * l) * kv_size * KV * 2
+            vc = kc + kv_size * KV * 2
+            if l == 0:
+                ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))  # norm + weight: one kernel, as the backend fuses them
+            # q, k, v projections on one activation: one call; V's also stores into the transposed F16 cache
+            arr = (ca.Mat * 3)()
+            for i, (nm, dst) in enumerate((("wq", q), ("wk", k), ("wv", v))):
+                t_, p_, N_, K_ = W[nm]
+                arr[i] = ca.Mat(t_, p_, dev.row_size(t_, K_), N_, dst.ptr, N_, None, 0)
+            if n <= 4:
+                arr[2].y_f16_t = vc + 2 * (n_kv - n)
+                arr[2].ld16 = kv_size
+            ck(L.chip_mul_mat_group(arr, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
+            if l == 0:                                                # one cos / sin table per step, as the backend keeps it
+                ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
+            ck(L.chip_rope_apply(q.ptr, hd, hd * n_head, rope_tab.ptr, hd, n_head, n, hd, 2, q.ptr, hd, hd * n_head, st))
+            # K: RoPE and the store into the F16 cache in one launch, as the backend runs the two nodes
+            ck(L.chip_rope_apply_store(k.ptr, hd, KV, rope_tab.ptr, hd, n_head_kv, n, hd, 2, k.ptr, hd, KV,
+                                       kc + 2 * KV * (n_kv - n), hd, KV, st))
+            if n > 4:
+                shp = A4(n, KV, 1, 1)
+                ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))
+            ck(L.chip_mul_mat_f16_batched(kc, 2 * KV, 2 * hd, hd, n_kv, n_head_kv, q.ptr, hd * n_head, hd, n, n_head, kq.ptr, n_kv,
+                                          n_kv * n, aws.ptr, aws_bytes, st))
+            ck(L.chip_soft_max(kq.ptr, n_kv, mask.ptr, ca.F16, n_kv, n, n_head * n, 0.0884, 0.0, kq.ptr, n_kv, st))
+            ck(L.chip_mul_mat_f16_batched(vc, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv, kq.ptr, n_kv, n_kv * n, n, n_head,
+                                          kqv.ptr, hd, hd * n, aws.ptr, aws_bytes, st))
+            ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
+                          A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
+            mm(*W["wo"], merged, att)
+            # residual + norm + weight: one kernel, as the backend fuses the three nodes
+            ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
+            (t_, wg, N_, K_), (_, wu, _, _) = W["gate"], W["up"]
+            ck(L.chip_mul_mat_pair(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, up.ptr, N_, ws.ptr, wsz, st))
+            ck(L.chip_silu_mul(gate.ptr, FF, up.ptr, FF, n, FF, gate.ptr, FF, st))                 # SiLU in its MUL's kernel, as the backend runs the pair
+            mm(*W["down"], gate, att)
+            # the layer's second residual with the next layer's (or the final) norm
+            ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
+        ck(L.chip_mul_mat(ca.Q6_K, trace.arena.ptr + trace.head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
+
+    step()
+    dev.sync(st)
+    launch, destroy = hip.capture(st, step)
+    ms, per = time_steps(dev, hip, st, launch, 10, 2)
+    destroy()
+    for bf in (resid, wn, pos, mask, cur, q, k, v, merged, att, kq, kqv, up, gate, caches, aws, rope_tab):
+        bf.free()
+    cache_bytes = NL * 2 * n_kv * KV * 2
+    return {"n_kv": n_kv, "us_per_step": round(ms * 1e3, 1), "step_us": percentiles(per), "tokens_per_s": round(n / (ms * 1e-3), 1),
+            "weight_and_cache_GBps": round((trace.total + cache_bytes) / ms / 1e6, 1)}
+
+
+def bench_trace_more(dev, hip, trace, eager):
+    """The same trace at 8 tokens (per step: 225 matmuls; shared quantized activations) and as one 512-token prefill chunk."""
+    st = trace.st
+    out = {}
+    for n in (8, 512):
+        run = trace.step(n)
+        run()
+        dev.sync(st)
+        if eager:
+            launch, destroy = run, (lambda: None)
+        else:
+            launch, destroy = hip.capture(st, run)
+        ms, per = time_steps(dev, hip, st, launch, 10, 2)
+        destroy()
+        b = trace.step_bytes(n)
+        e = {"us_per_step": round(ms * 1e3, 1), "step_us": percentiles(per), "tokens_per_s": round(n / (ms * 1e-3), 1),
+             "GBps": round(b / ms / 1e6, 1), "hbm_frac": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        if n > 8:
+            ops = 2.0 * n * (trace.NL * sum(N * K for (_, _, N, K) in trace.layer) + trace.V * trace.H)
+            e["TOPS"] = round(ops / ms / 1e9, 1)
+            e["int8_frac"] = round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4)
+        if not eager:
+            e["whole_layers"] = bench_whole_layers(dev, hip, trace, n, 512 if n == 512 else 4096)
+        out["config5_trace_n%d" % n] = e
+    if not eager:
+        out["config5_trace_n1_whole_layers"] = bench_whole_layers(dev, hip, trace, 1, 4096)
+    return out
+
+
+def backend_graph_timing():
+    """The same model as a ggml graph through the reference's scheduler and libggml-hip.so (every node on the device):
+    tests/backend_graph_timing.py in a child process - the host framework there is the reference's own ggml build, which
+    only the test tree may load.  Returns its figures, or the reason there are none."""
+    import re
+    import subprocess
+    script = os.path.join(ROOT, "tests", "backend_graph_timing.py")
+    ref_so = os.path.join(ROOT, "oracle", "_ref", "libggml_ref.so")
+    if not os.path.exists(ref_so):
+        return {"skipped": "no host framework on this machine (oracle/_ref/libggml_ref.so)"}
     res = {}
-    for n in (1, 8, 512):                                              # decode, small batch, one prefill chunk
-        x_h = dev.to_device(rng.standard_normal((n, H)).astype(np.float32))
-        x_ff = dev.to_device(rng.standard_normal((n, FF)).astype(np.float32))
-        y = dev.alloc(3 * n * V * 4)                                   # one output region per concurrent branch
-        wsz = max([L.chip_mul_mat_workspace_size_n(t, K, N, n) for (_, t, N, K, _) in layer] + [L.chip_mul_mat_workspace_size_n(ca.Q6_K, H, V, n)])
-        wss = [dev.alloc(wsz) for _ in range(3)]
-        fused = n <= 4            # chip_mul_mat quantizes in the GEMV prologue: one launch per matmul
-
-        def matmul(t, wptr, N, K, src, stream, lane, prepared):
-            yp = y.ptr + lane * n * V * 4
-            if fused:
-                dev.check(L.chip_mul_mat(t, wptr, dev.row_size(t, K), K, N, src.ptr, K, n, yp, N, wss[lane].ptr, wsz, stream))
-            else:
-                if not prepared:
-                    dev.check(L.chip_mul_mat_prepare(t, K, src.ptr, K, n, wss[lane].ptr, wsz, stream))
-                dev.check(L.chip_mul_mat_run_ws(t, wptr, dev.row_size(t, K), K, N, n, wss[lane].ptr, wsz, yp, N, stream))
-
-        def fork(streams):
-            e = hip.event()
-            hip.record(e, st)
-            for s_ in streams:
-                assert hl.hipStreamWaitEvent(s_, e, 0) == 0
-
-        def join(streams):
-            for s_ in streams:
-                e = hip.event()
-                hip.record(e, s_)
-                assert hl.hipStreamWaitEvent(st, e, 0) == 0
-
-        def one_step(parallel):
-            """serial: the 225 matmuls back to back on one stream (what a one-stream ggml backend issues).
-            parallel: matmuls of a layer that share an input and do not depend on each other (wq/wk/wv; up/gate)
-            run as concurrent branches of the graph; wo and down wait for them."""
-            for l in range(NL):
-                base = arena.ptr + l * layer_bytes
-                W = {name: (t, base + o, N, K) for (name, t, N, K, _), o in zip(layer, first)}
-                if parallel:
-                    fork(side)
-                    matmul(*W["wq"], x_h, st, 0, False)
-                    matmul(*W["wk"], x_h, side[0], 1, False)
-                    matmul(*W["wv"], x_h, side[1], 2, False)
-                    join(side)
-                    matmul(*W["wo"], x_h, st, 0, False)
-                    fork(side[:1])
-                    matmul(*W["up"], x_h, st, 0, False)
-                    matmul(*W["gate"], x_h, side[0], 1, False)
-                    join(side[:1])
-                    matmul(*W["down"], x_ff, st, 0, False)
-                else:
-                    matmul(*W["wq"], x_h, st, 0, False)
-                    matmul(*W["wk"], x_h, st, 0, True)          # wq/wk share the quantized input (both Q8_K planes)
-                    matmul(*W["wv"], x_h, st, 0, True)
-                    matmul(*W["wo"], x_h, st, 0, False)
-                    matmul(*W["up"], x_h, st, 0, False)
-                    matmul(*W["gate"], x_h, st, 0, True)
-                    matmul(*W["down"], x_ff, st, 0, False)
-            matmul(ca.Q6_K, arena.ptr + head_off, V, H, x_h, st, 0, False)
-
-        b = total + 4 * n * (NL * sum(K + N for (_, _, N, K, _) in layer) + H + V)
-        entry = {"weight_bytes": total, "matmuls": 7 * NL + 1}
-        for mode in (("serial", "parallel") if n <= 8 else ("serial",)):
-            one_step(mode == "parallel")
-            dev.sync(st)
-            graph, gexec = C.c_void_p(), C.c_void_p()
-            assert hl.hipStreamBeginCapture(st, 0) == 0
-            one_step(mode == "parallel")
-            assert hl.hipStreamEndCapture(st, C.byref(graph)) == 0
-            assert hl.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
-            us = time_runs(dev, hip, st, lambda: hl.hipGraphLaunch(gexec, st), 20, warm=2)
-            entry[mode] = {"us_per_step": round(us, 1), "tokens_per_s": round(n / (us * 1e-6), 1),
-                           "GBps": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
-            if n > 8:                                                   # prefill: the matrix pipe is the yardstick
-                ops = 2.0 * n * (NL * sum(N * K for (_, _, N, K, _) in layer) + V * H)
-                entry[mode]["TOPS"] = round(ops / us / 1e6, 1)
-                entry[mode]["int8_frac"] = round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)
-        entry["whole_layers"] = full_layers(n, 512 if n == 512 else 4096, wss[0], wsz)      # decode and the 8-token batch over 4096 cached positions
-        res["config5_llama3_8b_q4_K_M_trace_n%d" % n] = entry
-        for bf in [x_h, x_ff, y] + wss:
-            bf.free()
-    arena.free()
+    for n in (1, 8):
+        try:
+            txt = subprocess.run([sys.executable, "-u", script], env=dict(os.environ, NTOK=str(n)), capture_output=True, text=True,
+                                 timeout=240).stdout
+        except Exception as exc:                                            # noqa: BLE001
+            res["n%d" % n] = {"error": repr(exc)[:200]}
+            continue
+        m = re.search(r"graph_compute wall us: min (\d+) median (\d+) max (\d+)", txt)
+        i = re.search(r"host time to issue one graph us: median (\d+)", txt)
+        g = re.search(r"nodes (\d+)", txt)
+        if m:
+            res["n%d" % n] = {"graph_compute_us_median": int(m.group(2)), "min": int(m.group(1)), "max": int(m.group(3)),
+                              "host_issue_us": int(i.group(1)) if i else None, "graph_nodes": int(g.group(1)) if g else None,
+                              "tokens_per_s": round(n / (int(m.group(2)) * 1e-6), 1)}
+        else:
+            res["n%d" % n] = {"error": txt[-300:]}
+    res["what"] = ("Llama-3-8B-shaped graph (attention over 4096 cached positions + gated FFN, Q4_K_M type mix) run by the "
+                   "reference scheduler on the HIP backend, eager launches, wall time of graph_compute")
     return res
 
 
-def cpu_baseline(step_bytes_n):
-    """Reference ggml-cpu MUL_MAT (oracle/_ref) or the oracle port on the host cores, bounded sample:
-    the two headline shapes at n = 1 and n = 8."""
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def physical_cores():
+    """Distinct (package, core) pairs of the CPUs this process may run on, capped at the box's CPU share for one GPU."""
+    try:
+        allowed = sorted(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = list(range(os.cpu_count() or 1))
+    seen = set()
+    for c in allowed:
+        try:
+            pkg = open("/sys/devices/system/cpu/cpu%d/topology/physical_package_id" % c).read().strip()
+            core = open("/sys/devices/system/cpu/cpu%d/topology/core_id" % c).read().strip()
+            seen.add((pkg, core))
+        except OSError:
+            seen.add(("?", c))
+    return max(1, min(len(seen), 16))
+
+
+def cpu_baseline():
+    """Reference ggml-cpu MUL_MAT (oracle/_ref) or the oracle port on the host cores, bounded sample of the headline
+    workload: the seven weight matmuls of one layer of the trace at one token, each as its own one-node graph with a
+    persistent threadpool, at T = 1 and at T = the physical cores this process may use."""
     import oracle as O
-    cores = min(16, os.cpu_count() or 1)
     rng = np.random.default_rng(2)
     use_ref = O.Reference.available()
     eng = O.Reference() if use_ref else O.Oracle()
-    t_total, b_total, budget = 0.0, 0, 20.0
-    t_start = time.perf_counter()
-    for (N, K) in ((11008, 4096), (4096, 11008)):
-        w = rng.integers(0, 256, (N, K // 32, 34), dtype=np.uint8)
-        w[..., 0:2] = np.array([0.0107], np.float16).view(np.uint8)
-        w = w.reshape(N, -1)
-        for n in (1, 8):
-            x = rng.standard_normal((n, K)).astype(np.float32)
+    H, FF, KV = 4096, 14336, 1024
+    layer = [(O.Q4_K, H, H), (O.Q4_K, KV, H), (O.Q6_K, KV, H), (O.Q4_K, H, H), (O.Q4_K, FF, H), (O.Q4_K, FF, H), (O.Q6_K, H, FF)]
+    d = np.array([0.0107], np.float16).view(np.uint8)
+    mats = []
+    for (t, N, K) in layer:
+        bb = O.BLOCK_BYTES[t]
+        w = rng.integers(0, 256, (N, K // 256, bb), dtype=np.uint8)
+        if t == O.Q6_K:
+            w[..., 208:210] = d
+        else:
+            w[..., 0:2] = d
+            w[..., 2:4] = d
+        mats.append((t, w.reshape(N, -1), rng.standard_normal((1, K)).astype(np.float32)))
+    nbytes = sum(w.size + 4 * (w.shape[0] + x.shape[1]) for (_, w, x) in mats)
+    T = physical_cores()
+    legs, t_start = {}, time.perf_counter()
+    for threads in (T, 1):
+        total = 0.0
+        for (t, w, x) in mats:
             if use_ref:
-                _, times = eng.mul_mat_graph(O.Q8_0, w, x, nthreads=cores, repeat=12)
-                t = float(np.median(times[2:]))
+                _, times = eng.mul_mat_graph(t, w, x, nthreads=threads, repeat=8 if threads > 1 else 4)
+                total += float(np.median(times[1:]))
             else:
                 t0 = time.perf_counter()
-                eng.mul_mat(O.Q8_0, w, x, nthreads=cores)
-                t = time.perf_counter() - t0
-            t_total += t
-            b_total += w.size + 4 * n * (K + N)
-            if time.perf_counter() - t_start > budget:
-                break
-    return {"value": round(b_total / t_total / 1e9, 2), "unit": "GB/s", "cores": cores,
-            "kind": "reference" if use_ref else "port",
-            "sample": "Q8_0 W[11008x4096] and W[4096x11008] at n=1 and n=8, median of 10 calls each, "
-                      "%s with a persistent %d-thread pool" % ("reference ggml-cpu MUL_MAT graph (AVX2 build)" if use_ref
-                                                               else "oracle restatement", cores)}
+                eng.mul_mat(t, w, x, nthreads=threads)
+                total += time.perf_counter() - t0
+        legs["T%d" % threads] = {"threads": threads, "ms_per_layer": round(total * 1e3, 3), "GBps": round(nbytes / total / 1e9, 2)}
+        if time.perf_counter() - t_start > 60:
+            break
+    main_leg = legs["T%d" % T]
+    return {"value": main_leg["GBps"], "unit": "GB/s", "cores": T, "kind": "reference" if use_ref else "port",
+            "cpu_model": cpu_model(), "legs": legs,
+            "build": "gcc -O2 -mavx2 -mfma -mf16c -ffp-contract=off (AVX2 kernels of ggml-cpu-quants.c; no -march=native)" if use_ref
+                     else "gcc -O2 scalar restatement",
+            "sample": "one layer of the headline trace at one token (wq, wk, wv, wo, ffn_up, ffn_gate, ffn_down: 7 matmuls, "
+                      "%d bytes), %s, persistent threadpool, median of the calls after the first; random block bytes with a "
+                      "constant scale (timing is data independent)" % (nbytes, "reference ggml-cpu MUL_MAT graphs" if use_ref
+                                                                        else "oracle restatement")}
 
 
 def main():
@@ -668,16 +880,30 @@ def main():
     import cactus_amd as ca
     dev = ca.Device(0)
     hip = Hip()
-    value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, args.steps, args.warmup)
-    extra = {} if args.no_extra else bench_extra(dev, hip, trace=not args.no_trace)
-    cpu = None if args.no_cpu else cpu_baseline(step_bytes)
+    trace = Trace(dev, hip, np.random.default_rng(5))
+    value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, trace, args.steps, args.warmup, args.eager)
+    extra = {}
+    if not args.no_extra:
+        extra.update(bench_trace_more(dev, hip, trace, args.eager))
+    trace.free()
+    if not args.no_extra:
+        extra["config2_q8_0_ffn_gemv"] = bench_config2(dev, hip)
+        extra.update(bench_extra(dev, hip))
+        extra["mfma_i8_measured_peak"] = measured_mfma_peak()
+        if not args.no_backend and not args.eager:
+            extra["backend_graph"] = backend_graph_timing()
+    cpu = None if args.no_cpu else cpu_baseline()
     line = {
         "metric": "quant mul_mat GEMV HBM GB/s & prefill int8 TOPS (% of roofline), 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "BASELINE configs[1]: Q8_0 x Q8_0 decode GEMV, W[11008x4096] and W[4096x11008], "
-                               "n in {1,2,4,8}; step = 8 ops (GPU Q8_0 activation quantize + GEMV each); cold weights",
+        "dtype": "int8",
+        "data": "synthetic: random-init weights written directly as GGUF blocks (uniformly random quant and sub-scale bytes, "
+                "one constant fp16 block scale), fp32 activations ~N(0,1); kernel timing does not depend on the values",
+        "config": {"workload": "BASELINE configs[4]: decode-step MUL_MAT trace of a Llama-3-8B-shaped Q4_K_M model (32 layers, "
+                               "hidden 4096, FFN 14336, 32 q / 8 kv heads of 128, Q6_K output head 128256x4096; attn_v and "
+                               "ffn_down Q6_K, the rest Q4_K), every weight matmul of one token step at batch 1, serial on one "
+                               "stream; step = 225 matmuls in 129 calls (wq+wk+wv one call, ffn_gate+ffn_up one call)",
                    "bytes_per_step": step_bytes, "device": dev.info.arch.decode(), **info},
         "roofline": roof, "cpu_baseline": cpu, "extra": extra,
     }

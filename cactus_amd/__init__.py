@@ -35,10 +35,10 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
-    "chip_block_isums",
+    "chip_block_isums", "chip_verify_force_q6k_matrix_core",
     "chip_workspace_to_blocks",
 )
 
@@ -47,6 +47,12 @@ class DeviceInfo(C.Structure):
     _fields_ = [("device", C.c_int), ("compute_units", C.c_int), ("wavefront_size", C.c_int),
                 ("max_lds_per_block", C.c_int), ("clock_khz", C.c_int), ("xcd_count", C.c_int),
                 ("hbm_total", C.c_size_t), ("hbm_free", C.c_size_t), ("name", C.c_char * 128), ("arch", C.c_char * 64)]
+
+
+class Mat(C.Structure):
+    """struct chip_mat: one member of chip_mul_mat_group."""
+    _fields_ = [("type", C.c_int), ("W", C.c_void_p), ("nb01", C.c_size_t), ("N", C.c_int64), ("y", C.c_void_p),
+                ("ldy", C.c_int64), ("y_f16_t", C.c_void_p), ("ld16", C.c_int64)]
 
 
 class ChipError(RuntimeError):
@@ -101,6 +107,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_workspace_size_n.restype = sz
     L.chip_mul_mat_workspace_size_n.argtypes = [i32, i64, i64, i64]
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
+    L.chip_mul_mat_group.argtypes = [C.POINTER(Mat), i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
     L.chip_mul_mat_run_ws.argtypes = [i32, vp, sz, i64, i64, i64, vp, sz, vp, i64, vp]
@@ -131,6 +138,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
     L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
     L.chip_block_isums.argtypes = [i32, vp, sz, i64, i64, vp, i64, vp, vp, vp]
+    L.chip_verify_force_q6k_matrix_core.argtypes = [i32]
     L.chip_workspace_to_blocks.argtypes = [i32, i64, i64, vp, vp, vp]
     return L
 
@@ -257,6 +265,37 @@ class Device:
                                                  ws.ptr, wsz, None))
         self.sync()
         return dy.download(np.float32, n * N).reshape(n, N), dh.download(np.uint16, N * ld16).reshape(N, ld16)
+
+    def mul_mat_group(self, members, x, ld16=0):
+        """chip_mul_mat_group: members = [(wtype, W uint8 [N, row_size]), ...] on the activation rows x fp32 [n, K].
+        Returns a list of y fp32 [n, N]; with ld16 > 0 the last member also stores its transposed fp16 copy and the list
+        ends with that matrix [N, ld16] (untouched columns keep 0x7bff)."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, k = x.shape
+        dx = self.to_device(x)
+        arr = (Mat * len(members))()
+        keep, outs = [], []
+        wsz = 0
+        for i, (wt, W) in enumerate(members):
+            W = np.ascontiguousarray(W, np.uint8)
+            N = W.shape[0]
+            dW, dy = self.to_device(W), self.alloc(n * N * 4)
+            keep.append(dW)
+            outs.append((dy, N))
+            arr[i] = Mat(wt, dW.ptr, self.row_size(wt, k), N, dy.ptr, N, None, 0)
+            wsz = max(wsz, self.lib.chip_mul_mat_workspace_size_n(wt, k, N, n))
+        dh = None
+        if ld16:
+            dh = self.to_device(np.full(outs[-1][1] * ld16, 0x7bff, np.uint16))
+            arr[len(members) - 1].y_f16_t = dh.ptr
+            arr[len(members) - 1].ld16 = ld16
+        ws = self.alloc(wsz)
+        self.check(self.lib.chip_mul_mat_group(arr, len(members), k, dx.ptr, k, n, ws.ptr, wsz, None))
+        self.sync()
+        res = [dy.download(np.float32, n * N).reshape(n, N) for dy, N in outs]
+        if dh is not None:
+            res.append(dh.download(np.uint16, outs[-1][1] * ld16).reshape(outs[-1][1], ld16))
+        return res
 
     def mul_mat_pair(self, wtype, W1, W2, x):
         """Two matrices of one shape on the same activation (chip_mul_mat_pair): returns (y1, y2), each fp32 [n, N]."""

@@ -426,12 +426,12 @@ struct GemmPlan { bool use; size_t act_stride, off_perm, off_offsets, off_tiles,
 GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
     GemmPlan p{};
     const int64_t per_head = r2 * n;
-    static const int64_t min_cols = [] { const char *e = getenv("CHIP_ATTN_GEMM_MIN"); return e ? (int64_t)atoi(e) : GEMM_MIN_COLS; }();
+    const int64_t min_cols = tune("CHIP_ATTN_GEMM_MIN", GEMM_MIN_COLS);
     p.use = K >= 64 && K % 8 == 0 && N >= 32 && per_head >= min_cols && ne02 < (1 << MOE_EXPERT_BITS) && ne02 * per_head < (1LL << 30);
     if (!p.use) return p;
     p.act_stride = f16_stride(K);
-    // 128 x 128 tiles once they still give every CU four workgroups, else 64 x 64 (CHIP_ATTN_TILE forces one, for tuning)
-    static const int forced = [] { const char *e = getenv("CHIP_ATTN_TILE"); return e ? atoi(e) : 0; }();
+    // 128 x 128 tiles once they still give every CU four workgroups, else 64 x 64
+    const int forced = (int)tune("CHIP_ATTN_TILE", 0);
     p.tile = (N >= 128 && per_head >= 128 && ne02 * ceil_div(per_head, (int64_t)128) * ceil_div(N, (int64_t)128) >= 1024) ? 128 : 64;
     if (forced == 64 || forced == 128) p.tile = forced;
     p.n_tiles = ne02 * ceil_div(per_head, (int64_t)p.tile);
@@ -465,7 +465,7 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
                                       void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st) {
     if (N <= 0 || n <= 0 || ne02 <= 0 || r2 <= 0) return hipSuccess;
     if (!mul_mat_f16_batched_supported(K) || ne02 > 65535 || r2 * n > 0x7fffffff) return hipErrorInvalidValue;
-    static const bool mfma_rows = [] { const char *e = getenv("CHIP_ATTN_MFMA"); return !(e && e[0] == '0'); }();
+    const bool mfma_rows = tune("CHIP_ATTN_MFMA", 1) != 0;
     if (const size_t sp = slice_plan_bytes(K, N, ne02, r2, n); mfma_rows && sp > 0 && workspace && workspace_bytes >= sp &&
                                                               (((uintptr_t)workspace) & 15) == 0) {
         const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
@@ -490,7 +490,7 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
         // itself and rounds them while staging (measured: 1.3 % of a 128-token step over 4096 positions; with 2048 columns and two
         // row tiles the doubled staging traffic costs more than the rounding pass, and kq, with thousands of cache positions
         // as rows, reads the activations back once per row tile): the others get an fp16 copy first
-        static const bool f32_direct = [] { const char *e = getenv("CHIP_ATTN_F32_ROWS"); return !(e && e[0] == '0'); }();
+        const bool f32_direct = tune("CHIP_ATTN_F32_ROWS", 1) != 0;
         const int64_t row_tiles = ceil_div(N, (int64_t)plan.tile);
         const bool direct = f32_direct && (row_tiles == 1 || (row_tiles == 2 && r2 * n <= 1024)) && n <= 0x7fffffff &&
                             ne02 * r2 * n <= 0x7fffffff;

@@ -19,6 +19,11 @@ namespace {
 // From this many tokens on the matrix-core GEMV beats the dot-product GEMV (measured on Q8_0 4096x11008).
 constexpr int MMV_MIN_TOKENS = 5;
 
+}  // namespace
+namespace chip { std::atomic<int> g_force_mmv_q6k{0}; }
+
+namespace {
+
 std::mutex g_mu;
 bool g_limits_ready[64] = {};
 DeviceLimits g_limits[64];
@@ -345,7 +350,7 @@ static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t 
     // 5 tokens or more: integer sums on the matrix cores, up to 16 tokens per pass over the weights
     // (4-bit weights on a small matrix: the dot-product GEMV is still ahead up to 6 or 7 tokens)
     // (and Q4_K rows so wide that the kernel runs with six waves: from 7 tokens)
-    static const int mmv_forced = [] { const char *e = getenv("CHIP_MMV_MIN"); return e ? atoi(e) : 0; }();
+    const int mmv_forced = (int)tune("CHIP_MMV_MIN", 0);
     const int mmv_min = mmv_forced > 0 ? mmv_forced
                         : ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7)
                         : (type == T_Q4_K && K > 13312) ? 7 : MMV_MIN_TOKENS;
@@ -373,13 +378,13 @@ static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t 
 
 int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
                  float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
-    static const int mmv_forced = [] { const char *e = getenv("CHIP_MMV_MIN"); return e ? atoi(e) : 0; }();
+    const int mmv_forced = (int)tune("CHIP_MMV_MIN", 0);
     if (n >= 1 && n <= 4 && !(mmv_forced > 0 && n >= mmv_forced) && N > 0 && chip_mul_mat_supported(type, K)) {
         // decode: one launch that quantizes in the GEMV prologue (argument checks as in prepare + run)
         DeviceLimits lim;
         int rc0 = current_limits(lim);
         if (rc0) return rc0;
-        if (gemv_fused_applicable(type, K, (int)n, lim)) {
+            if (gemv_fused_applicable(type, K, (int)n, lim)) {
             if (!x || !workspace || ldx < K || !W || !y || ldy < N) return CHIP_EINVAL;
             if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0) return CHIP_EINVAL;
             if (!weights_aligned(type, W, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
@@ -414,6 +419,55 @@ int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int
     return mul_mat_run(type, W2, nb01, K, N, n, workspace, workspace_bytes, y2, ldy, stream);
 }
 
+// Several matmuls on one activation (wq / wk / wv).  Up to 4 tokens, members of one family: one launch of the
+// prologue-quantizing GEMV over all members; otherwise one quantizer and each member on its usual path.
+int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
+                       size_t workspace_bytes, void *stream) {
+    if (count < 0 || n < 0) return CHIP_EINVAL;
+    if (count == 0 || n == 0) return CHIP_OK;
+    if (!mats || count > CHIP_GROUP_MAX) return CHIP_EINVAL;
+    const int at = chip_vec_dot_type(mats[0].type);
+    size_t need = 0;
+    for (int i = 0; i < count; i++) {
+        const chip_mat &m = mats[i];
+        if (!chip_mul_mat_supported(m.type, K)) return CHIP_EUNSUPPORTED;
+        // one quantized activation serves every member: Q8_1 members read the Q8_0 planes, which carry block_q8_1.s
+        const int a = chip_vec_dot_type(m.type);
+        if (!(a == at || ((a == T_Q8_0 || a == T_Q8_1) && (at == T_Q8_0 || at == T_Q8_1)))) return CHIP_EUNSUPPORTED;
+        if (m.N < 0) return CHIP_EINVAL;
+        if (m.N == 0) continue;
+        if (!m.W || !m.y || m.ldy < m.N || (((uintptr_t)m.y) & 3) != 0) return CHIP_EINVAL;
+        if (!weights_aligned(m.type, m.W, m.nb01, K) || m.nb01 < chip_row_size(m.type, K)) return CHIP_EINVAL;
+        if (m.y_f16_t && (m.ld16 < n || (((uintptr_t)m.y_f16_t) & 1) != 0)) return CHIP_EINVAL;
+        const size_t w = chip_mul_mat_workspace_size(m.type, K, n);
+        if (w > need) need = w;
+    }
+    if (!x || !workspace || ldx < K || !aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace)) return CHIP_EINVAL;
+    if (workspace_bytes < need) return CHIP_ENOMEM;
+    DeviceLimits lim;
+    if (int rc = current_limits(lim); rc) return rc;
+    GroupMat gm[GROUP_MAX];
+    int live = 0;
+    for (int i = 0; i < count; i++)
+        if (mats[i].N > 0)
+            gm[live++] = GroupMat{mats[i].type, mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].y_f16_t, mats[i].ld16};
+    if (live == 0) return CHIP_OK;
+    if (n <= 4 && gemv_group_applicable(gm, live, K, (int)n, lim))
+        return hip_rc(launch_gemv_group(gm, live, K, x, ldx, (int)n, workspace, act_stride(at, K), lim, (hipStream_t)stream));
+    // more tokens, or members the one-launch form does not take: quantize once, then every member as chip_mul_mat_run would
+    if (int rc = chip_mul_mat_prepare(mats[0].type, K, x, ldx, n, workspace, workspace_bytes, stream); rc) return rc;
+    for (int i = 0; i < live; i++) {
+        const GroupMat &m = gm[i];
+        if (int rc = mul_mat_run(m.wtype, m.W, m.nb01, K, m.N, n, workspace, workspace_bytes, m.y, m.ldy, stream); rc) return rc;
+        if (m.t16) {
+            const int64_t ne[4] = {n, m.N, 1, 1};
+            const int64_t nbs[4] = {m.ldy * 4, 4, m.N * 4, m.N * 4}, nbd[4] = {2, m.t16_ld * 2, m.N * m.t16_ld * 2, m.N * m.t16_ld * 2};
+            if (hipError_t e = launch_cpy(m.y, 0, ne, nbs, m.t16, 1, ne, nbd, (hipStream_t)stream); e != hipSuccess) return (int)e;
+        }
+    }
+    return CHIP_OK;
+}
+
 // A matmul whose result is also stored transposed as fp16 (the V projection and the store into the transposed F16 V cache).
 int chip_mul_mat_store_t(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
                          float *y, int64_t ldy, uint16_t *y16t, int64_t ld16, void *workspace, size_t workspace_bytes, void *stream) {
@@ -421,7 +475,7 @@ int chip_mul_mat_store_t(int type, const void *W, size_t nb01, int64_t K, int64_
     if (n >= 1 && n <= 4 && N > 0 && chip_mul_mat_supported(type, K)) {
         DeviceLimits lim;
         if (int rc = current_limits(lim); rc) return rc;
-        if (gemv_fused_applicable(type, K, (int)n, lim)) {
+            if (gemv_fused_applicable(type, K, (int)n, lim)) {
             if (!x || !workspace || ldx < K || !W || !y || ldy < N) return CHIP_EINVAL;
             if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0) return CHIP_EINVAL;
             if (!weights_aligned(type, W, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
@@ -788,6 +842,11 @@ int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     if (!W || !aq || !isum) return CHIP_EINVAL;
     if (!weights_aligned(type, W, nb01, K) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;
     return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, (type == T_Q4_K || type == T_Q5_K) ? imin : nullptr, (hipStream_t)stream));
+}
+
+int chip_verify_force_q6k_matrix_core(int on) {
+    g_force_mmv_q6k.store(on ? 1 : 0, std::memory_order_relaxed);
+    return CHIP_OK;
 }
 
 int chip_workspace_to_blocks(int type, int64_t K, int64_t n, const void *workspace, void *y, void *stream) {

@@ -462,7 +462,7 @@ static int64_t gemm_blk32_min_tokens(int wtype, int64_t K, int64_t N, bool can_s
 bool gemm_blk32_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_split) {
     if (!(wtype == T_Q4_0 || wtype == T_Q8_0 || wtype == T_Q5_0 || wtype == T_IQ4_NL || wtype == T_Q4_1 || wtype == T_Q5_1)) return false;
     if (K % (32 * GEMM_KB) != 0 || N < 1) return false;
-    static const int64_t forced = [] { const char *e = getenv("CHIP_GEMM_MIN_TOKENS"); return e ? (int64_t)atoll(e) : (int64_t)0; }();
+    const int64_t forced = tune("CHIP_GEMM_MIN_TOKENS", 0);
     if (forced > 0) return n >= forced;
     return n >= gemm_blk32_min_tokens(wtype, K, N, can_split);
 }
@@ -518,7 +518,7 @@ hipError_t launch_sum_slices(const float *part, int slices, int64_t n, int64_t N
 // Slices of K for the 64 x 64 shape: about three workgroups per CU up to 128 tokens, two with more (the partial outputs
 // grow with the token count), at least eight stages each.
 static int blk32_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
-    static const int forced = [] { const char *e = getenv("CHIP_GEMM_SLICES"); return e ? atoi(e) : 0; }();
+    const int forced = (int)tune("CHIP_GEMM_SLICES", 0);
     const int64_t units = K / (32 * GEMM_KB), tiles = ceil_div(N, (int64_t)64) * ceil_div(M, (int64_t)64);
     if (forced > 0) {
         const int64_t per = ceil_div(units, (int64_t)(forced < units ? forced : units));
@@ -571,8 +571,7 @@ static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, 
     if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
         return launch_cfg<WT, 1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
-    const char *force = getenv("CHIP_GEMM_CFG");
-    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
+    const int cfg = (int)tune("CHIP_GEMM_CFG", g128 >= cus ? 0 : 1);
     switch (cfg) {
         case 0: return launch_cfg<WT, 1, 2, 4, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
         case 1: return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);

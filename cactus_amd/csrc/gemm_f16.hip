@@ -227,8 +227,7 @@ hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, con
     }
     if (f32_rows) return hipErrorInvalidValue;
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
-    const char *force = getenv("CHIP_GEMM_F16_CFG");
-    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 1);
+    const int cfg = (int)tune("CHIP_GEMM_F16_CFG", g128 >= cus ? 0 : 1);
     switch (cfg) {
         case 0: return launch_f16<2, 2, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 128, 4 waves
         case 1: return launch_f16<1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 64 x 64, 4 waves

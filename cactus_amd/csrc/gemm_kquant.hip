@@ -571,7 +571,7 @@ static int64_t gemm_kq_min_tokens(int wtype, int64_t K, int64_t N, bool can_spli
 }
 bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_split) {
     if (!(wtype == T_Q4_K || wtype == T_Q5_K || wtype == T_Q6_K) || K < QK_K || K % QK_K != 0 || N < 1) return false;
-    static const int64_t forced = [] { const char *e = getenv("CHIP_GEMM_MIN_TOKENS"); return e ? (int64_t)atoll(e) : (int64_t)0; }();
+    const int64_t forced = tune("CHIP_GEMM_MIN_TOKENS", 0);
     if (forced > 0) return n >= forced;
     return n >= gemm_kq_min_tokens(wtype, K, N, can_split);
 }
@@ -579,7 +579,7 @@ bool gemm_kq_supported(int wtype, int64_t K, int64_t N, int64_t n, bool can_spli
 // Slices of K for the 64 x 128 shape: up to two workgroups per CU with one token tile, one per CU with more (the partial
 // outputs grow with the token count), at least four super-blocks each.
 static int kq_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
-    static const int forced = [] { const char *e = getenv("CHIP_GEMM_SLICES"); return e ? atoi(e) : 0; }();
+    const int forced = (int)tune("CHIP_GEMM_SLICES", 0);
     const int64_t units = K / QK_K, tiles = ceil_div(N, (int64_t)64) * ceil_div(M, (int64_t)128);
     if (forced > 0) {
         const int64_t per = ceil_div(units, (int64_t)(forced < units ? forced : units));
@@ -632,13 +632,11 @@ static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t 
         if (slices > 1 && split.bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (((uintptr_t)split.part) & 15) == 0)
             return launch_kq<WT, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, slices, split.part);
     }
-    // 128 rows x 128 tokens per workgroup when that gives every CU one, else 64 x 128.  (CHIP_GEMM_KQ_CFG selects a
-    // shape by hand.)
+    // 128 rows x 128 tokens per workgroup when that gives every CU one, else 64 x 128.
     if (rg.perm)                                                                     // expert groups: 64 x 128 tiles
         return launch_kq<WT, 2, 2, 2, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
-    const char *force = getenv("CHIP_GEMM_KQ_CFG");
-    const int cfg = force ? atoi(force) : (g128 >= cus ? 0 : 2);
+    const int cfg = (int)tune("CHIP_GEMM_KQ_CFG", g128 >= cus ? 0 : 2);
     switch (cfg) {
         case 0: return launch_kq<WT, 4, 2, 3, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 128 x 128, 8 + 4 waves
         case 1: return launch_kq<WT, 4, 1, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 128 x 64, 4 + 4 waves

@@ -18,1002 +18,17 @@
 //     workgroup 0 then also writes the quantized activations to the workspace in the split layout;
 //   * integer dots use v_dot4_i32_i8; each lane keeps fp32 partial sums per (row, token) and the 64 lanes are
 //     combined at the end with a fixed DPP butterfly (no LDS round trip, deterministic order).
-#include "dev_common.h"
-#include "act_layout.h"
-#include "quant_dev.h"
-#include "kernels.h"
+#include "gemv_body.h"
 #include <cstdlib>
 
 namespace chip {
-
-// Weight loads are ordinary cached loads.  A lane's unit is 36..68 bytes, so neighbouring load instructions of
-// a wave touch the same 128-byte lines; with the non-temporal hint (-DCHIP_NT_WLOAD) those lines are not kept
-// between instructions and the kernel runs ~60 % slower (measured: 18 us instead of 11 us on a 48 MB matrix).
-#ifdef CHIP_NT_WLOAD
-#define WLOAD(ptr) __builtin_nontemporal_load(ptr)
-#else
-#define WLOAD(ptr) (*(ptr))
-#endif
-
-// ------------------------------------------------------------------------------------------------ traits
-// For each weight type: how a lane's unit maps to weight bytes and to activation planes.
-//   UNIT_ELEMS : K elements covered by one lane-unit
-//   QCH        : 16-byte activation chunks per unit
-//   AUX        : bytes of per-unit activation side data (scales, sums) kept in LDS
-template <int WT> struct Traits;
-
-template <> struct Traits<T_Q8_0> {
-    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
-    static constexpr bool A_HAS_SUMS = false;                   // A carries the per-block activation sums
-    struct W { uint32_t q[16]; float d0, d1; };
-    struct A { uint32_t q[16]; float d0, d1; };
-    struct Raw { u32x4 a, b, c, e; uint32_t f; };
-
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *p = row + (size_t)u * 68;                       // two 34-byte blocks, 4-byte aligned
-        r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
-        r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
-        r.c = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 32));
-        r.e = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 48));
-        r.f = WLOAD(reinterpret_cast<const uint32_t *>(p + 64));
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
-        const u32x4 a = r.a, b = r.b, c = r.c, e = r.e;
-        const uint32_t f = r.f;
-        // block 0: d at byte 0, quants at bytes 2..33 -> re-slice by 16 bits; block 1: d at 34, quants at 36..67
-        w.d0 = h2f(a.x);
-        w.q[0] = shr16(a.y, a.x); w.q[1] = shr16(a.z, a.y); w.q[2] = shr16(a.w, a.z); w.q[3] = shr16(b.x, a.w);
-        w.q[4] = shr16(b.y, b.x); w.q[5] = shr16(b.z, b.y); w.q[6] = shr16(b.w, b.z); w.q[7] = shr16(c.x, b.w);
-        w.d1 = h2f(c.x >> 16);
-        w.q[8] = c.y; w.q[9] = c.z; w.q[10] = c.w; w.q[11] = e.x;
-        w.q[12] = e.y; w.q[13] = e.z; w.q[14] = e.w; w.q[15] = f;
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-        const float2 d = reinterpret_cast<const float2 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
-        a.d0 = d.x; a.d1 = d.y;
-    }
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
-        i0 = 0; i1 = 0;
-#pragma unroll
-        for (int i = 0; i < 8; i++) { i0 = dot4(w.q[i], a.q[i], i0); i1 = dot4(w.q[8 + i], a.q[8 + i], i1); }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int i0, i1;
-        isums(w, a, i0, i1);
-        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
-        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
-    }
-    // staging: where unit u's chunk j and side data live in the split workspace planes of one token
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = float2;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) {
-        float2 d = make_float2(0.f, 0.f);
-        if (valid) d = reinterpret_cast<const float2 *>(ws + q8_0_off_d(K))[u];
-        return d;
-    }
-    // fused prologue: where the dword of elements e..e+3 and the side data of 32-block blk go in the LDS image
-    __device__ static __forceinline__ size_t img_qs(int, int e) {
-        const int b = e >> 5, u = b >> 1, off = 32 * (b & 1) + (e & 31);
-        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
-    }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int, float) {
-        reinterpret_cast<float *>(img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX)[blk & 1] = d;
-    }
-};
-
-template <> struct Traits<T_Q4_0> {
-    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
-    static constexpr bool A_HAS_SUMS = true;
-    struct W { uint32_t lo[8], hi[8]; float d0, d1; };          // nibbles spread to bytes, 0..15
-    struct A { uint32_t q[16]; float d0, d1; int s0, s1; };
-
-    struct Raw { u32x4 a, b; uint32_t c; };
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *p = row + (size_t)u * 36;                       // two 18-byte blocks, 4-byte aligned
-        r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
-        r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
-        r.c = WLOAD(reinterpret_cast<const uint32_t *>(p + 32));
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
-        const u32x4 a = r.a, b = r.b;
-        const uint32_t c = r.c;
-        uint32_t q[8];
-        w.d0 = h2f(a.x);
-        q[0] = shr16(a.y, a.x); q[1] = shr16(a.z, a.y); q[2] = shr16(a.w, a.z); q[3] = shr16(b.x, a.w);
-        w.d1 = h2f(b.x >> 16);
-        q[4] = b.y; q[5] = b.z; q[6] = b.w; q[7] = c;
-#pragma unroll
-        for (int i = 0; i < 8; i++) { w.lo[i] = q[i] & 0x0f0f0f0fu; w.hi[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-        const u32x4 x = reinterpret_cast<const u32x4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
-        a.d0 = __uint_as_float(x.x); a.d1 = __uint_as_float(x.y); a.s0 = (int)x.z; a.s1 = (int)x.w;
-    }
-    // byte i of qs holds element i (low nibble) and element i+16 (high nibble); value = nibble - 8
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
-        i0 = -8 * a.s0; i1 = -8 * a.s1;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            i0 = dot4(w.lo[i], a.q[i], i0);         i0 = dot4(w.hi[i], a.q[4 + i], i0);
-            i1 = dot4(w.lo[4 + i], a.q[8 + i], i1); i1 = dot4(w.hi[4 + i], a.q[12 + i], i1);
-        }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int i0, i1;
-        isums(w, a, i0, i1);
-        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
-        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = u32x4;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) {
-        u32x4 x = {0u, 0u, 0u, 0u};
-        if (valid) {
-            const u32x2 d = reinterpret_cast<const u32x2 *>(ws + q8_0_off_d(K))[u];
-            const u32x2 s = reinterpret_cast<const u32x2 *>(ws + q8_0_off_sum(K))[u];
-            x.x = d.x; x.y = d.y; x.z = s.x; x.w = s.y;
-        }
-        return x;
-    }
-    __device__ static __forceinline__ size_t img_qs(int, int e) {
-        const int b = e >> 5, u = b >> 1, off = 32 * (b & 1) + (e & 31);
-        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
-    }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float) {
-        uint8_t *a = img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX;
-        reinterpret_cast<float *>(a)[blk & 1] = d;
-        reinterpret_cast<int *>(a)[2 + (blk & 1)] = sum;
-    }
-};
-
-template <> struct Traits<T_Q4_K> {
-    // unit = (super-block sb, 64-value group jp of 4): the 32 qs bytes 32*jp..32*jp+31, whose low nibbles are
-    // elements 64*jp + [0,32) (sub-block 2*jp) and whose high nibbles are elements 64*jp + 32 + [0,32)
-    // (sub-block 2*jp+1).  The matching activations are the 64 contiguous quants 64*jp..64*jp+63.
-    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
-    static constexpr int KQ_STYLE = 0;                          // activation side data: two 32-value sub-block sums
-    struct W { uint32_t lo[8], hi[8]; float d, dmin; int sc0, sc1, m0, m1; };
-    struct A { uint32_t q[16]; float d; int s0, s1; };
-    struct Raw { u32x4 h, q0, q1; };
-
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const int sb = u >> 2, jp = u & 3;
-        const uint8_t *p = row + (size_t)sb * BYTES_Q4_K;              // 144-byte super-block, 16-byte aligned
-        r.h = WLOAD(reinterpret_cast<const u32x4 *>(p));
-        r.q0 = WLOAD(reinterpret_cast<const u32x4 *>(p + 16 + 32 * jp));
-        r.q1 = WLOAD(reinterpret_cast<const u32x4 *>(p + 32 + 32 * jp));
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
-        const int jp = u & 3;
-        const u32x4 h = r.h;
-        w.d = h2f(h.x); w.dmin = h2f(h.x >> 16);
-        // 6-bit scale/min of sub-blocks (2jp, 2jp+1) (reference ggml-quants.c:625-632)
-        const int sh = 16 * (jp & 1);
-        const uint32_t a1 = h.y >> sh, a2 = h.z >> sh, a3 = h.w >> sh;
-        uint32_t sc, mn;
-        if (jp < 2) { sc = a1 & 0x3f3fu; mn = a2 & 0x3f3fu; }
-        else        { sc = (a3 & 0x0f0fu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
-        w.sc0 = sc & 0xff; w.sc1 = sc >> 8; w.m0 = mn & 0xff; w.m1 = mn >> 8;
-        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-#pragma unroll
-        for (int i = 0; i < 8; i++) { w.lo[i] = q[i] & 0x0f0f0f0fu; w.hi[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-        const u32x2 x = reinterpret_cast<const u32x2 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
-        a.d = __uint_as_float(x.x);
-        a.s0 = (int)(int16_t)(x.y & 0xffff); a.s1 = (int)(int16_t)(x.y >> 16);
-    }
-    // this unit's share of the super-block sums: isum = sum_j sc_j * dot_j, imin = sum_j m_j * (sum of sub-block j)
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &im) {
-        int dl = 0, dh = 0;
-#pragma unroll
-        for (int i = 0; i < 8; i++) { dl = dot4(w.lo[i], a.q[i], dl); dh = dot4(w.hi[i], a.q[8 + i], dh); }
-        is = w.sc0 * dl + w.sc1 * dh;
-        im = w.m0 * a.s0 + w.m1 * a.s1;
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int is, im;
-        isums(w, a, is, im);
-        acc = __builtin_fmaf(w.d * a.d, (float)is, acc);
-        return __builtin_fmaf(-(w.dmin * a.d), (float)im, acc);
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = u32x2;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) {
-        u32x2 x = {0u, 0u};
-        if (valid) {
-            const int sb = u >> 2, jp = u & 3;
-            const int16_t *bs = reinterpret_cast<const int16_t *>(ws + q8_K_off_bsums(K)) + sb * 16 + 4 * jp;
-            x.x = reinterpret_cast<const uint32_t *>(ws + q8_K_off_d(K))[sb];
-            x.y = (uint32_t)(uint16_t)(bs[0] + bs[1]) | ((uint32_t)(uint16_t)(bs[2] + bs[3]) << 16);
-        }
-        return x;
-    }
-    // fused prologue (one wave per super-block sb; lane holds elements 4*lane..4*lane+3 of it)
-    static constexpr int UNITS_PER_SB = 4;
-    __device__ static __forceinline__ size_t img_qs(int, int e) {
-        const int u = e >> 6, off = e & 63;
-        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
-    }
-    __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return img + (size_t)NI * QCH * 1024 + (size_t)u * AUX; }
-    // called by all 64 lanes with the sum of their 16-value group: sub-block sums are two groups (8 lanes)
-    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int lane, int s16) {
-        const int s32 = s16 + __builtin_amdgcn_update_dpp(0, s16, 0x141, 0xf, 0xf, true);
-        if ((lane & 7) == 0) {
-            const int g32 = lane >> 3;                                  // sub-block index 0..7
-            reinterpret_cast<int16_t *>(img_aux(img, NI, sb * 4 + (g32 >> 1)) + 4)[g32 & 1] = (int16_t)s32;
-        }
-    }
-};
-
-template <> struct Traits<T_Q6_K> {
-    // unit = (super-block sb, half h, ip): 16 consecutive l = 16*ip + [0,16) of half h, i.e. the four
-    // 16-element groups {128h + 32v + 16ip + [0,16) : v = 0..3}; scale of group v is scales[8h + 2v + ip]
-    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
-    static constexpr int KQ_STYLE = 1;                          // four 16-value group sums
-    struct W { uint32_t q[16]; float d; int sc[4]; };            // q[4v + k]: 6-bit values 0..63 of group v
-    struct A { uint32_t q[16]; float d; int bs[4]; };
-
-    struct Raw { u32x4 l0, l1, qh; u32x2 s; uint32_t d; };
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
-        const uint8_t *p = row + (size_t)sb * BYTES_Q6_K;              // 210-byte super-block, 2-byte aligned
-        r.l0 = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 16 * ip));
-        r.l1 = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 64 * h + 32 + 16 * ip));
-        r.qh = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 128 + 32 * h + 16 * ip));
-        r.s  = WLOAD(reinterpret_cast<const u32x2_a2 *>(p + 192 + 8 * h));
-        r.d  = WLOAD(reinterpret_cast<const unsigned short *>(p + 208));
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
-        const int ip = u & 1;
-        const u32x4 l0 = r.l0, l1 = r.l1, qh = r.qh;
-        const u32x2 s = r.s;
-        w.d = h2f(r.d);
-        const uint32_t ql0[4] = {l0.x, l0.y, l0.z, l0.w}, ql1[4] = {l1.x, l1.y, l1.z, l1.w}, hh[4] = {qh.x, qh.y, qh.z, qh.w};
-#pragma unroll
-        for (int k = 0; k < 4; k++) {                                   // reference ggml-quants.c:1695-1711
-            w.q[k]      = (ql0[k] & 0x0f0f0f0fu)        | ((hh[k] << 4) & 0x30303030u);
-            w.q[4 + k]  = (ql1[k] & 0x0f0f0f0fu)        | ((hh[k] << 2) & 0x30303030u);
-            w.q[8 + k]  = ((ql0[k] >> 4) & 0x0f0f0f0fu) | (hh[k] & 0x30303030u);
-            w.q[12 + k] = ((ql1[k] >> 4) & 0x0f0f0f0fu) | ((hh[k] >> 2) & 0x30303030u);
-        }
-        const int b = 8 * ip;                                           // scales[8h + 2v + ip]: byte ip / ip+2 of each dword
-        w.sc[0] = (int)(int8_t)(s.x >> b); w.sc[1] = (int)(int8_t)(s.x >> (b + 16));
-        w.sc[2] = (int)(int8_t)(s.y >> b); w.sc[3] = (int)(int8_t)(s.y >> (b + 16));
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-        const u32x4 x = reinterpret_cast<const u32x4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
-        a.d = __uint_as_float(x.x);
-        a.bs[0] = (int)(int16_t)(x.y & 0xffff); a.bs[1] = (int)(int16_t)(x.y >> 16);
-        a.bs[2] = (int)(int16_t)(x.z & 0xffff); a.bs[3] = (int)(int16_t)(x.z >> 16);
-    }
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &unused) {
-        is = 0; unused = 0;
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            int dv = -32 * a.bs[v];                                     // sum (q-32)*a = sum q*a - 32*sum a
-#pragma unroll
-            for (int k = 0; k < 4; k++) dv = dot4(w.q[4 * v + k], a.q[4 * v + k], dv);
-            is += w.sc[v] * dv;
-        }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int is, unused;
-        isums(w, a, is, unused);
-        return __builtin_fmaf(w.d * a.d, (float)is, acc);
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) {
-        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
-        return (size_t)sb * 256 + 128 * h + 32 * j + 16 * ip;
-    }
-    using AuxT = u32x4;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) {
-        u32x4 x = {0u, 0u, 0u, 0u};
-        if (valid) {
-            const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
-            const int16_t *bs = reinterpret_cast<const int16_t *>(ws + q8_K_off_bsums(K)) + sb * 16 + 8 * h + ip;
-            x.x = reinterpret_cast<const uint32_t *>(ws + q8_K_off_d(K))[sb];
-            x.y = (uint32_t)(uint16_t)bs[0] | ((uint32_t)(uint16_t)bs[2] << 16);
-            x.z = (uint32_t)(uint16_t)bs[4] | ((uint32_t)(uint16_t)bs[6] << 16);
-        }
-        return x;
-    }
-    static constexpr int UNITS_PER_SB = 4;
-    __device__ static __forceinline__ size_t img_qs(int, int e) {
-        const int sb = e >> 8, o = e & 255;
-        const int h = o >> 7, v = (o >> 5) & 3, ip = (o >> 4) & 1, w = o & 15;
-        const int u = sb * 4 + 2 * h + ip;
-        return ((size_t)((u >> 6) * QCH + v) * 64 + (u & 63)) * 16 + w;
-    }
-    __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return img + (size_t)NI * QCH * 1024 + (size_t)u * AUX; }
-    // called by all 64 lanes with the sum of their 16-value group g = lane/4 = 8*h + 2*v + ip: unit 2*h + ip, slot v
-    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int lane, int s16) {
-        if ((lane & 3) == 0) {
-            const int g = lane >> 2;
-            const int u = sb * 4 + 2 * (g >> 3) + (g & 1);
-            reinterpret_cast<int16_t *>(img_aux(img, NI, u) + 4)[(g >> 1) & 3] = (int16_t)s16;
-        }
-    }
-};
-
-// ---- further weight types (reference type_traits_cpu[], ggml-cpu/ggml-cpu.c:198-367): same activation formats
-template <> struct Traits<T_Q5_0> {
-    // block_q5_0 (ggml-common.h:187-193): fp16 d, 32 high bits qh, 16 nibble bytes; value = d * (q5 - 16),
-    // q5 = nibble | bit << 4, bit j of qh for element j (low nibbles), bit j + 16 for element j + 16 (high nibbles)
-    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
-    static constexpr bool A_HAS_SUMS = true;
-    struct W { uint32_t lo[8], hi[8]; float d0, d1; };          // 5-bit values spread to bytes, 0..31
-    struct A { uint32_t q[16]; float d0, d1; int s0, s1; };
-    struct Raw { u32x4 a, b; u32x2 c; uint32_t e; };
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *p = row + (size_t)u * 44;                       // two 22-byte blocks, 4-byte aligned
-        r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
-        r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
-        r.c = WLOAD(reinterpret_cast<const u32x2_a4 *>(p + 32));
-        r.e = WLOAD(reinterpret_cast<const uint32_t *>(p + 40));
-    }
-    // four high bits -> bit 4 of four bytes
-    __device__ static __forceinline__ uint32_t spread4(uint32_t bits) { return (((bits & 0xFu) * 0x00204081u) & 0x01010101u) << 4; }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
-        const uint32_t d[11] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y, r.e};
-        // block 0: d at bytes 0..1, qh at 2..5, qs at 6..21; block 1: d at 22..23, qh at 24..27, qs at 28..43
-        w.d0 = h2f(d[0]);
-        w.d1 = h2f(d[5] >> 16);
-        const uint32_t qh0 = shr16(d[1], d[0]), qh1 = d[6];
-        const uint32_t q0[4] = {shr16(d[2], d[1]), shr16(d[3], d[2]), shr16(d[4], d[3]), shr16(d[5], d[4])};
-        const uint32_t q1[4] = {d[7], d[8], d[9], d[10]};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            w.lo[i]     = (q0[i] & 0x0f0f0f0fu)        | spread4(qh0 >> (4 * i));
-            w.hi[i]     = ((q0[i] >> 4) & 0x0f0f0f0fu) | spread4(qh0 >> (16 + 4 * i));
-            w.lo[4 + i] = (q1[i] & 0x0f0f0f0fu)        | spread4(qh1 >> (4 * i));
-            w.hi[4 + i] = ((q1[i] >> 4) & 0x0f0f0f0fu) | spread4(qh1 >> (16 + 4 * i));
-        }
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-        const u32x4 x = reinterpret_cast<const u32x4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
-        a.d0 = __uint_as_float(x.x); a.d1 = __uint_as_float(x.y); a.s0 = (int)x.z; a.s1 = (int)x.w;
-    }
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
-        i0 = -16 * a.s0; i1 = -16 * a.s1;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            i0 = dot4(w.lo[i], a.q[i], i0);         i0 = dot4(w.hi[i], a.q[4 + i], i0);
-            i1 = dot4(w.lo[4 + i], a.q[8 + i], i1); i1 = dot4(w.hi[4 + i], a.q[12 + i], i1);
-        }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int i0, i1;
-        isums(w, a, i0, i1);
-        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
-        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = u32x4;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q4_0>::aux_load(ws, K, u, valid); }
-    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_0>::img_qs(NI, e); }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float s) { Traits<T_Q4_0>::img_block_aux(img, NI, blk, d, sum, s); }
-};
-
-template <> struct Traits<T_IQ4_NL> {
-    // block_iq4_nl (ggml-common.h:405-410): fp16 d, 16 nibble bytes; value = d * codebook[nibble]
-    // (ggml-quants.c:2428), low nibbles are elements 0..15, high nibbles 16..31
-    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
-    static constexpr bool A_HAS_SUMS = false;
-    struct W { uint32_t q[16]; float d0, d1; };                 // signed code points, element order
-    using A = Traits<T_Q8_0>::A;
-    using Raw = Traits<T_Q4_0>::Raw;
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) { Traits<T_Q4_0>::load_raw(r, row, u); }
-    // four code indices (one per byte, 0..15) -> four code points, through two byte permutes of the 16-entry table
-    __device__ static __forceinline__ uint32_t lookup4(uint32_t idx) {
-        constexpr uint32_t T0 = 0xbfad9881u, T1 = 0xf6eaddcfu, T2 = 0x26190d01u, T3 = 0x71594535u;
-        const uint32_t sel = idx & 0x07070707u;
-        const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel), hi = __builtin_amdgcn_perm(T3, T2, sel);
-        const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xffu;
-        return (lo & ~m) | (hi & m);
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
-        const u32x4 a = r.a, b = r.b;
-        const uint32_t c = r.c;
-        uint32_t q[8];
-        w.d0 = h2f(a.x);
-        q[0] = shr16(a.y, a.x); q[1] = shr16(a.z, a.y); q[2] = shr16(a.w, a.z); q[3] = shr16(b.x, a.w);
-        w.d1 = h2f(b.x >> 16);
-        q[4] = b.y; q[5] = b.z; q[6] = b.w; q[7] = c;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            w.q[i]      = lookup4(q[i] & 0x0f0f0f0fu);        w.q[4 + i]  = lookup4((q[i] >> 4) & 0x0f0f0f0fu);
-            w.q[8 + i]  = lookup4(q[4 + i] & 0x0f0f0f0fu);    w.q[12 + i] = lookup4((q[4 + i] >> 4) & 0x0f0f0f0fu);
-        }
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) { Traits<T_Q8_0>::load_a(a, tok, NI, it, lane); }
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
-        i0 = 0; i1 = 0;
-#pragma unroll
-        for (int i = 0; i < 8; i++) { i0 = dot4(w.q[i], a.q[i], i0); i1 = dot4(w.q[8 + i], a.q[8 + i], i1); }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int i0, i1;
-        isums(w, a, i0, i1);
-        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
-        return __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = float2;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q8_0>::aux_load(ws, K, u, valid); }
-    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q8_0>::img_qs(NI, e); }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int sum, float s) { Traits<T_Q8_0>::img_block_aux(img, NI, blk, d, sum, s); }
-};
-
-// F16 weights (type_traits_cpu[LM_GGML_TYPE_F16], ggml-cpu/ggml-cpu.c:204-209): the activations are rounded to fp16
-// (lm_ggml_cpu_fp32_to_fp16) and lm_ggml_vec_dot_f16 (ggml-cpu/vec.cpp:122-162) accumulates the products of the
-// widened halves in fp32.  A unit is 32 elements = 64 weight bytes and 64 activation bytes; no side data.
-template <> struct Traits<T_F16> {
-    static constexpr int ACT = T_F16, UNIT_ELEMS = 32, QCH = 4, AUX = 0;
-    struct Raw { u32x4 q[4]; };
-    using W = Raw;
-    struct A { uint32_t q[16]; };
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const u32x4 *p = reinterpret_cast<const u32x4 *>(row + (size_t)u * 64);  // rows are multiples of 512 bytes
-#pragma unroll
-        for (int j = 0; j < 4; j++) r.q[j] = WLOAD(p + j);
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) { w = r; }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t wq[4] = {w.q[j].x, w.q[j].y, w.q[j].z, w.q[j].w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const half2_t wv = __builtin_bit_cast(half2_t, wq[i]), av = __builtin_bit_cast(half2_t, a.q[4 * j + i]);
-                acc = __builtin_fmaf((float)wv.x, (float)av.x, acc);      // v_fma_mix_f32: fp16 operands, fp32 accumulate
-                acc = __builtin_fmaf((float)wv.y, (float)av.y, acc);
-            }
-        }
-        return acc;
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = uint32_t;                                       // unused (AUX == 0)
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *, int64_t, int, bool) { return 0u; }
-    // fused prologue: byte position of element e (an fp16) in the LDS image
-    __device__ static __forceinline__ size_t img_h(int, int e) {
-        const int u = e >> 5, off = (e & 31) * 2;
-        return ((size_t)((u >> 6) * QCH + (off >> 4)) * 64 + (u & 63)) * 16 + (off & 15);
-    }
-};
-
-// Q4_1 / Q5_1 (ggml-common.h:175-185,196-207): value = d * u + m with an unsigned 4- or 5-bit u.  Their activation
-// format Q8_1 is Q8_0 plus s = fp16(d * sum q) per block (kept in the Q8_0 workspace planes), so
-// y += (dw * dx) * sum(u * q) + m * s (reference lm_ggml_vec_dot_q4_1_q8_1 / _q5_1_q8_1, AVX2 branches).
-template <int WT> struct TraitsMin32 {
-    static constexpr bool FIVE = (WT == T_Q5_1);
-    static constexpr int ACT = T_Q8_0, UNIT_ELEMS = 64, QCH = 4, AUX = 16;
-    static constexpr bool A_HAS_SUMS = false;
-    static constexpr int ABLK_BYTES = BYTES_Q8_1, ABLK_QOFF = 4;          // reference activation records (block_isums)
-    struct W { uint32_t lo[8], hi[8]; float d0, d1, m0, m1; };
-    struct A { uint32_t q[16]; float d0, d1, s0, s1; };
-    struct Raw { u32x4 a, b; u32x2 c; uint32_t e[2]; };
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        if constexpr (!FIVE) {
-            const uint8_t *p = row + (size_t)u * 40;                   // two 20-byte blocks, 4-byte aligned
-            r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
-            r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
-            r.c = WLOAD(reinterpret_cast<const u32x2_a4 *>(p + 32));
-        } else {
-            const uint8_t *p = row + (size_t)u * 48;                   // two 24-byte blocks, 4-byte aligned
-            r.a = WLOAD(reinterpret_cast<const u32x4_a4 *>(p));
-            r.b = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16));
-            r.c = WLOAD(reinterpret_cast<const u32x2_a4 *>(p + 32));
-            r.e[0] = WLOAD(reinterpret_cast<const uint32_t *>(p + 40));
-            r.e[1] = WLOAD(reinterpret_cast<const uint32_t *>(p + 44));
-        }
-    }
-    __device__ static __forceinline__ uint32_t spread4(uint32_t bits) { return (((bits & 0xFu) * 0x00204081u) & 0x01010101u) << 4; }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int) {
-        if constexpr (!FIVE) {
-            // block: d, m (one dword), 16 qs bytes
-            const uint32_t d[10] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y};
-            w.d0 = h2f(d[0]); w.m0 = h2f(d[0] >> 16);
-            w.d1 = h2f(d[5]); w.m1 = h2f(d[5] >> 16);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                w.lo[i]     = d[1 + i] & 0x0f0f0f0fu; w.hi[i]     = (d[1 + i] >> 4) & 0x0f0f0f0fu;
-                w.lo[4 + i] = d[6 + i] & 0x0f0f0f0fu; w.hi[4 + i] = (d[6 + i] >> 4) & 0x0f0f0f0fu;
-            }
-        } else {
-            // block: d, m (one dword), qh (one dword), 16 qs bytes
-            const uint32_t d[12] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y, r.e[0], r.e[1]};
-            w.d0 = h2f(d[0]); w.m0 = h2f(d[0] >> 16);
-            w.d1 = h2f(d[6]); w.m1 = h2f(d[6] >> 16);
-            const uint32_t qh0 = d[1], qh1 = d[7];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                w.lo[i]     = (d[2 + i] & 0x0f0f0f0fu)        | spread4(qh0 >> (4 * i));
-                w.hi[i]     = ((d[2 + i] >> 4) & 0x0f0f0f0fu) | spread4(qh0 >> (16 + 4 * i));
-                w.lo[4 + i] = (d[8 + i] & 0x0f0f0f0fu)        | spread4(qh1 >> (4 * i));
-                w.hi[4 + i] = ((d[8 + i] >> 4) & 0x0f0f0f0fu) | spread4(qh1 >> (16 + 4 * i));
-            }
-        }
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(tok) + (size_t)it * QCH * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < QCH; j++) {
-            const u32x4 v = q[j * 64];
-            a.q[4 * j] = v.x; a.q[4 * j + 1] = v.y; a.q[4 * j + 2] = v.z; a.q[4 * j + 3] = v.w;
-        }
-        const float4 x = reinterpret_cast<const float4 *>(tok + (size_t)NI * QCH * 1024)[it * 64 + lane];
-        a.d0 = x.x; a.d1 = x.y; a.s0 = x.z; a.s1 = x.w;
-    }
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &i0, int &i1) {
-        i0 = 0; i1 = 0;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            i0 = dot4(w.lo[i], a.q[i], i0);         i0 = dot4(w.hi[i], a.q[4 + i], i0);
-            i1 = dot4(w.lo[4 + i], a.q[8 + i], i1); i1 = dot4(w.hi[4 + i], a.q[12 + i], i1);
-        }
-    }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
-        int i0, i1;
-        isums(w, a, i0, i1);
-        acc = __builtin_fmaf(w.d0 * a.d0, (float)i0, acc);
-        acc = __builtin_fmaf(w.m0, a.s0, acc);
-        acc = __builtin_fmaf(w.d1 * a.d1, (float)i1, acc);
-        return __builtin_fmaf(w.m1, a.s1, acc);
-    }
-    __device__ static __forceinline__ size_t src_chunk(int64_t, int u, int j) { return (size_t)u * 64 + 16 * j; }
-    using AuxT = float4;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) {
-        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (valid) {
-            const float2 d = reinterpret_cast<const float2 *>(ws + q8_0_off_d(K))[u];
-            const float2 s = reinterpret_cast<const float2 *>(ws + q8_0_off_s(K))[u];
-            x = make_float4(d.x, d.y, s.x, s.y);
-        }
-        return x;
-    }
-    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_0>::img_qs(NI, e); }
-    __device__ static __forceinline__ void img_block_aux(uint8_t *img, int NI, int blk, float d, int, float s) {
-        float *a = reinterpret_cast<float *>(img + (size_t)NI * QCH * 1024 + (size_t)(blk >> 1) * AUX);
-        a[blk & 1] = d;
-        a[2 + (blk & 1)] = s;
-    }
-};
-template <> struct Traits<T_Q4_1> : TraitsMin32<T_Q4_1> {};
-template <> struct Traits<T_Q5_1> : TraitsMin32<T_Q5_1> {};
-
-template <> struct Traits<T_Q5_K> {
-    // block_q5_K (ggml-common.h:303-314): as q4_K plus qh[32]: bit 2jp of qh[l] is the fifth bit of element l of
-    // sub-block 2jp (low nibbles of the group's 32 qs bytes), bit 2jp+1 that of sub-block 2jp+1 (high nibbles)
-    static constexpr int ACT = T_Q8_K, UNIT_ELEMS = 64, QCH = 4, AUX = 8;
-    static constexpr int KQ_STYLE = 0;
-    using W = Traits<T_Q4_K>::W;
-    using A = Traits<T_Q4_K>::A;
-    struct Raw { u32x4 h, qh0, qh1, q0, q1; };
-    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const int sb = u >> 2, jp = u & 3;
-        const uint8_t *p = row + (size_t)sb * BYTES_Q5_K;              // 176-byte super-block, 16-byte aligned
-        r.h = WLOAD(reinterpret_cast<const u32x4 *>(p));
-        r.qh0 = WLOAD(reinterpret_cast<const u32x4 *>(p + 16));
-        r.qh1 = WLOAD(reinterpret_cast<const u32x4 *>(p + 32));
-        r.q0 = WLOAD(reinterpret_cast<const u32x4 *>(p + 48 + 32 * jp));
-        r.q1 = WLOAD(reinterpret_cast<const u32x4 *>(p + 64 + 32 * jp));
-    }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
-        const int jp = u & 3;
-        const u32x4 h = r.h;
-        w.d = h2f(h.x); w.dmin = h2f(h.x >> 16);
-        const int sh = 16 * (jp & 1);
-        const uint32_t a1 = h.y >> sh, a2 = h.z >> sh, a3 = h.w >> sh;
-        uint32_t sc, mn;
-        if (jp < 2) { sc = a1 & 0x3f3fu; mn = a2 & 0x3f3fu; }
-        else        { sc = (a3 & 0x0f0fu) | ((a1 >> 2) & 0x3030u); mn = ((a3 >> 4) & 0x0f0fu) | ((a2 >> 2) & 0x3030u); }
-        w.sc0 = sc & 0xff; w.sc1 = sc >> 8; w.m0 = mn & 0xff; w.m1 = mn >> 8;
-        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-        const uint32_t hb[8] = {r.qh0.x, r.qh0.y, r.qh0.z, r.qh0.w, r.qh1.x, r.qh1.y, r.qh1.z, r.qh1.w};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            w.lo[i] = (q[i] & 0x0f0f0f0fu)        | (((hb[i] >> (2 * jp)) & 0x01010101u) << 4);
-            w.hi[i] = ((q[i] >> 4) & 0x0f0f0f0fu) | (((hb[i] >> (2 * jp + 1)) & 0x01010101u) << 4);
-        }
-    }
-    __device__ static __forceinline__ void load_a(A &a, const uint8_t *tok, int NI, int it, int lane) { Traits<T_Q4_K>::load_a(a, tok, NI, it, lane); }
-    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &im) { Traits<T_Q4_K>::isums(w, a, is, im); }
-    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) { return Traits<T_Q4_K>::dot(w, a, acc); }
-    __device__ static __forceinline__ size_t src_chunk(int64_t K, int u, int j) { return Traits<T_Q4_K>::src_chunk(K, u, j); }
-    using AuxT = u32x2;
-    __device__ static __forceinline__ AuxT aux_load(const uint8_t *ws, int64_t K, int u, bool valid) { return Traits<T_Q4_K>::aux_load(ws, K, u, valid); }
-    static constexpr int UNITS_PER_SB = 4;
-    __device__ static __forceinline__ size_t img_qs(int NI, int e) { return Traits<T_Q4_K>::img_qs(NI, e); }
-    __device__ static __forceinline__ uint8_t *img_aux(uint8_t *img, int NI, int u) { return Traits<T_Q4_K>::img_aux(img, NI, u); }
-    __device__ static __forceinline__ void img_bsum(uint8_t *img, int NI, int sb, int lane, int s16) { Traits<T_Q4_K>::img_bsum(img, NI, sb, lane, s16); }
-};
-
-template <int WT> __host__ __device__ constexpr int units_per_row(int64_t K) { return (int)(K / Traits<WT>::UNIT_ELEMS); }
-template <int WT> __host__ __device__ constexpr int iters_per_row(int64_t K) { return (int)ceil_div(K / Traits<WT>::UNIT_ELEMS, 64); }
-template <int WT> __host__ __device__ constexpr size_t lds_image_bytes(int64_t K) {
-    return (size_t)iters_per_row<WT>(K) * (Traits<WT>::QCH * 1024 + 64 * Traits<WT>::AUX);
-}
-
-// ------------------------------------------------------------------------------------------------ kernel
-// Fused prologue: quantize NTOK fp32 rows straight into the LDS image; workgroup 0 also writes the split
-// workspace planes so the quantized activations exist in memory as the reference's wdata does.
-// The fp32 loads are split from their use (xload_* issues them, quantize_* consumes them) so that the caller
-// can put the weight prefetch between the two: all of a thread's loads are then in flight together and the
-// quantization waits only for the activations, which were issued first.
-constexpr int FUSE_MAX_VALUES = 16384;                     // n * K limit of the fused prologue
-
-// Register slots: token t owns slots [t*PER, (t+1)*PER); slot j of a token covers float4 chunk j*WGS + tid (Q8_0:
-// 8 lanes per 32-block) or super-block j*(WGS/64) + wave (Q8_K: one wave per 256 values).  n * K <= FUSE_MAX_VALUES
-// guarantees PER slots suffice; the loops stop at the first slot index that is out of range for the whole group.
-#ifndef FUSE_ILP
-#define FUSE_ILP 2
-#endif
-template <int NTOK, int WGS> struct XRegs {
-    static constexpr int PER = FUSE_MAX_VALUES / 4 / WGS / NTOK;
-    float4 v[NTOK][PER];
-};
-
-template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void xload(XRegs<NTOK, WGS> &xr, const float *__restrict__ x, int64_t ldx, int64_t K) {
-    using T = Traits<WT>;
-    constexpr int PER = XRegs<NTOK, WGS>::PER;
-    if constexpr (T::ACT == T_Q8_0 || T::ACT == T_F16) {
-        const int nchunk = (int)(K / 4);                                // float4 chunks per token
-#pragma unroll
-        for (int t = 0; t < NTOK; t++)
-#pragma unroll
-            for (int j = 0; j < PER; j++) {
-                const int c = j * WGS + (int)threadIdx.x;
-                xr.v[t][j] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (c < nchunk) xr.v[t][j] = *reinterpret_cast<const float4 *>(x + t * ldx + 4 * (int64_t)c);
-            }
-    } else {
-        const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-        const int nsb = (int)(K / 256);
-#pragma unroll
-        for (int t = 0; t < NTOK; t++)
-#pragma unroll
-            for (int j = 0; j < PER; j++) {
-                const int sb = j * (WGS / 64) + wv;
-                xr.v[t][j] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (sb < nsb) xr.v[t][j] = *reinterpret_cast<const float4 *>(x + t * ldx + (int64_t)sb * 256 + 4 * lane);
-            }
-    }
-}
-
-template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, uint8_t *lds, size_t img, int NI, int64_t K,
-                                                    uint8_t *__restrict__ ws, size_t ws_stride) {
-    using T = Traits<WT>;
-    constexpr int PER = XRegs<NTOK, WGS>::PER;
-    const bool dump = blockIdx.x == 0 && ws != nullptr;
-    if constexpr (T::ACT == T_F16) {
-        // plain conversion: four floats -> four halves (round to nearest even), 8 bytes into the image
-        const int nchunk = (int)(K / 4);
-#pragma unroll
-        for (int t = 0; t < NTOK; t++) {
-            uint8_t *im = lds + t * img;
-#pragma unroll
-            for (int j = 0; j < PER; j++) {
-                const int c = j * WGS + (int)threadIdx.x;
-                if (c < nchunk) {
-                    const float4 v = xr.v[t][j];
-                    u32x2 h;
-                    h.x = (uint32_t)f2h_rne(v.x) | ((uint32_t)f2h_rne(v.y) << 16);
-                    h.y = (uint32_t)f2h_rne(v.z) | ((uint32_t)f2h_rne(v.w) << 16);
-                    *reinterpret_cast<u32x2 *>(im + T::img_h(NI, 4 * c)) = h;
-                    if (dump) *reinterpret_cast<u32x2 *>(ws + t * ws_stride + 8 * (size_t)c) = h;
-                }
-            }
-        }
-    } else if constexpr (T::ACT == T_Q8_0) {
-        // 8 lanes per 32-block; K % 256 == 0 keeps every 64-lane group either fully inside or fully outside.
-        // Slots are quantized FUSE_ILP at a time so their dependent chains (DPP max, two divisions, DPP sum) overlap.
-        const int nchunk = (int)(K / 4);
-#pragma unroll
-        for (int t = 0; t < NTOK; t++) {
-            uint8_t *im = lds + t * img;
-#pragma unroll
-            for (int j0 = 0; j0 < PER; j0 += FUSE_ILP) {
-                if (j0 * WGS >= nchunk) break;                          // uniform over the group
-                Q8_0Lane q[FUSE_ILP];
-#pragma unroll
-                for (int u = 0; u < FUSE_ILP; u++)
-                    if (j0 + u < PER) q[u] = quantize_q8_0_lane(xr.v[t][j0 + u]);
-#pragma unroll
-                for (int u = 0; u < FUSE_ILP; u++) {
-                    if (j0 + u >= PER) continue;
-                    const int c = (j0 + u) * WGS + (int)threadIdx.x;
-                    if (c < nchunk) {
-                        const int e = 4 * c, blk = e >> 5;
-                        *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, e)) = q[u].packed;
-                        const float d = h2f(q[u].dh);
-                        if ((threadIdx.x & 7) == 0) T::img_block_aux(im, NI, blk, d, q[u].sum, h2f(q[u].sh));
-                        if (dump) {
-                            uint8_t *base = ws + t * ws_stride;
-                            *reinterpret_cast<uint32_t *>(base + e) = q[u].packed;
-                            if ((threadIdx.x & 7) == 0) {
-                                reinterpret_cast<float *>(base + q8_0_off_d(K))[blk] = d;
-                                reinterpret_cast<int32_t *>(base + q8_0_off_sum(K))[blk] = q[u].sum;
-                                reinterpret_cast<float *>(base + q8_0_off_s(K))[blk] = h2f(q[u].sh);
-                            }
-                        }
-                    }
-                }
-            }
-        }
-    } else {
-        // one wave per 256-value super-block, FUSE_ILP super-blocks in flight per wave
-        const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-        const int nsb = (int)(K / 256);
-#pragma unroll
-        for (int t = 0; t < NTOK; t++) {
-            uint8_t *im = lds + t * img;
-#pragma unroll
-            for (int j0 = 0; j0 < PER; j0 += FUSE_ILP) {
-                if (j0 * (WGS / 64) >= nsb) break;                      // uniform over the group
-                Q8_KLane q[FUSE_ILP];
-#pragma unroll
-                for (int u = 0; u < FUSE_ILP; u++)
-                    if (j0 + u < PER) q[u] = quantize_q8_K_lane(xr.v[t][j0 + u]);
-#pragma unroll
-                for (int u = 0; u < FUSE_ILP; u++) {
-                    if (j0 + u >= PER) continue;
-                    const int sb = (j0 + u) * (WGS / 64) + wv;
-                    if (sb < nsb) {                                     // uniform over the wave
-                        *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, sb * 256 + 4 * lane)) = q[u].packed;
-                        if (lane < T::UNITS_PER_SB) *reinterpret_cast<float *>(T::img_aux(im, NI, sb * T::UNITS_PER_SB + lane)) = q[u].d;
-                        T::img_bsum(im, NI, sb, lane, q[u].bsum);
-                        if (dump) {
-                            uint8_t *base = ws + t * ws_stride;
-                            *reinterpret_cast<uint32_t *>(base + (size_t)sb * 256 + 4 * lane) = q[u].packed;
-                            if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(K))[sb] = q[u].d;
-                            if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(K))[sb * 16 + (lane >> 2)] = (int16_t)q[u].bsum;
-                        }
-                    }
-                }
-            }
-        }
-    }
-}
-
-// Staging from an already quantized workspace: transpose the split planes to [it][chunk][lane].  The loads
-// are split from their LDS stores (stage_issue / stage_commit) so that the caller can request the first weight
-// tiles in between: loads return in issue order, so the staging data must be asked for first or it would wait
-// for the much slower weight stream.  Registers cover PQ chunks and one side-data record per token and thread;
-// longer rows finish in a plain loop inside stage_commit.
-template <int WT, int NTOK> struct StageRegs {
-    static constexpr int PQ = NTOK <= 4 ? 2 : 1;
-    u32x4 v[NTOK][PQ];
-    typename Traits<WT>::AuxT a[NTOK];
-};
-
-template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void stage_issue(StageRegs<WT, NTOK> &sr, int NI, int units, int64_t K,
-                                            const uint8_t *__restrict__ ws, size_t ws_stride) {
-    using T = Traits<WT>;
-    constexpr int PQ = StageRegs<WT, NTOK>::PQ;
-    const int nq = NI * T::QCH * 64;                                    // 16-byte chunks per token
-#pragma unroll
-    for (int j = 0; j < PQ; j++) {
-        const int r = j * WGS + (int)threadIdx.x;
-        const int lane = r & 63, c = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
-        const int u = it * 64 + lane;
-        const bool ok = r < nq && u < units;
-        const size_t off = T::src_chunk(K, u, c);
-#pragma unroll
-        for (int t = 0; t < NTOK; t++) {
-            sr.v[t][j] = u32x4{0u, 0u, 0u, 0u};
-            if (ok) sr.v[t][j] = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + off);
-        }
-    }
-    const int u = (int)threadIdx.x;
-#pragma unroll
-    for (int t = 0; t < NTOK; t++) sr.a[t] = T::aux_load(ws + t * ws_stride, K, u, u < units);   // no-op when AUX == 0
-}
-
-template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint8_t *lds, size_t img, int NI, int units,
-                                             int64_t K, const uint8_t *__restrict__ ws, size_t ws_stride) {
-    using T = Traits<WT>;
-    using AuxT = typename T::AuxT;
-    constexpr int PQ = StageRegs<WT, NTOK>::PQ;
-    const int nq = NI * T::QCH * 64, na = NI * 64;
-    const size_t aux0 = (size_t)NI * T::QCH * 1024;
-#pragma unroll
-    for (int j = 0; j < PQ; j++) {
-        const int r = j * WGS + (int)threadIdx.x;
-        if (r < nq) {
-#pragma unroll
-            for (int t = 0; t < NTOK; t++) reinterpret_cast<u32x4 *>(lds + t * img)[r] = sr.v[t][j];
-        }
-    }
-    if constexpr (T::AUX > 0) {
-        if ((int)threadIdx.x < na) {
-#pragma unroll
-            for (int t = 0; t < NTOK; t++) *reinterpret_cast<AuxT *>(lds + t * img + aux0 + (size_t)threadIdx.x * T::AUX) = sr.a[t];
-        }
-    }
-    // rows longer than the register slots
-    for (int r = PQ * WGS + (int)threadIdx.x; r < nq; r += WGS) {
-        const int lane = r & 63, c = (r >> 6) % T::QCH, it = (r >> 6) / T::QCH;
-        const int u = it * 64 + lane;
-        const size_t off = T::src_chunk(K, u, c);
-#pragma unroll
-        for (int t = 0; t < NTOK; t++) {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (u < units) v = *reinterpret_cast<const u32x4 *>(ws + t * ws_stride + off);
-            reinterpret_cast<u32x4 *>(lds + t * img)[r] = v;
-        }
-    }
-    if constexpr (T::AUX > 0) {
-        for (int u = WGS + (int)threadIdx.x; u < na; u += WGS) {
-#pragma unroll
-            for (int t = 0; t < NTOK; t++)
-                *reinterpret_cast<AuxT *>(lds + t * img + aux0 + (size_t)u * T::AUX) = T::aux_load(ws + t * ws_stride, K, u, u < units);
-        }
-    }
-}
-
-
-// Two matrices of one shape and type that read the same activation (ffn_gate and ffn_up) as one launch: rows
-// [0, n_first) are the first matrix, rows [n_first, N) the second one, whose weights and outputs lie w_off bytes / y_off
-// floats away from where the first matrix's row and output of that index would be.  One matrix: n_first = N.
-// t16 (one matrix only): the outputs also go, rounded to fp16, to t16[row * t16_ld + token] - the transposed store of V
-// into the F16 cache that follows the V projection (reference llama-kv-cache.cpp cpy_v without flash attention).
-struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; };
-constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0};
-
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
-__device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
-                                          const float *__restrict__ x, int64_t ldx,
-                                          uint8_t *__restrict__ ws, size_t ws_stride,
-                                          float *__restrict__ y, int64_t ldy, const SecondMatrix sec) {
-    using T = Traits<WT>;
-    extern __shared__ __align__(16) uint8_t lds[];
-    const int NI = iters_per_row<WT>(K);
-    const int units = units_per_row<WT>(K);
-    const size_t img = lds_image_bytes<WT>(K);
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * (WGS / 64) + (threadIdx.x >> 6);
-    const int64_t nwaves = (int64_t)gridDim.x * (WGS / 64);
-    const int64_t tiles = ceil_div(N, R);
-
-    // A wave walks the steps (tile, it) = (wave, 0), (wave, 1), ..., (wave + nwaves, 0), ...  Two cursors run
-    // over that sequence: the load cursor stays DEPTH steps ahead of the compute cursor, and the raw weight
-    // registers form a ring of DEPTH steps.  All cursor state is wave-uniform.
-    struct Cursor { int64_t tile; int it; bool have; };
-    auto advance = [&](Cursor &c) {
-        if (c.it + 1 == NI) { c.tile += nwaves; c.it = 0; } else c.it++;
-        c.have = c.tile < tiles;
-    };
-    typename T::Raw ring[DEPTH][R];
-    Cursor lc{wave, 0, wave < tiles};
-    auto issue = [&](typename T::Raw (&slot)[R]) {
-        if (lc.have) {
-            const int u = lc.it * 64 + lane;
-            if (u < units) {
-#pragma unroll
-                for (int r = 0; r < R; r++) {                            // tail tile: re-read the last row, never store it
-                    const int64_t row = min(lc.tile * R + r, N - 1);
-                    T::load_raw(slot[r], W + (size_t)row * nb01 + (row >= sec.n_first ? sec.w_off : (int64_t)0), u);
-                }
-            }
-            advance(lc);
-        }
-    };
-
-    // ---- prologue: activation loads first, then DEPTH steps of weight loads, then the activation image is
-    //      built in LDS while the weights are still in flight ----
-    if constexpr (FUSEQ) {
-        XRegs<NTOK, WGS> xr;
-        xload<WT, NTOK, WGS>(xr, x, ldx, K);
-#pragma unroll
-        for (int d = 0; d < DEPTH; d++) issue(ring[d]);
-        quantize_into_image<WT, NTOK, WGS>(xr, lds, img, NI, K, ws, ws_stride);
-    } else {
-        StageRegs<WT, NTOK> sr;
-        stage_issue<WT, NTOK, WGS>(sr, NI, units, K, ws, ws_stride);
-#pragma unroll
-        for (int d = 0; d < DEPTH; d++) issue(ring[d]);
-        stage_commit<WT, NTOK, WGS>(sr, lds, img, NI, units, K, ws, ws_stride);
-    }
-    __syncthreads();
-
-    // ---- main loop: consume ring slot d, refill it with the step DEPTH ahead, accumulate ----
-    Cursor cc{wave, 0, wave < tiles};
-    float acc[R][NTOK];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int t = 0; t < NTOK; t++) acc[r][t] = 0.f;
-
-    while (cc.have) {
-#pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
-            if (!cc.have) break;
-            const int u = cc.it * 64 + lane;
-            const bool active = u < units;
-            typename T::W w[R];
-            if (active) {
-#pragma unroll
-                for (int r = 0; r < R; r++) T::decode(w[r], ring[d][r], u);
-            }
-            issue(ring[d]);
-            if (active) {
-#pragma unroll
-                for (int t = 0; t < NTOK; t++) {
-                    typename T::A a;
-                    T::load_a(a, lds + t * img, NI, cc.it, lane);
-#pragma unroll
-                    for (int r = 0; r < R; r++) acc[r][t] = T::dot(w[r], a, acc[r][t]);
-                }
-            }
-            if (cc.it + 1 == NI) {
-                const int64_t row0 = cc.tile * R;
-#pragma unroll
-                for (int r = 0; r < R; r++)
-#pragma unroll
-                    for (int t = 0; t < NTOK; t++) {
-                        const float s = wave_sum_to_lane63(acc[r][t]);
-                        if (lane == 63 && row0 + r < N) {
-                            y[(int64_t)t * ldy + row0 + r + (row0 + r >= sec.n_first ? sec.y_off : (int64_t)0)] = s;
-                            if (sec.t16) sec.t16[(row0 + r) * sec.t16_ld + t] = f2h_rne(s);
-                        }
-                        acc[r][t] = 0.f;
-                    }
-            }
-            advance(cc);
-        }
-    }
-}
 
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
 __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                                    const float *__restrict__ x, int64_t ldx,
                                                    uint8_t *__restrict__ ws, size_t ws_stride,
                                                    float *__restrict__ y, int64_t ldy, SecondMatrix sec) {
-    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec);
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
 }
 
 // LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
@@ -1038,33 +53,30 @@ __global__ __launch_bounds__(WGS) void gemv_id_kernel(const uint8_t *__restrict_
     if (e < 0 || e >= m.n_as) return;
     const int64_t xrow = t * m.ne11 + s % m.ne11;
     gemv_body<WT, 1, R, WGS, FUSEQ, DEPTH>(W + (size_t)e * m.nb02, nb01, K, N, FUSEQ ? x + xrow * ldx : x, ldx,
-                                          ws + (size_t)xrow * ws_stride, ws_stride, y + pair * ldy, ldy, kNoSecond);
+                                          ws + (size_t)xrow * ws_stride, ws_stride, y + pair * ldy, ldy, kNoSecond, whole_grid());
 }
 
 // ------------------------------------------------------------------------------------------------ launch
-// Rows per wave step.  Two steps are in flight per wave (the next step's loads are issued before the current
-// step's arithmetic), so one row of a 48..68-byte unit (Q4_K, Q6_K, Q8_0) or two rows of a 36-byte unit (Q4_0)
-// keep about 100..140 bytes per lane outstanding, the depth at which a plain read kernel with the same access
-// pattern peaks on this GPU; measured sweeps over rows x group size x groups per CU agree.
-template <int WT> struct RowsPerWave { static constexpr int R = (WT == T_Q4_0) ? 2 : 1; };
-
-// Steps of weight loads a wave keeps in flight.  A step is one row of at most 64 units (36..68 bytes per lane).
-#ifndef GEMV_DEPTH
-#define GEMV_DEPTH 1
-#endif
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
-static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
-                             size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, const DeviceLimits &lim,
-                             hipStream_t st, const SecondMatrix &sec) {
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
+static hipError_t launch_depth(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
+                               size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, const DeviceLimits &lim,
+                               hipStream_t st, const SecondMatrix &sec) {
     const int64_t tiles = ceil_div(N, R);
     int64_t groups = ceil_div(tiles, WGS / 64);
     if (groups > max_groups) groups = max_groups;
-    auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, GEMV_DEPTH>;
+    auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
                        (uint8_t *)ws, ws_stride, y, ldy, sec);
     return hipGetLastError();
+}
+
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
+static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
+                             size_t ws_stride, float *y, int64_t ldy, size_t lds_bytes, int64_t max_groups, const DeviceLimits &lim,
+                             hipStream_t st, const SecondMatrix &sec) {
+    return launch_depth<WT, NTOK, R, WGS, FUSEQ, GEMV_DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, max_groups, lim, st, sec);
 }
 
 template <int WT, int NTOK, bool FUSEQ>
@@ -1075,22 +87,12 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     constexpr int R = RowsPerWave<WT>::R;
-#ifdef CHIP_TUNE
-    if constexpr (NTOK == 1 || NTOK == 4 || NTOK == 8) {
-        const char *ew = getenv("CHIP_TUNE_WGS"), *er = getenv("CHIP_TUNE_R"), *ec = getenv("CHIP_TUNE_CAP");
-        if (ew && er && ec) {
-            const int w = atoi(ew), r = atoi(er); const int64_t cap = (int64_t)cus * atoi(ec);
-#define TUNE_CASE(WW, RR) if (w == WW && r == RR) return launch_one<WT, NTOK, RR, WW, FUSEQ>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cap, lim, st, sec);
-            TUNE_CASE(256, 1) TUNE_CASE(256, 2) TUNE_CASE(256, 4) TUNE_CASE(512, 1) TUNE_CASE(512, 2) TUNE_CASE(512, 4)
-            TUNE_CASE(1024, 1) TUNE_CASE(1024, 2) TUNE_CASE(1024, 4)
-#undef TUNE_CASE
-        }
-    }
-#endif
     // The activation prologue (staging, or quantizing in the fused variant) is paid once per workgroup, so the
     // grid is persistent: one or two 8-wave groups per CU, each wave striding over the row tiles.  Matrices with
     // too few rows to give every CU an 8-wave group use 4-wave groups instead.
-    const int64_t per_cu = (lds_bytes <= 24 * 1024) ? 2 : 1;
+    // The one-token kernel that quantizes in its prologue runs three such groups per CU (24 waves: with one step of loads
+    // in flight per wave the bytes in flight per CU grow with the waves; measured on 66 MB and 431 MB: 3 % faster than two).
+    const int64_t per_cu = tune("CHIP_GEMV_PER_CU", (lds_bytes <= 24 * 1024) ? ((FUSEQ && NTOK == 1) ? 3 : 2) : 1);
     const int64_t tiles = ceil_div(N, R);
     if constexpr (FUSEQ) {
         // When the matrix gives each of 16 waves per CU at most one tile, the prologue is a large share of the
@@ -1106,8 +108,7 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         // waves read one tile each.  16-wave groups do that with a quarter of the values per lane and keep the same
         // number of waves reading weights, on fewer CUs.  Measured on a 32-layer decode graph (wk / wv of 1024 rows,
         // K = 4096): 4 tokens 8.5 % faster for the whole step, 2 tokens 3.7 % slower - so from 8192 values up only.
-        static const bool narrow_wide_groups = [] { const char *e = getenv("CHIP_GEMV_NARROW_WIDE"); return !e || atoi(e) != 0; }();
-        if (narrow_wide_groups && (int64_t)NTOK * K > 8192 && ceil_div(tiles, 8) < cus)
+        if (tune("CHIP_GEMV_NARROW_WIDE", 1) != 0 && (int64_t)NTOK * K > 8192 && ceil_div(tiles, 8) < cus)
             return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
     }
     if (ceil_div(tiles, 8) >= cus)

@@ -1,0 +1,195 @@
+// Several matmuls on one activation as one launch of the decode GEMV: wq / wk / wv of an attention block, or any set of
+// weight matrices (up to GROUP_MAX, types may differ within a family that shares the activation format) that read the
+// same rows x.  Every workgroup belongs to one matrix and runs the ordinary GEMV body of that matrix's type on it, so each
+// output equals the single-matrix launch's bit for bit; the prologue (activation quantization, launch latency) is paid
+// once for the group instead of once per matrix.
+// Reference: the same rows of lm_ggml_compute_forward_mul_mat (ggml-cpu/ggml-cpu.c:1257-1449), which quantizes src1
+// once per node; llama.cpp builds Qcur / Kcur / Vcur from one tensor (llama-model.cpp build_llama, llama-graph.cpp).
+#include "gemv_body.h"
+
+namespace chip {
+
+namespace {
+
+struct GroupKernelMat {
+    const uint8_t *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld;
+    int wtype; int first_block;
+};
+struct GroupKernelArgs { GroupKernelMat m[GROUP_MAX]; int count; };
+
+template <int WT, int NTOK, int WGS, int DEPTH>
+__device__ __forceinline__ void run_member(const GroupKernelMat &m, int64_t K, const float *x, int64_t ldx, uint8_t *ws,
+                                           size_t ws_stride, const GridPart gp) {
+    const SecondMatrix sec{INT64_MAX, 0, 0, m.t16, m.t16_ld};
+    gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, true, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
+}
+
+// FAMILY 0: K-quants (Q8_K activations); 1: 32-value blocks (Q8_0 / Q8_1 planes); 2: F16.
+template <int FAMILY, int NTOK, int WGS, int DEPTH>
+__global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs ga, int64_t K, const float *__restrict__ x,
+                                                         int64_t ldx, uint8_t *__restrict__ ws, size_t ws_stride) {
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < GROUP_MAX; j++)
+        if (j < ga.count && (int)blockIdx.x >= ga.m[j].first_block) i = j;
+    const GroupKernelMat &m = ga.m[i];
+    const int last = (i + 1 < ga.count) ? ga.m[i + 1].first_block : (int)gridDim.x;
+    const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), blockIdx.x == 0};
+    if constexpr (FAMILY == 0) {
+        switch (m.wtype) {                                              // uniform over the workgroup
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+        }
+    } else if constexpr (FAMILY == 1) {
+        switch (m.wtype) {
+            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            default:       run_member<T_Q8_0, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+        }
+    } else {
+        run_member<T_F16, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp);
+    }
+}
+
+size_t image_bytes(int wtype, int64_t K) {
+    switch (wtype) {
+        case T_Q4_0: return lds_image_bytes<T_Q4_0>(K);
+        case T_Q8_0: return lds_image_bytes<T_Q8_0>(K);
+        case T_Q4_K: return lds_image_bytes<T_Q4_K>(K);
+        case T_Q6_K: return lds_image_bytes<T_Q6_K>(K);
+        case T_Q5_0: return lds_image_bytes<T_Q5_0>(K);
+        case T_Q5_K: return lds_image_bytes<T_Q5_K>(K);
+        case T_IQ4_NL: return lds_image_bytes<T_IQ4_NL>(K);
+        case T_Q4_1: return lds_image_bytes<T_Q4_1>(K);
+        case T_Q5_1: return lds_image_bytes<T_Q5_1>(K);
+        case T_F16: return lds_image_bytes<T_F16>(K);
+        default: return 0;
+    }
+}
+int rows_per_step(int wtype) { return wtype == T_Q4_0 ? RowsPerWave<T_Q4_0>::R : 1; }
+
+template <int FAMILY, int NTOK, int WGS, int DEPTH>
+hipError_t launch_depth(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
+                        size_t lds_bytes, const DeviceLimits &lim, hipStream_t st) {
+    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, DEPTH>;
+    static LdsGrant grant;
+    if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(WGS), lds_bytes, st, ga, K, x, ldx, (uint8_t *)ws, ws_stride);
+    return hipGetLastError();
+}
+template <int FAMILY, int NTOK, int WGS>
+hipError_t launch_cfg(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
+                      size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool) {
+    return launch_depth<FAMILY, NTOK, WGS, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
+}
+template <int FAMILY, int NTOK>
+hipError_t launch_wgs(int wgs, const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws,
+                      size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool deep) {
+    return wgs == 1024 ? launch_cfg<FAMILY, NTOK, 1024>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep)
+                       : launch_cfg<FAMILY, NTOK, 512>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+}
+template <int FAMILY>
+hipError_t launch_ntok(int n, int wgs, const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws,
+                       size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool deep) {
+    switch (n) {
+        case 1: return launch_wgs<FAMILY, 1>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        case 2: return launch_wgs<FAMILY, 2>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        case 4: return launch_wgs<FAMILY, 4>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+int gemv_group_family(int wtype) {
+    switch (wtype) {
+        case T_Q4_K: case T_Q5_K: case T_Q6_K: return 0;
+        case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: return 1;
+        case T_F16: return 2;
+        default: return -1;
+    }
+}
+
+// One launch serves the group when the prologue-quantizing GEMV takes every member (n in {1, 2, 4}, n * K within its
+// limit, the largest member's activation image within LDS) and the members are of one family.
+bool gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim) {
+    if (count < 1 || count > GROUP_MAX) return false;
+    const int fam = gemv_group_family(mats[0].wtype);
+    if (fam < 0) return false;
+    int64_t rows = 0;
+    for (int i = 0; i < count; i++) {
+        if (gemv_group_family(mats[i].wtype) != fam || !gemv_fused_applicable(mats[i].wtype, K, n, lim)) return false;
+        if (mats[i].N <= 0 || mats[i].N > 0x7fffffff) return false;
+        rows += mats[i].N;
+    }
+    // Q8_1 members (Q4_1 / Q5_1) need the same planes as Q8_0 members: one workspace dump serves both
+    return rows <= 0x7fffffff;
+}
+
+hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const float *x, int64_t ldx, int n, void *ws,
+                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st) {
+    if (!gemv_group_applicable(mats, count, K, n, lim)) return hipErrorInvalidValue;
+    const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
+    const int fam = gemv_group_family(mats[0].wtype);
+    size_t img = 0;
+    int64_t tiles = 0;
+    double cost[GROUP_MAX], total_cost = 0;
+    for (int i = 0; i < count; i++) {
+        const size_t b = image_bytes(mats[i].wtype, K);
+        if (b > img) img = b;
+        tiles += ceil_div(mats[i].N, (int64_t)rows_per_step(mats[i].wtype));
+        cost[i] = (double)mats[i].N * (double)mats[i].nb01;              // bytes to stream
+        total_cost += cost[i];
+    }
+    const size_t lds_bytes = (size_t)n * img;
+    if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
+    // As the single-matrix launcher: a persistent grid; one 16-wave workgroup per CU while every wave gets at most a
+    // couple of tiles (the prologue is then most of the kernel and is paid once per CU), else two 8-wave workgroups.
+    const int wgs = tiles <= 32 * (int64_t)cus ? 1024 : 512;
+    const int per_cu = (wgs == 1024 || lds_bytes > 24 * 1024) ? 1 : (n == 1 ? 3 : 2);
+    int grid = cus * per_cu;
+    const int64_t max_useful = ceil_div(tiles, (int64_t)(wgs / 64));
+    if (grid > max_useful) grid = (int)max_useful;
+    if (grid < count) grid = count;
+    // workgroups in proportion to the bytes each member streams (largest remainder), at least one each
+    int blocks[GROUP_MAX], given = 0;
+    double frac[GROUP_MAX];
+    for (int i = 0; i < count; i++) {
+        const double share = cost[i] / total_cost * grid;
+        blocks[i] = (int)share;
+        if (blocks[i] < 1) blocks[i] = 1;
+        frac[i] = share - (double)blocks[i];
+        given += blocks[i];
+    }
+    while (given < grid) {
+        int best = 0;
+        for (int i = 1; i < count; i++) if (frac[i] > frac[best]) best = i;
+        blocks[best]++; frac[best] -= 1.0; given++;
+    }
+    while (given > grid) {                                                // the minimum of one each overshot
+        int best = -1;
+        for (int i = 0; i < count; i++) if (blocks[i] > 1 && (best < 0 || frac[i] < frac[best])) best = i;
+        if (best < 0) break;
+        blocks[best]--; frac[best] += 1.0; given--;
+    }
+    GroupKernelArgs ga{};
+    ga.count = count;
+    int first = 0;
+    for (int i = 0; i < count; i++) {
+        ga.m[i] = GroupKernelMat{(const uint8_t *)mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].t16,
+                                 mats[i].t16_ld, mats[i].wtype, first};
+        first += blocks[i];
+    }
+    const bool deep = tiles > (int64_t)first * (wgs / 64);              // some wave walks two or more tiles
+    switch (fam) {
+        case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+    }
+}
+
+}  // namespace chip

@@ -319,8 +319,7 @@ hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const vo
 
 // Tokens one launch takes for this shape: 16 if the 16-token image fits in LDS, else 8, else 0 (use the dot-product GEMV).
 int mmv_q4_0_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim) {
-    static const bool off = [] { const char *e = getenv("CHIP_MMV_Q4_0"); return e && e[0] == '0'; }();     // tuning: dot-product GEMV instead
-    if (off || K % 256 != 0) return 0;
+    if (tune("CHIP_MMV_Q4_0", 1) == 0 || K % 256 != 0) return 0;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
     if (N > (1 << 24) || K > (1 << 20)) return 0;                        // the kernel's 32-bit tile arithmetic

@@ -378,8 +378,7 @@ hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const 
 // Tokens one launch takes for this shape and type (Q4_K or Q5_K): 16 if the 16-token image fits in LDS, else 8, else 0
 // (use the dot-product GEMV).
 int mmv_q4k_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim) {
-    static const bool off = [] { const char *e = getenv("CHIP_MMV_Q4K"); return e && e[0] == '0'; }();      // tuning: dot-product GEMV instead
-    if (off || K % 256 != 0 || (wtype != T_Q4_K && wtype != T_Q5_K)) return 0;
+    if (tune("CHIP_MMV_Q4K", 1) == 0 || K % 256 != 0 || (wtype != T_Q4_K && wtype != T_Q5_K)) return 0;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
     if (N > (1 << 24) || K > (1 << 20)) return 0;                        // 32-bit tile arithmetic

@@ -268,16 +268,14 @@ hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const vo
 
 // Tokens one launch takes for this shape: 8 if the image fits in LDS, else 0 (use the dot-product GEMV).
 int mmv_q6k_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim) {
-    static const bool off = [] { const char *e = getenv("CHIP_MMV_Q6K"); return e && e[0] == '0'; }();      // tuning: dot-product GEMV instead
-    if (off || K % 256 != 0) return 0;
+    if (K % 256 != 0) return 0;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if (ceil_div(N, 16) < cus) return 0;                                 // too few 16-row tiles to occupy every CU
     if (N > (1 << 24) || K > (1 << 20)) return 0;                        // 32-bit tile arithmetic
     // Measured against the dot-product GEMV at 8 tokens: 128256 x 4096 131.5 vs 142.5 us, 14336 x 4096 22.0 vs 22.0 us,
     // 4096 x 14336 25.0 vs 21.5 us, 4096 x 4096 12.6 vs 9.4 us.  Two sub-blocks per MFMA mean 8-byte operand reads and
     // twice the LDS traffic per weight of the 16x16x64 kernels: it only pays on very large matrices (an output head).
-    static const bool force = [] { const char *e = getenv("CHIP_MMV_Q6K"); return e && e[0] == '1'; }();
-    if (!force && N * K < (128LL << 20)) return 0;
+    if (!g_force_mmv_q6k.load(std::memory_order_relaxed) && N * K < (128LL << 20)) return 0;
     return mmv_q6k_lds_bytes<8>(K) <= (size_t)lim.max_lds_per_block ? 8 : 0;
 }
 

@@ -4,9 +4,22 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <atomic>
+#include <cstdlib>
 #include "dev_common.h"
 
 namespace chip {
+
+// Dispatch thresholds and kernel shapes are constants of the library.  A build with -DCHIP_TUNING (make TUNING=1, never
+// the default) lets the environment variable `name` replace one of them for a measurement sweep.
+#ifdef CHIP_TUNING
+inline int64_t tune(const char *name, int64_t dflt) { const char *e = getenv(name); return e ? (int64_t)atoll(e) : dflt; }
+#else
+inline constexpr int64_t tune(const char *, int64_t dflt) { return dflt; }
+#endif
+
+// Verification hook (chip_verify_force_q6k_matrix_core): the Q6_K matrix-core GEMV on shapes below its size threshold.
+extern std::atomic<int> g_force_mmv_q6k;
+
 
 struct DeviceLimits {
     int compute_units;
@@ -139,6 +152,15 @@ hipError_t launch_gemv_fused_store_t(int wtype, const void *W, size_t nb01, int6
 hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                   int64_t ldx, int n, void *ws, size_t ws_stride, float *y1, float *y2, int64_t ldy,
                                   const DeviceLimits &lim, hipStream_t st);
+// gemv_group.hip: up to GROUP_MAX matrices that read the same activation rows in one launch of the prologue-quantizing
+// GEMV (members of one family: K-quants, 32-value block types, or F16).  t16: optional transposed fp16 copy of a member's
+// output, as launch_gemv_fused_store_t.
+constexpr int GROUP_MAX = 4;
+struct GroupMat { int wtype; const void *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld; };
+int        gemv_group_family(int wtype);
+bool       gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim);
+hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const float *x, int64_t ldx, int n, void *ws,
+                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st);
 // MUL_MAT_ID: every (token, slot) pair is a one-token GEMV on the expert ids[token][slot] names (W + id * nb02), its
 // activation row token * ne11 + slot % ne11, its output row token * n_used + slot.  fused: x is fp32 and is quantized in
 // the prologue; otherwise ws already holds the quantized rows.

@@ -64,8 +64,8 @@ __device__ __forceinline__ float silu1(float x) { return x / (1.0f + v_expf_lane
 // own elements), and the norm then runs over the stored sum.
 template <bool ADD, int QKIND = 0>
 __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, int64_t ldx, int64_t ne0, float eps,
-                                                              float *__restrict__ y, int64_t ldy, const float *__restrict__ w,
-                                                              float *__restrict__ yn, int64_t ldyn, const float *b, int64_t ldb,
+                                                              float *y, int64_t ldy, const float *__restrict__ w,
+                                                              float *yn, int64_t ldyn, const float *b, int64_t ldb,
                                                               float *xs, int64_t ldxs, uint8_t *__restrict__ qws, size_t qstride) {
     constexpr int qkind = QKIND;                                 // 0: no quantized copy; 1: Q8_0 / Q8_1 planes; 2: Q8_K planes
     __shared__ double part[EW_THREADS / 64];
@@ -203,9 +203,9 @@ template <int OP> __device__ __forceinline__ float ew_apply(float a, float b) {
     else return silu1(a);
 }
 template <int OP, bool VEC>
-__global__ __launch_bounds__(EW_THREADS) void elementwise_kernel(const float *__restrict__ a, int64_t lda,
-                                                                 const float *__restrict__ b, int64_t ldb, int64_t ne0,
-                                                                 int64_t n, float *__restrict__ y, int64_t ldy) {
+__global__ __launch_bounds__(EW_THREADS) void elementwise_kernel(const float *a, int64_t lda,
+                                                                 const float *b, int64_t ldb, int64_t ne0,
+                                                                 int64_t n, float *y, int64_t ldy) {
     for (int64_t row = blockIdx.y; row < n; row += gridDim.y) {
         const float *ar = a + (size_t)row * lda;
         const float *br = (OP == EW_SILU) ? nullptr : b + (size_t)row * ldb;       // ldb = 0: one row for all
@@ -239,8 +239,8 @@ template <int OP> __device__ __forceinline__ float unary_apply(float x, float s,
     }
 }
 template <int OP, bool VEC>
-__global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restrict__ x, int64_t ldx, int64_t ne0, int64_t n,
-                                                           float *__restrict__ y, int64_t ldy, float s,
+__global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *x, int64_t ldx, int64_t ne0, int64_t n,
+                                                           float *y, int64_t ldy, float s,
                                                            const unsigned short *__restrict__ table) {
     for (int64_t row = blockIdx.y; row < n; row += gridDim.y) {
         const float *xr = x + (size_t)row * ldx;
@@ -281,8 +281,8 @@ __device__ __forceinline__ float group_sum8(const float (&e)[8]) {
     return ((e[0] + e[4]) + (e[2] + e[6])) + ((e[1] + e[5]) + (e[3] + e[7]));
 }
 template <int MASK, int G>
-__global__ __launch_bounds__(EW_THREADS) void soft_max_kernel(const float *__restrict__ x, int64_t ldx, const void *__restrict__ mask,
-                                                              int64_t ne00, int64_t ne01, float scale, float *__restrict__ y,
+__global__ __launch_bounds__(EW_THREADS) void soft_max_kernel(const float *x, int64_t ldx, const void *__restrict__ mask,
+                                                              int64_t ne00, int64_t ne01, float scale, float *y,
                                                               int64_t ldy) {
     __shared__ float wmax[EW_THREADS / 64];
     __shared__ double wsum[EW_THREADS / 64];
@@ -631,8 +631,8 @@ hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st) {
 enum { ROPE_FULL = 0, ROPE_BUILD = 1, ROPE_APPLY = 2 };
 constexpr int ROPE_MAX_PAIRS = 256;
 template <int MODE>
-__global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *__restrict__ x, const int32_t *__restrict__ pos,
-                                                          const float *__restrict__ freq_factors, RopeArgs a, float *__restrict__ y,
+__global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *x, const int32_t *__restrict__ pos,
+                                                          const float *__restrict__ freq_factors, RopeArgs a, float *y,
                                                           float *__restrict__ table) {
     __shared__ float cs[ROPE_MAX_PAIRS], sn[ROPE_MAX_PAIRS];
     constexpr int PRE = 8;                                       // items per thread whose loads are issued before the table is built

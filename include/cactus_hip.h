@@ -156,6 +156,29 @@ CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, i
 CHIP_API int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                int64_t ldx, int64_t n, float *y1, float *y2, int64_t ldy, void *workspace, size_t workspace_bytes,
                                void *stream);
+/* Several matmuls that read the same activation rows (wq / wk / wv of an attention block: llama.cpp builds Qcur, Kcur,
+ * Vcur from one tensor, llama-model.cpp build_llama; the reference quantizes src1 once per MUL_MAT node,
+ * ggml-cpu/ggml-cpu.c:1319-1354) as one call: up to CHIP_GROUP_MAX weight matrices with the same K, each with its own
+ * type, row count, row stride and output.  The types must share one activation format (chip_vec_dot_type; Q8_0 and Q8_1
+ * count as one).  Up to 4 tokens, members of one family (K-quants / 32-value block types / F16): one launch of the GEMV that
+ * quantizes in its prologue, its workgroups divided among the members by the bytes each streams; otherwise one
+ * quantizer launch and every member on the path chip_mul_mat_run_ws would take.  A member with y_f16_t != NULL also gets
+ * its result rounded to fp16 at y_f16_t[row * ld16 + token], as chip_mul_mat_store_t.  Every output equals, bit for bit,
+ * what chip_mul_mat (chip_mul_mat_store_t) returns for that member alone.  The workspace must hold
+ * chip_mul_mat_workspace_size(type, K, n) bytes for the members' activation format. */
+#define CHIP_GROUP_MAX 4
+typedef struct chip_mat {
+    int         type;       /* weight type */
+    const void *W;          /* N rows of nb01 bytes */
+    size_t      nb01;
+    int64_t     N;
+    float      *y;          /* [n][N], row stride ldy elements */
+    int64_t     ldy;
+    uint16_t   *y_f16_t;    /* NULL, or the transposed fp16 copy [N][ld16] */
+    int64_t     ld16;
+} chip_mat;
+CHIP_API int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n,
+                                void *workspace, size_t workspace_bytes, void *stream);
 /* chip_mul_mat whose result also goes, rounded to fp16 (nearest even), to y_f16_t[row * ld16 + token]: the V projection
  * and its store into the transposed F16 V cache (llama-kv-cache.cpp cpy_v without flash attention) - one launch up to 4
  * tokens, otherwise the matmul followed by the copy.  Results as from chip_mul_mat and chip_cpy. */
@@ -313,6 +336,9 @@ CHIP_API int chip_rope_apply_store(const float *x, int64_t ldx1, int64_t ldx2, c
  *   imin : Q4_K and Q5_K only, [n][N][K/256] int32 (sum of min_j * bsum pairs); NULL otherwise */
 CHIP_API int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
                               const void *aq, int64_t n, int32_t *isum, int32_t *imin, void *stream);
+/* on != 0: Q6_K matmuls of 5 to 8 tokens take the matrix-core GEMV on every shape it supports, not only on the very
+ * large matrices where it is the default, so tests can run that kernel on small inputs; 0 restores the default. */
+CHIP_API int chip_verify_force_q6k_matrix_core(int on);
 /* Rebuilds the reference block layout from a prepared workspace (inverse of the kernel-private layout), so
  * tests can check that the fused prepare step quantizes bit-identically to chip_quantize_q8_0/_q8_K. */
 CHIP_API int chip_workspace_to_blocks(int type, int64_t K, int64_t n, const void *workspace, void *y, void *stream);

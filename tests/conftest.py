@@ -4,9 +4,6 @@ import sys
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-# The Q6_K matrix-core GEMV is only chosen for very large matrices (an output head); the parity tests run it on
-# ordinary shapes as well.  The library reads the variable once, at its first multi-token Q6_K call.
-os.environ.setdefault("CHIP_MMV_Q6K", "1")
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 

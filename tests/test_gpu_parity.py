@@ -35,6 +35,13 @@ def dev():
     return d
 
 
+@pytest.fixture
+def forced_q6k_matrix_core(dev):
+    dev.lib.chip_verify_force_q6k_matrix_core(1)
+    yield
+    dev.lib.chip_verify_force_q6k_matrix_core(0)
+
+
 def check_outputs(y_gpu, y_ref, sum_abs, what):
     err = np.abs(y_gpu.astype(np.float64) - y_ref.astype(np.float64))
     bound = REL_TOL * sum_abs
@@ -201,9 +208,11 @@ def test_mul_mat_q4_0_matrix_core_gemv(dev, orc, K, N, n):
 
 @pytest.mark.parametrize("K,N", [(256, 4100), (1024, 4111), (4096, 4096), (11008, 4099), (14336, 4096)])
 @pytest.mark.parametrize("n", [5, 8, 9, 16, 21])
-def test_mul_mat_q6_K_matrix_core_gemv(dev, orc, K, N, n):
+def test_mul_mat_q6_K_matrix_core_gemv(dev, orc, K, N, n, forced_q6k_matrix_core):
     # the Q6_K form: unsigned 6-bit operands, int8 sub-block scales, the -32 taken out through the activation block sums;
-    # rows that are only 2-byte aligned (210-byte super-blocks), ragged N, several launches of 8 tokens
+    # rows that are only 2-byte aligned (210-byte super-blocks), ragged N, several launches of 8 tokens.  By default the
+    # library takes this kernel only on very large matrices (an output head; tests/test_gpu_config5.py runs that shape
+    # with the default dispatch); the fixture makes it take these shapes too.
     print("mmv q6_K K", K, "N", N, "n", n, flush=True)
     wq = quantized_weights(O.Q6_K, K + N + 3, N, K)
     x = common.activations_f32(K + n + 3, n, K)
@@ -417,11 +426,9 @@ def test_config4_prefill_sampled(dev, orc, N, M):
     assert np.array_equal(y2[:, ::-1], y[:64])
 
 
-@pytest.mark.parametrize("K,N,n", [(256, 1, 32), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257), (64, 70, 40)])
+@pytest.mark.parametrize("K,N,n", [(256, 1, 32), (512, 40, 33), (1024, 131, 64), (4096, 300, 130), (2048, 260, 257)])
 def test_gemm_f16_vs_oracle(dev, orc, K, N, n):
     print("gemm f16 K", K, "N", N, "n", n, flush=True)
-    if K % 256:
-        pytest.skip("the C-ABI takes K in multiples of 256")
     wq = orc.quantize_weights(O.F16, common.weights_f32(K + N, N, K, outliers=True))
     x = common.activations_f32(K + n, n, K)
     x[3] = 0
@@ -429,6 +436,17 @@ def test_gemm_f16_vs_oracle(dev, orc, K, N, n):
     y, blocks = dev.mul_mat(O.F16, wq, x, want_workspace_blocks=True)
     assert np.array_equal(blocks, ref["wdata"])
     check_outputs(y, ref["y"], ref["sum_abs"], "f16 gemm")
+
+
+def test_f16_rows_of_k_not_a_multiple_of_256_are_rejected(dev):
+    """F16 weights (like the K-quants) are taken in rows of K % 256 == 0 only: the C-ABI says so instead of computing."""
+    K, N, n = 64, 70, 40
+    assert dev.lib.chip_mul_mat_supported(O.F16, K) == 0
+    assert dev.lib.chip_mul_mat_workspace_size(O.F16, K, n) == 0
+    buf = dev.alloc(1 << 16)
+    assert dev.lib.chip_mul_mat(O.F16, buf.ptr, 2 * K, K, N, buf.ptr, K, n, buf.ptr, N, buf.ptr, 1 << 16, None) == -2
+    assert dev.lib.chip_mul_mat_prepare(O.F16, K, buf.ptr, K, n, buf.ptr, 1 << 16, None) == -2
+    dev.sync()
 
 
 def test_gemm_f16_exact_small_integers(dev, orc):
@@ -656,3 +674,48 @@ def test_mul_mat_id_argument_errors(dev, orc):
     dev.sync()
     out = dy.download(np.float32, 2 * N).reshape(2, N)
     assert np.isfinite(out[0]).all() and np.isnan(out[1]).all()
+
+
+# ------------------------------------------------------------------------------------------ several matrices, one activation
+@pytest.mark.parametrize("members", [
+    ((O.Q4_K, 300), (O.Q6_K, 77), (O.Q5_K, 1)),                      # K-quants of three types, ragged row counts
+    ((O.Q4_0, 129), (O.Q8_0, 64), (O.Q5_1, 33), (O.IQ4_NL, 200)),    # 32-value block types incl. a Q8_1 member, two-row tiles
+    ((O.F16, 40), (O.F16, 3)),
+    ((O.Q6_K, 2000),),                                               # a group of one
+], ids=["kquants", "block32", "f16", "single"])
+@pytest.mark.parametrize("K", [1024, 4096])
+def test_mul_mat_group_equals_single_calls(dev, orc, members, K):
+    """chip_mul_mat_group: each member's output equals chip_mul_mat on that member alone, bit for bit, for every token
+    count class (1, 2, 4: one launch; 3, 7: one quantizer and the GEMVs; 40: the GEMMs), and the oracle within tolerance."""
+    ws = [(wt, quantized_weights(wt, K + N + 11, N, K)) for wt, N in members]
+    for n in (1, 2, 4, 3, 7, 40):
+        x = common.activations_f32(K + n + 5, n, K)
+        ys = dev.mul_mat_group(ws, x)
+        for (wt, W), y in zip(ws, ys):
+            assert y.tobytes() == dev.mul_mat(wt, W, x).tobytes(), (O.TYPE_NAMES[wt], n)
+        wt, W = ws[0]
+        ref = orc.mul_mat(wt, W, x, nthreads=8, want=("sum_abs",))
+        check_outputs(ys[0], ref["y"], ref["sum_abs"], "group member 0, n = %d" % n)
+
+
+def test_mul_mat_group_argument_errors(dev, orc):
+    import cactus_amd as ca
+    L = dev.lib
+    K, N = 1024, 8
+    buf, ws = dev.alloc(1 << 16), dev.alloc(1 << 16)
+    def mats(*types):
+        arr = (ca.Mat * len(types))()
+        for i, t in enumerate(types):
+            arr[i] = ca.Mat(t, buf.ptr, dev.row_size(t, K), N, buf.ptr, N, None, 0)
+        return arr
+    call = lambda arr, count, n=1, wsz=1 << 16: L.chip_mul_mat_group(arr, count, K, buf.ptr, K, n, ws.ptr, wsz, None)
+    assert call(mats(O.Q4_K, O.Q6_K), 2) == 0
+    assert call(mats(O.Q4_K, O.Q8_0), 2) == -2                   # different activation formats
+    assert call(mats(O.Q4_K, 30), 2) == -2                       # unknown type
+    assert call(mats(O.Q4_K), 5) == -1                           # more members than CHIP_GROUP_MAX
+    assert call(mats(O.Q4_K), 1, wsz=16) == -3
+    assert call(None, 1) == -1 and call(None, 0) == 0 and call(mats(O.Q4_K), 1, n=0) == 0
+    bad = mats(O.Q4_K)
+    bad[0].ldy = N - 1
+    assert call(bad, 1) == -1
+    dev.sync()
