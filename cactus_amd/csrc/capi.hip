@@ -14,6 +14,9 @@
 
 using namespace chip;
 
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];      // chip_mul_mat_noalloc's workspace
+
 namespace {
 
 // From this many tokens on the matrix-core GEMV beats the dot-product GEMV (measured on Q8_0 4096x11008).
@@ -27,6 +30,29 @@ namespace {
 std::mutex g_mu;
 bool g_limits_ready[64] = {};
 DeviceLimits g_limits[64];
+
+// Device memory of chip_mul_mat_noalloc: quantized activation rows and, behind them, the partial outputs of a GEMM whose
+// K is split.  Every GPU holds its own copy of the array for the life of the process; host code never uses the array's
+// name as an address, only the per-device pointer hipGetSymbolAddress returned (g_scratch_ptr).
+void *g_scratch_ptr[64] = {};
+
+// Address of the current device's scratch array, looked up once per device.
+int scratch_address(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return CHIP_EINVAL;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return CHIP_EINVAL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return CHIP_OK;
+}
 
 int hip_rc(hipError_t e) { return e == hipSuccess ? CHIP_OK : (int)e; }
 
@@ -99,7 +125,9 @@ int chip_init(int device) {
     if (e != hipSuccess) return (int)e;
     if (std::strncmp(p.gcnArchName, "gfx950", 6) != 0) return CHIP_ENODEVICE;   // the kernels are built for gfx950 only
     DeviceLimits lim;
-    return current_limits(lim);
+    if (int rc = current_limits(lim); rc) return rc;
+    void *sp = nullptr;
+    return scratch_address(&sp);                                        // chip_mul_mat_noalloc's memory on this device
 }
 
 int chip_get_device_info(chip_device_info *out) {
@@ -396,6 +424,20 @@ int chip_mul_mat(int type, const void *W, size_t nb01, int64_t K, int64_t N, con
     int rc = chip_mul_mat_prepare(type, K, x, ldx, n, workspace, workspace_bytes, stream);
     if (rc) return rc;
     return mul_mat_run(type, W, nb01, K, N, n, workspace, workspace_bytes, y, ldy, stream);
+}
+
+// chip_mul_mat on the library's own static device array instead of a caller's workspace: no allocation of any kind.
+size_t chip_mul_mat_noalloc_max_workspace(void) { return NOALLOC_SCRATCH_BYTES; }
+int chip_mul_mat_noalloc(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
+                         float *y, int64_t ldy, void *stream) {
+    if (N < 0 || n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n == 0) return CHIP_OK;
+    if (chip_mul_mat_workspace_size(type, K, n) > NOALLOC_SCRATCH_BYTES) return CHIP_ENOMEM;   // the activation rows must fit
+    void *sp = nullptr;
+    if (int rc = scratch_address(&sp); rc) return rc;
+    // With room behind the activation rows a GEMM may split K, exactly as chip_mul_mat does with a workspace of this size.
+    return chip_mul_mat(type, W, nb01, K, N, x, ldx, n, y, ldy, sp, NOALLOC_SCRATCH_BYTES, stream);
 }
 
 // Two matmuls on one activation (ffn_gate / ffn_up).  Up to 4 tokens: one launch of the prologue-quantizing GEMV over

@@ -190,6 +190,17 @@ CHIP_API int chip_mul_mat_store_t(int type, const void *W, size_t nb01, int64_t 
 CHIP_API int chip_mul_mat_run_ws(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n,
                                  void *workspace, size_t workspace_bytes, float *y, int64_t ldy, void *stream);
 
+/* chip_mul_mat for callers that cannot allocate device memory or hand one over (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is a static device
+ * array inside the library (chip_mul_mat_noalloc_max_workspace() bytes, 16 MiB, held by every GPU the library runs on
+ * until the process ends); the call allocates nothing and frees nothing.  Results equal chip_mul_mat's with a workspace
+ * of that size, bit for bit.  CHIP_ENOMEM when chip_mul_mat_workspace_size(type, K, n) exceeds the array (e.g. more than
+ * 3500 tokens of K = 4096).  All calls on one GPU share the array: calls that may overlap in time (different streams)
+ * race; calls on one stream are ordered and safe.  Nothing in the array has to start at zero. */
+CHIP_API size_t chip_mul_mat_noalloc_max_workspace(void);
+CHIP_API int    chip_mul_mat_noalloc(int type, const void *W, size_t nb01, int64_t K, int64_t N,
+                                     const float *x, int64_t ldx, int64_t n, float *y, int64_t ldy, void *stream);
+
 /* ---- LM_GGML_OP_MUL_MAT_ID: the expert matmul of mixture-of-experts layers ----
  * lm_ggml_compute_forward_mul_mat_id (ggml-cpu/ggml-cpu.c:1460-1710) with src0 = W (type, [K, N, n_as]: n_as expert
  * matrices, row stride nb01 and matrix stride nb02 bytes), src1 = x (F32 [K, ne11, n_tokens], row stride ldx
