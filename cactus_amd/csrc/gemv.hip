@@ -179,6 +179,10 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
 // small: n * K <= 16384 values (64 KB of fp32 per workgroup) and n in {1, 2, 4}.
 bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
     if (!(n == 1 || n == 2 || n == 4) || (int64_t)n * K > FUSE_MAX_VALUES) return false;
+    // Every workgroup repeats the quantizer, and its dependent chains (maximum, two divisions, sums) cost a wave about
+    // 0.9 us per 256 values: beyond 8192 values per workgroup the separate quantizer kernel (1.9 us) and the GEMV over
+    // prepared rows are ahead (Q6_K 4096 x 14336, one token: 1.97 + 12.6 us against 15.3-16.1 us in one launch).
+    if ((int64_t)n * K > 8192 && n == 1) return false;
     size_t img = 0;
     switch (wtype) {
         case T_Q4_0: img = lds_image_bytes<T_Q4_0>(K); break;

@@ -906,7 +906,12 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     const int64_t tiles = ceil_div(N, R);
 
     // A wave walks the steps (tile, it) = (wave, 0), (wave, 1), ..., (wave + nwaves, 0), ...; while it computes one step
-    // the loads of the next are in flight (deeper rings measured slower).  All of this state is wave-uniform.
+    // the loads of the next are in flight.  Measured and dropped: rings of two and three steps (3-8 % slower as a loop; the
+    // compiler cannot count the outstanding loads of a second register set across the back-edge and waits for all of
+    // them), all steps of a short wave requested up front as straight-line code (exact waits, but 12.6 -> 14.2 us on a
+    // 4096 x 14336 Q6_K matrix: four steps per wave at once thrash), tiles drawn from device-scope counters instead of
+    // fixed shares (waves on different CUs finish between 53 and 86 us on a 431 MB matrix, yet handing the slow waves' tiles
+    // to the fast ones changes nothing: the rate is the memory system's, not the distribution's).  All state is wave-uniform.
     struct Step { int64_t tile; int it; bool have; };
     auto after = [&](const Step &s) {
         Step n = s;
@@ -919,7 +924,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     // compiler wait for everything in flight, outstanding stores included, before the next use of a load register.
     // In the prologue the loads are issued whether or not the wave has a tile (one without re-reads row 0): behind any
     // branch, the wait for the activations - requested earlier - would turn into a wait for these weights as well.
-    typename T::Raw ring0[R];
+    typename T::Raw ring[R];
     auto load_step = [&](typename T::Raw (&set)[R], const Step &s, bool always) {
         if (always || s.have) {
             const int u = min(s.it * 64 + lane, units - 1);
@@ -937,12 +942,12 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     if constexpr (FUSEQ) {
         XRegs<NTOK, WGS> xr;
         xload<WT, NTOK, WGS>(xr, x, ldx, K);
-        load_step(ring0, s0, true);
+        load_step(ring, s0, true);
         quantize_into_image<WT, NTOK, WGS>(xr, lds, img, NI, K, ws, ws_stride, gp.writes_workspace);
     } else {
         StageRegs<WT, NTOK> sr;
         stage_issue<WT, NTOK, WGS>(sr, NI, units, K, ws, ws_stride);
-        load_step(ring0, s0, true);
+        load_step(ring, s0, true);
         stage_commit<WT, NTOK, WGS>(sr, lds, img, NI, units, K, ws, ws_stride);
     }
     __syncthreads();
@@ -974,7 +979,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     // one step: decode `set` (holding step s), refill it with step `next`, then the arithmetic of s
     auto consume = [&](typename T::Raw (&set)[R], const Step &s, const Step &next) {
         const int u = s.it * 64 + lane;
-        const bool active = u < units;
+        const bool active = s.have && u < units;
         typename T::W w[R];
         if (active) {
 #pragma unroll
@@ -990,7 +995,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
                 for (int r = 0; r < R; r++) acc[r][t] = T::dot(w[r], a, acc[r][t]);
             }
         }
-        if (s.it + 1 == NI) {
+        if (s.have && s.it + 1 == NI) {
 #pragma unroll
             for (int r = 0; r < R; r++)
 #pragma unroll
@@ -1009,7 +1014,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
         while (s0.have && nres < 64) {
             const Step cur = s0;
             s0 = after(cur);
-            consume(ring0, cur, s0);
+            consume(ring, cur, s0);
         }
         flush(nres);
         nres = 0;
