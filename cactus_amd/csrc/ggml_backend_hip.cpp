@@ -25,7 +25,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -212,6 +212,7 @@ void backend_synchronize(lm_ggml_backend_t backend) { chip_stream_synchronize(((
 void backend_set_tensor_async(lm_ggml_backend_t backend, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
     chip_memcpy_h2d((char *)t->data + offset, data, size, ((backend_ctx *)backend->context)->stream);
     g_uploaded += size;
+    g_uploaded_async += size;
 }
 void backend_get_tensor_async(lm_ggml_backend_t backend, const lm_ggml_tensor *t, void *data, size_t offset, size_t size) {
     chip_memcpy_d2h(data, (const char *)t->data + offset, size, ((backend_ctx *)backend->context)->stream);
@@ -1050,6 +1051,7 @@ void *reg_get_proc_address(lm_ggml_backend_reg_t, const char *name) {
     if (std::strcmp(name, "lm_ggml_backend_hip_get_fused_pairs") == 0) return (void *)lm_ggml_backend_hip_get_fused_pairs;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_quantizers_skipped") == 0) return (void *)lm_ggml_backend_hip_get_quantizers_skipped;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_rope_tables") == 0) return (void *)lm_ggml_backend_hip_get_rope_tables;
+    if (std::strcmp(name, "lm_ggml_backend_hip_get_async_uploaded") == 0) return (void *)lm_ggml_backend_hip_get_async_uploaded;
     return nullptr;         // no n_threads, no extra buffer types, no split buffer type, no feature list
 }
 const lm_ggml_backend_reg_i k_reg_i = {reg_name, reg_device_count, reg_get_device, reg_get_proc_address};
@@ -1112,5 +1114,6 @@ void lm_ggml_backend_hip_get_stats(unsigned long long *mul_mat_nodes, unsigned l
 unsigned long long lm_ggml_backend_hip_get_fused_pairs(void) { return g_fused_pairs.load(); }
 unsigned long long lm_ggml_backend_hip_get_quantizers_skipped(void) { return g_quantizers_skipped.load(); }
 unsigned long long lm_ggml_backend_hip_get_rope_tables(void) { return g_rope_tables.load(); }
+unsigned long long lm_ggml_backend_hip_get_async_uploaded(void) { return g_uploaded_async.load(); }
 
 }  // extern "C"

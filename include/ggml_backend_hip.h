@@ -49,6 +49,9 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_fused_pairs(void);
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_quantizers_skipped(void);   /* matmuls that reused the previous one's quantized input */
 /* cos / sin tables built for ROPE nodes (one per graph_compute call and set of parameters; the other ROPE nodes apply it). */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_tables(void);
+/* Bytes that arrived through set_tensor_async (the model loader's pinned-staging upload loop,
+ * cactus/llama-model-loader.cpp:1047-1064); a subset of uploaded_bytes above. */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_async_uploaded(void);
 
 #ifdef __cplusplus
 }
