@@ -189,6 +189,159 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
         }
 }
 
+// ---- the large-shape kernel: 256 x 256 output tile, 4 waves, each 128 x 128 (4 x 4 MFMA tiles, 256 accumulator registers) ----
+// One wave per SIMD, so nothing hides a wait but the wave's own instruction stream: the loop is software pipelined by
+// hand, one memory instruction after each MFMA.  Stages of 32 k (two k-groups of 16) in four LDS buffers.  During
+// stage s a wave runs the 32 MFMAs of the stage, reads the operand registers of the next k-group (the second group of s,
+// then the first group of s + 1) into the other half of a register double buffer, and issues its share of the loads of
+// stage s + 3.  One barrier per stage, in the middle: it publishes stage s + 1 and separates the last reads of stage s's
+// buffer from the loads the next stage aims at it.
+// The operands go straight from global memory into LDS (global_load_lds_dwordx4): no staging registers, no ds_write.
+// A wave instruction deposits 64 cells of 16 bytes at consecutive LDS addresses in lane order, and each lane chooses its
+// own global address: four neighbouring lanes fetch the four cells of one row's 64 contiguous bytes, 16 rows per
+// instruction, so LDS holds [row][4 cells] with a row pitch of 64 bytes.  A 64-byte pitch would put rows r, r + 4, r + 8,
+// r + 12 into the same banks when 16 lanes read the same cell of 16 rows; cell c of row r therefore sits in slot
+// c ^ ((r >> 2) & 3) (the lane that fills a slot fetches the matching cell).
+// Measured on one tile with K = 4096 (32 tiles in flight, 2.39 GHz): 55 us of MFMA issue alone; 63 us with the operand
+// reads (a ds_read_b128 between MFMAs costs the wave about 9 clocks); 70 us with the output stores (256 KB leave a CU at
+// about 16 bytes per clock); 87 us with the loads.  What the loads cost is not latency (a fifth buffer changes nothing;
+// loads that always hit the cache cost the same; half as many loads cost half) but about 37 clocks of the issuing wave
+// per 1 KB written to LDS - the same as a ds_write_b128 of register-staged data costs, while plain global loads into
+// registers cost nothing.  With all 256 CUs busy a tile takes 1.2 - 1.3 times longer (clock under load).
+constexpr int BIG_B = 256, BIG_K = 32;
+constexpr int D_NBUF = 4, D_AHEAD = D_NBUF - 1;                  // stage s + D_AHEAD is loaded during stage s
+constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }      // s_waitcnt vmcnt(n) only
+constexpr int D_OPER = BIG_B * 64;
+constexpr int D_STAGE = 2 * D_OPER;
+constexpr int D_LDS = D_NBUF * D_STAGE;
+
+// The load itself is inline assembly: the compiler, which cannot tell that a load into one stage buffer does not alias a
+// ds_read from another, would otherwise wait for every outstanding load before each LDS read.  The waits are placed by
+// hand instead (one vmcnt per stage, below).  M0 carries the LDS byte address of the wave's 1 KB destination.
+__device__ __forceinline__ void load16_to_lds(const uint8_t *src, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+}
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_f16_direct_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
+                            size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave >> 1, wc = wave & 1;
+    const int half = lane >> 5, l32 = lane & 31;
+    const TileCoord tc = xcd_tile(blockIdx.x, map);
+    if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;
+    const int64_t row_base = (int64_t)tc.row_tile * BIG_B, tok_base = (int64_t)tc.tok_tile * BIG_B;
+    const int nst = (int)(K / BIG_K);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+
+    // loads: wave w fills rows 64 w .. 64 w + 63 of both operands, instruction j rows 64 w + 16 j + lane / 4
+    const int cell = (lane & 3) ^ ((lane >> 4) & 3);
+    const uint8_t *wsrc[4], *xsrc[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int r = 64 * wave + 16 * j + (lane >> 2);
+        wsrc[j] = W + (size_t)min(row_base + r, N - 1) * nb01 + 16 * cell;
+        xsrc[j] = ws + (size_t)min(tok_base + r, M - 1) * ws_stride + 16 * cell;
+    }
+    const uint32_t ld_dst = lds0 + 64 * wave * 64;                   // + 1024 j, + D_OPER for the activations
+    auto load_one = [&](int i, size_t k_off, uint32_t buf_off) {     // i = 0..3 weights, 4..7 activations
+        if (i < 4) load16_to_lds(wsrc[i] + k_off, __builtin_amdgcn_readfirstlane(ld_dst + buf_off + 1024 * i));
+        else load16_to_lds(xsrc[i - 4] + k_off, __builtin_amdgcn_readfirstlane(ld_dst + buf_off + D_OPER + 1024 * (i - 4)));
+    };
+    // reads: row wr * 128 + 32 a + l32 (the swizzle term of such a row is (l32 >> 2) & 3), cell 2 g + half
+    const int sw = (l32 >> 2) & 3;
+    int a_rd[2], b_rd[2];
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        a_rd[g] = (wr * 128 + l32) * 64 + (((2 * g + half) ^ sw) << 4);
+        b_rd[g] = D_OPER + (wc * 128 + l32) * 64 + (((2 * g + half) ^ sw) << 4);
+    }
+    auto get_a = [&](int a, int g, int buf_off) { return *reinterpret_cast<const f16x8 *>(lds + buf_off + a_rd[g] + 2048 * a); };
+    auto get_b = [&](int c, int g, int buf_off) { return *reinterpret_cast<const f16x8 *>(lds + buf_off + b_rd[g] + 2048 * c); };
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[a][c][v] = 0.f;
+
+#pragma unroll
+    for (int p = 0; p < D_AHEAD; p++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) load_one(i, (size_t)min(p, nst - 1) * (BIG_K * 2), p * D_STAGE);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    __syncthreads();
+    f16x8 af[2][4], bf[2][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++) { af[0][a] = get_a(a, 0, 0); bf[0][a] = get_b(a, 0, 0); }
+
+    int cur = 0, nxt = D_STAGE, fill = D_AHEAD * D_STAGE;            // buffers of stages s, s + 1, s + D_AHEAD
+    for (int s = 0; s < nst; s++) {
+        const size_t fill_k = (size_t)min(s + D_AHEAD, nst - 1) * (BIG_K * 2);
+        // k-group 0: after each of its first 8 MFMAs one operand read of k-group 1, after each of the other 8 one load of stage s + 2
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int a = i >> 2, c = i & 3;
+            acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[0][c], af[0][a], acc[a][c], 0, 0, 0);
+            if (i < 4) af[1][i] = get_a(i, 1, cur);
+            else if (i < 8) bf[1][i - 4] = get_b(i - 4, 1, cur);
+            else {
+                load_one(i - 8, fill_k, fill);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Stage s + 1 has landed once at most the loads of the D_AHEAD - 1 stages after it are outstanding.  The barrier
+        // makes every wave's share of it visible; it also separates the last reads of stage s's buffer, made just
+        // above, from the loads the next stage will aim at it.
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(8 * (D_AHEAD - 1)));
+        __syncthreads();
+        // k-group 1: after each of its first 8 MFMAs one operand read of k-group 0 of stage s + 1
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int a = i >> 2, c = i & 3;
+            acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][c], af[1][a], acc[a][c], 0, 0, 0);
+            if (i < 4) af[0][i] = get_a(i, 0, nxt);
+            else if (i < 8) bf[0][i - 4] = get_b(i - 4, 0, nxt);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        cur = nxt;
+        nxt = nxt + D_STAGE == D_LDS ? 0 : nxt + D_STAGE;
+        fill = fill + D_STAGE == D_LDS ? 0 : fill + D_STAGE;
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                       // the clamped loads of the last stages
+
+    // The tokens are the MFMA's first operand and the weight rows its second, so a lane holds one weight row and its 16
+    // registers 16 tokens: register v of tile (a, c) is token 8 (v / 4) + 4 half + v % 4, row l32.  A store instruction
+    // then writes 128 contiguous bytes of two token rows.
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+        const int64_t row = row_base + (wr * 4 + a) * 32 + l32;
+        if (row >= N) continue;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t tok = tok_base + (wc * 4 + c) * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+                if (tok < M) y[(size_t)tok * ldy + row] = acc[a][c][v];
+            }
+        }
+    }
+}
+
+static hipError_t launch_f16_direct(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
+                                    float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    static LdsGrant grant;
+    if (hipError_t e = grant_dynamic_lds(gemm_f16_direct_kernel, D_LDS, lim, grant); e != hipSuccess) return e;
+    const TileMap map = make_tile_map(ceil_div(N, BIG_B), ceil_div(M, BIG_B), 32);
+    hipLaunchKernelGGL(gemm_f16_direct_kernel, dim3(map.grid), dim3(256), D_LDS, st, (const uint8_t *)W, nb01, K, N,
+                       (const uint8_t *)ws, ws_stride, M, y, ldy, map);
+    return hipGetLastError();
+}
+
 // rows must be 16-byte aligned (the weight alignment rule of the C-ABI) and K a multiple of the 64-value stage
 bool gemm_f16_supported(int64_t K, int64_t N, int64_t n) { return K >= 64 && K % (16 * F16_KG) == 0 && N >= 1 && n >= 32; }
 
@@ -226,13 +379,14 @@ hipError_t launch_gemm_f16(const void *W, size_t nb01, int64_t K, int64_t N, con
         return launch_f16<1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     }
     if (f32_rows) return hipErrorInvalidValue;
-    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
-    const int cfg = (int)tune("CHIP_GEMM_F16_CFG", g128 >= cus ? 0 : 1);
+    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128), g256 = ceil_div(N, 256) * ceil_div(M, 256);
+    const int cfg = (int)tune("CHIP_GEMM_F16_CFG", 2 * g256 >= cus && K >= 4 * BIG_K && n_as == 1 ? 9 : g128 >= cus ? 0 : 1);
     switch (cfg) {
         case 0: return launch_f16<2, 2, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 128, 4 waves
         case 1: return launch_f16<1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 64 x 64, 4 waves
         case 2: return launch_f16<2, 2, 2, 4, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 256, 8 waves
         case 3: return launch_f16<2, 4, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);       // 128 x 256, 4 waves
+        case 9: return launch_f16_direct(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st);                             // 256 x 256, 4 waves, direct to LDS
         default: return hipErrorInvalidValue;
     }
 }

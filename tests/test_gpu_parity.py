@@ -438,6 +438,34 @@ def test_gemm_f16_vs_oracle(dev, orc, K, N, n):
     check_outputs(y, ref["y"], ref["sum_abs"], "f16 gemm")
 
 
+@pytest.mark.parametrize("K,N,n", [(256, 4096, 2048), (512, 3841, 2305), (768, 8200, 1025)])
+def test_gemm_f16_large_shape_kernel_vs_oracle(dev, orc, K, N, n):
+    """Shapes with at least one 256 x 256 output tile for every second CU take the large-tile kernel (operands loaded
+    straight into LDS): whole and ragged edge tiles in both directions, a K loop shorter and longer than its pipeline."""
+    print("gemm f16 large K", K, "N", N, "n", n, flush=True)
+    assert -(-N // 256) * -(-n // 256) * 2 >= 256
+    wq = orc.quantize_weights(O.F16, common.weights_f32(K + N, N, K, outliers=True))
+    x = common.activations_f32(K + n, n, K)
+    x[3] = 0
+    y = dev.mul_mat(O.F16, wq, x)
+    rng = np.random.default_rng(K)
+    rows = np.unique(np.concatenate([[0, 1, 255, 256, N - 257, N - 2, N - 1], rng.choice(N, 160, replace=False)]))
+    toks = np.unique(np.concatenate([[0, 3, 255, 256, n - 257, n - 2, n - 1], rng.choice(n, 40, replace=False)]))
+    ref = orc.mul_mat(O.F16, wq[rows], x[toks], nthreads=8, want=("sum_abs",))
+    check_outputs(y[np.ix_(toks, rows)], ref["y"], ref["sum_abs"], "f16 large-shape gemm")
+    assert np.isfinite(y).all() and not y[3].any()
+
+
+def test_gemm_f16_large_shape_kernel_exact_small_integers(dev):
+    """Every output of the large-tile kernel, not a sample: integer operands whose dot products fp32 holds exactly."""
+    K, N, n = 512, 4100, 2050
+    rng = np.random.default_rng(4)
+    w = rng.integers(-32, 33, (N, K)).astype(np.float32)
+    x = rng.integers(-32, 33, (n, K)).astype(np.float32)
+    y = dev.mul_mat(O.F16, w.astype(np.float16).view(np.uint8).reshape(N, -1), x)
+    assert np.array_equal(y, x @ w.T)
+
+
 def test_f16_rows_of_k_not_a_multiple_of_256_are_rejected(dev):
     """F16 weights (like the K-quants) are taken in rows of K % 256 == 0 only: the C-ABI says so instead of computing."""
     K, N, n = 64, 70, 40
