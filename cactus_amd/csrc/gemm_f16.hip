@@ -208,6 +208,10 @@ void gemm_f16_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int6
 // loads that always hit the cache cost the same; half as many loads cost half) but about 37 clocks of the issuing wave
 // per 1 KB written to LDS - the same as a ds_write_b128 of register-staged data costs, while plain global loads into
 // registers cost nothing.  With all 256 CUs busy a tile takes 1.2 - 1.3 times longer (clock under load).
+// Tried and dropped: the same tile with register staging and ds_write_b128 (111 us per tile: the waits for the loads on
+// top of the write cost); a fifth stage buffer (no change); the token operands loaded by each wave from global memory
+// straight into registers in MFMA layout, only the weights through LDS (154 us per tile: 32 rows x 32 bytes per load
+// instruction is far slower through the texture path than it is cheap to issue).
 constexpr int BIG_B = 256, BIG_K = 32;
 constexpr int D_NBUF = 4, D_AHEAD = D_NBUF - 1;                  // stage s + D_AHEAD is loaded during stage s
 constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }      // s_waitcnt vmcnt(n) only
