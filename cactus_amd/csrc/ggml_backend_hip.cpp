@@ -25,7 +25,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -666,12 +666,16 @@ bool ranges_apart(const lm_ggml_tensor *p, const lm_ggml_tensor *q) {
     return disjoint(p, q);
 }
 template <typename F>
-int early_store_index(const lm_ggml_cgraph *g, int i, F wanted) {
+int early_store_index(const lm_ggml_cgraph *g, int i, F wanted, int run_at = -1) {
+    // run_at: the node at whose place the producer i itself runs (a projection grouped with an earlier one); the
+    // destination must stay untouched from there on
+    const int first = (run_at >= 0 ? run_at : i) + 1;
     const int end = i + 1 + STORE_LOOKAHEAD < g->n_nodes ? i + 1 + STORE_LOOKAHEAD : g->n_nodes;
     for (int j = i + 1; j < end; j++) {
         const lm_ggml_tensor *cp = g->nodes[j];
         if (cp->op != LM_GGML_OP_CPY || !wanted(cp)) continue;
-        for (int m = i + 1; m < j; m++) {
+        for (int m = first; m < j; m++) {
+            if (m == i) continue;
             const lm_ggml_tensor *t = g->nodes[m];
             if (is_view_op(t->op)) continue;
             if (!ranges_apart(t, cp)) return -1;
@@ -714,7 +718,7 @@ int paired_matmul_index(const lm_ggml_cgraph *g, int i) {
 // The V projection followed (views aside) by the CPY of its transpose into the transposed F16 V cache (reference
 // llama-kv-cache.cpp cpy_v without flash attention: dst is a 2-D view [n_tokens, n_embd_v] with rows kv_size apart).
 // Index of that CPY node, or -1.  The matmul still writes its own F32 result.
-int transposed_store_index(const lm_ggml_cgraph *g, int i) {
+int transposed_store_index(const lm_ggml_cgraph *g, int i, int run_at = -1) {
     const lm_ggml_tensor *mm = g->nodes[i];
     const int64_t N = mm->ne[0], n = mm->ne[1];
     return early_store_index(g, i, [mm, N, n](const lm_ggml_tensor *cp) {
@@ -727,7 +731,36 @@ int transposed_store_index(const lm_ggml_cgraph *g, int i) {
             return false;
         if (!is_hip_buffer(cp->view_src ? cp->view_src->buffer : cp->buffer)) return false;
         return disjoint(cp, mm) && disjoint(cp, mm->src[1]);
-    });
+    }, run_at);
+}
+
+// The projections of one activation tensor (llama.cpp builds Qcur, its RoPE, Kcur, its RoPE, Vcur, ... from the same
+// normed input: llama-model.cpp build_llama): MUL_MAT nodes within the next GROUP_LOOKAHEAD nodes after i that read the
+// same src[1] as node i and share its activation format.  Such a node may run at node i's place when nothing between the
+// two reads or writes the memory of its result (the allocator may have given it the place of a tensor that dies in
+// between, Qcur's for instance once its RoPE has read it).  Fills members[] (node i first) and returns their number.
+constexpr int GROUP_LOOKAHEAD = 12;
+int grouped_matmuls(const lm_ggml_cgraph *g, int i, int *members) {
+    const lm_ggml_tensor *first = g->nodes[i], *x = first->src[1];
+    const int vt = chip_vec_dot_type(first->src[0]->type);
+    int count = 0;
+    members[count++] = i;
+    const int end = i + 1 + GROUP_LOOKAHEAD < g->n_nodes ? i + 1 + GROUP_LOOKAHEAD : g->n_nodes;
+    for (int j = i + 1; j < end && count < CHIP_GROUP_MAX; j++) {
+        const lm_ggml_tensor *mm = g->nodes[j];
+        if (mm->op != LM_GGML_OP_MUL_MAT || mm->src[1] != x || !mul_mat_shape_ok(mm)) continue;
+        if (chip_vec_dot_type(mm->src[0]->type) != vt || !disjoint(mm, x)) continue;
+        bool safe = true;
+        for (int m = i; m < j && safe; m++) {
+            const lm_ggml_tensor *t = g->nodes[m];
+            if (is_view_op(t->op)) continue;
+            if (!ranges_apart(t, mm)) safe = false;
+            for (int k = 0; k < LM_GGML_MAX_SRC && safe; k++)
+                if (t->src[k] && !ranges_apart(t->src[k], mm)) safe = false;
+        }
+        if (safe) members[count++] = j;
+    }
+    return count;
 }
 
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
@@ -742,6 +775,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         return false;
     };
     int paired_matmul = -1;                           // index of an up projection that ran with its gate projection
+    int grouped[CHIP_GROUP_MAX] = {-1, -1, -1, -1};   // projections that already ran with an earlier one of the same input
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -887,6 +921,12 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: node %d (%s, op %d) is not supported by the HIP backend\n", __func__, i, node->name, node->op);
             return LM_GGML_STATUS_FAILED;
         }
+        {
+            bool done = false;
+            for (int &slot : grouped)
+                if (slot == i) { slot = -1; done = true; }
+            if (done) continue;
+        }
         const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
         const int64_t K = w->ne[0], N = w->ne[1], n = x->ne[1];
         if (N == 0 || n == 0) continue;
@@ -894,6 +934,51 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         int rc;
         const int64_t ldx = (int64_t)(x->nb[1] / 4);
         int store_t = -1;
+        int members[CHIP_GROUP_MAX];
+        int n_members = 1;
+        if (n <= 4 && fusion_enabled()) {
+            bool slots_free = true;
+            for (int slot : grouped) slots_free = slots_free && slot < 0;
+            if (slots_free) n_members = grouped_matmuls(cgraph, i, members);
+        }
+        if (n_members >= 2) {
+            chip_mat mats[CHIP_GROUP_MAX];
+            bool fits = true;
+            int stores = 0;
+            for (int k = 0; k < n_members; k++) fits = fits && cgraph->nodes[members[k]]->src[0]->ne[1] > 0;
+            for (int k = 0; fits && k < n_members; k++) {
+                lm_ggml_tensor *mm = cgraph->nodes[members[k]];
+                const lm_ggml_tensor *mw = mm->src[0];
+                mats[k] = chip_mat{(int)mw->type, mw->data, mw->nb[1], mw->ne[1], (float *)mm->data, (int64_t)(mm->nb[1] / 4), nullptr, 0};
+                if (!grow_workspace(c, chip_mul_mat_workspace_size_n(mw->type, K, mw->ne[1], n))) return LM_GGML_STATUS_ALLOC_FAILED;
+                const int st = transposed_store_index(cgraph, members[k], i);
+                if (st >= 0 && remember_store(st)) {
+                    lm_ggml_tensor *cp = cgraph->nodes[st];
+                    writes(cp);
+                    mats[k].y_f16_t = (uint16_t *)cp->data;
+                    mats[k].ld16 = (int64_t)(cp->nb[1] / 2);
+                    stores++;
+                }
+            }
+            if (fits) {
+                for (int k = 1; k < n_members; k++) {
+                    writes(cgraph->nodes[members[k]]);
+                    grouped[k] = members[k];
+                }
+                c->quantized.valid = false;
+                rc = chip_mul_mat_group(mats, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                if (rc != CHIP_OK) {
+                    HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT group of %d at %s failed: %s\n", __func__, n_members, node->name,
+                            chip_error_string(rc));
+                    return LM_GGML_STATUS_FAILED;
+                }
+                g_mul_mat_nodes += n_members;
+                g_grouped_matmuls += n_members;
+                g_elementwise_nodes += stores;
+                g_fused_pairs += n_members - 1 + stores;
+                continue;
+            }
+        }
         if (n <= 4 && fusion_enabled() && (store_t = transposed_store_index(cgraph, i)) >= 0 && remember_store(store_t)) {
             lm_ggml_tensor *cp = cgraph->nodes[store_t];
             writes(cp);
@@ -1052,6 +1137,7 @@ void *reg_get_proc_address(lm_ggml_backend_reg_t, const char *name) {
     if (std::strcmp(name, "lm_ggml_backend_hip_get_quantizers_skipped") == 0) return (void *)lm_ggml_backend_hip_get_quantizers_skipped;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_rope_tables") == 0) return (void *)lm_ggml_backend_hip_get_rope_tables;
     if (std::strcmp(name, "lm_ggml_backend_hip_get_async_uploaded") == 0) return (void *)lm_ggml_backend_hip_get_async_uploaded;
+    if (std::strcmp(name, "lm_ggml_backend_hip_get_grouped_matmuls") == 0) return (void *)lm_ggml_backend_hip_get_grouped_matmuls;
     return nullptr;         // no n_threads, no extra buffer types, no split buffer type, no feature list
 }
 const lm_ggml_backend_reg_i k_reg_i = {reg_name, reg_device_count, reg_get_device, reg_get_proc_address};
@@ -1115,5 +1201,6 @@ unsigned long long lm_ggml_backend_hip_get_fused_pairs(void) { return g_fused_pa
 unsigned long long lm_ggml_backend_hip_get_quantizers_skipped(void) { return g_quantizers_skipped.load(); }
 unsigned long long lm_ggml_backend_hip_get_rope_tables(void) { return g_rope_tables.load(); }
 unsigned long long lm_ggml_backend_hip_get_async_uploaded(void) { return g_uploaded_async.load(); }
+unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void) { return g_grouped_matmuls.load(); }
 
 }  // extern "C"

@@ -52,6 +52,9 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_tables(void);
 /* Bytes that arrived through set_tensor_async (the model loader's pinned-staging upload loop,
  * cactus/llama-model-loader.cpp:1047-1064); a subset of uploaded_bytes above. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_async_uploaded(void);
+/* MUL_MAT nodes that ran in one launch with other projections of the same activation tensor (Qcur / Kcur / Vcur of an
+ * attention block, cactus/llama-model.cpp build_llama), up to 4 tokens. */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void);
 
 #ifdef __cplusplus
 }

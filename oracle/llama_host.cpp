@@ -233,10 +233,11 @@ int run(int argc, char **argv) {
         typedef unsigned long long (*count_fn)(void);
         stats_fn stats = (stats_fn)lm_ggml_backend_reg_get_proc_address(reg, "lm_ggml_backend_hip_get_stats");
         count_fn async_up = (count_fn)lm_ggml_backend_reg_get_proc_address(reg, "lm_ggml_backend_hip_get_async_uploaded");
+        count_fn grouped = (count_fn)lm_ggml_backend_reg_get_proc_address(reg, "lm_ggml_backend_hip_get_grouped_matmuls");
         unsigned long long nodes = 0, uploaded = 0;
         if (stats) stats(&nodes, &uploaded);
-        std::printf("stat mul_mat_nodes %llu\nstat uploaded_bytes %llu\nstat async_uploaded_bytes %llu\n", nodes, uploaded,
-                    async_up ? async_up() : 0ull);
+        std::printf("stat mul_mat_nodes %llu\nstat uploaded_bytes %llu\nstat async_uploaded_bytes %llu\nstat grouped_matmuls %llu\n", nodes,
+                    uploaded, async_up ? async_up() : 0ull, grouped ? grouped() : 0ull);
     }
     cactus_free_context_c(handle);
     std::printf("stat bench_ok %d\nstat completion_ok %d\n", (int)bench_ok, (int)completion_ok);
