@@ -567,7 +567,9 @@ static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, 
             return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, slices, split.part);
     }
     // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
-    // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)
+    // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)  Larger per-wave tiles
+    // with fewer waves per SIMD measured slower on 14336 x 4096 x 2048 (Q4_0): 2 x 2 tiles at two waves 449 us against
+    // 447, 4 x 2 and 2 x 4 at one wave 719 and 667 us: the scaling work is vector-bound and wants waves, not tiles.
     if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
         return launch_cfg<WT, 1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
     const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
@@ -577,6 +579,7 @@ static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, 
         case 1: return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
         default: return hipErrorInvalidValue;
     }
+    return hipErrorInvalidValue;
 }
 
 int gemm_blk32_slices(int wtype, int64_t K, int64_t N, int64_t n, int compute_units) {

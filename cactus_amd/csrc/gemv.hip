@@ -79,14 +79,19 @@ static hipError_t launch_one(const void *W, size_t nb01, int64_t K, int64_t N, c
     return launch_depth<WT, NTOK, R, WGS, FUSEQ, GEMV_DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, max_groups, lim, st, sec);
 }
 
-template <int WT, int NTOK, bool FUSEQ>
+template <int WT, int NTOK, bool FUSEQ, int R = RowsPerWave<WT>::R>
 static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
                                size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st,
                                const SecondMatrix &sec = kNoSecond) {
     const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
-    constexpr int R = RowsPerWave<WT>::R;
+    if constexpr (R == 2 && NTOK == 1) {
+        // Two rows per step halve the tiles: a matrix with no more rows than the device has wave slots (16 per CU) would
+        // leave half of them without work, one step each for the others.  One row per step there.
+        if (tune("CHIP_GEMV_R1_SMALL", 1) != 0 && N <= 16 * (int64_t)cus)
+            return launch_typed<WT, NTOK, FUSEQ, 1>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+    }
     // The activation prologue (staging, or quantizing in the fused variant) is paid once per workgroup, so the
     // grid is persistent: one or two 8-wave groups per CU, each wave striding over the row tiles.  Matrices with
     // too few rows to give every CU an 8-wave group use 4-wave groups instead.
@@ -102,6 +107,11 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         const bool long_q8_0_row = Traits<WT>::ACT == T_Q8_0 && NTOK == 1 && K > 8192;
         if (one_tile_per_wave && !long_q8_0_row)
             return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
+    }
+    if constexpr (!FUSEQ && NTOK == 1) {
+        const bool one_tile_per_wave = tiles <= 16 * (int64_t)cus && tiles > 8 * (int64_t)cus;
+        if (tune("CHIP_GEMV_STAGED_WIDE", 0) != 0 && one_tile_per_wave)
+            return launch_one<WT, NTOK, R, 1024, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
     }
     if constexpr (FUSEQ && NTOK >= 2) {
         // A narrow matrix (fewer than 8 tiles per CU) is all prologue: every workgroup quantizes NTOK rows before its
