@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
@@ -108,6 +108,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_workspace_size_n.argtypes = [i32, i64, i64, i64]
     L.chip_mul_mat.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_group.argtypes = [C.POINTER(Mat), i32, i64, vp, i64, i64, vp, sz, vp]
+    L.chip_mul_mat_group_run.argtypes = [C.POINTER(Mat), i32, i64, i64, vp, sz, vp]
     L.chip_mul_mat_noalloc.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp]
     L.chip_mul_mat_noalloc_max_workspace.restype = sz
     L.chip_mul_mat_noalloc_max_workspace.argtypes = []
@@ -269,10 +270,11 @@ class Device:
         self.sync()
         return dy.download(np.float32, n * N).reshape(n, N), dh.download(np.uint16, N * ld16).reshape(N, ld16)
 
-    def mul_mat_group(self, members, x, ld16=0):
+    def mul_mat_group(self, members, x, ld16=0, prepared=False):
         """chip_mul_mat_group: members = [(wtype, W uint8 [N, row_size]), ...] on the activation rows x fp32 [n, K].
         Returns a list of y fp32 [n, N]; with ld16 > 0 the last member also stores its transposed fp16 copy and the list
-        ends with that matrix [N, ld16] (untouched columns keep 0x7bff)."""
+        ends with that matrix [N, ld16] (untouched columns keep 0x7bff).  prepared: chip_mul_mat_prepare first, then
+        chip_mul_mat_group_run over the workspace rows."""
         x = np.ascontiguousarray(x, np.float32)
         n, k = x.shape
         dx = self.to_device(x)
@@ -293,7 +295,11 @@ class Device:
             arr[len(members) - 1].y_f16_t = dh.ptr
             arr[len(members) - 1].ld16 = ld16
         ws = self.alloc(wsz)
-        self.check(self.lib.chip_mul_mat_group(arr, len(members), k, dx.ptr, k, n, ws.ptr, wsz, None))
+        if prepared:
+            self.check(self.lib.chip_mul_mat_prepare(members[0][0], k, dx.ptr, k, n, ws.ptr, wsz, None))
+            self.check(self.lib.chip_mul_mat_group_run(arr, len(members), k, n, ws.ptr, wsz, None))
+        else:
+            self.check(self.lib.chip_mul_mat_group(arr, len(members), k, dx.ptr, k, n, ws.ptr, wsz, None))
         self.sync()
         res = [dy.download(np.float32, n * N).reshape(n, N) for dy, N in outs]
         if dh is not None:

@@ -463,8 +463,9 @@ int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int
 
 // Several matmuls on one activation (wq / wk / wv).  Up to 4 tokens, members of one family: one launch of the
 // prologue-quantizing GEMV over all members; otherwise one quantizer and each member on its usual path.
-int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
-                       size_t workspace_bytes, void *stream) {
+// what chip_mul_mat_group and chip_mul_mat_group_run share: x == nullptr says the workspace already holds the rows
+static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
+                         size_t workspace_bytes, void *stream) {
     if (count < 0 || n < 0) return CHIP_EINVAL;
     if (count == 0 || n == 0) return CHIP_OK;
     if (!mats || count > CHIP_GROUP_MAX) return CHIP_EINVAL;
@@ -484,7 +485,9 @@ int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *
         const size_t w = chip_mul_mat_workspace_size(m.type, K, n);
         if (w > need) need = w;
     }
-    if (!x || !workspace || ldx < K || !aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace)) return CHIP_EINVAL;
+    const bool prepared = x == nullptr;
+    if (!workspace || !aligned16(workspace)) return CHIP_EINVAL;
+    if (!prepared && (ldx < K || !aligned16(x) || (ldx % 4) != 0)) return CHIP_EINVAL;
     if (workspace_bytes < need) return CHIP_ENOMEM;
     DeviceLimits lim;
     if (int rc = current_limits(lim); rc) return rc;
@@ -494,10 +497,27 @@ int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *
         if (mats[i].N > 0)
             gm[live++] = GroupMat{mats[i].type, mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].y_f16_t, mats[i].ld16};
     if (live == 0) return CHIP_OK;
-    if (n <= 4 && gemv_group_applicable(gm, live, K, (int)n, lim))
-        return hip_rc(launch_gemv_group(gm, live, K, x, ldx, (int)n, workspace, act_stride(at, K), lim, (hipStream_t)stream));
+    const size_t stride = act_stride(at, K);
+    hipStream_t st = (hipStream_t)stream;
+    // Up to 4 tokens.  One member, or two of one type, shape and row stride, take the single-matrix kernel (it keeps more
+    // waves per SIMD than the group kernel, whose register count is that of its most demanding member type): a pair runs
+    // as one matrix of twice the rows, a member with a transposed fp16 copy as chip_mul_mat_store_t does.
+    if (n <= 4 && gemv_group_applicable(gm, live, K, (int)n, lim, prepared)) {
+        const GroupMat &a = gm[0], &b = gm[live - 1];
+        if (live == 1 && a.t16)
+            return hip_rc(prepared ? launch_gemv_store_t(a.wtype, a.W, a.nb01, K, a.N, workspace, stride, (int)n, a.y, a.ldy, a.t16, a.t16_ld, lim, st)
+                                   : launch_gemv_fused_store_t(a.wtype, a.W, a.nb01, K, a.N, x, ldx, (int)n, workspace, stride, a.y, a.ldy, a.t16, a.t16_ld, lim, st));
+        if (live == 1)
+            return hip_rc(prepared ? launch_gemv(a.wtype, a.W, a.nb01, K, a.N, workspace, stride, (int)n, a.y, a.ldy, lim, st)
+                                   : launch_gemv_fused(a.wtype, a.W, a.nb01, K, a.N, x, ldx, (int)n, workspace, stride, a.y, a.ldy, lim, st));
+        if (live == 2 && a.wtype == b.wtype && a.N == b.N && a.nb01 == b.nb01 && a.ldy == b.ldy && !a.t16 && !b.t16 && 2 * a.N <= 0x7fffffff)
+            return hip_rc(prepared ? launch_gemv_pair(a.wtype, a.W, b.W, a.nb01, K, a.N, workspace, stride, (int)n, a.y, b.y, a.ldy, lim, st)
+                                   : launch_gemv_fused_pair(a.wtype, a.W, b.W, a.nb01, K, a.N, x, ldx, (int)n, workspace, stride, a.y, b.y, a.ldy, lim, st));
+        return hip_rc(launch_gemv_group(gm, live, K, x, ldx, (int)n, workspace, stride, lim, st, prepared));
+    }
     // more tokens, or members the one-launch form does not take: quantize once, then every member as chip_mul_mat_run would
-    if (int rc = chip_mul_mat_prepare(mats[0].type, K, x, ldx, n, workspace, workspace_bytes, stream); rc) return rc;
+    if (!prepared)
+        if (int rc = chip_mul_mat_prepare(mats[0].type, K, x, ldx, n, workspace, workspace_bytes, stream); rc) return rc;
     for (int i = 0; i < live; i++) {
         const GroupMat &m = gm[i];
         if (int rc = mul_mat_run(m.wtype, m.W, m.nb01, K, m.N, n, workspace, workspace_bytes, m.y, m.ldy, stream); rc) return rc;
@@ -508,6 +528,14 @@ int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *
         }
     }
     return CHIP_OK;
+}
+int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
+                       size_t workspace_bytes, void *stream) {
+    if (count > 0 && n > 0 && !x) return CHIP_EINVAL;
+    return mul_mat_group(mats, count, K, x, ldx, n, workspace, workspace_bytes, stream);
+}
+int chip_mul_mat_group_run(const chip_mat *mats, int count, int64_t K, int64_t n, void *workspace, size_t workspace_bytes, void *stream) {
+    return mul_mat_group(mats, count, K, nullptr, 0, n, workspace, workspace_bytes, stream);
 }
 
 // A matmul whose result is also stored transposed as fp16 (the V projection and the store into the transposed F16 V cache).

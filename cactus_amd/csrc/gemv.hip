@@ -185,6 +185,37 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
     }
 }
 
+// The GEMV over prepared rows with a second matrix behind the first (sec.split rows in) or a transposed fp16 copy of the
+// result (sec.t16): what launch_gemv_fused_pair / _store_t do, without the quantizer in the prologue.
+hipError_t launch_gemv_sec(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
+                           float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const SecondMatrix &sec) {
+    if (N <= 0 || n <= 0) return hipSuccess;
+    void *w = const_cast<void *>(ws);
+    switch (wtype) {
+        case T_Q4_0: return launch_ntok<T_Q4_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q8_0: return launch_ntok<T_Q8_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q4_K: return launch_ntok<T_Q4_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q6_K: return launch_ntok<T_Q6_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q5_0: return launch_ntok<T_Q5_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_IQ4_NL: return launch_ntok<T_IQ4_NL, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q4_1: return launch_ntok<T_Q4_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q5_1: return launch_ntok<T_Q5_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_F16: return launch_ntok<T_F16, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        default: return hipErrorInvalidValue;
+    }
+}
+hipError_t launch_gemv_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                            int n, float *y1, float *y2, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+    const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, (int64_t)(y2 - y1) - N, nullptr, 0};
+    return launch_gemv_sec(wtype, W1, nb01, K, 2 * N, ws, ws_stride, n, y1, ldy, lim, st, sec);
+}
+hipError_t launch_gemv_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
+                               float *y, int64_t ldy, unsigned short *y16t, int64_t ld16, const DeviceLimits &lim, hipStream_t st) {
+    const SecondMatrix sec{INT64_MAX, 0, 0, y16t, ld16};
+    return launch_gemv_sec(wtype, W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st, sec);
+}
+
 // One launch for the whole op: quantize in the prologue.  Worth it while a workgroup's share of that work stays
 // small: n * K <= 16384 values (64 KB of fp32 per workgroup) and n in {1, 2, 4}.
 bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {

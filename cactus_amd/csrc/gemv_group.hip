@@ -17,15 +17,17 @@ struct GroupKernelMat {
 };
 struct GroupKernelArgs { GroupKernelMat m[GROUP_MAX]; int count; };
 
-template <int WT, int NTOK, int WGS, int DEPTH>
+template <int WT, int NTOK, int WGS, bool FUSEQ, int DEPTH>
 __device__ __forceinline__ void run_member(const GroupKernelMat &m, int64_t K, const float *x, int64_t ldx, uint8_t *ws,
                                            size_t ws_stride, const GridPart gp) {
     const SecondMatrix sec{INT64_MAX, 0, 0, m.t16, m.t16_ld};
-    gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, true, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
+    gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
 }
 
 // FAMILY 0: K-quants (Q8_K activations); 1: 32-value blocks (Q8_0 / Q8_1 planes); 2: F16.
-template <int FAMILY, int NTOK, int WGS, int DEPTH>
+// FUSEQ: the workgroups quantize the fp32 rows x themselves; otherwise the workspace already holds the quantized rows
+// (written by chip_mul_mat_prepare or by the kernel that produced the activations) and is only read.
+template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH>
 __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs ga, int64_t K, const float *__restrict__ x,
                                                          int64_t ldx, uint8_t *__restrict__ ws, size_t ws_stride) {
     int i = 0;
@@ -34,24 +36,24 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
         if (j < ga.count && (int)blockIdx.x >= ga.m[j].first_block) i = j;
     const GroupKernelMat &m = ga.m[i];
     const int last = (i + 1 < ga.count) ? ga.m[i + 1].first_block : (int)gridDim.x;
-    const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), blockIdx.x == 0};
+    const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), FUSEQ && blockIdx.x == 0};
     if constexpr (FAMILY == 0) {
         switch (m.wtype) {                                              // uniform over the workgroup
-            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            default:     run_member<T_Q6_K, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else if constexpr (FAMILY == 1) {
         switch (m.wtype) {
-            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            default:       run_member<T_Q8_0, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else {
-        run_member<T_F16, NTOK, WGS, DEPTH>(m, K, x, ldx, ws, ws_stride, gp);
+        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp);
     }
 }
 
@@ -72,10 +74,10 @@ size_t image_bytes(int wtype, int64_t K) {
 }
 int rows_per_step(int wtype) { return wtype == T_Q4_0 ? RowsPerWave<T_Q4_0>::R : 1; }
 
-template <int FAMILY, int NTOK, int WGS, int DEPTH>
+template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH>
 hipError_t launch_depth(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
                         size_t lds_bytes, const DeviceLimits &lim, hipStream_t st) {
-    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, DEPTH>;
+    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, FUSEQ, DEPTH>;
     static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(WGS), lds_bytes, st, ga, K, x, ldx, (uint8_t *)ws, ws_stride);
@@ -83,22 +85,23 @@ hipError_t launch_depth(const GroupKernelArgs &ga, int grid, int64_t K, const fl
 }
 template <int FAMILY, int NTOK, int WGS>
 hipError_t launch_cfg(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
-                      size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool) {
-    return launch_depth<FAMILY, NTOK, WGS, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
+                      size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared) {
+    return prepared ? launch_depth<FAMILY, NTOK, WGS, false, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st)
+                    : launch_depth<FAMILY, NTOK, WGS, true, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
 }
 template <int FAMILY, int NTOK>
 hipError_t launch_wgs(int wgs, const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws,
-                      size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool deep) {
-    return wgs == 1024 ? launch_cfg<FAMILY, NTOK, 1024>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep)
-                       : launch_cfg<FAMILY, NTOK, 512>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+                      size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared) {
+    return wgs == 1024 ? launch_cfg<FAMILY, NTOK, 1024>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared)
+                       : launch_cfg<FAMILY, NTOK, 512>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
 }
 template <int FAMILY>
 hipError_t launch_ntok(int n, int wgs, const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws,
-                       size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool deep) {
+                       size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared) {
     switch (n) {
-        case 1: return launch_wgs<FAMILY, 1>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
-        case 2: return launch_wgs<FAMILY, 2>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
-        case 4: return launch_wgs<FAMILY, 4>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        case 1: return launch_wgs<FAMILY, 1>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        case 2: return launch_wgs<FAMILY, 2>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        case 4: return launch_wgs<FAMILY, 4>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
         default: return hipErrorInvalidValue;
     }
 }
@@ -116,13 +119,18 @@ int gemv_group_family(int wtype) {
 
 // One launch serves the group when the prologue-quantizing GEMV takes every member (n in {1, 2, 4}, n * K within its
 // limit, the largest member's activation image within LDS) and the members are of one family.
-bool gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim) {
+bool gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim, bool prepared) {
     if (count < 1 || count > GROUP_MAX) return false;
+    if (n != 1 && n != 2 && n != 4) return false;
     const int fam = gemv_group_family(mats[0].wtype);
     if (fam < 0) return false;
     int64_t rows = 0;
     for (int i = 0; i < count; i++) {
-        if (gemv_group_family(mats[i].wtype) != fam || !gemv_fused_applicable(mats[i].wtype, K, n, lim)) return false;
+        if (gemv_group_family(mats[i].wtype) != fam) return false;
+        // over prepared rows the only limit is the activation image of n rows in LDS; quantizing in the prologue has its own
+        if (prepared ? (size_t)n * image_bytes(mats[i].wtype, K) > (size_t)lim.max_lds_per_block || image_bytes(mats[i].wtype, K) == 0
+                     : !gemv_fused_applicable(mats[i].wtype, K, n, lim))
+            return false;
         if (mats[i].N <= 0 || mats[i].N > 0x7fffffff) return false;
         rows += mats[i].N;
     }
@@ -131,8 +139,8 @@ bool gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, co
 }
 
 hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const float *x, int64_t ldx, int n, void *ws,
-                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st) {
-    if (!gemv_group_applicable(mats, count, K, n, lim)) return hipErrorInvalidValue;
+                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st, bool prepared) {
+    if (!gemv_group_applicable(mats, count, K, n, lim, prepared)) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     const int fam = gemv_group_family(mats[0].wtype);
     size_t img = 0;
@@ -150,7 +158,9 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
     // As the single-matrix launcher: a persistent grid; one 16-wave workgroup per CU while every wave gets at most a
     // couple of tiles (the prologue is then most of the kernel and is paid once per CU), else two 8-wave workgroups.
     const int wgs = tiles <= 32 * (int64_t)cus ? 1024 : 512;
-    const int per_cu = (wgs == 1024 || lds_bytes > 24 * 1024) ? 1 : (n == 1 ? 3 : 2);
+    // the K-quant and block-32 kernels keep 4 - 5 waves per SIMD (the registers of their most demanding member type): two
+    // 8-wave workgroups per CU; the F16 kernel keeps 8 and takes three for one token
+    const int per_cu = (wgs == 1024 || lds_bytes > 24 * 1024) ? 1 : (fam == 2 && n == 1 && !prepared ? 3 : 2);
     int grid = cus * per_cu;
     const int64_t max_useful = ceil_div(tiles, (int64_t)(wgs / 64));
     if (grid > max_useful) grid = (int)max_useful;
@@ -184,11 +194,10 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
                                  mats[i].t16_ld, mats[i].wtype, first};
         first += blocks[i];
     }
-    const bool deep = tiles > (int64_t)first * (wgs / 64);              // some wave walks two or more tiles
     switch (fam) {
-        case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
-        case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
-        default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, deep);
+        case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
     }
 }
 

@@ -158,9 +158,14 @@ hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, siz
 constexpr int GROUP_MAX = 4;
 struct GroupMat { int wtype; const void *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld; };
 int        gemv_group_family(int wtype);
-bool       gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim);
+bool       gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim, bool prepared = false);
+// the GEMV over prepared rows for two matrices of one shape in one launch, and with a transposed fp16 copy of the result
+hipError_t launch_gemv_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
+                            int n, float *y1, float *y2, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+hipError_t launch_gemv_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
+                               float *y, int64_t ldy, unsigned short *y16t, int64_t ld16, const DeviceLimits &lim, hipStream_t st);
 hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const float *x, int64_t ldx, int n, void *ws,
-                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st);
+                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st, bool prepared = false);
 // MUL_MAT_ID: every (token, slot) pair is a one-token GEMV on the expert ids[token][slot] names (W + id * nb02), its
 // activation row token * ne11 + slot % ne11, its output row token * n_used + slot.  fused: x is fp32 and is quantized in
 // the prologue; otherwise ws already holds the quantized rows.

@@ -179,6 +179,13 @@ typedef struct chip_mat {
 } chip_mat;
 CHIP_API int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n,
                                 void *workspace, size_t workspace_bytes, void *stream);
+/* The same over rows the workspace already holds - Phase B of the op alone (ggml-cpu/ggml-cpu.c:1380-1448) for a group, as
+ * chip_mul_mat_run is for one matrix: the rows were written by chip_mul_mat_prepare or by the kernel that produced the
+ * activations (chip_rms_norm_quantized, chip_silu_mul_quantized).  Up to 4 tokens and members of one family: one launch of
+ * the GEMV that stages the rows from the workspace; any row length the activation image of n rows fits in LDS for.  Every
+ * output equals, bit for bit, chip_mul_mat_run's for that member (and the fp16 store of chip_mul_mat_store_t). */
+CHIP_API int chip_mul_mat_group_run(const chip_mat *mats, int count, int64_t K, int64_t n, void *workspace,
+                                    size_t workspace_bytes, void *stream);
 /* chip_mul_mat whose result also goes, rounded to fp16 (nearest even), to y_f16_t[row * ld16 + token]: the V projection
  * and its store into the transposed F16 V cache (llama-kv-cache.cpp cpy_v without flash attention) - one launch up to 4
  * tokens, otherwise the matmul followed by the copy.  Results as from chip_mul_mat and chip_cpy. */

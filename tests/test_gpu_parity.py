@@ -726,6 +726,27 @@ def test_mul_mat_group_equals_single_calls(dev, orc, members, K):
         check_outputs(ys[0], ref["y"], ref["sum_abs"], "group member 0, n = %d" % n)
 
 
+@pytest.mark.parametrize("members", [
+    ((O.Q4_K, 1100), (O.Q4_K, 256), (O.Q6_K, 260)),
+    ((O.Q4_0, 700), (O.Q8_0, 300), (O.Q5_1, 130)),
+    ((O.Q6_K, 2000),),
+], ids=["kquants", "block32", "single"])
+@pytest.mark.parametrize("K", [1024, 14336])
+def test_mul_mat_group_run_over_prepared_rows(dev, orc, members, K):
+    """chip_mul_mat_group_run: over rows the workspace already holds every member's output equals chip_mul_mat's, bit for
+    bit (the quantized rows are the same bytes and the GEMV's arithmetic does not depend on who staged them), also for
+    rows longer than the prologue quantizer takes (K = 14336), with the transposed fp16 store on the last member."""
+    ws = [(wt, quantized_weights(wt, K + N + 13, N, K)) for wt, N in members]
+    for n in (1, 2, 4, 3, 6):
+        x = common.activations_f32(K + n + 7, n, K)
+        ys = dev.mul_mat_group(ws, x, ld16=8, prepared=True)
+        for (wt, W), y in zip(ws, ys):
+            assert y.tobytes() == dev.mul_mat(wt, W, x).tobytes(), (O.TYPE_NAMES[wt], n)
+        t16 = ys[-1]
+        want = ys[len(ws) - 1].astype(np.float16).view(np.uint16).T
+        assert np.array_equal(t16[:, :n], want) and (t16[:, n:] == 0x7bff).all()
+
+
 def test_mul_mat_group_argument_errors(dev, orc):
     import cactus_amd as ca
     L = dev.lib
