@@ -518,6 +518,14 @@ static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float
     // more tokens, or members the one-launch form does not take: quantize once, then every member as chip_mul_mat_run would
     if (!prepared)
         if (int rc = chip_mul_mat_prepare(mats[0].type, K, x, ldx, n, workspace, workspace_bytes, stream); rc) return rc;
+    if (n == 8 && live >= 2 && gemv_group_applicable(gm, live, K, 8, lim, true)) {
+        // 8 tokens, several small matrices: one launch of the dot-product GEMV over all members when together they stream
+        // no more than 24 MB (larger ones are faster through a matrix-core GEMV each)
+        double bytes = 0;
+        for (int i = 0; i < live; i++) bytes += (double)gm[i].N * (double)gm[i].nb01;
+        if (bytes <= tune("CHIP_GROUP8_MAX_MB", 24) * 1048576.0)
+            return hip_rc(launch_gemv_group(gm, live, K, nullptr, 0, 8, workspace, stride, lim, st, true));
+    }
     for (int i = 0; i < live; i++) {
         const GroupMat &m = gm[i];
         if (int rc = mul_mat_run(m.wtype, m.W, m.nb01, K, m.N, n, workspace, workspace_bytes, m.y, m.ldy, stream); rc) return rc;

@@ -102,6 +102,10 @@ hipError_t launch_ntok(int n, int wgs, const GroupKernelArgs &ga, int grid, int6
         case 1: return launch_wgs<FAMILY, 1>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
         case 2: return launch_wgs<FAMILY, 2>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
         case 4: return launch_wgs<FAMILY, 4>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        case 8:                                                          // over prepared rows only
+            if (!prepared) return hipErrorInvalidValue;
+            return wgs == 1024 ? launch_depth<FAMILY, 8, 1024, false, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st)
+                               : launch_depth<FAMILY, 8, 512, false, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
         default: return hipErrorInvalidValue;
     }
 }
@@ -118,10 +122,12 @@ int gemv_group_family(int wtype) {
 }
 
 // One launch serves the group when the prologue-quantizing GEMV takes every member (n in {1, 2, 4}, n * K within its
-// limit, the largest member's activation image within LDS) and the members are of one family.
+// limit, the largest member's activation image within LDS) and the members are of one family.  Over prepared rows also
+// 8 tokens: for matrices that are small enough to be all latency (wq + wk + wv at 8 tokens: one quantizer and three
+// launches took 22 us) one launch of the dot-product GEMV beats a matrix-core GEMV launch per member.
 bool gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim, bool prepared) {
     if (count < 1 || count > GROUP_MAX) return false;
-    if (n != 1 && n != 2 && n != 4) return false;
+    if (n != 1 && n != 2 && n != 4 && !(prepared && n == 8)) return false;
     const int fam = gemv_group_family(mats[0].wtype);
     if (fam < 0) return false;
     int64_t rows = 0;

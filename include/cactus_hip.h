@@ -164,7 +164,10 @@ CHIP_API int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t 
  * quantizes in its prologue, its workgroups divided among the members by the bytes each streams; otherwise one
  * quantizer launch and every member on the path chip_mul_mat_run_ws would take.  A member with y_f16_t != NULL also gets
  * its result rounded to fp16 at y_f16_t[row * ld16 + token], as chip_mul_mat_store_t.  Every output equals, bit for bit,
- * what chip_mul_mat (chip_mul_mat_store_t) returns for that member alone.  The workspace must hold
+ * what chip_mul_mat (chip_mul_mat_store_t) returns for that member alone - except at exactly 8 tokens when the members
+ * together stream at most 24 MB: they then run as one launch of the dot-product GEMV over the quantized rows, while a
+ * member alone may take the matrix-core GEMV, which adds its partial sums in another order (same tolerance against the
+ * reference, not the same bits).  The workspace must hold
  * chip_mul_mat_workspace_size(type, K, n) bytes for the members' activation format. */
 #define CHIP_GROUP_MAX 4
 typedef struct chip_mat {

@@ -129,7 +129,10 @@ def test_config4_prefill_remaining_shapes(dev, orc, N, M):
 def test_trace_qkv_group(dev, orc):
     """wq (Q4_K 4096 rows), wk (Q4_K 1024), wv (Q6_K 1024, with its transposed fp16 cache store) on one activation as one
     call of chip_mul_mat_group, at the trace's shapes: every output equals the member's own chip_mul_mat /
-    chip_mul_mat_store_t bit for bit (1, 2, 4 tokens: one launch; 3 and 8: one quantizer, then each member)."""
+    chip_mul_mat_store_t bit for bit (1, 2, 4 tokens: one launch; 3: one quantizer, then each member).  At 8 tokens the
+    three run as one launch of the dot-product GEMV over prepared rows, where wq alone would take the matrix-core GEMV
+    (which splits K inside a workgroup): there every member is held to the oracle's tolerance instead, and the fp16 store to
+    the rounding of the group's own fp32 result."""
     K = 4096
     wq = np.tile(base_rows(orc, O.Q4_K, 5000 + 4096 + K, 1024, K), (4, 1))
     wk = base_rows(orc, O.Q4_K, 5000 + 1024 + K, 1024, K)
@@ -137,10 +140,16 @@ def test_trace_qkv_group(dev, orc):
     for n in (1, 2, 4, 3, 8):
         x = common.activations_f32(60 + n, n, K)
         yq, yk, yv, h = dev.mul_mat_group([(O.Q4_K, wq), (O.Q4_K, wk), (O.Q6_K, wv)], x, ld16=64)
-        assert yq.tobytes() == dev.mul_mat(O.Q4_K, wq, x).tobytes(), n
-        assert yk.tobytes() == dev.mul_mat(O.Q4_K, wk, x).tobytes(), n
-        y1, h1 = dev.mul_mat_store_t(O.Q6_K, wv, x, 64)
-        assert yv.tobytes() == y1.tobytes() and h.tobytes() == h1.tobytes(), n
+        if n != 8:
+            assert yq.tobytes() == dev.mul_mat(O.Q4_K, wq, x).tobytes(), n
+            assert yk.tobytes() == dev.mul_mat(O.Q4_K, wk, x).tobytes(), n
+            y1, h1 = dev.mul_mat_store_t(O.Q6_K, wv, x, 64)
+            assert yv.tobytes() == y1.tobytes() and h.tobytes() == h1.tobytes(), n
+        else:
+            for wt, W, y in ((O.Q4_K, wq, yq), (O.Q6_K, wv, yv)):
+                r = orc.mul_mat(wt, W, x, nthreads=8, want=("sum_abs",))
+                assert (np.abs(y.astype(np.float64) - r["y"].astype(np.float64)) <= REL_TOL * r["sum_abs"]).all(), n
+            assert np.array_equal(h[:, :n], yv.astype(np.float16).view(np.uint16).T) and (h[:, n:] == 0x7bff).all()
         ref = orc.mul_mat(O.Q4_K, wk, x, nthreads=8, want=("sum_abs",))
         err = np.abs(yk.astype(np.float64) - ref["y"].astype(np.float64))
         assert (err <= REL_TOL * ref["sum_abs"]).all(), n

@@ -716,10 +716,14 @@ def test_mul_mat_group_equals_single_calls(dev, orc, members, K):
     """chip_mul_mat_group: each member's output equals chip_mul_mat on that member alone, bit for bit, for every token
     count class (1, 2, 4: one launch; 3, 7: one quantizer and the GEMVs; 40: the GEMMs), and the oracle within tolerance."""
     ws = [(wt, quantized_weights(wt, K + N + 11, N, K)) for wt, N in members]
-    for n in (1, 2, 4, 3, 7, 40):
+    for n in (1, 2, 4, 3, 7, 8, 40):                                 # 8: small members as one launch over prepared rows
         x = common.activations_f32(K + n + 5, n, K)
         ys = dev.mul_mat_group(ws, x)
         for (wt, W), y in zip(ws, ys):
+            if n == 8 and len(ws) > 1:          # one launch of the dot-product GEMV; alone, a member may take the matrix-core GEMV
+                r = orc.mul_mat(wt, W, x, nthreads=8, want=("sum_abs",))
+                check_outputs(y, r["y"], r["sum_abs"], "group member at 8 tokens")
+                continue
             assert y.tobytes() == dev.mul_mat(wt, W, x).tobytes(), (O.TYPE_NAMES[wt], n)
         wt, W = ws[0]
         ref = orc.mul_mat(wt, W, x, nthreads=8, want=("sum_abs",))
@@ -737,10 +741,14 @@ def test_mul_mat_group_run_over_prepared_rows(dev, orc, members, K):
     bit (the quantized rows are the same bytes and the GEMV's arithmetic does not depend on who staged them), also for
     rows longer than the prologue quantizer takes (K = 14336), with the transposed fp16 store on the last member."""
     ws = [(wt, quantized_weights(wt, K + N + 13, N, K)) for wt, N in members]
-    for n in (1, 2, 4, 3, 6):
+    for n in (1, 2, 4, 3, 6, 8):
         x = common.activations_f32(K + n + 7, n, K)
         ys = dev.mul_mat_group(ws, x, ld16=8, prepared=True)
         for (wt, W), y in zip(ws, ys):
+            if n == 8 and len(ws) > 1:
+                r = orc.mul_mat(wt, W, x, nthreads=8, want=("sum_abs",))
+                check_outputs(y, r["y"], r["sum_abs"], "group member at 8 tokens")
+                continue
             assert y.tobytes() == dev.mul_mat(wt, W, x).tobytes(), (O.TYPE_NAMES[wt], n)
         t16 = ys[-1]
         want = ys[len(ws) - 1].astype(np.float16).view(np.uint16).T
