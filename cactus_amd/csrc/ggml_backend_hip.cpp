@@ -936,7 +936,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         int store_t = -1;
         int members[CHIP_GROUP_MAX];
         int n_members = 1;
-        if (n <= 4 && fusion_enabled()) {
+        if ((n <= 4 || n == 8) && fusion_enabled()) {      // the token counts chip_mul_mat_group has a one-launch form for
             bool slots_free = true;
             for (int slot : grouped) slots_free = slots_free && slot < 0;
             if (slots_free) n_members = grouped_matmuls(cgraph, i, members);
@@ -965,8 +965,19 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                     writes(cgraph->nodes[members[k]]);
                     grouped[k] = members[k];
                 }
-                c->quantized.valid = false;
-                rc = chip_mul_mat_group(mats, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                // more than 4 tokens: the workspace holds x's quantized rows afterwards, or already does (the norm in front
+                // left them there, or an earlier matmul of the same input)
+                quantized_key &q = c->quantized;
+                const int vt = chip_vec_dot_type(w->type);
+                const bool have_rows = n > 4 && q.valid && q.src == x->data && q.K == K && q.n == n && q.ldx == ldx && q.vec_dot_type == vt;
+                if (have_rows) {
+                    rc = chip_mul_mat_group_run(mats, n_members, K, n, c->workspace, c->workspace_size, c->stream);
+                    g_quantizers_skipped++;
+                } else {
+                    q.valid = false;
+                    rc = chip_mul_mat_group(mats, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                    if (rc == CHIP_OK && n > 4) q = quantized_key{true, x->data, lm_ggml_nbytes(x), K, n, ldx, vt};
+                }
                 if (rc != CHIP_OK) {
                     HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT group of %d at %s failed: %s\n", __func__, n_members, node->name,
                             chip_error_string(rc));

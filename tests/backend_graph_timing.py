@@ -124,6 +124,8 @@ f0 = blib.lm_ggml_backend_hip_get_fused_pairs()
 for it in range(3):
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
 print("fused per graph", (blib.lm_ggml_backend_hip_get_fused_pairs() - f0) / 3, flush=True)
+blib.lm_ggml_backend_hip_get_grouped_matmuls.restype = C.c_ulonglong
+print("projections run in group launches so far", blib.lm_ggml_backend_hip_get_grouped_matmuls(), "(3 graphs)", flush=True)
 blib.lm_ggml_backend_hip_get_quantizers_skipped.restype = C.c_ulonglong
 print("quantizers skipped so far", blib.lm_ggml_backend_hip_get_quantizers_skipped(), flush=True)
 ts = []
