@@ -221,9 +221,11 @@ hipError_t launch_gemv_store_t(int wtype, const void *W, size_t nb01, int64_t K,
 bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
     if (!(n == 1 || n == 2 || n == 4) || (int64_t)n * K > FUSE_MAX_VALUES) return false;
     // Every workgroup repeats the quantizer, and its dependent chains (maximum, two divisions, sums) cost a wave about
-    // 0.9 us per 256 values: beyond 8192 values per workgroup the separate quantizer kernel (1.9 us) and the GEMV over
-    // prepared rows are ahead (Q6_K 4096 x 14336, one token: 1.97 + 12.6 us against 15.3-16.1 us in one launch).
-    if ((int64_t)n * K > 8192 && n == 1) return false;
+    // 0.9 us per 256 values.  For Q6_K rows of more than 8192 values the separate quantizer kernel (1.9 us) and the GEMV over
+    // prepared rows are ahead (4096 x 14336, one token: 1.97 + 12.6 us against 15.3-16.1 us in one launch); the other
+    // types keep the single launch at every length it takes (4096 x 11008 Q8_0 10.7 against 12.3 us in two launches,
+    // 4096 x 14336 Q4_K 10.5 against 10.8, Q8_0 13.7 against 14.9, Q4_0 4096 x 11008 9.1 either way).
+    if (wtype == T_Q6_K && n == 1 && K > 8192) return false;
     size_t img = 0;
     switch (wtype) {
         case T_Q4_0: img = lds_image_bytes<T_Q4_0>(K); break;
