@@ -108,11 +108,6 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         if (one_tile_per_wave && !long_q8_0_row)
             return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
     }
-    if constexpr (!FUSEQ && NTOK == 1) {
-        const bool one_tile_per_wave = tiles <= 16 * (int64_t)cus && tiles > 8 * (int64_t)cus;
-        if (tune("CHIP_GEMV_STAGED_WIDE", 0) != 0 && one_tile_per_wave)
-            return launch_one<WT, NTOK, R, 1024, false>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
-    }
     if constexpr (FUSEQ && NTOK >= 2) {
         // A narrow matrix (fewer than 8 tiles per CU) is all prologue: every workgroup quantizes NTOK rows before its
         // waves read one tile each.  16-wave groups do that with a quarter of the values per lane and keep the same
