@@ -36,7 +36,7 @@ EXPORTS = (
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
-    "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
+    "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
     "chip_workspace_to_blocks",
@@ -126,6 +126,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_add_rms_norm_mul.argtypes = [vp, i64, vp, i64, vp, i64, i64, i64, C.c_float, vp, vp, i64, vp]
     L.chip_scale.argtypes = [vp, i64, i64, i64, C.c_float, vp, i64, vp]
     L.chip_rms_norm_quantized.argtypes = [vp, i64, vp, i64, vp, i64, i64, i64, C.c_float, vp, vp, i64, i32, vp, sz, vp]
+    L.chip_silu_mul_quantized.argtypes = [vp, i64, vp, i64, i64, i64, vp, i64, i32, vp, sz, vp]
     L.chip_gelu_table.argtypes = [vp]
     L.chip_gelu.argtypes = [vp, i64, i64, i64, vp, vp, i64, vp]
     L.chip_soft_max.argtypes = [vp, i64, vp, i32, i64, i64, i64, C.c_float, C.c_float, vp, i64, vp]
@@ -334,6 +335,15 @@ class Device:
         n, ne0 = x.shape
         dx, dy = self.to_device(x), self.alloc(x.nbytes)
         self.check(self.lib.chip_silu(dx.ptr, ne0, n, ne0, dy.ptr, ne0, None))
+        self.sync()
+        return dy.download(np.float32, n * ne0).reshape(n, ne0)
+
+    def silu_mul(self, a, b):
+        """silu(a) * b in one launch (the FFN's gate * up)."""
+        a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+        n, ne0 = a.shape
+        da, db, dy = self.to_device(a), self.to_device(b), self.alloc(a.nbytes)
+        self.check(self.lib.chip_silu_mul(da.ptr, ne0, db.ptr, ne0, n, ne0, dy.ptr, ne0, None))
         self.sync()
         return dy.download(np.float32, n * ne0).reshape(n, ne0)
 

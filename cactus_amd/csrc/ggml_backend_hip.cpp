@@ -524,14 +524,16 @@ static bool grow_workspace(backend_ctx *c, size_t need) {
     return true;
 }
 
-// The first node (views aside) after index `last` when it is a quantized weight matmul of more than 4 tokens that reads
-// `out`: the norm in front of it can then leave the quantized rows in the workspace.  NULL otherwise.
-const lm_ggml_tensor *quantized_consumer(const lm_ggml_cgraph *g, int last, const lm_ggml_tensor *out) {
+// The first node (views aside) after index `last` when it is a quantized weight matmul of at least min_tokens tokens that
+// reads `out`: the kernel in front of it can then leave the quantized rows in the workspace.  NULL otherwise.  A norm asks
+// for more than 4 tokens (up to 4 the projections behind it quantize in their own prologue, in one launch for all of
+// them); SiLU * up asks for 1: ffn_down's rows are long and its GEMV takes them ready-made at every token count.
+const lm_ggml_tensor *quantized_consumer(const lm_ggml_cgraph *g, int last, const lm_ggml_tensor *out, int64_t min_tokens = 5) {
     int j = last + 1;
     while (j < g->n_nodes && is_view_op(g->nodes[j]->op)) j++;
     if (j >= g->n_nodes) return nullptr;
     const lm_ggml_tensor *mm = g->nodes[j];
-    if (mm->op != LM_GGML_OP_MUL_MAT || mm->src[1] != out || !mul_mat_shape_ok(mm) || out->ne[1] <= 4) return nullptr;
+    if (mm->op != LM_GGML_OP_MUL_MAT || mm->src[1] != out || !mul_mat_shape_ok(mm) || out->ne[1] < min_tokens) return nullptr;
     if (mm->src[0]->type == LM_GGML_TYPE_F16 || out->ne[2] != 1 || out->ne[3] != 1) return nullptr;
     return mm;
 }
@@ -550,6 +552,26 @@ int norm_for_quantized_consumer(backend_ctx *c, const lm_ggml_cgraph *g, int las
         key = quantized_key{true, out->data, lm_ggml_nbytes(out), ne0, rows, ldy, chip_vec_dot_type(wtype)};
     }
     return rc;
+}
+
+// True when the workspace holds the quantized rows of x in the activation type that w's matmul reads.
+bool have_rows(const quantized_key &q, const lm_ggml_tensor *x, const lm_ggml_tensor *w, int64_t n, int64_t ldx) {
+    return q.valid && q.src == x->data && q.K == w->ne[0] && q.n == n && q.ldx == ldx && q.vec_dot_type == chip_vec_dot_type(w->type);
+}
+
+// silu(a) * b -> out, with the quantized rows going to the workspace when the next node is a quantized weight matmul that
+// reads out (ffn_down); sets key to what the workspace then holds.
+int silu_mul_for_consumer(backend_ctx *c, const lm_ggml_cgraph *g, int last, const float *a, int64_t lda, const float *b, int64_t ldb,
+                          int64_t rows, int64_t ne0, const lm_ggml_tensor *out, int64_t ldy, quantized_key &key) {
+    const lm_ggml_tensor *mm = fusion_enabled() ? quantized_consumer(g, last, out, 1) : nullptr;
+    if (mm && grow_workspace(c, chip_mul_mat_workspace_size_n(mm->src[0]->type, ne0, mm->src[0]->ne[1], rows))) {
+        const int wtype = mm->src[0]->type;
+        const int rc = chip_silu_mul_quantized(a, lda, b, ldb, rows, ne0, (float *)out->data, ldy, wtype, c->workspace, c->workspace_size,
+                                               c->stream);
+        if (rc == CHIP_OK) key = quantized_key{true, out->data, lm_ggml_nbytes(out), ne0, rows, ldy, chip_vec_dot_type(wtype)};
+        if (rc != CHIP_EUNSUPPORTED) return rc;
+    }
+    return chip_silu_mul(a, lda, b, ldb, rows, ne0, (float *)out->data, ldy, c->stream);
 }
 
 // RMS_NORM or SILU directly followed by the MUL that consumes it, the MUL written over the first node's output: the
@@ -580,8 +602,7 @@ int try_fused_pair(backend_ctx *c, const lm_ggml_cgraph *g, int i, const lm_ggml
     if (node->op == LM_GGML_OP_UNARY && node->op_params[0] == LM_GGML_UNARY_OP_SILU) {
         if (!same_shape(other, node)) return CHIP_OK;
         fused = true;
-        return chip_silu_mul((const float *)a->data, lda, (const float *)other->data, ldb, rows, a->ne[0], (float *)next->data, ldy,
-                             c->stream);
+        return silu_mul_for_consumer(c, g, i + 1, (const float *)a->data, lda, (const float *)other->data, ldb, rows, a->ne[0], next, ldy, key);
     }
     return CHIP_OK;
 }
@@ -795,8 +816,10 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             as_rows(silu->src[0], rows, lda);
             as_rows(other, rows, ldb);
             as_rows(node, rows, ldy);
-            const int rc = chip_silu_mul((const float *)silu->src[0]->data, lda, (const float *)other->data, ldb, rows, silu->ne[0],
-                                         (float *)node->data, ldy, c->stream);
+            quantized_key key;
+            const int rc = silu_mul_for_consumer(c, cgraph, i, (const float *)silu->src[0]->data, lda, (const float *)other->data, ldb, rows,
+                                                 silu->ne[0], node, ldy, key);
+            if (key.valid) c->quantized = key;
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (SILU run with its MUL) failed: %s\n", __func__, node->name, chip_error_string(rc));
                 return LM_GGML_STATUS_FAILED;
@@ -1007,11 +1030,12 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                                    (float *)up->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
             g_mul_mat_nodes++;
             g_fused_pairs++;
-        } else if (n > 4 && fusion_enabled()) {
-            // quantize once per source tensor: the matmuls that share an input follow each other closely
+        } else if ((n > 4 || have_rows(c->quantized, x, w, n, ldx)) && fusion_enabled()) {
+            // quantize once per source tensor: the matmuls that share an input follow each other closely (up to 4 tokens
+            // only a producer's kernel leaves rows here; without them the GEMV below quantizes in its prologue)
             quantized_key &q = c->quantized;
             const int vt = chip_vec_dot_type(w->type);
-            if (!(q.valid && q.src == x->data && q.K == K && q.n == n && q.ldx == ldx && q.vec_dot_type == vt)) {
+            if (!have_rows(q, x, w, n, ldx)) {
                 q.valid = false;
                 rc = chip_mul_mat_prepare(w->type, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
                 if (rc == CHIP_OK) q = quantized_key{true, x->data, lm_ggml_nbytes(x), K, n, ldx, vt};

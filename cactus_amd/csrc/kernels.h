@@ -256,6 +256,9 @@ bool norm_quantized_applicable(const float *a, int64_t lda, const float *b, int6
 hipError_t launch_norm_quantized(const float *a, int64_t lda, const float *b, int64_t ldb, float *xs, int64_t ldxs, int64_t n,
                                  int64_t ne0, float eps, const float *w, float *y, int64_t ldy, uint8_t *qws, size_t qstride,
                                  int act_kind, hipStream_t st);
+bool       silu_mul_quantized_applicable(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, const float *y, int64_t ldy);
+hipError_t launch_silu_mul_quantized(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y,
+                                     int64_t ldy, uint8_t *qws, size_t qstride, int act_kind, hipStream_t st);
 hipError_t launch_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy,
                            hipStream_t st);
 // SOFT_MAX over n_rows rows of ne00 values (a multiple of 8); row r adds row r % ne01 of the mask (fp32 or fp16, dense).

@@ -226,6 +226,53 @@ __global__ __launch_bounds__(EW_THREADS) void elementwise_kernel(const float *a,
     }
 }
 
+// silu(x) * b with the result also left as the quantized rows of the matmul that reads it (ffn_down reads
+// silu(ffn_gate) * ffn_up): what launch_quantize would write from y afterwards, without its launch.  Quantization is per
+// block, so the element-wise grid serves: a lane holds four consecutive values, eight lanes a 32-value block, a wave a
+// 256-value super-block, exactly the quantizer kernels' mapping (ne0 % 256 == 0 keeps every wave whole).
+// KIND 1: Q8_0 / Q8_1 planes; 2: Q8_K planes.
+template <int KIND>
+__global__ __launch_bounds__(EW_THREADS) void silu_mul_quantized_kernel(const float *x, int64_t ldx, const float *b, int64_t ldb,
+                                                                        int64_t ne0, float *y, int64_t ldy, uint8_t *qws, size_t qstride) {
+    const int64_t row = blockIdx.y;
+    const int64_t e0 = 4 * ((int64_t)blockIdx.x * EW_THREADS + threadIdx.x);
+    if (e0 >= ne0) return;                                                  // whole waves leave together
+    const float4 va = *reinterpret_cast<const float4 *>(x + (size_t)row * ldx + e0);
+    const float4 vb = *reinterpret_cast<const float4 *>(b + (size_t)row * ldb + e0);
+    const float4 v = make_float4(silu1(va.x) * vb.x, silu1(va.y) * vb.y, silu1(va.z) * vb.z, silu1(va.w) * vb.w);
+    *reinterpret_cast<float4 *>(y + (size_t)row * ldy + e0) = v;
+    uint8_t *base = qws + (size_t)row * qstride;
+    if constexpr (KIND == 2) {
+        const Q8_KLane q = quantize_q8_K_lane(v);
+        const int lane = threadIdx.x & 63;
+        const int64_t sb = e0 / QK_K;
+        *reinterpret_cast<uint32_t *>(base + e0) = q.packed;
+        if (lane == 0) reinterpret_cast<float *>(base + q8_K_off_d(ne0))[sb] = q.d;
+        if ((lane & 3) == 0) reinterpret_cast<int16_t *>(base + q8_K_off_bsums(ne0))[sb * 16 + (lane >> 2)] = (int16_t)q.bsum;
+    } else {
+        const Q8_0Lane q = quantize_q8_0_lane(v);
+        const int64_t blk = e0 / 32;
+        *reinterpret_cast<uint32_t *>(base + e0) = q.packed;
+        if ((threadIdx.x & 7) == 0) {
+            reinterpret_cast<float *>(base + q8_0_off_d(ne0))[blk] = h2f(q.dh);
+            reinterpret_cast<int32_t *>(base + q8_0_off_sum(ne0))[blk] = q.sum;
+            reinterpret_cast<float *>(base + q8_0_off_s(ne0))[blk] = h2f(q.sh);
+        }
+    }
+}
+bool silu_mul_quantized_applicable(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, const float *y, int64_t ldy) {
+    return ne0 > 0 && ne0 % 256 == 0 && ((ldx | ldb | ldy) & 3) == 0 && ((((uintptr_t)x) | ((uintptr_t)b) | ((uintptr_t)y)) & 15) == 0;
+}
+hipError_t launch_silu_mul_quantized(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y,
+                                     int64_t ldy, uint8_t *qws, size_t qstride, int act_kind, hipStream_t st) {
+    if (n <= 0 || ne0 <= 0) return hipSuccess;
+    if (n > 65535 || (act_kind != 1 && act_kind != 2) || !silu_mul_quantized_applicable(x, ldx, b, ldb, ne0, y, ldy)) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)ceil_div(ne0, 4 * EW_THREADS), (unsigned)n);
+    if (act_kind == 1) hipLaunchKernelGGL(silu_mul_quantized_kernel<1>, grid, dim3(EW_THREADS), 0, st, x, ldx, b, ldb, ne0, y, ldy, qws, qstride);
+    else               hipLaunchKernelGGL(silu_mul_quantized_kernel<2>, grid, dim3(EW_THREADS), 0, st, x, ldx, b, ldb, ne0, y, ldy, qws, qstride);
+    return hipGetLastError();
+}
+
 // ---- SCALE and GELU: one value in, one value out ----
 // GELU is the reference's table form (ggml-cpu/vec.h:452-466): 0 at or below -10, x at or above 10, else entry fp16(x) of
 // a 65536-entry fp16 table built on the host with the C library's tanhf (the caller uploads it).

@@ -275,6 +275,13 @@ CHIP_API int chip_gelu(const float *x, int64_t ldx, int64_t n, int64_t ne0, cons
 CHIP_API int chip_rms_norm_quantized(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
                                      int64_t ne0, float eps, const float *w, float *y, int64_t ldy, int wtype, void *workspace,
                                      size_t workspace_bytes, void *stream);
+/* chip_silu_mul in front of a matmul (ffn_down reads silu(ffn_gate) * ffn_up, reference llama-graph.cpp:562-690): y as
+ * chip_silu_mul writes it, and y quantized as the activation type of weight type `wtype` into `workspace`, exactly what
+ * chip_mul_mat_prepare(wtype, K = ne0, y, ...) would leave there.  Rows of any length that is a multiple of 256, 16-byte
+ * aligned with strides that are multiples of 4, at most 65535 rows; CHIP_EUNSUPPORTED otherwise (and for F16 weights), in
+ * which case nothing has been written. */
+CHIP_API int chip_silu_mul_quantized(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y,
+                                     int64_t ldy, int wtype, void *workspace, size_t workspace_bytes, void *stream);
 CHIP_API int chip_add_rms_norm_mul(const float *a, int64_t lda, const float *b, int64_t ldb, float *sum, int64_t ld_sum, int64_t n,
                                    int64_t ne0, float eps, const float *w, float *y, int64_t ldy, void *stream);
 

@@ -461,8 +461,9 @@ def test_ffn_block_stays_on_the_device(host, orc, n):
     # MUL's kernel
     # 5 tokens: the norm leaves its result quantized in the workspace, so neither gate nor up runs the quantizer.
     # 2 tokens: the two projections run as one launch of the GEMV that quantizes in its prologue (a third join)
+    # Either way SiLU * up leaves its result quantized for ffn_down, which runs no quantizer of its own.
     assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == (2 if n > 4 else 3)
-    assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - skipped_before == (2 if n > 4 else 0)
+    assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - skipped_before == (3 if n > 4 else 1)
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (cur, up, gate, act, down, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip

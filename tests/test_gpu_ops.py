@@ -202,6 +202,45 @@ def test_scale_and_gelu_equal_the_oracle(dev, orc):
     dt.free()
 
 
+@pytest.mark.parametrize("wt", ["Q6_K", "Q4_K", "Q8_0", "Q5_1"])
+@pytest.mark.parametrize("n,ne0", [(1, 14336), (4, 14336), (9, 4096), (3, 256), (40, 1024)])
+def test_silu_mul_that_leaves_quantized_rows(dev, orc, wt, n, ne0):
+    """chip_silu_mul_quantized: y equals chip_silu_mul's bit for bit, and the workspace holds what chip_mul_mat_prepare
+    writes from y (compared as the reference's activation blocks against the oracle's quantizer); a matmul over those rows
+    (chip_mul_mat_run) then equals chip_mul_mat on y."""
+    import cactus_amd as ca
+    t = getattr(ca, wt)
+    a, b = inputs(19 * n + ne0, n, ne0), inputs(23 * n + ne0, n, ne0)
+    da, db, dy = dev.to_device(a), dev.to_device(b), dev.alloc(a.nbytes)
+    N = 48
+    wsz = dev.lib.chip_mul_mat_workspace_size_n(t, ne0, N, n)
+    ws = dev.alloc(wsz)
+    dev.check(dev.lib.chip_silu_mul_quantized(da.ptr, ne0, db.ptr, ne0, n, ne0, dy.ptr, ne0, t, ws.ptr, wsz, None))
+    dev.sync()
+    y = dy.download(np.float32, a.size).reshape(n, ne0)
+    with np.errstate(all="ignore"):
+        want = dev.silu_mul(a, b)
+    assert y.tobytes() == want.tobytes()
+    at = dev.lib.chip_vec_dot_type(t)
+    rs = dev.row_size(at, ne0)
+    blk = dev.alloc(n * rs)
+    dev.check(dev.lib.chip_workspace_to_blocks(t, ne0, n, ws.ptr, blk.ptr, None))
+    dev.sync()
+    got = blk.download(np.uint8, n * rs).reshape(n, rs)
+    assert np.array_equal(got, orc.quantize_activation(at, y))
+    W = orc.quantize_weights(t, (np.random.default_rng(ne0).standard_normal((N, ne0)) * 0.05).astype(np.float32))
+    dW, dz = dev.to_device(W), dev.alloc(n * N * 4)
+    dev.check(dev.lib.chip_mul_mat_run_ws(t, dW.ptr, dev.row_size(t, ne0), ne0, N, n, ws.ptr, wsz, dz.ptr, N, None))
+    dev.sync()
+    assert dz.download(np.float32, n * N).reshape(n, N).tobytes() == dev.mul_mat(t, W, y).tobytes()
+    for tt in (da, db, dy, ws, blk, dW, dz):
+        tt.free()
+    # rows that are no multiple of 256 are declined, nothing written
+    dx = dev.to_device(inputs(3, 2, 320))
+    dyy, ws2 = dev.alloc(2 * 320 * 4), dev.alloc(4096)
+    assert dev.lib.chip_silu_mul_quantized(dx.ptr, 320, dx.ptr, 320, 2, 320, dyy.ptr, 320, ca.Q8_0, ws2.ptr, 4096, None) == ca.CHIP_EUNSUPPORTED
+
+
 @pytest.mark.parametrize("wt", ["Q4_K", "Q6_K", "Q8_0", "Q4_1"])
 @pytest.mark.parametrize("n,ne0", [(1, 4096), (9, 4096), (3, 256), (5, 8192), (40, 1024)])
 @pytest.mark.parametrize("with_add", [False, True])
