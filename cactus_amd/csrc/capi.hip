@@ -335,6 +335,23 @@ size_t chip_mul_mat_workspace_size_n(int type, int64_t K, int64_t N, int64_t n) 
     return slices > 1 ? act_rows_bytes(type, K, n) + (size_t)slices * (size_t)n * (size_t)N * sizeof(float) : act;
 }
 
+// Fewest tokens from which the matrix-core GEMV is taken for this matrix.
+// (4-bit weights on a small matrix: the dot-product GEMV is still ahead up to 6 or 7 tokens)
+// (and Q4_K rows so wide that the kernel runs with six waves: from 7 tokens)
+static int mmv_min_tokens(int type, int64_t K, int64_t N) {
+    const int mmv_forced = (int)tune("CHIP_MMV_MIN", 0);
+    return mmv_forced > 0 ? mmv_forced
+           : ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7)
+           : (type == T_Q4_K && K > 13312) ? 7 : MMV_MIN_TOKENS;
+}
+// Two Q4_K / Q5_K matrices of one shape on the same rows at 5..8 tokens (ffn_gate and ffn_up): true when each alone would
+// take one launch of the matrix-core GEMV whatever the workspace size - they then run as one launch whose grid is the two
+// launches' grids side by side (every tile is computed as in a launch of its own: the same bits).
+static bool mmv_pair_applicable(int type, int64_t K, int64_t N, int64_t n, const DeviceLimits &lim) {
+    if (n < 5 || n > 8 || !(type == T_Q4_K || type == T_Q5_K) || tune("CHIP_MMV_PAIR", 1) == 0) return false;
+    if (gemm_kq_supported(type, K, N, n, false) || gemm_kq_supported(type, K, N, n, true)) return false;
+    return n >= mmv_min_tokens(type, K, N) && n <= mmv_q4k_max_tokens(type, K, N, lim);
+}
 static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
                        size_t workspace_bytes, float *y, int64_t ldy, void *stream);
 int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t N, int64_t n, const void *workspace,
@@ -376,12 +393,7 @@ static int mul_mat_run(int type, const void *W, size_t nb01, int64_t K, int64_t 
         return hip_rc(launch_gemm_kq(type, W, nb01, K, N, workspace, stride, n, y, ldy, lim, st, nullptr, 1, split));
 
     // 5 tokens or more: integer sums on the matrix cores, up to 16 tokens per pass over the weights
-    // (4-bit weights on a small matrix: the dot-product GEMV is still ahead up to 6 or 7 tokens)
-    // (and Q4_K rows so wide that the kernel runs with six waves: from 7 tokens)
-    const int mmv_forced = (int)tune("CHIP_MMV_MIN", 0);
-    const int mmv_min = mmv_forced > 0 ? mmv_forced
-                        : ((type == T_Q4_K || type == T_Q5_K || type == T_Q4_0) && N * K < (32LL << 20)) ? (type == T_Q4_0 ? 8 : 7)
-                        : (type == T_Q4_K && K > 13312) ? 7 : MMV_MIN_TOKENS;
+    const int mmv_min = mmv_min_tokens(type, K, N);
     const int mgroup = (n >= mmv_min) ? mmv_max_tokens(type, K, N, lim) : 0;
     if (mgroup > 0) {
         for (int64_t t0 = 0; t0 < n; t0 += mgroup) {
@@ -457,6 +469,9 @@ int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int
         return hip_rc(launch_gemv_fused_pair(type, W1, W2, nb01, K, N, x, ldx, (int)n, workspace,
                                              act_stride(chip_vec_dot_type(type), K), y1, y2, ldy, lim, (hipStream_t)stream));
     if (int rc = chip_mul_mat_prepare(type, K, x, ldx, n, workspace, workspace_bytes, stream); rc) return rc;
+    if (mmv_pair_applicable(type, K, N, n, lim))
+        return hip_rc(launch_mmv_q4k(type, W1, nb01, K, N, workspace, act_stride(chip_vec_dot_type(type), K), (int)n, y1, ldy, lim,
+                                     (hipStream_t)stream, W2, y2));
     if (int rc = mul_mat_run(type, W1, nb01, K, N, n, workspace, workspace_bytes, y1, ldy, stream); rc) return rc;
     return mul_mat_run(type, W2, nb01, K, N, n, workspace, workspace_bytes, y2, ldy, stream);
 }
@@ -525,6 +540,12 @@ static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float
         for (int i = 0; i < live; i++) bytes += (double)gm[i].N * (double)gm[i].nb01;
         if (bytes <= tune("CHIP_GROUP8_MAX_MB", 24) * 1048576.0)
             return hip_rc(launch_gemv_group(gm, live, K, nullptr, 0, 8, workspace, stride, lim, st, true));
+    }
+    if (live == 2) {                                                   // ffn_gate and ffn_up at 5..8 tokens
+        const GroupMat &a = gm[0], &b = gm[1];
+        const bool twins = a.wtype == b.wtype && a.N == b.N && a.nb01 == b.nb01 && a.ldy == b.ldy && !a.t16 && !b.t16;
+        if (twins && mmv_pair_applicable(a.wtype, K, a.N, n, lim))
+            return hip_rc(launch_mmv_q4k(a.wtype, a.W, a.nb01, K, a.N, workspace, stride, (int)n, a.y, a.ldy, lim, st, b.W, b.y));
     }
     for (int i = 0; i < live; i++) {
         const GroupMat &m = gm[i];

@@ -54,7 +54,13 @@ template <int WT, int NT, int NW> __host__ __device__ constexpr size_t mmv_q4k_l
 template <int WT, int NT, int NW, int OCC>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
-                    size_t ws_stride, int n, float *__restrict__ y, int64_t ldy) {
+                    size_t ws_stride, int n, float *__restrict__ y, int64_t ldy, const uint8_t *__restrict__ W2,
+                    float *__restrict__ y2) {
+    // Two matrices of one shape on the same activation rows (ffn_gate and ffn_up): the second half of the grid works on
+    // W2 / y2 with the tile ranges the first half has on W / y, so either result is what a launch of its own returns.
+    const uint32_t grid = W2 ? gridDim.x / 2 : gridDim.x;
+    const uint32_t block = blockIdx.x >= grid ? blockIdx.x - grid : blockIdx.x;
+    if (blockIdx.x >= grid) { W = W2; y = y2; }
     constexpr int WGS = NW * 64;
     constexpr int KQ_ROW_BYTES = KqGeom<WT>::ROW_BYTES, KQ_MACRO_BYTES = KqGeom<WT>::MACRO_BYTES, KQ_CHUNKS = KqGeom<WT>::CHUNKS;
     constexpr int CPR = KqGeom<WT>::CHUNKS_PER_ROW;
@@ -82,7 +88,7 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     // tiles of 16 rows: a contiguous range per workgroup, in rounds of TC <= 4 tiles whose (tile, macro step) items are
     // split evenly over the waves; a wave's share touches at most two tiles
     const uint32_t tiles = (uint32_t)ceil_div(N, 16);
-    const uint32_t t_begin = tiles * blockIdx.x / gridDim.x, t_end = tiles * (blockIdx.x + 1) / gridDim.x;
+    const uint32_t t_begin = tiles * block / grid, t_end = tiles * (block + 1) / grid;
     const int T = (int)(t_end - t_begin);
     const int rounds = (T + 3) / 4;
     const int TCmax = rounds ? (T + rounds - 1) / rounds : 0;
@@ -338,7 +344,7 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
 
 template <int WT, int NT, int NW, int OCC>
 hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
-                      int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                      int64_t ldy, const DeviceLimits &lim, hipStream_t st, const void *W2, float *y2) {
     const size_t lds_bytes = mmv_q4k_lds_bytes<WT, NT, NW>(K);
     auto kfn = mmv_q4k_kernel<WT, NT, NW, OCC>;
     static LdsGrant grant;
@@ -347,8 +353,8 @@ hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const vo
     const int64_t tiles = ceil_div(N, 16);
     constexpr int per_cu = OCC * 4 / NW;
     const int64_t groups = tiles < (int64_t)cus * per_cu ? tiles : (int64_t)cus * per_cu;
-    hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(NW * 64), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
-                       (const uint8_t *)ws, ws_stride, n, y, ldy);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)(W2 ? 2 * groups : groups)), dim3(NW * 64), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                       (const uint8_t *)ws, ws_stride, n, y, ldy, (const uint8_t *)W2, y2);
     return hipGetLastError();
 }
 
@@ -361,16 +367,16 @@ template <int WT> int max_tokens_typed(int64_t K, const DeviceLimits &lim) {
 }
 template <int WT>
 hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,
-                        int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
+                        int64_t ldy, const DeviceLimits &lim, hipStream_t st, const void *W2, float *y2) {
     if (n <= 8) {
         if (mmv_q4k_lds_bytes<WT, 8, 8>(K) <= (size_t)lim.max_lds_per_block)
-            return launch_cfg<WT, 8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+            return launch_cfg<WT, 8, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st, W2, y2);
         if (mmv_q4k_lds_bytes<WT, 8, 6>(K) <= (size_t)lim.max_lds_per_block)
-            return launch_cfg<WT, 8, 6, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+            return launch_cfg<WT, 8, 6, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st, W2, y2);
         return hipErrorInvalidValue;
     }
     if (mmv_q4k_lds_bytes<WT, 16, 8>(K) > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
-    return launch_cfg<WT, 16, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+    return launch_cfg<WT, 16, 8, 2>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st, W2, y2);
 }
 
 }  // namespace
@@ -385,12 +391,13 @@ int mmv_q4k_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim)
     return wtype == T_Q4_K ? max_tokens_typed<T_Q4_K>(K, lim) : max_tokens_typed<T_Q5_K>(K, lim);
 }
 
+// W2 / y2: NULL, or a second matrix of the same type, shape and strides that reads the same rows (one launch for both).
 hipError_t launch_mmv_q4k(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
-                          float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st) {
-    if (n < 1 || n > 16 || (wtype != T_Q4_K && wtype != T_Q5_K)) return hipErrorInvalidValue;
+                          float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const void *W2, float *y2) {
+    if (n < 1 || n > 16 || (wtype != T_Q4_K && wtype != T_Q5_K) || (W2 == nullptr) != (y2 == nullptr)) return hipErrorInvalidValue;
     if (N <= 0) return hipSuccess;
-    return wtype == T_Q4_K ? launch_typed<T_Q4_K>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st)
-                           : launch_typed<T_Q5_K>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st);
+    return wtype == T_Q4_K ? launch_typed<T_Q4_K>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st, W2, y2)
+                           : launch_typed<T_Q5_K>(W, nb01, K, N, ws, ws_stride, n, y, ldy, lim, st, W2, y2);
 }
 
 }  // namespace chip

@@ -182,7 +182,7 @@ int        mmv_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &l
 // gemv_mfma_q4k.hip: the Q4_K / Q5_K form (activations in the split Q8_K layout); reached through the two functions above.
 int        mmv_q4k_max_tokens(int wtype, int64_t K, int64_t N, const DeviceLimits &lim);
 hipError_t launch_mmv_q4k(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
-                          float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st);
+                          float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const void *W2 = nullptr, float *y2 = nullptr);
 // gemv_mfma_q4_0.hip: the Q4_0 form (activations in the split Q8_0 layout).
 int        mmv_q4_0_max_tokens(int64_t K, int64_t N, const DeviceLimits &lim);
 hipError_t launch_mmv_q4_0(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n, float *y,

@@ -152,7 +152,8 @@ CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, i
                               const void *workspace, float *y, int64_t ldy, void *stream);
 /* Two matmuls of one type, shape and row stride on the same activation (ffn_gate and ffn_up, llama-graph.cpp:562-690):
  * up to 4 tokens both run in one launch of the GEMV that quantizes in its prologue; with more tokens the activation is
- * quantized once and each matrix takes its usual path.  Results as from two chip_mul_mat calls. */
+ * quantized once and each matrix takes its usual path (5..8 tokens, Q4_K / Q5_K matrices that would each take the
+ * matrix-core GEMV: one launch of it over both).  Results as from two chip_mul_mat calls, bit for bit. */
 CHIP_API int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                int64_t ldx, int64_t n, float *y1, float *y2, int64_t ldy, void *workspace, size_t workspace_bytes,
                                void *stream);

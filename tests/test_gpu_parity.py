@@ -321,6 +321,27 @@ def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
         check_outputs(y2, ref["y"], ref["sum_abs"], "second matrix of the pair, n = %d" % n)
 
 
+@pytest.mark.parametrize("wt,K,N", [(O.Q4_K, 4096, 8192), (O.Q4_K, 4096, 14336), (O.Q5_K, 2048, 16400), (O.Q4_K, 14336, 4096)],
+                         ids=["q4_K-8192x4096", "q4_K-14336x4096", "q5_K-16400x2048", "q4_K-4096x14336"])
+def test_mul_mat_pair_on_the_matrix_cores(dev, orc, wt, K, N):
+    """ffn_gate and ffn_up at 5..8 tokens: matrices large enough for the matrix-core GEMV run as one launch, through
+    chip_mul_mat_pair and through chip_mul_mat_group (fp32 rows and prepared rows); each output equals the single call's bit
+    for bit (a row count that is no multiple of 16 puts a partial tile at the end of each matrix), oracle within tolerance."""
+    w1 = quantized_weights(wt, K + N, N, K)
+    w2 = quantized_weights(wt, K + N + 1, N, K)
+    for n in (5, 7, 8):
+        x = common.activations_f32(K + n, n, K)
+        a, b = dev.mul_mat(wt, w1, x), dev.mul_mat(wt, w2, x)
+        y1, y2 = dev.mul_mat_pair(wt, w1, w2, x)
+        assert y1.tobytes() == a.tobytes() and y2.tobytes() == b.tobytes(), n
+        for prepared in (False, True):
+            g1, g2 = dev.mul_mat_group([(wt, w1), (wt, w2)], x, prepared=prepared)[:2]
+            assert g1.tobytes() == a.tobytes() and g2.tobytes() == b.tobytes(), (n, prepared)
+        if n == 8:
+            ref = orc.mul_mat(wt, w2, x, nthreads=8, want=("sum_abs",))
+            check_outputs(y2, ref["y"], ref["sum_abs"], "second matrix of the pair, n = 8")
+
+
 @pytest.mark.parametrize("wt", (O.Q6_K, O.Q4_K, O.Q8_0, O.Q4_0), ids=lambda t: O.TYPE_NAMES[t])
 def test_mul_mat_with_transposed_fp16_store(dev, wt):
     """chip_mul_mat_store_t (the V projection and its store into the transposed F16 cache): y equals chip_mul_mat's bit for
