@@ -25,6 +25,7 @@
 #include "dev_common.h"
 #include "act_layout.h"
 #include <cstdlib>
+#include <type_traits>
 
 namespace chip {
 
@@ -114,78 +115,117 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     };
 
     // ---- prologue: activation loads, then the first macro tile's weight loads, then the LDS images ----
+    // Every load instruction of the prologue costs the same whether one lane or all of them use its result, so the n rows
+    // are spread over the threads as flat lists of (token, piece) items - n * K / 16 chunks of quants, n * K / 256 scales,
+    // n * K / 32 pairs of block sums - with as many register slots as the workgroup needs for them; a thread past the end
+    // of a list loads the last item again and dumps it into the idle macro-tile buffers (all loads unconditional: a load
+    // inside a branch makes the compiler wait for everything in flight).  Rows n .. NT-1 of the images are zeros.
     u32x4 v[3];
     {
         const int nchunk = (int)(K / 16), nsb = (int)(K / 256), nsub = (int)(K / 32);
-        u32x4 qv[8][2];
-        float dv[8];
-        uint32_t bv[8];
-        auto load_batch = [&](int tb) {
+        const int q_items = n * nchunk, d_items = n * nsb, b_items = n * nsub;
+        const uint32_t dump = buf_off + 16u * (threadIdx.x % (NW * KQ_CHUNKS));
+        // item -> (token, piece): idx / den through the reciprocal, corrected by one (idx < 2^20)
+        auto divmod = [](int idx, int den, float rcp, int &q, int &r) {
+            q = (int)((float)idx * rcp);
+            r = idx - q * den;
+            if (r < 0) { q--; r += den; } else if (r >= den) { q++; r -= den; }
+        };
+        const float rc_chunk = 1.0f / (float)nchunk, rc_sb = 1.0f / (float)nsb, rc_sub = 1.0f / (float)nsub;
+        auto q_item = [&](int idx, const u32x4 *&src, uint32_t &dst) {
+            int t, c;
+            divmod(min(idx, q_items - 1), nchunk, rc_chunk, t, c);
+            src = reinterpret_cast<const u32x4 *>(ws + (size_t)t * ws_stride + 16 * (size_t)c);
+            dst = idx < q_items ? (uint32_t)t * q_stride + 16u * (uint32_t)c : dump;
+        };
+        auto d_item = [&](int idx, const float *&src, uint32_t &dst) {
+            int t, sb;
+            divmod(min(idx, d_items - 1), nsb, rc_sb, t, sb);
+            src = reinterpret_cast<const float *>(ws + (size_t)t * ws_stride + q8_K_off_d(K)) + sb;
+            dst = idx < d_items ? dx_base + 4u * (uint32_t)(sb * 16 + t) : dump;
+        };
+        auto b_item = [&](int idx, const uint32_t *&src, uint32_t &dst) {                  // two int16 block sums of a 32-value sub-block
+            int t, sub;
+            divmod(min(idx, b_items - 1), nsub, rc_sub, t, sub);
+            src = reinterpret_cast<const uint32_t *>(ws + (size_t)t * ws_stride + q8_K_off_bsums(K)) + sub;
+            dst = idx < b_items ? bs_base + 4u * (uint32_t)(sub * 16 + t) : dump;
+        };
+        auto pair_sum = [](uint32_t p) { return (int)(int16_t)(p & 0xffffu) + (int)(int16_t)(p >> 16); };
+        auto stage = [&](auto slots) {
+            constexpr int QL = decltype(slots)::value, BL = QL / 2, DL = 2;
+            u32x4 qv[QL];
+            uint32_t qdst[QL], bv[BL], bdst[BL], ddst[DL];
+            float dv[DL];
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const uint8_t *tokp = ws + (size_t)min(tb + i, n - 1) * ws_stride;
+            for (int j = 0; j < QL; j++) {
+                const u32x4 *src;
+                q_item(j * WGS + (int)threadIdx.x, src, qdst[j]);
+                qv[j] = *src;
+            }
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int c = min(j * WGS + (int)threadIdx.x, nchunk - 1);       // unconditional, clamped
-                    qv[i][j] = *reinterpret_cast<const u32x4 *>(tokp + 16 * (size_t)c);
-                }
-                dv[i] = reinterpret_cast<const float *>(tokp + q8_K_off_d(K))[min((int)threadIdx.x, nsb - 1)];
-                bv[i] = reinterpret_cast<const uint32_t *>(tokp + q8_K_off_bsums(K))[min((int)threadIdx.x, nsub - 1)];   // two int16 bsums
+            for (int j = 0; j < DL; j++) {
+                const float *src;
+                d_item(j * WGS + (int)threadIdx.x, src, ddst[j]);
+                dv[j] = *src;
+            }
+#pragma unroll
+            for (int j = 0; j < BL; j++) {
+                const uint32_t *src;
+                b_item(j * WGS + (int)threadIdx.x, src, bdst[j]);
+                bv[j] = *src;
+            }
+            __builtin_amdgcn_sched_barrier(0);                           // activations are requested before weights
+            {
+                Seg s0 = segment(0, 0);
+                s0.tile = min(s0.tile, tiles - 1);
+                s0.m0 = max(0, min(s0.m0, np - 1));
+                uint32_t co[3];
+                macro_offsets(co, s0.tile);
+                const uint8_t *tb = W + (size_t)s0.tile * 16 * nb01 + (size_t)s0.m0 * KQ_ROW_BYTES;
+#pragma unroll
+                for (int j = 0; j < 3; j++) v[j] = *reinterpret_cast<const u32x4 *>(tb + co[j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < QL; j++) *reinterpret_cast<u32x4 *>(lds + qdst[j]) = qv[j];
+#pragma unroll
+            for (int j = 0; j < DL; j++) *reinterpret_cast<float *>(lds + ddst[j]) = dv[j];
+#pragma unroll
+            for (int j = 0; j < BL; j++) *reinterpret_cast<int *>(lds + bdst[j]) = pair_sum(bv[j]);
+            // lists longer than the slots (rows wider than 16384 values at 8 tokens): the rest in plain loops
+            for (int idx = QL * WGS + (int)threadIdx.x; idx < q_items; idx += WGS) {
+                const u32x4 *src;
+                uint32_t dst;
+                q_item(idx, src, dst);
+                *reinterpret_cast<u32x4 *>(lds + dst) = *src;
+            }
+            for (int idx = DL * WGS + (int)threadIdx.x; idx < d_items; idx += WGS) {
+                const float *src;
+                uint32_t dst;
+                d_item(idx, src, dst);
+                *reinterpret_cast<float *>(lds + dst) = *src;
+            }
+            for (int idx = BL * WGS + (int)threadIdx.x; idx < b_items; idx += WGS) {
+                const uint32_t *src;
+                uint32_t dst;
+                b_item(idx, src, dst);
+                *reinterpret_cast<int *>(lds + dst) = pair_sum(*src);
             }
         };
-        auto store_batch = [&](int tb) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int c = j * WGS + (int)threadIdx.x;
-                    const u32x4 z = {0u, 0u, 0u, 0u};
-                    // a thread past the end of a row dumps its clamped duplicate into the idle macro-tile buffers
-                    const uint32_t dst = c < nchunk ? (uint32_t)(tb + i) * q_stride + 16u * c : buf_off + 16u * (threadIdx.x % (NW * KQ_CHUNKS));
-                    *reinterpret_cast<u32x4 *>(lds + dst) = (tb + i < n) ? qv[i][j] : z;
-                }
-                if ((int)threadIdx.x < nsb) reinterpret_cast<float *>(lds + dx_base)[threadIdx.x * 16 + tb + i] = (tb + i < n) ? dv[i] : 0.f;
-                if ((int)threadIdx.x < nsub) {
-                    const int s = (int)(int16_t)(bv[i] & 0xffffu) + (int)(int16_t)(bv[i] >> 16);
-                    reinterpret_cast<int *>(lds + bs_base)[threadIdx.x * 16 + tb + i] = (tb + i < n) ? s : 0;
-                }
-            }
-            for (int c = 2 * WGS + (int)threadIdx.x; c < nchunk; c += WGS)
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    u32x4 t = {0u, 0u, 0u, 0u};
-                    if (tb + i < n) t = *reinterpret_cast<const u32x4 *>(ws + (size_t)(tb + i) * ws_stride + 16 * (size_t)c);
-                    *reinterpret_cast<u32x4 *>(lds + (uint32_t)(tb + i) * q_stride + 16u * c) = t;
-                }
-            for (int b = WGS + (int)threadIdx.x; b < nsub; b += WGS)
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    int s = 0;
-                    if (tb + i < n) {
-                        const uint32_t p = reinterpret_cast<const uint32_t *>(ws + (size_t)(tb + i) * ws_stride + q8_K_off_bsums(K))[b];
-                        s = (int)(int16_t)(p & 0xffffu) + (int)(int16_t)(p >> 16);
-                    }
-                    reinterpret_cast<int *>(lds + bs_base)[b * 16 + tb + i] = s;
-                }
-        };
-        load_batch(0);
-        __builtin_amdgcn_sched_barrier(0);                               // activations are requested before weights
-        {
-            Seg s0 = segment(0, 0);
-            s0.tile = min(s0.tile, tiles - 1);
-            s0.m0 = max(0, min(s0.m0, np - 1));
-            uint32_t co[3];
-            macro_offsets(co, s0.tile);
-            const uint8_t *tb = W + (size_t)s0.tile * 16 * nb01 + (size_t)s0.m0 * KQ_ROW_BYTES;
-#pragma unroll
-            for (int j = 0; j < 3; j++) v[j] = *reinterpret_cast<const u32x4 *>(tb + co[j]);
+        const int need = (q_items + WGS - 1) / WGS;
+        if (need <= 4) stage(std::integral_constant<int, 4>{});
+        else if (need <= 8) stage(std::integral_constant<int, 8>{});
+        else stage(std::integral_constant<int, 16>{});
+        // rows n .. NT-1: zeros
+        for (int i = (int)threadIdx.x; i < (NT - n) * nchunk; i += WGS) {
+            int t, c;
+            divmod(i, nchunk, rc_chunk, t, c);
+            *reinterpret_cast<u32x4 *>(lds + (uint32_t)(n + t) * q_stride + 16u * (uint32_t)c) = u32x4{0u, 0u, 0u, 0u};
         }
-        __builtin_amdgcn_sched_barrier(0);
-        store_batch(0);
-        if constexpr (NT == 16) {
-            load_batch(8);
-            store_batch(8);
-        }
+        for (int i = (int)threadIdx.x; i < nsb * NT; i += WGS)
+            if ((i & (NT - 1)) >= n) reinterpret_cast<float *>(lds + dx_base)[(i / NT) * 16 + (i & (NT - 1))] = 0.f;
+        for (int i = (int)threadIdx.x; i < nsub * NT; i += WGS)
+            if ((i & (NT - 1)) >= n) reinterpret_cast<int *>(lds + bs_base)[(i / NT) * 16 + (i & (NT - 1))] = 0;
         if (threadIdx.x < 64) reinterpret_cast<uint32_t *>(lds + zero_off)[threadIdx.x] = 0u;
     }
     __syncthreads();
