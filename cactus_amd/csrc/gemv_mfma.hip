@@ -24,6 +24,7 @@
 #include "kernels.h"
 #include "dev_common.h"
 #include "act_layout.h"
+#include "mmv_stage.h"
 
 namespace chip {
 
@@ -98,60 +99,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OC
     // ---- prologue: activation loads, then the first macro tile's weight loads, then the LDS image ----
     u32x4 v[5];
     {
-        // activation loads: row-contiguous 16-byte chunks (two per token and thread cover K <= 32 * WGS), one scale
-        // per token and thread (K / 32 <= WGS); tokens in batches of 8 to bound the registers
-        const int nchunk = (int)(K / 16), nblk = (int)(K / 32);
-        u32x4 qv[8][2];
-        float dv[8];
-        auto load_batch = [&](int tb) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const uint8_t *tokp = ws + (size_t)min(tb + i, n - 1) * ws_stride;
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    // unconditional loads (clamped addresses) keep all of them in flight together
-                    const int c = min(j * WGS + (int)threadIdx.x, nchunk - 1);
-                    qv[i][j] = *reinterpret_cast<const u32x4 *>(tokp + 16 * (size_t)c);
-                }
-                dv[i] = reinterpret_cast<const float *>(tokp + q8_0_off_d(K))[min((int)threadIdx.x, nblk - 1)];
-            }
-        };
-        // The stores are unconditional as well (a conditional store lets the compiler sink its load into the
-        // branch, behind the weight loads): a thread past the end of a row dumps its clamped duplicate into the
-        // macro-tile buffers, which are idle during the prologue.
-        auto store_batch = [&](int tb) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int c = j * WGS + (int)threadIdx.x;
-                    const u32x4 z = {0u, 0u, 0u, 0u};
-                    const uint32_t dst = c < nchunk ? (uint32_t)(tb + i) * q_stride + 16u * c : buf_off + 16u * threadIdx.x;
-                    *reinterpret_cast<u32x4 *>(lds + dst) = (tb + i < n) ? qv[i][j] : z;
-                }
-                const uint32_t dd = (int)threadIdx.x < nblk ? q_bytes + 4u * (threadIdx.x * 16 + tb + i) : buf_off + 16u * WGS + 4u * threadIdx.x;
-                *reinterpret_cast<float *>(lds + dd) = (tb + i < n) ? dv[i] : 0.f;
-            }
-            // rows longer than the register slots
-            for (int c = 2 * WGS + (int)threadIdx.x; c < nchunk; c += WGS)
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    u32x4 t = {0u, 0u, 0u, 0u};
-                    if (tb + i < n) t = *reinterpret_cast<const u32x4 *>(ws + (size_t)(tb + i) * ws_stride + 16 * (size_t)c);
-                    *reinterpret_cast<u32x4 *>(lds + (uint32_t)(tb + i) * q_stride + 16u * c) = t;
-                }
-            for (int b = WGS + (int)threadIdx.x; b < nblk; b += WGS)
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    float t = 0.f;
-                    if (tb + i < n) t = reinterpret_cast<const float *>(ws + (size_t)(tb + i) * ws_stride + q8_0_off_d(K))[b];
-                    reinterpret_cast<float *>(lds + q_bytes)[b * 16 + tb + i] = t;
-                }
-        };
-        load_batch(0);
-        __builtin_amdgcn_sched_barrier(0);                               // activations are requested before weights
-        {
-            // the wave's first macro tile (clamped into the matrix if the wave has no work: loaded, never used)
+        // the n rows into the LDS image (mmv_stage.h); between their loads and their stores, the wave's first macro tile
+        // (clamped into the matrix if the wave has no work: loaded, never used)
+        mmv_stage_q8_0_rows<NT, WGS>(lds, ws, ws_stride, n, K, q_stride, q_bytes, buf_off + 32u * threadIdx.x, [&] {
             Seg s0 = segment(0, 0);
             s0.tile = min(s0.tile, tiles - 1);
             s0.m0 = max(0, min(s0.m0, np - 1));
@@ -160,13 +110,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OC
             const uint8_t *tb = W + (size_t)s0.tile * 16 * nb01 + (size_t)s0.m0 * MMV_ROW_BYTES;
 #pragma unroll
             for (int j = 0; j < 5; j++) v[j] = *reinterpret_cast<const u32x4 *>(tb + co[j]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        store_batch(0);
-        if constexpr (NT == 16) {                                        // NT == 8 never reads tokens 8..15 of the scale image
-            load_batch(8);
-            store_batch(8);
-        }
+        });
         if (threadIdx.x < 64) reinterpret_cast<uint32_t *>(lds + zero_off)[threadIdx.x] = 0u;
     }
     __syncthreads();

@@ -132,23 +132,47 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
             if (r < 0) { q--; r += den; } else if (r >= den) { q++; r -= den; }
         };
         const float rc_chunk = 1.0f / (float)nchunk, rc_sb = 1.0f / (float)nsb, rc_sub = 1.0f / (float)nsub;
+        // (token, piece) of item idx, the last item's past the end of the list
+        auto q_place = [&](int idx, int t, int c, const u32x4 *&src, uint32_t &dst) {
+            const bool in = idx < q_items;
+            t = in ? t : n - 1;
+            c = in ? c : nchunk - 1;
+            src = reinterpret_cast<const u32x4 *>(ws + (size_t)t * ws_stride + 16 * (size_t)c);
+            dst = in ? (uint32_t)t * q_stride + 16u * (uint32_t)c : dump;
+        };
+        auto d_place = [&](int idx, int t, int sb, const float *&src, uint32_t &dst) {
+            const bool in = idx < d_items;
+            t = in ? t : n - 1;
+            sb = in ? sb : nsb - 1;
+            src = reinterpret_cast<const float *>(ws + (size_t)t * ws_stride + q8_K_off_d(K)) + sb;
+            dst = in ? dx_base + 4u * (uint32_t)(sb * 16 + t) : dump;
+        };
+        auto b_place = [&](int idx, int t, int sub, const uint32_t *&src, uint32_t &dst) {   // two int16 block sums of a 32-value sub-block
+            const bool in = idx < b_items;
+            t = in ? t : n - 1;
+            sub = in ? sub : nsub - 1;
+            src = reinterpret_cast<const uint32_t *>(ws + (size_t)t * ws_stride + q8_K_off_bsums(K)) + sub;
+            dst = in ? bs_base + 4u * (uint32_t)(sub * 16 + t) : dump;
+        };
         auto q_item = [&](int idx, const u32x4 *&src, uint32_t &dst) {
             int t, c;
-            divmod(min(idx, q_items - 1), nchunk, rc_chunk, t, c);
-            src = reinterpret_cast<const u32x4 *>(ws + (size_t)t * ws_stride + 16 * (size_t)c);
-            dst = idx < q_items ? (uint32_t)t * q_stride + 16u * (uint32_t)c : dump;
+            divmod(idx, nchunk, rc_chunk, t, c);
+            q_place(idx, t, c, src, dst);
         };
         auto d_item = [&](int idx, const float *&src, uint32_t &dst) {
             int t, sb;
-            divmod(min(idx, d_items - 1), nsb, rc_sb, t, sb);
-            src = reinterpret_cast<const float *>(ws + (size_t)t * ws_stride + q8_K_off_d(K)) + sb;
-            dst = idx < d_items ? dx_base + 4u * (uint32_t)(sb * 16 + t) : dump;
+            divmod(idx, nsb, rc_sb, t, sb);
+            d_place(idx, t, sb, src, dst);
         };
-        auto b_item = [&](int idx, const uint32_t *&src, uint32_t &dst) {                  // two int16 block sums of a 32-value sub-block
+        auto b_item = [&](int idx, const uint32_t *&src, uint32_t &dst) {
             int t, sub;
-            divmod(min(idx, b_items - 1), nsub, rc_sub, t, sub);
-            src = reinterpret_cast<const uint32_t *>(ws + (size_t)t * ws_stride + q8_K_off_bsums(K)) + sub;
-            dst = idx < b_items ? bs_base + 4u * (uint32_t)(sub * 16 + t) : dump;
+            divmod(idx, nsub, rc_sub, t, sub);
+            b_place(idx, t, sub, src, dst);
+        };
+        // a thread's items are WGS apart: one division each for the first, then steps of (WGS / den, WGS % den) with a carry
+        auto advance = [](int &t, int &c, int den) {
+            t += WGS / den; c += WGS % den;
+            if (c >= den) { c -= den; t++; }
         };
         auto pair_sum = [](uint32_t p) { return (int)(int16_t)(p & 0xffffu) + (int)(int16_t)(p >> 16); };
         auto stage = [&](auto slots) {
@@ -156,23 +180,30 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
             u32x4 qv[QL];
             uint32_t qdst[QL], bv[BL], bdst[BL], ddst[DL];
             float dv[DL];
+            int t, c;
+            divmod((int)threadIdx.x, nchunk, rc_chunk, t, c);
 #pragma unroll
             for (int j = 0; j < QL; j++) {
                 const u32x4 *src;
-                q_item(j * WGS + (int)threadIdx.x, src, qdst[j]);
+                q_place(j * WGS + (int)threadIdx.x, t, c, src, qdst[j]);
                 qv[j] = *src;
+                advance(t, c, nchunk);
             }
+            divmod((int)threadIdx.x, nsb, rc_sb, t, c);
 #pragma unroll
             for (int j = 0; j < DL; j++) {
                 const float *src;
-                d_item(j * WGS + (int)threadIdx.x, src, ddst[j]);
+                d_place(j * WGS + (int)threadIdx.x, t, c, src, ddst[j]);
                 dv[j] = *src;
+                advance(t, c, nsb);
             }
+            divmod((int)threadIdx.x, nsub, rc_sub, t, c);
 #pragma unroll
             for (int j = 0; j < BL; j++) {
                 const uint32_t *src;
-                b_item(j * WGS + (int)threadIdx.x, src, bdst[j]);
+                b_place(j * WGS + (int)threadIdx.x, t, c, src, bdst[j]);
                 bv[j] = *src;
+                advance(t, c, nsub);
             }
             __builtin_amdgcn_sched_barrier(0);                           // activations are requested before weights
             {
@@ -215,6 +246,7 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
         const int need = (q_items + WGS - 1) / WGS;
         if (need <= 4) stage(std::integral_constant<int, 4>{});
         else if (need <= 8) stage(std::integral_constant<int, 8>{});
+        else if (need <= 12) stage(std::integral_constant<int, 12>{});
         else stage(std::integral_constant<int, 16>{});
         // rows n .. NT-1: zeros
         for (int i = (int)threadIdx.x; i < (NT - n) * nchunk; i += WGS) {
