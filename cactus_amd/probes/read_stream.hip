@@ -32,6 +32,36 @@ __global__ __launch_bounds__(256) void k_read(const uint8_t* __restrict__ cur, s
 }
 __global__ void k_empty(uint32_t* out){ if(threadIdx.x==9999) out[0]=1; }
 
+// How many bytes a wave keeps in flight: D loads of 16 bytes per lane and iteration (D KB per wave), and with AHEAD the next
+// iteration's loads are requested before the current ones are consumed (a ring of one step, as the GEMV has it).
+template<int D, bool AHEAD>
+__global__ __launch_bounds__(256) void k_depth(const uint8_t* __restrict__ p, size_t bytes, uint32_t* out){
+  const int lane=threadIdx.x&63; const size_t nw=(size_t)gridDim.x*4, wave=(size_t)blockIdx.x*4+(threadIdx.x>>6), per_wave=(size_t)D*1024;
+  uint32_t acc=0; u32x4 v[D], w[D];
+  size_t base=wave*per_wave;
+  if(AHEAD && base<bytes){
+    #pragma unroll
+    for(int j=0;j<D;j++) v[j]=*(const u32x4*)(p+base+j*1024+lane*16);
+  }
+  for(; base<bytes; base+=nw*per_wave){
+    if(AHEAD){
+      const size_t nb=base+nw*per_wave<bytes? base+nw*per_wave: base;      // the last iteration re-reads its own chunk
+      #pragma unroll
+      for(int j=0;j<D;j++) w[j]=*(const u32x4*)(p+nb+j*1024+lane*16);
+      #pragma unroll
+      for(int j=0;j<D;j++) acc+=v[j].x^v[j].y^v[j].z^v[j].w;
+      #pragma unroll
+      for(int j=0;j<D;j++) v[j]=w[j];
+    } else {
+      #pragma unroll
+      for(int j=0;j<D;j++) v[j]=*(const u32x4*)(p+base+j*1024+lane*16);
+      #pragma unroll
+      for(int j=0;j<D;j++) acc+=v[j].x^v[j].y^v[j].z^v[j].w;
+    }
+  }
+  if(acc==0x12345678) out[0]=acc;
+}
+
 int main(){
   const size_t total=(size_t)6<<30; uint8_t* d; CK(hipMalloc(&d,total)); CK(hipMemset(d,1,total)); uint32_t* out; CK(hipMalloc(&out,64));
   hipEvent_t e0,e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
@@ -52,6 +82,17 @@ int main(){
     }
     printf("read %6.1f MB (%-30s): cold %7.2f us = %4.0f GB/s = %4.1f %% of 8 TB/s (best of 512/1024/2048 workgroups: %d)   warm %7.2f us = %5.0f GB/s\n",
            bytes/1e6,c.what,best_cold,bytes/best_cold/1e3,bytes/best_cold/1e3/80.0,best_g,best_warm,bytes/best_warm/1e3);
+  }
+  // bytes in flight: D KB per wave and iteration, plain or one iteration ahead, 2 / 4 / 8 workgroups of four waves per CU
+  {
+    const size_t bytes=((size_t)(48.2e6))/(1<<16)*(1<<16); const int copies=(int)(total/bytes);
+    printf("48.2 MB cold, us per launch by KB per wave and iteration (plain | one iteration ahead), workgroups of 4 waves:\n");
+    auto run=[&](auto kfn,int G){ int idx=0; return elapsed([&]{ hipLaunchKernelGGL(kfn,dim3(G),dim3(256),0,0,d+(size_t)(idx++%copies)*bytes,bytes,out); }, copies<100?copies:100); };
+    for(int G:{512,1024,2048}){
+      printf("  %4d workgroups: 1 KB %6.2f | %6.2f   2 KB %6.2f | %6.2f   4 KB %6.2f | %6.2f   8 KB %6.2f | %6.2f   16 KB %6.2f | %6.2f\n",G,
+        run(k_depth<1,false>,G),run(k_depth<1,true>,G),run(k_depth<2,false>,G),run(k_depth<2,true>,G),run(k_depth<4,false>,G),run(k_depth<4,true>,G),
+        run(k_depth<8,false>,G),run(k_depth<8,true>,G),run(k_depth<16,false>,G),run(k_depth<16,true>,G));
+    }
   }
   // a chain of reads over rotating buffers, with P extra workgroups per kernel that already read the next buffer
   auto chain=[&](const char* name,std::vector<double> mbs,int G,int P){
