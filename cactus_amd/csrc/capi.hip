@@ -781,11 +781,11 @@ int chip_silu_mul(const float *x, int64_t ldx, const float *b, int64_t ldb, int6
 int chip_silu_mul_quantized(const float *x, int64_t ldx, const float *b, int64_t ldb, int64_t n, int64_t ne0, float *y, int64_t ldy,
                             int wtype, void *workspace, size_t workspace_bytes, void *stream) {
     if (n < 0 || ne0 < 0) return CHIP_EINVAL;
+    if (n == 0 || ne0 == 0) return CHIP_OK;
     if (!chip_mul_mat_supported(wtype, ne0)) return CHIP_EUNSUPPORTED;
     const int at = chip_vec_dot_type(wtype);
     const int kind = (at == T_Q8_0 || at == T_Q8_1) ? 1 : (at == T_Q8_K ? 2 : 0);
     if (kind == 0) return CHIP_EUNSUPPORTED;                               // F16 weights: plain fp16 rows, not done here
-    if (n == 0 || ne0 == 0) return CHIP_OK;
     if (!rows_ok(x, ldx, ne0) || !rows_ok(y, ldy, ne0) || !rows_ok(b, ldb, ne0) || n > 65535) return CHIP_EINVAL;
     if (!workspace || !aligned16(workspace)) return CHIP_EINVAL;
     if (workspace_bytes < chip_mul_mat_workspace_size(wtype, ne0, n)) return CHIP_ENOMEM;

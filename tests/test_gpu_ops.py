@@ -241,6 +241,28 @@ def test_silu_mul_that_leaves_quantized_rows(dev, orc, wt, n, ne0):
     assert dev.lib.chip_silu_mul_quantized(dx.ptr, 320, dx.ptr, 320, 2, 320, dyy.ptr, 320, ca.Q8_0, ws2.ptr, 4096, None) == ca.CHIP_EUNSUPPORTED
 
 
+def test_silu_mul_quantized_argument_errors(dev):
+    import cactus_amd as ca
+    L = dev.lib
+    ne0 = 512
+    a, ws = dev.to_device(inputs(5, 2, ne0)), dev.alloc(1 << 16)
+    y = dev.alloc(2 * ne0 * 4)
+    call = lambda **k: L.chip_silu_mul_quantized(k.get("x", a.ptr), k.get("ldx", ne0), k.get("b", a.ptr), ne0, k.get("n", 2), k.get("ne0", ne0),
+                                                 k.get("y", y.ptr), ne0, k.get("t", ca.Q4_K), k.get("ws", ws.ptr), k.get("wsz", 1 << 16), None)
+    assert call() == ca.CHIP_OK
+    assert call(n=0) == ca.CHIP_OK and call(ne0=0) == ca.CHIP_OK          # nothing to do
+    assert call(n=-1) == ca.CHIP_EINVAL
+    assert call(t=ca.F16) == ca.CHIP_EUNSUPPORTED                         # no quantized activation format
+    assert call(t=77) == ca.CHIP_EUNSUPPORTED
+    assert call(ws=None) == ca.CHIP_EINVAL and call(ws=ws.ptr + 4) == ca.CHIP_EINVAL
+    assert call(wsz=64) == ca.CHIP_ENOMEM
+    assert call(ldx=ne0 - 4) == ca.CHIP_EINVAL                            # rows overlap
+    assert call(x=a.ptr + 4) == ca.CHIP_EUNSUPPORTED                      # not 16-byte aligned: the caller takes chip_silu_mul
+    dev.sync()
+    for t in (a, ws, y):
+        t.free()
+
+
 @pytest.mark.parametrize("wt", ["Q4_K", "Q6_K", "Q8_0", "Q4_1"])
 @pytest.mark.parametrize("n,ne0", [(1, 4096), (9, 4096), (3, 256), (5, 8192), (40, 1024)])
 @pytest.mark.parametrize("with_add", [False, True])
