@@ -345,8 +345,9 @@ static int mmv_min_tokens(int type, int64_t K, int64_t N) {
            : (type == T_Q4_K && K > 13312) ? 7 : MMV_MIN_TOKENS;
 }
 // Two Q4_K / Q5_K matrices of one shape on the same rows at 5..8 tokens (ffn_gate and ffn_up): true when each alone would
-// take one launch of the matrix-core GEMV whatever the workspace size - they then run as one launch whose grid is the two
-// launches' grids side by side (every tile is computed as in a launch of its own: the same bits).
+// take one launch of the matrix-core GEMV whatever the workspace size - they then run as one launch in which every
+// workgroup, after its tiles of the first matrix, takes the same tiles of the second (the activation image is built once;
+// every tile is computed as in a launch of its own: the same bits).
 static bool mmv_pair_applicable(int type, int64_t K, int64_t N, int64_t n, const DeviceLimits &lim) {
     if (n < 5 || n > 8 || !(type == T_Q4_K || type == T_Q5_K) || tune("CHIP_MMV_PAIR", 1) == 0) return false;
     if (gemm_kq_supported(type, K, N, n, false) || gemm_kq_supported(type, K, N, n, true)) return false;

@@ -57,11 +57,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC, OC
 void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
                     size_t ws_stride, int n, float *__restrict__ y, int64_t ldy, const uint8_t *__restrict__ W2,
                     float *__restrict__ y2) {
-    // Two matrices of one shape on the same activation rows (ffn_gate and ffn_up): the second half of the grid works on
-    // W2 / y2 with the tile ranges the first half has on W / y, so either result is what a launch of its own returns.
-    const uint32_t grid = W2 ? gridDim.x / 2 : gridDim.x;
-    const uint32_t block = blockIdx.x >= grid ? blockIdx.x - grid : blockIdx.x;
-    if (blockIdx.x >= grid) { W = W2; y = y2; }
+    // Two matrices of one shape on the same activation rows (ffn_gate and ffn_up): after its tiles of W / y a workgroup
+    // takes the same tile range of W2 / y2, so either result is what a launch of its own returns and the activation
+    // image is built once.
+    const uint32_t grid = gridDim.x, block = blockIdx.x;
+    const int nmat = W2 ? 2 : 1;
     constexpr int WGS = NW * 64;
     constexpr int KQ_ROW_BYTES = KqGeom<WT>::ROW_BYTES, KQ_MACRO_BYTES = KqGeom<WT>::MACRO_BYTES, KQ_CHUNKS = KqGeom<WT>::CHUNKS;
     constexpr int CPR = KqGeom<WT>::CHUNKS_PER_ROW;
@@ -281,6 +281,8 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     const uint32_t qh_off = hdr + 16u + 16u * (g & 1);                  // Q5_K: the fifth bits of the same 16 elements
     const uint32_t nib_shift = 4u * (g >> 1);
 
+    for (int mat = 0; mat < nmat; mat++) {
+    if (mat == 1) { W = W2; y = y2; }
     for (int rd = 0; rd < rounds; rd++) {
         float4 part[2];
 #pragma unroll
@@ -291,7 +293,7 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
                 uint32_t co[3];
                 macro_offsets(co, sg.tile);
                 const uint8_t *tb = W + (size_t)sg.tile * 16 * nb01;
-                if (rd != 0 || seg != 0) {
+                if (rd != 0 || seg != 0 || mat != 0) {
 #pragma unroll
                     for (int j = 0; j < 3; j++) v[j] = *reinterpret_cast<const u32x4 *>(tb + (size_t)sg.m0 * KQ_ROW_BYTES + co[j]);
                 }
@@ -412,6 +414,7 @@ void mmv_q4k_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
         }
         __syncthreads();
     }
+    }
 }
 
 template <int WT, int NT, int NW, int OCC>
@@ -425,7 +428,7 @@ hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const vo
     const int64_t tiles = ceil_div(N, 16);
     constexpr int per_cu = OCC * 4 / NW;
     const int64_t groups = tiles < (int64_t)cus * per_cu ? tiles : (int64_t)cus * per_cu;
-    hipLaunchKernelGGL(kfn, dim3((unsigned)(W2 ? 2 * groups : groups)), dim3(NW * 64), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+    hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(NW * 64), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
                        (const uint8_t *)ws, ws_stride, n, y, ldy, (const uint8_t *)W2, y2);
     return hipGetLastError();
 }
