@@ -639,7 +639,7 @@ def bench_headline(dev, hip, trace, steps, warmup, eager):
     kernel_names = {"qkv": "gemv_group_kernel<K-quants, n=1> (wq Q4_K 4096x4096 + wk Q4_K 1024x4096 + wv Q6_K 1024x4096)",
                     "wo": "gemv_kernel<Q4_K, n=1, fused quantize> (4096x4096)",
                     "gate_up": "gemv_kernel<Q4_K, n=1, fused quantize> over ffn_gate + ffn_up (2 x 14336x4096, one launch)",
-                    "down": "quantize_q8_K_kernel + gemv_kernel<Q6_K, n=1, prepared rows> (4096x14336; Q6_K rows of more than 8192 values are quantized by their own launch)",
+                    "down": "gemv_kernel<Q6_K, n=1, fused quantize, image built a step's part at a time> (4096x14336)",
                     "head": "gemv_kernel<Q6_K, n=1, fused quantize> (128256x4096)"}
     roof = {"bound": "hbm", "achieved": d["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": d["hbm_frac"],
             "traffic": traffic_from_profile(dom), "kernel": kernel_names[dom], "op": dom,

@@ -23,12 +23,12 @@
 
 namespace chip {
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED>
 __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                                    const float *__restrict__ x, int64_t ldx,
                                                    uint8_t *__restrict__ ws, size_t ws_stride,
                                                    float *__restrict__ y, int64_t ldy, SecondMatrix sec) {
-    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
 }
 
 // LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
@@ -64,7 +64,21 @@ static hipError_t launch_depth(const void *W, size_t nb01, int64_t K, int64_t N,
     const int64_t tiles = ceil_div(N, R);
     int64_t groups = ceil_div(tiles, WGS / 64);
     if (groups > max_groups) groups = max_groups;
-    auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH>;
+    // Rows of more than one step whose activations the prologue quantizes to Q8_K: the kernel that builds the image a
+    // step's part at a time (gemv_body.h: PHASED)
+    if constexpr (FUSEQ && Traits<WT>::ACT == T_Q8_K && WGS >= 256) {
+        // (measured: 4096 x 14336 Q4_K 10.5 -> 9.5 us, 4096 x 11008 8.7 -> 8.0 us, Q6_K 4096 x 14336 15.3-16.1 -> 14.7 us;
+        //  two steps - K = 8192 - run 2 % slower that way and keep the plain prologue)
+        if (iters_per_row<WT>(K) > 2 && tune("CHIP_GEMV_PHASED", 1) != 0) {
+            auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, true>;
+            static LdsGrant grant;
+            if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
+            hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
+                               (uint8_t *)ws, ws_stride, y, ldy, sec);
+            return hipGetLastError();
+        }
+    }
+    auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false>;
     static LdsGrant grant;                                               // one per kernel instantiation
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
@@ -216,11 +230,11 @@ hipError_t launch_gemv_store_t(int wtype, const void *W, size_t nb01, int64_t K,
 bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
     if (!(n == 1 || n == 2 || n == 4) || (int64_t)n * K > FUSE_MAX_VALUES) return false;
     // Every workgroup repeats the quantizer, and its dependent chains (maximum, two divisions, sums) cost a wave about
-    // 0.9 us per 256 values.  For Q6_K rows of more than 8192 values the separate quantizer kernel (1.9 us) and the GEMV over
-    // prepared rows are ahead (4096 x 14336, one token: 1.97 + 12.6 us against 15.3-16.1 us in one launch); the other
-    // types keep the single launch at every length it takes (4096 x 11008 Q8_0 10.7 against 12.3 us in two launches,
-    // 4096 x 14336 Q4_K 10.5 against 10.8, Q8_0 13.7 against 14.9, Q4_0 4096 x 11008 9.1 either way).
-    if (wtype == T_Q6_K && n == 1 && K > 8192) return false;
+    // 0.9 us per 256 values.  With all of it in front of the first weight step, Q6_K rows of more than 8192 values ran
+    // faster as a quantizer kernel (1.9 us) and a GEMV over prepared rows (4096 x 14336, one token: 1.97 + 13.0 us against
+    // 15.3-16.1 us in one launch); with the image built a step's part at a time behind the previous step's arithmetic
+    // (gemv_body.h: PHASED) the single launch is ahead again (14.7 us), as it is for the other types at every length
+    // (4096 x 11008 Q8_0 10.7 against 12.3 us in two launches, 4096 x 14336 Q4_K 9.5 against 10.8, Q8_0 13.7 against 14.9).
     size_t img = 0;
     switch (wtype) {
         case T_Q4_0: img = lds_image_bytes<T_Q4_0>(K); break;

@@ -699,9 +699,12 @@ __device__ __forceinline__ void xload(XRegs<NTOK, WGS> &xr, const float *__restr
     }
 }
 
+// slot_lo, slot_hi (Q8_K activations only): the register slots [slot_lo, slot_hi) of every token, i.e. super-blocks
+// slot * (WGS / 64) .. - the caller may build the image a weight step's worth at a time.
 template <int WT, int NTOK, int WGS>
 __device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, uint8_t *lds, size_t img, int NI, int64_t K,
-                                                    uint8_t *__restrict__ ws, size_t ws_stride, bool first_block) {
+                                                    uint8_t *__restrict__ ws, size_t ws_stride, bool first_block,
+                                                    int slot_lo = 0, int slot_hi = XRegs<NTOK, WGS>::PER) {
     using T = Traits<WT>;
     constexpr int PER = XRegs<NTOK, WGS>::PER;
     const bool dump = first_block && ws != nullptr;
@@ -771,13 +774,14 @@ __device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, 
 #pragma unroll
             for (int j0 = 0; j0 < PER; j0 += FUSE_ILP) {
                 if (j0 * (WGS / 64) >= nsb) break;                      // uniform over the group
+                if (j0 + FUSE_ILP <= slot_lo || j0 >= slot_hi) continue;    // uniform: none of these slots is asked for
                 Q8_KLane q[FUSE_ILP];
 #pragma unroll
                 for (int u = 0; u < FUSE_ILP; u++)
-                    if (j0 + u < PER) q[u] = quantize_q8_K_lane(xr.v[t][j0 + u]);
+                    if (j0 + u < PER && j0 + u >= slot_lo && j0 + u < slot_hi) q[u] = quantize_q8_K_lane(xr.v[t][j0 + u]);
 #pragma unroll
                 for (int u = 0; u < FUSE_ILP; u++) {
-                    if (j0 + u >= PER) continue;
+                    if (j0 + u >= PER || j0 + u < slot_lo || j0 + u >= slot_hi) continue;
                     const int sb = (j0 + u) * (WGS / 64) + wv;
                     if (sb < nsb) {                                     // uniform over the wave
                         *reinterpret_cast<uint32_t *>(im + T::img_qs(NI, sb * 256 + 4 * lane)) = q[u].packed;
@@ -888,7 +892,7 @@ __device__ __forceinline__ GridPart whole_grid() { return GridPart{(int64_t)bloc
 struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; };
 constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0};
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH>
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                           const float *__restrict__ x, int64_t ldx,
                                           uint8_t *__restrict__ ws, size_t ws_stride,
@@ -939,7 +943,21 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
 
     // ---- prologue: activation loads first, then DEPTH steps of weight loads, then the activation image is built in LDS
     //      while the weights are still in flight ----
-    if constexpr (FUSEQ) {
+    // PHASED (rows of several steps with Q8_K activations, chosen by the launcher): a step reads the 16 super-blocks of its
+    // own part of the image, which are SPS register slots of every thread.  Only the first step's part is built before the
+    // first barrier; the part of step it + 1 is quantized behind the arithmetic of step it of the wave's first tile, while
+    // that step's weights are on their way - the quantizer's vector work (a third of a 14336-value row's kernel when it all
+    // stood in front) then fills time the waves would spend waiting.  Every wave, with or without a tile, takes part in
+    // every part and barrier.  The fp32 registers live until the last part, which is why this is a kernel of its own.
+    constexpr int SPS = 16 / (WGS / 64) > 0 ? 16 / (WGS / 64) : 1;      // slots per step
+    static_assert(!PHASED || (FUSEQ && T::ACT == T_Q8_K && WGS >= 256 && (SPS % FUSE_ILP == 0 || SPS == 1)),
+                  "parts of the image are whole quantizer slots");
+    [[maybe_unused]] XRegs<NTOK, (PHASED ? WGS : 64)> xr_parts;
+    if constexpr (FUSEQ && PHASED) {
+        xload<WT, NTOK, WGS>(xr_parts, x, ldx, K);
+        load_step(ring, s0, true);
+        quantize_into_image<WT, NTOK, WGS>(xr_parts, lds, img, NI, K, ws, ws_stride, gp.writes_workspace, 0, SPS);
+    } else if constexpr (FUSEQ) {
         XRegs<NTOK, WGS> xr;
         xload<WT, NTOK, WGS>(xr, x, ldx, K);
         load_step(ring, s0, true);
@@ -1009,6 +1027,19 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
         }
     };
 
+    if constexpr (PHASED) {
+        for (int it = 0; it < NI; it++) {                               // uniform over the workgroup
+            if (s0.have) {
+                const Step cur = s0;
+                s0 = after(cur);
+                consume(ring, cur, s0);
+            }
+            if (it + 1 < NI) {
+                quantize_into_image<WT, NTOK, WGS>(xr_parts, lds, img, NI, K, ws, ws_stride, gp.writes_workspace, (it + 1) * SPS, (it + 2) * SPS);
+                __syncthreads();
+            }
+        }
+    }
     // The stores of a batch of results stay out of the inner loop.
     while (s0.have) {
         while (s0.have && nres < 64) {
@@ -1019,6 +1050,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
         flush(nres);
         nres = 0;
     }
+    if constexpr (PHASED) flush(nres);                                  // a wave whose only tile went through the parts above
 }
 
 // Rows per wave step.  Two steps are in flight per wave (the next step's loads are issued before the current
