@@ -114,6 +114,27 @@ def test_mul_mat_vs_oracle(dev, orc, wt, K, N, n):
     check_outputs(y, ref["y"], ref["sum_abs"], "mul_mat")
 
 
+@pytest.mark.parametrize("wt,K,N", [(O.Q4_K, 11008, 5000), (O.Q6_K, 14336, 4500), (O.Q5_K, 12288, 2600), (O.Q6_K, 14336, 4096),
+                                    (O.Q4_K, 14336, 300)],
+                         ids=["q4_K-5000x11008", "q6_K-4500x14336", "q5_K-2600x12288", "q6_K-4096x14336", "q4_K-300x14336"])
+def test_long_rows_quantized_a_part_at_a_time(dev, orc, wt, K, N):
+    """One token, K-quant rows of three or four weight steps: the kernel builds its activation image a step's part at a time
+    behind the previous step's arithmetic, in workgroups of 4, 8 and 16 waves (by row count), with and without a second
+    tile per wave.  Activation bytes bit-exact, outputs within the tolerance and the same bits for every copy of a row; the
+    pair form (two matrices as one of twice the rows) returns the same bits."""
+    base = orc.quantize_weights(wt, common.weights_f32(K + N + wt, 100, K, outliers=(wt != O.Q6_K)))
+    W = np.tile(base, (N // 100 + 1, 1))[:N]
+    x = common.activations_f32(K + 3, 1, K)
+    ref = orc.mul_mat(wt, base, x, nthreads=8, want=("wdata", "sum_abs"))
+    y, blocks = dev.mul_mat(wt, W, x, want_workspace_blocks=True)
+    assert np.array_equal(blocks, ref["wdata"])
+    idx = np.arange(N) % 100
+    check_outputs(y, ref["y"][:, idx], ref["sum_abs"][:, idx], "rows of %d values" % K)
+    assert (y[0] == y[0, idx]).all()                                      # row r equals row r % 100
+    a, b = dev.mul_mat_pair(wt, W, np.ascontiguousarray(W[::-1]), x)
+    assert a.tobytes() == y.tobytes() and b.tobytes() == np.ascontiguousarray(y[:, ::-1]).tobytes()
+
+
 @pytest.mark.parametrize("wt", O.BLOCK_WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_block_integer_sums_bit_exact(dev, orc, wt):
     K, N, n = 2048, 9, 2
