@@ -8,29 +8,28 @@
 //     its K extent is exactly one 32-value quantization block, so each of the 1024 int32 results is one
 //     per-block integer sum isum[t][r][b], bit-exact.
 //   * Weight tiles are staged through LDS once per workgroup and k-stage: a block's packed quants are expanded into
-//     two 16-byte cells of signed int8 (elements 0..15 and 16..31), possibly times a power of two that the
-//     activation scale takes back (Q4_0: 16 * (nib - 8), Q5_0: 8 * (q - 16); IQ4_NL: the code point; Q8_0: as is);
-//     activations arrive as int8 from the split workspace layout.  Both sit in LDS as [k-block][half][row]
-//     16-byte cells, which is exactly what one lane feeds the MFMA (row = lane % 32, half = lane / 32).
+//     two 16-byte cells of signed int8 (elements 0..15 and 16..31), possibly times a power of two that is taken
+//     back exactly in the epilogue (Q4_0: 16 * (nib - 8), Q5_0: 8 * (q - 16); IQ4_NL: the code point; Q8_0: as is);
+//     activations arrive as int8 from the split workspace layout.
 //   * Per-block scales are applied in fp32 after the integer accumulate.  The MFMA's C input is a register
 //     vector holding the bit pattern of 12582912.0f (1.5 * 2^23): adding |isum| < 2^22 to those bits gives the
 //     bits of the float 12582912 + isum, so the accumulator can be used as a float with no conversion.  Then
 //         t   = fma(acc_as_float, dx, -12582912 * dx)      exactly round(isum * dx): 12582912*dx is exact
 //                                                           because dx comes from fp16 (11-bit significand)
-//         out = fma(t, dw, out)                            dw read as fp16 by the mixed-precision fma
+//         out = fma(t, dw, out)                            dw widened to fp32 exactly
 //     i.e. two VALU operations per integer sum, 32 per MFMA.  That VALU work, not the matrix pipe, bounds this
-//     kernel: an MFMA occupies the matrix unit for 32 cycles, 32 wave-wide fp32 operations occupy the vector
-//     unit for 128.
+//     kernel: an MFMA occupies the matrix unit for 32 cycles; the 32 fp32 operations, which read the MFMA's result
+//     registers, take 134 - 144 cycles per SIMD with two to four waves (measured in a register-only loop).
 //   * Q4_1 and Q5_1 add m * s per block (the weight block's minimum times the activation block's d * sum, the s of
 //     block_q8_1).  Both factors are fp16 numbers, so sum_b m[r][b] * s[t][b] over the 4 blocks of a stage is one
 //     v_mfma_f32_32x32x8f16 that adds straight into the fp32 accumulators: no vector work.
 //   * A workgroup is WR x WC waves, each wave owns TM x TN MFMA tiles (32*TM rows x 32*TN tokens); LDS is
-//     double buffered over stages of KB = 4 blocks with one barrier per stage and the next stage's global
-//     loads in flight during the current stage's arithmetic.
+//     double buffered over stages of KB = 4 blocks with one barrier per stage.
 #include "dev_common.h"
 #include "act_layout.h"
 #include "kernels.h"
 #include <cstdlib>
+#include <type_traits>
 
 namespace chip {
 
@@ -158,149 +157,164 @@ template <> struct Blk32<T_Q5_1> {
     }
 };
 
-template <int TM, int TN, int WR, int WC>
-struct GemmCfg {
+// ---- how the operands travel and how a wave orders its work ----
+//   * Quantized activations and their scales go from the workspace into LDS with global_load_lds_dwordx4: no staging
+//     registers, no ds_write, no vector instructions.  A token's 128 bytes of a stage are one LDS row of 8 cells; cell c of
+//     token t sits in slot c ^ ((t >> 1) & 7), so the 16 lanes that read one cell index of 16 consecutive tokens hit 16
+//     different bank groups (the lane that fills a slot fetches the matching cell).  The four fp32 scales of a token and
+//     stage are one more cell.
+//   * Weights pass through registers (their 18- to 34-byte blocks must be expanded to int8 cells); they are fetched
+//     two stages ahead and expanded one stage ahead, so a load has a whole stage to arrive.  The weight scales are
+//     widened to fp32 on the way into LDS: a mixed-precision FMA that reads them as fp16 issues at a lower rate than a
+//     plain one (measured: 16 + 16 plain FMAs behind an MFMA 56 - 60 ns per SIMD, with the second 16 mixed 67 - 80 ns).
+//   * Inside a stage the MFMA of tile i + 1 is issued before the 32 scaling operations of tile i, across k-blocks too,
+//     so one wave keeps the vector unit busy by itself and two waves per SIMD are enough; the stage loop is unrolled by
+//     two so that every LDS address is a register plus an immediate.
+//   * The power of two that the weight cells carry is taken back once, in the epilogue (exact), not per stage.
+// LDS cells: [k-block][half][row] 16-byte cells for the weights (exactly what one lane feeds the MFMA: row = lane % 32,
+// half = lane / 32), each plane padded by two cells: the threads that expand one stage walk the planes fastest, and a
+// plane stride that is 2 mod 16 cells puts 16 consecutive writers on 16 different bank groups.
+template <int TM, int TN, int WR, int WC, bool HAS_MIN>
+struct DirectCfg {
     static constexpr int NW = WR * WC, NT = NW * 64;
-    static constexpr int BM = 32 * TM * WR;                        // weight rows per workgroup
-    static constexpr int BN = 32 * TN * WC;                        // tokens per workgroup
-    // Each (k-block, half) plane of 16-byte cells is padded by two cells: the staging threads that write one
-    // stage walk the planes fastest, and a plane stride that is 2 mod 16 cells puts 16 consecutive writers on
-    // 16 different bank groups (unpadded, all of them hit the same banks).
-    static constexpr int A_PLANE = BM + 2, B_PLANE = BN + 2;
-    static constexpr int A_CELLS = GEMM_KB * 2 * A_PLANE;          // 16-byte cells
-    static constexpr int B_CELLS = GEMM_KB * 2 * B_PLANE;
+    static constexpr int BM = 32 * TM * WR, BN = 32 * TN * WC;
+    static constexpr int A_PLANE = BM + 2;                                        // cells
     static constexpr size_t OFF_A = 0;
-    static constexpr size_t OFF_B = OFF_A + (size_t)A_CELLS * 16;
-    static constexpr size_t OFF_SW = OFF_B + (size_t)B_CELLS * 16;                 // fp16 [KB][BM], permuted per 32 rows
-    static constexpr size_t OFF_SX = OFF_SW + (size_t)GEMM_KB * BM * 2;            // fp32 [KB][BN]
-    static constexpr size_t OFF_MW = OFF_SX + (size_t)GEMM_KB * BN * 4;            // fp16 [BM][KB]: block minimum (Q4_1, Q5_1)
-    static constexpr size_t OFF_MX = OFF_MW + (size_t)BM * GEMM_KB * 2;            // fp16 [BN][KB]: block_q8_1.s
-    static constexpr size_t STAGE = OFF_MX + (size_t)BN * GEMM_KB * 2;
-    static constexpr int W_ITEMS = BM * GEMM_KB;                   // (row, block) pairs per stage
-    static constexpr int W_PER_T = (W_ITEMS + NT - 1) / NT;
-    static constexpr int X_ITEMS = BN * GEMM_KB * 2;               // 16-byte activation cells per stage
-    static constexpr int X_PER_T = (X_ITEMS + NT - 1) / NT;
-    static constexpr int S_ITEMS = BN * GEMM_KB;                   // activation scales per stage
-    static constexpr int S_PER_T = (S_ITEMS + NT - 1) / NT;
+    static constexpr size_t OFF_B = OFF_A + (size_t)GEMM_KB * 2 * A_PLANE * 16;   // [token][8 cells], swizzled
+    static constexpr size_t OFF_SX = OFF_B + (size_t)BN * 128;                    // [token][4 floats]
+    static constexpr size_t OFF_SW = OFF_SX + (size_t)BN * 16;                    // fp32 [KB][BM], permuted per 32 rows
+    // plane b of the weight scales starts 8 * (b & 1) + 32 * (b >> 1) floats late: the 64 lanes that expand 16 rows x 4
+    // k-blocks then write to 64 different banks (a row's position inside its 32-row group is 0..7 or 16..23 for the first
+    // 16 rows, 8..15 or 24..31 for the others)
+    static constexpr int sw_plane(int b) { return b * BM + 8 * (b & 1) + 32 * (b >> 1); }
+    static constexpr size_t OFF_MW = OFF_SW + ((size_t)GEMM_KB * BM + 64) * 4;    // fp16 [BM][KB]
+    static constexpr size_t OFF_MX = OFF_MW + (HAS_MIN ? (size_t)BM * GEMM_KB * 2 : 0);   // fp16 [BN][KB]
+    static constexpr size_t STAGE = OFF_MX + (HAS_MIN ? (size_t)BN * GEMM_KB * 2 : 0);
+    static constexpr int W_ITEMS = BM * GEMM_KB, W_PER_T = (W_ITEMS + NT - 1) / NT;
+    static constexpr int B_INSTR = BN / 8;                                        // wave instructions that fill B: 8 tokens each
+    static constexpr int B_PER_W = B_INSTR / NW;
+    static constexpr int SX_INSTR = BN / 64;                                      // 64 tokens' scale cells each
+    static constexpr int S_ITEMS = BN * GEMM_KB, S_PER_T = (S_ITEMS + NT - 1) / NT;
+    static_assert(B_INSTR % NW == 0 && B_PER_W >= 1, "the activation loads divide evenly over the waves");
+    static_assert(SX_INSTR >= 1 && SX_INSTR <= NW, "one scale load instruction per wave at most");
+    static_assert(W_ITEMS % NT == 0, "the weight items divide evenly over the threads");
+    static_assert(STAGE % 16 == 0 && GEMM_KB == 4, "stage buffers keep 16-byte alignment; four scale planes");
 };
 
+constexpr int wait_vm0() { return 0x0F70; }                                      // s_waitcnt vmcnt(0) only
+
+// M0 carries the LDS byte address of the wave's 1 KB destination; lane i's 16 bytes land at M0 + 16 i.  Inline assembly,
+// because the compiler would make every later LDS read wait for a load it sees writing LDS; the kernel waits by hand
+// (vmcnt(0) in front of the stage barrier).  Nothing else in the kernel may use M0 (no dynamic register indexing).
+__device__ __forceinline__ void load16_into_lds(const uint8_t *src, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+}
+
 template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
-__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_blk32_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K,
-                                                                int64_t N, const uint8_t *__restrict__ ws,
-                                                                size_t ws_stride, int64_t M, float *__restrict__ y,
-                                                                int64_t ldy, TileMap map, RowGather rg, int slice_stages) {
-    using C = GemmCfg<TM, TN, WR, WC>;
+__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void gemm_blk32_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
+                              size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg,
+                              int slice_stages) {
     using T = Blk32<WT>;
+    using C = DirectCfg<TM, TN, WR, WC, T::HAS_MIN>;
     extern __shared__ __align__(16) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave / WC, wc = wave % WC;
     const int half = lane >> 5, l32 = lane & 31;
     const TileCoord tc = xcd_tile(blockIdx.x, map);
-    if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;        // padding of the tile map
+    if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;
     const int64_t row_base = (int64_t)tc.row_tile * C::BM;
     size_t w_offset;
-    const GatherView gv = resolve_gather<GATHER>(rg, w_offset, M);                   // MUL_MAT_ID: this expert's rows
+    const GatherView gv = resolve_gather<GATHER>(rg, w_offset, M);
     W += w_offset;
     if (gv.tok_tile < 0) return;
     const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
     if (tok_base >= M) return;
-    // split K (never with a gather, whose grid rows are the experts): grid row s takes the stages stage0 .. of every row and
-    // writes its partial tile to slice s of y
     int stage0 = 0, nstages = (int)(K / (32 * GEMM_KB));
     if (!GATHER && slice_stages > 0) {
         stage0 = (int)blockIdx.y * slice_stages;
         nstages = min(slice_stages, nstages - stage0);
         y += (size_t)blockIdx.y * (size_t)M * (size_t)ldy;
     }
-    const size_t off_d = q8_0_off_d(K);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
 
-    // ---- per-thread prefetch registers for one stage ----
+    // ---- sources of this thread's share of a stage (stage 0 of the slice; they advance by a constant per stage) ----
+    const uint8_t *wsrc[C::W_PER_T];
+#pragma unroll
+    for (int i = 0; i < C::W_PER_T; i++) {
+        const int item = tid + i * C::NT, r = item / GEMM_KB, b = item % GEMM_KB;
+        wsrc[i] = W + (size_t)min(row_base + r, N - 1) * nb01 + ((size_t)stage0 * GEMM_KB + b) * T::BYTES;
+    }
+    // activation cells: instruction q = wave * B_PER_W + j fills tokens 8 q .. 8 q + 7, lane -> token lane / 8, slot lane % 8
+    const uint8_t *bsrc[C::B_PER_W];
+#pragma unroll
+    for (int j = 0; j < C::B_PER_W; j++) {
+        const int t = (wave * C::B_PER_W + j) * 8 + (lane >> 3);
+        const int cell = (lane & 7) ^ ((t >> 1) & 7);
+        bsrc[j] = ws + (size_t)gv.act_row(min(tok_base + t, M - 1)) * ws_stride + (size_t)stage0 * (32 * GEMM_KB) + 16 * cell;
+    }
+    const uint8_t *sxsrc = ws + (size_t)gv.act_row(min(tok_base + (wave < C::SX_INSTR ? wave : 0) * 64 + lane, M - 1)) * ws_stride +
+                           q8_0_off_d(K) + (size_t)stage0 * (4 * GEMM_KB);
+    const uint8_t *msrc[C::S_PER_T];                                               // block_q8_1.s of the types with a minimum
+    if constexpr (T::HAS_MIN) {
+#pragma unroll
+        for (int i = 0; i < C::S_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            msrc[i] = ws + (size_t)gv.act_row(min(tok_base + min(item / GEMM_KB, C::BN - 1), M - 1)) * ws_stride + q8_0_off_s(K) +
+                      ((size_t)stage0 * GEMM_KB + item % GEMM_KB) * 4;
+        }
+    }
+
     typename T::Raw wq[C::W_PER_T];
     uint32_t wd[C::W_PER_T];
-    u32x4 xq[C::X_PER_T];
-    float xs[C::S_PER_T];
-    float xm[C::S_PER_T];                         // block_q8_1.s, for the types with a minimum
-    const size_t off_s = q8_0_off_s(K);
-    // activation rows of this thread's staging items (looked up once: with a gather they come from the pair list)
-    int64_t xrow[C::X_PER_T], srow[C::S_PER_T];
-#pragma unroll
-    for (int i = 0; i < C::X_PER_T; i++) xrow[i] = gv.act_row(min(tok_base + (tid + i * C::NT) / (GEMM_KB * 2), M - 1));
-#pragma unroll
-    for (int i = 0; i < C::S_PER_T; i++) srow[i] = gv.act_row(min(tok_base + (tid + i * C::NT) / GEMM_KB, M - 1));
-
-    auto fetch = [&](int stage) {
-        const int64_t kb0 = (int64_t)(stage0 + stage) * GEMM_KB;
+    float xm[C::S_PER_T];
+    auto fetch_w = [&](int s) {
 #pragma unroll
         for (int i = 0; i < C::W_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
-                const int r = item / GEMM_KB, b = item % GEMM_KB;
-                const int64_t row = min(row_base + r, N - 1);
-                const uint8_t *p = W + (size_t)row * nb01 + (size_t)(kb0 + b) * T::BYTES;
-                if constexpr (T::HAS_MIN) wd[i] = *reinterpret_cast<const uint32_t *>(p);          // d | m << 16
-                else wd[i] = *reinterpret_cast<const unsigned short *>(p);
-                T::fetch(wq[i], p);
-            }
+            const uint8_t *p = wsrc[i] + (size_t)s * (GEMM_KB * T::BYTES);
+            if constexpr (T::HAS_MIN) wd[i] = *reinterpret_cast<const uint32_t *>(p);
+            else wd[i] = *reinterpret_cast<const unsigned short *>(p);
+            T::fetch(wq[i], p);
         }
+        if constexpr (T::HAS_MIN) {
 #pragma unroll
-        for (int i = 0; i < C::X_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
-                const int c = item % (GEMM_KB * 2);                                 // c = 2*b + half
-                const int64_t tok = xrow[i];
-                xq[i] = *reinterpret_cast<const u32x4 *>(ws + (size_t)tok * ws_stride + (size_t)kb0 * 32 + 16 * c);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < C::S_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
-                const int b = item % GEMM_KB;
-                const int64_t tok = srow[i];
-                xs[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_d)[kb0 + b];
-                if constexpr (T::HAS_MIN) xm[i] = reinterpret_cast<const float *>(ws + (size_t)tok * ws_stride + off_s)[kb0 + b];
-            }
+            for (int i = 0; i < C::S_PER_T; i++) xm[i] = *reinterpret_cast<const float *>(msrc[i] + (size_t)s * (4 * GEMM_KB));
         }
     };
-
-    auto commit = [&](int buf) {
-        uint8_t *base = lds + (size_t)buf * C::STAGE;
+    auto issue_direct = [&](int s, uint32_t buf_off) {
+#pragma unroll
+        for (int j = 0; j < C::B_PER_W; j++)
+            load16_into_lds(bsrc[j] + (size_t)s * (32 * GEMM_KB),
+                            __builtin_amdgcn_readfirstlane(lds0 + buf_off + (uint32_t)C::OFF_B + (uint32_t)(wave * C::B_PER_W + j) * 1024u));
+        if (wave < C::SX_INSTR)
+            load16_into_lds(sxsrc + (size_t)s * (4 * GEMM_KB),
+                            __builtin_amdgcn_readfirstlane(lds0 + buf_off + (uint32_t)C::OFF_SX + (uint32_t)wave * 1024u));
+    };
+    auto commit_w = [&](uint32_t buf_off) {
+        uint8_t *base = lds + buf_off;
         u32x4 *A = reinterpret_cast<u32x4 *>(base + C::OFF_A);
-        u32x4 *B = reinterpret_cast<u32x4 *>(base + C::OFF_B);
-        unsigned short *SW = reinterpret_cast<unsigned short *>(base + C::OFF_SW);
-        float *SX = reinterpret_cast<float *>(base + C::OFF_SX);
+        float *SW = reinterpret_cast<float *>(base + C::OFF_SW);
 #pragma unroll
         for (int i = 0; i < C::W_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::W_ITEMS % C::NT == 0 || item < C::W_ITEMS) {
-                const int r = item / GEMM_KB, b = item % GEMM_KB;
-                u32x4 lo, hi;
-                T::emit(wq[i], lo, hi);
-                A[(b * 2 + 0) * C::A_PLANE + r] = lo;
-                A[(b * 2 + 1) * C::A_PLANE + r] = hi;
-                // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4;
-                // store the scale of row i at half*16 + (i/8)*4 + i%4 so each lane reads its 16 scales contiguously
-                const int i32 = r & 31;
-                const int pos = ((i32 >> 2) & 1) * 16 + (i32 >> 3) * 4 + (i32 & 3);
-                SW[b * C::BM + (r & ~31) + pos] = (unsigned short)wd[i];
-                if constexpr (T::HAS_MIN) reinterpret_cast<unsigned short *>(base + C::OFF_MW)[r * GEMM_KB + b] = (unsigned short)(wd[i] >> 16);
-            }
+            const int item = tid + i * C::NT, r = item / GEMM_KB, b = item % GEMM_KB;
+            u32x4 lo, hi;
+            T::emit(wq[i], lo, hi);
+            A[(b * 2 + 0) * C::A_PLANE + r] = lo;
+            A[(b * 2 + 1) * C::A_PLANE + r] = hi;
+            const int i32 = r & 31;
+            // the lane that owns MFMA result register v of a 32-row tile holds row 8*(v/4) + 4*half + v%4: the scale of
+            // row i goes to half*16 + (i/8)*4 + i%4, so a lane reads its 16 scales as one contiguous run
+            const int pos = ((i32 >> 2) & 1) * 16 + (i32 >> 3) * 4 + (i32 & 3);
+            SW[C::sw_plane(b) + (r & ~31) + pos] = h2f(wd[i]);
+            if constexpr (T::HAS_MIN) reinterpret_cast<unsigned short *>(base + C::OFF_MW)[r * GEMM_KB + b] = (unsigned short)(wd[i] >> 16);
         }
+        if constexpr (T::HAS_MIN) {
 #pragma unroll
-        for (int i = 0; i < C::X_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::X_ITEMS % C::NT == 0 || item < C::X_ITEMS) {
-                const int c = item % (GEMM_KB * 2), n = item / (GEMM_KB * 2);
-                B[c * C::B_PLANE + n] = xq[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < C::S_PER_T; i++) {
-            const int item = tid + i * C::NT;
-            if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS) {
-                const int b = item % GEMM_KB, n = item / GEMM_KB;
-                SX[b * C::BN + n] = xs[i] * T::INV_MULT;                   // takes back the power of two in the weight cells
-                if constexpr (T::HAS_MIN) reinterpret_cast<unsigned short *>(base + C::OFF_MX)[n * GEMM_KB + b] = f2h_rne(xm[i]);   // exact: s is an fp16 number
+            for (int i = 0; i < C::S_PER_T; i++) {
+                const int item = tid + i * C::NT;
+                if (C::S_ITEMS % C::NT == 0 || item < C::S_ITEMS)
+                    reinterpret_cast<unsigned short *>(base + C::OFF_MX)[item] = f2h_rne(xm[i]);      // [token][KB]; exact
             }
         }
     };
@@ -309,12 +323,9 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
 #pragma unroll
     for (int a = 0; a < TM; a++)
 #pragma unroll
-        for (int b = 0; b < TN; b++)
+        for (int c = 0; c < TN; c++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
-
-    // The magic constant lives in 16 registers for the whole kernel; the empty asm keeps the compiler from
-    // re-materialising it with 16 moves in front of every MFMA.
+            for (int v = 0; v < 16; v++) acc[a][c][v] = 0.f;
     i32x16 magic;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
@@ -323,31 +334,29 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
         magic[v] = m;
     }
 
-    fetch(0);
-    commit(0);
-    __syncthreads();
+    // per-lane LDS byte offsets inside a stage buffer; everything else is an immediate
+    const int r0 = wr * TM * 32, n0 = wc * TN * 32;
+    const uint32_t a_rd = (uint32_t)C::OFF_A + (uint32_t)(half * C::A_PLANE + r0 + l32) * 16u;
+    const uint32_t sw_rd = (uint32_t)C::OFF_SW + (uint32_t)(r0 + half * 16) * 4u;
+    const uint32_t sx_rd = (uint32_t)C::OFF_SX + (uint32_t)(n0 + l32) * 16u;
+    uint32_t b_rd[GEMM_KB];
+#pragma unroll
+    for (int b = 0; b < GEMM_KB; b++) b_rd[b] = (uint32_t)C::OFF_B + (uint32_t)(n0 + l32) * 128u + 16u * (uint32_t)((2 * b + half) ^ ((l32 >> 1) & 7));
 
-    for (int s = 0; s < nstages; s++) {
-        const int buf = s & 1;
-        if (s + 1 < nstages) fetch(s + 1);
-
-        const uint8_t *base = lds + (size_t)buf * C::STAGE;
-        const u32x4 *A = reinterpret_cast<const u32x4 *>(base + C::OFF_A);
-        const u32x4 *B = reinterpret_cast<const u32x4 *>(base + C::OFF_B);
-        const u32x4 *SW = reinterpret_cast<const u32x4 *>(base + C::OFF_SW);
-        const float *SX = reinterpret_cast<const float *>(base + C::OFF_SX);
-
+    // one stage from the buffer at byte offset BUF
+    auto compute = [&](auto buf_tag) {
+        constexpr uint32_t BUF = decltype(buf_tag)::value ? (uint32_t)C::STAGE : 0u;
+        const uint8_t *base = lds + BUF;
         if constexpr (T::HAS_MIN) {
-            // sum over the stage's 4 blocks of m[row][b] * s[token][b]: k = 0..3 live in lanes 0..31, k = 4..7 are zero
             f16x4 ma[TM], sb[TN];
 #pragma unroll
             for (int a = 0; a < TM; a++) {
-                const u32x2 t = reinterpret_cast<const u32x2 *>(base + C::OFF_MW)[(wr * TM + a) * 32 + l32];
+                const u32x2 t = reinterpret_cast<const u32x2 *>(base + C::OFF_MW)[r0 + a * 32 + l32];
                 ma[a] = __builtin_bit_cast(f16x4, half ? u32x2{0u, 0u} : t);
             }
 #pragma unroll
             for (int c = 0; c < TN; c++) {
-                const u32x2 t = reinterpret_cast<const u32x2 *>(base + C::OFF_MX)[(wc * TN + c) * 32 + l32];
+                const u32x2 t = reinterpret_cast<const u32x2 *>(base + C::OFF_MX)[n0 + c * 32 + l32];
                 sb[c] = __builtin_bit_cast(f16x4, half ? u32x2{0u, 0u} : t);
             }
 #pragma unroll
@@ -355,88 +364,136 @@ __global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC
 #pragma unroll
                 for (int c = 0; c < TN; c++) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x8f16(ma[a], sb[c], acc[a][c], 0, 0, 0);
         }
-#pragma unroll 1
-        for (int b = 0; b < GEMM_KB; b++) {
-            i32x4 af[TM], bf[TN];
-            u32x4 sw[TM][2];
-            float dx[TN], ndx[TN];
+        float dxs[TN][GEMM_KB];
+#pragma unroll
+        for (int c = 0; c < TN; c++) {
+            const float4 t = *reinterpret_cast<const float4 *>(base + sx_rd + c * 512);
+            dxs[c][0] = t.x; dxs[c][1] = t.y; dxs[c][2] = t.z; dxs[c][3] = t.w;
+            if constexpr (T::HAS_MIN) {
+#pragma unroll
+                for (int b = 0; b < GEMM_KB; b++) dxs[c][b] *= T::INV_MULT;       // the min term has no power of two to take back
+            }
+        }
+        // operand registers of two k-blocks: those of k-block b + 1 are requested while k-block b is worked on, and the
+        // first MFMA of k-block b + 1 is issued before the last scaling group of k-block b.  The 16 weight scales of a
+        // (k-block, row tile) pair - fp32 in LDS: a mixed-precision FMA that reads them as fp16 issues at a lower rate
+        // than a plain one - serve the pair's TN tiles and are requested one pair ahead, in two register sets.
+        i32x4 af[2][TM], bf[2][TN];
+        float swf[2][16];
+        auto load_operands = [&](int b, int slot) {
 #pragma unroll
             for (int a = 0; a < TM; a++) {
-                const int r0 = (wr * TM + a) * 32;
-                const u32x4 t = A[(b * 2 + half) * C::A_PLANE + r0 + l32];
-                af[a] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
-                const u32x4 *sp = SW + ((size_t)b * C::BM + r0 + half * 16) / 8;    // 8 halves per 16-byte cell
-                sw[a][0] = sp[0];
-                sw[a][1] = sp[1];
+                const u32x4 t = *reinterpret_cast<const u32x4 *>(base + a_rd + (b * 2 * C::A_PLANE + a * 32) * 16);
+                af[slot][a] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
             }
 #pragma unroll
             for (int c = 0; c < TN; c++) {
-                const int n0 = (wc * TN + c) * 32;
-                const u32x4 t = B[(b * 2 + half) * C::B_PLANE + n0 + l32];
-                bf[c] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
-                dx[c] = SX[b * C::BN + n0 + l32];
+                const u32x4 t = *reinterpret_cast<const u32x4 *>(base + b_rd[b] + c * 4096);
+                bf[slot][c] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
+            }
+        };
+        auto load_scales = [&](int g) {                                       // pair g = b * TM + a
+            const int b = g / TM, a = g % TM;
+            const float4 *sp = reinterpret_cast<const float4 *>(base + sw_rd + (C::sw_plane(b) + a * 32) * 4);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 t = sp[q];
+                swf[g & 1][4 * q] = t.x; swf[g & 1][4 * q + 1] = t.y; swf[g & 1][4 * q + 2] = t.z; swf[g & 1][4 * q + 3] = t.w;
+            }
+        };
+        load_operands(0, 0);
+        load_scales(0);
+        i32x16 d_cur = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0][0], bf[0][0], magic, 0, 0, 0);
+#pragma unroll
+        for (int b = 0; b < GEMM_KB; b++) {
+            const int slot = b & 1;
+            if (b + 1 < GEMM_KB) load_operands(b + 1, slot ^ 1);
+            float dx[TN], ndx[TN];
+#pragma unroll
+            for (int c = 0; c < TN; c++) {
+                dx[c] = dxs[c][b];
                 ndx[c] = -MAGIC_F * dx[c];
             }
-            if constexpr (OCC >= 4) {
-                // enough waves per SIMD to cover the MFMA latency: consume each result right away (16 fewer VGPRs)
 #pragma unroll
-                for (int i = 0; i < TM * TN; i++) {
-                    const int a = i / TN, c = i % TN;
-                    const i32x16 d = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bf[c], magic, 0, 0, 0);
-                    const uint32_t swd[8] = {sw[a][0].x, sw[a][0].y, sw[a][0].z, sw[a][0].w,
-                                             sw[a][1].x, sw[a][1].y, sw[a][1].z, sw[a][1].w};
+            for (int a = 0; a < TM; a++) {
+                const int g = b * TM + a;
+                if (g + 1 < GEMM_KB * TM) load_scales(g + 1);
 #pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const float t = __builtin_fmaf(__int_as_float(d[v]), dx[c], ndx[c]);
-                        const __half hw = __ushort_as_half((unsigned short)((v & 1) ? (swd[v >> 1] >> 16) : (swd[v >> 1] & 0xffffu)));
-                        acc[a][c][v] = __builtin_fmaf(t, __half2float(hw), acc[a][c][v]);
-                    }
-                }
-            } else {
-                // Software pipeline over the TM*TN tiles of this k-block: the MFMA of tile i+1 is issued before
-                // the 32 scaling operations of tile i.
-                i32x16 d_cur = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0], bf[0], magic, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < TM * TN; i++) {
-                    const int a = i / TN, c = i % TN;
+                for (int c = 0; c < TN; c++) {
                     i32x16 d_next = d_cur;
-                    if (i + 1 < TM * TN) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[(i + 1) / TN], bf[(i + 1) % TN], magic, 0, 0, 0);
-                    const uint32_t swd[8] = {sw[a][0].x, sw[a][0].y, sw[a][0].z, sw[a][0].w,
-                                             sw[a][1].x, sw[a][1].y, sw[a][1].z, sw[a][1].w};
+                    if (c + 1 < TN) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[slot][a], bf[slot][c + 1], magic, 0, 0, 0);
+                    else if (a + 1 < TM) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[slot][a + 1], bf[slot][0], magic, 0, 0, 0);
+                    else if (b + 1 < GEMM_KB) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[slot ^ 1][0], bf[slot ^ 1][0], magic, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);                // the MFMA goes first: it runs behind the scaling below
 #pragma unroll
                     for (int v = 0; v < 16; v++) {
                         const float t = __builtin_fmaf(__int_as_float(d_cur[v]), dx[c], ndx[c]);
-                        const __half hw = __ushort_as_half((unsigned short)((v & 1) ? (swd[v >> 1] >> 16) : (swd[v >> 1] & 0xffffu)));
-                        acc[a][c][v] = __builtin_fmaf(t, __half2float(hw), acc[a][c][v]);
+                        acc[a][c][v] = __builtin_fmaf(t, swf[g & 1][v], acc[a][c][v]);
                     }
                     d_cur = d_next;
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
+    };
 
-        if (s + 1 < nstages) commit(buf ^ 1);
-        __syncthreads();
+    // Every load gets a whole stage to arrive.  A stage begins by expanding the weights fetched during the previous stage
+    // into the idle buffer (the compiler's own wait for them is exact: nothing younger is outstanding then), then requests
+    // the next stage's activations (into that same idle buffer) and the weights of the stage after, and only then starts
+    // its arithmetic.  In front of the barrier a wave waits until at most its weight loads - the youngest requests - are
+    // outstanding, i.e. for the activations; the barrier publishes them and the expanded weights.
+    // Nothing inside a stage is conditional (a branch would end the scheduling region that keeps the MFMAs and their
+    // scaling interleaved): stages past the last one are the last one again, loaded and expanded into the idle buffer.
+    constexpr int W_LOADS = C::W_PER_T * 2 + (T::HAS_MIN ? C::S_PER_T : 0);          // vector loads of one fetch_w
+    constexpr int WAIT_ACTS = 0x0F70 | (W_LOADS & 15) | ((W_LOADS >> 4) << 14);      // s_waitcnt vmcnt(W_LOADS)
+    const int last = nstages - 1;
+    fetch_w(0);
+    issue_direct(0, 0u);
+    commit_w(0u);
+    fetch_w(min(1, last));
+    __builtin_amdgcn_s_waitcnt(WAIT_ACTS);
+    __syncthreads();
+    for (int s = 0; s < nstages; s += 2) {
+        {
+            commit_w((uint32_t)C::STAGE);
+            issue_direct(min(s + 1, last), (uint32_t)C::STAGE);
+            fetch_w(min(s + 2, last));
+            compute(std::false_type{});
+            __builtin_amdgcn_s_waitcnt(WAIT_ACTS);
+            __syncthreads();
+        }
+        if (s + 1 < nstages) {
+            commit_w(0u);
+            issue_direct(min(s + 2, last), 0u);
+            fetch_w(min(s + 3, last));
+            compute(std::true_type{});
+            __builtin_amdgcn_s_waitcnt(WAIT_ACTS);
+            __syncthreads();
+        }
     }
+    __builtin_amdgcn_s_waitcnt(wait_vm0());
 
     // ---- epilogue: register v of tile (a, c) is row 8*(v/4) + 4*half + v%4, token l32 ----
+    constexpr float POST = T::HAS_MIN ? 1.f : T::INV_MULT;
 #pragma unroll
     for (int a = 0; a < TM; a++)
 #pragma unroll
         for (int c = 0; c < TN; c++) {
-            const int64_t tok = tok_base + (wc * TN + c) * 32 + l32;
+            const int64_t tok = tok_base + n0 + c * 32 + l32;
             if (tok >= M) continue;
             const int64_t orow = gv.out_row(tok);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const int64_t row = row_base + (wr * TM + a) * 32 + 8 * g + 4 * half;
+                const int64_t row = row_base + r0 + a * 32 + 8 * g + 4 * half;
                 float *dst = y + (size_t)orow * ldy + row;
+                const float o0 = acc[a][c][4 * g] * POST, o1 = acc[a][c][4 * g + 1] * POST, o2 = acc[a][c][4 * g + 2] * POST, o3 = acc[a][c][4 * g + 3] * POST;
                 if (row + 3 < N && (((uintptr_t)dst) & 15) == 0) {
-                    *reinterpret_cast<float4 *>(dst) = make_float4(acc[a][c][4 * g], acc[a][c][4 * g + 1], acc[a][c][4 * g + 2], acc[a][c][4 * g + 3]);
+                    *reinterpret_cast<float4 *>(dst) = make_float4(o0, o1, o2, o3);
                 } else {
+                    const float o[4] = {o0, o1, o2, o3};
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (row + e < N) dst[e] = acc[a][c][4 * g + e];
+                        if (row + e < N) dst[e] = o[e];
                 }
             }
         }
@@ -534,16 +591,17 @@ static int blk32_slices_for(int64_t K, int64_t N, int64_t M, int64_t cus) {
 }
 
 template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
-static hipError_t launch_cfg(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
-                             float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
-                             int slices = 1, float *part = nullptr) {
-    using C = GemmCfg<TM, TN, WR, WC>;
+static hipError_t launch_direct(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
+                                float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
+                                int slices = 1, float *part = nullptr) {
+    using C = DirectCfg<TM, TN, WR, WC, Blk32<WT>::HAS_MIN>;
     const size_t lds_bytes = 2 * C::STAGE;
+    if ((int64_t)lds_bytes > lim.max_lds_per_block) return hipErrorInvalidValue;
     auto kfn = gemm_blk32_kernel<WT, TM, TN, WR, WC, OCC, GATHER>;
-    static LdsGrant grant;                                               // one per kernel instantiation
+    static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
-    // workgroups that share an XCD (OCC waves per SIMD, 32 CUs) take a compact block of output tiles
-    const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
+    const int per_cu = (int)(lds_bytes > 80 * 1024 ? 1 : (4 * OCC / C::NW > 0 ? 4 * OCC / C::NW : 1));
+    const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * per_cu);
     if (!GATHER && slices > 1) {
         const int slice_stages = (int)ceil_div(K / (32 * GEMM_KB), (int64_t)slices);
         hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)slices), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
@@ -563,20 +621,23 @@ static hipError_t launch_type(const void *W, size_t nb01, int64_t K, int64_t N, 
     const int64_t cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if (!rg.perm && split.part) {
         const int slices = blk32_slices_for(K, N, M, cus);
-        if (slices > 1 && split.bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (((uintptr_t)split.part) & 15) == 0)
-            return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, slices, split.part);
+        if (slices > 1 && split.bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (((uintptr_t)split.part) & 15) == 0) {
+            return launch_direct<WT, 1, 1, 2, 2, 3, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as, slices, split.part);
+        }
     }
-    // 128 rows x 128 tokens per 8-wave group, 4 waves per SIMD (two groups per CU); problems too small to give
-    // every CU such a group use 64 x 64 groups of 4 waves.  (CHIP_GEMM_CFG selects a shape by hand.)  Larger per-wave tiles
-    // with fewer waves per SIMD measured slower on 14336 x 4096 x 2048 (Q4_0): 2 x 2 tiles at two waves 449 us against
-    // 447, 4 x 2 and 2 x 4 at one wave 719 and 667 us: the scaling work is vector-bound and wants waves, not tiles.
-    if (rg.perm)                                                                     // expert groups: 64 x 64 tiles
-        return launch_cfg<WT, 1, 1, 2, 2, 4, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
-    const int cfg = (int)tune("CHIP_GEMM_CFG", g128 >= cus ? 0 : 1);
+    if (rg.perm) {                                                                   // expert groups: 64 x 64 tiles
+        return launch_direct<WT, 1, 1, 2, 2, 3, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+    }
+    // Two 4-wave workgroups of 128 x 128 per CU when that fills the device, else 64 x 128, else 64 x 64 (three workgroups
+    // per CU).  Measured on Q4_0 with K = 4096 (us; 128 x 128 / 64 x 128 / 64 x 64 / 128 x 256 with 8 waves): 14336 x 2048
+    // tokens 375 / 413 / 468 / 415, 4096 x 2048 106 / 115 / 130 / 106, 14336 x 512 103 / 110 / 114 / 102, 4096 x 512
+    // 63 / 38 / 38 / 81.
+    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128), g64x128 = ceil_div(N, 64) * ceil_div(M, 128);
+    const int cfg = (int)tune("CHIP_GEMM_CFG", 2 * g128 >= 3 * cus ? 3 : 2 * g64x128 >= 3 * cus ? 6 : 4);
     switch (cfg) {
-        case 0: return launch_cfg<WT, 1, 2, 4, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-        case 1: return launch_cfg<WT, 1, 1, 2, 2, 4, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
+        case 3: return launch_direct<WT, 2, 2, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);   // 128 x 128, 4 waves
+        case 4: return launch_direct<WT, 1, 1, 2, 2, 3, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);   // 64 x 64, 4 waves
+        case 6: return launch_direct<WT, 1, 2, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);   // 64 x 128, 4 waves
         default: return hipErrorInvalidValue;
     }
     return hipErrorInvalidValue;
@@ -587,7 +648,7 @@ int gemm_blk32_slices(int wtype, int64_t K, int64_t N, int64_t n, int compute_un
     return blk32_slices_for(K, N, n, compute_units > 0 ? compute_units : 256);
 }
 
-int gemm_blk32_moe_tile_tokens() { return GemmCfg<1, 1, 2, 2>::BN; }   // the 64 x 64 shape serves the expert groups
+int gemm_blk32_moe_tile_tokens() { return DirectCfg<1, 1, 2, 2, false>::BN; }   // the 64 x 64 shape serves the expert groups
 
 hipError_t launch_gemm_blk32(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                              int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather *rgp,
