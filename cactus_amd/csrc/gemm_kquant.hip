@@ -550,6 +550,317 @@ void gemm_kq_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64
     }
 }
 
+// ---- Q4_K and Q5_K at prefill sizes: one int8 plane, sub-block scales applied by the vector unit ----
+// The two digit planes above cost two MFMAs per 32 values.  Measured, an MFMA is worth more time (and power: these kernels
+// run clock-limited) than the 16 integer multiply-adds that apply a sub-block scale to its 16 results per lane.  So this
+// kernel feeds the quants themselves (Q4_K: 0..15, Q5_K: q - 16) as one plane: every MFMA result is the reference's
+// per-sub-block integer dot, and   sumi += isum_j * sc_j   is one v_mad_i32_i24 per result.  The activations are the MFMA's
+// first operand and the weights its second, so a lane owns one weight row and its 16 result registers 16 tokens: the
+// sub-block scale, d and dmin are one register per lane (no scale vectors from LDS), and a store instruction writes 32
+// consecutive rows of a token.  Per super-block the fold is, per output,  out += dx * (d * float(sumi) - dmin * summ)
+// with summ (and Q5_K's sum_j sc_j * bsum_j) from one fp16 MFMA as above: the same operations in the same order as
+// gemm_kq_kernel, so the outputs are bit-identical to it.
+// Skeleton as the block-32 kernel's: activations straight into swizzled LDS rows with global_load_lds_dwordx4, weights
+// through registers (a thread fetches its (row, x) item of a whole super-block during the super-block before and every
+// stage begins by expanding the next stage's half into the idle buffer), the MFMA of tile i + 1 issued before the 16
+// multiply-adds of tile i, two 4-wave workgroups per CU.
+template <int WT> struct KS;
+template <> struct KS<T_Q4_K> {
+    // 16 quant bytes -> the 16-value k-half of sub-blocks 2jp (low nibbles) and 2jp + 1 (high nibbles)
+    __device__ static __forceinline__ void emit(const KQ<T_Q4_K>::Raw &r, int h, int, u32x4 &c0, u32x4 &c1) {
+        const u32x4 q = r.q[h];
+#pragma unroll
+        for (int i = 0; i < 4; i++) { c0[i] = q[i] & 0x0f0f0f0fu; c1[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
+    }
+};
+template <> struct KS<T_Q5_K> {
+    // q - 16 as a signed byte: (q + 112) ^ 128 (q + 112 <= 143: no carries between bytes)
+    __device__ static __forceinline__ void emit(const KQ<T_Q5_K>::Raw &r, int h, int x, u32x4 &c0, u32x4 &c1) {
+        const int jp = 2 * h + (x >> 1);
+        const u32x4 q = r.q[h];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t hb = r.qh[i] >> (2 * jp);
+            const uint32_t lo = (q[i] & 0x0f0f0f0fu) | ((hb << 4) & 0x10101010u);
+            const uint32_t hi = ((q[i] >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
+            c0[i] = (lo + 0x70707070u) ^ 0x80808080u;
+            c1[i] = (hi + 0x70707070u) ^ 0x80808080u;
+        }
+    }
+};
+
+template <int WT, int TM, int TN, int WR, int WC>
+struct KsCfg {
+    using T = KQ<WT>;
+    static constexpr int NW = WR * WC, NT = NW * 64;
+    static constexpr int BM = 32 * TM * WR, BN = 32 * TN * WC;
+    static constexpr int A_PLANE = BM + 2;
+    static constexpr size_t OFF_A = 0;                                               // [k-block][half][row] cells
+    static constexpr size_t OFF_B = OFF_A + (size_t)KQ_KB * 2 * A_PLANE * 16;        // [token][8 cells], swizzled
+    static constexpr size_t STAGE = OFF_B + (size_t)BN * 128;
+    // one super-block buffer: written while half 0 is multiplied, read by the scaling of both halves and by the fold
+    static constexpr size_t OFF_FA = 0;                                              // fp16 cells [NF16][k-half][BM]
+    static constexpr size_t OFF_FB = OFF_FA + (size_t)T::NF16 * 2 * BM * 16;         // fp16 cells [k-half][BN]: the 16 bsums
+    static constexpr size_t OFF_SC = OFF_FB + (size_t)2 * BN * 16;                   // i32 [8][BM]: sub-block scales
+    static constexpr size_t OFF_SD = OFF_SC + (size_t)8 * BM * 4;                    // u32 [BM]: d | dmin << 16
+    static constexpr size_t OFF_SX = OFF_SD + (size_t)BM * 4;                        // f32 [BN]: activation scale
+    static constexpr size_t SBLK = OFF_SX + (size_t)BN * 4;
+    static constexpr size_t OFF_SBLK = 2 * STAGE;
+    static constexpr size_t TOTAL = OFF_SBLK + 2 * SBLK;                             // two: the next super-block's is written during half 1
+    static constexpr int W_ITEMS = BM * 4, W_PER_T = W_ITEMS / NT;
+    static constexpr int B_INSTR = BN / 8, B_PER_W = B_INSTR / NW;
+    static_assert(W_ITEMS % NT == 0 && W_PER_T >= 1, "the weight items divide evenly over the threads");
+    static_assert(B_INSTR % NW == 0 && B_PER_W >= 1, "the activation loads divide evenly over the waves");
+    static_assert(2 * BN <= NT, "two threads per token convert its block sums");
+    static_assert(STAGE % 16 == 0 && SBLK % 16 == 0, "buffers keep 16-byte alignment");
+};
+
+__device__ __forceinline__ void kq_load16_into_lds(const uint8_t *src, uint32_t lds_addr) {
+    // M0 = LDS byte address of the wave's 1 KB destination; lane i's 16 bytes land at M0 + 16 i.  Inline assembly so that
+    // the compiler does not make every later LDS read wait for it; the kernel waits by hand in front of the stage barrier.
+    // Nothing else in the kernel may use M0 (no dynamic register indexing).
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+}
+
+template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
+__global__ __launch_bounds__(WR *WC * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void gemm_ks_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N, const uint8_t *__restrict__ ws,
+                    size_t ws_stride, int64_t M, float *__restrict__ y, int64_t ldy, TileMap map, RowGather rg, int slice_sb) {
+    using T = KQ<WT>;
+    using C = KsCfg<WT, TM, TN, WR, WC>;
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int sb0 = 0, nsb = (int)(K / QK_K);
+    if (!GATHER && slice_sb > 0) {
+        sb0 = (int)blockIdx.y * slice_sb;
+        nsb = min(slice_sb, nsb - sb0);
+        y += (size_t)blockIdx.y * (size_t)M * (size_t)ldy;
+    }
+    const TileCoord tc = xcd_tile(blockIdx.x, map);
+    if (tc.row_tile >= map.row_tiles || tc.tok_tile >= map.tok_tiles) return;
+    size_t w_offset;
+    const GatherView gv = resolve_gather<GATHER>(rg, w_offset, M);
+    W += w_offset;
+    const int64_t row_base = (int64_t)tc.row_tile * C::BM;
+    if (gv.tok_tile < 0) return;
+    const int64_t tok_base = (int64_t)(GATHER ? gv.tok_tile : tc.tok_tile) * C::BN;
+    if (tok_base >= M) return;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    const size_t off_d = q8_K_off_d(K), off_bs = q8_K_off_bsums(K);
+
+    // ---- this thread's share of the staging ----
+    const uint8_t *wsrc[C::W_PER_T];
+#pragma unroll
+    for (int i = 0; i < C::W_PER_T; i++) wsrc[i] = W + (size_t)min(row_base + ((tid + i * C::NT) >> 2), N - 1) * nb01 + (size_t)sb0 * T::BYTES;
+    const uint8_t *bsrc[C::B_PER_W];
+#pragma unroll
+    for (int j = 0; j < C::B_PER_W; j++) {
+        const int t = (wave * C::B_PER_W + j) * 8 + (lane >> 3);
+        const int cell = (lane & 7) ^ ((t >> 1) & 7);
+        bsrc[j] = ws + (size_t)gv.act_row(min(tok_base + t, M - 1)) * ws_stride + (size_t)sb0 * QK_K + 16 * cell;
+    }
+    // activation scale: thread t < BN for token t; block sums: thread t < 2*BN for token t/2, k-half t&1
+    const uint8_t *ssrc = ws + (size_t)gv.act_row(min(tok_base + min(tid, C::BN - 1), M - 1)) * ws_stride + off_d + (size_t)sb0 * 4;
+    const uint8_t *bssrc = ws + (size_t)gv.act_row(min(tok_base + min(tid >> 1, C::BN - 1), M - 1)) * ws_stride + off_bs + 16 * (tid & 1) + (size_t)sb0 * 32;
+
+    typename T::Raw wq[C::W_PER_T];
+    u32x4 bs;
+    float xs;
+    auto fetch_sb = [&](int sb_wanted) {
+        const int sb = min(sb_wanted, nsb - 1);
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; i++) T::fetch(wq[i], wsrc[i] + (size_t)sb * T::BYTES, (tid + i * C::NT) & 3);
+        xs = reinterpret_cast<const float *>(ssrc)[sb];
+        bs = *reinterpret_cast<const u32x4 *>(bssrc + (size_t)sb * 32);
+    };
+    auto issue_direct = [&](int stage_wanted, uint32_t buf_off) {
+        const int stage = min(stage_wanted, 2 * nsb - 1);
+#pragma unroll
+        for (int j = 0; j < C::B_PER_W; j++)
+            kq_load16_into_lds(bsrc[j] + (size_t)stage * (32 * KQ_KB),
+                               __builtin_amdgcn_readfirstlane(lds0 + buf_off + (uint32_t)C::OFF_B + (uint32_t)(wave * C::B_PER_W + j) * 1024u));
+    };
+    // expand half H of the fetched super-block into the stage buffer at buf_off; with H = 0 also write that super-block's
+    // scales, fp16 cells and activation sums into super-block buffer sbp
+    auto commit = [&](uint32_t buf_off, int sbp, auto half_tag) {
+        constexpr int h = decltype(half_tag)::value ? 1 : 0;
+        uint8_t *base = lds + buf_off;
+        uint8_t *sblk = lds + C::OFF_SBLK + (size_t)sbp * C::SBLK;
+        u32x4 *A = reinterpret_cast<u32x4 *>(base + C::OFF_A);
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; i++) {
+            const int item = tid + i * C::NT;
+            const int r = item >> 2, x = item & 3, hf = x & 1;
+            u32x4 c0, c1;
+            KS<WT>::emit(wq[i], h, x, c0, c1);
+            A[(T::kb0(x) * 2 + hf) * C::A_PLANE + r] = c0;
+            A[(T::kb1(x) * 2 + hf) * C::A_PLANE + r] = c1;
+            if constexpr (h == 0) {
+                uint32_t sc, mn;
+                scale_min_pair(wq[i].hdr, x, sc, mn);                                      // sub-blocks 2x and 2x + 1
+                int *SC = reinterpret_cast<int *>(sblk + C::OFF_SC);
+                SC[(2 * x) * C::BM + r] = (int)(sc & 0xffu);
+                SC[(2 * x + 1) * C::BM + r] = (int)(sc >> 8);
+                if (x == 0) reinterpret_cast<uint32_t *>(sblk + C::OFF_SD)[r] = T::scales(wq[i]);
+                // items x < 2*NF16 of a row each build one fp16 operand cell [x/2][x&1][row]
+                if (x < 2 * T::NF16) *reinterpret_cast<u32x4 *>(sblk + C::OFF_FA + (size_t)(x * C::BM + r) * 16) = T::f16_cell(wq[i], x);
+            }
+        }
+        if constexpr (h == 0) {
+            if (tid < C::BN) reinterpret_cast<float *>(sblk + C::OFF_SX)[tid] = xs;
+            if (tid < 2 * C::BN) *reinterpret_cast<u32x4 *>(sblk + C::OFF_FB + (size_t)((tid & 1) * C::BN + (tid >> 1)) * 16) = i16x8_to_f16(bs);
+        }
+    };
+
+    // ---- this wave's tiles: register v of tile (a, c) is token n0 + 32 c + 8 (v / 4) + 4 half + v % 4, row r0 + 32 a + l32 ----
+    const int wr = wave / WC, wc = wave % WC;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int r0 = wr * TM * 32, n0 = wc * TN * 32;
+    const uint32_t a_rd = (uint32_t)C::OFF_A + (uint32_t)(half * C::A_PLANE + r0 + l32) * 16u;
+    uint32_t b_rd[KQ_KB];
+#pragma unroll
+    for (int b = 0; b < KQ_KB; b++) b_rd[b] = (uint32_t)C::OFF_B + (uint32_t)(n0 + l32) * 128u + 16u * (uint32_t)((2 * b + half) ^ ((l32 >> 1) & 7));
+
+    int sumi[TM][TN][16];
+    float out[TM][TN][16];
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int c = 0; c < TN; c++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) { out[a][c][v] = 0.f; sumi[a][c][v] = 0; }
+
+    // one stage (half H of a super-block whose scales sit in super-block buffer sbp) from the buffer at byte offset BUF
+    auto compute = [&](auto buf_tag, auto half_tag, int sbp) {
+        constexpr uint32_t BUF = decltype(buf_tag)::value ? (uint32_t)C::STAGE : 0u;
+        constexpr int h = decltype(half_tag)::value ? 1 : 0;
+        const uint8_t *base = lds + BUF;
+        const int *SC = reinterpret_cast<const int *>(lds + C::OFF_SBLK + (size_t)sbp * C::SBLK + C::OFF_SC);
+        i32x4 af[2][TM], bf[2][TN];
+        int sc[KQ_KB][TM];
+        auto load_operands = [&](int b, int slot) {
+#pragma unroll
+            for (int a = 0; a < TM; a++) {
+                const u32x4 t = *reinterpret_cast<const u32x4 *>(base + a_rd + (b * 2 * C::A_PLANE + a * 32) * 16);
+                af[slot][a] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
+            }
+#pragma unroll
+            for (int c = 0; c < TN; c++) {
+                const u32x4 t = *reinterpret_cast<const u32x4 *>(base + b_rd[b] + c * 4096);
+                bf[slot][c] = i32x4{(int)t.x, (int)t.y, (int)t.z, (int)t.w};
+            }
+        };
+#pragma unroll
+        for (int b = 0; b < KQ_KB; b++)
+#pragma unroll
+            for (int a = 0; a < TM; a++) sc[b][a] = SC[(4 * h + b) * C::BM + r0 + a * 32 + l32];
+        constexpr int TILES = TM * TN;
+        const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        load_operands(0, 0);
+        i32x16 d_cur = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[0][0], af[0][0], zero, 0, 0, 0);
+#pragma unroll
+        for (int b = 0; b < KQ_KB; b++) {
+            const int slot = b & 1;
+            if (b + 1 < KQ_KB) load_operands(b + 1, slot ^ 1);
+#pragma unroll
+            for (int i = 0; i < TILES; i++) {
+                const int a = i / TN, c = i % TN;
+                i32x16 d_next = d_cur;
+                if (i + 1 < TILES) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[slot][(i + 1) % TN], af[slot][(i + 1) / TN], zero, 0, 0, 0);
+                else if (b + 1 < KQ_KB) d_next = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[slot ^ 1][0], af[slot ^ 1][0], zero, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);                    // the MFMA goes first: it runs behind the multiply-adds below
+                // The first result of a stage is read right behind its MFMA: the compiler does not place the wait states
+                // that a vector read of a fresh MFMA result needs in front of inline assembly, so they are written out
+                // (later results are a whole group of multiply-adds old when they are read).
+                if (b == 0 && i == 0) asm volatile("s_nop 15\n\ts_nop 7");
+                // Inline assembly pins the multiply-adds here: as plain arithmetic the compiler gathers the stage's MFMAs in
+                // front and moves the multiply-adds behind the stage barrier, with every result register live in between.
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    if (h == 0 && b == 0) asm volatile("v_mul_i32_i24 %0, %1, %2" : "=v"(sumi[a][c][v]) : "v"(d_cur[v]), "v"(sc[b][a]));
+                    else asm volatile("v_mad_i32_i24 %0, %1, %2, %0" : "+v"(sumi[a][c][v]) : "v"(d_cur[v]), "v"(sc[b][a]));
+                }
+                d_cur = d_next;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    // once per super-block: out += dx * (d * float(sumi) - dmin * summ), the operations of KQ<WT>::value in their order
+    auto fold = [&](int sbp) {
+        const uint8_t *sblk = lds + C::OFF_SBLK + (size_t)sbp * C::SBLK;
+#pragma unroll
+        for (int a = 0; a < TM; a++) {
+            const uint32_t dd = reinterpret_cast<const uint32_t *>(sblk + C::OFF_SD)[r0 + a * 32 + l32];
+            f16x8 fa[T::NF16];
+#pragma unroll
+            for (int f = 0; f < T::NF16; f++)
+                fa[f] = *reinterpret_cast<const f16x8 *>(sblk + C::OFF_FA + (size_t)((2 * f + half) * C::BM + r0 + a * 32 + l32) * 16);
+#pragma unroll
+            for (int c = 0; c < TN; c++) {
+                const f16x8 fb = *reinterpret_cast<const f16x8 *>(sblk + C::OFF_FB + (size_t)(half * C::BN + n0 + c * 32 + l32) * 16);
+                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                f32x16 F[T::NF16];
+#pragma unroll
+                for (int f = 0; f < T::NF16; f++) F[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb, fa[f], zero, 0, 0, 0);
+                float dx[16];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4 t = *reinterpret_cast<const float4 *>(sblk + C::OFF_SX + (size_t)(n0 + c * 32 + 8 * g + 4 * half) * 4);
+                    dx[4 * g] = t.x; dx[4 * g + 1] = t.y; dx[4 * g + 2] = t.z; dx[4 * g + 3] = t.w;
+                }
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    float f[2] = {0.f, 0.f};
+#pragma unroll
+                    for (int j = 0; j < T::NF16; j++) f[j] = F[j][v];
+                    out[a][c][v] = __builtin_fmaf(T::value(0, sumi[a][c][v], f, dd, 0), dx[v], out[a][c][v]);
+                }
+            }
+        }
+    };
+
+    // Stage 2j is half 0 of super-block j, stage 2j + 1 its half 1.  Every stage begins by expanding the following stage
+    // into the idle buffer (an odd stage's expansion is half 0 of the next super-block and carries that super-block's
+    // scales into the other super-block buffer); after an even stage's expansion the registers are free and the next
+    // super-block is fetched into them.  Then the following stage's activations are requested, then the stage is
+    // multiplied.  In front of the barrier a wave waits for all its loads: they were issued a stage ago.
+    constexpr int WAIT0 = 0x0F70;                                          // s_waitcnt vmcnt(0)
+    fetch_sb(0);
+    issue_direct(0, 0u);
+    commit(0u, 0, std::false_type{});
+    __builtin_amdgcn_s_waitcnt(WAIT0);
+    __syncthreads();
+    for (int j = 0; j < nsb; j++) {
+        commit((uint32_t)C::STAGE, 0, std::true_type{});                     // half 1 of super-block j
+        issue_direct(2 * j + 1, (uint32_t)C::STAGE);
+        fetch_sb(j + 1);
+        compute(std::false_type{}, std::false_type{}, j & 1);                // stage 2j from buffer 0
+        __builtin_amdgcn_s_waitcnt(WAIT0);
+        __syncthreads();
+        commit(0u, (j + 1) & 1, std::false_type{});                          // half 0 of super-block j + 1 and its scales
+        issue_direct(2 * j + 2, 0u);
+        compute(std::true_type{}, std::true_type{}, j & 1);                  // stage 2j + 1 from buffer 1
+        fold(j & 1);
+        __builtin_amdgcn_s_waitcnt(WAIT0);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int a = 0; a < TM; a++) {
+        const int64_t row = row_base + r0 + a * 32 + l32;
+        if (row >= N) continue;
+#pragma unroll
+        for (int c = 0; c < TN; c++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t tok = tok_base + n0 + c * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+                if (tok < M) y[(size_t)gv.out_row(tok) * ldy + row] = out[a][c][v];
+            }
+        }
+    }
+}
+
 // With few tokens the GEMM's time is its walk over K (about 1.5 - 2 us per super-block, whatever the token count:
 // 28 - 35 us at K = 4096, 88 - 112 us at K = 14336), while the GEMV forms pass over the weights once per 8 or 16 tokens at
 // memory speed.  Up to 128 tokens on a matrix with few row tiles the walk is cut into slices (kq_slices_for below:
@@ -622,6 +933,33 @@ static hipError_t launch_kq(const void *W, size_t nb01, int64_t K, int64_t N, co
     return hipGetLastError();
 }
 
+template <int WT, int TM, int TN, int WR, int WC, int OCC, bool GATHER>
+static hipError_t launch_ks(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int64_t M,
+                            float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg, int64_t n_as,
+                            int slices = 1, float *part = nullptr) {
+    if constexpr (WT == T_Q6_K) return hipErrorInvalidValue;
+    else {
+        using C = KsCfg<WT, TM, TN, WR, WC>;
+        const size_t lds_bytes = C::TOTAL;
+        if ((int64_t)lds_bytes > lim.max_lds_per_block) return hipErrorInvalidValue;
+        auto kfn = gemm_ks_kernel<WT, TM, TN, WR, WC, OCC, GATHER>;
+        static LdsGrant grant;
+        if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
+        const int per_cu = lds_bytes > 80 * 1024 ? 1 : 2;
+        const TileMap map = make_tile_map(ceil_div(N, C::BM), GATHER ? 1 : ceil_div(M, C::BN), 32 * per_cu);
+        if (!GATHER && slices > 1) {
+            const int slice_sb = (int)ceil_div(K / QK_K, (int64_t)slices);
+            hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)slices), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                               (const uint8_t *)ws, ws_stride, M, part, N, map, rg, slice_sb);
+            if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+            return launch_sum_slices(part, slices, M, N, y, ldy, st);
+        }
+        hipLaunchKernelGGL(kfn, dim3(map.grid, (unsigned)n_as), dim3(C::NT), lds_bytes, st, (const uint8_t *)W, nb01, K, N,
+                           (const uint8_t *)ws, ws_stride, M, y, ldy, map, rg, 0);
+        return hipGetLastError();
+    }
+}
+
 template <int WT>
 static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride,
                                  int64_t M, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st, const RowGather &rg,
@@ -635,12 +973,17 @@ static hipError_t launch_kq_type(const void *W, size_t nb01, int64_t K, int64_t 
     // 128 rows x 128 tokens per workgroup when that gives every CU one, else 64 x 128.
     if (rg.perm)                                                                     // expert groups: 64 x 128 tiles
         return launch_kq<WT, 2, 2, 2, true>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);
-    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128);
-    const int cfg = (int)tune("CHIP_GEMM_KQ_CFG", g128 >= cus ? 0 : 2);
+    // Q4_K and Q5_K with enough 64 x 128 tiles to give every CU its two workgroups more than once: the single-plane kernel.
+    // Measured (us, K = 4096, tokens x rows; two-plane kernel -> single plane): Q4_K 2048 x 14336 432 -> 385, 2048 x 4096
+    // 118 -> 108, 512 x 4096 36 -> 39 (stays); Q5_K 553 -> 455, 150 -> 125, 43 -> 42; Q4_K 512 x 4096 with K = 14336 107 -> 124 (stays).
+    const int64_t g128 = ceil_div(N, 128) * ceil_div(M, 128), g64x128 = ceil_div(N, 64) * ceil_div(M, 128);
+    const bool single_plane = WT != T_Q6_K && g64x128 >= (WT == T_Q5_K ? 1 : 2) * cus;
+    const int cfg = (int)tune("CHIP_GEMM_KQ_CFG", single_plane ? 11 : g128 >= cus ? 0 : 2);
     switch (cfg) {
         case 0: return launch_kq<WT, 4, 2, 3, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 128 x 128, 8 + 4 waves
         case 1: return launch_kq<WT, 4, 1, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 128 x 64, 4 + 4 waves
         case 2: return launch_kq<WT, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);      // 64 x 128, 4 + 4 waves
+        case 11: return launch_ks<WT, 1, 2, 2, 2, 2, false>(W, nb01, K, N, ws, ws_stride, M, y, ldy, lim, st, rg, n_as);   // single plane, 64 x 128, 4 waves
         default: return hipErrorInvalidValue;
     }
 }

@@ -646,6 +646,40 @@ def test_gemm_kquant_prefill_shape_sampled(dev, orc, wt):
     assert np.array_equal(y2[:, ::-1], y[:64])
 
 
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q5_K), ids=lambda t: O.TYPE_NAMES[t])
+def test_gemm_kquant_single_plane_kernel(dev, orc, wt):
+    """Shapes with many output tiles take the kernel that feeds the quants as one int8 plane and applies the 6-bit
+    sub-block scales with integer multiply-adds.  (a) d = dmin = 1, activation scale 1, one super-block: the output is
+    sumi - summ itself, compared bit for bit with the reference's integer sums on a sample that covers the first and the
+    last (ragged) tiles; (b) real scales over four super-blocks against the oracle within the tolerance; (c) the same bits
+    whatever tile a row lands in."""
+    N, M = 4090, 1000                                    # 64 x 8 tiles of 64 rows x 128 tokens, both edges ragged
+    rng = np.random.default_rng(31 + wt)
+    rows = np.unique(np.concatenate([[0, 1, 63, 64, N - 1, N - 2], rng.choice(N, 40, replace=False)]))
+    toks = np.unique(np.concatenate([[0, 31, 32, 127, 128, M - 1], rng.choice(M, 18, replace=False)]))
+    # (a)
+    K = 256
+    w = random_kquant_rows(wt, rng, N, 1)
+    x = exact_q8_K_inputs(rng, M, K)
+    x[7, 1:] = 0.0
+    aq = orc.quantize_activation(O.Q8_K, x)
+    y = dev.mul_mat(wt, w, x, split_k=False)
+    for t in toks:
+        for i in rows:
+            _, isum, imin = orc.vec_dot(wt, K, w[i], aq[t], want_sums=True)
+            want = int(isum.sum()) - int(imin.sum())
+            assert abs(want) < 2 ** 24 and int(y[t, i]) == want and float(y[t, i]) == float(want), (t, i)
+    # (b), (c)
+    K = 1024
+    wq = orc.quantize_weights(wt, common.weights_f32(90 + wt, N, K, outliers=True))
+    x = common.activations_f32(90 + wt, M, K)
+    y = dev.mul_mat(wt, wq, x, split_k=False)
+    ref = orc.mul_mat(wt, wq[rows], x[toks], nthreads=8, want=("sum_abs",))
+    check_outputs(y[np.ix_(toks, rows)], ref["y"], ref["sum_abs"], "single-plane k-quant gemm")
+    y2 = dev.mul_mat(wt, wq[::-1].copy(), x, split_k=False)
+    assert np.array_equal(y2[:, ::-1], y)
+
+
 # ------------------------------------------------------------------------------------------ MUL_MAT_ID (expert matmul)
 def moe_case(orc, wt, K, N, n_as, n_used, n_tokens, ne11, seed):
     rng = np.random.default_rng(seed)
