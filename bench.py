@@ -442,6 +442,32 @@ def measured_mfma_peak():
     return {"instruction": "v_mfma_i32_32x32x32_i8", "TOPS": best, "datasheet_TOPS": INT8_PEAK_TOPS} if best else None
 
 
+def measured_read_floor():
+    """Runs the read-only streaming probe (a child process): what a kernel that only reads the bytes of each matrix of the
+    decode trace costs on this GPU, cold.  The sum over one step is the floor under a one-kernel-per-op decode step."""
+    import re
+    import subprocess
+    exe = os.path.join(ROOT, "cactus_amd", "probes", "bin", "read_stream")
+    if not os.path.exists(exe):
+        return None
+    try:
+        txt = subprocess.run([exe], capture_output=True, text=True, timeout=120).stdout
+    except Exception:
+        return None
+    out = {}
+    for line in txt.splitlines():
+        m = re.match(r"read\s+([\d.]+) MB \((.*?)\s*\): cold\s+([\d.]+) us", line)
+        if m:
+            out[m.group(2).strip()] = {"MB": float(m.group(1)), "cold_us": float(m.group(3))}
+        m = re.match(r"empty kernel, back to back: ([\d.]+) us", line)
+        if m:
+            out["empty_launch_us"] = float(m.group(1))
+    need = ("wq+wk+wv", "wo Q4_K 4096x4096 / config 1", "ffn_gate+ffn_up", "ffn_down Q6_K / config 2 Q8_0", "output head Q6_K 128256x4096")
+    if all(k in out for k in need):
+        out["decode_step_floor_us"] = round(32 * sum(out[k]["cold_us"] for k in need[:4]) + out[need[4]]["cold_us"], 1)
+    return out or None
+
+
 class Trace:
     """BASELINE configs[4]: the weight matmuls of a Llama-3-8B-shaped Q4_K_M model (32 layers; attn_v / ffn_down / the
     output head in Q6_K, the rest Q4_K) as random-init weights in one arena, and the launches of one step over them."""
@@ -775,11 +801,11 @@ def bench_trace_more(dev, hip, trace, eager):
 
 def backend_graph_timing():
     """The same model as a ggml graph through the reference's scheduler and libggml-hip.so (every node on the device):
-    tests/backend_graph_timing.py in a child process - the host framework there is the reference's own ggml build, which
-    only the test tree may load.  Returns its figures, or the reason there are none."""
+    bench_backend_graph.py in a child process - the host framework there is the reference's own ggml build (oracle/_ref),
+    which is there as the host of the backend, not as something measured.  Returns its figures, or the reason there are none."""
     import re
     import subprocess
-    script = os.path.join(ROOT, "tests", "backend_graph_timing.py")
+    script = os.path.join(ROOT, "bench_backend_graph.py")
     ref_so = os.path.join(ROOT, "oracle", "_ref", "libggml_ref.so")
     if not os.path.exists(ref_so):
         return {"skipped": "no host framework on this machine (oracle/_ref/libggml_ref.so)"}
@@ -806,13 +832,46 @@ def backend_graph_timing():
 
 
 def cpu_model():
+    """The first processor entry of /proc/cpuinfo: model string, family / model / stepping, and the SIMD flags that decide
+    which ggml-cpu kernels a native build would take (the reference build here is pinned to AVX2)."""
+    info = {}
     try:
         for line in open("/proc/cpuinfo"):
-            if line.startswith("model name"):
-                return line.split(":", 1)[1].strip()
+            if ":" not in line:
+                if info:
+                    break
+                continue
+            k, v = (p.strip() for p in line.split(":", 1))
+            if k in ("vendor_id", "cpu family", "model", "model name", "stepping", "cpu cores", "siblings"):
+                info[k] = v
+            elif k == "flags":
+                fl = set(v.split())
+                info["simd"] = " ".join(f for f in ("avx2", "fma", "f16c", "avx512f", "avx512bw", "avx512vl", "avx512_vnni", "avx_vnni", "amx_int8") if f in fl)
     except OSError:
         pass
-    return "unknown"
+    if not info:
+        return "unknown"
+    return "%s (%s family %s model %s stepping %s; %s cores / %s threads per package; %s)" % (
+        info.get("model name", "?"), info.get("vendor_id", "?"), info.get("cpu family", "?"), info.get("model", "?"),
+        info.get("stepping", "?"), info.get("cpu cores", "?"), info.get("siblings", "?"), info.get("simd", ""))
+
+
+def cpu_topology():
+    """Logical CPUs online, those this process may run on, and the distinct physical cores among them."""
+    try:
+        allowed = sorted(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = list(range(os.cpu_count() or 1))
+    cores = set()
+    for c in allowed:
+        try:
+            pkg = open("/sys/devices/system/cpu/cpu%d/topology/physical_package_id" % c).read().strip()
+            core = open("/sys/devices/system/cpu/cpu%d/topology/core_id" % c).read().strip()
+            cores.add((pkg, core))
+        except OSError:
+            cores.add(("?", c))
+    return {"logical_cpus_online": os.cpu_count(), "logical_cpus_allowed": len(allowed), "physical_cores_allowed": len(cores),
+            "threads_used_cap": 16}
 
 
 def physical_cores():
@@ -871,7 +930,7 @@ def cpu_baseline():
             break
     main_leg = legs["T%d" % T]
     return {"value": main_leg["GBps"], "unit": "GB/s", "cores": T, "kind": "reference" if use_ref else "port",
-            "cpu_model": cpu_model(), "legs": legs,
+            "cpu_model": cpu_model(), "cpu_topology": cpu_topology(), "legs": legs,
             "build": "gcc -O2 -mavx2 -mfma -mf16c -ffp-contract=off (AVX2 kernels of ggml-cpu-quants.c; no -march=native)" if use_ref
                      else "gcc -O2 scalar restatement",
             "sample": "one layer of the headline trace at one token (wq, wk, wv, wo, ffn_up, ffn_gate, ffn_down: 7 matmuls, "
@@ -899,6 +958,7 @@ def main():
         extra["config2_q8_0_ffn_gemv"] = bench_config2(dev, hip)
         extra.update(bench_extra(dev, hip))
         extra["mfma_i8_measured_peak"] = measured_mfma_peak()
+        extra["read_only_floor"] = measured_read_floor()
         if not args.no_backend and not args.eager:
             extra["backend_graph"] = backend_graph_timing()
     cpu = None if args.no_cpu else cpu_baseline()

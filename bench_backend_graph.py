@@ -4,7 +4,7 @@ ggml (oracle/_ref/libggml_ref.so), weights and caches live in HIP buffers, and t
 backend.  Prints the wall time of lm_ggml_backend_sched_graph_compute for NTOK new tokens (one launch per kernel, no
 HIP graph), and the backend's counters.  Not a test (pytest does not collect it):
 
-    NTOK=1 python tests/backend_graph_timing.py          # decode;  NTOK=8 / 32 / 512: small batches, a prefill chunk
+    NTOK=1 python bench_backend_graph.py          # decode;  NTOK=8 / 32 / 512: small batches, a prefill chunk
 """
 import ctypes as C
 import os
@@ -13,8 +13,9 @@ import time
 
 import numpy as np
 
-sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))          # ggml_host: the ctypes host over the reference's ggml build
 import oracle as O
 from ggml_host import Host
 

@@ -221,7 +221,9 @@ constexpr int D_LDS = D_NBUF * D_STAGE;
 
 // The load itself is inline assembly: the compiler, which cannot tell that a load into one stage buffer does not alias a
 // ds_read from another, would otherwise wait for every outstanding load before each LDS read.  The waits are placed by
-// hand instead (one vmcnt per stage, below).  M0 carries the LDS byte address of the wave's 1 KB destination.
+// hand instead (one vmcnt per stage, below).  M0 carries the LDS byte address of the wave's 1 KB destination.  The
+// compiler is not told about that write (it does not take M0 as a clobber of inline assembly), so nothing else in a kernel
+// that uses this may need M0: no dynamic indexing of register arrays, no s_sendmsg.
 __device__ __forceinline__ void load16_to_lds(const uint8_t *src, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
 }

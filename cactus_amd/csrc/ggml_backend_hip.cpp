@@ -962,7 +962,9 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         if ((n <= 4 || n == 8) && fusion_enabled()) {      // the token counts chip_mul_mat_group has a one-launch form for
             bool slots_free = true;
             for (int slot : grouped) slots_free = slots_free && slot < 0;
-            if (slots_free) n_members = grouped_matmuls(cgraph, i, members);
+            // A SILU held back for its MUL reads the gate projection's result only when that MUL runs, after this node:
+            // a later projection run here could be sitting in memory the allocator freed from under it, so no group then.
+            if (slots_free && !waiting_silu) n_members = grouped_matmuls(cgraph, i, members);
         }
         if (n_members >= 2) {
             chip_mat mats[CHIP_GROUP_MAX];

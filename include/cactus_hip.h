@@ -207,7 +207,10 @@ CHIP_API int chip_mul_mat_run_ws(int type, const void *W, size_t nb01, int64_t K
  * until the process ends); the call allocates nothing and frees nothing.  Results equal chip_mul_mat's with a workspace
  * of that size, bit for bit.  CHIP_ENOMEM when chip_mul_mat_workspace_size(type, K, n) exceeds the array (e.g. more than
  * 3500 tokens of K = 4096).  All calls on one GPU share the array: calls that may overlap in time (different streams)
- * race; calls on one stream are ordered and safe.  Nothing in the array has to start at zero. */
+ * race; calls on one stream are ordered and safe.  Nothing in the array has to start at zero.
+ * Set-up is not part of that promise: chip_init() on the device looks up the array's address, and the first launch of a
+ * kernel shape raises that kernel's LDS limit (a host call).  A caller under stream capture therefore calls chip_init()
+ * and makes one ordinary call of the same (type, K, N, n) before it captures; captured calls replay correctly. */
 CHIP_API size_t chip_mul_mat_noalloc_max_workspace(void);
 CHIP_API int    chip_mul_mat_noalloc(int type, const void *W, size_t nb01, int64_t K, int64_t N,
                                      const float *x, int64_t ldx, int64_t n, float *y, int64_t ldy, void *stream);

@@ -6,7 +6,8 @@ Q4_K and Q6_K rows against Q8_K activations quantized inside the op.
 
 Weights: a base block of rows quantized by the oracle's restatement of the reference quantizers, repeated down the matrix
 (quantizing 525 M values for the output head on the CPU would take minutes); every output row of every repetition is
-compared, so row tiles at every position of the grid are covered, first and last rows included.  Each case also prints how
+compared, so row tiles at every position of the grid are covered, first and last rows included.  A second test gives every
+repetition its own scale bytes, so that no two row tiles are alike, and checks a sample of rows of every repetition.  Each case also prints how
 far the GPU and the oracle (= the reference's AVX2 summation order) each are from the exact value of sum scale * isum
 evaluated in fp64, in units of the tolerance, on a sample of rows."""
 import numpy as np
@@ -81,6 +82,47 @@ def test_trace_matmul_vs_oracle(dev, orc, name, wt, N, K, nbase, n):
         assert (y == y[:, :1, :]).all()
     g, r = attribution(orc, wt, K, base, ref["wdata"], y[:, 0, :], ref["y"], ref["sum_abs"], "%s n=%d" % (name, n))
     assert g <= 1.0
+
+
+def distinct_repetitions(wt, base, reps, K):
+    """The base rows repeated `reps` times with one scale byte changed per repetition - the low mantissa byte of the fp16
+    super-block scale d of super-block (rep mod super-blocks per row), XORed with a value that differs between neighbouring
+    repetitions - so that no two row tiles of the matrix hold the same bytes: a kernel that swaps or aliases whole tiles
+    then gives wrong numbers somewhere, which identical repetitions cannot show."""
+    nbase, row_bytes = base.shape
+    bb = O.BLOCK_BYTES[wt]
+    d_off = 208 if wt == O.Q6_K else 0
+    W = np.tile(base, (reps, 1)).reshape(reps, nbase, row_bytes)
+    nsb = K // 256
+    for rep in range(reps):
+        W[rep, :, (rep % nsb) * bb + d_off] ^= np.uint8(1 + (rep * 37) % 255)
+    return W.reshape(reps * nbase, row_bytes)
+
+
+@pytest.mark.parametrize("name,wt,N,K,nbase", [m for m in TRACE_MATMULS if m[0] != "wk"], ids=[m[0] for m in TRACE_MATMULS if m[0] != "wk"])
+@pytest.mark.parametrize("n", [1, 8])
+def test_trace_matmul_no_two_tiles_alike(dev, orc, name, wt, N, K, nbase, n):
+    """The same shapes with every repetition of the base rows made distinct; the oracle evaluates a sample of rows of
+    every repetition (first and last row of the matrix included, at least 16 per repetition: 6144 rows of the output head)."""
+    print("config5 distinct", name, O.TYPE_NAMES[wt], "N", N, "K", K, "n", n, flush=True)
+    base = base_rows(orc, wt, 5000 + N + K, nbase, K)
+    reps = N // nbase
+    W = distinct_repetitions(wt, base, reps, K)
+    x = common.activations_f32(5 + n + K, n, K)
+    y = dev.mul_mat(wt, W, x)
+    rng = np.random.default_rng(N + n)
+    per_rep = 16 if reps >= 16 else 256 // reps
+    rows = np.concatenate([rep * nbase + np.sort(rng.choice(nbase, per_rep, replace=False)) for rep in range(reps)])
+    rows[0], rows[-1] = 0, N - 1
+    ref = orc.mul_mat(wt, W[rows], x, nthreads=8, want=("sum_abs",))
+    del W
+    err = np.abs(y[:, rows].astype(np.float64) - ref["y"].astype(np.float64))
+    bound = REL_TOL * ref["sum_abs"]
+    assert (err <= bound).all(), "%s n=%d: worst error %.3g x the tolerance" % (name, n, float((err / bound).max()))
+    # the changed scale moves a row's result by far more than the tolerance, so a tile read from the wrong repetition fails:
+    base_ref = orc.mul_mat(wt, base[rows[per_rep:2 * per_rep] % nbase], x, nthreads=8, want=("sum_abs",))
+    moved = np.abs(ref["y"][:, per_rep:2 * per_rep].astype(np.float64) - base_ref["y"].astype(np.float64))
+    assert (moved > 4 * bound[:, per_rep:2 * per_rep]).mean() > 0.5
 
 
 def test_trace_gate_up_pair_and_v_store(dev, orc):

@@ -787,7 +787,7 @@ def test_mul_mat_id_argument_errors(dev, orc):
     ((O.F16, 40), (O.F16, 3)),
     ((O.Q6_K, 2000),),                                               # a group of one
 ], ids=["kquants", "block32", "f16", "single"])
-@pytest.mark.parametrize("K", [1024, 4096])
+@pytest.mark.parametrize("K", [1024, 4096, 14336])                   # 14336: a single call builds its LDS image a step's part at a time
 def test_mul_mat_group_equals_single_calls(dev, orc, members, K):
     """chip_mul_mat_group: each member's output equals chip_mul_mat on that member alone, bit for bit, for every token
     count class (1, 2, 4: one launch; 3, 7: one quantizer and the GEMVs; 40: the GEMMs), and the oracle within tolerance."""

@@ -51,6 +51,51 @@ def test_noalloc_equals_mul_mat_two_calls_in_a_row(orc, wt):
         assert (err <= 1e-5 * ref["sum_abs"]).all(), (O.TYPE_NAMES[wt], n, rows)
 
 
+def test_noalloc_leaves_device_memory_alone_and_replays_from_a_graph(orc):
+    """After chip_init() and one warm call per shape (the first launch of a kernel raises its LDS limit, a host call), a
+    call changes nothing about the device's free memory, and a call recorded under stream capture replays - three times,
+    with other work and synchronizations in between - to the bits chip_mul_mat gives."""
+    import ctypes as C
+    import cactus_amd
+    dev = cactus_amd.Device(0)
+    L = dev.lib
+    hip = C.CDLL("libamdhip64.so")
+    K, N = 4096, 300
+    wt = O.Q4_K
+    W = orc.quantize_weights(wt, common.weights_f32(190, N, K))
+    nb01 = dev.row_size(wt, K)
+    dW = dev.to_device(W)
+    st = C.c_void_p()
+    dev.check(L.chip_stream_create(C.byref(st)))
+    for n in (1, 8, 64):
+        x = common.activations_f32(191 + n, n, K)
+        want = run_pair(dev, wt, W, x, False)
+        dx, dy = dev.to_device(x), dev.alloc(n * N * 4)
+        dev.check(L.chip_mul_mat_noalloc(wt, dW.ptr, nb01, K, N, dx.ptr, K, n, dy.ptr, N, st))     # warm call
+        dev.sync(st)
+        free0, free1, tot = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free0), C.byref(tot)) == 0
+        dev.check(L.chip_mul_mat_noalloc(wt, dW.ptr, nb01, K, N, dx.ptr, K, n, dy.ptr, N, st))
+        dev.sync(st)
+        assert hip.hipMemGetInfo(C.byref(free1), C.byref(tot)) == 0
+        assert free0.value == free1.value, "the call changed the device's free memory"
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(st, 0) == 0
+        rc = L.chip_mul_mat_noalloc(wt, dW.ptr, nb01, K, N, dx.ptr, K, n, dy.ptr, N, st)
+        assert hip.hipStreamEndCapture(st, C.byref(graph)) == 0 and rc == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for rep in range(3):
+            dev.check(L.chip_memset(dy.ptr, 0xFF, n * N * 4, st))
+            dev.sync(st)
+            assert hip.hipGraphLaunch(gexec, st) == 0
+            dev.sync(st)
+            got = dy.download(np.float32, n * N).reshape(n, N)
+            assert got.tobytes() == want.tobytes(), (n, rep)
+            run_pair(dev, wt, W[:50], common.activations_f32(5 + rep, 3, K), True)        # other work on the shared array
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+
+
 def test_noalloc_rejects_what_does_not_fit():
     import cactus_amd
     dev = cactus_amd.Device(0)
