@@ -741,10 +741,15 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
             ck(L.chip_mul_mat_f16_batched(kc, 2 * KV, 2 * hd, hd, n_kv, n_head_kv, q.ptr, hd * n_head, hd, n, n_head, kq.ptr, n_kv,
                                           n_kv * n, aws.ptr, aws_bytes, st))
             ck(L.chip_soft_max(kq.ptr, n_kv, mask.ptr, ca.F16, n_kv, n, n_head * n, 0.0884, 0.0, kq.ptr, n_kv, st))
-            ck(L.chip_mul_mat_f16_batched(vc, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv, kq.ptr, n_kv, n_kv * n, n, n_head,
-                                          kqv.ptr, hd, hd * n, aws.ptr, aws_bytes, st))
-            ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
-                          A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
+            if L.chip_mul_mat_f16_batched_second_copy_supported(n_head_kv, n_head, n) == 1:
+                # kqv and the head merge that follows it in one launch, as the backend runs the two nodes of a decode step
+                ck(L.chip_mul_mat_f16_batched_two_copies(vc, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv, kq.ptr, n_kv, n_kv * n, n,
+                                                         n_head, kqv.ptr, hd, hd * n, merged.ptr, H, hd, aws.ptr, aws_bytes, st))
+            else:
+                ck(L.chip_mul_mat_f16_batched(vc, 2 * kv_size, 2 * kv_size * hd, n_kv, hd, n_head_kv, kq.ptr, n_kv, n_kv * n, n, n_head,
+                                              kqv.ptr, hd, hd * n, aws.ptr, aws_bytes, st))
+                ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
+                              A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
             mm(*W["wo"], merged, att)
             # residual + norm + weight: one kernel, as the backend fuses the three nodes
             ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))

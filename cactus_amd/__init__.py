@@ -37,7 +37,7 @@ EXPORTS = (
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
-    "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size",
+    "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
     "chip_workspace_to_blocks",
 )
@@ -138,6 +138,8 @@ def load_library(path=KERNEL_LIB):
     L.chip_get_rows.argtypes = [i32, vp, sz, sz, sz, i64, i64, vp, i64, i64, i64, i64, i64, vp, i64, i64, i64, vp]
     L.chip_mul_mat_f16_batched.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_f16_batched_workspace_size.restype = sz
+    L.chip_mul_mat_f16_batched_second_copy_supported.argtypes = [i64, i64, i64]
+    L.chip_mul_mat_f16_batched_two_copies.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_f16_batched_workspace_size.argtypes = [i64, i64, i64, i64, i64]
     L.chip_mul_mat_id_workspace_size.restype = sz
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
@@ -449,10 +451,11 @@ class Device:
         self.sync()
         return dy.download(np.float32, ids.size * nc).reshape(ids.size, nc)
 
-    def mul_mat_f16_batched(self, W, x, workspace=True):
+    def mul_mat_f16_batched(self, W, x, workspace=True, merged=False):
         """W fp16 array or view [ne02, N, K] (K contiguous), x fp32 array or view [ne12, n, K] (K contiguous) ->
         y fp32 [ne12, n, N]; the views are uploaded with their own strides.  workspace=False withholds the workspace
-        (dot-product kernels only)."""
+        (dot-product kernels only).  merged=True: chip_mul_mat_f16_batched_two_copies, returns (y, the second copy laid
+        out [n, ne12 * N], a token's heads side by side)."""
         def upload(v):
             base = v
             while isinstance(base.base, np.ndarray):
@@ -467,6 +470,15 @@ class Device:
         dy = self.alloc(ne12 * n * N * 4)
         wsz = self.lib.chip_mul_mat_f16_batched_workspace_size(K, N, ne02, ne12, n) if workspace else 0
         ws = self.alloc(wsz) if wsz else None
+        if merged:
+            dy2 = self.alloc(ne12 * n * N * 4)
+            self.check(self.lib.chip_memset(dy2.ptr, 0xFF, ne12 * n * N * 4, None))          # NaN: unwritten values show
+            self.check(self.lib.chip_mul_mat_f16_batched_two_copies(dw.ptr + woff, W.strides[1], W.strides[0], K, N, ne02,
+                                                                    dx.ptr + xoff, x.strides[1] // 4, x.strides[0] // 4, n, ne12,
+                                                                    dy.ptr, N, n * N, dy2.ptr, ne12 * N, N, ws.ptr if ws else None,
+                                                                    wsz, None))
+            self.sync()
+            return (dy.download(np.float32, ne12 * n * N).reshape(ne12, n, N), dy2.download(np.float32, ne12 * n * N).reshape(n, ne12 * N))
         self.check(self.lib.chip_mul_mat_f16_batched(dw.ptr + woff, W.strides[1], W.strides[0], K, N, ne02, dx.ptr + xoff,
                                                      x.strides[1] // 4, x.strides[0] // 4, n, ne12, dy.ptr, N, n * N,
                                                      ws.ptr if ws else None, wsz, None))

@@ -74,6 +74,7 @@ struct BatchedArgs {
     const float *x; int64_t ldx1, ldx2;      // token and batch strides of src1, in floats
     int64_t n, r2;
     float *y; int64_t ldy1, ldy2;            // token and batch strides of dst, in floats
+    float *y2; int64_t ld2y1, ld2y2;         // optional second copy of dst under strides of its own (the dot-product kernels only)
 };
 // Column c of KV head b0: query head c % r2 of its group, token c / r2 (32-bit division: 64-bit is a long software routine).
 __device__ __forceinline__ const float *col_x(const BatchedArgs &a, int64_t b0, int64_t c) {
@@ -83,6 +84,10 @@ __device__ __forceinline__ const float *col_x(const BatchedArgs &a, int64_t b0, 
 __device__ __forceinline__ float *col_y(const BatchedArgs &a, int64_t b0, int64_t c) {
     const uint32_t r2 = (uint32_t)a.r2, t = (uint32_t)c / r2, h = (uint32_t)c - t * r2;
     return a.y + (b0 * a.r2 + h) * a.ldy2 + (int64_t)t * a.ldy1;
+}
+__device__ __forceinline__ float *col_y2(const BatchedArgs &a, int64_t b0, int64_t c) {
+    const uint32_t r2 = (uint32_t)a.r2, t = (uint32_t)c / r2, h = (uint32_t)c - t * r2;
+    return a.y2 + (b0 * a.r2 + h) * a.ld2y2 + (int64_t)t * a.ld2y1;
 }
 
 // ---- short rows: K <= 8 * LPR, one 16-byte chunk per lane ----
@@ -128,7 +133,10 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedAr
                 if (sub == 0 && row < a.N) {
 #pragma unroll
                     for (int j = 0; j < AM_COLS; j++)
-                        if (c0 + j < cols) col_y(a, b0, c0 + j)[row] = acc[j];
+                        if (c0 + j < cols) {
+                            col_y(a, b0, c0 + j)[row] = acc[j];
+                            if (a.y2) col_y2(a, b0, c0 + j)[row] = acc[j];
+                        }
                 }
             }
         }
@@ -181,8 +189,11 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArg
             __syncthreads();
             if (threadIdx.x < AM_ROWS * AM_COLS) {
                 const int r = threadIdx.x / AM_COLS, j = threadIdx.x % AM_COLS;
-                if (r0 + r < a.N && c0 + j < cols)
-                    col_y(a, b0, c0 + j)[r0 + r] = (part[0][r][j] + part[1][r][j]) + (part[2][r][j] + part[3][r][j]);
+                if (r0 + r < a.N && c0 + j < cols) {
+                    const float v = (part[0][r][j] + part[1][r][j]) + (part[2][r][j] + part[3][r][j]);
+                    col_y(a, b0, c0 + j)[r0 + r] = v;
+                    if (a.y2) col_y2(a, b0, c0 + j)[r0 + r] = v;
+                }
             }
             __syncthreads();
         }
@@ -446,6 +457,8 @@ GemmPlan gemm_plan(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
 }  // namespace
 
 bool mul_mat_f16_batched_supported(int64_t K) { return K > 0 && K % 8 == 0; }
+// the second copy of the result: written by the dot-product kernels, which take up to AM_COLS (query head, token) pairs per KV head
+bool mul_mat_f16_batched_second_copy_supported(int64_t r2, int64_t n) { return r2 > 0 && n > 0 && r2 * n <= AM_COLS; }
 
 // the split-K pair: 5 to AS_MAX_COLS columns per KV head, long rows, up to AS_MAX_ROWS rows (head sizes)
 static size_t slice_plan_bytes(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n) {
@@ -462,13 +475,15 @@ size_t mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne02, in
 
 hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
                                       int64_t ldx1, int64_t ldx2, int64_t n, int64_t r2, float *y, int64_t ldy1, int64_t ldy2,
-                                      void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st) {
+                                      void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st, float *y2,
+                                      int64_t ld2y1, int64_t ld2y2) {
     if (N <= 0 || n <= 0 || ne02 <= 0 || r2 <= 0) return hipSuccess;
     if (!mul_mat_f16_batched_supported(K) || ne02 > 65535 || r2 * n > 0x7fffffff) return hipErrorInvalidValue;
+    if (y2 && !mul_mat_f16_batched_second_copy_supported(r2, n)) return hipErrorInvalidValue;
     const bool mfma_rows = tune("CHIP_ATTN_MFMA", 1) != 0;
     if (const size_t sp = slice_plan_bytes(K, N, ne02, r2, n); mfma_rows && sp > 0 && workspace && workspace_bytes >= sp &&
                                                               (((uintptr_t)workspace) & 15) == 0) {
-        const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
+        const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2, nullptr, 0, 0};
         const int64_t cols = r2 * n, slices = ceil_div(K, (int64_t)AS_SLICE);
         const dim3 grid((unsigned)slices, (unsigned)ne02), block(AS_WAVES * 64);
         float *part = (float *)workspace;
@@ -483,7 +498,7 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
     }
     const GemmPlan plan = gemm_plan(K, N, ne02, r2, n);
     // the GEMM writes row R of y at R * ldy1: the batches of y must follow each other without a gap
-    if (plan.use && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {
+    if (plan.use && !y2 && workspace && workspace_bytes >= plan.bytes && ldy2 == n * ldy1 && n <= 65535 && ne02 * r2 <= 65535) {
         uint8_t *ws = (uint8_t *)workspace;
         int32_t *perm = (int32_t *)(ws + plan.off_perm), *offsets = (int32_t *)(ws + plan.off_offsets), *tiles = (int32_t *)(ws + plan.off_tiles);
         // one row tile, or two with at most 1024 columns per KV head (kqv: a head's rows): the GEMM reads the fp32 activations
@@ -506,7 +521,7 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
         return launch_gemm_f16(W, nb01, K, N, ws, plan.act_stride, ne02 * r2 * n, y, ldy1, lim, st, &rg, plan.n_tiles, plan.tile,
                                direct ? &fr : nullptr);
     }
-    const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2};
+    const BatchedArgs a{(const uint8_t *)W, nb01, nb02, K, N, x, ldx1, ldx2, n, r2, y, ldy1, ldy2, y2, ld2y1, ld2y2};
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     const int64_t cols = r2 * n;
     if (mfma_rows && cols > AM_COLS && cols <= 64 && N <= 16LL * 0x7fffffff) {

@@ -806,21 +806,39 @@ size_t chip_mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne0
     if (ne02 <= 0 || ne12 <= 0 || ne12 % ne02 != 0) return 0;
     return mul_mat_f16_batched_workspace_size(K, N, ne02, ne12 / ne02, n);
 }
-int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
-                             int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y, int64_t ldy1, int64_t ldy2,
-                             void *workspace, size_t workspace_bytes, void *stream) {
+static int mul_mat_f16_batched_checked(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
+                                       int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y, int64_t ldy1, int64_t ldy2, float *y2,
+                                       int64_t ld2y1, int64_t ld2y2, void *workspace, size_t workspace_bytes, void *stream) {
     if (K < 0 || N < 0 || n < 0 || ne02 < 0 || ne12 < 0) return CHIP_EINVAL;
     if (ne02 > 0 && ne12 % ne02 != 0) return CHIP_EINVAL;                   // src1's batch must be a multiple of src0's
     if (N == 0 || n == 0 || ne12 == 0) return CHIP_OK;
     if (K == 0 || K % 8 != 0 || ne02 > 65535) return CHIP_EUNSUPPORTED;
+    if (y2 && !mul_mat_f16_batched_second_copy_supported(ne12 / ne02, n)) return CHIP_EUNSUPPORTED;
     if (!W || !x || !y) return CHIP_EINVAL;
     if (!aligned16(W) || nb01 % 16 != 0 || nb02 % 16 != 0 || nb01 < (size_t)K * 2) return CHIP_EINVAL;
     if (!aligned16(x) || ((ldx1 | ldx2) & 3) != 0 || (((uintptr_t)y) & 3) != 0 || ldy1 < N) return CHIP_EINVAL;
+    if (y2 && ((((uintptr_t)y2) & 3) != 0 || ld2y1 < 0 || ld2y2 < 0)) return CHIP_EINVAL;
     if (workspace && !aligned16(workspace)) return CHIP_EINVAL;
     DeviceLimits lim;
     if (int rc = current_limits(lim); rc != CHIP_OK) return rc;
     return hip_rc(launch_mul_mat_f16_batched(W, nb01, nb02, K, N, ne02, x, ldx1, ldx2, n, ne12 / ne02, y, ldy1, ldy2, workspace,
-                                             workspace_bytes, lim, (hipStream_t)stream));
+                                             workspace_bytes, lim, (hipStream_t)stream, y2, ld2y1, ld2y2));
+}
+int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
+                             int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y, int64_t ldy1, int64_t ldy2,
+                             void *workspace, size_t workspace_bytes, void *stream) {
+    return mul_mat_f16_batched_checked(W, nb01, nb02, K, N, ne02, x, ldx1, ldx2, n, ne12, y, ldy1, ldy2, nullptr, 0, 0, workspace,
+                                       workspace_bytes, stream);
+}
+int chip_mul_mat_f16_batched_second_copy_supported(int64_t ne02, int64_t ne12, int64_t n) {
+    return ne02 > 0 && ne12 > 0 && ne12 % ne02 == 0 && mul_mat_f16_batched_second_copy_supported(ne12 / ne02, n) ? 1 : 0;
+}
+int chip_mul_mat_f16_batched_two_copies(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
+                                        int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y, int64_t ldy1, int64_t ldy2,
+                                        float *y2, int64_t ld2y1, int64_t ld2y2, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!y2) return CHIP_EINVAL;
+    return mul_mat_f16_batched_checked(W, nb01, nb02, K, N, ne02, x, ldx1, ldx2, n, ne12, y, ldy1, ldy2, y2, ld2y1, ld2y2, workspace,
+                                       workspace_bytes, stream);
 }
 
 // ---- attention-side ops ----

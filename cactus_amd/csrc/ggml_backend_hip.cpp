@@ -25,7 +25,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -784,6 +784,34 @@ int grouped_matmuls(const lm_ggml_cgraph *g, int i, int *members) {
     return count;
 }
 
+// The kqv matmul and the node that follows it (views aside) in build_attn_mha, CONT(PERMUTE(kqv, 0, 2, 1, 3)) (reference
+// llama-graph.cpp:1154-1158): with up to 4 (query head, token) pairs per KV head the matmul's kernel also writes the merged
+// layout.  Index of that CONT node, or -1.  The kernel writes both copies while workgroups still read its inputs: the CONT's
+// memory must lie apart from them and from the matmul's own result, whatever the allocator reused.
+int next_compute_node(const lm_ggml_cgraph *g, int i) {
+    for (int j = i + 1; j < g->n_nodes; j++)
+        if (!is_view_op(g->nodes[j]->op)) return j;
+    return -1;
+}
+int head_merge_index(const lm_ggml_cgraph *g, int i) {
+    const lm_ggml_tensor *kqv = g->nodes[i], *v = kqv->src[0], *p = kqv->src[1];
+    const int64_t hd = kqv->ne[0], n = kqv->ne[1], n_head = kqv->ne[2];
+    if (!chip_mul_mat_f16_batched_second_copy_supported(v->ne[2], n_head, n)) return -1;
+    const int j = next_compute_node(g, i);
+    if (j < 0) return -1;
+    const lm_ggml_tensor *ct = g->nodes[j], *pm = ct->src[0];
+    if (ct->op != LM_GGML_OP_CONT || ct->type != LM_GGML_TYPE_F32 || !pm || pm->op != LM_GGML_OP_PERMUTE || pm->src[0] != kqv ||
+        pm->view_src != kqv || pm->view_offs != 0 || !dense(ct) || n_elements(ct) != hd * n_head * n)
+        return -1;
+    // the permuted view: [hd, n_head, n] with kqv's strides of dimensions 0, 2, 1
+    if (pm->ne[0] != hd || pm->ne[1] != n_head || pm->ne[2] != n || pm->ne[3] != 1 || pm->nb[0] != 4 || pm->nb[1] != kqv->nb[2] ||
+        pm->nb[2] != kqv->nb[1])
+        return -1;
+    for (const lm_ggml_tensor *in : {v, p, kqv})
+        if (!ranges_apart(in, ct)) return -1;
+    return j;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
@@ -929,10 +957,29 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             if (w->ne[1] == 0 || x->ne[1] == 0 || x->ne[2] == 0) continue;
             if (!grow_workspace(c, chip_mul_mat_f16_batched_workspace_size(w->ne[0], w->ne[1], w->ne[2], x->ne[2], x->ne[1])))
                 return LM_GGML_STATUS_ALLOC_FAILED;
-            const int rc = chip_mul_mat_f16_batched(w->data, w->nb[1], w->nb[2], w->ne[0], w->ne[1], w->ne[2], (const float *)x->data,
-                                                    (int64_t)(x->nb[1] / 4), (int64_t)(x->nb[2] / 4), x->ne[1], x->ne[2],
-                                                    (float *)node->data, (int64_t)(node->nb[1] / 4), (int64_t)(node->nb[2] / 4),
-                                                    c->workspace, c->workspace_size, c->stream);
+            const int merge = fusion_enabled() ? head_merge_index(cgraph, i) : -1;
+            int rc;
+            if (merge >= 0) {
+                lm_ggml_tensor *ct = cgraph->nodes[merge];
+                writes(ct);
+                // merged[t][h * hd + d] = kqv[h][t][d]
+                rc = chip_mul_mat_f16_batched_two_copies(w->data, w->nb[1], w->nb[2], w->ne[0], w->ne[1], w->ne[2], (const float *)x->data,
+                                                         (int64_t)(x->nb[1] / 4), (int64_t)(x->nb[2] / 4), x->ne[1], x->ne[2],
+                                                         (float *)node->data, (int64_t)(node->nb[1] / 4), (int64_t)(node->nb[2] / 4),
+                                                         (float *)ct->data, node->ne[0] * node->ne[2], node->ne[0], c->workspace,
+                                                         c->workspace_size, c->stream);
+                if (rc == CHIP_OK) {
+                    g_elementwise_nodes++;
+                    g_fused_pairs++;
+                    g_head_merges++;
+                    i = merge;                        // only views lie between the two nodes
+                }
+            } else {
+                rc = chip_mul_mat_f16_batched(w->data, w->nb[1], w->nb[2], w->ne[0], w->ne[1], w->ne[2], (const float *)x->data,
+                                              (int64_t)(x->nb[1] / 4), (int64_t)(x->nb[2] / 4), x->ne[1], x->ne[2],
+                                              (float *)node->data, (int64_t)(node->nb[1] / 4), (int64_t)(node->nb[2] / 4),
+                                              c->workspace, c->workspace_size, c->stream);
+            }
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: batched F16 MUL_MAT %s failed: %s\n", __func__, node->name, chip_error_string(rc));
                 return LM_GGML_STATUS_FAILED;
@@ -1239,5 +1286,6 @@ unsigned long long lm_ggml_backend_hip_get_quantizers_skipped(void) { return g_q
 unsigned long long lm_ggml_backend_hip_get_rope_tables(void) { return g_rope_tables.load(); }
 unsigned long long lm_ggml_backend_hip_get_async_uploaded(void) { return g_uploaded_async.load(); }
 unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void) { return g_grouped_matmuls.load(); }
+unsigned long long lm_ggml_backend_hip_get_head_merges(void) { return g_head_merges.load(); }
 
 }  // extern "C"

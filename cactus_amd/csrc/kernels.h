@@ -232,11 +232,15 @@ hipError_t launch_gemm_kq(int wtype, const void *W, size_t nb01, int64_t K, int6
 // LM_GGML_OP_MUL_MAT with a batched, strided F16 src0 (the attention matmuls over the KV cache):
 // y[b][t][r] = sum_k W[b / r2][r][k] * fp16(x[b][t][k]); strides of W in bytes, of x and y in floats.
 // With a workspace of mul_mat_f16_batched_workspace_size bytes, many columns per KV head go through the fp16 GEMM.
+// y2 (optional): a second copy of the result under its own token and batch strides, for up to 4 (query head, token) pairs per
+// KV head (mul_mat_f16_batched_second_copy_supported): the head merge that follows kqv in the graph.
 bool mul_mat_f16_batched_supported(int64_t K);
+bool mul_mat_f16_batched_second_copy_supported(int64_t r2, int64_t n);
 size_t mul_mat_f16_batched_workspace_size(int64_t K, int64_t N, int64_t ne02, int64_t r2, int64_t n);
 hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02, const float *x,
                                       int64_t ldx1, int64_t ldx2, int64_t n, int64_t r2, float *y, int64_t ldy1, int64_t ldy2,
-                                      void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st);
+                                      void *workspace, size_t workspace_bytes, const DeviceLimits &lim, hipStream_t st,
+                                      float *y2 = nullptr, int64_t ld2y1 = 0, int64_t ld2y2 = 0);
 hipError_t launch_rms_norm(const float *x, int64_t ldx, int64_t n, int64_t ne0, float eps, float *y, int64_t ldy, hipStream_t st);
 hipError_t launch_add(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);
 hipError_t launch_mul(const float *a, int64_t lda, const float *b, int64_t ldb, int64_t ne0, int64_t n, float *y, int64_t ldy, hipStream_t st);

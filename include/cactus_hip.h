@@ -305,6 +305,19 @@ CHIP_API int chip_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
                                       const float *x, int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y,
                                       int64_t ldy1, int64_t ldy2, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The kqv matmul together with the node that follows it in build_attn_mha, cont(permute(kqv, 0, 2, 1, 3)) (reference
+ * llama-graph.cpp:1154-1158: the heads of a token put side by side for the output projection): the same matmul, each value
+ * also stored at y2[b * ld2y2 + t * ld2y1 + r] (for the merge ld2y2 = N, ld2y1 = ne12 * N), which saves the CONT's launch in a
+ * decode step.  Both copies hold the bits of chip_mul_mat_f16_batched.  Taken where that call runs its dot-product kernels
+ * (chip_mul_mat_f16_batched_second_copy_supported returns 1): at most 4 (query head, token) pairs per KV head, i.e.
+ * (ne12 / ne02) * n <= 4; CHIP_EUNSUPPORTED otherwise, nothing written, and the caller runs the two nodes.  y2 must not
+ * overlap W, x or y. */
+CHIP_API int chip_mul_mat_f16_batched_second_copy_supported(int64_t ne02, int64_t ne12, int64_t n);
+CHIP_API int chip_mul_mat_f16_batched_two_copies(const void *W, size_t nb01, size_t nb02, int64_t K, int64_t N, int64_t ne02,
+                                                 const float *x, int64_t ldx1, int64_t ldx2, int64_t n, int64_t ne12, float *y,
+                                                 int64_t ldy1, int64_t ldy2, float *y2, int64_t ld2y1, int64_t ld2y2,
+                                                 void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- the attention-side ops around the KV cache ----
  *   chip_soft_max : LM_GGML_OP_SOFT_MAX (lm_ggml_soft_max_ext), lm_ggml_compute_forward_soft_max_f32 (ggml-cpu/ops.cpp:4731-4827):
  *                   y[r] = softmax(x[r] * scale + mask[r % ne01]) over n_rows rows of ne00 values; mask NULL, or a dense

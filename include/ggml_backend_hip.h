@@ -55,6 +55,9 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_async_uploaded(void);
 /* MUL_MAT nodes that ran in one launch with other projections of the same activation tensor (Qcur / Kcur / Vcur of an
  * attention block, cactus/llama-model.cpp build_llama), up to 4 tokens. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void);
+/* kqv MUL_MAT nodes that also wrote the head merge that follows them, CONT(PERMUTE(kqv)) (cactus/llama-graph.cpp:1154-1158),
+ * up to 4 (query head, token) pairs per KV head. */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_head_merges(void);
 
 #ifdef __cplusplus
 }

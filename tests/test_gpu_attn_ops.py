@@ -293,6 +293,49 @@ def test_attention_matmuls_over_the_cache(dev, orc, hd, n_head, n_head_kv, n_tok
         assert (np.abs(got - want["y"]) <= 1e-5 * want["sum_abs"] + 1e-30).all()
 
 
+# (hd, n_head, n_head_kv, n_tokens, n_kv, kv_size): LLaMA-3-8B's decode step; multi-head attention with 1, 2 and 4 tokens; 3 and 2
+# query heads per KV head; a cache short enough for the short-rows kernel; ragged sizes
+MERGE_SHAPES = [(128, 32, 8, 1, 4096, 4096), (64, 4, 4, 1, 1000, 1024), (64, 4, 4, 4, 520, 1024), (128, 8, 8, 2, 264, 512),
+                (256, 6, 2, 1, 4104, 8192), (96, 4, 2, 2, 72, 128), (128, 2, 1, 1, 5000, 8192), (80, 8, 2, 1, 136, 256)]
+
+
+@pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", MERGE_SHAPES)
+def test_kqv_with_the_head_merge_in_one_launch(dev, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
+    """chip_mul_mat_f16_batched_two_copies: both copies hold the bits of chip_mul_mat_f16_batched, the second one laid out
+    like chip_cpy's CONT of the permuted result (a token's heads side by side)."""
+    _, vt_cache, _, p = attn_case(7 * hd + n_kv, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size)
+    vv = vt_cache[:, :, :n_kv]
+    assert dev.lib.chip_mul_mat_f16_batched_second_copy_supported(n_head_kv, n_head, n_tokens) == 1
+    want = dev.mul_mat_f16_batched(vv, p)
+    got, merged = dev.mul_mat_f16_batched(vv, p, merged=True)
+    assert got.tobytes() == want.tobytes()
+    assert merged.shape == (n_tokens, n_head * hd)
+    assert merged.tobytes() == np.ascontiguousarray(want.transpose(1, 0, 2)).tobytes()
+    assert merged.tobytes() == dev.cpy(want.transpose(1, 0, 2), np.float32).tobytes()
+
+
+def test_kqv_with_the_head_merge_declines_the_other_routes(dev):
+    import cactus_amd as ca
+    L = dev.lib
+    for ne02, ne12, n, ok in ((8, 32, 1, 1), (8, 8, 4, 1), (2, 4, 2, 1), (8, 32, 2, 0), (1, 8, 1, 0), (8, 8, 5, 0), (8, 30, 1, 0), (0, 8, 1, 0)):
+        assert L.chip_mul_mat_f16_batched_second_copy_supported(ne02, ne12, n) == ok
+    d = dev.alloc(1 << 20)
+    ok = [d.ptr, 1024, 1024 * 64, 512, 64, 2, d.ptr, 512, 512, 1, 4, d.ptr + (1 << 19), 64, 64, d.ptr + (1 << 18), 256, 64, None, 0, None]
+    assert L.chip_mul_mat_f16_batched_two_copies(*ok) == ca.CHIP_OK
+
+    def call(**kw):
+        a = list(ok)
+        for k, v in kw.items():
+            a[int(k[1:])] = v
+        return L.chip_mul_mat_f16_batched_two_copies(*a)
+    assert call(_14=None) == ca.CHIP_EINVAL                                      # no second destination
+    assert call(_10=16) == ca.CHIP_EUNSUPPORTED                                  # 8 query heads per KV head: the matrix-core kernels
+    assert call(_9=3) == ca.CHIP_EUNSUPPORTED                                    # 3 tokens x 2 heads
+    assert call(_14=d.ptr + (1 << 18) + 2) == ca.CHIP_EINVAL
+    assert call(_15=-1) == ca.CHIP_EINVAL
+    dev.sync()
+
+
 def test_attention_matmul_exact_small_integers(dev):
     # halves and activations that are small integers: every product and partial sum is exact in fp32, so any summation
     # order gives the same bits, and a wrong index or a dropped term shows

@@ -927,6 +927,89 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     L.lm_ggml_free(wctx)
 
 
+# (hd, n_head, n_head_kv, n_tokens, n_kv, kv_size): LLaMA-3-8B's block, one token; multi-head attention with 1 and 4 tokens; 8 query
+# heads per KV head and two tokens of LLaMA-3-8B, where the matmul takes kernels without the second copy and the CONT runs alone
+@pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", [(128, 32, 8, 1, 512, 1024), (128, 32, 8, 1, 4096, 4096),
+                                                                      (64, 4, 4, 1, 1000, 1024), (64, 4, 4, 4, 136, 256),
+                                                                      (128, 16, 2, 1, 512, 512), (128, 32, 8, 2, 520, 1024)])
+def test_kqv_writes_the_head_merge_that_follows_it(host, hd, n_head, n_head_kv, n_tokens, n_kv, kv_size):
+    """kq -> soft-max -> kqv -> merge (reference llama-graph.cpp:1120-1160) through the scheduler: with up to 4 (query head, token)
+    pairs per KV head the CONT runs inside the kqv matmul's launch, and the merged rows have the bits of the four ops called
+    one by one through the C-ABI."""
+    import cactus_amd
+    L = host.L
+    n_embd_kv = hd * n_head_kv
+    rng = np.random.default_rng(hd + n_kv)
+    kc0 = np.zeros((kv_size, n_embd_kv), np.float16)
+    kc0[:n_kv] = rng.standard_normal((n_kv, n_embd_kv)).astype(np.float16)
+    vc0 = np.zeros((n_embd_kv, kv_size), np.float16)
+    vc0[:, :n_kv] = rng.standard_normal((n_embd_kv, n_kv)).astype(np.float16)
+    q0 = rng.standard_normal((n_tokens, n_head, hd)).astype(np.float32)
+    mask = np.zeros((8, n_kv), np.float32)
+    mask[:n_tokens][rng.random((n_tokens, n_kv)) < 0.25] = -np.inf
+    mask[:, 0] = 0.0
+    mask16 = mask.astype(np.float16)
+    scale = float(1.0 / np.sqrt(hd))
+
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    cpu = L.lm_ggml_backend_cpu_init()
+    cctx = host.context(with_graph=False)
+    kc = host.tensor_2d(cctx, O.F16, n_embd_kv, kv_size, "cache_k")
+    vc = host.tensor_2d(cctx, O.F16, n_embd_kv, kv_size, "cache_v")
+    cbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(cctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    host.set(kc, kc0)
+    host.set(vc, vc0)
+    ctx = host.context(n_tensors=64)
+    tq = host.tensor_3d(ctx, O.F32, hd, n_head, n_tokens, "q")
+    tmask = host.tensor_2d(ctx, O.F16, n_kv, 8, "mask")
+    for t in (tq, tmask):
+        L.lm_ggml_set_input(t)
+    kview = L.lm_ggml_view_3d(ctx, kc, hd, n_head_kv, n_kv, 2 * hd, 2 * n_embd_kv, 0)
+    vview = L.lm_ggml_view_3d(ctx, vc, n_kv, n_head_kv, hd, 2 * kv_size * hd, 2 * kv_size, 0)
+    qp = L.lm_ggml_permute(ctx, tq, 0, 2, 1, 3)
+    kp = L.lm_ggml_permute(ctx, kview, 0, 2, 1, 3)
+    vp = L.lm_ggml_permute(ctx, vview, 0, 2, 1, 3)
+    kq = L.lm_ggml_mul_mat(ctx, kp, qp)
+    sm = L.lm_ggml_soft_max_ext(ctx, kq, tmask, scale, 0.0)
+    kqv = L.lm_ggml_mul_mat(ctx, vp, sm)
+    merged = L.lm_ggml_cont_2d(ctx, L.lm_ggml_permute(ctx, kqv, 0, 2, 1, 3), hd * n_head, n_tokens)
+    # outputs keep their memory to the end: the allocator cannot place the merged rows over the probabilities, which the matmul's
+    # workgroups still read while others already store (the backend checks for that and runs the CONT alone then)
+    for t in (merged, kqv, sm):
+        L.lm_ggml_set_output(t)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, merged)
+    backends = (C.c_void_p * 2)(hip, cpu)
+    sched = L.lm_ggml_backend_sched_new(backends, None, 2, 128, False, True)
+    assert L.lm_ggml_backend_sched_alloc_graph(sched, g)
+    host.set(tq, q0); host.set(tmask, mask16)
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    blib.lm_ggml_backend_hip_get_head_merges.restype = C.c_ulonglong
+    before = blib.lm_ggml_backend_hip_get_head_merges()
+    assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
+    taken = (n_head // n_head_kv) * n_tokens <= 4
+    assert blib.lm_ggml_backend_hip_get_head_merges() - before == (1 if taken else 0)
+    assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
+    y = host.get(merged, np.float32, (n_tokens, n_head, hd))
+    y_kqv = host.get(kqv, np.float32, (n_head, n_tokens, hd))
+
+    d = cactus_amd.Device(0)
+    kv = kc0[:n_kv].reshape(n_kv, n_head_kv, hd).transpose(1, 0, 2)
+    vv = vc0.reshape(n_head_kv, hd, kv_size)[:, :, :n_kv]
+    kq_ = d.mul_mat_f16_batched(kv, q0.transpose(1, 0, 2))
+    sm_ = d.soft_max(kq_, mask16, scale)
+    kqv_ = d.mul_mat_f16_batched(vv, sm_)
+    assert y_kqv.tobytes() == kqv_.tobytes()
+    assert y.tobytes() == np.ascontiguousarray(kqv_.transpose(1, 0, 2)).tobytes()
+    L.lm_ggml_backend_sched_free(sched)
+    L.lm_ggml_backend_buffer_free(cbuf)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_backend_free(cpu)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(cctx)
+
+
 def test_get_rows_from_a_device_resident_table(host, orc):
     """LM_GGML_OP_GET_ROWS over a quantized table in a HIP buffer (an embedding matrix kept on the device) runs on the HIP
     backend, bit for bit the reference's dequantized rows; a table in host memory is declined."""
