@@ -14,6 +14,7 @@
 #include "../../include/ggml_abi_mirror.h"
 #include "../../include/ggml_backend_hip.h"
 
+#include <algorithm>
 #include <atomic>
 #include <dlfcn.h>
 #include <cstdio>
@@ -21,6 +22,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <vector>
 
 namespace {
 
@@ -54,6 +56,7 @@ struct backend_ctx {
     rope_table_key rope_key = {};
     quantized_key quantized = {};
     uint16_t *gelu_table = nullptr;                  // device copy of the 65536-entry fp16 GELU table
+    float *group_scratch = nullptr; size_t group_slot_bytes = 0;     // CHIP_GROUP_MAX result slots for projections run early
 };
 
 lm_ggml_backend_buffer_type_t hip_buffer_type();
@@ -202,6 +205,7 @@ void backend_free(lm_ggml_backend_t backend) {
     chip_free(c->workspace);
     chip_free(c->rope_table);
     chip_free(c->gelu_table);
+    chip_free(c->group_scratch);
     chip_stream_destroy(c->stream);
     delete c;
     delete backend;
@@ -442,7 +446,8 @@ bool attn_side_shape_ok(const lm_ggml_tensor *op) {
     }
 }
 // store: the F32 -> F16 CPY of the RoPE's result into a dense destination (the K cache store), run in the RoPE's kernel
-int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *store = nullptr) {
+// src_at: where the ROPE's input really lies (a projection that ran early, into the backend's own memory)
+int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *store = nullptr, const void *src_at = nullptr) {
     const lm_ggml_tensor *a = op->src[0];
     switch (op->op) {
         case LM_GGML_OP_SOFT_MAX: {
@@ -455,6 +460,7 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *stor
         }
         case LM_GGML_OP_ROPE: {
             const lm_ggml_tensor *pos = op->src[1], *ff = op->src[2];
+            const float *xa = (const float *)(src_at ? src_at : a->data);
             float f[6];
             std::memcpy(f, op->op_params + 5, sizeof(f));        // freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow
             if (fusion_enabled()) {
@@ -484,15 +490,15 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *stor
                     g_rope_tables++;
                 }
                 if (store)
-                    return chip_rope_apply_store((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table,
+                    return chip_rope_apply_store(xa, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table,
                                                  a->ne[0], a->ne[1], a->ne[2], op->op_params[1], op->op_params[2], (float *)op->data,
                                                  (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), (uint16_t *)store->data, a->ne[0],
                                                  a->ne[0] * a->ne[1], c->stream);
-                return chip_rope_apply((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table, a->ne[0],
+                return chip_rope_apply(xa, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table, a->ne[0],
                                        a->ne[1], a->ne[2], op->op_params[1], op->op_params[2], (float *)op->data,
                                        (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), c->stream);
             }
-            return chip_rope((const float *)a->data, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), (const int32_t *)pos->data,
+            return chip_rope(xa, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), (const int32_t *)pos->data,
                              ff ? (const float *)ff->data : nullptr, a->ne[0], a->ne[1], a->ne[2], op->op_params[1], op->op_params[2],
                              op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], (float *)op->data, (int64_t)(op->nb[1] / 4),
                              (int64_t)(op->nb[2] / 4), c->stream);
@@ -761,17 +767,21 @@ int transposed_store_index(const lm_ggml_cgraph *g, int i, int run_at = -1) {
 // two reads or writes the memory of its result (the allocator may have given it the place of a tensor that dies in
 // between, Qcur's for instance once its RoPE has read it).  Fills members[] (node i first) and returns their number.
 constexpr int GROUP_LOOKAHEAD = 12;
-int grouped_matmuls(const lm_ggml_cgraph *g, int i, int *members) {
+// aliased[k]: member k's own memory is in use between node i and its node (the allocator gave it the place of a tensor that
+// dies in between: Kcur over Qcur, once Qcur's RoPE has read it and written elsewhere).  Such a member can still run at
+// node i when its result goes to memory of the backend's own; what happens to it then is the caller's business.
+int grouped_matmuls(const lm_ggml_cgraph *g, int i, int *members, bool *aliased) {
     const lm_ggml_tensor *first = g->nodes[i], *x = first->src[1];
     const int vt = chip_vec_dot_type(first->src[0]->type);
     int count = 0;
+    aliased[count] = false;
     members[count++] = i;
     const int end = i + 1 + GROUP_LOOKAHEAD < g->n_nodes ? i + 1 + GROUP_LOOKAHEAD : g->n_nodes;
     for (int j = i + 1; j < end && count < CHIP_GROUP_MAX; j++) {
         const lm_ggml_tensor *mm = g->nodes[j];
         if (mm->op != LM_GGML_OP_MUL_MAT || mm->src[1] != x || !mul_mat_shape_ok(mm)) continue;
-        if (chip_vec_dot_type(mm->src[0]->type) != vt || !disjoint(mm, x)) continue;
-        bool safe = true;
+        if (chip_vec_dot_type(mm->src[0]->type) != vt) continue;
+        bool safe = disjoint(mm, x);
         for (int m = i; m < j && safe; m++) {
             const lm_ggml_tensor *t = g->nodes[m];
             if (is_view_op(t->op)) continue;
@@ -779,9 +789,46 @@ int grouped_matmuls(const lm_ggml_cgraph *g, int i, int *members) {
             for (int k = 0; k < LM_GGML_MAX_SRC && safe; k++)
                 if (t->src[k] && !ranges_apart(t->src[k], mm)) safe = false;
         }
-        if (safe) members[count++] = j;
+        aliased[count] = !safe;
+        members[count++] = j;
     }
     return count;
+}
+
+// The tensors the graph's nodes read, views resolved to the tensor that owns the memory: built once per graph_compute,
+// when the first question about a tensor's readers comes up.
+struct graph_reads {
+    std::vector<const lm_ggml_tensor *> owner;       // one entry per (computing node, operand)
+    bool built = false;
+    void build(const lm_ggml_cgraph *g) {
+        owner.clear();
+        for (int k = 0; k < g->n_nodes; k++) {
+            const lm_ggml_tensor *nd = g->nodes[k];
+            if (is_view_op(nd->op)) continue;
+            for (int m = 0; m < LM_GGML_MAX_SRC; m++)
+                if (const lm_ggml_tensor *sr = nd->src[m]) owner.push_back(sr->view_src ? sr->view_src : sr);
+        }
+        built = true;
+    }
+    int readers_of(const lm_ggml_cgraph *g, const lm_ggml_tensor *t) {
+        if (!built) build(g);
+        int n = 0;
+        for (const lm_ggml_tensor *o : owner) n += o == t;
+        return n;
+    }
+};
+bool grow_group_scratch(backend_ctx *c, size_t slot_bytes) {
+    if (slot_bytes <= c->group_slot_bytes) return true;
+    chip_stream_synchronize(c->stream);                  // earlier nodes of this call may still use the old slots
+    chip_free(c->group_scratch);
+    c->group_scratch = nullptr;
+    c->group_slot_bytes = 0;
+    void *p = nullptr;
+    const size_t want = (slot_bytes + slot_bytes / 2 + 255) & ~(size_t)255;
+    if (chip_malloc(&p, want * CHIP_GROUP_MAX) != CHIP_OK) return false;
+    c->group_scratch = (float *)p;
+    c->group_slot_bytes = want;
+    return true;
 }
 
 // The kqv matmul and the node that follows it (views aside) in build_attn_mha, CONT(PERMUTE(kqv, 0, 2, 1, 3)) (reference
@@ -825,6 +872,10 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     };
     int paired_matmul = -1;                           // index of an up projection that ran with its gate projection
     int grouped[CHIP_GROUP_MAX] = {-1, -1, -1, -1};   // projections that already ran with an earlier one of the same input
+    const float *grouped_copy[CHIP_GROUP_MAX] = {nullptr, nullptr, nullptr, nullptr};   // ... into a scratch slot, still to be copied to their place
+    int rope_from_slot = -1;                          // a ROPE node whose input lies in a scratch slot instead
+    const float *rope_slot_src = nullptr;
+    graph_reads reads;
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -928,7 +979,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                     g_fused_pairs++;
                 }
             }
-            const int rc = run_attn_side(c, node, store);
+            const int rc = run_attn_side(c, node, store, i == rope_from_slot ? rope_slot_src : nullptr);
+            if (i == rope_from_slot) rope_from_slot = -1;
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
                 return LM_GGML_STATUS_FAILED;
@@ -993,8 +1045,22 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         }
         {
             bool done = false;
-            for (int &slot : grouped)
-                if (slot == i) { slot = -1; done = true; }
+            for (int k = 0; k < CHIP_GROUP_MAX; k++) {
+                if (grouped[k] != i) continue;
+                grouped[k] = -1;
+                done = true;
+                if (const float *from = grouped_copy[k]) {          // ran into a scratch slot: its own memory is free to take it now
+                    grouped_copy[k] = nullptr;
+                    const int64_t N = node->ne[0], n = node->ne[1];
+                    const int64_t ne[4] = {N, n, 1, 1}, nbs[4] = {4, N * 4, N * n * 4, N * n * 4};
+                    const int64_t nbd[4] = {4, (int64_t)node->nb[1], (int64_t)node->nb[1] * n, (int64_t)node->nb[1] * n};
+                    const int rc = chip_cpy(from, LM_GGML_TYPE_F32, ne, nbs, node->data, LM_GGML_TYPE_F32, ne, nbd, c->stream);
+                    if (rc != CHIP_OK) {
+                        HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: copy of the early result of %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+                        return LM_GGML_STATUS_FAILED;
+                    }
+                }
+            }
             if (done) continue;
         }
         const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
@@ -1005,23 +1071,33 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         const int64_t ldx = (int64_t)(x->nb[1] / 4);
         int store_t = -1;
         int members[CHIP_GROUP_MAX];
+        bool aliased[CHIP_GROUP_MAX] = {false, false, false, false};
         int n_members = 1;
         if ((n <= 4 || n == 8) && fusion_enabled()) {      // the token counts chip_mul_mat_group has a one-launch form for
             bool slots_free = true;
             for (int slot : grouped) slots_free = slots_free && slot < 0;
             // A SILU held back for its MUL reads the gate projection's result only when that MUL runs, after this node:
             // a later projection run here could be sitting in memory the allocator freed from under it, so no group then.
-            if (slots_free && !waiting_silu) n_members = grouped_matmuls(cgraph, i, members);
+            if (slots_free && !waiting_silu && rope_from_slot < 0) n_members = grouped_matmuls(cgraph, i, members, aliased);
         }
         if (n_members >= 2) {
             chip_mat mats[CHIP_GROUP_MAX];
             bool fits = true;
             int stores = 0;
             for (int k = 0; k < n_members; k++) fits = fits && cgraph->nodes[members[k]]->src[0]->ne[1] > 0;
+            size_t slot_bytes = 0;
+            for (int k = 1; k < n_members; k++)
+                if (aliased[k]) slot_bytes = std::max(slot_bytes, (size_t)(cgraph->nodes[members[k]]->ne[0] * n) * sizeof(float));
+            if (fits && slot_bytes > 0 && !grow_group_scratch(c, slot_bytes)) return LM_GGML_STATUS_ALLOC_FAILED;
+            bool stored[CHIP_GROUP_MAX] = {false, false, false, false};
             for (int k = 0; fits && k < n_members; k++) {
                 lm_ggml_tensor *mm = cgraph->nodes[members[k]];
                 const lm_ggml_tensor *mw = mm->src[0];
                 mats[k] = chip_mat{(int)mw->type, mw->data, mw->nb[1], mw->ne[1], (float *)mm->data, (int64_t)(mm->nb[1] / 4), nullptr, 0};
+                if (aliased[k]) {                      // its own memory is still in use: into the backend's slot k, rows side by side
+                    mats[k].y = (float *)((uint8_t *)c->group_scratch + (size_t)k * c->group_slot_bytes);
+                    mats[k].ldy = mw->ne[1];
+                }
                 if (!grow_workspace(c, chip_mul_mat_workspace_size_n(mw->type, K, mw->ne[1], n))) return LM_GGML_STATUS_ALLOC_FAILED;
                 const int st = transposed_store_index(cgraph, members[k], i);
                 if (st >= 0 && remember_store(st)) {
@@ -1030,12 +1106,32 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                     mats[k].y_f16_t = (uint16_t *)cp->data;
                     mats[k].ld16 = (int64_t)(cp->nb[1] / 2);
                     stores++;
+                    stored[k] = true;
                 }
             }
             if (fits) {
                 for (int k = 1; k < n_members; k++) {
-                    writes(cgraph->nodes[members[k]]);
+                    lm_ggml_tensor *mm = cgraph->nodes[members[k]];
+                    writes(mm);
                     grouped[k] = members[k];
+                    grouped_copy[k] = nullptr;
+                    if (!aliased[k]) continue;
+                    // What becomes of a result in a scratch slot.  Its only reader was the cache store that ran with it: nothing.
+                    // Its only reader is the ROPE that follows it (views aside) and takes its rows as they lie: that ROPE reads
+                    // the slot.  Otherwise it is copied to its own memory when the loop gets to its node.
+                    const int readers = reads.readers_of(cgraph, mm);
+                    const int nx = next_compute_node(cgraph, members[k]);
+                    const lm_ggml_tensor *rp = nx >= 0 ? cgraph->nodes[nx] : nullptr;
+                    const bool kept = (mm->flags & LM_GGML_TENSOR_FLAG_OUTPUT) != 0;     // the caller reads it afterwards
+                    if (!kept && readers == 1 && stored[k]) continue;
+                    if (!kept && readers == 1 && rope_from_slot < 0 && rp && rp->op == LM_GGML_OP_ROPE && rp->src[0] && attn_side_shape_ok(rp) &&
+                        (rp->src[0] == mm || rp->src[0]->view_src == mm) && rp->src[0]->data == mm->data && fusion_enabled() &&
+                        mm->nb[1] == (size_t)mm->ne[0] * sizeof(float)) {
+                        rope_from_slot = nx;
+                        rope_slot_src = mats[k].y;
+                        continue;
+                    }
+                    grouped_copy[k] = mats[k].y;
                 }
                 // more than 4 tokens: the workspace holds x's quantized rows afterwards, or already does (the norm in front
                 // left them there, or an earlier matmul of the same input)

@@ -44,6 +44,7 @@ enum {
     LM_GGML_OP_COUNT = 82,
 };
 enum { LM_GGML_UNARY_OP_GELU = 8, LM_GGML_UNARY_OP_SILU = 10 };
+enum { LM_GGML_TENSOR_FLAG_INPUT = 1, LM_GGML_TENSOR_FLAG_OUTPUT = 2 };      /* enum lm_ggml_tensor_flag (ggml.h:560-563) */
 enum { LM_GGML_STATUS_ALLOC_FAILED = -2, LM_GGML_STATUS_FAILED = -1, LM_GGML_STATUS_SUCCESS = 0, LM_GGML_STATUS_ABORTED = 1 };
 enum { LM_GGML_BACKEND_DEVICE_TYPE_CPU = 0, LM_GGML_BACKEND_DEVICE_TYPE_GPU = 1, LM_GGML_BACKEND_DEVICE_TYPE_ACCEL = 2 };
 enum { LM_GGML_BACKEND_BUFFER_USAGE_ANY = 0, LM_GGML_BACKEND_BUFFER_USAGE_WEIGHTS = 1, LM_GGML_BACKEND_BUFFER_USAGE_COMPUTE = 2 };

@@ -28,6 +28,8 @@ namespace mirror {
 #define LM_GGML_OP_MUL_MAT M_OP_MUL_MAT
 #define LM_GGML_UNARY_OP_SILU M_UNARY_OP_SILU
 #define LM_GGML_UNARY_OP_GELU M_UNARY_OP_GELU
+#define LM_GGML_TENSOR_FLAG_INPUT M_TENSOR_FLAG_INPUT
+#define LM_GGML_TENSOR_FLAG_OUTPUT M_TENSOR_FLAG_OUTPUT
 #define LM_GGML_OP_SCALE M_OP_SCALE
 #define LM_GGML_OP_UNARY M_OP_UNARY
 #define LM_GGML_OP_RMS_NORM M_OP_RMS_NORM
@@ -76,6 +78,8 @@ constexpr int k_max_dims = LM_GGML_MAX_DIMS, k_max_src = LM_GGML_MAX_SRC, k_max_
 #undef LM_GGML_OP_MUL_MAT
 #undef LM_GGML_UNARY_OP_SILU
 #undef LM_GGML_UNARY_OP_GELU
+#undef LM_GGML_TENSOR_FLAG_INPUT
+#undef LM_GGML_TENSOR_FLAG_OUTPUT
 #undef LM_GGML_OP_SCALE
 #undef LM_GGML_OP_UNARY
 #undef LM_GGML_OP_RMS_NORM
@@ -154,6 +158,7 @@ static_assert(mirror::M_OP_NONE == LM_GGML_OP_NONE && mirror::M_OP_MUL_MAT == LM
               mirror::M_OP_UNARY == LM_GGML_OP_UNARY && mirror::M_UNARY_OP_SILU == LM_GGML_UNARY_OP_SILU &&
               mirror::M_OP_DUP == LM_GGML_OP_DUP && mirror::M_OP_GET_ROWS == LM_GGML_OP_GET_ROWS && mirror::M_OP_CPY == LM_GGML_OP_CPY && mirror::M_OP_CONT == LM_GGML_OP_CONT && mirror::M_OP_SOFT_MAX == LM_GGML_OP_SOFT_MAX && mirror::M_OP_ROPE == LM_GGML_OP_ROPE &&
               mirror::M_OP_SCALE == LM_GGML_OP_SCALE && mirror::M_UNARY_OP_GELU == LM_GGML_UNARY_OP_GELU, "op ids");
+static_assert(mirror::M_TENSOR_FLAG_INPUT == LM_GGML_TENSOR_FLAG_INPUT && mirror::M_TENSOR_FLAG_OUTPUT == LM_GGML_TENSOR_FLAG_OUTPUT, "tensor flags");
 static_assert(mirror::M_STATUS_ALLOC_FAILED == LM_GGML_STATUS_ALLOC_FAILED && mirror::M_STATUS_FAILED == LM_GGML_STATUS_FAILED &&
               mirror::M_STATUS_SUCCESS == LM_GGML_STATUS_SUCCESS && mirror::M_STATUS_ABORTED == LM_GGML_STATUS_ABORTED, "status");
 static_assert(mirror::M_DEV_CPU == LM_GGML_BACKEND_DEVICE_TYPE_CPU && mirror::M_DEV_GPU == LM_GGML_BACKEND_DEVICE_TYPE_GPU &&
