@@ -731,10 +731,10 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
             ck(L.chip_mul_mat_group(arr, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
             if l == 0:                                                # one cos / sin table per step, as the backend keeps it
                 ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
-            ck(L.chip_rope_apply(q.ptr, hd, hd * n_head, rope_tab.ptr, hd, n_head, n, hd, 2, q.ptr, hd, hd * n_head, st))
-            # K: RoPE and the store into the F16 cache in one launch, as the backend runs the two nodes
-            ck(L.chip_rope_apply_store(k.ptr, hd, KV, rope_tab.ptr, hd, n_head_kv, n, hd, 2, k.ptr, hd, KV,
-                                       kc + 2 * KV * (n_kv - n), hd, KV, st))
+            # RoPE of Q and of K in one launch; K's also stores into the F16 cache, as the backend runs the three nodes
+            ra = ca.RopeOperand(q.ptr, hd, hd * n_head, n_head, q.ptr, hd, hd * n_head, None, 0, 0)
+            rb = ca.RopeOperand(k.ptr, hd, KV, n_head_kv, k.ptr, hd, KV, kc + 2 * KV * (n_kv - n), hd, KV)
+            ck(L.chip_rope_apply_two(C.byref(ra), C.byref(rb), rope_tab.ptr, hd, n, hd, 2, st))
             if n > 4:
                 shp = A4(n, KV, 1, 1)
                 ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))

@@ -37,7 +37,7 @@ EXPORTS = (
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
     "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
-    "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
+    "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_rope_apply_two", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
     "chip_workspace_to_blocks",
 )
@@ -53,6 +53,12 @@ class Mat(C.Structure):
     """struct chip_mat: one member of chip_mul_mat_group."""
     _fields_ = [("type", C.c_int), ("W", C.c_void_p), ("nb01", C.c_size_t), ("N", C.c_int64), ("y", C.c_void_p),
                 ("ldy", C.c_int64), ("y_f16_t", C.c_void_p), ("ld16", C.c_int64)]
+
+
+class RopeOperand(C.Structure):
+    """struct chip_rope_operand: one of the two tensors of chip_rope_apply_two."""
+    _fields_ = [("x", C.c_void_p), ("ldx1", C.c_int64), ("ldx2", C.c_int64), ("ne1", C.c_int64), ("y", C.c_void_p),
+                ("ldy1", C.c_int64), ("ldy2", C.c_int64), ("y_f16", C.c_void_p), ("ld16_1", C.c_int64), ("ld16_2", C.c_int64)]
 
 
 class ChipError(RuntimeError):
@@ -135,6 +141,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_rope_table.argtypes = [vp, vp, i64, i32, i32] + [C.c_float] * 6 + [vp, vp]
     L.chip_rope_apply.argtypes = [vp, i64, i64, vp, i64, i64, i64, i32, i32, vp, i64, i64, vp]
     L.chip_rope_apply_store.argtypes = [vp, i64, i64, vp, i64, i64, i64, i32, i32, vp, i64, i64, vp, i64, i64, vp]
+    L.chip_rope_apply_two.argtypes = [C.POINTER(RopeOperand), C.POINTER(RopeOperand), vp, i64, i64, i32, i32, vp]
     L.chip_get_rows.argtypes = [i32, vp, sz, sz, sz, i64, i64, vp, i64, i64, i64, i64, i64, vp, i64, i64, i64, vp]
     L.chip_mul_mat_f16_batched.argtypes = [vp, sz, sz, i64, i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_f16_batched_workspace_size.restype = sz
@@ -435,6 +442,39 @@ class Device:
                                           dy.ptr, ne0, ne0 * ne1, None))
         self.sync()
         return dy.download(np.float32, x.size).reshape(x.shape)
+
+    def rope_two(self, xa, xb, pos, n_dims, mode, want=(("f32",), ("f32", "f16")), freq_factors=None, n_ctx_orig=4096,
+                 freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0, beta_fast=32.0, beta_slow=1.0):
+        """chip_rope_table + chip_rope_apply_two: xa fp32 [n_tokens, heads_a, ne0], xb fp32 [n_tokens, heads_b, ne0] rotated in one
+        launch; want names the outputs of each ("f32", "f16").  Returns ({"f32": .., "f16": ..}, {..}); outputs not asked
+        for are absent."""
+        xs = [np.ascontiguousarray(xa, np.float32), np.ascontiguousarray(xb, np.float32)]
+        ne2, _, ne0 = xs[0].shape
+        dp = self.to_device(np.ascontiguousarray(pos, np.int32))
+        df = self.to_device(np.ascontiguousarray(freq_factors, np.float32)) if freq_factors is not None else None
+        dt = self.alloc(ne2 * n_dims * 4)
+        self.check(self.lib.chip_rope_table(dp.ptr, df.ptr if df else None, ne2, n_dims, n_ctx_orig, freq_base, freq_scale,
+                                            ext_factor, attn_factor, beta_fast, beta_slow, dt.ptr, None))
+        ops, bufs = [], []
+        for x, w in zip(xs, want):
+            ne1 = x.shape[1]
+            dx = self.to_device(x)
+            dy = self.alloc(x.nbytes) if "f32" in w else None
+            dh = self.alloc(x.size * 2) if "f16" in w else None
+            bufs.append((dx, dy, dh))
+            ops.append(RopeOperand(dx.ptr, ne0, ne0 * ne1, ne1, dy.ptr if dy else None, ne0, ne0 * ne1, dh.ptr if dh else None, ne0,
+                                   ne0 * ne1))
+        self.check(self.lib.chip_rope_apply_two(C.byref(ops[0]), C.byref(ops[1]), dt.ptr, ne0, ne2, n_dims, mode, None))
+        self.sync()
+        out = []
+        for x, (dx, dy, dh) in zip(xs, bufs):
+            r = {}
+            if dy:
+                r["f32"] = dy.download(np.float32, x.size).reshape(x.shape)
+            if dh:
+                r["f16"] = dh.download(np.float16, x.size).reshape(x.shape)
+            out.append(r)
+        return tuple(out)
 
     def get_rows(self, t, table, nc, ids):
         """table uint8 [ne01, row_size(t, nc)] (or float32 / float16 [ne01, nc] for F32 / F16), ids int32 [n] -> fp32 [n, nc];

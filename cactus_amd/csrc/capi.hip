@@ -967,6 +967,29 @@ int chip_rope_apply_store(const float *x, int64_t ldx1, int64_t ldx2, const floa
     return rope_apply_checked(x, ldx1, ldx2, table, ne0, ne1, ne2, n_dims, mode, y, ldy1, ldy2, y_f16, ld16_1, ld16_2, stream);
 }
 
+static int rope_operand_checked(const chip_rope_operand *o, int64_t ne0, int64_t ne2, int n_dims, int mode, RopeArgs &a) {
+    if (!o) return CHIP_EINVAL;
+    if (int rc = rope_dims_checked(ne0, o->ne1, ne2, n_dims, mode); rc != CHIP_OK) return rc;
+    if (ne0 <= 0 || o->ne1 <= 0 || ne2 <= 0 || ne2 > 0x7fffffff) return CHIP_EINVAL;
+    if (!o->x || (!o->y && !o->y_f16) || o->ldx1 < ne0 || (o->y && o->ldy1 < ne0)) return CHIP_EINVAL;
+    if ((((uintptr_t)o->x) | ((uintptr_t)o->y)) & 3) return CHIP_EINVAL;
+    if (o->y_f16 && (o->ld16_1 < ne0 || (((uintptr_t)o->y_f16) & 1) != 0)) return CHIP_EINVAL;
+    a.ne0 = ne0; a.ne1 = o->ne1; a.ne2 = ne2;
+    a.ldx1 = o->ldx1; a.ldx2 = o->ldx2; a.ldy1 = o->y ? o->ldy1 : 0; a.ldy2 = o->y ? o->ldy2 : 0;
+    a.n_dims = n_dims; a.neox = (mode & 2) != 0;
+    a.theta_scale = a.freq_scale = a.ext_factor = a.corr0 = a.corr1 = a.mscale = 0.0f;       // all in the table
+    a.y16 = o->y_f16; a.ld16_1 = o->y_f16 ? o->ld16_1 : 0; a.ld16_2 = o->y_f16 ? o->ld16_2 : 0;
+    return CHIP_OK;
+}
+int chip_rope_apply_two(const chip_rope_operand *a, const chip_rope_operand *b, const float *table, int64_t ne0, int64_t ne2,
+                        int n_dims, int mode, void *stream) {
+    RopeArgs ra, rb;
+    if (int rc = rope_operand_checked(a, ne0, ne2, n_dims, mode, ra); rc != CHIP_OK) return rc;
+    if (int rc = rope_operand_checked(b, ne0, ne2, n_dims, mode, rb); rc != CHIP_OK) return rc;
+    if (!table || (((uintptr_t)table) & 3)) return CHIP_EINVAL;
+    return hip_rc(launch_rope_apply_two(a->x, ra, a->y, b->x, rb, b->y, table, (hipStream_t)stream));
+}
+
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                      int32_t *isum, int32_t *imin, void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;

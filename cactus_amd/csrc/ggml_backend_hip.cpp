@@ -27,7 +27,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -446,8 +446,18 @@ bool attn_side_shape_ok(const lm_ggml_tensor *op) {
     }
 }
 // store: the F32 -> F16 CPY of the RoPE's result into a dense destination (the K cache store), run in the RoPE's kernel
+// A second ROPE node run in the first one's launch (K's with Q's): its input, the CPY of its result into the F16 cache that
+// runs with it (or null), and whether its own F32 result is written at all.
+struct rope_partner {
+    const lm_ggml_tensor *op = nullptr;
+    const void *src = nullptr;
+    const lm_ggml_tensor *store = nullptr;
+    int store_index = -1;
+    bool write_f32 = true;
+};
 // src_at: where the ROPE's input really lies (a projection that ran early, into the backend's own memory)
-int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *store = nullptr, const void *src_at = nullptr) {
+int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *store = nullptr, const void *src_at = nullptr,
+                  const rope_partner *partner = nullptr) {
     const lm_ggml_tensor *a = op->src[0];
     switch (op->op) {
         case LM_GGML_OP_SOFT_MAX: {
@@ -488,6 +498,17 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *stor
                     if (rc != CHIP_OK) return rc;
                     c->rope_key = k;
                     g_rope_tables++;
+                }
+                if (partner) {
+                    const lm_ggml_tensor *pb = partner->op, *ab = pb->src[0];
+                    chip_rope_operand oa = {xa, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), a->ne[1], (float *)op->data,
+                                            (int64_t)(op->nb[1] / 4), (int64_t)(op->nb[2] / 4), store ? (uint16_t *)store->data : nullptr,
+                                            a->ne[0], a->ne[0] * a->ne[1]};
+                    chip_rope_operand ob = {(const float *)partner->src, (int64_t)(ab->nb[1] / 4), (int64_t)(ab->nb[2] / 4), ab->ne[1],
+                                            partner->write_f32 ? (float *)pb->data : nullptr, (int64_t)(pb->nb[1] / 4),
+                                            (int64_t)(pb->nb[2] / 4), partner->store ? (uint16_t *)partner->store->data : nullptr,
+                                            ab->ne[0], ab->ne[0] * ab->ne[1]};
+                    return chip_rope_apply_two(&oa, &ob, c->rope_table, a->ne[0], a->ne[2], op->op_params[1], op->op_params[2], c->stream);
                 }
                 if (store)
                     return chip_rope_apply_store(xa, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), c->rope_table,
@@ -716,13 +737,13 @@ int early_store_index(const lm_ggml_cgraph *g, int i, F wanted, int run_at = -1)
 
 // The RoPE of K and the CPY of its result into the F16 cache (reference llama-kv-cache.cpp cpy_k: a dense 1-D view of the
 // cache): index of that CPY node, or -1.  The RoPE still writes its own F32 result.
-int rope_store_index(const lm_ggml_cgraph *g, int i) {
+int rope_store_index(const lm_ggml_cgraph *g, int i, int run_at = -1) {
     const lm_ggml_tensor *rope = g->nodes[i];
     if (rope->type != LM_GGML_TYPE_F32 || !dense(rope)) return -1;
     return early_store_index(g, i, [rope](const lm_ggml_tensor *cp) {
         return cp->src[0] == rope && cp->type == LM_GGML_TYPE_F16 && attn_side_shape_ok(cp) && dense(cp) &&
                n_elements(cp) == n_elements(rope) && disjoint(cp, rope) && disjoint(cp, rope->src[0]);
-    });
+    }, run_at);
 }
 
 // ffn_gate and ffn_up in llama.cpp's node order: gate matmul, SILU, up matmul, MUL.  With up to 4 tokens the two matmuls
@@ -859,6 +880,45 @@ int head_merge_index(const lm_ggml_cgraph *g, int i) {
     return j;
 }
 
+// Q's and K's ROPE of a layer (same positions, parameters, head size and token count) in one launch: index of a later ROPE
+// node that may run at node i's place, or -1.  Its input must be there already: the result of a projection that ran early
+// with node i's own (ran_early says where it lies).  Its F32 result is written early only if nothing in between touches
+// that memory; when the cache store that runs with it is its only reader, it is not written at all.
+constexpr int ROPE_LOOKAHEAD = 8;
+template <typename F>
+int rope_partner_index(const lm_ggml_cgraph *g, int i, graph_reads &reads, F ran_early, rope_partner &out) {
+    const lm_ggml_tensor *first = g->nodes[i];
+    const int end = i + 1 + ROPE_LOOKAHEAD < g->n_nodes ? i + 1 + ROPE_LOOKAHEAD : g->n_nodes;
+    for (int j = i + 1; j < end; j++) {
+        const lm_ggml_tensor *rp = g->nodes[j];
+        if (rp->op != LM_GGML_OP_ROPE) continue;
+        const lm_ggml_tensor *in = rp->src[0];
+        if (!attn_side_shape_ok(rp) || rp->src[1] != first->src[1] || rp->src[2] != first->src[2] ||
+            std::memcmp(rp->op_params, first->op_params, sizeof(rp->op_params)) != 0 || rp->ne[0] != first->ne[0] || rp->ne[2] != first->ne[2])
+            return -1;
+        const lm_ggml_tensor *owner = in->view_src ? in->view_src : in;
+        const void *at = ran_early(owner);
+        if (!at) return -1;
+        out.op = rp;
+        out.src = (const uint8_t *)at + ((const uint8_t *)in->data - (const uint8_t *)owner->data);
+        const int st = rope_store_index(g, j, i);
+        out.store = st >= 0 ? g->nodes[st] : nullptr;
+        out.store_index = st;
+        out.write_f32 = !(out.store && !(rp->flags & LM_GGML_TENSOR_FLAG_OUTPUT) && reads.readers_of(g, rp) == 1);
+        if (out.write_f32) {
+            for (int m = i; m < j; m++) {                // its memory may still belong to someone between the two nodes
+                const lm_ggml_tensor *t = g->nodes[m];
+                if (is_view_op(t->op)) continue;
+                if (!ranges_apart(t, rp)) return -1;
+                for (int k = 0; k < LM_GGML_MAX_SRC; k++)
+                    if (t->src[k] && !ranges_apart(t->src[k], rp)) return -1;
+            }
+        }
+        return j;
+    }
+    return -1;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
@@ -873,9 +933,10 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     int paired_matmul = -1;                           // index of an up projection that ran with its gate projection
     int grouped[CHIP_GROUP_MAX] = {-1, -1, -1, -1};   // projections that already ran with an earlier one of the same input
     const float *grouped_copy[CHIP_GROUP_MAX] = {nullptr, nullptr, nullptr, nullptr};   // ... into a scratch slot, still to be copied to their place
-    int rope_from_slot = -1;                          // a ROPE node whose input lies in a scratch slot instead
+    int rope_from_slot = -1, rope_from_slot_owner = -1;   // a ROPE node whose input lies in a scratch slot instead, and the projection's node
     const float *rope_slot_src = nullptr;
     graph_reads reads;
+    int rope_done = -1, rope_done_store = -1;         // a ROPE node (and its cache store) that already ran in an earlier ROPE's launch
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -968,8 +1029,12 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             paired_matmul = -1;
             continue;
         }
+        if (i == rope_done) { rope_done = -1; continue; }
+        if (i == rope_done_store) { rope_done_store = -1; continue; }
         if (is_attn_side_op(node->op) && attn_side_shape_ok(node)) {
             const lm_ggml_tensor *store = nullptr;
+            rope_partner partner;
+            bool paired = false;
             if (node->op == LM_GGML_OP_ROPE && fusion_enabled()) {
                 const int j = rope_store_index(cgraph, i);
                 if (j >= 0 && remember_store(j)) {
@@ -978,8 +1043,36 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                     g_elementwise_nodes++;
                     g_fused_pairs++;
                 }
+                if (rope_done < 0 && rope_done_store < 0) {
+                    // where the result of a projection that already ran with an earlier one lies: its slot or its own memory
+                    auto ran_early = [&](const lm_ggml_tensor *t) -> const void * {
+                        for (int k = 0; k < CHIP_GROUP_MAX; k++) {
+                            if (grouped[k] < 0 || cgraph->nodes[grouped[k]] != t) continue;
+                            if (rope_from_slot >= 0 && grouped[k] == rope_from_slot_owner) return rope_slot_src;
+                            if (grouped_copy[k]) return t->nb[1] == (size_t)t->ne[0] * sizeof(float) ? grouped_copy[k] : nullptr;
+                            return t->data;
+                        }
+                        return nullptr;
+                    };
+                    const int pj = rope_partner_index(cgraph, i, reads, ran_early, partner);
+                    if (pj >= 0) {
+                        paired = true;
+                        rope_done = pj;
+                        if (pj == rope_from_slot) rope_from_slot = -1;
+                        writes(cgraph->nodes[pj]);
+                        if (partner.store) {
+                            rope_done_store = partner.store_index;
+                            writes(partner.store);
+                            g_elementwise_nodes++;
+                            g_fused_pairs++;
+                        }
+                        g_elementwise_nodes++;
+                        g_fused_pairs++;
+                        g_rope_pairs++;
+                    }
+                }
             }
-            const int rc = run_attn_side(c, node, store, i == rope_from_slot ? rope_slot_src : nullptr);
+            const int rc = run_attn_side(c, node, store, i == rope_from_slot ? rope_slot_src : nullptr, paired ? &partner : nullptr);
             if (i == rope_from_slot) rope_from_slot = -1;
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d) failed: %s\n", __func__, node->name, node->op, chip_error_string(rc));
@@ -1128,6 +1221,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                         (rp->src[0] == mm || rp->src[0]->view_src == mm) && rp->src[0]->data == mm->data && fusion_enabled() &&
                         mm->nb[1] == (size_t)mm->ne[0] * sizeof(float)) {
                         rope_from_slot = nx;
+                        rope_from_slot_owner = members[k];
                         rope_slot_src = mats[k].y;
                         continue;
                     }
@@ -1383,5 +1477,6 @@ unsigned long long lm_ggml_backend_hip_get_rope_tables(void) { return g_rope_tab
 unsigned long long lm_ggml_backend_hip_get_async_uploaded(void) { return g_uploaded_async.load(); }
 unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void) { return g_grouped_matmuls.load(); }
 unsigned long long lm_ggml_backend_hip_get_head_merges(void) { return g_head_merges.load(); }
+unsigned long long lm_ggml_backend_hip_get_rope_pairs(void) { return g_rope_pairs.load(); }
 
 }  // extern "C"

@@ -287,6 +287,8 @@ struct GetRowsArgs {
     float *dst; int64_t ld1, ld2, ld3;                                         // dst strides in floats
 };
 hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st);
+hipError_t launch_rope_apply_two(const float *xa, const RopeArgs &a, float *ya, const float *xb, const RopeArgs &b, float *yb,
+                                 const float *table, hipStream_t st);
 hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, float *table,
                        bool build, hipStream_t st);
 

@@ -680,13 +680,15 @@ constexpr int ROPE_MAX_PAIRS = 256;
 template <int MODE>
 __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *x, const int32_t *__restrict__ pos,
                                                           const float *__restrict__ freq_factors, RopeArgs a, float *y,
-                                                          float *__restrict__ table) {
+                                                          float *__restrict__ table, const float *xb, RopeArgs ab, float *yb) {
     __shared__ float cs[ROPE_MAX_PAIRS], sn[ROPE_MAX_PAIRS];
+    // a second tensor with the same table (Q and K of a layer): the workgroups with blockIdx.y == 1 take it
+    if (blockIdx.y == 1) { x = xb; a = ab; y = yb; }
     constexpr int PRE = 8;                                       // items per thread whose loads are issued before the table is built
     const int64_t tok = blockIdx.x;
     const int half = a.n_dims / 2;
     const float *xt = x + tok * a.ldx2;
-    float *yt = y + tok * a.ldy2;
+    float *yt = y ? y + tok * a.ldy2 : nullptr;                  // no fp32 result wanted: only the fp16 copy
     const uint32_t per_head = (uint32_t)(a.ne0 - half);          // one item per rotated pair or per passed-through value
     const uint32_t items = (uint32_t)a.ne1 * per_head;           // 32-bit division: the 64-bit one is a long software routine
     // the operands of the first PRE * EW_THREADS items do not depend on the table: fetch them first
@@ -753,42 +755,54 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(const float *x, const 
         if (jj[u] < (uint32_t)half) {
             const float c = cs[jj[u]], s = sn[jj[u]];
             const float r0 = x0[u] * c - x1[u] * s, r1 = x0[u] * s + x1[u] * c;
-            yt[ia[u]] = r0;
-            yt[ib[u]] = r1;
+            if (yt) { yt[ia[u]] = r0; yt[ib[u]] = r1; }
             if (ht) { ht[ha[u]] = f2h_rne(r0); ht[hb[u]] = f2h_rne(r1); }
         } else {
-            yt[ia[u]] = x0[u];
+            if (yt) yt[ia[u]] = x0[u];
             if (ht) ht[ha[u]] = f2h_rne(x0[u]);
         }
     }
     for (uint32_t i = threadIdx.x + PRE * EW_THREADS; i < items; i += EW_THREADS) {
         const uint32_t h = i / per_head, j = i - h * per_head;
         const float *xr = xt + h * a.ldx1;
-        float *yr = yt + h * a.ldy1;
+        float *yr = yt ? yt + h * a.ldy1 : nullptr;
         unsigned short *hr = ht ? ht + h * a.ld16_1 : nullptr;
         if (j < (uint32_t)half) {
             const int64_t ka = a.neox ? j : 2 * j, kb = a.neox ? j + half : 2 * j + 1;
             const float v0 = xr[ka], v1 = xr[kb], c = cs[j], s = sn[j];
             const float r0 = v0 * c - v1 * s, r1 = v0 * s + v1 * c;
-            yr[ka] = r0;
-            yr[kb] = r1;
+            if (yr) { yr[ka] = r0; yr[kb] = r1; }
             if (hr) { hr[ka] = f2h_rne(r0); hr[kb] = f2h_rne(r1); }
         } else {
-            yr[j + half] = xr[j + half];
+            if (yr) yr[j + half] = xr[j + half];
             if (hr) hr[j + half] = f2h_rne(xr[j + half]);
         }
     }
 }
 // table == nullptr: one launch.  Otherwise build (x, y unused) or apply (pos, freq_factors unused) against table.
+static bool rope_args_ok(const RopeArgs &a) {
+    if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff || a.ne0 * a.ne1 > 0x7fffffff) return false;
+    return !(a.ne1 * a.ldx1 > 0x7fffffff || a.ne1 * a.ldy1 > 0x7fffffff || a.ne1 * a.ld16_1 > 0x7fffffff);   // 32-bit offsets inside a token
+}
 hipError_t launch_rope(const float *x, const int32_t *pos, const float *freq_factors, const RopeArgs &a, float *y, float *table,
                        bool build, hipStream_t st) {
     if (a.ne2 <= 0 || (!build && (a.ne0 <= 0 || a.ne1 <= 0))) return hipSuccess;
-    if (a.n_dims / 2 > ROPE_MAX_PAIRS || a.ne2 > 0x7fffffff || a.ne0 * a.ne1 > 0x7fffffff) return hipErrorInvalidValue;
-    if (a.ne1 * a.ldx1 > 0x7fffffff || a.ne1 * a.ldy1 > 0x7fffffff || a.ne1 * a.ld16_1 > 0x7fffffff) return hipErrorInvalidValue;   // 32-bit offsets inside a token
+    if (!rope_args_ok(a)) return hipErrorInvalidValue;
     const dim3 grid((unsigned)a.ne2), block(EW_THREADS);
-    if (!table) hipLaunchKernelGGL(rope_kernel<ROPE_FULL>, grid, block, 0, st, x, pos, freq_factors, a, y, (float *)nullptr);
-    else if (build) hipLaunchKernelGGL(rope_kernel<ROPE_BUILD>, grid, block, 0, st, x, pos, freq_factors, a, y, table);
-    else hipLaunchKernelGGL(rope_kernel<ROPE_APPLY>, grid, block, 0, st, x, pos, freq_factors, a, y, table);
+    if (!table) hipLaunchKernelGGL(rope_kernel<ROPE_FULL>, grid, block, 0, st, x, pos, freq_factors, a, y, (float *)nullptr, x, a, y);
+    else if (build) hipLaunchKernelGGL(rope_kernel<ROPE_BUILD>, grid, block, 0, st, x, pos, freq_factors, a, y, table, x, a, y);
+    else hipLaunchKernelGGL(rope_kernel<ROPE_APPLY>, grid, block, 0, st, x, pos, freq_factors, a, y, table, x, a, y);
+    return hipGetLastError();
+}
+// Two tensors rotated with one table in one launch (same ne0, ne2, n_dims and mode; heads, strides and outputs of their own;
+// y may be null where only the fp16 copy is wanted).
+hipError_t launch_rope_apply_two(const float *xa, const RopeArgs &a, float *ya, const float *xb, const RopeArgs &b, float *yb,
+                                 const float *table, hipStream_t st) {
+    if (a.ne2 <= 0 || a.ne0 <= 0 || a.ne1 <= 0 || b.ne1 <= 0) return hipErrorInvalidValue;
+    if (a.ne0 != b.ne0 || a.ne2 != b.ne2 || a.n_dims != b.n_dims || a.neox != b.neox || !rope_args_ok(a) || !rope_args_ok(b)) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)a.ne2, 2), block(EW_THREADS);
+    hipLaunchKernelGGL(rope_kernel<ROPE_APPLY>, grid, block, 0, st, xa, (const int32_t *)nullptr, (const float *)nullptr, a, ya,
+                       const_cast<float *>(table), xb, b, yb);
     return hipGetLastError();
 }
 

@@ -371,6 +371,20 @@ CHIP_API int chip_rope_apply(const float *x, int64_t ldx1, int64_t ldx2, const f
 CHIP_API int chip_rope_apply_store(const float *x, int64_t ldx1, int64_t ldx2, const float *table, int64_t ne0, int64_t ne1,
                                    int64_t ne2, int n_dims, int mode, float *y, int64_t ldy1, int64_t ldy2, uint16_t *y_f16,
                                    int64_t ld16_1, int64_t ld16_2, void *stream);
+/* Two tensors rotated with one table in one launch: Q and K of a layer, which the reference rotates in two ROPE nodes with the
+ * same positions and parameters (cactus/llama-model.cpp build_llama: lm_ggml_rope_ext on Qcur and on Kcur).  Each operand has
+ * its own heads (ne1), strides and outputs: y (F32) and / or y_f16 (the fp16 copy chip_rope_apply_store makes, i.e. the K
+ * cache store that follows K's ROPE); one of the two may be NULL - with y NULL only the fp16 copy is written, for a ROPE
+ * whose F32 result nobody else reads.  Every value written has the bits chip_rope_apply / chip_rope_apply_store give. */
+typedef struct chip_rope_operand {
+    const float *x; int64_t ldx1, ldx2;        /* input: head and token strides in floats */
+    int64_t ne1;                               /* heads */
+    float *y; int64_t ldy1, ldy2;              /* F32 result or NULL */
+    uint16_t *y_f16; int64_t ld16_1, ld16_2;   /* fp16 copy or NULL: head and token strides in halves */
+} chip_rope_operand;
+CHIP_API int chip_rope_apply_two(const chip_rope_operand *a, const chip_rope_operand *b, const float *table, int64_t ne0,
+                                 int64_t ne2, int n_dims, int mode, void *stream);
+
 
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,

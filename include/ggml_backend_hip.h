@@ -58,6 +58,8 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void)
 /* kqv MUL_MAT nodes that also wrote the head merge that follows them, CONT(PERMUTE(kqv)) (cactus/llama-graph.cpp:1154-1158),
  * up to 4 (query head, token) pairs per KV head. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_head_merges(void);
+/* ROPE nodes that ran in the launch of an earlier ROPE with the same positions and parameters (K's with Q's). */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_pairs(void);
 
 #ifdef __cplusplus
 }

@@ -257,6 +257,44 @@ def test_rope_with_the_cache_store_in_one_launch(dev, mode, ne0, n_dims, n_head,
     assert h.tobytes() == dev.cpy(y.reshape(-1, ne0), np.float16).tobytes() == y.astype(np.float16).tobytes()
 
 
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("ne0,n_dims,heads_a,heads_b,n_tokens", [(128, 128, 32, 8, 1), (128, 128, 32, 8, 5), (64, 32, 3, 1, 2), (256, 256, 40, 40, 3)])
+def test_rope_of_q_and_k_in_one_launch(dev, mode, ne0, n_dims, heads_a, heads_b, n_tokens):
+    """chip_rope_apply_two: every output equals what chip_rope / chip_rope_apply_store give for that tensor alone, bit for
+    bit, also when one tensor asks for its fp16 copy only."""
+    rng = np.random.default_rng(ne0 + heads_a + mode)
+    xa = (rng.standard_normal((n_tokens, heads_a, ne0)) * 3).astype(np.float32)
+    xb = (rng.standard_normal((n_tokens, heads_b, ne0)) * 3).astype(np.float32)
+    pos = np.array([5, 0, 4095, 17, 100000][:n_tokens], np.int32)
+    ya = dev.rope(xa, pos, n_dims, mode, freq_base=500000.0)
+    yb, hb = dev.rope(xb, pos, n_dims, mode, freq_base=500000.0, store_f16=True)
+    a, b = dev.rope_two(xa, xb, pos, n_dims, mode, freq_base=500000.0)
+    assert a["f32"].tobytes() == ya.tobytes() and "f16" not in a
+    assert b["f32"].tobytes() == yb.tobytes() and b["f16"].tobytes() == hb.tobytes()
+    a, b = dev.rope_two(xa, xb, pos, n_dims, mode, want=(("f32", "f16"), ("f16",)), freq_base=500000.0)
+    assert a["f32"].tobytes() == ya.tobytes() and a["f16"].tobytes() == ya.astype(np.float16).tobytes()
+    assert b["f16"].tobytes() == hb.tobytes() and "f32" not in b
+
+
+def test_rope_of_two_tensors_rejects_bad_operands(dev):
+    import cactus_amd as ca
+    L = dev.lib
+    d = dev.alloc(1 << 16)
+    good = lambda: ca.RopeOperand(d.ptr, 64, 256, 4, d.ptr + 4096, 64, 256, None, 0, 0)
+    a, b = good(), good()
+    assert L.chip_rope_apply_two(C.byref(a), C.byref(b), d.ptr + 8192, 64, 1, 64, 2, None) == ca.CHIP_OK
+    assert L.chip_rope_apply_two(C.byref(a), None, d.ptr + 8192, 64, 1, 64, 2, None) == ca.CHIP_EINVAL
+    assert L.chip_rope_apply_two(C.byref(a), C.byref(b), None, 64, 1, 64, 2, None) == ca.CHIP_EINVAL
+    assert L.chip_rope_apply_two(C.byref(a), C.byref(b), d.ptr + 8192, 64, 1, 64, 8, None) == ca.CHIP_EUNSUPPORTED
+    b.y = None                                                                    # neither output
+    assert L.chip_rope_apply_two(C.byref(a), C.byref(b), d.ptr + 8192, 64, 1, 64, 2, None) == ca.CHIP_EINVAL
+    b = good(); b.ldx1 = 32
+    assert L.chip_rope_apply_two(C.byref(a), C.byref(b), d.ptr + 8192, 64, 1, 64, 2, None) == ca.CHIP_EINVAL
+    b = good(); b.y_f16 = d.ptr + 16384 + 1; b.ld16_1 = 64
+    assert L.chip_rope_apply_two(C.byref(a), C.byref(b), d.ptr + 8192, 64, 1, 64, 2, None) == ca.CHIP_EINVAL
+    dev.sync()
+
+
 ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8, 3, 96, 128), (256, 4, 2, 2, 160, 160),
                (96, 6, 2, 5, 72, 80), (128, 28, 4, 2, 104, 128), (128, 8, 2, 70, 128, 128), (128, 32, 8, 130, 320, 512),
                (64, 4, 4, 100, 192, 256), (96, 6, 2, 40, 104, 128), (128, 32, 8, 512, 1056, 2048),

@@ -881,15 +881,20 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     fused_before = blib.lm_ggml_backend_hip_get_fused_pairs()
     blib.lm_ggml_backend_hip_get_grouped_matmuls.restype = C.c_ulonglong
     grouped_before = blib.lm_ggml_backend_hip_get_grouped_matmuls()
+    blib.lm_ggml_backend_hip_get_rope_pairs.restype = C.c_ulonglong
+    pairs_before = blib.lm_ggml_backend_hip_get_rope_pairs()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     assert blib.lm_ggml_backend_hip_get_rope_tables() - tables_before == 1      # Q and K share one cos / sin table
     # The K store ran in the kernel of K's RoPE.  With up to 4 tokens the transposed V store ran in the V projection's
-    # launch, and the projections whose results the graph allocator did not place over a tensor that is still read in
-    # between (Kcur over Qcur, which dies at its RoPE, say) ran as one launch: all three, two of them, or none.
+    # launch, and the three projections ran as one launch: one whose own memory the graph allocator placed over a tensor
+    # that is still read in between (Kcur over Qcur, which dies at its RoPE, say) wrote into a slot of the backend's instead.
     grouped = blib.lm_ggml_backend_hip_get_grouped_matmuls() - grouped_before
-    assert grouped == 0 if n_tokens > 4 else grouped in (0, 2, 3), grouped
+    assert grouped == (0 if n_tokens > 4 else 3), grouped
     fused = blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before
-    assert fused == (1 if n_tokens > 4 else 2 + max(grouped - 1, 0)), (fused, grouped)
+    # K's RoPE (with its store) in the launch of Q's when K's projection had already run with Q's
+    pairs = blib.lm_ggml_backend_hip_get_rope_pairs() - pairs_before
+    assert pairs == (1 if grouped >= 2 else 0), (pairs, grouped)
+    assert fused == (1 if n_tokens > 4 else 2 + max(grouped - 1, 0) + pairs), (fused, grouped, pairs)
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
