@@ -754,11 +754,16 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
             # residual + norm + weight: one kernel, as the backend fuses the three nodes
             ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
             (t_, wg, N_, K_), (_, wu, _, _) = W["gate"], W["up"]
-            ck(L.chip_mul_mat_pair(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, up.ptr, N_, ws.ptr, wsz, st))
-            # SiLU in its MUL's kernel, which also leaves ffn_down's quantized rows in the workspace, as the backend runs the three nodes
-            t_, wd, N_, K_ = W["down"]
-            ck(L.chip_silu_mul_quantized(gate.ptr, FF, up.ptr, FF, n, FF, gate.ptr, FF, t_, ws.ptr, wsz, st))
-            ck(L.chip_mul_mat_run_ws(t_, wd, dev.row_size(t_, K_), K_, N_, n, ws.ptr, wsz, att.ptr, N_, st))
+            td, wd, Nd, Kd = W["down"]
+            if n <= 4 and L.chip_mul_mat_pair_silu_mul_supported(t_, K_, N_, n) == 1:
+                # gate, SILU, up and their MUL in one launch; ffn_down quantizes its input itself, as the backend runs the five nodes
+                ck(L.chip_mul_mat_pair_silu_mul(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, N_, ws.ptr, wsz, st))
+                ck(L.chip_mul_mat(td, wd, dev.row_size(td, Kd), Kd, Nd, gate.ptr, Kd, n, att.ptr, Nd, ws.ptr, wsz, st))
+            else:
+                ck(L.chip_mul_mat_pair(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, up.ptr, N_, ws.ptr, wsz, st))
+                # SiLU in its MUL's kernel, which also leaves ffn_down's quantized rows in the workspace, as the backend runs the three nodes
+                ck(L.chip_silu_mul_quantized(gate.ptr, FF, up.ptr, FF, n, FF, gate.ptr, FF, td, ws.ptr, wsz, st))
+                ck(L.chip_mul_mat_run_ws(td, wd, dev.row_size(td, Kd), Kd, Nd, n, ws.ptr, wsz, att.ptr, Nd, st))
             # the layer's second residual with the next layer's (or the final) norm
             ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
         ck(L.chip_mul_mat(ca.Q6_K, trace.arena.ptr + trace.head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))

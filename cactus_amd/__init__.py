@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_pair_silu_mul", "chip_mul_mat_pair_silu_mul_supported", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_rope_apply_two", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
@@ -122,6 +122,8 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
     L.chip_mul_mat_run_ws.argtypes = [i32, vp, sz, i64, i64, i64, vp, sz, vp, i64, vp]
     L.chip_mul_mat_pair.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, vp, i64, vp, sz, vp]
+    L.chip_mul_mat_pair_silu_mul.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
+    L.chip_mul_mat_pair_silu_mul_supported.argtypes = [i32, i64, i64, i64]
     L.chip_mul_mat_store_t.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, i64, vp, sz, vp]
     L.chip_rms_norm.argtypes = [vp, i64, i64, i64, C.c_float, vp, i64, vp]
     L.chip_add.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
@@ -330,6 +332,22 @@ class Device:
         self.check(self.lib.chip_mul_mat_pair(wtype, d1.ptr, d2.ptr, nb01, k, N, dx.ptr, k, n, y1.ptr, y2.ptr, N, ws.ptr, wsz, None))
         self.sync()
         return y1.download(np.float32, n * N).reshape(n, N), y2.download(np.float32, n * N).reshape(n, N)
+
+    def mul_mat_pair_silu_mul(self, wtype, W1, W2, x):
+        """silu(W1 x) * (W2 x) in one launch (chip_mul_mat_pair_silu_mul): fp32 [n, N]."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, k = x.shape
+        W1, W2 = np.ascontiguousarray(W1, np.uint8), np.ascontiguousarray(W2, np.uint8)
+        N = W1.shape[0]
+        nb01 = self.row_size(wtype, k)
+        d1, d2, dx = self.to_device(W1), self.to_device(W2), self.to_device(x)
+        y = self.alloc(n * N * 4)
+        self.check(self.lib.chip_memset(y.ptr, 0xFF, n * N * 4, None))                   # NaN: unwritten rows show
+        wsz = self.lib.chip_mul_mat_workspace_size_n(wtype, k, N, n)
+        ws = self.alloc(wsz)
+        self.check(self.lib.chip_mul_mat_pair_silu_mul(wtype, d1.ptr, d2.ptr, nb01, k, N, dx.ptr, k, n, y.ptr, N, ws.ptr, wsz, None))
+        self.sync()
+        return y.download(np.float32, n * N).reshape(n, N)
 
     def rms_norm(self, x, eps):
         x = np.ascontiguousarray(x, np.float32)

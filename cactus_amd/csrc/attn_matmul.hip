@@ -100,35 +100,46 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedAr
     const int64_t b0 = blockIdx.y;
     const uint8_t *Wb = a.W + b0 * a.nb02;
     const bool has_chunk = sub < a.K / 8;
+    const int subc = has_chunk ? sub : 0;                            // lanes past the row's end load chunk 0 and count zeros
     const int64_t cols = a.r2 * a.n;
     const int64_t row_step = (int64_t)gridDim.x * AM_WAVES * RPS;
     const int64_t row0 = ((int64_t)blockIdx.x * AM_WAVES + wave) * RPS + grp;
+    const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
+    // Every load is unconditional, from a clamped address, so that the columns' and the first rows' requests leave together:
+    // one round trip to memory instead of one per column and then one for the rows.
+    auto load_rows = [&](int64_t rbase, u32x4 (&w)[UNROLL]) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int64_t row = rbase + u * row_step;
+            w[u] = *reinterpret_cast<const u32x4 *>(Wb + (row < a.N ? row : a.N - 1) * a.nb01 + 16 * subc);
+        }
+    };
     for (int64_t c0 = 0; c0 < cols; c0 += AM_COLS) {
-        u32x4 xh[AM_COLS];
+        float4 xlo[AM_COLS], xhi[AM_COLS];
 #pragma unroll
         for (int j = 0; j < AM_COLS; j++) {
             const int64_t c = c0 + j < cols ? c0 + j : cols - 1;                  // clamped: the load stays in bounds, the result is unused
-            xh[j] = u32x4{0u, 0u, 0u, 0u};
-            if (has_chunk) {
-                const float4 *xp = reinterpret_cast<const float4 *>(col_x(a, b0, c) + 8 * sub);
-                xh[j] = round8(xp[0], xp[1]);
-            }
+            const float4 *xp = reinterpret_cast<const float4 *>(col_x(a, b0, c) + 8 * subc);
+            xlo[j] = xp[0];
+            xhi[j] = xp[1];
         }
-        for (int64_t rbase = row0; rbase < a.N; rbase += UNROLL * row_step) {
-            u32x4 w[UNROLL];
+        u32x4 w[UNROLL];
+        if (row0 < a.N) load_rows(row0, w);
+        u32x4 xh[AM_COLS];
+#pragma unroll
+        for (int j = 0; j < AM_COLS; j++) xh[j] = has_chunk ? round8(xlo[j], xhi[j]) : zero;
+        for (int64_t rbase = row0; rbase < a.N;) {
+            const int64_t next = rbase + UNROLL * row_step;
+            u32x4 wn[UNROLL];
+            if (next < a.N) load_rows(next, wn);
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
                 const int64_t row = rbase + u * row_step;
-                w[u] = u32x4{0u, 0u, 0u, 0u};
-                if (row < a.N && has_chunk) w[u] = *reinterpret_cast<const u32x4 *>(Wb + row * a.nb01 + 16 * sub);
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const int64_t row = rbase + u * row_step;
+                const u32x4 wu = has_chunk ? w[u] : zero;
                 float acc[AM_COLS];
 #pragma unroll
                 for (int j = 0; j < AM_COLS; j++) {
-                    acc[j] = group_sum<LPR>(dot8(w[u], xh[j], 0.0f));
+                    acc[j] = group_sum<LPR>(dot8(wu, xh[j], 0.0f));
                 }
                 if (sub == 0 && row < a.N) {
 #pragma unroll
@@ -139,6 +150,11 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedAr
                         }
                 }
             }
+            if (next < a.N) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) w[u] = wn[u];
+            }
+            rbase = next;
         }
     }
 }

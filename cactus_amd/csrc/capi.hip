@@ -477,6 +477,30 @@ int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int
     return mul_mat_run(type, W2, nb01, K, N, n, workspace, workspace_bytes, y2, ldy, stream);
 }
 
+// MUL(SILU(MUL_MAT(W1, x)), MUL_MAT(W2, x)) in one launch, where chip_mul_mat_pair runs its one-launch GEMV
+int chip_mul_mat_pair_silu_mul_supported(int type, int64_t K, int64_t N, int64_t n) {
+    if (!chip_mul_mat_supported(type, K) || N <= 0 || n < 1 || n > 4 || 2 * N > 0x7fffffff) return 0;
+    if (N % 8 != 0) return 0;                                               // as chip_silu: the reference's row tail uses the C library's expf
+    DeviceLimits lim;
+    if (current_limits(lim) != CHIP_OK) return 0;
+    return gemv_fused_applicable(type, K, (int)n, lim) ? 1 : 0;
+}
+int chip_mul_mat_pair_silu_mul(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                               int64_t n, float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (N < 0 || n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n == 0) return CHIP_OK;
+    if (!chip_mul_mat_pair_silu_mul_supported(type, K, N, n)) return CHIP_EUNSUPPORTED;
+    if (!W1 || !W2 || !x || !y || !workspace || ldx < K || ldy < N) return CHIP_EINVAL;
+    if (!weights_aligned(type, W1, nb01, K) || !weights_aligned(type, W2, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
+    if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || (((uintptr_t)y) & 3) != 0) return CHIP_EINVAL;
+    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+    DeviceLimits lim;
+    if (int rc = current_limits(lim); rc) return rc;
+    return hip_rc(launch_gemv_fused_pair_silu_mul(type, W1, W2, nb01, K, N, x, ldx, (int)n, workspace,
+                                                  act_stride(chip_vec_dot_type(type), K), y, ldy, lim, (hipStream_t)stream));
+}
+
 // Several matmuls on one activation (wq / wk / wv).  Up to 4 tokens, members of one family: one launch of the
 // prologue-quantizing GEMV over all members; otherwise one quantizer and each member on its usual path.
 // what chip_mul_mat_group and chip_mul_mat_group_run share: x == nullptr says the workspace already holds the rows

@@ -23,12 +23,12 @@
 
 namespace chip {
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED>
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED, bool GATED = false>
 __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                                    const float *__restrict__ x, int64_t ldx,
                                                    uint8_t *__restrict__ ws, size_t ws_stride,
                                                    float *__restrict__ y, int64_t ldy, SecondMatrix sec) {
-    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED, GATED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
 }
 
 // LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
@@ -64,26 +64,31 @@ static hipError_t launch_depth(const void *W, size_t nb01, int64_t K, int64_t N,
     const int64_t tiles = ceil_div(N, R);
     int64_t groups = ceil_div(tiles, WGS / 64);
     if (groups > max_groups) groups = max_groups;
+    auto launch = [&](auto kfn, LdsGrant &grant) {
+        if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
+        hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
+                           (uint8_t *)ws, ws_stride, y, ldy, sec);
+        return hipGetLastError();
+    };
     // Rows of more than one step whose activations the prologue quantizes to Q8_K: the kernel that builds the image a
     // step's part at a time (gemv_body.h: PHASED)
     if constexpr (FUSEQ && Traits<WT>::ACT == T_Q8_K && WGS >= 256) {
         // (measured: 4096 x 14336 Q4_K 10.5 -> 9.5 us, 4096 x 11008 8.7 -> 8.0 us, Q6_K 4096 x 14336 15.3-16.1 -> 14.7 us;
         //  two steps - K = 8192 - run 2 % slower that way and keep the plain prologue)
         if (iters_per_row<WT>(K) > 2 && tune("CHIP_GEMV_PHASED", 1) != 0) {
-            auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, true>;
-            static LdsGrant grant;
-            if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
-            hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
-                               (uint8_t *)ws, ws_stride, y, ldy, sec);
-            return hipGetLastError();
+            static LdsGrant grant, grant_gated;                          // one per kernel instantiation
+            if (sec.gated) return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, true, true>, grant_gated);
+            return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, true>, grant);
         }
     }
-    auto kfn = gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false>;
-    static LdsGrant grant;                                               // one per kernel instantiation
-    if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kfn, dim3((unsigned)groups), dim3(WGS), lds_bytes, st, (const uint8_t *)W, nb01, K, N, x, ldx,
-                       (uint8_t *)ws, ws_stride, y, ldy, sec);
-    return hipGetLastError();
+    static LdsGrant grant;
+    if constexpr (FUSEQ) {                                                // the gated pair exists with the quantizing prologue only
+        static LdsGrant grant_gated;
+        if (sec.gated) return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false, true>, grant_gated);
+    } else {
+        if (sec.gated) return hipErrorInvalidValue;
+    }
+    return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false>, grant);
 }
 
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ>
@@ -265,6 +270,13 @@ hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, siz
                                   const DeviceLimits &lim, hipStream_t st) {
     const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, (int64_t)(y2 - y1) - N, nullptr, 0};
     return launch_gemv_fused_sec(wtype, W1, nb01, K, 2 * N, x, ldx, n, ws, ws_stride, y1, ldy, lim, st, sec);
+}
+// silu(W1 x) * (W2 x) -> y, one launch (gemv_body.h: gated)
+hipError_t launch_gemv_fused_pair_silu_mul(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
+                                           int64_t ldx, int n, void *ws, size_t ws_stride, float *y, int64_t ldy,
+                                           const DeviceLimits &lim, hipStream_t st) {
+    const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, 0, nullptr, 0, 1};
+    return launch_gemv_fused_sec(wtype, W1, nb01, K, 2 * N, x, ldx, n, ws, ws_stride, y, ldy, lim, st, sec);
 }
 // y16t: element (token t, row r) of the result also goes to y16t[r * ld16 + t] as fp16
 hipError_t launch_gemv_fused_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int n,

@@ -889,10 +889,13 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
 struct GridPart { int64_t block, blocks; bool writes_workspace; };
 __device__ __forceinline__ GridPart whole_grid() { return GridPart{(int64_t)blockIdx.x, (int64_t)gridDim.x, blockIdx.x == 0}; }
 
-struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; };
-constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0};
+// gated (two matrices only): a wave takes row r of the first matrix and then row r of the second, and what is stored, at y's
+// row r, is silu(first) * second - the SILU and MUL nodes that follow ffn_gate and ffn_up (reference llama-graph.cpp:562-690,
+// LLM_FFN_SILU with LLM_FFN_PAR), with lm_ggml_vec_silu_f32's arithmetic; the two projections themselves are not stored.
+struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; int gated; };
+constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0, 0};
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false>
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false, bool GATED = false>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                           const float *__restrict__ x, int64_t ldx,
                                           uint8_t *__restrict__ ws, size_t ws_stride,
@@ -907,7 +910,10 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     const int lane = threadIdx.x & 63;
     const int64_t wave = gp.block * (WGS / 64) + (threadIdx.x >> 6);
     const int64_t nwaves = gp.blocks * (WGS / 64);
-    const int64_t tiles = ceil_div(N, R);
+    // gated: tile T is row tile T / 2 of matrix T % 2; a wave walks 2 * wave, 2 * wave + 1, 2 * (wave + nwaves), ...
+    constexpr bool gated = GATED;                      // a kernel of its own: sec.gated picks it in the launcher
+    const int64_t tiles = gated ? 2 * ceil_div(sec.n_first, (int64_t)R) : ceil_div(N, R);
+    const int64_t first_tile = gated ? 2 * wave : wave;
 
     // A wave walks the steps (tile, it) = (wave, 0), (wave, 1), ..., (wave + nwaves, 0), ...; while it computes one step
     // the loads of the next are in flight.  Measured and dropped: rings of two and three steps (3-8 % slower as a loop; the
@@ -919,7 +925,10 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     struct Step { int64_t tile; int it; bool have; };
     auto after = [&](const Step &s) {
         Step n = s;
-        if (s.it + 1 == NI) { n.tile = s.tile + nwaves; n.it = 0; } else n.it = s.it + 1;
+        if (s.it + 1 == NI) {
+            n.tile = !gated ? s.tile + nwaves : ((s.tile & 1) ? s.tile + 2 * nwaves - 1 : s.tile + 1);
+            n.it = 0;
+        } else n.it = s.it + 1;
         n.have = s.have && n.tile < tiles;
         return n;
     };
@@ -934,12 +943,13 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
             const int u = min(s.it * 64 + lane, units - 1);
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const int64_t row = s.have ? min(s.tile * R + r, N - 1) : (int64_t)0;
+                int64_t row = s.have ? min(s.tile * R + r, N - 1) : (int64_t)0;
+                if (gated) row = s.have ? min((s.tile >> 1) * R + r, sec.n_first - 1) + (s.tile & 1) * sec.n_first : (int64_t)0;
                 T::load_raw(set[r], W + (size_t)row * nb01 + (row >= sec.n_first ? sec.w_off : (int64_t)0), u);
             }
         }
     };
-    Step s0{wave, 0, wave < tiles};
+    Step s0{first_tile, 0, first_tile < tiles};
 
     // ---- prologue: activation loads first, then DEPTH steps of weight loads, then the activation image is built in LDS
     //      while the weights are still in flight ----
@@ -980,6 +990,18 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
 #pragma unroll
         for (int t = 0; t < NTOK; t++) { acc[r][t] = 0.f; res[r][t] = 0.f; }
     auto flush = [&](int count) {
+        if (gated) {                                     // lanes 2j and 2j + 1 hold the two projections of one row tile
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int64_t row = (int64_t)res_row + r;
+#pragma unroll
+                for (int t = 0; t < NTOK; t++) {
+                    const float up = __shfl_down(res[r][t], 1);
+                    if (lane < count && !(lane & 1) && row < sec.n_first) y[(int64_t)t * ldy + row] = silu1(res[r][t]) * up;
+                }
+            }
+            return;
+        }
         if (lane < count) {
 #pragma unroll
             for (int r = 0; r < R; r++) {
@@ -1022,7 +1044,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
                     res[r][t] = lane == nres ? sum : res[r][t];
                     acc[r][t] = 0.f;
                 }
-            res_row = lane == nres ? (int)(s.tile * R) : res_row;
+            res_row = lane == nres ? (int)((gated ? s.tile >> 1 : s.tile) * R) : res_row;
             nres++;
         }
     };

@@ -27,7 +27,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -1163,6 +1163,33 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         int rc;
         const int64_t ldx = (int64_t)(x->nb[1] / 4);
         int store_t = -1;
+        if (n <= 4 && fusion_enabled()) {
+            // gate, SILU, up, MUL with nobody else reading the three intermediate results: one launch that stores the MUL's
+            // result only.  Its workgroups store while others still read the activation, so the two must lie apart.
+            const int up_index = paired_matmul_index(cgraph, i);
+            if (up_index >= 0) {
+                lm_ggml_tensor *up = cgraph->nodes[up_index], *silu = cgraph->nodes[i + 1], *mul = cgraph->nodes[i + 3];
+                const bool kept = ((node->flags | silu->flags | up->flags) & LM_GGML_TENSOR_FLAG_OUTPUT) != 0;
+                int64_t mrows, ldm;
+                if (!kept && chip_mul_mat_pair_silu_mul_supported(w->type, K, N, n) && as_rows(mul, mrows, ldm) && mrows == n && disjoint(mul, x) &&
+                    reads.readers_of(cgraph, node) == 1 && reads.readers_of(cgraph, silu) == 1 && reads.readers_of(cgraph, up) == 1) {
+                    c->quantized.valid = false;
+                    rc = chip_mul_mat_pair_silu_mul(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)x->data, ldx, n,
+                                                    (float *)mul->data, ldm, c->workspace, c->workspace_size, c->stream);
+                    if (rc != CHIP_OK) {
+                        HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: gated MUL_MAT pair at %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+                        return LM_GGML_STATUS_FAILED;
+                    }
+                    for (int k = 1; k <= 3; k++) writes(cgraph->nodes[i + k]);
+                    g_mul_mat_nodes += 2;
+                    g_elementwise_nodes += 2;
+                    g_fused_pairs += 3;
+                    g_gated_pairs++;
+                    i += 3;
+                    continue;
+                }
+            }
+        }
         int members[CHIP_GROUP_MAX];
         bool aliased[CHIP_GROUP_MAX] = {false, false, false, false};
         int n_members = 1;
@@ -1478,5 +1505,6 @@ unsigned long long lm_ggml_backend_hip_get_async_uploaded(void) { return g_uploa
 unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void) { return g_grouped_matmuls.load(); }
 unsigned long long lm_ggml_backend_hip_get_head_merges(void) { return g_head_merges.load(); }
 unsigned long long lm_ggml_backend_hip_get_rope_pairs(void) { return g_rope_pairs.load(); }
+unsigned long long lm_ggml_backend_hip_get_gated_pairs(void) { return g_gated_pairs.load(); }
 
 }  // extern "C"

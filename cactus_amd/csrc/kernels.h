@@ -152,6 +152,10 @@ hipError_t launch_gemv_fused_store_t(int wtype, const void *W, size_t nb01, int6
 hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                   int64_t ldx, int n, void *ws, size_t ws_stride, float *y1, float *y2, int64_t ldy,
                                   const DeviceLimits &lim, hipStream_t st);
+// silu(W1 x) * (W2 x) -> y in one launch: the gated FFN's four nodes up to ffn_down's input (shapes as launch_gemv_fused_pair)
+hipError_t launch_gemv_fused_pair_silu_mul(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
+                                           int64_t ldx, int n, void *ws, size_t ws_stride, float *y, int64_t ldy,
+                                           const DeviceLimits &lim, hipStream_t st);
 // gemv_group.hip: up to GROUP_MAX matrices that read the same activation rows in one launch of the prologue-quantizing
 // GEMV (members of one family: K-quants, 32-value block types, or F16).  t16: optional transposed fp16 copy of a member's
 // output, as launch_gemv_fused_store_t.

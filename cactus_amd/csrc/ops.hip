@@ -36,25 +36,6 @@ namespace chip {
 
 constexpr int EW_THREADS = 256;
 
-// one lane of lm_ggml_v_expf (AVX2 + FMA)
-__device__ __forceinline__ float v_expf_lane(float x) {
-    const float r = 0x1.8p23f;
-    const float z = __builtin_fmaf(x, 0x1.715476p+0f, r);
-    const float n = z - r;
-    const float b = __builtin_fmaf(-n, 0x1.7f7d1cp-20f, __builtin_fmaf(-n, 0x1.62e4p-1f, x));
-    const uint32_t e = __float_as_uint(z) << 23;
-    const float k = __uint_as_float(e + __float_as_uint(1.0f));
-    const float u = b * b;
-    const float j = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(0x1.0e4020p-7f, b, 0x1.573e2ep-5f), u,
-                                                  __builtin_fmaf(0x1.555e66p-3f, b, 0x1.fffdb6p-2f)),
-                                   u, 0x1.ffffecp-1f * b);
-    if (!(__builtin_fabsf(n) > 126.0f)) return __builtin_fmaf(j, k, k);
-    const uint32_t g = (n <= 0.0f) ? 0x82000000u : 0u;
-    const float s1 = __uint_as_float(g + 0x7f000000u), s2 = __uint_as_float(e - g);
-    if (__builtin_fabsf(n) > 192.0f) return s1 * s1;
-    return __builtin_fmaf(s2, j, s2) * s1;
-}
-__device__ __forceinline__ float silu1(float x) { return x / (1.0f + v_expf_lane(0.0f - x)); }
 
 // ---- RMS_NORM: one workgroup per row ----
 // With w, the row is also multiplied by the weight row w (the MUL node that follows a norm): y = (x * scale) * w, two

@@ -157,6 +157,16 @@ CHIP_API int chip_mul_mat_run(int type, const void *W, size_t nb01, int64_t K, i
 CHIP_API int chip_mul_mat_pair(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                int64_t ldx, int64_t n, float *y1, float *y2, int64_t ldy, void *workspace, size_t workspace_bytes,
                                void *stream);
+/* The gated FFN up to ffn_down's input in one launch: MUL(SILU(MUL_MAT(W1, x)), MUL_MAT(W2, x)), the four nodes of
+ * LLM_FFN_SILU with LLM_FFN_PAR (reference llama-graph.cpp:562-690; lm_ggml_vec_silu_f32, ggml-cpu/vec.cpp:164-186).  Arguments
+ * as chip_mul_mat_pair with one output: y[t * ldy + r] = silu(y1[t][r]) * y2[t][r], bit for bit what chip_mul_mat_pair
+ * followed by chip_silu_mul gives; the two projections themselves are not stored.  For 1, 2 or 4 tokens and N a multiple
+ * of 8 (as chip_silu) where chip_mul_mat_pair runs as one GEMV launch (chip_mul_mat_pair_silu_mul_supported returns 1); CHIP_EUNSUPPORTED
+ * otherwise, nothing written.  The workspace holds the quantized rows of x afterwards, as after chip_mul_mat. */
+CHIP_API int chip_mul_mat_pair_silu_mul_supported(int type, int64_t K, int64_t N, int64_t n);
+CHIP_API int chip_mul_mat_pair_silu_mul(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N,
+                                        const float *x, int64_t ldx, int64_t n, float *y, int64_t ldy, void *workspace,
+                                        size_t workspace_bytes, void *stream);
 /* Several matmuls that read the same activation rows (wq / wk / wv of an attention block: llama.cpp builds Qcur, Kcur,
  * Vcur from one tensor, llama-model.cpp build_llama; the reference quantizes src1 once per MUL_MAT node,
  * ggml-cpu/ggml-cpu.c:1319-1354) as one call: up to CHIP_GROUP_MAX weight matrices with the same K, each with its own

@@ -60,6 +60,8 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void)
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_head_merges(void);
 /* ROPE nodes that ran in the launch of an earlier ROPE with the same positions and parameters (K's with Q's). */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_pairs(void);
+/* Gated FFNs whose four nodes ffn_gate, SILU, ffn_up, MUL (cactus/llama-graph.cpp:562-690) ran as one launch, up to 4 tokens. */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_gated_pairs(void);
 
 #ifdef __cplusplus
 }

@@ -455,15 +455,19 @@ def test_ffn_block_stays_on_the_device(host, orc, n):
     fused_before = blib.lm_ggml_backend_hip_get_fused_pairs()
     blib.lm_ggml_backend_hip_get_quantizers_skipped.restype = C.c_ulonglong
     skipped_before = blib.lm_ggml_backend_hip_get_quantizers_skipped()
+    blib.lm_ggml_backend_hip_get_gated_pairs.restype = C.c_ulonglong
+    gated_before = blib.lm_ggml_backend_hip_get_gated_pairs()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     # norm + weight ran as one kernel (the allocator writes the MUL over its only producer); SiLU and its MUL are not
     # neighbours in the node order (the up projection sits between them): the SiLU waits for that matmul and runs in the
     # MUL's kernel
-    # 5 tokens: the norm leaves its result quantized in the workspace, so neither gate nor up runs the quantizer.
-    # 2 tokens: the two projections run as one launch of the GEMV that quantizes in its prologue (a third join)
-    # Either way SiLU * up leaves its result quantized for ffn_down, which runs no quantizer of its own.
-    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == (2 if n > 4 else 3)
-    assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - skipped_before == (3 if n > 4 else 1)
+    # 5 tokens: the norm leaves its result quantized in the workspace, so neither gate nor up runs the quantizer, and
+    # SiLU * up leaves its result quantized for ffn_down, which runs no quantizer of its own.
+    # 2 tokens: gate, SiLU, up and the MUL run as one launch of the GEMV that quantizes in its prologue (three joins), and
+    # ffn_down's GEMV quantizes in its own prologue.
+    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == (2 if n > 4 else 4)
+    assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - skipped_before == (3 if n > 4 else 0)
+    assert blib.lm_ggml_backend_hip_get_gated_pairs() - gated_before == (0 if n > 4 else 1)
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (cur, up, gate, act, down, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip

@@ -342,6 +342,33 @@ def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
         check_outputs(y2, ref["y"], ref["sum_abs"], "second matrix of the pair, n = %d" % n)
 
 
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N", [(1024, 336), (4096, 1032), (4096, 14336), (256, 8), (2048, 4104)])
+def test_gated_pair_equals_the_pair_and_silu_mul(dev, wt, K, N):
+    """chip_mul_mat_pair_silu_mul (ffn_gate, SILU, ffn_up and their MUL in one launch): bit for bit chip_silu_mul of
+    chip_mul_mat_pair's two outputs, for a few rows, more rows than a pass of the grid takes, and 1, 2 and 4 tokens; declined
+    for other token counts and for row counts that are no multiple of 8 (chip_silu's rule)."""
+    import cactus_amd as ca
+    if (K, N) == (4096, 14336) and wt not in (O.Q4_K, O.Q4_0):
+        pytest.skip("the large shape once per activation family")
+    w1 = quantized_weights(wt, K + N, N, K)
+    w2 = quantized_weights(wt, K + N + 1, N, K)
+    for n in (1, 2, 4):
+        x = common.activations_f32(K + n, n, K)
+        if not dev.lib.chip_mul_mat_pair_silu_mul_supported(wt, K, N, n):
+            assert n * K > 16384
+            continue
+        y1, y2 = dev.mul_mat_pair(wt, w1, w2, x)
+        want = dev.silu_mul(y1, y2)
+        got = dev.mul_mat_pair_silu_mul(wt, w1, w2, x)
+        assert got.tobytes() == want.tobytes(), n
+    assert dev.lib.chip_mul_mat_pair_silu_mul_supported(wt, K, N, 3) == 0
+    assert dev.lib.chip_mul_mat_pair_silu_mul_supported(wt, K, N, 8) == 0
+    assert dev.lib.chip_mul_mat_pair_silu_mul_supported(wt, K, N + 4, 1) == 0
+    d = dev.alloc(4096)
+    assert dev.lib.chip_mul_mat_pair_silu_mul(wt, d.ptr, d.ptr, 16, K, N, d.ptr, K, 3, d.ptr, N, d.ptr, 4096, None) == ca.CHIP_EUNSUPPORTED
+
+
 @pytest.mark.parametrize("wt,K,N", [(O.Q4_K, 4096, 8192), (O.Q4_K, 4096, 14336), (O.Q5_K, 2048, 16400), (O.Q4_K, 14336, 4096)],
                          ids=["q4_K-8192x4096", "q4_K-14336x4096", "q5_K-16400x2048", "q4_K-4096x14336"])
 def test_mul_mat_pair_on_the_matrix_cores(dev, orc, wt, K, N):
