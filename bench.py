@@ -49,6 +49,9 @@ def parse():
                     help="issue every launch of the trace directly instead of replaying a HIP graph, and skip everything that "
                          "replays one (for runs under rocprofv3 --kernel-trace; the host then bounds the step time)")
     ap.add_argument("--no-backend", action="store_true", help="skip the ggml-backend graph timing (a child process)")
+    ap.add_argument("--only-trace", type=int, default=0, metavar="N", choices=(0, 1, 8, 512),
+                    help="run nothing but the trace step at N tokens, every launch issued directly, --warmup + --steps times, and "
+                         "print its time (for a per-kernel table of that step under rocprofv3 --kernel-trace --stats)")
     return ap.parse_args()
 
 
@@ -959,6 +962,13 @@ def main():
     dev = ca.Device(0)
     hip = Hip()
     trace = Trace(dev, hip, np.random.default_rng(5))
+    if args.only_trace:
+        run = trace.step(args.only_trace)
+        ms, per = time_steps(dev, hip, trace.st, run, args.steps, args.warmup)
+        print(json.dumps({"only_trace": args.only_trace, "launches": "eager", "steps": args.steps, "warmup": args.warmup,
+                          "us_per_step": round(ms * 1e3, 1), "step_us": percentiles(per)}))
+        trace.free()
+        return
     value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, trace, args.steps, args.warmup, args.eager)
     extra = {}
     if not args.no_extra:
