@@ -728,16 +728,23 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
             for i, (nm, dst) in enumerate((("wq", q), ("wk", k), ("wv", v))):
                 t_, p_, N_, K_ = W[nm]
                 arr[i] = ca.Mat(t_, p_, dev.row_size(t_, K_), N_, dst.ptr, N_, None, 0)
-            if n <= 4:
-                arr[2].y_f16_t = vc + 2 * (n_kv - n)
-                arr[2].ld16 = kv_size
-            ck(L.chip_mul_mat_group(arr, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
             if l == 0:                                                # one cos / sin table per step, as the backend keeps it
                 ck(L.chip_rope_table(pos.ptr, None, n, hd, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, rope_tab.ptr, st))
-            # RoPE of Q and of K in one launch; K's also stores into the F16 cache, as the backend runs the three nodes
-            ra = ca.RopeOperand(q.ptr, hd, hd * n_head, n_head, q.ptr, hd, hd * n_head, None, 0, 0)
-            rb = ca.RopeOperand(k.ptr, hd, KV, n_head_kv, k.ptr, hd, KV, kc + 2 * KV * (n_kv - n), hd, KV)
-            ck(L.chip_rope_apply_two(C.byref(ra), C.byref(rb), rope_tab.ptr, hd, n, hd, 2, st))
+            if n <= 4:
+                # up to 4 tokens also the RoPE of Q and of K in the projections' epilogue, K's result going to the F16 cache only
+                # (its F32 form has no other reader), as the backend runs the six nodes
+                arr[2].y_f16_t = vc + 2 * (n_kv - n)
+                arr[2].ld16 = kv_size
+                rp = (ca.RopeAfter * 3)()
+                rp[0] = ca.RopeAfter(rope_tab.ptr, hd, hd, 2, q.ptr, hd * n_head, None, 0)
+                rp[1] = ca.RopeAfter(rope_tab.ptr, hd, hd, 2, None, 0, kc + 2 * KV * (n_kv - n), KV)
+                ck(L.chip_mul_mat_group_rope(arr, rp, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
+            else:
+                ck(L.chip_mul_mat_group(arr, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
+                # RoPE of Q and of K in one launch; K's also stores into the F16 cache
+                ra = ca.RopeOperand(q.ptr, hd, hd * n_head, n_head, q.ptr, hd, hd * n_head, None, 0, 0)
+                rb = ca.RopeOperand(k.ptr, hd, KV, n_head_kv, k.ptr, hd, KV, kc + 2 * KV * (n_kv - n), hd, KV)
+                ck(L.chip_rope_apply_two(C.byref(ra), C.byref(rb), rope_tab.ptr, hd, n, hd, 2, st))
             if n > 4:
                 shp = A4(n, KV, 1, 1)
                 ck(L.chip_cpy(v.ptr, ca.F32, shp, A4(KV * 4, 4, 0, 0), vc + 2 * (n_kv - n), ca.F16, shp, A4(2, kv_size * 2, 0, 0), st))

@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_pair_silu_mul", "chip_mul_mat_pair_silu_mul_supported", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_pair_silu_mul", "chip_mul_mat_pair_silu_mul_supported", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_rope", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_rope_apply_two", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
@@ -59,6 +59,12 @@ class RopeOperand(C.Structure):
     """struct chip_rope_operand: one of the two tensors of chip_rope_apply_two."""
     _fields_ = [("x", C.c_void_p), ("ldx1", C.c_int64), ("ldx2", C.c_int64), ("ne1", C.c_int64), ("y", C.c_void_p),
                 ("ldy1", C.c_int64), ("ldy2", C.c_int64), ("y_f16", C.c_void_p), ("ld16_1", C.c_int64), ("ld16_2", C.c_int64)]
+
+
+class RopeAfter(C.Structure):
+    """struct chip_rope_after: the ROPE node behind a member of chip_mul_mat_group_rope."""
+    _fields_ = [("table", C.c_void_p), ("head_dim", C.c_int64), ("n_dims", C.c_int), ("mode", C.c_int), ("y", C.c_void_p),
+                ("ldy", C.c_int64), ("y_f16", C.c_void_p), ("ld16", C.c_int64)]
 
 
 class ChipError(RuntimeError):
@@ -121,6 +127,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_prepare.argtypes = [i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_run.argtypes = [i32, vp, sz, i64, i64, i64, vp, vp, i64, vp]
     L.chip_mul_mat_run_ws.argtypes = [i32, vp, sz, i64, i64, i64, vp, sz, vp, i64, vp]
+    L.chip_mul_mat_group_rope.argtypes = [C.POINTER(Mat), C.POINTER(RopeAfter), i32, i64, vp, i64, i64, vp, sz, vp]
     L.chip_mul_mat_pair.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, vp, i64, vp, sz, vp]
     L.chip_mul_mat_pair_silu_mul.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_pair_silu_mul_supported.argtypes = [i32, i64, i64, i64]
@@ -317,6 +324,55 @@ class Device:
         if dh is not None:
             res.append(dh.download(np.uint16, outs[-1][1] * ld16).reshape(outs[-1][1], ld16))
         return res
+
+    def mul_mat_group_rope(self, members, x, pos, ropes, freq_base=10000.0, check=True):
+        """chip_rope_table + chip_mul_mat_group_rope: members as mul_mat_group; ropes[i] = None or (head_dim, n_dims, mode,
+        wants) with wants a subset of ("f32", "f16").  Returns (rc, list of dicts): a roped member's dict holds "f32" / "f16"
+        arrays [n, N], an unroped member's "y"."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, k = x.shape
+        dx = self.to_device(x)
+        dp = self.to_device(np.ascontiguousarray(pos, np.int32))
+        arr = (Mat * len(members))()
+        rp = (RopeAfter * len(members))()
+        keep, outs = [], []
+        wsz = 0
+        for i, (wt, W) in enumerate(members):
+            W = np.ascontiguousarray(W, np.uint8)
+            N = W.shape[0]
+            dW = self.to_device(W)
+            keep.append(dW)
+            wsz = max(wsz, self.lib.chip_mul_mat_workspace_size_n(wt, k, N, n))
+            if ropes[i] is None:
+                dy = self.alloc(n * N * 4)
+                self.check(self.lib.chip_memset(dy.ptr, 0xFF, n * N * 4, None))
+                arr[i] = Mat(wt, dW.ptr, self.row_size(wt, k), N, dy.ptr, N, None, 0)
+                outs.append({"y": (dy, np.float32)})
+                continue
+            hd, n_dims, mode, wants = ropes[i]
+            dt = self.alloc(n * n_dims * 4)
+            self.check(self.lib.chip_rope_table(dp.ptr, None, n, n_dims, 4096, freq_base, 1.0, 0.0, 1.0, 32.0, 1.0, dt.ptr, None))
+            keep.append(dt)
+            o = {}
+            if "f32" in wants:
+                o["f32"] = (self.alloc(n * N * 4), np.float32)
+                self.check(self.lib.chip_memset(o["f32"][0].ptr, 0xFF, n * N * 4, None))
+            if "f16" in wants:
+                o["f16"] = (self.alloc(n * N * 2), np.float16)
+                self.check(self.lib.chip_memset(o["f16"][0].ptr, 0xFF, n * N * 2, None))
+            arr[i] = Mat(wt, dW.ptr, self.row_size(wt, k), N, None, 0, None, 0)
+            rp[i] = RopeAfter(dt.ptr, hd, n_dims, mode, o["f32"][0].ptr if "f32" in o else None, N, o["f16"][0].ptr if "f16" in o else None, N)
+            outs.append(o)
+        ws = self.alloc(max(wsz, 16))
+        rc = self.lib.chip_mul_mat_group_rope(arr, rp, len(members), k, dx.ptr, k, n, ws.ptr, wsz, None)
+        if check:
+            self.check(rc)
+        self.sync()
+        res = []
+        for (wt, W), o in zip(members, outs):
+            N = np.asarray(W).shape[0]
+            res.append({key: buf.download(dt_, n * N).reshape(n, N) for key, (buf, dt_) in o.items()})
+        return rc, res
 
     def mul_mat_pair(self, wtype, W1, W2, x):
         """Two matrices of one shape on the same activation (chip_mul_mat_pair): returns (y1, y2), each fp32 [n, N]."""

@@ -501,11 +501,13 @@ int chip_mul_mat_pair_silu_mul(int type, const void *W1, const void *W2, size_t 
                                                   act_stride(chip_vec_dot_type(type), K), y, ldy, lim, (hipStream_t)stream));
 }
 
+static int rope_dims_checked(int64_t ne0, int64_t ne1, int64_t ne2, int n_dims, int mode);
+
 // Several matmuls on one activation (wq / wk / wv).  Up to 4 tokens, members of one family: one launch of the
 // prologue-quantizing GEMV over all members; otherwise one quantizer and each member on its usual path.
 // what chip_mul_mat_group and chip_mul_mat_group_run share: x == nullptr says the workspace already holds the rows
 static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
-                         size_t workspace_bytes, void *stream) {
+                         size_t workspace_bytes, void *stream, const chip_rope_after *ropes = nullptr) {
     if (count < 0 || n < 0) return CHIP_EINVAL;
     if (count == 0 || n == 0) return CHIP_OK;
     if (!mats || count > CHIP_GROUP_MAX) return CHIP_EINVAL;
@@ -519,9 +521,18 @@ static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float
         if (!(a == at || ((a == T_Q8_0 || a == T_Q8_1) && (at == T_Q8_0 || at == T_Q8_1)))) return CHIP_EUNSUPPORTED;
         if (m.N < 0) return CHIP_EINVAL;
         if (m.N == 0) continue;
-        if (!m.W || !m.y || m.ldy < m.N || (((uintptr_t)m.y) & 3) != 0) return CHIP_EINVAL;
+        const bool roped = ropes && ropes[i].table;                    // the member's own result is then not stored
+        if (!m.W || (!roped && (!m.y || m.ldy < m.N || (((uintptr_t)m.y) & 3) != 0))) return CHIP_EINVAL;
         if (!weights_aligned(m.type, m.W, m.nb01, K) || m.nb01 < chip_row_size(m.type, K)) return CHIP_EINVAL;
         if (m.y_f16_t && (m.ld16 < n || (((uintptr_t)m.y_f16_t) & 1) != 0)) return CHIP_EINVAL;
+        if (roped) {
+            const chip_rope_after &r = ropes[i];
+            if (int rc = rope_dims_checked(r.head_dim, m.N / (r.head_dim > 0 ? r.head_dim : 1), n, r.n_dims, r.mode); rc != CHIP_OK) return rc;
+            if (r.head_dim <= 0 || (r.head_dim & 1) || m.N % r.head_dim != 0 || r.head_dim > 0x7fffffff) return CHIP_EUNSUPPORTED;
+            if ((!r.y && !r.y_f16) || m.y_f16_t || (((uintptr_t)r.table) & 3) != 0) return CHIP_EINVAL;
+            if (r.y && (r.ldy < m.N || (((uintptr_t)r.y) & 3) != 0)) return CHIP_EINVAL;
+            if (r.y_f16 && (r.ld16 < m.N || (((uintptr_t)r.y_f16) & 1) != 0)) return CHIP_EINVAL;
+        }
         const size_t w = chip_mul_mat_workspace_size(m.type, K, n);
         if (w > need) need = w;
     }
@@ -533,10 +544,25 @@ static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float
     if (int rc = current_limits(lim); rc) return rc;
     GroupMat gm[GROUP_MAX];
     int live = 0;
+    bool any_rope = false;
     for (int i = 0; i < count; i++)
-        if (mats[i].N > 0)
-            gm[live++] = GroupMat{mats[i].type, mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].y_f16_t, mats[i].ld16};
+        if (mats[i].N > 0) {
+            gm[live] = GroupMat{mats[i].type, mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].y_f16_t, mats[i].ld16};
+            if (ropes && ropes[i].table) {
+                const chip_rope_after &r = ropes[i];
+                gm[live].y = r.y;
+                gm[live].ldy = r.y ? r.ldy : 0;
+                gm[live].rope = RopeEpilogue{r.table, (int)r.head_dim, r.n_dims, (r.mode & 2) != 0, r.y != nullptr, r.y_f16, r.y_f16 ? r.ld16 : 0};
+                any_rope = true;
+            }
+            live++;
+        }
     if (live == 0) return CHIP_OK;
+    if (any_rope) {                                                      // only the one-launch form has the epilogue
+        if (prepared || n > 4 || !gemv_group_applicable(gm, live, K, (int)n, lim, false) || gemv_group_family(gm[0].wtype) == 2)
+            return CHIP_EUNSUPPORTED;
+        return hip_rc(launch_gemv_group(gm, live, K, x, ldx, (int)n, workspace, act_stride(at, K), lim, (hipStream_t)stream, false));
+    }
     const size_t stride = act_stride(at, K);
     hipStream_t st = (hipStream_t)stream;
     // Up to 4 tokens.  One member, or two of one type, shape and row stride, take the single-matrix kernel (it keeps more
@@ -587,6 +613,11 @@ int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *
                        size_t workspace_bytes, void *stream) {
     if (count > 0 && n > 0 && !x) return CHIP_EINVAL;
     return mul_mat_group(mats, count, K, x, ldx, n, workspace, workspace_bytes, stream);
+}
+int chip_mul_mat_group_rope(const chip_mat *mats, const chip_rope_after *ropes, int count, int64_t K, const float *x, int64_t ldx,
+                            int64_t n, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!ropes || (count > 0 && n > 0 && !x)) return CHIP_EINVAL;
+    return mul_mat_group(mats, count, K, x, ldx, n, workspace, workspace_bytes, stream, ropes);
 }
 int chip_mul_mat_group_run(const chip_mat *mats, int count, int64_t K, int64_t n, void *workspace, size_t workspace_bytes, void *stream) {
     return mul_mat_group(mats, count, K, nullptr, 0, n, workspace, workspace_bytes, stream);

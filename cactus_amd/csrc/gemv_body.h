@@ -895,12 +895,14 @@ __device__ __forceinline__ GridPart whole_grid() { return GridPart{(int64_t)bloc
 struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; int gated; };
 constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0, 0};
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false, bool GATED = false>
+
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false, bool GATED = false, bool ROPED = false>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                           const float *__restrict__ x, int64_t ldx,
                                           uint8_t *__restrict__ ws, size_t ws_stride,
                                           float *__restrict__ y, int64_t ldy, const SecondMatrix sec,
-                                          const GridPart gp) {
+                                          const GridPart gp, const RopeEpilogue rope = kNoRope) {
+    static_assert(!ROPED || (R == 1 && !GATED && !PHASED && FUSEQ), "the pair walk of the rotated rows takes one row per step");
     using T = Traits<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     static_assert(DEPTH == 1, "one step of weight loads is in flight beyond the one being computed");
@@ -912,8 +914,17 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     const int64_t nwaves = gp.blocks * (WGS / 64);
     // gated: tile T is row tile T / 2 of matrix T % 2; a wave walks 2 * wave, 2 * wave + 1, 2 * (wave + nwaves), ...
     constexpr bool gated = GATED;                      // a kernel of its own: sec.gated picks it in the launcher
+    // ROPED: tile T is half T % 2 of rotated pair T / 2; a wave walks 2 * wave, 2 * wave + 1, 2 * (wave + nwaves), ...
+    constexpr bool paired = GATED || ROPED;
     const int64_t tiles = gated ? 2 * ceil_div(sec.n_first, (int64_t)R) : ceil_div(N, R);
-    const int64_t first_tile = gated ? 2 * wave : wave;
+    const int64_t first_tile = paired ? 2 * wave : wave;
+    [[maybe_unused]] auto rope_row = [&](int64_t T) -> int64_t {        // the row of tile T (32-bit division: wave-uniform, once per tile)
+        const uint32_t p = (uint32_t)(T >> 1), hp = (uint32_t)rope.head_dim >> 1, rot = (uint32_t)rope.n_dims >> 1;
+        const uint32_t h = p / hp, j = p - h * hp;
+        const uint32_t ra = j < rot ? (rope.neox ? j : 2 * j) : (uint32_t)rope.n_dims + 2 * (j - rot);
+        const uint32_t step = (j < rot && rope.neox) ? rot : 1u;
+        return (int64_t)h * rope.head_dim + ra + (uint32_t)(T & 1) * step;
+    };
 
     // A wave walks the steps (tile, it) = (wave, 0), (wave, 1), ..., (wave + nwaves, 0), ...; while it computes one step
     // the loads of the next are in flight.  Measured and dropped: rings of two and three steps (3-8 % slower as a loop; the
@@ -926,7 +937,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     auto after = [&](const Step &s) {
         Step n = s;
         if (s.it + 1 == NI) {
-            n.tile = !gated ? s.tile + nwaves : ((s.tile & 1) ? s.tile + 2 * nwaves - 1 : s.tile + 1);
+            n.tile = !paired ? s.tile + nwaves : ((s.tile & 1) ? s.tile + 2 * nwaves - 1 : s.tile + 1);
             n.it = 0;
         } else n.it = s.it + 1;
         n.have = s.have && n.tile < tiles;
@@ -945,6 +956,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
             for (int r = 0; r < R; r++) {
                 int64_t row = s.have ? min(s.tile * R + r, N - 1) : (int64_t)0;
                 if (gated) row = s.have ? min((s.tile >> 1) * R + r, sec.n_first - 1) + (s.tile & 1) * sec.n_first : (int64_t)0;
+                if constexpr (ROPED) row = s.have ? rope_row(s.tile) : (int64_t)0;
                 T::load_raw(set[r], W + (size_t)row * nb01 + (row >= sec.n_first ? sec.w_off : (int64_t)0), u);
             }
         }
@@ -970,8 +982,17 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     } else if constexpr (FUSEQ) {
         XRegs<NTOK, WGS> xr;
         xload<WT, NTOK, WGS>(xr, x, ldx, K);
+        [[maybe_unused]] float rope_cs = 0.f;                           // this thread's entry of the tokens' cos / sin table
+        if constexpr (ROPED) {
+            if ((int)threadIdx.x < NTOK * rope.n_dims) rope_cs = rope.table[threadIdx.x];
+        }
         load_step(ring, s0, true);
         quantize_into_image<WT, NTOK, WGS>(xr, lds, img, NI, K, ws, ws_stride, gp.writes_workspace);
+        if constexpr (ROPED) {                                          // behind the image: [token][cos | sin]
+            float *tab = reinterpret_cast<float *>(lds + (size_t)NTOK * img);
+            if ((int)threadIdx.x < NTOK * rope.n_dims) tab[threadIdx.x] = rope_cs;
+            for (int i = WGS + (int)threadIdx.x; i < NTOK * rope.n_dims; i += WGS) tab[i] = rope.table[i];
+        }
     } else {
         StageRegs<WT, NTOK> sr;
         stage_issue<WT, NTOK, WGS>(sr, NI, units, K, ws, ws_stride);
@@ -990,6 +1011,29 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
 #pragma unroll
         for (int t = 0; t < NTOK; t++) { acc[r][t] = 0.f; res[r][t] = 0.f; }
     auto flush = [&](int count) {
+        if constexpr (ROPED) {                           // lanes 2k and 2k + 1 hold the two values of one rotated pair
+            const float *tab = reinterpret_cast<const float *>(lds + (size_t)NTOK * img);
+            const int row = res_row, rowb = __shfl_down(res_row, 1);
+            const uint32_t off = (uint32_t)row % (uint32_t)rope.head_dim;
+            const bool mine = lane < count && !(lane & 1) && row < N;
+            const bool rotated = off < (uint32_t)rope.n_dims;
+            const uint32_t j = rope.neox ? off : off >> 1;
+#pragma unroll
+            for (int t = 0; t < NTOK; t++) {
+                const float x0 = res[0][t], x1 = __shfl_down(res[0][t], 1);
+                if (mine) {
+                    float y0 = x0, y1 = x1;
+                    if (rotated) {
+                        const float c = tab[t * rope.n_dims + j], sn = tab[t * rope.n_dims + (rope.n_dims >> 1) + j];
+                        y0 = x0 * c - x1 * sn;
+                        y1 = x0 * sn + x1 * c;
+                    }
+                    if (rope.write_f32) { y[(int64_t)t * ldy + row] = y0; y[(int64_t)t * ldy + rowb] = y1; }
+                    if (rope.h16) { rope.h16[(int64_t)t * rope.h16_ld + row] = f2h_rne(y0); rope.h16[(int64_t)t * rope.h16_ld + rowb] = f2h_rne(y1); }
+                }
+            }
+            return;
+        }
         if (gated) {                                     // lanes 2j and 2j + 1 hold the two projections of one row tile
 #pragma unroll
             for (int r = 0; r < R; r++) {
@@ -1044,7 +1088,8 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
                     res[r][t] = lane == nres ? sum : res[r][t];
                     acc[r][t] = 0.f;
                 }
-            res_row = lane == nres ? (int)((gated ? s.tile >> 1 : s.tile) * R) : res_row;
+            if constexpr (ROPED) res_row = lane == nres ? (int)rope_row(s.tile) : res_row;
+            else res_row = lane == nres ? (int)((gated ? s.tile >> 1 : s.tile) * R) : res_row;
             nres++;
         }
     };

@@ -14,20 +14,30 @@ namespace {
 struct GroupKernelMat {
     const uint8_t *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld;
     int wtype; int first_block;
+    RopeEpilogue rope;                                  // table != nullptr: the member's ROPE node runs in its epilogue
 };
 struct GroupKernelArgs { GroupKernelMat m[GROUP_MAX]; int count; };
 
-template <int WT, int NTOK, int WGS, bool FUSEQ, int DEPTH>
+template <int WT, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE>
 __device__ __forceinline__ void run_member(const GroupKernelMat &m, int64_t K, const float *x, int64_t ldx, uint8_t *ws,
                                            size_t ws_stride, const GridPart gp) {
     const SecondMatrix sec{INT64_MAX, 0, 0, m.t16, m.t16_ld};
+    if constexpr (ROPE && FUSEQ) {
+        if (m.rope.table) {                                             // uniform over the workgroup; one row per step (pairs)
+            gemv_body<WT, NTOK, 1, WGS, FUSEQ, DEPTH, false, false, true>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, kNoSecond,
+                                                                            gp, m.rope);
+            return;
+        }
+    }
     gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
 }
 
 // FAMILY 0: K-quants (Q8_K activations); 1: 32-value blocks (Q8_0 / Q8_1 planes); 2: F16.
 // FUSEQ: the workgroups quantize the fp32 rows x themselves; otherwise the workspace already holds the quantized rows
 // (written by chip_mul_mat_prepare or by the kernel that produced the activations) and is only read.
-template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH>
+// ROPE: a kernel of its own for groups in which a member's ROPE node runs in its epilogue (gemv_body.h: ROPED), so that the
+// plain group kernel keeps its registers.
+template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE = false>
 __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs ga, int64_t K, const float *__restrict__ x,
                                                          int64_t ldx, uint8_t *__restrict__ ws, size_t ws_stride) {
     int i = 0;
@@ -39,21 +49,21 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
     const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), FUSEQ && blockIdx.x == 0};
     if constexpr (FAMILY == 0) {
         switch (m.wtype) {                                              // uniform over the workgroup
-            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else if constexpr (FAMILY == 1) {
         switch (m.wtype) {
-            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
-            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else {
-        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH>(m, K, x, ldx, ws, ws_stride, gp);
+        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp);
     }
 }
 
@@ -74,10 +84,10 @@ size_t image_bytes(int wtype, int64_t K) {
 }
 int rows_per_step(int wtype) { return wtype == T_Q4_0 ? RowsPerWave<T_Q4_0>::R : 1; }
 
-template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH>
+template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE = false>
 hipError_t launch_depth(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
                         size_t lds_bytes, const DeviceLimits &lim, hipStream_t st) {
-    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, FUSEQ, DEPTH>;
+    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, FUSEQ, DEPTH, ROPE>;
     static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(WGS), lds_bytes, st, ga, K, x, ldx, (uint8_t *)ws, ws_stride);
@@ -85,25 +95,31 @@ hipError_t launch_depth(const GroupKernelArgs &ga, int grid, int64_t K, const fl
 }
 template <int FAMILY, int NTOK, int WGS>
 hipError_t launch_cfg(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
-                      size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared) {
+                      size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared, bool rope) {
+    if (rope) {
+        if constexpr (FAMILY != 2) {
+            if (!prepared) return launch_depth<FAMILY, NTOK, WGS, true, GEMV_DEPTH, true>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
+        }
+        return hipErrorInvalidValue;
+    }
     return prepared ? launch_depth<FAMILY, NTOK, WGS, false, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st)
                     : launch_depth<FAMILY, NTOK, WGS, true, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
 }
 template <int FAMILY, int NTOK>
 hipError_t launch_wgs(int wgs, const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws,
-                      size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared) {
-    return wgs == 1024 ? launch_cfg<FAMILY, NTOK, 1024>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared)
-                       : launch_cfg<FAMILY, NTOK, 512>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+                      size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared, bool rope) {
+    return wgs == 1024 ? launch_cfg<FAMILY, NTOK, 1024>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope)
+                       : launch_cfg<FAMILY, NTOK, 512>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
 }
 template <int FAMILY>
 hipError_t launch_ntok(int n, int wgs, const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws,
-                       size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared) {
+                       size_t ws_stride, size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared, bool rope) {
     switch (n) {
-        case 1: return launch_wgs<FAMILY, 1>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
-        case 2: return launch_wgs<FAMILY, 2>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
-        case 4: return launch_wgs<FAMILY, 4>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        case 1: return launch_wgs<FAMILY, 1>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
+        case 2: return launch_wgs<FAMILY, 2>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
+        case 4: return launch_wgs<FAMILY, 4>(wgs, ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         case 8:                                                          // over prepared rows only
-            if (!prepared) return hipErrorInvalidValue;
+            if (!prepared || rope) return hipErrorInvalidValue;
             return wgs == 1024 ? launch_depth<FAMILY, 8, 1024, false, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st)
                                : launch_depth<FAMILY, 8, 512, false, GEMV_DEPTH>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
         default: return hipErrorInvalidValue;
@@ -159,7 +175,20 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
         cost[i] = (double)mats[i].N * (double)mats[i].nb01;              // bytes to stream
         total_cost += cost[i];
     }
-    const size_t lds_bytes = (size_t)n * img;
+    // members whose ROPE node runs in their epilogue: one row per step (pairs of rows per wave), the cos / sin table behind the image
+    bool rope = false;
+    int rope_dims = 0;
+    for (int i = 0; i < count; i++) {
+        const RopeEpilogue &r = mats[i].rope;
+        if (!r.table) continue;
+        if (prepared || fam == 2 || r.head_dim <= 0 || (r.head_dim & 1) || r.n_dims <= 0 || (r.n_dims & 1) || r.n_dims > r.head_dim ||
+            mats[i].N % r.head_dim != 0 || (!r.write_f32 && !r.h16) || mats[i].t16)
+            return hipErrorInvalidValue;
+        rope = true;
+        if (r.n_dims > rope_dims) rope_dims = r.n_dims;
+        tiles += mats[i].N - ceil_div(mats[i].N, (int64_t)rows_per_step(mats[i].wtype));
+    }
+    const size_t lds_bytes = (size_t)n * img + (size_t)n * rope_dims * sizeof(float);
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     // As the single-matrix launcher: a persistent grid; one 16-wave workgroup per CU while every wave gets at most a
     // couple of tiles (the prologue is then most of the kernel and is paid once per CU), else two 8-wave workgroups.
@@ -197,13 +226,13 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
     int first = 0;
     for (int i = 0; i < count; i++) {
         ga.m[i] = GroupKernelMat{(const uint8_t *)mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].t16,
-                                 mats[i].t16_ld, mats[i].wtype, first};
+                                 mats[i].t16_ld, mats[i].wtype, first, mats[i].rope};
         first += blocks[i];
     }
     switch (fam) {
-        case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
-        case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
-        default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared);
+        case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
+        case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
+        default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
     }
 }
 

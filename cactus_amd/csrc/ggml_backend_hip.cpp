@@ -27,7 +27,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0}, g_rope_epilogues{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -446,6 +446,37 @@ bool attn_side_shape_ok(const lm_ggml_tensor *op) {
     }
 }
 // store: the F32 -> F16 CPY of the RoPE's result into a dense destination (the K cache store), run in the RoPE's kernel
+// The cos / sin table of a ROPE node (positions, frequency factors and parameters; built by the first node of a
+// graph_compute call that needs it, kept until a node with another key comes): leaves it in c->rope_table.
+int ensure_rope_table(backend_ctx *c, const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *a = op->src[0], *pos = op->src[1], *ff = op->src[2];
+    float f[6];
+    std::memcpy(f, op->op_params + 5, sizeof(f));        // freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow
+    rope_table_key k = {pos->data, ff ? ff->data : nullptr, a->ne[2], {}, true};
+    k.params[0] = op->op_params[1];
+    std::memcpy(k.params + 1, op->op_params + 3, 8 * sizeof(int32_t));
+    const size_t need = (size_t)a->ne[2] * (size_t)op->op_params[1] * sizeof(float);
+    const bool have = c->rope_key.valid && c->rope_key.pos == k.pos && c->rope_key.ff == k.ff && c->rope_key.ne2 == k.ne2 &&
+                      std::memcmp(c->rope_key.params, k.params, sizeof(k.params)) == 0;
+    if (have) return CHIP_OK;
+    if (need > c->rope_table_bytes) {
+        chip_stream_synchronize(c->stream);          // earlier nodes of this call may still read the old table
+        chip_free(c->rope_table);
+        c->rope_table = nullptr;
+        c->rope_table_bytes = 0;
+        void *p = nullptr;
+        if (chip_malloc(&p, need + need / 2) != CHIP_OK) return CHIP_ENOMEM;
+        c->rope_table = (float *)p;
+        c->rope_table_bytes = need + need / 2;
+    }
+    const int rc = chip_rope_table((const int32_t *)pos->data, ff ? (const float *)ff->data : nullptr, a->ne[2], op->op_params[1],
+                                   op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], c->rope_table, c->stream);
+    if (rc != CHIP_OK) return rc;
+    c->rope_key = k;
+    g_rope_tables++;
+    return CHIP_OK;
+}
+
 // A second ROPE node run in the first one's launch (K's with Q's): its input, the CPY of its result into the F16 cache that
 // runs with it (or null), and whether its own F32 result is written at all.
 struct rope_partner {
@@ -474,31 +505,7 @@ int run_attn_side(backend_ctx *c, lm_ggml_tensor *op, const lm_ggml_tensor *stor
             float f[6];
             std::memcpy(f, op->op_params + 5, sizeof(f));        // freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow
             if (fusion_enabled()) {
-                // the table of this call, built by its first ROPE node (or by the first one with other parameters)
-                rope_table_key k = {pos->data, ff ? ff->data : nullptr, a->ne[2], {}, true};
-                k.params[0] = op->op_params[1];
-                std::memcpy(k.params + 1, op->op_params + 3, 8 * sizeof(int32_t));
-                const size_t need = (size_t)a->ne[2] * (size_t)op->op_params[1] * sizeof(float);
-                bool have = c->rope_key.valid && c->rope_key.pos == k.pos && c->rope_key.ff == k.ff && c->rope_key.ne2 == k.ne2 &&
-                            std::memcmp(c->rope_key.params, k.params, sizeof(k.params)) == 0;
-                if (!have) {
-                    if (need > c->rope_table_bytes) {
-                        chip_stream_synchronize(c->stream);          // earlier nodes of this call may still read the old table
-                        chip_free(c->rope_table);
-                        c->rope_table = nullptr;
-                        c->rope_table_bytes = 0;
-                        void *p = nullptr;
-                        if (chip_malloc(&p, need + need / 2) != CHIP_OK) return CHIP_ENOMEM;
-                        c->rope_table = (float *)p;
-                        c->rope_table_bytes = need + need / 2;
-                    }
-                    const int rc = chip_rope_table((const int32_t *)pos->data, ff ? (const float *)ff->data : nullptr, a->ne[2],
-                                                   op->op_params[1], op->op_params[4], f[0], f[1], f[2], f[3], f[4], f[5], c->rope_table,
-                                                   c->stream);
-                    if (rc != CHIP_OK) return rc;
-                    c->rope_key = k;
-                    g_rope_tables++;
-                }
+                if (const int trc = ensure_rope_table(c, op); trc != CHIP_OK) return trc;
                 if (partner) {
                     const lm_ggml_tensor *pb = partner->op, *ab = pb->src[0];
                     chip_rope_operand oa = {xa, (int64_t)(a->nb[1] / 4), (int64_t)(a->nb[2] / 4), a->ne[1], (float *)op->data,
@@ -919,6 +926,39 @@ int rope_partner_index(const lm_ggml_cgraph *g, int i, graph_reads &reads, F ran
     return -1;
 }
 
+// The ROPE node behind a projection that runs in a group at node i, to be run in that projection's epilogue
+// (chip_mul_mat_group_rope): the projection is read by nothing else, its rows are the ROPE's heads as they lie, and whatever
+// the ROPE writes at node i's place is not in use there.  Returns the ROPE's index and fills rope (the table pointer is left
+// to the caller), store_index (the cache store that runs with it, or -1); -1: no such node.
+int rope_epilogue_index(const lm_ggml_cgraph *g, int i, int member, int64_t n, graph_reads &reads, chip_rope_after &rope, int &store_index) {
+    const lm_ggml_tensor *mm = g->nodes[member];
+    const int nx = next_compute_node(g, member);
+    if (nx < 0 || nx > member + ROPE_LOOKAHEAD) return -1;
+    const lm_ggml_tensor *rp = g->nodes[nx], *in = rp->src[0];
+    if (rp->op != LM_GGML_OP_ROPE || !in || !attn_side_shape_ok(rp) || (mm->flags & LM_GGML_TENSOR_FLAG_OUTPUT)) return -1;
+    if ((in != mm && in->view_src != mm) || in->data != mm->data || reads.readers_of(g, mm) != 1) return -1;
+    const int64_t hd = in->ne[0], N = mm->ne[0];
+    if (hd <= 0 || (hd & 1) || in->ne[1] * hd != N || in->ne[2] != n || in->ne[3] != 1 || mm->nb[1] != (size_t)N * 4) return -1;
+    if (in->nb[1] != (size_t)hd * 4 || in->nb[2] != (size_t)N * 4 || rp->nb[1] != (size_t)hd * 4 || rp->nb[2] != (size_t)N * 4) return -1;
+    store_index = rope_store_index(g, nx, i);
+    const lm_ggml_tensor *store = store_index >= 0 ? g->nodes[store_index] : nullptr;
+    const bool write_f32 = !(store && !(rp->flags & LM_GGML_TENSOR_FLAG_OUTPUT) && reads.readers_of(g, rp) == 1);
+    if (write_f32) {
+        for (int m = i; m < nx; m++) {                       // the ROPE's own memory, between node i and its node
+            const lm_ggml_tensor *t = g->nodes[m];
+            if (is_view_op(t->op) || t == mm) continue;      // (over the projection it replaces it may lie: that is not stored)
+            if (!ranges_apart(t, rp)) return -1;
+            for (int k = 0; k < LM_GGML_MAX_SRC; k++) {
+                const lm_ggml_tensor *sr = t->src[k];
+                if (sr && sr != mm && sr->view_src != mm && !ranges_apart(sr, rp)) return -1;
+            }
+        }
+    }
+    rope = chip_rope_after{nullptr, hd, rp->op_params[1], rp->op_params[2], write_f32 ? (float *)rp->data : nullptr, N,
+                           store ? (uint16_t *)store->data : nullptr, N};
+    return nx;
+}
+
 int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     backend_ctx *c = (backend_ctx *)backend->context;
     c->rope_key.valid = false;                        // positions may have changed since the last call
@@ -937,6 +977,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     const float *rope_slot_src = nullptr;
     graph_reads reads;
     int rope_done = -1, rope_done_store = -1;         // a ROPE node (and its cache store) that already ran in an earlier ROPE's launch
+    int roped_early[CHIP_GROUP_MAX] = {-1, -1, -1, -1};   // ROPE nodes that ran in the epilogue of their projection
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
@@ -1030,6 +1071,12 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             continue;
         }
         if (i == rope_done) { rope_done = -1; continue; }
+        {
+            bool done = false;
+            for (int &slot : roped_early)
+                if (slot == i) { slot = -1; done = true; }
+            if (done) continue;
+        }
         if (i == rope_done_store) { rope_done_store = -1; continue; }
         if (is_attn_side_op(node->op) && attn_side_shape_ok(node)) {
             const lm_ggml_tensor *store = nullptr;
@@ -1230,12 +1277,86 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 }
             }
             if (fits) {
+                // ROPE nodes behind members, run in the members' epilogue (up to 4 tokens, fp32 rows)
+                chip_rope_after ropes[CHIP_GROUP_MAX] = {};
+                int rope_node[CHIP_GROUP_MAX] = {-1, -1, -1, -1}, rope_store[CHIP_GROUP_MAX] = {-1, -1, -1, -1};
+                bool any_rope = false;
+                int free_store_slots = 0;
+                for (int slot : stored_early) free_store_slots += slot < 0;
+                if (n <= 4 && rope_done < 0 && rope_done_store < 0) {
+                    for (int k = 0; k < n_members; k++) {
+                        if (stored[k]) continue;
+                        int st = -1;
+                        const int nx = rope_epilogue_index(cgraph, i, members[k], n, reads, ropes[k], st);
+                        if (nx < 0) continue;
+                        if (st >= 0 && free_store_slots == 0) { ropes[k] = chip_rope_after{}; continue; }
+                        if (ensure_rope_table(c, cgraph->nodes[nx]) != CHIP_OK) { ropes[k] = chip_rope_after{}; continue; }
+                        // one table serves the launch: a member whose ROPE has another key (positions, parameters) stays as it is
+                        bool same_key = true;
+                        for (int m = 0; m < k; m++)
+                            if (rope_node[m] >= 0 && (cgraph->nodes[rope_node[m]]->src[1] != cgraph->nodes[nx]->src[1] ||
+                                                      cgraph->nodes[rope_node[m]]->src[2] != cgraph->nodes[nx]->src[2] ||
+                                                      std::memcmp(cgraph->nodes[rope_node[m]]->op_params, cgraph->nodes[nx]->op_params,
+                                                                  sizeof(node->op_params)) != 0))
+                                same_key = false;
+                        if (!same_key) { ropes[k] = chip_rope_after{}; continue; }
+                        ropes[k].table = c->rope_table;
+                        rope_node[k] = nx;
+                        rope_store[k] = st;
+                        if (st >= 0) free_store_slots--;
+                        any_rope = true;
+                    }
+                }
+                quantized_key &q = c->quantized;
+                const int vt = chip_vec_dot_type(w->type);
+                rc = CHIP_EUNSUPPORTED;
+                if (any_rope) {
+                    q.valid = false;
+                    rc = chip_mul_mat_group_rope(mats, ropes, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                    if (rc == CHIP_EUNSUPPORTED) {               // not a one-launch group: the ROPE nodes run at their own places
+                        any_rope = false;
+                        for (int k = 0; k < n_members; k++) { ropes[k] = chip_rope_after{}; rope_node[k] = rope_store[k] = -1; }
+                    }
+                }
+                if (!any_rope) {
+                    // more than 4 tokens: the workspace holds x's quantized rows afterwards, or already does (the norm in front
+                    // left them there, or an earlier matmul of the same input)
+                    const bool have_rows = n > 4 && q.valid && q.src == x->data && q.K == K && q.n == n && q.ldx == ldx && q.vec_dot_type == vt;
+                    if (have_rows) {
+                        rc = chip_mul_mat_group_run(mats, n_members, K, n, c->workspace, c->workspace_size, c->stream);
+                        g_quantizers_skipped++;
+                    } else {
+                        q.valid = false;
+                        rc = chip_mul_mat_group(mats, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                        if (rc == CHIP_OK && n > 4) q = quantized_key{true, x->data, lm_ggml_nbytes(x), K, n, ldx, vt};
+                    }
+                }
+                if (rc != CHIP_OK) {
+                    HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT group of %d at %s failed: %s\n", __func__, n_members, node->name,
+                            chip_error_string(rc));
+                    return LM_GGML_STATUS_FAILED;
+                }
+                for (int k = 0; k < n_members; k++) {
+                    if (rope_node[k] < 0) continue;               // this member's ROPE (and its cache store) ran with it
+                    lm_ggml_tensor *rp = cgraph->nodes[rope_node[k]];
+                    writes(rp);
+                    roped_early[k] = rope_node[k];
+                    if (rope_store[k] >= 0) {
+                        remember_store(rope_store[k]);
+                        writes(cgraph->nodes[rope_store[k]]);
+                        g_elementwise_nodes++;
+                        g_fused_pairs++;
+                    }
+                    g_elementwise_nodes++;
+                    g_fused_pairs++;
+                    g_rope_epilogues++;
+                }
                 for (int k = 1; k < n_members; k++) {
                     lm_ggml_tensor *mm = cgraph->nodes[members[k]];
                     writes(mm);
                     grouped[k] = members[k];
                     grouped_copy[k] = nullptr;
-                    if (!aliased[k]) continue;
+                    if (!aliased[k] || rope_node[k] >= 0) continue;
                     // What becomes of a result in a scratch slot.  Its only reader was the cache store that ran with it: nothing.
                     // Its only reader is the ROPE that follows it (views aside) and takes its rows as they lie: that ROPE reads
                     // the slot.  Otherwise it is copied to its own memory when the loop gets to its node.
@@ -1253,24 +1374,6 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                         continue;
                     }
                     grouped_copy[k] = mats[k].y;
-                }
-                // more than 4 tokens: the workspace holds x's quantized rows afterwards, or already does (the norm in front
-                // left them there, or an earlier matmul of the same input)
-                quantized_key &q = c->quantized;
-                const int vt = chip_vec_dot_type(w->type);
-                const bool have_rows = n > 4 && q.valid && q.src == x->data && q.K == K && q.n == n && q.ldx == ldx && q.vec_dot_type == vt;
-                if (have_rows) {
-                    rc = chip_mul_mat_group_run(mats, n_members, K, n, c->workspace, c->workspace_size, c->stream);
-                    g_quantizers_skipped++;
-                } else {
-                    q.valid = false;
-                    rc = chip_mul_mat_group(mats, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
-                    if (rc == CHIP_OK && n > 4) q = quantized_key{true, x->data, lm_ggml_nbytes(x), K, n, ldx, vt};
-                }
-                if (rc != CHIP_OK) {
-                    HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: MUL_MAT group of %d at %s failed: %s\n", __func__, n_members, node->name,
-                            chip_error_string(rc));
-                    return LM_GGML_STATUS_FAILED;
                 }
                 g_mul_mat_nodes += n_members;
                 g_grouped_matmuls += n_members;
@@ -1506,5 +1609,6 @@ unsigned long long lm_ggml_backend_hip_get_grouped_matmuls(void) { return g_grou
 unsigned long long lm_ggml_backend_hip_get_head_merges(void) { return g_head_merges.load(); }
 unsigned long long lm_ggml_backend_hip_get_rope_pairs(void) { return g_rope_pairs.load(); }
 unsigned long long lm_ggml_backend_hip_get_gated_pairs(void) { return g_gated_pairs.load(); }
+unsigned long long lm_ggml_backend_hip_get_rope_epilogues(void) { return g_rope_epilogues.load(); }
 
 }  // extern "C"

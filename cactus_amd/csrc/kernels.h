@@ -159,8 +159,19 @@ hipError_t launch_gemv_fused_pair_silu_mul(int wtype, const void *W1, const void
 // gemv_group.hip: up to GROUP_MAX matrices that read the same activation rows in one launch of the prologue-quantizing
 // GEMV (members of one family: K-quants, 32-value block types, or F16).  t16: optional transposed fp16 copy of a member's
 // output, as launch_gemv_fused_store_t.
+// The ROPE node that follows a projection (reference llama-model.cpp build_llama: lm_ggml_rope_ext on Qcur and on Kcur;
+// lm_ggml_compute_forward_rope_f32, ggml-cpu/ops.cpp:5178-5361, modes 0 and NEOX) run in the projection's kernel (ROPED): the
+// rows are heads of head_dim values; a wave takes the two rows of a rotated pair one after the other - (2j, 2j + 1) of a
+// head, or (j, j + n_dims / 2) in NEOX mode; rows past n_dims pass through - so both values sit in neighbouring lanes of its
+// result registers, and what is stored is the pair rotated by the cos / sin of token t and pair j from table (the layout
+// chip_rope_table writes: per token the n_dims / 2 cosines, then the sines), with the ROPE kernel's two expressions.  The
+// projection's own result is not stored.  y: the ROPE's F32 result (if write_f32), h16: its fp16 copy [token][row] (the K
+// cache store), or nullptr.
+struct RopeEpilogue { const float *table; int head_dim, n_dims, neox, write_f32; unsigned short *h16; int64_t h16_ld; };
+constexpr RopeEpilogue kNoRope = {nullptr, 0, 0, 0, 0, nullptr, 0};
 constexpr int GROUP_MAX = 4;
-struct GroupMat { int wtype; const void *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld; };
+struct GroupMat { int wtype; const void *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld;
+                  RopeEpilogue rope = kNoRope; };
 int        gemv_group_family(int wtype);
 bool       gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim, bool prepared = false);
 // the GEMV over prepared rows for two matrices of one shape in one launch, and with a transposed fp16 copy of the result

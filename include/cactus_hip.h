@@ -193,6 +193,27 @@ typedef struct chip_mat {
 } chip_mat;
 CHIP_API int chip_mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n,
                                 void *workspace, size_t workspace_bytes, void *stream);
+/* chip_mul_mat_group with the ROPE node that follows a member run in that member's epilogue (reference
+ * cactus/llama-model.cpp build_llama: Qcur / Kcur = lm_ggml_rope_ext(...) right after their projections;
+ * lm_ggml_compute_forward_rope_f32, ggml-cpu/ops.cpp:5178-5361, modes 0 and LM_GGML_ROPE_TYPE_NEOX = 2).  ropes[i].table != NULL:
+ * member i's rows are heads of head_dim values (N a multiple of head_dim), a wave computes the two rows of a rotated pair one
+ * after the other and stores the pair rotated with table (chip_rope_table's output for the n tokens): y receives what
+ * chip_rope_apply would write from the member's result, y_f16 its fp16 copy as chip_rope_apply_store (the K cache store);
+ * either may be NULL, not both.  mats[i].y is not written for such a member (it may be NULL).  Every value has the bits of
+ * chip_mul_mat_group followed by chip_rope_apply / chip_rope_apply_store.  Only where chip_mul_mat_group is one launch (1, 2
+ * or 4 tokens, members of one family, K-quants or 32-value block types, fp32 rows x): CHIP_EUNSUPPORTED otherwise, nothing
+ * written, and the caller runs the nodes one by one. */
+typedef struct chip_rope_after {
+    const float *table;      /* NULL: no ROPE behind this member */
+    int64_t      head_dim;   /* ne0 of the ROPE */
+    int          n_dims, mode;
+    float       *y;          /* F32 result [n][N], row stride ldy, or NULL */
+    int64_t      ldy;
+    uint16_t    *y_f16;      /* fp16 copy [n][N], row stride ld16 halves, or NULL */
+    int64_t      ld16;
+} chip_rope_after;
+CHIP_API int chip_mul_mat_group_rope(const chip_mat *mats, const chip_rope_after *ropes, int count, int64_t K, const float *x,
+                                     int64_t ldx, int64_t n, void *workspace, size_t workspace_bytes, void *stream);
 /* The same over rows the workspace already holds - Phase B of the op alone (ggml-cpu/ggml-cpu.c:1380-1448) for a group, as
  * chip_mul_mat_run is for one matrix: the rows were written by chip_mul_mat_prepare or by the kernel that produced the
  * activations (chip_rms_norm_quantized, chip_silu_mul_quantized).  Up to 4 tokens and members of one family: one launch of

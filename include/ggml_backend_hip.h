@@ -62,6 +62,8 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_head_merges(void);
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_pairs(void);
 /* Gated FFNs whose four nodes ffn_gate, SILU, ffn_up, MUL (cactus/llama-graph.cpp:562-690) ran as one launch, up to 4 tokens. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_gated_pairs(void);
+/* ROPE nodes that ran in the epilogue of the projection in front of them (Q's and K's, in the group launch of wq / wk / wv). */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_epilogues(void);
 
 #ifdef __cplusplus
 }

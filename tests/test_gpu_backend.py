@@ -887,6 +887,8 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     grouped_before = blib.lm_ggml_backend_hip_get_grouped_matmuls()
     blib.lm_ggml_backend_hip_get_rope_pairs.restype = C.c_ulonglong
     pairs_before = blib.lm_ggml_backend_hip_get_rope_pairs()
+    blib.lm_ggml_backend_hip_get_rope_epilogues.restype = C.c_ulonglong
+    epilogues_before = blib.lm_ggml_backend_hip_get_rope_epilogues()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     assert blib.lm_ggml_backend_hip_get_rope_tables() - tables_before == 1      # Q and K share one cos / sin table
     # The K store ran in the kernel of K's RoPE.  With up to 4 tokens the transposed V store ran in the V projection's
@@ -895,10 +897,11 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     grouped = blib.lm_ggml_backend_hip_get_grouped_matmuls() - grouped_before
     assert grouped == (0 if n_tokens > 4 else 3), grouped
     fused = blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before
-    # K's RoPE (with its store) in the launch of Q's when K's projection had already run with Q's
+    # Up to 4 tokens the RoPE of Q and of K (with K's store) ran in the epilogue of their projections, so no ROPE kernel at all
     pairs = blib.lm_ggml_backend_hip_get_rope_pairs() - pairs_before
-    assert pairs == (1 if grouped >= 2 else 0), (pairs, grouped)
-    assert fused == (1 if n_tokens > 4 else 2 + max(grouped - 1, 0) + pairs), (fused, grouped, pairs)
+    epilogues = blib.lm_ggml_backend_hip_get_rope_epilogues() - epilogues_before
+    assert (epilogues, pairs) == ((0, 0) if n_tokens > 4 else (2, 0)), (epilogues, pairs, grouped)
+    assert fused == (1 if n_tokens > 4 else 2 + max(grouped - 1, 0) + epilogues), (fused, grouped, epilogues)
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip

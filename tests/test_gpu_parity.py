@@ -342,6 +342,47 @@ def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
         check_outputs(y2, ref["y"], ref["sum_abs"], "second matrix of the pair, n = %d" % n)
 
 
+# (types of wq, wk, wv), K, heads, KV heads, head size, rotated dims, mode: LLaMA-3-8B's attention block in a Q4_K_M file (NORM and
+# NEOX pairs); 32-value block types incl. Q4_0 (two rows per step in the plain kernel, one in the pair walk); partial rotation
+# (pass-through rows); a head size that is no power of two; more pairs than one pass of the grid takes
+GROUP_ROPE_CASES = [((O.Q4_K, O.Q4_K, O.Q6_K), 4096, 32, 8, 128, 128, 0), ((O.Q4_K, O.Q4_K, O.Q6_K), 4096, 32, 8, 128, 128, 2),
+                    ((O.Q4_0, O.Q8_0, O.Q5_1), 1024, 8, 2, 64, 32, 2), ((O.Q6_K, O.Q5_K, O.Q4_K), 2048, 6, 2, 96, 64, 0),
+                    ((O.Q8_0, O.Q8_0, O.Q8_0), 512, 160, 160, 128, 128, 2)]
+
+
+@pytest.mark.parametrize("types,K,n_head,n_head_kv,hd,n_dims,mode", GROUP_ROPE_CASES)
+def test_group_with_rope_in_the_epilogue_equals_group_then_rope(dev, types, K, n_head, n_head_kv, hd, n_dims, mode):
+    """chip_mul_mat_group_rope: Q and K rotated in their projections' epilogue (K as F32 and as the fp16 cache copy, or the fp16
+    copy alone), V untouched - every value bit for bit what chip_mul_mat_group followed by chip_rope_apply_two gives."""
+    wq = quantized_weights(types[0], K + 1, n_head * hd, K)
+    wk = quantized_weights(types[1], K + 2, n_head_kv * hd, K)
+    wv = quantized_weights(types[2], K + 3, n_head_kv * hd, K)
+    members = [(types[0], wq), (types[1], wk), (types[2], wv)]
+    for n in (1, 2, 4):
+        x = common.activations_f32(K + n, n, K)
+        pos = np.array([37, 0, 4095, 100000][:n], np.int32)
+        q, k, v = dev.mul_mat_group(members, x)
+        a, b = dev.rope_two(q.reshape(n, n_head, hd), k.reshape(n, n_head_kv, hd), pos, n_dims, mode, want=(("f32",), ("f32", "f16")),
+                            freq_base=500000.0)
+        ropes = [(hd, n_dims, mode, ("f32",)), (hd, n_dims, mode, ("f32", "f16")), None]
+        rc, got = dev.mul_mat_group_rope(members, x, pos, ropes, freq_base=500000.0)
+        assert got[0]["f32"].tobytes() == a["f32"].tobytes(), n
+        assert got[1]["f32"].tobytes() == b["f32"].tobytes() and got[1]["f16"].tobytes() == b["f16"].tobytes(), n
+        assert got[2]["y"].tobytes() == v.tobytes(), n
+        ropes = [(hd, n_dims, mode, ("f32",)), (hd, n_dims, mode, ("f16",)), None]       # K's F32 result has no other reader
+        rc, got = dev.mul_mat_group_rope(members, x, pos, ropes, freq_base=500000.0)
+        assert got[0]["f32"].tobytes() == a["f32"].tobytes() and got[1]["f16"].tobytes() == b["f16"].tobytes(), n
+    import cactus_amd as ca
+    x = common.activations_f32(K, 3, K)
+    rc, _ = dev.mul_mat_group_rope(members, x, np.arange(3, dtype=np.int32), [(hd, n_dims, mode, ("f32",)), None, None], check=False)
+    assert rc == ca.CHIP_EUNSUPPORTED                                            # 3 tokens: no one-launch form
+    x = common.activations_f32(K, 1, K)
+    rc, _ = dev.mul_mat_group_rope(members, x, np.zeros(1, np.int32), [(hd + 2, n_dims, mode, ("f32",)), None, None], check=False)
+    assert rc in (ca.CHIP_EUNSUPPORTED, ca.CHIP_EINVAL)                          # rows are no whole heads of that size
+    rc, _ = dev.mul_mat_group_rope(members, x, np.zeros(1, np.int32), [(hd, n_dims, 8, ("f32",)), None, None], check=False)
+    assert rc == ca.CHIP_EUNSUPPORTED                                            # multi-section mode
+
+
 @pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(1024, 336), (4096, 1032), (4096, 14336), (256, 8), (2048, 4104)])
 def test_gated_pair_equals_the_pair_and_silu_mul(dev, wt, K, N):
