@@ -680,7 +680,7 @@ def bench_headline(dev, hip, trace, steps, warmup, eager):
     return value, ms_per_step, b, roof, info
 
 
-def bench_whole_layers(dev, hip, trace, n, n_kv):
+def bench_whole_layers(dev, hip, trace, n, n_kv, fold=True):
     """Every node of the 32 layers as llama.cpp builds them without flash attention (norms, projections, RoPE, cache
     stores, kq, soft-max, kqv, head merge, residuals, SiLU * up), n new tokens against n_kv cached positions, as one
     HIP graph on one stream: what a decode step costs when no activation leaves the device."""
@@ -706,6 +706,13 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
     aws = dev.alloc(aws_bytes)
     rope_tab = dev.alloc(n * hd * 4)
     ck = dev.check
+    # up to 4 tokens the norms run in the prologue of the projections that read them and the residual ADDs in the store of
+    # the projections in front of them, where the library has those forms for the model's types
+    Wl = trace.weights(0)
+    deferred = (fold and n <= 4 and all(L.chip_norm_before_supported(Wl[nm][0], H, n) == 1 for nm in ("wq", "wk", "wv", "gate")) and
+                L.chip_mul_mat_pair_silu_mul_supported(Wl["gate"][0], H, FF, n) == 1 and
+                L.chip_mul_mat_add_supported(Wl["wo"][0], H, H, n) == 1 and L.chip_mul_mat_add_supported(Wl["down"][0], FF, H, n) == 1)
+    nb = ca.NormBefore(wn.ptr, 1e-5, cur.ptr, H)
 
     def mm(t, wptr, N, K, src, dst, shared=False):
         """shared: src was quantized by the previous matmul (same tensor, same activation type), as the backend reuses it"""
@@ -721,7 +728,7 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
             W = trace.weights(l)
             kc = caches.ptr + (2 * l) * kv_size * KV * 2
             vc = kc + kv_size * KV * 2
-            if l == 0:
+            if l == 0 and not deferred:
                 ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))  # norm + weight: one kernel, as the backend fuses them
             # q, k, v projections on one activation: one call; V's also stores into the transposed F16 cache
             arr = (ca.Mat * 3)()
@@ -738,7 +745,10 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
                 rp = (ca.RopeAfter * 3)()
                 rp[0] = ca.RopeAfter(rope_tab.ptr, hd, hd, 2, q.ptr, hd * n_head, None, 0)
                 rp[1] = ca.RopeAfter(rope_tab.ptr, hd, hd, 2, None, 0, kc + 2 * KV * (n_kv - n), KV)
-                ck(L.chip_mul_mat_group_rope(arr, rp, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
+                if deferred:                                          # attn_norm and its weight MUL in the same launch's prologue
+                    ck(L.chip_mul_mat_group_rope_norm(arr, rp, C.byref(nb), 3, H, resid.ptr, H, n, ws.ptr, wsz, st))
+                else:
+                    ck(L.chip_mul_mat_group_rope(arr, rp, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
             else:
                 ck(L.chip_mul_mat_group(arr, 3, H, cur.ptr, H, n, ws.ptr, wsz, st))
                 # RoPE of Q and of K in one launch; K's also stores into the F16 cache
@@ -760,11 +770,20 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
                                               kqv.ptr, hd, hd * n, aws.ptr, aws_bytes, st))
                 ck(L.chip_cpy(kqv.ptr, ca.F32, A4(hd, n_head, n, 1), A4(4, 4 * hd * n, 4 * hd, 0), merged.ptr, ca.F32, A4(H, n, 1, 1),
                               A4(4, 4 * H, 4 * H * n, 4 * H * n), st))
+            (t_, wg, N_, K_), (_, wu, _, _) = W["gate"], W["up"]
+            td, wd, Nd, Kd = W["down"]
+            if deferred:
+                # wo with the residual ADD in its store; ffn_norm and its weight MUL in the gated pair's prologue; ffn_down with
+                # the second residual ADD in its store: four launches for the eleven nodes, as the backend runs them
+                to_, wo_, No_, Ko_ = W["wo"]
+                ck(L.chip_mul_mat_add(to_, wo_, dev.row_size(to_, Ko_), Ko_, No_, merged.ptr, Ko_, n, resid.ptr, H, resid.ptr, H, ws.ptr, wsz, st))
+                ck(L.chip_mul_mat_pair_silu_mul_norm(t_, wg, wu, dev.row_size(t_, K_), K_, N_, resid.ptr, K_, n, C.byref(nb), gate.ptr, N_,
+                                                     ws.ptr, wsz, st))
+                ck(L.chip_mul_mat_add(td, wd, dev.row_size(td, Kd), Kd, Nd, gate.ptr, Kd, n, resid.ptr, H, resid.ptr, H, ws.ptr, wsz, st))
+                continue
             mm(*W["wo"], merged, att)
             # residual + norm + weight: one kernel, as the backend fuses the three nodes
             ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
-            (t_, wg, N_, K_), (_, wu, _, _) = W["gate"], W["up"]
-            td, wd, Nd, Kd = W["down"]
             if n <= 4 and L.chip_mul_mat_pair_silu_mul_supported(t_, K_, N_, n) == 1:
                 # gate, SILU, up and their MUL in one launch; ffn_down quantizes its input itself, as the backend runs the five nodes
                 ck(L.chip_mul_mat_pair_silu_mul(t_, wg, wu, dev.row_size(t_, K_), K_, N_, cur.ptr, K_, n, gate.ptr, N_, ws.ptr, wsz, st))
@@ -776,6 +795,8 @@ def bench_whole_layers(dev, hip, trace, n, n_kv):
                 ck(L.chip_mul_mat_run_ws(td, wd, dev.row_size(td, Kd), Kd, Nd, n, ws.ptr, wsz, att.ptr, Nd, st))
             # the layer's second residual with the next layer's (or the final) norm
             ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
+        if deferred:                                                  # the final norm has no projection of this kind behind it
+            ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))
         ck(L.chip_mul_mat(ca.Q6_K, trace.arena.ptr + trace.head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
 
     step()

@@ -35,7 +35,7 @@ EXPORTS = (
     "chip_event_destroy", "chip_event_record", "chip_event_synchronize", "chip_stream_wait_event", "chip_block_elems", "chip_block_bytes", "chip_row_size",
     "chip_vec_dot_type", "chip_mul_mat_supported", "chip_quantize_q8_0", "chip_quantize_q8_K",
     "chip_quantize_q8_1", "chip_convert_f32_to_f16",
-    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_pair_silu_mul", "chip_mul_mat_pair_silu_mul_supported", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_rope", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
+    "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_pair_silu_mul", "chip_mul_mat_pair_silu_mul_supported", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_rope", "chip_mul_mat_group_rope_norm", "chip_mul_mat_pair_silu_mul_norm", "chip_norm_before_supported", "chip_mul_mat_add", "chip_mul_mat_add_supported", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_rope_apply_two", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
     "chip_block_isums", "chip_verify_force_q6k_matrix_core",
@@ -65,6 +65,11 @@ class RopeAfter(C.Structure):
     """struct chip_rope_after: the ROPE node behind a member of chip_mul_mat_group_rope."""
     _fields_ = [("table", C.c_void_p), ("head_dim", C.c_int64), ("n_dims", C.c_int), ("mode", C.c_int), ("y", C.c_void_p),
                 ("ldy", C.c_int64), ("y_f16", C.c_void_p), ("ld16", C.c_int64)]
+
+
+class NormBefore(C.Structure):
+    """struct chip_norm_before: the RMS norm and weight MUL run in a projection's prologue."""
+    _fields_ = [("w", C.c_void_p), ("eps", C.c_float), ("y", C.c_void_p), ("ldy", C.c_int64)]
 
 
 class ChipError(RuntimeError):
@@ -131,6 +136,11 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_pair.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, vp, i64, vp, sz, vp]
     L.chip_mul_mat_pair_silu_mul.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_pair_silu_mul_supported.argtypes = [i32, i64, i64, i64]
+    L.chip_mul_mat_group_rope_norm.argtypes = [C.POINTER(Mat), C.POINTER(RopeAfter), C.POINTER(NormBefore), i32, i64, vp, i64, i64, vp, sz, vp]
+    L.chip_mul_mat_pair_silu_mul_norm.argtypes = [i32, vp, vp, sz, i64, i64, vp, i64, i64, C.POINTER(NormBefore), vp, i64, vp, sz, vp]
+    L.chip_norm_before_supported.argtypes = [i32, i64, i64]
+    L.chip_mul_mat_add_supported.argtypes = [i32, i64, i64, i64]
+    L.chip_mul_mat_add.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, i64, vp, sz, vp]
     L.chip_mul_mat_store_t.argtypes = [i32, vp, sz, i64, i64, vp, i64, i64, vp, i64, vp, i64, vp, sz, vp]
     L.chip_rms_norm.argtypes = [vp, i64, i64, i64, C.c_float, vp, i64, vp]
     L.chip_add.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, i64, vp]
@@ -325,10 +335,11 @@ class Device:
             res.append(dh.download(np.uint16, outs[-1][1] * ld16).reshape(outs[-1][1], ld16))
         return res
 
-    def mul_mat_group_rope(self, members, x, pos, ropes, freq_base=10000.0, check=True):
+    def mul_mat_group_rope(self, members, x, pos, ropes, freq_base=10000.0, check=True, norm=None):
         """chip_rope_table + chip_mul_mat_group_rope: members as mul_mat_group; ropes[i] = None or (head_dim, n_dims, mode,
         wants) with wants a subset of ("f32", "f16").  Returns (rc, list of dicts): a roped member's dict holds "f32" / "f16"
-        arrays [n, N], an unroped member's "y"."""
+        arrays [n, N], an unroped member's "y".  norm = (weight row, eps): chip_mul_mat_group_rope_norm, and one more dict
+        {"normed": [n, K]} at the end of the list."""
         x = np.ascontiguousarray(x, np.float32)
         n, k = x.shape
         dx = self.to_device(x)
@@ -364,7 +375,13 @@ class Device:
             rp[i] = RopeAfter(dt.ptr, hd, n_dims, mode, o["f32"][0].ptr if "f32" in o else None, N, o["f16"][0].ptr if "f16" in o else None, N)
             outs.append(o)
         ws = self.alloc(max(wsz, 16))
-        rc = self.lib.chip_mul_mat_group_rope(arr, rp, len(members), k, dx.ptr, k, n, ws.ptr, wsz, None)
+        if norm is None:
+            rc = self.lib.chip_mul_mat_group_rope(arr, rp, len(members), k, dx.ptr, k, n, ws.ptr, wsz, None)
+        else:
+            dw, dn = self.to_device(np.ascontiguousarray(norm[0], np.float32)), self.alloc(n * k * 4)
+            self.check(self.lib.chip_memset(dn.ptr, 0xFF, n * k * 4, None))
+            nb = NormBefore(dw.ptr, norm[1], dn.ptr, k)
+            rc = self.lib.chip_mul_mat_group_rope_norm(arr, rp, C.byref(nb), len(members), k, dx.ptr, k, n, ws.ptr, wsz, None)
         if check:
             self.check(rc)
         self.sync()
@@ -372,6 +389,8 @@ class Device:
         for (wt, W), o in zip(members, outs):
             N = np.asarray(W).shape[0]
             res.append({key: buf.download(dt_, n * N).reshape(n, N) for key, (buf, dt_) in o.items()})
+        if norm is not None:
+            res.append({"normed": dn.download(np.float32, n * k).reshape(n, k)})
         return rc, res
 
     def mul_mat_pair(self, wtype, W1, W2, x):
@@ -389,8 +408,9 @@ class Device:
         self.sync()
         return y1.download(np.float32, n * N).reshape(n, N), y2.download(np.float32, n * N).reshape(n, N)
 
-    def mul_mat_pair_silu_mul(self, wtype, W1, W2, x):
-        """silu(W1 x) * (W2 x) in one launch (chip_mul_mat_pair_silu_mul): fp32 [n, N]."""
+    def mul_mat_pair_silu_mul(self, wtype, W1, W2, x, norm=None):
+        """silu(W1 x) * (W2 x) in one launch (chip_mul_mat_pair_silu_mul): fp32 [n, N].  norm = (weight row, eps): the rows are
+        normed in the prologue (chip_mul_mat_pair_silu_mul_norm) and (y, normed rows) is returned."""
         x = np.ascontiguousarray(x, np.float32)
         n, k = x.shape
         W1, W2 = np.ascontiguousarray(W1, np.uint8), np.ascontiguousarray(W2, np.uint8)
@@ -401,9 +421,42 @@ class Device:
         self.check(self.lib.chip_memset(y.ptr, 0xFF, n * N * 4, None))                   # NaN: unwritten rows show
         wsz = self.lib.chip_mul_mat_workspace_size_n(wtype, k, N, n)
         ws = self.alloc(wsz)
+        if norm is not None:
+            dw, dn = self.to_device(np.ascontiguousarray(norm[0], np.float32)), self.alloc(n * k * 4)
+            self.check(self.lib.chip_memset(dn.ptr, 0xFF, n * k * 4, None))
+            nb = NormBefore(dw.ptr, norm[1], dn.ptr, k)
+            self.check(self.lib.chip_mul_mat_pair_silu_mul_norm(wtype, d1.ptr, d2.ptr, nb01, k, N, dx.ptr, k, n, C.byref(nb), y.ptr, N,
+                                                                ws.ptr, wsz, None))
+            self.sync()
+            return y.download(np.float32, n * N).reshape(n, N), dn.download(np.float32, n * k).reshape(n, k)
         self.check(self.lib.chip_mul_mat_pair_silu_mul(wtype, d1.ptr, d2.ptr, nb01, k, N, dx.ptr, k, n, y.ptr, N, ws.ptr, wsz, None))
         self.sync()
         return y.download(np.float32, n * N).reshape(n, N)
+
+    def mul_mat_add(self, wtype, W, x, addend, in_place=False):
+        """W x + addend in one launch (chip_mul_mat_add): fp32 [n, N]; in_place: the result goes over the addend."""
+        x, addend = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(addend, np.float32)
+        n, k = x.shape
+        W = np.ascontiguousarray(W, np.uint8)
+        N = W.shape[0]
+        dW, dx, da = self.to_device(W), self.to_device(x), self.to_device(addend)
+        y = da if in_place else self.alloc(n * N * 4)
+        if not in_place:
+            self.check(self.lib.chip_memset(y.ptr, 0xFF, n * N * 4, None))
+        wsz = self.lib.chip_mul_mat_workspace_size_n(wtype, k, N, n)
+        ws = self.alloc(wsz)
+        self.check(self.lib.chip_mul_mat_add(wtype, dW.ptr, self.row_size(wtype, k), k, N, dx.ptr, k, n, da.ptr, N, y.ptr, N, ws.ptr, wsz, None))
+        self.sync()
+        return y.download(np.float32, n * N).reshape(n, N)
+
+    def rms_norm_mul(self, x, w, eps):
+        """chip_rms_norm_mul: the norm of every row times the weight row."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, ne0 = x.shape
+        dx, dw, dy = self.to_device(x), self.to_device(np.ascontiguousarray(w, np.float32)), self.alloc(x.nbytes)
+        self.check(self.lib.chip_rms_norm_mul(dx.ptr, ne0, n, ne0, eps, dw.ptr, None, 0, dy.ptr, ne0, None))
+        self.sync()
+        return dy.download(np.float32, n * ne0).reshape(n, ne0)
 
     def rms_norm(self, x, eps):
         x = np.ascontiguousarray(x, np.float32)

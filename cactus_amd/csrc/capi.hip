@@ -485,8 +485,33 @@ int chip_mul_mat_pair_silu_mul_supported(int type, int64_t K, int64_t N, int64_t
     if (current_limits(lim) != CHIP_OK) return 0;
     return gemv_fused_applicable(type, K, (int)n, lim) ? 1 : 0;
 }
+static int norm_before_checked(const chip_norm_before *norm, int type, int64_t K, int64_t n, const DeviceLimits &lim) {
+    if (!norm || !norm->w || !aligned16(norm->w)) return CHIP_EINVAL;
+    if (norm->y && (!aligned16(norm->y) || norm->ldy < K || (norm->ldy % 4) != 0)) return CHIP_EINVAL;
+    return gemv_norm_prologue_applicable(type, K, (int)n, lim) ? CHIP_OK : CHIP_EUNSUPPORTED;
+}
+int chip_norm_before_supported(int type, int64_t K, int64_t n) {
+    if (!chip_mul_mat_supported(type, K) || n < 1 || n > 4) return 0;
+    DeviceLimits lim;
+    if (current_limits(lim) != CHIP_OK) return 0;
+    return gemv_norm_prologue_applicable(type, K, (int)n, lim) ? 1 : 0;
+}
+static int pair_silu_mul(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                         int64_t n, const chip_norm_before *norm, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                         void *stream);
 int chip_mul_mat_pair_silu_mul(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
                                int64_t n, float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    return pair_silu_mul(type, W1, W2, nb01, K, N, x, ldx, n, nullptr, y, ldy, workspace, workspace_bytes, stream);
+}
+int chip_mul_mat_pair_silu_mul_norm(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                                    int64_t n, const chip_norm_before *norm, float *y, int64_t ldy, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+    if (!norm) return CHIP_EINVAL;
+    return pair_silu_mul(type, W1, W2, nb01, K, N, x, ldx, n, norm, y, ldy, workspace, workspace_bytes, stream);
+}
+static int pair_silu_mul(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
+                         int64_t n, const chip_norm_before *norm, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                         void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;
     if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
     if (N == 0 || n == 0) return CHIP_OK;
@@ -497,8 +522,33 @@ int chip_mul_mat_pair_silu_mul(int type, const void *W1, const void *W2, size_t 
     if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
     DeviceLimits lim;
     if (int rc = current_limits(lim); rc) return rc;
+    if (norm)
+        if (int rc = norm_before_checked(norm, type, K, n, lim); rc) return rc;
     return hip_rc(launch_gemv_fused_pair_silu_mul(type, W1, W2, nb01, K, N, x, ldx, (int)n, workspace,
-                                                  act_stride(chip_vec_dot_type(type), K), y, ldy, lim, (hipStream_t)stream));
+                                                  act_stride(chip_vec_dot_type(type), K), y, ldy, lim, (hipStream_t)stream,
+                                                  norm ? norm->w : nullptr, norm ? norm->eps : 0.f, norm ? norm->y : nullptr,
+                                                  norm ? norm->ldy : 0));
+}
+int chip_mul_mat_add_supported(int type, int64_t K, int64_t N, int64_t n) {
+    if (!chip_mul_mat_supported(type, K) || N <= 0 || n < 1 || n > 4) return 0;
+    DeviceLimits lim;
+    if (current_limits(lim) != CHIP_OK) return 0;
+    return gemv_fused_applicable(type, K, (int)n, lim) ? 1 : 0;
+}
+int chip_mul_mat_add(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
+                     const float *addend, int64_t ld_add, float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (N < 0 || n < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(type, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0 || n == 0) return CHIP_OK;
+    if (!chip_mul_mat_add_supported(type, K, N, n)) return CHIP_EUNSUPPORTED;
+    if (!x || !workspace || ldx < K || !W || !y || ldy < N || !addend || ld_add < N) return CHIP_EINVAL;
+    if (!aligned16(x) || (ldx % 4) != 0 || !aligned16(workspace) || ((((uintptr_t)y) | ((uintptr_t)addend)) & 3) != 0) return CHIP_EINVAL;
+    if (!weights_aligned(type, W, nb01, K) || nb01 < chip_row_size(type, K)) return CHIP_EINVAL;
+    if (workspace_bytes < chip_mul_mat_workspace_size(type, K, n)) return CHIP_ENOMEM;
+    DeviceLimits lim;
+    if (int rc = current_limits(lim); rc) return rc;
+    return hip_rc(launch_gemv_fused_add(type, W, nb01, K, N, x, ldx, (int)n, workspace, act_stride(chip_vec_dot_type(type), K), addend,
+                                        ld_add, y, ldy, lim, (hipStream_t)stream));
 }
 
 static int rope_dims_checked(int64_t ne0, int64_t ne1, int64_t ne2, int n_dims, int mode);
@@ -507,7 +557,8 @@ static int rope_dims_checked(int64_t ne0, int64_t ne1, int64_t ne2, int n_dims, 
 // prologue-quantizing GEMV over all members; otherwise one quantizer and each member on its usual path.
 // what chip_mul_mat_group and chip_mul_mat_group_run share: x == nullptr says the workspace already holds the rows
 static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace,
-                         size_t workspace_bytes, void *stream, const chip_rope_after *ropes = nullptr) {
+                         size_t workspace_bytes, void *stream, const chip_rope_after *ropes = nullptr,
+                         const chip_norm_before *norm = nullptr) {
     if (count < 0 || n < 0) return CHIP_EINVAL;
     if (count == 0 || n == 0) return CHIP_OK;
     if (!mats || count > CHIP_GROUP_MAX) return CHIP_EINVAL;
@@ -561,8 +612,15 @@ static int mul_mat_group(const chip_mat *mats, int count, int64_t K, const float
     if (any_rope) {                                                      // only the one-launch form has the epilogue
         if (prepared || n > 4 || !gemv_group_applicable(gm, live, K, (int)n, lim, false) || gemv_group_family(gm[0].wtype) == 2)
             return CHIP_EUNSUPPORTED;
-        return hip_rc(launch_gemv_group(gm, live, K, x, ldx, (int)n, workspace, act_stride(at, K), lim, (hipStream_t)stream, false));
+        GroupNorm gn{nullptr, 0.f, nullptr, 0};
+        if (norm) {
+            for (int i = 0; i < live; i++)
+                if (int rc = norm_before_checked(norm, gm[i].wtype, K, n, lim); rc) return rc;
+            gn = GroupNorm{norm->w, norm->eps, norm->y, norm->ldy};
+        }
+        return hip_rc(launch_gemv_group(gm, live, K, x, ldx, (int)n, workspace, act_stride(at, K), lim, (hipStream_t)stream, false, &gn));
     }
+    if (norm) return CHIP_EUNSUPPORTED;
     const size_t stride = act_stride(at, K);
     hipStream_t st = (hipStream_t)stream;
     // Up to 4 tokens.  One member, or two of one type, shape and row stride, take the single-matrix kernel (it keeps more
@@ -618,6 +676,11 @@ int chip_mul_mat_group_rope(const chip_mat *mats, const chip_rope_after *ropes, 
                             int64_t n, void *workspace, size_t workspace_bytes, void *stream) {
     if (!ropes || (count > 0 && n > 0 && !x)) return CHIP_EINVAL;
     return mul_mat_group(mats, count, K, x, ldx, n, workspace, workspace_bytes, stream, ropes);
+}
+int chip_mul_mat_group_rope_norm(const chip_mat *mats, const chip_rope_after *ropes, const chip_norm_before *norm, int count, int64_t K,
+                                 const float *x, int64_t ldx, int64_t n, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!ropes || !norm || (count > 0 && n > 0 && !x)) return CHIP_EINVAL;
+    return mul_mat_group(mats, count, K, x, ldx, n, workspace, workspace_bytes, stream, ropes, norm);
 }
 int chip_mul_mat_group_run(const chip_mat *mats, int count, int64_t K, int64_t n, void *workspace, size_t workspace_bytes, void *stream) {
     return mul_mat_group(mats, count, K, nullptr, 0, n, workspace, workspace_bytes, stream);

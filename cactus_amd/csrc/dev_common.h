@@ -68,6 +68,46 @@ __device__ __forceinline__ float wave_max_all(float v) {
     return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
+// The same butterfly for a double (two 32-bit moves per step); the total ends up in lane 63.
+template <int CTRL, int ROW_MASK = 0xf, bool BOUND = true>
+__device__ __forceinline__ double dpp_get_f64(double v) {
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, ROW_MASK, 0xf, BOUND);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, ROW_MASK, 0xf, BOUND);
+    return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double wave_sum_f64_to_lane63(double v) {
+    v += dpp_get_f64<0xB1>(v);
+    v += dpp_get_f64<0x4E>(v);
+    v += dpp_get_f64<0x141>(v);
+    v += dpp_get_f64<0x140>(v);
+    v += dpp_get_f64<0x142, 0xa, false>(v);
+    v += dpp_get_f64<0x143, 0xc, false>(v);
+    return v;
+}
+// The sum of squares of a row for the RMS norm (reference lm_ggml_compute_forward_rms_norm_f32, ggml-cpu/ops.cpp: sum +=
+// (lm_ggml_float)(x * x), squares rounded to float, added in double), in an order fixed by where a value lies in the row, so that
+// every kernel that forms it gets the same bits whatever its thread layout:
+//   a float4 chunk      d = ((x0^2 + x1^2) + x2^2) + x3^2                       (norm_chunk_squares)
+//   a 256-value block   B = the butterfly sum of its 64 chunks, lane = chunk % 64  (wave_sum_f64_to_lane63; absent chunks 0.0)
+//   S_r = B(r) + B(r + 4) + B(r + 8) + ... for r = 0..3, and the total = ((S_0 + S_1) + S_2) + S_3.
+__device__ __forceinline__ double norm_chunk_squares(const float4 v) {
+    return (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+}
+constexpr int NORM_BLOCKS_MAX = 32;       // blocks of a row whose B values a kernel may keep side by side (rows up to 8192 values)
+// total from the B values of a row (all threads read the same addresses)
+__device__ __forceinline__ double norm_total_from_blocks(const double *B, int blocks) {
+    double s[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int b = 0; b < blocks; b += 4) {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            if (b + r < blocks) s[r] += B[b + r];
+    }
+    double total = 0.0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) total += s[r];
+    return total;
+}
+
 // One lane of lm_ggml_v_expf in its AVX2 + FMA form (reference ggml-cpu/vec.h:615-656), operation by operation: the fused
 // operations are explicit fmaf calls and the library is built with -ffp-contract=off, so nothing else is contracted.
 __device__ __forceinline__ float v_expf_lane(float x) {

@@ -19,6 +19,7 @@
 //   * integer dots use v_dot4_i32_i8; each lane keeps fp32 partial sums per (row, token) and the 64 lanes are
 //     combined at the end with a fixed DPP butterfly (no LDS round trip, deterministic order).
 #include "gemv_body.h"
+#include <algorithm>
 #include <cstdlib>
 
 namespace chip {
@@ -28,7 +29,9 @@ __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W
                                                    const float *__restrict__ x, int64_t ldx,
                                                    uint8_t *__restrict__ ws, size_t ws_stride,
                                                    float *__restrict__ y, int64_t ldy, SecondMatrix sec) {
-    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED, GATED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
+    // the gated pair may also take the RMS norm of its input rows into its prologue (gemv_body.h: NORMABLE)
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED, GATED, false, GATED && FUSEQ && !PHASED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec,
+                                                                                                whole_grid());
 }
 
 // LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
@@ -76,6 +79,7 @@ static hipError_t launch_depth(const void *W, size_t nb01, int64_t K, int64_t N,
         // (measured: 4096 x 14336 Q4_K 10.5 -> 9.5 us, 4096 x 11008 8.7 -> 8.0 us, Q6_K 4096 x 14336 15.3-16.1 -> 14.7 us;
         //  two steps - K = 8192 - run 2 % slower that way and keep the plain prologue)
         if (iters_per_row<WT>(K) > 2 && tune("CHIP_GEMV_PHASED", 1) != 0) {
+            if (sec.norm_w) return hipErrorInvalidValue;                 // the phased prologue never holds the whole row
             static LdsGrant grant, grant_gated;                          // one per kernel instantiation
             if (sec.gated) return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, true, true>, grant_gated);
             return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, true>, grant);
@@ -88,6 +92,7 @@ static hipError_t launch_depth(const void *W, size_t nb01, int64_t K, int64_t N,
     } else {
         if (sec.gated) return hipErrorInvalidValue;
     }
+    if (sec.norm_w) return hipErrorInvalidValue;                         // only the gated pair's kernel is built with the norm
     return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false>, grant);
 }
 
@@ -102,7 +107,8 @@ template <int WT, int NTOK, bool FUSEQ, int R = RowsPerWave<WT>::R>
 static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, void *ws,
                                size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim, hipStream_t st,
                                const SecondMatrix &sec = kNoSecond) {
-    const size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
+    size_t lds_bytes = (size_t)NTOK * lds_image_bytes<WT>(K);
+    if (sec.norm_w) lds_bytes = ((lds_bytes + 7) & ~(size_t)7) + (size_t)NTOK * NORM_BLOCKS_MAX * sizeof(double);   // the norm's block sums
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     if constexpr (R == 2 && NTOK == 1) {
@@ -257,6 +263,20 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
     return (size_t)n * img <= (size_t)lim.max_lds_per_block;
 }
 
+// The RMS norm of the rows in the prologue (gemv_body.h: NORMABLE): the prologue that holds whole rows in registers, i.e.
+// not the one that builds the image a step's part at a time, and rows of at most NORM_BLOCKS_MAX blocks of 256 values.
+bool gemv_norm_prologue_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
+    if (!gemv_fused_applicable(wtype, K, n, lim) || K > 256 * NORM_BLOCKS_MAX) return false;
+    int iters = 0;
+    switch (wtype) {                                                     // the types with Q8_K activations
+        case T_Q4_K: iters = iters_per_row<T_Q4_K>(K); break;
+        case T_Q5_K: iters = iters_per_row<T_Q5_K>(K); break;
+        case T_Q6_K: iters = iters_per_row<T_Q6_K>(K); break;
+        default: break;
+    }
+    return iters <= 2;
+}
+
 static hipError_t launch_gemv_fused_sec(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx,
                                         int n, void *ws, size_t ws_stride, float *y, int64_t ldy, const DeviceLimits &lim,
                                         hipStream_t st, const SecondMatrix &sec);
@@ -274,9 +294,22 @@ hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, siz
 // silu(W1 x) * (W2 x) -> y, one launch (gemv_body.h: gated)
 hipError_t launch_gemv_fused_pair_silu_mul(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                            int64_t ldx, int n, void *ws, size_t ws_stride, float *y, int64_t ldy,
-                                           const DeviceLimits &lim, hipStream_t st) {
-    const SecondMatrix sec{N, (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01, 0, nullptr, 0, 1};
+                                           const DeviceLimits &lim, hipStream_t st, const float *norm_w, float norm_eps, float *norm_y,
+                                           int64_t norm_ldy) {
+    SecondMatrix sec = kNoSecond;
+    sec.n_first = N;
+    sec.w_off = (int64_t)((const uint8_t *)W2 - (const uint8_t *)W1) - N * (int64_t)nb01;
+    sec.gated = 1;
+    sec.norm_w = norm_w; sec.norm_eps = norm_eps; sec.norm_y = norm_y; sec.norm_ldy = norm_ldy;
     return launch_gemv_fused_sec(wtype, W1, nb01, K, 2 * N, x, ldx, n, ws, ws_stride, y, ldy, lim, st, sec);
+}
+// y = W x + addend in one launch (the residual ADD behind wo / ffn_down)
+hipError_t launch_gemv_fused_add(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int n, void *ws,
+                                 size_t ws_stride, const float *addend, int64_t ld_add, float *y, int64_t ldy, const DeviceLimits &lim,
+                                 hipStream_t st) {
+    SecondMatrix sec = kNoSecond;
+    sec.addend = addend; sec.ld_add = ld_add;
+    return launch_gemv_fused_sec(wtype, W, nb01, K, N, x, ldx, n, ws, ws_stride, y, ldy, lim, st, sec);
 }
 // y16t: element (token t, row r) of the result also goes to y16t[r * ld16 + t] as fp16
 hipError_t launch_gemv_fused_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int n,

@@ -879,6 +879,80 @@ __device__ __forceinline__ void stage_commit(const StageRegs<WT, NTOK> &sr, uint
 }
 
 
+// The float4 chunk of a row that register slot j of this thread holds after xload (-1: none), the first chunk of the
+// 256-value block that slot j of this wave covers (wave-uniform), and the RMS norm of the rows in those registers: a slot of a
+// wave is one 256-value block with lane = chunk % 64 in both register layouts, which is how dev_common.h orders the sum of
+// squares.  Lane 63 of every wave leaves the butterfly totals of its blocks in LDS (B, NORM_BLOCKS_MAX doubles per token, in a
+// place the image does not reach), one barrier, every thread adds them up and scales its registers by 1 / sqrt(mean + eps)
+// and then by the weight row: the same bits as rms_norm_kernel with a weight (ops.hip).
+template <int WT, int WGS> __device__ __forceinline__ int xreg_chunk(int j, int64_t K) {
+    using T = Traits<WT>;
+    if constexpr (T::ACT == T_Q8_0 || T::ACT == T_F16) {
+        const int c = j * WGS + (int)threadIdx.x;
+        return c < (int)(K / 4) ? c : -1;
+    } else {
+        const int sb = j * (WGS / 64) + ((int)threadIdx.x >> 6);
+        return sb < (int)(K / 256) ? sb * 64 + ((int)threadIdx.x & 63) : -1;
+    }
+}
+template <int WGS> __device__ __forceinline__ int xreg_block_first_chunk(int j) {
+    return j * WGS + ((int)threadIdx.x & ~63);            // both layouts: slot j of wave w starts at chunk j * WGS + 64 w
+}
+// (rows of at most 256 * NORM_BLOCKS_MAX values: the first NPER slots of a token)
+template <int WT, int NTOK, int WGS> struct NormRegs {
+    static constexpr int FULL = XRegs<NTOK, WGS>::PER, CAP = 64 * NORM_BLOCKS_MAX / WGS > 0 ? 64 * NORM_BLOCKS_MAX / WGS : 1;
+    static constexpr int NPER = FULL < CAP ? FULL : CAP;
+    float4 w[NPER];
+};
+template <int WT, int NTOK, int WGS>
+__device__ __forceinline__ void norm_issue(NormRegs<WT, NTOK, WGS> &nr, const float *__restrict__ w, int64_t K) {
+#pragma unroll
+    for (int j = 0; j < NormRegs<WT, NTOK, WGS>::NPER; j++) {
+        const int c = xreg_chunk<WT, WGS>(j, K);
+        nr.w[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c >= 0) nr.w[j] = *reinterpret_cast<const float4 *>(w + 4 * (int64_t)c);
+    }
+}
+template <int WT, int NTOK, int WGS>
+__device__ __forceinline__ void norm_apply(XRegs<NTOK, WGS> &xr, const NormRegs<WT, NTOK, WGS> &nr, int64_t K, float eps, float *y,
+                                           int64_t ldy, bool store, double *B) {
+    constexpr int PER = NormRegs<WT, NTOK, WGS>::NPER;
+    const int chunks = (int)(K / 4), blocks = (chunks + 63) >> 6;
+#pragma unroll
+    for (int t = 0; t < NTOK; t++)
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int first = xreg_block_first_chunk<WGS>(j);
+            if (first < chunks) {                                        // wave-uniform: all 64 lanes take part in the butterfly
+                const double d = xreg_chunk<WT, WGS>(j, K) >= 0 ? norm_chunk_squares(xr.v[t][j]) : 0.0;
+                const double total = wave_sum_f64_to_lane63(d);
+                if ((threadIdx.x & 63) == 63) B[t * NORM_BLOCKS_MAX + (first >> 6)] = total;
+            }
+        }
+    __syncthreads();
+    float scale[NTOK];
+#pragma unroll
+    for (int t = 0; t < NTOK; t++) {
+        const double total = norm_total_from_blocks(B + t * NORM_BLOCKS_MAX, blocks);
+        const float mean = (float)(total / (double)K);
+        scale[t] = 1.0f / sqrtf(mean + eps);
+    }
+#pragma unroll
+    for (int t = 0; t < NTOK; t++)
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int c = xreg_chunk<WT, WGS>(j, K);
+            if (c >= 0) {
+                float4 v = xr.v[t][j];
+                v.x *= scale[t]; v.y *= scale[t]; v.z *= scale[t]; v.w *= scale[t];
+                const float4 g = nr.w[j];
+                v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w;
+                xr.v[t][j] = v;
+                if (store) *reinterpret_cast<float4 *>(y + (int64_t)t * ldy + 4 * (int64_t)c) = v;
+            }
+        }
+}
+
 // Two matrices of one shape and type that read the same activation (ffn_gate and ffn_up) as one launch: rows
 // [0, n_first) are the first matrix, rows [n_first, N) the second one, whose weights and outputs lie w_off bytes / y_off
 // floats away from where the first matrix's row and output of that index would be.  One matrix: n_first = N.
@@ -892,17 +966,28 @@ __device__ __forceinline__ GridPart whole_grid() { return GridPart{(int64_t)bloc
 // gated (two matrices only): a wave takes row r of the first matrix and then row r of the second, and what is stored, at y's
 // row r, is silu(first) * second - the SILU and MUL nodes that follow ffn_gate and ffn_up (reference llama-graph.cpp:562-690,
 // LLM_FFN_SILU with LLM_FFN_PAR), with lm_ggml_vec_silu_f32's arithmetic; the two projections themselves are not stored.
-struct SecondMatrix { int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; int gated; };
-constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0, 0};
+// addend: a tensor of y's shape added to every output as it is stored (the residual ADD that follows wo and ffn_down, reference
+// llama-model.cpp build_llama: ffn_inp = add(cur, inpSA), cur = add(cur, ffn_inp)): y = W x + addend, one IEEE addition as the
+// ADD node's.  norm_w (kernels built NORMABLE only): the rows x are RMS-normed and multiplied by the weight row norm_w in the
+// prologue, before they are quantized - the RMS_NORM and MUL nodes in front of the projections (build_norm, llama-graph.cpp:527-560)
+// - with rms_norm_kernel's arithmetic and order of additions; norm_y, if given, receives the normed rows (workgroup 0 stores them).
+struct SecondMatrix {
+    int64_t n_first, w_off, y_off; unsigned short *t16; int64_t t16_ld; int gated;
+    const float *addend; int64_t ld_add;
+    const float *norm_w; float norm_eps; float *norm_y; int64_t norm_ldy;
+};
+constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0, 0, nullptr, 0, nullptr, 0.f, nullptr, 0};
 
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false, bool GATED = false, bool ROPED = false>
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false, bool GATED = false, bool ROPED = false,
+          bool NORMABLE = false>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                           const float *__restrict__ x, int64_t ldx,
                                           uint8_t *__restrict__ ws, size_t ws_stride,
                                           float *__restrict__ y, int64_t ldy, const SecondMatrix sec,
                                           const GridPart gp, const RopeEpilogue rope = kNoRope) {
     static_assert(!ROPED || (R == 1 && !GATED && !PHASED && FUSEQ), "the pair walk of the rotated rows takes one row per step");
+    static_assert(!NORMABLE || (FUSEQ && !PHASED), "the norm runs on the whole row in the prologue's registers");
     using T = Traits<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     static_assert(DEPTH == 1, "one step of weight loads is in flight beyond the one being computed");
@@ -982,11 +1067,23 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
     } else if constexpr (FUSEQ) {
         XRegs<NTOK, WGS> xr;
         xload<WT, NTOK, WGS>(xr, x, ldx, K);
+        [[maybe_unused]] NormRegs<WT, NTOK, WGS> nr;
+        if constexpr (NORMABLE) {
+            if (sec.norm_w) norm_issue<WT, NTOK, WGS>(nr, sec.norm_w, K);  // uniform; requested before the weights, needed before them
+        }
         [[maybe_unused]] float rope_cs = 0.f;                           // this thread's entry of the tokens' cos / sin table
         if constexpr (ROPED) {
             if ((int)threadIdx.x < NTOK * rope.n_dims) rope_cs = rope.table[threadIdx.x];
         }
         load_step(ring, s0, true);
+        if constexpr (NORMABLE) {
+            if (sec.norm_w) {                                           // the block sums go behind the image (and the cos / sin table)
+                size_t at = (size_t)NTOK * img;
+                if constexpr (ROPED) at += (size_t)NTOK * rope.n_dims * sizeof(float);
+                norm_apply<WT, NTOK, WGS>(xr, nr, K, sec.norm_eps, sec.norm_y, sec.norm_ldy, gp.writes_workspace && sec.norm_y,
+                                          reinterpret_cast<double *>(lds + ((at + 7) & ~(size_t)7)));
+            }
+        }
         quantize_into_image<WT, NTOK, WGS>(xr, lds, img, NI, K, ws, ws_stride, gp.writes_workspace);
         if constexpr (ROPED) {                                          // behind the image: [token][cos | sin]
             float *tab = reinterpret_cast<float *>(lds + (size_t)NTOK * img);
@@ -1053,7 +1150,9 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
                 if (row < N) {
 #pragma unroll
                     for (int t = 0; t < NTOK; t++) {
-                        y[(int64_t)t * ldy + row + (row >= sec.n_first ? sec.y_off : (int64_t)0)] = res[r][t];
+                        float v = res[r][t];
+                        if (sec.addend) v += sec.addend[(int64_t)t * sec.ld_add + row];
+                        y[(int64_t)t * ldy + row + (row >= sec.n_first ? sec.y_off : (int64_t)0)] = v;
                         if (sec.t16) sec.t16[row * sec.t16_ld + t] = f2h_rne(res[r][t]);
                     }
                 }

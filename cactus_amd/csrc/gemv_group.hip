@@ -16,18 +16,23 @@ struct GroupKernelMat {
     int wtype; int first_block;
     RopeEpilogue rope;                                  // table != nullptr: the member's ROPE node runs in its epilogue
 };
-struct GroupKernelArgs { GroupKernelMat m[GROUP_MAX]; int count; };
+struct GroupKernelArgs { GroupKernelMat m[GROUP_MAX]; int count; GroupNorm norm; };
 
 template <int WT, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE>
-__device__ __forceinline__ void run_member(const GroupKernelMat &m, int64_t K, const float *x, int64_t ldx, uint8_t *ws,
+__device__ __forceinline__ void run_member(const GroupKernelMat &m, const GroupNorm &nm, int64_t K, const float *x, int64_t ldx, uint8_t *ws,
                                            size_t ws_stride, const GridPart gp) {
-    const SecondMatrix sec{INT64_MAX, 0, 0, m.t16, m.t16_ld};
+    SecondMatrix sec = kNoSecond;
+    sec.t16 = m.t16; sec.t16_ld = m.t16_ld;
     if constexpr (ROPE && FUSEQ) {
-        if (m.rope.table) {                                             // uniform over the workgroup; one row per step (pairs)
-            gemv_body<WT, NTOK, 1, WGS, FUSEQ, DEPTH, false, false, true>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, kNoSecond,
-                                                                            gp, m.rope);
-            return;
-        }
+        // the kernel for groups with ROPE epilogues: its bodies may also take the RMS norm of the rows into their prologue
+        // (gemv_body.h: NORMABLE; short rows only: the phased prologue never holds a whole row), one row per step
+        sec.norm_w = nm.w; sec.norm_eps = nm.eps; sec.norm_y = nm.y; sec.norm_ldy = nm.ldy;
+        if (m.rope.table)                                               // uniform over the workgroup
+            gemv_body<WT, NTOK, 1, WGS, FUSEQ, DEPTH, false, false, true, true>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp, m.rope);
+        else
+            gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH, false, false, false, true>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y,
+                                                                                                  m.ldy, sec, gp);
+        return;
     }
     gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
 }
@@ -49,21 +54,21 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
     const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), FUSEQ && blockIdx.x == 0};
     if constexpr (FAMILY == 0) {
         switch (m.wtype) {                                              // uniform over the workgroup
-            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else if constexpr (FAMILY == 1) {
         switch (m.wtype) {
-            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
-            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else {
-        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, K, x, ldx, ws, ws_stride, gp);
+        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp);
     }
 }
 
@@ -161,7 +166,7 @@ bool gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, co
 }
 
 hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const float *x, int64_t ldx, int n, void *ws,
-                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st, bool prepared) {
+                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st, bool prepared, const GroupNorm *norm) {
     if (!gemv_group_applicable(mats, count, K, n, lim, prepared)) return hipErrorInvalidValue;
     const int cus = lim.compute_units > 0 ? lim.compute_units : 256;
     const int fam = gemv_group_family(mats[0].wtype);
@@ -188,7 +193,11 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
         if (r.n_dims > rope_dims) rope_dims = r.n_dims;
         tiles += mats[i].N - ceil_div(mats[i].N, (int64_t)rows_per_step(mats[i].wtype));
     }
-    const size_t lds_bytes = (size_t)n * img + (size_t)n * rope_dims * sizeof(float);
+    size_t lds_bytes = (size_t)n * img + (size_t)n * rope_dims * sizeof(float);
+    if (norm && norm->w) {                                               // only the kernel with ROPE epilogues is built with it
+        if (!rope || K > 256 * NORM_BLOCKS_MAX) return hipErrorInvalidValue;
+        lds_bytes = ((lds_bytes + 7) & ~(size_t)7) + (size_t)n * NORM_BLOCKS_MAX * sizeof(double);   // the block sums, behind image and table
+    }
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     // As the single-matrix launcher: a persistent grid; one 16-wave workgroup per CU while every wave gets at most a
     // couple of tiles (the prologue is then most of the kernel and is paid once per CU), else two 8-wave workgroups.
@@ -223,6 +232,7 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
     }
     GroupKernelArgs ga{};
     ga.count = count;
+    ga.norm = (norm && norm->w) ? *norm : GroupNorm{nullptr, 0.f, nullptr, 0};
     int first = 0;
     for (int i = 0; i < count; i++) {
         ga.m[i] = GroupKernelMat{(const uint8_t *)mats[i].W, mats[i].nb01, mats[i].N, mats[i].y, mats[i].ldy, mats[i].t16,

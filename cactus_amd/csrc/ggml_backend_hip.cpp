@@ -27,7 +27,7 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0}, g_rope_epilogues{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0}, g_rope_epilogues{0}, g_norms_in_prologue{0}, g_residual_adds{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
@@ -612,9 +612,12 @@ int silu_mul_for_consumer(backend_ctx *c, const lm_ggml_cgraph *g, int last, con
 // allocator reuses a node's memory for its consumer only when nothing else reads it (reference ggml-alloc.c in-place
 // rule: one child, no views), so the first node's own result is not needed and the pair runs as one kernel.
 // Returns CHIP_OK and sets fused, or leaves fused false.
+struct held_norm;
+bool norm_can_wait(const lm_ggml_cgraph *g, int mul_index, const lm_ggml_tensor *a, const lm_ggml_tensor *mul, const lm_ggml_tensor *wt);
 int try_fused_pair(backend_ctx *c, const lm_ggml_cgraph *g, int i, const lm_ggml_tensor *node, const lm_ggml_tensor *next, bool &fused,
-                   quantized_key &key) {
+                   quantized_key &key, bool &held) {
     fused = false;
+    held = false;
     if (!next || next->op != LM_GGML_OP_MUL || next->data != node->data || !elementwise_shape_ok(next)) return CHIP_OK;
     const lm_ggml_tensor *other = next->src[0] == node ? next->src[1] : (next->src[1] == node ? next->src[0] : nullptr);
     if (!other || other == node || !same_shape(next, node)) return CHIP_OK;
@@ -626,6 +629,10 @@ int try_fused_pair(backend_ctx *c, const lm_ggml_cgraph *g, int i, const lm_ggml
         float eps;
         std::memcpy(&eps, node->op_params, sizeof(float));
         fused = true;
+        if (norm_can_wait(g, i + 1, a, next, other)) {                     // the projections behind the MUL run the pair
+            held = true;
+            return CHIP_OK;
+        }
         if (const int rc = norm_for_quantized_consumer(c, g, i + 1, (const float *)a->data, lda, nullptr, 0, nullptr, 0, rows, a->ne[0], eps,
                                                        (const float *)other->data, next, ldy, key);
             rc != CHIP_EUNSUPPORTED)
@@ -926,6 +933,46 @@ int rope_partner_index(const lm_ggml_cgraph *g, int i, graph_reads &reads, F ran
     return -1;
 }
 
+// The residual ADD behind a projection (reference cactus/llama-model.cpp build_llama: ffn_inp = lm_ggml_add(cur, inpSA) after wo,
+// cur = lm_ggml_add(cur, ffn_inp) after ffn_down), to be run where the projection's GEMV stores its result (chip_mul_mat_add):
+// the next computing node, adding a tensor of the projection's shape to it; nothing else reads the projection; the sum's
+// rows lie apart from the projection's input and are the other operand's rows or apart from them.  Returns its index or -1.
+int residual_add_index(const lm_ggml_cgraph *g, int i, graph_reads &reads) {
+    const lm_ggml_tensor *mm = g->nodes[i], *w = mm->src[0], *x = mm->src[1];
+    const int j = next_compute_node(g, i);
+    if (j < 0 || (mm->flags & LM_GGML_TENSOR_FLAG_OUTPUT)) return -1;
+    const lm_ggml_tensor *add = g->nodes[j];
+    if (add->op != LM_GGML_OP_ADD || !elementwise_shape_ok(add)) return -1;
+    const lm_ggml_tensor *other = add->src[0] == mm ? add->src[1] : (add->src[1] == mm ? add->src[0] : nullptr);
+    if (!other || other == mm || !same_shape(other, mm) || !same_shape(add, mm) || reads.readers_of(g, mm) != 1) return -1;
+    int64_t rows, ldo, lda;
+    if (!as_rows(other, rows, ldo) || !as_rows(add, rows, lda) || rows != x->ne[1] || !other->data) return -1;
+    if (!chip_mul_mat_add_supported(w->type, w->ne[0], w->ne[1], rows)) return -1;
+    if (!ranges_apart(add, x) || !same_or_disjoint(add->data, lda, other->data, ldo, rows, mm->ne[0])) return -1;
+    return j;
+}
+
+// An RMS_NORM and the MUL with its weight held back for the projections that read the result: they run the two nodes in
+// their prologue (chip_mul_mat_group_rope_norm, chip_mul_mat_pair_silu_mul_norm).  src: the norm's input, out: the MUL node.
+struct held_norm {
+    const lm_ggml_tensor *src = nullptr, *out = nullptr, *weight = nullptr;
+    float eps = 0.f;
+    bool held() const { return out != nullptr; }
+};
+// True when the norm of `a` (RMS_NORM node, then `mul` with the one-row weight `wt`) may wait for the node after the MUL: up
+// to 4 tokens, that node a weight matmul of the MUL's result with a prologue that takes the norm, and the norm's input still
+// whole when that matmul runs (the MUL's rows lie apart from it).
+bool norm_can_wait(const lm_ggml_cgraph *g, int mul_index, const lm_ggml_tensor *a, const lm_ggml_tensor *mul, const lm_ggml_tensor *wt) {
+    const int j = next_compute_node(g, mul_index);
+    if (j < 0 || (mul->flags & LM_GGML_TENSOR_FLAG_OUTPUT)) return false;
+    const lm_ggml_tensor *mm = g->nodes[j];
+    if (mm->op != LM_GGML_OP_MUL_MAT || mm->src[1] != mul || !mul_mat_shape_ok(mm)) return false;
+    const int64_t n = mul->ne[1];
+    if (mul->ne[2] != 1 || mul->ne[3] != 1 || n > 4 || !chip_norm_before_supported(mm->src[0]->type, mul->ne[0], n)) return false;
+    if (((uintptr_t)wt->data & 15) != 0 || ((uintptr_t)mul->data & 15) != 0 || (mul->nb[1] % 16) != 0) return false;
+    return ranges_apart(a, mul) && ranges_apart(wt, mul);
+}
+
 // The ROPE node behind a projection that runs in a group at node i, to be run in that projection's epilogue
 // (chip_mul_mat_group_rope): the projection is read by nothing else, its rows are the ROPE's heads as they lie, and whatever
 // the ROPE writes at node i's place is not in use there.  Returns the ROPE's index and fills rope (the table pointer is left
@@ -978,9 +1025,26 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
     graph_reads reads;
     int rope_done = -1, rope_done_store = -1;         // a ROPE node (and its cache store) that already ran in an earlier ROPE's launch
     int roped_early[CHIP_GROUP_MAX] = {-1, -1, -1, -1};   // ROPE nodes that ran in the epilogue of their projection
+    int add_done = -1;                                // a residual ADD that ran in the store of the projection before it
+    held_norm held;                                   // a norm and its weight MUL waiting for the projections that read them
+    // the held norm as a kernel of its own after all: the matmul that was to run it took a path without that prologue
+    auto run_held_norm = [&]() -> int {
+        if (!held.held()) return CHIP_OK;
+        const lm_ggml_tensor *a = held.src, *out = held.out;
+        held.out = nullptr;
+        return chip_rms_norm_mul((const float *)a->data, (int64_t)(a->nb[1] / 4), out->ne[1], a->ne[0], held.eps, (const float *)held.weight->data,
+                                 nullptr, 0, (float *)out->data, (int64_t)(out->nb[1] / 4), c->stream);
+    };
     for (int i = 0; i < cgraph->n_nodes; i++) {
         lm_ggml_tensor *node = cgraph->nodes[i];
         if (is_view_op(node->op)) continue;
+        if (held.held() && !(node->op == LM_GGML_OP_MUL_MAT && node->src[1] == held.out)) {
+            if (const int rc = run_held_norm(); rc != CHIP_OK) {
+                HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: RMS_NORM held for %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+                return LM_GGML_STATUS_FAILED;
+            }
+        }
+        if (i == add_done) { add_done = -1; continue; }
         // a node that writes into the tensor the workspace was quantized from, or that uses the workspace itself, ends
         // the reuse of the quantized rows (every node is seen here, also those run inside a neighbour's kernel)
         auto writes = [c](const lm_ggml_tensor *t) {
@@ -1029,9 +1093,9 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         }
         if ((node->op == LM_GGML_OP_RMS_NORM || (node->op == LM_GGML_OP_UNARY && node->op_params[0] == LM_GGML_UNARY_OP_SILU)) &&
             elementwise_shape_ok(node) && fusion_enabled()) {
-            bool fused = false;
+            bool fused = false, waits = false;
             quantized_key key;
-            const int rc = try_fused_pair(c, cgraph, i, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused, key);
+            const int rc = try_fused_pair(c, cgraph, i, node, i + 1 < cgraph->n_nodes ? cgraph->nodes[i + 1] : nullptr, fused, key, waits);
             if (rc != CHIP_OK) {
                 HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: %s (op %d, fused with the next node) failed: %s\n", __func__, node->name, node->op,
                         chip_error_string(rc));
@@ -1040,6 +1104,13 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             if (fused) {
                 writes(cgraph->nodes[i + 1]);
                 if (key.valid) c->quantized = key;
+                if (waits) {
+                    const lm_ggml_tensor *mul = cgraph->nodes[i + 1];
+                    held.src = node->src[0];
+                    held.out = mul;
+                    held.weight = mul->src[0] == node ? mul->src[1] : mul->src[0];
+                    std::memcpy(&held.eps, node->op_params, sizeof(float));
+                }
                 g_elementwise_nodes += 2;
                 g_fused_pairs++;
                 i++;
@@ -1221,8 +1292,17 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 if (!kept && chip_mul_mat_pair_silu_mul_supported(w->type, K, N, n) && as_rows(mul, mrows, ldm) && mrows == n && disjoint(mul, x) &&
                     reads.readers_of(cgraph, node) == 1 && reads.readers_of(cgraph, silu) == 1 && reads.readers_of(cgraph, up) == 1) {
                     c->quantized.valid = false;
-                    rc = chip_mul_mat_pair_silu_mul(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)x->data, ldx, n,
-                                                    (float *)mul->data, ldm, c->workspace, c->workspace_size, c->stream);
+                    rc = CHIP_EUNSUPPORTED;
+                    if (held.held() && ranges_apart(mul, held.src)) {     // ffn_norm and its weight MUL in the same launch
+                        const chip_norm_before nb{(const float *)held.weight->data, held.eps, (float *)x->data, ldx};
+                        rc = chip_mul_mat_pair_silu_mul_norm(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)held.src->data,
+                                                             (int64_t)(held.src->nb[1] / 4), n, &nb, (float *)mul->data, ldm, c->workspace,
+                                                             c->workspace_size, c->stream);
+                        if (rc == CHIP_OK) { held.out = nullptr; g_norms_in_prologue++; }
+                    }
+                    if (rc == CHIP_EUNSUPPORTED && (rc = run_held_norm()) == CHIP_OK)
+                        rc = chip_mul_mat_pair_silu_mul(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)x->data, ldx, n,
+                                                        (float *)mul->data, ldm, c->workspace, c->workspace_size, c->stream);
                     if (rc != CHIP_OK) {
                         HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: gated MUL_MAT pair at %s failed: %s\n", __func__, node->name, chip_error_string(rc));
                         return LM_GGML_STATUS_FAILED;
@@ -1312,11 +1392,27 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 rc = CHIP_EUNSUPPORTED;
                 if (any_rope) {
                     q.valid = false;
-                    rc = chip_mul_mat_group_rope(mats, ropes, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
+                    bool apart = held.held();                     // everything the launch writes, apart from the held norm's input
+                    for (int k = 0; apart && k < n_members; k++) {
+                        apart = ranges_apart(cgraph->nodes[members[k]], held.src);
+                        if (rope_node[k] >= 0) apart = apart && ranges_apart(cgraph->nodes[rope_node[k]], held.src);
+                    }
+                    if (apart) {                                  // attn_norm and its weight MUL in the same launch
+                        const chip_norm_before nb{(const float *)held.weight->data, held.eps, (float *)x->data, ldx};
+                        rc = chip_mul_mat_group_rope_norm(mats, ropes, &nb, n_members, K, (const float *)held.src->data,
+                                                          (int64_t)(held.src->nb[1] / 4), n, c->workspace, c->workspace_size, c->stream);
+                        if (rc == CHIP_OK) { held.out = nullptr; g_norms_in_prologue++; }
+                    }
+                    if (rc == CHIP_EUNSUPPORTED && (rc = run_held_norm()) == CHIP_OK)
+                        rc = chip_mul_mat_group_rope(mats, ropes, n_members, K, (const float *)x->data, ldx, n, c->workspace, c->workspace_size, c->stream);
                     if (rc == CHIP_EUNSUPPORTED) {               // not a one-launch group: the ROPE nodes run at their own places
                         any_rope = false;
                         for (int k = 0; k < n_members; k++) { ropes[k] = chip_rope_after{}; rope_node[k] = rope_store[k] = -1; }
                     }
+                }
+                if (!any_rope && (rc = run_held_norm()) != CHIP_OK) {
+                    HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: RMS_NORM held for %s failed: %s\n", __func__, node->name, chip_error_string(rc));
+                    return LM_GGML_STATUS_FAILED;
                 }
                 if (!any_rope) {
                     // more than 4 tokens: the workspace holds x's quantized rows afterwards, or already does (the norm in front
@@ -1382,6 +1478,11 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 continue;
             }
         }
+        if (const int hrc = run_held_norm(); hrc != CHIP_OK) {     // none of the paths below has the norm in its prologue
+            HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: RMS_NORM held for %s failed: %s\n", __func__, node->name, chip_error_string(hrc));
+            return LM_GGML_STATUS_FAILED;
+        }
+        int add_index = -1;
         if (n <= 4 && fusion_enabled() && (store_t = transposed_store_index(cgraph, i)) >= 0 && remember_store(store_t)) {
             lm_ggml_tensor *cp = cgraph->nodes[store_t];
             writes(cp);
@@ -1415,6 +1516,19 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             if (rc == CHIP_OK)
                 rc = chip_mul_mat_run_ws(w->type, w->data, w->nb[1], K, N, n, c->workspace, c->workspace_size, (float *)node->data,
                                          (int64_t)(node->nb[1] / 4), c->stream);
+        } else if (n <= 4 && fusion_enabled() && add_done < 0 && (add_index = residual_add_index(cgraph, i, reads)) >= 0) {
+            // wo / ffn_down and the residual ADD behind them: the GEMV adds the other operand as it stores, into the ADD's rows
+            lm_ggml_tensor *add = cgraph->nodes[add_index];
+            const lm_ggml_tensor *other = add->src[0] == node ? add->src[1] : add->src[0];
+            c->quantized.valid = false;
+            writes(add);
+            rc = chip_mul_mat_add(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (const float *)other->data,
+                                  (int64_t)(other->nb[1] / 4), (float *)add->data, (int64_t)(add->nb[1] / 4), c->workspace, c->workspace_size,
+                                  c->stream);
+            add_done = add_index;
+            g_elementwise_nodes++;
+            g_fused_pairs++;
+            g_residual_adds++;
         } else {
             c->quantized.valid = false;               // up to 4 tokens the GEMV quantizes in its own prologue, into the workspace
             rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
@@ -1426,6 +1540,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         }
         g_mul_mat_nodes++;
     }
+    if (run_held_norm() != CHIP_OK) return LM_GGML_STATUS_FAILED;
     return LM_GGML_STATUS_SUCCESS;
 }
 
@@ -1610,5 +1725,7 @@ unsigned long long lm_ggml_backend_hip_get_head_merges(void) { return g_head_mer
 unsigned long long lm_ggml_backend_hip_get_rope_pairs(void) { return g_rope_pairs.load(); }
 unsigned long long lm_ggml_backend_hip_get_gated_pairs(void) { return g_gated_pairs.load(); }
 unsigned long long lm_ggml_backend_hip_get_rope_epilogues(void) { return g_rope_epilogues.load(); }
+unsigned long long lm_ggml_backend_hip_get_norms_in_prologue(void) { return g_norms_in_prologue.load(); }
+unsigned long long lm_ggml_backend_hip_get_residual_adds(void) { return g_residual_adds.load(); }
 
 }  // extern "C"

@@ -153,9 +153,16 @@ hipError_t launch_gemv_fused_pair(int wtype, const void *W1, const void *W2, siz
                                   int64_t ldx, int n, void *ws, size_t ws_stride, float *y1, float *y2, int64_t ldy,
                                   const DeviceLimits &lim, hipStream_t st);
 // silu(W1 x) * (W2 x) -> y in one launch: the gated FFN's four nodes up to ffn_down's input (shapes as launch_gemv_fused_pair)
+bool gemv_norm_prologue_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim);
+// norm_w != nullptr: the rows x are RMS-normed (norm_eps) and multiplied by norm_w in the prologue; norm_y may receive them
 hipError_t launch_gemv_fused_pair_silu_mul(int wtype, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
                                            int64_t ldx, int n, void *ws, size_t ws_stride, float *y, int64_t ldy,
-                                           const DeviceLimits &lim, hipStream_t st);
+                                           const DeviceLimits &lim, hipStream_t st, const float *norm_w = nullptr, float norm_eps = 0.f,
+                                           float *norm_y = nullptr, int64_t norm_ldy = 0);
+// y = W x + addend (addend [n][N] at ld_add): the GEMV that quantizes in its prologue with the residual ADD in its store
+hipError_t launch_gemv_fused_add(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int n, void *ws,
+                                 size_t ws_stride, const float *addend, int64_t ld_add, float *y, int64_t ldy, const DeviceLimits &lim,
+                                 hipStream_t st);
 // gemv_group.hip: up to GROUP_MAX matrices that read the same activation rows in one launch of the prologue-quantizing
 // GEMV (members of one family: K-quants, 32-value block types, or F16).  t16: optional transposed fp16 copy of a member's
 // output, as launch_gemv_fused_store_t.
@@ -172,6 +179,8 @@ constexpr RopeEpilogue kNoRope = {nullptr, 0, 0, 0, 0, nullptr, 0};
 constexpr int GROUP_MAX = 4;
 struct GroupMat { int wtype; const void *W; size_t nb01; int64_t N; float *y; int64_t ldy; unsigned short *t16; int64_t t16_ld;
                   RopeEpilogue rope = kNoRope; };
+// the RMS norm (and weight MUL) of the rows x in the prologue of a group launch whose members carry ROPE epilogues
+struct GroupNorm { const float *w; float eps; float *y; int64_t ldy; };
 int        gemv_group_family(int wtype);
 bool       gemv_group_applicable(const GroupMat *mats, int count, int64_t K, int n, const DeviceLimits &lim, bool prepared = false);
 // the GEMV over prepared rows for two matrices of one shape in one launch, and with a transposed fp16 copy of the result
@@ -180,7 +189,8 @@ hipError_t launch_gemv_pair(int wtype, const void *W1, const void *W2, size_t nb
 hipError_t launch_gemv_store_t(int wtype, const void *W, size_t nb01, int64_t K, int64_t N, const void *ws, size_t ws_stride, int n,
                                float *y, int64_t ldy, unsigned short *y16t, int64_t ld16, const DeviceLimits &lim, hipStream_t st);
 hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const float *x, int64_t ldx, int n, void *ws,
-                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st, bool prepared = false);
+                             size_t ws_stride, const DeviceLimits &lim, hipStream_t st, bool prepared = false,
+                             const GroupNorm *norm = nullptr);
 // MUL_MAT_ID: every (token, slot) pair is a one-token GEMV on the expert ids[token][slot] names (W + id * nb02), its
 // activation row token * ne11 + slot % ne11, its output row token * n_used + slot.  fused: x is fp32 and is quantized in
 // the prologue; otherwise ws already holds the quantized rows.

@@ -58,7 +58,12 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
     float *ynr = yn ? yn + (size_t)blockIdx.x * ldyn : nullptr;
     const bool vecw = vec && (!w || ((uintptr_t)w & 15) == 0) && (!yn || ((ldyn & 3) == 0 && ((uintptr_t)yn & 15) == 0));
     double sum = 0.0;
-    // rows of up to 8192 values stay in registers between the two passes (same order of additions as the loops below)
+    // Vector paths: the squares are added in the order dev_common.h fixes for a row (chunk, 256-value block, blocks four
+    // apart, four partial sums).  Thread tid's k-th chunk is chunk tid + 256 k, i.e. lane tid % 64 of block tid / 64 + 4 k, so
+    // a wave adds the butterfly totals of its blocks as it walks the row; every lane of a wave takes part in each butterfly
+    // (lanes past the end with 0.0), hence the wave-uniform bounds.  Lane 63 holds the wave's sum.
+    const int64_t wave_first = 4 * (int64_t)(tid & ~63);
+    // rows of up to 8192 values stay in registers between the two passes
     constexpr int RC = 8;
     const bool cached = vecw && ne0 <= 4 * EW_THREADS * RC;
     float4 keep[RC], wk[RC];                                     // wk: the weight row, asked for before the reduction
@@ -68,6 +73,7 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
 #pragma unroll
         for (int k = 0; k < RC; k++) {
             const int64_t i = 4 * tid + (int64_t)k * 4 * EW_THREADS;
+            double d = 0.0;
             if (i < ne0) {
                 float4 v = *reinterpret_cast<const float4 *>(xr + i);
                 if (ADD) {
@@ -77,39 +83,45 @@ __global__ __launch_bounds__(EW_THREADS) void rms_norm_kernel(const float *x, in
                 }
                 keep[k] = v;
                 if (w) wk[k] = *reinterpret_cast<const float4 *>(w + i);
-                sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+                d = norm_chunk_squares(v);
             }
+            if (wave_first + (int64_t)k * 4 * EW_THREADS < ne0) sum += wave_sum_f64_to_lane63(d);
         }
-    } else if (ADD) {
-        const float *br = b + (size_t)blockIdx.x * ldb;
-        float *sr = xs + (size_t)blockIdx.x * ldxs;
-        if (vec) {
-            for (int64_t i = 4 * tid; i < ne0; i += 4 * EW_THREADS) {
+    } else if (vec) {
+        const float *br = ADD ? b + (size_t)blockIdx.x * ldb : nullptr;
+        float *sr = ADD ? xs + (size_t)blockIdx.x * ldxs : nullptr;
+        for (int64_t i0 = wave_first; i0 < ne0; i0 += 4 * EW_THREADS) {
+            const int64_t i = i0 + 4 * (tid & 63);
+            double d = 0.0;
+            if (i < ne0) {
                 float4 v = *reinterpret_cast<const float4 *>(xr + i);
-                const float4 u = *reinterpret_cast<const float4 *>(br + i);
-                v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
-                *reinterpret_cast<float4 *>(sr + i) = v;
-                sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+                if (ADD) {
+                    const float4 u = *reinterpret_cast<const float4 *>(br + i);
+                    v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+                    *reinterpret_cast<float4 *>(sr + i) = v;
+                }
+                d = norm_chunk_squares(v);
             }
-        } else {
+            sum += wave_sum_f64_to_lane63(d);
+        }
+        if (ADD) xr = sr;
+    } else {
+        if (ADD) {
+            const float *br = b + (size_t)blockIdx.x * ldb;
+            float *sr = xs + (size_t)blockIdx.x * ldxs;
             for (int64_t i = tid; i < ne0; i += EW_THREADS) {
                 const float v = xr[i] + br[i];
                 sr[i] = v;
                 sum += (double)(v * v);
             }
+            xr = sr;
+        } else {
+            for (int64_t i = tid; i < ne0; i += EW_THREADS) sum += (double)(xr[i] * xr[i]);
         }
-        xr = sr;
-    } else if (vec) {
-        for (int64_t i = 4 * tid; i < ne0; i += 4 * EW_THREADS) {
-            const float4 v = *reinterpret_cast<const float4 *>(xr + i);
-            sum += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
-        }
-    } else {
-        for (int64_t i = tid; i < ne0; i += EW_THREADS) sum += (double)(xr[i] * xr[i]);
-    }
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    if ((tid & 63) == 0) part[tid >> 6] = sum;
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);      // rows that are not 16-byte aligned: element by element
+    }
+    if ((tid & 63) == 63) part[tid >> 6] = sum;
     __syncthreads();
     double total = 0.0;
 #pragma unroll

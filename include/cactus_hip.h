@@ -214,6 +214,37 @@ typedef struct chip_rope_after {
 } chip_rope_after;
 CHIP_API int chip_mul_mat_group_rope(const chip_mat *mats, const chip_rope_after *ropes, int count, int64_t K, const float *x,
                                      int64_t ldx, int64_t n, void *workspace, size_t workspace_bytes, void *stream);
+/* The RMS norm and the MUL with the norm weight that precede a projection, run in the projection's prologue (reference
+ * cactus/llama-graph.cpp build_norm, LLM_NORM_RMS: lm_ggml_rms_norm then lm_ggml_mul with the weight; lm_ggml_compute_forward_rms_norm_f32,
+ * ggml-cpu/ops.cpp).  x is then the norm's input; every workgroup norms the rows it has loaded for quantizing, with the
+ * additions in chip_rms_norm_mul's order, so every value has the bits of chip_rms_norm_mul followed by the plain call.
+ * y (optional) receives the normed rows, as the MUL node's tensor would hold them. */
+typedef struct chip_norm_before {
+    const float *w;          /* the norm weight, K floats, 16-byte aligned */
+    float        eps;
+    float       *y;          /* [n][K] at row stride ldy (16-byte aligned, ldy a multiple of 4), or NULL */
+    int64_t      ldy;
+} chip_norm_before;
+/* chip_mul_mat_group_rope on rows normed in the prologue.  CHIP_EUNSUPPORTED where chip_mul_mat_group_rope is, and for rows
+ * the prologue does not hold whole (K-quant rows of more than two steps, K > 8192): nothing written then. */
+CHIP_API int chip_mul_mat_group_rope_norm(const chip_mat *mats, const chip_rope_after *ropes, const chip_norm_before *norm, int count,
+                                          int64_t K, const float *x, int64_t ldx, int64_t n, void *workspace, size_t workspace_bytes,
+                                          void *stream);
+/* chip_mul_mat_pair_silu_mul on rows normed in the prologue (ffn_norm in front of ffn_gate / ffn_up); same conditions. */
+CHIP_API int chip_mul_mat_pair_silu_mul_norm(int type, const void *W1, const void *W2, size_t nb01, int64_t K, int64_t N, const float *x,
+                                             int64_t ldx, int64_t n, const chip_norm_before *norm, float *y, int64_t ldy, void *workspace,
+                                             size_t workspace_bytes, void *stream);
+/* 1 when the two calls above take rows of K values of this weight type at n tokens */
+CHIP_API int chip_norm_before_supported(int type, int64_t K, int64_t n);
+/* y = W x + addend: the residual ADD that follows wo and ffn_down (reference cactus/llama-model.cpp build_llama: ffn_inp =
+ * lm_ggml_add(cur, inpSA), cur = lm_ggml_add(cur, ffn_inp)) done where the GEMV stores its result.  addend [n][N] at row stride
+ * ld_add; it may be y itself (same pointer and stride) or lie apart from it.  Bits of chip_mul_mat followed by chip_add
+ * (matmul result first operand).  One launch, 1, 2 or 4 tokens where chip_mul_mat quantizes in its prologue
+ * (chip_mul_mat_add_supported); CHIP_EUNSUPPORTED otherwise, nothing written. */
+CHIP_API int chip_mul_mat_add_supported(int type, int64_t K, int64_t N, int64_t n);
+CHIP_API int chip_mul_mat_add(int type, const void *W, size_t nb01, int64_t K, int64_t N, const float *x, int64_t ldx, int64_t n,
+                              const float *addend, int64_t ld_add, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                              void *stream);
 /* The same over rows the workspace already holds - Phase B of the op alone (ggml-cpu/ggml-cpu.c:1380-1448) for a group, as
  * chip_mul_mat_run is for one matrix: the rows were written by chip_mul_mat_prepare or by the kernel that produced the
  * activations (chip_rms_norm_quantized, chip_silu_mul_quantized).  Up to 4 tokens and members of one family: one launch of

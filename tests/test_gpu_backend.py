@@ -457,17 +457,24 @@ def test_ffn_block_stays_on_the_device(host, orc, n):
     skipped_before = blib.lm_ggml_backend_hip_get_quantizers_skipped()
     blib.lm_ggml_backend_hip_get_gated_pairs.restype = C.c_ulonglong
     gated_before = blib.lm_ggml_backend_hip_get_gated_pairs()
+    blib.lm_ggml_backend_hip_get_norms_in_prologue.restype = C.c_ulonglong
+    norms_before = blib.lm_ggml_backend_hip_get_norms_in_prologue()
+    blib.lm_ggml_backend_hip_get_residual_adds.restype = C.c_ulonglong
+    adds_before = blib.lm_ggml_backend_hip_get_residual_adds()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     # norm + weight ran as one kernel (the allocator writes the MUL over its only producer); SiLU and its MUL are not
     # neighbours in the node order (the up projection sits between them): the SiLU waits for that matmul and runs in the
     # MUL's kernel
     # 5 tokens: the norm leaves its result quantized in the workspace, so neither gate nor up runs the quantizer, and
     # SiLU * up leaves its result quantized for ffn_down, which runs no quantizer of its own.
-    # 2 tokens: gate, SiLU, up and the MUL run as one launch of the GEMV that quantizes in its prologue (three joins), and
-    # ffn_down's GEMV quantizes in its own prologue.
-    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == (2 if n > 4 else 4)
+    # 2 tokens: gate, SiLU, up and the MUL run as one launch of the GEMV that quantizes in its prologue (three joins), with
+    # the norm and its weight MUL (one join) in that prologue too; ffn_down's GEMV quantizes in its own prologue and adds the
+    # residual as it stores (one join): two launches for the eight nodes.
+    assert blib.lm_ggml_backend_hip_get_fused_pairs() - fused_before == (2 if n > 4 else 5)
     assert blib.lm_ggml_backend_hip_get_quantizers_skipped() - skipped_before == (3 if n > 4 else 0)
     assert blib.lm_ggml_backend_hip_get_gated_pairs() - gated_before == (0 if n > 4 else 1)
+    assert blib.lm_ggml_backend_hip_get_norms_in_prologue() - norms_before == (0 if n > 4 else 1)
+    assert blib.lm_ggml_backend_hip_get_residual_adds() - adds_before == (0 if n > 4 else 1)
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
     for t in (cur, up, gate, act, down, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
@@ -799,8 +806,8 @@ def test_attention_side_ops_outside_the_restated_cases_are_declined(host):
 
 @pytest.mark.parametrize("n_tokens", [5, 2])
 def test_attention_block_stays_on_the_device(host, orc, n_tokens):
-    """A whole attention block as llama.cpp builds it without flash attention (reference llama-graph.cpp build_attn /
-    build_attn_mha :1060-1170, llama-kv-cache.cpp get_k / get_v / cpy_k / cpy_v): q/k/v projections, RoPE, the cache stores,
+    """A whole attention block as llama.cpp builds it without flash attention (reference llama-graph.cpp build_norm, build_attn /
+    build_attn_mha :1060-1170, llama-kv-cache.cpp get_k / get_v / cpy_k / cpy_v): attn_norm, q/k/v projections, RoPE, the cache stores,
     kq over the F16 K cache, masked soft-max, kqv over the transposed F16 V cache, the merge of the heads, the output
     projection and the residual.  Weights and caches live in HIP buffers: the reference scheduler puts everything into
     one HIP split."""
@@ -813,6 +820,8 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     wv = orc.quantize_weights(O.Q6_K, common.weights_f32(43, n_embd_kv, H))
     wo = orc.quantize_weights(O.Q4_K, common.weights_f32(44, H, n_head * hd))
     x = common.activations_f32(45, n_tokens, H)
+    wn = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    eps = 1e-5
     pos = np.arange(head, head + n_tokens, dtype=np.int32)
     mask = np.full((8, n_kv), -np.inf, np.float32)
     for i in range(n_tokens):
@@ -831,13 +840,14 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     hip = L.lm_ggml_backend_dev_init(dev, None)
     cpu = L.lm_ggml_backend_cpu_init()
     wctx = host.context(with_graph=False)
+    tn = L.lm_ggml_new_tensor_1d(wctx, O.F32, H)
     twq = host.tensor_2d(wctx, O.Q4_K, H, n_head * hd, "wq")
     twk = host.tensor_2d(wctx, O.Q4_K, H, n_embd_kv, "wk")
     twv = host.tensor_2d(wctx, O.Q6_K, H, n_embd_kv, "wv")
     two = host.tensor_2d(wctx, O.Q4_K, n_head * hd, H, "wo")
     wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
     L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
-    for t, a in ((twq, wq), (twk, wk), (twv, wv), (two, wo)):
+    for t, a in ((twq, wq), (twk, wk), (twv, wv), (two, wo), (tn, wn)):
         host.set(t, a)
     cctx = host.context(with_graph=False)
     kc = host.tensor_2d(cctx, O.F16, n_embd_kv, kv_size, "cache_k")
@@ -854,9 +864,10 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
         L.lm_ggml_set_input(t)
     rope = lambda t, nh: L.lm_ggml_rope_ext(ctx, L.lm_ggml_reshape_3d(ctx, t, hd, nh, n_tokens), tpos, None, hd, 2, 4096, 10000.0, 1.0,
                                          0.0, 1.0, 32.0, 1.0)
-    q = rope(L.lm_ggml_mul_mat(ctx, twq, tx), n_head)
-    k = rope(L.lm_ggml_mul_mat(ctx, twk, tx), n_head_kv)
-    v = L.lm_ggml_mul_mat(ctx, twv, tx)
+    cur = L.lm_ggml_mul(ctx, L.lm_ggml_rms_norm(ctx, tx, eps), tn)
+    q = rope(L.lm_ggml_mul_mat(ctx, twq, cur), n_head)
+    k = rope(L.lm_ggml_mul_mat(ctx, twk, cur), n_head_kv)
+    v = L.lm_ggml_mul_mat(ctx, twv, cur)
     k_store = L.lm_ggml_cpy(ctx, k, L.lm_ggml_view_1d(ctx, kc, n_tokens * n_embd_kv, 2 * n_embd_kv * head))
     v_store = L.lm_ggml_cpy(ctx, L.lm_ggml_transpose(ctx, v), L.lm_ggml_view_2d(ctx, vc, n_tokens, n_embd_kv, kv_size * 2, head * 2))
     kview = L.lm_ggml_view_3d(ctx, kc, hd, n_head_kv, n_kv, 2 * hd, 2 * n_embd_kv, 0)
@@ -889,6 +900,10 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     pairs_before = blib.lm_ggml_backend_hip_get_rope_pairs()
     blib.lm_ggml_backend_hip_get_rope_epilogues.restype = C.c_ulonglong
     epilogues_before = blib.lm_ggml_backend_hip_get_rope_epilogues()
+    blib.lm_ggml_backend_hip_get_residual_adds.restype = C.c_ulonglong
+    adds_before = blib.lm_ggml_backend_hip_get_residual_adds()
+    blib.lm_ggml_backend_hip_get_norms_in_prologue.restype = C.c_ulonglong
+    norms_before = blib.lm_ggml_backend_hip_get_norms_in_prologue()
     assert L.lm_ggml_backend_sched_graph_compute(sched, g) == 0
     assert blib.lm_ggml_backend_hip_get_rope_tables() - tables_before == 1      # Q and K share one cos / sin table
     # The K store ran in the kernel of K's RoPE.  With up to 4 tokens the transposed V store ran in the V projection's
@@ -901,18 +916,24 @@ def test_attention_block_stays_on_the_device(host, orc, n_tokens):
     pairs = blib.lm_ggml_backend_hip_get_rope_pairs() - pairs_before
     epilogues = blib.lm_ggml_backend_hip_get_rope_epilogues() - epilogues_before
     assert (epilogues, pairs) == ((0, 0) if n_tokens > 4 else (2, 0)), (epilogues, pairs, grouped)
-    assert fused == (1 if n_tokens > 4 else 2 + max(grouped - 1, 0) + epilogues), (fused, grouped, epilogues)
+    adds = blib.lm_ggml_backend_hip_get_residual_adds() - adds_before        # up to 4 tokens wo's GEMV adds the residual as it stores
+    assert adds == (0 if n_tokens > 4 else 1), adds
+    # attn_norm and its weight MUL are one join at every token count; up to 4 tokens they ran in the prologue of the group launch
+    norms = blib.lm_ggml_backend_hip_get_norms_in_prologue() - norms_before
+    assert norms == (0 if n_tokens > 4 else 1), norms
+    assert fused == 1 + (1 if n_tokens > 4 else 2 + max(grouped - 1, 0) + epilogues + adds), (fused, grouped, epilogues, adds)
     assert L.lm_ggml_backend_sched_get_n_splits(sched) == 1
-    for t in (q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
+    for t in (cur, q, k, v, k_store, v_store, kq, sm, kqv, merged, out):
         assert L.lm_ggml_backend_sched_get_tensor_backend(sched, t) == hip
     y = host.get(out, np.float32, (n_tokens, H))
     y_kc = host.get(kc, np.float16, (kv_size, n_embd_kv))
     y_vc = host.get(vc, np.float16, (n_embd_kv, kv_size))
 
     # the same chain on the oracle
-    q_ = orc.rope(orc.mul_mat(O.Q4_K, wq, x)["y"].reshape(n_tokens, n_head, hd), pos, hd, 2)
-    k_ = orc.rope(orc.mul_mat(O.Q4_K, wk, x)["y"].reshape(n_tokens, n_head_kv, hd), pos, hd, 2)
-    v_ = orc.mul_mat(O.Q6_K, wv, x)["y"]
+    c_ = orc.rms_norm(x, eps) * wn
+    q_ = orc.rope(orc.mul_mat(O.Q4_K, wq, c_)["y"].reshape(n_tokens, n_head, hd), pos, hd, 2)
+    k_ = orc.rope(orc.mul_mat(O.Q4_K, wk, c_)["y"].reshape(n_tokens, n_head_kv, hd), pos, hd, 2)
+    v_ = orc.mul_mat(O.Q6_K, wv, c_)["y"]
     kc_ = kc0.copy()
     kc_[head:head + n_tokens] = k_.reshape(n_tokens, n_embd_kv).astype(np.float16)
     vc_ = vc0.copy()

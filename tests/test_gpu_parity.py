@@ -410,6 +410,86 @@ def test_gated_pair_equals_the_pair_and_silu_mul(dev, wt, K, N):
     assert dev.lib.chip_mul_mat_pair_silu_mul(wt, d.ptr, d.ptr, 16, K, N, d.ptr, K, 3, d.ptr, N, d.ptr, 4096, None) == ca.CHIP_EUNSUPPORTED
 
 
+def norm_weight(seed, K):
+    return (1.0 + 0.25 * np.random.default_rng(seed).standard_normal(K)).astype(np.float32)
+
+
+@pytest.mark.parametrize("types,K,n_head,n_head_kv,hd,n_dims,mode", GROUP_ROPE_CASES)
+def test_group_with_the_norm_in_its_prologue_equals_norm_then_group(dev, types, K, n_head, n_head_kv, hd, n_dims, mode):
+    """chip_mul_mat_group_rope_norm (attn_norm, its weight MUL, wq / wk / wv, both ROPE nodes and the K cache store in one
+    launch): every value, the normed rows included, bit for bit what chip_rms_norm_mul followed by chip_mul_mat_group_rope
+    gives."""
+    members = [(types[0], quantized_weights(types[0], K + 1, n_head * hd, K)), (types[1], quantized_weights(types[1], K + 2, n_head_kv * hd, K)),
+               (types[2], quantized_weights(types[2], K + 3, n_head_kv * hd, K))]
+    w = norm_weight(K, K)
+    ropes = [(hd, n_dims, mode, ("f32",)), (hd, n_dims, mode, ("f32", "f16")), None]
+    for n in (1, 2, 4):
+        x = common.activations_f32(K + n, n, K) * np.float32(3.0)
+        pos = np.array([37, 0, 4095, 100000][:n], np.int32)
+        assert dev.lib.chip_norm_before_supported(types[0], K, n) == 1
+        normed = dev.rms_norm_mul(x, w, 1e-5)
+        rc, want = dev.mul_mat_group_rope(members, normed, pos, ropes, freq_base=500000.0)
+        rc, got = dev.mul_mat_group_rope(members, x, pos, ropes, freq_base=500000.0, norm=(w, 1e-5))
+        assert got[3]["normed"].tobytes() == normed.tobytes(), n
+        assert got[0]["f32"].tobytes() == want[0]["f32"].tobytes(), n
+        assert got[1]["f32"].tobytes() == want[1]["f32"].tobytes() and got[1]["f16"].tobytes() == want[1]["f16"].tobytes(), n
+        assert got[2]["y"].tobytes() == want[2]["y"].tobytes(), n
+
+
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N", [(1024, 336), (4096, 14336), (256, 8), (8192, 1032)])
+def test_gated_pair_with_the_norm_in_its_prologue(dev, wt, K, N):
+    """chip_mul_mat_pair_silu_mul_norm (ffn_norm, its weight MUL and the gated pair in one launch): bit for bit chip_rms_norm_mul
+    followed by chip_mul_mat_pair_silu_mul; rows the prologue does not hold whole are declined."""
+    import cactus_amd as ca
+    if (K, N) == (4096, 14336) and wt not in (O.Q4_K, O.Q4_0):
+        return
+    w1 = quantized_weights(wt, K + N, N, K)
+    w2 = quantized_weights(wt, K + N + 1, N, K)
+    w = norm_weight(N, K)
+    for n in (1, 2, 4):
+        if not dev.lib.chip_mul_mat_pair_silu_mul_supported(wt, K, N, n):
+            assert n * K > 16384
+            continue
+        x = common.activations_f32(K + n, n, K) * np.float32(0.25)
+        assert dev.lib.chip_norm_before_supported(wt, K, n) == 1
+        normed = dev.rms_norm_mul(x, w, 1e-6)
+        want = dev.mul_mat_pair_silu_mul(wt, w1, w2, normed)
+        got, got_normed = dev.mul_mat_pair_silu_mul(wt, w1, w2, x, norm=(w, 1e-6))
+        assert got_normed.tobytes() == normed.tobytes(), n
+        assert got.tobytes() == want.tobytes(), n
+    assert dev.lib.chip_norm_before_supported(O.Q4_K, 14336, 1) == 0           # the image of such a row is built a step's part at a time
+    assert dev.lib.chip_norm_before_supported(wt, K, 3) == 0
+    d = dev.alloc(4096)
+    nb = ca.NormBefore(d.ptr, 1e-6, None, 0)
+    import ctypes
+    assert dev.lib.chip_mul_mat_pair_silu_mul_norm(O.Q4_K, d.ptr, d.ptr, 8064, 14336, 8, d.ptr, 14336, 1, ctypes.byref(nb), d.ptr, 8, d.ptr,
+                                                   65536, None) == ca.CHIP_EUNSUPPORTED
+
+
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("K,N", [(1024, 333), (4096, 4096), (14336, 4096), (256, 7)])
+def test_matmul_with_the_residual_add_in_its_store(dev, wt, K, N):
+    """chip_mul_mat_add (wo / ffn_down and the residual ADD behind them in one launch): bit for bit chip_mul_mat followed by
+    chip_add, with the result written apart from the addend and over it."""
+    import cactus_amd as ca
+    if K == 14336 and wt not in (O.Q4_K, O.Q6_K, O.Q8_0):
+        return
+    W = quantized_weights(wt, K + N, N, K)
+    for n in (1, 2, 4):
+        if not dev.lib.chip_mul_mat_add_supported(wt, K, N, n):
+            assert n * K > 16384
+            continue
+        x = common.activations_f32(K + n, n, K)
+        b = common.activations_f32(N + n, n, N) * np.float32(5.0)
+        want = dev.binary("add", dev.mul_mat(wt, W, x), b)
+        assert dev.mul_mat_add(wt, W, x, b).tobytes() == want.tobytes(), n
+        assert dev.mul_mat_add(wt, W, x, b, in_place=True).tobytes() == want.tobytes(), n
+    assert dev.lib.chip_mul_mat_add_supported(wt, K, N, 3) == 0
+    d = dev.alloc(4096)
+    assert dev.lib.chip_mul_mat_add(wt, d.ptr, 16, K, N, d.ptr, K, 8, d.ptr, N, d.ptr, N, d.ptr, 4096, None) == ca.CHIP_EUNSUPPORTED
+
+
 @pytest.mark.parametrize("wt,K,N", [(O.Q4_K, 4096, 8192), (O.Q4_K, 4096, 14336), (O.Q5_K, 2048, 16400), (O.Q4_K, 14336, 4096)],
                          ids=["q4_K-8192x4096", "q4_K-14336x4096", "q5_K-16400x2048", "q4_K-4096x14336"])
 def test_mul_mat_pair_on_the_matrix_cores(dev, orc, wt, K, N):
