@@ -24,14 +24,13 @@
 
 namespace chip {
 
-template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED, bool GATED = false>
+// NORMED (gated pair only): the RMS norm of the input rows and the MUL with its weight in the prologue (gemv_body.h)
+template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED, bool GATED = false, bool NORMED = false>
 __global__ __launch_bounds__(WGS) void gemv_kernel(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                                    const float *__restrict__ x, int64_t ldx,
                                                    uint8_t *__restrict__ ws, size_t ws_stride,
                                                    float *__restrict__ y, int64_t ldy, SecondMatrix sec) {
-    // the gated pair may also take the RMS norm of its input rows into its prologue (gemv_body.h: NORMABLE)
-    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED, GATED, false, GATED && FUSEQ && !PHASED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec,
-                                                                                                whole_grid());
+    gemv_body<WT, NTOK, R, WGS, FUSEQ, DEPTH, PHASED, GATED, false, NORMED>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, sec, whole_grid());
 }
 
 // LM_GGML_OP_MUL_MAT_ID (reference ggml-cpu/ggml-cpu.c:1460-1710): blockIdx.y is a (token, slot) pair; its expert
@@ -87,7 +86,8 @@ static hipError_t launch_depth(const void *W, size_t nb01, int64_t K, int64_t N,
     }
     static LdsGrant grant;
     if constexpr (FUSEQ) {                                                // the gated pair exists with the quantizing prologue only
-        static LdsGrant grant_gated;
+        static LdsGrant grant_gated, grant_normed;
+        if (sec.gated && sec.norm_w) return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false, true, true>, grant_normed);
         if (sec.gated) return launch(gemv_kernel<WT, NTOK, R, WGS, FUSEQ, DEPTH, false, true>, grant_gated);
     } else {
         if (sec.gated) return hipErrorInvalidValue;
@@ -263,7 +263,7 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
     return (size_t)n * img <= (size_t)lim.max_lds_per_block;
 }
 
-// The RMS norm of the rows in the prologue (gemv_body.h: NORMABLE): the prologue that holds whole rows in registers, i.e.
+// The RMS norm of the rows in the prologue (gemv_body.h: NORMED): the prologue that holds whole rows in registers, i.e.
 // not the one that builds the image a step's part at a time, and rows of at most NORM_BLOCKS_MAX blocks of 256 values.
 bool gemv_norm_prologue_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim) {
     if (!gemv_fused_applicable(wtype, K, n, lim) || K > 256 * NORM_BLOCKS_MAX) return false;

@@ -666,15 +666,15 @@ constexpr int FUSE_MAX_VALUES = 16384;                     // n * K limit of the
 // 8 lanes per 32-block) or super-block j*(WGS/64) + wave (Q8_K: one wave per 256 values).  n * K <= FUSE_MAX_VALUES
 // guarantees PER slots suffice; the loops stop at the first slot index that is out of range for the whole group.
 constexpr int FUSE_ILP = 2;
-template <int NTOK, int WGS> struct XRegs {
-    static constexpr int PER = FUSE_MAX_VALUES / 4 / WGS / NTOK;
+template <int NTOK, int WGS, int MAXV = FUSE_MAX_VALUES> struct XRegs {      // MAXV: the n * K the registers are sized for
+    static constexpr int PER = MAXV / 4 / WGS / NTOK > 0 ? MAXV / 4 / WGS / NTOK : 1;
     float4 v[NTOK][PER];
 };
 
-template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void xload(XRegs<NTOK, WGS> &xr, const float *__restrict__ x, int64_t ldx, int64_t K) {
+template <int WT, int NTOK, int WGS, int MAXV>
+__device__ __forceinline__ void xload(XRegs<NTOK, WGS, MAXV> &xr, const float *__restrict__ x, int64_t ldx, int64_t K) {
     using T = Traits<WT>;
-    constexpr int PER = XRegs<NTOK, WGS>::PER;
+    constexpr int PER = XRegs<NTOK, WGS, MAXV>::PER;
     if constexpr (T::ACT == T_Q8_0 || T::ACT == T_F16) {
         const int nchunk = (int)(K / 4);                                // float4 chunks per token
 #pragma unroll
@@ -701,12 +701,12 @@ __device__ __forceinline__ void xload(XRegs<NTOK, WGS> &xr, const float *__restr
 
 // slot_lo, slot_hi (Q8_K activations only): the register slots [slot_lo, slot_hi) of every token, i.e. super-blocks
 // slot * (WGS / 64) .. - the caller may build the image a weight step's worth at a time.
-template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS> &xr, uint8_t *lds, size_t img, int NI, int64_t K,
+template <int WT, int NTOK, int WGS, int MAXV>
+__device__ __forceinline__ void quantize_into_image(const XRegs<NTOK, WGS, MAXV> &xr, uint8_t *lds, size_t img, int NI, int64_t K,
                                                     uint8_t *__restrict__ ws, size_t ws_stride, bool first_block,
-                                                    int slot_lo = 0, int slot_hi = XRegs<NTOK, WGS>::PER) {
+                                                    int slot_lo = 0, int slot_hi = XRegs<NTOK, WGS, MAXV>::PER) {
     using T = Traits<WT>;
-    constexpr int PER = XRegs<NTOK, WGS>::PER;
+    constexpr int PER = XRegs<NTOK, WGS, MAXV>::PER;
     const bool dump = first_block && ws != nullptr;
     if constexpr (T::ACT == T_F16) {
         // plain conversion: four floats -> four halves (round to nearest even), 8 bytes into the image
@@ -898,10 +898,12 @@ template <int WT, int WGS> __device__ __forceinline__ int xreg_chunk(int j, int6
 template <int WGS> __device__ __forceinline__ int xreg_block_first_chunk(int j) {
     return j * WGS + ((int)threadIdx.x & ~63);            // both layouts: slot j of wave w starts at chunk j * WGS + 64 w
 }
-// (rows of at most 256 * NORM_BLOCKS_MAX values: the first NPER slots of a token)
+// A kernel with the norm takes rows of at most 256 * NORM_BLOCKS_MAX values and sizes its registers for that.
+template <int NTOK> constexpr int norm_max_values() {
+    return 256 * NORM_BLOCKS_MAX * NTOK < FUSE_MAX_VALUES ? 256 * NORM_BLOCKS_MAX * NTOK : FUSE_MAX_VALUES;
+}
 template <int WT, int NTOK, int WGS> struct NormRegs {
-    static constexpr int FULL = XRegs<NTOK, WGS>::PER, CAP = 64 * NORM_BLOCKS_MAX / WGS > 0 ? 64 * NORM_BLOCKS_MAX / WGS : 1;
-    static constexpr int NPER = FULL < CAP ? FULL : CAP;
+    static constexpr int NPER = XRegs<NTOK, WGS, norm_max_values<NTOK>()>::PER;
     float4 w[NPER];
 };
 template <int WT, int NTOK, int WGS>
@@ -914,7 +916,7 @@ __device__ __forceinline__ void norm_issue(NormRegs<WT, NTOK, WGS> &nr, const fl
     }
 }
 template <int WT, int NTOK, int WGS>
-__device__ __forceinline__ void norm_apply(XRegs<NTOK, WGS> &xr, const NormRegs<WT, NTOK, WGS> &nr, int64_t K, float eps, float *y,
+__device__ __forceinline__ void norm_apply(XRegs<NTOK, WGS, norm_max_values<NTOK>()> &xr, const NormRegs<WT, NTOK, WGS> &nr, int64_t K, float eps, float *y,
                                            int64_t ldy, bool store, double *B) {
     constexpr int PER = NormRegs<WT, NTOK, WGS>::NPER;
     const int chunks = (int)(K / 4), blocks = (chunks + 63) >> 6;
@@ -968,7 +970,7 @@ __device__ __forceinline__ GridPart whole_grid() { return GridPart{(int64_t)bloc
 // LLM_FFN_SILU with LLM_FFN_PAR), with lm_ggml_vec_silu_f32's arithmetic; the two projections themselves are not stored.
 // addend: a tensor of y's shape added to every output as it is stored (the residual ADD that follows wo and ffn_down, reference
 // llama-model.cpp build_llama: ffn_inp = add(cur, inpSA), cur = add(cur, ffn_inp)): y = W x + addend, one IEEE addition as the
-// ADD node's.  norm_w (kernels built NORMABLE only): the rows x are RMS-normed and multiplied by the weight row norm_w in the
+// ADD node's.  norm_w (kernels built NORMED, which always have one): the rows x are RMS-normed and multiplied by the weight row norm_w in the
 // prologue, before they are quantized - the RMS_NORM and MUL nodes in front of the projections (build_norm, llama-graph.cpp:527-560)
 // - with rms_norm_kernel's arithmetic and order of additions; norm_y, if given, receives the normed rows (workgroup 0 stores them).
 struct SecondMatrix {
@@ -980,14 +982,14 @@ constexpr SecondMatrix kNoSecond = {INT64_MAX, 0, 0, nullptr, 0, 0, nullptr, 0, 
 
 
 template <int WT, int NTOK, int R, int WGS, bool FUSEQ, int DEPTH, bool PHASED = false, bool GATED = false, bool ROPED = false,
-          bool NORMABLE = false>
+          bool NORMED = false>
 __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t nb01, int64_t K, int64_t N,
                                           const float *__restrict__ x, int64_t ldx,
                                           uint8_t *__restrict__ ws, size_t ws_stride,
                                           float *__restrict__ y, int64_t ldy, const SecondMatrix sec,
                                           const GridPart gp, const RopeEpilogue rope = kNoRope) {
     static_assert(!ROPED || (R == 1 && !GATED && !PHASED && FUSEQ), "the pair walk of the rotated rows takes one row per step");
-    static_assert(!NORMABLE || (FUSEQ && !PHASED), "the norm runs on the whole row in the prologue's registers");
+    static_assert(!NORMED || (FUSEQ && !PHASED), "the norm runs on the whole row in the prologue's registers");
     using T = Traits<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     static_assert(DEPTH == 1, "one step of weight loads is in flight beyond the one being computed");
@@ -1065,24 +1067,21 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, size_t 
         load_step(ring, s0, true);
         quantize_into_image<WT, NTOK, WGS>(xr_parts, lds, img, NI, K, ws, ws_stride, gp.writes_workspace, 0, SPS);
     } else if constexpr (FUSEQ) {
-        XRegs<NTOK, WGS> xr;
+        // NORMED: a kernel of its own (the launcher picks it when there is a norm), with registers for the shorter rows it takes
+        XRegs<NTOK, WGS, (NORMED ? norm_max_values<NTOK>() : FUSE_MAX_VALUES)> xr;
         xload<WT, NTOK, WGS>(xr, x, ldx, K);
         [[maybe_unused]] NormRegs<WT, NTOK, WGS> nr;
-        if constexpr (NORMABLE) {
-            if (sec.norm_w) norm_issue<WT, NTOK, WGS>(nr, sec.norm_w, K);  // uniform; requested before the weights, needed before them
-        }
+        if constexpr (NORMED) norm_issue<WT, NTOK, WGS>(nr, sec.norm_w, K);   // requested before the weights, needed before them
         [[maybe_unused]] float rope_cs = 0.f;                           // this thread's entry of the tokens' cos / sin table
         if constexpr (ROPED) {
             if ((int)threadIdx.x < NTOK * rope.n_dims) rope_cs = rope.table[threadIdx.x];
         }
         load_step(ring, s0, true);
-        if constexpr (NORMABLE) {
-            if (sec.norm_w) {                                           // the block sums go behind the image (and the cos / sin table)
-                size_t at = (size_t)NTOK * img;
-                if constexpr (ROPED) at += (size_t)NTOK * rope.n_dims * sizeof(float);
-                norm_apply<WT, NTOK, WGS>(xr, nr, K, sec.norm_eps, sec.norm_y, sec.norm_ldy, gp.writes_workspace && sec.norm_y,
-                                          reinterpret_cast<double *>(lds + ((at + 7) & ~(size_t)7)));
-            }
+        if constexpr (NORMED) {                                         // the block sums go behind the image (and the cos / sin table)
+            size_t at = (size_t)NTOK * img;
+            if constexpr (ROPED) at += (size_t)NTOK * rope.n_dims * sizeof(float);
+            norm_apply<WT, NTOK, WGS>(xr, nr, K, sec.norm_eps, sec.norm_y, sec.norm_ldy, gp.writes_workspace && sec.norm_y,
+                                      reinterpret_cast<double *>(lds + ((at + 7) & ~(size_t)7)));
         }
         quantize_into_image<WT, NTOK, WGS>(xr, lds, img, NI, K, ws, ws_stride, gp.writes_workspace);
         if constexpr (ROPED) {                                          // behind the image: [token][cos | sin]

@@ -18,20 +18,21 @@ struct GroupKernelMat {
 };
 struct GroupKernelArgs { GroupKernelMat m[GROUP_MAX]; int count; GroupNorm norm; };
 
-template <int WT, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE>
+template <int WT, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE, bool NORMED>
 __device__ __forceinline__ void run_member(const GroupKernelMat &m, const GroupNorm &nm, int64_t K, const float *x, int64_t ldx, uint8_t *ws,
                                            size_t ws_stride, const GridPart gp) {
     SecondMatrix sec = kNoSecond;
     sec.t16 = m.t16; sec.t16_ld = m.t16_ld;
     if constexpr (ROPE && FUSEQ) {
-        // the kernel for groups with ROPE epilogues: its bodies may also take the RMS norm of the rows into their prologue
-        // (gemv_body.h: NORMABLE; short rows only: the phased prologue never holds a whole row), one row per step
-        sec.norm_w = nm.w; sec.norm_eps = nm.eps; sec.norm_y = nm.y; sec.norm_ldy = nm.ldy;
+        // the kernel for groups with ROPE epilogues, one row per step in the members that have one; NORMED: every body also runs
+        // the RMS norm of the rows and the MUL with its weight in its prologue (gemv_body.h)
+        if constexpr (NORMED) { sec.norm_w = nm.w; sec.norm_eps = nm.eps; sec.norm_y = nm.y; sec.norm_ldy = nm.ldy; }
         if (m.rope.table)                                               // uniform over the workgroup
-            gemv_body<WT, NTOK, 1, WGS, FUSEQ, DEPTH, false, false, true, true>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp, m.rope);
+            gemv_body<WT, NTOK, 1, WGS, FUSEQ, DEPTH, false, false, true, NORMED>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp,
+                                                                                  m.rope);
         else
-            gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH, false, false, false, true>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y,
-                                                                                                  m.ldy, sec, gp);
+            gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH, false, false, false, NORMED>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y,
+                                                                                                    m.ldy, sec, gp);
         return;
     }
     gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
@@ -41,8 +42,8 @@ __device__ __forceinline__ void run_member(const GroupKernelMat &m, const GroupN
 // FUSEQ: the workgroups quantize the fp32 rows x themselves; otherwise the workspace already holds the quantized rows
 // (written by chip_mul_mat_prepare or by the kernel that produced the activations) and is only read.
 // ROPE: a kernel of its own for groups in which a member's ROPE node runs in its epilogue (gemv_body.h: ROPED), so that the
-// plain group kernel keeps its registers.
-template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE = false>
+// plain group kernel keeps its registers; NORMED: that kernel with the norm in front (ga.norm), again one of its own.
+template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE = false, bool NORMED = false>
 __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs ga, int64_t K, const float *__restrict__ x,
                                                          int64_t ldx, uint8_t *__restrict__ ws, size_t ws_stride) {
     int i = 0;
@@ -54,21 +55,21 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
     const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), FUSEQ && blockIdx.x == 0};
     if constexpr (FAMILY == 0) {
         switch (m.wtype) {                                              // uniform over the workgroup
-            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else if constexpr (FAMILY == 1) {
         switch (m.wtype) {
-            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
-            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_0:   run_member<T_Q4_0, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_0:   run_member<T_Q5_0, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_IQ4_NL: run_member<T_IQ4_NL, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q4_1:   run_member<T_Q4_1, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_1:   run_member<T_Q5_1, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            default:       run_member<T_Q8_0, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else {
-        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH, ROPE>(m, ga.norm, K, x, ldx, ws, ws_stride, gp);
+        run_member<T_F16, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp);
     }
 }
 
@@ -89,10 +90,10 @@ size_t image_bytes(int wtype, int64_t K) {
 }
 int rows_per_step(int wtype) { return wtype == T_Q4_0 ? RowsPerWave<T_Q4_0>::R : 1; }
 
-template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE = false>
+template <int FAMILY, int NTOK, int WGS, bool FUSEQ, int DEPTH, bool ROPE = false, bool NORMED = false>
 hipError_t launch_depth(const GroupKernelArgs &ga, int grid, int64_t K, const float *x, int64_t ldx, void *ws, size_t ws_stride,
                         size_t lds_bytes, const DeviceLimits &lim, hipStream_t st) {
-    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, FUSEQ, DEPTH, ROPE>;
+    auto kfn = gemv_group_kernel<FAMILY, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>;
     static LdsGrant grant;
     if (hipError_t e = grant_dynamic_lds(kfn, lds_bytes, lim, grant); e != hipSuccess) return e;
     hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(WGS), lds_bytes, st, ga, K, x, ldx, (uint8_t *)ws, ws_stride);
@@ -103,6 +104,8 @@ hipError_t launch_cfg(const GroupKernelArgs &ga, int grid, int64_t K, const floa
                       size_t lds_bytes, const DeviceLimits &lim, hipStream_t st, bool prepared, bool rope) {
     if (rope) {
         if constexpr (FAMILY != 2) {
+            if (!prepared && ga.norm.w)
+                return launch_depth<FAMILY, NTOK, WGS, true, GEMV_DEPTH, true, true>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
             if (!prepared) return launch_depth<FAMILY, NTOK, WGS, true, GEMV_DEPTH, true>(ga, grid, K, x, ldx, ws, ws_stride, lds_bytes, lim, st);
         }
         return hipErrorInvalidValue;
