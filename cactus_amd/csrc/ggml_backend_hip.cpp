@@ -267,6 +267,25 @@ bool mul_mat_f16_batched_shape_ok(const lm_ggml_tensor *op) {
     return true;
 }
 
+// MUL_MAT with batch dimensions over a weight of a supported block type: src0 [K, N, ne02, ne03], src1 [K, n, ne12, ne13]
+// with ne12 / ne13 multiples of ne02 / ne03 (slice (i12, i13) of src1 meets slice (i12 / r2, i13 / r3) of src0: reference
+// ggml-cpu/ggml-cpu.c:1188-1189, 1294-1295).  Every slice is a 2-D matmul of the kind above; what the two paths above take goes
+// there first.
+bool mul_mat_batched_shape_ok(const lm_ggml_tensor *op) {
+    const lm_ggml_tensor *w = op->src[0], *x = op->src[1];
+    if (!w || !x || !chip_mul_mat_supported(w->type, w->ne[0])) return false;
+    if (x->type != LM_GGML_TYPE_F32 || op->type != LM_GGML_TYPE_F32) return false;
+    if (w->ne[2] < 1 || w->ne[3] < 1 || x->ne[2] % w->ne[2] != 0 || x->ne[3] % w->ne[3] != 0) return false;
+    if (x->ne[2] * x->ne[3] <= 1 || x->ne[2] * x->ne[3] > 65536) return false;
+    if (x->ne[0] != w->ne[0] || op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1] || op->ne[2] != x->ne[2] || op->ne[3] != x->ne[3]) return false;
+    const size_t a = w->type == LM_GGML_TYPE_Q6_K ? 2 : (w->ne[0] % 256 != 0 ? 4 : 16);
+    if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, w->ne[0]) || w->nb[1] % a != 0) return false;
+    if (w->nb[2] % a != 0 || w->nb[3] % a != 0) return false;
+    if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)x->ne[0] * 4 || x->nb[2] % 16 != 0 || x->nb[3] % 16 != 0) return false;
+    if (op->nb[0] != sizeof(float) || op->nb[1] % 4 != 0 || op->nb[1] < (size_t)op->ne[0] * 4 || op->nb[2] % 4 != 0 || op->nb[3] % 4 != 0) return false;
+    return true;
+}
+
 // The MUL_MAT_ID shapes: experts [K, N, n_as] stored one matrix after the other, F32 activations [K, ne11, n_tokens]
 // with ne11 = 1 or n_used and the rows of a token adjacent, I32 ids [n_used, n_tokens], F32 result
 // [N, n_used, n_tokens] with adjacent rows (reference ggml.c lm_ggml_mul_mat_id, ggml-cpu/ggml-cpu.c:1531-1710).
@@ -1250,6 +1269,30 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             g_mul_mat_nodes++;
             continue;
         }
+        if (node->op == LM_GGML_OP_MUL_MAT && !mul_mat_shape_ok(node) && mul_mat_batched_shape_ok(node)) {
+            // one 2-D matmul per slice of src1, on the slice of src0 that the broadcast assigns to it
+            const lm_ggml_tensor *w = node->src[0], *x = node->src[1];
+            const int64_t K = w->ne[0], N = w->ne[1], n = x->ne[1];
+            if (N == 0 || n == 0) continue;
+            if (!grow_workspace(c, chip_mul_mat_workspace_size_n(w->type, K, N, n))) return LM_GGML_STATUS_ALLOC_FAILED;
+            const int64_t r2 = x->ne[2] / w->ne[2], r3 = x->ne[3] / w->ne[3];
+            c->quantized.valid = false;
+            for (int64_t i13 = 0; i13 < x->ne[3]; i13++)
+                for (int64_t i12 = 0; i12 < x->ne[2]; i12++) {
+                    const uint8_t *ws = (const uint8_t *)w->data + (size_t)(i12 / r2) * w->nb[2] + (size_t)(i13 / r3) * w->nb[3];
+                    const float *xs = (const float *)((const uint8_t *)x->data + (size_t)i12 * x->nb[2] + (size_t)i13 * x->nb[3]);
+                    float *ys = (float *)((uint8_t *)node->data + (size_t)i12 * node->nb[2] + (size_t)i13 * node->nb[3]);
+                    const int rc = chip_mul_mat(w->type, ws, w->nb[1], K, N, xs, (int64_t)(x->nb[1] / 4), n, ys, (int64_t)(node->nb[1] / 4),
+                                                c->workspace, c->workspace_size, c->stream);
+                    if (rc != CHIP_OK) {
+                        HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: batched MUL_MAT %s failed at slice (%lld, %lld): %s\n", __func__, node->name,
+                                (long long)i12, (long long)i13, chip_error_string(rc));
+                        return LM_GGML_STATUS_FAILED;
+                    }
+                }
+            g_mul_mat_nodes++;
+            continue;
+        }
         if (node->op != LM_GGML_OP_MUL_MAT || !mul_mat_shape_ok(node)) {
             HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: node %d (%s, op %d) is not supported by the HIP backend\n", __func__, i, node->name, node->op);
             return LM_GGML_STATUS_FAILED;
@@ -1624,7 +1667,7 @@ bool dev_supports_op(lm_ggml_backend_dev_t, const lm_ggml_tensor *op) {
     const lm_ggml_tensor *w = op->src[0];
     const lm_ggml_backend_buffer_t wbuf = !w ? nullptr : (w->view_src ? w->view_src->buffer : w->buffer);
     if (!wbuf || !is_hip_buffer(wbuf)) return false;
-    return op->op == LM_GGML_OP_MUL_MAT ? (mul_mat_shape_ok(op) || mul_mat_f16_batched_shape_ok(op)) : mul_mat_id_shape_ok(op);
+    return op->op == LM_GGML_OP_MUL_MAT ? (mul_mat_shape_ok(op) || mul_mat_f16_batched_shape_ok(op) || mul_mat_batched_shape_ok(op)) : mul_mat_id_shape_ok(op);
 }
 bool dev_supports_buft(lm_ggml_backend_dev_t, lm_ggml_backend_buffer_type_t buft) { return buft == hip_buffer_type(); }
 

@@ -114,6 +114,59 @@ def test_one_node_graph_with_a_hidden_size_that_is_no_multiple_of_256(host, orc,
     L.lm_ggml_free(ctx)
 
 
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q6_K, O.Q4_0), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("n,ne02,ne03,ne12,ne13", [(1, 2, 1, 4, 1), (3, 2, 2, 2, 4), (40, 3, 1, 3, 2)])
+def test_batched_and_broadcast_matmul_over_quantized_weights(host, orc, wt, n, ne02, ne03, ne12, ne13):
+    """MUL_MAT with batch dimensions over a quantized src0 (reference ggml-cpu/ggml-cpu.c:1188-1189, 1294-1295: slice (i12, i13)
+    of src1 meets slice (i12 / r2, i13 / r3) of src0): every slice equals, bit for bit, the one-node graph of that slice's two
+    matrices on the same backend, and meets the oracle's tolerance."""
+    L = host.L
+    K, N = 512, 72
+    rng_seed = wt * 100 + n
+    wq = np.stack([orc.quantize_weights(wt, common.weights_f32(rng_seed + i, N, K)) for i in range(ne02 * ne03)])
+    x = np.stack([common.activations_f32(rng_seed + 50 + i, n, K) for i in range(ne12 * ne13)])
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    be = L.lm_ggml_backend_dev_init(dev, None)
+    ctx = host.context()
+    a = L.lm_ggml_new_tensor_4d(ctx, wt, K, N, ne02, ne03)
+    b = L.lm_ggml_new_tensor_4d(ctx, O.F32, K, n, ne12, ne13)
+    c = L.lm_ggml_mul_mat(ctx, a, b)
+    wf = L.lm_ggml_new_tensor_4d(ctx, O.F32, K, N, ne02, ne03)
+    cf = L.lm_ggml_mul_mat(ctx, wf, b)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, c)
+    ctx2 = host.context()                                                # the slice's one-node graph, in a context of its own
+    a2 = host.tensor_2d(ctx2, wt, K, N, "w")
+    b2 = host.tensor_2d(ctx2, O.F32, K, n, "x")
+    c2 = L.lm_ggml_mul_mat(ctx2, a2, b2)
+    g2 = L.lm_ggml_new_graph(ctx2)
+    L.lm_ggml_build_forward_expand(g2, c2)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    buf2 = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx2, L.lm_ggml_backend_dev_buffer_type(dev))
+    assert L.lm_ggml_backend_dev_supports_op(dev, c) is True
+    assert L.lm_ggml_backend_dev_supports_op(dev, cf) is False           # F32 weights stay declined
+    host.set(a, wq)
+    host.set(b, x)
+    assert L.lm_ggml_backend_graph_compute(be, g) == 0
+    y = host.get(c, np.float32, (ne13, ne12, n, N))
+    r2, r3 = ne12 // ne02, ne13 // ne03
+    for i13 in range(ne13):
+        for i12 in range(ne12):
+            wi = (i13 // r3) * ne02 + i12 // r2
+            xi = i13 * ne12 + i12
+            host.set(a2, wq[wi])
+            host.set(b2, x[xi])
+            assert L.lm_ggml_backend_graph_compute(be, g2) == 0
+            assert y[i13, i12].tobytes() == host.get(c2, np.float32, (n, N)).tobytes(), (i12, i13)
+            ref = orc.mul_mat(wt, wq[wi], x[xi], nthreads=8, want=("sum_abs",))
+            assert (np.abs(y[i13, i12].astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all(), (i12, i13)
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_buffer_free(buf2)
+    L.lm_ggml_backend_free(be)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(ctx2)
+
+
 def test_unsupported_ops_are_declined(host):
     L = host.L
     dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
