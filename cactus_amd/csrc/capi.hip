@@ -83,7 +83,7 @@ int current_limits(DeviceLimits &out) {
 
 bool is_weight_type(int t) {
     return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K || t == T_Q5_0 || t == T_Q5_K || t == T_IQ4_NL ||
-           t == T_Q4_1 || t == T_Q5_1 || t == T_F16;
+           t == T_Q4_1 || t == T_Q5_1 || t == T_F16 || t == T_Q3_K || t == T_Q2_K;
 }
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -95,7 +95,8 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 // dot-product GEMV; the GEMM, whose staging reads single blocks, when K % 128 == 0).
 bool is_block32_type(int t) { return t == T_Q4_0 || t == T_Q8_0 || t == T_Q5_0 || t == T_IQ4_NL || t == T_Q4_1 || t == T_Q5_1; }
 bool weights_aligned(int type, const void *W, size_t nb01, int64_t K = 256) {
-    const size_t a = (type == T_Q6_K) ? 2 : (is_block32_type(type) && K % 256 != 0) ? 4 : 16;
+    // (Q3_K: 110-byte super-blocks, as Q6_K's 210; Q2_K: 84 bytes)
+    const size_t a = (type == T_Q6_K || type == T_Q3_K) ? 2 : (type == T_Q2_K || (is_block32_type(type) && K % 256 != 0)) ? 4 : 16;
     return ((uintptr_t)W % a) == 0 && (nb01 % a) == 0;
 }
 
@@ -232,7 +233,7 @@ int chip_block_elems(int type) {
     switch (type) {
         case T_F32: case T_F16: return 1;
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: case T_Q8_1: return 32;
-        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: return 256;
+        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: return 256;
         default: return 0;
     }
 }
@@ -251,6 +252,8 @@ size_t chip_block_bytes(int type) {
         case T_Q4_1: return BYTES_Q4_1;
         case T_Q5_1: return BYTES_Q5_1;
         case T_Q8_1: return BYTES_Q8_1;
+        case T_Q3_K: return BYTES_Q3_K;
+        case T_Q2_K: return BYTES_Q2_K;
         default: return 0;
     }
 }
@@ -261,7 +264,7 @@ size_t chip_row_size(int type, int64_t k) {
 int chip_vec_dot_type(int type) {
     switch (type) {
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return T_Q8_0;
-        case T_Q4_K: case T_Q6_K: case T_Q5_K: return T_Q8_K;
+        case T_Q4_K: case T_Q6_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: return T_Q8_K;
         case T_Q4_1: case T_Q5_1: return T_Q8_1;
         case T_F16: return T_F16;
         default: return -1;
@@ -745,7 +748,8 @@ int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K
     hipStream_t st = (hipStream_t)stream;
 
     const bool kq = type == T_Q4_K || type == T_Q5_K || type == T_Q6_K;
-    const bool have_gemm = type == T_F16 ? K % 64 == 0 : (kq ? true : K % 128 == 0);
+    // (the 2- and 3-bit K-quants have no GEMM of their own: every pair takes the GEMV)
+    const bool have_gemm = (type == T_Q3_K || type == T_Q2_K) ? false : type == T_F16 ? K % 64 == 0 : (kq ? true : K % 128 == 0);
     if (pairs >= MOE_GEMM_MIN_PAIRS && have_gemm && moe_group_supported(n_as, pairs)) {
         rc = chip_mul_mat_prepare(type, K, x, ldx, rows, workspace, workspace_bytes, stream);
         if (rc) return rc;
@@ -1115,7 +1119,7 @@ int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N,
     if (N == 0 || n == 0) return CHIP_OK;
     if (!W || !aq || !isum) return CHIP_EINVAL;
     if (!weights_aligned(type, W, nb01, K) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;
-    return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, (type == T_Q4_K || type == T_Q5_K) ? imin : nullptr, (hipStream_t)stream));
+    return hip_rc(launch_block_isums(type, W, nb01, K, N, aq, n, isum, (type == T_Q4_K || type == T_Q5_K || type == T_Q2_K) ? imin : nullptr, (hipStream_t)stream));
 }
 
 int chip_verify_force_q6k_matrix_core(int on) {

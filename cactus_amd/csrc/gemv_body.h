@@ -340,6 +340,106 @@ template <> struct Traits<T_Q6_K> {
     }
 };
 
+// ---- the 3- and 2-bit K-quants (reference type_traits_cpu[], ggml-cpu/ggml-cpu.c:257-268; lm_ggml_vec_dot_q3_K_q8_K and
+// lm_ggml_vec_dot_q2_K_q8_K, ggml-cpu/ggml-cpu-quants.c:5521 ff. / 4506 ff.; dequantize_row_q3_K / _q2_K, ggml-quants.c:1050 / 706).
+// Their 64 bytes of qs hold element 128 h + 32 v + l (l < 32) in bits 2 v of byte 32 h + l, and sub-block 8 h + 2 v + (l >= 16)
+// carries the scale: the unit (sb, h, ip) of Q6_K - the 16 bytes 32 h + 16 ip ... of qs, four 16-value groups v with scales
+// 8 h + 2 v + ip - fits both, so the activation side (image layout, block sums of 16, staging) is Q6_K's unchanged.
+template <> struct Traits<T_Q3_K> : Traits<T_Q6_K> {
+    // block_q3_K (ggml-common.h:273-278): hmask[32] | qs[64] | scales[12] | fp16 d, 110 bytes, 2-byte aligned.
+    // value = d * (scale - 32) * (q - 4), q = the two bits of qs plus 4 where the bit 4 h + v of hmask[l] is set
+    struct W { uint32_t q[16]; float d; int sc[4]; };            // q[4v + k]: values 0..7 of group v; the 4 comes off through the block sums
+    struct Raw { u32x4 qs, hm; uint32_t s0, s1, s2, d; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
+        const uint8_t *p = row + (size_t)sb * BYTES_Q3_K;
+        r.qs = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 32 + 32 * h + 16 * ip));
+        r.hm = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 16 * ip));
+        r.s0 = WLOAD(reinterpret_cast<const u32_a2 *>(p + 96));
+        r.s1 = WLOAD(reinterpret_cast<const u32_a2 *>(p + 100));
+        r.s2 = WLOAD(reinterpret_cast<const u32_a2 *>(p + 104));
+        r.d  = WLOAD(reinterpret_cast<const unsigned short *>(p + 108));
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+        const int h = (u >> 1) & 1, ip = u & 1;
+        w.d = h2f(r.d);
+        const uint32_t lo[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w}, hm[4] = {r.hm.x, r.hm.y, r.hm.z, r.hm.w};
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                w.q[4 * v + k] = ((lo[k] >> (2 * v)) & 0x03030303u) | (((hm[k] >> (4 * h + v)) & 0x01010101u) << 2);
+        // the sixteen 6-bit scales (ggml-quants.c:1062-1071): scale 4 w + i is byte i of word w below; this unit wants
+        // 8 h + 2 v + ip, i.e. bytes ip and 2 + ip of words 2 h and 2 h + 1
+        const uint32_t hi2 = r.s2 >> (4 * h);
+        const uint32_t wa = ((r.s0 >> (4 * h)) & 0x0f0f0f0fu) | ((hi2 & 0x03030303u) << 4);
+        const uint32_t wb = ((r.s1 >> (4 * h)) & 0x0f0f0f0fu) | (((hi2 >> 2) & 0x03030303u) << 4);
+        const int b = 8 * ip;
+        w.sc[0] = (int)((wa >> b) & 0xffu) - 32; w.sc[1] = (int)((wa >> (b + 16)) & 0xffu) - 32;
+        w.sc[2] = (int)((wb >> b) & 0xffu) - 32; w.sc[3] = (int)((wb >> (b + 16)) & 0xffu) - 32;
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &unused) {
+        is = 0; unused = 0;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            int dv = -4 * a.bs[v];                                      // sum (q-4)*a = sum q*a - 4*sum a
+#pragma unroll
+            for (int k = 0; k < 4; k++) dv = dot4(w.q[4 * v + k], a.q[4 * v + k], dv);
+            is += w.sc[v] * dv;
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int is, unused;
+        isums(w, a, is, unused);
+        return __builtin_fmaf(w.d * a.d, (float)is, acc);
+    }
+};
+
+template <> struct Traits<T_Q2_K> : Traits<T_Q6_K> {
+    // block_q2_K (ggml-common.h:254-266): scales[16] (scale in the low, min in the high nibble) | qs[64] | fp16 d | fp16 dmin,
+    // 84 bytes, 4-byte aligned.  value = d * sc * q - dmin * m, q = the two bits of qs
+    struct W { uint32_t q[16]; float d, dmin; int sc[4], m[4]; };
+    struct Raw { u32x4 qs; uint32_t s0, s1, dd; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
+        const uint8_t *p = row + (size_t)sb * BYTES_Q2_K;
+        r.qs = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 16 + 32 * h + 16 * ip));
+        r.s0 = WLOAD(reinterpret_cast<const uint32_t *>(p + 8 * h));
+        r.s1 = WLOAD(reinterpret_cast<const uint32_t *>(p + 8 * h + 4));
+        r.dd = WLOAD(reinterpret_cast<const uint32_t *>(p + 80));
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+        const int ip = u & 1;
+        w.d = h2f(r.dd); w.dmin = h2f(r.dd >> 16);
+        const uint32_t lo[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) w.q[4 * v + k] = (lo[k] >> (2 * v)) & 0x03030303u;
+        const int b = 8 * ip;                                           // scales[8h + 2v + ip]: bytes ip and 2 + ip of the two words
+        const uint32_t c0 = r.s0 >> b, c1 = r.s0 >> (b + 16), c2 = r.s1 >> b, c3 = r.s1 >> (b + 16);
+        w.sc[0] = (int)(c0 & 15u); w.m[0] = (int)((c0 >> 4) & 15u); w.sc[1] = (int)(c1 & 15u); w.m[1] = (int)((c1 >> 4) & 15u);
+        w.sc[2] = (int)(c2 & 15u); w.m[2] = (int)((c2 >> 4) & 15u); w.sc[3] = (int)(c3 & 15u); w.m[3] = (int)((c3 >> 4) & 15u);
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &im) {
+        is = 0; im = 0;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            int dv = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) dv = dot4(w.q[4 * v + k], a.q[4 * v + k], dv);
+            is += w.sc[v] * dv;
+            im += w.m[v] * a.bs[v];
+        }
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int is, im;
+        isums(w, a, is, im);
+        acc = __builtin_fmaf(w.d * a.d, (float)is, acc);
+        return __builtin_fmaf(-(w.dmin * a.d), (float)im, acc);
+    }
+};
+
 // ---- further weight types (reference type_traits_cpu[], ggml-cpu/ggml-cpu.c:198-367): same activation formats
 template <> struct Traits<T_Q5_0> {
     // block_q5_0 (ggml-common.h:187-193): fp16 d, 32 high bits qh, 16 nibble bytes; value = d * (q5 - 16),

@@ -233,6 +233,12 @@ bool is_view_op(int op) {
            op == LM_GGML_OP_TRANSPOSE;
 }
 
+// What a weight row's start and stride must be a multiple of: super-blocks of 210 (Q6_K) and 110 bytes (Q3_K) allow 2, of 84
+// bytes (Q2_K) and rows of K % 256 != 0 (32-value block types only) 4, everything else 16.
+size_t weight_alignment(const lm_ggml_tensor *w) {
+    if (w->type == LM_GGML_TYPE_Q6_K || w->type == LM_GGML_TYPE_Q3_K) return 2;
+    return (w->type == LM_GGML_TYPE_Q2_K || w->ne[0] % 256 != 0) ? 4 : 16;
+}
 // The MUL_MAT shapes the kernels take: weights [K, N] of a supported block type with whole-row strides, F32
 // activations [K, n] and F32 result [N, n] with element-contiguous rows, no batch dimensions.
 bool mul_mat_shape_ok(const lm_ggml_tensor *op) {
@@ -243,8 +249,7 @@ bool mul_mat_shape_ok(const lm_ggml_tensor *op) {
     if (w->ne[2] != 1 || w->ne[3] != 1 || x->ne[2] != 1 || x->ne[3] != 1) return false;
     if (x->ne[0] != w->ne[0] || op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1]) return false;
     if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, w->ne[0])) return false;
-    // rows of K % 256 != 0 (32-value block types only) are multiples of 4 bytes
-    if (w->nb[1] % (w->type == LM_GGML_TYPE_Q6_K ? 2 : (w->ne[0] % 256 != 0 ? 4 : 16)) != 0) return false;
+    if (w->nb[1] % weight_alignment(w) != 0) return false;
     if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)x->ne[0] * 4) return false;
     if (op->nb[0] != sizeof(float) || op->nb[1] % 4 != 0 || op->nb[1] < (size_t)op->ne[0] * 4) return false;
     return true;
@@ -278,7 +283,7 @@ bool mul_mat_batched_shape_ok(const lm_ggml_tensor *op) {
     if (w->ne[2] < 1 || w->ne[3] < 1 || x->ne[2] % w->ne[2] != 0 || x->ne[3] % w->ne[3] != 0) return false;
     if (x->ne[2] * x->ne[3] <= 1 || x->ne[2] * x->ne[3] > 65536) return false;
     if (x->ne[0] != w->ne[0] || op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1] || op->ne[2] != x->ne[2] || op->ne[3] != x->ne[3]) return false;
-    const size_t a = w->type == LM_GGML_TYPE_Q6_K ? 2 : (w->ne[0] % 256 != 0 ? 4 : 16);
+    const size_t a = weight_alignment(w);
     if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, w->ne[0]) || w->nb[1] % a != 0) return false;
     if (w->nb[2] % a != 0 || w->nb[3] % a != 0) return false;
     if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)x->ne[0] * 4 || x->nb[2] % 16 != 0 || x->nb[3] % 16 != 0) return false;
@@ -299,7 +304,7 @@ bool mul_mat_id_shape_ok(const lm_ggml_tensor *op) {
     if (w->ne[3] != 1 || x->ne[3] != 1 || op->ne[3] != 1 || ids->ne[2] != 1 || ids->ne[3] != 1) return false;
     if (x->ne[0] != K || x->ne[2] != n_tokens || !(x->ne[1] == 1 || x->ne[1] == n_used)) return false;
     if (op->ne[0] != N || op->ne[1] != n_used || op->ne[2] != n_tokens) return false;
-    const size_t a = (w->type == LM_GGML_TYPE_Q6_K) ? 2 : 16;
+    const size_t a = weight_alignment(w);
     if (w->nb[0] != chip_block_bytes(w->type) || w->nb[1] < chip_row_size(w->type, K) || w->nb[1] % a != 0) return false;
     if (w->nb[2] < (size_t)N * w->nb[1] || w->nb[2] % a != 0) return false;
     if (x->nb[0] != sizeof(float) || x->nb[1] % 16 != 0 || x->nb[1] < (size_t)K * 4 || x->nb[2] != (size_t)x->ne[1] * x->nb[1]) return false;

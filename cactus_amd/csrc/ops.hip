@@ -620,6 +620,23 @@ template <int WT> __device__ __forceinline__ float dequant_at(const uint8_t *row
         int v = hi ? (q >> 4) : (q & 0xF);
         if constexpr (WT == T_Q5_K) v += (b[16 + ll] & (1u << (2 * j64 + hi))) ? 16 : 0;
         return d1 * (float)v - m1;
+    } else if constexpr (WT == T_Q2_K) {                                // scales[16] qs[64] d dmin (reference ggml-quants.c:706-737)
+        const uint8_t *b = row + (size_t)(i >> 8) * BYTES_Q2_K;
+        const uint32_t r = i & 255, h = r >> 7, j = (r >> 5) & 3, l = r & 31;
+        const float d = h2f(reinterpret_cast<const uint16_t *>(b + 80)[0]), mn = h2f(reinterpret_cast<const uint16_t *>(b + 80)[1]);
+        const int sc = b[8 * h + 2 * j + (l >> 4)];
+        const float dl = d * (float)(sc & 0xF), ml = mn * (float)(sc >> 4);
+        return dl * (float)(int8_t)((b[16 + 32 * h + l] >> (2 * j)) & 3) - ml;
+    } else if constexpr (WT == T_Q3_K) {                                // hmask[32] qs[64] scales[12] d (ggml-quants.c:1050-1098)
+        const uint8_t *b = row + (size_t)(i >> 8) * BYTES_Q3_K;
+        const uint32_t r = i & 255, h = r >> 7, j = (r >> 5) & 3, l = r & 31;
+        const uint32_t is = 8 * h + 2 * j + (l >> 4);                   // scale index: low nibbles in bytes 0..7, high bit pairs in 8..11
+        const uint8_t *s = b + 96;
+        const int lo4 = is < 8 ? (s[is] & 0xF) : (s[is - 8] >> 4);
+        const int hi2 = (s[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+        const float dl = h2f(reinterpret_cast<const uint16_t *>(b + 108)[0]) * (float)((lo4 | (hi2 << 4)) - 32);
+        const int q = (int)(int8_t)((b[32 + 32 * h + l] >> (2 * j)) & 3) - ((b[l] & (1u << (4 * h + j))) ? 0 : 4);
+        return dl * (float)q;
     } else {                                                            // T_Q6_K: ql[128] qh[64] scales[16] d
         const uint8_t *b = row + (size_t)(i >> 8) * BYTES_Q6_K;
         const uint32_t r = i & 255, h = r >> 7, rr = r & 127, quarter = rr >> 5, l = rr & 31;
@@ -656,7 +673,7 @@ hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st) {
 #define GR_CASE(TT) case TT: hipLaunchKernelGGL(get_rows_kernel<TT>, grid, dim3(EW_THREADS), 0, st, a); break;
     switch (type) {
         GR_CASE(T_F32) GR_CASE(T_F16) GR_CASE(T_Q4_0) GR_CASE(T_Q4_1) GR_CASE(T_Q5_0) GR_CASE(T_Q5_1) GR_CASE(T_Q8_0)
-        GR_CASE(T_Q4_K) GR_CASE(T_Q5_K) GR_CASE(T_Q6_K) GR_CASE(T_IQ4_NL)
+        GR_CASE(T_Q4_K) GR_CASE(T_Q5_K) GR_CASE(T_Q6_K) GR_CASE(T_IQ4_NL) GR_CASE(T_Q3_K) GR_CASE(T_Q2_K)
         default: return hipErrorInvalidValue;
     }
 #undef GR_CASE

@@ -19,18 +19,21 @@ F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
 F16 = 1
-TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
+Q2_K, Q3_K = 10, 11
+TYPE_NAMES = {Q2_K: "q2_K", Q3_K: "q3_K", F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
               Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16"}
-BLOCK_ELEMS = {F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32,
+BLOCK_ELEMS = {Q2_K: 256, Q3_K: 256, F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32,
                Q4_1: 32, Q5_1: 32, Q8_1: 32, F16: 1}
-BLOCK_BYTES = {F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18,
+BLOCK_BYTES = {Q2_K: 84, Q3_K: 110, F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18,
                Q4_1: 20, Q5_1: 24, Q8_1: 36, F16: 2}
-VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0,
+VEC_DOT_TYPE = {Q2_K: Q8_K, Q3_K: Q8_K, Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0,
                 Q4_1: Q8_1, Q5_1: Q8_1, F16: F16}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, F16)
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, Q3_K, Q2_K, F16)
 BLOCK_WEIGHT_TYPES = WEIGHT_TYPES[:-1]        # the types with per-block integer sums
-# types whose weight quantizer is restated in the oracle (IQ4_NL weights come from the reference build, from the
-# golden fixture, or are random bytes: any byte string is a valid block)
+# the 2- and 3-bit K-quants: decode and small batches on the GEMV kernels, no matrix-core kernels of their own
+LOW_BIT_K_TYPES = (Q3_K, Q2_K)
+# types whose weight quantizer is restated in the oracle (IQ4_NL, Q3_K and Q2_K weights come from the reference build, from
+# the golden fixture, from a plain quantizer here, or are random bytes: any byte string is a valid block)
 ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, Q4_1, Q5_1, F16)
 
 
@@ -66,6 +69,73 @@ def random_iq4_nl_rows(seed, n, k):
     blk[..., :2] = d.view(np.uint8).reshape(n, nb, 2)
     blk[..., 2:] = rng.integers(0, 256, (n, nb, 16), dtype=np.uint8)
     return blk.reshape(n, nb * 18)
+
+
+def _k_sub_blocks(w):
+    """fp32 [N, K] -> [N, K/256, 2 halves, 4 shifts, 2 parts, 16]: element 128 h + 32 j + 16 p + l of a super-block, i.e.
+    bits 2 j of byte 32 h + 16 p + l of qs in the 2- and 3-bit K-quants; sub-block (scale) index 8 h + 2 j + p."""
+    w = np.ascontiguousarray(w, np.float32)
+    n, k = w.shape
+    return w.reshape(n, k // 256, 2, 4, 2, 16)
+
+
+def _pack_2bit(q):
+    """q uint8 [N, nb, 2, 4, 2, 16] with values 0..3 -> qs uint8 [N, nb, 64]"""
+    n, nb = q.shape[:2]
+    out = np.zeros((n, nb, 2, 2, 16), np.uint8)
+    for j in range(4):
+        out |= (q[:, :, :, j] & 3) << (2 * j)
+    return out.reshape(n, nb, 64)
+
+
+def plain_q3_K_rows(w):
+    """fp32 [N, K] -> Q3_K rows by a plain round-to-nearest quantizer: sub-block scale = max|x| / 4, super-block d =
+    largest scale / 31, codes 0..31 (+32), q = round(x / (d code)) in [-4, 3].  Not the reference's search: it only makes
+    meaningful bytes (any byte string is a valid block; the op's parity surface starts at the bytes)."""
+    blk = _k_sub_blocks(w)
+    n, nb = blk.shape[:2]
+    s = np.abs(blk).max(-1) / np.float32(4)                          # [n, nb, 2, 4, 2]
+    d = (s.reshape(n, nb, -1).max(-1) / np.float32(31)).astype(np.float16)
+    df = d.astype(np.float32)[:, :, None, None, None]
+    code = np.where(df > 0, np.rint(s / np.where(df > 0, df, 1)), 0).clip(0, 31).astype(np.int32)
+    step = df * code
+    q = np.where(step[..., None] > 0, np.rint(blk / np.where(step[..., None] > 0, step[..., None], 1)), 0).clip(-4, 3).astype(np.int32) + 4
+    out = np.zeros((n, nb, 110), np.uint8)
+    hm = np.zeros((n, nb, 2, 16), np.uint8)                          # hmask[16 p + l], bit 4 h + j
+    for h in range(2):
+        for j in range(4):
+            hm |= ((q[:, :, h, j] >> 2) & 1).astype(np.uint8) << (4 * h + j)
+    out[..., :32] = hm.reshape(n, nb, 32)
+    out[..., 32:96] = _pack_2bit(q.astype(np.uint8))
+    sc = (code + 32).transpose(0, 1, 2, 3, 4).reshape(n, nb, 16)      # index 8 h + 2 j + p
+    lo, hi = (sc & 15).astype(np.uint8), (sc >> 4).astype(np.uint8)
+    out[..., 96:100] = lo[..., 0:4] | (lo[..., 8:12] << 4)
+    out[..., 100:104] = lo[..., 4:8] | (lo[..., 12:16] << 4)
+    out[..., 104:108] = hi[..., 0:4] | (hi[..., 4:8] << 2) | (hi[..., 8:12] << 4) | (hi[..., 12:16] << 6)
+    out[..., 108:110] = d.view(np.uint8).reshape(n, nb, 2)
+    return out.reshape(n, nb * 110)
+
+
+def plain_q2_K_rows(w):
+    """fp32 [N, K] -> Q2_K rows by a plain quantizer: sub-block min m = max(0, -min x), scale = (max x + m) / 3, 4-bit
+    codes of both against the super-block's largest, q = round((x + dmin m) / (d sc)) in [0, 3].  Not the reference's."""
+    blk = _k_sub_blocks(w)
+    n, nb = blk.shape[:2]
+    mn = np.maximum(0, -blk.min(-1))
+    sc = (blk.max(-1) + mn) / np.float32(3)
+    d = (sc.reshape(n, nb, -1).max(-1) / np.float32(15)).astype(np.float16)
+    dm = (mn.reshape(n, nb, -1).max(-1) / np.float32(15)).astype(np.float16)
+    df, dmf = d.astype(np.float32)[:, :, None, None, None], dm.astype(np.float32)[:, :, None, None, None]
+    csc = np.where(df > 0, np.rint(sc / np.where(df > 0, df, 1)), 0).clip(0, 15).astype(np.int32)
+    cmn = np.where(dmf > 0, np.rint(mn / np.where(dmf > 0, dmf, 1)), 0).clip(0, 15).astype(np.int32)
+    step = (df * csc)[..., None]
+    q = np.where(step > 0, np.rint((blk + (dmf * cmn)[..., None]) / np.where(step > 0, step, 1)), 0).clip(0, 3).astype(np.uint8)
+    out = np.zeros((n, nb, 84), np.uint8)
+    out[..., :16] = (csc | (cmn << 4)).reshape(n, nb, 16).astype(np.uint8)
+    out[..., 16:80] = _pack_2bit(q)
+    out[..., 80:82] = d.view(np.uint8).reshape(n, nb, 2)
+    out[..., 82:84] = dm.view(np.uint8).reshape(n, nb, 2)
+    return out.reshape(n, nb * 84)
 
 
 def row_size(t, k):
@@ -116,11 +186,11 @@ class Oracle:
         L.orc_quantize_rows.argtypes = [_i32, _vp, _vp, _i64, _i64]
         L.orc_dequantize_row.restype = None
         L.orc_dequantize_row.argtypes = [_i32, _vp, _vp, _i64]
-        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0", "q4_1_q8_1", "q5_1_q8_1"):
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0", "q4_1_q8_1", "q5_1_q8_1", "q3_K_q8_K"):
             f = getattr(L, "orc_vec_dot_" + n)
             f.restype = C.c_float
             f.argtypes = [_i64, _vp, _vp, _vp]
-        for n in ("q4_K_q8_K", "q5_K_q8_K"):
+        for n in ("q4_K_q8_K", "q5_K_q8_K", "q2_K_q8_K"):
             f = getattr(L, "orc_vec_dot_" + n)
             f.restype = C.c_float
             f.argtypes = [_i64, _vp, _vp, _vp, _vp]
@@ -177,6 +247,10 @@ class Oracle:
         n, k = w.shape
         if wtype == IQ4_NL:
             return nearest_iq4_nl_rows(w)
+        if wtype == Q3_K:
+            return plain_q3_K_rows(w)
+        if wtype == Q2_K:
+            return plain_q2_K_rows(w)
         out = np.zeros((n, row_size(wtype, k)), np.uint8)
         got = self.lib.orc_quantize_rows(wtype, _ptr(w), _ptr(out), n, k)
         assert got == out.size
@@ -213,6 +287,10 @@ class Oracle:
             v = self.lib.orc_vec_dot_q5_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
         elif wtype == F16:
             v = self.lib.orc_vec_dot_f16(k, _ptr(wrow), _ptr(arow))
+        elif wtype == Q2_K:
+            v = self.lib.orc_vec_dot_q2_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
+        elif wtype == Q3_K:
+            v = self.lib.orc_vec_dot_q3_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q4_1:
             v = self.lib.orc_vec_dot_q4_1_q8_1(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q5_1:
@@ -391,16 +469,17 @@ class Reference:
                   "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref",
                   "quantize_row_q5_0_ref", "quantize_row_q5_K_ref", "quantize_row_iq4_nl_ref",
                   "quantize_row_q4_1_ref", "quantize_row_q5_1_ref", "quantize_row_q8_1",
+                  "quantize_row_q2_K_ref", "quantize_row_q3_K_ref",
                   "lm_ggml_fp32_to_fp16_row", "lm_ggml_cpu_fp32_to_fp16", "lm_ggml_fp16_to_fp32_row"):
             f = getattr(L, n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
-        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl", "q4_1", "q5_1"):
+        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl", "q4_1", "q5_1", "q2_K", "q3_K"):
             f = getattr(L, "dequantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
         for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "q5_0_q8_0", "q5_K_q8_K", "iq4_nl_q8_0",
-                  "q4_1_q8_1", "q5_1_q8_1", "f16"):
+                  "q4_1_q8_1", "q5_1_q8_1", "f16", "q2_K_q8_K", "q3_K_q8_K"):
             f = getattr(L, "lm_ggml_vec_dot_" + n)
             f.restype = None
             f.argtypes = [C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, _vp, C.c_size_t, C.c_int]
@@ -467,11 +546,13 @@ class Reference:
     _WQ = {Q4_0: "quantize_row_q4_0_ref", Q8_0: "quantize_row_q8_0_ref",
            Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref",
            Q5_0: "quantize_row_q5_0_ref", Q5_K: "quantize_row_q5_K_ref", IQ4_NL: "quantize_row_iq4_nl_ref",
-           Q4_1: "quantize_row_q4_1_ref", Q5_1: "quantize_row_q5_1_ref", F16: "lm_ggml_fp32_to_fp16_row"}
+           Q4_1: "quantize_row_q4_1_ref", Q5_1: "quantize_row_q5_1_ref", F16: "lm_ggml_fp32_to_fp16_row",
+           Q2_K: "quantize_row_q2_K_ref", Q3_K: "quantize_row_q3_K_ref"}
     _DOT = {Q4_0: "lm_ggml_vec_dot_q4_0_q8_0", Q8_0: "lm_ggml_vec_dot_q8_0_q8_0",
             Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K",
             Q5_0: "lm_ggml_vec_dot_q5_0_q8_0", Q5_K: "lm_ggml_vec_dot_q5_K_q8_K", IQ4_NL: "lm_ggml_vec_dot_iq4_nl_q8_0",
-            Q4_1: "lm_ggml_vec_dot_q4_1_q8_1", Q5_1: "lm_ggml_vec_dot_q5_1_q8_1", F16: "lm_ggml_vec_dot_f16"}
+            Q4_1: "lm_ggml_vec_dot_q4_1_q8_1", Q5_1: "lm_ggml_vec_dot_q5_1_q8_1", F16: "lm_ggml_vec_dot_f16",
+            Q2_K: "lm_ggml_vec_dot_q2_K_q8_K", Q3_K: "lm_ggml_vec_dot_q3_K_q8_K"}
 
     def quantize_activation(self, act_type, x):
         x = _f32(x)

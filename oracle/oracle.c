@@ -28,6 +28,9 @@ typedef struct { uint16_t d; uint8_t qs[16]; } blk_iq4_nl;
 typedef struct { uint16_t d; uint16_t m; uint8_t qs[16]; } blk_q4_1;
 typedef struct { uint16_t d; uint16_t m; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_1;
 typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } blk_q8_1;
+/* 2- and 3-bit K-quants: ggml-common.h:254-266 (q2_K), :273-278 (q3_K) */
+typedef struct { uint8_t scales[16]; uint8_t qs[64]; uint16_t d; uint16_t dmin; } blk_q2_K;
+typedef struct { uint8_t hmask[32]; uint8_t qs[64]; uint8_t scales[12]; uint16_t d; } blk_q3_K;
 #pragma pack(pop)
 
 _Static_assert(sizeof(blk_q4_0) == 18, "q4_0");
@@ -41,6 +44,8 @@ _Static_assert(sizeof(blk_iq4_nl) == 18, "iq4_nl");
 _Static_assert(sizeof(blk_q4_1) == 20, "q4_1");
 _Static_assert(sizeof(blk_q5_1) == 24, "q5_1");
 _Static_assert(sizeof(blk_q8_1) == 36, "q8_1");
+_Static_assert(sizeof(blk_q2_K) == 84, "q2_K");
+_Static_assert(sizeof(blk_q3_K) == 110, "q3_K");
 
 /* ggml-quants.c:2428: the 16 code points of the non-linear 4-bit types. */
 static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
@@ -51,6 +56,7 @@ int orc_block_elems(int type) {
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL:
         case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: case ORC_TYPE_Q8_1: return 32;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
+        case ORC_TYPE_Q2_K: case ORC_TYPE_Q3_K: return 256;
         default: return 0;
     }
 }
@@ -69,6 +75,8 @@ size_t orc_block_bytes(int type) {
         case ORC_TYPE_Q4_1: return 20;
         case ORC_TYPE_Q5_1: return 24;
         case ORC_TYPE_Q8_1: return 36;
+        case ORC_TYPE_Q2_K: return 84;
+        case ORC_TYPE_Q3_K: return 110;
         default: return 0;
     }
 }
@@ -80,6 +88,7 @@ int orc_vec_dot_type(int type) {
     switch (type) { /* ggml-cpu/ggml-cpu.c:213,245,272,284; :229 (q5_0), :278 (q5_K), :340 (iq4_nl) */
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return ORC_TYPE_Q8_0;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
+        case ORC_TYPE_Q2_K: case ORC_TYPE_Q3_K: return ORC_TYPE_Q8_K;   /* ggml-cpu/ggml-cpu.c:257-268 */
         case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: return ORC_TYPE_Q8_1;   /* ggml-cpu/ggml-cpu.c:221,237 */
         case ORC_TYPE_F16: return ORC_TYPE_F16;                        /* ggml-cpu/ggml-cpu.c:204-209 */
         default: return -1;
@@ -600,6 +609,19 @@ size_t orc_quantize_rows(int type, const float *x, void *y, int64_t nrows, int64
     return rs * (size_t)nrows;
 }
 
+/* The sixteen 6-bit scales of a q3_K super-block, still biased by 32 (ggml-quants.c:1062-1071, the same unpacking in
+ * ggml-cpu/ggml-cpu-quants.c:5815-5822): byte k of the four words is scale k. */
+static void q3_K_scales(const uint8_t *s12, int8_t out[16]) {
+    uint32_t aux[4];
+    memcpy(aux, s12, 12);
+    const uint32_t tmp = aux[2];
+    aux[2] = ((aux[0] >> 4) & 0x0f0f0f0fu) | (((tmp >> 4) & 0x03030303u) << 4);
+    aux[3] = ((aux[1] >> 4) & 0x0f0f0f0fu) | (((tmp >> 6) & 0x03030303u) << 4);
+    aux[0] = (aux[0] & 0x0f0f0f0fu) | (((tmp >> 0) & 0x03030303u) << 4);
+    aux[1] = (aux[1] & 0x0f0f0f0fu) | (((tmp >> 2) & 0x03030303u) << 4);
+    memcpy(out, aux, 16);
+}
+
 /* ---------------------------------------------------------------- dequantizers (closed forms)
  * q4_0 ggml-quants.c:249-267 ; q8_0 :343-357 ; q4_K :1274-1296 ; q6_K :1684-1713 ; q8_K :2512-2521 */
 void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
@@ -650,6 +672,41 @@ void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
                     y[l + 32] = d * sc[is + 2] * q2;
                     y[l + 64] = d * sc[is + 4] * q3;
                     y[l + 96] = d * sc[is + 6] * q4;
+                }
+            }
+        }
+    } else if (type == ORC_TYPE_Q2_K) {                 /* ggml-quants.c:706-737 */
+        const blk_q2_K *x = (const blk_q2_K *)vx;
+        for (int64_t b = 0; b < k / 256; b++) {
+            const float d = H2F(x[b].d), mn = H2F(x[b].dmin);
+            const uint8_t *q = x[b].qs;
+            int is = 0;
+            for (int h = 0; h < 2; h++, q += 32) {
+                for (int j = 0; j < 4; j++) {
+                    for (int half = 0; half < 2; half++) {
+                        const uint8_t sc = x[b].scales[is++];
+                        const float dl = d * (sc & 0xF), ml = mn * (sc >> 4);
+                        for (int l = 0; l < 16; l++) *y++ = dl * ((int8_t)((q[l + 16 * half] >> (2 * j)) & 3)) - ml;
+                    }
+                }
+            }
+        }
+    } else if (type == ORC_TYPE_Q3_K) {                 /* ggml-quants.c:1050-1098 */
+        const blk_q3_K *x = (const blk_q3_K *)vx;
+        for (int64_t b = 0; b < k / 256; b++) {
+            const float d_all = H2F(x[b].d);
+            int8_t scales[16];
+            q3_K_scales(x[b].scales, scales);
+            const uint8_t *q = x[b].qs, *hm = x[b].hmask;
+            uint8_t m = 1;
+            int is = 0;
+            for (int h = 0; h < 2; h++, q += 32) {
+                for (int j = 0; j < 4; j++, m <<= 1) {
+                    for (int half = 0; half < 2; half++) {
+                        const float dl = d_all * (scales[is++] - 32);
+                        for (int l = 16 * half; l < 16 * half + 16; l++)
+                            *y++ = dl * ((int8_t)((q[l] >> (2 * j)) & 3) - ((hm[l] & m) ? 0 : 4));
+                    }
                 }
             }
         }
@@ -1069,6 +1126,76 @@ float orc_vec_dot_q5_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *
     return hsum8(acc) + summs;
 }
 
+/* ggml-cpu/ggml-cpu-quants.c:4831-4894 (AVX2).  Eight int32 lanes: lane m of a 32-value vector v of half h holds
+ * scale[8h + 2v + (m >= 4)] * sum_{t<4} q2 * q8 over bytes 4m .. 4m+3; the mins go first, into the same eight float
+ * lanes, as mins[2m] * bsums[2m] + mins[2m+1] * bsums[2m+1]. */
+float orc_vec_dot_q2_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin) {
+    const blk_q2_K *x = (const blk_q2_K *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float d = y[b].d * H2F(x[b].d);
+        const float dmin = -y[b].d * H2F(x[b].dmin);
+        int32_t mtot = 0;
+        for (int m = 0; m < 8; m++) {
+            const int32_t p = (int32_t)(x[b].scales[2 * m] >> 4) * y[b].bsums[2 * m] + (int32_t)(x[b].scales[2 * m + 1] >> 4) * y[b].bsums[2 * m + 1];
+            mtot += p;
+            acc[m] = fmaf(dmin, (float)p, acc[m]);
+        }
+        int32_t lane[8] = {0};
+        const uint8_t *q2 = x[b].qs;
+        const int8_t *q8 = y[b].qs;
+        for (int h = 0; h < 2; h++, q2 += 32, q8 += 128) {
+            for (int v = 0; v < 4; v++) {
+                for (int m = 0; m < 8; m++) {
+                    int32_t p = 0;
+                    for (int t = 0; t < 4; t++) p += (int32_t)((q2[4 * m + t] >> (2 * v)) & 3) * q8[32 * v + 4 * m + t];
+                    lane[m] += (int32_t)(x[b].scales[8 * h + 2 * v + (m >= 4)] & 0xF) * p;
+                }
+            }
+        }
+        int32_t tot = 0;
+        for (int m = 0; m < 8; m++) { tot += lane[m]; acc[m] = fmaf(d, (float)lane[m], acc[m]); }
+        if (isum) isum[b] = tot;
+        if (imin) imin[b] = mtot;
+    }
+    return hsum8(acc);
+}
+
+/* ggml-cpu/ggml-cpu-quants.c:5806-5911 (AVX2): as q2_K without mins; the quant is the two low bits minus 4 where the
+ * high bit is clear, the scales are biased by 32. */
+float orc_vec_dot_q3_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_q3_K *x = (const blk_q3_K *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float d = y[b].d * H2F(x[b].d);
+        int8_t sc[16];
+        q3_K_scales(x[b].scales, sc);
+        int32_t lane[8] = {0};
+        const uint8_t *q3 = x[b].qs, *hm = x[b].hmask;
+        const int8_t *q8 = y[b].qs;
+        for (int h = 0; h < 2; h++, q3 += 32, q8 += 128) {
+            for (int v = 0; v < 4; v++) {
+                const uint8_t bit = (uint8_t)(1u << (4 * h + v));
+                for (int m = 0; m < 8; m++) {
+                    int32_t p = 0;
+                    for (int t = 0; t < 4; t++) {
+                        const int i = 4 * m + t;
+                        const int q = (int)((q3[i] >> (2 * v)) & 3) - ((hm[i] & bit) ? 0 : 4);
+                        p += q * (int32_t)q8[32 * v + i];
+                    }
+                    lane[m] += (int32_t)(sc[8 * h + 2 * v + (m >= 4)] - 32) * p;
+                }
+            }
+        }
+        int32_t tot = 0;
+        for (int m = 0; m < 8; m++) { tot += lane[m]; acc[m] = fmaf(d, (float)lane[m], acc[m]); }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc);
+}
+
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
     switch (type) {
         case ORC_TYPE_Q4_0: return orc_vec_dot_q4_0_q8_0(k, vx, vy, NULL);
@@ -1081,6 +1208,8 @@ float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
         case ORC_TYPE_Q4_1: return orc_vec_dot_q4_1_q8_1(k, vx, vy, NULL);
         case ORC_TYPE_Q5_1: return orc_vec_dot_q5_1_q8_1(k, vx, vy, NULL);
         case ORC_TYPE_F16: return orc_vec_dot_f16(k, vx, vy);
+        case ORC_TYPE_Q2_K: return orc_vec_dot_q2_K_q8_K(k, vx, vy, NULL, NULL);
+        case ORC_TYPE_Q3_K: return orc_vec_dot_q3_K_q8_K(k, vx, vy, NULL);
         default: return NAN;
     }
 }
@@ -1184,6 +1313,40 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
             }
         }
         free(wi); free(tmp);
+    } else if (type == ORC_TYPE_Q2_K || type == ORC_TYPE_Q3_K) {
+        /* terms at sub-block granularity (16 values): d*sc_g*dot_g, and for q2_K dmin*m_g*bsum_g */
+        float *wi = (float *)malloc(sizeof(float) * (size_t)(k > 0 ? k : 1));
+        const blk_q8_K *y = (const blk_q8_K *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            double d, dm = 0;
+            int sc[16], mn[16];
+            if (type == ORC_TYPE_Q2_K) {
+                blk_q2_K t = ((const blk_q2_K *)vx)[b];
+                d = (double)y[b].d * (double)H2F(t.d); dm = (double)y[b].d * (double)H2F(t.dmin);
+                for (int g = 0; g < 16; g++) { sc[g] = t.scales[g] & 0xF; mn[g] = t.scales[g] >> 4; t.scales[g] = 1; }
+                t.d = 0x3c00; t.dmin = 0;                 /* d = 1, unit scales, no mins: the integers q in element order */
+                orc_dequantize_row(ORC_TYPE_Q2_K, &t, wi + 256 * b, 256);
+            } else {
+                blk_q3_K t = ((const blk_q3_K *)vx)[b];
+                int8_t s8[16];
+                d = (double)y[b].d * (double)H2F(t.d);
+                q3_K_scales(t.scales, s8);
+                for (int g = 0; g < 16; g++) { sc[g] = s8[g] - 32; mn[g] = 0; }
+                /* scales of 33 - 32 = 1 in every position: low nibbles 1, high bit pairs 2 */
+                for (int i = 0; i < 8; i++) t.scales[i] = 0x11;
+                for (int i = 8; i < 12; i++) t.scales[i] = 0xAA;
+                t.d = 0x3c00;
+                orc_dequantize_row(ORC_TYPE_Q3_K, &t, wi + 256 * b, 256);
+            }
+            for (int g = 0; g < 16; g++) {
+                int64_t dot = 0;
+                for (int l = 0; l < 16; l++) dot += (int64_t)wi[256 * b + 16 * g + l] * y[b].qs[16 * g + l];
+                const double t1 = d * (double)sc[g] * (double)dot;
+                const double t2 = dm * (double)mn[g] * (double)y[b].bsums[g];
+                s += t1 - t2; sa += fabs(t1) + fabs(t2);
+            }
+        }
+        free(wi);
     } else { s = NAN; }
     free(is);
     if (sum_abs) *sum_abs = sa;

@@ -1,6 +1,7 @@
 """Writes tests/golden/*.npz from the reference's own compiled code (oracle/_ref/libggml_ref.so).
 
-Run in the build container, where the reference tree is mounted:  python tests/golden/make_golden.py
+Run in the build container, where the reference tree is mounted:  python tests/golden/make_golden.py [type names]
+(with type names, e.g. "q3_K q2_K", only the mul_mat fixtures of those types are written).
 The fixtures hold data only: seeded inputs and the bytes / floats the reference produced for them.
 """
 import os
@@ -20,8 +21,11 @@ def main():
     O.build()
     r = O.Reference()
     K, N, n = 512, 3, 2
+    only = sys.argv[1:]
     for wt in O.WEIGHT_TYPES:
         name = O.TYPE_NAMES[wt]
+        if only and name not in only:
+            continue
         w = common.weights_f32(100 + wt, N, K, outliers=(wt in (O.Q4_K, O.Q6_K)))
         x = common.activations_f32(100 + wt, n, K)
         wq = r.quantize_weights(wt, w)
@@ -35,6 +39,8 @@ def main():
         np.savez_compressed(os.path.join(HERE, "mul_mat_%s.npz" % name),
                             wtype=np.int32(wt), K=np.int32(K), w=w, x=x, wq=wq, xq=xq,
                             w_deq=r.dequantize(wt, wq, K), y_dot=y_dot, y_graph=y_graph)
+    if only:
+        return
     # LM_GGML_OP_MUL_MAT_ID from the reference's CPU graph: 5 experts, 3 used per token, per-slot activations for one
     # type and activations shared by a token's slots for the other
     for wt, ne11 in ((O.Q4_K, 1), (O.Q8_0, 3)):

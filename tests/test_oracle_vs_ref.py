@@ -47,6 +47,32 @@ def test_weight_quantizers_and_dots(orc, ref, wt):
             assert orc.vec_dot(wt, K, b[i], xq[t]).tobytes() == ref.vec_dot(wt, K, b[i], xq[t]).tobytes()
 
 
+@pytest.mark.parametrize("wt", O.LOW_BIT_K_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+def test_low_bit_k_quants_on_random_bytes(orc, ref, wt):
+    """Q3_K and Q2_K over random block bytes with sane fp16 super-block scales: every code of the packed scales (Q3_K's below
+    32, i.e. negative ones, included), every quant and high-bit pattern; dequantizer and dot bit for bit the reference's."""
+    K, N, n = 1024, 16, 2
+    rng = np.random.default_rng(77 + wt)
+    bb, nb = O.BLOCK_BYTES[wt], K // 256
+    b = rng.integers(0, 256, (N, nb, bb), dtype=np.uint8)
+    d = (0.01 * np.exp(rng.uniform(-1, 1, (N, nb)))).astype(np.float16)
+    d[rng.random((N, nb)) < 0.2] *= np.float16(-1)
+    off = 108 if wt == O.Q3_K else 80
+    b[..., off:off + 2] = d.view(np.uint8).reshape(N, nb, 2)
+    if wt == O.Q2_K:
+        b[..., 82:84] = (d * np.float16(0.5)).view(np.uint8).reshape(N, nb, 2)
+    b = b.reshape(N, nb * bb)
+    assert np.array_equal(orc.dequantize(wt, b, K), ref.dequantize(wt, b, K))
+    xq = ref.quantize_activation(O.Q8_K, common.activations_f32(wt, n, K))
+    for t in range(n):
+        for i in range(N):
+            assert orc.vec_dot(wt, K, b[i], xq[t]).tobytes() == ref.vec_dot(wt, K, b[i], xq[t]).tobytes()
+            # the integer sums are those of the dequantized integers (d = 1: the super-block scale taken out)
+            v, isum, imin = orc.vec_dot(wt, K, b[i], xq[t], want_sums=True)
+            exact, sum_abs = orc.vec_dot_exact(wt, K, b[i], xq[t])
+            assert abs(float(v) - exact) <= 1e-5 * sum_abs
+
+
 @pytest.mark.parametrize("wt", O.WEIGHT_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("n,threads", [(1, 1), (5, 3)])
 def test_mul_mat_graph(orc, ref, wt, n, threads):
