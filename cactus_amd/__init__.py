@@ -20,14 +20,14 @@ BACKEND_LIB = os.path.join(LIB_DIR, "libggml-hip.so")
 
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
-Q2_K, Q3_K = 10, 11
+Q2_K, Q3_K, IQ4_XS = 10, 11, 23
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
 F16 = 1
 CHIP_OK, CHIP_EINVAL, CHIP_EUNSUPPORTED, CHIP_ENOMEM = 0, -1, -2, -3        # include/cactus_hip.h
 TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
               Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16", Q3_K: "q3_K",
-              Q2_K: "q2_K"}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, Q3_K, Q2_K, F16)
+              Q2_K: "q2_K", IQ4_XS: "iq4_xs"}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, Q3_K, Q2_K, IQ4_XS, F16)
 
 # every symbol include/cactus_hip.h declares
 EXPORTS = (

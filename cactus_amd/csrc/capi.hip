@@ -83,7 +83,7 @@ int current_limits(DeviceLimits &out) {
 
 bool is_weight_type(int t) {
     return t == T_Q4_0 || t == T_Q8_0 || t == T_Q4_K || t == T_Q6_K || t == T_Q5_0 || t == T_Q5_K || t == T_IQ4_NL ||
-           t == T_Q4_1 || t == T_Q5_1 || t == T_F16 || t == T_Q3_K || t == T_Q2_K;
+           t == T_Q4_1 || t == T_Q5_1 || t == T_F16 || t == T_Q3_K || t == T_Q2_K || t == T_IQ4_XS;
 }
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -95,8 +95,8 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 // dot-product GEMV; the GEMM, whose staging reads single blocks, when K % 128 == 0).
 bool is_block32_type(int t) { return t == T_Q4_0 || t == T_Q8_0 || t == T_Q5_0 || t == T_IQ4_NL || t == T_Q4_1 || t == T_Q5_1; }
 bool weights_aligned(int type, const void *W, size_t nb01, int64_t K = 256) {
-    // (Q3_K: 110-byte super-blocks, as Q6_K's 210; Q2_K: 84 bytes)
-    const size_t a = (type == T_Q6_K || type == T_Q3_K) ? 2 : (type == T_Q2_K || (is_block32_type(type) && K % 256 != 0)) ? 4 : 16;
+    // (Q3_K: 110-byte super-blocks, as Q6_K's 210; Q2_K: 84 bytes; IQ4_XS: 136 bytes, loaded as an 8-byte and 4-byte aligned pieces)
+    const size_t a = (type == T_Q6_K || type == T_Q3_K) ? 2 : type == T_Q2_K ? 4 : type == T_IQ4_XS ? 8 : (is_block32_type(type) && K % 256 != 0) ? 4 : 16;
     return ((uintptr_t)W % a) == 0 && (nb01 % a) == 0;
 }
 
@@ -233,7 +233,7 @@ int chip_block_elems(int type) {
     switch (type) {
         case T_F32: case T_F16: return 1;
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: case T_Q8_1: return 32;
-        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: return 256;
+        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: return 256;
         default: return 0;
     }
 }
@@ -254,6 +254,7 @@ size_t chip_block_bytes(int type) {
         case T_Q8_1: return BYTES_Q8_1;
         case T_Q3_K: return BYTES_Q3_K;
         case T_Q2_K: return BYTES_Q2_K;
+        case T_IQ4_XS: return BYTES_IQ4_XS;
         default: return 0;
     }
 }
@@ -264,7 +265,7 @@ size_t chip_row_size(int type, int64_t k) {
 int chip_vec_dot_type(int type) {
     switch (type) {
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return T_Q8_0;
-        case T_Q4_K: case T_Q6_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: return T_Q8_K;
+        case T_Q4_K: case T_Q6_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: return T_Q8_K;
         case T_Q4_1: case T_Q5_1: return T_Q8_1;
         case T_F16: return T_F16;
         default: return -1;
@@ -749,7 +750,7 @@ int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K
 
     const bool kq = type == T_Q4_K || type == T_Q5_K || type == T_Q6_K;
     // (the 2- and 3-bit K-quants have no GEMM of their own: every pair takes the GEMV)
-    const bool have_gemm = (type == T_Q3_K || type == T_Q2_K) ? false : type == T_F16 ? K % 64 == 0 : (kq ? true : K % 128 == 0);
+    const bool have_gemm = (type == T_Q3_K || type == T_Q2_K || type == T_IQ4_XS) ? false : type == T_F16 ? K % 64 == 0 : (kq ? true : K % 128 == 0);
     if (pairs >= MOE_GEMM_MIN_PAIRS && have_gemm && moe_group_supported(n_as, pairs)) {
         rc = chip_mul_mat_prepare(type, K, x, ldx, rows, workspace, workspace_bytes, stream);
         if (rc) return rc;

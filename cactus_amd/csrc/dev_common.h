@@ -14,9 +14,10 @@ constexpr int QK_K     = 256;    // elements per K-quant super-block
 constexpr int BYTES_Q4_0 = 18, BYTES_Q8_0 = 34, BYTES_Q4_K = 144, BYTES_Q6_K = 210, BYTES_Q8_K = 292;
 constexpr int BYTES_Q5_0 = 22, BYTES_Q5_K = 176, BYTES_IQ4_NL = 18, BYTES_Q4_1 = 20, BYTES_Q5_1 = 24, BYTES_Q8_1 = 36;
 constexpr int BYTES_Q2_K = 84, BYTES_Q3_K = 110;   // reference ggml-common.h:254-266, 273-278
+constexpr int BYTES_IQ4_XS = 136;                  // ggml-common.h:412-417
 
 enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15, T_Q5_0 = 6, T_Q5_K = 13, T_IQ4_NL = 20,
-              T_Q4_1 = 3, T_Q5_1 = 7, T_Q8_1 = 9, T_F16 = 1, T_Q2_K = 10, T_Q3_K = 11 };
+              T_Q4_1 = 3, T_Q5_1 = 7, T_Q8_1 = 9, T_F16 = 1, T_Q2_K = 10, T_Q3_K = 11, T_IQ4_XS = 23 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

@@ -180,6 +180,7 @@ int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
         case T_Q5_K: return max_tokens_typed<T_Q5_K>(K, lim);
         case T_Q3_K: return max_tokens_typed<T_Q3_K>(K, lim);
         case T_Q2_K: return max_tokens_typed<T_Q2_K>(K, lim);
+        case T_IQ4_XS: return max_tokens_typed<T_IQ4_XS>(K, lim);
         case T_IQ4_NL: return max_tokens_typed<T_IQ4_NL>(K, lim);
         case T_Q4_1: return max_tokens_typed<T_Q4_1>(K, lim);
         case T_Q5_1: return max_tokens_typed<T_Q5_1>(K, lim);
@@ -201,6 +202,7 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
         case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q3_K: return launch_ntok<T_Q3_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q2_K: return launch_ntok<T_Q2_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_IQ4_XS: return launch_ntok<T_IQ4_XS, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q4_1: return launch_ntok<T_Q4_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q5_1: return launch_ntok<T_Q5_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
@@ -224,6 +226,7 @@ hipError_t launch_gemv_sec(int wtype, const void *W, size_t nb01, int64_t K, int
         case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q3_K: return launch_ntok<T_Q3_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q2_K: return launch_ntok<T_Q2_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_IQ4_XS: return launch_ntok<T_IQ4_XS, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q4_1: return launch_ntok<T_Q4_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q5_1: return launch_ntok<T_Q5_1, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
@@ -262,6 +265,7 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
         case T_Q5_K: img = lds_image_bytes<T_Q5_K>(K); break;
         case T_Q3_K: img = lds_image_bytes<T_Q3_K>(K); break;
         case T_Q2_K: img = lds_image_bytes<T_Q2_K>(K); break;
+        case T_IQ4_XS: img = lds_image_bytes<T_IQ4_XS>(K); break;
         case T_IQ4_NL: img = lds_image_bytes<T_IQ4_NL>(K); break;
         case T_Q4_1: img = lds_image_bytes<T_Q4_1>(K); break;
         case T_Q5_1: img = lds_image_bytes<T_Q5_1>(K); break;
@@ -281,6 +285,7 @@ bool gemv_norm_prologue_applicable(int wtype, int64_t K, int n, const DeviceLimi
         case T_Q5_K: iters = iters_per_row<T_Q5_K>(K); break;
         case T_Q3_K: iters = iters_per_row<T_Q3_K>(K); break;
         case T_Q2_K: iters = iters_per_row<T_Q2_K>(K); break;
+        case T_IQ4_XS: iters = iters_per_row<T_IQ4_XS>(K); break;
         case T_Q6_K: iters = iters_per_row<T_Q6_K>(K); break;
         default: break;
     }
@@ -341,6 +346,7 @@ static hipError_t launch_gemv_fused_sec(int wtype, const void *W, size_t nb01, i
         case T_Q5_K: return launch_ntok<T_Q5_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q3_K: return launch_ntok<T_Q3_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q2_K: return launch_ntok<T_Q2_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_IQ4_XS: return launch_ntok<T_IQ4_XS, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_IQ4_NL: return launch_ntok<T_IQ4_NL, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q4_1: return launch_ntok<T_Q4_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q5_1: return launch_ntok<T_Q5_1, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
@@ -388,7 +394,7 @@ hipError_t launch_gemv_id(int wtype, bool fused, const void *W, size_t nb01, siz
                                           : launch_id_typed<TT, false>(W, nb01, K, N, nullptr, 0, ws, ws_stride, y, ldy, m, pairs, lim, st);
     switch (wtype) {
         ID_CASE(T_Q4_0) ID_CASE(T_Q8_0) ID_CASE(T_Q4_K) ID_CASE(T_Q6_K) ID_CASE(T_Q5_0) ID_CASE(T_Q5_K) ID_CASE(T_IQ4_NL)
-        ID_CASE(T_Q4_1) ID_CASE(T_Q5_1) ID_CASE(T_F16) ID_CASE(T_Q3_K) ID_CASE(T_Q2_K)
+        ID_CASE(T_Q4_1) ID_CASE(T_Q5_1) ID_CASE(T_F16) ID_CASE(T_Q3_K) ID_CASE(T_Q2_K) ID_CASE(T_IQ4_XS)
         default: return hipErrorInvalidValue;
     }
 #undef ID_CASE
@@ -488,6 +494,7 @@ hipError_t launch_block_isums(int wtype, const void *W, size_t nb01, int64_t K, 
         case T_Q5_K: hipLaunchKernelGGL(block_isums_kernel<T_Q5_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q3_K: hipLaunchKernelGGL(block_isums_kernel<T_Q3_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q2_K: hipLaunchKernelGGL(block_isums_kernel<T_Q2_K>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
+        case T_IQ4_XS: hipLaunchKernelGGL(block_isums_kernel<T_IQ4_XS>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_IQ4_NL: hipLaunchKernelGGL(block_isums_kernel<T_IQ4_NL>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q4_1: hipLaunchKernelGGL(block_isums_kernel<T_Q4_1>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;
         case T_Q5_1: hipLaunchKernelGGL(block_isums_kernel<T_Q5_1>, grid, dim3(64), 0, st, (const uint8_t *)W, nb01, K, N, (const uint8_t *)aq, isum, imin); break;

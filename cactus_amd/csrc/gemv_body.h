@@ -754,6 +754,48 @@ template <int WT> __host__ __device__ constexpr size_t lds_image_bytes(int64_t K
     return (size_t)iters_per_row<WT>(K) * (Traits<WT>::QCH * 1024 + 64 * Traits<WT>::AUX);
 }
 
+// IQ4_XS (reference type_traits_cpu[], ggml-cpu/ggml-cpu.c:340-345; lm_ggml_vec_dot_iq4_xs_q8_K, ggml-cpu/ggml-cpu-quants.c:12965 ff.;
+// dequantize_row_iq4_xs, ggml-quants.c): IQ4_NL's code points in 256-value super-blocks with a 6-bit scale (biased by 32) per
+// 32-value sub-block and Q8_K activations.  block_iq4_xs (ggml-common.h:412-417): fp16 d | u16 scales_h | scales_l[4] | qs[128],
+// 136 bytes, 8-byte aligned.  Sub-block ib is the 16 bytes qs[16 ib ...]: low nibbles elements 0..15, high nibbles 16..31.
+// Q4_K's unit (super-block, 64-value group jp = sub-blocks 2 jp and 2 jp + 1, 64 consecutive activation quants) carries it.
+template <> struct Traits<T_IQ4_XS> : Traits<T_Q4_K> {
+    struct W { uint32_t q[16]; float d; int ls0, ls1; };          // signed code points in element order
+    struct Raw { u32x2 h; u32x4 q0, q1; };
+    __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
+        const int sb = u >> 2, jp = u & 3;
+        const uint8_t *p = row + (size_t)sb * BYTES_IQ4_XS;
+        r.h = WLOAD(reinterpret_cast<const u32x2 *>(p));
+        r.q0 = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 8 + 32 * jp));
+        r.q1 = WLOAD(reinterpret_cast<const u32x4_a4 *>(p + 24 + 32 * jp));
+    }
+    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+        const int jp = u & 3;
+        w.d = h2f(r.h.x);
+        const uint32_t sh = (r.h.x >> 16) >> (4 * jp), sl = (r.h.y >> (8 * jp)) & 0xffu;   // scales_h bits of 2jp, 2jp+1; scales_l[jp]
+        w.ls0 = (int)((sl & 0xfu) | ((sh & 3u) << 4)) - 32;
+        w.ls1 = (int)((sl >> 4) | (((sh >> 2) & 3u) << 4)) - 32;
+        const uint32_t a[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w}, b[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w.q[i]      = Traits<T_IQ4_NL>::lookup4(a[i] & 0x0f0f0f0fu);   w.q[4 + i]  = Traits<T_IQ4_NL>::lookup4((a[i] >> 4) & 0x0f0f0f0fu);
+            w.q[8 + i]  = Traits<T_IQ4_NL>::lookup4(b[i] & 0x0f0f0f0fu);   w.q[12 + i] = Traits<T_IQ4_NL>::lookup4((b[i] >> 4) & 0x0f0f0f0fu);
+        }
+    }
+    __device__ static __forceinline__ void isums(const W &w, const A &a, int &is, int &unused) {
+        int d0 = 0, d1 = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { d0 = dot4(w.q[i], a.q[i], d0); d1 = dot4(w.q[8 + i], a.q[8 + i], d1); }
+        is = w.ls0 * d0 + w.ls1 * d1;
+        unused = 0;
+    }
+    __device__ static __forceinline__ float dot(const W &w, const A &a, float acc) {
+        int is, unused;
+        isums(w, a, is, unused);
+        return __builtin_fmaf(w.d * a.d, (float)is, acc);
+    }
+};
+
 // ------------------------------------------------------------------------------------------------ kernel
 // Fused prologue: quantize NTOK fp32 rows straight into the LDS image; workgroup 0 also writes the split
 // workspace planes so the quantized activations exist in memory as the reference's wdata does.

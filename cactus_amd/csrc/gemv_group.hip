@@ -59,6 +59,7 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
             case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             case T_Q3_K: run_member<T_Q3_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             case T_Q2_K: run_member<T_Q2_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_IQ4_XS: run_member<T_IQ4_XS, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else if constexpr (FAMILY == 1) {
@@ -85,6 +86,7 @@ size_t image_bytes(int wtype, int64_t K) {
         case T_Q5_K: return lds_image_bytes<T_Q5_K>(K);
         case T_Q3_K: return lds_image_bytes<T_Q3_K>(K);
         case T_Q2_K: return lds_image_bytes<T_Q2_K>(K);
+        case T_IQ4_XS: return lds_image_bytes<T_IQ4_XS>(K);
         case T_IQ4_NL: return lds_image_bytes<T_IQ4_NL>(K);
         case T_Q4_1: return lds_image_bytes<T_Q4_1>(K);
         case T_Q5_1: return lds_image_bytes<T_Q5_1>(K);
@@ -142,7 +144,7 @@ hipError_t launch_ntok(int n, int wgs, const GroupKernelArgs &ga, int grid, int6
 
 int gemv_group_family(int wtype) {
     switch (wtype) {
-        case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_Q3_K: case T_Q2_K: return 0;
+        case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: return 0;
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: return 1;
         case T_F16: return 2;
         default: return -1;

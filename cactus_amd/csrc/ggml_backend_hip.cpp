@@ -237,6 +237,7 @@ bool is_view_op(int op) {
 // bytes (Q2_K) and rows of K % 256 != 0 (32-value block types only) 4, everything else 16.
 size_t weight_alignment(const lm_ggml_tensor *w) {
     if (w->type == LM_GGML_TYPE_Q6_K || w->type == LM_GGML_TYPE_Q3_K) return 2;
+    if (w->type == LM_GGML_TYPE_IQ4_XS) return 8;                     // 136-byte super-blocks
     return (w->type == LM_GGML_TYPE_Q2_K || w->ne[0] % 256 != 0) ? 4 : 16;
 }
 // The MUL_MAT shapes the kernels take: weights [K, N] of a supported block type with whole-row strides, F32

@@ -620,6 +620,13 @@ template <int WT> __device__ __forceinline__ float dequant_at(const uint8_t *row
         int v = hi ? (q >> 4) : (q & 0xF);
         if constexpr (WT == T_Q5_K) v += (b[16 + ll] & (1u << (2 * j64 + hi))) ? 16 : 0;
         return d1 * (float)v - m1;
+    } else if constexpr (WT == T_IQ4_XS) {                              // d scales_h scales_l[4] qs[128] (ggml-quants.c dequantize_row_iq4_xs)
+        const uint8_t *b = row + (size_t)(i >> 8) * BYTES_IQ4_XS;
+        const uint32_t r = i & 255, ib = r >> 5, j = r & 31;
+        const uint32_t sh = reinterpret_cast<const uint16_t *>(b)[1];
+        const int ls = (int)(((b[4 + (ib >> 1)] >> (4 * (ib & 1))) & 0xFu) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+        const int q = b[8 + 16 * ib + (j & 15)], nib = j < 16 ? (q & 0xF) : (q >> 4);
+        return h2f(reinterpret_cast<const uint16_t *>(b)[0]) * (float)ls * (float)k_iq4nl_values[nib];
     } else if constexpr (WT == T_Q2_K) {                                // scales[16] qs[64] d dmin (reference ggml-quants.c:706-737)
         const uint8_t *b = row + (size_t)(i >> 8) * BYTES_Q2_K;
         const uint32_t r = i & 255, h = r >> 7, j = (r >> 5) & 3, l = r & 31;
@@ -673,7 +680,7 @@ hipError_t launch_get_rows(int type, const GetRowsArgs &a, hipStream_t st) {
 #define GR_CASE(TT) case TT: hipLaunchKernelGGL(get_rows_kernel<TT>, grid, dim3(EW_THREADS), 0, st, a); break;
     switch (type) {
         GR_CASE(T_F32) GR_CASE(T_F16) GR_CASE(T_Q4_0) GR_CASE(T_Q4_1) GR_CASE(T_Q5_0) GR_CASE(T_Q5_1) GR_CASE(T_Q8_0)
-        GR_CASE(T_Q4_K) GR_CASE(T_Q5_K) GR_CASE(T_Q6_K) GR_CASE(T_IQ4_NL) GR_CASE(T_Q3_K) GR_CASE(T_Q2_K)
+        GR_CASE(T_Q4_K) GR_CASE(T_Q5_K) GR_CASE(T_Q6_K) GR_CASE(T_IQ4_NL) GR_CASE(T_Q3_K) GR_CASE(T_Q2_K) GR_CASE(T_IQ4_XS)
         default: return hipErrorInvalidValue;
     }
 #undef GR_CASE

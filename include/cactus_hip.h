@@ -39,10 +39,11 @@ enum chip_type {
     CHIP_TYPE_Q4_1   = 3,
     CHIP_TYPE_Q5_1   = 7,
     CHIP_TYPE_Q8_1   = 9,    /* activation format of Q4_1 / Q5_1 (ggml-cpu/ggml-cpu.c:221,237) */
-    /* the 2- and 3-bit K-quants (ggml-cpu/ggml-cpu.c:257-268; Q8_K activations): dot-product GEMV at every token count (in
-     * passes of up to 8 tokens), GET_ROWS, MUL_MAT_ID per pair; no matrix-core kernels of their own */
+    /* the 2- and 3-bit K-quants and IQ4_XS (ggml-cpu/ggml-cpu.c:257-268, 340-345; Q8_K activations): dot-product GEMV at every
+     * token count (in passes of up to 8 tokens), GET_ROWS, MUL_MAT_ID per pair; no matrix-core kernels of their own */
     CHIP_TYPE_Q2_K   = 10,
     CHIP_TYPE_Q3_K   = 11,
+    CHIP_TYPE_IQ4_XS = 23,
 };
 
 enum chip_status {

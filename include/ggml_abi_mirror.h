@@ -34,7 +34,7 @@ extern "C" {
 /* enum values used on this path (the enums themselves are plain ints in the ABI) */
 enum {
     LM_GGML_TYPE_F32 = 0, LM_GGML_TYPE_F16 = 1, LM_GGML_TYPE_Q4_0 = 2, LM_GGML_TYPE_Q8_0 = 8,
-    LM_GGML_TYPE_Q2_K = 10, LM_GGML_TYPE_Q3_K = 11,
+    LM_GGML_TYPE_Q2_K = 10, LM_GGML_TYPE_Q3_K = 11, LM_GGML_TYPE_IQ4_XS = 23,
     LM_GGML_TYPE_Q4_K = 12, LM_GGML_TYPE_Q6_K = 14, LM_GGML_TYPE_Q8_K = 15, LM_GGML_TYPE_I32 = 26,
 };
 enum {

@@ -19,19 +19,19 @@ F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
 F16 = 1
-Q2_K, Q3_K = 10, 11
-TYPE_NAMES = {Q2_K: "q2_K", Q3_K: "q3_K", F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
+Q2_K, Q3_K, IQ4_XS = 10, 11, 23
+TYPE_NAMES = {Q2_K: "q2_K", Q3_K: "q3_K", IQ4_XS: "iq4_xs", F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
               Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16"}
-BLOCK_ELEMS = {Q2_K: 256, Q3_K: 256, F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32,
+BLOCK_ELEMS = {Q2_K: 256, Q3_K: 256, IQ4_XS: 256, F32: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256, Q5_0: 32, Q5_K: 256, IQ4_NL: 32,
                Q4_1: 32, Q5_1: 32, Q8_1: 32, F16: 1}
-BLOCK_BYTES = {Q2_K: 84, Q3_K: 110, F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18,
+BLOCK_BYTES = {Q2_K: 84, Q3_K: 110, IQ4_XS: 136, F32: 4, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292, Q5_0: 22, Q5_K: 176, IQ4_NL: 18,
                Q4_1: 20, Q5_1: 24, Q8_1: 36, F16: 2}
-VEC_DOT_TYPE = {Q2_K: Q8_K, Q3_K: Q8_K, Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0,
+VEC_DOT_TYPE = {Q2_K: Q8_K, Q3_K: Q8_K, IQ4_XS: Q8_K, Q4_0: Q8_0, Q8_0: Q8_0, Q4_K: Q8_K, Q6_K: Q8_K, Q5_0: Q8_0, Q5_K: Q8_K, IQ4_NL: Q8_0,
                 Q4_1: Q8_1, Q5_1: Q8_1, F16: F16}
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, Q3_K, Q2_K, F16)
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, Q3_K, Q2_K, IQ4_XS, F16)
 BLOCK_WEIGHT_TYPES = WEIGHT_TYPES[:-1]        # the types with per-block integer sums
-# the 2- and 3-bit K-quants: decode and small batches on the GEMV kernels, no matrix-core kernels of their own
-LOW_BIT_K_TYPES = (Q3_K, Q2_K)
+# the 2- and 3-bit K-quants and IQ4_XS: decode and small batches on the GEMV kernels, no matrix-core kernels of their own
+LOW_BIT_K_TYPES = (Q3_K, Q2_K, IQ4_XS)
 # types whose weight quantizer is restated in the oracle (IQ4_NL, Q3_K and Q2_K weights come from the reference build, from
 # the golden fixture, from a plain quantizer here, or are random bytes: any byte string is a valid block)
 ORACLE_QUANTIZED = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, Q4_1, Q5_1, F16)
@@ -138,6 +138,35 @@ def plain_q2_K_rows(w):
     return out.reshape(n, nb * 84)
 
 
+def plain_iq4_xs_rows(w):
+    """fp32 [N, K] -> IQ4_XS rows by a plain quantizer: 32-value sub-block scale = max|x| / 127 (signed like the largest
+    element), super-block d = largest |scale| / 31, 6-bit codes ls = round(scale / d) + 32, index = nearest code point of
+    x / (d (ls - 32)).  Not the reference's search."""
+    w = np.ascontiguousarray(w, np.float32)
+    n, k = w.shape
+    nb = k // 256
+    blk = w.reshape(n, nb, 8, 32)
+    imax = np.abs(blk).argmax(-1)
+    mx = np.take_along_axis(blk, imax[..., None], -1)[..., 0]
+    sc = mx / np.float32(-127)
+    d = (np.abs(sc).max(-1) / np.float32(31)).astype(np.float16)
+    df = d.astype(np.float32)[..., None]
+    ls = np.where(df > 0, np.rint(sc / np.where(df > 0, df, 1)), 0).clip(-32, 31).astype(np.int32)
+    step = (df * ls)[..., None]
+    idx = np.abs(np.where(step != 0, blk / np.where(step != 0, step, 1), 0)[..., None] - IQ4_NL_VALUES).argmin(-1).astype(np.uint8)
+    code = (ls + 32).astype(np.uint16)
+    out = np.zeros((n, nb, 136), np.uint8)
+    out[..., 0:2] = d.view(np.uint8).reshape(n, nb, 2)
+    sh = np.zeros((n, nb), np.uint16)
+    for ib in range(8):
+        sh |= ((code[..., ib] >> 4) & 3) << (2 * ib)
+    out[..., 2:4] = sh.view(np.uint8).reshape(n, nb, 2)
+    lo = (code & 15).astype(np.uint8)
+    out[..., 4:8] = lo[..., 0::2] | (lo[..., 1::2] << 4)
+    out[..., 8:] = (idx[..., :16] | (idx[..., 16:] << 4)).reshape(n, nb, 128)
+    return out.reshape(n, nb * 136)
+
+
 def row_size(t, k):
     return (k // BLOCK_ELEMS[t]) * BLOCK_BYTES[t]
 
@@ -186,7 +215,7 @@ class Oracle:
         L.orc_quantize_rows.argtypes = [_i32, _vp, _vp, _i64, _i64]
         L.orc_dequantize_row.restype = None
         L.orc_dequantize_row.argtypes = [_i32, _vp, _vp, _i64]
-        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0", "q4_1_q8_1", "q5_1_q8_1", "q3_K_q8_K"):
+        for n in ("q4_0_q8_0", "q8_0_q8_0", "q6_K_q8_K", "q5_0_q8_0", "iq4_nl_q8_0", "q4_1_q8_1", "q5_1_q8_1", "q3_K_q8_K", "iq4_xs_q8_K"):
             f = getattr(L, "orc_vec_dot_" + n)
             f.restype = C.c_float
             f.argtypes = [_i64, _vp, _vp, _vp]
@@ -251,6 +280,8 @@ class Oracle:
             return plain_q3_K_rows(w)
         if wtype == Q2_K:
             return plain_q2_K_rows(w)
+        if wtype == IQ4_XS:
+            return plain_iq4_xs_rows(w)
         out = np.zeros((n, row_size(wtype, k)), np.uint8)
         got = self.lib.orc_quantize_rows(wtype, _ptr(w), _ptr(out), n, k)
         assert got == out.size
@@ -291,6 +322,8 @@ class Oracle:
             v = self.lib.orc_vec_dot_q2_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum), _ptr(imin))
         elif wtype == Q3_K:
             v = self.lib.orc_vec_dot_q3_K_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum))
+        elif wtype == IQ4_XS:
+            v = self.lib.orc_vec_dot_iq4_xs_q8_K(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q4_1:
             v = self.lib.orc_vec_dot_q4_1_q8_1(k, _ptr(wrow), _ptr(arow), _ptr(isum))
         elif wtype == Q5_1:
@@ -469,17 +502,17 @@ class Reference:
                   "quantize_row_q4_K_ref", "quantize_row_q6_K_ref", "quantize_row_q8_K_ref",
                   "quantize_row_q5_0_ref", "quantize_row_q5_K_ref", "quantize_row_iq4_nl_ref",
                   "quantize_row_q4_1_ref", "quantize_row_q5_1_ref", "quantize_row_q8_1",
-                  "quantize_row_q2_K_ref", "quantize_row_q3_K_ref",
+                  "quantize_row_q2_K_ref", "quantize_row_q3_K_ref", "quantize_row_iq4_xs_ref",
                   "lm_ggml_fp32_to_fp16_row", "lm_ggml_cpu_fp32_to_fp16", "lm_ggml_fp16_to_fp32_row"):
             f = getattr(L, n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
-        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl", "q4_1", "q5_1", "q2_K", "q3_K"):
+        for n in ("q4_0", "q8_0", "q4_K", "q6_K", "q8_K", "q5_0", "q5_K", "iq4_nl", "q4_1", "q5_1", "q2_K", "q3_K", "iq4_xs"):
             f = getattr(L, "dequantize_row_" + n)
             f.restype = None
             f.argtypes = [_vp, _vp, _i64]
         for n in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "q5_0_q8_0", "q5_K_q8_K", "iq4_nl_q8_0",
-                  "q4_1_q8_1", "q5_1_q8_1", "f16", "q2_K_q8_K", "q3_K_q8_K"):
+                  "q4_1_q8_1", "q5_1_q8_1", "f16", "q2_K_q8_K", "q3_K_q8_K", "iq4_xs_q8_K"):
             f = getattr(L, "lm_ggml_vec_dot_" + n)
             f.restype = None
             f.argtypes = [C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, _vp, C.c_size_t, C.c_int]
@@ -547,12 +580,12 @@ class Reference:
            Q4_K: "quantize_row_q4_K_ref", Q6_K: "quantize_row_q6_K_ref",
            Q5_0: "quantize_row_q5_0_ref", Q5_K: "quantize_row_q5_K_ref", IQ4_NL: "quantize_row_iq4_nl_ref",
            Q4_1: "quantize_row_q4_1_ref", Q5_1: "quantize_row_q5_1_ref", F16: "lm_ggml_fp32_to_fp16_row",
-           Q2_K: "quantize_row_q2_K_ref", Q3_K: "quantize_row_q3_K_ref"}
+           Q2_K: "quantize_row_q2_K_ref", Q3_K: "quantize_row_q3_K_ref", IQ4_XS: "quantize_row_iq4_xs_ref"}
     _DOT = {Q4_0: "lm_ggml_vec_dot_q4_0_q8_0", Q8_0: "lm_ggml_vec_dot_q8_0_q8_0",
             Q4_K: "lm_ggml_vec_dot_q4_K_q8_K", Q6_K: "lm_ggml_vec_dot_q6_K_q8_K",
             Q5_0: "lm_ggml_vec_dot_q5_0_q8_0", Q5_K: "lm_ggml_vec_dot_q5_K_q8_K", IQ4_NL: "lm_ggml_vec_dot_iq4_nl_q8_0",
             Q4_1: "lm_ggml_vec_dot_q4_1_q8_1", Q5_1: "lm_ggml_vec_dot_q5_1_q8_1", F16: "lm_ggml_vec_dot_f16",
-            Q2_K: "lm_ggml_vec_dot_q2_K_q8_K", Q3_K: "lm_ggml_vec_dot_q3_K_q8_K"}
+            Q2_K: "lm_ggml_vec_dot_q2_K_q8_K", Q3_K: "lm_ggml_vec_dot_q3_K_q8_K", IQ4_XS: "lm_ggml_vec_dot_iq4_xs_q8_K"}
 
     def quantize_activation(self, act_type, x):
         x = _f32(x)

@@ -31,6 +31,8 @@ typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } blk_q8_1;
 /* 2- and 3-bit K-quants: ggml-common.h:254-266 (q2_K), :273-278 (q3_K) */
 typedef struct { uint8_t scales[16]; uint8_t qs[64]; uint16_t d; uint16_t dmin; } blk_q2_K;
 typedef struct { uint8_t hmask[32]; uint8_t qs[64]; uint8_t scales[12]; uint16_t d; } blk_q3_K;
+/* ggml-common.h:412-417: the non-linear 4-bit code points with 6-bit sub-block scales */
+typedef struct { uint16_t d; uint16_t scales_h; uint8_t scales_l[4]; uint8_t qs[128]; } blk_iq4_xs;
 #pragma pack(pop)
 
 _Static_assert(sizeof(blk_q4_0) == 18, "q4_0");
@@ -46,6 +48,7 @@ _Static_assert(sizeof(blk_q5_1) == 24, "q5_1");
 _Static_assert(sizeof(blk_q8_1) == 36, "q8_1");
 _Static_assert(sizeof(blk_q2_K) == 84, "q2_K");
 _Static_assert(sizeof(blk_q3_K) == 110, "q3_K");
+_Static_assert(sizeof(blk_iq4_xs) == 136, "iq4_xs");
 
 /* ggml-quants.c:2428: the 16 code points of the non-linear 4-bit types. */
 static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
@@ -56,7 +59,7 @@ int orc_block_elems(int type) {
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL:
         case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: case ORC_TYPE_Q8_1: return 32;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: case ORC_TYPE_Q8_K: return 256;
-        case ORC_TYPE_Q2_K: case ORC_TYPE_Q3_K: return 256;
+        case ORC_TYPE_Q2_K: case ORC_TYPE_Q3_K: case ORC_TYPE_IQ4_XS: return 256;
         default: return 0;
     }
 }
@@ -77,6 +80,7 @@ size_t orc_block_bytes(int type) {
         case ORC_TYPE_Q8_1: return 36;
         case ORC_TYPE_Q2_K: return 84;
         case ORC_TYPE_Q3_K: return 110;
+        case ORC_TYPE_IQ4_XS: return 136;
         default: return 0;
     }
 }
@@ -89,6 +93,7 @@ int orc_vec_dot_type(int type) {
         case ORC_TYPE_Q4_0: case ORC_TYPE_Q8_0: case ORC_TYPE_Q5_0: case ORC_TYPE_IQ4_NL: return ORC_TYPE_Q8_0;
         case ORC_TYPE_Q4_K: case ORC_TYPE_Q5_K: case ORC_TYPE_Q6_K: return ORC_TYPE_Q8_K;
         case ORC_TYPE_Q2_K: case ORC_TYPE_Q3_K: return ORC_TYPE_Q8_K;   /* ggml-cpu/ggml-cpu.c:257-268 */
+        case ORC_TYPE_IQ4_XS: return ORC_TYPE_Q8_K;                     /* ggml-cpu/ggml-cpu.c:340-345 */
         case ORC_TYPE_Q4_1: case ORC_TYPE_Q5_1: return ORC_TYPE_Q8_1;   /* ggml-cpu/ggml-cpu.c:221,237 */
         case ORC_TYPE_F16: return ORC_TYPE_F16;                        /* ggml-cpu/ggml-cpu.c:204-209 */
         default: return -1;
@@ -710,6 +715,20 @@ void orc_dequantize_row(int type, const void *vx, float *y, int64_t k) {
                 }
             }
         }
+    } else if (type == ORC_TYPE_IQ4_XS) {               /* ggml-quants.c dequantize_row_iq4_xs */
+        const blk_iq4_xs *x = (const blk_iq4_xs *)vx;
+        for (int64_t b = 0; b < k / 256; b++) {
+            const float d = H2F(x[b].d);
+            const uint8_t *qs = x[b].qs;
+            for (int ib = 0; ib < 8; ib++, y += 32, qs += 16) {
+                const int ls = ((x[b].scales_l[ib / 2] >> 4 * (ib % 2)) & 0xf) | (((x[b].scales_h >> 2 * ib) & 3) << 4);
+                const float dl = d * (ls - 32);
+                for (int j = 0; j < 16; j++) {
+                    y[j]      = dl * iq4nl_values[qs[j] & 0xf];
+                    y[j + 16] = dl * iq4nl_values[qs[j] >> 4];
+                }
+            }
+        }
     } else if (type == ORC_TYPE_Q8_K) {
         const blk_q8_K *x = (const blk_q8_K *)vx;
         for (int64_t b = 0; b < k / 256; b++)
@@ -1196,6 +1215,37 @@ float orc_vec_dot_q3_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *
     return hsum8(acc);
 }
 
+/* ggml-cpu/ggml-cpu-quants.c lm_ggml_vec_dot_iq4_xs_q8_K, AVX2 branch: a 32-value sub-block is 16 qs bytes, the code points of
+ * the low nibbles (elements 0..15) then those of the high nibbles (16..31) against 32 consecutive q8; lane m of eight holds
+ * (ls - 32) * sum over bytes 4m .. 4m+3 of that vector; the super-block's scale is h2f(d) * y.d. */
+float orc_vec_dot_iq4_xs_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum) {
+    const blk_iq4_xs *x = (const blk_iq4_xs *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    float acc[8] = {0};
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float d = H2F(x[b].d) * y[b].d;
+        int32_t lane[8] = {0};
+        const uint8_t *qs = x[b].qs;
+        const int8_t *q8 = y[b].qs;
+        for (int ib = 0; ib < 8; ib++, qs += 16, q8 += 32) {
+            const int ls = (((x[b].scales_l[ib / 2] >> 4 * (ib % 2)) & 0xf) | (((x[b].scales_h >> 2 * ib) & 3) << 4)) - 32;
+            for (int m = 0; m < 8; m++) {
+                int32_t p = 0;
+                for (int t = 0; t < 4; t++) {
+                    const int e = 4 * m + t;                          /* element of the sub-block */
+                    const int nib = e < 16 ? (qs[e] & 0xf) : (qs[e - 16] >> 4);
+                    p += (int32_t)iq4nl_values[nib] * q8[e];
+                }
+                lane[m] += ls * p;
+            }
+        }
+        int32_t tot = 0;
+        for (int m = 0; m < 8; m++) { tot += lane[m]; acc[m] = fmaf(d, (float)lane[m], acc[m]); }
+        if (isum) isum[b] = tot;
+    }
+    return hsum8(acc);
+}
+
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
     switch (type) {
         case ORC_TYPE_Q4_0: return orc_vec_dot_q4_0_q8_0(k, vx, vy, NULL);
@@ -1210,6 +1260,7 @@ float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy) {
         case ORC_TYPE_F16: return orc_vec_dot_f16(k, vx, vy);
         case ORC_TYPE_Q2_K: return orc_vec_dot_q2_K_q8_K(k, vx, vy, NULL, NULL);
         case ORC_TYPE_Q3_K: return orc_vec_dot_q3_K_q8_K(k, vx, vy, NULL);
+        case ORC_TYPE_IQ4_XS: return orc_vec_dot_iq4_xs_q8_K(k, vx, vy, NULL);
         default: return NAN;
     }
 }
@@ -1347,6 +1398,23 @@ double orc_vec_dot_exact(int type, int64_t k, const void *vx, const void *vy, do
             }
         }
         free(wi);
+    } else if (type == ORC_TYPE_IQ4_XS) {
+        /* terms at sub-block granularity (32 values with their own 6-bit scale) */
+        const blk_iq4_xs *x = (const blk_iq4_xs *)vx;
+        const blk_q8_K *y = (const blk_q8_K *)vy;
+        for (int64_t b = 0; b < nb; b++) {
+            const double d = (double)H2F(x[b].d) * (double)y[b].d;
+            for (int ib = 0; ib < 8; ib++) {
+                const int ls = (((x[b].scales_l[ib / 2] >> 4 * (ib % 2)) & 0xf) | (((x[b].scales_h >> 2 * ib) & 3) << 4)) - 32;
+                int64_t dot = 0;
+                for (int j = 0; j < 16; j++) {
+                    dot += (int64_t)iq4nl_values[x[b].qs[16 * ib + j] & 0xf] * y[b].qs[32 * ib + j];
+                    dot += (int64_t)iq4nl_values[x[b].qs[16 * ib + j] >> 4] * y[b].qs[32 * ib + 16 + j];
+                }
+                const double t = d * (double)ls * (double)dot;
+                s += t; sa += fabs(t);
+            }
+        }
     } else { s = NAN; }
     free(is);
     if (sum_abs) *sum_abs = sa;

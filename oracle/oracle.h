@@ -22,7 +22,7 @@
  *   orc_quantize_row_q4_1_ref/_q5_1_ref  bit-exact vs oracle/_ref + golden; dequant closed form d*u + m
  *   orc_quantize_row_q8_1            bit-exact vs oracle/_ref on seeded data + golden edge rows; quants and d
  *                                    equal orc_quantize_row_q8_0's, s == fp16(d * sum q) on finite rows
- *   (iq4_nl, q2_K and q3_K have no quantizer here: their weights come from oracle/_ref, committed in the golden
+ *   (iq4_nl, iq4_xs, q2_K and q3_K have no quantizer here: their weights come from oracle/_ref, committed in the golden
  *    fixtures, or are random quant bits with plausible scales -- any byte string is a valid block of these types)
  *   orc_dequantize_row_*             closed forms; vs oracle/_ref + golden
  *   orc_vec_dot_*                    integer sums: brute force from dequantised integers; float result: bit-exact
@@ -64,6 +64,7 @@ enum orc_type {
     ORC_TYPE_Q8_1 = 9,      /* activation format of Q4_1 / Q5_1 */
     ORC_TYPE_Q2_K = 10,
     ORC_TYPE_Q3_K = 11,
+    ORC_TYPE_IQ4_XS = 23,
 };
 
 /* elements per block / bytes per block / bytes per row of k elements; 0 for an unknown type */
@@ -119,6 +120,8 @@ float orc_vec_dot_q5_1_q8_1(int64_t k, const void *vx, const void *vy, int32_t *
  * q3_K: isum[k/256] = sum_g (scale_g - 32) * sum_{i<16} (q3 - 4)*q8   (g: the sixteen 16-value sub-blocks) */
 float orc_vec_dot_q2_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum, int32_t *imin);
 float orc_vec_dot_q3_K_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum);
+/* iq4_xs: isum[k/256] = sum_ib (ls_ib - 32) * sum_{i<32} codebook[nib]*q8   (ib: the eight 32-value sub-blocks) */
+float orc_vec_dot_iq4_xs_q8_K(int64_t k, const void *vx, const void *vy, int32_t *isum);
 float orc_vec_dot_f16(int64_t k, const void *vx, const void *vy);   /* both operands fp16, fp32 fmadd lanes */
 float orc_vec_dot(int type, int64_t k, const void *vx, const void *vy);
 

@@ -23,6 +23,9 @@ namespace mirror {
 #define LM_GGML_TYPE_Q4_K M_TYPE_Q4_K
 #define LM_GGML_TYPE_Q6_K M_TYPE_Q6_K
 #define LM_GGML_TYPE_Q8_K M_TYPE_Q8_K
+#define LM_GGML_TYPE_Q2_K M_TYPE_Q2_K
+#define LM_GGML_TYPE_Q3_K M_TYPE_Q3_K
+#define LM_GGML_TYPE_IQ4_XS M_TYPE_IQ4_XS
 #define LM_GGML_TYPE_I32 M_TYPE_I32
 #define LM_GGML_OP_NONE M_OP_NONE
 #define LM_GGML_OP_MUL_MAT M_OP_MUL_MAT
@@ -72,6 +75,9 @@ constexpr int k_max_dims = LM_GGML_MAX_DIMS, k_max_src = LM_GGML_MAX_SRC, k_max_
 #undef LM_GGML_TYPE_Q8_0
 #undef LM_GGML_TYPE_Q4_K
 #undef LM_GGML_TYPE_Q6_K
+#undef LM_GGML_TYPE_Q2_K
+#undef LM_GGML_TYPE_Q3_K
+#undef LM_GGML_TYPE_IQ4_XS
 #undef LM_GGML_TYPE_Q8_K
 #undef LM_GGML_TYPE_I32
 #undef LM_GGML_OP_NONE
@@ -150,7 +156,8 @@ static_assert(mirror::k_max_op_params == LM_GGML_MAX_OP_PARAMS && mirror::k_max_
 static_assert(mirror::k_api == LM_GGML_BACKEND_API_VERSION, "api version");
 static_assert(mirror::M_TYPE_F32 == LM_GGML_TYPE_F32 && mirror::M_TYPE_F16 == LM_GGML_TYPE_F16 && mirror::M_TYPE_Q4_0 == LM_GGML_TYPE_Q4_0 &&
               mirror::M_TYPE_Q8_0 == LM_GGML_TYPE_Q8_0 && mirror::M_TYPE_Q4_K == LM_GGML_TYPE_Q4_K && mirror::M_TYPE_Q6_K == LM_GGML_TYPE_Q6_K &&
-              mirror::M_TYPE_Q8_K == LM_GGML_TYPE_Q8_K && mirror::M_TYPE_I32 == LM_GGML_TYPE_I32, "type ids");
+              mirror::M_TYPE_Q8_K == LM_GGML_TYPE_Q8_K && mirror::M_TYPE_I32 == LM_GGML_TYPE_I32 && mirror::M_TYPE_Q2_K == LM_GGML_TYPE_Q2_K &&
+              mirror::M_TYPE_Q3_K == LM_GGML_TYPE_Q3_K && mirror::M_TYPE_IQ4_XS == LM_GGML_TYPE_IQ4_XS, "type ids");
 static_assert(mirror::M_OP_NONE == LM_GGML_OP_NONE && mirror::M_OP_MUL_MAT == LM_GGML_OP_MUL_MAT && mirror::M_OP_RESHAPE == LM_GGML_OP_RESHAPE &&
               mirror::M_OP_VIEW == LM_GGML_OP_VIEW && mirror::M_OP_PERMUTE == LM_GGML_OP_PERMUTE && mirror::M_OP_TRANSPOSE == LM_GGML_OP_TRANSPOSE &&
               mirror::M_OP_COUNT == LM_GGML_OP_COUNT && mirror::M_OP_MUL_MAT_ID == LM_GGML_OP_MUL_MAT_ID &&

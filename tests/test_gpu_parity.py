@@ -326,7 +326,7 @@ def test_argument_errors(dev):
 
 
 # ------------------------------------------------------------------------------------------ two matrices, one activation
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q3_K, O.Q2_K), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(1024, 333), (4096, 1030)])
 def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
     """chip_mul_mat_pair (ffn_gate and ffn_up in one launch up to 4 tokens; an odd row count puts a two-row tile of Q4_0
@@ -347,7 +347,8 @@ def test_mul_mat_pair_equals_two_mul_mats(dev, orc, wt, K, N):
 # (pass-through rows); a head size that is no power of two; more pairs than one pass of the grid takes
 GROUP_ROPE_CASES = [((O.Q4_K, O.Q4_K, O.Q6_K), 4096, 32, 8, 128, 128, 0), ((O.Q4_K, O.Q4_K, O.Q6_K), 4096, 32, 8, 128, 128, 2),
                     ((O.Q4_0, O.Q8_0, O.Q5_1), 1024, 8, 2, 64, 32, 2), ((O.Q6_K, O.Q5_K, O.Q4_K), 2048, 6, 2, 96, 64, 0),
-                    ((O.Q8_0, O.Q8_0, O.Q8_0), 512, 160, 160, 128, 128, 2), ((O.Q3_K, O.Q2_K, O.Q4_K), 1024, 8, 4, 64, 64, 0)]
+                    ((O.Q8_0, O.Q8_0, O.Q8_0), 512, 160, 160, 128, 128, 2), ((O.Q3_K, O.Q2_K, O.Q4_K), 1024, 8, 4, 64, 64, 0),
+                    ((O.IQ4_XS, O.IQ4_XS, O.Q6_K), 2048, 16, 4, 128, 64, 2)]
 
 
 @pytest.mark.parametrize("types,K,n_head,n_head_kv,hd,n_dims,mode", GROUP_ROPE_CASES)
@@ -383,7 +384,7 @@ def test_group_with_rope_in_the_epilogue_equals_group_then_rope(dev, types, K, n
     assert rc == ca.CHIP_EUNSUPPORTED                                            # multi-section mode
 
 
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(1024, 336), (4096, 1032), (4096, 14336), (256, 8), (2048, 4104)])
 def test_gated_pair_equals_the_pair_and_silu_mul(dev, wt, K, N):
     """chip_mul_mat_pair_silu_mul (ffn_gate, SILU, ffn_up and their MUL in one launch): bit for bit chip_silu_mul of
@@ -436,7 +437,7 @@ def test_group_with_the_norm_in_its_prologue_equals_norm_then_group(dev, types, 
         assert got[2]["y"].tobytes() == want[2]["y"].tobytes(), n
 
 
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(1024, 336), (4096, 14336), (256, 8), (8192, 1032)])
 def test_gated_pair_with_the_norm_in_its_prologue(dev, wt, K, N):
     """chip_mul_mat_pair_silu_mul_norm (ffn_norm, its weight MUL and the gated pair in one launch): bit for bit chip_rms_norm_mul
@@ -467,7 +468,7 @@ def test_gated_pair_with_the_norm_in_its_prologue(dev, wt, K, N):
                                                    65536, None) == ca.CHIP_EUNSUPPORTED
 
 
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K), ids=lambda t: O.TYPE_NAMES[t])
+@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
 @pytest.mark.parametrize("K,N", [(1024, 333), (4096, 4096), (14336, 4096), (256, 7)])
 def test_matmul_with_the_residual_add_in_its_store(dev, wt, K, N):
     """chip_mul_mat_add (wo / ffn_down and the residual ADD behind them in one launch): bit for bit chip_mul_mat followed by

@@ -49,7 +49,7 @@ def test_weight_quantizers_and_dots(orc, ref, wt):
 
 @pytest.mark.parametrize("wt", O.LOW_BIT_K_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_low_bit_k_quants_on_random_bytes(orc, ref, wt):
-    """Q3_K and Q2_K over random block bytes with sane fp16 super-block scales: every code of the packed scales (Q3_K's below
+    """Q3_K, Q2_K and IQ4_XS over random block bytes with sane fp16 super-block scales: every code of the packed scales (Q3_K's below
     32, i.e. negative ones, included), every quant and high-bit pattern; dequantizer and dot bit for bit the reference's."""
     K, N, n = 1024, 16, 2
     rng = np.random.default_rng(77 + wt)
@@ -57,7 +57,7 @@ def test_low_bit_k_quants_on_random_bytes(orc, ref, wt):
     b = rng.integers(0, 256, (N, nb, bb), dtype=np.uint8)
     d = (0.01 * np.exp(rng.uniform(-1, 1, (N, nb)))).astype(np.float16)
     d[rng.random((N, nb)) < 0.2] *= np.float16(-1)
-    off = 108 if wt == O.Q3_K else 80
+    off = {O.Q3_K: 108, O.Q2_K: 80, O.IQ4_XS: 0}[wt]
     b[..., off:off + 2] = d.view(np.uint8).reshape(N, nb, 2)
     if wt == O.Q2_K:
         b[..., 82:84] = (d * np.float16(0.5)).view(np.uint8).reshape(N, nb, 2)
