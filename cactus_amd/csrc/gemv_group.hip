@@ -38,7 +38,9 @@ __device__ __forceinline__ void run_member(const GroupKernelMat &m, const GroupN
     gemv_body<WT, NTOK, RowsPerWave<WT>::R, WGS, FUSEQ, DEPTH>(m.W, m.nb01, K, m.N, x, ldx, ws, ws_stride, m.y, m.ldy, sec, gp);
 }
 
-// FAMILY 0: K-quants (Q8_K activations); 1: 32-value blocks (Q8_0 / Q8_1 planes); 2: F16.
+// FAMILY 0: Q4_K / Q5_K / Q6_K (Q8_K activations); 1: 32-value blocks (Q8_0 / Q8_1 planes); 2: F16; 3: family 0 with Q3_K, Q2_K and
+// IQ4_XS members as well - a kernel of its own, so that the kernel the common type mixes run (Q4_K_M: 0) stays as small as it was
+// (with six member bodies in it the one-token wq + wk + wv launch measured 8.1 instead of 7.6 us).
 // FUSEQ: the workgroups quantize the fp32 rows x themselves; otherwise the workspace already holds the quantized rows
 // (written by chip_mul_mat_prepare or by the kernel that produced the activations) and is only read.
 // ROPE: a kernel of its own for groups in which a member's ROPE node runs in its epilogue (gemv_body.h: ROPED), so that the
@@ -55,6 +57,12 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
     const GridPart gp{(int64_t)((int)blockIdx.x - m.first_block), (int64_t)(last - m.first_block), FUSEQ && blockIdx.x == 0};
     if constexpr (FAMILY == 0) {
         switch (m.wtype) {                                              // uniform over the workgroup
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+        }
+    } else if constexpr (FAMILY == 3) {
+        switch (m.wtype) {
             case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             case T_Q3_K: run_member<T_Q3_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
@@ -248,7 +256,10 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
                                  mats[i].t16_ld, mats[i].wtype, first, mats[i].rope};
         first += blocks[i];
     }
-    switch (fam) {
+    bool low_bit = false;
+    for (int i = 0; i < count; i++) low_bit = low_bit || mats[i].wtype == T_Q3_K || mats[i].wtype == T_Q2_K || mats[i].wtype == T_IQ4_XS;
+    switch (fam == 0 && low_bit ? 3 : fam) {
+        case 3: return launch_ntok<3>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
