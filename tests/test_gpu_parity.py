@@ -384,15 +384,21 @@ def test_group_with_rope_in_the_epilogue_equals_group_then_rope(dev, types, K, n
     assert rc == ca.CHIP_EUNSUPPORTED                                            # multi-section mode
 
 
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N", [(1024, 336), (4096, 1032), (4096, 14336), (256, 8), (2048, 4104)])
+FUSED_FORM_TYPES = (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS)
+
+
+def types_and_shapes(shapes, large, large_types):
+    """(type, K, N) for every type and shape; the large shape only for large_types (once per activation family is enough)."""
+    return [pytest.param(wt, K, N, id="%s-%dx%d" % (O.TYPE_NAMES[wt], N, K)) for (K, N) in shapes for wt in FUSED_FORM_TYPES
+            if (K, N) != large or wt in large_types]
+
+
+@pytest.mark.parametrize("wt,K,N", types_and_shapes([(1024, 336), (4096, 1032), (4096, 14336), (256, 8), (2048, 4104)], (4096, 14336), (O.Q4_K, O.Q4_0)))
 def test_gated_pair_equals_the_pair_and_silu_mul(dev, wt, K, N):
     """chip_mul_mat_pair_silu_mul (ffn_gate, SILU, ffn_up and their MUL in one launch): bit for bit chip_silu_mul of
     chip_mul_mat_pair's two outputs, for a few rows, more rows than a pass of the grid takes, and 1, 2 and 4 tokens; declined
     for other token counts and for row counts that are no multiple of 8 (chip_silu's rule)."""
     import cactus_amd as ca
-    if (K, N) == (4096, 14336) and wt not in (O.Q4_K, O.Q4_0):
-        pytest.skip("the large shape once per activation family")
     w1 = quantized_weights(wt, K + N, N, K)
     w2 = quantized_weights(wt, K + N + 1, N, K)
     for n in (1, 2, 4):
@@ -437,14 +443,11 @@ def test_group_with_the_norm_in_its_prologue_equals_norm_then_group(dev, types, 
         assert got[2]["y"].tobytes() == want[2]["y"].tobytes(), n
 
 
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N", [(1024, 336), (4096, 14336), (256, 8), (8192, 1032)])
+@pytest.mark.parametrize("wt,K,N", types_and_shapes([(1024, 336), (4096, 14336), (256, 8), (8192, 1032)], (4096, 14336), (O.Q4_K, O.Q4_0)))
 def test_gated_pair_with_the_norm_in_its_prologue(dev, wt, K, N):
     """chip_mul_mat_pair_silu_mul_norm (ffn_norm, its weight MUL and the gated pair in one launch): bit for bit chip_rms_norm_mul
     followed by chip_mul_mat_pair_silu_mul; rows the prologue does not hold whole are declined."""
     import cactus_amd as ca
-    if (K, N) == (4096, 14336) and wt not in (O.Q4_K, O.Q4_0):
-        return
     w1 = quantized_weights(wt, K + N, N, K)
     w2 = quantized_weights(wt, K + N + 1, N, K)
     w = norm_weight(N, K)
@@ -468,14 +471,11 @@ def test_gated_pair_with_the_norm_in_its_prologue(dev, wt, K, N):
                                                    65536, None) == ca.CHIP_EUNSUPPORTED
 
 
-@pytest.mark.parametrize("wt", (O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_1, O.F16, O.Q5_K, O.IQ4_NL, O.Q3_K, O.Q2_K, O.IQ4_XS), ids=lambda t: O.TYPE_NAMES[t])
-@pytest.mark.parametrize("K,N", [(1024, 333), (4096, 4096), (14336, 4096), (256, 7)])
+@pytest.mark.parametrize("wt,K,N", types_and_shapes([(1024, 333), (4096, 4096), (14336, 4096), (256, 7)], (14336, 4096), (O.Q4_K, O.Q6_K, O.Q8_0)))
 def test_matmul_with_the_residual_add_in_its_store(dev, wt, K, N):
     """chip_mul_mat_add (wo / ffn_down and the residual ADD behind them in one launch): bit for bit chip_mul_mat followed by
     chip_add, with the result written apart from the addend and over it."""
     import cactus_amd as ca
-    if K == 14336 and wt not in (O.Q4_K, O.Q6_K, O.Q8_0):
-        return
     W = quantized_weights(wt, K + N, N, K)
     for n in (1, 2, 4):
         if not dev.lib.chip_mul_mat_add_supported(wt, K, N, n):
