@@ -49,6 +49,9 @@ def parse():
                     help="issue every launch of the trace directly instead of replaying a HIP graph, and skip everything that "
                          "replays one (for runs under rocprofv3 --kernel-trace; the host then bounds the step time)")
     ap.add_argument("--no-backend", action="store_true", help="skip the ggml-backend graph timing (a child process)")
+    ap.add_argument("--block-order", action="store_true",
+                    help="keep the Q6_K weights as block_q6_K rows for the one-token step too (default: rows in planes, as the "
+                         "backend keeps them for matmuls of up to 4 tokens)")
     ap.add_argument("--only-trace", type=int, default=0, metavar="N", choices=(0, 1, 8, 512),
                     help="run nothing but the trace step at N tokens, every launch issued directly, --warmup + --steps times, and "
                          "print its time (for a per-kernel table of that step under rocprofv3 --kernel-trace --stats)")
@@ -504,6 +507,23 @@ class Trace:
         self.st = C.c_void_p()
         dev.check(L.chip_stream_create(C.byref(self.st)))
         self.bufs = {}
+        self.head_type = ca.Q6_K
+
+    def q6_K_to(self, planes):
+        """Every Q6_K matrix of the arena to planes (what the backend keeps for its decode GEMVs) or back to block order,
+        in place; the launches that follow name the layout by its type."""
+        ca, dev, L = self.ca, self.dev, self.dev.lib
+        want, have = (ca.Q6_K_PLANES, ca.Q6_K) if planes else (ca.Q6_K, ca.Q6_K_PLANES)
+        for l in range(self.NL):
+            for nm, (t, p, N, K) in self.weights(l).items():
+                if t == have:
+                    dev.check(L.chip_repack_q6_K(p, dev.row_size(t, K), p, dev.row_size(t, K), K, N, int(planes), None))
+        if self.head_type == have:
+            p = self.arena.ptr + self.head_off
+            dev.check(L.chip_repack_q6_K(p, dev.row_size(have, self.H), p, dev.row_size(have, self.H), self.H, self.V, int(planes), None))
+        dev.sync()
+        self.layer = [(nm, want if t == have else t, N, K) for (nm, t, N, K) in self.layer]
+        self.head_type = want if self.head_type == have else self.head_type
 
     def weights(self, l):
         base = self.arena.ptr + l * self.layer_bytes
@@ -555,7 +575,7 @@ class Trace:
             ck(L.chip_mul_mat_pair(t, pg, pu, dev.row_size(t, K), K, N, xh, K, n, y, y + nV, N, ws, wsz, st))
 
         def head(_l):
-            ck(L.chip_mul_mat(ca.Q6_K, self.arena.ptr + self.head_off, dev.row_size(ca.Q6_K, H), H, V, xh, H, n, y, V, ws, wsz, st))
+            ck(L.chip_mul_mat(self.head_type, self.arena.ptr + self.head_off, dev.row_size(ca.Q6_K, H), H, V, xh, H, n, y, V, ws, wsz, st))
 
         return {"qkv": qkv, "wo": single("wo", xh), "gate_up": gate_up, "down": single("down", xff), "head": head}
 
@@ -665,11 +685,12 @@ def bench_headline(dev, hip, trace, steps, warmup, eager):
                       "share_of_step": round(count * us / (ms_per_step * 1e3), 3), "launches_timed": launches}
     dom = max(per_op, key=lambda k: per_op[k]["share_of_step"])
     d = per_op[dom]
-    kernel_names = {"qkv": "gemv_group_kernel<K-quants, n=1> (wq Q4_K 4096x4096 + wk Q4_K 1024x4096 + wv Q6_K 1024x4096)",
+    q6 = "Q6_K in planes" if trace.head_type == trace.ca.Q6_K_PLANES else "Q6_K"
+    kernel_names = {"qkv": "gemv_group_kernel<K-quants, n=1> (wq Q4_K 4096x4096 + wk Q4_K 1024x4096 + wv %s 1024x4096)" % q6,
                     "wo": "gemv_kernel<Q4_K, n=1, fused quantize> (4096x4096)",
                     "gate_up": "gemv_kernel<Q4_K, n=1, fused quantize> over ffn_gate + ffn_up (2 x 14336x4096, one launch)",
-                    "down": "gemv_kernel<Q6_K, n=1, fused quantize, image built a step's part at a time> (4096x14336)",
-                    "head": "gemv_kernel<Q6_K, n=1, fused quantize> (128256x4096)"}
+                    "down": "gemv_kernel<%s, n=1, fused quantize, image built a step's part at a time> (4096x14336)" % q6,
+                    "head": "gemv_kernel<%s, n=1, fused quantize> (128256x4096)" % q6}
     roof = {"bound": "hbm", "achieved": d["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": d["hbm_frac"],
             "traffic": traffic_from_profile(dom), "kernel": kernel_names[dom], "op": dom,
             "bytes_per_launch": d["bytes_per_launch"], "us_per_launch": d["us_per_launch"],
@@ -797,7 +818,7 @@ def bench_whole_layers(dev, hip, trace, n, n_kv, fold=True):
             ck(L.chip_add_rms_norm_mul(att.ptr, H, resid.ptr, H, resid.ptr, H, n, H, 1e-5, wn.ptr, cur.ptr, H, st))
         if deferred:                                                  # the final norm has no projection of this kind behind it
             ck(L.chip_rms_norm_mul(resid.ptr, H, n, H, 1e-5, wn.ptr, None, 0, cur.ptr, H, st))
-        ck(L.chip_mul_mat(ca.Q6_K, trace.arena.ptr + trace.head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
+        ck(L.chip_mul_mat(trace.head_type, trace.arena.ptr + trace.head_off, dev.row_size(ca.Q6_K, H), H, V, cur.ptr, H, n, y.ptr, V, ws.ptr, wsz, st))
 
     step()
     dev.sync(st)
@@ -811,10 +832,12 @@ def bench_whole_layers(dev, hip, trace, n, n_kv, fold=True):
             "weight_and_cache_GBps": round((trace.total + cache_bytes) / ms / 1e6, 1)}
 
 
-def bench_trace_more(dev, hip, trace, eager):
-    """The same trace at 8 tokens (per step: 225 matmuls; shared quantized activations) and as one 512-token prefill chunk."""
+def bench_trace_more(dev, hip, trace, eager, planes=True):
+    """The same trace at 8 tokens (per step: 225 matmuls; shared quantized activations) and as one 512-token prefill chunk,
+    both on block-order Q6_K rows (the backend reads its copy in planes up to 4 tokens only)."""
     st = trace.st
     out = {}
+    trace.q6_K_to(False)
     for n in (8, 512):
         run = trace.step(n)
         run()
@@ -836,6 +859,7 @@ def bench_trace_more(dev, hip, trace, eager):
             e["whole_layers"] = bench_whole_layers(dev, hip, trace, n, 512 if n == 512 else 4096)
         out["config5_trace_n%d" % n] = e
     if not eager:
+        trace.q6_K_to(planes)
         out["config5_trace_n1_whole_layers"] = bench_whole_layers(dev, hip, trace, 1, 4096)
     return out
 
@@ -990,17 +1014,27 @@ def main():
     dev = ca.Device(0)
     hip = Hip()
     trace = Trace(dev, hip, np.random.default_rng(5))
+    # Q6_K weights as the backend keeps them for matmuls of up to 4 tokens: rows in planes (made once, outside the timed region)
+    planes = not args.block_order
     if args.only_trace:
+        trace.q6_K_to(planes and args.only_trace <= 4)
         run = trace.step(args.only_trace)
         ms, per = time_steps(dev, hip, trace.st, run, args.steps, args.warmup)
         print(json.dumps({"only_trace": args.only_trace, "launches": "eager", "steps": args.steps, "warmup": args.warmup,
                           "us_per_step": round(ms * 1e3, 1), "step_us": percentiles(per)}))
         trace.free()
         return
-    value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, trace, args.steps, args.warmup, args.eager)
     extra = {}
+    if planes and not args.no_extra:                                   # the same step on block_q6_K rows as the file stores them
+        _, ms_blocks, _, _, info_blocks = bench_headline(dev, hip, trace, min(args.steps, 10), min(args.warmup, 2), args.eager)
+        extra["q6_K_in_block_order"] = {"ms_per_step": round(ms_blocks, 4),
+                                        "us_per_launch": {k: v["us_per_launch"] for k, v in info_blocks["per_op"].items()}}
+    trace.q6_K_to(planes)
+    value, ms_per_step, step_bytes, roof, info = bench_headline(dev, hip, trace, args.steps, args.warmup, args.eager)
+    info["q6_K_layout"] = ("planes: chip_repack_q6_K at set-up, what the backend keeps for matmuls of up to 4 tokens" if planes
+                           else "block_q6_K as stored in the file")
     if not args.no_extra:
-        extra.update(bench_trace_more(dev, hip, trace, args.eager))
+        extra.update(bench_trace_more(dev, hip, trace, args.eager, planes))
     trace.free()
     if not args.no_extra:
         extra["config2_q8_0_ffn_gemv"] = bench_config2(dev, hip)

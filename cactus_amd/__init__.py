@@ -21,12 +21,13 @@ BACKEND_LIB = os.path.join(LIB_DIR, "libggml-hip.so")
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 Q5_0, Q5_K, IQ4_NL = 6, 13, 20
 Q2_K, Q3_K, IQ4_XS = 10, 11, 23
+Q6_K_PLANES = 114           # CHIP_TYPE_Q6_K_PLANES: Q6_K rows repacked by chip_repack_q6_K (no type of the reference)
 Q4_1, Q5_1, Q8_1 = 3, 7, 9
 F16 = 1
 CHIP_OK, CHIP_EINVAL, CHIP_EUNSUPPORTED, CHIP_ENOMEM = 0, -1, -2, -3        # include/cactus_hip.h
 TYPE_NAMES = {F32: "f32", Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", Q8_K: "q8_K",
               Q5_0: "q5_0", Q5_K: "q5_K", IQ4_NL: "iq4_nl", Q4_1: "q4_1", Q5_1: "q5_1", Q8_1: "q8_1", F16: "f16", Q3_K: "q3_K",
-              Q2_K: "q2_K", IQ4_XS: "iq4_xs"}
+              Q2_K: "q2_K", IQ4_XS: "iq4_xs", Q6_K_PLANES: "q6_K_planes"}
 WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, IQ4_NL, Q4_1, Q5_1, Q3_K, Q2_K, IQ4_XS, F16)
 
 # every symbol include/cactus_hip.h declares
@@ -40,7 +41,7 @@ EXPORTS = (
     "chip_mul_mat_workspace_size", "chip_mul_mat_workspace_size_n", "chip_mul_mat", "chip_mul_mat_prepare", "chip_mul_mat_run", "chip_mul_mat_run_ws", "chip_mul_mat_pair", "chip_mul_mat_pair_silu_mul", "chip_mul_mat_pair_silu_mul_supported", "chip_mul_mat_store_t", "chip_mul_mat_group", "chip_mul_mat_group_rope", "chip_mul_mat_group_rope_norm", "chip_mul_mat_pair_silu_mul_norm", "chip_norm_before_supported", "chip_mul_mat_add", "chip_mul_mat_add_supported", "chip_mul_mat_group_run", "chip_mul_mat_noalloc", "chip_mul_mat_noalloc_max_workspace", "chip_mul_mat_id",
     "chip_mul_mat_id_workspace_size", "chip_rms_norm", "chip_add", "chip_mul", "chip_silu", "chip_rms_norm_mul", "chip_silu_mul", "chip_add_rms_norm_mul", "chip_rms_norm_quantized", "chip_silu_mul_quantized", "chip_scale", "chip_gelu_table", "chip_gelu",
     "chip_soft_max", "chip_cpy", "chip_rope", "chip_rope_table", "chip_rope_apply", "chip_rope_apply_store", "chip_rope_apply_two", "chip_get_rows", "chip_mul_mat_f16_batched", "chip_mul_mat_f16_batched_workspace_size", "chip_mul_mat_f16_batched_two_copies", "chip_mul_mat_f16_batched_second_copy_supported",
-    "chip_block_isums", "chip_verify_force_q6k_matrix_core",
+    "chip_repack_q6_K", "chip_block_isums", "chip_verify_force_q6k_matrix_core",
     "chip_workspace_to_blocks",
 )
 
@@ -172,6 +173,7 @@ def load_library(path=KERNEL_LIB):
     L.chip_mul_mat_id_workspace_size.restype = sz
     L.chip_mul_mat_id_workspace_size.argtypes = [i32, i64, i64, i64, i64, i64]
     L.chip_mul_mat_id.argtypes = [i32, vp, sz, sz, i64, i64, i64, vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, sz, vp]
+    L.chip_repack_q6_K.argtypes = [vp, sz, vp, sz, i64, i64, i32, vp]
     L.chip_block_isums.argtypes = [i32, vp, sz, i64, i64, vp, i64, vp, vp, vp]
     L.chip_verify_force_q6k_matrix_core.argtypes = [i32]
     L.chip_workspace_to_blocks.argtypes = [i32, i64, i64, vp, vp, vp]
@@ -673,6 +675,16 @@ class Device:
                                             n_used, n_tokens, dy.ptr, N, ws.ptr, wsz, None))
         self.sync()
         return dy.download(np.float32, n_tokens * n_used * N).reshape(n_tokens, n_used, N)
+
+    def repack_q6_K(self, W, k, to_planes=True, in_place=False):
+        """chip_repack_q6_K on a host matrix W uint8 [N, row_size(Q6_K, K)]: returns the repacked bytes."""
+        W = np.ascontiguousarray(W, np.uint8)
+        N, nb01 = W.shape
+        src = self.to_device(W)
+        dst = src if in_place else self.alloc(W.size)
+        self.check(self.lib.chip_repack_q6_K(src.ptr, nb01, dst.ptr, nb01, k, N, 1 if to_planes else 0, None))
+        self.sync()
+        return dst.download(np.uint8, W.size).reshape(N, nb01)
 
     def block_isums(self, wtype, W, aq, k):
         """Per-block integer sums [n, N, K/block] (and imin for Q4_K / Q5_K) from reference-layout activation blocks."""

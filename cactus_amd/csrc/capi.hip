@@ -96,6 +96,7 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 bool is_block32_type(int t) { return t == T_Q4_0 || t == T_Q8_0 || t == T_Q5_0 || t == T_IQ4_NL || t == T_Q4_1 || t == T_Q5_1; }
 bool weights_aligned(int type, const void *W, size_t nb01, int64_t K = 256) {
     // (Q3_K: 110-byte super-blocks, as Q6_K's 210; Q2_K: 84 bytes; IQ4_XS: 136 bytes, loaded as an 8-byte and 4-byte aligned pieces)
+    // (Q6_K rows in planes: 210 * K / 256 bytes with K % 2048 == 0, a multiple of 16)
     const size_t a = (type == T_Q6_K || type == T_Q3_K) ? 2 : type == T_Q2_K ? 4 : type == T_IQ4_XS ? 8 : (is_block32_type(type) && K % 256 != 0) ? 4 : 16;
     return ((uintptr_t)W % a) == 0 && (nb01 % a) == 0;
 }
@@ -171,7 +172,12 @@ int chip_malloc(void **dptr, size_t bytes) {
     if (!dptr) return CHIP_EINVAL;
     *dptr = nullptr;
     if (bytes == 0) return CHIP_OK;
-    return hip_rc(hipMalloc(dptr, bytes));
+    const hipError_t e = hipMalloc(dptr, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();                     // or the next kernel launch's own check would report this failure again
+        *dptr = nullptr;
+    }
+    return hip_rc(e);
 }
 int chip_free(void *dptr) { return dptr ? hip_rc(hipFree(dptr)) : CHIP_OK; }
 
@@ -233,7 +239,7 @@ int chip_block_elems(int type) {
     switch (type) {
         case T_F32: case T_F16: return 1;
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: case T_Q8_1: return 32;
-        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: return 256;
+        case T_Q4_K: case T_Q6_K: case T_Q8_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: case T_Q6_K_P: return 256;
         default: return 0;
     }
 }
@@ -244,7 +250,7 @@ size_t chip_block_bytes(int type) {
         case T_Q4_0: return BYTES_Q4_0;
         case T_Q8_0: return BYTES_Q8_0;
         case T_Q4_K: return BYTES_Q4_K;
-        case T_Q6_K: return BYTES_Q6_K;
+        case T_Q6_K: case T_Q6_K_P: return BYTES_Q6_K;
         case T_Q8_K: return BYTES_Q8_K;
         case T_Q5_0: return BYTES_Q5_0;
         case T_Q5_K: return BYTES_Q5_K;
@@ -265,14 +271,33 @@ size_t chip_row_size(int type, int64_t k) {
 int chip_vec_dot_type(int type) {
     switch (type) {
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: return T_Q8_0;
-        case T_Q4_K: case T_Q6_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: return T_Q8_K;
+        case T_Q4_K: case T_Q6_K: case T_Q5_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: case T_Q6_K_P: return T_Q8_K;
         case T_Q4_1: case T_Q5_1: return T_Q8_1;
         case T_F16: return T_F16;
         default: return -1;
     }
 }
 int chip_mul_mat_supported(int type, int64_t K) {
+    // Q6_K rows in planes: every field of a row starts at a multiple of 16 bytes when the row has a multiple of 8 super-blocks
+    if (type == T_Q6_K_P) return K > 0 && K % 2048 == 0 && K <= (1 << 20);
     return is_weight_type(type) && K > 0 && K % (is_block32_type(type) ? 64 : 256) == 0 && K <= (1 << 20);
+}
+
+int chip_repack_q6_K(const void *src, size_t nb01_src, void *dst, size_t nb01_dst, int64_t K, int64_t N, int to_planes, void *stream) {
+    if (N < 0) return CHIP_EINVAL;
+    if (!chip_mul_mat_supported(T_Q6_K_P, K)) return CHIP_EUNSUPPORTED;
+    if (N == 0) return CHIP_OK;
+    const size_t row = chip_row_size(T_Q6_K, K);
+    if (!src || !dst || nb01_src < row || nb01_dst < row || (nb01_src % 2) != 0 || (nb01_dst % 2) != 0) return CHIP_EINVAL;
+    if (((uintptr_t)src & 1) != 0 || ((uintptr_t)dst & 1) != 0) return CHIP_EINVAL;
+    // the same rows (in place), or rows that do not overlap at all
+    const uint8_t *s0 = (const uint8_t *)src, *d0 = (const uint8_t *)dst;
+    const size_t s_span = (size_t)(N - 1) * nb01_src + row, d_span = (size_t)(N - 1) * nb01_dst + row;
+    if (!(s0 == d0 && nb01_src == nb01_dst) && s0 < d0 + d_span && d0 < s0 + s_span) return CHIP_EINVAL;
+    DeviceLimits lim;
+    if (int rc = current_limits(lim); rc) return rc;
+    if (row > (size_t)lim.max_lds_per_block) return CHIP_EUNSUPPORTED;
+    return hip_rc(launch_repack_q6_K(src, nb01_src, dst, nb01_dst, K, N, to_planes != 0, lim.max_lds_per_block, (hipStream_t)stream));
 }
 
 static int quantize_public(int act_type, const float *x, int64_t ldx, int64_t n, int64_t k, void *y, void *stream) {
@@ -731,7 +756,7 @@ int chip_mul_mat_id(int type, const void *W, size_t nb01, size_t nb02, int64_t K
                     int64_t ldx, int64_t ne11, const int32_t *ids, int64_t ids_stride, int64_t n_used, int64_t n_tokens,
                     float *y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream) {
     if (N < 0 || n_as < 0 || n_used < 0 || n_tokens < 0 || ne11 < 0) return CHIP_EINVAL;
-    if (!chip_mul_mat_supported(type, K) || K % 256 != 0) return CHIP_EUNSUPPORTED;
+    if (!chip_mul_mat_supported(type, K) || K % 256 != 0 || type == T_Q6_K_P) return CHIP_EUNSUPPORTED;
     if (N == 0 || n_used == 0 || n_tokens == 0) return CHIP_OK;
     if (n_as == 0 || !(ne11 == 1 || ne11 == n_used)) return CHIP_EINVAL;
     if (!W || !x || !ids || !y || !workspace || ldx < K || ldy < N || ids_stride < n_used) return CHIP_EINVAL;
@@ -1116,7 +1141,7 @@ int chip_rope_apply_two(const chip_rope_operand *a, const chip_rope_operand *b, 
 int chip_block_isums(int type, const void *W, size_t nb01, int64_t K, int64_t N, const void *aq, int64_t n,
                      int32_t *isum, int32_t *imin, void *stream) {
     if (N < 0 || n < 0) return CHIP_EINVAL;
-    if (!chip_mul_mat_supported(type, K) || type == T_F16) return CHIP_EUNSUPPORTED;   // F16 has no integer sums
+    if (!chip_mul_mat_supported(type, K) || type == T_F16 || type == T_Q6_K_P) return CHIP_EUNSUPPORTED;   // F16 has no integer sums
     if (N == 0 || n == 0) return CHIP_OK;
     if (!W || !aq || !isum) return CHIP_EINVAL;
     if (!weights_aligned(type, W, nb01, K) || N > 0x7fffffff || n > 65535) return CHIP_EINVAL;

@@ -17,7 +17,9 @@ constexpr int BYTES_Q2_K = 84, BYTES_Q3_K = 110;   // reference ggml-common.h:25
 constexpr int BYTES_IQ4_XS = 136;                  // ggml-common.h:412-417
 
 enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15, T_Q5_0 = 6, T_Q5_K = 13, T_IQ4_NL = 20,
-              T_Q4_1 = 3, T_Q5_1 = 7, T_Q8_1 = 9, T_F16 = 1, T_Q2_K = 10, T_Q3_K = 11, T_IQ4_XS = 23 };
+              T_Q4_1 = 3, T_Q5_1 = 7, T_Q8_1 = 9, T_F16 = 1, T_Q2_K = 10, T_Q3_K = 11, T_IQ4_XS = 23,
+              // not a type of the reference: Q6_K rows whose four fields lie in planes (chip_repack_q6_K), read by the GEMV kernels only
+              T_Q6_K_P = 114 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

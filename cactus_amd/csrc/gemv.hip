@@ -176,6 +176,7 @@ int gemv_max_tokens(int wtype, int64_t K, const DeviceLimits &lim) {
         case T_Q8_0: return max_tokens_typed<T_Q8_0>(K, lim);
         case T_Q4_K: return max_tokens_typed<T_Q4_K>(K, lim);
         case T_Q6_K: return max_tokens_typed<T_Q6_K>(K, lim);
+        case T_Q6_K_P: return max_tokens_typed<T_Q6_K_P>(K, lim);
         case T_Q5_0: return max_tokens_typed<T_Q5_0>(K, lim);
         case T_Q5_K: return max_tokens_typed<T_Q5_K>(K, lim);
         case T_Q3_K: return max_tokens_typed<T_Q3_K>(K, lim);
@@ -198,6 +199,7 @@ hipError_t launch_gemv(int wtype, const void *W, size_t nb01, int64_t K, int64_t
         case T_Q8_0: return launch_ntok<T_Q8_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q4_K: return launch_ntok<T_Q4_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q6_K: return launch_ntok<T_Q6_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
+        case T_Q6_K_P: return launch_ntok<T_Q6_K_P, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q5_0: return launch_ntok<T_Q5_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
         case T_Q3_K: return launch_ntok<T_Q3_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st);
@@ -222,6 +224,7 @@ hipError_t launch_gemv_sec(int wtype, const void *W, size_t nb01, int64_t K, int
         case T_Q8_0: return launch_ntok<T_Q8_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q4_K: return launch_ntok<T_Q4_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q6_K: return launch_ntok<T_Q6_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
+        case T_Q6_K_P: return launch_ntok<T_Q6_K_P, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q5_0: return launch_ntok<T_Q5_0, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q5_K: return launch_ntok<T_Q5_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
         case T_Q3_K: return launch_ntok<T_Q3_K, false>(n, W, nb01, K, N, nullptr, 0, w, ws_stride, y, ldy, lim, st, sec);
@@ -261,6 +264,7 @@ bool gemv_fused_applicable(int wtype, int64_t K, int n, const DeviceLimits &lim)
         case T_Q8_0: img = lds_image_bytes<T_Q8_0>(K); break;
         case T_Q4_K: img = lds_image_bytes<T_Q4_K>(K); break;
         case T_Q6_K: img = lds_image_bytes<T_Q6_K>(K); break;
+        case T_Q6_K_P: img = lds_image_bytes<T_Q6_K_P>(K); break;
         case T_Q5_0: img = lds_image_bytes<T_Q5_0>(K); break;
         case T_Q5_K: img = lds_image_bytes<T_Q5_K>(K); break;
         case T_Q3_K: img = lds_image_bytes<T_Q3_K>(K); break;
@@ -287,6 +291,7 @@ bool gemv_norm_prologue_applicable(int wtype, int64_t K, int n, const DeviceLimi
         case T_Q2_K: iters = iters_per_row<T_Q2_K>(K); break;
         case T_IQ4_XS: iters = iters_per_row<T_IQ4_XS>(K); break;
         case T_Q6_K: iters = iters_per_row<T_Q6_K>(K); break;
+        case T_Q6_K_P: iters = iters_per_row<T_Q6_K_P>(K); break;
         default: break;
     }
     return iters <= 2;
@@ -342,6 +347,7 @@ static hipError_t launch_gemv_fused_sec(int wtype, const void *W, size_t nb01, i
         case T_Q8_0: return launch_ntok<T_Q8_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q4_K: return launch_ntok<T_Q4_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q6_K: return launch_ntok<T_Q6_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
+        case T_Q6_K_P: return launch_ntok<T_Q6_K_P, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q5_0: return launch_ntok<T_Q5_0, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q5_K: return launch_ntok<T_Q5_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);
         case T_Q3_K: return launch_ntok<T_Q3_K, true>(n, W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lim, st, sec);

@@ -40,7 +40,8 @@ __device__ __forceinline__ void run_member(const GroupKernelMat &m, const GroupN
 
 // FAMILY 0: Q4_K / Q5_K / Q6_K (Q8_K activations); 1: 32-value blocks (Q8_0 / Q8_1 planes); 2: F16; 3: family 0 with Q3_K, Q2_K and
 // IQ4_XS members as well - a kernel of its own, so that the kernel the common type mixes run (Q4_K_M: 0) stays as small as it was
-// (with six member bodies in it the one-token wq + wk + wv launch measured 8.1 instead of 7.6 us).
+// (with six member bodies in it the one-token wq + wk + wv launch measured 8.1 instead of 7.6 us); 4: Q4_K / Q5_K with Q6_K rows in
+// planes (T_Q6_K_P), again three bodies; any other mix that contains T_Q6_K_P runs in family 3.
 // FUSEQ: the workgroups quantize the fp32 rows x themselves; otherwise the workspace already holds the quantized rows
 // (written by chip_mul_mat_prepare or by the kernel that produced the activations) and is only read.
 // ROPE: a kernel of its own for groups in which a member's ROPE node runs in its epilogue (gemv_body.h: ROPED), so that the
@@ -61,6 +62,12 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
             case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
+    } else if constexpr (FAMILY == 4) {                                 // Q4_K / Q5_K with Q6_K rows in planes: the decode mix of a Q4_K_M file
+        switch (m.wtype) {
+            case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q5_K: run_member<T_Q5_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            default:     run_member<T_Q6_K_P, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+        }
     } else if constexpr (FAMILY == 3) {
         switch (m.wtype) {
             case T_Q4_K: run_member<T_Q4_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
@@ -68,6 +75,7 @@ __global__ __launch_bounds__(WGS) void gemv_group_kernel(const GroupKernelArgs g
             case T_Q3_K: run_member<T_Q3_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             case T_Q2_K: run_member<T_Q2_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             case T_IQ4_XS: run_member<T_IQ4_XS, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
+            case T_Q6_K_P: run_member<T_Q6_K_P, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
             default:     run_member<T_Q6_K, NTOK, WGS, FUSEQ, DEPTH, ROPE, NORMED>(m, ga.norm, K, x, ldx, ws, ws_stride, gp); break;
         }
     } else if constexpr (FAMILY == 1) {
@@ -89,7 +97,7 @@ size_t image_bytes(int wtype, int64_t K) {
         case T_Q4_0: return lds_image_bytes<T_Q4_0>(K);
         case T_Q8_0: return lds_image_bytes<T_Q8_0>(K);
         case T_Q4_K: return lds_image_bytes<T_Q4_K>(K);
-        case T_Q6_K: return lds_image_bytes<T_Q6_K>(K);
+        case T_Q6_K: case T_Q6_K_P: return lds_image_bytes<T_Q6_K>(K);
         case T_Q5_0: return lds_image_bytes<T_Q5_0>(K);
         case T_Q5_K: return lds_image_bytes<T_Q5_K>(K);
         case T_Q3_K: return lds_image_bytes<T_Q3_K>(K);
@@ -152,7 +160,7 @@ hipError_t launch_ntok(int n, int wgs, const GroupKernelArgs &ga, int grid, int6
 
 int gemv_group_family(int wtype) {
     switch (wtype) {
-        case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: return 0;
+        case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_Q3_K: case T_Q2_K: case T_IQ4_XS: case T_Q6_K_P: return 0;
         case T_Q4_0: case T_Q8_0: case T_Q5_0: case T_IQ4_NL: case T_Q4_1: case T_Q5_1: return 1;
         case T_F16: return 2;
         default: return -1;
@@ -256,10 +264,15 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
                                  mats[i].t16_ld, mats[i].wtype, first, mats[i].rope};
         first += blocks[i];
     }
-    bool low_bit = false;
-    for (int i = 0; i < count; i++) low_bit = low_bit || mats[i].wtype == T_Q3_K || mats[i].wtype == T_Q2_K || mats[i].wtype == T_IQ4_XS;
-    switch (fam == 0 && low_bit ? 3 : fam) {
+    bool low_bit = false, planes = false, raw6 = false;
+    for (int i = 0; i < count; i++) {
+        low_bit = low_bit || mats[i].wtype == T_Q3_K || mats[i].wtype == T_Q2_K || mats[i].wtype == T_IQ4_XS;
+        planes = planes || mats[i].wtype == T_Q6_K_P;
+        raw6 = raw6 || mats[i].wtype == T_Q6_K;
+    }
+    switch (fam != 0 ? fam : (low_bit || (planes && raw6)) ? 3 : planes ? 4 : 0) {
         case 3: return launch_ntok<3>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
+        case 4: return launch_ntok<4>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         case 0: return launch_ntok<0>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         case 1: return launch_ntok<1>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);
         default: return launch_ntok<2>(n, wgs, ga, first, K, x, ldx, ws, ws_stride, lds_bytes, lim, st, prepared, rope);

@@ -17,6 +17,7 @@
 #include <algorithm>
 #include <atomic>
 #include <dlfcn.h>
+#include <map>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -27,11 +28,25 @@
 namespace {
 
 std::atomic<unsigned long long> g_mul_mat_nodes{0}, g_uploaded{0}, g_elementwise_nodes{0}, g_fused_pairs{0}, g_rope_tables{0},
-    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0}, g_rope_epilogues{0}, g_norms_in_prologue{0}, g_residual_adds{0};
+    g_quantizers_skipped{0}, g_uploaded_async{0}, g_grouped_matmuls{0}, g_head_merges{0}, g_rope_pairs{0}, g_gated_pairs{0}, g_rope_epilogues{0}, g_norms_in_prologue{0}, g_residual_adds{0}, g_planes_copies{0}, g_planes_bytes{0}, g_planes_dropped{0}, g_planes_matmuls{0};
 
 #define HIP_LOG(level, ...) lm_ggml_log_internal(level, __VA_ARGS__)
 
-struct buffer_ctx { void *base; size_t size; };
+// A 2-D Q6_K weight's second copy with its rows in planes (chip_repack_q6_K), which the decode GEMVs (up to 4 tokens) read
+// instead: block_q6_K's 210-byte pitch leaves every load of those kernels 2-byte aligned, the planes 16-byte aligned, and the
+// kernels then run 10 to 15 % faster on the same bits.  The tensor's own bytes stay as they are for every other reader (GEMM,
+// MUL_MAT_ID, GET_ROWS, get_tensor); the copy is made at the weight's first decode matmul, kept with the buffer and dropped
+// when anything writes over the weight.
+struct planes_copy { void *data; size_t src_span; size_t nb01; int64_t K, N; };
+struct buffer_ctx {
+    void *base; size_t size;
+    std::mutex mu;
+    std::map<const uint8_t *, planes_copy> planes;     // by the weight's address
+    std::atomic<int> n_planes{0};
+    size_t max_span = 0;                               // the largest src_span ever entered
+    bool planes_failed = false;                        // an allocation failed: no further copies for this buffer
+    buffer_ctx(void *b, size_t s) : base(b), size(s) {}
+};
 // The cos / sin table of the ROPE nodes of one graph_compute call: Q and K of every layer are rotated by the same
 // positions, so the first ROPE node of a call builds the table and the others apply it.  The key is only valid inside
 // the call (the position tensor keeps its address from call to call while its contents change).
@@ -76,17 +91,43 @@ bool is_host_buffer(const lm_ggml_backend_buffer *b) {
 bool is_hip_buffer(const lm_ggml_backend_buffer *b) { return b && b->buft == hip_buffer_type(); }
 
 // ------------------------------------------------------------------------------------------------ buffer
+// Drops the planes copies of the weights that [lo, lo + bytes) touches: called by everything that writes into a buffer.
+// (chip_free waits for the device, so a GEMV still reading a copy finishes first)
+void drop_planes(buffer_ctx *bc, const void *lo, size_t bytes) {
+    if (!bc || bc->n_planes.load(std::memory_order_acquire) == 0 || bytes == 0) return;
+    std::lock_guard<std::mutex> lk(bc->mu);
+    const uint8_t *a = (const uint8_t *)lo, *b = a + bytes;
+    // the weights that start below b, from the highest down to the last one a span of the largest size could still reach
+    auto it = bc->planes.lower_bound(b);
+    while (it != bc->planes.begin()) {
+        --it;
+        if (it->first + bc->max_span <= a) break;
+        if (a < it->first + it->second.src_span) {
+            chip_free(it->second.data);
+            it = bc->planes.erase(it);
+            bc->n_planes--;
+            g_planes_dropped++;
+        }
+    }
+}
+buffer_ctx *hip_buffer_ctx_of(const lm_ggml_tensor *t) {
+    const lm_ggml_backend_buffer *b = t->view_src ? t->view_src->buffer : t->buffer;
+    return is_hip_buffer(b) ? (buffer_ctx *)b->context : nullptr;
+}
 void buf_free(lm_ggml_backend_buffer_t buffer) {
     buffer_ctx *c = (buffer_ctx *)buffer->context;
+    drop_planes(c, c->base, c->size);
     chip_free(c->base);
     delete c;
 }
 void *buf_get_base(lm_ggml_backend_buffer_t buffer) { return ((buffer_ctx *)buffer->context)->base; }
-void buf_memset_tensor(lm_ggml_backend_buffer_t, lm_ggml_tensor *t, uint8_t value, size_t offset, size_t size) {
+void buf_memset_tensor(lm_ggml_backend_buffer_t buffer, lm_ggml_tensor *t, uint8_t value, size_t offset, size_t size) {
+    drop_planes((buffer_ctx *)buffer->context, (char *)t->data + offset, size);
     chip_memset((char *)t->data + offset, value, size, nullptr);
     chip_stream_synchronize(nullptr);
 }
-void buf_set_tensor(lm_ggml_backend_buffer_t, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
+void buf_set_tensor(lm_ggml_backend_buffer_t buffer, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
+    drop_planes((buffer_ctx *)buffer->context, (char *)t->data + offset, size);
     chip_memcpy_h2d((char *)t->data + offset, data, size, nullptr);          // synchronous
     g_uploaded += size;
 }
@@ -94,8 +135,9 @@ void buf_get_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *t, void *dat
     chip_stream_synchronize(nullptr);
     chip_memcpy_d2h(data, (const char *)t->data + offset, size, nullptr);    // synchronous
 }
-bool buf_cpy_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *src, lm_ggml_tensor *dst) {
+bool buf_cpy_tensor(lm_ggml_backend_buffer_t buffer, const lm_ggml_tensor *src, lm_ggml_tensor *dst) {
     const size_t n = lm_ggml_nbytes(src);
+    drop_planes((buffer_ctx *)buffer->context, dst->data, n);
     if (is_host_buffer(src->buffer)) {
         chip_memcpy_h2d(dst->data, src->data, n, nullptr);
         return true;
@@ -109,6 +151,7 @@ bool buf_cpy_tensor(lm_ggml_backend_buffer_t, const lm_ggml_tensor *src, lm_ggml
 }
 void buf_clear(lm_ggml_backend_buffer_t buffer, uint8_t value) {
     buffer_ctx *c = (buffer_ctx *)buffer->context;
+    drop_planes(c, c->base, c->size);
     chip_memset(c->base, value, c->size, nullptr);
     chip_stream_synchronize(nullptr);
 }
@@ -133,7 +176,7 @@ lm_ggml_backend_buffer_t buft_alloc(lm_ggml_backend_buffer_type_t buft, size_t s
         HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: hipMalloc of %zu bytes failed\n", __func__, size);
         return nullptr;
     }
-    buffer_ctx *c = new (std::nothrow) buffer_ctx{p, size};
+    buffer_ctx *c = new (std::nothrow) buffer_ctx(p, size);
     if (!c) { chip_free(p); return nullptr; }
     return lm_ggml_backend_buffer_init(buft, k_buffer_i, c, size);
 }
@@ -186,7 +229,7 @@ lm_ggml_backend_buffer_t hbuft_alloc(lm_ggml_backend_buffer_type_t buft, size_t 
         HIP_LOG(LM_GGML_LOG_LEVEL_WARN, "%s: pinned allocation of %zu bytes failed\n", __func__, size);
         return nullptr;
     }
-    buffer_ctx *c = new (std::nothrow) buffer_ctx{p, size};
+    buffer_ctx *c = new (std::nothrow) buffer_ctx(p, size);
     if (!c) { chip_host_free(p); return nullptr; }
     return lm_ggml_backend_buffer_init(buft, k_host_buffer_i, c, size);
 }
@@ -214,6 +257,7 @@ void backend_synchronize(lm_ggml_backend_t backend) { chip_stream_synchronize(((
 // Asynchronous on the backend's stream, ordered with graph_compute; the host memory must stay untouched until the
 // stream (or an event recorded after the call) has been waited for.
 void backend_set_tensor_async(lm_ggml_backend_t backend, lm_ggml_tensor *t, const void *data, size_t offset, size_t size) {
+    drop_planes(hip_buffer_ctx_of(t), (char *)t->data + offset, size);
     chip_memcpy_h2d((char *)t->data + offset, data, size, ((backend_ctx *)backend->context)->stream);
     g_uploaded += size;
     g_uploaded_async += size;
@@ -334,6 +378,60 @@ bool elementwise_enabled() {
 bool fusion_enabled() {
     static const bool on = [] { const char *e = std::getenv("CACTUS_HIP_FUSE"); return !(e && std::strcmp(e, "0") == 0); }();
     return on;
+}
+bool planes_enabled() {
+    static const bool on = [] { const char *e = std::getenv("CACTUS_HIP_Q6K_PLANES"); return !(e && std::strcmp(e, "0") == 0); }();
+    return on;
+}
+// The weight operand of a matmul of n tokens as the kernels take it: the tensor's own bytes, or for a Q6_K weight at up to
+// 4 tokens its copy in planes (made here, on the backend's stream, at the first such matmul).
+struct weight_arg { int type; const void *data; size_t nb01; };
+weight_arg weight_for(backend_ctx *c, const lm_ggml_tensor *w, int64_t n) {
+    const weight_arg own{(int)w->type, w->data, w->nb[1]};
+    if (w->type != LM_GGML_TYPE_Q6_K || n < 1 || n > 4 || w->ne[2] != 1 || w->ne[3] != 1 || w->ne[1] <= 0 || !planes_enabled()) return own;
+    const int64_t K = w->ne[0], N = w->ne[1];
+    const size_t row = chip_row_size(CHIP_TYPE_Q6_K, K);
+    if (!chip_mul_mat_supported(CHIP_TYPE_Q6_K_PLANES, K) || row > 160 * 1024 || w->nb[1] < row || w->nb[1] % 2 != 0) return own;
+    buffer_ctx *bc = hip_buffer_ctx_of(w);
+    if (!bc || bc->planes_failed) return own;
+    std::lock_guard<std::mutex> lk(bc->mu);
+    const uint8_t *key = (const uint8_t *)w->data;
+    auto it = bc->planes.find(key);
+    if (it != bc->planes.end()) {
+        const planes_copy &pc = it->second;
+        if (pc.K == K && pc.N == N && pc.nb01 == w->nb[1]) {
+            g_planes_matmuls++;
+            return weight_arg{CHIP_TYPE_Q6_K_PLANES, pc.data, row};
+        }
+        chip_free(pc.data);                            // the same address read as another shape
+        bc->planes.erase(it);
+        bc->n_planes--;
+        g_planes_dropped++;
+    }
+    const size_t bytes = (size_t)N * row;
+    chip_device_info info;
+    if (chip_get_device_info(&info) != CHIP_OK || info.hbm_free < bytes + ((size_t)1 << 30)) {   // leave the caller a GiB
+        bc->planes_failed = true;
+        return own;
+    }
+    void *p = nullptr;
+    if (chip_malloc(&p, bytes) != CHIP_OK || !p) {
+        bc->planes_failed = true;
+        return own;
+    }
+    if (chip_repack_q6_K(w->data, w->nb[1], p, row, K, N, 1, c->stream) != CHIP_OK) {
+        chip_free(p);
+        bc->planes_failed = true;
+        return own;
+    }
+    const size_t span = (size_t)(N - 1) * w->nb[1] + row;
+    bc->planes.emplace(key, planes_copy{p, span, w->nb[1], K, N});
+    bc->max_span = std::max(bc->max_span, span);
+    bc->n_planes++;
+    g_planes_copies++;
+    g_planes_bytes += bytes;
+    g_planes_matmuls++;
+    return weight_arg{CHIP_TYPE_Q6_K_PLANES, p, row};
 }
 bool elementwise_shape_ok(const lm_ggml_tensor *op) {
     if (!elementwise_enabled()) return false;
@@ -1073,6 +1171,7 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
         // a node that writes into the tensor the workspace was quantized from, or that uses the workspace itself, ends
         // the reuse of the quantized rows (every node is seen here, also those run inside a neighbour's kernel)
         auto writes = [c](const lm_ggml_tensor *t) {
+            drop_planes(hip_buffer_ctx_of(t), t->data, lm_ggml_nbytes(t));
             if (!c->quantized.valid) return;
             const uintptr_t a = (uintptr_t)t->data, b = (uintptr_t)c->quantized.src;
             const bool apart = a + lm_ggml_nbytes(t) <= b || b + c->quantized.src_bytes <= a;
@@ -1342,15 +1441,17 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                     reads.readers_of(cgraph, node) == 1 && reads.readers_of(cgraph, silu) == 1 && reads.readers_of(cgraph, up) == 1) {
                     c->quantized.valid = false;
                     rc = CHIP_EUNSUPPORTED;
+                    weight_arg wg = weight_for(c, w, n), wu = weight_for(c, up->src[0], n);
+                    if (wg.type != wu.type) wg = weight_arg{(int)w->type, w->data, w->nb[1]}, wu = weight_arg{(int)w->type, up->src[0]->data, w->nb[1]};
                     if (held.held() && ranges_apart(mul, held.src)) {     // ffn_norm and its weight MUL in the same launch
                         const chip_norm_before nb{(const float *)held.weight->data, held.eps, (float *)x->data, ldx};
-                        rc = chip_mul_mat_pair_silu_mul_norm(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)held.src->data,
+                        rc = chip_mul_mat_pair_silu_mul_norm(wg.type, wg.data, wu.data, wg.nb01, K, N, (const float *)held.src->data,
                                                              (int64_t)(held.src->nb[1] / 4), n, &nb, (float *)mul->data, ldm, c->workspace,
                                                              c->workspace_size, c->stream);
                         if (rc == CHIP_OK) { held.out = nullptr; g_norms_in_prologue++; }
                     }
                     if (rc == CHIP_EUNSUPPORTED && (rc = run_held_norm()) == CHIP_OK)
-                        rc = chip_mul_mat_pair_silu_mul(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)x->data, ldx, n,
+                        rc = chip_mul_mat_pair_silu_mul(wg.type, wg.data, wu.data, wg.nb01, K, N, (const float *)x->data, ldx, n,
                                                         (float *)mul->data, ldm, c->workspace, c->workspace_size, c->stream);
                     if (rc != CHIP_OK) {
                         HIP_LOG(LM_GGML_LOG_LEVEL_ERROR, "%s: gated MUL_MAT pair at %s failed: %s\n", __func__, node->name, chip_error_string(rc));
@@ -1389,7 +1490,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             for (int k = 0; fits && k < n_members; k++) {
                 lm_ggml_tensor *mm = cgraph->nodes[members[k]];
                 const lm_ggml_tensor *mw = mm->src[0];
-                mats[k] = chip_mat{(int)mw->type, mw->data, mw->nb[1], mw->ne[1], (float *)mm->data, (int64_t)(mm->nb[1] / 4), nullptr, 0};
+                const weight_arg wa = weight_for(c, mw, n);
+                mats[k] = chip_mat{wa.type, wa.data, wa.nb01, mw->ne[1], (float *)mm->data, (int64_t)(mm->nb[1] / 4), nullptr, 0};
                 if (aliased[k]) {                      // its own memory is still in use: into the backend's slot k, rows side by side
                     mats[k].y = (float *)((uint8_t *)c->group_scratch + (size_t)k * c->group_slot_bytes);
                     mats[k].ldy = mw->ne[1];
@@ -1536,7 +1638,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             lm_ggml_tensor *cp = cgraph->nodes[store_t];
             writes(cp);
             c->quantized.valid = false;
-            rc = chip_mul_mat_store_t(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
+            const weight_arg wa = weight_for(c, w, n);
+            rc = chip_mul_mat_store_t(wa.type, wa.data, wa.nb01, K, N, (const float *)x->data, ldx, n, (float *)node->data,
                                       (int64_t)(node->nb[1] / 4), (uint16_t *)cp->data, (int64_t)(cp->nb[1] / 2), c->workspace,
                                       c->workspace_size, c->stream);
             g_elementwise_nodes++;
@@ -1545,7 +1648,9 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             lm_ggml_tensor *up = cgraph->nodes[paired_matmul];
             writes(up);
             c->quantized.valid = false;
-            rc = chip_mul_mat_pair(w->type, w->data, up->src[0]->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
+            weight_arg wg = weight_for(c, w, n), wu = weight_for(c, up->src[0], n);
+            if (wg.type != wu.type) wg = weight_arg{(int)w->type, w->data, w->nb[1]}, wu = weight_arg{(int)w->type, up->src[0]->data, w->nb[1]};
+            rc = chip_mul_mat_pair(wg.type, wg.data, wu.data, wg.nb01, K, N, (const float *)x->data, ldx, n, (float *)node->data,
                                    (float *)up->data, (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
             g_mul_mat_nodes++;
             g_fused_pairs++;
@@ -1563,15 +1668,19 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
                 g_quantizers_skipped++;
             }
             if (rc == CHIP_OK)
-                rc = chip_mul_mat_run_ws(w->type, w->data, w->nb[1], K, N, n, c->workspace, c->workspace_size, (float *)node->data,
+                {
+                const weight_arg wa = weight_for(c, w, n);
+                rc = chip_mul_mat_run_ws(wa.type, wa.data, wa.nb01, K, N, n, c->workspace, c->workspace_size, (float *)node->data,
                                          (int64_t)(node->nb[1] / 4), c->stream);
+            }
         } else if (n <= 4 && fusion_enabled() && add_done < 0 && (add_index = residual_add_index(cgraph, i, reads)) >= 0) {
             // wo / ffn_down and the residual ADD behind them: the GEMV adds the other operand as it stores, into the ADD's rows
             lm_ggml_tensor *add = cgraph->nodes[add_index];
             const lm_ggml_tensor *other = add->src[0] == node ? add->src[1] : add->src[0];
             c->quantized.valid = false;
             writes(add);
-            rc = chip_mul_mat_add(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (const float *)other->data,
+            const weight_arg wa = weight_for(c, w, n);
+            rc = chip_mul_mat_add(wa.type, wa.data, wa.nb01, K, N, (const float *)x->data, ldx, n, (const float *)other->data,
                                   (int64_t)(other->nb[1] / 4), (float *)add->data, (int64_t)(add->nb[1] / 4), c->workspace, c->workspace_size,
                                   c->stream);
             add_done = add_index;
@@ -1580,7 +1689,8 @@ int backend_graph_compute(lm_ggml_backend_t backend, lm_ggml_cgraph *cgraph) {
             g_residual_adds++;
         } else {
             c->quantized.valid = false;               // up to 4 tokens the GEMV quantizes in its own prologue, into the workspace
-            rc = chip_mul_mat(w->type, w->data, w->nb[1], K, N, (const float *)x->data, ldx, n, (float *)node->data,
+            const weight_arg wa = weight_for(c, w, n);
+            rc = chip_mul_mat(wa.type, wa.data, wa.nb01, K, N, (const float *)x->data, ldx, n, (float *)node->data,
                               (int64_t)(node->nb[1] / 4), c->workspace, c->workspace_size, c->stream);
         }
         if (rc != CHIP_OK) {
@@ -1776,5 +1886,9 @@ unsigned long long lm_ggml_backend_hip_get_gated_pairs(void) { return g_gated_pa
 unsigned long long lm_ggml_backend_hip_get_rope_epilogues(void) { return g_rope_epilogues.load(); }
 unsigned long long lm_ggml_backend_hip_get_norms_in_prologue(void) { return g_norms_in_prologue.load(); }
 unsigned long long lm_ggml_backend_hip_get_residual_adds(void) { return g_residual_adds.load(); }
+unsigned long long lm_ggml_backend_hip_get_planes_copies(void) { return g_planes_copies.load(); }
+unsigned long long lm_ggml_backend_hip_get_planes_bytes(void) { return g_planes_bytes.load(); }
+unsigned long long lm_ggml_backend_hip_get_planes_dropped(void) { return g_planes_dropped.load(); }
+unsigned long long lm_ggml_backend_hip_get_planes_matmuls(void) { return g_planes_matmuls.load(); }
 
 }  // extern "C"

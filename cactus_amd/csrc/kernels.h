@@ -278,6 +278,9 @@ hipError_t launch_add_rms_norm_mul(const float *a, int64_t lda, const float *b, 
                                    int64_t ne0, float eps, const float *w, float *yn, int64_t ldyn, float *y, int64_t ldy,
                                    hipStream_t st);
 hipError_t launch_scale(const float *x, int64_t ldx, int64_t ne0, int64_t n, float s, float *y, int64_t ldy, hipStream_t st);
+// Q6_K rows between block order and planes (T_Q6_K_P), in place (dst == src) or into another matrix; rows of at most max_lds bytes
+hipError_t launch_repack_q6_K(const void *src, size_t nb01_src, void *dst, size_t nb01_dst, int64_t K, int64_t N, bool to_planes,
+                              int max_lds, hipStream_t st);
 hipError_t launch_gelu(const float *x, int64_t ldx, int64_t ne0, int64_t n, const unsigned short *table, float *y, int64_t ldy,
                        hipStream_t st);
 bool norm_quantized_applicable(const float *a, int64_t lda, const float *b, int64_t ldb, const float *xs, int64_t ldxs, int64_t ne0,

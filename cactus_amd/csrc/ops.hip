@@ -920,6 +920,38 @@ static hipError_t launch_unary(const float *x, int64_t ldx, int64_t ne0, int64_t
     }
     return hipGetLastError();
 }
+// ---- Q6_K rows between block_q6_K order and planes (ql | qh | scales | d per row): one workgroup per row takes the row
+// into LDS and writes it in the other order, to the same place or to another matrix; rows of up to 160 KB ----
+template <bool TO_PLANES>
+__global__ __launch_bounds__(256) void repack_q6_K_kernel(const uint8_t *src, size_t nb01_src, uint8_t *dst, size_t nb01_dst, int nsb) {
+    extern __shared__ __align__(16) uint8_t rowbuf[];
+    const uint16_t *in = reinterpret_cast<const uint16_t *>(src + (size_t)blockIdx.x * nb01_src);
+    uint16_t *row = reinterpret_cast<uint16_t *>(dst + (size_t)blockIdx.x * nb01_dst);
+    uint16_t *buf = reinterpret_cast<uint16_t *>(rowbuf);
+    const int halves = nsb * (BYTES_Q6_K / 2);                        // the row in 2-byte pieces (its fields are multiples of 2 bytes)
+    for (int i = threadIdx.x; i < halves; i += 256) buf[i] = in[i];
+    __syncthreads();
+    // piece p of super-block sb in block order: ql 0..63 | qh 64..95 | scales 96..103 | d 104; in planes: its field's plane
+    for (int i = threadIdx.x; i < halves; i += 256) {
+        const int sb = i / 105, p = i - sb * 105;
+        const int q = p < 64 ? sb * 64 + p : p < 96 ? nsb * 64 + sb * 32 + (p - 64) : p < 104 ? nsb * 96 + sb * 8 + (p - 96) : nsb * 104 + sb;
+        if (TO_PLANES) row[q] = buf[i];
+        else row[i] = buf[q];
+    }
+}
+hipError_t launch_repack_q6_K(const void *src, size_t nb01_src, void *dst, size_t nb01_dst, int64_t K, int64_t N, bool to_planes,
+                              int max_lds, hipStream_t st) {
+    const int64_t nsb = K / 256;
+    const size_t bytes = (size_t)nsb * BYTES_Q6_K;
+    if (N <= 0 || nsb <= 0) return hipSuccess;
+    if (bytes > (size_t)max_lds || N > 0x7fffffff) return hipErrorInvalidValue;
+    auto kfn = to_planes ? repack_q6_K_kernel<true> : repack_q6_K_kernel<false>;
+    if (bytes > 48 * 1024)
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kfn, dim3((unsigned)N), dim3(256), bytes, st, (const uint8_t *)src, nb01_src, (uint8_t *)dst, nb01_dst, (int)nsb);
+    return hipGetLastError();
+}
+
 hipError_t launch_scale(const float *x, int64_t ldx, int64_t ne0, int64_t n, float s, float *y, int64_t ldy, hipStream_t st) {
     return launch_unary<UN_SCALE>(x, ldx, ne0, n, y, ldy, s, nullptr, st);
 }

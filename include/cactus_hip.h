@@ -44,6 +44,10 @@ enum chip_type {
     CHIP_TYPE_Q2_K   = 10,
     CHIP_TYPE_Q3_K   = 11,
     CHIP_TYPE_IQ4_XS = 23,
+    /* Not a type of the reference: a Q6_K matrix whose rows chip_repack_q6_K has laid out in planes.  Accepted as the weight
+     * type of the matmul entry points only (not by chip_get_rows, chip_mul_mat_id, chip_block_isums); every token count runs
+     * on the dot-product GEMV, in passes of up to 8 tokens, so this layout is meant for decode (1..4 tokens). */
+    CHIP_TYPE_Q6_K_PLANES = 114,
 };
 
 enum chip_status {
@@ -452,6 +456,19 @@ typedef struct chip_rope_operand {
 CHIP_API int chip_rope_apply_two(const chip_rope_operand *a, const chip_rope_operand *b, const float *table, int64_t ne0,
                                  int64_t ne2, int n_dims, int mode, void *stream);
 
+
+/* ---- Q6_K rows in planes ----
+ * No counterpart in the reference, whose CPU kernels read block_q6_K (ggml-common.h:332-338) as stored in the file.
+ * A row of K / 256 super-blocks of 210 bytes is laid out as four planes instead - all ql fields (128 bytes each), then all
+ * qh (64), then all scales (16), then all d (2) - in the same 210 * K / 256 bytes.  With K % 2048 == 0 every load of the
+ * decode GEMV then starts at a multiple of its own size, where block_q6_K's 210-byte pitch leaves them 2-byte aligned;
+ * results are the same bits as on the block layout.
+ *   to_planes != 0: block order -> planes; 0: planes -> block order (the inverse, byte for byte)
+ *   dst == src with nb01_dst == nb01_src repacks in place; otherwise the two matrices must not overlap
+ *   K % 2048 == 0, rows of at most the device's LDS per workgroup (160 KB: K <= 196608); src, dst, strides 2-byte aligned
+ *   (chip_mul_mat and the other matmul entry points ask 16-byte alignment of a CHIP_TYPE_Q6_K_PLANES matrix and stride) */
+CHIP_API int chip_repack_q6_K(const void *src, size_t nb01_src, void *dst, size_t nb01_dst, int64_t K, int64_t N,
+                              int to_planes, void *stream);
 
 /* ---- verification hooks ----
  * Per-block integer sums of lm_ggml_vec_dot_{q4_0_q8_0,q8_0_q8_0,q4_K_q8_K,q6_K_q8_K,q5_0_q8_0,q5_K_q8_K,

@@ -69,6 +69,15 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_epilogues(void);
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_norms_in_prologue(void);
 /* Residual ADD nodes that ran where the projection in front of them (wo, ffn_down) stores its result, up to 4 tokens. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_residual_adds(void);
+/* Q6_K weights in planes.  The decode GEMVs (up to 4 tokens) read a 2-D Q6_K weight of K % 2048 == 0 from a second copy whose
+ * rows chip_repack_q6_K laid out in planes; the backend makes the copy at the weight's first such matmul (210 * K / 256 bytes
+ * per row of device memory more, skipped when less than that plus 1 GiB is free) and drops it when set_tensor, memset_tensor,
+ * cpy_tensor, clear or a graph node writes over the weight.  CACTUS_HIP_Q6K_PLANES=0 in the environment turns this off.
+ * Counters: copies made, their bytes, copies dropped, matmul operands read from a copy. */
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_planes_copies(void);
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_planes_bytes(void);
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_planes_dropped(void);
+CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_planes_matmuls(void);
 
 #ifdef __cplusplus
 }

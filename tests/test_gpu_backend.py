@@ -1137,3 +1137,79 @@ def test_get_rows_from_a_device_resident_table(host, orc):
     L.lm_ggml_backend_free(cpu)
     L.lm_ggml_free(ctx)
     L.lm_ggml_free(wctx)
+
+
+def test_q6_K_weights_are_read_from_a_copy_in_planes_at_decode(host, orc):
+    """A 2-D Q6_K weight of K % 2048 == 0: its first matmul of up to 4 tokens makes the copy in planes and reads it (the same
+    bits as the C-ABI gives on the block-order rows), the next one reads the same copy, get_tensor still returns the bytes that
+    were set, set_tensor and memset_tensor drop the copy (the matmul after them sees the new weights), and a matmul of 8 tokens
+    reads the tensor's own bytes."""
+    import cactus_amd
+    L = host.L
+    K, N = 2048, 520
+    w1 = orc.quantize_weights(O.Q6_K, common.weights_f32(81, N, K))
+    w2 = orc.quantize_weights(O.Q6_K, common.weights_f32(82, N, K))
+    cdev = cactus_amd.Device(0)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    wctx = host.context(with_graph=False)
+    tw = host.tensor_2d(wctx, O.Q6_K, K, N, "w")
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    L.lm_ggml_backend_buffer_set_usage(wbuf, 1)
+    host.set(tw, w1)
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    counters = {}
+    for name in ("copies", "bytes", "dropped", "matmuls"):
+        f = getattr(blib, "lm_ggml_backend_hip_get_planes_" + name)
+        f.restype = C.c_ulonglong
+        counters[name] = f
+    def counts():
+        return {k: f() for k, f in counters.items()}
+    graphs = {}
+    for n in (2, 8):
+        ctx = host.context()
+        tx = host.tensor_2d(ctx, O.F32, K, n, "x")
+        ty = L.lm_ggml_mul_mat(ctx, tw, tx)
+        g = L.lm_ggml_new_graph(ctx)
+        L.lm_ggml_build_forward_expand(g, ty)
+        buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+        graphs[n] = (ctx, tx, ty, g, buf)
+    x2, x8 = common.activations_f32(83, 2, K), common.activations_f32(84, 8, K)
+
+    def run(n, x):
+        ctx, tx, ty, g, buf = graphs[n]
+        host.set(tx, x)
+        assert L.lm_ggml_backend_graph_compute(hip, g) == 0
+        return host.get(ty, np.float32, (n, N))
+
+    c0 = counts()
+    y = run(2, x2)
+    c1 = counts()
+    assert c1["copies"] - c0["copies"] == 1 and c1["bytes"] - c0["bytes"] == w1.size and c1["matmuls"] - c0["matmuls"] == 1
+    assert y.tobytes() == cdev.mul_mat(O.Q6_K, w1, x2).tobytes()
+    ref = orc.mul_mat(O.Q6_K, w1, x2, nthreads=8, want=("sum_abs",))
+    assert (np.abs(y.astype(np.float64) - ref["y"]) <= REL_TOL * ref["sum_abs"]).all()
+    assert run(2, x2).tobytes() == y.tobytes()
+    c2 = counts()
+    assert c2["copies"] == c1["copies"] and c2["matmuls"] - c1["matmuls"] == 1 and c2["dropped"] == c0["dropped"]
+    assert np.array_equal(host.get(tw, np.uint8, w1.shape), w1)                    # the tensor's own bytes stay in block order
+    y8 = run(8, x8)
+    assert counts() == c2                                                          # 8 tokens: no copy read, none made
+    assert y8.tobytes() == cdev.mul_mat(O.Q6_K, w1, x8).tobytes()
+    host.set(tw, w2)                                                               # new weights: the copy is stale
+    c3 = counts()
+    assert c3["dropped"] - c2["dropped"] == 1
+    y = run(2, x2)
+    assert y.tobytes() == cdev.mul_mat(O.Q6_K, w2, x2).tobytes()
+    assert counts()["copies"] - c3["copies"] == 1
+    L.lm_ggml_backend_tensor_memset(tw, 0, 0, w2.size)                             # d = 0 in every block
+    assert counts()["dropped"] - c3["dropped"] == 1
+    assert not run(2, x2).any()
+    before_free = counts()["dropped"]
+    L.lm_ggml_backend_buffer_free(wbuf)                                            # the copy goes with the buffer
+    assert counts()["dropped"] - before_free == 1
+    for ctx, tx, ty, g, buf in graphs.values():
+        L.lm_ggml_backend_buffer_free(buf)
+        L.lm_ggml_free(ctx)
+    L.lm_ggml_backend_free(hip)
+    L.lm_ggml_free(wctx)

@@ -1001,3 +1001,118 @@ def test_mul_mat_group_argument_errors(dev, orc):
     bad[0].ldy = N - 1
     assert call(bad, 1) == -1
     dev.sync()
+
+
+# ------------------------------------------------------------------------------------------ Q6_K rows in planes
+def q6_K_planes_of(W, K):
+    """What chip_repack_q6_K writes, on the host: per row every ql field, then every qh, every scales, every d."""
+    N, nsb = W.shape[0], K // 256
+    b = W.reshape(N, nsb, 210)
+    return np.concatenate([b[:, :, 0:128].reshape(N, -1), b[:, :, 128:192].reshape(N, -1), b[:, :, 192:208].reshape(N, -1),
+                           b[:, :, 208:210].reshape(N, -1)], axis=1)
+
+
+@pytest.mark.parametrize("K,N", [(2048, 64), (4096, 1032), (14336, 304), (6144, 77), (196608, 3)])
+def test_q6_K_repack_to_planes_and_back(dev, K, N):
+    """chip_repack_q6_K moves every byte of a row to its plane (checked against the same permutation on the host), out of
+    place and in place, and the other direction gives the block order back; row lengths that leave a plane misaligned, rows
+    longer than the LDS and overlapping matrices are rejected."""
+    import cactus_amd as ca
+    W = np.random.default_rng(K + N).integers(0, 256, (N, K // 256 * 210), dtype=np.uint8)
+    P = dev.repack_q6_K(W, K, True)
+    assert np.array_equal(P, q6_K_planes_of(W, K))
+    assert np.array_equal(dev.repack_q6_K(W, K, True, in_place=True), P)
+    assert np.array_equal(dev.repack_q6_K(P, K, False), W)
+    assert np.array_equal(dev.repack_q6_K(P, K, False, in_place=True), W)
+    d = dev.alloc(1 << 20)
+    L = dev.lib
+    for bad_k in (256, 1024, 2048 + 256, 0):
+        assert L.chip_repack_q6_K(d.ptr, 210 * bad_k // 256, d.ptr + (1 << 19), 210 * bad_k // 256, bad_k, 2, 1, None) == ca.CHIP_EUNSUPPORTED
+        assert L.chip_mul_mat_supported(ca.Q6_K_PLANES, bad_k) == 0
+    assert L.chip_mul_mat_supported(ca.Q6_K_PLANES, 2048) == 1
+    assert L.chip_repack_q6_K(d.ptr, 1680, d.ptr + 1680, 1680, 2048, 4, 1, None) == ca.CHIP_EINVAL      # the two overlap
+    assert L.chip_repack_q6_K(d.ptr, 1678, d.ptr + (1 << 19), 1680, 2048, 4, 1, None) == ca.CHIP_EINVAL  # stride below a row
+    assert L.chip_repack_q6_K(d.ptr, 1680, d.ptr + (1 << 19), 1680, 2048, 0, 1, None) == ca.CHIP_OK
+    assert L.chip_repack_q6_K(d.ptr, 210 * 1024, d.ptr, 210 * 1024, 262144, 1, 1, None) == ca.CHIP_EUNSUPPORTED   # 215 040-byte rows
+
+
+@pytest.mark.parametrize("K,N", [(2048, 72), (4096, 1032), (14336, 4096), (8192, 264)])
+def test_q6_K_in_planes_gives_the_bits_of_q6_K(dev, orc, K, N):
+    """CHIP_TYPE_Q6_K_PLANES through every matmul entry point that takes it: bit for bit what the same entry point gives on
+    the block_q6_K rows the planes were made from (1, 2, 3, 4 tokens; larger batches against single passes of the GEMV), and
+    the oracle within tolerance; the entry points that read other layouts reject the type."""
+    import cactus_amd as ca
+    W = quantized_weights(O.Q6_K, K + N, N, K)
+    W2 = quantized_weights(O.Q6_K, K + N + 1, N, K)
+    P, P2 = dev.repack_q6_K(W, K), dev.repack_q6_K(W2, K)
+    PL = ca.Q6_K_PLANES
+    for n in (1, 2, 3, 4):
+        x = common.activations_f32(K + n, n, K)
+        y = dev.mul_mat(PL, P, x)
+        assert y.tobytes() == dev.mul_mat(O.Q6_K, W, x).tobytes(), n
+        if n == 1:
+            ref = orc.mul_mat(O.Q6_K, W, x, nthreads=8, want=("sum_abs",))
+            check_outputs(y, ref["y"], ref["sum_abs"], "Q6_K planes")
+        if dev.lib.chip_mul_mat_add_supported(O.Q6_K, K, N, n):
+            assert dev.lib.chip_mul_mat_add_supported(PL, K, N, n) == 1
+            b = common.activations_f32(N + n, n, N)
+            assert dev.mul_mat_add(PL, P, x, b).tobytes() == dev.mul_mat_add(O.Q6_K, W, x, b).tobytes(), n
+        y1, y2 = dev.mul_mat_pair(PL, P, P2, x)
+        w1, w2 = dev.mul_mat_pair(O.Q6_K, W, W2, x)
+        assert y1.tobytes() == w1.tobytes() and y2.tobytes() == w2.tobytes(), n
+        yt, ht = dev.mul_mat_store_t(PL, P, x, 8)
+        wt_, hw = dev.mul_mat_store_t(O.Q6_K, W, x, 8)
+        assert yt.tobytes() == wt_.tobytes() and ht.tobytes() == hw.tobytes(), n
+        if n != 3 and dev.lib.chip_mul_mat_pair_silu_mul_supported(O.Q6_K, K, N, n):
+            assert dev.lib.chip_mul_mat_pair_silu_mul_supported(PL, K, N, n) == 1
+            assert dev.mul_mat_pair_silu_mul(PL, P, P2, x).tobytes() == dev.mul_mat_pair_silu_mul(O.Q6_K, W, W2, x).tobytes(), n
+            if dev.lib.chip_norm_before_supported(O.Q6_K, K, n):
+                assert dev.lib.chip_norm_before_supported(PL, K, n) == 1
+                nw = norm_weight(N, K)
+                got, got_normed = dev.mul_mat_pair_silu_mul(PL, P, P2, x, norm=(nw, 1e-6))
+                want, want_normed = dev.mul_mat_pair_silu_mul(O.Q6_K, W, W2, x, norm=(nw, 1e-6))
+                assert got.tobytes() == want.tobytes() and got_normed.tobytes() == want_normed.tobytes(), n
+    if N <= 1032:
+        for n in (5, 8, 11):                    # passes of up to 8 tokens of the same kernel
+            x = common.activations_f32(K + n, n, K)
+            want = np.concatenate([dev.mul_mat(O.Q6_K, W, x[i:i + 1]) for i in range(n)])
+            assert dev.mul_mat(PL, P, x).tobytes() == want.tobytes(), n
+    d = dev.alloc(1 << 16)
+    L = dev.lib
+    assert L.chip_get_rows(PL, d.ptr, 1680, 0, 0, 2048, 4, d.ptr, 1, 1, 1, 0, 0, d.ptr, 8192, 0, 0, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_block_isums(PL, d.ptr, 1680, 2048, 4, d.ptr, 1, d.ptr, d.ptr, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_mul_mat_id(PL, d.ptr, 1680, 4 * 1680, 2048, 4, 2, d.ptr + 32768, 2048, 1, d.ptr + 49152, 1, 1, 1, d.ptr + 49408, 4,
+                             d.ptr + 16384, 16384, None) == ca.CHIP_EUNSUPPORTED
+    assert L.chip_mul_mat(PL, d.ptr + 2, 1680, 2048, 4, d.ptr + 32768, 2048, 1, d.ptr + 49152, 4, d.ptr + 16384, 16384, None) == ca.CHIP_EINVAL
+
+
+@pytest.mark.parametrize("K,members", [(4096, ((O.Q4_K, 4096), (O.Q4_K, 1024), ("planes", 1024))), (2048, (("planes", 520), ("planes", 8), ("planes", 264))),
+                                       (2048, ((O.Q6_K, 520), (O.Q5_K, 72), ("planes", 264))), (2048, ((O.Q3_K, 136), ("planes", 264), (O.Q2_K, 64)))],
+                         ids=["q4_K_M-qkv", "planes-only", "blocks-and-planes", "with-q3_K"])
+def test_group_members_in_planes(dev, K, members):
+    """chip_mul_mat_group and chip_mul_mat_group_rope_norm with Q6_K members in planes (beside Q4_K / Q5_K members: the kernel
+    family of the Q4_K_M mix; beside block-order Q6_K or low-bit members: the wide family): every output bit for bit the group
+    with those members in block order."""
+    import cactus_amd as ca
+    blocks, planes = [], []
+    for i, (wt, N) in enumerate(members):
+        real = O.Q6_K if wt == "planes" else wt
+        W = quantized_weights(real, K + N + i, N, K)
+        blocks.append((real, W))
+        planes.append((ca.Q6_K_PLANES, dev.repack_q6_K(W, K)) if wt == "planes" else (real, W))
+    for n in (1, 2, 4, 3, 8):
+        x = common.activations_f32(K + n + 5, n, K)
+        for got, want in zip(dev.mul_mat_group(planes, x), dev.mul_mat_group(blocks, x)):
+            assert got.tobytes() == want.tobytes(), n
+    if members[0][1] % 128 == 0 and blocks[0][0] in (O.Q4_K, O.Q6_K):
+        hd = 128
+        ropes = [(hd, hd, 0, ("f32",)), (hd, hd, 0, ("f32", "f16")), None]
+        nw = norm_weight(K, K)
+        for n in (1, 2, 4):
+            x = common.activations_f32(K + n, n, K)
+            pos = np.array([37, 0, 4095, 100000][:n], np.int32)
+            rc, want = dev.mul_mat_group_rope(blocks, x, pos, ropes, freq_base=500000.0, norm=(nw, 1e-5))
+            rc, got = dev.mul_mat_group_rope(planes, x, pos, ropes, freq_base=500000.0, norm=(nw, 1e-5))
+            for g, w in zip(got, want):
+                for key in w:
+                    assert g[key].tobytes() == w[key].tobytes(), (n, key)
