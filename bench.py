@@ -509,7 +509,7 @@ class Trace:
         self.bufs = {}
         self.head_type = ca.Q6_K
 
-    def q6_K_to(self, planes):
+    def q6_K_to(self, planes, head=True):
         """Every Q6_K matrix of the arena to planes (what the backend keeps for its decode GEMVs) or back to block order,
         in place; the launches that follow name the layout by its type."""
         ca, dev, L = self.ca, self.dev, self.dev.lib
@@ -518,7 +518,7 @@ class Trace:
             for nm, (t, p, N, K) in self.weights(l).items():
                 if t == have:
                     dev.check(L.chip_repack_q6_K(p, dev.row_size(t, K), p, dev.row_size(t, K), K, N, int(planes), None))
-        if self.head_type == have:
+        if self.head_type == have and (head or not planes):
             p = self.arena.ptr + self.head_off
             dev.check(L.chip_repack_q6_K(p, dev.row_size(have, self.H), p, dev.row_size(have, self.H), self.H, self.V, int(planes), None))
         dev.sync()

@@ -122,7 +122,8 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
     // too few rows to give every CU an 8-wave group use 4-wave groups instead.
     // The one-token kernel that quantizes in its prologue runs three such groups per CU (24 waves: with one step of loads
     // in flight per wave the bytes in flight per CU grow with the waves; measured on 66 MB and 431 MB: 3 % faster than two).
-    const int64_t per_cu = tune("CHIP_GEMV_PER_CU", (lds_bytes <= 24 * 1024) ? ((FUSEQ && NTOK == 1) ? 3 : 2) : 1);
+    // (Q6_K rows in planes: two - the 128256 x 4096 output head 81.5 -> 77.2 us; its aligned loads saturate with 16 waves)
+    const int64_t per_cu = tune("CHIP_GEMV_PER_CU", (lds_bytes <= 24 * 1024) ? ((FUSEQ && NTOK == 1 && WT != T_Q6_K_P) ? 3 : 2) : 1);
     const int64_t tiles = ceil_div(N, R);
     if constexpr (FUSEQ) {
         // When the matrix gives each of 16 waves per CU at most one tile, the prologue is a large share of the
@@ -130,7 +131,7 @@ static hipError_t launch_typed(const void *W, size_t nb01, int64_t K, int64_t N,
         // every such shape except long Q8_0 rows (K > 8192), where two 8-wave groups win.
         const bool one_tile_per_wave = tiles <= 16 * (int64_t)cus && tiles > 8 * (int64_t)cus;
         const bool long_q8_0_row = Traits<WT>::ACT == T_Q8_0 && NTOK == 1 && K > 8192;
-        if (one_tile_per_wave && !long_q8_0_row)
+        if (one_tile_per_wave && !long_q8_0_row && tune("CHIP_GEMV_ONE_TILE_WIDE", 1) != 0)
             return launch_one<WT, NTOK, R, 1024, true>(W, nb01, K, N, x, ldx, ws, ws_stride, y, ldy, lds_bytes, cus, lim, st, sec);
     }
     if constexpr (FUSEQ && NTOK >= 2) {

@@ -197,13 +197,10 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
     const int fam = gemv_group_family(mats[0].wtype);
     size_t img = 0;
     int64_t tiles = 0;
-    double cost[GROUP_MAX], total_cost = 0;
     for (int i = 0; i < count; i++) {
         const size_t b = image_bytes(mats[i].wtype, K);
         if (b > img) img = b;
         tiles += ceil_div(mats[i].N, (int64_t)rows_per_step(mats[i].wtype));
-        cost[i] = (double)mats[i].N * (double)mats[i].nb01;              // bytes to stream
-        total_cost += cost[i];
     }
     // members whose ROPE node runs in their epilogue: one row per step (pairs of rows per wave), the cos / sin table behind the image
     bool rope = false;
@@ -226,34 +223,39 @@ hipError_t launch_gemv_group(const GroupMat *mats, int count, int64_t K, const f
     if (lds_bytes > (size_t)lim.max_lds_per_block) return hipErrorInvalidValue;
     // As the single-matrix launcher: a persistent grid; one 16-wave workgroup per CU while every wave gets at most a
     // couple of tiles (the prologue is then most of the kernel and is paid once per CU), else two 8-wave workgroups.
-    const int wgs = tiles <= 32 * (int64_t)cus ? 1024 : 512;
+    const int wgs = (int)tune("CHIP_GROUP_WGS", tiles <= 32 * (int64_t)cus ? 1024 : 512);
     // the K-quant and block-32 kernels keep 4 - 5 waves per SIMD (the registers of their most demanding member type): two
     // 8-wave workgroups per CU; the F16 kernel keeps 8 and takes three for one token
-    const int per_cu = (wgs == 1024 || lds_bytes > 24 * 1024) ? 1 : (fam == 2 && n == 1 && !prepared ? 3 : 2);
+    const int per_cu = (int)tune("CHIP_GROUP_PER_CU", (wgs == 1024 || lds_bytes > 24 * 1024) ? 1 : (fam == 2 && n == 1 && !prepared ? 3 : 2));
     int grid = cus * per_cu;
     const int64_t max_useful = ceil_div(tiles, (int64_t)(wgs / 64));
     if (grid > max_useful) grid = (int)max_useful;
     if (grid < count) grid = count;
-    // workgroups in proportion to the bytes each member streams (largest remainder), at least one each
-    int blocks[GROUP_MAX], given = 0;
-    double frac[GROUP_MAX];
+    // Workgroups per member so that the waves that stream the most bytes stream as few as possible.  A member's waves walk its
+    // tiles (a row, R rows, or the two rows of a rotated pair) in turn, so each streams ceil(tiles / waves) tiles: every member
+    // starts with one workgroup, each further one goes to the member whose waves stream the most, and at the end a member keeps
+    // only as many as that load needs.  (In proportion to the members' bytes, wq + wk + wv of a Q4_K_M layer left wv's waves two
+    // 3360-byte rows each while wq's took two 2304-byte rows: 6.6 us against 5.8 us this way.)
+    const int waves = wgs / 64;
+    int64_t mtiles[GROUP_MAX];
+    double tile_bytes[GROUP_MAX];
     for (int i = 0; i < count; i++) {
-        const double share = cost[i] / total_cost * grid;
-        blocks[i] = (int)share;
-        if (blocks[i] < 1) blocks[i] = 1;
-        frac[i] = share - (double)blocks[i];
-        given += blocks[i];
+        const int64_t r = mats[i].rope.table ? 2 : rows_per_step(mats[i].wtype);
+        mtiles[i] = ceil_div(mats[i].N, r);
+        tile_bytes[i] = (double)r * (double)mats[i].nb01;
     }
+    auto wave_load = [&](int i, int b) { return (double)ceil_div(mtiles[i], (int64_t)b * waves) * tile_bytes[i]; };
+    int blocks[GROUP_MAX], given = count;
+    for (int i = 0; i < count; i++) blocks[i] = 1;
     while (given < grid) {
-        int best = 0;
-        for (int i = 1; i < count; i++) if (frac[i] > frac[best]) best = i;
-        blocks[best]++; frac[best] -= 1.0; given++;
+        int worst = 0;
+        for (int i = 1; i < count; i++) if (wave_load(i, blocks[i]) > wave_load(worst, blocks[worst])) worst = i;
+        if (ceil_div(mtiles[worst], (int64_t)blocks[worst] * waves) <= 1) break;      // one tile per wave already: nothing left to split
+        blocks[worst]++; given++;
     }
-    while (given > grid) {                                                // the minimum of one each overshot
-        int best = -1;
-        for (int i = 0; i < count; i++) if (blocks[i] > 1 && (best < 0 || frac[i] < frac[best])) best = i;
-        if (best < 0) break;
-        blocks[best]--; frac[best] += 1.0; given--;
+    for (int i = 0; i < count; i++) {
+        const int64_t per_wave = ceil_div(mtiles[i], (int64_t)blocks[i] * waves);
+        blocks[i] = (int)ceil_div(ceil_div(mtiles[i], per_wave), (int64_t)waves);
     }
     GroupKernelArgs ga{};
     ga.count = count;
