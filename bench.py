@@ -730,7 +730,7 @@ def bench_whole_layers(dev, hip, trace, n, n_kv, fold=True):
     # up to 4 tokens the norms run in the prologue of the projections that read them and the residual ADDs in the store of
     # the projections in front of them, where the library has those forms for the model's types
     Wl = trace.weights(0)
-    deferred = (fold and n <= 4 and all(L.chip_norm_before_supported(Wl[nm][0], H, n) == 1 for nm in ("wq", "wk", "wv", "gate")) and
+    deferred = (fold and n <= 2 and all(L.chip_norm_before_supported(Wl[nm][0], H, n) == 1 for nm in ("wq", "wk", "wv", "gate")) and
                 L.chip_mul_mat_pair_silu_mul_supported(Wl["gate"][0], H, FF, n) == 1 and
                 L.chip_mul_mat_add_supported(Wl["wo"][0], H, H, n) == 1 and L.chip_mul_mat_add_supported(Wl["down"][0], FF, H, n) == 1)
     nb = ca.NormBefore(wn.ptr, 1e-5, cur.ptr, H)

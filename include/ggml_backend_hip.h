@@ -65,7 +65,7 @@ CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_gated_pairs(void);
 /* ROPE nodes that ran in the epilogue of the projection in front of them (Q's and K's, in the group launch of wq / wk / wv). */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_rope_epilogues(void);
 /* RMS_NORM + weight MUL pairs (cactus/llama-graph.cpp build_norm) that ran in the prologue of the projections reading them (the
- * group launch of wq / wk / wv, the gated FFN launch), up to 4 tokens. */
+ * group launch of wq / wk / wv, the gated FFN launch), up to 2 tokens (at 4 the norm's own launch is the faster form). */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_norms_in_prologue(void);
 /* Residual ADD nodes that ran where the projection in front of them (wo, ffn_down) stores its result, up to 4 tokens. */
 CACTUS_GGML_API unsigned long long lm_ggml_backend_hip_get_residual_adds(void);
