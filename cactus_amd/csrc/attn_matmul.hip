@@ -94,7 +94,7 @@ __device__ __forceinline__ float *col_y2(const BatchedArgs &a, int64_t b0, int64
 template <int LPR>
 __global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedArgs a) {
     constexpr int RPS = 64 / LPR;                                    // rows per wave step
-    constexpr int UNROLL = 4;                                        // row steps in flight
+    constexpr int UNROLL = 4;                                        // row steps in flight (2 and 8 measured slower: kq of a decode step 5.7 -> 5.95 / 6.65 us)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPR, grp = lane / LPR;
     const int64_t b0 = blockIdx.y;
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(AM_THREADS) void mm_f16_short_rows_kernel(BatchedAr
 }
 
 // ---- long rows: a workgroup takes AM_ROWS rows, wave w the chunks w * 64 + lane, + 256, ... of each ----
-constexpr int AM_ROWS = 4;
+template <int AM_ROWS>
 __global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArgs a) {
     __shared__ float part[AM_WAVES][AM_ROWS][AM_COLS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -578,10 +578,15 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
             default: hipLaunchKernelGGL(mm_f16_short_rows_kernel<32>, grid, dim3(AM_THREADS), 0, st, a); break;
         }
     } else {
-        int64_t gx = ceil_div(N, (int64_t)AM_ROWS);
+        // four rows per workgroup; two while that leaves fewer than two workgroups per CU (kqv of a decode step: 128 rows per
+        // KV head - twice the workgroups re-read the activation columns from L2 and stream the cache rows with twice the waves:
+        // 6.57 -> 6.01 us over a cold 8 MB cache; one row per workgroup 6.54 us)
+        const int rows = (int)tune("CHIP_KQV_ROWS", ceil_div(N, (int64_t)4) * ne02 < 2 * (int64_t)cus ? 2 : 4);
+        int64_t gx = ceil_div(N, (int64_t)rows);
         const int64_t cap = ceil_div((int64_t)cus * 8, ne02);
         if (gx > cap) gx = cap;
-        hipLaunchKernelGGL(mm_f16_long_rows_kernel, dim3((unsigned)gx, (unsigned)ne02), dim3(AM_THREADS), 0, st, a);
+        if (rows == 2) hipLaunchKernelGGL(mm_f16_long_rows_kernel<2>, dim3((unsigned)gx, (unsigned)ne02), dim3(AM_THREADS), 0, st, a);
+        else           hipLaunchKernelGGL(mm_f16_long_rows_kernel<4>, dim3((unsigned)gx, (unsigned)ne02), dim3(AM_THREADS), 0, st, a);
     }
     return hipGetLastError();
 }

@@ -419,7 +419,8 @@ weight_arg weight_for(backend_ctx *c, const lm_ggml_tensor *w, int64_t n) {
         bc->planes_failed = true;
         return own;
     }
-    if (chip_repack_q6_K(w->data, w->nb[1], p, row, K, N, 1, c->stream) != CHIP_OK) {
+    // finished before the copy is entered: another backend instance on the same buffer reads it from its own stream
+    if (chip_repack_q6_K(w->data, w->nb[1], p, row, K, N, 1, c->stream) != CHIP_OK || chip_stream_synchronize(c->stream) != CHIP_OK) {
         chip_free(p);
         bc->planes_failed = true;
         return own;
