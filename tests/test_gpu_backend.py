@@ -1213,3 +1213,54 @@ def test_q6_K_weights_are_read_from_a_copy_in_planes_at_decode(host, orc):
         L.lm_ggml_free(ctx)
     L.lm_ggml_backend_free(hip)
     L.lm_ggml_free(wctx)
+
+
+def test_planes_copy_of_a_weight_that_is_a_view(host, orc):
+    """A Q6_K weight that is a row range of a larger tensor (as a loader slices a fused matrix): the decode matmul reads a copy
+    in planes of that range, a set_tensor on the parent drops it, rows of K % 2048 != 0 get no copy."""
+    import cactus_amd
+    L = host.L
+    K, N_all, r0, N = 2048, 96, 32, 40
+    w_all = orc.quantize_weights(O.Q6_K, common.weights_f32(91, N_all, K))
+    w_new = orc.quantize_weights(O.Q6_K, common.weights_f32(92, N_all, K))
+    cdev = cactus_amd.Device(0)
+    dev = L.lm_ggml_backend_reg_dev_get(host.reg, 0)
+    hip = L.lm_ggml_backend_dev_init(dev, None)
+    wctx = host.context(with_graph=False)
+    tw = host.tensor_2d(wctx, O.Q6_K, K, N_all, "w_all")
+    t768 = host.tensor_2d(wctx, O.Q6_K, 768, 24, "w_768")
+    wbuf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(wctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    host.set(tw, w_all)
+    w768 = orc.quantize_weights(O.Q6_K, common.weights_f32(93, 24, 768))
+    host.set(t768, w768)
+    row = w_all.shape[1]
+    blib = C.CDLL(cactus_amd.BACKEND_LIB)
+    for name in ("copies", "dropped", "matmuls"):
+        getattr(blib, "lm_ggml_backend_hip_get_planes_" + name).restype = C.c_ulonglong
+    ctx = host.context()
+    view = L.lm_ggml_view_2d(ctx, tw, K, N, row, r0 * row)
+    tx = host.tensor_2d(ctx, O.F32, K, 1, "x")
+    ty = L.lm_ggml_mul_mat(ctx, view, tx)
+    tx7 = host.tensor_2d(ctx, O.F32, 768, 1, "x7")
+    ty7 = L.lm_ggml_mul_mat(ctx, t768, tx7)
+    g = L.lm_ggml_new_graph(ctx)
+    L.lm_ggml_build_forward_expand(g, ty)
+    L.lm_ggml_build_forward_expand(g, ty7)
+    buf = L.lm_ggml_backend_alloc_ctx_tensors_from_buft(ctx, L.lm_ggml_backend_dev_buffer_type(dev))
+    x, x7 = common.activations_f32(94, 1, K), common.activations_f32(95, 1, 768)
+    host.set(tx, x)
+    host.set(tx7, x7)
+    copies, dropped = blib.lm_ggml_backend_hip_get_planes_copies(), blib.lm_ggml_backend_hip_get_planes_dropped()
+    assert L.lm_ggml_backend_graph_compute(hip, g) == 0
+    assert blib.lm_ggml_backend_hip_get_planes_copies() - copies == 1                      # the view's rows; none for K = 768
+    assert host.get(ty, np.float32, (1, N)).tobytes() == cdev.mul_mat(O.Q6_K, w_all[r0:r0 + N], x).tobytes()
+    assert host.get(ty7, np.float32, (1, 24)).tobytes() == cdev.mul_mat(O.Q6_K, w768, x7).tobytes()
+    host.set(tw, w_new)                                                                    # through the parent: overlaps the copy
+    assert blib.lm_ggml_backend_hip_get_planes_dropped() - dropped == 1
+    assert L.lm_ggml_backend_graph_compute(hip, g) == 0
+    assert host.get(ty, np.float32, (1, N)).tobytes() == cdev.mul_mat(O.Q6_K, w_new[r0:r0 + N], x).tobytes()
+    L.lm_ggml_backend_buffer_free(buf)
+    L.lm_ggml_backend_buffer_free(wbuf)
+    L.lm_ggml_free(ctx)
+    L.lm_ggml_free(wctx)
+    L.lm_ggml_backend_free(hip)

@@ -1024,8 +1024,17 @@ def test_q6_K_repack_to_planes_and_back(dev, K, N):
     assert np.array_equal(dev.repack_q6_K(W, K, True, in_place=True), P)
     assert np.array_equal(dev.repack_q6_K(P, K, False), W)
     assert np.array_equal(dev.repack_q6_K(P, K, False, in_place=True), W)
-    d = dev.alloc(1 << 20)
     L = dev.lib
+    if N <= 304:                                         # rows wider apart than they are long, on both sides
+        row, ps, pd = W.shape[1], W.shape[1] + 420, W.shape[1] + 64
+        src = np.full((N, ps), 0xa5, np.uint8)
+        src[:, :row] = W
+        ds, dd = dev.to_device(src), dev.to_device(np.full((N, pd), 0x5a, np.uint8))
+        dev.check(L.chip_repack_q6_K(ds.ptr, ps, dd.ptr, pd, K, N, 1, None))
+        dev.sync()
+        out = dd.download(np.uint8, N * pd).reshape(N, pd)
+        assert np.array_equal(out[:, :row], P) and (out[:, row:] == 0x5a).all()
+    d = dev.alloc(1 << 20)
     for bad_k in (256, 1024, 2048 + 256, 0):
         assert L.chip_repack_q6_K(d.ptr, 210 * bad_k // 256, d.ptr + (1 << 19), 210 * bad_k // 256, bad_k, 2, 1, None) == ca.CHIP_EUNSUPPORTED
         assert L.chip_mul_mat_supported(ca.Q6_K_PLANES, bad_k) == 0
