@@ -581,7 +581,9 @@ hipError_t launch_mul_mat_f16_batched(const void *W, size_t nb01, size_t nb02, i
         // four rows per workgroup; two while that leaves fewer than two workgroups per CU (kqv of a decode step: 128 rows per
         // KV head - twice the workgroups re-read the activation columns from L2 and stream the cache rows with twice the waves:
         // 6.57 -> 6.01 us over a cold 8 MB cache; one row per workgroup 6.54 us)
-        const int rows = (int)tune("CHIP_KQV_ROWS", ceil_div(N, (int64_t)4) * ne02 < 2 * (int64_t)cus ? 2 : 4);
+        // (up to 8192 cached positions: with longer rows the columns' re-reads cost more than the waves gain - 16384 positions
+        // 13.7 -> 14.6 us, 32768 22.8 -> 26.8 us; 1024 positions 5.14 -> 4.47 us)
+        const int rows = (int)tune("CHIP_KQV_ROWS", (K <= 8192 && ceil_div(N, (int64_t)4) * ne02 < 2 * (int64_t)cus) ? 2 : 4);
         int64_t gx = ceil_div(N, (int64_t)rows);
         const int64_t cap = ceil_div((int64_t)cus * 8, ne02);
         if (gx > cap) gx = cap;
