@@ -138,22 +138,37 @@ int chip_get_device_info(chip_device_info *out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
-    hipDeviceProp_t p;
-    e = hipGetDeviceProperties(&p, dev);
-    if (e != hipSuccess) return (int)e;
-    DeviceLimits lim;
-    int rc = current_limits(lim);
-    if (rc) return rc;
-    out->device = dev;
-    out->compute_units = p.multiProcessorCount;
-    out->wavefront_size = p.warpSize;
-    out->max_lds_per_block = lim.max_lds_per_block;
-    out->clock_khz = p.clockRate;
-    out->xcd_count = 0;
+    constexpr int MAX_DEVICES = 64;
+    if (dev < 0 || dev >= MAX_DEVICES) return CHIP_EINVAL;
+    // the properties are read once per device (the query takes milliseconds); the memory figures every time
+    static chip_device_info fixed[MAX_DEVICES];
+    static bool have[MAX_DEVICES];
+    static std::mutex mu;
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        if (!have[dev]) {
+            hipDeviceProp_t p;
+            e = hipGetDeviceProperties(&p, dev);
+            if (e != hipSuccess) return (int)e;
+            DeviceLimits lim;
+            int rc = current_limits(lim);
+            if (rc) return rc;
+            chip_device_info &f = fixed[dev];
+            std::memset(&f, 0, sizeof(f));
+            f.device = dev;
+            f.compute_units = p.multiProcessorCount;
+            f.wavefront_size = p.warpSize;
+            f.max_lds_per_block = lim.max_lds_per_block;
+            f.clock_khz = p.clockRate;
+            f.xcd_count = 0;
+            std::snprintf(f.name, sizeof(f.name), "%s", p.name);
+            std::snprintf(f.arch, sizeof(f.arch), "%s", p.gcnArchName);
+            have[dev] = true;
+        }
+        *out = fixed[dev];
+    }
     size_t fr = 0, tot = 0;
     if (hipMemGetInfo(&fr, &tot) == hipSuccess) { out->hbm_free = fr; out->hbm_total = tot; }
-    std::snprintf(out->name, sizeof(out->name), "%s", p.name);
-    std::snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
     return CHIP_OK;
 }
 
