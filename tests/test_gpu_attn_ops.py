@@ -69,6 +69,28 @@ def test_soft_max_in_place_and_strided(dev, orc):
     assert np.array_equal(out[:, ne00:], buf[:, ne00:])                      # the padding between rows is untouched
 
 
+@pytest.mark.parametrize("ne00", [8192, 16384, 40960, 131072])
+def test_soft_max_of_few_long_rows_equals_the_same_rows_in_a_large_batch(dev, orc, ne00):
+    """Few rows of 8192 values or more (a decode step over a long context) run with 1024 threads per row: bit for bit what the
+    same rows give among more rows than that kernel takes (256 threads per row), with an F16 causal mask and in place; the
+    oracle within the soft-max tolerance."""
+    import cactus_amd as ca
+    rng = np.random.default_rng(ne00)
+    few, many = 6, 134
+    x = (rng.standard_normal((many, ne00)) * 5).astype(np.float32)
+    x[0, :8] = [30.0, -30.0, 88.0, -104.0, 0.0, 1e-3, -200.0, 50.0]
+    mask = np.zeros((1, ne00), np.float16)
+    mask[0, ne00 - 37:] = -np.inf
+    y_many = dev.soft_max(x[:, None, :], mask, 0.0884)[:, 0]
+    y_few = dev.soft_max(x[:few, None, :], mask, 0.0884)[:, 0]
+    assert y_few.tobytes() == y_many[:few].tobytes()
+    assert_soft_max_close(y_few[None], orc.soft_max(x[None, :few], np.repeat(mask, few, 0), 0.0884))
+    d, dm = dev.to_device(x[:few]), dev.to_device(mask)
+    dev.check(dev.lib.chip_soft_max(d.ptr, ne00, dm.ptr, ca.F16, ne00, 1, few, 0.0884, 0.0, d.ptr, ne00, None))
+    dev.sync()
+    assert d.download(np.float32, few * ne00).tobytes() == y_few.tobytes()
+
+
 def test_soft_max_declines_what_it_does_not_restate(dev):
     import cactus_amd as ca
     x = dev.to_device(np.zeros((2, 64), np.float32))
