@@ -326,7 +326,9 @@ ATTN_SHAPES = [(128, 32, 8, 1, 4096, 4096), (128, 32, 8, 7, 288, 512), (64, 8, 8
                # 65 to 128 pairs: kqv with K split over workgroups (eight column groups), kq through the GEMM
                (128, 32, 8, 32, 1048, 2048), (96, 12, 2, 17, 520, 1024),
                # more than 128 pairs over a long cache (K not a multiple of the GEMM's 64-value stage)
-               (128, 8, 2, 40, 2056, 4096), (64, 8, 2, 64, 4104, 4352)]
+               (128, 8, 2, 40, 2056, 4096), (64, 8, 2, 64, 4104, 4352),
+               # a decode step over a long context (kqv rows of more than 8192 values: four cache rows per workgroup)
+               (128, 32, 8, 1, 16384, 16384), (128, 8, 2, 1, 9008, 12288)]
 
 
 @pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", ATTN_SHAPES)
@@ -356,7 +358,8 @@ def test_attention_matmuls_over_the_cache(dev, orc, hd, n_head, n_head_kv, n_tok
 # (hd, n_head, n_head_kv, n_tokens, n_kv, kv_size): LLaMA-3-8B's decode step; multi-head attention with 1, 2 and 4 tokens; 3 and 2
 # query heads per KV head; a cache short enough for the short-rows kernel; ragged sizes
 MERGE_SHAPES = [(128, 32, 8, 1, 4096, 4096), (64, 4, 4, 1, 1000, 1024), (64, 4, 4, 4, 520, 1024), (128, 8, 8, 2, 264, 512),
-                (256, 6, 2, 1, 4104, 8192), (96, 4, 2, 2, 72, 128), (128, 2, 1, 1, 5000, 8192), (80, 8, 2, 1, 136, 256)]
+                (256, 6, 2, 1, 4104, 8192), (96, 4, 2, 2, 72, 128), (128, 2, 1, 1, 5000, 8192), (80, 8, 2, 1, 136, 256),
+                (128, 8, 2, 1, 16392, 16640)]
 
 
 @pytest.mark.parametrize("hd,n_head,n_head_kv,n_tokens,n_kv,kv_size", MERGE_SHAPES)
