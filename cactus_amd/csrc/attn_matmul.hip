@@ -164,11 +164,15 @@ template <int AM_ROWS>
 __global__ __launch_bounds__(AM_THREADS) void mm_f16_long_rows_kernel(BatchedArgs a) {
     __shared__ float part[AM_WAVES][AM_ROWS][AM_COLS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t b0 = blockIdx.y;
+    // Workgroups are handed to the 8 XCDs in turn, in the order of their linear index (x fastest).  The KV head is that index
+    // modulo the number of heads, so that with 8 KV heads all workgroups of a head run on one XCD and the head's activation
+    // columns (the probabilities: 64 KB per head at 4096 positions) reach one L2 instead of all eight.
+    const uint32_t linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int64_t b0 = linear % gridDim.y, bx = linear / gridDim.y;
     const uint8_t *Wb = a.W + b0 * a.nb02;
     const int64_t chunks = a.K / 8;
     const int64_t cols = a.r2 * a.n;
-    for (int64_t r0 = (int64_t)blockIdx.x * AM_ROWS; r0 < a.N; r0 += (int64_t)gridDim.x * AM_ROWS) {
+    for (int64_t r0 = bx * AM_ROWS; r0 < a.N; r0 += (int64_t)gridDim.x * AM_ROWS) {
         const uint8_t *wrow[AM_ROWS];
 #pragma unroll
         for (int r = 0; r < AM_ROWS; r++) wrow[r] = Wb + (r0 + r < a.N ? r0 + r : a.N - 1) * a.nb01;      // clamped, unused past N
