@@ -129,6 +129,10 @@ blib.lm_ggml_backend_hip_get_grouped_matmuls.restype = C.c_ulonglong
 print("projections run in group launches so far", blib.lm_ggml_backend_hip_get_grouped_matmuls(), "(3 graphs)", flush=True)
 blib.lm_ggml_backend_hip_get_quantizers_skipped.restype = C.c_ulonglong
 print("quantizers skipped so far", blib.lm_ggml_backend_hip_get_quantizers_skipped(), flush=True)
+blib.lm_ggml_backend_hip_get_planes_copies.restype = C.c_ulonglong
+blib.lm_ggml_backend_hip_get_planes_bytes.restype = C.c_ulonglong
+print("Q6_K weights read from a copy in planes:", blib.lm_ggml_backend_hip_get_planes_copies(), "copies,",
+      blib.lm_ggml_backend_hip_get_planes_bytes() >> 20, "MiB", flush=True)
 ts = []
 for it in range(20):
     t0 = time.perf_counter()
