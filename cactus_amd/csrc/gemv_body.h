@@ -367,18 +367,25 @@ template <> struct Traits<T_Q3_K> : Traits<T_Q6_K> {
     // block_q3_K (ggml-common.h:273-278): hmask[32] | qs[64] | scales[12] | fp16 d, 110 bytes, 2-byte aligned.
     // value = d * (scale - 32) * (q - 4), q = the two bits of qs plus 4 where the bit 4 h + v of hmask[l] is set
     struct W { uint32_t q[16]; float d; int sc[4]; };            // q[4v + k]: values 0..7 of group v; the 4 comes off through the block sums
-    struct Raw { u32x4 qs, hm; uint32_t s0, s1, s2, d; };
+    // The 14 bytes behind qs (12 of packed scales, fp16 d) belong to all four lanes of a super-block: lane j of the quad fetches
+    // one dword of them (bytes 96, 100, 104 and, for the fourth, 106: the last two scale bytes and d - no byte past the block)
+    // and the quad hands them round by DPP: three load instructions per step instead of six (4096 x 14336 at one token
+    // 12.2 -> 11.7 us, the other shapes within 2 %).
+    struct Raw { u32x4 qs, hm; uint32_t tail; };
     __device__ static __forceinline__ void load_raw(Raw &r, const uint8_t *row, int u) {
-        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1;
+        const int sb = u >> 2, h = (u >> 1) & 1, ip = u & 1, j = u & 3;
         const uint8_t *p = row + (size_t)sb * BYTES_Q3_K;
         r.qs = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 32 + 32 * h + 16 * ip));
         r.hm = WLOAD(reinterpret_cast<const u32x4_a2 *>(p + 16 * ip));
-        r.s0 = WLOAD(reinterpret_cast<const u32_a2 *>(p + 96));
-        r.s1 = WLOAD(reinterpret_cast<const u32_a2 *>(p + 100));
-        r.s2 = WLOAD(reinterpret_cast<const u32_a2 *>(p + 104));
-        r.d  = WLOAD(reinterpret_cast<const unsigned short *>(p + 108));
+        r.tail = WLOAD(reinterpret_cast<const u32_a2 *>(p + 96 + (j < 3 ? 4 * j : 10)));
     }
-    __device__ static __forceinline__ void decode(W &w, const Raw &r, int u) {
+    __device__ static __forceinline__ void decode(W &w, const Raw &rr, int u) {
+        struct { u32x4 qs, hm; uint32_t s0, s1, s2, d; } r;
+        r.qs = rr.qs; r.hm = rr.hm;
+        r.s0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)rr.tail, 0x00, 0xf, 0xf, false);
+        r.s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)rr.tail, 0x55, 0xf, 0xf, false);
+        r.s2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)rr.tail, 0xAA, 0xf, 0xf, false);
+        r.d = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)rr.tail, 0xFF, 0xf, 0xf, false) >> 16;
         const int h = (u >> 1) & 1, ip = u & 1;
         w.d = h2f(r.d);
         const uint32_t lo[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w}, hm[4] = {r.hm.x, r.hm.y, r.hm.z, r.hm.w};
